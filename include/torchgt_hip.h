@@ -1,0 +1,122 @@
+/*
+ * torchgt_hip.h — C ABI of the MI355X (gfx950) sparse-attention library.
+ *
+ * The reference (zxmeng98/torchgt) has no FFI layer: its hot path is the Python
+ * method CoreAttention.sparse_attention / sparse_attention_bias, a chain of a
+ * dozen ATen / torch_scatter kernels.  These entry points are what a binding for
+ * that path attaches to; each comment names the reference code it replaces.
+ *
+ * Conventions
+ *   - every pointer named d_* is DEVICE memory of the current HIP device; h_* is
+ *     host memory; `stream` is a hipStream_t passed as void*.
+ *   - all functions return 0 (TGT_OK) or a negative error code and write no
+ *     output on error; tgt_last_error() gives a per-thread message.
+ *   - inputs are borrowed and never modified; nothing here synchronises the
+ *     stream except tgt_plan_create / tgt_plan_export.
+ *   - node features are row-major [N, H, d] (the reference's [b, S, H, d] view
+ *     flattened over b*S, attn_module.py:141-143).
+ */
+#ifndef TORCHGT_HIP_H
+#define TORCHGT_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TGT_OK                 0
+#define TGT_ERR_INVALID_ARG   -1   /* null pointer, negative size, bad enum        */
+#define TGT_ERR_INDEX_RANGE   -2   /* an edge endpoint is outside [0, N)            */
+#define TGT_ERR_UNSUPPORTED   -3   /* (H, d, dtype) combination has no kernel       */
+#define TGT_ERR_HIP           -4   /* a HIP runtime call failed                     */
+#define TGT_ERR_WORKSPACE     -5   /* workspace too small / misaligned              */
+
+/* element type of q, k, v, out, bias and the gradients */
+#define TGT_DTYPE_F32   0
+#define TGT_DTYPE_BF16  1
+
+/* how the additive attention bias is supplied (added AFTER the +-5 clamp,
+ * models/graphormer_dist_graph_level.py:262-267) */
+#define TGT_BIAS_NONE      0
+#define TGT_BIAS_EDGE_HEAD 1   /* [E, H], one value per edge and head, caller's edge order */
+#define TGT_BIAS_EDGE      2   /* [E], one value per edge broadcast over heads
+                                  (graphormer_dist_node_level.py:384)                     */
+
+typedef struct tgt_plan tgt_plan_t;   /* opaque, owns device memory */
+
+int          tgt_version(void);
+const char*  tgt_error_string(int code);
+const char*  tgt_last_error(void);
+
+/* ---- graph plan ---------------------------------------------------------
+ * Replaces the per-call gathers `k[edge_index[0]]`, `q[edge_index[1]]` and the
+ * atomic scatter-adds `scatter(msg, edge_index[1], ...)` (attn_module.py:146-147,
+ * 180, 185) by two sorted views of the edge list built ONCE per edge_index:
+ *   CSR by destination: rowptr_dst[N+1], col_dst[E] (= source of the edge),
+ *                       eid_dst[E] (= index of the edge in the caller's order)
+ *   CSC by source:      rowptr_src[N+1], col_src[E] (= destination), eid_src[E]
+ * Both orders are the STABLE sort of the caller's edge list (ties keep the
+ * caller's order), i.e. what `argsort(kind='stable')` gives — the same contract
+ * as the reference's edge sort (gt_sp/utils.py:354-356).  On top of that the
+ * plan holds a degree-binned row schedule (long rows split into segments).
+ *
+ * d_src / d_dst: int64 device arrays of length E (edge_index[0], edge_index[1]).
+ * Synchronises `stream`.  TGT_ERR_INDEX_RANGE if any endpoint is outside [0,N).
+ */
+int tgt_plan_create(const int64_t* d_src, const int64_t* d_dst, int64_t E, int64_t N,
+                    void* stream, tgt_plan_t** out_plan);
+int tgt_plan_destroy(tgt_plan_t* plan);
+
+/* info[0]=N, [1]=E, [2]=#schedule items (dst side), [3]=#split rows (dst),
+ * [4]=#partial segments (dst), [5..7]= the same for the src side,
+ * [8]=segment length limit, [9..15] reserved (0). */
+int tgt_plan_info(const tgt_plan_t* plan, int64_t info[16]);
+
+#define TGT_PLAN_ROWPTR_DST 0
+#define TGT_PLAN_COL_DST    1
+#define TGT_PLAN_EID_DST    2
+#define TGT_PLAN_ROWPTR_SRC 3
+#define TGT_PLAN_COL_SRC    4
+#define TGT_PLAN_EID_SRC    5
+#define TGT_PLAN_ITEMS_DST  6   /* int32 x4 per item: row, first edge, length, partial slot (-1 = whole row) */
+#define TGT_PLAN_ITEMS_SRC  7
+/* number of int32 values in array `which` */
+int64_t tgt_plan_array_len(const tgt_plan_t* plan, int which);
+/* copy array `which` to host memory (capacity in int32 elements); synchronous */
+int tgt_plan_export(const tgt_plan_t* plan, int which, int32_t* h_out, int64_t capacity);
+
+/* ---- sparse attention ---------------------------------------------------
+ * Workspace (device memory, 256-byte aligned) needed by fwd/bwd for partial
+ * sums of split rows and per-node side vectors; depends on the plan and H*d. */
+int64_t tgt_sparse_attn_workspace_bytes(const tgt_plan_t* plan, int H, int d);
+
+/* Forward of CoreAttention.sparse_attention (attn_module.py:133-189) /
+ * sparse_attention_bias (models/graphormer_dist_node_level.py:69-127):
+ *   s_e   = clamp(sum_c k[src,h,c] q[dst,h,c] / sqrt(d), -5, 5) + bias_e[h]
+ *   w_e   = exp(s_e)                       (no max subtraction)
+ *   Z_i   = sum_{e: dst=i} w_e ;  out_i = sum_e w_e v[src] / (Z_i + 1e-6)
+ * d_out: [N, H, d] dtype;  d_Z: [N, H] float32 (saved for backward).
+ */
+int tgt_sparse_attn_fwd(const tgt_plan_t* plan,
+                        const void* d_q, const void* d_k, const void* d_v,
+                        const void* d_bias, int bias_mode,
+                        int H, int d, int dtype,
+                        void* d_out, float* d_Z,
+                        void* d_workspace, int64_t workspace_bytes, void* stream);
+
+/* Backward of the same function (autograd in the reference).  d_dout, d_dq,
+ * d_dk, d_dv: [N, H, d] dtype; d_dbias: same shape/dtype as d_bias or NULL.
+ * Every gradient is written exactly once (no atomics, no pre-zeroing needed). */
+int tgt_sparse_attn_bwd(const tgt_plan_t* plan,
+                        const void* d_q, const void* d_k, const void* d_v,
+                        const void* d_bias, int bias_mode,
+                        int H, int d, int dtype,
+                        const void* d_out, const float* d_Z, const void* d_dout,
+                        void* d_dq, void* d_dk, void* d_dv, void* d_dbias,
+                        void* d_workspace, int64_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TORCHGT_HIP_H */

@@ -1,0 +1,33 @@
+"""CPU oracle for the TorchGT sparse-attention hot path.
+
+TEST INFRASTRUCTURE ONLY.  Nothing in the shipped package may import this
+directory: only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline``
+leg of ``bench.py`` use it, and there only as the checker (or as the CPU
+baseline being timed), never as the thing that produces a result.
+
+Every function restates, in plain PyTorch / numpy, the algorithm of a reference
+function and cites the reference file:line it follows.  The reference ships no
+tests, fixtures or golden vectors, and it cannot be imported offline (it imports
+torch_scatter / dgl / torch_geometric at module top), so each function is pinned
+by independent checks in ``tests/test_oracle_*.py``:
+
+=============================  ================================================
+function                       pinned by
+=============================  ================================================
+sparse_attention               dense-softmax equivalence (torch.softmax), fp64
+                               brute-force loops, closed-form special cases,
+                               permutation / relabel invariants
+sparse_attention (gradients)   torch autograd of the restatement; analytic
+                               formulas checked by fp64 gradcheck
+dense_bias_to_edge_bias        brute-force indexing loops
+dense_attention                torch.softmax/matmul library routine with the
+                               q*sqrt(d) quirk; brute-force loops
+fix_edge_index                 hand-computed known answer (N=3)
+relabel_by_partition           hand-computed known answer
+blockize / reformat_graph      hand-computed known answer (k=1, N=32, bs=16)
+                               + structural invariants
+build_csr                      numpy stable argsort + round-trip invariants
+metis partition labels         PARITY UNPINNED: dgl/METIS is absent; partition
+                               ids are always an explicit input here
+=============================  ================================================
+"""

@@ -1,0 +1,76 @@
+"""Oracle: dense biased attention for graph-level batches (test infrastructure).
+
+Restates ``CoreAttention.forward`` of ``models/graphormer_graph_level.py:186-214``
+(same body: ``attn_module.py:99-127``, ``graphormer_dist_graph_level.py:211-235``)
+and the bias producer ``GraphAttnBias.forward``
+(``models/graphormer_graph_level.py:94-156``, edge_type != 'multi_hop' branch).
+"""
+import math
+
+import torch
+
+
+def dense_attention(q, k, v, attn_bias=None, mask=None):
+    """q, k, v: [b, S, H, d]; attn_bias [b, H, S, S] (additive, -inf on padded
+    keys); mask [b, S, S] bool or None.  NOTE the reference MULTIPLIES q by
+    sqrt(d) (graphormer_graph_level.py:198).  Dropout is the identity here
+    (eval / p = 0).  Returns [b, S, H*d]."""
+    b, S, H, d = q.shape
+    scale = math.sqrt(d)
+    qt = q.transpose(1, 2)                      # :192  [b, H, S, d]
+    vt = v.transpose(1, 2)                      # :193
+    kt = k.transpose(1, 2).transpose(2, 3)      # :194  [b, H, d, S]
+    qt = qt * scale                             # :198
+    x = torch.matmul(qt, kt)                    # :199
+    if attn_bias is not None:
+        x = x + attn_bias                       # :202
+    if mask is not None:
+        x = x.masked_fill(mask.unsqueeze(1), 0)  # :204-205
+    x = torch.softmax(x, dim=3)                 # :207
+    x = x.matmul(vt)                            # :209
+    x = x.transpose(1, 2).contiguous()          # :211
+    return x.view(b, S, -1)                     # :212
+
+
+def graph_attn_bias(attn_bias, spatial_pos, attn_edge_type, spatial_table, edge_table, virtual_dist):
+    """``GraphAttnBias.forward`` (graphormer_graph_level.py:94-156), simple
+    edge-type branch (:150).
+
+    attn_bias       [b, S+1, S+1] float (0 / -inf from the collator)
+    spatial_pos     [b, S, S] int64   (shortest-path distance + 1, 0 = pad)
+    attn_edge_type  [b, S, S, F] int64 (edge feature ids + 1, 0 = none)
+    spatial_table   [num_spatial, H]  (row 0 = padding_idx, zeros)
+    edge_table      [num_edges, H]    (row 0 = padding_idx, zeros)
+    virtual_dist    [1, H]
+    Returns [b, H, S+1, S+1].
+    """
+    H = spatial_table.shape[1]
+    g = attn_bias.clone().unsqueeze(1).repeat(1, H, 1, 1)             # :104-107
+    sp = spatial_table[spatial_pos].permute(0, 3, 1, 2)               # :110
+    g[:, :, 1:, 1:] = g[:, :, 1:, 1:] + sp                            # :111
+    t = virtual_dist.view(1, H, 1)                                    # :115
+    g[:, :, 1:, 0] = g[:, :, 1:, 0] + t                               # :116
+    g[:, :, 0, :] = g[:, :, 0, :] + t                                 # :117
+    ei = edge_table[attn_edge_type].mean(-2).permute(0, 3, 1, 2)      # :150
+    g[:, :, 1:, 1:] = g[:, :, 1:, 1:] + ei                            # :152
+    g = g + attn_bias.unsqueeze(1)                                    # :153
+    return g
+
+
+def dense_attention_bruteforce(q, k, v, attn_bias=None):
+    """fp64 loops from the definition; pins ``dense_attention`` on tiny inputs."""
+    b, S, H, d = q.shape
+    q, k, v = q.double(), k.double(), v.double()
+    out = torch.zeros(b, S, H * d, dtype=torch.float64)
+    for g in range(b):
+        for h in range(H):
+            for i in range(S):
+                sc = torch.empty(S, dtype=torch.float64)
+                for j in range(S):
+                    sc[j] = (q[g, i, h] * math.sqrt(d) * k[g, j, h]).sum()
+                    if attn_bias is not None:
+                        sc[j] = sc[j] + float(attn_bias[g, h, i, j])
+                m = sc.max()
+                w = torch.exp(sc - m)
+                out[g, i, h * d:(h + 1) * d] = (w.unsqueeze(1) * v[g, :, h]).sum(0) / w.sum()
+    return out

@@ -1,0 +1,146 @@
+"""Oracle: edge construction and ordering (test infrastructure, CPU, numpy).
+
+Restates the integer side of the reference's batch preparation:
+
+* ``fix_edge_index``                 gt_sp/utils.py:34-50
+* ``adjust_edge_index_nomerge``      gt_sp/utils.py:53-58
+* relabel by partition               gt_sp/utils.py:329-335
+* ``generate_new_edges_optimized``   gt_sp/utils.py:223-305   (cluster "blockize")
+* ``reformat_graph`` tail            gt_sp/utils.py:350-359   (sort by source)
+
+``dgl.metis_partition_assignment`` (gt_sp/utils.py:326; dgl-cu111 0.9.1, absent
+here) is NOT restated: partition ids are an explicit argument.  PARITY UNPINNED
+for the METIS labels themselves.
+
+``build_csr`` is the oracle for the plan the HIP library builds (stable
+counting sort of the edge list by destination or by source).
+"""
+import numpy as np
+
+
+def fix_edge_index(x, num_node):
+    """gt_sp/utils.py:34-50.  x: int64 [2, E0].  Real nodes shift by +1, the
+    virtual node is 0; appended: num_node edges (i+1 -> 0), then num_node
+    edges (0 -> i+1).  No self-loop on the virtual node."""
+    x = np.asarray(x, dtype=np.int64)
+    ar = np.arange(num_node, dtype=np.int64) + 1
+    zeros = np.zeros(num_node, dtype=np.int64)
+    to_virtual = np.stack([ar, zeros])
+    from_virtual = np.stack([zeros, ar])
+    return np.concatenate([x + 1, to_virtual, from_virtual], axis=1)
+
+
+def adjust_edge_index_nomerge(edge_index, sub_seq_len):
+    """gt_sp/utils.py:53-58: idx + (idx-1)//L for idx > 0 (float floor-divide
+    in the reference; exact for idx < 2**24).  Identity when every idx <= L."""
+    e = np.asarray(edge_index, dtype=np.int64)
+    out = e.copy()
+    mask = e > 0
+    out[mask] = e[mask] + ((e[mask].astype(np.float32) - 1) // sub_seq_len).astype(np.int64)
+    return out
+
+
+def relabel_by_partition(partition_ids, k):
+    """gt_sp/utils.py:329-335: parts in order 0..k-1, members in ascending old
+    id get consecutive new ids.  Returns new_id_mapping[old] = new."""
+    partition_ids = np.asarray(partition_ids)
+    mapping = np.empty(partition_ids.shape[0], dtype=np.int64)
+    nxt = 0
+    for part in range(k):
+        members = np.nonzero(partition_ids == part)[0]
+        mapping[members] = nxt + np.arange(members.shape[0])
+        nxt += members.shape[0]
+    return mapping
+
+
+def blockize(edge_index, k, partition_ids, p, blocksize, new_id_mapping):
+    """gt_sp/utils.py:223-305.  Returns int64 [2, E'] in emission order.
+
+    Faithful to the reference including its quirk: per-(part_src, part_dst)
+    edge counts are stored COMPACTLY in order of the non-empty pairs
+    (:237-245) but read back as [i*k+j] (:270), so they are misaligned when a
+    pair is empty.
+    """
+    src = np.asarray(edge_index[0], dtype=np.int64)
+    dst = np.asarray(edge_index[1], dtype=np.int64)
+    part = np.asarray(partition_ids, dtype=np.int64)
+    ps, pd = part[src], part[dst]
+    # :230-235  sorted by ((part_src, part_dst), (src, dst))
+    order = np.lexsort((dst, src, pd, ps))
+    s_ps, s_pd, s_src, s_dst = ps[order], pd[order], src[order], dst[order]
+    E = src.shape[0]
+    # :237-245  run lengths of equal (part_src, part_dst), stored compactly
+    counts = np.zeros(k * k, dtype=np.int64)
+    if E > 0:
+        change = np.nonzero((s_ps[1:] != s_ps[:-1]) | (s_pd[1:] != s_pd[:-1]))[0] + 1
+        bounds = np.concatenate([[0], change, [E]])
+        runs = np.diff(bounds)
+        counts[: runs.shape[0]] = runs
+    cum = np.concatenate([[0], np.cumsum(counts)])                # :246
+    node_counts = np.bincount(part, minlength=k).astype(np.int64)  # :257-260
+    offsets = np.concatenate([[0], np.cumsum(node_counts)[:-1]]).astype(np.int64)  # :262-263
+    out_src, out_dst = [], []
+    keep_cnt = 0
+    per_block = blocksize * blocksize
+    for i in range(k):
+        for j in range(k):
+            total = node_counts[i] * node_counts[j]
+            with np.errstate(divide="ignore", invalid="ignore"):
+                sparsity = counts[i * k + j] / total               # :270 (float64)
+            if sparsity > p:                                        # :274-279
+                lo, hi = cum[i * k + j], cum[i * k + j + 1]
+                out_src.append(new_id_mapping[s_src[lo:hi]])
+                out_dst.append(new_id_mapping[s_dst[lo:hi]])
+            else:                                                   # :284-299
+                nblk = int(sparsity * total / per_block) + 1
+                rng = np.random.RandomState(keep_cnt)               # == np.random.seed(keep_cnt)
+                if node_counts[i] >= blocksize and node_counts[j] >= blocksize:
+                    for _ in range(nblk):
+                        br = rng.randint(0, node_counts[i] // blocksize)
+                        bc = rng.randint(0, node_counts[j] // blocksize)
+                        keep_cnt += 1
+                        r0 = br * blocksize + offsets[i]
+                        c0 = bc * blocksize + offsets[j]
+                        a = np.repeat(np.arange(r0, r0 + blocksize), blocksize)   # :218-220 row-major pairs
+                        b = np.tile(np.arange(c0, c0 + blocksize), blocksize)
+                        out_src.append(a)
+                        out_dst.append(b)
+    if not out_src:
+        return np.zeros((2, 0), dtype=np.int64)
+    return np.stack([np.concatenate(out_src), np.concatenate(out_dst)]).astype(np.int64)
+
+
+def reformat_graph(edge_index, partition_ids, k, block_size):
+    """gt_sp/utils.py:319-359 with the METIS call replaced by explicit
+    ``partition_ids``.  p is hard-wired to 1 (:344).  Returns
+    (sorted_edge_index [2,E'], sorted_indices [N]) where sorted_indices is
+    argsort(new_id_mapping) (new -> old) and edges are STABLY sorted by source.
+    """
+    mapping = relabel_by_partition(partition_ids, k)
+    new_edges = blockize(edge_index, k, partition_ids, 1, block_size, mapping)
+    sorted_indices = np.argsort(mapping, kind="stable")           # :352
+    order = np.argsort(new_edges[0], kind="stable")               # :354
+    return new_edges[:, order], sorted_indices
+
+
+def relabel_and_sort(edge_index, partition_ids, k):
+    """Relabel with :329-335 and stably sort by source (:354-356) WITHOUT the
+    blockize replacement (the commented-out alternative at :347)."""
+    mapping = relabel_by_partition(partition_ids, k)
+    e = mapping[np.asarray(edge_index, dtype=np.int64)]
+    order = np.argsort(e[0], kind="stable")
+    return e[:, order], np.argsort(mapping, kind="stable")
+
+
+def build_csr(edge_index, num_nodes, by="dst"):
+    """Stable counting sort of the edges by destination (by='dst', CSR of the
+    in-neighbour lists) or by source (by='src').  Returns int32
+    (rowptr [N+1], col [E], eid [E]) where eid[p] is the original edge id at
+    sorted position p and col[p] is the other endpoint."""
+    e = np.asarray(edge_index, dtype=np.int64)
+    key, other = (e[1], e[0]) if by == "dst" else (e[0], e[1])
+    eid = np.argsort(key, kind="stable")
+    rowptr = np.zeros(num_nodes + 1, dtype=np.int64)
+    np.add.at(rowptr, key + 1, 1)
+    rowptr = np.cumsum(rowptr)
+    return rowptr.astype(np.int32), other[eid].astype(np.int32), eid.astype(np.int32)

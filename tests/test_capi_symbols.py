@@ -1,0 +1,52 @@
+"""The C-ABI library loads without a GPU and exports every symbol that
+include/torchgt_hip.h declares; host-only entry points behave."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "torchgt_hip.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tgt_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_expected_entry_points():
+    names = declared_functions()
+    for must in ("tgt_plan_create", "tgt_plan_destroy", "tgt_sparse_attn_fwd", "tgt_sparse_attn_bwd",
+                 "tgt_sparse_attn_workspace_bytes", "tgt_plan_export"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    from torchgt_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.fail(f"{_lib.LIB_PATH} not built (python -m torchgt_amd.build)")
+    handle = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared_functions():
+        assert hasattr(handle, name), f"{name} declared in torchgt_hip.h but not exported"
+    # the ctypes table covers the same set
+    assert sorted(_lib.SIGNATURES) == declared_functions()
+
+
+def test_host_only_entry_points():
+    from torchgt_amd import _lib
+    L = _lib.lib()
+    assert L.tgt_version() >= 1
+    assert L.tgt_error_string(0) == b"ok"
+    assert b"range" in L.tgt_error_string(_lib.ERR_INDEX_RANGE)
+    # argument validation happens before any GPU call
+    out = ctypes.c_void_p()
+    assert L.tgt_plan_create(None, None, -1, 10, None, ctypes.byref(out)) == _lib.ERR_INVALID_ARG
+    assert L.tgt_plan_create(None, None, 5, 10, None, ctypes.byref(out)) == _lib.ERR_INVALID_ARG
+    assert L.tgt_plan_create(None, None, 0, 0, None, ctypes.byref(out)) == _lib.ERR_INVALID_ARG
+    assert L.tgt_last_error() != b""
+    assert L.tgt_plan_destroy(None) == 0
+    assert L.tgt_sparse_attn_workspace_bytes(None, 8, 8) == -1
+    assert L.tgt_sparse_attn_fwd(None, None, None, None, None, 0, 8, 8, 0, None, None, None, 0, None) \
+        == _lib.ERR_INVALID_ARG

@@ -1,0 +1,117 @@
+"""Pins of the graph-preparation oracle (CPU only): hand-computed known answers
+and structural invariants for fix_edge_index / relabel / blockize / sort / CSR."""
+import numpy as np
+import pytest
+
+from oracle import graph_prep as gp
+
+
+def test_fix_edge_index_known_answer():
+    # N = 3 real nodes, one edge 0 -> 1 (gt_sp/utils.py:34-50 worked by hand)
+    out = gp.fix_edge_index(np.array([[0], [1]]), 3)
+    expect = np.array([[1, 1, 2, 3, 0, 0, 0],
+                       [2, 0, 0, 0, 1, 2, 3]])
+    np.testing.assert_array_equal(out, expect)
+    assert out.dtype == np.int64
+
+
+def test_fix_edge_index_no_self_loop_on_virtual_node():
+    e = gp.fix_edge_index(np.zeros((2, 0), dtype=np.int64), 5)
+    assert e.shape == (2, 10)
+    assert not np.any((e[0] == 0) & (e[1] == 0))
+    np.testing.assert_array_equal(np.bincount(e[1], minlength=6), [5, 1, 1, 1, 1, 1])
+
+
+def test_adjust_edge_index_nomerge_identity_at_p1_and_shift_at_p2():
+    e = np.array([[0, 1, 5, 8], [8, 4, 0, 1]])
+    np.testing.assert_array_equal(gp.adjust_edge_index_nomerge(e, 8), e)       # every idx <= L
+    # L = 4: idx 5..8 belong to the second rank and shift by one slot (its global-token copy)
+    np.testing.assert_array_equal(gp.adjust_edge_index_nomerge(e, 4), [[0, 1, 6, 9], [9, 4, 0, 1]])
+
+
+def test_relabel_known_answer():
+    # parts: node0->1, node1->0, node2->1, node3->0  => part 0 = {1,3} -> ids 0,1 ; part 1 = {0,2} -> 2,3
+    m = gp.relabel_by_partition(np.array([1, 0, 1, 0]), 2)
+    np.testing.assert_array_equal(m, [2, 0, 3, 1])
+
+
+def test_blockize_known_answer_single_partition():
+    # k = 1, N = 32, block 16: 5 edges -> sparsity 5/1024 <= 1 -> int(5/256)+1 = 1 random block,
+    # drawn exactly as the reference does: np.random.seed(0); randint(0, 2); randint(0, 2)
+    N, bs = 32, 16
+    part = np.zeros(N, dtype=np.int64)
+    ei = np.array([[0, 3, 7, 20, 31], [1, 9, 2, 5, 30]])
+    mapping = gp.relabel_by_partition(part, 1)
+    np.testing.assert_array_equal(mapping, np.arange(N))
+    out = gp.blockize(ei, 1, part, 1, bs, mapping)
+    np.random.seed(0)
+    br = np.random.randint(0, N // bs)
+    bc = np.random.randint(0, N // bs)
+    a = np.repeat(np.arange(br * bs, br * bs + bs), bs)
+    b = np.tile(np.arange(bc * bs, bc * bs + bs), bs)
+    np.testing.assert_array_equal(out, np.stack([a, b]))
+    assert out.shape == (2, 256)
+
+
+def test_blockize_counts_and_offsets_two_partitions():
+    # k = 2 with 32 nodes each and every partition pair non-empty (so the compact-count quirk is
+    # inactive): pair (i,j) with c edges emits int(c/256)+1 blocks inside [off_i, off_i+32) x [off_j, off_j+32)
+    rng = np.random.default_rng(0)
+    N, k, bs = 64, 2, 16
+    part = np.repeat([0, 1], 32)
+    counts = {(0, 0): 300, (0, 1): 10, (1, 0): 257, (1, 1): 600}
+    src, dst = [], []
+    for (i, j), c in counts.items():
+        src.append(rng.integers(0, 32, c) + 32 * i)
+        dst.append(rng.integers(0, 32, c) + 32 * j)
+    ei = np.stack([np.concatenate(src), np.concatenate(dst)])
+    mapping = gp.relabel_by_partition(part, k)
+    out = gp.blockize(ei, k, part, 1, bs, mapping)
+    pos = 0
+    for (i, j), c in counts.items():
+        nblk = c // 256 + 1
+        blk = out[:, pos:pos + nblk * 256]
+        assert blk[0].min() >= 32 * i and blk[0].max() < 32 * (i + 1)
+        assert blk[1].min() >= 32 * j and blk[1].max() < 32 * (j + 1)
+        for t in range(nblk):
+            one = blk[:, t * 256:(t + 1) * 256]
+            r0, c0 = one[0, 0], one[1, 0]
+            assert r0 % bs == 0 and c0 % bs == 0
+            np.testing.assert_array_equal(one[0], np.repeat(np.arange(r0, r0 + bs), bs))
+            np.testing.assert_array_equal(one[1], np.tile(np.arange(c0, c0 + bs), bs))
+        pos += nblk * 256
+    assert pos == out.shape[1]
+
+
+def test_reformat_graph_sorted_by_source_stably():
+    rng = np.random.default_rng(1)
+    N, k = 96, 3
+    part = rng.integers(0, k, N)
+    part[:48] = np.repeat([0, 1, 2], 16)           # every part has >= 16 nodes
+    ei = rng.integers(0, N, (2, 400))
+    edges, sorted_indices = gp.reformat_graph(ei, part, k, 16)
+    assert np.all(np.diff(edges[0]) >= 0)
+    mapping = gp.relabel_by_partition(part, k)
+    np.testing.assert_array_equal(mapping[sorted_indices], np.arange(N))   # new -> old inverse
+    raw = gp.blockize(ei, k, part, 1, 16, mapping)
+    # stable: among equal sources the emission order is kept
+    for s in np.unique(raw[0])[:10]:
+        np.testing.assert_array_equal(edges[1][edges[0] == s], raw[1][raw[0] == s])
+
+
+@pytest.mark.parametrize("by", ["dst", "src"])
+def test_build_csr_invariants(by):
+    rng = np.random.default_rng(2)
+    N, E = 50, 600
+    ei = rng.integers(0, N, (2, E))
+    ei[:, :100] = ei[:, 100:200]                    # duplicates
+    rowptr, col, eid = gp.build_csr(ei, N, by)
+    key, other = (ei[1], ei[0]) if by == "dst" else (ei[0], ei[1])
+    assert rowptr[0] == 0 and rowptr[-1] == E and np.all(np.diff(rowptr) >= 0)
+    np.testing.assert_array_equal(np.sort(eid), np.arange(E))
+    np.testing.assert_array_equal(np.diff(rowptr), np.bincount(key, minlength=N))
+    for r in range(N):
+        seg = eid[rowptr[r]:rowptr[r + 1]]
+        assert np.all(key[seg] == r)
+        assert np.all(np.diff(seg) > 0)             # stable: caller's order inside a row
+    np.testing.assert_array_equal(col, other[eid])

@@ -1,0 +1,11 @@
+"""torchgt_amd — MI355X (gfx950) implementation of TorchGT's topology-aware
+sparse attention behind the reference's ``CoreAttention`` module API.
+
+The compute lives in ``libtorchgt_hip.so`` (sources in ``csrc/``, C ABI in
+``include/torchgt_hip.h``); this package is the thin host side.
+"""
+from .core_attention import CoreAttention, SparseAttentionFunction, sparse_attention, gather_dense_bias
+from .plan import GraphPlan, get_plan, clear_plan_cache
+
+__all__ = ["CoreAttention", "SparseAttentionFunction", "sparse_attention", "gather_dense_bias",
+           "GraphPlan", "get_plan", "clear_plan_cache"]

@@ -1,0 +1,69 @@
+"""ctypes binding of libtorchgt_hip.so (the C ABI in include/torchgt_hip.h).
+
+The library is loaded from the package directory.  There is no fallback: if the
+shared object is missing or a call fails, an exception is raised.
+"""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libtorchgt_hip.so")
+
+OK = 0
+ERR_INVALID_ARG, ERR_INDEX_RANGE, ERR_UNSUPPORTED, ERR_HIP, ERR_WORKSPACE = -1, -2, -3, -4, -5
+DTYPE_F32, DTYPE_BF16 = 0, 1
+BIAS_NONE, BIAS_EDGE_HEAD, BIAS_EDGE = 0, 1, 2
+(PLAN_ROWPTR_DST, PLAN_COL_DST, PLAN_EID_DST, PLAN_ROWPTR_SRC, PLAN_COL_SRC, PLAN_EID_SRC,
+ PLAN_ITEMS_DST, PLAN_ITEMS_SRC) = range(8)
+
+_c = ctypes
+_vp, _i64, _i32 = _c.c_void_p, _c.c_int64, _c.c_int
+
+# name -> (restype, argtypes); one entry per declaration in include/torchgt_hip.h
+SIGNATURES = {
+    "tgt_version": (_i32, []),
+    "tgt_error_string": (_c.c_char_p, [_i32]),
+    "tgt_last_error": (_c.c_char_p, []),
+    "tgt_plan_create": (_i32, [_vp, _vp, _i64, _i64, _vp, _c.POINTER(_vp)]),
+    "tgt_plan_destroy": (_i32, [_vp]),
+    "tgt_plan_info": (_i32, [_vp, _c.POINTER(_i64)]),
+    "tgt_plan_array_len": (_i64, [_vp, _i32]),
+    "tgt_plan_export": (_i32, [_vp, _i32, _vp, _i64]),
+    "tgt_sparse_attn_workspace_bytes": (_i64, [_vp, _i32, _i32]),
+    "tgt_sparse_attn_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _i64, _vp]),
+    "tgt_sparse_attn_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp,
+                                   _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
+}
+
+
+class TorchGTHipError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__(f"libtorchgt_hip error {code}: {message}")
+        self.code = code
+
+
+_lib = None
+
+
+def lib():
+    """The loaded library (loads on first use; raises if it is not built)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is not built; run `python -m torchgt_amd.build` "
+                "(there is no fallback implementation)")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(code):
+    if code != OK:
+        l = lib()
+        detail = l.tgt_last_error().decode() or l.tgt_error_string(code).decode()
+        raise TorchGTHipError(code, detail)

@@ -1,0 +1,202 @@
+"""Drop-in ``CoreAttention`` for TorchGT's node-level models, backed by the
+gfx950 library.
+
+Mirrors the reference classes
+  * ``models/graphormer_dist_node_level.py:42-221``  (4-argument constructor,
+    ``sparse_attention_bias(k, q, v, edge_index, attn_bias)``, forward dispatch)
+  * ``models/gt_dist_node_level.py:30-166`` / ``graphormer_dist_graph_level.py``
+    (3-argument constructor)
+  * ``attn_module.py:87-229`` (``(hidden, dropout, heads, device)`` constructor,
+    ``forward(q, k, v, edge_index, flash_attn=False, full=False, mask=None)``)
+with sequence-parallel size 1 (``num_attention_heads_per_partition == num_heads``).
+
+There is no CPU or eager fallback: tensors must live on the GPU and the HIP
+library must be built, otherwise an exception is raised.
+"""
+import math
+
+import torch
+import torch.nn as nn
+
+from . import _lib
+from .plan import GraphPlan, get_plan
+
+_DTYPES = {torch.float32: _lib.DTYPE_F32, torch.bfloat16: _lib.DTYPE_BF16}
+
+
+def _ptr(t):
+    return t.data_ptr() if t is not None else None
+
+
+class SparseAttentionFunction(torch.autograd.Function):
+    """out[N,H,d] = sparse_attention(q, k, v, plan, edge_bias) with the backward
+    kernels of the library (the reference relies on autograd through ATen /
+    torch_scatter ops, attn_module.py:146-187)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, edge_bias, plan):
+        if not (q.is_cuda and k.is_cuda and v.is_cuda):
+            raise RuntimeError("sparse attention needs GPU tensors (no CPU implementation)")
+        if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
+            raise TypeError(f"q/k/v must share dtype float32 or bfloat16, got {q.dtype}/{k.dtype}/{v.dtype}")
+        if q.dim() != 3 or q.shape != k.shape or q.shape != v.shape:
+            raise ValueError("q, k, v must be [N, H, d] with equal shapes")
+        N, H, d = q.shape
+        if N != plan.num_nodes:
+            raise ValueError(f"q has {N} rows but the plan was built for {plan.num_nodes} nodes")
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        mode = _lib.BIAS_NONE
+        if edge_bias is not None:
+            if edge_bias.dtype != q.dtype:
+                edge_bias = edge_bias.to(q.dtype)
+            edge_bias = edge_bias.contiguous()
+            E = plan.num_edges
+            if edge_bias.dim() == 2 and edge_bias.shape == (E, H) and H != 1:
+                mode = _lib.BIAS_EDGE_HEAD
+            elif edge_bias.numel() == E:
+                mode = _lib.BIAS_EDGE
+            else:
+                raise ValueError(f"edge bias must be [E] or [E, H] with E={E}, H={H}; got {tuple(edge_bias.shape)}")
+        out = torch.empty_like(q)
+        Z = torch.empty((N, H), dtype=torch.float32, device=q.device)
+        ws = plan.workspace(H, d)
+        with torch.cuda.device(q.device):
+            stream = torch.cuda.current_stream(q.device).cuda_stream
+            _lib.check(_lib.lib().tgt_sparse_attn_fwd(
+                plan.handle, _ptr(q), _ptr(k), _ptr(v), _ptr(edge_bias), mode, H, d, _DTYPES[q.dtype],
+                _ptr(out), _ptr(Z), _ptr(ws), ws.numel(), stream))
+        ctx.plan = plan
+        ctx.mode = mode
+        ctx.has_bias = edge_bias is not None
+        ctx.save_for_backward(q, k, v, edge_bias, out, Z)
+        ctx.mark_non_differentiable(Z)
+        return out, Z
+
+    @staticmethod
+    def backward(ctx, dout, _dZ):
+        q, k, v, edge_bias, out, Z = ctx.saved_tensors
+        plan = ctx.plan
+        N, H, d = q.shape
+        dout = dout.contiguous()
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        dbias = None
+        if ctx.has_bias and ctx.needs_input_grad[3]:
+            dbias = torch.empty_like(edge_bias)
+        ws = plan.workspace(H, d)
+        with torch.cuda.device(q.device):
+            stream = torch.cuda.current_stream(q.device).cuda_stream
+            _lib.check(_lib.lib().tgt_sparse_attn_bwd(
+                plan.handle, _ptr(q), _ptr(k), _ptr(v), _ptr(edge_bias), ctx.mode, H, d, _DTYPES[q.dtype],
+                _ptr(out), _ptr(Z), _ptr(dout), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(dbias),
+                _ptr(ws), ws.numel(), stream))
+        return dq, dk, dv, dbias, None
+
+
+def sparse_attention(q, k, v, edge_index=None, edge_bias=None, plan=None, return_z=False):
+    """Functional form.  q, k, v: [N, H, d] (or [b, S, H, d], flattened over b*S
+    as in attn_module.py:141-143); ``edge_index`` int64 [2, E] (row 0 = source /
+    key node, row 1 = destination / query node) or a prebuilt ``plan``;
+    ``edge_bias``: None, [E] or [E, H] in the order of ``edge_index``."""
+    H, d = q.shape[-2], q.shape[-1]
+    q3, k3, v3 = q.reshape(-1, H, d), k.reshape(-1, H, d), v.reshape(-1, H, d)
+    if plan is None:
+        if edge_index is None:
+            raise ValueError("need edge_index or plan")
+        plan = get_plan(edge_index, q3.shape[0])
+    out, Z = SparseAttentionFunction.apply(q3, k3, v3, edge_bias, plan)
+    return (out, Z) if return_z else out
+
+
+def gather_dense_bias(attn_bias, edge_index, layout):
+    """Per-edge view ``bias[src, dst, :]`` of a dense bias, the indexing of
+    models/graphormer_dist_graph_level.py:262-267.  layout 'bhss' = [b, H, S, S]
+    (graph-level), 'bssh' = [b, S, S, H'] (node-level,
+    graphormer_dist_node_level.py:100-106).  The dense [b*S, b*S, H] tensor the
+    reference builds is never materialised.  Differentiable (torch indexing)."""
+    if layout == "bhss":
+        attn_bias = attn_bias.permute(0, 2, 3, 1)
+    S = attn_bias.shape[1]
+    src, dst = edge_index[0].long(), edge_index[1].long()
+    return attn_bias[src // S, src % S, dst % S, :]
+
+
+class CoreAttention(nn.Module):
+    """Same constructor and call conventions as the reference's ``CoreAttention``
+    classes (see the module docstring for the three flavours)."""
+
+    def __init__(self, hidden_size, attention_dropout_rate, num_heads, *extra, **kw):
+        super().__init__()
+        self.hidden_size_per_partition = hidden_size
+        self.hidden_size_per_attention_head = hidden_size // num_heads
+        self.num_attention_heads_per_partition = num_heads      # sequence-parallel size 1
+        self.scale = math.sqrt(self.hidden_size_per_attention_head)
+        self.num_heads = num_heads
+        self.att_dropout = nn.Dropout(attention_dropout_rate)
+        self.attention_dropout_rate = attention_dropout_rate
+        self.drop_out_rate = attention_dropout_rate
+        # 4th positional argument: attn_bias_dim (node-level Graphormer) or a device (attn_module.py)
+        fourth = extra[0] if extra else kw.get("attn_bias_dim", kw.get("device"))
+        self.attn_bias_dim = fourth if isinstance(fourth, int) else None
+        self.dense_bias_layout = "bssh" if self.attn_bias_dim is not None else "bhss"
+
+    # -- helpers ---------------------------------------------------------
+    def _edge_bias(self, attn_bias, edge_index):
+        if attn_bias is None:
+            return None
+        if attn_bias.dim() <= 2:
+            return attn_bias                       # already per edge: [E], [E, 1] or [E, H]
+        eb = gather_dense_bias(attn_bias, edge_index, self.dense_bias_layout)
+        if eb.shape[-1] == 1:
+            eb = eb.squeeze(-1)
+        return eb
+
+    def _sparse(self, q, k, v, edge_index, attn_bias):
+        H, d = self.num_heads, self.hidden_size_per_attention_head
+        q3 = q.reshape(-1, H, d)
+        k3 = k.reshape(-1, H, d)
+        v3 = v.reshape(-1, H, d)
+        plan = edge_index if isinstance(edge_index, GraphPlan) else get_plan(edge_index, q3.shape[0])
+        eb = self._edge_bias(attn_bias, edge_index)
+        out, _ = SparseAttentionFunction.apply(q3, k3, v3, eb, plan)
+        return out
+
+    # -- reference method names -------------------------------------------
+    def sparse_attention_bias(self, k, q, v, edge_index, attn_bias):
+        """models/graphormer_dist_node_level.py:69-127 — note the (k, q, v) order.
+        Returns [b*S, H, d]."""
+        return self._sparse(q, k, v, edge_index, attn_bias)
+
+    def sparse_attention(self, q, k, v, edge_index, attn_bias=None):
+        """attn_module.py:133-189.  Returns [b, S, H*d]."""
+        b, S = k.size(0), k.size(1)
+        return self._sparse(q, k, v, edge_index, attn_bias).view(b, S, -1)
+
+    def full_attention(self, *args, **kw):
+        raise NotImplementedError(
+            "dense attention (attn_type='full') is served by torchgt_amd.dense_attention; "
+            "it is not wired into this class yet")
+
+    def forward(self, q, k, v, attn_bias=None, edge_index=None, attn_type=None, mask=None,
+                flash_attn=False, full=False):
+        """Node-level convention (graphormer_dist_node_level.py:199-221):
+        ``forward(q, k, v, attn_bias, edge_index, attn_type)`` with q, k, v
+        [b, S, H, d]; returns [b, S, H*d].  The benchmark convention of
+        attn_module.py:221-229, ``forward(q, k, v, edge_index)``, is recognised
+        by an integer [2, E] fourth argument."""
+        if (edge_index is None and isinstance(attn_bias, torch.Tensor) and attn_bias.dim() == 2
+                and attn_bias.size(0) == 2 and not attn_bias.is_floating_point()):
+            edge_index, attn_bias = attn_bias, None
+            if attn_type is None:
+                attn_type = "full" if full else ("flash" if flash_attn else "sparse")
+        b, S = q.size(0), q.size(1)
+        if attn_type == "sparse":
+            x = self._sparse(q, k, v, edge_index, attn_bias)
+        elif attn_type == "full":
+            x = self.full_attention(k, q, v, attn_bias)
+        elif attn_type == "flash":
+            raise NotImplementedError(
+                "attn_type='flash' calls the CUDA-only flash_attn package in the reference "
+                "(graphormer_dist_node_level.py:211-216); it has no counterpart here")
+        else:
+            raise ValueError(f"unknown attn_type {attn_type!r}")
+        return x.view(b, S, -1)

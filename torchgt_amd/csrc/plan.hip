@@ -1,0 +1,464 @@
+// Graph plan: stable CSR-by-destination / CSC-by-source build and the
+// degree-binned row schedule.
+//
+// Replaces, once per edge_index, what the reference redoes on every attention
+// call: the per-edge gathers k[edge_index[0]], q[edge_index[1]] and the atomic
+// scatter-adds over edge_index[1] (attn_module.py:146-147,180,185).  The sorted
+// order is the stable one (ties keep the caller's edge order), the contract of
+// the reference's edge sort (gt_sp/utils.py:354-356).
+//
+// The sort is a hand-written LSD radix sort (8-bit digits) whose ranking is
+// position-based, so the result is bit-reproducible: integer LDS counters only
+// count, they never decide an order.
+#include "common.h"
+#include <vector>
+#include <new>
+
+namespace tgt {
+
+static thread_local char g_err[512] = "";
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+const char* last_error() { return g_err; }
+
+// ---------------------------------------------------------------------------
+// kernels
+// ---------------------------------------------------------------------------
+constexpr int RS_THREADS = 256;
+constexpr int RS_ITEMS = 16;
+constexpr int RS_TILE = RS_THREADS * RS_ITEMS;   // 4096 keys per workgroup
+constexpr int RS_WAVE_SPAN = kWave * RS_ITEMS;   // 1024 consecutive keys per wave
+
+// int64 endpoints -> uint32, with a range check (flag[0] = 1 on a bad index).
+__global__ void k_convert_validate(const int64_t* __restrict__ src, const int64_t* __restrict__ dst,
+                                   int64_t E, int64_t N, uint32_t* __restrict__ s32,
+                                   uint32_t* __restrict__ d32, int* __restrict__ flag) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= E) return;
+    int64_t s = src[i], d = dst[i];
+    bool bad = (s < 0) | (s >= N) | (d < 0) | (d >= N);
+    if (bad) { flag[0] = 1; s = 0; d = 0; }
+    s32[i] = (uint32_t)s;
+    d32[i] = (uint32_t)d;
+}
+
+// Per-workgroup digit histogram, stored digit-major: hist[digit * nblocks + block].
+__global__ __launch_bounds__(RS_THREADS) void k_rs_hist(const uint32_t* __restrict__ keys, int64_t n,
+                                                        int shift, uint32_t* __restrict__ hist,
+                                                        int nblocks) {
+    __shared__ uint32_t h[256];
+    const int tid = threadIdx.x;
+    h[tid] = 0;
+    __syncthreads();
+    const int64_t base = (int64_t)blockIdx.x * RS_TILE;
+#pragma unroll
+    for (int i = 0; i < RS_ITEMS; ++i) {
+        int64_t idx = base + i * RS_THREADS + tid;
+        if (idx < n) atomicAdd(&h[(keys[idx] >> shift) & 255u], 1u);   // integer count: order-free
+    }
+    __syncthreads();
+    hist[(int64_t)tid * nblocks + blockIdx.x] = h[tid];
+}
+
+// Workgroup `digit` turns its row of per-block counts into exclusive offsets and
+// records the row total.
+__global__ __launch_bounds__(256) void k_rs_scan_rows(uint32_t* __restrict__ hist, int nblocks,
+                                                      uint32_t* __restrict__ totals) {
+    __shared__ uint32_t part[256];
+    const int tid = threadIdx.x;
+    uint32_t* row = hist + (int64_t)blockIdx.x * nblocks;
+    const int chunk = (nblocks + 255) / 256;
+    const int b = tid * chunk;
+    const int e = min(b + chunk, nblocks);
+    uint32_t s = 0;
+    for (int i = b; i < e; ++i) s += row[i];
+    part[tid] = s;
+    __syncthreads();
+    for (int off = 1; off < 256; off <<= 1) {
+        uint32_t x = tid >= off ? part[tid - off] : 0u;
+        __syncthreads();
+        part[tid] += x;
+        __syncthreads();
+    }
+    uint32_t run = tid ? part[tid - 1] : 0u;
+    for (int i = b; i < e; ++i) {
+        uint32_t x = row[i];
+        row[i] = run;
+        run += x;
+    }
+    if (tid == 255) totals[blockIdx.x] = part[255];
+}
+
+// Stable scatter of one radix pass.  Each wave owns 1024 consecutive keys of the
+// tile and ranks them in 16 rounds of 64; the rank of a key among equal digits is
+// (count in earlier rounds) + (number of lower lanes with the same digit).
+__global__ __launch_bounds__(RS_THREADS) void k_rs_scatter(
+    const uint32_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in,
+    uint32_t* __restrict__ keys_out, uint32_t* __restrict__ vals_out, int64_t n, int shift,
+    const uint32_t* __restrict__ hist, const uint32_t* __restrict__ totals, int nblocks) {
+    __shared__ uint32_t cnt[4][256];
+    __shared__ uint32_t base[256];
+    __shared__ uint32_t scan[256];
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    for (int i = tid; i < 4 * 256; i += RS_THREADS) (&cnt[0][0])[i] = 0;
+    scan[tid] = totals[tid];
+    __syncthreads();
+
+    volatile uint32_t* wcnt = &cnt[wave][0];
+    uint32_t key[RS_ITEMS], rank[RS_ITEMS];
+    const int64_t wbase = (int64_t)blockIdx.x * RS_TILE + (int64_t)wave * RS_WAVE_SPAN;
+    const uint64_t lower_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+#pragma unroll
+    for (int r = 0; r < RS_ITEMS; ++r) {
+        const int64_t idx = wbase + r * kWave + lane;
+        const bool valid = idx < n;
+        const uint32_t kk = valid ? keys_in[idx] : 0u;
+        key[r] = kk;
+        const uint32_t dg = (kk >> shift) & 255u;
+        uint64_t same = __ballot(valid);
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            const bool bit = (dg >> b) & 1u;
+            const uint64_t bal = __ballot(bit);
+            same &= bit ? bal : ~bal;
+        }
+        uint32_t prior = 0;
+        if (valid) prior = wcnt[dg];
+        const uint32_t lower = (uint32_t)__popcll(same & lower_mask);
+        rank[r] = prior + lower;
+        if (valid && lower == 0) wcnt[dg] = prior + (uint32_t)__popcll(same);
+    }
+    __syncthreads();
+    // exclusive prefix over the 4 waves (thread = digit) and over the 256 digit totals
+    {
+        uint32_t c0 = cnt[0][tid], c1 = cnt[1][tid], c2 = cnt[2][tid];
+        cnt[0][tid] = 0;
+        cnt[1][tid] = c0;
+        cnt[2][tid] = c0 + c1;
+        cnt[3][tid] = c0 + c1 + c2;
+    }
+    for (int off = 1; off < 256; off <<= 1) {
+        uint32_t x = tid >= off ? scan[tid - off] : 0u;
+        __syncthreads();
+        scan[tid] += x;
+        __syncthreads();
+    }
+    base[tid] = (tid ? scan[tid - 1] : 0u) + hist[(int64_t)tid * nblocks + blockIdx.x];
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < RS_ITEMS; ++r) {
+        const int64_t idx = wbase + r * kWave + lane;
+        if (idx < n) {
+            const uint32_t dg = (key[r] >> shift) & 255u;
+            const uint32_t pos = base[dg] + cnt[wave][dg] + rank[r];
+            keys_out[pos] = key[r];
+            vals_out[pos] = vals_in ? vals_in[idx] : (uint32_t)idx;
+        }
+    }
+}
+
+// rowptr[r] = first sorted position whose key is >= r.
+__global__ void k_fill_rowptr(const uint32_t* __restrict__ keys, int64_t E, int64_t N,
+                              int32_t* __restrict__ rowptr) {
+    int64_t pos = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (pos > E) return;
+    int64_t prev = pos == 0 ? -1 : (int64_t)keys[pos - 1];
+    int64_t cur = pos == E ? N : (int64_t)keys[pos];
+    for (int64_t r = prev + 1; r <= cur; ++r) rowptr[r] = (int32_t)pos;
+}
+
+__global__ void k_gather_col(const uint32_t* __restrict__ eid, const uint32_t* __restrict__ other,
+                             int64_t E, int32_t* __restrict__ col, int32_t* __restrict__ eid_out) {
+    int64_t pos = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (pos >= E) return;
+    uint32_t e = eid[pos];
+    col[pos] = (int32_t)other[e];
+    eid_out[pos] = (int32_t)e;
+}
+
+// ---------------------------------------------------------------------------
+// host helpers
+// ---------------------------------------------------------------------------
+struct DevBuf {
+    void* p = nullptr;
+    ~DevBuf() { if (p) (void)hipFree(p); }
+    hipError_t alloc(size_t bytes) { return hipMalloc(&p, bytes ? bytes : 4); }
+    template <typename T> T* as() { return (T*)p; }
+};
+
+static int radix_passes(int64_t N) {
+    int bits = 1;
+    while (bits < 32 && ((int64_t)1 << bits) < N) ++bits;
+    return (bits + 7) / 8;
+}
+
+struct SortScratch {
+    DevBuf keysA, keysB, valsA, valsB, hist, totals;
+    int nblocks = 0;
+};
+
+// Sort edge ids by `keys32` (stable) and fill one Side's rowptr / col / eid.
+static int build_side(const uint32_t* keys32, const uint32_t* other32, int64_t E, int64_t N,
+                      SortScratch& sc, Side& side, hipStream_t st) {
+    const int passes = radix_passes(N);
+    const uint32_t* kin = keys32;
+    const uint32_t* vin = nullptr;
+    uint32_t* kout = sc.keysA.as<uint32_t>();
+    uint32_t* vout = sc.valsA.as<uint32_t>();
+    if (E > 0) {
+        for (int p = 0; p < passes; ++p) {
+            const int shift = 8 * p;
+            hipLaunchKernelGGL(k_rs_hist, dim3(sc.nblocks), dim3(RS_THREADS), 0, st, kin, E, shift,
+                               sc.hist.as<uint32_t>(), sc.nblocks);
+            hipLaunchKernelGGL(k_rs_scan_rows, dim3(256), dim3(256), 0, st, sc.hist.as<uint32_t>(),
+                               sc.nblocks, sc.totals.as<uint32_t>());
+            hipLaunchKernelGGL(k_rs_scatter, dim3(sc.nblocks), dim3(RS_THREADS), 0, st, kin, vin, kout,
+                               vout, E, shift, sc.hist.as<uint32_t>(), sc.totals.as<uint32_t>(),
+                               sc.nblocks);
+            kin = kout;
+            vin = vout;
+            const bool toB = (kout == sc.keysA.as<uint32_t>());
+            kout = toB ? sc.keysB.as<uint32_t>() : sc.keysA.as<uint32_t>();
+            vout = toB ? sc.valsB.as<uint32_t>() : sc.valsA.as<uint32_t>();
+        }
+    }
+    const int T = 256;
+    hipLaunchKernelGGL(k_fill_rowptr, dim3((unsigned)((E + 1 + T - 1) / T)), dim3(T), 0, st, kin, E, N,
+                       side.rowptr);
+    if (E > 0)
+        hipLaunchKernelGGL(k_gather_col, dim3((unsigned)((E + T - 1) / T)), dim3(T), 0, st, vin, other32,
+                           E, side.col, side.eid);
+    TGT_HIP_CHECK(hipGetLastError());
+    return TGT_OK;
+}
+
+static int length_class(int len) {
+    if (len > 32) return 0;
+    if (len > 16) return 1;
+    if (len > 8) return 2;
+    if (len > 4) return 3;
+    return 4;
+}
+
+// Row schedule from a host copy of rowptr: every row becomes one item, a row
+// longer than kSegLen becomes ceil(len/kSegLen) balanced segments.  Items are
+// grouped by length class (longest first) and keep row order inside a class, so
+// waves see uniform lengths and neighbouring rows stay together.
+static int build_schedule(const std::vector<int32_t>& rowptr, int64_t N, Side& side, hipStream_t st) {
+    std::vector<Item> cls[kNumClass];
+    std::vector<int32_t> split_row, split_off;
+    int32_t n_parts = 0;
+    for (int64_t r = 0; r < N; ++r) {
+        const int32_t b = rowptr[r], len = rowptr[r + 1] - b;
+        if (len <= kSegLen) {
+            cls[length_class(len)].push_back(Item{(int32_t)r, b, len, -1});
+        } else {
+            const int nseg = (len + kSegLen - 1) / kSegLen;
+            const int seg = (len + nseg - 1) / nseg;
+            split_row.push_back((int32_t)r);
+            split_off.push_back(n_parts);
+            for (int s = 0; s < nseg; ++s) {
+                const int o = s * seg;
+                const int l = (o + seg <= len) ? seg : (len - o);
+                cls[length_class(l)].push_back(Item{(int32_t)r, b + o, l, n_parts++});
+            }
+        }
+    }
+    split_off.push_back(n_parts);
+    std::vector<Item> items;
+    items.reserve((size_t)N + n_parts);
+    for (int c = 0; c < kNumClass; ++c) {
+        side.class_off[c] = (int32_t)items.size();
+        items.insert(items.end(), cls[c].begin(), cls[c].end());
+    }
+    side.class_off[kNumClass] = (int32_t)items.size();
+    side.n_items = (int32_t)items.size();
+    side.n_split = (int32_t)split_row.size();
+    side.n_parts = n_parts;
+    TGT_HIP_CHECK(hipMalloc((void**)&side.items, sizeof(Item) * (items.size() + 1)));
+    TGT_HIP_CHECK(hipMalloc((void**)&side.split_row, sizeof(int32_t) * (split_row.size() + 1)));
+    TGT_HIP_CHECK(hipMalloc((void**)&side.split_off, sizeof(int32_t) * split_off.size()));
+    TGT_HIP_CHECK(hipMemcpyAsync(side.items, items.data(), sizeof(Item) * items.size(),
+                                 hipMemcpyHostToDevice, st));
+    if (!split_row.empty())
+        TGT_HIP_CHECK(hipMemcpyAsync(side.split_row, split_row.data(), sizeof(int32_t) * split_row.size(),
+                                     hipMemcpyHostToDevice, st));
+    TGT_HIP_CHECK(hipMemcpyAsync(side.split_off, split_off.data(), sizeof(int32_t) * split_off.size(),
+                                 hipMemcpyHostToDevice, st));
+    TGT_HIP_CHECK(hipStreamSynchronize(st));   // the host vectors die at return
+    return TGT_OK;
+}
+
+static void free_side(Side& s) {
+    if (s.rowptr) (void)hipFree(s.rowptr);
+    if (s.col) (void)hipFree(s.col);
+    if (s.eid) (void)hipFree(s.eid);
+    if (s.items) (void)hipFree(s.items);
+    if (s.split_row) (void)hipFree(s.split_row);
+    if (s.split_off) (void)hipFree(s.split_off);
+    s = Side();
+}
+
+static int create_impl(const int64_t* d_src, const int64_t* d_dst, int64_t E, int64_t N, hipStream_t st,
+                       tgt_plan* plan) {
+    plan->N = N;
+    plan->E = E;
+    TGT_HIP_CHECK(hipGetDevice(&plan->device));
+    for (Side* s : {&plan->dst, &plan->src}) {
+        TGT_HIP_CHECK(hipMalloc((void**)&s->rowptr, sizeof(int32_t) * (N + 1)));
+        TGT_HIP_CHECK(hipMalloc((void**)&s->col, sizeof(int32_t) * (E ? E : 1)));
+        TGT_HIP_CHECK(hipMalloc((void**)&s->eid, sizeof(int32_t) * (E ? E : 1)));
+    }
+    DevBuf s32, d32, flag;
+    SortScratch sc;
+    sc.nblocks = (int)((E + RS_TILE - 1) / RS_TILE);
+    if (sc.nblocks < 1) sc.nblocks = 1;
+    const size_t eb = sizeof(uint32_t) * (size_t)(E ? E : 1);
+    TGT_HIP_CHECK(s32.alloc(eb));
+    TGT_HIP_CHECK(d32.alloc(eb));
+    TGT_HIP_CHECK(flag.alloc(sizeof(int)));
+    TGT_HIP_CHECK(sc.keysA.alloc(eb));
+    TGT_HIP_CHECK(sc.keysB.alloc(eb));
+    TGT_HIP_CHECK(sc.valsA.alloc(eb));
+    TGT_HIP_CHECK(sc.valsB.alloc(eb));
+    TGT_HIP_CHECK(sc.hist.alloc(sizeof(uint32_t) * 256 * (size_t)sc.nblocks));
+    TGT_HIP_CHECK(sc.totals.alloc(sizeof(uint32_t) * 256));
+    TGT_HIP_CHECK(hipMemsetAsync(flag.p, 0, sizeof(int), st));
+    if (E > 0) {
+        const int T = 256;
+        hipLaunchKernelGGL(k_convert_validate, dim3((unsigned)((E + T - 1) / T)), dim3(T), 0, st, d_src,
+                           d_dst, E, N, s32.as<uint32_t>(), d32.as<uint32_t>(), flag.as<int>());
+        TGT_HIP_CHECK(hipGetLastError());
+    }
+    int h_flag = 0;
+    TGT_HIP_CHECK(hipMemcpyAsync(&h_flag, flag.p, sizeof(int), hipMemcpyDeviceToHost, st));
+    TGT_HIP_CHECK(hipStreamSynchronize(st));
+    if (h_flag) {
+        set_error("edge_index holds a node id outside [0, %lld)", (long long)N);
+        return TGT_ERR_INDEX_RANGE;
+    }
+    int rc = build_side(d32.as<uint32_t>(), s32.as<uint32_t>(), E, N, sc, plan->dst, st);
+    if (rc) return rc;
+    rc = build_side(s32.as<uint32_t>(), d32.as<uint32_t>(), E, N, sc, plan->src, st);
+    if (rc) return rc;
+    std::vector<int32_t> rp_dst((size_t)N + 1), rp_src((size_t)N + 1);
+    TGT_HIP_CHECK(hipMemcpyAsync(rp_dst.data(), plan->dst.rowptr, sizeof(int32_t) * (N + 1),
+                                 hipMemcpyDeviceToHost, st));
+    TGT_HIP_CHECK(hipMemcpyAsync(rp_src.data(), plan->src.rowptr, sizeof(int32_t) * (N + 1),
+                                 hipMemcpyDeviceToHost, st));
+    TGT_HIP_CHECK(hipStreamSynchronize(st));
+    rc = build_schedule(rp_dst, N, plan->dst, st);
+    if (rc) return rc;
+    return build_schedule(rp_src, N, plan->src, st);
+}
+
+}  // namespace tgt
+
+// ---------------------------------------------------------------------------
+// C ABI
+// ---------------------------------------------------------------------------
+extern "C" {
+
+int tgt_version(void) { return 1; }
+
+const char* tgt_error_string(int code) {
+    switch (code) {
+        case TGT_OK: return "ok";
+        case TGT_ERR_INVALID_ARG: return "invalid argument";
+        case TGT_ERR_INDEX_RANGE: return "edge endpoint out of range";
+        case TGT_ERR_UNSUPPORTED: return "unsupported (H, d, dtype) combination";
+        case TGT_ERR_HIP: return "HIP runtime error";
+        case TGT_ERR_WORKSPACE: return "workspace too small or misaligned";
+        default: return "unknown error";
+    }
+}
+
+const char* tgt_last_error(void) { return tgt::last_error(); }
+
+int tgt_plan_create(const int64_t* d_src, const int64_t* d_dst, int64_t E, int64_t N, void* stream,
+                    tgt_plan_t** out_plan) {
+    if (!out_plan || E < 0 || N < 1 || (E > 0 && (!d_src || !d_dst))) {
+        tgt::set_error("tgt_plan_create: null pointer, E < 0 or N < 1");
+        return TGT_ERR_INVALID_ARG;
+    }
+    if (E > 0x7fff0000LL || N > 0x7fff0000LL) {
+        tgt::set_error("tgt_plan_create: E and N must fit 31 bits");
+        return TGT_ERR_INVALID_ARG;
+    }
+    tgt_plan* plan = new (std::nothrow) tgt_plan();
+    if (!plan) return TGT_ERR_INVALID_ARG;
+    int rc = tgt::create_impl(d_src, d_dst, E, N, (hipStream_t)stream, plan);
+    if (rc != TGT_OK) {
+        tgt::free_side(plan->dst);
+        tgt::free_side(plan->src);
+        delete plan;
+        return rc;
+    }
+    *out_plan = plan;
+    return TGT_OK;
+}
+
+int tgt_plan_destroy(tgt_plan_t* plan) {
+    if (!plan) return TGT_OK;
+    tgt::free_side(plan->dst);
+    tgt::free_side(plan->src);
+    delete plan;
+    return TGT_OK;
+}
+
+int tgt_plan_info(const tgt_plan_t* plan, int64_t info[16]) {
+    if (!plan || !info) return TGT_ERR_INVALID_ARG;
+    for (int i = 0; i < 16; ++i) info[i] = 0;
+    info[0] = plan->N;
+    info[1] = plan->E;
+    info[2] = plan->dst.n_items;
+    info[3] = plan->dst.n_split;
+    info[4] = plan->dst.n_parts;
+    info[5] = plan->src.n_items;
+    info[6] = plan->src.n_split;
+    info[7] = plan->src.n_parts;
+    info[8] = tgt::kSegLen;
+    return TGT_OK;
+}
+
+int64_t tgt_plan_array_len(const tgt_plan_t* plan, int which) {
+    if (!plan) return -1;
+    switch (which) {
+        case TGT_PLAN_ROWPTR_DST: case TGT_PLAN_ROWPTR_SRC: return plan->N + 1;
+        case TGT_PLAN_COL_DST: case TGT_PLAN_EID_DST:
+        case TGT_PLAN_COL_SRC: case TGT_PLAN_EID_SRC: return plan->E;
+        case TGT_PLAN_ITEMS_DST: return 4 * (int64_t)plan->dst.n_items;
+        case TGT_PLAN_ITEMS_SRC: return 4 * (int64_t)plan->src.n_items;
+        default: return -1;
+    }
+}
+
+int tgt_plan_export(const tgt_plan_t* plan, int which, int32_t* h_out, int64_t capacity) {
+    const int64_t n = tgt_plan_array_len(plan, which);
+    if (n < 0 || !h_out || capacity < n) {
+        tgt::set_error("tgt_plan_export: bad array id or capacity");
+        return TGT_ERR_INVALID_ARG;
+    }
+    const void* p = nullptr;
+    switch (which) {
+        case TGT_PLAN_ROWPTR_DST: p = plan->dst.rowptr; break;
+        case TGT_PLAN_COL_DST: p = plan->dst.col; break;
+        case TGT_PLAN_EID_DST: p = plan->dst.eid; break;
+        case TGT_PLAN_ROWPTR_SRC: p = plan->src.rowptr; break;
+        case TGT_PLAN_COL_SRC: p = plan->src.col; break;
+        case TGT_PLAN_EID_SRC: p = plan->src.eid; break;
+        case TGT_PLAN_ITEMS_DST: p = plan->dst.items; break;
+        case TGT_PLAN_ITEMS_SRC: p = plan->src.items; break;
+    }
+    if (n == 0) return TGT_OK;
+    TGT_HIP_CHECK(hipMemcpy(h_out, p, sizeof(int32_t) * n, hipMemcpyDeviceToHost));
+    return TGT_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,113 @@
+"""Graph plan: Python handle on ``tgt_plan_t`` (include/torchgt_hip.h).
+
+The reference re-gathers ``k[edge_index[0]]`` / ``q[edge_index[1]]`` and
+scatter-adds over ``edge_index[1]`` on every attention call of every layer
+(attn_module.py:146-147,180,185) although ``edge_index`` is shared by all layers
+of a step and by all steps of a pre-packed batch
+(main_sp_sparse_node_level.py:155-161).  A plan is the sorted form of one
+``edge_index``; it is built once and reused.
+"""
+import collections
+import ctypes
+
+import numpy as np
+import torch
+
+from . import _lib
+
+
+class GraphPlan:
+    """Stable CSR-by-destination / CSC-by-source views of ``edge_index`` plus the
+    row schedule, resident on the GPU."""
+
+    def __init__(self, edge_index, num_nodes):
+        if not isinstance(edge_index, torch.Tensor) or edge_index.dim() != 2 or edge_index.size(0) != 2:
+            raise ValueError("edge_index must be a [2, E] tensor")
+        if not edge_index.is_cuda:
+            raise RuntimeError("GraphPlan needs edge_index on the GPU (there is no CPU implementation)")
+        ei = edge_index.to(torch.int64).contiguous()
+        self.num_nodes = int(num_nodes)
+        self.num_edges = int(ei.size(1))
+        self.device = ei.device
+        self._handle = ctypes.c_void_p()
+        self._workspaces = {}
+        L = _lib.lib()
+        with torch.cuda.device(self.device):
+            stream = torch.cuda.current_stream(self.device).cuda_stream
+            src_ptr = ei[0].data_ptr() if self.num_edges else None
+            dst_ptr = ei[1].data_ptr() if self.num_edges else None
+            _lib.check(L.tgt_plan_create(src_ptr, dst_ptr, self.num_edges, self.num_nodes, stream,
+                                         ctypes.byref(self._handle)))
+
+    @property
+    def handle(self):
+        if not self._handle:
+            raise RuntimeError("plan was destroyed")
+        return self._handle
+
+    def close(self):
+        if getattr(self, "_handle", None):
+            _lib.lib().tgt_plan_destroy(self._handle)
+            self._handle = ctypes.c_void_p()
+            self._workspaces = {}
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def info(self):
+        arr = (ctypes.c_int64 * 16)()
+        _lib.check(_lib.lib().tgt_plan_info(self.handle, arr))
+        keys = ["N", "E", "items_dst", "split_rows_dst", "segments_dst", "items_src", "split_rows_src",
+                "segments_src", "segment_len"]
+        return {k: int(arr[i]) for i, k in enumerate(keys)}
+
+    def export(self, which):
+        """Copy one plan array to host as int32 numpy (tests compare it with the oracle)."""
+        L = _lib.lib()
+        n = L.tgt_plan_array_len(self.handle, which)
+        if n < 0:
+            raise ValueError(f"bad plan array id {which}")
+        out = np.empty(n, dtype=np.int32)
+        _lib.check(L.tgt_plan_export(self.handle, which, out.ctypes.data_as(ctypes.c_void_p), n))
+        return out
+
+    def workspace(self, H, d):
+        """Device scratch for the attention calls on this plan (cached per (H, d)).
+        Calls that share it must be ordered on one stream."""
+        key = (H, d)
+        ws = self._workspaces.get(key)
+        if ws is None:
+            nbytes = _lib.lib().tgt_sparse_attn_workspace_bytes(self.handle, H, d)
+            if nbytes < 0:
+                raise ValueError("bad H / d")
+            ws = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=self.device)
+            self._workspaces[key] = ws
+        return ws
+
+
+_CACHE = collections.OrderedDict()
+_CACHE_SIZE = 16
+
+
+def get_plan(edge_index, num_nodes):
+    """Plan for ``edge_index``, cached on (storage address, shape, version, N) so
+    that the layers of a model and the iterations over a pre-packed batch share
+    one plan.  The cache keeps the tensor alive, so the address cannot be reused."""
+    key = (edge_index.data_ptr(), tuple(edge_index.shape), edge_index._version, edge_index.dtype,
+           str(edge_index.device), int(num_nodes))
+    hit = _CACHE.get(key)
+    if hit is not None:
+        _CACHE.move_to_end(key)
+        return hit[0]
+    plan = GraphPlan(edge_index, num_nodes)
+    _CACHE[key] = (plan, edge_index)
+    while len(_CACHE) > _CACHE_SIZE:
+        _CACHE.popitem(last=False)
+    return plan
+
+
+def clear_plan_cache():
+    _CACHE.clear()
