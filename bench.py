@@ -1,0 +1,208 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse-attention hot path on one MI355X.
+
+A step is one forward + backward of one layer's sparse attention (the C-ABI calls
+tgt_sparse_attn_fwd + tgt_sparse_attn_bwd) on the 64 K-node power-law graph of
+BASELINE.json configs[1]: N = 64 001, E ~ 530 K, H = 8, d = 8, per-edge bias
+[E, 8] with gradient, inputs resident in HBM, plan prebuilt (its build time is
+reported separately).  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype f32|bf16]
+                    [--workload config2|config1] [--no-cpu-baseline]
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0     # MI355X HBM3E, published
+
+
+def alg_bytes(N, E, H, d, esize, bias_bytes_per_edge, bias_grad):
+    """Compulsory bytes of one fwd+bwd (every operand once per pass, gathers cache-served),
+    and the share of each pass.  R = H*d*esize."""
+    R = H * d * esize
+    fwd = 3 * N * R + N * R + 4 * N * H + 4 * (N + 1) + 4 * E + E * bias_bytes_per_edge
+    bwd = (5 * N * R + 3 * N * R + 4 * N * H + 2 * (4 * (N + 1) + 4 * E) + 4 * E
+           + E * bias_bytes_per_edge * (2 if bias_grad else 1))
+    return fwd, bwd
+
+
+def kernel_alg_bytes(name, N, E, H, d, esize, bpe):
+    """Compulsory bytes of ONE launch of a named kernel (what it must read and write once)."""
+    R = H * d * esize
+    csr = 4 * (N + 1) + 4 * E + 4 * E      # rowptr, col, edge ids (bias is addressed through them)
+    table = {
+        # q,k,v in, out + Z out, one sorted view, bias
+        "attn_fwd": 3 * N * R + N * R + 4 * N * H + csr + E * bpe,
+        "bwd_node_side": 2 * N * R + 4 * N * H + 8 * N * H,
+        # q,k,v,dout + nd in, dq,dk,dv out, both sorted views, bias in (once), dbias out
+        "attn_bwd": 4 * N * R + 8 * N * H + 3 * N * R + 2 * csr + 2 * E * bpe,
+    }
+    return table.get(name)
+
+
+def build_workload(name):
+    import numpy as np
+    from torchgt_amd import workloads
+    if name == "config2":
+        e, n = workloads.power_law_graph(n=64000, exponent=2.1, directed_edges=530_000, seed=42)
+        label = "configs[1]: power-law (exp 2.1) 64000 nodes + 1 global node"
+    elif name == "config1":
+        e, n = workloads.barabasi_albert(n=4096, m=4, seed=42)
+        label = "configs[0]: Barabasi-Albert 4096 nodes m=4 + 1 global node"
+    else:
+        raise SystemExit(f"unknown workload {name}")
+    return e, n, label, workloads.describe(e, n)
+
+
+def cpu_baseline(e, n, H, d, seconds_budget=25.0):
+    """The oracle (op-for-op restatement of the reference's PyTorch path, fp32,
+    autograd backward) timed on this host's cores with the same seeded inputs."""
+    import torch
+    from oracle import sparse_attention as osa
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    g = torch.Generator().manual_seed(42)
+    ei = torch.from_numpy(e)
+    E = e.shape[1]
+    q, k, v = (torch.randn(n, H, d, generator=g).requires_grad_(True) for _ in range(3))
+    bias = (torch.randn(E, H, generator=g) * 0.02).requires_grad_(True)
+    dout = torch.randn(n, H, d, generator=g)
+
+    def step():
+        out, _ = osa.sparse_attention(q, k, v, ei, bias)
+        torch.autograd.grad(out, (q, k, v, bias), dout)
+
+    times = []
+    t_start = time.perf_counter()
+    step()                                       # warm-up
+    while len(times) < 10 and (time.perf_counter() - t_start) < seconds_budget:
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+    med = statistics.median(times)
+    return {"value": E / med, "unit": "edges/s", "cores": cores, "kind": "port",
+            "sample": f"full workload (E={E}), fp32, {len(times)} fwd+bwd iterations after 1 warm-up, median",
+            "ms_per_step": med * 1e3}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--dtype", default="f32", choices=["f32", "bf16"])
+    ap.add_argument("--workload", default="config2")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py: this build runs on ONE GPU (sequence-parallel size 1); "
+                         "--gpus N with N > 1 is not supported")
+
+    import torch
+    from torchgt_amd import _lib
+    from torchgt_amd.plan import GraphPlan
+
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU")
+    dev = torch.device("cuda:0")
+    H, d = 8, 8
+    tdt = torch.float32 if args.dtype == "f32" else torch.bfloat16
+    esize = 4 if args.dtype == "f32" else 2
+    e, n, label, desc = build_workload(args.workload)
+    E = e.shape[1]
+
+    ei = torch.from_numpy(e).to(dev)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    plan = GraphPlan(ei, n)
+    torch.cuda.synchronize()
+    plan_first_ms = (time.perf_counter() - t0) * 1e3
+    t0 = time.perf_counter()
+    plan2 = GraphPlan(ei, n)
+    torch.cuda.synchronize()
+    plan_ms = (time.perf_counter() - t0) * 1e3
+    plan2.close()
+
+    g = torch.Generator().manual_seed(42)
+    q, k, v = (torch.randn(n, H, d, generator=g).to(dev, tdt) for _ in range(3))
+    bias = (torch.randn(E, H, generator=g) * 0.02).to(dev, tdt)
+    dout = torch.randn(n, H, d, generator=g).to(dev, tdt)
+    out = torch.empty_like(q)
+    Z = torch.empty(n, H, dtype=torch.float32, device=dev)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+    dbias = torch.empty_like(bias)
+    ws = plan.workspace(H, d)
+    L = _lib.lib()
+    dt_code = _lib.DTYPE_F32 if args.dtype == "f32" else _lib.DTYPE_BF16
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    P = lambda t: t.data_ptr()
+
+    def step():
+        _lib.check(L.tgt_sparse_attn_fwd(plan.handle, P(q), P(k), P(v), P(bias), _lib.BIAS_EDGE_HEAD, H, d,
+                                         dt_code, P(out), P(Z), P(ws), ws.numel(), stream))
+        _lib.check(L.tgt_sparse_attn_bwd(plan.handle, P(q), P(k), P(v), P(bias), _lib.BIAS_EDGE_HEAD, H, d,
+                                         dt_code, P(out), P(Z), P(dout), P(dq), P(dk), P(dv), P(dbias),
+                                         P(ws), ws.numel(), stream))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    sec = time.perf_counter() - t0
+    ms_per_step = sec / args.steps * 1e3
+
+    # per-kernel durations: HIP events on the launch stream around every kernel, same K steps
+    L.tgt_timing_reset()
+    L.tgt_timing_enable(1)
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    L.tgt_timing_enable(0)
+    timings = _lib.kernel_timings()
+    kernels = {name: {"avg_us": ms / cnt * 1e3, "launches": cnt} for name, (ms, cnt) in timings.items() if cnt}
+    bpe = H * esize
+    dom = max((kk for kk in kernels if kernel_alg_bytes(kk, n, E, H, d, esize, bpe)),
+              key=lambda kk: kernels[kk]["avg_us"])
+    dom_bytes = kernel_alg_bytes(dom, n, E, H, d, esize, bpe)
+    dom_gbs = dom_bytes / (kernels[dom]["avg_us"] * 1e-6) / 1e9
+    fwd_b, bwd_b = alg_bytes(n, E, H, d, esize, bpe, True)
+    step_gbs = (fwd_b + bwd_b) / (ms_per_step * 1e-3) / 1e9
+
+    result = {
+        "metric": "fwd+bwd sparse-attn edges/sec at 64K nodes; % HBM roofline; ms/layer",
+        "value": E / (ms_per_step * 1e-3),
+        "unit": "edges/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic",
+        "config": {"workload": label, "N": n, "E": E, "H": H, "d": d, "bias": "[E,H] with gradient",
+                   "max_in_degree": desc["max_in_degree"], "edge_index_sha256": desc["sha256"],
+                   "step": "tgt_sparse_attn_fwd + tgt_sparse_attn_bwd (one layer)", "parallelism": "1 GPU, SP=1"},
+        "hbm_roofline_frac_step": step_gbs / HBM_PEAK_GBS,
+        "alg_bytes_step": fwd_b + bwd_b,
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": dom_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": dom_gbs / HBM_PEAK_GBS, "traffic": None, "alg_bytes": dom_bytes,
+                     "avg_us": kernels[dom]["avg_us"]},
+        "kernels": kernels,
+        "plan_build_ms": plan_ms, "plan_build_first_ms": plan_first_ms,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(e, n, H, d)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -70,7 +70,8 @@ int tgt_plan_destroy(tgt_plan_t* plan);
 
 /* info[0]=N, [1]=E, [2]=#schedule items (dst side), [3]=#split rows (dst),
  * [4]=#partial segments (dst), [5..7]= the same for the src side,
- * [8]=segment length limit, [9..15] reserved (0). */
+ * [8]=segment length limit, [9]=longest row one wave walks, [10],[11]=#workgroup
+ * items (dst, src), [12..15] reserved (0). */
 int tgt_plan_info(const tgt_plan_t* plan, int64_t info[16]);
 
 #define TGT_PLAN_ROWPTR_DST 0
@@ -88,7 +89,10 @@ int tgt_plan_export(const tgt_plan_t* plan, int which, int32_t* h_out, int64_t c
 
 /* ---- sparse attention ---------------------------------------------------
  * Workspace (device memory, 256-byte aligned) needed by fwd/bwd for partial
- * sums of split rows and per-node side vectors; depends on the plan and H*d. */
+ * sums of split rows, their arrival counters and per-node side vectors; depends
+ * on the plan and H*d.  The caller ZEROES it once after allocating it; after that
+ * only this library writes it (the counters return to zero at the end of every
+ * call).  Calls that share a workspace must be ordered on one stream. */
 int64_t tgt_sparse_attn_workspace_bytes(const tgt_plan_t* plan, int H, int d);
 
 /* Forward of CoreAttention.sparse_attention (attn_module.py:133-189) /
@@ -115,6 +119,17 @@ int tgt_sparse_attn_bwd(const tgt_plan_t* plan,
                         const void* d_out, const float* d_Z, const void* d_dout,
                         void* d_dq, void* d_dk, void* d_dv, void* d_dbias,
                         void* d_workspace, int64_t workspace_bytes, void* stream);
+
+/* ---- per-kernel timing --------------------------------------------------
+ * The reference times this path with torch.profiler around whole iterations
+ * (attn_module.py:415-438).  When enabled, every kernel the library launches is
+ * bracketed by two hipEvents on the launch stream; tgt_timing_read waits for the
+ * recorded pairs and returns the summed duration and launch count of one kernel
+ * slot (0 <= slot < tgt_timing_slots()).  Off by default. */
+int tgt_timing_enable(int on);
+int tgt_timing_reset(void);
+int tgt_timing_slots(void);
+int tgt_timing_read(int slot, const char** name, double* total_ms, int64_t* launches);
 
 #ifdef __cplusplus
 }

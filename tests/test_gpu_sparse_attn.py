@@ -114,8 +114,8 @@ def test_head_shapes(cuda, H, d):
 
 
 def test_all_length_classes_and_ragged_rows(cuda):
-    # rows of in-degree 0,1,...,70 and a few long ones (300, 1000): every slot width and the split path
-    degs = list(range(0, 71)) + [300, 1000, 0, 0, 257, 256, 255]
+    # rows of in-degree 0..70 (every slot width), 255..1024 (one wave / one workgroup) and 1025, 2500 (split rows)
+    degs = list(range(0, 71)) + [300, 1000, 0, 0, 257, 256, 255, 1024, 1025, 2500]
     N = len(degs)
     rng = np.random.default_rng(5)
     src = np.concatenate([rng.integers(0, N, dg) for dg in degs]).astype(np.int64)

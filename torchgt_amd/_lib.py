@@ -33,7 +33,22 @@ SIGNATURES = {
     "tgt_sparse_attn_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _i64, _vp]),
     "tgt_sparse_attn_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp,
                                    _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
+    "tgt_timing_enable": (_i32, [_i32]),
+    "tgt_timing_reset": (_i32, []),
+    "tgt_timing_slots": (_i32, []),
+    "tgt_timing_read": (_i32, [_i32, _c.POINTER(_c.c_char_p), _c.POINTER(_c.c_double), _c.POINTER(_i64)]),
 }
+
+
+def kernel_timings():
+    """{kernel name: (total ms, launches)} since the last tgt_timing_reset()."""
+    L = lib()
+    out = {}
+    for slot in range(L.tgt_timing_slots()):
+        name, ms, n = _c.c_char_p(), _c.c_double(), _i64()
+        check(L.tgt_timing_read(slot, _c.byref(name), _c.byref(ms), _c.byref(n)))
+        out[name.value.decode()] = (ms.value, n.value)
+    return out
 
 
 class TorchGTHipError(RuntimeError):

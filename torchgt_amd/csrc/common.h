@@ -10,8 +10,9 @@ namespace tgt {
 
 constexpr int kWave = 64;            // CDNA wavefront width
 constexpr int kBlock = 256;          // threads per workgroup of the attention kernels (4 waves)
-constexpr int kSegLen = 256;         // a row longer than this is split into segments of this many edges
-constexpr int kNumClass = 5;         // item length classes: >32, <=32, <=16, <=8, <=4
+constexpr int kWaveRowMax = 256;     // a row of up to this many edges is walked by (part of) one wave
+constexpr int kBlockSeg = 1024;      // longer rows are walked by whole workgroups, in segments of at most this many edges
+constexpr int kNumClass = 5;         // wave item length classes: >32, <=32, <=16, <=8, <=4
 
 void set_error(const char* fmt, ...);
 
@@ -27,8 +28,8 @@ void set_error(const char* fmt, ...);
 
 // One schedule entry: `len` consecutive edges starting at sorted position
 // `start`, all belonging to node `row`.  part < 0: the item covers the whole row
-// and its result is final; part >= 0: the row is split and this item's partial
-// sums go to slot `part` of the workspace.
+// and its result is final; part >= 0: the row is split over several workgroups
+// and this item's partial sums go to slot `part` of the workspace.
 struct Item { int32_t row, start, len, part; };
 
 // One sorted view of the edge list plus its row schedule.
@@ -36,11 +37,30 @@ struct Side {
     int32_t* rowptr = nullptr;   // [N+1]
     int32_t* col = nullptr;      // [E] other endpoint
     int32_t* eid = nullptr;      // [E] caller's edge id
-    Item* items = nullptr;       // [n_items], ordered by length class, longest class first
+    Item* items = nullptr;       // [n_items]: workgroup items first, then wave items by length class (longest first)
     int32_t* split_row = nullptr;   // [n_split] rows that were split
     int32_t* split_off = nullptr;   // [n_split+1] first partial slot of each split row
+    int32_t* part2split = nullptr;  // [n_parts] index into split_row of the row a partial slot belongs to
     int32_t n_items = 0, n_split = 0, n_parts = 0;
-    int32_t class_off[kNumClass + 1] = {0, 0, 0, 0, 0, 0};   // item index where each class begins
+    int32_t n_block_items = 0;      // items [0, n_block_items) are walked by one workgroup each
+    int32_t class_off[kNumClass + 1] = {0, 0, 0, 0, 0, 0};   // item index where each wave class begins
+};
+
+// Kernel names of the optional per-kernel timing (timing.hip).
+enum KernelSlot { KS_FWD = 0, KS_NODE_SIDE, KS_BWD, KS_COUNT };
+
+// Scope guard: records a hipEvent on `st` before and after the launches made in
+// its scope when timing is enabled; does nothing otherwise.
+class KernelTimer {
+public:
+    KernelTimer(int slot, hipStream_t st);
+    ~KernelTimer();
+    KernelTimer(const KernelTimer&) = delete;
+    KernelTimer& operator=(const KernelTimer&) = delete;
+private:
+    int slot_;
+    hipStream_t st_;
+    hipEvent_t start_;
 };
 
 }  // namespace tgt

@@ -246,33 +246,40 @@ static int length_class(int len) {
     return 4;
 }
 
-// Row schedule from a host copy of rowptr: every row becomes one item, a row
-// longer than kSegLen becomes ceil(len/kSegLen) balanced segments.  Items are
-// grouped by length class (longest first) and keep row order inside a class, so
-// waves see uniform lengths and neighbouring rows stay together.
+// Row schedule from a host copy of rowptr.  A row of up to kWaveRowMax edges is
+// one wave item; items are grouped by length class (longest first) and keep row
+// order inside a class, so the lanes of a wave see uniform lengths and
+// neighbouring rows stay together.  A longer row is walked by whole workgroups:
+// ceil(len / kBlockSeg) balanced segments, each a workgroup item; if there is more
+// than one segment their partial sums meet in the workspace.
 static int build_schedule(const std::vector<int32_t>& rowptr, int64_t N, Side& side, hipStream_t st) {
     std::vector<Item> cls[kNumClass];
-    std::vector<int32_t> split_row, split_off;
+    std::vector<Item> items;
+    std::vector<int32_t> split_row, split_off, part2split;
     int32_t n_parts = 0;
     for (int64_t r = 0; r < N; ++r) {
         const int32_t b = rowptr[r], len = rowptr[r + 1] - b;
-        if (len <= kSegLen) {
+        if (len <= kWaveRowMax) {
             cls[length_class(len)].push_back(Item{(int32_t)r, b, len, -1});
-        } else {
-            const int nseg = (len + kSegLen - 1) / kSegLen;
-            const int seg = (len + nseg - 1) / nseg;
-            split_row.push_back((int32_t)r);
-            split_off.push_back(n_parts);
-            for (int s = 0; s < nseg; ++s) {
-                const int o = s * seg;
-                const int l = (o + seg <= len) ? seg : (len - o);
-                cls[length_class(l)].push_back(Item{(int32_t)r, b + o, l, n_parts++});
-            }
+            continue;
         }
+        const int nseg = (len + kBlockSeg - 1) / kBlockSeg;
+        if (nseg == 1) {
+            items.push_back(Item{(int32_t)r, b, len, -1});
+            continue;
+        }
+        const int seg = (len + nseg - 1) / nseg;
+        split_off.push_back(n_parts);
+        for (int s = 0; s < nseg; ++s) {
+            const int o = s * seg;
+            const int l = (o + seg <= len) ? seg : (len - o);
+            part2split.push_back((int32_t)split_row.size());
+            items.push_back(Item{(int32_t)r, b + o, l, n_parts++});
+        }
+        split_row.push_back((int32_t)r);
     }
     split_off.push_back(n_parts);
-    std::vector<Item> items;
-    items.reserve((size_t)N + n_parts);
+    side.n_block_items = (int32_t)items.size();
     for (int c = 0; c < kNumClass; ++c) {
         side.class_off[c] = (int32_t)items.size();
         items.insert(items.end(), cls[c].begin(), cls[c].end());
@@ -284,11 +291,15 @@ static int build_schedule(const std::vector<int32_t>& rowptr, int64_t N, Side& s
     TGT_HIP_CHECK(hipMalloc((void**)&side.items, sizeof(Item) * (items.size() + 1)));
     TGT_HIP_CHECK(hipMalloc((void**)&side.split_row, sizeof(int32_t) * (split_row.size() + 1)));
     TGT_HIP_CHECK(hipMalloc((void**)&side.split_off, sizeof(int32_t) * split_off.size()));
+    TGT_HIP_CHECK(hipMalloc((void**)&side.part2split, sizeof(int32_t) * (part2split.size() + 1)));
     TGT_HIP_CHECK(hipMemcpyAsync(side.items, items.data(), sizeof(Item) * items.size(),
                                  hipMemcpyHostToDevice, st));
-    if (!split_row.empty())
+    if (!split_row.empty()) {
         TGT_HIP_CHECK(hipMemcpyAsync(side.split_row, split_row.data(), sizeof(int32_t) * split_row.size(),
                                      hipMemcpyHostToDevice, st));
+        TGT_HIP_CHECK(hipMemcpyAsync(side.part2split, part2split.data(), sizeof(int32_t) * part2split.size(),
+                                     hipMemcpyHostToDevice, st));
+    }
     TGT_HIP_CHECK(hipMemcpyAsync(side.split_off, split_off.data(), sizeof(int32_t) * split_off.size(),
                                  hipMemcpyHostToDevice, st));
     TGT_HIP_CHECK(hipStreamSynchronize(st));   // the host vectors die at return
@@ -302,6 +313,7 @@ static void free_side(Side& s) {
     if (s.items) (void)hipFree(s.items);
     if (s.split_row) (void)hipFree(s.split_row);
     if (s.split_off) (void)hipFree(s.split_off);
+    if (s.part2split) (void)hipFree(s.part2split);
     s = Side();
 }
 
@@ -423,7 +435,10 @@ int tgt_plan_info(const tgt_plan_t* plan, int64_t info[16]) {
     info[5] = plan->src.n_items;
     info[6] = plan->src.n_split;
     info[7] = plan->src.n_parts;
-    info[8] = tgt::kSegLen;
+    info[8] = tgt::kBlockSeg;
+    info[9] = tgt::kWaveRowMax;
+    info[10] = plan->dst.n_block_items;
+    info[11] = plan->src.n_block_items;
     return TGT_OK;
 }
 

@@ -12,8 +12,9 @@
 // a chunk of 8 consecutive elements, so LPE = H*d/8 lanes cover one edge and
 // LPH = d/8 lanes cover one head.  S "edge slots" work on S edges of the same
 // row at once (S*LPE lanes per row); short rows use small S and several rows
-// share a wave, long rows use the whole wave, rows longer than kSegLen are split
-// into segments whose partial sums a small second kernel adds in a fixed order.
+// share a wave, rows up to kWaveRowMax edges use a whole wave, longer rows are
+// walked by whole workgroups in segments of kBlockSeg edges whose partial sums the
+// last-arriving workgroup adds in a fixed order.
 #include "common.h"
 
 namespace tgt {
@@ -83,85 +84,94 @@ __host__ __device__ constexpr int slots_for_class(int lpe, int cls) {
     return nat < cap ? nat : cap;
 }
 
-// Which walk a launch performs.
+// Which walk a workgroup performs.
 enum { MODE_FWD = 0, MODE_BWD_DST = 1, MODE_BWD_SRC = 2 };
 
-struct WalkArgs {
-    // row-side and edge-side node features; meaning depends on the mode
+// Operands shared by both views.
+struct Common {
     const void* q;
     const void* k;
     const void* v;
     const void* g;        // dout (backward)
     const void* bias;
     const float2* nd;     // [N, H] (1/(Z+eps), D) (backward)
-    const Item* items;
-    const int32_t* col;
-    const int32_t* eid;
-    void* out0;           // fwd: out      bwd_dst: dq     bwd_src: dk
-    void* out1;           // fwd: -        bwd_dst: dbias  bwd_src: dv
-    float* Z;             // fwd: Z
-    float* part;          // partial slots of split rows
-    int32_t class_off[kNumClass + 1];
-    int32_t wave_off[kNumClass + 1];
-    int32_t n_parts;
     int32_t bias_mode;
     float inv_scale;
 };
 
+// One sorted view (by destination or by source) with its schedule and outputs.
+struct SideArgs {
+    const Item* items;
+    const int32_t* col;
+    const int32_t* eid;
+    const int32_t* split_off;
+    const int32_t* part2split;
+    void* out0;           // fwd: out      bwd_dst: dq     bwd_src: dk
+    void* out1;           // fwd: -        bwd_dst: dbias  bwd_src: dv
+    float* Z;             // fwd: Z
+    float* part;          // partial sums of split rows
+    int32_t* counters;    // one arrival counter per split row, zero between calls
+    int32_t n_block_items;
+    int32_t n_wave_blocks;
+    int32_t class_off[kNumClass + 1];
+    int32_t wave_off[kNumClass + 1];
+};
+
+struct Acc {
+    float a0[8];   // fwd: sum w v | bwd_dst: dq | bwd_src: dk
+    float a1[8];   // bwd_src: dv
+    float z;       // fwd: sum w
+};
+
+// Floats one partial slot holds.
+template <int MODE, int HD, int H>
+__host__ __device__ constexpr int part_stride() {
+    return MODE == MODE_FWD ? HD + H : (MODE == MODE_BWD_DST ? HD : 2 * HD);
+}
+
+// Walks `len` edges starting at sorted position `start` of node `row` with S edge
+// slots (this lane is slot `slot`, element chunk `el`).  On return every lane of
+// the S*LPE-lane group holds the sums over all S slots.
 template <typename T, int LPE, int LPH, int S, int MODE>
-__device__ __forceinline__ void walk_items(const WalkArgs& a, const int item_begin, const int item_end,
-                                           const int wave_in_class) {
-    constexpr int G = LPE * S;        // lanes per item
-    constexpr int IPW = kWave / G;    // items per wave
+__device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, const int row, const int start,
+                                           const int len, const int slot, const int el, const bool valid,
+                                           Acc& acc) {
+    constexpr int G = LPE * S;
     constexpr int H = LPE / LPH;
     constexpr int HD = LPE * 8;
-    const int lane = threadIdx.x & (kWave - 1);
-    const int sub = lane / G;
-    const int gl = lane % G;
-    const int slot = gl / LPE;
-    const int el = gl % LPE;
     const int head = el / LPH;
-    const int item = item_begin + wave_in_class * IPW + sub;
-    const bool valid = item < item_end;
-    Item it{0, 0, 0, -1};
-    if (valid) it = a.items[item];
+    const T* __restrict__ Q = static_cast<const T*>(c.q);
+    const T* __restrict__ K = static_cast<const T*>(c.k);
+    const T* __restrict__ V = static_cast<const T*>(c.v);
+    const T* __restrict__ Gd = static_cast<const T*>(c.g);
+    const T* __restrict__ B = static_cast<const T*>(c.bias);
+    const int64_t row_off = (int64_t)row * HD + el * 8;
 
-    const T* __restrict__ Q = static_cast<const T*>(a.q);
-    const T* __restrict__ K = static_cast<const T*>(a.k);
-    const T* __restrict__ V = static_cast<const T*>(a.v);
-    const T* __restrict__ Gd = static_cast<const T*>(a.g);
-    const T* __restrict__ B = static_cast<const T*>(a.bias);
-    const int64_t row_off = (int64_t)it.row * HD + el * 8;
-
-    // row-resident operands
-    float r0[8], r1[8];      // fwd: q | bwd_dst: q, g | bwd_src: k, v
+    float r0[8], r1[8];      // row-resident: fwd q | bwd_dst q, g | bwd_src k, v
     float rz = 0.f, Dh = 0.f;
 #pragma unroll
-    for (int c = 0; c < 8; ++c) { r0[c] = 0.f; r1[c] = 0.f; }
+    for (int i = 0; i < 8; ++i) { r0[i] = 0.f; r1[i] = 0.f; acc.a0[i] = 0.f; acc.a1[i] = 0.f; }
+    acc.z = 0.f;
     if (valid) {
         if (MODE == MODE_FWD) {
             load8(Q + row_off, r0);
         } else if (MODE == MODE_BWD_DST) {
             load8(Q + row_off, r0);
             load8(Gd + row_off, r1);
-            const float2 nd = a.nd[(int64_t)it.row * H + head];
+            const float2 nd = c.nd[(int64_t)row * H + head];
             rz = nd.x; Dh = nd.y;
         } else {
             load8(K + row_off, r0);
             load8(V + row_off, r1);
         }
     }
-    float acc0[8], acc1[8];  // fwd: sum w v | bwd_dst: dq | bwd_src: dk, dv
-    float z = 0.f;
-#pragma unroll
-    for (int c = 0; c < 8; ++c) { acc0[c] = 0.f; acc1[c] = 0.f; }
+    const int32_t* __restrict__ col = s.col + start;
+    const int32_t* __restrict__ eid = s.eid + start;
+    const int bias_mode = c.bias_mode;
+    const float inv_scale = c.inv_scale;
+    const int n = valid ? len : 0;
 
-    const int32_t* __restrict__ col = a.col + it.start;
-    const int32_t* __restrict__ eid = a.eid + it.start;
-    const int bias_mode = a.bias_mode;
-    const float inv_scale = a.inv_scale;
-
-    for (int e0 = slot; e0 < it.len; e0 += S * kUnroll) {
+    for (int e0 = slot; e0 < n; e0 += S * kUnroll) {
         int nb[kUnroll], ed[kUnroll];
         bool ok[kUnroll];
         float x0[kUnroll][8], x1[kUnroll][8], bb[kUnroll];
@@ -169,7 +179,7 @@ __device__ __forceinline__ void walk_items(const WalkArgs& a, const int item_beg
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             const int e = e0 + u * S;
-            ok[u] = e < it.len;
+            ok[u] = e < n;
             nb[u] = 0; ed[u] = 0;
             if (ok[u]) {
                 nb[u] = col[e];
@@ -181,13 +191,13 @@ __device__ __forceinline__ void walk_items(const WalkArgs& a, const int item_beg
             bb[u] = 0.f;
             ndv[u] = make_float2(0.f, 0.f);
 #pragma unroll
-            for (int c = 0; c < 8; ++c) { x0[u][c] = 0.f; x1[u][c] = 0.f; }
+            for (int i = 0; i < 8; ++i) { x0[u][i] = 0.f; x1[u][i] = 0.f; }
             if (ok[u]) {
                 const int64_t o = (int64_t)nb[u] * HD + el * 8;
                 if (MODE == MODE_BWD_SRC) {
                     load8(Q + o, x0[u]);
                     load8(Gd + o, x1[u]);
-                    ndv[u] = a.nd[(int64_t)nb[u] * H + head];
+                    ndv[u] = c.nd[(int64_t)nb[u] * H + head];
                 } else {
                     load8(K + o, x0[u]);
                     load8(V + o, x1[u]);
@@ -204,142 +214,271 @@ __device__ __forceinline__ void walk_items(const WalkArgs& a, const int item_beg
                 const float raw = head_sum<LPH>(dot8(r0, x0[u])) * inv_scale;
                 const float w = expf(clamp5(raw) + bb[u]);
                 if (MODE == MODE_FWD) {
-                    z += w;
+                    acc.z += w;
 #pragma unroll
-                    for (int c = 0; c < 8; ++c) acc0[c] = fmaf(w, x1[u][c], acc0[c]);
+                    for (int i = 0; i < 8; ++i) acc.a0[i] = fmaf(w, x1[u][i], acc.a0[i]);
                 } else {
                     const bool inside = (raw >= -5.0f) & (raw <= 5.0f);   // torch clamp backward: inclusive
                     if (MODE == MODE_BWD_DST) {
                         const float t = head_sum<LPH>(dot8(r1, x1[u]));   // g_dst . v_src
                         const float dS = w * rz * (t - Dh);
-                        T* __restrict__ dB = static_cast<T*>(a.out1);
+                        T* __restrict__ dB = static_cast<T*>(s.out1);
                         if (dB != nullptr) {
                             if (bias_mode == TGT_BIAS_EDGE_HEAD) {
                                 if (el % LPH == 0) store1(dB + (int64_t)ed[u] * H + head, dS);
                             } else if (bias_mode == TGT_BIAS_EDGE) {
-                                float s = dS;   // sum over heads; every head is held by LPH lanes
+                                float t2 = dS;   // sum over heads; every head is held by LPH lanes
 #pragma unroll
-                                for (int off = 1; off < LPE; off <<= 1) s += __shfl_xor(s, off);
-                                if (el == 0) store1(dB + ed[u], s * (1.0f / LPH));
+                                for (int off = 1; off < LPE; off <<= 1) t2 += __shfl_xor(t2, off);
+                                if (el == 0) store1(dB + ed[u], t2 * (1.0f / LPH));
                             }
                         }
                         const float md = inside ? dS : 0.f;
 #pragma unroll
-                        for (int c = 0; c < 8; ++c) acc0[c] = fmaf(md, x0[u][c], acc0[c]);
+                        for (int i = 0; i < 8; ++i) acc.a0[i] = fmaf(md, x0[u][i], acc.a0[i]);
                     } else {
                         const float p = w * ndv[u].x;
                         const float t = head_sum<LPH>(dot8(x1[u], r1));   // g_dst . v_src
                         const float dS = p * (t - ndv[u].y);
                         const float md = inside ? dS : 0.f;
 #pragma unroll
-                        for (int c = 0; c < 8; ++c) {
-                            acc0[c] = fmaf(md, x0[u][c], acc0[c]);   // dk += m dS q_dst
-                            acc1[c] = fmaf(p, x1[u][c], acc1[c]);    // dv += p g_dst
+                        for (int i = 0; i < 8; ++i) {
+                            acc.a0[i] = fmaf(md, x0[u][i], acc.a0[i]);   // dk += m dS q_dst
+                            acc.a1[i] = fmaf(p, x1[u][i], acc.a1[i]);    // dv += p g_dst
                         }
                     }
                 }
             }
         }
     }
-
-    // add the S edge slots of an item (all lanes take part)
+    // add the S edge slots (all lanes take part)
 #pragma unroll
     for (int off = LPE; off < G; off <<= 1) {
-        if (MODE == MODE_FWD) z += __shfl_xor(z, off);
+        if (MODE == MODE_FWD) acc.z += __shfl_xor(acc.z, off);
 #pragma unroll
-        for (int c = 0; c < 8; ++c) {
-            acc0[c] += __shfl_xor(acc0[c], off);
-            if (MODE == MODE_BWD_SRC) acc1[c] += __shfl_xor(acc1[c], off);
+        for (int i = 0; i < 8; ++i) {
+            acc.a0[i] += __shfl_xor(acc.a0[i], off);
+            if (MODE == MODE_BWD_SRC) acc.a1[i] += __shfl_xor(acc.a1[i], off);
         }
     }
-    if (!valid || slot != 0) return;
+}
 
-    if (MODE != MODE_FWD) {
+// Final value of a row from its sums, written by the LPE lanes that own the chunks.
+template <typename T, int LPE, int LPH, int MODE>
+__device__ __forceinline__ void write_row(const Common& c, const SideArgs& s, const int row, const int el,
+                                          Acc& acc) {
+    constexpr int H = LPE / LPH;
+    constexpr int HD = LPE * 8;
+    const int64_t row_off = (int64_t)row * HD + el * 8;
+    if (MODE == MODE_FWD) {
+        const float den = acc.z + kEps;
 #pragma unroll
-        for (int c = 0; c < 8; ++c) acc0[c] *= inv_scale;
-    }
-    if (it.part < 0) {
-        if (MODE == MODE_FWD) {
-            const float den = z + kEps;
-#pragma unroll
-            for (int c = 0; c < 8; ++c) acc0[c] = acc0[c] / den;
-            store8(static_cast<T*>(a.out0) + row_off, acc0);
-            if (el % LPH == 0) a.Z[(int64_t)it.row * H + head] = z;
-        } else if (MODE == MODE_BWD_DST) {
-            store8(static_cast<T*>(a.out0) + row_off, acc0);
-        } else {
-            store8(static_cast<T*>(a.out0) + row_off, acc0);
-            store8(static_cast<T*>(a.out1) + row_off, acc1);
-        }
+        for (int i = 0; i < 8; ++i) acc.a0[i] = acc.a0[i] / den;
+        store8(static_cast<T*>(s.out0) + row_off, acc.a0);
+        if (el % LPH == 0) s.Z[(int64_t)row * H + el / LPH] = acc.z;
     } else {
-        // partial slot layout: fwd [n_parts][HD] then [n_parts][H]; bwd_dst [n_parts][HD];
-        // bwd_src [n_parts][2][HD]
-        if (MODE == MODE_FWD) {
-            store8(a.part + (int64_t)it.part * HD + el * 8, acc0);
-            if (el % LPH == 0) a.part[(int64_t)a.n_parts * HD + (int64_t)it.part * H + head] = z;
-        } else if (MODE == MODE_BWD_DST) {
-            store8(a.part + (int64_t)it.part * HD + el * 8, acc0);
-        } else {
-            store8(a.part + (int64_t)it.part * 2 * HD + el * 8, acc0);
-            store8(a.part + (int64_t)it.part * 2 * HD + HD + el * 8, acc1);
-        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc.a0[i] *= c.inv_scale;
+        store8(static_cast<T*>(s.out0) + row_off, acc.a0);
+        if (MODE == MODE_BWD_SRC) store8(static_cast<T*>(s.out1) + row_off, acc.a1);
     }
+}
+
+// Wave items: rows of at most kWaveRowMax edges, 64 / (LPE*S) rows per wave.
+template <typename T, int LPE, int LPH, int S, int MODE>
+__device__ __forceinline__ void wave_items(const Common& c, const SideArgs& s, const int item_begin,
+                                           const int item_end, const int wave_in_class) {
+    constexpr int G = LPE * S;
+    constexpr int IPW = kWave / G;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int sub = lane / G, gl = lane % G;
+    const int slot = gl / LPE, el = gl % LPE;
+    const int item = item_begin + wave_in_class * IPW + sub;
+    const bool valid = item < item_end;
+    Item it{0, 0, 0, -1};
+    if (valid) it = s.items[item];
+    Acc acc;
+    walk_range<T, LPE, LPH, S, MODE>(c, s, it.row, it.start, it.len, slot, el, valid, acc);
+    if (valid && slot == 0) write_row<T, LPE, LPH, MODE>(c, s, it.row, el, acc);
 }
 
 template <typename T, int LPE, int LPH, int MODE>
-__global__ __launch_bounds__(kBlock) void k_walk(const WalkArgs a) {
-    const int gw = blockIdx.x * (kBlock / kWave) + (threadIdx.x >> 6);   // global wave index
+__device__ __forceinline__ void wave_block(const Common& c, const SideArgs& s, const int block) {
+    const int gw = block * (kBlock / kWave) + (threadIdx.x >> 6);
     int cls = 0;
 #pragma unroll
-    for (int c = 1; c < kNumClass; ++c) cls += (gw >= a.wave_off[c]) ? 1 : 0;
+    for (int k = 1; k < kNumClass; ++k) cls += (gw >= s.wave_off[k]) ? 1 : 0;
     cls = __builtin_amdgcn_readfirstlane(cls);
-    if (gw >= a.wave_off[kNumClass]) return;
-    const int w = gw - a.wave_off[cls];
-    const int b = a.class_off[cls], e = a.class_off[cls + 1];
+    if (gw >= s.wave_off[kNumClass]) return;
+    const int w = gw - s.wave_off[cls];
+    const int b = s.class_off[cls], e = s.class_off[cls + 1];
     switch (cls) {
-        case 0: walk_items<T, LPE, LPH, slots_for_class(LPE, 0), MODE>(a, b, e, w); break;
-        case 1: walk_items<T, LPE, LPH, slots_for_class(LPE, 1), MODE>(a, b, e, w); break;
-        case 2: walk_items<T, LPE, LPH, slots_for_class(LPE, 2), MODE>(a, b, e, w); break;
-        case 3: walk_items<T, LPE, LPH, slots_for_class(LPE, 3), MODE>(a, b, e, w); break;
-        default: walk_items<T, LPE, LPH, slots_for_class(LPE, 4), MODE>(a, b, e, w); break;
+        case 0: wave_items<T, LPE, LPH, slots_for_class(LPE, 0), MODE>(c, s, b, e, w); break;
+        case 1: wave_items<T, LPE, LPH, slots_for_class(LPE, 1), MODE>(c, s, b, e, w); break;
+        case 2: wave_items<T, LPE, LPH, slots_for_class(LPE, 2), MODE>(c, s, b, e, w); break;
+        case 3: wave_items<T, LPE, LPH, slots_for_class(LPE, 3), MODE>(c, s, b, e, w); break;
+        default: wave_items<T, LPE, LPH, slots_for_class(LPE, 4), MODE>(c, s, b, e, w); break;
     }
 }
 
-// Adds the partial slots of every split row in slot order (fixed order ->
-// reproducible) and writes the row.  One workgroup of 64 threads per split row.
-template <typename T, int MODE>
-__global__ __launch_bounds__(64) void k_combine(const int32_t* __restrict__ split_row,
-                                                const int32_t* __restrict__ split_off,
-                                                const float* __restrict__ part, int n_parts, int H, int d,
-                                                void* out0, void* out1, float* Z) {
-    const int r = blockIdx.x;
-    const int row = split_row[r];
-    const int p0 = split_off[r], p1 = split_off[r + 1];
-    const int HD = H * d;
-    for (int c = threadIdx.x; c < HD; c += 64) {
-        if (MODE == MODE_FWD) {
-            float acc = 0.f, z = 0.f;
-            const int h = c / d;
-            for (int p = p0; p < p1; ++p) {
-                acc += part[(int64_t)p * HD + c];
-                z += part[(int64_t)n_parts * HD + (int64_t)p * H + h];
+// LDS of one workgroup: sums of its lane groups, then (last arriver only) sums of
+// the partial slots of a split row.
+template <int LPE>
+struct BlockLds {
+    static constexpr int HD = LPE * 8;
+    static constexpr int STRIDE = 2 * HD + LPE;               // a0 | a1 | z (one float per chunk)
+    static constexpr int NGROUP = kBlock / LPE;               // combine groups
+    float red[NGROUP * STRIDE];
+    int last;
+};
+
+// Workgroup item: one segment (<= kBlockSeg edges) of a long row.  The lane groups
+// of the 4 waves each walk a share of the segment, LDS adds them in a fixed order.
+// If the row has several segments each workgroup stores its sums in a partial
+// slot, and the workgroup that arrives last adds the slots in slot order and
+// writes the row - no second launch, no floating-point atomics, and the order of
+// the additions does not depend on which workgroup is last.
+template <typename T, int LPE, int LPH, int MODE>
+__device__ __forceinline__ void block_item(const Common& c, const SideArgs& s, const int item,
+                                           BlockLds<LPE>& lds) {
+    constexpr int S = slots_for_class(LPE, 0);
+    constexpr int G = LPE * S;
+    constexpr int IPW = kWave / G;
+    constexpr int NG = (kBlock / kWave) * IPW;    // lane groups in the workgroup
+    constexpr int H = LPE / LPH;
+    constexpr int HD = LPE * 8;
+    constexpr int STRIDE = BlockLds<LPE>::STRIDE;
+    constexpr int PS = part_stride<MODE, HD, H>();
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int sub = lane / G, gl = lane % G;
+    const int slot = gl / LPE, el = gl % LPE;
+    const int grp = (tid >> 6) * IPW + sub;
+    const Item it = s.items[item];
+    // share of this lane group: consecutive chunk of the segment
+    const int share = (it.len + NG - 1) / NG;
+    const int lo = min(grp * share, it.len);
+    const int hi = min(lo + share, it.len);
+    Acc acc;
+    walk_range<T, LPE, LPH, S, MODE>(c, s, it.row, it.start + lo, hi - lo, slot, el, true, acc);
+    if (slot == 0) {
+        float* r = lds.red + grp * STRIDE;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            r[el * 8 + i] = acc.a0[i];
+            if (MODE == MODE_BWD_SRC) r[HD + el * 8 + i] = acc.a1[i];
+        }
+        if (MODE == MODE_FWD) r[2 * HD + el] = acc.z;
+    }
+    __syncthreads();
+    if (tid < LPE) {   // tid == el here
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { acc.a0[i] = 0.f; acc.a1[i] = 0.f; }
+        acc.z = 0.f;
+        for (int gI = 0; gI < NG; ++gI) {
+            const float* r = lds.red + gI * STRIDE;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                acc.a0[i] += r[tid * 8 + i];
+                if (MODE == MODE_BWD_SRC) acc.a1[i] += r[HD + tid * 8 + i];
             }
-            store1(static_cast<T*>(out0) + (int64_t)row * HD + c, acc / (z + kEps));
-            if (c % d == 0) Z[(int64_t)row * H + h] = z;
-        } else if (MODE == MODE_BWD_DST) {
-            float acc = 0.f;
-            for (int p = p0; p < p1; ++p) acc += part[(int64_t)p * HD + c];
-            store1(static_cast<T*>(out0) + (int64_t)row * HD + c, acc);
+            if (MODE == MODE_FWD) acc.z += r[2 * HD + tid];
+        }
+        if (it.part < 0) {
+            write_row<T, LPE, LPH, MODE>(c, s, it.row, tid, acc);
         } else {
-            float a0 = 0.f, a1 = 0.f;
-            for (int p = p0; p < p1; ++p) {
-                a0 += part[(int64_t)p * 2 * HD + c];
-                a1 += part[(int64_t)p * 2 * HD + HD + c];
-            }
-            store1(static_cast<T*>(out0) + (int64_t)row * HD + c, a0);
-            store1(static_cast<T*>(out1) + (int64_t)row * HD + c, a1);
+            float* p = s.part + (int64_t)it.part * PS;
+            store8(p + tid * 8, acc.a0);
+            if (MODE == MODE_BWD_SRC) store8(p + HD + tid * 8, acc.a1);
+            if (MODE == MODE_FWD && tid % LPH == 0) p[HD + tid / LPH] = acc.z;
         }
     }
+    if (it.part < 0) return;   // uniform over the workgroup
+
+    // arrival: the partial slot is published before the counter moves
+    const int sidx = s.part2split[it.part];
+    const int p0 = s.split_off[sidx], p1 = s.split_off[sidx + 1];
+    if (tid < kWave) {          // wave 0 holds every writer of the slot
+        __threadfence();
+        if (tid == 0) {
+            const int old = atomicAdd(&s.counters[sidx], 1);
+            lds.last = (old == p1 - p0 - 1) ? 1 : 0;
+        }
+    }
+    __syncthreads();
+    if (!lds.last) return;
+    __threadfence();
+    // last arriver: NGROUP groups of LPE threads add slots p0 + grp2, p0 + grp2 + NGROUP, ...
+    constexpr int NGROUP = BlockLds<LPE>::NGROUP;
+    const int grp2 = tid / LPE, el2 = tid % LPE;
+    {
+        float a0[8], a1[8], z = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { a0[i] = 0.f; a1[i] = 0.f; }
+        for (int p = p0 + grp2; p < p1; p += NGROUP) {
+            const float* src = s.part + (int64_t)p * PS;
+            float t0[8], t1[8];
+            load8(src + el2 * 8, t0);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) a0[i] += t0[i];
+            if (MODE == MODE_BWD_SRC) {
+                load8(src + HD + el2 * 8, t1);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) a1[i] += t1[i];
+            }
+            if (MODE == MODE_FWD) z += src[HD + el2 / LPH];
+        }
+        float* r = lds.red + grp2 * STRIDE;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            r[el2 * 8 + i] = a0[i];
+            if (MODE == MODE_BWD_SRC) r[HD + el2 * 8 + i] = a1[i];
+        }
+        if (MODE == MODE_FWD) r[2 * HD + el2] = z;
+    }
+    __syncthreads();
+    if (tid < LPE) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { acc.a0[i] = 0.f; acc.a1[i] = 0.f; }
+        acc.z = 0.f;
+        for (int gI = 0; gI < NGROUP; ++gI) {
+            const float* r = lds.red + gI * STRIDE;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                acc.a0[i] += r[tid * 8 + i];
+                if (MODE == MODE_BWD_SRC) acc.a1[i] += r[HD + tid * 8 + i];
+            }
+            if (MODE == MODE_FWD) acc.z += r[2 * HD + tid];
+        }
+        write_row<T, LPE, LPH, MODE>(c, s, it.row, tid, acc);
+        if (tid == 0) s.counters[sidx] = 0;   // ready for the next call
+    }
+}
+
+// Forward: workgroup items of the destination view first (longest work first),
+// then its wave items.
+template <typename T, int LPE, int LPH>
+__global__ __launch_bounds__(kBlock) void k_attn_fwd(const Common c, const SideArgs s) {
+    __shared__ BlockLds<LPE> lds;
+    const int b = blockIdx.x;
+    if (b < s.n_block_items) block_item<T, LPE, LPH, MODE_FWD>(c, s, b, lds);
+    else wave_block<T, LPE, LPH, MODE_FWD>(c, s, b - s.n_block_items);
+}
+
+// Backward: both views in one launch (they are independent once nd is known):
+// workgroup items of the destination view, workgroup items of the source view,
+// wave items of the destination view, wave items of the source view.
+template <typename T, int LPE, int LPH>
+__global__ __launch_bounds__(kBlock) void k_attn_bwd(const Common c, const SideArgs sd, const SideArgs ss) {
+    __shared__ BlockLds<LPE> lds;
+    int b = blockIdx.x;
+    if (b < sd.n_block_items) { block_item<T, LPE, LPH, MODE_BWD_DST>(c, sd, b, lds); return; }
+    b -= sd.n_block_items;
+    if (b < ss.n_block_items) { block_item<T, LPE, LPH, MODE_BWD_SRC>(c, ss, b, lds); return; }
+    b -= ss.n_block_items;
+    if (b < sd.n_wave_blocks) { wave_block<T, LPE, LPH, MODE_BWD_DST>(c, sd, b); return; }
+    b -= sd.n_wave_blocks;
+    wave_block<T, LPE, LPH, MODE_BWD_SRC>(c, ss, b);
 }
 
 // Per-node side vector of the backward: nd[i,h] = (1 / (Z[i,h] + eps), sum_c dout[i,h,c] out[i,h,c]).
@@ -355,7 +494,7 @@ __global__ __launch_bounds__(kBlock) void k_node_side(const T* __restrict__ out,
     const bool valid = row < N;
     float o[8], g[8];
 #pragma unroll
-    for (int c = 0; c < 8; ++c) { o[c] = 0.f; g[c] = 0.f; }
+    for (int i = 0; i < 8; ++i) { o[i] = 0.f; g[i] = 0.f; }
     if (valid) {
         load8(out + row * HD + el * 8, o);
         load8(dout + row * HD + el * 8, g);
@@ -373,7 +512,7 @@ __global__ __launch_bounds__(kBlock) void k_node_side(const T* __restrict__ out,
 static inline int64_t align256(int64_t x) { return (x + 255) & ~(int64_t)255; }
 
 struct WsLayout {
-    int64_t nd, fwd_part, dq_part, dkv_part, total;
+    int64_t nd, fwd_part, dq_part, dkv_part, counters, total;
 };
 static WsLayout ws_layout(const tgt_plan* p, int H, int d) {
     const int64_t HD = (int64_t)H * d;
@@ -382,11 +521,15 @@ static WsLayout ws_layout(const tgt_plan* p, int H, int d) {
     w.fwd_part = align256(p->N * H * 8);
     w.dq_part = w.fwd_part + align256((int64_t)p->dst.n_parts * (HD + H) * 4);
     w.dkv_part = w.dq_part + align256((int64_t)p->dst.n_parts * HD * 4);
-    w.total = w.dkv_part + align256((int64_t)p->src.n_parts * 2 * HD * 4);
+    w.counters = w.dkv_part + align256((int64_t)p->src.n_parts * 2 * HD * 4);
+    w.total = w.counters + align256(((int64_t)2 * p->dst.n_split + p->src.n_split + 1) * 4);
     return w;
 }
 
-static void fill_schedule(WalkArgs& a, const Side& s, int lpe, int* n_blocks) {
+static void fill_side(SideArgs& a, const Side& s, int lpe) {
+    a.items = s.items; a.col = s.col; a.eid = s.eid;
+    a.split_off = s.split_off; a.part2split = s.part2split;
+    a.n_block_items = s.n_block_items;
     int waves = 0;
     for (int c = 0; c < kNumClass; ++c) {
         a.class_off[c] = s.class_off[c];
@@ -397,8 +540,7 @@ static void fill_schedule(WalkArgs& a, const Side& s, int lpe, int* n_blocks) {
     }
     a.class_off[kNumClass] = s.class_off[kNumClass];
     a.wave_off[kNumClass] = waves;
-    a.n_parts = s.n_parts;
-    *n_blocks = (waves + (kBlock / kWave) - 1) / (kBlock / kWave);
+    a.n_wave_blocks = (waves + (kBlock / kWave) - 1) / (kBlock / kWave);
 }
 
 struct Call {
@@ -416,20 +558,20 @@ struct Call {
 template <typename T, int LPE, int LPH>
 static int run_fwd(const Call& c) {
     const WsLayout L = ws_layout(c.plan, c.H, c.d);
-    WalkArgs a{};
-    a.q = c.q; a.k = c.k; a.v = c.v; a.g = nullptr; a.bias = c.bias; a.nd = nullptr;
-    a.items = c.plan->dst.items; a.col = c.plan->dst.col; a.eid = c.plan->dst.eid;
+    Common cm{};
+    cm.q = c.q; cm.k = c.k; cm.v = c.v; cm.g = nullptr; cm.bias = c.bias; cm.nd = nullptr;
+    cm.bias_mode = c.bias_mode;
+    cm.inv_scale = 1.0f / sqrtf((float)c.d);
+    SideArgs a{};
+    fill_side(a, c.plan->dst, LPE);
     a.out0 = c.o_out; a.out1 = nullptr; a.Z = c.o_Z;
     a.part = reinterpret_cast<float*>(c.ws + L.fwd_part);
-    a.bias_mode = c.bias_mode;
-    a.inv_scale = 1.0f / sqrtf((float)c.d);
-    int nb = 0;
-    fill_schedule(a, c.plan->dst, LPE, &nb);
-    if (nb > 0) hipLaunchKernelGGL((k_walk<T, LPE, LPH, MODE_FWD>), dim3(nb), dim3(kBlock), 0, c.st, a);
-    if (c.plan->dst.n_split > 0)
-        hipLaunchKernelGGL((k_combine<T, MODE_FWD>), dim3(c.plan->dst.n_split), dim3(64), 0, c.st,
-                           c.plan->dst.split_row, c.plan->dst.split_off, a.part, c.plan->dst.n_parts, c.H,
-                           c.d, c.o_out, nullptr, c.o_Z);
+    a.counters = reinterpret_cast<int32_t*>(c.ws + L.counters);
+    const int nb = a.n_block_items + a.n_wave_blocks;
+    if (nb > 0) {
+        KernelTimer t(KS_FWD, c.st);
+        hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH>), dim3(nb), dim3(kBlock), 0, c.st, cm, a);
+    }
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
 }
@@ -442,35 +584,29 @@ static int run_bwd(const Call& c) {
     {
         constexpr int RPB = kBlock / LPE;
         const int nb = (int)((N + RPB - 1) / RPB);
+        KernelTimer t(KS_NODE_SIDE, c.st);
         hipLaunchKernelGGL((k_node_side<T, LPE, LPH>), dim3(nb), dim3(kBlock), 0, c.st,
                            static_cast<const T*>(c.out), static_cast<const T*>(c.dout), c.Z, N, nd);
     }
-    WalkArgs a{};
-    a.q = c.q; a.k = c.k; a.v = c.v; a.g = c.dout; a.bias = c.bias; a.nd = nd;
-    a.bias_mode = c.bias_mode;
-    a.inv_scale = 1.0f / sqrtf((float)c.d);
-    a.Z = nullptr;
-    int nb = 0;
-    // destination view: dq, dbias
-    a.items = c.plan->dst.items; a.col = c.plan->dst.col; a.eid = c.plan->dst.eid;
-    a.out0 = c.dq; a.out1 = c.dbias;
-    a.part = reinterpret_cast<float*>(c.ws + L.dq_part);
-    fill_schedule(a, c.plan->dst, LPE, &nb);
-    if (nb > 0) hipLaunchKernelGGL((k_walk<T, LPE, LPH, MODE_BWD_DST>), dim3(nb), dim3(kBlock), 0, c.st, a);
-    if (c.plan->dst.n_split > 0)
-        hipLaunchKernelGGL((k_combine<T, MODE_BWD_DST>), dim3(c.plan->dst.n_split), dim3(64), 0, c.st,
-                           c.plan->dst.split_row, c.plan->dst.split_off, a.part, c.plan->dst.n_parts, c.H,
-                           c.d, c.dq, nullptr, nullptr);
-    // source view: dk, dv
-    a.items = c.plan->src.items; a.col = c.plan->src.col; a.eid = c.plan->src.eid;
-    a.out0 = c.dk; a.out1 = c.dv;
-    a.part = reinterpret_cast<float*>(c.ws + L.dkv_part);
-    fill_schedule(a, c.plan->src, LPE, &nb);
-    if (nb > 0) hipLaunchKernelGGL((k_walk<T, LPE, LPH, MODE_BWD_SRC>), dim3(nb), dim3(kBlock), 0, c.st, a);
-    if (c.plan->src.n_split > 0)
-        hipLaunchKernelGGL((k_combine<T, MODE_BWD_SRC>), dim3(c.plan->src.n_split), dim3(64), 0, c.st,
-                           c.plan->src.split_row, c.plan->src.split_off, a.part, c.plan->src.n_parts, c.H,
-                           c.d, c.dk, c.dv, nullptr);
+    Common cm{};
+    cm.q = c.q; cm.k = c.k; cm.v = c.v; cm.g = c.dout; cm.bias = c.bias; cm.nd = nd;
+    cm.bias_mode = c.bias_mode;
+    cm.inv_scale = 1.0f / sqrtf((float)c.d);
+    int32_t* counters = reinterpret_cast<int32_t*>(c.ws + L.counters);
+    SideArgs sd{}, ss{};
+    fill_side(sd, c.plan->dst, LPE);
+    sd.out0 = c.dq; sd.out1 = c.dbias; sd.Z = nullptr;
+    sd.part = reinterpret_cast<float*>(c.ws + L.dq_part);
+    sd.counters = counters + c.plan->dst.n_split;
+    fill_side(ss, c.plan->src, LPE);
+    ss.out0 = c.dk; ss.out1 = c.dv; ss.Z = nullptr;
+    ss.part = reinterpret_cast<float*>(c.ws + L.dkv_part);
+    ss.counters = counters + 2 * c.plan->dst.n_split;
+    const int nb = sd.n_block_items + ss.n_block_items + sd.n_wave_blocks + ss.n_wave_blocks;
+    if (nb > 0) {
+        KernelTimer t(KS_BWD, c.st);
+        hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss);
+    }
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
 }

@@ -61,7 +61,7 @@ class GraphPlan:
         arr = (ctypes.c_int64 * 16)()
         _lib.check(_lib.lib().tgt_plan_info(self.handle, arr))
         keys = ["N", "E", "items_dst", "split_rows_dst", "segments_dst", "items_src", "split_rows_src",
-                "segments_src", "segment_len"]
+                "segments_src", "segment_len", "wave_row_max", "block_items_dst", "block_items_src"]
         return {k: int(arr[i]) for i, k in enumerate(keys)}
 
     def export(self, which):
@@ -83,7 +83,7 @@ class GraphPlan:
             nbytes = _lib.lib().tgt_sparse_attn_workspace_bytes(self.handle, H, d)
             if nbytes < 0:
                 raise ValueError("bad H / d")
-            ws = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=self.device)
+            ws = torch.zeros(max(int(nbytes), 256), dtype=torch.uint8, device=self.device)   # counters start at 0
             self._workspaces[key] = ws
         return ws
 
