@@ -102,6 +102,9 @@ def main():
     ap.add_argument("--dtype", default="f32", choices=["f32", "bf16"])
     ap.add_argument("--workload", default="config2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run one 256 MiB device copy (a kernel of known traffic, for scaling rocprofv3 "
+                         "FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on ONE GPU (sequence-parallel size 1); "
@@ -153,6 +156,14 @@ def main():
                                          dt_code, P(out), P(Z), P(dout), P(dq), P(dk), P(dv), P(dbias),
                                          P(ws), ws.numel(), stream))
 
+    if args.calibration_copy:
+        # reads 256 MiB and writes 256 MiB in one elementwise kernel (name contains "elementwise")
+        b = torch.ones(64 << 20, dtype=torch.float32, device=dev)
+        a = torch.empty_like(b)
+        torch.cuda.synchronize()
+        torch.neg(b, out=a)
+        torch.cuda.synchronize()
+        del a, b
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()

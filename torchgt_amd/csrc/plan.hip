@@ -13,6 +13,7 @@
 #include "common.h"
 #include <vector>
 #include <new>
+#include <stdlib.h>
 
 namespace tgt {
 
@@ -252,7 +253,17 @@ static int length_class(int len) {
 // neighbouring rows stay together.  A longer row is walked by whole workgroups:
 // ceil(len / kBlockSeg) balanced segments, each a workgroup item; if there is more
 // than one segment their partial sums meet in the workspace.
+static int env_int(const char* name, int dflt) {
+    const char* v = getenv(name);
+    if (!v || !*v) return dflt;
+    const int x = atoi(v);
+    return x > 0 ? x : dflt;
+}
+
 static int build_schedule(const std::vector<int32_t>& rowptr, int64_t N, Side& side, hipStream_t st) {
+    // tuning overrides (experiments only; the defaults are the measured best)
+    const int kWaveRowMax = env_int("TGT_WAVE_ROW_MAX", tgt::kWaveRowMax);
+    const int kBlockSeg = env_int("TGT_BLOCK_SEG", tgt::kBlockSeg);
     std::vector<Item> cls[kNumClass];
     std::vector<Item> items;
     std::vector<int32_t> split_row, split_off, part2split;

@@ -22,10 +22,9 @@ namespace tgt {
 struct bf16_t { uint16_t x; };
 
 __device__ __forceinline__ float bf16_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
-__device__ __forceinline__ uint32_t f32_to_bf16(float f) {   // round to nearest even, NaN kept quiet
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
-    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+__device__ __forceinline__ uint32_t f32_to_bf16(float f) {   // gfx950 converts in hardware (round to nearest even)
+    const __bf16 b = static_cast<__bf16>(f);
+    return (uint32_t)__builtin_bit_cast(uint16_t, b);
 }
 
 __device__ __forceinline__ void load8(const float* __restrict__ p, float (&x)[8]) {
@@ -171,6 +170,7 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
     const float inv_scale = c.inv_scale;
     const int n = valid ? len : 0;
 
+#pragma unroll 1
     for (int e0 = slot; e0 < n; e0 += S * kUnroll) {
         int nb[kUnroll], ed[kUnroll];
         bool ok[kUnroll];
@@ -618,6 +618,7 @@ static int dispatch(const Call& c, bool bwd) {
     if (lpe == LPE_ && lph == LPH_)                                            \
         return bwd ? run_bwd<T, LPE_, LPH_>(c) : run_fwd<T, LPE_, LPH_>(c);
     TGT_CASE(8, 1)    // H=8  d=8   (Graphormer-Slim / GT node level, hidden 64)
+#ifndef TGT_ONLY_8x8   // -DTGT_ONLY_8x8: compile one shape only (quick experiments)
     TGT_CASE(8, 2)    // H=4  d=16  (attention micro-benchmark, attn_module.py:387)
     TGT_CASE(16, 2)   // H=8  d=16  (hidden 128, the parser default)
     TGT_CASE(16, 1)   // H=16 d=8
@@ -626,6 +627,7 @@ static int dispatch(const Call& c, bool bwd) {
     TGT_CASE(1, 1)    // H=1  d=8
     TGT_CASE(4, 2)    // H=2  d=16
     TGT_CASE(2, 2)    // H=1  d=16
+#endif
 #undef TGT_CASE
     set_error("no kernel for H=%d d=%d (d must be 8 or 16 and H*d/8 one of 1,2,4,8,16)", c.H, c.d);
     return TGT_ERR_UNSUPPORTED;
