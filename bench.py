@@ -48,6 +48,16 @@ def kernel_alg_bytes(name, N, E, H, d, esize, bpe):
     return table.get(name)
 
 
+# HBM-side bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each
+# scaled by the reading of a copy kernel of known size: FETCH x2.000, WRITE x1.000); the summary is
+# profiles/sparse_attn_config2_hbm_traffic_pmc.txt.  Counters cannot be read from inside this process,
+# so the figures are carried here and only reported for the workload / dtype they were measured on.
+MEASURED_TRAFFIC = {
+    ("config2", "f32"): {"attn_fwd": 254.3e6, "bwd_node_side": 38.9e6, "attn_bwd": 638.5e6},
+    ("config2", "bf16"): {"attn_fwd": 143.1e6, "bwd_node_side": 22.6e6, "attn_bwd": 378.2e6},
+}
+
+
 def build_workload(name):
     import numpy as np
     from torchgt_amd import workloads
@@ -205,7 +215,9 @@ def main():
         "hbm_roofline_frac_step": step_gbs / HBM_PEAK_GBS,
         "alg_bytes_step": fwd_b + bwd_b,
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": dom_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": dom_gbs / HBM_PEAK_GBS, "traffic": None, "alg_bytes": dom_bytes,
+                     "frac": dom_gbs / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC.get((args.workload, args.dtype), {}).get(dom),
+                     "alg_bytes": dom_bytes,
                      "avg_us": kernels[dom]["avg_us"]},
         "kernels": kernels,
         "plan_build_ms": plan_ms, "plan_build_first_ms": plan_first_ms,
