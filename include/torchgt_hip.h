@@ -120,6 +120,37 @@ int tgt_sparse_attn_bwd(const tgt_plan_t* plan,
                         void* d_dq, void* d_dk, void* d_dv, void* d_dbias,
                         void* d_workspace, int64_t workspace_bytes, void* stream);
 
+/* ---- edge construction and ordering ------------------------------------
+ * fix_edge_index (gt_sp/utils.py:34-50): d_edge_index int64 [2, E0] over real
+ * nodes 0..num_node-1 -> d_out int64 [2, E0 + 2*num_node]: real nodes shift by +1,
+ * then num_node edges (i+1 -> 0), then num_node edges (0 -> i+1).  Global node 0
+ * gets no self-loop. */
+int tgt_fix_edge_index(const int64_t* d_edge_index, int64_t E0, int64_t num_node, int64_t* d_out, void* stream);
+
+/* reformat_graph (gt_sp/utils.py:319-359) with the METIS call replaced by the
+ * explicit d_partition_ids int64 [N] in [0, k):
+ *   relabel: parts in order 0..k-1, members in ascending old id (:329-335);
+ *   blockize != 0: generate_new_edges_optimized (:223-305) - the edges of every
+ *     partition pair are REPLACED by int(count/bs^2)+1 random dense bs x bs blocks
+ *     drawn from numpy's legacy MT19937 stream exactly as the reference draws them
+ *     (including its compact-count quirk and p hard-wired to 1);
+ *   blockize == 0: keep the real edges (the alternative commented out at :347);
+ *   stable sort of the new edge list by source (:354-356).
+ * Synchronises `stream`.  Results are read with tgt_reformat_export:
+ * d_edge_index int64 [2, E'] (E' = tgt_reformat_num_edges), d_sorted_indices
+ * int64 [N] = argsort(new_id_mapping) (new id -> old id, :352). */
+typedef struct tgt_reformat tgt_reformat_t;
+int tgt_reformat_create(const int64_t* d_src, const int64_t* d_dst, int64_t E, int64_t N,
+                        const int64_t* d_partition_ids, int k, int block_size, int blockize,
+                        void* stream, tgt_reformat_t** out);
+int64_t tgt_reformat_num_edges(const tgt_reformat_t* r);
+int tgt_reformat_export(const tgt_reformat_t* r, int64_t* d_edge_index, int64_t* d_sorted_indices, void* stream);
+int tgt_reformat_destroy(tgt_reformat_t* r);
+
+/* Host only: the n values np.random.randint(0, h_highs[i]) returns after
+ * np.random.seed(seed) (legacy MT19937 stream used by gt_sp/utils.py:290-295). */
+int tgt_np_legacy_randint(uint32_t seed, const int64_t* h_highs, int n, int64_t* h_out);
+
 /* ---- per-kernel timing --------------------------------------------------
  * The reference times this path with torch.profiler around whole iterations
  * (attn_module.py:415-438).  When enabled, every kernel the library launches is

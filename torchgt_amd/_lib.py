@@ -33,6 +33,12 @@ SIGNATURES = {
     "tgt_sparse_attn_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _i64, _vp]),
     "tgt_sparse_attn_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp,
                                    _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
+    "tgt_fix_edge_index": (_i32, [_vp, _i64, _i64, _vp, _vp]),
+    "tgt_reformat_create": (_i32, [_vp, _vp, _i64, _i64, _vp, _i32, _i32, _i32, _vp, _c.POINTER(_vp)]),
+    "tgt_reformat_num_edges": (_i64, [_vp]),
+    "tgt_reformat_export": (_i32, [_vp, _vp, _vp, _vp]),
+    "tgt_reformat_destroy": (_i32, [_vp]),
+    "tgt_np_legacy_randint": (_i32, [_c.c_uint32, _vp, _i32, _vp]),
     "tgt_timing_enable": (_i32, [_i32]),
     "tgt_timing_reset": (_i32, []),
     "tgt_timing_slots": (_i32, []),

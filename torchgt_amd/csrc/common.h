@@ -46,6 +46,34 @@ struct Side {
     int32_t class_off[kNumClass + 1] = {0, 0, 0, 0, 0, 0};   // item index where each wave class begins
 };
 
+// Device buffer that frees itself.
+struct DevBuf {
+    void* p = nullptr;
+    DevBuf() = default;
+    DevBuf(const DevBuf&) = delete;
+    DevBuf& operator=(const DevBuf&) = delete;
+    ~DevBuf();
+    hipError_t alloc(size_t bytes);
+    template <typename T> T* as() const { return (T*)p; }
+};
+
+int bits_for(int64_t n);   // bits needed to hold values in [0, n)
+
+// Stable LSD radix sort of (uint32 key, uint32 value) pairs (radix_sort.hip).
+class RadixSorter {
+public:
+    int init(int64_t capacity);
+    // Sorts by the low `bits` bits of the keys.  vals_in == nullptr means values 0..n-1.
+    // The results live in the sorter's buffers until the next sort() call; copy a
+    // result before passing it as input of another sort().
+    int sort(const uint32_t* keys_in, const uint32_t* vals_in, int64_t n, int bits, hipStream_t st,
+             const uint32_t** keys_out, const uint32_t** vals_out);
+private:
+    DevBuf keysA_, keysB_, valsA_, valsB_, hist_, totals_;
+    int64_t cap_ = 0;
+    int nblocks_ = 0;
+};
+
 // Kernel names of the optional per-kernel timing (timing.hip).
 enum KernelSlot { KS_FWD = 0, KS_NODE_SIDE, KS_BWD, KS_COUNT };
 

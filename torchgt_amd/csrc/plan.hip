@@ -29,11 +29,6 @@ const char* last_error() { return g_err; }
 // ---------------------------------------------------------------------------
 // kernels
 // ---------------------------------------------------------------------------
-constexpr int RS_THREADS = 256;
-constexpr int RS_ITEMS = 16;
-constexpr int RS_TILE = RS_THREADS * RS_ITEMS;   // 4096 keys per workgroup
-constexpr int RS_WAVE_SPAN = kWave * RS_ITEMS;   // 1024 consecutive keys per wave
-
 // int64 endpoints -> uint32, with a range check (flag[0] = 1 on a bad index).
 __global__ void k_convert_validate(const int64_t* __restrict__ src, const int64_t* __restrict__ dst,
                                    int64_t E, int64_t N, uint32_t* __restrict__ s32,
@@ -45,123 +40,6 @@ __global__ void k_convert_validate(const int64_t* __restrict__ src, const int64_
     if (bad) { flag[0] = 1; s = 0; d = 0; }
     s32[i] = (uint32_t)s;
     d32[i] = (uint32_t)d;
-}
-
-// Per-workgroup digit histogram, stored digit-major: hist[digit * nblocks + block].
-__global__ __launch_bounds__(RS_THREADS) void k_rs_hist(const uint32_t* __restrict__ keys, int64_t n,
-                                                        int shift, uint32_t* __restrict__ hist,
-                                                        int nblocks) {
-    __shared__ uint32_t h[256];
-    const int tid = threadIdx.x;
-    h[tid] = 0;
-    __syncthreads();
-    const int64_t base = (int64_t)blockIdx.x * RS_TILE;
-#pragma unroll
-    for (int i = 0; i < RS_ITEMS; ++i) {
-        int64_t idx = base + i * RS_THREADS + tid;
-        if (idx < n) atomicAdd(&h[(keys[idx] >> shift) & 255u], 1u);   // integer count: order-free
-    }
-    __syncthreads();
-    hist[(int64_t)tid * nblocks + blockIdx.x] = h[tid];
-}
-
-// Workgroup `digit` turns its row of per-block counts into exclusive offsets and
-// records the row total.
-__global__ __launch_bounds__(256) void k_rs_scan_rows(uint32_t* __restrict__ hist, int nblocks,
-                                                      uint32_t* __restrict__ totals) {
-    __shared__ uint32_t part[256];
-    const int tid = threadIdx.x;
-    uint32_t* row = hist + (int64_t)blockIdx.x * nblocks;
-    const int chunk = (nblocks + 255) / 256;
-    const int b = tid * chunk;
-    const int e = min(b + chunk, nblocks);
-    uint32_t s = 0;
-    for (int i = b; i < e; ++i) s += row[i];
-    part[tid] = s;
-    __syncthreads();
-    for (int off = 1; off < 256; off <<= 1) {
-        uint32_t x = tid >= off ? part[tid - off] : 0u;
-        __syncthreads();
-        part[tid] += x;
-        __syncthreads();
-    }
-    uint32_t run = tid ? part[tid - 1] : 0u;
-    for (int i = b; i < e; ++i) {
-        uint32_t x = row[i];
-        row[i] = run;
-        run += x;
-    }
-    if (tid == 255) totals[blockIdx.x] = part[255];
-}
-
-// Stable scatter of one radix pass.  Each wave owns 1024 consecutive keys of the
-// tile and ranks them in 16 rounds of 64; the rank of a key among equal digits is
-// (count in earlier rounds) + (number of lower lanes with the same digit).
-__global__ __launch_bounds__(RS_THREADS) void k_rs_scatter(
-    const uint32_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in,
-    uint32_t* __restrict__ keys_out, uint32_t* __restrict__ vals_out, int64_t n, int shift,
-    const uint32_t* __restrict__ hist, const uint32_t* __restrict__ totals, int nblocks) {
-    __shared__ uint32_t cnt[4][256];
-    __shared__ uint32_t base[256];
-    __shared__ uint32_t scan[256];
-    const int tid = threadIdx.x;
-    const int wave = tid >> 6;
-    const int lane = tid & 63;
-    for (int i = tid; i < 4 * 256; i += RS_THREADS) (&cnt[0][0])[i] = 0;
-    scan[tid] = totals[tid];
-    __syncthreads();
-
-    volatile uint32_t* wcnt = &cnt[wave][0];
-    uint32_t key[RS_ITEMS], rank[RS_ITEMS];
-    const int64_t wbase = (int64_t)blockIdx.x * RS_TILE + (int64_t)wave * RS_WAVE_SPAN;
-    const uint64_t lower_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-#pragma unroll
-    for (int r = 0; r < RS_ITEMS; ++r) {
-        const int64_t idx = wbase + r * kWave + lane;
-        const bool valid = idx < n;
-        const uint32_t kk = valid ? keys_in[idx] : 0u;
-        key[r] = kk;
-        const uint32_t dg = (kk >> shift) & 255u;
-        uint64_t same = __ballot(valid);
-#pragma unroll
-        for (int b = 0; b < 8; ++b) {
-            const bool bit = (dg >> b) & 1u;
-            const uint64_t bal = __ballot(bit);
-            same &= bit ? bal : ~bal;
-        }
-        uint32_t prior = 0;
-        if (valid) prior = wcnt[dg];
-        const uint32_t lower = (uint32_t)__popcll(same & lower_mask);
-        rank[r] = prior + lower;
-        if (valid && lower == 0) wcnt[dg] = prior + (uint32_t)__popcll(same);
-    }
-    __syncthreads();
-    // exclusive prefix over the 4 waves (thread = digit) and over the 256 digit totals
-    {
-        uint32_t c0 = cnt[0][tid], c1 = cnt[1][tid], c2 = cnt[2][tid];
-        cnt[0][tid] = 0;
-        cnt[1][tid] = c0;
-        cnt[2][tid] = c0 + c1;
-        cnt[3][tid] = c0 + c1 + c2;
-    }
-    for (int off = 1; off < 256; off <<= 1) {
-        uint32_t x = tid >= off ? scan[tid - off] : 0u;
-        __syncthreads();
-        scan[tid] += x;
-        __syncthreads();
-    }
-    base[tid] = (tid ? scan[tid - 1] : 0u) + hist[(int64_t)tid * nblocks + blockIdx.x];
-    __syncthreads();
-#pragma unroll
-    for (int r = 0; r < RS_ITEMS; ++r) {
-        const int64_t idx = wbase + r * kWave + lane;
-        if (idx < n) {
-            const uint32_t dg = (key[r] >> shift) & 255u;
-            const uint32_t pos = base[dg] + cnt[wave][dg] + rank[r];
-            keys_out[pos] = key[r];
-            vals_out[pos] = vals_in ? vals_in[idx] : (uint32_t)idx;
-        }
-    }
 }
 
 // rowptr[r] = first sorted position whose key is >= r.
@@ -186,48 +64,14 @@ __global__ void k_gather_col(const uint32_t* __restrict__ eid, const uint32_t* _
 // ---------------------------------------------------------------------------
 // host helpers
 // ---------------------------------------------------------------------------
-struct DevBuf {
-    void* p = nullptr;
-    ~DevBuf() { if (p) (void)hipFree(p); }
-    hipError_t alloc(size_t bytes) { return hipMalloc(&p, bytes ? bytes : 4); }
-    template <typename T> T* as() { return (T*)p; }
-};
-
-static int radix_passes(int64_t N) {
-    int bits = 1;
-    while (bits < 32 && ((int64_t)1 << bits) < N) ++bits;
-    return (bits + 7) / 8;
-}
-
-struct SortScratch {
-    DevBuf keysA, keysB, valsA, valsB, hist, totals;
-    int nblocks = 0;
-};
-
 // Sort edge ids by `keys32` (stable) and fill one Side's rowptr / col / eid.
 static int build_side(const uint32_t* keys32, const uint32_t* other32, int64_t E, int64_t N,
-                      SortScratch& sc, Side& side, hipStream_t st) {
-    const int passes = radix_passes(N);
+                      RadixSorter& sorter, Side& side, hipStream_t st) {
     const uint32_t* kin = keys32;
     const uint32_t* vin = nullptr;
-    uint32_t* kout = sc.keysA.as<uint32_t>();
-    uint32_t* vout = sc.valsA.as<uint32_t>();
     if (E > 0) {
-        for (int p = 0; p < passes; ++p) {
-            const int shift = 8 * p;
-            hipLaunchKernelGGL(k_rs_hist, dim3(sc.nblocks), dim3(RS_THREADS), 0, st, kin, E, shift,
-                               sc.hist.as<uint32_t>(), sc.nblocks);
-            hipLaunchKernelGGL(k_rs_scan_rows, dim3(256), dim3(256), 0, st, sc.hist.as<uint32_t>(),
-                               sc.nblocks, sc.totals.as<uint32_t>());
-            hipLaunchKernelGGL(k_rs_scatter, dim3(sc.nblocks), dim3(RS_THREADS), 0, st, kin, vin, kout,
-                               vout, E, shift, sc.hist.as<uint32_t>(), sc.totals.as<uint32_t>(),
-                               sc.nblocks);
-            kin = kout;
-            vin = vout;
-            const bool toB = (kout == sc.keysA.as<uint32_t>());
-            kout = toB ? sc.keysB.as<uint32_t>() : sc.keysA.as<uint32_t>();
-            vout = toB ? sc.valsB.as<uint32_t>() : sc.valsA.as<uint32_t>();
-        }
+        int rc = sorter.sort(keys32, nullptr, E, bits_for(N), st, &kin, &vin);
+        if (rc) return rc;
     }
     const int T = 256;
     hipLaunchKernelGGL(k_fill_rowptr, dim3((unsigned)((E + 1 + T - 1) / T)), dim3(T), 0, st, kin, E, N,
@@ -339,19 +183,15 @@ static int create_impl(const int64_t* d_src, const int64_t* d_dst, int64_t E, in
         TGT_HIP_CHECK(hipMalloc((void**)&s->eid, sizeof(int32_t) * (E ? E : 1)));
     }
     DevBuf s32, d32, flag;
-    SortScratch sc;
-    sc.nblocks = (int)((E + RS_TILE - 1) / RS_TILE);
-    if (sc.nblocks < 1) sc.nblocks = 1;
+    RadixSorter sorter;
     const size_t eb = sizeof(uint32_t) * (size_t)(E ? E : 1);
     TGT_HIP_CHECK(s32.alloc(eb));
     TGT_HIP_CHECK(d32.alloc(eb));
     TGT_HIP_CHECK(flag.alloc(sizeof(int)));
-    TGT_HIP_CHECK(sc.keysA.alloc(eb));
-    TGT_HIP_CHECK(sc.keysB.alloc(eb));
-    TGT_HIP_CHECK(sc.valsA.alloc(eb));
-    TGT_HIP_CHECK(sc.valsB.alloc(eb));
-    TGT_HIP_CHECK(sc.hist.alloc(sizeof(uint32_t) * 256 * (size_t)sc.nblocks));
-    TGT_HIP_CHECK(sc.totals.alloc(sizeof(uint32_t) * 256));
+    {
+        int rc0 = sorter.init(E);
+        if (rc0) return rc0;
+    }
     TGT_HIP_CHECK(hipMemsetAsync(flag.p, 0, sizeof(int), st));
     if (E > 0) {
         const int T = 256;
@@ -366,9 +206,9 @@ static int create_impl(const int64_t* d_src, const int64_t* d_dst, int64_t E, in
         set_error("edge_index holds a node id outside [0, %lld)", (long long)N);
         return TGT_ERR_INDEX_RANGE;
     }
-    int rc = build_side(d32.as<uint32_t>(), s32.as<uint32_t>(), E, N, sc, plan->dst, st);
+    int rc = build_side(d32.as<uint32_t>(), s32.as<uint32_t>(), E, N, sorter, plan->dst, st);
     if (rc) return rc;
-    rc = build_side(s32.as<uint32_t>(), d32.as<uint32_t>(), E, N, sc, plan->src, st);
+    rc = build_side(s32.as<uint32_t>(), d32.as<uint32_t>(), E, N, sorter, plan->src, st);
     if (rc) return rc;
     std::vector<int32_t> rp_dst((size_t)N + 1), rp_src((size_t)N + 1);
     TGT_HIP_CHECK(hipMemcpyAsync(rp_dst.data(), plan->dst.rowptr, sizeof(int32_t) * (N + 1),

@@ -1,0 +1,189 @@
+// Stable LSD radix sort of (uint32 key, uint32 value) pairs, 8-bit digits.
+//
+// The ranking is position-based (ballots and prefix counts), so the output is
+// the stable order - what numpy's argsort(kind='stable') gives - and is
+// bit-reproducible: integer LDS counters only count, they never decide an order.
+// Used for the CSR/CSC build (keys = destination / source node) and for the
+// graph reordering (keys = partition id, new source id).
+#include "common.h"
+
+namespace tgt {
+
+constexpr int RS_THREADS = 256;
+constexpr int RS_ITEMS = 16;
+constexpr int RS_TILE = RS_THREADS * RS_ITEMS;   // 4096 keys per workgroup
+constexpr int RS_WAVE_SPAN = kWave * RS_ITEMS;   // 1024 consecutive keys per wave
+
+// Per-workgroup digit histogram, stored digit-major: hist[digit * nblocks + block].
+__global__ __launch_bounds__(RS_THREADS) void k_rs_hist(const uint32_t* __restrict__ keys, int64_t n,
+                                                        int shift, uint32_t* __restrict__ hist,
+                                                        int nblocks) {
+    __shared__ uint32_t h[256];
+    const int tid = threadIdx.x;
+    h[tid] = 0;
+    __syncthreads();
+    const int64_t base = (int64_t)blockIdx.x * RS_TILE;
+#pragma unroll
+    for (int i = 0; i < RS_ITEMS; ++i) {
+        int64_t idx = base + i * RS_THREADS + tid;
+        if (idx < n) atomicAdd(&h[(keys[idx] >> shift) & 255u], 1u);   // integer count: order-free
+    }
+    __syncthreads();
+    hist[(int64_t)tid * nblocks + blockIdx.x] = h[tid];
+}
+
+// Workgroup `digit` turns its row of per-block counts into exclusive offsets and
+// records the row total.
+__global__ __launch_bounds__(256) void k_rs_scan_rows(uint32_t* __restrict__ hist, int nblocks,
+                                                      uint32_t* __restrict__ totals) {
+    __shared__ uint32_t part[256];
+    const int tid = threadIdx.x;
+    uint32_t* row = hist + (int64_t)blockIdx.x * nblocks;
+    const int chunk = (nblocks + 255) / 256;
+    const int b = tid * chunk;
+    const int e = min(b + chunk, nblocks);
+    uint32_t s = 0;
+    for (int i = b; i < e; ++i) s += row[i];
+    part[tid] = s;
+    __syncthreads();
+    for (int off = 1; off < 256; off <<= 1) {
+        uint32_t x = tid >= off ? part[tid - off] : 0u;
+        __syncthreads();
+        part[tid] += x;
+        __syncthreads();
+    }
+    uint32_t run = tid ? part[tid - 1] : 0u;
+    for (int i = b; i < e; ++i) {
+        uint32_t x = row[i];
+        row[i] = run;
+        run += x;
+    }
+    if (tid == 255) totals[blockIdx.x] = part[255];
+}
+
+// Stable scatter of one radix pass.  Each wave owns 1024 consecutive keys of the
+// tile and ranks them in 16 rounds of 64; the rank of a key among equal digits is
+// (count in earlier rounds) + (number of lower lanes with the same digit).
+__global__ __launch_bounds__(RS_THREADS) void k_rs_scatter(
+    const uint32_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in,
+    uint32_t* __restrict__ keys_out, uint32_t* __restrict__ vals_out, int64_t n, int shift,
+    const uint32_t* __restrict__ hist, const uint32_t* __restrict__ totals, int nblocks) {
+    __shared__ uint32_t cnt[4][256];
+    __shared__ uint32_t base[256];
+    __shared__ uint32_t scan[256];
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    for (int i = tid; i < 4 * 256; i += RS_THREADS) (&cnt[0][0])[i] = 0;
+    scan[tid] = totals[tid];
+    __syncthreads();
+
+    volatile uint32_t* wcnt = &cnt[wave][0];
+    uint32_t key[RS_ITEMS], rank[RS_ITEMS];
+    const int64_t wbase = (int64_t)blockIdx.x * RS_TILE + (int64_t)wave * RS_WAVE_SPAN;
+    const uint64_t lower_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+#pragma unroll
+    for (int r = 0; r < RS_ITEMS; ++r) {
+        const int64_t idx = wbase + r * kWave + lane;
+        const bool valid = idx < n;
+        const uint32_t kk = valid ? keys_in[idx] : 0u;
+        key[r] = kk;
+        const uint32_t dg = (kk >> shift) & 255u;
+        uint64_t same = __ballot(valid);
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            const bool bit = (dg >> b) & 1u;
+            const uint64_t bal = __ballot(bit);
+            same &= bit ? bal : ~bal;
+        }
+        uint32_t prior = 0;
+        if (valid) prior = wcnt[dg];
+        const uint32_t lower = (uint32_t)__popcll(same & lower_mask);
+        rank[r] = prior + lower;
+        if (valid && lower == 0) wcnt[dg] = prior + (uint32_t)__popcll(same);
+    }
+    __syncthreads();
+    // exclusive prefix over the 4 waves (thread = digit) and over the 256 digit totals
+    {
+        uint32_t c0 = cnt[0][tid], c1 = cnt[1][tid], c2 = cnt[2][tid];
+        cnt[0][tid] = 0;
+        cnt[1][tid] = c0;
+        cnt[2][tid] = c0 + c1;
+        cnt[3][tid] = c0 + c1 + c2;
+    }
+    for (int off = 1; off < 256; off <<= 1) {
+        uint32_t x = tid >= off ? scan[tid - off] : 0u;
+        __syncthreads();
+        scan[tid] += x;
+        __syncthreads();
+    }
+    base[tid] = (tid ? scan[tid - 1] : 0u) + hist[(int64_t)tid * nblocks + blockIdx.x];
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < RS_ITEMS; ++r) {
+        const int64_t idx = wbase + r * kWave + lane;
+        if (idx < n) {
+            const uint32_t dg = (key[r] >> shift) & 255u;
+            const uint32_t pos = base[dg] + cnt[wave][dg] + rank[r];
+            keys_out[pos] = key[r];
+            vals_out[pos] = vals_in ? vals_in[idx] : (uint32_t)idx;
+        }
+    }
+}
+
+
+hipError_t DevBuf::alloc(size_t bytes) {
+    if (p) { (void)hipFree(p); p = nullptr; }
+    return hipMalloc(&p, bytes ? bytes : 4);
+}
+DevBuf::~DevBuf() { if (p) (void)hipFree(p); }
+
+int bits_for(int64_t n) {
+    int bits = 1;
+    while (bits < 32 && ((int64_t)1 << bits) < n) ++bits;
+    return bits;
+}
+
+int RadixSorter::init(int64_t n) {
+    cap_ = n > 0 ? n : 1;
+    nblocks_ = (int)((cap_ + RS_TILE - 1) / RS_TILE);
+    const size_t eb = sizeof(uint32_t) * (size_t)cap_;
+    TGT_HIP_CHECK(keysA_.alloc(eb));
+    TGT_HIP_CHECK(keysB_.alloc(eb));
+    TGT_HIP_CHECK(valsA_.alloc(eb));
+    TGT_HIP_CHECK(valsB_.alloc(eb));
+    TGT_HIP_CHECK(hist_.alloc(sizeof(uint32_t) * 256 * (size_t)nblocks_));
+    TGT_HIP_CHECK(totals_.alloc(sizeof(uint32_t) * 256));
+    return TGT_OK;
+}
+
+int RadixSorter::sort(const uint32_t* keys_in, const uint32_t* vals_in, int64_t n, int bits, hipStream_t st,
+                      const uint32_t** keys_out, const uint32_t** vals_out) {
+    if (n > cap_) { set_error("RadixSorter: n exceeds capacity"); return TGT_ERR_INVALID_ARG; }
+    const int passes = (bits + 7) / 8 > 0 ? (bits + 7) / 8 : 1;
+    const int nblocks = (int)((n + RS_TILE - 1) / RS_TILE);
+    const uint32_t* kin = keys_in;
+    const uint32_t* vin = vals_in;
+    uint32_t* kout = keysA_.as<uint32_t>();
+    uint32_t* vout = valsA_.as<uint32_t>();
+    for (int p = 0; p < passes && n > 0; ++p) {
+        const int shift = 8 * p;
+        hipLaunchKernelGGL(k_rs_hist, dim3(nblocks), dim3(RS_THREADS), 0, st, kin, n, shift,
+                           hist_.as<uint32_t>(), nblocks);
+        hipLaunchKernelGGL(k_rs_scan_rows, dim3(256), dim3(256), 0, st, hist_.as<uint32_t>(), nblocks,
+                           totals_.as<uint32_t>());
+        hipLaunchKernelGGL(k_rs_scatter, dim3(nblocks), dim3(RS_THREADS), 0, st, kin, vin, kout, vout, n,
+                           shift, hist_.as<uint32_t>(), totals_.as<uint32_t>(), nblocks);
+        kin = kout;
+        vin = vout;
+        const bool toB = (kout == keysA_.as<uint32_t>());
+        kout = toB ? keysB_.as<uint32_t>() : keysA_.as<uint32_t>();
+        vout = toB ? valsB_.as<uint32_t>() : valsA_.as<uint32_t>();
+    }
+    TGT_HIP_CHECK(hipGetLastError());
+    *keys_out = kin;
+    *vals_out = vin;
+    return TGT_OK;
+}
+
+}  // namespace tgt
