@@ -120,6 +120,24 @@ int tgt_sparse_attn_bwd(const tgt_plan_t* plan,
                         void* d_dq, void* d_dk, void* d_dv, void* d_dbias,
                         void* d_workspace, int64_t workspace_bytes, void* stream);
 
+/* ---- dense biased attention (graph-level batches) -------------------------
+ * CoreAttention.forward of models/graphormer_graph_level.py:186-214 (same body:
+ * attn_module.py:99-127):  x = (q * sqrt(d)) k^T + bias ; softmax over keys ; x v.
+ * d_q, d_k, d_v: [b, S, H, d]; d_bias: [b, H, S, S] (may hold -inf on padded
+ * keys) or NULL; d_out: [b, S, H*d]; all of `dtype`.  d_lse: [b, H, S] float32
+ * (log-sum-exp of every score row, saved for the backward).  bf16 matrix
+ * instructions with fp32 accumulation and fp32 softmax; float32 inputs are rounded
+ * to bf16 on load.  d in {8, 16, 32}, S <= 256.  Dropout and the reference's
+ * unused `mask` argument are not applied. */
+int tgt_dense_attn_fwd(const void* d_q, const void* d_k, const void* d_v, const void* d_bias,
+                       int b, int S, int H, int d, int dtype,
+                       void* d_out, float* d_lse, void* stream);
+/* Backward (autograd in the reference).  d_dbias: [b, H, S, S] or NULL. */
+int tgt_dense_attn_bwd(const void* d_q, const void* d_k, const void* d_v, const void* d_bias,
+                       int b, int S, int H, int d, int dtype,
+                       const void* d_out, const float* d_lse, const void* d_dout,
+                       void* d_dq, void* d_dk, void* d_dv, void* d_dbias, void* stream);
+
 /* ---- edge construction and ordering ------------------------------------
  * fix_edge_index (gt_sp/utils.py:34-50): d_edge_index int64 [2, E0] over real
  * nodes 0..num_node-1 -> d_out int64 [2, E0 + 2*num_node]: real nodes shift by +1,

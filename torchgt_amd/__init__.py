@@ -4,8 +4,10 @@ sparse attention behind the reference's ``CoreAttention`` module API.
 The compute lives in ``libtorchgt_hip.so`` (sources in ``csrc/``, C ABI in
 ``include/torchgt_hip.h``); this package is the thin host side.
 """
-from .core_attention import CoreAttention, SparseAttentionFunction, sparse_attention, gather_dense_bias
+from .core_attention import (CoreAttention, SparseAttentionFunction, DenseAttentionFunction, sparse_attention,
+                             dense_attention, gather_dense_bias)
 from .plan import GraphPlan, get_plan, clear_plan_cache
 
-__all__ = ["CoreAttention", "SparseAttentionFunction", "sparse_attention", "gather_dense_bias",
+__all__ = ["CoreAttention", "SparseAttentionFunction", "DenseAttentionFunction", "sparse_attention",
+           "dense_attention", "gather_dense_bias",
            "GraphPlan", "get_plan", "clear_plan_cache"]

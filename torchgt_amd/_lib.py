@@ -33,6 +33,9 @@ SIGNATURES = {
     "tgt_sparse_attn_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _i64, _vp]),
     "tgt_sparse_attn_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp,
                                    _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
+    "tgt_dense_attn_fwd": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp]),
+    "tgt_dense_attn_bwd": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp,
+                                  _vp, _vp, _vp, _vp, _vp]),
     "tgt_fix_edge_index": (_i32, [_vp, _i64, _i64, _vp, _vp]),
     "tgt_reformat_create": (_i32, [_vp, _vp, _i64, _i64, _vp, _i32, _i32, _i32, _vp, _c.POINTER(_vp)]),
     "tgt_reformat_num_edges": (_i64, [_vp]),

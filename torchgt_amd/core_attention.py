@@ -48,7 +48,7 @@ class SparseAttentionFunction(torch.autograd.Function):
         mode = _lib.BIAS_NONE
         if edge_bias is not None:
             if edge_bias.dtype != q.dtype:
-                edge_bias = edge_bias.to(q.dtype)
+                raise TypeError("edge bias must have the dtype of q (convert it outside, where autograd sees it)")
             edge_bias = edge_bias.contiguous()
             E = plan.num_edges
             if edge_bias.dim() == 2 and edge_bias.shape == (E, H) and H != 1:
@@ -92,6 +92,62 @@ class SparseAttentionFunction(torch.autograd.Function):
         return dq, dk, dv, dbias, None
 
 
+class DenseAttentionFunction(torch.autograd.Function):
+    """out[b,S,H*d] = softmax((q*sqrt(d)) k^T + bias) v, the dense ``CoreAttention.forward`` of
+    models/graphormer_graph_level.py:186-214, on the library's MFMA kernels."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, bias):
+        if not (q.is_cuda and k.is_cuda and v.is_cuda):
+            raise RuntimeError("dense attention needs GPU tensors (no CPU implementation)")
+        if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
+            raise TypeError(f"q/k/v must share dtype float32 or bfloat16, got {q.dtype}/{k.dtype}/{v.dtype}")
+        if q.dim() != 4 or q.shape != k.shape or q.shape != v.shape:
+            raise ValueError("q, k, v must be [b, S, H, d] with equal shapes")
+        b, S, H, d = q.shape
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        if bias is not None:
+            if tuple(bias.shape) != (b, H, S, S) or bias.dtype != q.dtype:
+                raise ValueError(f"attn_bias must be {q.dtype} [b, H, S, S] = {(b, H, S, S)}, "
+                                 f"got {bias.dtype} {tuple(bias.shape)}")
+            bias = bias.contiguous()
+        out = torch.empty((b, S, H * d), dtype=q.dtype, device=q.device)
+        lse = torch.empty((b, H, S), dtype=torch.float32, device=q.device)
+        with torch.cuda.device(q.device):
+            stream = torch.cuda.current_stream(q.device).cuda_stream
+            _lib.check(_lib.lib().tgt_dense_attn_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(bias), b, S, H, d,
+                                                     _DTYPES[q.dtype], _ptr(out), _ptr(lse), stream))
+        ctx.save_for_backward(q, k, v, bias, out, lse)
+        ctx.has_bias = bias is not None
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, bias, out, lse = ctx.saved_tensors
+        b, S, H, d = q.shape
+        dout = dout.contiguous()
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        dbias = torch.empty_like(bias) if (ctx.has_bias and ctx.needs_input_grad[3]) else None
+        with torch.cuda.device(q.device):
+            stream = torch.cuda.current_stream(q.device).cuda_stream
+            _lib.check(_lib.lib().tgt_dense_attn_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(bias), b, S, H, d,
+                                                     _DTYPES[q.dtype], _ptr(out), _ptr(lse), _ptr(dout),
+                                                     _ptr(dq), _ptr(dk), _ptr(dv), _ptr(dbias), stream))
+        return dq, dk, dv, dbias
+
+
+def dense_attention(q, k, v, attn_bias=None):
+    """Functional form of the dense path: q, k, v [b, S, H, d], attn_bias [b, H, S, S] or None;
+    returns [b, S, H*d].  A bias of another float dtype or with a broadcast head axis
+    ([b, 1, S, S]) is converted / expanded here, where autograd sees it."""
+    if attn_bias is not None:
+        b, S, H = q.shape[0], q.shape[1], q.shape[2]
+        if attn_bias.dim() == 4 and attn_bias.shape[1] == 1 and H != 1:
+            attn_bias = attn_bias.expand(b, H, S, S)
+        attn_bias = attn_bias.to(q.dtype)
+    return DenseAttentionFunction.apply(q, k, v, attn_bias)
+
+
 def sparse_attention(q, k, v, edge_index=None, edge_bias=None, plan=None, return_z=False):
     """Functional form.  q, k, v: [N, H, d] (or [b, S, H, d], flattened over b*S
     as in attn_module.py:141-143); ``edge_index`` int64 [2, E] (row 0 = source /
@@ -103,6 +159,8 @@ def sparse_attention(q, k, v, edge_index=None, edge_bias=None, plan=None, return
         if edge_index is None:
             raise ValueError("need edge_index or plan")
         plan = get_plan(edge_index, q3.shape[0])
+    if edge_bias is not None:
+        edge_bias = edge_bias.to(q3.dtype)
     out, Z = SparseAttentionFunction.apply(q3, k3, v3, edge_bias, plan)
     return (out, Z) if return_z else out
 
@@ -157,6 +215,8 @@ class CoreAttention(nn.Module):
         v3 = v.reshape(-1, H, d)
         plan = edge_index if isinstance(edge_index, GraphPlan) else get_plan(edge_index, q3.shape[0])
         eb = self._edge_bias(attn_bias, edge_index)
+        if eb is not None:
+            eb = eb.to(q3.dtype)
         out, _ = SparseAttentionFunction.apply(q3, k3, v3, eb, plan)
         return out
 
@@ -171,10 +231,17 @@ class CoreAttention(nn.Module):
         b, S = k.size(0), k.size(1)
         return self._sparse(q, k, v, edge_index, attn_bias).view(b, S, -1)
 
-    def full_attention(self, *args, **kw):
-        raise NotImplementedError(
-            "dense attention (attn_type='full') is served by torchgt_amd.dense_attention; "
-            "it is not wired into this class yet")
+    def full_attention(self, q, k, v, attn_bias=None, mask=None):
+        """attn_module.py:99-127 / graphormer_graph_level.py:186-214: dense attention with an
+        additive [b, H, S, S] bias.  Returns [b, S, H*d]."""
+        if mask is not None:
+            raise NotImplementedError("the reference never passes `mask` (graphormer_graph_level.py:380); "
+                                      "it is not supported")
+        if self.training and self.attention_dropout_rate > 0:
+            raise NotImplementedError(
+                "attention dropout inside the dense kernel is not implemented; construct CoreAttention "
+                "with attention_dropout_rate=0 or call it in eval mode")
+        return dense_attention(q, k, v, attn_bias)
 
     def forward(self, q, k, v, attn_bias=None, edge_index=None, attn_type=None, mask=None,
                 flash_attn=False, full=False):
@@ -182,17 +249,21 @@ class CoreAttention(nn.Module):
         ``forward(q, k, v, attn_bias, edge_index, attn_type)`` with q, k, v
         [b, S, H, d]; returns [b, S, H*d].  The benchmark convention of
         attn_module.py:221-229, ``forward(q, k, v, edge_index)``, is recognised
-        by an integer [2, E] fourth argument."""
+        by an integer [2, E] fourth argument; the graph-level convention of
+        graphormer_graph_level.py:186, ``forward(q, k, v, attn_bias, mask)``, by
+        the absence of both edge_index and attn_type."""
         if (edge_index is None and isinstance(attn_bias, torch.Tensor) and attn_bias.dim() == 2
                 and attn_bias.size(0) == 2 and not attn_bias.is_floating_point()):
             edge_index, attn_bias = attn_bias, None
             if attn_type is None:
                 attn_type = "full" if full else ("flash" if flash_attn else "sparse")
+        if attn_type is None and edge_index is None:
+            attn_type = "full"        # graph-level convention: forward(q, k, v, attn_bias, mask)
         b, S = q.size(0), q.size(1)
         if attn_type == "sparse":
             x = self._sparse(q, k, v, edge_index, attn_bias)
         elif attn_type == "full":
-            x = self.full_attention(k, q, v, attn_bias)
+            x = self.full_attention(q, k, v, attn_bias, mask)
         elif attn_type == "flash":
             raise NotImplementedError(
                 "attn_type='flash' calls the CUDA-only flash_attn package in the reference "
