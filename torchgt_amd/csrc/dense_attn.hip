@@ -16,7 +16,8 @@
 // and its registers run over keys: the softmax reductions are register-local plus
 // one cross-half shuffle, and the probabilities sit exactly in the B-operand
 // layout of the next product (O^T = V^T P^T), no shuffle or LDS round trip.
-// The bias tile is transposed through LDS so that its global reads are coalesced.
+// The bias is staged in LDS strip by strip with 16-byte loads (a strip of 32 query
+// rows is contiguous in memory) and read from there in whichever layout a phase needs.
 #include "common.h"
 
 namespace tgt {
@@ -69,8 +70,6 @@ __device__ __forceinline__ float16_t zero16() {
 }
 __device__ __forceinline__ short4_t zero4() { short4_t z; z.x = 0; z.y = 0; z.z = 0; z.w = 0; return z; }
 
-constexpr int kTilePad = 33;   // LDS row stride of a 32x32 fp32 tile (conflict-free transposed reads)
-
 // LDS images of X[g, :, h, :]: row-major [SP][D] and transposed [D][SP+4] (bf16 bits).
 template <int D, int SP> constexpr int rm_elems() { return SP * D; }
 template <int D, int SP> constexpr int tr_elems() { return D * (SP + 4); }
@@ -93,35 +92,103 @@ __device__ __forceinline__ void load_head(const T* __restrict__ X, int g, int h,
     }
 }
 
-// dynamic LDS sizes (bytes)
-template <int D, int NT> constexpr int fwd_lds_bytes() {
-    return 2 * (rm_elems<D, NT * 32>() + tr_elems<D, NT * 32>()) + 4 * NT * 32 * kTilePad;
-}
-template <int D, int NT> constexpr int bwd_lds_bytes() {
-    return 2 * (4 * rm_elems<D, NT * 32>() + 3 * tr_elems<D, NT * 32>()) + 4 * 2 * NT * 32 + 4 * NT * 32 * kTilePad;
+// One wave's strip of the bias: rows q0 .. q0+31 of bias[g, h] are CONTIGUOUS in
+// the [b, H, S, S] tensor, so the strip is fetched with 16-byte loads from the
+// aligned-down start and kept in LDS as bf16 with row stride strip_stride(S)
+// (never a multiple of 4 elements, so that 32 lanes reading one key of 32
+// different rows hit different banks).  Chunks that straddle the tensor's ends
+// are read element by element.
+template <int SP> constexpr int strip_elems() { return 32 * (SP + 2) + 16; }
+__device__ __forceinline__ int strip_stride(int S) { return (S & 3) == 0 ? S + 2 : S; }
+
+// Returns the offset of strip element 0 inside `strip` (readers add it).
+template <typename T>
+__device__ __forceinline__ int stage_strip(const T* __restrict__ bias, int64_t e0, int count, int S,
+                                           int64_t total, short* __restrict__ strip, int lane) {
+    constexpr int EPC = 16 / (int)sizeof(T);
+    const int SL = strip_stride(S);
+    const uintptr_t A = reinterpret_cast<uintptr_t>(bias + e0);
+    const uintptr_t A0 = A & ~(uintptr_t)15;
+    const int head = (int)((A - A0) / sizeof(T));
+    const int nchunk = (head + count + EPC - 1) / EPC;
+    const T* base0 = reinterpret_cast<const T*>(A0);
+    const T* t_begin = bias;
+    const T* t_end = bias + total;
+    for (int c = lane; c < nchunk; c += 64) {
+        const T* p = base0 + (int64_t)c * EPC;
+        short vals[EPC];
+        if (p >= t_begin && p + EPC <= t_end) {
+            if (sizeof(T) == 2) {
+                const uint4 u = *reinterpret_cast<const uint4*>(p);
+                vals[0] = (short)(u.x & 0xffffu); vals[1] = (short)(u.x >> 16);
+                vals[2] = (short)(u.y & 0xffffu); vals[3] = (short)(u.y >> 16);
+                vals[4 % EPC] = (short)(u.z & 0xffffu); vals[5 % EPC] = (short)(u.z >> 16);
+                vals[6 % EPC] = (short)(u.w & 0xffffu); vals[7 % EPC] = (short)(u.w >> 16);
+            } else {
+                const float4_t f = *reinterpret_cast<const float4_t*>(p);
+                vals[0] = f2bf(f.x); vals[1] = f2bf(f.y); vals[2] = f2bf(f.z); vals[3] = f2bf(f.w);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < EPC; ++i) {
+                const T* q = p + i;
+                vals[i] = (q >= t_begin && q < t_end) ? f2bf(ld1(q)) : (short)0;
+            }
+        }
+        if (SL == S) {          // rows stay contiguous: the chunk goes to LDS as it came, shifted by `head`
+#pragma unroll
+            for (int i = 0; i < EPC; ++i) strip[c * EPC + i] = vals[i];
+            continue;
+        }
+        // element i of the chunk is strip element e = c*EPC + i - head: (row, key) = (e / S, e % S)
+        int e = c * EPC - head;
+        int row = e >= 0 ? e / S : -1;
+        int key = e >= 0 ? e - row * S : 0;
+#pragma unroll
+        for (int i = 0; i < EPC; ++i, ++e) {
+            if (e >= 0 && e < count) strip[row * SL + key] = vals[i];
+            if (e >= 0 && ++key == S) { key = 0; ++row; }
+            if (e < 0 && e + 1 == 0) { row = 0; key = 0; }
+        }
+    }
+    return SL == S ? head : 0;
 }
 
+// dynamic LDS sizes (bytes)
+template <int D, int NT> constexpr int fwd_lds_bytes() {
+    return 2 * (rm_elems<D, NT * 32>() + tr_elems<D, NT * 32>() + NT * strip_elems<NT * 32>());
+}
+template <int D, int NT> constexpr int bwd_lds_bytes() {
+    return 2 * (4 * rm_elems<D, NT * 32>() + 3 * tr_elems<D, NT * 32>() + NT * strip_elems<NT * 32>()) +
+           4 * 2 * NT * 32 + 4 * 8;
+}
+constexpr int kLdsLimit = 160 * 1024;
+
 // ---------------------------------------------------------------------------
-// forward
+// forward: online softmax over key tiles
 // ---------------------------------------------------------------------------
 template <typename T, int D, int NT>
 __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, const T* __restrict__ K,
                                                        const T* __restrict__ V, const T* __restrict__ bias,
                                                        T* __restrict__ out, float* __restrict__ lse, int S,
-                                                       int H, float scale) {
+                                                       int H, float scale, int64_t bias_total) {
     constexpr int KS = D / 8;
     constexpr int SP = NT * 32;
     extern __shared__ __align__(16) char smem[];
     short* k_rm = reinterpret_cast<short*>(smem);
     short* v_tr = k_rm + rm_elems<D, SP>();
-    float* bias_all = reinterpret_cast<float*>(v_tr + tr_elems<D, SP>());
     const int g = blockIdx.x / H, h = blockIdx.x % H;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int col = lane & 31, half = lane >> 5;
-    float* bias_l = bias_all + wave * 32 * kTilePad;
+    short* strip = v_tr + tr_elems<D, SP>() + wave * strip_elems<SP>();
+    const int q0 = wave * 32, qi = q0 + col;
+    int head = 0;
+    if (bias != nullptr) {
+        const int rows = min(32, S - q0);
+        head = stage_strip<T>(bias, (((int64_t)g * H + h) * S + q0) * S, rows * S, S, bias_total, strip, lane);
+    }
     load_head<T, D, SP>(K, g, h, S, H, k_rm, nullptr);
     load_head<T, D, SP>(V, g, h, S, H, nullptr, v_tr);
-    const int q0 = wave * 32, qi = q0 + col;
     short4_t bq[KS];
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
@@ -129,67 +196,53 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
         if (qi < S) bq[s] = ld4(Q + (((int64_t)g * S + qi) * H + h) * D + s * 8 + half * 4);
     }
     __syncthreads();
-    float16_t acc[NT];
-#pragma unroll
+    const short* brow = strip + head + col * strip_stride(S);     // this lane's query row of the bias
+    float m = -INFINITY, l = 0.f;
+    float16_t o = zero16();
+#pragma unroll 1
     for (int kt = 0; kt < NT; ++kt) {
-        acc[kt] = zero16();
+        float16_t sc = zero16();
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
             const short4_t a = *reinterpret_cast<const short4_t*>(&k_rm[(kt * 32 + col) * D + s * 8 + half * 4]);
-            acc[kt] = mfma(a, bq[s], acc[kt]);
+            sc = mfma(a, bq[s], sc);
         }
-    }
-    // scale, bias (transposed through LDS), key padding
-    float m = -INFINITY;
-#pragma unroll
-    for (int kt = 0; kt < NT; ++kt) {
-        if (bias != nullptr) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = r * 2 + half, key = kt * 32 + col;
-                float bv = 0.f;
-                if (q0 + row < S && key < S)
-                    bv = ld1(bias + (((int64_t)g * H + h) * S + q0 + row) * S + key);
-                bias_l[row * kTilePad + col] = bv;
-            }
-        }
-        __syncthreads();
+        float tmax = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const int kk = 8 * (r / 4) + 4 * half + (r % 4);
-            float s = acc[kt][r] * scale;
-            if (bias != nullptr) s += bias_l[col * kTilePad + kk];
-            if (kt * 32 + kk >= S) s = -INFINITY;
-            acc[kt][r] = s;
-            m = fmaxf(m, s);
+            const int key = kt * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+            float x = sc[r] * scale;
+            const bool ok = key < S && qi < S;
+            if (bias != nullptr && ok) x += bf2f(brow[key]);
+            if (!ok) x = -INFINITY;
+            sc[r] = x;
+            tmax = fmaxf(tmax, x);
         }
-        __syncthreads();
-    }
-    m = fmaxf(m, __shfl_xor(m, 32));
-    if (m == -INFINITY) m = 0.f;
-    float l = 0.f;
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+        const float m_new = fmaxf(m, tmax);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = __expf(m - m_use);
+        l *= alpha;
 #pragma unroll
-    for (int kt = 0; kt < NT; ++kt)
+        for (int r = 0; r < 4 * KS; ++r) o[r] *= alpha;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const float p = __expf(acc[kt][r] - m);
-            acc[kt][r] = p;
-            l += p;
+            const float pv = __expf(sc[r] - m_use);
+            sc[r] = pv;
+            l += pv;
         }
-    l += __shfl_xor(l, 32);
-    // O^T = V^T P^T
-    float16_t o = zero16();
-#pragma unroll
-    for (int kt = 0; kt < NT; ++kt)
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             short4_t pb;
-            pb.x = f2bf(acc[kt][4 * t + 0]); pb.y = f2bf(acc[kt][4 * t + 1]);
-            pb.z = f2bf(acc[kt][4 * t + 2]); pb.w = f2bf(acc[kt][4 * t + 3]);
+            pb.x = f2bf(sc[4 * t + 0]); pb.y = f2bf(sc[4 * t + 1]);
+            pb.z = f2bf(sc[4 * t + 2]); pb.w = f2bf(sc[4 * t + 3]);
             short4_t av = zero4();
             if (col < D) av = *reinterpret_cast<const short4_t*>(&v_tr[col * (SP + 4) + kt * 32 + t * 8 + half * 4]);
-            o = mfma(av, pb, o);
+            o = mfma(av, pb, o);        // O^T += V^T P^T
         }
+        m = m_new;
+    }
+    l += __shfl_xor(l, 32);
     if (qi < S) {
         const float inv = 1.0f / l;
         T* op = out + (((int64_t)g * S + qi) * H + h) * D;
@@ -197,23 +250,25 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
         for (int rb = 0; rb < KS; ++rb)
             st4(op + 8 * rb + 4 * half, o[4 * rb + 0] * inv, o[4 * rb + 1] * inv, o[4 * rb + 2] * inv,
                 o[4 * rb + 3] * inv);
-        if (half == 0) lse[((int64_t)g * H + h) * S + qi] = m + __logf(l);
+        if (half == 0) lse[((int64_t)g * H + h) * S + qi] = (m == -INFINITY ? 0.f : m) + __logf(l);
     }
 }
 
 // ---------------------------------------------------------------------------
 // backward
 // ---------------------------------------------------------------------------
-// Wave w first acts on query tile w (transposed scores, lane = query): dQ and the
-// per-query D = dout . out.  Then on key tile w (direct scores, lane = key): dK, dV
-// and dBias, with coalesced bias reads and dBias writes.
+// Wave w first acts on query tile w (transposed scores, lane = query): dQ.  Then
+// on key tile w (direct scores, lane = key): dK, dV and dBias.  The bias is read
+// from HBM once: every wave stages its strip, and the second phase reads all
+// strips from LDS.
 template <typename T, int D, int NT>
 __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, const T* __restrict__ K,
                                                        const T* __restrict__ V, const T* __restrict__ bias,
                                                        const T* __restrict__ O, const float* __restrict__ lse,
                                                        const T* __restrict__ dO, T* __restrict__ dQ,
                                                        T* __restrict__ dK, T* __restrict__ dV,
-                                                       T* __restrict__ dbias, int S, int H, float scale) {
+                                                       T* __restrict__ dbias, int S, int H, float scale,
+                                                       int64_t bias_total) {
     constexpr int KS = D / 8;
     constexpr int SP = NT * 32;
     extern __shared__ __align__(16) char smem[];
@@ -225,32 +280,40 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
     short* q_tr = g_rm + RM;
     short* k_tr = q_tr + TR;
     short* g_tr = k_tr + TR;
-    float* lse_l = reinterpret_cast<float*>(g_tr + TR);
+    short* strips = g_tr + TR;
+    float* lse_l = reinterpret_cast<float*>(strips + NT * strip_elems<SP>());
     float* dd_l = lse_l + SP;
+    int* heads = reinterpret_cast<int*>(dd_l + SP);
     const int g = blockIdx.x / H, h = blockIdx.x % H;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int col = lane & 31, half = lane >> 5;
-    float* bias_l = dd_l + SP + wave * 32 * kTilePad;
+    if (bias != nullptr) {
+        const int q0 = wave * 32;
+        const int rows = min(32, S - q0);
+        const int hd = stage_strip<T>(bias, (((int64_t)g * H + h) * S + q0) * S, rows * S, S, bias_total,
+                                      strips + wave * strip_elems<SP>(), lane);
+        if (lane == 0) heads[wave] = hd;
+    }
     load_head<T, D, SP>(Q, g, h, S, H, q_rm, q_tr);
     load_head<T, D, SP>(K, g, h, S, H, k_rm, k_tr);
     load_head<T, D, SP>(V, g, h, S, H, v_rm, nullptr);
     load_head<T, D, SP>(dO, g, h, S, H, g_rm, g_tr);
-    for (int i = threadIdx.x; i < SP; i += blockDim.x)
-        lse_l[i] = i < S ? lse[((int64_t)g * H + h) * S + i] : 0.f;
-    // D[q] = sum_dd dout[q,dd] out[q,dd]
     for (int i = threadIdx.x; i < SP; i += blockDim.x) {
-        float dsum = 0.f;
+        float dsum = 0.f, L = 0.f;
         if (i < S) {
+            L = lse[((int64_t)g * H + h) * S + i];
             const T* op = O + (((int64_t)g * S + i) * H + h) * D;
+            const T* gp = dO + (((int64_t)g * S + i) * H + h) * D;
 #pragma unroll
             for (int c = 0; c < D; c += 4) {
                 const short4_t ov = ld4(op + c);
-                const short4_t gv = ld4(dO + (((int64_t)g * S + i) * H + h) * D + c);
+                const short4_t gv = ld4(gp + c);
                 dsum += bf2f(ov.x) * bf2f(gv.x) + bf2f(ov.y) * bf2f(gv.y) + bf2f(ov.z) * bf2f(gv.z) +
                         bf2f(ov.w) * bf2f(gv.w);
             }
         }
-        dd_l[i] = dsum;
+        lse_l[i] = L;
+        dd_l[i] = dsum;          // D[q] = sum_dd dout[q,dd] out[q,dd]
     }
     __syncthreads();
 
@@ -264,8 +327,9 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
             bg[s] = *reinterpret_cast<const short4_t*>(&g_rm[qi * D + s * 8 + half * 4]);
         }
         const float L = lse_l[qi], Dq = dd_l[qi];
+        const short* brow = strips + wave * strip_elems<SP>() + (bias != nullptr ? heads[wave] : 0) + col * strip_stride(S);
         float16_t dq = zero16();
-#pragma unroll
+#pragma unroll 1
         for (int kt = 0; kt < NT; ++kt) {
             float16_t sc = zero16(), dp = zero16();
 #pragma unroll
@@ -275,27 +339,15 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
                 sc = mfma(ak, bq[s], sc);     // S^T[key, query]
                 dp = mfma(av, bg[s], dp);     // dP^T[key, query] = V dout^T
             }
-            if (bias != nullptr) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int row = r * 2 + half, key = kt * 32 + col;
-                    float bv = 0.f;
-                    if (q0 + row < S && key < S)
-                        bv = ld1(bias + (((int64_t)g * H + h) * S + q0 + row) * S + key);
-                    bias_l[row * kTilePad + col] = bv;
-                }
-            }
-            __syncthreads();
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int kk = 8 * (r / 4) + 4 * half + (r % 4);
-                float s = sc[r] * scale;
-                if (bias != nullptr) s += bias_l[col * kTilePad + kk];
-                float p = __expf(s - L);
-                if (kt * 32 + kk >= S || qi >= S) p = 0.f;
-                sc[r] = p * (dp[r] - Dq);      // dS^T
+                const int key = kt * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+                const bool ok = key < S && qi < S;
+                float x = sc[r] * scale;
+                if (bias != nullptr && ok) x += bf2f(brow[key]);
+                const float pv = ok ? __expf(x - L) : 0.f;
+                sc[r] = pv * (dp[r] - Dq);    // dS^T
             }
-            __syncthreads();
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
                 short4_t db;
@@ -325,7 +377,7 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
             bv[s] = *reinterpret_cast<const short4_t*>(&v_rm[ki * D + s * 8 + half * 4]);
         }
         float16_t dk = zero16(), dv = zero16();
-#pragma unroll
+#pragma unroll 1
         for (int qt = 0; qt < NT; ++qt) {
             float16_t sc = zero16(), dp = zero16();
 #pragma unroll
@@ -335,17 +387,20 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
                 sc = mfma(aq, bk[s], sc);     // S[query, key]
                 dp = mfma(ag, bv[s], dp);     // dP[query, key] = dout V^T
             }
+            const short* bt = strips + qt * strip_elems<SP>() + (bias != nullptr ? heads[qt] : 0) + ki;
+            const int SL = strip_stride(S);
             float pr[16];
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int qq = qt * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-                float s = sc[r] * scale;
+                const int qr = 8 * (r / 4) + 4 * half + (r % 4);
+                const int qq = qt * 32 + qr;
                 const bool ok = qq < S && ki < S;
-                if (bias != nullptr && ok) s += ld1(bias + (((int64_t)g * H + h) * S + qq) * S + ki);
-                float p = ok ? __expf(s - lse_l[qq]) : 0.f;
-                const float ds = p * (dp[r] - dd_l[qq]);
+                float x = sc[r] * scale;
+                if (bias != nullptr && ok) x += bf2f(bt[qr * SL]);
+                const float pv = ok ? __expf(x - lse_l[qq]) : 0.f;
+                const float ds = pv * (dp[r] - dd_l[qq]);
                 if (dbias != nullptr && ok) st1(dbias + (((int64_t)g * H + h) * S + qq) * S + ki, ds);
-                pr[r] = p;
+                pr[r] = pv;
                 sc[r] = ds;
             }
 #pragma unroll
@@ -391,32 +446,38 @@ struct DenseCall {
 
 template <typename T, int D, int NT>
 static int launch_dense(const DenseCall& c, bool bwd) {
-    const float scale = sqrtf((float)c.d);     // the reference MULTIPLIES q by sqrt(d)
-    const dim3 grid((unsigned)(c.b * c.H)), block(64 * NT);
     constexpr int lds_f = fwd_lds_bytes<D, NT>(), lds_b = bwd_lds_bytes<D, NT>();
-    static_assert(lds_b <= 160 * 1024, "backward LDS image exceeds the 160 KB of a CU");
-    static bool attr_done = false;     // raise the dynamic-LDS cap once per instantiation
-    if (!attr_done) {
-        if (lds_f > 48 * 1024)
-            TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_dense_fwd<T, D, NT>),
-                                              hipFuncAttributeMaxDynamicSharedMemorySize, lds_f));
-        if (lds_b > 48 * 1024)
-            TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_dense_bwd<T, D, NT>),
-                                              hipFuncAttributeMaxDynamicSharedMemorySize, lds_b));
-        attr_done = true;
-    }
-    if (!bwd) {
-        KernelTimer t(KS_DENSE_FWD, c.st);
-        hipLaunchKernelGGL((k_dense_fwd<T, D, NT>), grid, block, lds_f, c.st, (const T*)c.q, (const T*)c.k,
-                           (const T*)c.v, (const T*)c.bias, (T*)c.o_out, c.o_lse, c.S, c.H, scale);
+    if constexpr (lds_f > kLdsLimit || lds_b > kLdsLimit) {
+        set_error("dense attention: S=%d with head dim %d needs %d bytes of LDS (limit %d)", c.S, c.d,
+                  lds_b > lds_f ? lds_b : lds_f, kLdsLimit);
+        return TGT_ERR_UNSUPPORTED;
     } else {
-        KernelTimer t(KS_DENSE_BWD, c.st);
-        hipLaunchKernelGGL((k_dense_bwd<T, D, NT>), grid, block, lds_b, c.st, (const T*)c.q, (const T*)c.k,
-                           (const T*)c.v, (const T*)c.bias, (const T*)c.out, c.lse, (const T*)c.dout, (T*)c.dq,
-                           (T*)c.dk, (T*)c.dv, (T*)c.dbias, c.S, c.H, scale);
+        const float scale = sqrtf((float)c.d);     // the reference MULTIPLIES q by sqrt(d)
+        const dim3 grid((unsigned)(c.b * c.H)), block(64 * NT);
+        const int64_t bias_total = (int64_t)c.b * c.H * c.S * c.S;
+        static bool attr_done = false;     // raise the dynamic-LDS cap once per instantiation
+        if (!attr_done) {
+            if (lds_f > 48 * 1024)
+                TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_dense_fwd<T, D, NT>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_f));
+            if (lds_b > 48 * 1024)
+                TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_dense_bwd<T, D, NT>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_b));
+            attr_done = true;
+        }
+        if (!bwd) {
+            KernelTimer t(KS_DENSE_FWD, c.st);
+            hipLaunchKernelGGL((k_dense_fwd<T, D, NT>), grid, block, lds_f, c.st, (const T*)c.q, (const T*)c.k,
+                               (const T*)c.v, (const T*)c.bias, (T*)c.o_out, c.o_lse, c.S, c.H, scale, bias_total);
+        } else {
+            KernelTimer t(KS_DENSE_BWD, c.st);
+            hipLaunchKernelGGL((k_dense_bwd<T, D, NT>), grid, block, lds_b, c.st, (const T*)c.q, (const T*)c.k,
+                               (const T*)c.v, (const T*)c.bias, (const T*)c.out, c.lse, (const T*)c.dout,
+                               (T*)c.dq, (T*)c.dk, (T*)c.dv, (T*)c.dbias, c.S, c.H, scale, bias_total);
+        }
+        TGT_HIP_CHECK(hipGetLastError());
+        return TGT_OK;
     }
-    TGT_HIP_CHECK(hipGetLastError());
-    return TGT_OK;
 }
 
 template <typename T, int D>
