@@ -161,7 +161,10 @@ def bench_dense(args):
                    "b": b, "S": S, "H": H, "d": d, "bias": "[b,H,S,S] with gradient, -inf on padded keys",
                    "step": "tgt_dense_attn_fwd + tgt_dense_attn_bwd", "parallelism": "1 GPU"},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": gbs / HBM_PEAK_GBS, "traffic": None, "alg_bytes": alg[dom],
+                     "frac": gbs / HBM_PEAK_GBS,
+                     # rocprofv3 FETCH_SIZE x2.000 + WRITE_SIZE x1.000, profiles/dense_attn_config4_bf16.txt
+                     "traffic": {"dense_fwd": 86.3e6, "dense_bwd": 171.4e6}.get(dom) if args.dtype == "bf16" else None,
+                     "alg_bytes": alg[dom],
                      "avg_us": kernels[dom]["avg_us"]},
         "mfma": {n: {"alg_tflops": flops[n] / (kernels[n]["avg_us"] * 1e-6) / 1e12, "peak_tflops": 2500.0}
                  for n in kernels},

@@ -171,13 +171,18 @@ template <typename T, int D, int NT>
 __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, const T* __restrict__ K,
                                                        const T* __restrict__ V, const T* __restrict__ bias,
                                                        T* __restrict__ out, float* __restrict__ lse, int S,
-                                                       int H, float scale, int64_t bias_total) {
+                                                       int H, float scale, int64_t bias_total, int nb) {
     constexpr int KS = D / 8;
     constexpr int SP = NT * 32;
     extern __shared__ __align__(16) char smem[];
     short* k_rm = reinterpret_cast<short*>(smem);
     short* v_tr = k_rm + rm_elems<D, SP>();
-    const int g = blockIdx.x / H, h = blockIdx.x % H;
+    // XCD-aware placement: workgroups go to the 8 XCDs round-robin, and the H heads of a graph
+    // share every 128-byte line of q/k/v ([b,S,H,d] layout), so the heads of graph g are given the
+    // workgroup ids congruent to g mod 8 inside a window of 8*H ids - same XCD, same L2, same time.
+    const int win = blockIdx.x / (8 * H), rem = blockIdx.x % (8 * H);
+    const int g = win * 8 + (rem & 7), h = rem >> 3;
+    if (g >= nb) return;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int col = lane & 31, half = lane >> 5;
     short* strip = v_tr + tr_elems<D, SP>() + wave * strip_elems<SP>();
@@ -268,7 +273,7 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
                                                        const T* __restrict__ dO, T* __restrict__ dQ,
                                                        T* __restrict__ dK, T* __restrict__ dV,
                                                        T* __restrict__ dbias, int S, int H, float scale,
-                                                       int64_t bias_total) {
+                                                       int64_t bias_total, int nb) {
     constexpr int KS = D / 8;
     constexpr int SP = NT * 32;
     extern __shared__ __align__(16) char smem[];
@@ -284,7 +289,12 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
     float* lse_l = reinterpret_cast<float*>(strips + NT * strip_elems<SP>());
     float* dd_l = lse_l + SP;
     int* heads = reinterpret_cast<int*>(dd_l + SP);
-    const int g = blockIdx.x / H, h = blockIdx.x % H;
+    // XCD-aware placement: workgroups go to the 8 XCDs round-robin, and the H heads of a graph
+    // share every 128-byte line of q/k/v ([b,S,H,d] layout), so the heads of graph g are given the
+    // workgroup ids congruent to g mod 8 inside a window of 8*H ids - same XCD, same L2, same time.
+    const int win = blockIdx.x / (8 * H), rem = blockIdx.x % (8 * H);
+    const int g = win * 8 + (rem & 7), h = rem >> 3;
+    if (g >= nb) return;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int col = lane & 31, half = lane >> 5;
     if (bias != nullptr) {
@@ -453,7 +463,7 @@ static int launch_dense(const DenseCall& c, bool bwd) {
         return TGT_ERR_UNSUPPORTED;
     } else {
         const float scale = sqrtf((float)c.d);     // the reference MULTIPLIES q by sqrt(d)
-        const dim3 grid((unsigned)(c.b * c.H)), block(64 * NT);
+        const dim3 grid((unsigned)(((c.b + 7) / 8) * 8 * c.H)), block(64 * NT);
         const int64_t bias_total = (int64_t)c.b * c.H * c.S * c.S;
         static bool attr_done = false;     // raise the dynamic-LDS cap once per instantiation
         if (!attr_done) {
@@ -468,12 +478,12 @@ static int launch_dense(const DenseCall& c, bool bwd) {
         if (!bwd) {
             KernelTimer t(KS_DENSE_FWD, c.st);
             hipLaunchKernelGGL((k_dense_fwd<T, D, NT>), grid, block, lds_f, c.st, (const T*)c.q, (const T*)c.k,
-                               (const T*)c.v, (const T*)c.bias, (T*)c.o_out, c.o_lse, c.S, c.H, scale, bias_total);
+                               (const T*)c.v, (const T*)c.bias, (T*)c.o_out, c.o_lse, c.S, c.H, scale, bias_total, c.b);
         } else {
             KernelTimer t(KS_DENSE_BWD, c.st);
             hipLaunchKernelGGL((k_dense_bwd<T, D, NT>), grid, block, lds_b, c.st, (const T*)c.q, (const T*)c.k,
                                (const T*)c.v, (const T*)c.bias, (const T*)c.out, c.lse, (const T*)c.dout,
-                               (T*)c.dq, (T*)c.dk, (T*)c.dv, (T*)c.dbias, c.S, c.H, scale, bias_total);
+                               (T*)c.dq, (T*)c.dk, (T*)c.dv, (T*)c.dbias, c.S, c.H, scale, bias_total, c.b);
         }
         TGT_HIP_CHECK(hipGetLastError());
         return TGT_OK;
