@@ -16,6 +16,7 @@
 // walked by whole workgroups in segments of kBlockSeg edges whose partial sums the
 // last-arriving workgroup adds in a fixed order.
 #include "common.h"
+#include <stdlib.h>
 
 namespace tgt {
 
@@ -95,6 +96,7 @@ struct Common {
     const void* bias;
     const float2* nd;     // [N, H] (1/(Z+eps), D) (backward)
     int32_t bias_mode;
+    int32_t bias_se, bias_sh;   // element strides of the bias per edge / per head: (H, 1) or (1, 0)
     float inv_scale;
 };
 
@@ -111,9 +113,12 @@ struct SideArgs {
     float* part;          // partial sums of split rows
     int32_t* counters;    // one arrival counter per split row, zero between calls
     int32_t n_block_items;
-    int32_t n_wave_blocks;
-    int32_t class_off[kNumClass + 1];
-    int32_t wave_off[kNumClass + 1];
+    int32_t n_wave_blocks;               // multiple of 8
+    int32_t class_off[kNumClass + 1];    // item index where each wave class begins
+    int32_t nwaves[kNumClass];           // waves of each class
+    int32_t chunk[kNumClass];            // waves of each class given to one XCD (ceil(nwaves / 8))
+    int32_t voff[kNumClass + 1];         // prefix sums of chunk: wave slots of one XCD
+    int32_t interleave;                  // experiment switch: XCD x takes waves x, x+8, ... instead of a chunk
 };
 
 struct Acc {
@@ -131,7 +136,7 @@ __host__ __device__ constexpr int part_stride() {
 // Walks `len` edges starting at sorted position `start` of node `row` with S edge
 // slots (this lane is slot `slot`, element chunk `el`).  On return every lane of
 // the S*LPE-lane group holds the sums over all S slots.
-template <typename T, int LPE, int LPH, int S, int MODE>
+template <typename T, int LPE, int LPH, int S, int MODE, bool HASB>
 __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, const int row, const int start,
                                            const int len, const int slot, const int el, const bool valid,
                                            Acc& acc) {
@@ -166,7 +171,7 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
     }
     const int32_t* __restrict__ col = s.col + start;
     const int32_t* __restrict__ eid = s.eid + start;
-    const int bias_mode = c.bias_mode;
+    const int bias_se = c.bias_se, bias_sh = c.bias_sh;
     const float inv_scale = c.inv_scale;
     const int n = valid ? len : 0;
 
@@ -183,7 +188,7 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
             nb[u] = 0; ed[u] = 0;
             if (ok[u]) {
                 nb[u] = col[e];
-                if (bias_mode != TGT_BIAS_NONE) ed[u] = eid[e];
+                if (HASB) ed[u] = eid[e];
             }
         }
 #pragma unroll
@@ -202,8 +207,7 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
                     load8(K + o, x0[u]);
                     load8(V + o, x1[u]);
                 }
-                if (bias_mode == TGT_BIAS_EDGE_HEAD) bb[u] = load1(B + (int64_t)ed[u] * H + head);
-                else if (bias_mode == TGT_BIAS_EDGE) bb[u] = load1(B + ed[u]);
+                if (HASB) bb[u] = load1(B + (int64_t)ed[u] * bias_se + head * bias_sh);
             }
         }
 #pragma unroll
@@ -212,7 +216,7 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
                 // raw score: identical arithmetic in all three walks so that the
                 // recomputed weights and the clamp mask agree bit for bit
                 const float raw = head_sum<LPH>(dot8(r0, x0[u])) * inv_scale;
-                const float w = expf(clamp5(raw) + bb[u]);
+                const float w = __expf(clamp5(raw) + bb[u]);
                 if (MODE == MODE_FWD) {
                     acc.z += w;
 #pragma unroll
@@ -223,10 +227,10 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
                         const float t = head_sum<LPH>(dot8(r1, x1[u]));   // g_dst . v_src
                         const float dS = w * rz * (t - Dh);
                         T* __restrict__ dB = static_cast<T*>(s.out1);
-                        if (dB != nullptr) {
-                            if (bias_mode == TGT_BIAS_EDGE_HEAD) {
+                        if (HASB && dB != nullptr) {
+                            if (bias_sh != 0) {       // one value per edge and head
                                 if (el % LPH == 0) store1(dB + (int64_t)ed[u] * H + head, dS);
-                            } else if (bias_mode == TGT_BIAS_EDGE) {
+                            } else {                  // one value per edge: sum over heads
                                 float t2 = dS;   // sum over heads; every head is held by LPH lanes
 #pragma unroll
                                 for (int off = 1; off < LPE; off <<= 1) t2 += __shfl_xor(t2, off);
@@ -285,7 +289,7 @@ __device__ __forceinline__ void write_row(const Common& c, const SideArgs& s, co
 }
 
 // Wave items: rows of at most kWaveRowMax edges, 64 / (LPE*S) rows per wave.
-template <typename T, int LPE, int LPH, int S, int MODE>
+template <typename T, int LPE, int LPH, int S, int MODE, bool HASB>
 __device__ __forceinline__ void wave_items(const Common& c, const SideArgs& s, const int item_begin,
                                            const int item_end, const int wave_in_class) {
     constexpr int G = LPE * S;
@@ -298,26 +302,34 @@ __device__ __forceinline__ void wave_items(const Common& c, const SideArgs& s, c
     Item it{0, 0, 0, -1};
     if (valid) it = s.items[item];
     Acc acc;
-    walk_range<T, LPE, LPH, S, MODE>(c, s, it.row, it.start, it.len, slot, el, valid, acc);
+    walk_range<T, LPE, LPH, S, MODE, HASB>(c, s, it.row, it.start, it.len, slot, el, valid, acc);
     if (valid && slot == 0) write_row<T, LPE, LPH, MODE>(c, s, it.row, el, acc);
 }
 
-template <typename T, int LPE, int LPH, int MODE>
+// Wave items, XCD-aware.  Workgroups go to the 8 XCDs round-robin (workgroup id mod 8), each
+// XCD has its own L2, and neighbouring rows tend to share sources (clustered / reordered
+// graphs).  So every class's waves are cut into 8 contiguous chunks and XCD x walks chunk x of
+// every class, longest class first: rows that are neighbours in the schedule meet in one L2.
+// `block` counts from the start of this view's wave region, which begins at a workgroup id
+// that is a multiple of 8.
+template <typename T, int LPE, int LPH, int MODE, bool HASB>
 __device__ __forceinline__ void wave_block(const Common& c, const SideArgs& s, const int block) {
-    const int gw = block * (kBlock / kWave) + (threadIdx.x >> 6);
+    const int xcd = block & 7;
+    const int v = (block >> 3) * (kBlock / kWave) + (threadIdx.x >> 6);   // wave slot inside the XCD
     int cls = 0;
 #pragma unroll
-    for (int k = 1; k < kNumClass; ++k) cls += (gw >= s.wave_off[k]) ? 1 : 0;
+    for (int k = 1; k < kNumClass; ++k) cls += (v >= s.voff[k]) ? 1 : 0;
     cls = __builtin_amdgcn_readfirstlane(cls);
-    if (gw >= s.wave_off[kNumClass]) return;
-    const int w = gw - s.wave_off[cls];
+    if (v >= s.voff[kNumClass]) return;
+    const int w = s.interleave ? (v - s.voff[cls]) * 8 + xcd : xcd * s.chunk[cls] + (v - s.voff[cls]);
+    if (w >= s.nwaves[cls]) return;
     const int b = s.class_off[cls], e = s.class_off[cls + 1];
     switch (cls) {
-        case 0: wave_items<T, LPE, LPH, slots_for_class(LPE, 0), MODE>(c, s, b, e, w); break;
-        case 1: wave_items<T, LPE, LPH, slots_for_class(LPE, 1), MODE>(c, s, b, e, w); break;
-        case 2: wave_items<T, LPE, LPH, slots_for_class(LPE, 2), MODE>(c, s, b, e, w); break;
-        case 3: wave_items<T, LPE, LPH, slots_for_class(LPE, 3), MODE>(c, s, b, e, w); break;
-        default: wave_items<T, LPE, LPH, slots_for_class(LPE, 4), MODE>(c, s, b, e, w); break;
+        case 0: wave_items<T, LPE, LPH, slots_for_class(LPE, 0), MODE, HASB>(c, s, b, e, w); break;
+        case 1: wave_items<T, LPE, LPH, slots_for_class(LPE, 1), MODE, HASB>(c, s, b, e, w); break;
+        case 2: wave_items<T, LPE, LPH, slots_for_class(LPE, 2), MODE, HASB>(c, s, b, e, w); break;
+        case 3: wave_items<T, LPE, LPH, slots_for_class(LPE, 3), MODE, HASB>(c, s, b, e, w); break;
+        default: wave_items<T, LPE, LPH, slots_for_class(LPE, 4), MODE, HASB>(c, s, b, e, w); break;
     }
 }
 
@@ -338,7 +350,7 @@ struct BlockLds {
 // slot, and the workgroup that arrives last adds the slots in slot order and
 // writes the row - no second launch, no floating-point atomics, and the order of
 // the additions does not depend on which workgroup is last.
-template <typename T, int LPE, int LPH, int MODE>
+template <typename T, int LPE, int LPH, int MODE, bool HASB>
 __device__ __forceinline__ void block_item(const Common& c, const SideArgs& s, const int item,
                                            BlockLds<LPE>& lds) {
     constexpr int S = slots_for_class(LPE, 0);
@@ -360,7 +372,7 @@ __device__ __forceinline__ void block_item(const Common& c, const SideArgs& s, c
     const int lo = min(grp * share, it.len);
     const int hi = min(lo + share, it.len);
     Acc acc;
-    walk_range<T, LPE, LPH, S, MODE>(c, s, it.row, it.start + lo, hi - lo, slot, el, true, acc);
+    walk_range<T, LPE, LPH, S, MODE, HASB>(c, s, it.row, it.start + lo, hi - lo, slot, el, true, acc);
     if (slot == 0) {
         float* r = lds.red + grp * STRIDE;
 #pragma unroll
@@ -457,28 +469,32 @@ __device__ __forceinline__ void block_item(const Common& c, const SideArgs& s, c
 
 // Forward: workgroup items of the destination view first (longest work first),
 // then its wave items.
-template <typename T, int LPE, int LPH>
-__global__ __launch_bounds__(kBlock) void k_attn_fwd(const Common c, const SideArgs s) {
+template <typename T, int LPE, int LPH, bool HASB>
+__global__ __launch_bounds__(kBlock) void k_attn_fwd(const Common c, const SideArgs s, const int items_pad) {
     __shared__ BlockLds<LPE> lds;
     const int b = blockIdx.x;
-    if (b < s.n_block_items) block_item<T, LPE, LPH, MODE_FWD>(c, s, b, lds);
-    else wave_block<T, LPE, LPH, MODE_FWD>(c, s, b - s.n_block_items);
+    if (b < s.n_block_items) block_item<T, LPE, LPH, MODE_FWD, HASB>(c, s, b, lds);
+    else if (b >= items_pad) wave_block<T, LPE, LPH, MODE_FWD, HASB>(c, s, b - items_pad);
 }
 
 // Backward: both views in one launch (they are independent once nd is known):
 // workgroup items of the destination view, workgroup items of the source view,
 // wave items of the destination view, wave items of the source view.
-template <typename T, int LPE, int LPH>
-__global__ __launch_bounds__(kBlock) void k_attn_bwd(const Common c, const SideArgs sd, const SideArgs ss) {
+template <typename T, int LPE, int LPH, bool HASB>
+__global__ __launch_bounds__(kBlock) void k_attn_bwd(const Common c, const SideArgs sd, const SideArgs ss,
+                                                     const int items_pad) {
     __shared__ BlockLds<LPE> lds;
     int b = blockIdx.x;
-    if (b < sd.n_block_items) { block_item<T, LPE, LPH, MODE_BWD_DST>(c, sd, b, lds); return; }
-    b -= sd.n_block_items;
-    if (b < ss.n_block_items) { block_item<T, LPE, LPH, MODE_BWD_SRC>(c, ss, b, lds); return; }
-    b -= ss.n_block_items;
-    if (b < sd.n_wave_blocks) { wave_block<T, LPE, LPH, MODE_BWD_DST>(c, sd, b); return; }
+    if (b < sd.n_block_items) { block_item<T, LPE, LPH, MODE_BWD_DST, HASB>(c, sd, b, lds); return; }
+    if (b < sd.n_block_items + ss.n_block_items) {
+        block_item<T, LPE, LPH, MODE_BWD_SRC, HASB>(c, ss, b - sd.n_block_items, lds);
+        return;
+    }
+    if (b < items_pad) return;     // padding: the wave regions start at a multiple of 8
+    b -= items_pad;
+    if (b < sd.n_wave_blocks) { wave_block<T, LPE, LPH, MODE_BWD_DST, HASB>(c, sd, b); return; }
     b -= sd.n_wave_blocks;
-    wave_block<T, LPE, LPH, MODE_BWD_SRC>(c, ss, b);
+    wave_block<T, LPE, LPH, MODE_BWD_SRC, HASB>(c, ss, b);
 }
 
 // Per-node side vector of the backward: nd[i,h] = (1 / (Z[i,h] + eps), sum_c dout[i,h,c] out[i,h,c]).
@@ -530,18 +546,23 @@ static void fill_side(SideArgs& a, const Side& s, int lpe) {
     a.items = s.items; a.col = s.col; a.eid = s.eid;
     a.split_off = s.split_off; a.part2split = s.part2split;
     a.n_block_items = s.n_block_items;
-    int waves = 0;
+    int slots = 0;
     for (int c = 0; c < kNumClass; ++c) {
         a.class_off[c] = s.class_off[c];
-        a.wave_off[c] = waves;
         const int ipw = kWave / (lpe * slots_for_class(lpe, c));
         const int n = s.class_off[c + 1] - s.class_off[c];
-        waves += (n + ipw - 1) / ipw;
+        a.nwaves[c] = (n + ipw - 1) / ipw;
+        a.chunk[c] = (a.nwaves[c] + 7) / 8;
+        a.voff[c] = slots;
+        slots += a.chunk[c];
     }
     a.class_off[kNumClass] = s.class_off[kNumClass];
-    a.wave_off[kNumClass] = waves;
-    a.n_wave_blocks = (waves + (kBlock / kWave) - 1) / (kBlock / kWave);
+    a.voff[kNumClass] = slots;
+    a.n_wave_blocks = 8 * ((slots + (kBlock / kWave) - 1) / (kBlock / kWave));
+    const char* il = getenv("TGT_XCD_INTERLEAVE");
+    a.interleave = (il && il[0] == '1') ? 1 : 0;
 }
+static inline int pad8(int x) { return (x + 7) & ~7; }
 
 struct Call {
     const tgt_plan* plan;
@@ -561,16 +582,22 @@ static int run_fwd(const Call& c) {
     Common cm{};
     cm.q = c.q; cm.k = c.k; cm.v = c.v; cm.g = nullptr; cm.bias = c.bias; cm.nd = nullptr;
     cm.bias_mode = c.bias_mode;
+    cm.bias_se = c.bias_mode == TGT_BIAS_EDGE_HEAD ? c.H : 1;
+    cm.bias_sh = c.bias_mode == TGT_BIAS_EDGE_HEAD ? 1 : 0;
     cm.inv_scale = 1.0f / sqrtf((float)c.d);
     SideArgs a{};
     fill_side(a, c.plan->dst, LPE);
     a.out0 = c.o_out; a.out1 = nullptr; a.Z = c.o_Z;
     a.part = reinterpret_cast<float*>(c.ws + L.fwd_part);
     a.counters = reinterpret_cast<int32_t*>(c.ws + L.counters);
-    const int nb = a.n_block_items + a.n_wave_blocks;
+    const int items_pad = pad8(a.n_block_items);
+    const int nb = items_pad + a.n_wave_blocks;
     if (nb > 0) {
         KernelTimer t(KS_FWD, c.st);
-        hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH>), dim3(nb), dim3(kBlock), 0, c.st, cm, a);
+        if (c.bias_mode != TGT_BIAS_NONE)
+            hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
+        else
+            hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
     }
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
@@ -591,6 +618,8 @@ static int run_bwd(const Call& c) {
     Common cm{};
     cm.q = c.q; cm.k = c.k; cm.v = c.v; cm.g = c.dout; cm.bias = c.bias; cm.nd = nd;
     cm.bias_mode = c.bias_mode;
+    cm.bias_se = c.bias_mode == TGT_BIAS_EDGE_HEAD ? c.H : 1;
+    cm.bias_sh = c.bias_mode == TGT_BIAS_EDGE_HEAD ? 1 : 0;
     cm.inv_scale = 1.0f / sqrtf((float)c.d);
     int32_t* counters = reinterpret_cast<int32_t*>(c.ws + L.counters);
     SideArgs sd{}, ss{};
@@ -602,10 +631,14 @@ static int run_bwd(const Call& c) {
     ss.out0 = c.dk; ss.out1 = c.dv; ss.Z = nullptr;
     ss.part = reinterpret_cast<float*>(c.ws + L.dkv_part);
     ss.counters = counters + 2 * c.plan->dst.n_split;
-    const int nb = sd.n_block_items + ss.n_block_items + sd.n_wave_blocks + ss.n_wave_blocks;
+    const int items_pad = pad8(sd.n_block_items + ss.n_block_items);
+    const int nb = items_pad + sd.n_wave_blocks + ss.n_wave_blocks;
     if (nb > 0) {
         KernelTimer t(KS_BWD, c.st);
-        hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss);
+        if (c.bias_mode != TGT_BIAS_NONE)
+            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, items_pad);
+        else
+            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, items_pad);
     }
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;

@@ -110,33 +110,73 @@ def spd_edge_ids(edge_index, clamp=5):
 
 
 def stochastic_block_model(n_clusters=64, cluster_size=4096, p_intra=0.004, inter_fraction=0.05, seed=42):
-    """Config 5: nodes ordered contiguously by cluster, one DIRECTED edge per
-    sampled ordered pair; intra-cluster pairs with probability p_intra, plus
-    inter-cluster edges amounting to ``inter_fraction`` of the total.  No global
-    node, no self-loops.  Returns (edge_index, N, cluster_of_node)."""
+    """Config 5: nodes ordered contiguously by cluster.  Every UNORDERED intra-cluster pair is
+    sampled with probability p_intra and becomes ONE directed edge with a random direction;
+    inter-cluster edges (random ordered pairs of different clusters) make up ``inter_fraction``
+    of the total.  No global node, no self-loops.  Returns (edge_index, N, cluster_of_node)."""
     rng = np.random.default_rng(seed)
     n = n_clusters * cluster_size
     srcs, dsts = [], []
-    per = cluster_size * cluster_size
+    pairs = cluster_size * (cluster_size - 1) // 2
     for c in range(n_clusters):
-        m = rng.binomial(per, p_intra)
-        flat = np.unique(rng.integers(0, per, size=int(m * 1.02), dtype=np.int64))[:m]
-        a, b = flat // cluster_size, flat % cluster_size
+        m = rng.binomial(pairs, p_intra)
+        # sample m distinct unordered pairs by rejection on ordered draws
+        a = rng.integers(0, cluster_size, size=int(m * 1.05) + 16, dtype=np.int64)
+        b = rng.integers(0, cluster_size, size=a.shape[0], dtype=np.int64)
         keep = a != b
-        srcs.append(a[keep] + c * cluster_size)
-        dsts.append(b[keep] + c * cluster_size)
+        lo, hi = np.minimum(a[keep], b[keep]), np.maximum(a[keep], b[keep])
+        _, first = np.unique(lo * cluster_size + hi, return_index=True)
+        first = np.sort(first)[:m]
+        lo, hi = lo[first], hi[first]
+        flip = rng.random(lo.shape[0]) < 0.5
+        srcs.append(np.where(flip, hi, lo) + c * cluster_size)
+        dsts.append(np.where(flip, lo, hi) + c * cluster_size)
     intra = sum(x.shape[0] for x in srcs)
     m_inter = int(intra * inter_fraction / (1.0 - inter_fraction))
-    a = rng.integers(0, n, size=m_inter, dtype=np.int64)
-    b = rng.integers(0, n, size=m_inter, dtype=np.int64)
+    a = rng.integers(0, n, size=int(m_inter * 1.03), dtype=np.int64)
+    b = rng.integers(0, n, size=a.shape[0], dtype=np.int64)
     keep = (a // cluster_size) != (b // cluster_size)
-    srcs.append(a[keep])
-    dsts.append(b[keep])
+    srcs.append(a[keep][:m_inter])
+    dsts.append(b[keep][:m_inter])
     e = np.stack([np.concatenate(srcs), np.concatenate(dsts)])
     key = np.unique(e[0] * np.int64(n) + e[1])
     e = np.stack([key // n, key % n])
     e = e[:, rng.permutation(e.shape[1])]
     return e, n, np.repeat(np.arange(n_clusters, dtype=np.int64), cluster_size)
+
+
+def clustered_power_law_graph(n=870_000, exponent=2.0, directed_edges=44_000_000, n_clusters=64,
+                              intra_fraction=0.8, seed=42, oversample=None):
+    """Config 3: power-law graph (mean degree ~50) whose nodes are grouped into contiguous
+    clusters, the order a cluster / degree reordering leaves behind: a fraction
+    ``intra_fraction`` of every node's stubs is matched inside its cluster, the rest globally.
+    Bidirectional, self-loops, global node 0.  N = n + 1."""
+    rng = np.random.default_rng(seed)
+    m_target = (directed_edges - 3 * n) // 2
+    kmax = int(np.sqrt(2.0 * m_target))
+    first_pass = oversample is None
+    deg = power_law_degrees(n, exponent, int(2 * m_target * (oversample or 1.0)), kmax, rng)
+    csize = (n + n_clusters - 1) // n_clusters
+    intra = rng.binomial(deg, intra_fraction)
+    pairs = []
+    for c in range(n_clusters):
+        lo, hi = c * csize, min(n, (c + 1) * csize)
+        stubs = np.repeat(np.arange(lo, hi, dtype=np.int64), intra[lo:hi])
+        rng.shuffle(stubs)
+        h = stubs.shape[0] // 2
+        pairs.append(np.stack([stubs[:h], stubs[h:2 * h]], axis=1))
+    stubs = np.repeat(np.arange(n, dtype=np.int64), deg - intra)
+    rng.shuffle(stubs)
+    h = stubs.shape[0] // 2
+    pairs.append(np.stack([stubs[:h], stubs[h:2 * h]], axis=1))
+    allp = np.concatenate(pairs)
+    und = _simple_pairs(allp[:, 0], allp[:, 1], n)
+    loss = m_target / max(1, und.shape[0])
+    if first_pass and abs(loss - 1.0) > 0.02:      # the erased model drops multi-edges: one corrective pass
+        return clustered_power_law_graph(n, exponent, directed_edges, n_clusters, intra_fraction, seed,
+                                         oversample=loss)
+    e = _symmetrize_with_self_loops(und, n)
+    return add_global_node(e, n), n + 1
 
 
 def erdos_renyi_batch(batch=256, n_min=16, n_max=128, p=0.1, n_edge_types=4, spd_clamp=20, seed=42):
