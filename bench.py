@@ -67,6 +67,12 @@ def build_workload(name):
     elif name == "config1":
         e, n = workloads.barabasi_albert(n=4096, m=4, seed=42)
         label = "configs[0]: Barabasi-Albert 4096 nodes m=4 + 1 global node"
+    elif name == "config3":
+        e, n = workloads.clustered_power_law_graph(n=870_000, exponent=2.0, directed_edges=44_000_000, seed=42)
+        label = "configs[2]: clustered power-law (exp 2.0) 870000 nodes + 1 global node, cluster-ordered"
+    elif name == "config5":
+        e, n, _ = workloads.stochastic_block_model(seed=42)
+        label = "configs[4]: SBM 64 x 4096 nodes, p_intra 0.004, 5% inter-cluster, cluster-ordered"
     else:
         raise SystemExit(f"unknown workload {name}")
     return e, n, label, workloads.describe(e, n)
@@ -199,10 +205,12 @@ def main():
     H, d = 8, 8
     tdt = torch.float32 if args.dtype == "f32" else torch.bfloat16
     esize = 4 if args.dtype == "f32" else 2
+    if args.workload in ("config3", "config4", "config5") and "--dtype" not in sys.argv:
+        args.dtype = "bf16"              # the dtype those configurations are quoted on
     if args.workload == "config4":
-        if args.dtype == "f32" and "--dtype" not in sys.argv:
-            args.dtype = "bf16"
         return bench_dense(args)
+    if args.workload in ("config3", "config5"):
+        args.no_cpu_baseline = True      # the CPU restatement needs minutes per step at this size
     e, n, label, desc = build_workload(args.workload)
     E = e.shape[1]
 

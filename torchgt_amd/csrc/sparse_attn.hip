@@ -473,8 +473,14 @@ template <typename T, int LPE, int LPH, bool HASB>
 __global__ __launch_bounds__(kBlock) void k_attn_fwd(const Common c, const SideArgs s, const int items_pad) {
     __shared__ BlockLds<LPE> lds;
     const int b = blockIdx.x;
-    if (b < s.n_block_items) block_item<T, LPE, LPH, MODE_FWD, HASB>(c, s, b, lds);
-    else if (b >= items_pad) wave_block<T, LPE, LPH, MODE_FWD, HASB>(c, s, b - items_pad);
+    if (b < items_pad) {
+        // workgroup items are in row order; XCD x (= workgroup id mod 8) takes the x-th contiguous
+        // eighth of them, so the rows of a cluster (and the segments of a split row) share an L2
+        const int it = (b & 7) * (items_pad >> 3) + (b >> 3);
+        if (it < s.n_block_items) block_item<T, LPE, LPH, MODE_FWD, HASB>(c, s, it, lds);
+    } else {
+        wave_block<T, LPE, LPH, MODE_FWD, HASB>(c, s, b - items_pad);
+    }
 }
 
 // Backward: both views in one launch (they are independent once nd is known):
@@ -482,16 +488,21 @@ __global__ __launch_bounds__(kBlock) void k_attn_fwd(const Common c, const SideA
 // wave items of the destination view, wave items of the source view.
 template <typename T, int LPE, int LPH, bool HASB>
 __global__ __launch_bounds__(kBlock) void k_attn_bwd(const Common c, const SideArgs sd, const SideArgs ss,
-                                                     const int items_pad) {
+                                                     const int pad_d, const int pad_s) {
     __shared__ BlockLds<LPE> lds;
     int b = blockIdx.x;
-    if (b < sd.n_block_items) { block_item<T, LPE, LPH, MODE_BWD_DST, HASB>(c, sd, b, lds); return; }
-    if (b < sd.n_block_items + ss.n_block_items) {
-        block_item<T, LPE, LPH, MODE_BWD_SRC, HASB>(c, ss, b - sd.n_block_items, lds);
+    if (b < pad_d) {
+        const int it = (b & 7) * (pad_d >> 3) + (b >> 3);
+        if (it < sd.n_block_items) block_item<T, LPE, LPH, MODE_BWD_DST, HASB>(c, sd, it, lds);
         return;
     }
-    if (b < items_pad) return;     // padding: the wave regions start at a multiple of 8
-    b -= items_pad;
+    b -= pad_d;
+    if (b < pad_s) {
+        const int it = (b & 7) * (pad_s >> 3) + (b >> 3);
+        if (it < ss.n_block_items) block_item<T, LPE, LPH, MODE_BWD_SRC, HASB>(c, ss, it, lds);
+        return;
+    }
+    b -= pad_s;
     if (b < sd.n_wave_blocks) { wave_block<T, LPE, LPH, MODE_BWD_DST, HASB>(c, sd, b); return; }
     b -= sd.n_wave_blocks;
     wave_block<T, LPE, LPH, MODE_BWD_SRC, HASB>(c, ss, b);
@@ -631,14 +642,14 @@ static int run_bwd(const Call& c) {
     ss.out0 = c.dk; ss.out1 = c.dv; ss.Z = nullptr;
     ss.part = reinterpret_cast<float*>(c.ws + L.dkv_part);
     ss.counters = counters + 2 * c.plan->dst.n_split;
-    const int items_pad = pad8(sd.n_block_items + ss.n_block_items);
-    const int nb = items_pad + sd.n_wave_blocks + ss.n_wave_blocks;
+    const int pad_d = pad8(sd.n_block_items), pad_s = pad8(ss.n_block_items);
+    const int nb = pad_d + pad_s + sd.n_wave_blocks + ss.n_wave_blocks;
     if (nb > 0) {
         KernelTimer t(KS_BWD, c.st);
         if (c.bias_mode != TGT_BIAS_NONE)
-            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, items_pad);
+            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
         else
-            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, items_pad);
+            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
     }
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
