@@ -138,6 +138,34 @@ int tgt_dense_attn_bwd(const void* d_q, const void* d_k, const void* d_v, const 
                        const void* d_out, const float* d_lse, const void* d_dout,
                        void* d_dq, void* d_dk, void* d_dv, void* d_dbias, void* stream);
 
+/* ---- block path: dense 16 x 16 tiles + remaining edges, one softmax per node ----
+ * A tile (r0, c0) stands for the 256 edges a -> b, a in [r0, r0+16), b in
+ * [c0, c0+16) that the reference's cluster reordering emits as an expanded edge
+ * list (gt_sp/utils.py:284-299, create_pairs :218-220) and then feeds to
+ * sparse_attention (attn_module.py:133-189).  The result equals sparse attention
+ * over the expanded tiles plus the edges of `plan` (tiles carry no bias, like the
+ * reference, which forces attn_bias to None on this path, gt_sp/utils.py:465,470).
+ * Tile products run on bf16 matrix instructions with fp32 accumulation (float32
+ * inputs are rounded to bf16 for them); the remaining edges run on the sparse
+ * kernels.  h_tiles: HOST int32 [T, 2]; destination blocks (and source blocks) of
+ * different tiles must be identical or disjoint.  `plan` holds the remaining edges
+ * (it may have E = 0) and fixes N.  Workspace: as for tgt_sparse_attn_*, zeroed once. */
+typedef struct tgt_tiles tgt_tiles_t;
+int tgt_tiles_create(const int32_t* h_tiles, int64_t T, int block_size, int64_t N, void* stream,
+                     tgt_tiles_t** out);
+int tgt_tiles_destroy(tgt_tiles_t* tiles);
+int64_t tgt_block_attn_workspace_bytes(const tgt_tiles_t* tiles, const tgt_plan_t* plan, int H, int d);
+int tgt_block_attn_fwd(const tgt_tiles_t* tiles, const tgt_plan_t* plan,
+                       const void* d_q, const void* d_k, const void* d_v,
+                       const void* d_bias, int bias_mode, int H, int d, int dtype,
+                       void* d_out, float* d_Z, void* d_workspace, int64_t workspace_bytes, void* stream);
+int tgt_block_attn_bwd(const tgt_tiles_t* tiles, const tgt_plan_t* plan,
+                       const void* d_q, const void* d_k, const void* d_v,
+                       const void* d_bias, int bias_mode, int H, int d, int dtype,
+                       const void* d_out, const float* d_Z, const void* d_dout,
+                       void* d_dq, void* d_dk, void* d_dv, void* d_dbias,
+                       void* d_workspace, int64_t workspace_bytes, void* stream);
+
 /* ---- edge construction and ordering ------------------------------------
  * fix_edge_index (gt_sp/utils.py:34-50): d_edge_index int64 [2, E0] over real
  * nodes 0..num_node-1 -> d_out int64 [2, E0 + 2*num_node]: real nodes shift by +1,
@@ -164,6 +192,13 @@ int tgt_reformat_create(const int64_t* d_src, const int64_t* d_dst, int64_t E, i
 int64_t tgt_reformat_num_edges(const tgt_reformat_t* r);
 int tgt_reformat_export(const tgt_reformat_t* r, int64_t* d_edge_index, int64_t* d_sorted_indices, void* stream);
 int tgt_reformat_destroy(tgt_reformat_t* r);
+/* The same result as a tile list: every emitted block as (first source, first
+ * destination) in new ids (h_tiles, HOST int32 [T, 2], T = tgt_reformat_num_tiles)
+ * plus the edges that were kept as they are (d_raw_edge_index, DEVICE int64
+ * [2, E_raw], relabelled) - the input of tgt_block_attn_*. */
+int64_t tgt_reformat_num_tiles(const tgt_reformat_t* r);
+int64_t tgt_reformat_num_raw_edges(const tgt_reformat_t* r);
+int tgt_reformat_export_tiles(const tgt_reformat_t* r, int32_t* h_tiles, int64_t* d_raw_edge_index, void* stream);
 
 /* Host only: the n values np.random.randint(0, h_highs[i]) returns after
  * np.random.seed(seed) (legacy MT19937 stream used by gt_sp/utils.py:290-295). */

@@ -36,6 +36,15 @@ SIGNATURES = {
     "tgt_dense_attn_fwd": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp]),
     "tgt_dense_attn_bwd": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp,
                                   _vp, _vp, _vp, _vp, _vp]),
+    "tgt_tiles_create": (_i32, [_vp, _i64, _i32, _i64, _vp, _c.POINTER(_vp)]),
+    "tgt_tiles_destroy": (_i32, [_vp]),
+    "tgt_block_attn_workspace_bytes": (_i64, [_vp, _vp, _i32, _i32]),
+    "tgt_block_attn_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _i64, _vp]),
+    "tgt_block_attn_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp,
+                                  _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
+    "tgt_reformat_num_tiles": (_i64, [_vp]),
+    "tgt_reformat_num_raw_edges": (_i64, [_vp]),
+    "tgt_reformat_export_tiles": (_i32, [_vp, _vp, _vp, _vp]),
     "tgt_fix_edge_index": (_i32, [_vp, _i64, _i64, _vp, _vp]),
     "tgt_reformat_create": (_i32, [_vp, _vp, _i64, _i64, _vp, _i32, _i32, _i32, _vp, _c.POINTER(_vp)]),
     "tgt_reformat_num_edges": (_i64, [_vp]),

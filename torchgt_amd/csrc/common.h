@@ -75,7 +75,7 @@ private:
 };
 
 // Kernel names of the optional per-kernel timing (timing.hip).
-enum KernelSlot { KS_FWD = 0, KS_NODE_SIDE, KS_BWD, KS_DENSE_FWD, KS_DENSE_BWD, KS_COUNT };
+enum KernelSlot { KS_FWD = 0, KS_NODE_SIDE, KS_BWD, KS_DENSE_FWD, KS_DENSE_BWD, KS_TILE_FWD, KS_TILE_BWD, KS_COUNT };
 
 // Scope guard: records a hipEvent on `st` before and after the launches made in
 // its scope when timing is enabled; does nothing otherwise.
@@ -91,6 +91,32 @@ private:
     hipEvent_t start_;
 };
 
+// Sums of the dense tiles of the block path, added by the sparse kernels when they write a row.
+struct TileInit {
+    const float* acc;          // [N, H, d] sum w v
+    const float* Z;            // [N, H]
+    const float* dq;           // [N, H, d]
+    const float* dk;           // [N, H, d]
+    const float* dv;           // [N, H, d]
+    const uint8_t* cover_dst;  // [N] 1 where the node is a destination of some tile
+    const uint8_t* cover_src;  // [N] 1 where the node is a source of some tile
+};
+
+}  // namespace tgt
+
+struct tgt_plan;
+namespace tgt {
+int sparse_attn_fwd_impl(const tgt_plan* plan, const void* d_q, const void* d_k, const void* d_v, const void* d_bias,
+                         int bias_mode, int H, int d, int dtype, void* d_out, float* d_Z, void* d_workspace,
+                         int64_t workspace_bytes, void* stream, const TileInit* init);
+int sparse_attn_bwd_impl(const tgt_plan* plan, const void* d_q, const void* d_k, const void* d_v, const void* d_bias,
+                         int bias_mode, int H, int d, int dtype, const void* d_out, const float* d_Z,
+                         const void* d_dout, void* d_dq, void* d_dk, void* d_dv, void* d_dbias, void* d_workspace,
+                         int64_t workspace_bytes, void* stream, const TileInit* init, bool skip_node_side);
+// nd[i,h] = (1/(Z+eps), dout.out) into the head of the workspace (what the backward walks read)
+int sparse_attn_node_side(const tgt_plan* plan, int H, int d, int dtype, const void* d_out, const float* d_Z,
+                          const void* d_dout, void* d_workspace, void* stream);
+const float2* sparse_attn_nd_ptr(void* d_workspace);
 }  // namespace tgt
 
 struct tgt_plan {

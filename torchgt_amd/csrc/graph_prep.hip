@@ -157,6 +157,14 @@ __global__ void k_emit_blocks(const int64_t* __restrict__ blk_off, const uint32_
     }
 }
 
+__global__ void k_write_raw(const uint32_t* __restrict__ ns, const uint32_t* __restrict__ nd, int64_t off,
+                            int64_t cnt, int64_t dst_off, int64_t E_raw, int64_t* __restrict__ out) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= cnt) return;
+    out[dst_off + i] = (int64_t)ns[off + i];
+    out[E_raw + dst_off + i] = (int64_t)nd[off + i];
+}
+
 __global__ void k_write_sorted(const uint32_t* __restrict__ keys_sorted, const uint32_t* __restrict__ order,
                                const uint32_t* __restrict__ nd, int64_t n, int64_t* __restrict__ out) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -173,6 +181,9 @@ struct tgt_reformat {
     int64_t N = 0, E_out = 0;
     tgt::DevBuf edge_index;       // int64 [2, E_out], stably sorted by source
     tgt::DevBuf sorted_indices;   // int64 [N], new id -> old id
+    std::vector<int32_t> tiles;   // (first source, first destination) of every emitted block, emission order
+    int64_t E_raw = 0;            // edges kept as they are (the sparsity > p branch, or everything if !blockize)
+    tgt::DevBuf raw;              // int64 [2, E_raw], relabelled, emission order
 };
 
 namespace tgt {
@@ -338,6 +349,30 @@ static int reformat_impl(const int64_t* d_src, const int64_t* d_dst, int64_t E, 
             TGT_HIP_CHECK(hipStreamSynchronize(st));   // the descriptor buffers die here
         }
     }
+    // the blocks as a tile list and the edges kept as they are, for the block attention path
+    for (size_t i = 0; i < blk_r0.size(); ++i) {
+        R->tiles.push_back((int32_t)blk_r0[i]);
+        R->tiles.push_back((int32_t)blk_c0[i]);
+    }
+    {
+        int64_t e_raw = blockize ? 0 : E;
+        for (const RawSlice& r : raws) e_raw += r.cnt;
+        R->E_raw = e_raw;
+        TGT_HIP_CHECK(R->raw.alloc(sizeof(int64_t) * 2 * (size_t)(e_raw ? e_raw : 1)));
+        if (!blockize) {
+            if (E > 0)
+                hipLaunchKernelGGL(k_write_raw, dim3(nblk(E)), dim3(256), 0, st, ns.as<uint32_t>(), nd.as<uint32_t>(),
+                                   (int64_t)0, E, (int64_t)0, e_raw, R->raw.as<int64_t>());
+        } else {
+            int64_t pos = 0;
+            for (const RawSlice& r : raws) {
+                if (r.cnt > 0)
+                    hipLaunchKernelGGL(k_write_raw, dim3(nblk(r.cnt)), dim3(256), 0, st, ns.as<uint32_t>(),
+                                       nd.as<uint32_t>(), r.out_off, r.cnt, pos, e_raw, R->raw.as<int64_t>());
+                pos += r.cnt;
+            }
+        }
+    }
     // stable sort by new source (gt_sp/utils.py:354-356)
     if (E_out > 0) {
         const uint32_t *ko = nullptr, *vo = nullptr;
@@ -412,6 +447,21 @@ int tgt_reformat_export(const tgt_reformat_t* r, int64_t* d_edge_index, int64_t*
                                      hipMemcpyDeviceToDevice, st));
     TGT_HIP_CHECK(hipMemcpyAsync(d_sorted_indices, r->sorted_indices.p, sizeof(int64_t) * r->N,
                                  hipMemcpyDeviceToDevice, st));
+    return TGT_OK;
+}
+
+int64_t tgt_reformat_num_tiles(const tgt_reformat_t* r) { return r ? (int64_t)(r->tiles.size() / 2) : -1; }
+int64_t tgt_reformat_num_raw_edges(const tgt_reformat_t* r) { return r ? r->E_raw : -1; }
+
+int tgt_reformat_export_tiles(const tgt_reformat_t* r, int32_t* h_tiles, int64_t* d_raw_edge_index, void* stream) {
+    if (!r || (!r->tiles.empty() && !h_tiles) || (r->E_raw > 0 && !d_raw_edge_index)) {
+        tgt::set_error("tgt_reformat_export_tiles: null pointer");
+        return TGT_ERR_INVALID_ARG;
+    }
+    for (size_t i = 0; i < r->tiles.size(); ++i) h_tiles[i] = r->tiles[i];
+    if (r->E_raw > 0)
+        TGT_HIP_CHECK(hipMemcpyAsync(d_raw_edge_index, r->raw.p, sizeof(int64_t) * 2 * r->E_raw,
+                                     hipMemcpyDeviceToDevice, (hipStream_t)stream));
     return TGT_OK;
 }
 

@@ -112,6 +112,12 @@ struct SideArgs {
     float* Z;             // fwd: Z
     float* part;          // partial sums of split rows
     int32_t* counters;    // one arrival counter per split row, zero between calls
+    // optional sums computed elsewhere for the same rows (dense tiles of the block path), fp32,
+    // added when the row is written: fwd (sum w v, Z) | bwd_dst dq | bwd_src (dk, dv)
+    const float* init0;
+    const float* init1;
+    const float* initZ;
+    const uint8_t* cover; // [N] 1 where the row has such sums
     int32_t n_block_items;
     int32_t n_wave_blocks;               // multiple of 8
     int32_t class_off[kNumClass + 1];    // item index where each wave class begins
@@ -274,6 +280,23 @@ __device__ __forceinline__ void write_row(const Common& c, const SideArgs& s, co
     constexpr int H = LPE / LPH;
     constexpr int HD = LPE * 8;
     const int64_t row_off = (int64_t)row * HD + el * 8;
+    const bool extra = s.init0 != nullptr && s.cover[row] != 0;
+    if (MODE != MODE_FWD) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc.a0[i] *= c.inv_scale;
+    }
+    if (extra) {
+        float t[8];
+        load8(s.init0 + row_off, t);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc.a0[i] += t[i];
+        if (MODE == MODE_FWD) acc.z += s.initZ[(int64_t)row * H + el / LPH];
+        if (MODE == MODE_BWD_SRC) {
+            load8(s.init1 + row_off, t);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc.a1[i] += t[i];
+        }
+    }
     if (MODE == MODE_FWD) {
         const float den = acc.z + kEps;
 #pragma unroll
@@ -281,8 +304,6 @@ __device__ __forceinline__ void write_row(const Common& c, const SideArgs& s, co
         store8(static_cast<T*>(s.out0) + row_off, acc.a0);
         if (el % LPH == 0) s.Z[(int64_t)row * H + el / LPH] = acc.z;
     } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) acc.a0[i] *= c.inv_scale;
         store8(static_cast<T*>(s.out0) + row_off, acc.a0);
         if (MODE == MODE_BWD_SRC) store8(static_cast<T*>(s.out1) + row_off, acc.a1);
     }
@@ -585,6 +606,9 @@ struct Call {
     float* o_Z;
     char* ws;
     hipStream_t st;
+    const TileInit* init;
+    bool skip_node_side;   // nd was already computed into the workspace by sparse_attn_node_side
+    bool only_node_side;
 };
 
 template <typename T, int LPE, int LPH>
@@ -599,6 +623,7 @@ static int run_fwd(const Call& c) {
     SideArgs a{};
     fill_side(a, c.plan->dst, LPE);
     a.out0 = c.o_out; a.out1 = nullptr; a.Z = c.o_Z;
+    if (c.init) { a.init0 = c.init->acc; a.initZ = c.init->Z; a.cover = c.init->cover_dst; }
     a.part = reinterpret_cast<float*>(c.ws + L.fwd_part);
     a.counters = reinterpret_cast<int32_t*>(c.ws + L.counters);
     const int items_pad = pad8(a.n_block_items);
@@ -619,13 +644,15 @@ static int run_bwd(const Call& c) {
     const WsLayout L = ws_layout(c.plan, c.H, c.d);
     const int64_t N = c.plan->N;
     float2* nd = reinterpret_cast<float2*>(c.ws + L.nd);
-    {
+    if (!c.skip_node_side) {
         constexpr int RPB = kBlock / LPE;
         const int nb = (int)((N + RPB - 1) / RPB);
         KernelTimer t(KS_NODE_SIDE, c.st);
         hipLaunchKernelGGL((k_node_side<T, LPE, LPH>), dim3(nb), dim3(kBlock), 0, c.st,
                            static_cast<const T*>(c.out), static_cast<const T*>(c.dout), c.Z, N, nd);
+        TGT_HIP_CHECK(hipGetLastError());
     }
+    if (c.only_node_side) return TGT_OK;
     Common cm{};
     cm.q = c.q; cm.k = c.k; cm.v = c.v; cm.g = c.dout; cm.bias = c.bias; cm.nd = nd;
     cm.bias_mode = c.bias_mode;
@@ -636,10 +663,12 @@ static int run_bwd(const Call& c) {
     SideArgs sd{}, ss{};
     fill_side(sd, c.plan->dst, LPE);
     sd.out0 = c.dq; sd.out1 = c.dbias; sd.Z = nullptr;
+    if (c.init) { sd.init0 = c.init->dq; sd.cover = c.init->cover_dst; }
     sd.part = reinterpret_cast<float*>(c.ws + L.dq_part);
     sd.counters = counters + c.plan->dst.n_split;
     fill_side(ss, c.plan->src, LPE);
     ss.out0 = c.dk; ss.out1 = c.dv; ss.Z = nullptr;
+    if (c.init) { ss.init0 = c.init->dk; ss.init1 = c.init->dv; ss.cover = c.init->cover_src; }
     ss.part = reinterpret_cast<float*>(c.ws + L.dkv_part);
     ss.counters = counters + 2 * c.plan->dst.n_split;
     const int pad_d = pad8(sd.n_block_items), pad_s = pad8(ss.n_block_items);
@@ -693,6 +722,54 @@ static int check_common(const tgt_plan* plan, const void* q, const void* k, cons
     return TGT_OK;
 }
 
+int sparse_attn_fwd_impl(const tgt_plan_t* plan, const void* d_q, const void* d_k, const void* d_v,
+                         const void* d_bias, int bias_mode, int H, int d, int dtype, void* d_out, float* d_Z,
+                         void* d_workspace, int64_t workspace_bytes, void* stream, const TileInit* init) {
+    int rc = check_common(plan, d_q, d_k, d_v, d_bias, bias_mode, H, d, dtype, d_workspace, workspace_bytes);
+    if (rc) return rc;
+    if (!d_out || !d_Z) { set_error("null out or Z"); return TGT_ERR_INVALID_ARG; }
+    Call c{};
+    c.plan = plan; c.q = d_q; c.k = d_k; c.v = d_v; c.bias = d_bias; c.bias_mode = bias_mode;
+    c.H = H; c.d = d; c.o_out = d_out; c.o_Z = d_Z; c.ws = static_cast<char*>(d_workspace);
+    c.st = static_cast<hipStream_t>(stream);
+    c.init = init;
+    return dtype == TGT_DTYPE_F32 ? dispatch<float>(c, false) : dispatch<bf16_t>(c, false);
+}
+
+int sparse_attn_bwd_impl(const tgt_plan_t* plan, const void* d_q, const void* d_k, const void* d_v,
+                         const void* d_bias, int bias_mode, int H, int d, int dtype, const void* d_out,
+                         const float* d_Z, const void* d_dout, void* d_dq, void* d_dk, void* d_dv,
+                         void* d_dbias, void* d_workspace, int64_t workspace_bytes, void* stream,
+                         const TileInit* init, bool skip_node_side) {
+    int rc = check_common(plan, d_q, d_k, d_v, d_bias, bias_mode, H, d, dtype, d_workspace, workspace_bytes);
+    if (rc) return rc;
+    if (!d_out || !d_Z || !d_dout || !d_dq || !d_dk || !d_dv) {
+        set_error("null out/Z/dout/dq/dk/dv");
+        return TGT_ERR_INVALID_ARG;
+    }
+    Call c{};
+    c.plan = plan; c.q = d_q; c.k = d_k; c.v = d_v; c.bias = d_bias; c.bias_mode = bias_mode;
+    c.H = H; c.d = d; c.out = d_out; c.Z = d_Z; c.dout = d_dout;
+    c.dq = d_dq; c.dk = d_dk; c.dv = d_dv; c.dbias = (bias_mode == TGT_BIAS_NONE) ? nullptr : d_dbias;
+    c.ws = static_cast<char*>(d_workspace);
+    c.st = static_cast<hipStream_t>(stream);
+    c.init = init;
+    c.skip_node_side = skip_node_side;
+    return dtype == TGT_DTYPE_F32 ? dispatch<float>(c, true) : dispatch<bf16_t>(c, true);
+}
+
+int sparse_attn_node_side(const tgt_plan_t* plan, int H, int d, int dtype, const void* d_out, const float* d_Z,
+                          const void* d_dout, void* d_workspace, void* stream) {
+    Call c{};
+    c.plan = plan; c.H = H; c.d = d; c.out = d_out; c.Z = d_Z; c.dout = d_dout;
+    c.ws = static_cast<char*>(d_workspace);
+    c.st = static_cast<hipStream_t>(stream);
+    c.only_node_side = true;
+    return dtype == TGT_DTYPE_F32 ? dispatch<float>(c, true) : dispatch<bf16_t>(c, true);
+}
+
+const float2* sparse_attn_nd_ptr(void* d_workspace) { return reinterpret_cast<const float2*>(d_workspace); }
+
 }  // namespace tgt
 
 extern "C" {
@@ -705,33 +782,16 @@ int64_t tgt_sparse_attn_workspace_bytes(const tgt_plan_t* plan, int H, int d) {
 int tgt_sparse_attn_fwd(const tgt_plan_t* plan, const void* d_q, const void* d_k, const void* d_v,
                         const void* d_bias, int bias_mode, int H, int d, int dtype, void* d_out, float* d_Z,
                         void* d_workspace, int64_t workspace_bytes, void* stream) {
-    int rc = tgt::check_common(plan, d_q, d_k, d_v, d_bias, bias_mode, H, d, dtype, d_workspace, workspace_bytes);
-    if (rc) return rc;
-    if (!d_out || !d_Z) { tgt::set_error("null out or Z"); return TGT_ERR_INVALID_ARG; }
-    tgt::Call c{};
-    c.plan = plan; c.q = d_q; c.k = d_k; c.v = d_v; c.bias = d_bias; c.bias_mode = bias_mode;
-    c.H = H; c.d = d; c.o_out = d_out; c.o_Z = d_Z; c.ws = static_cast<char*>(d_workspace);
-    c.st = static_cast<hipStream_t>(stream);
-    return dtype == TGT_DTYPE_F32 ? tgt::dispatch<float>(c, false) : tgt::dispatch<tgt::bf16_t>(c, false);
+    return tgt::sparse_attn_fwd_impl(plan, d_q, d_k, d_v, d_bias, bias_mode, H, d, dtype, d_out, d_Z, d_workspace,
+                                     workspace_bytes, stream, nullptr);
 }
 
 int tgt_sparse_attn_bwd(const tgt_plan_t* plan, const void* d_q, const void* d_k, const void* d_v,
                         const void* d_bias, int bias_mode, int H, int d, int dtype, const void* d_out,
                         const float* d_Z, const void* d_dout, void* d_dq, void* d_dk, void* d_dv,
                         void* d_dbias, void* d_workspace, int64_t workspace_bytes, void* stream) {
-    int rc = tgt::check_common(plan, d_q, d_k, d_v, d_bias, bias_mode, H, d, dtype, d_workspace, workspace_bytes);
-    if (rc) return rc;
-    if (!d_out || !d_Z || !d_dout || !d_dq || !d_dk || !d_dv) {
-        tgt::set_error("null out/Z/dout/dq/dk/dv");
-        return TGT_ERR_INVALID_ARG;
-    }
-    tgt::Call c{};
-    c.plan = plan; c.q = d_q; c.k = d_k; c.v = d_v; c.bias = d_bias; c.bias_mode = bias_mode;
-    c.H = H; c.d = d; c.out = d_out; c.Z = d_Z; c.dout = d_dout;
-    c.dq = d_dq; c.dk = d_dk; c.dv = d_dv; c.dbias = (bias_mode == TGT_BIAS_NONE) ? nullptr : d_dbias;
-    c.ws = static_cast<char*>(d_workspace);
-    c.st = static_cast<hipStream_t>(stream);
-    return dtype == TGT_DTYPE_F32 ? tgt::dispatch<float>(c, true) : tgt::dispatch<tgt::bf16_t>(c, true);
+    return tgt::sparse_attn_bwd_impl(plan, d_q, d_k, d_v, d_bias, bias_mode, H, d, dtype, d_out, d_Z, d_dout, d_dq,
+                                     d_dk, d_dv, d_dbias, d_workspace, workspace_bytes, stream, nullptr, false);
 }
 
 }  // extern "C"

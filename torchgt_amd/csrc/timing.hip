@@ -12,7 +12,7 @@
 namespace tgt {
 
 static const char* kSlotNames[KS_COUNT] = {
-    "attn_fwd", "bwd_node_side", "attn_bwd", "dense_fwd", "dense_bwd",
+    "attn_fwd", "bwd_node_side", "attn_bwd", "dense_fwd", "dense_bwd", "tile_fwd", "tile_bwd",
 };
 
 struct Pending { hipEvent_t start, stop; int slot; };

@@ -35,14 +35,19 @@ def adjust_edge_index_nomerge(edge_index, sub_seq_len):
     return torch.where(edge_index > 0, edge_index + shift, edge_index)
 
 
-def reformat_graph(edge_index, k, block_size, beta_coeffi="1", partition_ids=None, blockize=True):
+def reformat_graph(edge_index, k, block_size, beta_coeffi="1", partition_ids=None, blockize=True,
+                   return_tiles=False):
     """Relabel nodes by partition, (optionally) replace the edges of every partition pair by
     random dense blocks, and stably sort the edges by source.  Same return value as the
     reference: (sorted_edge_index [2, E'], sorted_indices [N]).
 
     The reference obtains ``partition_ids`` from dgl's METIS binding, which does not exist
     here; they must be passed in (int64 [N], values in [0, k)).  ``beta_coeffi`` is accepted
-    and ignored, as in the reference (p is overwritten with 1, gt_sp/utils.py:344)."""
+    and ignored, as in the reference (p is overwritten with 1, gt_sp/utils.py:344).
+
+    ``return_tiles=True`` additionally returns the emitted blocks as a tile list (numpy int32
+    [T, 2], first source / first destination in new ids) and the edges that were kept as they
+    are (int64 [2, E_raw]), the inputs of ``torchgt_amd.block_attention``."""
     if partition_ids is None:
         raise ValueError("reformat_graph: partition_ids must be given (METIS is not available)")
     if not edge_index.is_cuda:
@@ -64,7 +69,17 @@ def reformat_graph(edge_index, k, block_size, beta_coeffi="1", partition_ids=Non
             sorted_indices = torch.empty(N, dtype=torch.int64, device=dev)
             _lib.check(L.tgt_reformat_export(handle, out.data_ptr() if E_out else None,
                                              sorted_indices.data_ptr(), st))
+            tiles = raw = None
+            if return_tiles:
+                import numpy as np
+                T, E_raw = L.tgt_reformat_num_tiles(handle), L.tgt_reformat_num_raw_edges(handle)
+                tiles = np.empty((T, 2), dtype=np.int32)
+                raw = torch.empty((2, E_raw), dtype=torch.int64, device=dev)
+                _lib.check(L.tgt_reformat_export_tiles(handle, tiles.ctypes.data_as(ctypes.c_void_p) if T else None,
+                                                       raw.data_ptr() if E_raw else None, st))
             torch.cuda.current_stream(dev).synchronize()
         finally:
             L.tgt_reformat_destroy(handle)
+    if return_tiles:
+        return out, sorted_indices, tiles, raw
     return out, sorted_indices
