@@ -179,6 +179,95 @@ def bench_dense(args):
     print(json.dumps(result))
 
 
+def bench_block(args):
+    """BASELINE configs[4] through the reference's pipeline: SBM 64 x 4096, the reference's
+    cluster reordering with the clusters as partitions (every partition pair's edges become
+    dense 16 x 16 blocks), then attention.  A step = tgt_block_attn_fwd + _bwd on the tile list;
+    the same edges through the sparse kernels (expanded list) are timed next to it."""
+    import numpy as np
+    import torch
+    from torchgt_amd import _lib, graph_prep, workloads
+    from torchgt_amd.block_attention import TileSet
+    from torchgt_amd.plan import GraphPlan
+    dev = torch.device("cuda:0")
+    H, d = 8, 8
+    tdt = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    e, n, cluster = workloads.stochastic_block_model(seed=42)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    new_e, _, tiles, raw = graph_prep.reformat_graph(torch.from_numpy(e).to(dev), 64, 16,
+                                                     partition_ids=torch.from_numpy(cluster), return_tiles=True)
+    torch.cuda.synchronize()
+    reorder_ms = (time.perf_counter() - t0) * 1e3
+    E = int(new_e.shape[1])
+    ts = TileSet(tiles, n, dev)
+    plan_rest = GraphPlan(raw, n)
+    plan_full = GraphPlan(new_e, n)
+    g = torch.Generator().manual_seed(42)
+    q, k, v, dout = (torch.randn(n, H, d, generator=g).to(dev, tdt) for _ in range(4))
+    out = torch.empty_like(q)
+    Z = torch.empty(n, H, device=dev)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+    L = _lib.lib()
+    code = _lib.DTYPE_BF16 if args.dtype == "bf16" else _lib.DTYPE_F32
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    P = lambda t: t.data_ptr()
+    wsb = ts.workspace(plan_rest, H, d)
+    wss = plan_full.workspace(H, d)
+
+    def step_block():
+        _lib.check(L.tgt_block_attn_fwd(ts.handle, plan_rest.handle, P(q), P(k), P(v), None, 0, H, d, code, P(out),
+                                        P(Z), P(wsb), wsb.numel(), stream))
+        _lib.check(L.tgt_block_attn_bwd(ts.handle, plan_rest.handle, P(q), P(k), P(v), None, 0, H, d, code, P(out),
+                                        P(Z), P(dout), P(dq), P(dk), P(dv), None, P(wsb), wsb.numel(), stream))
+
+    def step_sparse():
+        _lib.check(L.tgt_sparse_attn_fwd(plan_full.handle, P(q), P(k), P(v), None, 0, H, d, code, P(out), P(Z),
+                                         P(wss), wss.numel(), stream))
+        _lib.check(L.tgt_sparse_attn_bwd(plan_full.handle, P(q), P(k), P(v), None, 0, H, d, code, P(out), P(Z),
+                                         P(dout), P(dq), P(dk), P(dv), None, P(wss), wss.numel(), stream))
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / args.steps * 1e3
+
+    ms_block = timed(step_block)
+    L.tgt_timing_reset()
+    L.tgt_timing_enable(1)
+    for _ in range(args.steps):
+        step_block()
+    torch.cuda.synchronize()
+    L.tgt_timing_enable(0)
+    kernels = {nm: {"avg_us": t / c * 1e3, "launches": c} for nm, (t, c) in _lib.kernel_timings().items() if c}
+    ms_sparse = timed(step_sparse)
+    esize = 2 if args.dtype == "bf16" else 4
+    R = H * d * esize
+    # every node row once per pass; a tile is 8 bytes; fp32 tile sums written and read once per pass
+    alg = 12 * n * R + 8 * n * H + 3 * 8 * len(tiles) + 2 * 4 * (n * H * d * 4 + n * H)
+    result = {
+        "metric": "fwd+bwd block attention (16x16 tiles on MFMA + sparse remainder) edges/sec; ms/layer",
+        "value": E / (ms_block * 1e-3), "unit": "edges/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_block, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic",
+        "config": {"workload": "configs[4]: SBM 64 x 4096 reordered by the reference's blockize (k=64, 16x16 blocks)",
+                   "N": n, "tiles": int(len(tiles)), "E_expanded": E, "E_remainder": int(raw.shape[1]), "H": H, "d": d,
+                   "step": "tgt_block_attn_fwd + tgt_block_attn_bwd", "parallelism": "1 GPU"},
+        "roofline": {"bound": "hbm", "kernel": "whole step", "achieved": alg / (ms_block * 1e-3) / 1e9,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": alg / (ms_block * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "traffic": None, "alg_bytes": alg},
+        "kernels": kernels,
+        "sparse_path_same_edges_ms": ms_sparse,
+        "reorder_ms": reorder_ms,
+    }
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -205,10 +294,12 @@ def main():
     H, d = 8, 8
     tdt = torch.float32 if args.dtype == "f32" else torch.bfloat16
     esize = 4 if args.dtype == "f32" else 2
-    if args.workload in ("config3", "config4", "config5") and "--dtype" not in sys.argv:
+    if args.workload in ("config3", "config4", "config5", "config5-blockized") and "--dtype" not in sys.argv:
         args.dtype = "bf16"              # the dtype those configurations are quoted on
     if args.workload == "config4":
         return bench_dense(args)
+    if args.workload == "config5-blockized":
+        return bench_block(args)
     if args.workload in ("config3", "config5"):
         args.no_cpu_baseline = True      # the CPU restatement needs minutes per step at this size
     e, n, label, desc = build_workload(args.workload)

@@ -12,6 +12,7 @@ constexpr int kWave = 64;            // CDNA wavefront width
 constexpr int kBlock = 256;          // threads per workgroup of the attention kernels (4 waves)
 constexpr int kWaveRowMax = 256;     // a row of up to this many edges is walked by (part of) one wave
 constexpr int kBlockSeg = 1024;      // longer rows are walked by whole workgroups, in segments of at most this many edges
+constexpr int kSpreadSegs = 8;       // rows with more segments than this are spread over all XCDs
 constexpr int kNumClass = 5;         // wave item length classes: >32, <=32, <=16, <=8, <=4
 
 void set_error(const char* fmt, ...);
@@ -43,6 +44,9 @@ struct Side {
     int32_t* part2split = nullptr;  // [n_parts] index into split_row of the row a partial slot belongs to
     int32_t n_items = 0, n_split = 0, n_parts = 0;
     int32_t n_block_items = 0;      // items [0, n_block_items) are walked by one workgroup each
+    int32_t n_spread_items = 0;     // the first of them: segments of rows with more than kSpreadSegs segments,
+                                    // handed to the XCDs round-robin
+    int32_t blk_chunk[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0};   // the others cut into 8 contiguous runs of equal edge count
     int32_t class_off[kNumClass + 1] = {0, 0, 0, 0, 0, 0};   // item index where each wave class begins
 };
 

@@ -109,7 +109,8 @@ static int build_schedule(const std::vector<int32_t>& rowptr, int64_t N, Side& s
     const int kWaveRowMax = env_int("TGT_WAVE_ROW_MAX", tgt::kWaveRowMax);
     const int kBlockSeg = env_int("TGT_BLOCK_SEG", tgt::kBlockSeg);
     std::vector<Item> cls[kNumClass];
-    std::vector<Item> items;
+    std::vector<Item> items;       // segments of very long rows: spread over all XCDs
+    std::vector<Item> local;       // other workgroup items: contiguous runs per XCD
     std::vector<int32_t> split_row, split_off, part2split;
     int32_t n_parts = 0;
     for (int64_t r = 0; r < N; ++r) {
@@ -120,20 +121,36 @@ static int build_schedule(const std::vector<int32_t>& rowptr, int64_t N, Side& s
         }
         const int nseg = (len + kBlockSeg - 1) / kBlockSeg;
         if (nseg == 1) {
-            items.push_back(Item{(int32_t)r, b, len, -1});
+            local.push_back(Item{(int32_t)r, b, len, -1});
             continue;
         }
+        std::vector<Item>& where = nseg > kSpreadSegs ? items : local;
         const int seg = (len + nseg - 1) / nseg;
         split_off.push_back(n_parts);
         for (int s = 0; s < nseg; ++s) {
             const int o = s * seg;
             const int l = (o + seg <= len) ? seg : (len - o);
             part2split.push_back((int32_t)split_row.size());
-            items.push_back(Item{(int32_t)r, b + o, l, n_parts++});
+            where.push_back(Item{(int32_t)r, b + o, l, n_parts++});
         }
         split_row.push_back((int32_t)r);
     }
     split_off.push_back(n_parts);
+    side.n_spread_items = (int32_t)items.size();
+    {   // 8 contiguous runs of the other workgroup items with (nearly) equal numbers of edges, one per XCD
+        const int32_t base = side.n_spread_items;
+        int64_t total = 0;
+        for (const Item& it : local) total += it.len;
+        int64_t run = 0;
+        int x = 1;
+        side.blk_chunk[0] = base;
+        for (size_t i = 0; i < local.size() && x < 8; ++i) {
+            run += local[i].len;
+            while (x < 8 && run * 8 >= total * x) side.blk_chunk[x++] = base + (int32_t)(i + 1);
+        }
+        while (x <= 8) side.blk_chunk[x++] = base + (int32_t)local.size();
+    }
+    items.insert(items.end(), local.begin(), local.end());
     side.n_block_items = (int32_t)items.size();
     for (int c = 0; c < kNumClass; ++c) {
         side.class_off[c] = (int32_t)items.size();

@@ -17,6 +17,7 @@
 // last-arriving workgroup adds in a fixed order.
 #include "common.h"
 #include <stdlib.h>
+#include <algorithm>
 
 namespace tgt {
 
@@ -119,6 +120,9 @@ struct SideArgs {
     const float* initZ;
     const uint8_t* cover; // [N] 1 where the row has such sums
     int32_t n_block_items;
+    int32_t n_spread;                    // workgroup items [0, n_spread) go to the XCDs round-robin
+    int32_t spread_pad;                  // n_spread rounded up to a multiple of 8
+    int32_t blk_chunk[9];                // XCD x walks workgroup items [blk_chunk[x], blk_chunk[x+1])
     int32_t n_wave_blocks;               // multiple of 8
     int32_t class_off[kNumClass + 1];    // item index where each wave class begins
     int32_t nwaves[kNumClass];           // waves of each class
@@ -274,27 +278,28 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
 }
 
 // Final value of a row from its sums, written by the LPE lanes that own the chunks.
-template <typename T, int LPE, int LPH, int MODE>
+template <typename T, int LPE, int LPH, int MODE, bool TILES>
 __device__ __forceinline__ void write_row(const Common& c, const SideArgs& s, const int row, const int el,
                                           Acc& acc) {
     constexpr int H = LPE / LPH;
     constexpr int HD = LPE * 8;
     const int64_t row_off = (int64_t)row * HD + el * 8;
-    const bool extra = s.init0 != nullptr && s.cover[row] != 0;
     if (MODE != MODE_FWD) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc.a0[i] *= c.inv_scale;
     }
-    if (extra) {
-        float t[8];
-        load8(s.init0 + row_off, t);
+    if (TILES) {   // sums of the dense tiles of the block path for this row, if it has any
+        if (s.cover[row] != 0) {
+            float t[8];
+            load8(s.init0 + row_off, t);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc.a0[i] += t[i];
-        if (MODE == MODE_FWD) acc.z += s.initZ[(int64_t)row * H + el / LPH];
-        if (MODE == MODE_BWD_SRC) {
-            load8(s.init1 + row_off, t);
+            for (int i = 0; i < 8; ++i) acc.a0[i] += t[i];
+            if (MODE == MODE_FWD) acc.z += s.initZ[(int64_t)row * H + el / LPH];
+            if (MODE == MODE_BWD_SRC) {
+                load8(s.init1 + row_off, t);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) acc.a1[i] += t[i];
+                for (int i = 0; i < 8; ++i) acc.a1[i] += t[i];
+            }
         }
     }
     if (MODE == MODE_FWD) {
@@ -310,7 +315,7 @@ __device__ __forceinline__ void write_row(const Common& c, const SideArgs& s, co
 }
 
 // Wave items: rows of at most kWaveRowMax edges, 64 / (LPE*S) rows per wave.
-template <typename T, int LPE, int LPH, int S, int MODE, bool HASB>
+template <typename T, int LPE, int LPH, int S, int MODE, bool HASB, bool TILES>
 __device__ __forceinline__ void wave_items(const Common& c, const SideArgs& s, const int item_begin,
                                            const int item_end, const int wave_in_class) {
     constexpr int G = LPE * S;
@@ -324,7 +329,7 @@ __device__ __forceinline__ void wave_items(const Common& c, const SideArgs& s, c
     if (valid) it = s.items[item];
     Acc acc;
     walk_range<T, LPE, LPH, S, MODE, HASB>(c, s, it.row, it.start, it.len, slot, el, valid, acc);
-    if (valid && slot == 0) write_row<T, LPE, LPH, MODE>(c, s, it.row, el, acc);
+    if (valid && slot == 0) write_row<T, LPE, LPH, MODE, TILES>(c, s, it.row, el, acc);
 }
 
 // Wave items, XCD-aware.  Workgroups go to the 8 XCDs round-robin (workgroup id mod 8), each
@@ -333,7 +338,7 @@ __device__ __forceinline__ void wave_items(const Common& c, const SideArgs& s, c
 // every class, longest class first: rows that are neighbours in the schedule meet in one L2.
 // `block` counts from the start of this view's wave region, which begins at a workgroup id
 // that is a multiple of 8.
-template <typename T, int LPE, int LPH, int MODE, bool HASB>
+template <typename T, int LPE, int LPH, int MODE, bool HASB, bool TILES>
 __device__ __forceinline__ void wave_block(const Common& c, const SideArgs& s, const int block) {
     const int xcd = block & 7;
     const int v = (block >> 3) * (kBlock / kWave) + (threadIdx.x >> 6);   // wave slot inside the XCD
@@ -346,11 +351,11 @@ __device__ __forceinline__ void wave_block(const Common& c, const SideArgs& s, c
     if (w >= s.nwaves[cls]) return;
     const int b = s.class_off[cls], e = s.class_off[cls + 1];
     switch (cls) {
-        case 0: wave_items<T, LPE, LPH, slots_for_class(LPE, 0), MODE, HASB>(c, s, b, e, w); break;
-        case 1: wave_items<T, LPE, LPH, slots_for_class(LPE, 1), MODE, HASB>(c, s, b, e, w); break;
-        case 2: wave_items<T, LPE, LPH, slots_for_class(LPE, 2), MODE, HASB>(c, s, b, e, w); break;
-        case 3: wave_items<T, LPE, LPH, slots_for_class(LPE, 3), MODE, HASB>(c, s, b, e, w); break;
-        default: wave_items<T, LPE, LPH, slots_for_class(LPE, 4), MODE, HASB>(c, s, b, e, w); break;
+        case 0: wave_items<T, LPE, LPH, slots_for_class(LPE, 0), MODE, HASB, TILES>(c, s, b, e, w); break;
+        case 1: wave_items<T, LPE, LPH, slots_for_class(LPE, 1), MODE, HASB, TILES>(c, s, b, e, w); break;
+        case 2: wave_items<T, LPE, LPH, slots_for_class(LPE, 2), MODE, HASB, TILES>(c, s, b, e, w); break;
+        case 3: wave_items<T, LPE, LPH, slots_for_class(LPE, 3), MODE, HASB, TILES>(c, s, b, e, w); break;
+        default: wave_items<T, LPE, LPH, slots_for_class(LPE, 4), MODE, HASB, TILES>(c, s, b, e, w); break;
     }
 }
 
@@ -371,7 +376,7 @@ struct BlockLds {
 // slot, and the workgroup that arrives last adds the slots in slot order and
 // writes the row - no second launch, no floating-point atomics, and the order of
 // the additions does not depend on which workgroup is last.
-template <typename T, int LPE, int LPH, int MODE, bool HASB>
+template <typename T, int LPE, int LPH, int MODE, bool HASB, bool TILES>
 __device__ __forceinline__ void block_item(const Common& c, const SideArgs& s, const int item,
                                            BlockLds<LPE>& lds) {
     constexpr int S = slots_for_class(LPE, 0);
@@ -418,7 +423,7 @@ __device__ __forceinline__ void block_item(const Common& c, const SideArgs& s, c
             if (MODE == MODE_FWD) acc.z += r[2 * HD + tid];
         }
         if (it.part < 0) {
-            write_row<T, LPE, LPH, MODE>(c, s, it.row, tid, acc);
+            write_row<T, LPE, LPH, MODE, TILES>(c, s, it.row, tid, acc);
         } else {
             float* p = s.part + (int64_t)it.part * PS;
             store8(p + tid * 8, acc.a0);
@@ -483,50 +488,65 @@ __device__ __forceinline__ void block_item(const Common& c, const SideArgs& s, c
             }
             if (MODE == MODE_FWD) acc.z += r[2 * HD + tid];
         }
-        write_row<T, LPE, LPH, MODE>(c, s, it.row, tid, acc);
+        write_row<T, LPE, LPH, MODE, TILES>(c, s, it.row, tid, acc);
         if (tid == 0) s.counters[sidx] = 0;   // ready for the next call
     }
 }
 
 // Forward: workgroup items of the destination view first (longest work first),
 // then its wave items.
-template <typename T, int LPE, int LPH, bool HASB>
+template <typename T, int LPE, int LPH, bool HASB, bool TILES>
 __global__ __launch_bounds__(kBlock) void k_attn_fwd(const Common c, const SideArgs s, const int items_pad) {
     __shared__ BlockLds<LPE> lds;
     const int b = blockIdx.x;
     if (b < items_pad) {
         // workgroup items are in row order; XCD x (= workgroup id mod 8) takes the x-th contiguous
-        // eighth of them, so the rows of a cluster (and the segments of a split row) share an L2
-        const int it = (b & 7) * (items_pad >> 3) + (b >> 3);
-        if (it < s.n_block_items) block_item<T, LPE, LPH, MODE_FWD, HASB>(c, s, it, lds);
+        // run of them (runs of equal edge count), so the rows of a cluster share an L2
+        if (b < s.spread_pad) {
+            if (b < s.n_spread) block_item<T, LPE, LPH, MODE_FWD, HASB, TILES>(c, s, b, lds);
+        } else {
+            const int bb = b - s.spread_pad;
+            const int it = s.blk_chunk[bb & 7] + (bb >> 3);
+            if (it < s.blk_chunk[(bb & 7) + 1]) block_item<T, LPE, LPH, MODE_FWD, HASB, TILES>(c, s, it, lds);
+        }
     } else {
-        wave_block<T, LPE, LPH, MODE_FWD, HASB>(c, s, b - items_pad);
+        wave_block<T, LPE, LPH, MODE_FWD, HASB, TILES>(c, s, b - items_pad);
     }
 }
 
 // Backward: both views in one launch (they are independent once nd is known):
 // workgroup items of the destination view, workgroup items of the source view,
 // wave items of the destination view, wave items of the source view.
-template <typename T, int LPE, int LPH, bool HASB>
+template <typename T, int LPE, int LPH, bool HASB, bool TILES>
 __global__ __launch_bounds__(kBlock) void k_attn_bwd(const Common c, const SideArgs sd, const SideArgs ss,
                                                      const int pad_d, const int pad_s) {
     __shared__ BlockLds<LPE> lds;
     int b = blockIdx.x;
     if (b < pad_d) {
-        const int it = (b & 7) * (pad_d >> 3) + (b >> 3);
-        if (it < sd.n_block_items) block_item<T, LPE, LPH, MODE_BWD_DST, HASB>(c, sd, it, lds);
+        if (b < sd.spread_pad) {
+            if (b < sd.n_spread) block_item<T, LPE, LPH, MODE_BWD_DST, HASB, TILES>(c, sd, b, lds);
+        } else {
+            const int bb = b - sd.spread_pad;
+            const int it = sd.blk_chunk[bb & 7] + (bb >> 3);
+            if (it < sd.blk_chunk[(bb & 7) + 1]) block_item<T, LPE, LPH, MODE_BWD_DST, HASB, TILES>(c, sd, it, lds);
+        }
         return;
     }
     b -= pad_d;
     if (b < pad_s) {
-        const int it = (b & 7) * (pad_s >> 3) + (b >> 3);
-        if (it < ss.n_block_items) block_item<T, LPE, LPH, MODE_BWD_SRC, HASB>(c, ss, it, lds);
+        if (b < ss.spread_pad) {
+            if (b < ss.n_spread) block_item<T, LPE, LPH, MODE_BWD_SRC, HASB, TILES>(c, ss, b, lds);
+        } else {
+            const int bb = b - ss.spread_pad;
+            const int it = ss.blk_chunk[bb & 7] + (bb >> 3);
+            if (it < ss.blk_chunk[(bb & 7) + 1]) block_item<T, LPE, LPH, MODE_BWD_SRC, HASB, TILES>(c, ss, it, lds);
+        }
         return;
     }
     b -= pad_s;
-    if (b < sd.n_wave_blocks) { wave_block<T, LPE, LPH, MODE_BWD_DST, HASB>(c, sd, b); return; }
+    if (b < sd.n_wave_blocks) { wave_block<T, LPE, LPH, MODE_BWD_DST, HASB, TILES>(c, sd, b); return; }
     b -= sd.n_wave_blocks;
-    wave_block<T, LPE, LPH, MODE_BWD_SRC, HASB>(c, ss, b);
+    wave_block<T, LPE, LPH, MODE_BWD_SRC, HASB, TILES>(c, ss, b);
 }
 
 // Per-node side vector of the backward: nd[i,h] = (1 / (Z[i,h] + eps), sum_c dout[i,h,c] out[i,h,c]).
@@ -578,6 +598,9 @@ static void fill_side(SideArgs& a, const Side& s, int lpe) {
     a.items = s.items; a.col = s.col; a.eid = s.eid;
     a.split_off = s.split_off; a.part2split = s.part2split;
     a.n_block_items = s.n_block_items;
+    for (int x = 0; x < 9; ++x) a.blk_chunk[x] = s.blk_chunk[x];
+    a.n_spread = s.n_spread_items;
+    a.spread_pad = (s.n_spread_items + 7) & ~7;
     int slots = 0;
     for (int c = 0; c < kNumClass; ++c) {
         a.class_off[c] = s.class_off[c];
@@ -594,7 +617,16 @@ static void fill_side(SideArgs& a, const Side& s, int lpe) {
     const char* il = getenv("TGT_XCD_INTERLEAVE");
     a.interleave = (il && il[0] == '1') ? 1 : 0;
 }
-static inline int pad8(int x) { return (x + 7) & ~7; }
+// workgroups needed so that every XCD can walk its run of workgroup items
+static inline int blk_grid(const Side& s) {
+    int m = 0;
+    for (int x = 0; x < 8; ++x) m = std::max(m, s.blk_chunk[x + 1] - s.blk_chunk[x]);
+    return ((s.n_spread_items + 7) & ~7) + 8 * m;
+}
+// shapes for which the variant that adds the block path's tile sums is compiled
+template <int LPE, int LPH>
+constexpr bool kTilesShape = (LPE == 8 && LPH == 1) || (LPE == 8 && LPH == 2) || (LPE == 16 && LPH == 2) ||
+                             (LPE == 2 && LPH == 1);
 
 struct Call {
     const tgt_plan* plan;
@@ -626,14 +658,24 @@ static int run_fwd(const Call& c) {
     if (c.init) { a.init0 = c.init->acc; a.initZ = c.init->Z; a.cover = c.init->cover_dst; }
     a.part = reinterpret_cast<float*>(c.ws + L.fwd_part);
     a.counters = reinterpret_cast<int32_t*>(c.ws + L.counters);
-    const int items_pad = pad8(a.n_block_items);
+    const int items_pad = blk_grid(c.plan->dst);
     const int nb = items_pad + a.n_wave_blocks;
     if (nb > 0) {
         KernelTimer t(KS_FWD, c.st);
-        if (c.bias_mode != TGT_BIAS_NONE)
-            hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
-        else
-            hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
+        const bool hb = c.bias_mode != TGT_BIAS_NONE;
+        if (c.init != nullptr) {
+            if constexpr (kTilesShape<LPE, LPH>) {
+                if (hb) hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, true, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
+                else hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, false, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
+            } else {
+                set_error("block attention: no kernel for this (H, d)");
+                return TGT_ERR_UNSUPPORTED;
+            }
+        } else if (hb) {
+            hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, true, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
+        } else {
+            hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, false, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
+        }
     }
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
@@ -671,14 +713,24 @@ static int run_bwd(const Call& c) {
     if (c.init) { ss.init0 = c.init->dk; ss.init1 = c.init->dv; ss.cover = c.init->cover_src; }
     ss.part = reinterpret_cast<float*>(c.ws + L.dkv_part);
     ss.counters = counters + 2 * c.plan->dst.n_split;
-    const int pad_d = pad8(sd.n_block_items), pad_s = pad8(ss.n_block_items);
+    const int pad_d = blk_grid(c.plan->dst), pad_s = blk_grid(c.plan->src);
     const int nb = pad_d + pad_s + sd.n_wave_blocks + ss.n_wave_blocks;
     if (nb > 0) {
         KernelTimer t(KS_BWD, c.st);
-        if (c.bias_mode != TGT_BIAS_NONE)
-            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
-        else
-            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
+        const bool hb = c.bias_mode != TGT_BIAS_NONE;
+        if (c.init != nullptr) {
+            if constexpr (kTilesShape<LPE, LPH>) {
+                if (hb) hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, true, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
+                else hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, false, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
+            } else {
+                set_error("block attention: no kernel for this (H, d)");
+                return TGT_ERR_UNSUPPORTED;
+            }
+        } else if (hb) {
+            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, true, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
+        } else {
+            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, false, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
+        }
     }
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
