@@ -53,8 +53,8 @@ def kernel_alg_bytes(name, N, E, H, d, esize, bpe):
 # profiles/sparse_attn_config2_hbm_traffic_pmc.txt.  Counters cannot be read from inside this process,
 # so the figures are carried here and only reported for the workload / dtype they were measured on.
 MEASURED_TRAFFIC = {
-    ("config2", "f32"): {"attn_fwd": 254.3e6, "bwd_node_side": 38.9e6, "attn_bwd": 638.5e6},
-    ("config2", "bf16"): {"attn_fwd": 143.1e6, "bwd_node_side": 22.6e6, "attn_bwd": 378.2e6},
+    ("config2", "f32"): {"attn_fwd": 251.8e6, "bwd_node_side": 38.9e6, "attn_bwd": 633.2e6},
+    ("config2", "bf16"): {"attn_fwd": 137.5e6, "bwd_node_side": 22.5e6, "attn_bwd": 367.6e6},
 }
 
 
