@@ -518,7 +518,7 @@ __global__ __launch_bounds__(kBlock) void k_attn_fwd(const Common c, const SideA
 // workgroup items of the destination view, workgroup items of the source view,
 // wave items of the destination view, wave items of the source view.
 template <typename T, int LPE, int LPH, bool HASB, bool TILES>
-__global__ __launch_bounds__(kBlock) void k_attn_bwd(const Common c, const SideArgs sd, const SideArgs ss,
+__global__ __launch_bounds__(kBlock, 4) void k_attn_bwd(const Common c, const SideArgs sd, const SideArgs ss,
                                                      const int pad_d, const int pad_s) {
     __shared__ BlockLds<LPE> lds;
     int b = blockIdx.x;
