@@ -110,6 +110,44 @@ def cpu_baseline(e, n, H, d, seconds_budget=25.0):
             "ms_per_step": med * 1e3}
 
 
+def gather_probe(plan, n, E, row_bytes, stream, repeats=20):
+    """Rate the memory system sustains for the bare access pattern of the forward walk: the same
+    source rows in the same (destination-sorted) order, k then v (two tables of n rows of
+    row_bytes each), read by the library's row-gather probe kernel: no index chain, no arithmetic,
+    no outputs.  Also the same number of uniformly random rows.  Returns None if the row size
+    has no probe variant."""
+    import torch
+    from torchgt_amd import _lib
+    if row_bytes not in (128, 256):
+        return None
+    dev = torch.device("cuda:0")
+    L = _lib.lib()
+    col = torch.from_numpy(plan.export(_lib.PLAN_COL_DST)).to(dev, torch.int32)
+    idx_real = torch.cat([col, col + n]).contiguous()
+    idx_real = idx_real[: idx_real.numel() // 4 * 4]
+    gen = torch.Generator().manual_seed(7)
+    idx_rand = torch.randint(0, 2 * n, (idx_real.numel(),), generator=gen, dtype=torch.int32).to(dev)
+    table = torch.ones(2 * n * row_bytes // 4, dtype=torch.int32, device=dev)
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    out = {"row_bytes": row_bytes, "table_bytes": 2 * n * row_bytes, "rows_gathered": int(idx_real.numel())}
+    for tag, idx in (("graph_order", idx_real), ("uniform_random", idx_rand)):
+        for _ in range(3):
+            _lib.check(L.tgt_probe_row_gather(table.data_ptr(), 2 * n, row_bytes, idx.data_ptr(), idx.numel(),
+                                              sink.data_ptr(), stream))
+        torch.cuda.synchronize()
+        L.tgt_timing_reset()
+        L.tgt_timing_enable(1)
+        for _ in range(repeats):
+            _lib.check(L.tgt_probe_row_gather(table.data_ptr(), 2 * n, row_bytes, idx.data_ptr(), idx.numel(),
+                                              sink.data_ptr(), stream))
+        torch.cuda.synchronize()
+        L.tgt_timing_enable(0)
+        ms, cnt = _lib.kernel_timings()["probe_row_gather"]
+        us = ms / cnt * 1e3
+        out[tag] = {"avg_us": us, "GB/s": idx.numel() * row_bytes / (us * 1e-6) / 1e9}
+    return out
+
+
 def bench_dense(args):
     """BASELINE configs[3]: dense biased attention on a batch of 256 padded ER graphs (S = 129,
     H = 8, d = 8, bf16, bias [b,H,S,S] with gradient).  A step = tgt_dense_attn_fwd + _bwd."""
@@ -365,6 +403,7 @@ def main():
     L.tgt_timing_enable(0)
     timings = _lib.kernel_timings()
     kernels = {name: {"avg_us": ms / cnt * 1e3, "launches": cnt} for name, (ms, cnt) in timings.items() if cnt}
+    probe = gather_probe(plan, n, E, H * d * esize, stream)
     bpe = H * esize
     dom = max((kk for kk in kernels if kernel_alg_bytes(kk, n, E, H, d, esize, bpe)),
               key=lambda kk: kernels[kk]["avg_us"])
@@ -392,6 +431,8 @@ def main():
                      "alg_bytes": dom_bytes,
                      "avg_us": kernels[dom]["avg_us"]},
         "kernels": kernels,
+        # what a bare gather of the forward walk's k and v rows costs (no arithmetic, no index chain)
+        "row_gather_probe": probe,
         "plan_build_ms": plan_ms, "plan_build_first_ms": plan_first_ms,
     }
     if not args.no_cpu_baseline:

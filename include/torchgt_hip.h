@@ -215,6 +215,17 @@ int tgt_timing_reset(void);
 int tgt_timing_slots(void);
 int tgt_timing_read(int slot, const char** name, double* total_ms, int64_t* launches);
 
+/* ---- row-gather probe ----------------------------------------------------
+ * Measurement aid with no counterpart in the reference.  Launches one kernel in
+ * which every group of 8 lanes reads the rows d_idx[4g .. 4g+3] (row_bytes = 128
+ * or 256, values in [0, n_rows), not checked) of d_table and discards them: the
+ * per-edge k[src] / v[src] access of tgt_sparse_attn_fwd (attn_module.py:146-147)
+ * without arithmetic, index chains or outputs.  Its rate (n_idx * row_bytes over
+ * the "probe_row_gather" timing slot) is what the memory system sustains for
+ * this access pattern at this table size.  d_sink: 4 writable bytes. */
+int tgt_probe_row_gather(const void* d_table, int64_t n_rows, int row_bytes, const int32_t* d_idx,
+                         int64_t n_idx, void* d_sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

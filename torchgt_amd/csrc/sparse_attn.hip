@@ -59,6 +59,25 @@ __device__ __forceinline__ float load1(const bf16_t* p) { return bf16_to_f32(p->
 __device__ __forceinline__ void store1(float* p, float v) { *p = v; }
 __device__ __forceinline__ void store1(bf16_t* p, float v) { p->x = (uint16_t)f32_to_bf16(v); }
 
+// Partial sums of a split row travel between workgroups that may sit on different XCDs, whose L2s
+// are not coherent with each other.  A device-wide fence would write back and invalidate a whole
+// L2 for every segment; instead the few floats of a partial slot are stored and loaded with
+// device-scope accesses (they go through to the memory side), nothing else is disturbed.
+__device__ __forceinline__ void store_dev(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_dev(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store8_dev(float* p, const float (&x)[8]) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) store_dev(p + i, x[i]);
+}
+__device__ __forceinline__ void load8_dev(const float* p, float (&x)[8]) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = load_dev(p + i);
+}
+
 __device__ __forceinline__ float dot8(const float (&a)[8], const float (&b)[8]) {
     float s = a[0] * b[0];
 #pragma unroll
@@ -426,26 +445,26 @@ __device__ __forceinline__ void block_item(const Common& c, const SideArgs& s, c
             write_row<T, LPE, LPH, MODE, TILES>(c, s, it.row, tid, acc);
         } else {
             float* p = s.part + (int64_t)it.part * PS;
-            store8(p + tid * 8, acc.a0);
-            if (MODE == MODE_BWD_SRC) store8(p + HD + tid * 8, acc.a1);
-            if (MODE == MODE_FWD && tid % LPH == 0) p[HD + tid / LPH] = acc.z;
+            store8_dev(p + tid * 8, acc.a0);
+            if (MODE == MODE_BWD_SRC) store8_dev(p + HD + tid * 8, acc.a1);
+            if (MODE == MODE_FWD && tid % LPH == 0) store_dev(p + HD + tid / LPH, acc.z);
         }
     }
     if (it.part < 0) return;   // uniform over the workgroup
 
-    // arrival: the partial slot is published before the counter moves
+    // arrival: the partial slot is published before the counter moves.  Wave 0 holds every writer
+    // of the slot; once its device-scope stores are acknowledged the slot is visible to all XCDs.
     const int sidx = s.part2split[it.part];
     const int p0 = s.split_off[sidx], p1 = s.split_off[sidx + 1];
-    if (tid < kWave) {          // wave 0 holds every writer of the slot
-        __threadfence();
+    if (tid < kWave) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         if (tid == 0) {
-            const int old = atomicAdd(&s.counters[sidx], 1);
+            const int old = __hip_atomic_fetch_add(&s.counters[sidx], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             lds.last = (old == p1 - p0 - 1) ? 1 : 0;
         }
     }
     __syncthreads();
     if (!lds.last) return;
-    __threadfence();
     // last arriver: NGROUP groups of LPE threads add slots p0 + grp2, p0 + grp2 + NGROUP, ...
     constexpr int NGROUP = BlockLds<LPE>::NGROUP;
     const int grp2 = tid / LPE, el2 = tid % LPE;
@@ -456,15 +475,15 @@ __device__ __forceinline__ void block_item(const Common& c, const SideArgs& s, c
         for (int p = p0 + grp2; p < p1; p += NGROUP) {
             const float* src = s.part + (int64_t)p * PS;
             float t0[8], t1[8];
-            load8(src + el2 * 8, t0);
+            load8_dev(src + el2 * 8, t0);
 #pragma unroll
             for (int i = 0; i < 8; ++i) a0[i] += t0[i];
             if (MODE == MODE_BWD_SRC) {
-                load8(src + HD + el2 * 8, t1);
+                load8_dev(src + HD + el2 * 8, t1);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) a1[i] += t1[i];
             }
-            if (MODE == MODE_FWD) z += src[HD + el2 / LPH];
+            if (MODE == MODE_FWD) z += load_dev(src + HD + el2 / LPH);
         }
         float* r = lds.red + grp2 * STRIDE;
 #pragma unroll
