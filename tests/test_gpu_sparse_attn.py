@@ -209,6 +209,32 @@ def test_bitwise_reproducible(cuda):
         assert torch.equal(x, y)
 
 
+def test_split_rows_fresh_inputs_every_call(cuda):
+    """Rows long enough to be split over several workgroups (in both views), called again and
+    again on ONE plan and workspace with new operands: a partial sum left over from an earlier
+    call, or read before it was published, would show against the oracle."""
+    N = 600
+    g = torch.Generator().manual_seed(71)
+    hubs = torch.arange(0, 24)
+    parts = []
+    for h in hubs:   # every hub receives from and sends to 1500..4500 random nodes
+        deg = int(torch.randint(1500, 4500, (1,), generator=g))
+        other = torch.randint(0, N, (deg,), generator=g)
+        parts.append(torch.stack([other, torch.full((deg,), int(h))]))
+        parts.append(torch.stack([torch.full((deg,), int(h)), other]))
+    parts.append(rand_graph(N, 3000, 72))
+    ei = torch.cat(parts, dim=1)
+    ei = ei[:, torch.randperm(ei.shape[1], generator=g)]
+    ei = ei.to(cuda)          # one tensor: the plan (and its workspace) is cached on it
+    plan = GraphPlan(ei, N)
+    info = plan.info()
+    assert info["segments_dst"] >= 48 and info["segments_src"] >= 48
+    plan.close()
+    for call in range(6):
+        for dtype in (torch.float32, torch.bfloat16):
+            run_case(f"split rows call {call}", N, ei, 8, 8, dtype, "edge_head", 700 + call, cuda, scale=0.5)
+
+
 def test_module_api_matches_reference_conventions(cuda):
     # forward(q,k,v,attn_bias,edge_index,'sparse') with [b,S,H,d] and a dense [b,H,S,S] bias,
     # sparse_attention_bias(k,q,v,...) with the k-first order, and the attn_module.py convention

@@ -54,6 +54,30 @@ __device__ __forceinline__ void store8(bf16_t* __restrict__ p, const float (&x)[
     u.w = f32_to_bf16(x[6]) | (f32_to_bf16(x[7]) << 16);
     *reinterpret_cast<uint4*>(p) = u;
 }
+// A gathered row chunk as it arrives from memory.  The walk issues all gathers of a step first and
+// converts only when a value is used: a conversion placed next to its load would make the wave
+// wait for that load before the next one is issued.
+template <typename T> struct Raw8;
+template <> struct Raw8<float> { float x[8]; };
+template <> struct Raw8<bf16_t> { uint4 u; };
+__device__ __forceinline__ void load_raw(const float* __restrict__ p, Raw8<float>& r) { load8(p, r.x); }
+__device__ __forceinline__ void load_raw(const bf16_t* __restrict__ p, Raw8<bf16_t>& r) {
+    r.u = *reinterpret_cast<const uint4*>(p);
+}
+__device__ __forceinline__ void unpack(const Raw8<float>& r, float (&x)[8]) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = r.x[i];
+}
+__device__ __forceinline__ void unpack(const Raw8<bf16_t>& r, float (&x)[8]) {
+    x[0] = bf16_to_f32(r.u.x & 0xffffu); x[1] = __uint_as_float(r.u.x & 0xffff0000u);
+    x[2] = bf16_to_f32(r.u.y & 0xffffu); x[3] = __uint_as_float(r.u.y & 0xffff0000u);
+    x[4] = bf16_to_f32(r.u.z & 0xffffu); x[5] = __uint_as_float(r.u.z & 0xffff0000u);
+    x[6] = bf16_to_f32(r.u.w & 0xffffu); x[7] = __uint_as_float(r.u.w & 0xffff0000u);
+}
+__device__ __forceinline__ float raw1(const float* p) { return *p; }
+__device__ __forceinline__ uint32_t raw1(const bf16_t* p) { return p->x; }
+__device__ __forceinline__ float cvt1(float x) { return x; }
+__device__ __forceinline__ float cvt1(uint32_t x) { return bf16_to_f32(x); }
 __device__ __forceinline__ float load1(const float* p) { return *p; }
 __device__ __forceinline__ float load1(const bf16_t* p) { return bf16_to_f32(p->x); }
 __device__ __forceinline__ void store1(float* p, float v) { *p = v; }
@@ -208,52 +232,85 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
     for (int e0 = slot; e0 < n; e0 += S * kUnroll) {
         int nb[kUnroll], ed[kUnroll];
         bool ok[kUnroll];
-        float x0[kUnroll][8], x1[kUnroll][8], bb[kUnroll];
+        Raw8<T> g0[kUnroll], g1[kUnroll];          // gathered rows, unconverted
+        decltype(raw1(B)) braw[kUnroll];
         float2 ndv[kUnroll];
+        if constexpr (sizeof(T) == 4) {
+            // fp32: lanes past the end of the row load nothing and hold zeros
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                const int e = e0 + u * S;
+                ok[u] = e < n;
+                nb[u] = 0; ed[u] = 0;
+                if (ok[u]) {
+                    nb[u] = col[e];
+                    if (HASB) ed[u] = eid[e];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) {
+                braw[u] = 0;
+                ndv[u] = make_float2(0.f, 0.f);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) { g0[u].x[i] = 0.f; g1[u].x[i] = 0.f; }
+                if (ok[u]) {
+                    const int64_t o = (int64_t)nb[u] * HD + el * 8;
+                    if (MODE == MODE_BWD_SRC) {
+                        load_raw(Q + o, g0[u]);
+                        load_raw(Gd + o, g1[u]);
+                        ndv[u] = c.nd[(int64_t)nb[u] * H + head];
+                    } else {
+                        load_raw(K + o, g0[u]);
+                        load_raw(V + o, g1[u]);
+                    }
+                    if (HASB) braw[u] = raw1(B + (int64_t)ed[u] * bias_se + head * bias_sh);
+                }
+            }
+        } else {
+        // 16-bit rows: lanes past the end of the row repeat its last edge (a line the wave is reading
+        // anyway) and skip the arithmetic; with no lane-dependent branch around them the loads of a
+        // step are issued back to back, and the rows stay packed until they are used.
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             const int e = e0 + u * S;
             ok[u] = e < n;
-            nb[u] = 0; ed[u] = 0;
-            if (ok[u]) {
-                nb[u] = col[e];
-                if (HASB) ed[u] = eid[e];
-            }
+            const int ec = min(e, n - 1);
+            nb[u] = col[ec];
+            ed[u] = HASB ? eid[ec] : 0;
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            bb[u] = 0.f;
-            ndv[u] = make_float2(0.f, 0.f);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) { x0[u][i] = 0.f; x1[u][i] = 0.f; }
-            if (ok[u]) {
-                const int64_t o = (int64_t)nb[u] * HD + el * 8;
-                if (MODE == MODE_BWD_SRC) {
-                    load8(Q + o, x0[u]);
-                    load8(Gd + o, x1[u]);
-                    ndv[u] = c.nd[(int64_t)nb[u] * H + head];
-                } else {
-                    load8(K + o, x0[u]);
-                    load8(V + o, x1[u]);
-                }
-                if (HASB) bb[u] = load1(B + (int64_t)ed[u] * bias_se + head * bias_sh);
+            const int64_t o = (int64_t)nb[u] * HD + el * 8;
+            if (MODE == MODE_BWD_SRC) {
+                load_raw(Q + o, g0[u]);
+                load_raw(Gd + o, g1[u]);
+                ndv[u] = c.nd[(int64_t)nb[u] * H + head];
+            } else {
+                load_raw(K + o, g0[u]);
+                load_raw(V + o, g1[u]);
             }
+            if (HASB) braw[u] = raw1(B + (int64_t)ed[u] * bias_se + head * bias_sh);
+        }
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             if (ok[u]) {
+                float x0[8], x1[8];
+                unpack(g0[u], x0);
+                unpack(g1[u], x1);
+                const float bbu = HASB ? cvt1(braw[u]) : 0.f;
                 // raw score: identical arithmetic in all three walks so that the
                 // recomputed weights and the clamp mask agree bit for bit
-                const float raw = head_sum<LPH>(dot8(r0, x0[u])) * inv_scale;
-                const float w = __expf(clamp5(raw) + bb[u]);
+                const float raw = head_sum<LPH>(dot8(r0, x0)) * inv_scale;
+                const float w = __expf(clamp5(raw) + bbu);
                 if (MODE == MODE_FWD) {
                     acc.z += w;
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) acc.a0[i] = fmaf(w, x1[u][i], acc.a0[i]);
+                    for (int i = 0; i < 8; ++i) acc.a0[i] = fmaf(w, x1[i], acc.a0[i]);
                 } else {
                     const bool inside = (raw >= -5.0f) & (raw <= 5.0f);   // torch clamp backward: inclusive
                     if (MODE == MODE_BWD_DST) {
-                        const float t = head_sum<LPH>(dot8(r1, x1[u]));   // g_dst . v_src
+                        const float t = head_sum<LPH>(dot8(r1, x1));   // g_dst . v_src
                         const float dS = w * rz * (t - Dh);
                         T* __restrict__ dB = static_cast<T*>(s.out1);
                         if (HASB && dB != nullptr) {
@@ -268,16 +325,16 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
                         }
                         const float md = inside ? dS : 0.f;
 #pragma unroll
-                        for (int i = 0; i < 8; ++i) acc.a0[i] = fmaf(md, x0[u][i], acc.a0[i]);
+                        for (int i = 0; i < 8; ++i) acc.a0[i] = fmaf(md, x0[i], acc.a0[i]);
                     } else {
                         const float p = w * ndv[u].x;
-                        const float t = head_sum<LPH>(dot8(x1[u], r1));   // g_dst . v_src
+                        const float t = head_sum<LPH>(dot8(x1, r1));   // g_dst . v_src
                         const float dS = p * (t - ndv[u].y);
                         const float md = inside ? dS : 0.f;
 #pragma unroll
                         for (int i = 0; i < 8; ++i) {
-                            acc.a0[i] = fmaf(md, x0[u][i], acc.a0[i]);   // dk += m dS q_dst
-                            acc.a1[i] = fmaf(p, x1[u][i], acc.a1[i]);    // dv += p g_dst
+                            acc.a0[i] = fmaf(md, x0[i], acc.a0[i]);   // dk += m dS q_dst
+                            acc.a1[i] = fmaf(p, x1[i], acc.a1[i]);    // dv += p g_dst
                         }
                     }
                 }
