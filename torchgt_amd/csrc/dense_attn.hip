@@ -16,9 +16,11 @@
 // and its registers run over keys: the softmax reductions are register-local plus
 // one cross-half shuffle, and the probabilities sit exactly in the B-operand
 // layout of the next product (O^T = V^T P^T), no shuffle or LDS round trip.
-// The bias is staged in LDS strip by strip with 16-byte loads (a strip of 32 query
-// rows is contiguous in memory) and read from there in whichever layout a phase needs.
+// The bias is read straight from global memory in the layout each walk needs (see
+// key_of_row and the backward kernel); only q/k/v/dout heads are staged in LDS.
 #include "common.h"
+#include <algorithm>
+#include <stdlib.h>
 
 namespace tgt {
 
@@ -92,86 +94,99 @@ __device__ __forceinline__ void load_head(const T* __restrict__ X, int g, int h,
     }
 }
 
-// One wave's strip of the bias: rows q0 .. q0+31 of bias[g, h] are CONTIGUOUS in
-// the [b, H, S, S] tensor, so the strip is fetched with 16-byte loads from the
-// aligned-down start and kept in LDS as bf16 with row stride strip_stride(S)
-// (never a multiple of 4 elements, so that 32 lanes reading one key of 32
-// different rows hit different banks).  Chunks that straddle the tensor's ends
-// are read element by element.
-template <int SP> constexpr int strip_elems() { return 32 * (SP + 2) + 16; }
-__device__ __forceinline__ int strip_stride(int S) { return (S & 3) == 0 ? S + 2 : S; }
-
-// Returns the offset of strip element 0 inside `strip` (readers add it).
-template <typename T>
-__device__ __forceinline__ int stage_strip(const T* __restrict__ bias, int64_t e0, int count, int S,
-                                           int64_t total, short* __restrict__ strip, int lane) {
-    constexpr int EPC = 16 / (int)sizeof(T);
-    const int SL = strip_stride(S);
-    const uintptr_t A = reinterpret_cast<uintptr_t>(bias + e0);
-    const uintptr_t A0 = A & ~(uintptr_t)15;
-    const int head = (int)((A - A0) / sizeof(T));
-    const int nchunk = (head + count + EPC - 1) / EPC;
-    const T* base0 = reinterpret_cast<const T*>(A0);
-    const T* t_begin = bias;
-    const T* t_end = bias + total;
-    for (int c = lane; c < nchunk; c += 64) {
-        const T* p = base0 + (int64_t)c * EPC;
-        short vals[EPC];
-        if (p >= t_begin && p + EPC <= t_end) {
-            if (sizeof(T) == 2) {
-                const uint4 u = *reinterpret_cast<const uint4*>(p);
-                vals[0] = (short)(u.x & 0xffffu); vals[1] = (short)(u.x >> 16);
-                vals[2] = (short)(u.y & 0xffffu); vals[3] = (short)(u.y >> 16);
-                vals[4 % EPC] = (short)(u.z & 0xffffu); vals[5 % EPC] = (short)(u.z >> 16);
-                vals[6 % EPC] = (short)(u.w & 0xffffu); vals[7 % EPC] = (short)(u.w >> 16);
-            } else {
-                const float4_t f = *reinterpret_cast<const float4_t*>(p);
-                vals[0] = f2bf(f.x); vals[1] = f2bf(f.y); vals[2] = f2bf(f.z); vals[3] = f2bf(f.w);
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < EPC; ++i) {
-                const T* q = p + i;
-                vals[i] = (q >= t_begin && q < t_end) ? f2bf(ld1(q)) : (short)0;
-            }
-        }
-        if (SL == S) {          // rows stay contiguous: the chunk goes to LDS as it came, shifted by `head`
-#pragma unroll
-            for (int i = 0; i < EPC; ++i) strip[c * EPC + i] = vals[i];
-            continue;
-        }
-        // element i of the chunk is strip element e = c*EPC + i - head: (row, key) = (e / S, e % S)
-        int e = c * EPC - head;
-        int row = e >= 0 ? e / S : -1;
-        int key = e >= 0 ? e - row * S : 0;
-#pragma unroll
-        for (int i = 0; i < EPC; ++i, ++e) {
-            if (e >= 0 && e < count) strip[row * SL + key] = vals[i];
-            if (e >= 0 && ++key == S) { key = 0; ++row; }
-            if (e < 0 && e + 1 == 0) { row = 0; key = 0; }
-        }
+// Sixteen consecutive elements of one bias row, as they come from memory.  A bias row of
+// [b, H, S, S] starts at an arbitrary 2- or 4-byte boundary (S is odd for a batch with a virtual
+// node); gfx950 global loads take any alignment, so a full group is fetched with 16-byte loads
+// and the values are converted when they are used, not when they arrive.
+template <typename T> struct Bias16;
+template <> struct Bias16<dbf16> {
+    uint32_t w[8];
+    __device__ __forceinline__ float get(int r) const {
+        return (r & 1) ? __uint_as_float(w[r >> 1] & 0xffff0000u) : __uint_as_float(w[r >> 1] << 16);
     }
-    return SL == S ? head : 0;
+};
+template <> struct Bias16<float> {
+    float w[16];
+    __device__ __forceinline__ float get(int r) const { return w[r]; }
+};
+// elements p[0 .. n_valid) (n_valid <= 16); the others read as 0
+__device__ __forceinline__ void load_bias16(const dbf16* __restrict__ p, int n_valid, Bias16<dbf16>& b) {
+    if (n_valid >= 16) {
+        // A row of an odd-length bias starts on a 2-byte boundary half of the time, and a vector load
+        // from such an address is split into many cache accesses.  So the nine aligned dwords that
+        // hold the group are loaded and funnel-shifted into place.  (With the shift the ninth dword
+        // holds element 15; its upper half may lie 2 bytes past a tensor that ends there, inside the
+        // allocation's granule.)
+        const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+        const uint32_t* __restrict__ q = reinterpret_cast<const uint32_t*>(a & ~(uintptr_t)3);
+        const uint32_t sh = (uint32_t)(a & 2) * 8;      // 0 or 16 bits
+        uint32_t w9[9];
+        __builtin_memcpy(w9, q, 32);
+        w9[8] = sh ? q[8] : 0u;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) b.w[i] = __builtin_amdgcn_alignbit(w9[i + 1], w9[i], sh);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) b.w[i] = 0;
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            if (r < n_valid) b.w[r >> 1] |= ((uint32_t)p[r].x) << (16 * (r & 1));
+    }
 }
+__device__ __forceinline__ void load_bias16(const float* __restrict__ p, int n_valid, Bias16<float>& b) {
+    if (n_valid >= 16) {
+        __builtin_memcpy(b.w, p, 64);
+    } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) b.w[r] = r < n_valid ? p[r] : 0.f;
+    }
+}
+template <typename T>
+__device__ __forceinline__ void zero_bias16(Bias16<T>& b) {
+#pragma unroll
+    for (int i = 0; i < (int)(sizeof(b.w) / sizeof(b.w[0])); ++i) b.w[i] = 0;
+}
+// raw single elements (the key-major walk of the backward reads one element per query)
+__device__ __forceinline__ uint32_t raw1(const dbf16* p) { return p->x; }
+__device__ __forceinline__ float raw1(const float* p) { return *p; }
+__device__ __forceinline__ float cvt1(uint32_t x) { return __uint_as_float(x << 16); }
+__device__ __forceinline__ float cvt1(float x) { return x; }
+
+// The keys of a 32-key tile are assigned to the rows of the MFMA A operand in a permuted order,
+// row 8j + 4h + t  <->  key 16h + 4j + t, so that in the transposed score tile (lane = query,
+// half h = lane / 32) register r of a lane is key 16h + r: sixteen CONSECUTIVE keys per lane,
+// which is 32 contiguous bytes of that query's bias row.
+__device__ __forceinline__ int key_of_row(int row) { return 16 * ((row >> 2) & 1) + 4 * (row >> 3) + (row & 3); }
+
+// 2^x as the bare hardware instruction (inputs here are <= 0 or row maxima differences; results
+// below the normal range flush to zero, which is what a softmax weight of that size is worth)
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float d;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+    return d;
+}
+
+constexpr float kLog2e = 1.4426950408889634f;
 
 // dynamic LDS sizes (bytes)
 template <int D, int NT> constexpr int fwd_lds_bytes() {
-    return 2 * (rm_elems<D, NT * 32>() + tr_elems<D, NT * 32>() + NT * strip_elems<NT * 32>());
+    return 2 * (rm_elems<D, NT * 32>() + tr_elems<D, NT * 32>());
 }
 template <int D, int NT> constexpr int bwd_lds_bytes() {
-    return 2 * (4 * rm_elems<D, NT * 32>() + 3 * tr_elems<D, NT * 32>() + NT * strip_elems<NT * 32>()) +
-           4 * 2 * NT * 32 + 4 * 8;
+    return 2 * (4 * rm_elems<D, NT * 32>() + 3 * tr_elems<D, NT * 32>()) + 4 * 2 * NT * 32;
 }
 constexpr int kLdsLimit = 160 * 1024;
 
 // ---------------------------------------------------------------------------
-// forward: online softmax over key tiles
+// forward: online softmax over key tiles, in the base-2 domain
 // ---------------------------------------------------------------------------
 template <typename T, int D, int NT>
 __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, const T* __restrict__ K,
                                                        const T* __restrict__ V, const T* __restrict__ bias,
                                                        T* __restrict__ out, float* __restrict__ lse, int S,
-                                                       int H, float scale, int64_t bias_total, int nb) {
+                                                       int H, float scale, int nb) {
     constexpr int KS = D / 8;
     constexpr int SP = NT * 32;
     extern __shared__ __align__(16) char smem[];
@@ -180,61 +195,87 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
     // XCD-aware placement: workgroups go to the 8 XCDs round-robin, and the H heads of a graph
     // share every 128-byte line of q/k/v ([b,S,H,d] layout), so the heads of graph g are given the
     // workgroup ids congruent to g mod 8 inside a window of 8*H ids - same XCD, same L2, same time.
-    const int win = blockIdx.x / (8 * H), rem = blockIdx.x % (8 * H);
+    // Workgroups are persistent: the grid holds as many as the GPU keeps resident and each walks the
+    // (graph, head) pairs pair, pair + gridDim.x, ... (gridDim.x is a multiple of 8, so a workgroup
+    // stays on the XCD its pairs were assigned to).
+    const int total_pairs = ((nb + 7) / 8) * 8 * H;
+    for (int pair = blockIdx.x; pair < total_pairs; pair += gridDim.x) {
+    const int win = pair / (8 * H), rem = pair % (8 * H);
     const int g = win * 8 + (rem & 7), h = rem >> 3;
-    if (g >= nb) return;
+    if (g >= nb) continue;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int col = lane & 31, half = lane >> 5;
-    short* strip = v_tr + tr_elems<D, SP>() + wave * strip_elems<SP>();
     const int q0 = wave * 32, qi = q0 + col;
-    int head = 0;
-    if (bias != nullptr) {
-        const int rows = min(32, S - q0);
-        head = stage_strip<T>(bias, (((int64_t)g * H + h) * S + q0) * S, rows * S, S, bias_total, strip, lane);
-    }
+#ifdef TGT_DENSE_TRACE
+    long long tr_t[12]; int tr_n = 0;
+    tr_t[tr_n++] = clock64();
+#define TR_MARK() tr_t[tr_n++] = clock64()
+#else
+#define TR_MARK()
+#endif
+    const bool qok = qi < S;
+    const bool hasb = bias != nullptr;
+    // this lane's query row of the bias; the first tile's group of it is requested before anything else
+    const T* brow = hasb ? bias + (((int64_t)g * H + h) * S + (qok ? qi : 0)) * S : nullptr;
+    Bias16<T> bcur, bnext;
+    zero_bias16(bcur);
+    zero_bias16(bnext);
+    if (hasb && qok) load_bias16(brow + 16 * half, min(16, S - 16 * half), bcur);
+    TR_MARK();
     load_head<T, D, SP>(K, g, h, S, H, k_rm, nullptr);
     load_head<T, D, SP>(V, g, h, S, H, nullptr, v_tr);
     short4_t bq[KS];
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
         bq[s] = zero4();
-        if (qi < S) bq[s] = ld4(Q + (((int64_t)g * S + qi) * H + h) * D + s * 8 + half * 4);
+        if (qok) bq[s] = ld4(Q + (((int64_t)g * S + qi) * H + h) * D + s * 8 + half * 4);
     }
+    TR_MARK();
     __syncthreads();
-    const short* brow = strip + head + col * strip_stride(S);     // this lane's query row of the bias
-    float m = -INFINITY, l = 0.f;
+    TR_MARK();
+    const int krow = key_of_row(col);            // key (inside a tile) of this lane's A-operand row
+    // Row sums on the matrix unit: with a head dim below 32 the A operand of O^T = V^T P^T has idle
+    // rows, and a row of ones there makes row D of the product the sum of the (bf16-rounded)
+    // probabilities, the very numbers the numerator was built from.  It is C register 4*KS of the lower half.
+    constexpr bool kSumOnMfma = D < 32;
+    const short one_bits = 0x3f80;               // bf16 1.0
+    float m = -INFINITY, l = 0.f;                // running maximum and sum (natural units)
     float16_t o = zero16();
 #pragma unroll 1
     for (int kt = 0; kt < NT; ++kt) {
+        const int kb = kt * 32 + 16 * half;      // this lane's keys: kb .. kb + 15
+        if (kt + 1 < NT && hasb && qok) {        // the next tile's group, a whole tile ahead of its use
+            const int nv = S - (kb + 32);
+            if (nv > 0) load_bias16(brow + kb + 32, min(16, nv), bnext);
+        }
         float16_t sc = zero16();
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
-            const short4_t a = *reinterpret_cast<const short4_t*>(&k_rm[(kt * 32 + col) * D + s * 8 + half * 4]);
+            const short4_t a = *reinterpret_cast<const short4_t*>(&k_rm[(kt * 32 + krow) * D + s * 8 + half * 4]);
             sc = mfma(a, bq[s], sc);
         }
-        float tmax = -INFINITY;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int key = kt * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-            float x = sc[r] * scale;
-            const bool ok = key < S && qi < S;
-            if (bias != nullptr && ok) x += bf2f(brow[key]);
-            if (!ok) x = -INFINITY;
-            sc[r] = x;
-            tmax = fmaxf(tmax, x);
+        for (int r = 0; r < 16; ++r) sc[r] = fmaf(sc[r], scale, bcur.get(r));
+        if (kt * 32 + 32 > S) {                  // the row ends inside this tile (wave-uniform)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sc[r] = kb + r < S ? sc[r] : -INFINITY;
         }
+        float tmax = max3(sc[0], sc[1], sc[2]);
+#pragma unroll
+        for (int r = 3; r < 15; r += 2) tmax = max3(tmax, sc[r], sc[r + 1]);
+        tmax = fmaxf(tmax, sc[15]);
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
         const float m_new = fmaxf(m, tmax);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = __expf(m - m_use);
-        l *= alpha;
+        const float alpha = fast_exp2((m - m_use) * kLog2e);
+        const float nm2 = -m_use * kLog2e;
 #pragma unroll
-        for (int r = 0; r < 4 * KS; ++r) o[r] *= alpha;
+        for (int r = 0; r < 4 * KS + (kSumOnMfma ? 4 : 0); ++r) o[r] *= alpha;
+        if (!kSumOnMfma) l *= alpha;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const float pv = __expf(sc[r] - m_use);
-            sc[r] = pv;
-            l += pv;
+            sc[r] = fast_exp2(fmaf(sc[r], kLog2e, nm2));
+            if (!kSumOnMfma) l += sc[r];
         }
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
@@ -242,13 +283,17 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
             pb.x = f2bf(sc[4 * t + 0]); pb.y = f2bf(sc[4 * t + 1]);
             pb.z = f2bf(sc[4 * t + 2]); pb.w = f2bf(sc[4 * t + 3]);
             short4_t av = zero4();
-            if (col < D) av = *reinterpret_cast<const short4_t*>(&v_tr[col * (SP + 4) + kt * 32 + t * 8 + half * 4]);
-            o = mfma(av, pb, o);        // O^T += V^T P^T
+            if (col < D) av = *reinterpret_cast<const short4_t*>(&v_tr[col * (SP + 4) + kb + 4 * t]);
+            if (kSumOnMfma && col == D) { av.x = one_bits; av.y = one_bits; av.z = one_bits; av.w = one_bits; }
+            o = mfma(av, pb, o);        // O^T += V^T P^T (the B operand's keys are kb + 4t .. +3)
         }
         m = m_new;
+        bcur = bnext;
+        TR_MARK();
     }
-    l += __shfl_xor(l, 32);
-    if (qi < S) {
+    if (kSumOnMfma) l = __shfl(o[4 * KS], col);      // row D sits in the lower half's register 4*KS
+    else l += __shfl_xor(l, 32);
+    if (qok) {
         const float inv = 1.0f / l;
         T* op = out + (((int64_t)g * S + qi) * H + h) * D;
 #pragma unroll
@@ -257,23 +302,29 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
                 o[4 * rb + 3] * inv);
         if (half == 0) lse[((int64_t)g * H + h) * S + qi] = (m == -INFINITY ? 0.f : m) + __logf(l);
     }
+#ifdef TGT_DENSE_TRACE
+    if (lane == 0 && pair == blockIdx.x) for (int i = 1; i < tr_n; ++i) lse[((int64_t)g * H + h) * S + wave * 12 + i - 1] = (float)(tr_t[i] - tr_t[0]);
+#endif
+    __syncthreads();     // the LDS images are rewritten for the next pair
+    }
 }
 
 // ---------------------------------------------------------------------------
 // backward
 // ---------------------------------------------------------------------------
 // Wave w first acts on query tile w (transposed scores, lane = query): dQ.  Then
-// on key tile w (direct scores, lane = key): dK, dV and dBias.  The bias is read
-// from HBM once: every wave stages its strip, and the second phase reads all
-// strips from LDS.
+// on key tile w (direct scores, lane = key): dK and dV.  dBias = dS is written by the first walk
+// (a lane holds 16 consecutive keys of one row there: vector stores).  Both walks read the
+// bias straight from global memory in the layout their lanes need (a lane's own row
+// in the first, 32 lanes on 32 consecutive keys of one row in the second); the second
+// read of a (graph, head) slice comes from L2.
 template <typename T, int D, int NT>
 __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, const T* __restrict__ K,
                                                        const T* __restrict__ V, const T* __restrict__ bias,
                                                        const T* __restrict__ O, const float* __restrict__ lse,
                                                        const T* __restrict__ dO, T* __restrict__ dQ,
                                                        T* __restrict__ dK, T* __restrict__ dV,
-                                                       T* __restrict__ dbias, int S, int H, float scale,
-                                                       int64_t bias_total, int nb) {
+                                                       T* __restrict__ dbias, int S, int H, float scale, int nb) {
     constexpr int KS = D / 8;
     constexpr int SP = NT * 32;
     extern __shared__ __align__(16) char smem[];
@@ -285,25 +336,24 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
     short* q_tr = g_rm + RM;
     short* k_tr = q_tr + TR;
     short* g_tr = k_tr + TR;
-    short* strips = g_tr + TR;
-    float* lse_l = reinterpret_cast<float*>(strips + NT * strip_elems<SP>());
+    float* lse_l = reinterpret_cast<float*>(g_tr + TR);   // lse * log2(e)
     float* dd_l = lse_l + SP;
-    int* heads = reinterpret_cast<int*>(dd_l + SP);
-    // XCD-aware placement: workgroups go to the 8 XCDs round-robin, and the H heads of a graph
-    // share every 128-byte line of q/k/v ([b,S,H,d] layout), so the heads of graph g are given the
-    // workgroup ids congruent to g mod 8 inside a window of 8*H ids - same XCD, same L2, same time.
+    // XCD-aware placement as in the forward; one workgroup per (graph, head) pair
     const int win = blockIdx.x / (8 * H), rem = blockIdx.x % (8 * H);
     const int g = win * 8 + (rem & 7), h = rem >> 3;
     if (g >= nb) return;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int col = lane & 31, half = lane >> 5;
-    if (bias != nullptr) {
-        const int q0 = wave * 32;
-        const int rows = min(32, S - q0);
-        const int hd = stage_strip<T>(bias, (((int64_t)g * H + h) * S + q0) * S, rows * S, S, bias_total,
-                                      strips + wave * strip_elems<SP>(), lane);
-        if (lane == 0) heads[wave] = hd;
-    }
+    const bool hasb = bias != nullptr;
+    const T* bias_gh = hasb ? bias + ((int64_t)g * H + h) * S * S : nullptr;
+    // the first query-major group of this lane's bias row, requested before anything else
+    const int qi = wave * 32 + col;
+    const bool qok = qi < S;
+    const T* brow = hasb ? bias_gh + (int64_t)(qok ? qi : 0) * S : nullptr;
+    Bias16<T> bcur, bnext;
+    zero_bias16(bcur);
+    zero_bias16(bnext);
+    if (hasb && qok) load_bias16(brow + 16 * half, min(16, S - 16 * half), bcur);
     load_head<T, D, SP>(Q, g, h, S, H, q_rm, q_tr);
     load_head<T, D, SP>(K, g, h, S, H, k_rm, k_tr);
     load_head<T, D, SP>(V, g, h, S, H, v_rm, nullptr);
@@ -322,53 +372,79 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
                         bf2f(ov.w) * bf2f(gv.w);
             }
         }
-        lse_l[i] = L;
+        lse_l[i] = L * kLog2e;
         dd_l[i] = dsum;          // D[q] = sum_dd dout[q,dd] out[q,dd]
     }
     __syncthreads();
 
     // ---- query tile `wave`: dQ -------------------------------------------------
     {
-        const int q0 = wave * 32, qi = q0 + col;
         short4_t bq[KS], bg[KS];
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
             bq[s] = *reinterpret_cast<const short4_t*>(&q_rm[qi * D + s * 8 + half * 4]);
             bg[s] = *reinterpret_cast<const short4_t*>(&g_rm[qi * D + s * 8 + half * 4]);
         }
-        const float L = lse_l[qi], Dq = dd_l[qi];
-        const short* brow = strips + wave * strip_elems<SP>() + (bias != nullptr ? heads[wave] : 0) + col * strip_stride(S);
+        const float nL2 = -lse_l[qi], Dq = dd_l[qi];
+        const float scale2 = scale * kLog2e;
+        const int krow = key_of_row(col);
+        T* dbrow = dbias != nullptr ? dbias + (((int64_t)g * H + h) * S + (qok ? qi : 0)) * S : nullptr;
         float16_t dq = zero16();
 #pragma unroll 1
         for (int kt = 0; kt < NT; ++kt) {
+            const int kb = kt * 32 + 16 * half;
+            if (kt + 1 < NT && hasb && qok) {
+                const int nv = S - (kb + 32);
+                if (nv > 0) load_bias16(brow + kb + 32, min(16, nv), bnext);
+            }
             float16_t sc = zero16(), dp = zero16();
 #pragma unroll
             for (int s = 0; s < KS; ++s) {
-                const short4_t ak = *reinterpret_cast<const short4_t*>(&k_rm[(kt * 32 + col) * D + s * 8 + half * 4]);
-                const short4_t av = *reinterpret_cast<const short4_t*>(&v_rm[(kt * 32 + col) * D + s * 8 + half * 4]);
+                const short4_t ak = *reinterpret_cast<const short4_t*>(&k_rm[(kt * 32 + krow) * D + s * 8 + half * 4]);
+                const short4_t av = *reinterpret_cast<const short4_t*>(&v_rm[(kt * 32 + krow) * D + s * 8 + half * 4]);
                 sc = mfma(ak, bq[s], sc);     // S^T[key, query]
                 dp = mfma(av, bg[s], dp);     // dP^T[key, query] = V dout^T
             }
+            // p = 2^(s*scale*log2e + (bias*log2e - lse*log2e)); dS^T = p (dP^T - D)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int key = kt * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-                const bool ok = key < S && qi < S;
-                float x = sc[r] * scale;
-                if (bias != nullptr && ok) x += bf2f(brow[key]);
-                const float pv = ok ? __expf(x - L) : 0.f;
-                sc[r] = pv * (dp[r] - Dq);    // dS^T
+                const float pv = fast_exp2(fmaf(sc[r], scale2, fmaf(bcur.get(r), kLog2e, nL2)));
+                sc[r] = pv * (dp[r] - Dq);
+            }
+            if (kt * 32 + 32 > S) {               // the row ends inside this tile (wave-uniform)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sc[r] = kb + r < S ? sc[r] : 0.f;
+            }
+            short4_t db[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                db[t].x = f2bf(sc[4 * t + 0]); db[t].y = f2bf(sc[4 * t + 1]);
+                db[t].z = f2bf(sc[4 * t + 2]); db[t].w = f2bf(sc[4 * t + 3]);
+            }
+            // dBias = dS: this lane holds 16 consecutive keys of its query row, one 32/64-byte piece
+            if (dbrow != nullptr && qok) {
+                if (kb + 16 <= S) {
+                    if (sizeof(T) == 2) {
+                        __builtin_memcpy(dbrow + kb, db, 32);
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) st1(dbrow + kb + r, sc[r]);
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        if (kb + r < S) st1(dbrow + kb + r, sc[r]);
+                }
             }
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-                short4_t db;
-                db.x = f2bf(sc[4 * t + 0]); db.y = f2bf(sc[4 * t + 1]);
-                db.z = f2bf(sc[4 * t + 2]); db.w = f2bf(sc[4 * t + 3]);
                 short4_t ak = zero4();
-                if (col < D) ak = *reinterpret_cast<const short4_t*>(&k_tr[col * (SP + 4) + kt * 32 + t * 8 + half * 4]);
-                dq = mfma(ak, db, dq);        // dQ^T[dd, query] += K^T dS^T
+                if (col < D) ak = *reinterpret_cast<const short4_t*>(&k_tr[col * (SP + 4) + kb + 4 * t]);
+                dq = mfma(ak, db[t], dq);     // dQ^T[dd, query] += K^T dS^T
             }
+            bcur = bnext;
         }
-        if (qi < S) {
+        if (qok) {
             T* p = dQ + (((int64_t)g * S + qi) * H + h) * D;
 #pragma unroll
             for (int rb = 0; rb < KS; ++rb)
@@ -380,15 +456,37 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
     // ---- key tile `wave`: dK, dV, dBias -----------------------------------------
     {
         const int k0 = wave * 32, ki = k0 + col;
+        const bool kok = ki < S;
         short4_t bk[KS], bv[KS];
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
             bk[s] = *reinterpret_cast<const short4_t*>(&k_rm[ki * D + s * 8 + half * 4]);
             bv[s] = *reinterpret_cast<const short4_t*>(&v_rm[ki * D + s * 8 + half * 4]);
         }
+        // register r of a lane is query qt*32 + 8*(r/4) + 4*half + r%4; for one r the 32 lanes of a
+        // half read 32 consecutive keys of that query's bias row (second read of the slice: L2)
+        const T* bcol = hasb ? bias_gh + (kok ? ki : 0) : nullptr;
+        decltype(raw1(bcol)) braw[16], braw_next[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { braw[r] = 0; braw_next[r] = 0; }
+        if (hasb && kok) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int qq = 8 * (r / 4) + 4 * half + (r % 4);
+                if (qq < S) braw[r] = raw1(bcol + (int64_t)qq * S);
+            }
+        }
+        const float scale2 = scale * kLog2e;
         float16_t dk = zero16(), dv = zero16();
 #pragma unroll 1
         for (int qt = 0; qt < NT; ++qt) {
+            if (qt + 1 < NT && hasb && kok) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int qq = (qt + 1) * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+                    if (qq < S) braw_next[r] = raw1(bcol + (int64_t)qq * S);
+                }
+            }
             float16_t sc = zero16(), dp = zero16();
 #pragma unroll
             for (int s = 0; s < KS; ++s) {
@@ -397,21 +495,27 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
                 sc = mfma(aq, bk[s], sc);     // S[query, key]
                 dp = mfma(ag, bv[s], dp);     // dP[query, key] = dout V^T
             }
-            const short* bt = strips + qt * strip_elems<SP>() + (bias != nullptr ? heads[qt] : 0) + ki;
-            const int SL = strip_stride(S);
+            const bool full = qt * 32 + 32 <= S;
             float pr[16];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int qr = 8 * (r / 4) + 4 * half + (r % 4);
-                const int qq = qt * 32 + qr;
-                const bool ok = qq < S && ki < S;
-                float x = sc[r] * scale;
-                if (bias != nullptr && ok) x += bf2f(bt[qr * SL]);
-                const float pv = ok ? __expf(x - lse_l[qq]) : 0.f;
-                const float ds = pv * (dp[r] - dd_l[qq]);
-                if (dbias != nullptr && ok) st1(dbias + (((int64_t)g * H + h) * S + qq) * S + ki, ds);
-                pr[r] = pv;
-                sc[r] = ds;
+            for (int j = 0; j < 4; ++j) {
+                const int qb = qt * 32 + 8 * j + 4 * half;          // four consecutive queries
+                const float4_t L4 = *reinterpret_cast<const float4_t*>(&lse_l[qb]);
+                const float4_t D4 = *reinterpret_cast<const float4_t*>(&dd_l[qb]);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const int r = 4 * j + t;
+                    pr[r] = fast_exp2(fmaf(sc[r], scale2, fmaf(cvt1(braw[r]), kLog2e, -L4[t])));
+                    sc[r] = pr[r] * (dp[r] - D4[t]);
+                }
+            }
+            if (!full) {                          // queries past the end of the batch entry (wave-uniform branch)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const bool in = qt * 32 + 8 * (r / 4) + 4 * half + (r % 4) < S;
+                    pr[r] = in ? pr[r] : 0.f;
+                    sc[r] = in ? sc[r] : 0.f;
+                }
             }
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
@@ -428,8 +532,10 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
                 dk = mfma(aq, db, dk);        // dK^T[dd, key] += Q^T dS
                 dv = mfma(ag, pb, dv);        // dV^T[dd, key] += dout^T P
             }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) braw[r] = braw_next[r];
         }
-        if (ki < S) {
+        if (kok) {
             T* pk = dK + (((int64_t)g * S + ki) * H + h) * D;
             T* pv = dV + (((int64_t)g * S + ki) * H + h) * D;
 #pragma unroll
@@ -463,8 +569,7 @@ static int launch_dense(const DenseCall& c, bool bwd) {
         return TGT_ERR_UNSUPPORTED;
     } else {
         const float scale = sqrtf((float)c.d);     // the reference MULTIPLIES q by sqrt(d)
-        const dim3 grid((unsigned)(((c.b + 7) / 8) * 8 * c.H)), block(64 * NT);
-        const int64_t bias_total = (int64_t)c.b * c.H * c.S * c.S;
+        const dim3 block(64 * NT);
         static bool attr_done = false;     // raise the dynamic-LDS cap once per instantiation
         if (!attr_done) {
             if (lds_f > 48 * 1024)
@@ -475,15 +580,29 @@ static int launch_dense(const DenseCall& c, bool bwd) {
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds_b));
             attr_done = true;
         }
+        const int total_pairs = ((c.b + 7) / 8) * 8 * c.H;
+        // Forward: a persistent grid of about three workgroups per CU (measured best; more resident
+        // workgroups only add cache pressure), a multiple of 8 (one share per XCD).  Backward: one
+        // workgroup per pair (it runs longer per pair, persistence does not pay there).
+        static int fwd_grid = 0;
+        if (fwd_grid == 0) {
+            int dev = 0, cus = 0;
+            TGT_HIP_CHECK(hipGetDevice(&dev));
+            TGT_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+            fwd_grid = std::max(8, (3 * cus) & ~7);
+        }
+        int nblk = bwd ? total_pairs : std::min(total_pairs, fwd_grid);
+        if (const char* e = getenv("TGT_DENSE_GRID")) { if (atoi(e) >= 8) nblk = std::min(total_pairs, atoi(e) & ~7); }
+        const dim3 grid((unsigned)nblk);
         if (!bwd) {
             KernelTimer t(KS_DENSE_FWD, c.st);
             hipLaunchKernelGGL((k_dense_fwd<T, D, NT>), grid, block, lds_f, c.st, (const T*)c.q, (const T*)c.k,
-                               (const T*)c.v, (const T*)c.bias, (T*)c.o_out, c.o_lse, c.S, c.H, scale, bias_total, c.b);
+                               (const T*)c.v, (const T*)c.bias, (T*)c.o_out, c.o_lse, c.S, c.H, scale, c.b);
         } else {
             KernelTimer t(KS_DENSE_BWD, c.st);
             hipLaunchKernelGGL((k_dense_bwd<T, D, NT>), grid, block, lds_b, c.st, (const T*)c.q, (const T*)c.k,
                                (const T*)c.v, (const T*)c.bias, (const T*)c.out, c.lse, (const T*)c.dout,
-                               (T*)c.dq, (T*)c.dk, (T*)c.dv, (T*)c.dbias, c.S, c.H, scale, bias_total, c.b);
+                               (T*)c.dq, (T*)c.dk, (T*)c.dv, (T*)c.dbias, c.S, c.H, scale, c.b);
         }
         TGT_HIP_CHECK(hipGetLastError());
         return TGT_OK;
