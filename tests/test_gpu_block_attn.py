@@ -84,6 +84,11 @@ def test_other_shapes(cuda):
     run_case("H4d16", N, tiles, rest, 4, 16, torch.bfloat16, "edge_head", 5, cuda)
     run_case("H8d16", N, tiles, rest, 8, 16, torch.bfloat16, "none", 6, cuda)
     run_case("H2d8", N, tiles, rest, 2, 8, torch.bfloat16, "edge", 7, cuda)
+    # no remaining edges: the tile kernels write the final rows (and zeros on rows without tiles)
+    none = torch.zeros(2, 0, dtype=torch.int64)
+    run_case("H4d16 tiles-only", N, tiles, none, 4, 16, torch.bfloat16, "none", 8, cuda)
+    run_case("H8d16 tiles-only", N, tiles, none, 8, 16, torch.float32, "none", 9, cuda)
+    run_case("H2d8 tiles-only", N, tiles, none, 2, 8, torch.bfloat16, "none", 10, cuda)
 
 
 def test_reference_pipeline_blockize_then_attention(cuda):

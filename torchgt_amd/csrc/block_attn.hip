@@ -53,153 +53,325 @@ __device__ __forceinline__ bshort4 t_pack(const float (&x)[4]) {
     r.x = t_f2bf(x[0]); r.y = t_f2bf(x[1]); r.z = t_f2bf(x[2]); r.w = t_f2bf(x[3]);
     return r;
 }
-// column `c` of four consecutive node rows starting at `row0` (the transposed operand)
-template <typename T>
-__device__ __forceinline__ bshort4 t_ld_col(const T* __restrict__ X, int row0, int h, int H, int D, int c, bool ok) {
-    bshort4 r = t_zero4();
-    if (ok) {
-        r.x = t_ld1(X + ((int64_t)(row0 + 0) * H + h) * D + c);
-        r.y = t_ld1(X + ((int64_t)(row0 + 1) * H + h) * D + c);
-        r.z = t_ld1(X + ((int64_t)(row0 + 2) * H + h) * D + c);
-        r.w = t_ld1(X + ((int64_t)(row0 + 3) * H + h) * D + c);
-    }
-    return r;
+constexpr int kTile = 16;
+constexpr float kTileEps = 1e-6f;   // attn_module.py:187
+
+__device__ __forceinline__ void t_st4(float* p, float a, float b, float c, float d) {
+    bfloat4 r; r.x = a; r.y = b; r.z = c; r.w = d;
+    *reinterpret_cast<bfloat4*>(p) = r;
+}
+__device__ __forceinline__ void t_st4(tbf16* p, float a, float b, float c, float d) {
+    bshort4 r; r.x = t_f2bf(a); r.y = t_f2bf(b); r.z = t_f2bf(c); r.w = t_f2bf(d);
+    *reinterpret_cast<bshort4*>(p) = r;
 }
 
-constexpr int kTile = 16;
+// Rows no tile covers get zeros when the tile kernels write final results (no remaining edges).
+template <typename T>
+__global__ void k_zero_uncovered(const uint8_t* __restrict__ cover, int64_t N, int HD, int H, T* __restrict__ a,
+                                 T* __restrict__ b, float* __restrict__ Z) {
+    const int64_t row = (int64_t)blockIdx.x * (blockDim.x / 8) + threadIdx.x / 8;
+    const int part = threadIdx.x % 8;
+    if (row >= N || cover[row]) return;
+    for (int e = part; e < HD; e += 8) {
+        if (a) a[row * HD + e] = T{};
+        if (b) b[row * HD + e] = T{};
+    }
+    if (Z) for (int h = part; h < H; h += 8) Z[row * H + h] = 0.f;
+}
+// waves (= tile groups) per workgroup of the tile kernels: as many as keep the static LDS under 64 KB
+template <int HD> constexpr int tile_waves() { return HD > 64 ? 2 : 4; }
 
-// One wave per group of tiles that share their 16 destinations: sum w v and Z of the tiles.
-template <typename T, int D>
-__global__ __launch_bounds__(64) void k_tile_fwd(const int32_t* __restrict__ grp_c0, const int32_t* __restrict__ grp_off,
-                                                 const int32_t* __restrict__ tile_r0, const T* __restrict__ Q,
-                                                 const T* __restrict__ K, const T* __restrict__ V,
-                                                 float* __restrict__ acc, float* __restrict__ Zp, int H,
-                                                 float inv_scale) {
-    const int g = blockIdx.x, lane = threadIdx.x;
+// LDS images of a block of 16 node rows (all heads, HD = H*D elements per row, bf16 bits):
+//   row-major   rm[row * (HD + 4) + e]   - the A operand "16 rows x 4 consecutive elements"
+//   transposed  tr[e * 20 + row]         - the A operand "element e x 4 consecutive rows"
+// The strides (HD + 4 and 20 elements) keep the 8-byte reads of 16 lanes on different banks.
+template <int HD> constexpr int rm_size() { return kTile * (HD + 4); }
+template <int HD> constexpr int tr_size() { return HD * 20; }
+
+// Coalesced copy of rows row0 .. row0+15 of X ([N, HD]) into the LDS images (either may be null):
+// every lane fetches 16-byte pieces of consecutive memory.
+template <typename T, int HD>
+__device__ __forceinline__ void stage_rows(const T* __restrict__ X, int row0, short* __restrict__ rm,
+                                           short* __restrict__ tr, int lane) {
+    constexpr int CPR = HD / 8;                     // 8-element pieces per row
+#pragma unroll
+    for (int i = 0; i < (kTile * CPR + 63) / 64; ++i) {
+        const int c = i * 64 + lane;
+        if (kTile * CPR % 64 != 0 && c >= kTile * CPR) break;
+        const int row = c / CPR, e0 = (c % CPR) * 8;
+        const T* p = X + (int64_t)(row0 + row) * HD + e0;
+        short v[8];
+        if (sizeof(T) == 2) {
+            const uint4 u = *reinterpret_cast<const uint4*>(p);
+            v[0] = (short)(u.x & 0xffffu); v[1] = (short)(u.x >> 16);
+            v[2] = (short)(u.y & 0xffffu); v[3] = (short)(u.y >> 16);
+            v[4] = (short)(u.z & 0xffffu); v[5] = (short)(u.z >> 16);
+            v[6] = (short)(u.w & 0xffffu); v[7] = (short)(u.w >> 16);
+        } else {
+            const bfloat4 f0 = *reinterpret_cast<const bfloat4*>(p);
+            const bfloat4 f1 = *reinterpret_cast<const bfloat4*>(reinterpret_cast<const float*>(p) + 4);
+            v[0] = t_f2bf(f0.x); v[1] = t_f2bf(f0.y); v[2] = t_f2bf(f0.z); v[3] = t_f2bf(f0.w);
+            v[4] = t_f2bf(f1.x); v[5] = t_f2bf(f1.y); v[6] = t_f2bf(f1.z); v[7] = t_f2bf(f1.w);
+        }
+        if (rm) {
+            bshort4 lo, hi;
+            lo.x = v[0]; lo.y = v[1]; lo.z = v[2]; lo.w = v[3];
+            hi.x = v[4]; hi.y = v[5]; hi.z = v[6]; hi.w = v[7];
+            *reinterpret_cast<bshort4*>(&rm[row * (HD + 4) + e0]) = lo;
+            *reinterpret_cast<bshort4*>(&rm[row * (HD + 4) + e0 + 4]) = hi;
+        }
+        if (tr) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) tr[(e0 + j) * 20 + row] = v[j];
+        }
+    }
+}
+// A operand "rows x 4 consecutive elements": lane (col, kq) reads row `col`, elements e .. e+3
+template <int HD>
+__device__ __forceinline__ bshort4 a_rows(const short* __restrict__ rm, int col, int e) {
+    return *reinterpret_cast<const bshort4*>(&rm[col * (HD + 4) + e]);
+}
+// A operand "element x 4 consecutive rows": lane reads element e of rows 4kq .. 4kq+3
+__device__ __forceinline__ bshort4 a_cols(const short* __restrict__ tr, int e, int kq) {
+    return *reinterpret_cast<const bshort4*>(&tr[e * 20 + 4 * kq]);
+}
+// in-wave ordering of LDS traffic: the images are written and read by the same wave only
+__device__ __forceinline__ void wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// One wave per group of tiles that share their 16 destinations: sum w v and Z of the tiles, all
+// heads at once.  The K and V rows of a tile are staged in LDS once (coalesced) and every head's
+// two products take their operands from there.
+// FINAL: the tiles are all there is (no remaining edges): the kernel divides by Z + eps and writes
+// the output rows and Z themselves; otherwise it leaves fp32 sums for the sparse kernel to add.
+template <typename T, int D, int H, bool FINAL>
+__global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_fwd(const int32_t* __restrict__ grp_c0,
+                                                              const int32_t* __restrict__ grp_off,
+                                                              const int32_t* __restrict__ tile_r0, int n_groups,
+                                                              const T* __restrict__ Q, const T* __restrict__ K,
+                                                              const T* __restrict__ V, float* __restrict__ acc,
+                                                              float* __restrict__ Zp, T* __restrict__ out,
+                                                              float inv_scale) {
+    constexpr int HD = H * D;
+    constexpr int kTileWaves = tile_waves<HD>();
+    __shared__ short lds[kTileWaves * (rm_size<HD>() + tr_size<HD>())];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int g = blockIdx.x * kTileWaves + wave;
+    if (g >= n_groups) return;
+    short* k_rm = lds + wave * (rm_size<HD>() + tr_size<HD>());
+    short* v_tr = k_rm + rm_size<HD>();
     const int col = lane & 15, kq = lane >> 4;
     const bool kval = kq * 4 < D;
     const int c0 = grp_c0[g], t0 = grp_off[g], t1 = grp_off[g + 1];
+    bshort4 bq[H];
+#pragma unroll
     for (int h = 0; h < H; ++h) {
-        bshort4 bq = t_zero4();
-        if (kval) bq = t_ld4(Q + ((int64_t)(c0 + col) * H + h) * D + kq * 4);
-        bfloat4 o = t_zerof();
-        float z = 0.f;
-        for (int t = t0; t < t1; ++t) {
-            const int r0 = tile_r0[t];
+        bq[h] = t_zero4();
+        if (kval) bq[h] = t_ld4(Q + (int64_t)(c0 + col) * HD + h * D + kq * 4);
+    }
+    bfloat4 o[H];
+    float z[H];
+#pragma unroll
+    for (int h = 0; h < H; ++h) { o[h] = t_zerof(); z[h] = 0.f; }
+    for (int t = t0; t < t1; ++t) {
+        const int r0 = tile_r0[t];
+        wave_lds_fence();                      // the previous tile's reads are done
+        stage_rows<T, HD>(K, r0, k_rm, nullptr, lane);
+        stage_rows<T, HD>(V, r0, nullptr, v_tr, lane);
+        wave_lds_fence();
+#pragma unroll
+        for (int h = 0; h < H; ++h) {
             bshort4 ak = t_zero4();
-            if (kval) ak = t_ld4(K + ((int64_t)(r0 + col) * H + h) * D + kq * 4);
-            const bfloat4 sc = mfma16(ak, bq, t_zerof());          // S^T[source 4kq+r][destination col]
+            if (kval) ak = a_rows<HD>(k_rm, col, h * D + kq * 4);
+            const bfloat4 sc = mfma16(ak, bq[h], t_zerof());       // S^T[source 4kq+r][destination col]
             float w[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 w[r] = __expf(t_clamp5(sc[r] * inv_scale));
-                z += w[r];
+                z[h] += w[r];
             }
-            const bshort4 av = t_ld_col<T>(V, r0 + 4 * kq, h, H, D, col, col < D);
-            o = mfma16(av, t_pack(w), o);                          // O^T[dd 4kq+r][destination col]
+            bshort4 av = t_zero4();
+            if (col < D) av = a_cols(v_tr, h * D + col, kq);
+            o[h] = mfma16(av, t_pack(w), o[h]);                    // O^T[dd 4kq+r][destination col]
         }
-        z += __shfl_xor(z, 16);
-        z += __shfl_xor(z, 32);
-        if (kval) *reinterpret_cast<bfloat4*>(acc + ((int64_t)(c0 + col) * H + h) * D + kq * 4) = o;
-        if (kq == 0) Zp[(int64_t)(c0 + col) * H + h] = z;
+    }
+#pragma unroll
+    for (int h = 0; h < H; ++h) {
+        float zz = z[h];
+        zz += __shfl_xor(zz, 16);
+        zz += __shfl_xor(zz, 32);
+        if (FINAL) {
+            const float inv = 1.0f / (zz + kTileEps);
+            if (kval) t_st4(out + (int64_t)(c0 + col) * HD + h * D + kq * 4, o[h].x * inv, o[h].y * inv, o[h].z * inv, o[h].w * inv);
+        } else if (kval) {
+            *reinterpret_cast<bfloat4*>(acc + (int64_t)(c0 + col) * HD + h * D + kq * 4) = o[h];
+        }
+        if (kq == 0) Zp[(int64_t)(c0 + col) * H + h] = zz;
     }
 }
 
 // Same grouping: dQ of the tiles.  nd[i,h] = (1/(Z+eps), dout.out) of the FINAL output.
-template <typename T, int D>
-__global__ __launch_bounds__(64) void k_tile_bwd_dst(const int32_t* __restrict__ grp_c0, const int32_t* __restrict__ grp_off,
-                                                     const int32_t* __restrict__ tile_r0, const T* __restrict__ Q,
-                                                     const T* __restrict__ K, const T* __restrict__ V,
-                                                     const T* __restrict__ dO, const float2* __restrict__ nd,
-                                                     float* __restrict__ dq_part, int H, float inv_scale) {
-    const int g = blockIdx.x, lane = threadIdx.x;
+template <typename T, int D, int H, bool FINAL>
+__global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_bwd_dst(const int32_t* __restrict__ grp_c0,
+                                                                  const int32_t* __restrict__ grp_off,
+                                                                  const int32_t* __restrict__ tile_r0, int n_groups,
+                                                                  const T* __restrict__ Q, const T* __restrict__ K,
+                                                                  const T* __restrict__ V, const T* __restrict__ dO,
+                                                                  const float2* __restrict__ nd,
+                                                                  float* __restrict__ dq_part, T* __restrict__ dq_out,
+                                                                  float inv_scale) {
+    constexpr int HD = H * D;
+    constexpr int kTileWaves = tile_waves<HD>();
+    constexpr int PER_WAVE = 2 * rm_size<HD>() + tr_size<HD>();
+    __shared__ short lds[kTileWaves * PER_WAVE];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int g = blockIdx.x * kTileWaves + wave;
+    if (g >= n_groups) return;
+    short* k_rm = lds + wave * PER_WAVE;
+    short* v_rm = k_rm + rm_size<HD>();
+    short* k_tr = v_rm + rm_size<HD>();
     const int col = lane & 15, kq = lane >> 4;
     const bool kval = kq * 4 < D;
     const int c0 = grp_c0[g], t0 = grp_off[g], t1 = grp_off[g + 1];
+    bshort4 bq[H], bg[H];
+    float2 ndv[H];
+    bfloat4 dq[H];
+#pragma unroll
     for (int h = 0; h < H; ++h) {
-        bshort4 bq = t_zero4(), bg = t_zero4();
+        bq[h] = t_zero4(); bg[h] = t_zero4();
         if (kval) {
-            bq = t_ld4(Q + ((int64_t)(c0 + col) * H + h) * D + kq * 4);
-            bg = t_ld4(dO + ((int64_t)(c0 + col) * H + h) * D + kq * 4);
+            bq[h] = t_ld4(Q + (int64_t)(c0 + col) * HD + h * D + kq * 4);
+            bg[h] = t_ld4(dO + (int64_t)(c0 + col) * HD + h * D + kq * 4);
         }
-        const float2 ndv = nd[(int64_t)(c0 + col) * H + h];
-        bfloat4 dq = t_zerof();
-        for (int t = t0; t < t1; ++t) {
-            const int r0 = tile_r0[t];
+        ndv[h] = nd[(int64_t)(c0 + col) * H + h];
+        dq[h] = t_zerof();
+    }
+    for (int t = t0; t < t1; ++t) {
+        const int r0 = tile_r0[t];
+        wave_lds_fence();
+        stage_rows<T, HD>(K, r0, k_rm, k_tr, lane);
+        stage_rows<T, HD>(V, r0, v_rm, nullptr, lane);
+        wave_lds_fence();
+#pragma unroll
+        for (int h = 0; h < H; ++h) {
             bshort4 ak = t_zero4(), av = t_zero4();
             if (kval) {
-                ak = t_ld4(K + ((int64_t)(r0 + col) * H + h) * D + kq * 4);
-                av = t_ld4(V + ((int64_t)(r0 + col) * H + h) * D + kq * 4);
+                ak = a_rows<HD>(k_rm, col, h * D + kq * 4);
+                av = a_rows<HD>(v_rm, col, h * D + kq * 4);
             }
-            const bfloat4 sc = mfma16(ak, bq, t_zerof());          // S^T[source][destination]
-            const bfloat4 dp = mfma16(av, bg, t_zerof());          // dP^T = V dout^T
+            const bfloat4 sc = mfma16(ak, bq[h], t_zerof());       // S^T[source][destination]
+            const bfloat4 dp = mfma16(av, bg[h], t_zerof());       // dP^T = V dout^T
             float md[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const float raw = sc[r] * inv_scale;
                 const float wv = __expf(t_clamp5(raw));
-                const float dS = wv * ndv.x * (dp[r] - ndv.y);
+                const float dS = wv * ndv[h].x * (dp[r] - ndv[h].y);
                 md[r] = ((raw >= -5.0f) & (raw <= 5.0f)) ? dS : 0.f;
             }
-            const bshort4 akT = t_ld_col<T>(K, r0 + 4 * kq, h, H, D, col, col < D);
-            dq = mfma16(akT, t_pack(md), dq);                      // dQ^T[dd][destination] += K^T (m dS)^T
+            bshort4 akT = t_zero4();
+            if (col < D) akT = a_cols(k_tr, h * D + col, kq);
+            dq[h] = mfma16(akT, t_pack(md), dq[h]);                // dQ^T[dd][destination] += K^T (m dS)^T
         }
-        if (kval) {
+    }
+    if (kval) {
+#pragma unroll
+        for (int h = 0; h < H; ++h) {
             bfloat4 o;
-            o.x = dq.x * inv_scale; o.y = dq.y * inv_scale; o.z = dq.z * inv_scale; o.w = dq.w * inv_scale;
-            *reinterpret_cast<bfloat4*>(dq_part + ((int64_t)(c0 + col) * H + h) * D + kq * 4) = o;
+            o.x = dq[h].x * inv_scale; o.y = dq[h].y * inv_scale; o.z = dq[h].z * inv_scale; o.w = dq[h].w * inv_scale;
+            if (FINAL) t_st4(dq_out + (int64_t)(c0 + col) * HD + h * D + kq * 4, o.x, o.y, o.z, o.w);
+            else *reinterpret_cast<bfloat4*>(dq_part + (int64_t)(c0 + col) * HD + h * D + kq * 4) = o;
         }
     }
 }
 
 // One wave per group of tiles that share their 16 SOURCES: dK and dV of the tiles.
-template <typename T, int D>
-__global__ __launch_bounds__(64) void k_tile_bwd_src(const int32_t* __restrict__ grp_r0, const int32_t* __restrict__ grp_off,
-                                                     const int32_t* __restrict__ tile_c0, const T* __restrict__ Q,
-                                                     const T* __restrict__ K, const T* __restrict__ V,
-                                                     const T* __restrict__ dO, const float2* __restrict__ nd,
-                                                     float* __restrict__ dk_part, float* __restrict__ dv_part, int H,
-                                                     float inv_scale) {
-    const int g = blockIdx.x, lane = threadIdx.x;
+template <typename T, int D, int H, bool FINAL>
+__global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_bwd_src(const int32_t* __restrict__ grp_r0,
+                                                                  const int32_t* __restrict__ grp_off,
+                                                                  const int32_t* __restrict__ tile_c0, int n_groups,
+                                                                  const T* __restrict__ Q, const T* __restrict__ K,
+                                                                  const T* __restrict__ V, const T* __restrict__ dO,
+                                                                  const float2* __restrict__ nd,
+                                                                  float* __restrict__ dk_part,
+                                                                  float* __restrict__ dv_part, T* __restrict__ dk_out,
+                                                                  T* __restrict__ dv_out, float inv_scale) {
+    constexpr int HD = H * D;
+    constexpr int kTileWaves = tile_waves<HD>();
+    constexpr int PER_WAVE = 2 * rm_size<HD>() + 2 * tr_size<HD>() + 4 * kTile * H;   // + nd tile (float2 = 4 shorts)
+    __shared__ __align__(16) short lds[kTileWaves * PER_WAVE];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int g = blockIdx.x * kTileWaves + wave;
+    if (g >= n_groups) return;
+    short* q_rm = lds + wave * PER_WAVE;
+    short* g_rm = q_rm + rm_size<HD>();
+    short* q_tr = g_rm + rm_size<HD>();
+    short* g_tr = q_tr + tr_size<HD>();
+    float2* nd_l = reinterpret_cast<float2*>(g_tr + tr_size<HD>());     // [16 destinations][H]
     const int col = lane & 15, kq = lane >> 4;
     const bool kval = kq * 4 < D;
     const int r0 = grp_r0[g], t0 = grp_off[g], t1 = grp_off[g + 1];
+    bshort4 bk[H], bv[H];
+    bfloat4 dk[H], dv[H];
+#pragma unroll
     for (int h = 0; h < H; ++h) {
-        bshort4 bk = t_zero4(), bv = t_zero4();
+        bk[h] = t_zero4(); bv[h] = t_zero4();
         if (kval) {
-            bk = t_ld4(K + ((int64_t)(r0 + col) * H + h) * D + kq * 4);
-            bv = t_ld4(V + ((int64_t)(r0 + col) * H + h) * D + kq * 4);
+            bk[h] = t_ld4(K + (int64_t)(r0 + col) * HD + h * D + kq * 4);
+            bv[h] = t_ld4(V + (int64_t)(r0 + col) * HD + h * D + kq * 4);
         }
-        bfloat4 dk = t_zerof(), dv = t_zerof();
-        for (int t = t0; t < t1; ++t) {
-            const int c0 = tile_c0[t];
+        dk[h] = t_zerof(); dv[h] = t_zerof();
+    }
+    for (int t = t0; t < t1; ++t) {
+        const int c0 = tile_c0[t];
+        wave_lds_fence();
+        stage_rows<T, HD>(Q, c0, q_rm, q_tr, lane);
+        stage_rows<T, HD>(dO, c0, g_rm, g_tr, lane);
+        for (int i = lane; i < kTile * H; i += 64) nd_l[i] = nd[(int64_t)c0 * H + i];   // rows c0..c0+15 are contiguous
+        wave_lds_fence();
+#pragma unroll
+        for (int h = 0; h < H; ++h) {
             bshort4 aq = t_zero4(), ag = t_zero4();
             if (kval) {
-                aq = t_ld4(Q + ((int64_t)(c0 + col) * H + h) * D + kq * 4);
-                ag = t_ld4(dO + ((int64_t)(c0 + col) * H + h) * D + kq * 4);
+                aq = a_rows<HD>(q_rm, col, h * D + kq * 4);
+                ag = a_rows<HD>(g_rm, col, h * D + kq * 4);
             }
-            const bfloat4 sc = mfma16(aq, bk, t_zerof());          // S[destination 4kq+r][source col]
-            const bfloat4 dp = mfma16(ag, bv, t_zerof());          // dP = dout V^T
+            const bfloat4 sc = mfma16(aq, bk[h], t_zerof());       // S[destination 4kq+r][source col]
+            const bfloat4 dp = mfma16(ag, bv[h], t_zerof());       // dP = dout V^T
             float pw[4], md[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const float2 ndv = nd[(int64_t)(c0 + 4 * kq + r) * H + h];
+                const float2 ndv = nd_l[(4 * kq + r) * H + h];
                 const float raw = sc[r] * inv_scale;
                 const float p = __expf(t_clamp5(raw)) * ndv.x;
                 const float dS = p * (dp[r] - ndv.y);
                 pw[r] = p;
                 md[r] = ((raw >= -5.0f) & (raw <= 5.0f)) ? dS : 0.f;
             }
-            const bshort4 agT = t_ld_col<T>(dO, c0 + 4 * kq, h, H, D, col, col < D);
-            const bshort4 aqT = t_ld_col<T>(Q, c0 + 4 * kq, h, H, D, col, col < D);
-            dv = mfma16(agT, t_pack(pw), dv);                      // dV^T[dd][source] += dout^T p
-            dk = mfma16(aqT, t_pack(md), dk);                      // dK^T[dd][source] += Q^T (m dS)
+            bshort4 agT = t_zero4(), aqT = t_zero4();
+            if (col < D) {
+                agT = a_cols(g_tr, h * D + col, kq);
+                aqT = a_cols(q_tr, h * D + col, kq);
+            }
+            dv[h] = mfma16(agT, t_pack(pw), dv[h]);                // dV^T[dd][source] += dout^T p
+            dk[h] = mfma16(aqT, t_pack(md), dk[h]);                // dK^T[dd][source] += Q^T (m dS)
         }
-        if (kval) {
+    }
+    if (kval) {
+#pragma unroll
+        for (int h = 0; h < H; ++h) {
             bfloat4 o;
-            o.x = dk.x * inv_scale; o.y = dk.y * inv_scale; o.z = dk.z * inv_scale; o.w = dk.w * inv_scale;
-            *reinterpret_cast<bfloat4*>(dk_part + ((int64_t)(r0 + col) * H + h) * D + kq * 4) = o;
-            *reinterpret_cast<bfloat4*>(dv_part + ((int64_t)(r0 + col) * H + h) * D + kq * 4) = dv;
+            o.x = dk[h].x * inv_scale; o.y = dk[h].y * inv_scale; o.z = dk[h].z * inv_scale; o.w = dk[h].w * inv_scale;
+            if (FINAL) {
+                t_st4(dk_out + (int64_t)(r0 + col) * HD + h * D + kq * 4, o.x, o.y, o.z, o.w);
+                t_st4(dv_out + (int64_t)(r0 + col) * HD + h * D + kq * 4, dv[h].x, dv[h].y, dv[h].z, dv[h].w);
+            } else {
+                *reinterpret_cast<bfloat4*>(dk_part + (int64_t)(r0 + col) * HD + h * D + kq * 4) = o;
+                *reinterpret_cast<bfloat4*>(dv_part + (int64_t)(r0 + col) * HD + h * D + kq * 4) = dv[h];
+            }
         }
     }
 }
@@ -263,39 +435,91 @@ static int upload(DevBuf& b, const std::vector<X>& v, hipStream_t st) {
     return TGT_OK;
 }
 
-template <typename T>
-static int tile_fwd_launch(const tgt_tiles* tl, const void* q, const void* k, const void* v, float* acc, float* Zp,
-                           int H, int d, hipStream_t st) {
-    if (tl->n_dst_groups == 0) return TGT_OK;
-    const float inv_scale = 1.0f / sqrtf((float)d);
+// `final_out` non-null: the tiles are all there is; the kernels write final results (and zeros on
+// rows without tiles) and the sparse kernels are not run.
+template <typename T, int D, int H>
+static int tile_fwd_launch_s(const tgt_tiles* tl, const void* q, const void* k, const void* v, float* acc, float* Zp,
+                             void* final_out, hipStream_t st) {
+    constexpr int W = tile_waves<H * D>();
+    const float inv_scale = 1.0f / sqrtf((float)D);
     KernelTimer t(KS_TILE_FWD, st);
-    if (d == 8)
-        hipLaunchKernelGGL((k_tile_fwd<T, 8>), dim3(tl->n_dst_groups), dim3(64), 0, st, tl->dst_c0.as<int32_t>(),
-                           tl->dst_off.as<int32_t>(), tl->dst_r0.as<int32_t>(), (const T*)q, (const T*)k, (const T*)v,
-                           acc, Zp, H, inv_scale);
-    else
-        hipLaunchKernelGGL((k_tile_fwd<T, 16>), dim3(tl->n_dst_groups), dim3(64), 0, st, tl->dst_c0.as<int32_t>(),
-                           tl->dst_off.as<int32_t>(), tl->dst_r0.as<int32_t>(), (const T*)q, (const T*)k, (const T*)v,
-                           acc, Zp, H, inv_scale);
+    const dim3 grid((tl->n_dst_groups + W - 1) / W), block(64 * W);
+    if (final_out) {
+        hipLaunchKernelGGL((k_zero_uncovered<T>), dim3((unsigned)((tl->N + 31) / 32)), dim3(256), 0, st,
+                           tl->cover_dst.as<uint8_t>(), tl->N, H * D, H, (T*)final_out, (T*)nullptr, Zp);
+        if (tl->n_dst_groups > 0)
+            hipLaunchKernelGGL((k_tile_fwd<T, D, H, true>), grid, block, 0, st, tl->dst_c0.as<int32_t>(),
+                               tl->dst_off.as<int32_t>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
+                               (const T*)k, (const T*)v, acc, Zp, (T*)final_out, inv_scale);
+    } else if (tl->n_dst_groups > 0) {
+        hipLaunchKernelGGL((k_tile_fwd<T, D, H, false>), grid, block, 0, st, tl->dst_c0.as<int32_t>(),
+                           tl->dst_off.as<int32_t>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
+                           (const T*)k, (const T*)v, acc, Zp, (T*)nullptr, inv_scale);
+    }
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
 }
 
-template <typename T, int D>
-static int tile_bwd_launch_d(const tgt_tiles* tl, const void* q, const void* k, const void* v, const void* dout,
-                             const float2* nd, float* dq, float* dk, float* dv, int H, hipStream_t st) {
+template <typename T, int D, int H>
+static int tile_bwd_launch_s(const tgt_tiles* tl, const void* q, const void* k, const void* v, const void* dout,
+                             const float2* nd, float* dq, float* dk, float* dv, void* f_dq, void* f_dk, void* f_dv,
+                             hipStream_t st) {
+    constexpr int W = tile_waves<H * D>();
     const float inv_scale = 1.0f / sqrtf((float)D);
     KernelTimer t(KS_TILE_BWD, st);
-    if (tl->n_dst_groups > 0)
-        hipLaunchKernelGGL((k_tile_bwd_dst<T, D>), dim3(tl->n_dst_groups), dim3(64), 0, st, tl->dst_c0.as<int32_t>(),
-                           tl->dst_off.as<int32_t>(), tl->dst_r0.as<int32_t>(), (const T*)q, (const T*)k, (const T*)v,
-                           (const T*)dout, nd, dq, H, inv_scale);
-    if (tl->n_src_groups > 0)
-        hipLaunchKernelGGL((k_tile_bwd_src<T, D>), dim3(tl->n_src_groups), dim3(64), 0, st, tl->src_r0.as<int32_t>(),
-                           tl->src_off.as<int32_t>(), tl->src_c0.as<int32_t>(), (const T*)q, (const T*)k, (const T*)v,
-                           (const T*)dout, nd, dk, dv, H, inv_scale);
+    const dim3 gd((tl->n_dst_groups + W - 1) / W), gs((tl->n_src_groups + W - 1) / W), block(64 * W);
+    if (f_dq) {
+        const dim3 gz((unsigned)((tl->N + 31) / 32));
+        hipLaunchKernelGGL((k_zero_uncovered<T>), gz, dim3(256), 0, st, tl->cover_dst.as<uint8_t>(), tl->N, H * D, H,
+                           (T*)f_dq, (T*)nullptr, (float*)nullptr);
+        hipLaunchKernelGGL((k_zero_uncovered<T>), gz, dim3(256), 0, st, tl->cover_src.as<uint8_t>(), tl->N, H * D, H,
+                           (T*)f_dk, (T*)f_dv, (float*)nullptr);
+        if (tl->n_dst_groups > 0)
+            hipLaunchKernelGGL((k_tile_bwd_dst<T, D, H, true>), gd, block, 0, st, tl->dst_c0.as<int32_t>(),
+                               tl->dst_off.as<int32_t>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
+                               (const T*)k, (const T*)v, (const T*)dout, nd, dq, (T*)f_dq, inv_scale);
+        if (tl->n_src_groups > 0)
+            hipLaunchKernelGGL((k_tile_bwd_src<T, D, H, true>), gs, block, 0, st, tl->src_r0.as<int32_t>(),
+                               tl->src_off.as<int32_t>(), tl->src_c0.as<int32_t>(), tl->n_src_groups, (const T*)q,
+                               (const T*)k, (const T*)v, (const T*)dout, nd, dk, dv, (T*)f_dk, (T*)f_dv, inv_scale);
+    } else {
+        if (tl->n_dst_groups > 0)
+            hipLaunchKernelGGL((k_tile_bwd_dst<T, D, H, false>), gd, block, 0, st, tl->dst_c0.as<int32_t>(),
+                               tl->dst_off.as<int32_t>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
+                               (const T*)k, (const T*)v, (const T*)dout, nd, dq, (T*)nullptr, inv_scale);
+        if (tl->n_src_groups > 0)
+            hipLaunchKernelGGL((k_tile_bwd_src<T, D, H, false>), gs, block, 0, st, tl->src_r0.as<int32_t>(),
+                               tl->src_off.as<int32_t>(), tl->src_c0.as<int32_t>(), tl->n_src_groups, (const T*)q,
+                               (const T*)k, (const T*)v, (const T*)dout, nd, dk, dv, (T*)nullptr, (T*)nullptr,
+                               inv_scale);
+    }
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
+}
+
+// the (d, H) shapes the tile kernels are compiled for (the same ones the sparse kernels' tile-sum hook has)
+#define TGT_TILE_SHAPES(X) X(8, 8) X(16, 4) X(16, 8) X(8, 2)
+
+template <typename T>
+static int tile_fwd_launch(const tgt_tiles* tl, const void* q, const void* k, const void* v, float* acc, float* Zp,
+                           void* final_out, int H, int d, hipStream_t st) {
+#define X(D_, H_) if (d == D_ && H == H_) return tile_fwd_launch_s<T, D_, H_>(tl, q, k, v, acc, Zp, final_out, st);
+    TGT_TILE_SHAPES(X)
+#undef X
+    set_error("block attention: no tile kernel for H=%d, d=%d", H, d);
+    return TGT_ERR_UNSUPPORTED;
+}
+
+template <typename T>
+static int tile_bwd_launch(const tgt_tiles* tl, const void* q, const void* k, const void* v, const void* dout,
+                           const float2* nd, float* dq, float* dk, float* dv, void* f_dq, void* f_dk, void* f_dv,
+                           int H, int d, hipStream_t st) {
+#define X(D_, H_) \
+    if (d == D_ && H == H_) return tile_bwd_launch_s<T, D_, H_>(tl, q, k, v, dout, nd, dq, dk, dv, f_dq, f_dk, f_dv, st);
+    TGT_TILE_SHAPES(X)
+#undef X
+    set_error("block attention: no tile kernel for H=%d, d=%d", H, d);
+    return TGT_ERR_UNSUPPORTED;
 }
 
 static int check_block(const tgt_tiles* tl, const tgt_plan* plan, int H, int d, int dtype, const void* ws,
@@ -384,9 +608,13 @@ int tgt_block_attn_fwd(const tgt_tiles_t* tiles, const tgt_plan_t* plan, const v
     float* acc = reinterpret_cast<float*>(ws + L.acc);
     float* Zp = reinterpret_cast<float*>(ws + L.Z);
     hipStream_t st = (hipStream_t)stream;
-    rc = dtype == TGT_DTYPE_F32 ? tgt::tile_fwd_launch<float>(tiles, d_q, d_k, d_v, acc, Zp, H, d, st)
-                                : tgt::tile_fwd_launch<tgt::tbf16>(tiles, d_q, d_k, d_v, acc, Zp, H, d, st);
-    if (rc) return rc;
+    // no remaining edges: the tile kernels write out and Z themselves and nothing else runs
+    const bool tiles_only = plan->E == 0;
+    void* fin = tiles_only ? d_out : nullptr;
+    float* Zdst = tiles_only ? d_Z : Zp;
+    rc = dtype == TGT_DTYPE_F32 ? tgt::tile_fwd_launch<float>(tiles, d_q, d_k, d_v, acc, Zdst, fin, H, d, st)
+                                : tgt::tile_fwd_launch<tgt::tbf16>(tiles, d_q, d_k, d_v, acc, Zdst, fin, H, d, st);
+    if (rc || tiles_only) return rc;
     tgt::TileInit init{};
     init.acc = acc; init.Z = Zp; init.cover_dst = tiles->cover_dst.as<uint8_t>();
     return tgt::sparse_attn_fwd_impl(plan, d_q, d_k, d_v, d_bias, bias_mode, H, d, dtype, d_out, d_Z, ws + L.sparse,
@@ -412,13 +640,14 @@ int tgt_block_attn_bwd(const tgt_tiles_t* tiles, const tgt_plan_t* plan, const v
     float* dq = reinterpret_cast<float*>(ws + L.dq);
     float* dk = reinterpret_cast<float*>(ws + L.dk);
     float* dv = reinterpret_cast<float*>(ws + L.dv);
-    if (dtype == TGT_DTYPE_F32)
-        rc = d == 8 ? tgt::tile_bwd_launch_d<float, 8>(tiles, d_q, d_k, d_v, d_dout, nd, dq, dk, dv, H, st)
-                    : tgt::tile_bwd_launch_d<float, 16>(tiles, d_q, d_k, d_v, d_dout, nd, dq, dk, dv, H, st);
-    else
-        rc = d == 8 ? tgt::tile_bwd_launch_d<tgt::tbf16, 8>(tiles, d_q, d_k, d_v, d_dout, nd, dq, dk, dv, H, st)
-                    : tgt::tile_bwd_launch_d<tgt::tbf16, 16>(tiles, d_q, d_k, d_v, d_dout, nd, dq, dk, dv, H, st);
-    if (rc) return rc;
+    const bool tiles_only = plan->E == 0;
+    void* f_dq = tiles_only ? d_dq : nullptr;
+    void* f_dk = tiles_only ? d_dk : nullptr;
+    void* f_dv = tiles_only ? d_dv : nullptr;
+    rc = dtype == TGT_DTYPE_F32
+             ? tgt::tile_bwd_launch<float>(tiles, d_q, d_k, d_v, d_dout, nd, dq, dk, dv, f_dq, f_dk, f_dv, H, d, st)
+             : tgt::tile_bwd_launch<tgt::tbf16>(tiles, d_q, d_k, d_v, d_dout, nd, dq, dk, dv, f_dq, f_dk, f_dv, H, d, st);
+    if (rc || tiles_only) return rc;     // (no edges: there is no per-edge bias gradient to write either)
     tgt::TileInit init{};
     init.dq = dq; init.dk = dk; init.dv = dv;
     init.cover_dst = tiles->cover_dst.as<uint8_t>();
