@@ -53,8 +53,8 @@ def kernel_alg_bytes(name, N, E, H, d, esize, bpe):
 # profiles/sparse_attn_config2_hbm_traffic_pmc.txt.  Counters cannot be read from inside this process,
 # so the figures are carried here and only reported for the workload / dtype they were measured on.
 MEASURED_TRAFFIC = {
-    ("config2", "f32"): {"attn_fwd": 251.8e6, "bwd_node_side": 38.9e6, "attn_bwd": 633.2e6},
-    ("config2", "bf16"): {"attn_fwd": 137.5e6, "bwd_node_side": 22.5e6, "attn_bwd": 367.6e6},
+    ("config2", "f32"): {"attn_fwd": 252.0e6, "bwd_node_side": 38.9e6, "attn_bwd": 636.0e6},
+    ("config2", "bf16"): {"attn_fwd": 137.7e6, "bwd_node_side": 22.6e6, "attn_bwd": 371.7e6},
 }
 
 
@@ -207,7 +207,7 @@ def bench_dense(args):
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": gbs / HBM_PEAK_GBS,
                      # rocprofv3 FETCH_SIZE x2.000 + WRITE_SIZE x1.000, profiles/dense_attn_config4_bf16.txt
-                     "traffic": {"dense_fwd": 86.3e6, "dense_bwd": 171.4e6}.get(dom) if args.dtype == "bf16" else None,
+                     "traffic": {"dense_fwd": 107.5e6, "dense_bwd": 203.9e6}.get(dom) if args.dtype == "bf16" else None,
                      "alg_bytes": alg[dom],
                      "avg_us": kernels[dom]["avg_us"]},
         "mfma": {n: {"alg_tflops": flops[n] / (kernels[n]["avg_us"] * 1e-6) / 1e12, "peak_tflops": 2500.0}
@@ -330,10 +330,10 @@ def main():
         raise SystemExit("bench.py needs a GPU")
     dev = torch.device("cuda:0")
     H, d = 8, 8
-    tdt = torch.float32 if args.dtype == "f32" else torch.bfloat16
-    esize = 4 if args.dtype == "f32" else 2
     if args.workload in ("config3", "config4", "config5", "config5-blockized") and "--dtype" not in sys.argv:
         args.dtype = "bf16"              # the dtype those configurations are quoted on
+    tdt = torch.float32 if args.dtype == "f32" else torch.bfloat16
+    esize = 4 if args.dtype == "f32" else 2
     if args.workload == "config4":
         return bench_dense(args)
     if args.workload == "config5-blockized":
