@@ -110,6 +110,36 @@ def cpu_baseline(e, n, H, d, seconds_budget=25.0):
             "ms_per_step": med * 1e3}
 
 
+def reference_ops_on_gpu(ei, q, k, v, bias, dout, steps=20):
+    """The reference's formulation on this GPU: its chain of stock PyTorch-ROCm ops (gathers,
+    elementwise ops, index_add_ scatter-adds, autograd backward; attn_module.py:146-187), fp32, same
+    inputs.  A datapoint beside the HIP path, not a checker: nothing is compared with it."""
+    import torch
+    H, d = q.shape[1], q.shape[2]
+    src, dst = ei[0], ei[1]
+    qf, kf, vf, bf = (t.detach().float().requires_grad_(True) for t in (q, k, v, bias))
+    g = dout.float()
+
+    def step():
+        s = (kf[src] * qf[dst] / (d ** 0.5)).sum(-1).clamp(-5, 5) + bf
+        w = torch.exp(s)
+        wv = torch.zeros_like(qf).index_add_(0, dst, w.unsqueeze(-1) * vf[src])
+        z = torch.zeros(qf.shape[0], H, device=qf.device).index_add_(0, dst, w)
+        out = wv / (z.unsqueeze(-1) + 1e-6)
+        torch.autograd.grad(out, (qf, kf, vf, bf), g)
+
+    for _ in range(3):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    return {"ms_per_step": ms, "edges_per_s": ei.shape[1] / (ms * 1e-3), "dtype": "f32",
+            "what": "reference op chain with stock PyTorch-ROCm kernels (index gathers + index_add_, autograd)"}
+
+
 def gather_probe(plan, n, E, row_bytes, stream, repeats=20):
     """Rate the memory system sustains for the bare access pattern of the forward walk: the same
     source rows in the same (destination-sorted) order, k then v (two tables of n rows of
@@ -435,6 +465,8 @@ def main():
         "row_gather_probe": probe,
         "plan_build_ms": plan_ms, "plan_build_first_ms": plan_first_ms,
     }
+    if E <= 4_000_000:      # the op chain materialises several [E,H,d] fp32 tensors
+        result["reference_ops_on_gpu"] = reference_ops_on_gpu(ei, q, k, v, bias, dout)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(e, n, H, d)
     print(json.dumps(result))
