@@ -591,8 +591,7 @@ static int launch_dense(const DenseCall& c, bool bwd) {
             TGT_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
             fwd_grid = std::max(8, (3 * cus) & ~7);
         }
-        int nblk = bwd ? total_pairs : std::min(total_pairs, fwd_grid);
-        if (const char* e = getenv("TGT_DENSE_GRID")) { if (atoi(e) >= 8) nblk = std::min(total_pairs, atoi(e) & ~7); }
+        const int nblk = bwd ? total_pairs : std::min(total_pairs, fwd_grid);
         const dim3 grid((unsigned)nblk);
         if (!bwd) {
             KernelTimer t(KS_DENSE_FWD, c.st);

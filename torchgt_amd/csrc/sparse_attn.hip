@@ -171,7 +171,6 @@ struct SideArgs {
     int32_t nwaves[kNumClass];           // waves of each class
     int32_t chunk[kNumClass];            // waves of each class given to one XCD (ceil(nwaves / 8))
     int32_t voff[kNumClass + 1];         // prefix sums of chunk: wave slots of one XCD
-    int32_t interleave;                  // experiment switch: XCD x takes waves x, x+8, ... instead of a chunk
 };
 
 struct Acc {
@@ -423,7 +422,7 @@ __device__ __forceinline__ void wave_block(const Common& c, const SideArgs& s, c
     for (int k = 1; k < kNumClass; ++k) cls += (v >= s.voff[k]) ? 1 : 0;
     cls = __builtin_amdgcn_readfirstlane(cls);
     if (v >= s.voff[kNumClass]) return;
-    const int w = s.interleave ? (v - s.voff[cls]) * 8 + xcd : xcd * s.chunk[cls] + (v - s.voff[cls]);
+    const int w = xcd * s.chunk[cls] + (v - s.voff[cls]);
     if (w >= s.nwaves[cls]) return;
     const int b = s.class_off[cls], e = s.class_off[cls + 1];
     switch (cls) {
@@ -690,8 +689,6 @@ static void fill_side(SideArgs& a, const Side& s, int lpe) {
     a.class_off[kNumClass] = s.class_off[kNumClass];
     a.voff[kNumClass] = slots;
     a.n_wave_blocks = 8 * ((slots + (kBlock / kWave) - 1) / (kBlock / kWave));
-    const char* il = getenv("TGT_XCD_INTERLEAVE");
-    a.interleave = (il && il[0] == '1') ? 1 : 0;
 }
 // workgroups needed so that every XCD can walk its run of workgroup items
 static inline int blk_grid(const Side& s) {
