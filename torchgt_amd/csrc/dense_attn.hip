@@ -206,13 +206,6 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int col = lane & 31, half = lane >> 5;
     const int q0 = wave * 32, qi = q0 + col;
-#ifdef TGT_DENSE_TRACE
-    long long tr_t[12]; int tr_n = 0;
-    tr_t[tr_n++] = clock64();
-#define TR_MARK() tr_t[tr_n++] = clock64()
-#else
-#define TR_MARK()
-#endif
     const bool qok = qi < S;
     const bool hasb = bias != nullptr;
     // this lane's query row of the bias; the first tile's group of it is requested before anything else
@@ -221,7 +214,6 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
     zero_bias16(bcur);
     zero_bias16(bnext);
     if (hasb && qok) load_bias16(brow + 16 * half, min(16, S - 16 * half), bcur);
-    TR_MARK();
     load_head<T, D, SP>(K, g, h, S, H, k_rm, nullptr);
     load_head<T, D, SP>(V, g, h, S, H, nullptr, v_tr);
     short4_t bq[KS];
@@ -230,9 +222,7 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
         bq[s] = zero4();
         if (qok) bq[s] = ld4(Q + (((int64_t)g * S + qi) * H + h) * D + s * 8 + half * 4);
     }
-    TR_MARK();
     __syncthreads();
-    TR_MARK();
     const int krow = key_of_row(col);            // key (inside a tile) of this lane's A-operand row
     // Row sums on the matrix unit: with a head dim below 32 the A operand of O^T = V^T P^T has idle
     // rows, and a row of ones there makes row D of the product the sum of the (bf16-rounded)
@@ -289,8 +279,7 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
         }
         m = m_new;
         bcur = bnext;
-        TR_MARK();
-    }
+        }
     if (kSumOnMfma) l = __shfl(o[4 * KS], col);      // row D sits in the lower half's register 4*KS
     else l += __shfl_xor(l, 32);
     if (qok) {
@@ -302,9 +291,6 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
                 o[4 * rb + 3] * inv);
         if (half == 0) lse[((int64_t)g * H + h) * S + qi] = (m == -INFINITY ? 0.f : m) + __logf(l);
     }
-#ifdef TGT_DENSE_TRACE
-    if (lane == 0 && pair == blockIdx.x) for (int i = 1; i < tr_n; ++i) lse[((int64_t)g * H + h) * S + wave * 12 + i - 1] = (float)(tr_t[i] - tr_t[0]);
-#endif
     __syncthreads();     // the LDS images are rewritten for the next pair
     }
 }
