@@ -3,12 +3,15 @@
 
 A step is one forward + backward of one layer's sparse attention (the C-ABI calls
 tgt_sparse_attn_fwd + tgt_sparse_attn_bwd) on the 64 K-node power-law graph of
-BASELINE.json configs[1]: N = 64 001, E ~ 530 K, H = 8, d = 8, per-edge bias
+the benchmark configuration "configs[1]": N = 64 001, E ~ 530 K, H = 8, d = 8, per-edge bias
 [E, 8] with gradient, inputs resident in HBM, plan prebuilt (its build time is
 reported separately).  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype f32|bf16]
-                    [--workload config2|config1] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype f32|bf16] [--no-cpu-baseline]
+                    [--workload config1|config2|config3|config4|config5|config5-blockized]
+
+config3 / config5: larger sparse workloads (bf16); config4: dense biased attention of a graph-level
+batch; config5-blockized: the block path on the reordered config5 graph.
 """
 import argparse
 import json
@@ -179,7 +182,7 @@ def gather_probe(plan, n, E, row_bytes, stream, repeats=20):
 
 
 def bench_dense(args):
-    """BASELINE configs[3]: dense biased attention on a batch of 256 padded ER graphs (S = 129,
+    """Benchmark configuration configs[3]: dense biased attention on a batch of 256 padded ER graphs (S = 129,
     H = 8, d = 8, bf16, bias [b,H,S,S] with gradient).  A step = tgt_dense_attn_fwd + _bwd."""
     import torch
     from torchgt_amd import _lib, workloads
@@ -248,7 +251,7 @@ def bench_dense(args):
 
 
 def bench_block(args):
-    """BASELINE configs[4] through the reference's pipeline: SBM 64 x 4096, the reference's
+    """Benchmark configuration configs[4] through the reference's pipeline: SBM 64 x 4096, the reference's
     cluster reordering with the clusters as partitions (every partition pair's edges become
     dense 16 x 16 blocks), then attention.  A step = tgt_block_attn_fwd + _bwd on the tile list;
     the same edges through the sparse kernels (expanded list) are timed next to it."""

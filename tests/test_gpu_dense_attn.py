@@ -72,7 +72,7 @@ def test_other_head_dims(cuda, d):
 
 
 def test_config4_batch_with_bias_from_tables(cuda):
-    # BASELINE config 4 (reduced batch for the fp64 oracle): ER graphs padded to 128 + virtual node,
+    # benchmark config 4 (reduced batch for the fp64 oracle): ER graphs padded to 128 + virtual node,
     # bias built by the reference's GraphAttnBias recipe from SPD / edge-type ids and N(0, 0.02) tables
     data = workloads.erdos_renyi_batch(batch=16, seed=42)
     S, H, d, b = data["S"], 8, 8, 16

@@ -78,7 +78,7 @@ def test_config1_barabasi_albert(cuda, dtype, bias_kind):
 
 
 def test_config1_with_learned_spd_table(cuda):
-    # BASELINE config 1: per-edge scalar bias = table[spd id], table ~ N(0, 0.02), grads reach the table
+    # benchmark config 1: per-edge scalar bias = table[spd id], table ~ N(0, 0.02), grads reach the table
     e, n = workloads.barabasi_albert()
     ids = torch.from_numpy(workloads.spd_edge_ids(e))
     ei = torch.from_numpy(e)
