@@ -42,14 +42,20 @@ __global__ void k_convert_validate(const int64_t* __restrict__ src, const int64_
     d32[i] = (uint32_t)d;
 }
 
-// rowptr[r] = first sorted position whose key is >= r.
+// rowptr[r] = first sorted position whose key is >= r (r = 0 .. N): one thread per row, binary
+// search in the sorted keys (a thread per position walking the gap to the next key would leave
+// all the work to one thread when the keys are few or far apart).
 __global__ void k_fill_rowptr(const uint32_t* __restrict__ keys, int64_t E, int64_t N,
                               int32_t* __restrict__ rowptr) {
-    int64_t pos = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (pos > E) return;
-    int64_t prev = pos == 0 ? -1 : (int64_t)keys[pos - 1];
-    int64_t cur = pos == E ? N : (int64_t)keys[pos];
-    for (int64_t r = prev + 1; r <= cur; ++r) rowptr[r] = (int32_t)pos;
+    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (r > N) return;
+    int64_t lo = 0, hi = E;            // answer in [lo, hi]
+    while (lo < hi) {
+        const int64_t mid = (lo + hi) >> 1;
+        if ((int64_t)keys[mid] < r) lo = mid + 1;
+        else hi = mid;
+    }
+    rowptr[r] = (int32_t)lo;
 }
 
 __global__ void k_gather_col(const uint32_t* __restrict__ eid, const uint32_t* __restrict__ other,
@@ -59,6 +65,77 @@ __global__ void k_gather_col(const uint32_t* __restrict__ eid, const uint32_t* _
     uint32_t e = eid[pos];
     col[pos] = (int32_t)other[e];
     eid_out[pos] = (int32_t)e;
+}
+
+// ---------------------------------------------------------------------------
+// schedule kernels: rows are binned on the device, only the few long rows visit the host
+// ---------------------------------------------------------------------------
+constexpr int kSchedCats = kNumClass + 1;   // the wave classes, then "longer than a wave row"
+constexpr int kSchedBlock = 256;
+
+__device__ __forceinline__ int sched_category(int len, int wave_row_max) {
+    if (len > wave_row_max) return kNumClass;
+    if (len > 32) return 0;
+    if (len > 16) return 1;
+    if (len > 8) return 2;
+    if (len > 4) return 3;
+    return 4;
+}
+
+// counts[cat * nblocks + block] = rows of that category among the block's 256 rows
+__global__ __launch_bounds__(kSchedBlock) void k_sched_count(const int32_t* __restrict__ rowptr, int64_t N,
+                                                            int wave_row_max, uint32_t* __restrict__ counts,
+                                                            int nblocks) {
+    __shared__ uint32_t c[kSchedCats];
+    if (threadIdx.x < kSchedCats) c[threadIdx.x] = 0;
+    __syncthreads();
+    const int64_t r = (int64_t)blockIdx.x * kSchedBlock + threadIdx.x;
+    const int cat = r < N ? sched_category(rowptr[r + 1] - rowptr[r], wave_row_max) : -1;
+#pragma unroll
+    for (int k = 0; k < kSchedCats; ++k) {
+        const uint64_t b = __ballot(cat == k);
+        if ((threadIdx.x & 63) == 0 && b) atomicAdd(&c[k], (uint32_t)__popcll(b));   // integer count: order-free
+    }
+    __syncthreads();
+    if (threadIdx.x < kSchedCats) counts[(int64_t)threadIdx.x * nblocks + blockIdx.x] = c[threadIdx.x];
+}
+
+// Rows keep their order inside a category: position = (rows of the category in earlier blocks)
+// + (rank among the block's rows).  Wave-class rows become schedule items at
+// items[class_base[cat] + position]; long rows are listed (row, first edge, length) for the host.
+struct SchedBases { int32_t v[kSchedCats]; };
+__global__ __launch_bounds__(kSchedBlock) void k_sched_fill(const int32_t* __restrict__ rowptr, int64_t N,
+                                                           int wave_row_max, const uint32_t* __restrict__ offs,
+                                                           int nblocks, SchedBases base, Item* __restrict__ items,
+                                                           int32_t* __restrict__ long_rows) {
+    __shared__ uint32_t wave_cnt[kSchedBlock / 64][kSchedCats];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t r = (int64_t)blockIdx.x * kSchedBlock + threadIdx.x;
+    int start = 0, len = 0, cat = -1;
+    if (r < N) {
+        start = rowptr[r];
+        len = rowptr[r + 1] - start;
+        cat = sched_category(len, wave_row_max);
+    }
+    const uint64_t lower = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+    uint32_t rank = 0;
+#pragma unroll
+    for (int k = 0; k < kSchedCats; ++k) {
+        const uint64_t b = __ballot(cat == k);
+        if (cat == k) rank = (uint32_t)__popcll(b & lower);
+        if (lane == 0) wave_cnt[wave][k] = (uint32_t)__popcll(b);
+    }
+    __syncthreads();
+    if (cat < 0) return;
+    uint32_t pos = offs[(int64_t)cat * nblocks + blockIdx.x] + rank;
+    for (int w = 0; w < wave; ++w) pos += wave_cnt[w][cat];
+    if (cat < kNumClass) {
+        if (items) items[(int64_t)base.v[cat] + pos] = Item{(int32_t)r, start, len, -1};
+    } else if (long_rows) {
+        long_rows[3 * (int64_t)pos + 0] = (int32_t)r;
+        long_rows[3 * (int64_t)pos + 1] = start;
+        long_rows[3 * (int64_t)pos + 2] = len;
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -74,7 +151,7 @@ static int build_side(const uint32_t* keys32, const uint32_t* other32, int64_t E
         if (rc) return rc;
     }
     const int T = 256;
-    hipLaunchKernelGGL(k_fill_rowptr, dim3((unsigned)((E + 1 + T - 1) / T)), dim3(T), 0, st, kin, E, N,
+    hipLaunchKernelGGL(k_fill_rowptr, dim3((unsigned)((N + 1 + T - 1) / T)), dim3(T), 0, st, kin, E, N,
                        side.rowptr);
     if (E > 0)
         hipLaunchKernelGGL(k_gather_col, dim3((unsigned)((E + T - 1) / T)), dim3(T), 0, st, vin, other32,
@@ -83,13 +160,6 @@ static int build_side(const uint32_t* keys32, const uint32_t* other32, int64_t E
     return TGT_OK;
 }
 
-static int length_class(int len) {
-    if (len > 32) return 0;
-    if (len > 16) return 1;
-    if (len > 8) return 2;
-    if (len > 4) return 3;
-    return 4;
-}
 
 // Row schedule from a host copy of rowptr.  A row of up to kWaveRowMax edges is
 // one wave item; items are grouped by length class (longest first) and keep row
@@ -104,24 +174,69 @@ static int env_int(const char* name, int dflt) {
     return x > 0 ? x : dflt;
 }
 
-static int build_schedule(const std::vector<int32_t>& rowptr, int64_t N, Side& side, hipStream_t st) {
+// exclusive prefix over the blocks of every category (one workgroup per category) + totals
+__global__ __launch_bounds__(256) void k_sched_scan(uint32_t* __restrict__ counts, int nblocks,
+                                                    uint32_t* __restrict__ totals) {
+    __shared__ uint32_t part[256];
+    const int tid = threadIdx.x;
+    uint32_t* row = counts + (int64_t)blockIdx.x * nblocks;
+    const int chunk = (nblocks + 255) / 256;
+    const int b = tid * chunk, e = min(b + chunk, nblocks);
+    uint32_t sum = 0;
+    for (int i = b; i < e; ++i) sum += row[i];
+    part[tid] = sum;
+    __syncthreads();
+    for (int off = 1; off < 256; off <<= 1) {
+        const uint32_t x = tid >= off ? part[tid - off] : 0u;
+        __syncthreads();
+        part[tid] += x;
+        __syncthreads();
+    }
+    uint32_t run = tid ? part[tid - 1] : 0u;
+    for (int i = b; i < e; ++i) {
+        const uint32_t x = row[i];
+        row[i] = run;
+        run += x;
+    }
+    if (tid == 255) totals[blockIdx.x] = part[255];
+}
+
+static int build_schedule(int64_t N, Side& side, hipStream_t st) {
     // tuning overrides (experiments only; the defaults are the measured best)
     const int kWaveRowMax = env_int("TGT_WAVE_ROW_MAX", tgt::kWaveRowMax);
     const int kBlockSeg = env_int("TGT_BLOCK_SEG", tgt::kBlockSeg);
-    std::vector<Item> cls[kNumClass];
+    const int nblocks = (int)((N + kSchedBlock - 1) / kSchedBlock);
+    DevBuf counts, totals_d, long_d;
+    TGT_HIP_CHECK(counts.alloc(sizeof(uint32_t) * (size_t)kSchedCats * nblocks));
+    TGT_HIP_CHECK(totals_d.alloc(sizeof(uint32_t) * kSchedCats));
+    hipLaunchKernelGGL(k_sched_count, dim3(nblocks), dim3(kSchedBlock), 0, st, side.rowptr, N, kWaveRowMax,
+                       counts.as<uint32_t>(), nblocks);
+    hipLaunchKernelGGL(k_sched_scan, dim3(kSchedCats), dim3(256), 0, st, counts.as<uint32_t>(), nblocks,
+                       totals_d.as<uint32_t>());
+    TGT_HIP_CHECK(hipGetLastError());
+    uint32_t totals[kSchedCats];
+    TGT_HIP_CHECK(hipMemcpyAsync(totals, totals_d.p, sizeof(totals), hipMemcpyDeviceToHost, st));
+    TGT_HIP_CHECK(hipStreamSynchronize(st));
+    // the long rows (few) come to the host, which cuts them into workgroup items
+    const int64_t n_long = totals[kNumClass];
+    std::vector<int32_t> longs((size_t)(3 * n_long));
+    if (n_long > 0) {
+        TGT_HIP_CHECK(long_d.alloc(sizeof(int32_t) * (size_t)(3 * n_long)));
+        hipLaunchKernelGGL(k_sched_fill, dim3(nblocks), dim3(kSchedBlock), 0, st, side.rowptr, N, kWaveRowMax,
+                           counts.as<uint32_t>(), nblocks, SchedBases{}, (Item*)nullptr, long_d.as<int32_t>());
+        TGT_HIP_CHECK(hipGetLastError());
+        TGT_HIP_CHECK(hipMemcpyAsync(longs.data(), long_d.p, sizeof(int32_t) * longs.size(), hipMemcpyDeviceToHost, st));
+        TGT_HIP_CHECK(hipStreamSynchronize(st));
+    }
     std::vector<Item> items;       // segments of very long rows: spread over all XCDs
     std::vector<Item> local;       // other workgroup items: contiguous runs per XCD
     std::vector<int32_t> split_row, split_off, part2split;
     int32_t n_parts = 0;
-    for (int64_t r = 0; r < N; ++r) {
-        const int32_t b = rowptr[r], len = rowptr[r + 1] - b;
-        if (len <= kWaveRowMax) {
-            cls[length_class(len)].push_back(Item{(int32_t)r, b, len, -1});
-            continue;
-        }
+    for (int64_t i = 0; i < n_long; ++i) {
+        const int32_t r = longs[3 * i], b = longs[3 * i + 1], len = longs[3 * i + 2];
         const int nseg = (len + kBlockSeg - 1) / kBlockSeg;
         if (nseg == 1) {
-            local.push_back(Item{(int32_t)r, b, len, -1});
+            local.push_back(Item{r, b, len, -1});
             continue;
         }
         std::vector<Item>& where = nseg > kSpreadSegs ? items : local;
@@ -131,9 +246,9 @@ static int build_schedule(const std::vector<int32_t>& rowptr, int64_t N, Side& s
             const int o = s * seg;
             const int l = (o + seg <= len) ? seg : (len - o);
             part2split.push_back((int32_t)split_row.size());
-            where.push_back(Item{(int32_t)r, b + o, l, n_parts++});
+            where.push_back(Item{r, b + o, l, n_parts++});
         }
-        split_row.push_back((int32_t)r);
+        split_row.push_back(r);
     }
     split_off.push_back(n_parts);
     side.n_spread_items = (int32_t)items.size();
@@ -152,20 +267,23 @@ static int build_schedule(const std::vector<int32_t>& rowptr, int64_t N, Side& s
     }
     items.insert(items.end(), local.begin(), local.end());
     side.n_block_items = (int32_t)items.size();
+    SchedBases base{};
+    int64_t at = side.n_block_items;
     for (int c = 0; c < kNumClass; ++c) {
-        side.class_off[c] = (int32_t)items.size();
-        items.insert(items.end(), cls[c].begin(), cls[c].end());
+        side.class_off[c] = (int32_t)at;
+        base.v[c] = (int32_t)at;
+        at += totals[c];
     }
-    side.class_off[kNumClass] = (int32_t)items.size();
-    side.n_items = (int32_t)items.size();
+    side.class_off[kNumClass] = (int32_t)at;
+    side.n_items = (int32_t)at;
     side.n_split = (int32_t)split_row.size();
     side.n_parts = n_parts;
-    TGT_HIP_CHECK(hipMalloc((void**)&side.items, sizeof(Item) * (items.size() + 1)));
+    TGT_HIP_CHECK(hipMalloc((void**)&side.items, sizeof(Item) * ((size_t)at + 1)));
     TGT_HIP_CHECK(hipMalloc((void**)&side.split_row, sizeof(int32_t) * (split_row.size() + 1)));
     TGT_HIP_CHECK(hipMalloc((void**)&side.split_off, sizeof(int32_t) * split_off.size()));
     TGT_HIP_CHECK(hipMalloc((void**)&side.part2split, sizeof(int32_t) * (part2split.size() + 1)));
-    TGT_HIP_CHECK(hipMemcpyAsync(side.items, items.data(), sizeof(Item) * items.size(),
-                                 hipMemcpyHostToDevice, st));
+    if (!items.empty())
+        TGT_HIP_CHECK(hipMemcpyAsync(side.items, items.data(), sizeof(Item) * items.size(), hipMemcpyHostToDevice, st));
     if (!split_row.empty()) {
         TGT_HIP_CHECK(hipMemcpyAsync(side.split_row, split_row.data(), sizeof(int32_t) * split_row.size(),
                                      hipMemcpyHostToDevice, st));
@@ -174,7 +292,11 @@ static int build_schedule(const std::vector<int32_t>& rowptr, int64_t N, Side& s
     }
     TGT_HIP_CHECK(hipMemcpyAsync(side.split_off, split_off.data(), sizeof(int32_t) * split_off.size(),
                                  hipMemcpyHostToDevice, st));
-    TGT_HIP_CHECK(hipStreamSynchronize(st));   // the host vectors die at return
+    // the wave items (the bulk) are written by the device, in row order inside every class
+    hipLaunchKernelGGL(k_sched_fill, dim3(nblocks), dim3(kSchedBlock), 0, st, side.rowptr, N, kWaveRowMax,
+                       counts.as<uint32_t>(), nblocks, base, side.items, (int32_t*)nullptr);
+    TGT_HIP_CHECK(hipGetLastError());
+    TGT_HIP_CHECK(hipStreamSynchronize(st));   // the host vectors and the scratch buffers die at return
     return TGT_OK;
 }
 
@@ -227,15 +349,9 @@ static int create_impl(const int64_t* d_src, const int64_t* d_dst, int64_t E, in
     if (rc) return rc;
     rc = build_side(s32.as<uint32_t>(), d32.as<uint32_t>(), E, N, sorter, plan->src, st);
     if (rc) return rc;
-    std::vector<int32_t> rp_dst((size_t)N + 1), rp_src((size_t)N + 1);
-    TGT_HIP_CHECK(hipMemcpyAsync(rp_dst.data(), plan->dst.rowptr, sizeof(int32_t) * (N + 1),
-                                 hipMemcpyDeviceToHost, st));
-    TGT_HIP_CHECK(hipMemcpyAsync(rp_src.data(), plan->src.rowptr, sizeof(int32_t) * (N + 1),
-                                 hipMemcpyDeviceToHost, st));
-    TGT_HIP_CHECK(hipStreamSynchronize(st));
-    rc = build_schedule(rp_dst, N, plan->dst, st);
+    rc = build_schedule(N, plan->dst, st);
     if (rc) return rc;
-    return build_schedule(rp_src, N, plan->src, st);
+    return build_schedule(N, plan->src, st);
 }
 
 }  // namespace tgt
