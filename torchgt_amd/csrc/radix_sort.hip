@@ -63,14 +63,20 @@ __global__ __launch_bounds__(256) void k_rs_scan_rows(uint32_t* __restrict__ his
 
 // Stable scatter of one radix pass.  Each wave owns 1024 consecutive keys of the
 // tile and ranks them in 16 rounds of 64; the rank of a key among equal digits is
-// (count in earlier rounds) + (number of lower lanes with the same digit).
+// (count in earlier rounds) + (number of lower lanes with the same digit).  The tile
+// is then put in digit order in LDS (stable), so that the writes to global memory go
+// out as runs of consecutive addresses, one run per digit, instead of one scattered
+// 4-byte store per key.
 __global__ __launch_bounds__(RS_THREADS) void k_rs_scatter(
     const uint32_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in,
     uint32_t* __restrict__ keys_out, uint32_t* __restrict__ vals_out, int64_t n, int shift,
     const uint32_t* __restrict__ hist, const uint32_t* __restrict__ totals, int nblocks) {
     __shared__ uint32_t cnt[4][256];
-    __shared__ uint32_t base[256];
-    __shared__ uint32_t scan[256];
+    __shared__ uint32_t base[256];        // first output position of this tile's keys of a digit
+    __shared__ uint32_t scan[256];        // scan of the global digit totals
+    __shared__ uint32_t tstart[256];      // scan of the tile's digit counts: first LDS slot of a digit
+    __shared__ uint32_t lkey[RS_TILE];
+    __shared__ uint32_t lval[RS_TILE];
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
     const int lane = tid & 63;
@@ -80,7 +86,8 @@ __global__ __launch_bounds__(RS_THREADS) void k_rs_scatter(
 
     volatile uint32_t* wcnt = &cnt[wave][0];
     uint32_t key[RS_ITEMS], rank[RS_ITEMS];
-    const int64_t wbase = (int64_t)blockIdx.x * RS_TILE + (int64_t)wave * RS_WAVE_SPAN;
+    const int64_t tbase = (int64_t)blockIdx.x * RS_TILE;
+    const int64_t wbase = tbase + (int64_t)wave * RS_WAVE_SPAN;
     const uint64_t lower_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
 #pragma unroll
     for (int r = 0; r < RS_ITEMS; ++r) {
@@ -103,31 +110,49 @@ __global__ __launch_bounds__(RS_THREADS) void k_rs_scatter(
         if (valid && lower == 0) wcnt[dg] = prior + (uint32_t)__popcll(same);
     }
     __syncthreads();
-    // exclusive prefix over the 4 waves (thread = digit) and over the 256 digit totals
+    // exclusive prefix over the 4 waves (thread = digit); the tile's count of the digit
     {
-        uint32_t c0 = cnt[0][tid], c1 = cnt[1][tid], c2 = cnt[2][tid];
+        const uint32_t c0 = cnt[0][tid], c1 = cnt[1][tid], c2 = cnt[2][tid], c3 = cnt[3][tid];
         cnt[0][tid] = 0;
         cnt[1][tid] = c0;
         cnt[2][tid] = c0 + c1;
         cnt[3][tid] = c0 + c1 + c2;
+        tstart[tid] = c0 + c1 + c2 + c3;
     }
+    __syncthreads();
+    // inclusive scans over the 256 digits: global totals and tile counts
     for (int off = 1; off < 256; off <<= 1) {
-        uint32_t x = tid >= off ? scan[tid - off] : 0u;
+        const uint32_t x = tid >= off ? scan[tid - off] : 0u;
+        const uint32_t y = tid >= off ? tstart[tid - off] : 0u;
         __syncthreads();
         scan[tid] += x;
+        tstart[tid] += y;
         __syncthreads();
     }
+    const uint32_t my_tstart = tid ? tstart[tid - 1] : 0u;
     base[tid] = (tid ? scan[tid - 1] : 0u) + hist[(int64_t)tid * nblocks + blockIdx.x];
     __syncthreads();
+    tstart[tid] = my_tstart;              // now exclusive
+    __syncthreads();
+    // the tile in digit order (stable) in LDS
 #pragma unroll
     for (int r = 0; r < RS_ITEMS; ++r) {
         const int64_t idx = wbase + r * kWave + lane;
         if (idx < n) {
             const uint32_t dg = (key[r] >> shift) & 255u;
-            const uint32_t pos = base[dg] + cnt[wave][dg] + rank[r];
-            keys_out[pos] = key[r];
-            vals_out[pos] = vals_in ? vals_in[idx] : (uint32_t)idx;
+            const uint32_t slot = tstart[dg] + cnt[wave][dg] + rank[r];
+            lkey[slot] = key[r];
+            lval[slot] = vals_in ? vals_in[idx] : (uint32_t)idx;
         }
+    }
+    __syncthreads();
+    const int tile_n = (int)min((int64_t)RS_TILE, n - tbase);
+    for (int i = tid; i < tile_n; i += RS_THREADS) {
+        const uint32_t kk = lkey[i];
+        const uint32_t dg = (kk >> shift) & 255u;
+        const uint32_t pos = base[dg] + ((uint32_t)i - tstart[dg]);
+        keys_out[pos] = kk;
+        vals_out[pos] = lval[i];
     }
 }
 
