@@ -109,9 +109,44 @@ __global__ void k_invert(const uint32_t* __restrict__ sorted_old, int64_t N, uin
     sorted_out[i] = (int64_t)o;
 }
 
-__global__ void k_count(const uint32_t* __restrict__ keys, int64_t n, unsigned long long* __restrict__ cnt) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) atomicAdd(&cnt[keys[i]], 1ull);   // integer count: order-free
+// Histogram of keys in [0, nbins).  The bins are few (k or k*k partition pairs) and neighbouring
+// keys are often equal, so equal keys of a wave are first merged with ballots (one LDS add per
+// distinct key and wave), workgroups count in LDS, and only non-empty bins reach global memory.
+// Integer counts: the order of the additions does not matter.
+constexpr int kCountLdsBins = 4096;
+__global__ __launch_bounds__(256) void k_count(const uint32_t* __restrict__ keys, int64_t n, int nbins, int key_bits,
+                                               unsigned long long* __restrict__ cnt) {
+    __shared__ uint32_t h[kCountLdsBins];
+    const bool lds = nbins <= kCountLdsBins;
+    if (lds) {
+        for (int b = threadIdx.x; b < nbins; b += blockDim.x) h[b] = 0;
+        __syncthreads();
+    }
+    const int lane = threadIdx.x & 63;
+    const uint64_t lower = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    const int64_t rounds = (n + stride - 1) / stride;          // the same for every thread: ballots need whole waves
+    for (int64_t t = 0; t < rounds; ++t) {
+        const int64_t i = t * stride + (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+        const bool valid = i < n;
+        const uint32_t key = valid ? keys[i] : 0u;
+        uint64_t same = __ballot(valid);
+        for (int b = 0; b < key_bits; ++b) {
+            const bool bit = (key >> b) & 1u;
+            const uint64_t bal = __ballot(bit);
+            same &= bit ? bal : ~bal;
+        }
+        if (valid && (same & lower) == 0) {                    // lowest lane of its group of equal keys
+            const uint32_t c = (uint32_t)__popcll(same);
+            if (lds) atomicAdd(&h[key], c);
+            else atomicAdd(&cnt[key], (unsigned long long)c);
+        }
+    }
+    if (lds) {
+        __syncthreads();
+        for (int b = threadIdx.x; b < nbins; b += blockDim.x)
+            if (h[b]) atomicAdd(&cnt[b], (unsigned long long)h[b]);
+    }
 }
 
 // per-edge keys: pair = part[src]*k + part[dst], s32 = src, d32 = dst
@@ -223,7 +258,8 @@ static int reformat_impl(const int64_t* d_src, const int64_t* d_dst, int64_t E, 
     TGT_HIP_CHECK(cnt_pairs.alloc(sizeof(unsigned long long) * k * k));
     TGT_HIP_CHECK(hipMemsetAsync(cnt_nodes.p, 0, sizeof(unsigned long long) * k, st));
     TGT_HIP_CHECK(hipMemsetAsync(cnt_pairs.p, 0, sizeof(unsigned long long) * k * k, st));
-    hipLaunchKernelGGL(k_count, dim3(nblk(N)), dim3(256), 0, st, p32.as<uint32_t>(), N,
+    const auto count_grid = [](int64_t n) { return dim3((unsigned)std::min<int64_t>(256, (n + 255) / 256)); };
+    hipLaunchKernelGGL(k_count, count_grid(N), dim3(256), 0, st, p32.as<uint32_t>(), N, k, bits_for(k),
                        cnt_nodes.as<unsigned long long>());
     DevBuf pair, s32, d32;
     const size_t eb = sizeof(uint32_t) * (size_t)(E ? E : 1);
@@ -233,8 +269,8 @@ static int reformat_impl(const int64_t* d_src, const int64_t* d_dst, int64_t E, 
     if (E > 0) {
         hipLaunchKernelGGL(k_edge_keys, dim3(nblk(E)), dim3(256), 0, st, d_src, d_dst, E, p32.as<uint32_t>(), k,
                            pair.as<uint32_t>(), s32.as<uint32_t>(), d32.as<uint32_t>());
-        hipLaunchKernelGGL(k_count, dim3(nblk(E)), dim3(256), 0, st, pair.as<uint32_t>(), E,
-                           cnt_pairs.as<unsigned long long>());
+        hipLaunchKernelGGL(k_count, count_grid(E), dim3(256), 0, st, pair.as<uint32_t>(), E, k * k,
+                           bits_for((int64_t)k * k), cnt_pairs.as<unsigned long long>());
     }
     std::vector<unsigned long long> h_nodes(k), h_pairs((size_t)k * k);
     TGT_HIP_CHECK(hipMemcpyAsync(h_nodes.data(), cnt_nodes.p, sizeof(unsigned long long) * k,
