@@ -13,6 +13,7 @@ constexpr int kBlock = 256;          // threads per workgroup of the attention k
 constexpr int kWaveRowMax = 256;     // a row of up to this many edges is walked by (part of) one wave
 constexpr int kBlockSeg = 1024;      // longer rows are walked by whole workgroups, in segments of at most this many edges
 constexpr int kSpreadSegs = 8;       // rows with more segments than this are spread over all XCDs
+constexpr int kSpreadSeg = 512;      // segment length of such a row (it is alone on the critical path: more, shorter segments)
 constexpr int kNumClass = 5;         // wave item length classes: >32, <=32, <=16, <=8, <=4
 
 void set_error(const char* fmt, ...);

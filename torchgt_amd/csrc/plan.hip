@@ -205,6 +205,7 @@ static int build_schedule(int64_t N, Side& side, hipStream_t st) {
     // tuning overrides (experiments only; the defaults are the measured best)
     const int kWaveRowMax = env_int("TGT_WAVE_ROW_MAX", tgt::kWaveRowMax);
     const int kBlockSeg = env_int("TGT_BLOCK_SEG", tgt::kBlockSeg);
+    const int kSpreadSeg = env_int("TGT_SPREAD_SEG", tgt::kSpreadSeg);
     const int nblocks = (int)((N + kSchedBlock - 1) / kSchedBlock);
     DevBuf counts, totals_d, long_d;
     TGT_HIP_CHECK(counts.alloc(sizeof(uint32_t) * (size_t)kSchedCats * nblocks));
@@ -234,7 +235,10 @@ static int build_schedule(int64_t N, Side& side, hipStream_t st) {
     int32_t n_parts = 0;
     for (int64_t i = 0; i < n_long; ++i) {
         const int32_t r = longs[3 * i], b = longs[3 * i + 1], len = longs[3 * i + 2];
-        const int nseg = (len + kBlockSeg - 1) / kBlockSeg;
+        int nseg = (len + kBlockSeg - 1) / kBlockSeg;
+        // a row long enough to be spread over all XCDs is alone on the critical path of the launch:
+        // it gets shorter segments (more workgroups, fewer steps each)
+        if (nseg > kSpreadSegs) nseg = (len + kSpreadSeg - 1) / kSpreadSeg;
         if (nseg == 1) {
             local.push_back(Item{r, b, len, -1});
             continue;
