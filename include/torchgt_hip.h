@@ -204,6 +204,33 @@ int tgt_reformat_export_tiles(const tgt_reformat_t* r, int32_t* h_tiles, int64_t
  * np.random.seed(seed) (legacy MT19937 stream used by gt_sp/utils.py:290-295). */
 int tgt_np_legacy_randint(uint32_t seed, const int64_t* h_highs, int n, int64_t* h_out);
 
+/* ---- projections around the attention -------------------------------------
+ * MultiHeadAttention.forward (models/graphormer_dist_node_level.py:246-273; same
+ * module in models/gt_dist_node_level.py and models/graphormer_dist_graph_level.py):
+ * linear_q / linear_k / linear_v (:255-257, n_out = 3: one pass over x writes q, k
+ * and v in the [N, H, d] layout the attention reads) and output_layer (:271,
+ * n_out = 1).  y_j = x W_j^T + b_j for j < n_out.
+ * d_x: [N, in_features]; d_W[j]: [out_features, in_features] row-major
+ * (nn.Linear.weight); d_b[j]: [out_features] (d_b or an entry may be NULL: no
+ * bias); d_y[j]: [N, out_features]; all of `dtype`, fp32 accumulation.  d_W, d_b,
+ * d_y are HOST arrays of n_out device pointers.  in_features and out_features
+ * must be multiples of 8. */
+int tgt_linear_fwd(const void* d_x, const void* const* d_W, const void* const* d_b, void* const* d_y, int n_out,
+                   int64_t N, int in_features, int out_features, int dtype, void* stream);
+
+/* Backward of the same (autograd of nn.Linear in the reference):
+ *   dx = sum_j dy_j W_j ;  dW_j = dy_j^T x ;  db_j = column sums of dy_j.
+ * d_dx: [N, in_features] or NULL (not wanted).  d_dW: HOST array of n_out device
+ * pointers [out_features, in_features], or NULL (then d_db must be NULL too);
+ * d_db: HOST array of n_out device pointers [out_features] (or NULL, entries may
+ * be NULL).  The weight gradients are summed in a fixed order (same inputs give
+ * the same bits).  d_workspace: tgt_linear_bwd_workspace_bytes(...) bytes,
+ * 16-byte aligned, needed when d_dW is given; contents need no initialisation. */
+int64_t tgt_linear_bwd_workspace_bytes(int n_out, int in_features, int out_features);
+int tgt_linear_bwd(const void* d_x, const void* const* d_W, const void* const* d_dy, int n_out, int64_t N,
+                   int in_features, int out_features, int dtype, void* d_dx, void* const* d_dW, void* const* d_db,
+                   void* d_workspace, int64_t workspace_bytes, void* stream);
+
 /* ---- per-kernel timing --------------------------------------------------
  * The reference times this path with torch.profiler around whole iterations
  * (attn_module.py:415-438).  When enabled, every kernel the library launches is

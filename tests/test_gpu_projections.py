@@ -1,0 +1,165 @@
+"""GPU parity of the projections (tgt_linear_fwd / tgt_linear_bwd) and of the
+MultiHeadAttention module with the oracle.
+
+Error measure: max|a - b| / max|b| against the oracle in float64 on the same
+inputs.  Bars: float32 1e-5 (fp32 matrix instructions, exact products, fp32
+accumulation), bf16 2e-2 (bf16 inputs and outputs, fp32 accumulation).
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import projections as P
+from torchgt_amd import MultiHeadAttention, _lib, fused_linear, workloads
+from torchgt_amd.multi_head_attention import LinearFunction
+
+pytestmark = pytest.mark.gpu
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2}
+
+
+def err(a, b):
+    a = a.detach().double().cpu().numpy()
+    b = np.asarray(b, np.float64)
+    assert a.shape == b.shape, (a.shape, b.shape)
+    denom = np.abs(b).max()
+    return np.abs(a - b).max() / (denom if denom > 0 else 1.0)
+
+
+def run_linear(name, N, in_f, out_f, n, dtype, cuda, seed, bias=True):
+    print(f"linear case {name}: N={N} in={in_f} out={out_f} n={n} {dtype} bias={bias} seed={seed}", flush=True)
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(N, in_f, generator=g).to(dtype)
+    Ws = [(torch.randn(out_f, in_f, generator=g) / in_f ** 0.5).to(dtype) for _ in range(n)]
+    bs = [torch.randn(out_f, generator=g).to(dtype) if bias else None for _ in range(n)]
+    dys = [torch.randn(N, out_f, generator=g).to(dtype) for _ in range(n)]
+    xc = x.to(cuda).requires_grad_(True)
+    Wc = [W.to(cuda).requires_grad_(True) for W in Ws]
+    bc = [None if b is None else b.to(cuda).requires_grad_(True) for b in bs]
+    args = []
+    for W, b in zip(Wc, bc):
+        args += [W, b]
+    ys = LinearFunction.apply(xc, *args)
+    leaves = [xc] + Wc + [b for b in bc if b is not None]
+    grads = torch.autograd.grad(ys, leaves, [dy.to(cuda) for dy in dys])
+    tol = TOL[dtype]
+    dx_ref = 0
+    for j in range(n):
+        y_ref = P.linear_forward(x.double().numpy(), Ws[j].double().numpy(), None if bs[j] is None else bs[j].double().numpy())
+        assert ys[j].dtype == dtype
+        assert err(ys[j], y_ref) <= tol, f"y{j} err {err(ys[j], y_ref)}"
+        dx_j, dW_j, db_j = P.linear_backward(x.double().numpy(), Ws[j].double().numpy(), dys[j].double().numpy())
+        dx_ref = dx_ref + dx_j
+        assert err(grads[1 + j], dW_j) <= tol, f"dW{j} err {err(grads[1 + j], dW_j)}"
+        if bias:
+            assert err(grads[1 + n + j], db_j) <= tol, f"db{j} err {err(grads[1 + n + j], db_j)}"
+    assert err(grads[0], dx_ref) <= tol, f"dx err {err(grads[0], dx_ref)}"
+    return ys, grads
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_linear_shapes(cuda, dtype):
+    run_linear("qkv-64", 1000, 64, 64, 3, dtype, cuda, 1)
+    run_linear("out-64", 777, 64, 64, 1, dtype, cuda, 2)
+    run_linear("ragged-panel", 129, 64, 64, 3, dtype, cuda, 3)        # one row past a 128-row panel
+    run_linear("tiny", 5, 8, 8, 2, dtype, cuda, 4)                     # narrower than one tile
+    run_linear("wide", 300, 128, 192, 3, dtype, cuda, 5)               # several contraction chunks and column tiles
+    run_linear("odd-tiles", 201, 72, 40, 1, dtype, cuda, 6, bias=False)  # partial chunks both ways, no bias
+    run_linear("gt-128", 513, 128, 128, 3, dtype, cuda, 7)
+
+
+def test_linear_weight_gradient_is_reproducible(cuda):
+    """The weight gradients are summed in a fixed order: two runs give the same bits."""
+    a = run_linear("repro-a", 20000, 64, 64, 3, torch.float32, cuda, 9)[1]
+    b = run_linear("repro-b", 20000, 64, 64, 3, torch.float32, cuda, 9)[1]
+    for ga, gb in zip(a, b):
+        assert torch.equal(ga, gb)
+
+
+def test_linear_empty_input(cuda):
+    x = torch.zeros(0, 64, device=cuda, requires_grad=True)
+    W = torch.randn(64, 64, device=cuda, requires_grad=True)
+    b = torch.randn(64, device=cuda, requires_grad=True)
+    (y,) = LinearFunction.apply(x, W, b)
+    assert y.shape == (0, 64)
+    dx, dW, db = torch.autograd.grad(y, [x, W, b], torch.zeros(0, 64, device=cuda))
+    assert dx.shape == (0, 64) and not dW.any() and not db.any()
+
+
+def test_linear_rejects_bad_arguments(cuda):
+    L = _lib.lib()
+    arr = (ctypes.c_void_p * 3)()
+    x = torch.zeros(16, 12, device=cuda)
+    W = torch.zeros(8, 12, device=cuda)
+    y = torch.zeros(16, 8, device=cuda)
+    arr_w = (ctypes.c_void_p * 3)(W.data_ptr())
+    arr_y = (ctypes.c_void_p * 3)(y.data_ptr())
+    assert L.tgt_linear_fwd(x.data_ptr(), arr_w, arr, arr_y, 1, 16, 12, 8, 0, None) == _lib.ERR_UNSUPPORTED   # 12 % 8
+    assert L.tgt_linear_fwd(x.data_ptr(), arr_w, arr, arr_y, 4, 16, 16, 8, 0, None) == _lib.ERR_INVALID_ARG   # n_out
+    assert L.tgt_linear_fwd(x.data_ptr(), arr, arr, arr_y, 1, 16, 16, 8, 0, None) == _lib.ERR_INVALID_ARG     # null weight
+    assert L.tgt_linear_bwd(x.data_ptr(), arr_w, arr_y, 1, 16, 16, 8, 0, None, arr_w, None, None, 0, None) == _lib.ERR_WORKSPACE
+    with pytest.raises(RuntimeError):
+        LinearFunction.apply(torch.zeros(4, 8), torch.zeros(8, 8), None)          # CPU tensors: no fallback
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_module_matches_oracle_and_reference_state_dict(cuda, dtype):
+    """MultiHeadAttention(hidden 64, 8 heads) on the 4 097-node configuration-1 graph:
+    forward against the oracle's module forward; parameter names are the reference's."""
+    torch.manual_seed(0)
+    e, n_nodes = workloads.barabasi_albert()
+    ei = torch.as_tensor(e)
+    hidden, H = 64, 8
+    m = MultiHeadAttention(hidden, 0.0, H, 1)
+    assert sorted(m.state_dict()) == sorted(
+        f"{l}.{p}" for l in ("linear_q", "linear_k", "linear_v", "output_layer") for p in ("weight", "bias"))
+    x = torch.randn(1, n_nodes, hidden)
+    if dtype == torch.bfloat16:      # the oracle sees the rounded values
+        x = x.bfloat16()
+        m = m.bfloat16()
+    params = {k: v.detach().double().numpy() for k, v in m.state_dict().items()}
+    want = P.multi_head_attention_forward(x.double().numpy(), params, ei.numpy(), H)
+    mc = m.to(cuda)
+    xc = x.to(cuda).requires_grad_(True)
+    got = mc(xc, None, ei.to(cuda), "sparse")
+    assert got.shape == (1, n_nodes, hidden) and got.dtype == dtype
+    assert err(got, want) <= TOL[dtype], err(got, want)
+    # backward against torch autograd through the oracle's pieces in float64
+    from oracle import sparse_attention as osa
+    xd = x.double().requires_grad_(True)
+    pd = {k: torch.tensor(v, requires_grad=True) for k, v in params.items()}
+    lin = torch.nn.functional.linear
+    q, k, v = (lin(xd[0], pd[f"linear_{c}.weight"], pd[f"linear_{c}.bias"]).view(1, n_nodes, H, hidden // H) for c in "qkv")
+    o, _ = osa.sparse_attention(q, k, v, ei)
+    y = lin(o.reshape(n_nodes, hidden), pd["output_layer.weight"], pd["output_layer.bias"])
+    gy = torch.randn(n_nodes, hidden, generator=torch.Generator().manual_seed(5)).to(dtype)
+    names = sorted(pd)
+    ref = torch.autograd.grad(y, [xd] + [pd[n] for n in names], gy.double())
+    got_g = torch.autograd.grad(got, [xc] + [dict(mc.named_parameters())[n] for n in names], gy.to(cuda).view(1, n_nodes, hidden))
+    # the bf16 module rounds q, k, v, the attention output and every gradient to bf16 between its four kernels
+    tol = TOL[dtype] * (3 if dtype == torch.bfloat16 else 1)
+    ref_by_name = dict(zip(["x"] + names, ref))
+    for nm, a, r in zip(["x"] + names, got_g, ref):
+        if nm == "linear_k.bias":
+            # shifting every key by one vector shifts all scores of a destination alike, which the
+            # normalisation cancels: this gradient is a sum of terms that cancel to ~0, so it is
+            # measured against the size of the query-bias gradient (same terms, no cancellation)
+            scale = ref_by_name["linear_q.bias"].abs().max().item()
+            e = (a.detach().double().cpu() - r).abs().max().item() / scale
+        else:
+            e = err(a, r.numpy())
+        assert e <= tol, f"d{nm} err {e}"
+
+
+def test_module_without_output_layer(cuda):
+    """GT flavour (no attn_bias_dim): no output layer, output = attention output."""
+    m = MultiHeadAttention(64, 0.0, 8).to(cuda)
+    assert m.output_layer is None
+    e, n_nodes = workloads.barabasi_albert()
+    ei = torch.as_tensor(e)
+    x = torch.randn(1, n_nodes, 64, generator=torch.Generator().manual_seed(1))
+    params = {k: v.detach().double().cpu().numpy() for k, v in m.state_dict().items()}
+    want = P.multi_head_attention_forward(x.double().numpy(), params, ei.numpy(), 8)
+    got = m(x.to(cuda), None, ei.to(cuda), "sparse")
+    assert err(got, want) <= 1e-5

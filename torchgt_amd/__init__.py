@@ -7,9 +7,10 @@ The compute lives in ``libtorchgt_hip.so`` (sources in ``csrc/``, C ABI in
 from .core_attention import (CoreAttention, SparseAttentionFunction, DenseAttentionFunction, sparse_attention,
                              dense_attention, gather_dense_bias)
 from .plan import GraphPlan, get_plan, clear_plan_cache
+from .multi_head_attention import MultiHeadAttention, LinearFunction, fused_linear
 from .block_attention import BlockAttentionFunction, TileSet, block_attention, expand_tiles
 
 __all__ = ["CoreAttention", "SparseAttentionFunction", "DenseAttentionFunction", "sparse_attention",
            "dense_attention", "gather_dense_bias",
            "GraphPlan", "get_plan", "clear_plan_cache", "BlockAttentionFunction", "TileSet", "block_attention",
-           "expand_tiles"]
+           "expand_tiles", "MultiHeadAttention", "LinearFunction", "fused_linear"]

@@ -51,6 +51,9 @@ SIGNATURES = {
     "tgt_reformat_export": (_i32, [_vp, _vp, _vp, _vp]),
     "tgt_reformat_destroy": (_i32, [_vp]),
     "tgt_np_legacy_randint": (_i32, [_c.c_uint32, _vp, _i32, _vp]),
+    "tgt_linear_fwd": (_i32, [_vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp]),
+    "tgt_linear_bwd_workspace_bytes": (_i64, [_i32, _i32, _i32]),
+    "tgt_linear_bwd": (_i32, [_vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _i64, _vp]),
     "tgt_probe_row_gather": (_i32, [_vp, _i64, _i32, _vp, _i64, _vp, _vp]),
     "tgt_timing_enable": (_i32, [_i32]),
     "tgt_timing_reset": (_i32, []),

@@ -1,0 +1,430 @@
+// The projections on either side of the attention: y_j = x W_j^T + b_j for up to
+// three weights in one pass over x, and the backward of that.
+//
+// Replaces linear_q / linear_k / linear_v and output_layer of MultiHeadAttention
+// (models/graphormer_dist_node_level.py:233-241 construct them, :255-257 and :271
+// apply them; same module in models/gt_dist_node_level.py and
+// models/graphormer_dist_graph_level.py).  In the reference these are three
+// separate GEMMs that each read x, plus one for the output; their backward is two
+// GEMMs and a column sum per weight.
+//
+// N (nodes) is large and the feature widths are small (64 in the node-level
+// configurations), so every kernel walks panels of node rows and keeps the
+// weights / weight gradients on chip:
+//   k_linear<DX=false>   y_j = x W_j^T + b_j         panel of 128 rows, x staged once
+//   k_linear<DX=true>    dx  = sum_j dy_j W_j         same walk, W staged transposed
+//   k_linear_gradw       dW_j = dy_j^T x, db_j = colsum(dy_j): each workgroup keeps a
+//                        64 x 64 tile of every dW_j in registers over its share of the
+//                        panels and writes one partial; k_linear_gradw_reduce adds the
+//                        partials in a fixed order (no atomics: results are reproducible)
+// Matrix instructions: v_mfma_f32_32x32x2_f32 for float32 (exact fp32 products,
+// fp32 accumulation), v_mfma_f32_32x32x8_bf16_1k for bf16 (fp32 accumulation).
+//   A 32xk : lane l holds A[l%32][k-slice of half l/32]
+//   B kx32 : lane l holds B[k-slice of half l/32][l%32]
+//   C 32x32: lane l, register r holds C[8*(r/4) + 4*(l/32) + r%4][l%32]
+// Both operands are kept in LDS with the contraction index contiguous, and half
+// l/32 of the wave takes the contraction indices [half*KC/2, (half+1)*KC/2): a
+// lane then fetches the operands of four (fp32) or two (bf16) instructions with one
+// 16-byte LDS read.  (Any assignment of contraction indices to instructions gives
+// the same product as long as A and B use the same one.)
+#include "common.h"
+#include <algorithm>
+
+namespace tgt {
+namespace {
+
+typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+struct pbf16 { uint16_t x; };
+
+constexpr int kThreads = 256;
+constexpr int kPanel = 128;     // node rows per workgroup of the forward / input-gradient kernel
+constexpr int kChunk = 64;      // contraction indices per LDS stage
+constexpr int kCols = 64;       // output columns per accumulation pass
+constexpr int kGradRows = 64;   // node rows per step of the weight-gradient kernel
+constexpr int kGradWorkers = 512;   // workgroups (partials) of the weight-gradient kernel per output tile set
+
+template <typename T> constexpr int lds_stride(int inner) { return inner + 16 / (int)sizeof(T); }
+
+__device__ __forceinline__ float ld1(const float* p) { return *p; }
+__device__ __forceinline__ float ld1(const pbf16* p) { return __uint_as_float(((uint32_t)p->x) << 16); }
+__device__ __forceinline__ void st1(float* p, float v) { *p = v; }
+__device__ __forceinline__ void st1(pbf16* p, float v) {
+    const __bf16 b = static_cast<__bf16>(v);
+    p->x = __builtin_bit_cast(uint16_t, b);
+}
+
+__device__ __forceinline__ float16_t zero16() {
+    float16_t z;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) z[i] = 0.f;
+    return z;
+}
+
+// tile[r][c] = src[(row0 + r) * ld + col0 + c], r < R, c < 64; zero outside [0,nrows) x [0,ncols)
+template <typename T, int R, int STRIDE>
+__device__ __forceinline__ void stage_natural(T* __restrict__ tile, const T* __restrict__ src, int64_t ld,
+                                              int64_t row0, int64_t nrows, int col0, int ncols) {
+    constexpr int VE = 16 / (int)sizeof(T);
+    constexpr int VPR = kChunk / VE;
+#pragma unroll
+    for (int v = threadIdx.x; v < R * VPR; v += kThreads) {
+        const int r = v / VPR, c = (v % VPR) * VE;
+        uint4 val = make_uint4(0u, 0u, 0u, 0u);
+        if (row0 + r < nrows && col0 + c < ncols)
+            val = *reinterpret_cast<const uint4*>(src + (row0 + r) * ld + col0 + c);
+        *reinterpret_cast<uint4*>(tile + r * STRIDE + c) = val;
+    }
+}
+
+// tile[c][r] = src[(row0 + r) * ld + col0 + c], r < R, c < 64; zero outside.  Four
+// lanes read 64 consecutive bytes of one source row and sixteen rows go per
+// instruction, which keeps the scattered LDS writes to two per bank.
+template <typename T, int R, int STRIDE>
+__device__ __forceinline__ void stage_transposed(T* __restrict__ tile, const T* __restrict__ src, int64_t ld,
+                                                 int64_t row0, int64_t nrows, int col0, int ncols) {
+    constexpr int VE = 16 / (int)sizeof(T);
+    constexpr int VPR = kChunk / VE;
+    static_assert(R % 16 == 0 && VPR % 4 == 0, "tile shape");
+#pragma unroll
+    for (int v = threadIdx.x; v < R * VPR; v += kThreads) {
+        const int cq = v & 3, r_lo = (v >> 2) & 15, rest = v >> 6;
+        const int r = (rest % (R / 16)) * 16 + r_lo;
+        const int c = ((rest / (R / 16)) * 4 + cq) * VE;
+        uint4 val = make_uint4(0u, 0u, 0u, 0u);
+        if (row0 + r < nrows && col0 + c < ncols)
+            val = *reinterpret_cast<const uint4*>(src + (row0 + r) * ld + col0 + c);
+        const T* e = reinterpret_cast<const T*>(&val);
+#pragma unroll
+        for (int t = 0; t < VE; ++t) tile[(c + t) * STRIDE + r] = e[t];
+    }
+}
+
+// acc += A B over KC contraction indices; a, b: the lane's operand rows in LDS,
+// already offset by its half's first contraction index.
+template <typename T, int KC> struct Mma;
+template <int KC> struct Mma<float, KC> {
+    static __device__ __forceinline__ void run(const float* a, const float* b, float16_t& acc) {
+#pragma unroll
+        for (int i = 0; i < KC / 2; i += 4) {
+            const float4 av = *reinterpret_cast<const float4*>(a + i);
+            const float4 bv = *reinterpret_cast<const float4*>(b + i);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.x, bv.x, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.y, bv.y, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.z, bv.z, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av.w, bv.w, acc, 0, 0, 0);
+        }
+    }
+};
+template <int KC> struct Mma<pbf16, KC> {
+    static __device__ __forceinline__ void run(const pbf16* a, const pbf16* b, float16_t& acc) {
+#pragma unroll
+        for (int i = 0; i < KC / 2; i += 8) {
+            const uint4 av = *reinterpret_cast<const uint4*>(a + i);
+            const uint4 bv = *reinterpret_cast<const uint4*>(b + i);
+            acc = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(__builtin_bit_cast(short4_t, make_uint2(av.x, av.y)),
+                                                           __builtin_bit_cast(short4_t, make_uint2(bv.x, bv.y)),
+                                                           acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(__builtin_bit_cast(short4_t, make_uint2(av.z, av.w)),
+                                                           __builtin_bit_cast(short4_t, make_uint2(bv.z, bv.w)),
+                                                           acc, 0, 0, 0);
+        }
+    }
+};
+
+struct LinArgs {
+    const void* A[3];      // forward: A[0] = x [N, K]; input gradient: A[j] = dy_j [N, M]
+    const void* W[3];      // [M, K] row-major (nn.Linear.weight)
+    const void* bias[3];   // forward only; entries may be null
+    void* out[3];          // forward: y_j [N, M]; input gradient: out[0] = dx [N, K]
+    int nw;
+    int64_t N;
+    int K, M;
+};
+
+// One workgroup per panel of 128 node rows; wave w owns rows [32w, 32w+32) and two
+// 32-column blocks of the current 64 output columns.
+template <typename T, bool DX>
+__global__ __launch_bounds__(kThreads) void k_linear(LinArgs a) {
+    constexpr int S = lds_stride<T>(kChunk);
+    __shared__ __align__(16) T tA[kPanel * S];
+    __shared__ __align__(16) T tB[kCols * S];
+    const int L = DX ? a.M : a.K;          // contraction length
+    const int C = DX ? a.K : a.M;          // output columns
+    const int n_out = DX ? 1 : a.nw, n_src = DX ? a.nw : 1;
+    const int64_t row0 = (int64_t)blockIdx.x * kPanel;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, h = lane >> 5;
+    const bool a_resident = (n_src == 1 && L <= kChunk);   // the source panel is staged once for all outputs
+    bool a_loaded = false;
+    for (int o = 0; o < n_out; ++o) {
+        for (int c0 = 0; c0 < C; c0 += kCols) {
+            float16_t acc0 = zero16(), acc1 = zero16();
+            for (int s = 0; s < n_src; ++s) {
+                const T* W = reinterpret_cast<const T*>(a.W[DX ? s : o]);
+                for (int l0 = 0; l0 < L; l0 += kChunk) {
+                    __syncthreads();
+                    if (!(a_resident && a_loaded)) {
+                        stage_natural<T, kPanel, S>(tA, reinterpret_cast<const T*>(a.A[s]), L, row0, a.N, l0, L);
+                        a_loaded = true;
+                    }
+                    if (!DX) stage_natural<T, kCols, S>(tB, W, a.K, c0, a.M, l0, a.K);       // rows = output columns
+                    else stage_transposed<T, kChunk, S>(tB, W, a.K, l0, a.M, c0, a.K);       // rows of W = contraction
+                    __syncthreads();
+                    const T* ap = tA + (wave * 32 + l32) * S + h * (kChunk / 2);
+                    Mma<T, kChunk>::run(ap, tB + l32 * S + h * (kChunk / 2), acc0);
+                    Mma<T, kChunk>::run(ap, tB + (32 + l32) * S + h * (kChunk / 2), acc1);
+                }
+            }
+            T* out = reinterpret_cast<T*>(a.out[o]);
+            const T* bias = DX ? nullptr : reinterpret_cast<const T*>(a.bias[o]);
+#pragma unroll
+            for (int cb = 0; cb < 2; ++cb) {
+                const int col = c0 + 32 * cb + l32;
+                if (col >= C) continue;
+                const float bv = bias ? ld1(bias + col) : 0.f;
+                const float16_t& acc = cb ? acc1 : acc0;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int64_t row = row0 + wave * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+                    if (row < a.N) st1(out + row * C + col, acc[r] + bv);
+                }
+            }
+        }
+    }
+}
+
+struct GradWArgs {
+    const void* x;         // [N, K]
+    const void* dy[3];     // [N, M]
+    float* partial;        // [workers][nw][M*K + M]
+    int64_t N;
+    int K, M;
+};
+
+// blockIdx.y picks a 64 x 64 tile (mt, kt) of the weight gradients, blockIdx.x a
+// worker; wave w owns the 32 x 32 block (w/2, w%2) of the tile for every weight.
+template <typename T, int NW>
+__global__ __launch_bounds__(kThreads) void k_linear_gradw(GradWArgs a) {
+    constexpr int S = lds_stride<T>(kGradRows);
+    extern __shared__ __align__(16) unsigned char smem[];
+    T* tX = reinterpret_cast<T*>(smem);          // [64 k][64 nodes]
+    T* tD = tX + kCols * S;                      // NW x [64 m][64 nodes]
+    const int kt_n = (a.K + kCols - 1) / kCols;
+    const int mt = blockIdx.y / kt_n, kt = blockIdx.y % kt_n;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, h = lane >> 5;
+    const int mi = wave >> 1, ki = wave & 1;
+    float16_t acc[NW];
+#pragma unroll
+    for (int j = 0; j < NW; ++j) acc[j] = zero16();
+    float colsum = 0.f;
+    const int64_t n_panels = (a.N + kGradRows - 1) / kGradRows;
+    for (int64_t p = blockIdx.x; p < n_panels; p += gridDim.x) {
+        __syncthreads();
+        stage_transposed<T, kGradRows, S>(tX, reinterpret_cast<const T*>(a.x), a.K, p * kGradRows, a.N, kt * kCols, a.K);
+#pragma unroll
+        for (int j = 0; j < NW; ++j)
+            stage_transposed<T, kGradRows, S>(tD + j * kCols * S, reinterpret_cast<const T*>(a.dy[j]), a.M,
+                                              p * kGradRows, a.N, mt * kCols, a.M);
+        __syncthreads();
+        const T* bp = tX + (32 * ki + l32) * S + h * (kGradRows / 2);
+#pragma unroll
+        for (int j = 0; j < NW; ++j)
+            Mma<T, kGradRows>::run(tD + j * kCols * S + (32 * mi + l32) * S + h * (kGradRows / 2), bp, acc[j]);
+        if (kt == 0 && wave < NW) {      // wave j adds up the columns of dy_j: lane = column
+            const T* row = tD + wave * kCols * S + lane * S;
+            float s = 0.f;
+#pragma unroll 16
+            for (int i = 0; i < kGradRows; ++i) s += ld1(row + i);
+            colsum += s;
+        }
+    }
+    const int64_t per = (int64_t)a.M * a.K + a.M;
+    float* mine = a.partial + (int64_t)blockIdx.x * NW * per;
+#pragma unroll
+    for (int j = 0; j < NW; ++j) {
+        const int k = kt * kCols + 32 * ki + l32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m = mt * kCols + 32 * mi + 8 * (r >> 2) + 4 * h + (r & 3);
+            if (m < a.M && k < a.K) mine[j * per + (int64_t)m * a.K + k] = acc[j][r];
+        }
+    }
+    if (kt == 0 && wave < NW) {
+        const int m = mt * kCols + lane;
+        if (m < a.M) mine[wave * per + (int64_t)a.M * a.K + m] = colsum;
+    }
+}
+
+struct ReduceArgs {
+    const float* partial;
+    void* dW[3];
+    void* db[3];           // entries may be null
+    int workers, nw, K, M;
+};
+
+// 64 consecutive elements x 16 slices of the workers per workgroup; the slices are
+// added in order, so the sum does not depend on the launch.
+template <typename T>
+__global__ __launch_bounds__(1024) void k_linear_gradw_reduce(ReduceArgs a) {
+    __shared__ float part[16][64];
+    const int el = threadIdx.x & 63, sl = threadIdx.x >> 6;
+    const int64_t per = (int64_t)a.M * a.K + a.M;
+    const int64_t total = per * a.nw;
+    const int64_t e = (int64_t)blockIdx.x * 64 + el;
+    const int w0 = (int)((int64_t)a.workers * sl / 16), w1 = (int)((int64_t)a.workers * (sl + 1) / 16);
+    float s = 0.f;
+    if (e < total)
+        for (int w = w0; w < w1; ++w) s += a.partial[(int64_t)w * total + e];
+    part[sl][el] = s;
+    __syncthreads();
+    if (sl == 0 && e < total) {
+        float t = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) t += part[i][el];
+        const int j = (int)(e / per);
+        const int64_t off = e % per;
+        if (off < (int64_t)a.M * a.K) st1(reinterpret_cast<T*>(a.dW[j]) + off, t);
+        else if (a.db[j]) st1(reinterpret_cast<T*>(a.db[j]) + (off - (int64_t)a.M * a.K), t);
+    }
+}
+
+int check_shape(int n_out, int64_t N, int in_features, int out_features, int dtype) {
+    if (n_out < 1 || n_out > 3 || N < 0 || in_features <= 0 || out_features <= 0) {
+        set_error("linear: n_out must be 1..3 and sizes positive (n_out=%d N=%lld in=%d out=%d)", n_out, (long long)N,
+                  in_features, out_features);
+        return TGT_ERR_INVALID_ARG;
+    }
+    if (dtype != TGT_DTYPE_F32 && dtype != TGT_DTYPE_BF16) {
+        set_error("linear: unknown dtype %d", dtype);
+        return TGT_ERR_INVALID_ARG;
+    }
+    if (in_features % 8 || out_features % 8) {
+        set_error("linear: in_features and out_features must be multiples of 8 (got %d, %d)", in_features, out_features);
+        return TGT_ERR_UNSUPPORTED;
+    }
+    if (N > (int64_t)INT32_MAX * kGradRows) {
+        set_error("linear: N too large");
+        return TGT_ERR_UNSUPPORTED;
+    }
+    return TGT_OK;
+}
+
+int grad_workers(int in_features, int out_features) {
+    const int tiles = ((in_features + kCols - 1) / kCols) * ((out_features + kCols - 1) / kCols);
+    return std::max(1, kGradWorkers / tiles);
+}
+
+template <typename T, int NW>
+int launch_gradw(const GradWArgs& g, int workers, int tiles, hipStream_t st) {
+    const size_t lds = sizeof(T) * (size_t)(1 + NW) * kCols * lds_stride<T>(kGradRows);
+    static bool raised = false;   // per instantiation; the attribute is per function and sticks
+    if (!raised && lds > 48 * 1024) {
+        TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_linear_gradw<T, NW>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        raised = true;
+    }
+    hipLaunchKernelGGL((k_linear_gradw<T, NW>), dim3(workers, tiles), dim3(kThreads), lds, st, g);
+    return TGT_OK;
+}
+
+template <typename T>
+int linear_bwd_t(const void* d_x, const void* const* d_W, const void* const* d_dy, int n_out, int64_t N, int K, int M,
+                 void* d_dx, void* const* d_dW, void* const* d_db, float* partial, hipStream_t st) {
+    if (d_dx && N > 0) {
+        LinArgs a{};
+        for (int j = 0; j < n_out; ++j) { a.A[j] = d_dy[j]; a.W[j] = d_W[j]; }
+        a.out[0] = d_dx;
+        a.nw = n_out; a.N = N; a.K = K; a.M = M;
+        KernelTimer t(KS_LINEAR_DX, st);
+        hipLaunchKernelGGL((k_linear<T, true>), dim3((unsigned)((N + kPanel - 1) / kPanel)), dim3(kThreads), 0, st, a);
+    }
+    if (d_dW) {
+        const int tiles = ((K + kCols - 1) / kCols) * ((M + kCols - 1) / kCols);
+        const int64_t n_panels = (N + kGradRows - 1) / kGradRows;
+        const int workers = (int)std::max<int64_t>(1, std::min<int64_t>(n_panels, grad_workers(K, M)));
+        GradWArgs g{};
+        g.x = d_x;
+        for (int j = 0; j < n_out; ++j) g.dy[j] = d_dy[j];
+        g.partial = partial; g.N = N; g.K = K; g.M = M;
+        KernelTimer t(KS_LINEAR_DW, st);
+        int rc = TGT_OK;
+        if (n_out == 1) rc = launch_gradw<T, 1>(g, workers, tiles, st);
+        else if (n_out == 2) rc = launch_gradw<T, 2>(g, workers, tiles, st);
+        else rc = launch_gradw<T, 3>(g, workers, tiles, st);
+        if (rc != TGT_OK) return rc;
+        ReduceArgs r{};
+        r.partial = partial; r.workers = workers; r.nw = n_out; r.K = K; r.M = M;
+        for (int j = 0; j < n_out; ++j) { r.dW[j] = d_dW[j]; r.db[j] = d_db ? d_db[j] : nullptr; }
+        const int64_t total = ((int64_t)M * K + M) * n_out;
+        hipLaunchKernelGGL((k_linear_gradw_reduce<T>), dim3((unsigned)((total + 63) / 64)), dim3(1024), 0, st, r);
+    }
+    TGT_HIP_CHECK(hipGetLastError());
+    return TGT_OK;
+}
+
+}  // namespace
+}  // namespace tgt
+
+extern "C" {
+
+int tgt_linear_fwd(const void* d_x, const void* const* d_W, const void* const* d_b, void* const* d_y, int n_out,
+                   int64_t N, int in_features, int out_features, int dtype, void* stream) {
+    using namespace tgt;
+    const int rc = check_shape(n_out, N, in_features, out_features, dtype);
+    if (rc != TGT_OK) return rc;
+    if (!d_W || !d_y || (N > 0 && !d_x)) { set_error("linear_fwd: null pointer"); return TGT_ERR_INVALID_ARG; }
+    LinArgs a{};
+    a.A[0] = d_x;
+    for (int j = 0; j < n_out; ++j) {
+        if (!d_W[j] || (N > 0 && !d_y[j])) { set_error("linear_fwd: null weight or output %d", j); return TGT_ERR_INVALID_ARG; }
+        a.W[j] = d_W[j];
+        a.bias[j] = d_b ? d_b[j] : nullptr;
+        a.out[j] = d_y[j];
+    }
+    a.nw = n_out; a.N = N; a.K = in_features; a.M = out_features;
+    if (N == 0) return TGT_OK;
+    hipStream_t st = (hipStream_t)stream;
+    KernelTimer t(KS_LINEAR_FWD, st);
+    const dim3 grid((unsigned)((N + kPanel - 1) / kPanel));
+    if (dtype == TGT_DTYPE_F32) hipLaunchKernelGGL((k_linear<float, false>), grid, dim3(kThreads), 0, st, a);
+    else hipLaunchKernelGGL((k_linear<pbf16, false>), grid, dim3(kThreads), 0, st, a);
+    TGT_HIP_CHECK(hipGetLastError());
+    return TGT_OK;
+}
+
+int64_t tgt_linear_bwd_workspace_bytes(int n_out, int in_features, int out_features) {
+    using namespace tgt;
+    if (n_out < 1 || n_out > 3 || in_features <= 0 || out_features <= 0) return 0;
+    return (int64_t)sizeof(float) * grad_workers(in_features, out_features) * n_out *
+           ((int64_t)in_features * out_features + out_features);
+}
+
+int tgt_linear_bwd(const void* d_x, const void* const* d_W, const void* const* d_dy, int n_out, int64_t N,
+                   int in_features, int out_features, int dtype, void* d_dx, void* const* d_dW, void* const* d_db,
+                   void* d_workspace, int64_t workspace_bytes, void* stream) {
+    using namespace tgt;
+    const int rc = check_shape(n_out, N, in_features, out_features, dtype);
+    if (rc != TGT_OK) return rc;
+    if (!d_W || !d_dy || (N > 0 && !d_x)) { set_error("linear_bwd: null pointer"); return TGT_ERR_INVALID_ARG; }
+    for (int j = 0; j < n_out; ++j) {
+        if (!d_W[j] || (N > 0 && !d_dy[j]) || (d_dW && !d_dW[j])) {
+            set_error("linear_bwd: null weight, gradient or output %d", j);
+            return TGT_ERR_INVALID_ARG;
+        }
+    }
+    if (d_db && !d_dW) { set_error("linear_bwd: bias gradients are produced with the weight gradients"); return TGT_ERR_INVALID_ARG; }
+    if (d_dW && (!d_workspace || workspace_bytes < tgt_linear_bwd_workspace_bytes(n_out, in_features, out_features) ||
+                 ((uintptr_t)d_workspace & 15))) {
+        set_error("linear_bwd: workspace of %lld bytes (16-byte aligned) needed, got %lld",
+                  (long long)tgt_linear_bwd_workspace_bytes(n_out, in_features, out_features), (long long)workspace_bytes);
+        return TGT_ERR_WORKSPACE;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == TGT_DTYPE_F32)
+        return linear_bwd_t<float>(d_x, d_W, d_dy, n_out, N, in_features, out_features, d_dx, d_dW, d_db,
+                                   (float*)d_workspace, st);
+    return linear_bwd_t<pbf16>(d_x, d_W, d_dy, n_out, N, in_features, out_features, d_dx, d_dW, d_db,
+                               (float*)d_workspace, st);
+}
+
+}  // extern "C"
