@@ -8,10 +8,11 @@ the benchmark configuration "configs[1]": N = 64 001, E ~ 530 K, H = 8, d = 8, p
 reported separately).  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype f32|bf16] [--no-cpu-baseline]
-                    [--workload config1|config2|config3|config4|config5|config5-blockized]
+                    [--workload config1|config2|config2-mha|config3|config4|config5|config5-blockized]
 
 config3 / config5: larger sparse workloads (bf16); config4: dense biased attention of a graph-level
-batch; config5-blockized: the block path on the reordered config5 graph.
+batch; config5-blockized: the block path on the reordered config5 graph; config2-mha: one whole
+MultiHeadAttention layer (projections + sparse attention) on the config2 graph.
 """
 import argparse
 import json
@@ -339,6 +340,71 @@ def bench_block(args):
     print(json.dumps(result))
 
 
+def bench_mha(args):
+    """One MultiHeadAttention layer of configs[1] (hidden 64, 8 heads, N = 64 001, E ~ 530 K, no bias as in the
+    shipped node-level runs): q/k/v projections, sparse attention, output projection, forward + backward with all
+    parameter gradients.  A step = tgt_linear_fwd(3) + tgt_sparse_attn_fwd + tgt_linear_fwd(1) and their backwards,
+    driven through the module (torch autograd bookkeeping included in the wall time)."""
+    import torch
+    from torchgt_amd import MultiHeadAttention, _lib
+    dev = torch.device("cuda:0")
+    hidden, H = 64, 8
+    e, n, label, desc = build_workload("config2")
+    tdt = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    esize = 2 if args.dtype == "bf16" else 4
+    torch.manual_seed(42)
+    m = MultiHeadAttention(hidden, 0.0, H, 1).to(dev, tdt)
+    ei = torch.from_numpy(e).to(dev)
+    x = torch.randn(1, n, hidden, device=dev).to(tdt).requires_grad_(True)
+    gy = torch.randn(1, n, hidden, device=dev).to(tdt)
+    params = list(m.parameters())
+
+    def step():
+        y = m(x, None, ei, "sparse")
+        torch.autograd.grad(y, [x] + params, gy)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    L = _lib.lib()
+    L.tgt_timing_reset()
+    L.tgt_timing_enable(1)
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    L.tgt_timing_enable(0)
+    # per step: linear_fwd runs twice (q/k/v and output), linear_dx and linear_dw twice
+    kernels = {k: {"avg_us": t / c * 1e3, "launches_per_step": c / args.steps} for k, (t, c) in _lib.kernel_timings().items() if c}
+    gpu_us = sum(v["avg_us"] * v["launches_per_step"] for v in kernels.values())
+    row = n * hidden * esize
+    # projections, every operand once: forward reads x and writes q, k, v (4 rows), output layer 2 rows;
+    # input gradients read 3 + 1 and write 1 + 1 rows; weight gradients read 4 + 2 rows
+    lin_bytes = (4 + 2 + 4 + 2 + 4 + 2) * row
+    lin_us = sum(kernels[k]["avg_us"] * kernels[k]["launches_per_step"] for k in kernels if k.startswith("linear"))
+    lin_flops = 2 * n * hidden * hidden * 4 * 3       # four 64 x 64 weights, forward + two backward products
+    result = {
+        "metric": "fwd+bwd of one MultiHeadAttention layer (projections + sparse attention)",
+        "value": e.shape[1] / (ms * 1e-3), "unit": "edges/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic",
+        "config": {"workload": "configs[1] graph, MultiHeadAttention(hidden 64, 8 heads) layer, no bias", "N": n,
+                   "E": int(e.shape[1]), "step": "module forward + autograd backward (x and all parameters)",
+                   "parallelism": "1 GPU"},
+        "gpu_kernel_us_per_step": gpu_us,
+        "projections": {"us_per_step": lin_us, "alg_bytes": lin_bytes,
+                        "hbm_frac": lin_bytes / (lin_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
+                        "alg_tflops": lin_flops / (lin_us * 1e-6) / 1e12,
+                        "mfma_peak_tflops": 157.3 if args.dtype == "f32" else 2500.0},
+        "kernels": kernels,
+    }
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -371,6 +437,8 @@ def main():
         return bench_dense(args)
     if args.workload == "config5-blockized":
         return bench_block(args)
+    if args.workload == "config2-mha":
+        return bench_mha(args)
     if args.workload in ("config3", "config5"):
         args.no_cpu_baseline = True      # the CPU restatement needs minutes per step at this size
     e, n, label, desc = build_workload(args.workload)

@@ -100,6 +100,45 @@ __device__ __forceinline__ void stage_transposed(T* __restrict__ tile, const T* 
     }
 }
 
+// The same transposed tile in two steps, so that the loads of the next tile can be
+// in flight during the products of the current one: fetch_t reads the thread's
+// 16-byte pieces into registers, put_t scatters them into the LDS tile.
+template <typename T> struct PieceRegs { uint4 v[(64 * 64 * sizeof(T)) / (16 * kThreads)]; };
+
+template <typename T, int R>
+__device__ __forceinline__ void piece_pos(int i, int& r, int& c) {
+    constexpr int VE = 16 / (int)sizeof(T);
+    const int v = threadIdx.x + i * kThreads;
+    const int cq = v & 3, r_lo = (v >> 2) & 15, rest = v >> 6;
+    r = (rest % (R / 16)) * 16 + r_lo;
+    c = ((rest / (R / 16)) * 4 + cq) * VE;
+}
+template <typename T>
+__device__ __forceinline__ void fetch_t(PieceRegs<T>& t, const T* __restrict__ src, int64_t ld, int64_t row0,
+                                        int64_t nrows, int col0, int ncols) {
+    constexpr int NV = (int)(sizeof(PieceRegs<T>) / 16);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        int r, c;
+        piece_pos<T, 64>(i, r, c);
+        uint4 u = make_uint4(0u, 0u, 0u, 0u);
+        if (row0 + r < nrows && col0 + c < ncols) u = *reinterpret_cast<const uint4*>(src + (row0 + r) * ld + col0 + c);
+        t.v[i] = u;
+    }
+}
+template <typename T, int STRIDE>
+__device__ __forceinline__ void put_t(const PieceRegs<T>& t, T* __restrict__ tile) {
+    constexpr int VE = 16 / (int)sizeof(T), NV = (int)(sizeof(PieceRegs<T>) / 16);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        int r, c;
+        piece_pos<T, 64>(i, r, c);
+        const T* e = reinterpret_cast<const T*>(&t.v[i]);
+#pragma unroll
+        for (int k = 0; k < VE; ++k) tile[(c + k) * STRIDE + r] = e[k];
+    }
+}
+
 // acc += A B over KC contraction indices; a, b: the lane's operand rows in LDS,
 // already offset by its half's first contraction index.
 template <typename T, int KC> struct Mma;
@@ -193,6 +232,133 @@ __global__ __launch_bounds__(kThreads) void k_linear(LinArgs a) {
     }
 }
 
+// A 64-row x 64-column tile on its way from global memory to LDS: each thread
+// holds 16-byte pieces in registers, so the loads of the next panel can be in
+// flight while the current one is multiplied.
+template <typename T> struct TileRegs { uint4 v[(64 * 64 * sizeof(T)) / (16 * kThreads)]; };
+
+template <typename T>
+__device__ __forceinline__ void tile_fetch(TileRegs<T>& t, const T* __restrict__ src, int64_t row0, int64_t nrows) {
+    constexpr int VE = 16 / (int)sizeof(T), VPR = 64 / VE, NV = (int)(sizeof(TileRegs<T>) / 16);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int v = threadIdx.x + i * kThreads, r = v / VPR, c = (v % VPR) * VE;
+        uint4 u = make_uint4(0u, 0u, 0u, 0u);
+        if (row0 + r < nrows) u = *reinterpret_cast<const uint4*>(src + (row0 + r) * 64 + c);
+        t.v[i] = u;
+    }
+}
+template <typename T, int STRIDE>
+__device__ __forceinline__ void tile_put(const TileRegs<T>& t, T* __restrict__ tile) {
+    constexpr int VE = 16 / (int)sizeof(T), VPR = 64 / VE, NV = (int)(sizeof(TileRegs<T>) / 16);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int v = threadIdx.x + i * kThreads, r = v / VPR, c = (v % VPR) * VE;
+        *reinterpret_cast<uint4*>(tile + r * STRIDE + c) = t.v[i];
+    }
+}
+
+// in_features = out_features = 64 (the node-level models).  The weights stay in LDS
+// for the life of the workgroup, which walks panels of 64 node rows; the next
+// panel's rows are fetched into registers while the current panel is multiplied.
+// Wave w owns the 32 x 32 block (w/2, w%2) of every 64 x 64 output tile.
+template <typename T, bool DX, int NW>
+__global__ __launch_bounds__(kThreads) void k_linear64(LinArgs a) {
+    constexpr int S = lds_stride<T>(64);
+    constexpr int NA = DX ? NW : 1;      // source tiles per panel
+    constexpr int NO = DX ? 1 : NW;      // output tiles per panel
+    extern __shared__ __align__(16) unsigned char smem[];
+    T* tW = reinterpret_cast<T*>(smem);          // [NW][64][S]
+    T* tA = tW + NW * 64 * S;                    // [NA][64][S]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, h = lane >> 5;
+    const int rb = wave >> 1, cb = wave & 1;
+    const int64_t n_panels = (a.N + 63) / 64;
+    TileRegs<T> next[NA];
+    int64_t p = blockIdx.x;
+    if (p < n_panels) {
+#pragma unroll
+        for (int s = 0; s < NA; ++s) tile_fetch(next[s], reinterpret_cast<const T*>(a.A[s]), p * 64, a.N);
+    }
+#pragma unroll
+    for (int j = 0; j < NW; ++j) {
+        const T* W = reinterpret_cast<const T*>(a.W[j]);
+        if (!DX) stage_natural<T, 64, S>(tW + j * 64 * S, W, 64, 0, 64, 0, 64);        // rows = output columns
+        else stage_transposed<T, 64, S>(tW + j * 64 * S, W, 64, 0, 64, 0, 64);         // rows = columns of W
+    }
+    float bv[NO];
+#pragma unroll
+    for (int o = 0; o < NO; ++o) {
+        const T* bias = DX ? nullptr : reinterpret_cast<const T*>(a.bias[o]);
+        bv[o] = bias ? ld1(bias + 32 * cb + l32) : 0.f;
+    }
+    for (; p < n_panels; p += gridDim.x) {
+        __syncthreads();                 // the previous panel has been read
+#pragma unroll
+        for (int s = 0; s < NA; ++s) tile_put<T, S>(next[s], tA + s * 64 * S);
+        __syncthreads();
+        if (p + gridDim.x < n_panels) {
+#pragma unroll
+            for (int s = 0; s < NA; ++s)
+                tile_fetch(next[s], reinterpret_cast<const T*>(a.A[s]), (p + gridDim.x) * 64, a.N);
+        }
+#pragma unroll
+        for (int o = 0; o < NO; ++o) {
+            float16_t acc = zero16();
+#pragma unroll
+            for (int s = 0; s < NA; ++s)
+                Mma<T, 64>::run(tA + (s * 64 + 32 * rb + l32) * S + h * 32,
+                                tW + ((DX ? s : o) * 64 + 32 * cb + l32) * S + h * 32, acc);
+            T* out = reinterpret_cast<T*>(a.out[o]) + 32 * cb + l32;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int64_t row = p * 64 + 32 * rb + 8 * (r >> 2) + 4 * h + (r & 3);
+                if (row < a.N) st1(out + row * 64, acc[r] + bv[o]);
+            }
+        }
+    }
+}
+
+int num_cus() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            cus = n;
+        else
+            cus = 256;
+    }
+    return cus;
+}
+
+template <typename T, bool DX, int NW>
+int launch_linear64(const LinArgs& a, hipStream_t st) {
+    constexpr int NA = DX ? NW : 1;
+    const size_t lds = sizeof(T) * (size_t)(NW + NA) * 64 * lds_stride<T>(64);
+    static bool raised = false;
+    if (!raised && lds > 48 * 1024) {
+        TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_linear64<T, DX, NW>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        raised = true;
+    }
+    const int64_t n_panels = (a.N + 63) / 64;
+    const int per_cu = (int)std::max<size_t>(1, std::min<size_t>(4, (size_t)(150 * 1024) / lds));
+    const unsigned grid = (unsigned)std::min<int64_t>(n_panels, (int64_t)num_cus() * per_cu);
+    hipLaunchKernelGGL((k_linear64<T, DX, NW>), dim3(grid), dim3(kThreads), lds, st, a);
+    return TGT_OK;
+}
+
+template <typename T, bool DX>
+int launch_linear(const LinArgs& a, hipStream_t st) {
+    if (a.K == 64 && a.M == 64) {
+        if (a.nw == 1) return launch_linear64<T, DX, 1>(a, st);
+        if (a.nw == 2) return launch_linear64<T, DX, 2>(a, st);
+        return launch_linear64<T, DX, 3>(a, st);
+    }
+    hipLaunchKernelGGL((k_linear<T, DX>), dim3((unsigned)((a.N + kPanel - 1) / kPanel)), dim3(kThreads), 0, st, a);
+    return TGT_OK;
+}
+
 struct GradWArgs {
     const void* x;         // [N, K]
     const void* dy[3];     // [N, M]
@@ -217,15 +383,29 @@ __global__ __launch_bounds__(kThreads) void k_linear_gradw(GradWArgs a) {
 #pragma unroll
     for (int j = 0; j < NW; ++j) acc[j] = zero16();
     float colsum = 0.f;
+    static_assert(kGradRows == 64, "piece layout");
     const int64_t n_panels = (a.N + kGradRows - 1) / kGradRows;
-    for (int64_t p = blockIdx.x; p < n_panels; p += gridDim.x) {
-        __syncthreads();
-        stage_transposed<T, kGradRows, S>(tX, reinterpret_cast<const T*>(a.x), a.K, p * kGradRows, a.N, kt * kCols, a.K);
+    PieceRegs<T> nx, nd[NW];
+    int64_t p = blockIdx.x;
+    if (p < n_panels) {
+        fetch_t(nx, reinterpret_cast<const T*>(a.x), a.K, p * kGradRows, a.N, kt * kCols, a.K);
 #pragma unroll
         for (int j = 0; j < NW; ++j)
-            stage_transposed<T, kGradRows, S>(tD + j * kCols * S, reinterpret_cast<const T*>(a.dy[j]), a.M,
-                                              p * kGradRows, a.N, mt * kCols, a.M);
+            fetch_t(nd[j], reinterpret_cast<const T*>(a.dy[j]), a.M, p * kGradRows, a.N, mt * kCols, a.M);
+    }
+    for (; p < n_panels; p += gridDim.x) {
         __syncthreads();
+        put_t<T, S>(nx, tX);
+#pragma unroll
+        for (int j = 0; j < NW; ++j) put_t<T, S>(nd[j], tD + j * kCols * S);
+        __syncthreads();
+        if (p + gridDim.x < n_panels) {
+            const int64_t q = p + gridDim.x;
+            fetch_t(nx, reinterpret_cast<const T*>(a.x), a.K, q * kGradRows, a.N, kt * kCols, a.K);
+#pragma unroll
+            for (int j = 0; j < NW; ++j)
+                fetch_t(nd[j], reinterpret_cast<const T*>(a.dy[j]), a.M, q * kGradRows, a.N, mt * kCols, a.M);
+        }
         const T* bp = tX + (32 * ki + l32) * S + h * (kGradRows / 2);
 #pragma unroll
         for (int j = 0; j < NW; ++j)
@@ -273,8 +453,18 @@ __global__ __launch_bounds__(1024) void k_linear_gradw_reduce(ReduceArgs a) {
     const int64_t e = (int64_t)blockIdx.x * 64 + el;
     const int w0 = (int)((int64_t)a.workers * sl / 16), w1 = (int)((int64_t)a.workers * (sl + 1) / 16);
     float s = 0.f;
-    if (e < total)
-        for (int w = w0; w < w1; ++w) s += a.partial[(int64_t)w * total + e];
+    if (e < total) {
+        const float* __restrict__ src = a.partial + e;
+        int w = w0;
+        for (; w + 8 <= w1; w += 8) {      // eight loads in flight, added in worker order
+            float t[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) t[i] = src[(int64_t)(w + i) * total];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s += t[i];
+        }
+        for (; w < w1; ++w) s += src[(int64_t)w * total];
+    }
     part[sl][el] = s;
     __syncthreads();
     if (sl == 0 && e < total) {
@@ -336,7 +526,8 @@ int linear_bwd_t(const void* d_x, const void* const* d_W, const void* const* d_d
         a.out[0] = d_dx;
         a.nw = n_out; a.N = N; a.K = K; a.M = M;
         KernelTimer t(KS_LINEAR_DX, st);
-        hipLaunchKernelGGL((k_linear<T, true>), dim3((unsigned)((N + kPanel - 1) / kPanel)), dim3(kThreads), 0, st, a);
+        const int rc = launch_linear<T, true>(a, st);
+        if (rc != TGT_OK) return rc;
     }
     if (d_dW) {
         const int tiles = ((K + kCols - 1) / kCols) * ((M + kCols - 1) / kCols);
@@ -385,9 +576,8 @@ int tgt_linear_fwd(const void* d_x, const void* const* d_W, const void* const* d
     if (N == 0) return TGT_OK;
     hipStream_t st = (hipStream_t)stream;
     KernelTimer t(KS_LINEAR_FWD, st);
-    const dim3 grid((unsigned)((N + kPanel - 1) / kPanel));
-    if (dtype == TGT_DTYPE_F32) hipLaunchKernelGGL((k_linear<float, false>), grid, dim3(kThreads), 0, st, a);
-    else hipLaunchKernelGGL((k_linear<pbf16, false>), grid, dim3(kThreads), 0, st, a);
+    const int lrc = dtype == TGT_DTYPE_F32 ? launch_linear<float, false>(a, st) : launch_linear<pbf16, false>(a, st);
+    if (lrc != TGT_OK) return lrc;
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
 }
