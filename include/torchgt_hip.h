@@ -173,6 +173,22 @@ int tgt_block_attn_bwd(const tgt_tiles_t* tiles, const tgt_plan_t* plan,
  * gets no self-loop. */
 int tgt_fix_edge_index(const int64_t* d_edge_index, int64_t E0, int64_t num_node, int64_t* d_out, void* stream);
 
+/* gen_sub_edge_index (gt_sp/utils.py:202-215): the edges among the nodes of a
+ * batch, renamed to batch positions.  The reference calls torch_geometric
+ * 2.0.0 (requirements.txt:208): remove_self_loops, add_self_loops(num_nodes=N),
+ * subgraph(idx_batch, relabel_nodes=True).  Result, in this order: every edge
+ * (s, d) of d_edge_index (int64 [2, E]) with s != d and both ends in
+ * d_idx_batch (int64 [S], values in [0, N)), in the input's edge order; then one
+ * self-loop per distinct batch node in ascending ORIGINAL node id.  Node
+ * idx_batch[p] is renamed p; a node listed more than once takes its last
+ * position.  d_out: int64, row 0 (sources) at d_out, row 1 (destinations) at
+ * d_out + capacity; capacity >= E + min(S, N) always suffices.  *h_num_edges
+ * (HOST) receives the number of edges written.  Synchronises `stream`.
+ * TGT_ERR_INDEX_RANGE for ids outside [0, N), TGT_ERR_WORKSPACE if capacity is
+ * too small (*h_num_edges then holds the needed size). */
+int tgt_sub_edge_index(const int64_t* d_edge_index, int64_t E, int64_t N, const int64_t* d_idx_batch, int64_t S,
+                       int64_t* d_out, int64_t capacity, int64_t* h_num_edges, void* stream);
+
 /* reformat_graph (gt_sp/utils.py:319-359) with the METIS call replaced by the
  * explicit d_partition_ids int64 [N] in [0, k):
  *   relabel: parts in order 0..k-1, members in ascending old id (:329-335);

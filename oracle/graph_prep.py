@@ -30,6 +30,35 @@ def fix_edge_index(x, num_node):
     return np.concatenate([x + 1, to_virtual, from_virtual], axis=1)
 
 
+def gen_sub_edge_index(edge_index, idx_batch, N):
+    """gt_sp/utils.py:202-215.  The reference calls three torch_geometric
+    functions (torch-geometric==2.0.0, requirements.txt:208; the package is absent
+    here, so their published algorithms are restated):
+
+    * ``remove_self_loops``: ``edge_index[:, row != col]``;
+    * ``add_self_loops(num_nodes=N)``: append ``[[0..N-1], [0..N-1]]``;
+    * ``subgraph(subset, edge_index, relabel_nodes=True, num_nodes=N)`` with an
+      index ``subset``: ``n_mask[subset] = 1``, ``n_idx[subset] = arange(len(subset))``,
+      keep the edges whose two ends are in the mask (order kept), return
+      ``n_idx[edge_index]``.
+
+    A node listed twice in ``idx_batch`` keeps the position written last
+    (sequential index assignment).  Returns int64 [2, E'].
+    """
+    e = np.asarray(edge_index, dtype=np.int64)
+    idx = np.asarray(idx_batch, dtype=np.int64)
+    e = e[:, e[0] != e[1]]                                   # remove_self_loops
+    loops = np.arange(N, dtype=np.int64)
+    e = np.concatenate([e, np.stack([loops, loops])], axis=1)   # add_self_loops
+    n_mask = np.zeros(N, dtype=bool)
+    n_mask[idx] = True
+    n_idx = np.zeros(N, dtype=np.int64)
+    for p, v in enumerate(idx):                               # n_idx[subset] = arange(S), in order
+        n_idx[v] = p
+    keep = n_mask[e[0]] & n_mask[e[1]]
+    return n_idx[e[:, keep]]
+
+
 def adjust_edge_index_nomerge(edge_index, sub_seq_len):
     """gt_sp/utils.py:53-58: idx + (idx-1)//L for idx > 0 (float floor-divide
     in the reference; exact for idx < 2**24).  Identity when every idx <= L."""

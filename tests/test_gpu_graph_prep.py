@@ -91,3 +91,64 @@ def test_reformat_errors(cuda):
     assert exc.value.code == _lib.ERR_INVALID_ARG
     with pytest.raises(ValueError):
         graph_prep.reformat_graph(ei, 2, 16)
+
+
+def _check_sub(e, idx, N, cuda):
+    print(f"sub_edge_index case: N={N} E={e.shape[1]} S={len(idx)}", flush=True)
+    want = ogp.gen_sub_edge_index(e, idx, N)
+    got = graph_prep.gen_sub_edge_index(torch.as_tensor(e, dtype=torch.int64).to(cuda), torch.as_tensor(np.asarray(idx), dtype=torch.int64), N)
+    assert got.dtype == torch.int64 and got.is_contiguous()
+    np.testing.assert_array_equal(got.cpu().numpy(), want)
+
+
+def test_gen_sub_edge_index_matches_oracle(cuda):
+    rng = np.random.default_rng(0)
+    _check_sub(np.array([[0, 1, 2, 3, 4, 1, 5, 2], [1, 1, 3, 2, 5, 0, 5, 0]]), [3, 0, 2], 6, cuda)      # known answer
+    _check_sub(rng.integers(0, 50, size=(2, 400)), rng.permutation(50)[:17], 50, cuda)
+    _check_sub(rng.integers(0, 50, size=(2, 400)), rng.integers(0, 50, size=23), 50, cuda)              # repeated nodes
+    _check_sub(np.zeros((2, 0), dtype=np.int64), [2, 1], 4, cuda)                                       # no edges
+    _check_sub(np.array([[0, 1], [1, 0]]), [], 3, cuda)                                                 # empty batch
+    _check_sub(rng.integers(0, 5000, size=(2, 70001)), rng.permutation(5000)[:1025], 5000, cuda)        # ragged tiles
+    e, n = workloads.power_law_graph()                       # 64 K nodes, 530 K edges; a 16 K-node batch
+    _check_sub(e, rng.permutation(n)[:16384], n, cuda)
+    _check_sub(e, np.arange(n), n, cuda)                     # the whole graph: every edge survives
+
+
+def test_gen_sub_edge_index_errors(cuda):
+    e = torch.tensor([[0, 1], [1, 7]], device=cuda)
+    with pytest.raises(_lib.TorchGTHipError) as ei:
+        graph_prep.gen_sub_edge_index(e, torch.tensor([0, 1]), 4)          # endpoint 7 outside [0, 4)
+    assert ei.value.code == _lib.ERR_INDEX_RANGE
+    with pytest.raises(_lib.TorchGTHipError) as ei:
+        graph_prep.gen_sub_edge_index(torch.tensor([[0], [1]], device=cuda), torch.tensor([0, 9]), 4)
+    assert ei.value.code == _lib.ERR_INDEX_RANGE
+    with pytest.raises(RuntimeError):
+        graph_prep.gen_sub_edge_index(torch.tensor([[0], [1]]), torch.tensor([0]), 4)      # CPU tensor
+
+
+def test_prepare_batch_composes_the_reference_steps(cuda):
+    """prepare_batch = the oracle's gen_sub_edge_index -> fix_edge_index -> reformat_graph ->
+    adjust_edge_index_nomerge, with x and y permuted by the sorted indices (gt_sp/utils.py:409-520, one rank)."""
+    rng = np.random.default_rng(5)
+    e, n = workloads.power_law_graph(n=4000, directed_edges=40000)
+    S, k, bs = 1024, 4, 16
+    idx = rng.permutation(n)[:S]
+    x = torch.randn(n, 12, generator=torch.Generator().manual_seed(0))
+    y = torch.randint(0, 40, (n,), generator=torch.Generator().manual_seed(1))
+    part = rng.integers(0, k, size=S + 1)
+    sub = ogp.fix_edge_index(ogp.gen_sub_edge_index(e, idx, n), S)
+    want_ei, want_sorted = ogp.reformat_graph(sub, part, k, bs)
+    want_ei = ogp.adjust_edge_index_nomerge(want_ei, S)
+    order = want_sorted[want_sorted != 0] - 1
+    x_i, y_i, ei, bias = graph_prep.prepare_batch(x.to(cuda), y.to(cuda), torch.as_tensor(idx), torch.as_tensor(e).to(cuda), n, k, bs,
+                                                  torch.as_tensor(part))
+    assert bias is None
+    np.testing.assert_array_equal(ei.cpu().numpy(), want_ei)
+    assert torch.equal(x_i.cpu(), x[idx][order]) and torch.equal(y_i.cpu(), y[idx][order])
+    # a callable partitioner sees the sub-graph
+    seen = {}
+    def partition(ei_sub, n_sub, kk):
+        seen["args"] = (tuple(ei_sub.shape), n_sub, kk)
+        return torch.as_tensor(part)
+    out2 = graph_prep.prepare_batch(x.to(cuda), y.to(cuda), torch.as_tensor(idx), torch.as_tensor(e).to(cuda), n, k, bs, partition)
+    assert seen["args"] == ((2, sub.shape[1]), S + 1, k) and torch.equal(out2[2], ei)

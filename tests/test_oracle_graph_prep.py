@@ -115,3 +115,51 @@ def test_build_csr_invariants(by):
         assert np.all(key[seg] == r)
         assert np.all(np.diff(seg) > 0)             # stable: caller's order inside a row
     np.testing.assert_array_equal(col, other[eid])
+
+
+def test_gen_sub_edge_index_known_answer():
+    # N = 6; batch [3, 0, 2] renames 3 -> 0, 0 -> 1, 2 -> 2.  Input self-loops (1,1), (5,5) are dropped;
+    # kept, in input order: (2,3) (3,2) (2,0); then the batch nodes' self-loops in ascending ORIGINAL id 0, 2, 3.
+    e = np.array([[0, 1, 2, 3, 4, 1, 5, 2],
+                  [1, 1, 3, 2, 5, 0, 5, 0]])
+    got = gp.gen_sub_edge_index(e, [3, 0, 2], 6)
+    want = np.array([[2, 0, 2, 1, 2, 0],
+                     [0, 2, 1, 1, 2, 0]])
+    np.testing.assert_array_equal(got, want)
+
+
+def _sub_edge_index_bruteforce(e, idx, N):
+    """Independent statement: Python loops and a dict."""
+    pos = {}
+    for p, v in enumerate(idx):
+        pos[int(v)] = p                      # the last position of a repeated node wins
+    out = []
+    for s, d in zip(e[0].tolist(), e[1].tolist()):
+        if s != d and s in pos and d in pos:
+            out.append((pos[s], pos[d]))
+    for v in range(N):
+        if v in pos:
+            out.append((pos[v], pos[v]))
+    return np.array(out, dtype=np.int64).reshape(-1, 2).T
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_gen_sub_edge_index_matches_bruteforce(seed):
+    rng = np.random.default_rng(seed)
+    N, E = 50, 400
+    e = rng.integers(0, N, size=(2, E))
+    idx = rng.permutation(N)[:17] if seed < 2 else rng.integers(0, N, size=23)     # seed 2: repeated nodes
+    got = gp.gen_sub_edge_index(e, idx, N)
+    np.testing.assert_array_equal(got, _sub_edge_index_bruteforce(e, idx, N))
+    # every kept edge maps back to an input edge or to a self-loop of a batch node
+    back = np.asarray(idx)[got]
+    pairs = set(zip(e[0].tolist(), e[1].tolist()))
+    for s, d in zip(back[0].tolist(), back[1].tolist()):
+        assert s == d or (s, d) in pairs
+    assert (got[0] == got[1]).sum() == len(set(np.asarray(idx).tolist()))
+
+
+def test_gen_sub_edge_index_empty_batch_and_no_edges():
+    e = np.zeros((2, 0), dtype=np.int64)
+    np.testing.assert_array_equal(gp.gen_sub_edge_index(e, [2, 1], 4), np.array([[1, 0], [1, 0]]))
+    assert gp.gen_sub_edge_index(np.array([[0, 1], [1, 0]]), [], 3).shape == (2, 0)

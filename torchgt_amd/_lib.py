@@ -46,6 +46,7 @@ SIGNATURES = {
     "tgt_reformat_num_raw_edges": (_i64, [_vp]),
     "tgt_reformat_export_tiles": (_i32, [_vp, _vp, _vp, _vp]),
     "tgt_fix_edge_index": (_i32, [_vp, _i64, _i64, _vp, _vp]),
+    "tgt_sub_edge_index": (_i32, [_vp, _i64, _i64, _vp, _i64, _vp, _i64, _c.POINTER(_i64), _vp]),
     "tgt_reformat_create": (_i32, [_vp, _vp, _i64, _i64, _vp, _i32, _i32, _i32, _vp, _c.POINTER(_vp)]),
     "tgt_reformat_num_edges": (_i64, [_vp]),
     "tgt_reformat_export": (_i32, [_vp, _vp, _vp, _vp]),

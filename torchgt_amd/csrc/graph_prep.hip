@@ -2,6 +2,7 @@
 // batch preparation.
 //
 //   tgt_fix_edge_index      gt_sp/utils.py:34-50   (global node 0, edges to and from it)
+//   tgt_sub_edge_index      gt_sp/utils.py:202-215 (edges among the nodes of a batch, renamed)
 //   tgt_reformat_*          gt_sp/utils.py:319-359 (relabel by partition, cluster
 //                           "blockize" of gt_sp/utils.py:223-305, stable sort by source)
 //
@@ -422,6 +423,150 @@ static int reformat_impl(const int64_t* d_src, const int64_t* d_dst, int64_t E, 
     return TGT_OK;
 }
 
+// ---------------------------------------------------------------------------
+// Sub-graph of a node batch (gen_sub_edge_index, gt_sp/utils.py:202-215): the
+// sequence of torch_geometric 2.0.0 calls
+//   remove_self_loops(edge_index)              keep edges with src != dst, in order
+//   add_self_loops(.., num_nodes=N)            append (i, i) for i = 0..N-1
+//   subgraph(idx_batch, .., relabel_nodes=True, num_nodes=N)
+//                                              keep edges with both ends in the batch, in
+//                                              order, and rename node idx_batch[p] to p
+// as one order-preserving compaction over the E edges followed by the N
+// self-loops.  A node that occurs more than once in idx_batch takes its LAST
+// position (what the sequential index assignment n_idx[subset] = arange gives).
+// ---------------------------------------------------------------------------
+constexpr int kSubItems = 1024;     // items per workgroup of the compaction (4 rounds of 256)
+
+__global__ void k_sub_fill(int32_t* __restrict__ pos, int64_t N) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < N) pos[i] = -1;
+}
+
+__global__ void k_sub_positions(const int64_t* __restrict__ idx, int64_t S, int64_t N, int32_t* __restrict__ pos,
+                                int* __restrict__ bad) {
+    const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= S) return;
+    const int64_t v = idx[p];
+    if (v < 0 || v >= N) { atomicOr(bad, 1); return; }
+    atomicMax(&pos[v], (int32_t)p);
+}
+
+// item i < E: edge i; item E + v: self-loop of node v.  Returns the renamed endpoints.
+__device__ __forceinline__ bool sub_item(const int64_t* __restrict__ ei, int64_t E, int64_t N,
+                                         const int32_t* __restrict__ pos, int64_t i, int32_t& a, int32_t& b,
+                                         int* __restrict__ bad) {
+    if (i < E) {
+        const int64_t s = ei[i], d = ei[E + i];
+        if (s < 0 || s >= N || d < 0 || d >= N) { atomicOr(bad, 2); return false; }
+        if (s == d) return false;
+        a = pos[s]; b = pos[d];
+        return a >= 0 && b >= 0;
+    }
+    a = b = pos[i - E];
+    return a >= 0;
+}
+
+// pass 0 counts the kept items of every workgroup; pass 1 writes them behind the
+// workgroup's offset, in item order (ballot ranks inside a wave, wave totals in LDS).
+template <int PASS>
+__global__ __launch_bounds__(256) void k_sub_compact(const int64_t* __restrict__ ei, int64_t E, int64_t N,
+                                                     const int32_t* __restrict__ pos, uint32_t* __restrict__ counts,
+                                                     int64_t* __restrict__ out, int64_t capacity,
+                                                     int* __restrict__ bad) {
+    __shared__ uint32_t wave_n[4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t total = E + N;
+    uint32_t run = PASS ? counts[blockIdx.x] : 0u;          // pass 1: exclusive prefix of this workgroup
+    for (int round = 0; round < kSubItems / 256; ++round) {
+        const int64_t i = (int64_t)blockIdx.x * kSubItems + round * 256 + threadIdx.x;
+        int32_t a = 0, b = 0;
+        const bool keep = i < total && sub_item(ei, E, N, pos, i, a, b, bad);
+        const uint64_t m = __ballot(keep);
+        if (lane == 0) wave_n[wave] = (uint32_t)__popcll(m);
+        __syncthreads();
+        uint32_t before = 0, all = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            if (w < wave) before += wave_n[w];
+            all += wave_n[w];
+        }
+        if (PASS && keep) {
+            const int64_t o = (int64_t)run + before + __popcll(m & ((1ull << lane) - 1ull));
+            out[o] = a;
+            out[capacity + o] = b;
+        }
+        run += all;
+        __syncthreads();
+    }
+    if (!PASS && threadIdx.x == 0) counts[blockIdx.x] = run;
+}
+
+// exclusive prefix of the workgroup counts in place (one workgroup), total to counts[n]
+__global__ __launch_bounds__(256) void k_sub_scan(uint32_t* __restrict__ counts, int n) {
+    __shared__ uint32_t part[256];
+    const int tid = threadIdx.x;
+    const int chunk = (n + 255) / 256;
+    const int b = min(tid * chunk, n), e = min(b + chunk, n);
+    uint32_t sum = 0;
+    for (int i = b; i < e; ++i) sum += counts[i];
+    part[tid] = sum;
+    __syncthreads();
+    for (int off = 1; off < 256; off <<= 1) {
+        const uint32_t x = tid >= off ? part[tid - off] : 0u;
+        __syncthreads();
+        part[tid] += x;
+        __syncthreads();
+    }
+    uint32_t run = tid ? part[tid - 1] : 0u;
+    for (int i = b; i < e; ++i) {
+        const uint32_t x = counts[i];
+        counts[i] = run;
+        run += x;
+    }
+    if (tid == 255) counts[n] = part[255];
+}
+
+static int sub_edge_index_impl(const int64_t* d_ei, int64_t E, int64_t N, const int64_t* d_idx, int64_t S,
+                               int64_t* d_out, int64_t capacity, int64_t* h_num, hipStream_t st) {
+    const int64_t total = E + N;
+    const int nblocks = (int)((total + kSubItems - 1) / kSubItems);
+    DevBuf pos, counts, bad;
+    TGT_HIP_CHECK(pos.alloc(sizeof(int32_t) * (size_t)N));
+    TGT_HIP_CHECK(counts.alloc(sizeof(uint32_t) * (size_t)(nblocks + 1)));
+    TGT_HIP_CHECK(bad.alloc(sizeof(int)));
+    TGT_HIP_CHECK(hipMemsetAsync(bad.p, 0, sizeof(int), st));
+    hipLaunchKernelGGL(k_sub_fill, dim3(nblk(N)), dim3(256), 0, st, pos.as<int32_t>(), N);
+    if (S > 0)
+        hipLaunchKernelGGL(k_sub_positions, dim3(nblk(S)), dim3(256), 0, st, d_idx, S, N, pos.as<int32_t>(),
+                           bad.as<int>());
+    hipLaunchKernelGGL((k_sub_compact<0>), dim3(nblocks), dim3(256), 0, st, d_ei, E, N, pos.as<int32_t>(),
+                       counts.as<uint32_t>(), (int64_t*)nullptr, (int64_t)0, bad.as<int>());
+    hipLaunchKernelGGL(k_sub_scan, dim3(1), dim3(256), 0, st, counts.as<uint32_t>(), nblocks);
+    TGT_HIP_CHECK(hipGetLastError());
+    uint32_t n_keep = 0;
+    int h_bad = 0;
+    TGT_HIP_CHECK(hipMemcpyAsync(&n_keep, counts.as<uint32_t>() + nblocks, sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+    TGT_HIP_CHECK(hipMemcpyAsync(&h_bad, bad.p, sizeof(int), hipMemcpyDeviceToHost, st));
+    TGT_HIP_CHECK(hipStreamSynchronize(st));
+    if (h_bad) {
+        set_error("tgt_sub_edge_index: %s outside [0, %lld)", (h_bad & 1) ? "a batch node id is" : "an edge endpoint is",
+                  (long long)N);
+        return TGT_ERR_INDEX_RANGE;
+    }
+    *h_num = (int64_t)n_keep;
+    if ((int64_t)n_keep > capacity) {
+        set_error("tgt_sub_edge_index: %lld edges kept, room for %lld", (long long)n_keep, (long long)capacity);
+        return TGT_ERR_WORKSPACE;
+    }
+    if (n_keep > 0) {
+        hipLaunchKernelGGL((k_sub_compact<1>), dim3(nblocks), dim3(256), 0, st, d_ei, E, N, pos.as<int32_t>(),
+                           counts.as<uint32_t>(), d_out, capacity, bad.as<int>());
+        TGT_HIP_CHECK(hipGetLastError());
+        TGT_HIP_CHECK(hipStreamSynchronize(st));      // the scratch buffers are freed on return
+    }
+    return TGT_OK;
+}
+
 }  // namespace tgt
 
 extern "C" {
@@ -437,6 +582,21 @@ int tgt_fix_edge_index(const int64_t* d_edge_index, int64_t E0, int64_t num_node
                        E0, num_node, d_out);
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
+}
+
+int tgt_sub_edge_index(const int64_t* d_edge_index, int64_t E, int64_t N, const int64_t* d_idx_batch, int64_t S,
+                       int64_t* d_out, int64_t capacity, int64_t* h_num_edges, void* stream) {
+    if (E < 0 || N < 1 || S < 0 || capacity < 0 || !h_num_edges || (E > 0 && !d_edge_index) || (S > 0 && !d_idx_batch) ||
+        (capacity > 0 && !d_out)) {
+        tgt::set_error("tgt_sub_edge_index: null pointer or bad size");
+        return TGT_ERR_INVALID_ARG;
+    }
+    if (E > 0x7fff0000LL || N > 0x7fff0000LL || S > 0x7fff0000LL) {
+        tgt::set_error("tgt_sub_edge_index: E, N and the batch size must fit 31 bits");
+        return TGT_ERR_INVALID_ARG;
+    }
+    return tgt::sub_edge_index_impl(d_edge_index, E, N, d_idx_batch, S, d_out, capacity, h_num_edges,
+                                    (hipStream_t)stream);
 }
 
 int tgt_np_legacy_randint(uint32_t seed, const int64_t* h_highs, int n, int64_t* h_out) {
