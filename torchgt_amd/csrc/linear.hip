@@ -61,19 +61,68 @@ __device__ __forceinline__ float16_t zero16() {
     return z;
 }
 
+// The 16 accumulator values of a lane (rows 8*(r/4) + r%4 below its first row, one
+// column) plus a bias.  All values are formed before the first store and a wave
+// whose rows all exist stores without per-row branches: with a branch per store
+// the compiler reuses one data register and waits for each store to finish.
+template <typename T>
+__device__ __forceinline__ void store_rows(T* __restrict__ out, int64_t ld, const float16_t& acc, float bias,
+                                           int64_t rows_left) {
+    float v[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) v[r] = acc[r] + bias;
+    // a lane writes rows 0..27 below its first row and the lanes of a wave differ by 4 in rows_left:
+    // 32 rows left for the first lane means every row of every lane exists
+    if (__builtin_amdgcn_readfirstlane(rows_left >= 32 ? 1 : 0)) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) st1(out + (8 * (r >> 2) + (r & 3)) * ld, v[r]);
+    } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            if (8 * (r >> 2) + (r & 3) < rows_left) st1(out + (8 * (r >> 2) + (r & 3)) * ld, v[r]);
+    }
+}
+
+// 16 bytes of src[row * ld + col ..], zero if (row, col) lies outside [0,nrows) x [0,ncols).
+// The address is clamped into the array and the result selected, so the load is
+// unconditional: a branch around it would make the compiler wait for every load
+// before issuing the next.  nrows >= 1; ncols is a multiple of the vector width.
+template <typename T>
+__device__ __forceinline__ uint4 load16_clamped(const T* __restrict__ src, int64_t ld, int64_t row, int64_t nrows,
+                                                int col, int ncols) {
+    constexpr int VE = 16 / (int)sizeof(T);
+    const int64_t rr = row < nrows ? row : nrows - 1;
+    const int cc = col < ncols ? col : ncols - VE;
+    return *reinterpret_cast<const uint4*>(src + rr * ld + cc);
+}
+__device__ __forceinline__ uint4 zero_unless(bool ok, uint4 u) {
+    u.x = ok ? u.x : 0u; u.y = ok ? u.y : 0u; u.z = ok ? u.z : 0u; u.w = ok ? u.w : 0u;
+    return u;
+}
+template <typename T>
+__device__ __forceinline__ uint4 load16_or_zero(const T* __restrict__ src, int64_t ld, int64_t row, int64_t nrows,
+                                                int col, int ncols) {
+    return zero_unless(row < nrows && col < ncols, load16_clamped(src, ld, row, nrows, col, ncols));
+}
+
 // tile[r][c] = src[(row0 + r) * ld + col0 + c], r < R, c < 64; zero outside [0,nrows) x [0,ncols)
 template <typename T, int R, int STRIDE>
 __device__ __forceinline__ void stage_natural(T* __restrict__ tile, const T* __restrict__ src, int64_t ld,
                                               int64_t row0, int64_t nrows, int col0, int ncols) {
     constexpr int VE = 16 / (int)sizeof(T);
     constexpr int VPR = kChunk / VE;
+    constexpr int NV = R * VPR / kThreads;
+    static_assert(R * VPR % kThreads == 0, "tile shape");
+    uint4 val[NV];            // all loads are issued before the first LDS write
 #pragma unroll
-    for (int v = threadIdx.x; v < R * VPR; v += kThreads) {
-        const int r = v / VPR, c = (v % VPR) * VE;
-        uint4 val = make_uint4(0u, 0u, 0u, 0u);
-        if (row0 + r < nrows && col0 + c < ncols)
-            val = *reinterpret_cast<const uint4*>(src + (row0 + r) * ld + col0 + c);
-        *reinterpret_cast<uint4*>(tile + r * STRIDE + c) = val;
+    for (int i = 0; i < NV; ++i) {
+        const int v = threadIdx.x + i * kThreads, r = v / VPR, c = (v % VPR) * VE;
+        val[i] = load16_or_zero(src, ld, row0 + r, nrows, col0 + c, ncols);
+    }
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int v = threadIdx.x + i * kThreads, r = v / VPR, c = (v % VPR) * VE;
+        *reinterpret_cast<uint4*>(tile + r * STRIDE + c) = val[i];
     }
 }
 
@@ -85,16 +134,24 @@ __device__ __forceinline__ void stage_transposed(T* __restrict__ tile, const T* 
                                                  int64_t row0, int64_t nrows, int col0, int ncols) {
     constexpr int VE = 16 / (int)sizeof(T);
     constexpr int VPR = kChunk / VE;
-    static_assert(R % 16 == 0 && VPR % 4 == 0, "tile shape");
+    constexpr int NV = R * VPR / kThreads;
+    static_assert(R % 16 == 0 && VPR % 4 == 0 && R * VPR % kThreads == 0, "tile shape");
+    uint4 val[NV];
 #pragma unroll
-    for (int v = threadIdx.x; v < R * VPR; v += kThreads) {
+    for (int i = 0; i < NV; ++i) {
+        const int v = threadIdx.x + i * kThreads;
         const int cq = v & 3, r_lo = (v >> 2) & 15, rest = v >> 6;
         const int r = (rest % (R / 16)) * 16 + r_lo;
         const int c = ((rest / (R / 16)) * 4 + cq) * VE;
-        uint4 val = make_uint4(0u, 0u, 0u, 0u);
-        if (row0 + r < nrows && col0 + c < ncols)
-            val = *reinterpret_cast<const uint4*>(src + (row0 + r) * ld + col0 + c);
-        const T* e = reinterpret_cast<const T*>(&val);
+        val[i] = load16_or_zero(src, ld, row0 + r, nrows, col0 + c, ncols);
+    }
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int v = threadIdx.x + i * kThreads;
+        const int cq = v & 3, r_lo = (v >> 2) & 15, rest = v >> 6;
+        const int r = (rest % (R / 16)) * 16 + r_lo;
+        const int c = ((rest / (R / 16)) * 4 + cq) * VE;
+        const T* e = reinterpret_cast<const T*>(&val[i]);
 #pragma unroll
         for (int t = 0; t < VE; ++t) tile[(c + t) * STRIDE + r] = e[t];
     }
@@ -121,19 +178,21 @@ __device__ __forceinline__ void fetch_t(PieceRegs<T>& t, const T* __restrict__ s
     for (int i = 0; i < NV; ++i) {
         int r, c;
         piece_pos<T, 64>(i, r, c);
-        uint4 u = make_uint4(0u, 0u, 0u, 0u);
-        if (row0 + r < nrows && col0 + c < ncols) u = *reinterpret_cast<const uint4*>(src + (row0 + r) * ld + col0 + c);
-        t.v[i] = u;
+        t.v[i] = load16_clamped(src, ld, row0 + r, nrows, col0 + c, ncols);
     }
 }
+// (the pieces outside the array are zeroed here, not in fetch_t: touching the loaded
+// values there would make the wave wait for the loads at once)
 template <typename T, int STRIDE>
-__device__ __forceinline__ void put_t(const PieceRegs<T>& t, T* __restrict__ tile) {
+__device__ __forceinline__ void put_t(const PieceRegs<T>& t, T* __restrict__ tile, int64_t row0, int64_t nrows,
+                                      int col0, int ncols) {
     constexpr int VE = 16 / (int)sizeof(T), NV = (int)(sizeof(PieceRegs<T>) / 16);
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         int r, c;
         piece_pos<T, 64>(i, r, c);
-        const T* e = reinterpret_cast<const T*>(&t.v[i]);
+        const uint4 u = zero_unless(row0 + r < nrows && col0 + c < ncols, t.v[i]);
+        const T* e = reinterpret_cast<const T*>(&u);
 #pragma unroll
         for (int k = 0; k < VE; ++k) tile[(c + k) * STRIDE + r] = e[k];
     }
@@ -222,11 +281,8 @@ __global__ __launch_bounds__(kThreads) void k_linear(LinArgs a) {
                 if (col >= C) continue;
                 const float bv = bias ? ld1(bias + col) : 0.f;
                 const float16_t& acc = cb ? acc1 : acc0;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int64_t row = row0 + wave * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                    if (row < a.N) st1(out + row * C + col, acc[r] + bv);
-                }
+                const int64_t first = row0 + wave * 32 + 4 * h;
+                store_rows<T>(out + first * C + col, C, acc, bv, a.N - first);
             }
         }
     }
@@ -243,9 +299,8 @@ __device__ __forceinline__ void tile_fetch(TileRegs<T>& t, const T* __restrict__
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int v = threadIdx.x + i * kThreads, r = v / VPR, c = (v % VPR) * VE;
-        uint4 u = make_uint4(0u, 0u, 0u, 0u);
-        if (row0 + r < nrows) u = *reinterpret_cast<const uint4*>(src + (row0 + r) * 64 + c);
-        t.v[i] = u;
+        t.v[i] = load16_clamped(src, 64, row0 + r, nrows, c, 64);     // rows past the end repeat the last row: their
+                                                                      // products land in output rows that are not stored
     }
 }
 template <typename T, int STRIDE>
@@ -291,6 +346,10 @@ __global__ __launch_bounds__(kThreads) void k_linear64(LinArgs a) {
         const T* bias = DX ? nullptr : reinterpret_cast<const T*>(a.bias[o]);
         bv[o] = bias ? ld1(bias + 32 * cb + l32) : 0.f;
     }
+    // use the bias values once here, so that the wait for their loads stands before the loop and
+    // not inside it, where it would also wait for the prefetched panel
+#pragma unroll
+    for (int o = 0; o < NO; ++o) asm volatile("" ::"v"(bv[o]));
     for (; p < n_panels; p += gridDim.x) {
         __syncthreads();                 // the previous panel has been read
 #pragma unroll
@@ -308,12 +367,8 @@ __global__ __launch_bounds__(kThreads) void k_linear64(LinArgs a) {
             for (int s = 0; s < NA; ++s)
                 Mma<T, 64>::run(tA + (s * 64 + 32 * rb + l32) * S + h * 32,
                                 tW + ((DX ? s : o) * 64 + 32 * cb + l32) * S + h * 32, acc);
-            T* out = reinterpret_cast<T*>(a.out[o]) + 32 * cb + l32;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int64_t row = p * 64 + 32 * rb + 8 * (r >> 2) + 4 * h + (r & 3);
-                if (row < a.N) st1(out + row * 64, acc[r] + bv[o]);
-            }
+            T* out = reinterpret_cast<T*>(a.out[o]) + (p * 64 + 32 * rb + 4 * h) * 64 + 32 * cb + l32;
+            store_rows<T>(out, 64, acc, bv[o], a.N - (p * 64 + 32 * rb + 4 * h));
         }
     }
 }
@@ -395,9 +450,9 @@ __global__ __launch_bounds__(kThreads) void k_linear_gradw(GradWArgs a) {
     }
     for (; p < n_panels; p += gridDim.x) {
         __syncthreads();
-        put_t<T, S>(nx, tX);
+        put_t<T, S>(nx, tX, p * kGradRows, a.N, kt * kCols, a.K);
 #pragma unroll
-        for (int j = 0; j < NW; ++j) put_t<T, S>(nd[j], tD + j * kCols * S);
+        for (int j = 0; j < NW; ++j) put_t<T, S>(nd[j], tD + j * kCols * S, p * kGradRows, a.N, mt * kCols, a.M);
         __syncthreads();
         if (p + gridDim.x < n_panels) {
             const int64_t q = p + gridDim.x;
