@@ -230,7 +230,7 @@ int tgt_np_legacy_randint(uint32_t seed, const int64_t* h_highs, int n, int64_t*
  * (nn.Linear.weight); d_b[j]: [out_features] (d_b or an entry may be NULL: no
  * bias); d_y[j]: [N, out_features]; all of `dtype`, fp32 accumulation.  d_W, d_b,
  * d_y are HOST arrays of n_out device pointers.  in_features and out_features
- * must be multiples of 8. */
+ * must be multiples of 4 (fp32) or 8 (bf16): rows are read in 16-byte pieces. */
 int tgt_linear_fwd(const void* d_x, const void* const* d_W, const void* const* d_b, void* const* d_y, int n_out,
                    int64_t N, int in_features, int out_features, int dtype, void* stream);
 
@@ -246,6 +246,34 @@ int64_t tgt_linear_bwd_workspace_bytes(int n_out, int in_features, int out_featu
 int tgt_linear_bwd(const void* d_x, const void* const* d_W, const void* const* d_dy, int n_out, int64_t N,
                    int in_features, int out_features, int dtype, void* d_dx, void* const* d_dW, void* const* d_db,
                    void* d_workspace, int64_t workspace_bytes, void* stream);
+
+/* ---- the rest of the encoder layer ------------------------------------------
+ * EncoderLayer.forward (models/graphormer_dist_node_level.py:296-314): each residual
+ * block is  x = x + f(LayerNorm(x)).  One pass forms the residual sum and the
+ * LayerNorm that follows it:
+ *   s = x (+ r when d_r != NULL), written to d_sum when d_sum != NULL;
+ *   y = (s - mean) / sqrt(var + eps) * gamma + beta   (nn.LayerNorm: biased variance
+ *   over the C features of a row), written to d_y when d_y != NULL.
+ * d_x, d_r, d_sum, d_y: [N, C]; d_gamma, d_beta: [C]; all of `dtype`, statistics in
+ * fp32.  d_mean, d_rstd: float32 [N], saved for the backward (may be NULL).
+ * C must be 16-byte vectors times a power of two of at most 64 lanes
+ * (fp32: 8, 16, ..., 256; bf16: 16, 32, ..., 512). */
+int tgt_add_layer_norm_fwd(const void* d_x, const void* d_r, const void* d_gamma, const void* d_beta, int64_t N, int C,
+                           float eps, int dtype, void* d_sum, void* d_y, float* d_mean, float* d_rstd, void* stream);
+/* Backward of y = LayerNorm(s) (autograd of nn.LayerNorm in the reference):
+ *   ds = LayerNorm-backward(dy) (+ d_ds_extra when != NULL: the gradient that reaches s
+ *   through the residual path), dgamma = sum_rows dy * xhat, dbeta = sum_rows dy.
+ * The column sums are formed per workgroup and added in a fixed order.
+ * d_workspace: tgt_layer_norm_bwd_workspace_bytes(C) bytes, 16-byte aligned. */
+int64_t tgt_layer_norm_bwd_workspace_bytes(int C);
+int tgt_layer_norm_bwd(const void* d_s, const void* d_gamma, const float* d_mean, const float* d_rstd, const void* d_dy,
+                       const void* d_ds_extra, int64_t N, int C, int dtype, void* d_ds, void* d_dgamma, void* d_dbeta,
+                       void* d_workspace, int64_t workspace_bytes, void* stream);
+/* nn.GELU() of FeedForwardNetwork (models/graphormer_dist_node_level.py:32,37), exact
+ * erf form, on n elements (n a multiple of 4 for fp32, 8 for bf16):
+ * h = 0.5 u (1 + erf(u / sqrt 2));  backward: du = dh * dh/du evaluated at u. */
+int tgt_gelu_fwd(const void* d_u, int64_t n, int dtype, void* d_h, void* stream);
+int tgt_gelu_bwd(const void* d_u, const void* d_dh, int64_t n, int dtype, void* d_du, void* stream);
 
 /* ---- per-kernel timing --------------------------------------------------
  * The reference times this path with torch.profiler around whole iterations

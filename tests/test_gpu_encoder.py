@@ -1,0 +1,171 @@
+"""GPU parity of the encoder-layer kernels (residual add + LayerNorm, GELU) and of the
+EncoderLayer / Graphormer modules with the oracle.
+
+Error measure: max|a - b| / max|b| against float64 on the same inputs.  Bars:
+float32 1e-5; bf16 2e-2 for single kernels, 3x that for whole modules (every
+intermediate tensor is rounded to bf16 between kernels).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import encoder_layer as E
+from oracle import graph_prep as ogp
+from oracle import sparse_attention as osa
+from torchgt_amd import EncoderLayer, Graphormer, _lib, workloads
+from torchgt_amd.encoder import AddFunction, AddLayerNormFunction, GeluFunction
+
+pytestmark = pytest.mark.gpu
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2}
+
+
+def err(a, b):
+    a = a.detach().double().cpu().numpy()
+    b = b.detach().double().cpu().numpy() if isinstance(b, torch.Tensor) else np.asarray(b, np.float64)
+    assert a.shape == b.shape, (a.shape, b.shape)
+    denom = np.abs(b).max()
+    return np.abs(a - b).max() / (denom if denom > 0 else 1.0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("C", [64, 16, 128, 256])
+def test_add_layer_norm_forward_backward(cuda, dtype, C):
+    for N, with_r in ((1000, True), (37, False), (1, True)):
+        print(f"add_layer_norm case: N={N} C={C} {dtype} residual={with_r}", flush=True)
+        g = torch.Generator().manual_seed(N + C)
+        x = (torch.randn(N, C, generator=g) * 2 + 0.5).to(dtype)
+        r = torch.randn(N, C, generator=g).to(dtype) if with_r else None
+        gamma, beta = (torch.randn(C, generator=g) + 1).to(dtype), torch.randn(C, generator=g).to(dtype)
+        ds_out, dy = torch.randn(N, C, generator=g).to(dtype), torch.randn(N, C, generator=g).to(dtype)
+        # float64 with torch's own layer_norm + autograd
+        leaves = [t.double().requires_grad_(True) for t in ([x, r] if with_r else [x]) + [gamma, beta]]
+        s_ref = leaves[0] + leaves[1] if with_r else leaves[0] * 1.0
+        y_ref = torch.nn.functional.layer_norm(s_ref, (C,), leaves[-2], leaves[-1], 1e-5)
+        g_ref = torch.autograd.grad([s_ref, y_ref], leaves, [ds_out.double(), dy.double()])
+        cl = [t.to(cuda).requires_grad_(True) for t in ([x, r] if with_r else [x]) + [gamma, beta]]
+        s, y = AddLayerNormFunction.apply(cl[0], cl[1] if with_r else None, cl[-2], cl[-1], 1e-5)
+        g_got = torch.autograd.grad([s, y], cl, [ds_out.to(cuda), dy.to(cuda)])
+        tol = TOL[dtype]
+        assert err(s, s_ref) <= tol and err(y, y_ref) <= tol, (err(s, s_ref), err(y, y_ref))
+        for nm, a, b in zip(["x"] + (["r"] if with_r else []) + ["gamma", "beta"], g_got, g_ref):
+            assert err(a, b) <= tol, f"d{nm} err {err(a, b)}"
+
+
+def test_layer_norm_rejects_unsupported_width(cuda):
+    x = torch.zeros(4, 24, device=cuda)
+    w = torch.ones(24, device=cuda)
+    with pytest.raises(_lib.TorchGTHipError) as ei:
+        AddLayerNormFunction.apply(x, None, w, w, 1e-5)          # 24 / 4 = 6 lanes: not a power of two
+    assert ei.value.code == _lib.ERR_UNSUPPORTED
+    with pytest.raises(RuntimeError):
+        GeluFunction.apply(torch.zeros(8))                        # CPU tensor: no fallback
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gelu_and_add(cuda, dtype):
+    g = torch.Generator().manual_seed(0)
+    u = (torch.randn(3001, 64, generator=g) * 3).to(dtype)
+    dh = torch.randn(3001, 64, generator=g).to(dtype)
+    ud = u.double().requires_grad_(True)
+    h_ref = torch.nn.functional.gelu(ud)
+    (du_ref,) = torch.autograd.grad(h_ref, ud, dh.double())
+    uc = u.to(cuda).requires_grad_(True)
+    h = GeluFunction.apply(uc)
+    (du,) = torch.autograd.grad(h, uc, dh.to(cuda))
+    np.testing.assert_allclose(h.detach().double().cpu().numpy(), E.gelu(u.double().numpy()), rtol=0, atol=TOL[dtype] * 10)
+    assert err(h, h_ref) <= TOL[dtype] and err(du, du_ref) <= TOL[dtype]
+    s = AddFunction.apply(uc, dh.to(cuda))
+    assert torch.equal(s.detach().cpu(), u + dh)        # one rounding of the exact sum, in either dtype
+
+
+def _ref_layer(p, x, ei, H, prefix=""):
+    """The layer with torch.nn.functional pieces in float64 (differentiable)."""
+    F, lin = torch.nn.functional, torch.nn.functional.linear
+    b, S, hidden = x.shape
+    g = lambda n: p[prefix + n]
+    y = F.layer_norm(x, (hidden,), g("self_attention_norm.weight"), g("self_attention_norm.bias"))
+    q, k, v = (lin(y, g(f"self_attention.linear_{c}.weight"), g(f"self_attention.linear_{c}.bias")).view(b, S, H, hidden // H)
+               for c in "qkv")
+    o, _ = osa.sparse_attention(q, k, v, ei)
+    x1 = x + lin(o.reshape(b, S, hidden), g("self_attention.output_layer.weight"), g("self_attention.output_layer.bias"))
+    y = F.layer_norm(x1, (hidden,), g("ffn_norm.weight"), g("ffn_norm.bias"))
+    return x1 + lin(F.gelu(lin(y, g("ffn.layer1.weight"), g("ffn.layer1.bias"))), g("ffn.layer2.weight"), g("ffn.layer2.bias"))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_encoder_layer_matches_oracle(cuda, dtype):
+    torch.manual_seed(0)
+    e, n_nodes = workloads.barabasi_albert()
+    ei = torch.as_tensor(e)
+    hidden, H = 64, 8
+    m = EncoderLayer(hidden, 64, 0.0, 0.0, H, 1)
+    with torch.no_grad():
+        # weights large enough for the attention and the FFN to matter, small enough that scores stay inside the
+        # clamp (a score within rounding distance of +-5 flips the clamp mask and with it whole gradient terms)
+        for p in m.parameters():
+            if p.dim() == 2:
+                p.normal_(0, 0.1)
+    x = torch.randn(1, n_nodes, hidden)
+    if dtype == torch.bfloat16:
+        x, m = x.bfloat16(), m.bfloat16()
+    params = {k: v.detach().double().numpy() for k, v in m.state_dict().items()}
+    want = E.encoder_layer_forward(x.double().numpy(), params, e, H)
+    mc = m.to(cuda)
+    xc = x.to(cuda).requires_grad_(True)
+    got = mc(xc, None, ei.to(cuda), "sparse")
+    tol = TOL[dtype] * (3 if dtype == torch.bfloat16 else 1)
+    assert got.shape == (1, n_nodes, hidden) and got.dtype == dtype
+    assert err(got, want) <= tol, err(got, want)
+    # gradients against autograd through the float64 composition
+    pd = {k: torch.tensor(v, requires_grad=True) for k, v in params.items()}
+    xd = x.double().requires_grad_(True)
+    gy = torch.randn(1, n_nodes, hidden, generator=torch.Generator().manual_seed(5)).to(dtype)
+    names = sorted(pd)
+    ref = torch.autograd.grad(_ref_layer(pd, xd, ei, H), [xd] + [pd[n] for n in names], gy.double())
+    got_g = torch.autograd.grad(got, [xc] + [dict(mc.named_parameters())[n] for n in names], gy.to(cuda))
+    ref_by = dict(zip(["x"] + names, ref))
+    for nm, a, r in zip(["x"] + names, got_g, ref):
+        if nm == "self_attention.linear_k.bias":       # cancels to ~0 (see test_gpu_projections): scale by the q-bias gradient
+            ev = (a.detach().double().cpu() - r).abs().max().item() / ref_by["self_attention.linear_q.bias"].abs().max().item()
+            # in bf16 it is the sum of 4 097 rows of dk, each rounded to bf16, whose exact sum cancels:
+            # the rounding noise does not cancel, so this one quantity gets twice the module bar
+            ev = ev / 2 if dtype == torch.bfloat16 else ev
+        else:
+            ev = err(a, r)
+        assert ev <= tol, f"d{nm} err {ev}"
+
+
+def test_graphormer_forward_backward_matches_oracle(cuda):
+    """Graphormer-Slim of the benchmark (4 layers, hidden 64, ffn 64, 8 heads; 128-d input, 40 classes) on a
+    2 000-node batch with the global node: log-probabilities against the oracle, input gradient against autograd
+    through the float64 composition."""
+    torch.manual_seed(1)
+    rng = np.random.default_rng(3)
+    S = 2000
+    e, _ = workloads.power_law_graph(n=S, directed_edges=20000)        # already holds the global node 0: S + 1 nodes
+    m = Graphormer(4, 8, 128, 64, 40, 1, 0.0, 0.0, 0.0, 64, 1)
+    with torch.no_grad():
+        for p in m.parameters():
+            if p.dim() == 2 and p.shape[0] > 1:
+                p.normal_(0, 0.15)
+    x = torch.randn(S, 128)
+    params = {k: v.detach().double().numpy() for k, v in m.state_dict().items()}
+    want = E.graphormer_forward(x.double().numpy(), params, e, 4, 8)
+    mc = m.to(cuda)
+    xc = x.to(cuda).requires_grad_(True)
+    got = mc(xc, None, torch.as_tensor(e).to(cuda), attn_type="sparse")
+    assert got.shape == (S, 40)
+    assert np.abs(got.detach().double().cpu().numpy() - want).max() <= 1e-4, np.abs(got.detach().double().cpu().numpy() - want).max()
+    # loss = nll of random labels, as the training loop computes it (main_sp_node_level.py); gradient of the input
+    y = torch.as_tensor(rng.integers(0, 40, S))
+    (gx,) = torch.autograd.grad(torch.nn.functional.nll_loss(got, y.to(cuda)), xc)
+    pd = {k: torch.tensor(v) for k, v in params.items()}
+    xd = x.double().requires_grad_(True)
+    lin = torch.nn.functional.linear
+    h = torch.cat([pd["graph_token.weight"], lin(xd, pd["node_encoder.weight"], pd["node_encoder.bias"])], 0)[None]
+    for i in range(4):
+        h = _ref_layer(pd, h, torch.as_tensor(e), 8, prefix=f"layers.{i}.")
+    h = torch.nn.functional.layer_norm(h, (64,), pd["final_ln.weight"], pd["final_ln.bias"])
+    out = torch.log_softmax(lin(h[0, 1:, :], pd["downstream_out_proj.weight"], pd["downstream_out_proj.bias"]), 1)
+    (gx_ref,) = torch.autograd.grad(torch.nn.functional.nll_loss(out, y), xd)
+    assert err(gx, gx_ref) <= 1e-4, err(gx, gx_ref)

@@ -67,6 +67,8 @@ def test_linear_shapes(cuda, dtype):
     run_linear("wide", 300, 128, 192, 3, dtype, cuda, 5)               # several contraction chunks and column tiles
     run_linear("odd-tiles", 201, 72, 40, 1, dtype, cuda, 6, bias=False)  # partial chunks both ways, no bias
     run_linear("gt-128", 513, 128, 128, 3, dtype, cuda, 7)
+    if dtype == torch.float32:
+        run_linear("in-100-out-44", 333, 100, 44, 1, dtype, cuda, 8)     # multiples of 4 only (100-d node features)
 
 
 def test_linear_weight_gradient_is_reproducible(cuda):
@@ -90,12 +92,12 @@ def test_linear_empty_input(cuda):
 def test_linear_rejects_bad_arguments(cuda):
     L = _lib.lib()
     arr = (ctypes.c_void_p * 3)()
-    x = torch.zeros(16, 12, device=cuda)
-    W = torch.zeros(8, 12, device=cuda)
+    x = torch.zeros(16, 10, device=cuda)
+    W = torch.zeros(8, 10, device=cuda)
     y = torch.zeros(16, 8, device=cuda)
     arr_w = (ctypes.c_void_p * 3)(W.data_ptr())
     arr_y = (ctypes.c_void_p * 3)(y.data_ptr())
-    assert L.tgt_linear_fwd(x.data_ptr(), arr_w, arr, arr_y, 1, 16, 12, 8, 0, None) == _lib.ERR_UNSUPPORTED   # 12 % 8
+    assert L.tgt_linear_fwd(x.data_ptr(), arr_w, arr, arr_y, 1, 16, 10, 8, 0, None) == _lib.ERR_UNSUPPORTED   # 10 % 4
     assert L.tgt_linear_fwd(x.data_ptr(), arr_w, arr, arr_y, 4, 16, 16, 8, 0, None) == _lib.ERR_INVALID_ARG   # n_out
     assert L.tgt_linear_fwd(x.data_ptr(), arr, arr, arr_y, 1, 16, 16, 8, 0, None) == _lib.ERR_INVALID_ARG     # null weight
     assert L.tgt_linear_bwd(x.data_ptr(), arr_w, arr_y, 1, 16, 16, 8, 0, None, arr_w, None, None, 0, None) == _lib.ERR_WORKSPACE

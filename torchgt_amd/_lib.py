@@ -55,6 +55,11 @@ SIGNATURES = {
     "tgt_linear_fwd": (_i32, [_vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp]),
     "tgt_linear_bwd_workspace_bytes": (_i64, [_i32, _i32, _i32]),
     "tgt_linear_bwd": (_i32, [_vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _i64, _vp]),
+    "tgt_add_layer_norm_fwd": (_i32, [_vp, _vp, _vp, _vp, _i64, _i32, _c.c_float, _i32, _vp, _vp, _vp, _vp, _vp]),
+    "tgt_layer_norm_bwd_workspace_bytes": (_i64, [_i32]),
+    "tgt_layer_norm_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _i64, _vp]),
+    "tgt_gelu_fwd": (_i32, [_vp, _i64, _i32, _vp, _vp]),
+    "tgt_gelu_bwd": (_i32, [_vp, _vp, _i64, _i32, _vp, _vp]),
     "tgt_probe_row_gather": (_i32, [_vp, _i64, _i32, _vp, _i64, _vp, _vp]),
     "tgt_timing_enable": (_i32, [_i32]),
     "tgt_timing_reset": (_i32, []),

@@ -543,8 +543,10 @@ int check_shape(int n_out, int64_t N, int in_features, int out_features, int dty
         set_error("linear: unknown dtype %d", dtype);
         return TGT_ERR_INVALID_ARG;
     }
-    if (in_features % 8 || out_features % 8) {
-        set_error("linear: in_features and out_features must be multiples of 8 (got %d, %d)", in_features, out_features);
+    const int ve = dtype == TGT_DTYPE_F32 ? 4 : 8;      // rows are read in 16-byte pieces
+    if (in_features % ve || out_features % ve) {
+        set_error("linear: in_features and out_features must be multiples of %d for this dtype (got %d, %d)", ve,
+                  in_features, out_features);
         return TGT_ERR_UNSUPPORTED;
     }
     if (N > (int64_t)INT32_MAX * kGradRows) {

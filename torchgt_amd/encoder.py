@@ -1,0 +1,216 @@
+"""The encoder layer and the node-level Graphormer around ``MultiHeadAttention``.
+
+Mirrors of ``FeedForwardNetwork``, ``EncoderLayer`` and ``Graphormer`` of
+models/graphormer_dist_node_level.py (:27-39, :276-314, :316-392): same
+constructors, same parameter names (a reference ``state_dict`` loads; the
+parameter counts 111 913 / 110 576 of README.md:70,114 are reproduced), same
+``forward`` signatures.  Every residual add is folded into the LayerNorm that
+follows it (``tgt_add_layer_norm_fwd``), GELU and all linears run on the
+library's kernels; torch only keeps the autograd graph.
+
+Dropout: the fused path covers rate 0 and eval mode (what the attention
+supports); with a positive rate in training mode torch's dropout is applied at
+the reference's places, with torch's random stream.
+"""
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import _lib
+from .multi_head_attention import MultiHeadAttention, fused_linear, _DT
+
+
+def _stream(t):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+class AddLayerNormFunction(torch.autograd.Function):
+    """``s = x + r`` (r may be None) and ``y = LayerNorm(s)`` in one pass; returns (s, y)."""
+
+    @staticmethod
+    def forward(ctx, x, r, gamma, beta, eps):
+        if not x.is_cuda:
+            raise RuntimeError("torchgt_amd encoder kernels run on the GPU only (no CPU fallback)")
+        if x.dtype not in _DT:
+            raise TypeError(f"unsupported dtype {x.dtype}")
+        C = x.shape[-1]
+        x2 = x.reshape(-1, C).contiguous()
+        r2 = None if r is None else r.reshape(-1, C).contiguous()
+        N = x2.shape[0]
+        s = x2 if r2 is None else torch.empty_like(x2)
+        y = torch.empty_like(x2)
+        mean = torch.empty(N, dtype=torch.float32, device=x.device)
+        rstd = torch.empty(N, dtype=torch.float32, device=x.device)
+        g, b = gamma.contiguous(), beta.contiguous()
+        with torch.cuda.device(x.device):
+            _lib.check(_lib.lib().tgt_add_layer_norm_fwd(
+                x2.data_ptr(), None if r2 is None else r2.data_ptr(), g.data_ptr(), b.data_ptr(), N, C, float(eps),
+                _DT[x.dtype], None if r2 is None else s.data_ptr(), y.data_ptr(), mean.data_ptr(), rstd.data_ptr(),
+                _stream(x)))
+        ctx.save_for_backward(s, g, mean, rstd)
+        ctx.has_r = r is not None
+        ctx.shape = x.shape
+        return s.view(x.shape), y.view(x.shape)
+
+    @staticmethod
+    def backward(ctx, ds_out, dy):
+        s, g, mean, rstd = ctx.saved_tensors
+        N, C = s.shape
+        L = _lib.lib()
+        if dy is None:
+            dy = torch.zeros_like(s)
+        dy2 = dy.reshape(N, C).contiguous()
+        extra = None if ds_out is None else ds_out.reshape(N, C).contiguous()
+        ds = torch.empty_like(s)
+        dg, db = torch.empty_like(g), torch.empty_like(g)
+        nbytes = L.tgt_layer_norm_bwd_workspace_bytes(C)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=s.device)
+        with torch.cuda.device(s.device):
+            _lib.check(L.tgt_layer_norm_bwd(s.data_ptr(), g.data_ptr(), mean.data_ptr(), rstd.data_ptr(), dy2.data_ptr(),
+                                            None if extra is None else extra.data_ptr(), N, C, _DT[s.dtype],
+                                            ds.data_ptr(), dg.data_ptr(), db.data_ptr(), ws.data_ptr(), nbytes, _stream(s)))
+        ds = ds.view(ctx.shape)
+        return ds, (ds if ctx.has_r else None), dg, db, None
+
+
+class AddFunction(torch.autograd.Function):
+    """``x + r`` through the same kernel (no normalisation)."""
+
+    @staticmethod
+    def forward(ctx, x, r):
+        C = x.shape[-1]
+        x2, r2 = x.reshape(-1, C).contiguous(), r.reshape(-1, C).contiguous()
+        s = torch.empty_like(x2)
+        with torch.cuda.device(x.device):
+            _lib.check(_lib.lib().tgt_add_layer_norm_fwd(x2.data_ptr(), r2.data_ptr(), None, None, x2.shape[0], C, 0.0,
+                                                         _DT[x.dtype], s.data_ptr(), None, None, None, _stream(x)))
+        return s.view(x.shape)
+
+    @staticmethod
+    def backward(ctx, ds):
+        return ds, ds
+
+
+class GeluFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, u):
+        if not u.is_cuda:
+            raise RuntimeError("torchgt_amd encoder kernels run on the GPU only (no CPU fallback)")
+        u2 = u.contiguous()
+        h = torch.empty_like(u2)
+        with torch.cuda.device(u.device):
+            _lib.check(_lib.lib().tgt_gelu_fwd(u2.data_ptr(), u2.numel(), _DT[u.dtype], h.data_ptr(), _stream(u)))
+        ctx.save_for_backward(u2)
+        return h
+
+    @staticmethod
+    def backward(ctx, dh):
+        (u,) = ctx.saved_tensors
+        dh2 = dh.contiguous()
+        du = torch.empty_like(u)
+        with torch.cuda.device(u.device):
+            _lib.check(_lib.lib().tgt_gelu_bwd(u.data_ptr(), dh2.data_ptr(), u.numel(), _DT[u.dtype], du.data_ptr(), _stream(u)))
+        return du
+
+
+def init_params(module, n_layers):
+    """models/graphormer_dist_node_level.py:18-24."""
+    if isinstance(module, nn.Linear):
+        module.weight.data.normal_(mean=0.0, std=0.02 / math.sqrt(n_layers))
+        if module.bias is not None:
+            module.bias.data.zero_()
+    if isinstance(module, nn.Embedding):
+        module.weight.data.normal_(mean=0.0, std=0.02)
+
+
+class FeedForwardNetwork(nn.Module):
+    def __init__(self, hidden_size, ffn_size, dropout_rate):
+        super().__init__()
+        self.layer1 = nn.Linear(hidden_size, ffn_size)
+        self.gelu = nn.GELU()            # kept for the reference's module tree; the library kernel computes it
+        self.layer2 = nn.Linear(ffn_size, hidden_size)
+
+    def forward(self, x):
+        (u,) = fused_linear(x, self.layer1)
+        h = GeluFunction.apply(u)
+        (y,) = fused_linear(h, self.layer2)
+        return y
+
+
+class EncoderLayer(nn.Module):
+    def __init__(self, hidden_size, ffn_size, dropout_rate, attention_dropout_rate, num_heads, attn_bias_dim):
+        super().__init__()
+        self.self_attention_norm = nn.LayerNorm(hidden_size)
+        self.self_attention = MultiHeadAttention(hidden_size, attention_dropout_rate, num_heads, attn_bias_dim)
+        self.self_attention_dropout = nn.Dropout(dropout_rate)
+        self.ffn_norm = nn.LayerNorm(hidden_size)
+        self.ffn = FeedForwardNetwork(hidden_size, ffn_size, dropout_rate)
+        self.ffn_dropout = nn.Dropout(dropout_rate)
+
+    def forward(self, x, attn_bias=None, edge_index=None, attn_type=None, residual=None, defer_residual=False):
+        """``residual``: a tensor still to be added to x (the previous layer's FFN output when it was
+        called with ``defer_residual=True``); the add rides on this layer's first LayerNorm.
+        ``defer_residual=True`` returns (x, ffn_output) instead of their sum."""
+        n1, n2 = self.self_attention_norm, self.ffn_norm
+        x, y = AddLayerNormFunction.apply(x, residual, n1.weight, n1.bias, n1.eps)
+        y = self.self_attention(y, attn_bias, edge_index, attn_type=attn_type)
+        y = self.self_attention_dropout(y)
+        x, y = AddLayerNormFunction.apply(x, y, n2.weight, n2.bias, n2.eps)
+        y = self.ffn(y)
+        y = self.ffn_dropout(y)
+        if defer_residual:
+            return x, y
+        return AddFunction.apply(x, y)
+
+
+class Graphormer(nn.Module):
+    """Graphormer for node-level tasks, global token at index 0
+    (models/graphormer_dist_node_level.py:316-392)."""
+
+    def __init__(self, n_layers, num_heads, input_dim, hidden_dim, output_dim, attn_bias_dim, dropout_rate,
+                 input_dropout_rate, attention_dropout_rate, ffn_dim, num_global_node):
+        super().__init__()
+        self.num_heads = num_heads
+        self.node_encoder = nn.Linear(input_dim, hidden_dim)
+        self.input_dropout = nn.Dropout(input_dropout_rate)
+        self.layers = nn.ModuleList([EncoderLayer(hidden_dim, ffn_dim, dropout_rate, attention_dropout_rate, num_heads,
+                                                  attn_bias_dim) for _ in range(n_layers)])
+        self.n_layers = n_layers
+        self.final_ln = nn.LayerNorm(hidden_dim)
+        self.downstream_out_proj = nn.Linear(hidden_dim, output_dim)
+        self.hidden_dim = hidden_dim
+        self.num_global_node = num_global_node
+        self.graph_token = nn.Embedding(self.num_global_node, hidden_dim)
+        self.graph_token_virtual_distance = nn.Embedding(self.num_global_node, attn_bias_dim)
+        self.apply(lambda module: init_params(module, n_layers=n_layers))
+
+    def forward(self, x, attn_bias, edge_index, perturb=None, attn_type=None):
+        x = x.unsqueeze(0)
+        n_graph = x.shape[0]
+        (node_feature,) = fused_linear(x, self.node_encoder)
+        if perturb is not None:
+            node_feature = node_feature + perturb
+        global_node_feature = self.graph_token.weight.unsqueeze(0).repeat(n_graph, 1, 1)
+        node_feature = torch.cat([global_node_feature, node_feature], dim=1)
+        output = self.input_dropout(node_feature)
+        if attn_bias is not None:
+            # the dense bias of the reference (:363-376); only practical for short sequences
+            attn_bias = attn_bias.unsqueeze(0)
+            n_graph, subseq_len, seq_len = attn_bias.size()[:3]
+            vd = self.graph_token_virtual_distance.weight
+            graph_attn_bias = torch.cat([vd.unsqueeze(0).unsqueeze(2).repeat(n_graph, 1, seq_len, 1), attn_bias.clone()], dim=1)
+            graph_attn_bias = torch.cat([vd.unsqueeze(0).unsqueeze(0).repeat(n_graph, subseq_len + self.num_global_node, 1, 1),
+                                         graph_attn_bias], dim=2)
+            graph_attn_bias = graph_attn_bias.repeat(1, 1, 1, self.num_heads)
+        else:
+            graph_attn_bias = None
+        pending = None
+        for enc_layer in self.layers:
+            output, pending = enc_layer(output, attn_bias=graph_attn_bias, edge_index=edge_index, attn_type=attn_type,
+                                        residual=pending, defer_residual=True)
+        fl = self.final_ln
+        _, output = AddLayerNormFunction.apply(output, pending, fl.weight, fl.bias, fl.eps)
+        (output,) = fused_linear(output[0, 1:, :], self.downstream_out_proj)
+        return F.log_softmax(output, dim=1)
