@@ -8,11 +8,12 @@ the benchmark configuration "configs[1]": N = 64 001, E ~ 530 K, H = 8, d = 8, p
 reported separately).  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype f32|bf16] [--no-cpu-baseline]
-                    [--workload config1|config2|config2-mha|config3|config4|config5|config5-blockized]
+                    [--workload config1|config2|config2-mha|config2-model|config3|config4|config5|config5-blockized]
 
 config3 / config5: larger sparse workloads (bf16); config4: dense biased attention of a graph-level
 batch; config5-blockized: the block path on the reordered config5 graph; config2-mha: one whole
-MultiHeadAttention layer (projections + sparse attention) on the config2 graph.
+MultiHeadAttention layer (projections + sparse attention) on the config2 graph; config2-model: a training
+step of the 4-layer Graphormer-Slim on that graph.
 """
 import argparse
 import json
@@ -405,6 +406,67 @@ def bench_mha(args):
     print(json.dumps(result))
 
 
+def bench_model(args):
+    """One training step of the Graphormer-Slim of configs[1] (4 layers, hidden 64, ffn 64, 8 heads, 128-d input,
+    40 classes; 111 913 parameters) on the whole 64 K-node graph as one sequence: forward, nll loss, backward,
+    AdamW step (torch's optimizer, as in the reference's training loop)."""
+    import torch
+    from torchgt_amd import Graphormer, _lib
+    dev = torch.device("cuda:0")
+    e, n, label, desc = build_workload("config2")
+    tdt = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    torch.manual_seed(42)
+    m = Graphormer(4, 8, 128, 64, 40, 1, 0.0, 0.0, 0.0, 64, 1).to(dev, tdt)
+    opt = torch.optim.AdamW(m.parameters(), lr=1e-3, weight_decay=0.01)
+    ei = torch.from_numpy(e).to(dev)
+    x = torch.randn(n - 1, 128, device=dev).to(tdt)
+    y = torch.randint(0, 40, (n - 1,), device=dev)
+
+    def step():
+        opt.zero_grad(set_to_none=True)
+        out = m(x, None, ei, attn_type="sparse")
+        loss = torch.nn.functional.nll_loss(out.float(), y)
+        loss.backward()
+        opt.step()
+        return loss
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss = step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    L = _lib.lib()
+    L.tgt_timing_reset()
+    L.tgt_timing_enable(1)
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    L.tgt_timing_enable(0)
+    kernels = {k: {"avg_us": t / c * 1e3, "launches_per_step": c / args.steps} for k, (t, c) in _lib.kernel_timings().items() if c}
+    lib_us = sum(v["avg_us"] * v["launches_per_step"] for v in kernels.values())
+    groups = {"attention": ("attn_fwd", "bwd_node_side", "attn_bwd"), "projections and ffn linears": ("linear_fwd", "linear_dx", "linear_dw"),
+              "layer norm + residual": ("layer_norm_fwd", "layer_norm_bwd"), "gelu": ("gelu",)}
+    result = {
+        "metric": "training step of the 4-layer Graphormer-Slim on one 64 K-node sequence",
+        "value": 1e3 / ms, "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic",
+        "config": {"workload": "configs[1] graph as one sequence, Graphormer-Slim 4 x (hidden 64, ffn 64, 8 heads), "
+                               "128-d features, 40 classes, no bias, dropout 0", "N": n, "E": int(e.shape[1]),
+                   "parameters": sum(p.numel() for p in m.parameters()),
+                   "step": "forward + nll_loss + backward + torch AdamW", "parallelism": "1 GPU"},
+        "loss": float(loss.detach()),
+        "library_kernel_us_per_step": lib_us,
+        "kernel_groups_us": {g: sum(kernels[k]["avg_us"] * kernels[k]["launches_per_step"] for k in ks if k in kernels)
+                             for g, ks in groups.items()},
+        "kernels": kernels,
+    }
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -439,6 +501,8 @@ def main():
         return bench_block(args)
     if args.workload == "config2-mha":
         return bench_mha(args)
+    if args.workload == "config2-model":
+        return bench_model(args)
     if args.workload in ("config3", "config5"):
         args.no_cpu_baseline = True      # the CPU restatement needs minutes per step at this size
     e, n, label, desc = build_workload(args.workload)

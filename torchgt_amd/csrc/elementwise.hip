@@ -166,27 +166,39 @@ __global__ __launch_bounds__(kEwBlock) void k_layer_norm_bwd(const T* __restrict
     }
 }
 
-// out[e] = sum over workers of partial[w][e], in worker order; e < n
+// out[e] = sum over workers of partial[w][e], e < n: 64 consecutive elements x 16
+// slices of the workers per workgroup; the slices are added in order, so the sum
+// does not depend on the launch.
 template <typename T>
-__global__ __launch_bounds__(256) void k_reduce_workers(const float* __restrict__ partial, int workers, int n,
-                                                        T* __restrict__ out_a, T* __restrict__ out_b, int split) {
-    const int e = blockIdx.x * 256 + threadIdx.x;
-    if (e >= n) return;
+__global__ __launch_bounds__(1024) void k_reduce_workers(const float* __restrict__ partial, int workers, int n,
+                                                         T* __restrict__ out_a, T* __restrict__ out_b, int split) {
+    __shared__ float part[16][64];
+    const int el = threadIdx.x & 63, sl = threadIdx.x >> 6;
+    const int e = blockIdx.x * 64 + el;
+    const int w0 = (int)((int64_t)workers * sl / 16), w1 = (int)((int64_t)workers * (sl + 1) / 16);
     float t = 0.f;
-    int w = 0;
-    for (; w + 8 <= workers; w += 8) {
-        float v[8];
+    if (e < n) {
+        const float* __restrict__ src = partial + e;
+        int w = w0;
+        for (; w + 8 <= w1; w += 8) {
+            float v[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = partial[(int64_t)(w + i) * n + e];
+            for (int i = 0; i < 8; ++i) v[i] = src[(int64_t)(w + i) * n];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) t += v[i];
+            for (int i = 0; i < 8; ++i) t += v[i];
+        }
+        for (; w < w1; ++w) t += src[(int64_t)w * n];
     }
-    for (; w < workers; ++w) t += partial[(int64_t)w * n + e];
-    T* dst = e < split ? out_a + e : out_b + (e - split);
-    if (dst) {
-        if constexpr (sizeof(T) == 4) *reinterpret_cast<float*>(dst) = t;
+    part[sl][el] = t;
+    __syncthreads();
+    if (sl == 0 && e < n) {
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sum += part[i][el];
+        T* dst = e < split ? out_a + e : out_b + (e - split);
+        if constexpr (sizeof(T) == 4) *reinterpret_cast<float*>(dst) = sum;
         else {
-            const __bf16 b = static_cast<__bf16>(t);
+            const __bf16 b = static_cast<__bf16>(sum);
             reinterpret_cast<ebf16*>(dst)->x = __builtin_bit_cast(uint16_t, b);
         }
     }
@@ -312,12 +324,12 @@ int tgt_layer_norm_bwd(const void* d_s, const void* d_gamma, const float* d_mean
     KernelTimer t(KS_LAYER_NORM_BWD, st);
     if (dtype == TGT_DTYPE_F32) launch_ln_bwd<float>(lpr, workers, d_s, d_gamma, d_mean, d_rstd, d_dy, d_ds_extra, N, d_ds, partial, st);
     else launch_ln_bwd<ebf16>(lpr, workers, d_s, d_gamma, d_mean, d_rstd, d_dy, d_ds_extra, N, d_ds, partial, st);
-    const unsigned rgrid = (unsigned)((2 * C + 255) / 256);
+    const unsigned rgrid = (unsigned)((2 * C + 63) / 64);
     if (dtype == TGT_DTYPE_F32)
-        hipLaunchKernelGGL((k_reduce_workers<float>), dim3(rgrid), dim3(256), 0, st, partial, workers, 2 * C,
+        hipLaunchKernelGGL((k_reduce_workers<float>), dim3(rgrid), dim3(1024), 0, st, partial, workers, 2 * C,
                            (float*)d_dgamma, (float*)d_dbeta, C);
     else
-        hipLaunchKernelGGL((k_reduce_workers<ebf16>), dim3(rgrid), dim3(256), 0, st, partial, workers, 2 * C,
+        hipLaunchKernelGGL((k_reduce_workers<ebf16>), dim3(rgrid), dim3(1024), 0, st, partial, workers, 2 * C,
                            (ebf16*)d_dgamma, (ebf16*)d_dbeta, C);
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
