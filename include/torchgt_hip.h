@@ -275,6 +275,41 @@ int tgt_layer_norm_bwd(const void* d_s, const void* d_gamma, const float* d_mean
 int tgt_gelu_fwd(const void* d_u, int64_t n, int dtype, void* d_h, void* stream);
 int tgt_gelu_bwd(const void* d_u, const void* d_dh, int64_t n, int dtype, void* d_du, void* stream);
 
+/* ---- graph-level attention bias ---------------------------------------------
+ * GraphAttnBias.forward (models/graphormer_graph_level.py:94-156), edge_type other than
+ * 'multi_hop' (:148-150).  With S1 = s + 1 (virtual node first):
+ *   out[g,h,i,j] = 2 * attn_bias[g,i,j]                                   (:104 and :153)
+ *                + spatial_table[spatial_pos[g,i-1,j-1]][h]               (i, j >= 1; :110-111)
+ *                + mean_f edge_table[edge_type[g,i-1,j-1,f]][h]           (i, j >= 1; :150-152)
+ *                + virtual_dist[h]                                         (i == 0 or j == 0; :115-117)
+ * d_attn_bias: [b, S1, S1]; d_spatial_pos: int64 [b, s, s]; d_edge_type: int64
+ * [b, s, s, F]; tables [num_spatial, H], [num_edges, H], [H]; d_out: [b, H, S1, S1];
+ * float tensors of `dtype`.  Ids outside a table are clamped to its range (the
+ * reference's embedding lookup would raise). */
+int tgt_graph_attn_bias_fwd(const void* d_attn_bias, const int64_t* d_spatial_pos, const int64_t* d_edge_type, int F,
+                            const void* d_spatial_table, int num_spatial, const void* d_edge_table, int num_edges,
+                            const void* d_virtual_dist, int b, int s, int H, int dtype, void* d_out, void* stream);
+/* Gradients of the three tables for the upstream gradient d_dout [b, H, S1, S1]
+ * (autograd of the embedding lookups in the reference; row 0 of the spatial and edge
+ * tables is the padding index and gets zero).  Sums are formed in LDS per workgroup
+ * with floating-point atomics and the workgroup partials are added in a fixed order:
+ * results agree to rounding between runs, not bit for bit.
+ * (num_spatial + num_edges + 1) * H must not exceed 15 360. */
+int64_t tgt_graph_attn_bias_bwd_workspace_bytes(int num_spatial, int num_edges, int H);
+int tgt_graph_attn_bias_bwd(const void* d_dout, const int64_t* d_spatial_pos, const int64_t* d_edge_type, int F,
+                            int num_spatial, int num_edges, int b, int s, int H, int dtype, void* d_dspatial_table,
+                            void* d_dedge_table, void* d_dvirtual_dist, void* d_workspace, int64_t workspace_bytes,
+                            void* stream);
+/* floyd_warshall (data/algos.pyx:9-54) for a batch of graphs of at most 128 nodes.
+ * d_adj: uint8 [num_graphs, n_max, n_max], entry = edge weight, 0 = no edge;
+ * d_n_nodes: int32 [num_graphs] node counts (NULL: all n_max).  d_dist, d_path:
+ * int32 [num_graphs, n_max, n_max]; entries with i or j >= n_nodes[g] are left
+ * untouched.  dist = shortest distance (0 on the diagonal, 510 if unreachable),
+ * path = the intermediate node recorded by the last strict improvement (-1 for
+ * direct edges, 510 if unreachable): both exactly what the reference's loop yields. */
+int tgt_floyd_warshall(const uint8_t* d_adj, const int32_t* d_n_nodes, int num_graphs, int n_max, int32_t* d_dist,
+                       int32_t* d_path, void* stream);
+
 /* ---- per-kernel timing --------------------------------------------------
  * The reference times this path with torch.profiler around whole iterations
  * (attn_module.py:415-438).  When enabled, every kernel the library launches is

@@ -173,3 +173,34 @@ def build_csr(edge_index, num_nodes, by="dst"):
     np.add.at(rowptr, key + 1, 1)
     rowptr = np.cumsum(rowptr)
     return rowptr.astype(np.int32), other[eid].astype(np.int32), eid.astype(np.int32)
+
+
+FW_UNREACHABLE = 510      # data/algos.pyx:30
+
+
+def floyd_warshall(adjacency_matrix):
+    """data/algos.pyx:9-54, loop for loop (use on small graphs).  Returns (M, path) int64 [n, n]:
+    M = shortest distances (0 on the diagonal, 510 = unreachable), path[i][j] = the intermediate
+    node k of the last strict improvement of M[i][j] (-1 if none, 510 if unreachable)."""
+    M = np.array(adjacency_matrix, dtype=np.int64)
+    n = M.shape[0]
+    assert M.shape == (n, n)
+    path = -np.ones((n, n), dtype=np.int64)
+    for i in range(n):                                  # :27-32
+        for j in range(n):
+            if i == j:
+                M[i, j] = 0
+            elif M[i, j] == 0:
+                M[i, j] = FW_UNREACHABLE
+    for k in range(n):                                  # :35-45
+        for i in range(n):
+            M_ik = M[i, k]
+            for j in range(n):
+                cost = M_ik + M[k, j]
+                if M[i, j] > cost:
+                    M[i, j] = cost
+                    path[i, j] = k
+    far = M >= FW_UNREACHABLE                           # :48-52
+    path[far] = FW_UNREACHABLE
+    M[far] = FW_UNREACHABLE
+    return M, path

@@ -1,0 +1,120 @@
+"""GPU parity of GraphAttnBias (forward and table gradients) and of the Floyd-Warshall
+kernel with the oracle.  Floyd-Warshall is integer work: bit-exact.  The bias is a sum of
+table entries: float32 1e-5 / bf16 2e-2 on max|a-b| / max|b| (finite entries; -inf stays -inf).
+"""
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import dense_attention as oda
+from oracle import graph_prep as ogp
+from torchgt_amd import GraphAttnBias, _lib, floyd_warshall, workloads
+
+pytestmark = pytest.mark.gpu
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2}
+
+
+def err(a, b):
+    a, b = a.detach().double().cpu(), b.detach().double().cpu()
+    fin = torch.isfinite(b)
+    assert torch.equal(torch.isfinite(a), fin)
+    assert torch.equal(a[~fin], b[~fin])
+    denom = b[fin].abs().max().item()
+    return (a[fin] - b[fin]).abs().max().item() / (denom if denom > 0 else 1.0)
+
+
+def test_floyd_warshall_matches_oracle_bit_for_bit(cuda):
+    rng = np.random.default_rng(0)
+    # single graphs, the reference's call shape
+    for n, p in ((1, 0.0), (5, 0.5), (23, 0.12), (64, 0.05), (128, 0.03)):
+        print(f"floyd_warshall case: n={n} p={p}", flush=True)
+        a = (rng.random((n, n)) < p).astype(np.int64)
+        a = np.maximum(a, a.T)
+        M, path = floyd_warshall(a)
+        M_ref, path_ref = ogp.floyd_warshall(a)
+        assert M.dtype == np.int64 and path.dtype == np.int64
+        np.testing.assert_array_equal(M, M_ref)
+        np.testing.assert_array_equal(path, path_ref)
+    # directed, weighted, with self-loops in the input (the diagonal is reset to 0)
+    a = rng.integers(0, 4, size=(17, 17)) * (rng.random((17, 17)) < 0.2)
+    M, path = floyd_warshall(a)
+    M_ref, path_ref = ogp.floyd_warshall(a)
+    np.testing.assert_array_equal(M, M_ref)
+    np.testing.assert_array_equal(path, path_ref)
+    # a padded batch of graphs of different sizes: the configuration-4 generator
+    data = workloads.erdos_renyi_batch(batch=12, seed=3)
+    sizes = data["n_nodes"]
+    n_max = int(sizes.max())
+    adj = np.zeros((12, n_max, n_max), dtype=np.uint8)
+    for g in range(12):
+        n = int(sizes[g])
+        sp = data["spatial_pos"][g][:n, :n]
+        adj[g, :n, :n] = (sp == 2)                # spatial_pos = distance + 1: direct neighbours
+    dist, path = floyd_warshall(torch.from_numpy(adj), sizes)
+    for g in range(12):
+        n = int(sizes[g])
+        M_ref, path_ref = ogp.floyd_warshall(adj[g, :n, :n])
+        np.testing.assert_array_equal(dist[g, :n, :n].cpu().numpy(), M_ref)
+        np.testing.assert_array_equal(path[g, :n, :n].cpu().numpy(), path_ref)
+        assert not dist[g, n:, :].any() and not dist[g, :, n:].any()
+
+
+def test_floyd_warshall_rejects_large_graphs(cuda):
+    with pytest.raises(_lib.TorchGTHipError) as ei:
+        floyd_warshall(np.zeros((129, 129), dtype=np.int64))
+    assert ei.value.code == _lib.ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_graph_attn_bias_matches_oracle(cuda, dtype):
+    data = workloads.erdos_renyi_batch(batch=16, seed=42)
+    H, F = 8, 3
+    g = torch.Generator().manual_seed(1)
+    m = GraphAttnBias(H, 512, 5, 22, 128, 64, "single_hop", 5)
+    with torch.no_grad():
+        m.spatial_pos_encoder.weight.normal_(0, 0.5, generator=g); m.spatial_pos_encoder.weight[0] = 0
+        m.edge_encoder.weight.normal_(0, 0.5, generator=g); m.edge_encoder.weight[0] = 0
+        m.graph_token_virtual_distance.weight.normal_(0, 0.5, generator=g)
+    assert sorted(n for n, _ in m.named_parameters()) == ["edge_encoder.weight", "graph_token_virtual_distance.weight",
+                                                          "spatial_pos_encoder.weight"]
+    m = m.to(dtype)
+    attn_bias = torch.from_numpy(data["attn_bias"])                       # 0 / -inf, [b, S1, S1]
+    spatial_pos = torch.from_numpy(data["spatial_pos"]).long()
+    et1 = torch.from_numpy(data["edge_type"]).long()
+    edge_type = torch.stack([et1, (et1 * 2) % 5, torch.zeros_like(et1)], -1)       # F = 3 edge features per pair
+    st, et, vd = (p.detach().double() for p in (m.spatial_pos_encoder.weight, m.edge_encoder.weight, m.graph_token_virtual_distance.weight))
+    st.requires_grad_(True); et.requires_grad_(True); vd.requires_grad_(True)
+    want = oda.graph_attn_bias(attn_bias.double(), spatial_pos, edge_type, st, et, vd)
+    mc = m.to(cuda)
+    batch = types.SimpleNamespace(attn_bias=attn_bias.to(cuda), spatial_pos=spatial_pos.to(cuda), attn_edge_type=edge_type.to(cuda),
+                                  edge_input=None)
+    got = mc(batch)
+    assert got.shape == want.shape and got.dtype == dtype
+    assert err(got, want) <= TOL[dtype], err(got, want)
+    # table gradients; the upstream gradient is zero on the masked (-inf) entries, as the attention's is
+    dout = torch.randn(want.shape, generator=g)
+    dout[~torch.isfinite(want)] = 0
+    dout = dout.to(dtype)
+    finite = torch.where(torch.isfinite(want), want, torch.zeros_like(want))
+    ref = [r.clone() for r in torch.autograd.grad((finite * dout.double()).sum(), [st, et, vd])]
+    # the oracle indexes plain tensors; the module's tables are nn.Embedding(padding_idx=0), whose row 0 gets no
+    # gradient (checked here on torch's own embedding), although padded query rows do look it up
+    w = torch.ones(3, 2, requires_grad=True)
+    torch.nn.functional.embedding(torch.tensor([0, 0, 1]), w, padding_idx=0).sum().backward()
+    assert w.grad[0].abs().sum() == 0 and w.grad[1].sum() == 2
+    assert ref[0][0].abs().max() > 0          # the case is exercised
+    ref[0][0] = 0
+    ref[1][0] = 0
+    got_g = torch.autograd.grad(got, [mc.spatial_pos_encoder.weight, mc.edge_encoder.weight, mc.graph_token_virtual_distance.weight],
+                                dout.to(cuda))
+    for nm, a, r in zip(("spatial", "edge", "virtual"), got_g, ref):
+        assert err(a, r) <= TOL[dtype], f"d{nm} err {err(a, r)}"
+    assert not got_g[0][0].any() and not got_g[1][0].any()              # padding index rows get no gradient
+
+
+def test_graph_attn_bias_multi_hop_is_not_built(cuda):
+    m = GraphAttnBias(8, 512, 5, 22, 128, 64, "multi_hop", 5)
+    with pytest.raises(NotImplementedError):
+        m(types.SimpleNamespace())

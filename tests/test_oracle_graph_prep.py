@@ -163,3 +163,34 @@ def test_gen_sub_edge_index_empty_batch_and_no_edges():
     e = np.zeros((2, 0), dtype=np.int64)
     np.testing.assert_array_equal(gp.gen_sub_edge_index(e, [2, 1], 4), np.array([[1, 0], [1, 0]]))
     assert gp.gen_sub_edge_index(np.array([[0, 1], [1, 0]]), [], 3).shape == (2, 0)
+
+
+def test_floyd_warshall_known_answer_and_scipy():
+    # path graph 0-1-2-3 plus an isolated node 4
+    adj = np.zeros((5, 5), dtype=np.int64)
+    for a, b in ((0, 1), (1, 2), (2, 3)):
+        adj[a, b] = adj[b, a] = 1
+    M, path = gp.floyd_warshall(adj)
+    want = np.array([[0, 1, 2, 3, 510], [1, 0, 1, 2, 510], [2, 1, 0, 1, 510], [3, 2, 1, 0, 510], [510] * 4 + [0]])
+    np.testing.assert_array_equal(M, want)
+    assert path[0, 1] == -1 and path[0, 2] == 1 and path[0, 4] == 510 and path[4, 4] == -1
+    assert path[0, 3] == 2        # the improvement through k = 2 comes last (k = 1 gave 0-1-..-3 only after 1-3 was known)
+    # distances against scipy's shortest paths on random graphs
+    from scipy.sparse.csgraph import shortest_path
+    rng = np.random.default_rng(0)
+    for n in (7, 20):
+        a = (rng.random((n, n)) < 0.15).astype(np.int64)
+        a = np.maximum(a, a.T)
+        np.fill_diagonal(a, 0)
+        M, path = gp.floyd_warshall(a)
+        d = shortest_path(a, method="D", unweighted=True)
+        d[np.isinf(d)] = 510
+        np.testing.assert_array_equal(M, d.astype(np.int64))
+        # every recorded intermediate node splits the distance exactly
+        for i in range(n):
+            for j in range(n):
+                k = path[i, j]
+                if 0 <= k < 510:
+                    assert M[i, j] == M[i, k] + M[k, j]
+                elif k == -1:
+                    assert i == j or a[i, j] == 1
