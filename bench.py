@@ -447,6 +447,43 @@ def bench_model(args):
     L.tgt_timing_enable(0)
     kernels = {k: {"avg_us": t / c * 1e3, "launches_per_step": c / args.steps} for k, (t, c) in _lib.kernel_timings().items() if c}
     lib_us = sum(v["avg_us"] * v["launches_per_step"] for v in kernels.values())
+    loss_value = float(loss.detach())
+    # The same step captured once into a HIP graph (the library calls only launch kernels) and replayed.  A fresh
+    # model and optimizer are used, warmed up on a side stream: autograd nodes that earlier eager steps created on
+    # the default stream (kept alive by their loss tensor) must not take part in a capture.
+    graph_ms = None
+    if args.hip_graph:
+        del loss
+        torch.manual_seed(42)
+        gm = Graphormer(4, 8, 128, 64, 40, 1, 0.0, 0.0, 0.0, 64, 1).to(dev, tdt)
+        gopt = torch.optim.AdamW(gm.parameters(), lr=1e-3, weight_decay=0.01, capturable=True)
+
+        def gstep():
+            gloss = torch.nn.functional.nll_loss(gm(x, None, ei, attn_type="sparse").float(), y)
+            gloss.backward()
+            gopt.step()
+            return gloss
+
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                gopt.zero_grad(set_to_none=True)
+                gstep()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        gr = torch.cuda.CUDAGraph()
+        gopt.zero_grad(set_to_none=True)
+        with torch.cuda.graph(gr):
+            gstep()
+        for _ in range(args.warmup):
+            gr.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            gr.replay()
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - t0) / args.steps * 1e3
     groups = {"attention": ("attn_fwd", "bwd_node_side", "attn_bwd"), "projections and ffn linears": ("linear_fwd", "linear_dx", "linear_dw"),
               "layer norm + residual": ("layer_norm_fwd", "layer_norm_bwd"), "gelu": ("gelu",)}
     result = {
@@ -458,7 +495,8 @@ def bench_model(args):
                                "128-d features, 40 classes, no bias, dropout 0", "N": n, "E": int(e.shape[1]),
                    "parameters": sum(p.numel() for p in m.parameters()),
                    "step": "forward + nll_loss + backward + torch AdamW", "parallelism": "1 GPU"},
-        "loss": float(loss.detach()),
+        "loss": loss_value,
+        "ms_per_step_hip_graph": graph_ms,
         "library_kernel_us_per_step": lib_us,
         "kernel_groups_us": {g: sum(kernels[k]["avg_us"] * kernels[k]["launches_per_step"] for k in ks if k in kernels)
                              for g, ks in groups.items()},
@@ -475,6 +513,8 @@ def main():
     ap.add_argument("--dtype", default="f32", choices=["f32", "bf16"])
     ap.add_argument("--workload", default="config2")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--hip-graph", action="store_true",
+                    help="config2-model: also time the step captured into a HIP graph and replayed")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device copy (a kernel of known traffic, for scaling rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings)")

@@ -58,3 +58,56 @@ def test_sparse_step_replays_from_a_graph(cuda, dtype):
         for a, b in zip(got, (out, Z, dq, dk, dv, db)):
             assert torch.equal(a, b), f"replay {replay} differs from the eager step"
     plan.close()
+
+
+def test_model_training_step_replays_from_a_graph(cuda):
+    """A whole training step of the Graphormer mirror (forward, nll loss, backward, AdamW) captured once and
+    replayed on fresh inputs: every replay gives the loss of the eager step bit for bit, with eager work and
+    synchronisations between the replays, and the weights end up identical."""
+    from torchgt_amd import Graphormer
+    e, n = workloads.power_law_graph(n=3000, directed_edges=30000)
+    ei = torch.from_numpy(e).to(cuda)
+    g = torch.Generator().manual_seed(0)
+    xs = [torch.randn(n - 1, 32, generator=g).to(cuda) for _ in range(4)]
+    y = torch.randint(0, 10, (n - 1,), generator=g).to(cuda)
+
+    def make():
+        torch.manual_seed(7)
+        m = Graphormer(2, 8, 32, 64, 10, 1, 0.0, 0.0, 0.0, 64, 1).to(cuda)
+        return m, torch.optim.AdamW(m.parameters(), lr=1e-2, capturable=True)
+
+    def step(m, opt, x):
+        opt.zero_grad(set_to_none=True)
+        loss = torch.nn.functional.nll_loss(m(x, None, ei, attn_type="sparse"), y)
+        loss.backward()
+        opt.step()
+        return loss
+
+    m, opt = make()
+    for _ in range(3):
+        step(m, opt, xs[0])
+    eager = [step(m, opt, xs[i]).item() for i in range(1, 4)]
+    w_eager = [p.detach().clone() for p in m.parameters()]
+
+    m, opt = make()
+    static_x = xs[0].clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step(m, opt, static_x)
+    torch.cuda.current_stream().wait_stream(side)
+    gr = torch.cuda.CUDAGraph()
+    opt.zero_grad(set_to_none=True)
+    with torch.cuda.graph(gr):
+        static_loss = torch.nn.functional.nll_loss(m(static_x, None, ei, attn_type="sparse"), y)
+        static_loss.backward()
+        opt.step()
+    for i in range(1, 4):
+        static_x.copy_(xs[i])
+        gr.replay()
+        torch.cuda.synchronize()
+        assert static_loss.item() == eager[i - 1], (i, static_loss.item(), eager[i - 1])
+        assert torch.isfinite(torch.randn(1000, device=cuda).sum()).item()        # eager work between replays
+    for a, b in zip(w_eager, m.parameters()):
+        assert torch.equal(a, b.detach())

@@ -165,3 +165,23 @@ def test_module_without_output_layer(cuda):
     want = P.multi_head_attention_forward(x.double().numpy(), params, ei.numpy(), 8)
     got = m(x.to(cuda), None, ei.to(cuda), "sparse")
     assert err(got, want) <= 1e-5
+
+
+def test_fused_linear_pads_widths_that_do_not_fit(cuda):
+    """47 classes / 100-d bf16 features: the module-level helper pads to the vector width and slices back."""
+    for dtype, in_f, out_f in ((torch.float32, 64, 47), (torch.bfloat16, 100, 47)):
+        torch.manual_seed(0)
+        lin = torch.nn.Linear(in_f, out_f).to(dtype)
+        x = torch.randn(301, in_f).to(dtype)
+        dy = torch.randn(301, out_f).to(dtype)
+        xd = x.double().requires_grad_(True)
+        Wd, bd = lin.weight.detach().double().requires_grad_(True), lin.bias.detach().double().requires_grad_(True)
+        ref = torch.autograd.grad(torch.nn.functional.linear(xd, Wd, bd), [xd, Wd, bd], dy.double())
+        lc = lin.to(cuda)
+        xc = x.to(cuda).requires_grad_(True)
+        (y,) = fused_linear(xc, lc)
+        assert y.shape == (301, out_f)
+        got = torch.autograd.grad(y, [xc, lc.weight, lc.bias], dy.to(cuda))
+        assert err(y, torch.nn.functional.linear(xd, Wd, bd).detach().numpy()) <= TOL[dtype]
+        for a, r in zip(got, ref):
+            assert a.shape == r.shape and err(a, r.numpy()) <= TOL[dtype]
