@@ -42,6 +42,13 @@ extern "C" {
 #define TGT_BIAS_EDGE_HEAD 1   /* [E, H], one value per edge and head, caller's edge order */
 #define TGT_BIAS_EDGE      2   /* [E], one value per edge broadcast over heads
                                   (graphormer_dist_node_level.py:384)                     */
+/* OR'ed to TGT_BIAS_EDGE_HEAD / TGT_BIAS_EDGE: bias and dbias rows are in the plan's
+ * destination-sorted edge order (row i belongs to the caller's edge
+ * tgt_plan_edge_order()[i]) instead of the caller's order.  The walks by destination then
+ * read the bias and write dbias sequentially instead of through the edge permutation
+ * (random 16 / 32-byte accesses that cost as much as the K/V row gathers on large graphs);
+ * a bias shared by several layers is permuted once.  Needs tgt_plan_enable_bias_order(). */
+#define TGT_BIAS_PLAN_ORDER 0x10
 
 typedef struct tgt_plan tgt_plan_t;   /* opaque, owns device memory */
 
@@ -82,10 +89,24 @@ int tgt_plan_info(const tgt_plan_t* plan, int64_t info[16]);
 #define TGT_PLAN_EID_SRC    5
 #define TGT_PLAN_ITEMS_DST  6   /* int32 x4 per item: row, first edge, length, partial slot (-1 = whole row) */
 #define TGT_PLAN_ITEMS_SRC  7
+#define TGT_PLAN_POS_SRC    8   /* after tgt_plan_enable_bias_order: destination-sorted position of every edge of the source-sorted order */
 /* number of int32 values in array `which` */
 int64_t tgt_plan_array_len(const tgt_plan_t* plan, int which);
 /* copy array `which` to host memory (capacity in int32 elements); synchronous */
 int tgt_plan_export(const tgt_plan_t* plan, int which, int32_t* h_out, int64_t capacity);
+
+/* Support for TGT_BIAS_PLAN_ORDER.  tgt_plan_enable_bias_order builds (once; later calls return
+ * at once) the map from the source-sorted to the destination-sorted edge order that the walk by
+ * source needs; it allocates 4 bytes per edge and synchronises `stream`.  Call it before the
+ * first attention call that uses the flag (not from a graph capture).  tgt_plan_edge_order writes
+ * the permutation itself, int64 [E] on the device: d_out[i] = caller's index of the i-th edge in
+ * destination-sorted order (stable), so  bias_sorted = bias[d_out]  and  dbias[d_out] = dbias_sorted. */
+int tgt_plan_enable_bias_order(tgt_plan_t* plan, void* stream);
+int tgt_plan_edge_order(const tgt_plan_t* plan, int64_t* d_out, void* stream);
+/* Rows of row_bytes bytes, one per edge, between the two orders: inverse == 0 writes
+ * d_out[i] = d_in[edge_order[i]] (caller's order -> plan order: a bias), inverse != 0 writes
+ * d_out[edge_order[i]] = d_in[i] (plan order -> caller's order: its gradient).  d_in != d_out. */
+int tgt_plan_sort_rows(const tgt_plan_t* plan, const void* d_in, int row_bytes, void* d_out, int inverse, void* stream);
 
 /* ---- sparse attention ---------------------------------------------------
  * Workspace (device memory, 256-byte aligned) needed by fwd/bwd for partial

@@ -316,3 +316,55 @@ def test_config2_size_independent_properties(cuda):
     # weights are a convex combination: out lies within the range of v over the row's sources
     assert torch.isfinite(base[0]).all()
     assert base[0].abs().max() <= v.abs().max() + 1e-4
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("per_head", [True, False])
+def test_bias_in_plan_order_is_the_same_computation(cuda, dtype, per_head):
+    """TGT_BIAS_PLAN_ORDER: the bias permuted into the plan's destination-sorted order gives bit-identical
+    outputs and gradients, and the bias gradient comes back in the caller's order (graphs with split rows,
+    workgroup rows and all wave classes)."""
+    from torchgt_amd import get_plan, sparse_attention
+    for name, (e, n) in (("config1", workloads.barabasi_albert()),
+                         ("power-law", workloads.power_law_graph(n=20000, directed_edges=200000))):
+        print(f"plan-order bias case: {name} {dtype} per_head={per_head}", flush=True)
+        ei = torch.from_numpy(e).to(cuda)
+        E, H, d = e.shape[1], 8, 8
+        g = torch.Generator().manual_seed(3)
+        q, k, v, dout = (torch.randn(n, H, d, generator=g).to(cuda, dtype) for _ in range(4))
+        bias = (torch.randn(E, H, generator=g) if per_head else torch.randn(E, generator=g)).to(cuda, dtype)
+        plan = get_plan(ei, n)
+        order = plan.edge_order()
+        # the permutation is the stable sort of the destinations
+        want_order = torch.sort(ei[1], stable=True).indices
+        assert torch.equal(order, want_order)
+        outs = []
+        for sorted_mode in (False, True):
+            t = [x.clone().requires_grad_(True) for x in (q, k, v)]
+            b = bias.clone().requires_grad_(True)
+            bb = plan.sort_bias(b) if sorted_mode else b
+            o = sparse_attention(t[0], t[1], t[2], plan=plan, edge_bias=bb, bias_in_plan_order=sorted_mode)
+            outs.append((o, torch.autograd.grad(o, t + [b], dout)))
+        (o0, g0), (o1, g1) = outs
+        assert torch.equal(o0, o1)
+        for nm, a, b_ in zip(("dq", "dk", "dv", "dbias"), g0, g1):
+            assert torch.equal(a, b_), nm
+
+
+def test_plan_order_needs_the_map(cuda):
+    e, n = workloads.barabasi_albert()
+    ei = torch.from_numpy(e).to(cuda)
+    plan = GraphPlan(ei, n)
+    L = _lib.lib()
+    H = d = 8
+    q = torch.zeros(n, H, d, device=cuda)
+    b = torch.zeros(e.shape[1], H, device=cuda)
+    Z = torch.zeros(n, H, device=cuda)
+    ws = plan.workspace(H, d)
+    rc = L.tgt_sparse_attn_fwd(plan.handle, q.data_ptr(), q.data_ptr(), q.data_ptr(), b.data_ptr(),
+                               _lib.BIAS_EDGE_HEAD | _lib.BIAS_PLAN_ORDER, H, d, _lib.DTYPE_F32, q.data_ptr(), Z.data_ptr(),
+                               ws.data_ptr(), ws.numel(), None)
+    assert rc == _lib.ERR_INVALID_ARG and b"tgt_plan_enable_bias_order" in L.tgt_last_error()
+    assert L.tgt_sparse_attn_fwd(plan.handle, q.data_ptr(), q.data_ptr(), q.data_ptr(), b.data_ptr(), 0x13, H, d,
+                                 _lib.DTYPE_F32, q.data_ptr(), Z.data_ptr(), ws.data_ptr(), ws.numel(), None) == _lib.ERR_INVALID_ARG
+    plan.close()

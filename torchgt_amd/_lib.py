@@ -13,8 +13,9 @@ OK = 0
 ERR_INVALID_ARG, ERR_INDEX_RANGE, ERR_UNSUPPORTED, ERR_HIP, ERR_WORKSPACE = -1, -2, -3, -4, -5
 DTYPE_F32, DTYPE_BF16 = 0, 1
 BIAS_NONE, BIAS_EDGE_HEAD, BIAS_EDGE = 0, 1, 2
+BIAS_PLAN_ORDER = 0x10
 (PLAN_ROWPTR_DST, PLAN_COL_DST, PLAN_EID_DST, PLAN_ROWPTR_SRC, PLAN_COL_SRC, PLAN_EID_SRC,
- PLAN_ITEMS_DST, PLAN_ITEMS_SRC) = range(8)
+ PLAN_ITEMS_DST, PLAN_ITEMS_SRC, PLAN_POS_SRC) = range(9)
 
 _c = ctypes
 _vp, _i64, _i32 = _c.c_void_p, _c.c_int64, _c.c_int
@@ -29,6 +30,9 @@ SIGNATURES = {
     "tgt_plan_info": (_i32, [_vp, _c.POINTER(_i64)]),
     "tgt_plan_array_len": (_i64, [_vp, _i32]),
     "tgt_plan_export": (_i32, [_vp, _i32, _vp, _i64]),
+    "tgt_plan_enable_bias_order": (_i32, [_vp, _vp]),
+    "tgt_plan_edge_order": (_i32, [_vp, _vp, _vp]),
+    "tgt_plan_sort_rows": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp]),
     "tgt_sparse_attn_workspace_bytes": (_i64, [_vp, _i32, _i32]),
     "tgt_sparse_attn_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _i64, _vp]),
     "tgt_sparse_attn_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp,

@@ -34,7 +34,7 @@ class SparseAttentionFunction(torch.autograd.Function):
     torch_scatter ops, attn_module.py:146-187)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, edge_bias, plan):
+    def forward(ctx, q, k, v, edge_bias, plan, bias_in_plan_order=False):
         if not (q.is_cuda and k.is_cuda and v.is_cuda):
             raise RuntimeError("sparse attention needs GPU tensors (no CPU implementation)")
         if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
@@ -57,6 +57,9 @@ class SparseAttentionFunction(torch.autograd.Function):
                 mode = _lib.BIAS_EDGE
             else:
                 raise ValueError(f"edge bias must be [E] or [E, H] with E={E}, H={H}; got {tuple(edge_bias.shape)}")
+            if bias_in_plan_order:
+                plan.edge_order()               # makes sure the plan holds the map for this mode
+                mode |= _lib.BIAS_PLAN_ORDER
         out = torch.empty_like(q)
         Z = torch.empty((N, H), dtype=torch.float32, device=q.device)
         ws = plan.workspace(H, d)
@@ -89,7 +92,7 @@ class SparseAttentionFunction(torch.autograd.Function):
                 plan.handle, _ptr(q), _ptr(k), _ptr(v), _ptr(edge_bias), ctx.mode, H, d, _DTYPES[q.dtype],
                 _ptr(out), _ptr(Z), _ptr(dout), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(dbias),
                 _ptr(ws), ws.numel(), stream))
-        return dq, dk, dv, dbias, None
+        return dq, dk, dv, dbias, None, None
 
 
 class DenseAttentionFunction(torch.autograd.Function):
@@ -148,11 +151,13 @@ def dense_attention(q, k, v, attn_bias=None):
     return DenseAttentionFunction.apply(q, k, v, attn_bias)
 
 
-def sparse_attention(q, k, v, edge_index=None, edge_bias=None, plan=None, return_z=False):
+def sparse_attention(q, k, v, edge_index=None, edge_bias=None, plan=None, return_z=False, bias_in_plan_order=False):
     """Functional form.  q, k, v: [N, H, d] (or [b, S, H, d], flattened over b*S
     as in attn_module.py:141-143); ``edge_index`` int64 [2, E] (row 0 = source /
     key node, row 1 = destination / query node) or a prebuilt ``plan``;
-    ``edge_bias``: None, [E] or [E, H] in the order of ``edge_index``."""
+    ``edge_bias``: None, [E] or [E, H] in the order of ``edge_index`` - or, with
+    ``bias_in_plan_order=True``, already permuted with ``plan.sort_bias(bias)``
+    (worth it when several layers share one bias: see ``GraphPlan.sort_bias``)."""
     H, d = q.shape[-2], q.shape[-1]
     q3, k3, v3 = q.reshape(-1, H, d), k.reshape(-1, H, d), v.reshape(-1, H, d)
     if plan is None:
@@ -161,7 +166,7 @@ def sparse_attention(q, k, v, edge_index=None, edge_bias=None, plan=None, return
         plan = get_plan(edge_index, q3.shape[0])
     if edge_bias is not None:
         edge_bias = edge_bias.to(q3.dtype)
-    out, Z = SparseAttentionFunction.apply(q3, k3, v3, edge_bias, plan)
+    out, Z = SparseAttentionFunction.apply(q3, k3, v3, edge_bias, plan, bias_in_plan_order)
     return (out, Z) if return_z else out
 
 

@@ -39,6 +39,7 @@ struct Side {
     int32_t* rowptr = nullptr;   // [N+1]
     int32_t* col = nullptr;      // [E] other endpoint
     int32_t* eid = nullptr;      // [E] caller's edge id
+    int32_t* pos = nullptr;      // [E] source side only, built on request: position of the edge in the destination-sorted order
     Item* items = nullptr;       // [n_items]: workgroup items first, then wave items by length class (longest first)
     int32_t* split_row = nullptr;   // [n_split] rows that were split
     int32_t* split_off = nullptr;   // [n_split+1] first partial slot of each split row

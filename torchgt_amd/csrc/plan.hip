@@ -304,10 +304,41 @@ static int build_schedule(int64_t N, Side& side, hipStream_t st) {
     return TGT_OK;
 }
 
+// inv[eid[c]] = c, then pos[p] = inv[eid_src[p]]: where each edge of the source-sorted order sits in the
+// destination-sorted order
+__global__ void k_invert_perm(const int32_t* __restrict__ eid, int64_t E, int32_t* __restrict__ inv) {
+    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c < E) inv[eid[c]] = (int32_t)c;
+}
+__global__ void k_compose_perm(const int32_t* __restrict__ eid, const int32_t* __restrict__ inv, int64_t E,
+                               int32_t* __restrict__ pos) {
+    const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p < E) pos[p] = inv[eid[p]];
+}
+
+__global__ void k_widen(const int32_t* __restrict__ in, int64_t n, int64_t* __restrict__ out) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = in[i];
+}
+
+// rows of nv vectors: out[i] = in[eid[i]] (inverse: out[eid[i]] = in[i])
+template <typename V>
+__global__ void k_permute_rows(const V* __restrict__ in, const int32_t* __restrict__ eid, int64_t E, int nv,
+                               V* __restrict__ out, bool inverse) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= E * nv) return;
+    const int64_t i = t / nv;
+    const int v = (int)(t % nv);
+    const int64_t j = eid[i];
+    if (!inverse) out[i * nv + v] = in[j * nv + v];
+    else out[j * nv + v] = in[i * nv + v];
+}
+
 static void free_side(Side& s) {
     if (s.rowptr) (void)hipFree(s.rowptr);
     if (s.col) (void)hipFree(s.col);
     if (s.eid) (void)hipFree(s.eid);
+    if (s.pos) (void)hipFree(s.pos);
     if (s.items) (void)hipFree(s.items);
     if (s.split_row) (void)hipFree(s.split_row);
     if (s.split_off) (void)hipFree(s.split_off);
@@ -366,6 +397,24 @@ static int create_impl(const int64_t* d_src, const int64_t* d_dst, int64_t E, in
 extern "C" {
 
 int tgt_version(void) { return 1; }
+
+int tgt_plan_enable_bias_order(tgt_plan_t* plan, void* stream) {
+    if (!plan) { tgt::set_error("tgt_plan_enable_bias_order: null plan"); return TGT_ERR_INVALID_ARG; }
+    if (plan->src.pos) return TGT_OK;
+    const int64_t E = plan->E;
+    hipStream_t st = (hipStream_t)stream;
+    TGT_HIP_CHECK(hipMalloc((void**)&plan->src.pos, sizeof(int32_t) * (size_t)(E ? E : 1)));
+    if (E == 0) return TGT_OK;
+    tgt::DevBuf inv;
+    TGT_HIP_CHECK(inv.alloc(sizeof(int32_t) * (size_t)E));
+    const unsigned grid = (unsigned)((E + 255) / 256);
+    hipLaunchKernelGGL(tgt::k_invert_perm, dim3(grid), dim3(256), 0, st, plan->dst.eid, E, inv.as<int32_t>());
+    hipLaunchKernelGGL(tgt::k_compose_perm, dim3(grid), dim3(256), 0, st, plan->src.eid, inv.as<int32_t>(), E,
+                       plan->src.pos);
+    TGT_HIP_CHECK(hipGetLastError());
+    TGT_HIP_CHECK(hipStreamSynchronize(st));      // the scratch buffer is freed on return
+    return TGT_OK;
+}
 
 const char* tgt_error_string(int code) {
     switch (code) {
@@ -436,6 +485,7 @@ int64_t tgt_plan_array_len(const tgt_plan_t* plan, int which) {
         case TGT_PLAN_ROWPTR_DST: case TGT_PLAN_ROWPTR_SRC: return plan->N + 1;
         case TGT_PLAN_COL_DST: case TGT_PLAN_EID_DST:
         case TGT_PLAN_COL_SRC: case TGT_PLAN_EID_SRC: return plan->E;
+        case TGT_PLAN_POS_SRC: return plan->src.pos ? plan->E : 0;
         case TGT_PLAN_ITEMS_DST: return 4 * (int64_t)plan->dst.n_items;
         case TGT_PLAN_ITEMS_SRC: return 4 * (int64_t)plan->src.n_items;
         default: return -1;
@@ -456,11 +506,49 @@ int tgt_plan_export(const tgt_plan_t* plan, int which, int32_t* h_out, int64_t c
         case TGT_PLAN_ROWPTR_SRC: p = plan->src.rowptr; break;
         case TGT_PLAN_COL_SRC: p = plan->src.col; break;
         case TGT_PLAN_EID_SRC: p = plan->src.eid; break;
+        case TGT_PLAN_POS_SRC: p = plan->src.pos; break;
         case TGT_PLAN_ITEMS_DST: p = plan->dst.items; break;
         case TGT_PLAN_ITEMS_SRC: p = plan->src.items; break;
     }
     if (n == 0) return TGT_OK;
     TGT_HIP_CHECK(hipMemcpy(h_out, p, sizeof(int32_t) * n, hipMemcpyDeviceToHost));
+    return TGT_OK;
+}
+
+int tgt_plan_sort_rows(const tgt_plan_t* plan, const void* d_in, int row_bytes, void* d_out, int inverse, void* stream) {
+    if (!plan || row_bytes < 1 || (plan->E > 0 && (!d_in || !d_out))) {
+        tgt::set_error("tgt_plan_sort_rows: null pointer or bad row size");
+        return TGT_ERR_INVALID_ARG;
+    }
+    if (plan->E == 0) return TGT_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t E = plan->E;
+    const int32_t* eid = plan->dst.eid;
+    const bool inv = inverse != 0;
+#define TGT_LAUNCH_PERMUTE(V)                                                                                  \
+    do {                                                                                                       \
+        const int nv = row_bytes / (int)sizeof(V);                                                             \
+        const int64_t total = E * nv;                                                                          \
+        hipLaunchKernelGGL((tgt::k_permute_rows<V>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,  \
+                           (const V*)d_in, eid, E, nv, (V*)d_out, inv);                                        \
+    } while (0)
+    const uintptr_t al = (uintptr_t)d_in | (uintptr_t)d_out | (uintptr_t)row_bytes;
+    if (al % 16 == 0) TGT_LAUNCH_PERMUTE(uint4);
+    else if (al % 8 == 0) TGT_LAUNCH_PERMUTE(uint2);
+    else if (al % 4 == 0) TGT_LAUNCH_PERMUTE(uint32_t);
+    else if (al % 2 == 0) TGT_LAUNCH_PERMUTE(uint16_t);
+    else TGT_LAUNCH_PERMUTE(uint8_t);
+#undef TGT_LAUNCH_PERMUTE
+    TGT_HIP_CHECK(hipGetLastError());
+    return TGT_OK;
+}
+
+int tgt_plan_edge_order(const tgt_plan_t* plan, int64_t* d_out, void* stream) {
+    if (!plan || (plan->E > 0 && !d_out)) { tgt::set_error("tgt_plan_edge_order: null pointer"); return TGT_ERR_INVALID_ARG; }
+    if (plan->E == 0) return TGT_OK;
+    hipLaunchKernelGGL(tgt::k_widen, dim3((unsigned)((plan->E + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       plan->dst.eid, plan->E, d_out);
+    TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
 }
 

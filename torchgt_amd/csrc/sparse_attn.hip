@@ -188,7 +188,7 @@ __host__ __device__ constexpr int part_stride() {
 // Walks `len` edges starting at sorted position `start` of node `row` with S edge
 // slots (this lane is slot `slot`, element chunk `el`).  On return every lane of
 // the S*LPE-lane group holds the sums over all S slots.
-template <typename T, int LPE, int LPH, int S, int MODE, bool HASB>
+template <typename T, int LPE, int LPH, int S, int MODE, int HASB>
 __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, const int row, const int start,
                                            const int len, const int slot, const int el, const bool valid,
                                            Acc& acc) {
@@ -222,7 +222,9 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
         }
     }
     const int32_t* __restrict__ col = s.col + start;
-    const int32_t* __restrict__ eid = s.eid + start;
+    // HASB == 2: no edge-id array, the bias rows are in this side's own sorted order (row = sorted position)
+    constexpr bool ident = HASB == 2;
+    const int32_t* __restrict__ eid = ident ? nullptr : s.eid + start;
     const int bias_se = c.bias_se, bias_sh = c.bias_sh;
     const float inv_scale = c.inv_scale;
     const int n = valid ? len : 0;
@@ -243,7 +245,7 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
                 nb[u] = 0; ed[u] = 0;
                 if (ok[u]) {
                     nb[u] = col[e];
-                    if (HASB) ed[u] = eid[e];
+                    if (HASB) ed[u] = ident ? start + e : eid[e];
                 }
             }
 #pragma unroll
@@ -275,7 +277,7 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
             ok[u] = e < n;
             const int ec = min(e, n - 1);
             nb[u] = col[ec];
-            ed[u] = HASB ? eid[ec] : 0;
+            ed[u] = HASB ? (ident ? start + ec : eid[ec]) : 0;
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
@@ -390,7 +392,7 @@ __device__ __forceinline__ void write_row(const Common& c, const SideArgs& s, co
 }
 
 // Wave items: rows of at most kWaveRowMax edges, 64 / (LPE*S) rows per wave.
-template <typename T, int LPE, int LPH, int S, int MODE, bool HASB, bool TILES>
+template <typename T, int LPE, int LPH, int S, int MODE, int HASB, bool TILES>
 __device__ __forceinline__ void wave_items(const Common& c, const SideArgs& s, const int item_begin,
                                            const int item_end, const int wave_in_class) {
     constexpr int G = LPE * S;
@@ -413,7 +415,7 @@ __device__ __forceinline__ void wave_items(const Common& c, const SideArgs& s, c
 // every class, longest class first: rows that are neighbours in the schedule meet in one L2.
 // `block` counts from the start of this view's wave region, which begins at a workgroup id
 // that is a multiple of 8.
-template <typename T, int LPE, int LPH, int MODE, bool HASB, bool TILES>
+template <typename T, int LPE, int LPH, int MODE, int HASB, bool TILES>
 __device__ __forceinline__ void wave_block(const Common& c, const SideArgs& s, const int block) {
     const int xcd = block & 7;
     const int v = (block >> 3) * (kBlock / kWave) + (threadIdx.x >> 6);   // wave slot inside the XCD
@@ -451,7 +453,7 @@ struct BlockLds {
 // slot, and the workgroup that arrives last adds the slots in slot order and
 // writes the row - no second launch, no floating-point atomics, and the order of
 // the additions does not depend on which workgroup is last.
-template <typename T, int LPE, int LPH, int MODE, bool HASB, bool TILES>
+template <typename T, int LPE, int LPH, int MODE, int HASB, bool TILES>
 __device__ __forceinline__ void block_item(const Common& c, const SideArgs& s, const int item,
                                            BlockLds<LPE>& lds) {
     constexpr int S = slots_for_class(LPE, 0);
@@ -570,7 +572,7 @@ __device__ __forceinline__ void block_item(const Common& c, const SideArgs& s, c
 
 // Forward: workgroup items of the destination view first (longest work first),
 // then its wave items.
-template <typename T, int LPE, int LPH, bool HASB, bool TILES>
+template <typename T, int LPE, int LPH, int HASB, bool TILES>
 __global__ __launch_bounds__(kBlock) void k_attn_fwd(const Common c, const SideArgs s, const int items_pad) {
     __shared__ BlockLds<LPE> lds;
     const int b = blockIdx.x;
@@ -592,7 +594,7 @@ __global__ __launch_bounds__(kBlock) void k_attn_fwd(const Common c, const SideA
 // Backward: both views in one launch (they are independent once nd is known):
 // workgroup items of the destination view, workgroup items of the source view,
 // wave items of the destination view, wave items of the source view.
-template <typename T, int LPE, int LPH, bool HASB, bool TILES>
+template <typename T, int LPE, int LPH, int HASB, bool TILES>
 __global__ __launch_bounds__(kBlock, 4) void k_attn_bwd(const Common c, const SideArgs sd, const SideArgs ss,
                                                      const int pad_d, const int pad_s) {
     __shared__ BlockLds<LPE> lds;
@@ -610,18 +612,18 @@ __global__ __launch_bounds__(kBlock, 4) void k_attn_bwd(const Common c, const Si
     b -= pad_d;
     if (b < pad_s) {
         if (b < ss.spread_pad) {
-            if (b < ss.n_spread) block_item<T, LPE, LPH, MODE_BWD_SRC, HASB, TILES>(c, ss, b, lds);
+            if (b < ss.n_spread) block_item<T, LPE, LPH, MODE_BWD_SRC, (HASB ? 1 : 0), TILES>(c, ss, b, lds);
         } else {
             const int bb = b - ss.spread_pad;
             const int it = ss.blk_chunk[bb & 7] + (bb >> 3);
-            if (it < ss.blk_chunk[(bb & 7) + 1]) block_item<T, LPE, LPH, MODE_BWD_SRC, HASB, TILES>(c, ss, it, lds);
+            if (it < ss.blk_chunk[(bb & 7) + 1]) block_item<T, LPE, LPH, MODE_BWD_SRC, (HASB ? 1 : 0), TILES>(c, ss, it, lds);
         }
         return;
     }
     b -= pad_s;
     if (b < sd.n_wave_blocks) { wave_block<T, LPE, LPH, MODE_BWD_DST, HASB, TILES>(c, sd, b); return; }
     b -= sd.n_wave_blocks;
-    wave_block<T, LPE, LPH, MODE_BWD_SRC, HASB, TILES>(c, ss, b);
+    wave_block<T, LPE, LPH, MODE_BWD_SRC, (HASB ? 1 : 0), TILES>(c, ss, b);
 }
 
 // Per-node side vector of the backward: nd[i,h] = (1 / (Z[i,h] + eps), sum_c dout[i,h,c] out[i,h,c]).
@@ -722,11 +724,12 @@ static int run_fwd(const Call& c) {
     Common cm{};
     cm.q = c.q; cm.k = c.k; cm.v = c.v; cm.g = nullptr; cm.bias = c.bias; cm.nd = nullptr;
     cm.bias_mode = c.bias_mode;
-    cm.bias_se = c.bias_mode == TGT_BIAS_EDGE_HEAD ? c.H : 1;
-    cm.bias_sh = c.bias_mode == TGT_BIAS_EDGE_HEAD ? 1 : 0;
+    cm.bias_se = (c.bias_mode & 0xf) == TGT_BIAS_EDGE_HEAD ? c.H : 1;
+    cm.bias_sh = (c.bias_mode & 0xf) == TGT_BIAS_EDGE_HEAD ? 1 : 0;
     cm.inv_scale = 1.0f / sqrtf((float)c.d);
     SideArgs a{};
     fill_side(a, c.plan->dst, LPE);
+    if (c.bias_mode & TGT_BIAS_PLAN_ORDER) a.eid = nullptr;             // bias rows in destination-sorted order
     a.out0 = c.o_out; a.out1 = nullptr; a.Z = c.o_Z;
     if (c.init) { a.init0 = c.init->acc; a.initZ = c.init->Z; a.cover = c.init->cover_dst; }
     a.part = reinterpret_cast<float*>(c.ws + L.fwd_part);
@@ -736,18 +739,24 @@ static int run_fwd(const Call& c) {
     if (nb > 0) {
         KernelTimer t(KS_FWD, c.st);
         const bool hb = c.bias_mode != TGT_BIAS_NONE;
+        if (c.init != nullptr && (c.bias_mode & TGT_BIAS_PLAN_ORDER)) {
+            set_error("block attention takes the bias in the caller's edge order");
+            return TGT_ERR_UNSUPPORTED;
+        }
         if (c.init != nullptr) {
             if constexpr (kTilesShape<LPE, LPH>) {
-                if (hb) hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, true, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
-                else hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, false, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
+                if (hb) hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, 1, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
+                else hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, 0, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
             } else {
                 set_error("block attention: no kernel for this (H, d)");
                 return TGT_ERR_UNSUPPORTED;
             }
+        } else if (hb && (c.bias_mode & TGT_BIAS_PLAN_ORDER)) {
+            hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, 2, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
         } else if (hb) {
-            hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, true, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
+            hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, 1, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
         } else {
-            hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, false, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
+            hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, 0, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
         }
     }
     TGT_HIP_CHECK(hipGetLastError());
@@ -771,17 +780,19 @@ static int run_bwd(const Call& c) {
     Common cm{};
     cm.q = c.q; cm.k = c.k; cm.v = c.v; cm.g = c.dout; cm.bias = c.bias; cm.nd = nd;
     cm.bias_mode = c.bias_mode;
-    cm.bias_se = c.bias_mode == TGT_BIAS_EDGE_HEAD ? c.H : 1;
-    cm.bias_sh = c.bias_mode == TGT_BIAS_EDGE_HEAD ? 1 : 0;
+    cm.bias_se = (c.bias_mode & 0xf) == TGT_BIAS_EDGE_HEAD ? c.H : 1;
+    cm.bias_sh = (c.bias_mode & 0xf) == TGT_BIAS_EDGE_HEAD ? 1 : 0;
     cm.inv_scale = 1.0f / sqrtf((float)c.d);
     int32_t* counters = reinterpret_cast<int32_t*>(c.ws + L.counters);
     SideArgs sd{}, ss{};
     fill_side(sd, c.plan->dst, LPE);
+    if (c.bias_mode & TGT_BIAS_PLAN_ORDER) sd.eid = nullptr;
     sd.out0 = c.dq; sd.out1 = c.dbias; sd.Z = nullptr;
     if (c.init) { sd.init0 = c.init->dq; sd.cover = c.init->cover_dst; }
     sd.part = reinterpret_cast<float*>(c.ws + L.dq_part);
     sd.counters = counters + c.plan->dst.n_split;
     fill_side(ss, c.plan->src, LPE);
+    if (c.bias_mode & TGT_BIAS_PLAN_ORDER) ss.eid = c.plan->src.pos;    // source-sorted -> destination-sorted position
     ss.out0 = c.dk; ss.out1 = c.dv; ss.Z = nullptr;
     if (c.init) { ss.init0 = c.init->dk; ss.init1 = c.init->dv; ss.cover = c.init->cover_src; }
     ss.part = reinterpret_cast<float*>(c.ws + L.dkv_part);
@@ -791,18 +802,24 @@ static int run_bwd(const Call& c) {
     if (nb > 0) {
         KernelTimer t(KS_BWD, c.st);
         const bool hb = c.bias_mode != TGT_BIAS_NONE;
+        if (c.init != nullptr && (c.bias_mode & TGT_BIAS_PLAN_ORDER)) {
+            set_error("block attention takes the bias in the caller's edge order");
+            return TGT_ERR_UNSUPPORTED;
+        }
         if (c.init != nullptr) {
             if constexpr (kTilesShape<LPE, LPH>) {
-                if (hb) hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, true, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
-                else hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, false, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
+                if (hb) hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, 1, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
+                else hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, 0, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
             } else {
                 set_error("block attention: no kernel for this (H, d)");
                 return TGT_ERR_UNSUPPORTED;
             }
+        } else if (hb && (c.bias_mode & TGT_BIAS_PLAN_ORDER)) {
+            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, 2, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
         } else if (hb) {
-            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, true, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
+            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, 1, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
         } else {
-            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, false, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
+            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, 0, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
         }
     }
     TGT_HIP_CHECK(hipGetLastError());
@@ -834,7 +851,18 @@ static int dispatch(const Call& c, bool bwd) {
 static int check_common(const tgt_plan* plan, const void* q, const void* k, const void* v, const void* bias,
                         int bias_mode, int H, int d, int dtype, const void* ws, int64_t ws_bytes) {
     if (!plan || !q || !k || !v) { set_error("null plan or q/k/v"); return TGT_ERR_INVALID_ARG; }
-    if (bias_mode < TGT_BIAS_NONE || bias_mode > TGT_BIAS_EDGE) { set_error("bad bias_mode %d", bias_mode); return TGT_ERR_INVALID_ARG; }
+    {
+        const int base = bias_mode & 0xf;
+        if (bias_mode < 0 || (bias_mode & ~(0xf | TGT_BIAS_PLAN_ORDER)) || base > TGT_BIAS_EDGE ||
+            (base == TGT_BIAS_NONE && bias_mode != TGT_BIAS_NONE)) {
+            set_error("bad bias_mode %d", bias_mode);
+            return TGT_ERR_INVALID_ARG;
+        }
+        if ((bias_mode & TGT_BIAS_PLAN_ORDER) && !plan->src.pos) {
+            set_error("TGT_BIAS_PLAN_ORDER needs tgt_plan_enable_bias_order(plan) first");
+            return TGT_ERR_INVALID_ARG;
+        }
+    }
     if (bias_mode != TGT_BIAS_NONE && !bias && plan->E > 0) { set_error("bias_mode %d needs a bias pointer", bias_mode); return TGT_ERR_INVALID_ARG; }
     if (dtype != TGT_DTYPE_F32 && dtype != TGT_DTYPE_BF16) { set_error("bad dtype %d", dtype); return TGT_ERR_INVALID_ARG; }
     if (H < 1 || d < 1) { set_error("H and d must be positive"); return TGT_ERR_INVALID_ARG; }

@@ -74,6 +74,41 @@ class GraphPlan:
         _lib.check(L.tgt_plan_export(self.handle, which, out.ctypes.data_as(ctypes.c_void_p), n))
         return out
 
+    def edge_order(self):
+        """int64 [E] on the GPU: the caller's index of every edge in the plan's destination-sorted (stable)
+        order.  ``bias[plan.edge_order()]`` is a bias in plan order (see ``sort_bias``).  Also builds, once,
+        the map the walk by source needs for such a bias."""
+        if getattr(self, "_edge_order", None) is None:
+            L = _lib.lib()
+            out = torch.empty(self.num_edges, dtype=torch.int64, device=self.device)
+            with torch.cuda.device(self.device):
+                stream = torch.cuda.current_stream(self.device).cuda_stream
+                _lib.check(L.tgt_plan_enable_bias_order(self.handle, stream))
+                _lib.check(L.tgt_plan_edge_order(self.handle, out.data_ptr() if self.num_edges else None, stream))
+            self._edge_order = out
+        return self._edge_order
+
+    def sort_bias(self, edge_bias):
+        """A per-edge bias ([E] or [E, H], caller's edge order) in plan order, for
+        ``sparse_attention(..., bias_in_plan_order=True)``.  Differentiable: the gradient comes back in the
+        caller's order.  Permute a bias that several layers share once and pass the result to all of them: the
+        destination walks then stream it instead of gathering 16/32-byte pieces through the edge permutation."""
+        return _SortRows.apply(edge_bias, self)
+
+    def _permute(self, t, inverse):
+        self.edge_order()
+        t = t.contiguous()
+        if t.shape[0] != self.num_edges:
+            raise ValueError(f"expected {self.num_edges} rows, got {t.shape[0]}")
+        out = torch.empty_like(t)
+        if self.num_edges:
+            row_bytes = t.element_size() * (t.numel() // self.num_edges)
+            with torch.cuda.device(self.device):
+                _lib.check(_lib.lib().tgt_plan_sort_rows(self.handle, t.data_ptr(), row_bytes, out.data_ptr(),
+                                                         1 if inverse else 0,
+                                                         torch.cuda.current_stream(self.device).cuda_stream))
+        return out
+
     def workspace(self, H, d):
         """Device scratch for the attention calls on this plan (cached per (H, d)).
         Calls that share it must be ordered on one stream."""
@@ -86,6 +121,19 @@ class GraphPlan:
             ws = torch.zeros(max(int(nbytes), 256), dtype=torch.uint8, device=self.device)   # counters start at 0
             self._workspaces[key] = ws
         return ws
+
+
+class _SortRows(torch.autograd.Function):
+    """bias in plan order; the gradient is carried back to the caller's order."""
+
+    @staticmethod
+    def forward(ctx, t, plan):
+        ctx.plan = plan
+        return plan._permute(t, inverse=False)
+
+    @staticmethod
+    def backward(ctx, g):
+        return ctx.plan._permute(g, inverse=True), None
 
 
 _CACHE = collections.OrderedDict()
