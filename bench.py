@@ -608,6 +608,40 @@ def main():
     L.tgt_timing_enable(0)
     timings = _lib.kernel_timings()
     kernels = {name: {"avg_us": ms / cnt * 1e3, "launches": cnt} for name, (ms, cnt) in timings.items() if cnt}
+
+    # Second datapoint, not the headline: the same step with the bias already in the plan's destination-sorted
+    # order (TGT_BIAS_PLAN_ORDER; a bias shared by the layers of a model is permuted once per step), plus what
+    # the permutation of the bias and of its gradient costs.
+    def plan_order_point():
+        order_mode = _lib.BIAS_EDGE_HEAD | _lib.BIAS_PLAN_ORDER
+        bias_sorted = plan._permute(bias, inverse=False)
+
+        def ostep():
+            _lib.check(L.tgt_sparse_attn_fwd(plan.handle, P(q), P(k), P(v), P(bias_sorted), order_mode, H, d,
+                                             dt_code, P(out), P(Z), P(ws), ws.numel(), stream))
+            _lib.check(L.tgt_sparse_attn_bwd(plan.handle, P(q), P(k), P(v), P(bias_sorted), order_mode, H, d,
+                                             dt_code, P(out), P(Z), P(dout), P(dq), P(dk), P(dv), P(dbias),
+                                             P(ws), ws.numel(), stream))
+
+        n_it = max(5, args.steps // 4)
+        for _ in range(3):
+            ostep()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n_it):
+            ostep()
+        torch.cuda.synchronize()
+        step_us = (time.perf_counter() - t0) / n_it * 1e6
+        t0 = time.perf_counter()
+        for _ in range(n_it):
+            plan._permute(bias, inverse=False)
+            plan._permute(dbias, inverse=True)
+        torch.cuda.synchronize()
+        perm_us = (time.perf_counter() - t0) / n_it * 1e6
+        return {"step_us": step_us, "edges_per_s": E / (step_us * 1e-6),
+                "permute_bias_and_gradient_us_once_per_model_step": perm_us}
+
+    plan_order = plan_order_point()
     probe = gather_probe(plan, n, E, H * d * esize, stream)
     bpe = H * esize
     dom = max((kk for kk in kernels if kernel_alg_bytes(kk, n, E, H, d, esize, bpe)),
@@ -636,6 +670,7 @@ def main():
                      "alg_bytes": dom_bytes,
                      "avg_us": kernels[dom]["avg_us"]},
         "kernels": kernels,
+        "bias_in_plan_order": plan_order,
         # what a bare gather of the forward walk's k and v rows costs (no arithmetic, no index chain)
         "row_gather_probe": probe,
         "plan_build_ms": plan_ms, "plan_build_first_ms": plan_first_ms,

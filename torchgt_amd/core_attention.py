@@ -183,6 +183,30 @@ def gather_dense_bias(attn_bias, edge_index, layout):
     return attn_bias[src // S, src % S, dst % S, :]
 
 
+_BIAS_CACHE = {}      # one entry: (bias tensor, its version, plan, dtype, layout) -> per-edge bias in plan order
+
+
+def _plan_order_bias(module, attn_bias, edge_index, plan, dtype):
+    """Per-edge bias in the plan's destination-sorted order for a dense or per-edge ``attn_bias``; the last
+    result is kept (with the tensor it came from, so its identity cannot be recycled) and reused while the same
+    bias object comes in again - the other layers of the same step.  Differentiable."""
+    key = (id(attn_bias), attn_bias._version, id(plan), dtype, module.dense_bias_layout)
+    hit = _BIAS_CACHE.get("entry")
+    if hit is not None and hit[0] == key and hit[1] is attn_bias and hit[2] is plan:
+        return hit[3]
+    if attn_bias.dim() <= 2:
+        eb = plan.sort_bias(attn_bias.to(dtype))
+    else:
+        if isinstance(edge_index, GraphPlan):
+            raise ValueError("a dense attn_bias needs the edge_index tensor (not a prebuilt plan)")
+        eb = gather_dense_bias(attn_bias, edge_index.index_select(1, plan.edge_order()), module.dense_bias_layout)
+        if eb.shape[-1] == 1:
+            eb = eb.squeeze(-1)
+        eb = eb.to(dtype)
+    _BIAS_CACHE["entry"] = (key, attn_bias, plan, eb)
+    return eb
+
+
 class CoreAttention(nn.Module):
     """Same constructor and call conventions as the reference's ``CoreAttention``
     classes (see the module docstring for the three flavours)."""
@@ -219,10 +243,13 @@ class CoreAttention(nn.Module):
         k3 = k.reshape(-1, H, d)
         v3 = v.reshape(-1, H, d)
         plan = edge_index if isinstance(edge_index, GraphPlan) else get_plan(edge_index, q3.shape[0])
-        eb = self._edge_bias(attn_bias, edge_index)
-        if eb is not None:
-            eb = eb.to(q3.dtype)
-        out, _ = SparseAttentionFunction.apply(q3, k3, v3, eb, plan)
+        if attn_bias is None:
+            out, _ = SparseAttentionFunction.apply(q3, k3, v3, None, plan)
+            return out
+        # The layers of a model get one and the same bias tensor: it is brought into the plan's edge order once
+        # (by the first layer that sees it) and every layer then streams it.
+        eb = _plan_order_bias(self, attn_bias, edge_index, plan, q3.dtype)
+        out, _ = SparseAttentionFunction.apply(q3, k3, v3, eb, plan, True)
         return out
 
     # -- reference method names -------------------------------------------

@@ -159,3 +159,5 @@ def get_plan(edge_index, num_nodes):
 
 def clear_plan_cache():
     _CACHE.clear()
+    from . import core_attention
+    core_attention._BIAS_CACHE.clear()
