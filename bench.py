@@ -613,14 +613,21 @@ def main():
     # order (TGT_BIAS_PLAN_ORDER; a bias shared by the layers of a model is permuted once per step), plus what
     # the permutation of the bias and of its gradient costs.
     def plan_order_point():
-        order_mode = _lib.BIAS_EDGE_HEAD | _lib.BIAS_PLAN_ORDER
-        bias_sorted = plan._permute(bias, inverse=False)
+        order_mode = _lib.BIAS_EDGE_HEAD | _lib.BIAS_PLAN_ORDER | _lib.BIAS_BOTH_ORDERS
+        bias2 = torch.empty((2 * E, H), dtype=bias.dtype, device=dev)     # destination-sorted rows, then source-sorted
+        dbias2 = torch.empty_like(bias2)
+
+        def permute():
+            plan._permute(bias, 0, out=bias2[:E])
+            plan._permute(bias, 2, out=bias2[E:])
+
+        permute()
 
         def ostep():
-            _lib.check(L.tgt_sparse_attn_fwd(plan.handle, P(q), P(k), P(v), P(bias_sorted), order_mode, H, d,
+            _lib.check(L.tgt_sparse_attn_fwd(plan.handle, P(q), P(k), P(v), P(bias2), order_mode, H, d,
                                              dt_code, P(out), P(Z), P(ws), ws.numel(), stream))
-            _lib.check(L.tgt_sparse_attn_bwd(plan.handle, P(q), P(k), P(v), P(bias_sorted), order_mode, H, d,
-                                             dt_code, P(out), P(Z), P(dout), P(dq), P(dk), P(dv), P(dbias),
+            _lib.check(L.tgt_sparse_attn_bwd(plan.handle, P(q), P(k), P(v), P(bias2), order_mode, H, d,
+                                             dt_code, P(out), P(Z), P(dout), P(dq), P(dk), P(dv), P(dbias2),
                                              P(ws), ws.numel(), stream))
 
         n_it = max(5, args.steps // 4)
@@ -634,12 +641,13 @@ def main():
         step_us = (time.perf_counter() - t0) / n_it * 1e6
         t0 = time.perf_counter()
         for _ in range(n_it):
-            plan._permute(bias, inverse=False)
-            plan._permute(dbias, inverse=True)
+            permute()
+            plan._permute(dbias2[:E], 1, out=dbias)
         torch.cuda.synchronize()
         perm_us = (time.perf_counter() - t0) / n_it * 1e6
         return {"step_us": step_us, "edges_per_s": E / (step_us * 1e-6),
-                "permute_bias_and_gradient_us_once_per_model_step": perm_us}
+                "permute_bias_and_gradient_us_once_per_model_step": perm_us,
+                "mode": "TGT_BIAS_PLAN_ORDER | TGT_BIAS_BOTH_ORDERS"}
 
     plan_order = plan_order_point()
     probe = gather_probe(plan, n, E, H * d * esize, stream)

@@ -49,6 +49,12 @@ extern "C" {
  * (random 16 / 32-byte accesses that cost as much as the K/V row gathers on large graphs);
  * a bias shared by several layers is permuted once.  Needs tgt_plan_enable_bias_order(). */
 #define TGT_BIAS_PLAN_ORDER 0x10
+/* OR'ed to TGT_BIAS_PLAN_ORDER: d_bias holds the bias twice, 2 * E rows: first in
+ * destination-sorted order, then in source-sorted order (tgt_plan_sort_rows with
+ * direction 0 and 2).  The backward's walk by source then streams its copy as well: no
+ * walk gathers the bias any more, and tgt_plan_enable_bias_order is not needed.  The
+ * forward reads the first copy only; d_dbias is [E] / [E, H] in destination-sorted order. */
+#define TGT_BIAS_BOTH_ORDERS 0x20
 
 typedef struct tgt_plan tgt_plan_t;   /* opaque, owns device memory */
 
@@ -103,10 +109,13 @@ int tgt_plan_export(const tgt_plan_t* plan, int which, int32_t* h_out, int64_t c
  * destination-sorted order (stable), so  bias_sorted = bias[d_out]  and  dbias[d_out] = dbias_sorted. */
 int tgt_plan_enable_bias_order(tgt_plan_t* plan, void* stream);
 int tgt_plan_edge_order(const tgt_plan_t* plan, int64_t* d_out, void* stream);
-/* Rows of row_bytes bytes, one per edge, between the two orders: inverse == 0 writes
- * d_out[i] = d_in[edge_order[i]] (caller's order -> plan order: a bias), inverse != 0 writes
- * d_out[edge_order[i]] = d_in[i] (plan order -> caller's order: its gradient).  d_in != d_out. */
-int tgt_plan_sort_rows(const tgt_plan_t* plan, const void* d_in, int row_bytes, void* d_out, int inverse, void* stream);
+/* the same for the source-sorted (stable) order */
+int tgt_plan_edge_order_src(const tgt_plan_t* plan, int64_t* d_out, void* stream);
+/* Rows of row_bytes bytes, one per edge, between the orders.  direction 0: d_out[i] =
+ * d_in[edge_order[i]] (caller's order -> destination-sorted: a bias); 1: d_out[edge_order[i]] =
+ * d_in[i] (destination-sorted -> caller's order: its gradient); 2: caller's order ->
+ * source-sorted (the second copy of TGT_BIAS_BOTH_ORDERS).  d_in != d_out. */
+int tgt_plan_sort_rows(const tgt_plan_t* plan, const void* d_in, int row_bytes, void* d_out, int direction, void* stream);
 
 /* ---- sparse attention ---------------------------------------------------
  * Workspace (device memory, 256-byte aligned) needed by fwd/bwd for partial

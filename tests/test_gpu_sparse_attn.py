@@ -338,17 +338,20 @@ def test_bias_in_plan_order_is_the_same_computation(cuda, dtype, per_head):
         # the permutation is the stable sort of the destinations
         want_order = torch.sort(ei[1], stable=True).indices
         assert torch.equal(order, want_order)
+        assert torch.equal(plan.edge_order_src(), torch.sort(ei[0], stable=True).indices)
         outs = []
-        for sorted_mode in (False, True):
+        for sorted_mode in (None, "dst", "both"):
             t = [x.clone().requires_grad_(True) for x in (q, k, v)]
             b = bias.clone().requires_grad_(True)
-            bb = plan.sort_bias(b) if sorted_mode else b
-            o = sparse_attention(t[0], t[1], t[2], plan=plan, edge_bias=bb, bias_in_plan_order=sorted_mode)
+            bb = b if sorted_mode is None else plan.sort_bias(b, both_orders=(sorted_mode == "both"))
+            assert bb.shape[0] == (2 * E if sorted_mode == "both" else E)
+            o = sparse_attention(t[0], t[1], t[2], plan=plan, edge_bias=bb, bias_in_plan_order=sorted_mode is not None)
             outs.append((o, torch.autograd.grad(o, t + [b], dout)))
-        (o0, g0), (o1, g1) = outs
-        assert torch.equal(o0, o1)
-        for nm, a, b_ in zip(("dq", "dk", "dv", "dbias"), g0, g1):
-            assert torch.equal(a, b_), nm
+        (o0, g0) = outs[0]
+        for o1, g1 in outs[1:]:
+            assert torch.equal(o0, o1)
+            for nm, a, b_ in zip(("dq", "dk", "dv", "dbias"), g0, g1):
+                assert torch.equal(a, b_), nm
 
 
 def test_plan_order_needs_the_map(cuda):
@@ -365,6 +368,6 @@ def test_plan_order_needs_the_map(cuda):
                                _lib.BIAS_EDGE_HEAD | _lib.BIAS_PLAN_ORDER, H, d, _lib.DTYPE_F32, q.data_ptr(), Z.data_ptr(),
                                ws.data_ptr(), ws.numel(), None)
     assert rc == _lib.ERR_INVALID_ARG and b"tgt_plan_enable_bias_order" in L.tgt_last_error()
-    assert L.tgt_sparse_attn_fwd(plan.handle, q.data_ptr(), q.data_ptr(), q.data_ptr(), b.data_ptr(), 0x13, H, d,
+    assert L.tgt_sparse_attn_fwd(plan.handle, q.data_ptr(), q.data_ptr(), q.data_ptr(), b.data_ptr(), 0x23, H, d,
                                  _lib.DTYPE_F32, q.data_ptr(), Z.data_ptr(), ws.data_ptr(), ws.numel(), None) == _lib.ERR_INVALID_ARG
     plan.close()

@@ -14,6 +14,7 @@ ERR_INVALID_ARG, ERR_INDEX_RANGE, ERR_UNSUPPORTED, ERR_HIP, ERR_WORKSPACE = -1, 
 DTYPE_F32, DTYPE_BF16 = 0, 1
 BIAS_NONE, BIAS_EDGE_HEAD, BIAS_EDGE = 0, 1, 2
 BIAS_PLAN_ORDER = 0x10
+BIAS_BOTH_ORDERS = 0x20
 (PLAN_ROWPTR_DST, PLAN_COL_DST, PLAN_EID_DST, PLAN_ROWPTR_SRC, PLAN_COL_SRC, PLAN_EID_SRC,
  PLAN_ITEMS_DST, PLAN_ITEMS_SRC, PLAN_POS_SRC) = range(9)
 
@@ -32,6 +33,7 @@ SIGNATURES = {
     "tgt_plan_export": (_i32, [_vp, _i32, _vp, _i64]),
     "tgt_plan_enable_bias_order": (_i32, [_vp, _vp]),
     "tgt_plan_edge_order": (_i32, [_vp, _vp, _vp]),
+    "tgt_plan_edge_order_src": (_i32, [_vp, _vp, _vp]),
     "tgt_plan_sort_rows": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp]),
     "tgt_sparse_attn_workspace_bytes": (_i64, [_vp, _i32, _i32]),
     "tgt_sparse_attn_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _i64, _vp]),

@@ -51,15 +51,20 @@ class SparseAttentionFunction(torch.autograd.Function):
                 raise TypeError("edge bias must have the dtype of q (convert it outside, where autograd sees it)")
             edge_bias = edge_bias.contiguous()
             E = plan.num_edges
-            if edge_bias.dim() == 2 and edge_bias.shape == (E, H) and H != 1:
+            both = bias_in_plan_order and edge_bias.shape[0] == 2 * E and E > 0
+            rows = 2 * E if both else E
+            if edge_bias.dim() == 2 and edge_bias.shape == (rows, H) and H != 1:
                 mode = _lib.BIAS_EDGE_HEAD
-            elif edge_bias.numel() == E:
+            elif edge_bias.numel() == rows:
                 mode = _lib.BIAS_EDGE
             else:
                 raise ValueError(f"edge bias must be [E] or [E, H] with E={E}, H={H}; got {tuple(edge_bias.shape)}")
             if bias_in_plan_order:
-                plan.edge_order()               # makes sure the plan holds the map for this mode
                 mode |= _lib.BIAS_PLAN_ORDER
+                if both:
+                    mode |= _lib.BIAS_BOTH_ORDERS      # [2E, ...]: destination-sorted rows, then source-sorted rows
+                else:
+                    plan.edge_order()                  # makes sure the plan holds the map for this mode
         out = torch.empty_like(q)
         Z = torch.empty((N, H), dtype=torch.float32, device=q.device)
         ws = plan.workspace(H, d)
@@ -85,6 +90,8 @@ class SparseAttentionFunction(torch.autograd.Function):
         dbias = None
         if ctx.has_bias and ctx.needs_input_grad[3]:
             dbias = torch.empty_like(edge_bias)
+            if ctx.mode & _lib.BIAS_BOTH_ORDERS:
+                dbias[plan.num_edges:].zero_()      # the source-sorted copy gets no gradient of its own
         ws = plan.workspace(H, d)
         with torch.cuda.device(q.device):
             stream = torch.cuda.current_stream(q.device).cuda_stream
@@ -199,7 +206,8 @@ def _plan_order_bias(module, attn_bias, edge_index, plan, dtype):
     else:
         if isinstance(edge_index, GraphPlan):
             raise ValueError("a dense attn_bias needs the edge_index tensor (not a prebuilt plan)")
-        eb = gather_dense_bias(attn_bias, edge_index.index_select(1, plan.edge_order()), module.dense_bias_layout)
+        both = torch.cat([plan.edge_order(), plan.edge_order_src()])       # destination-sorted rows, then source-sorted
+        eb = gather_dense_bias(attn_bias, edge_index.index_select(1, both), module.dense_bias_layout)
         if eb.shape[-1] == 1:
             eb = eb.squeeze(-1)
         eb = eb.to(dtype)

@@ -515,16 +515,16 @@ int tgt_plan_export(const tgt_plan_t* plan, int which, int32_t* h_out, int64_t c
     return TGT_OK;
 }
 
-int tgt_plan_sort_rows(const tgt_plan_t* plan, const void* d_in, int row_bytes, void* d_out, int inverse, void* stream) {
-    if (!plan || row_bytes < 1 || (plan->E > 0 && (!d_in || !d_out))) {
+int tgt_plan_sort_rows(const tgt_plan_t* plan, const void* d_in, int row_bytes, void* d_out, int direction, void* stream) {
+    if (!plan || row_bytes < 1 || direction < 0 || direction > 2 || (plan->E > 0 && (!d_in || !d_out))) {
         tgt::set_error("tgt_plan_sort_rows: null pointer or bad row size");
         return TGT_ERR_INVALID_ARG;
     }
     if (plan->E == 0) return TGT_OK;
     hipStream_t st = (hipStream_t)stream;
     const int64_t E = plan->E;
-    const int32_t* eid = plan->dst.eid;
-    const bool inv = inverse != 0;
+    const int32_t* eid = direction == 2 ? plan->src.eid : plan->dst.eid;
+    const bool inv = direction == 1;
 #define TGT_LAUNCH_PERMUTE(V)                                                                                  \
     do {                                                                                                       \
         const int nv = row_bytes / (int)sizeof(V);                                                             \
@@ -539,6 +539,15 @@ int tgt_plan_sort_rows(const tgt_plan_t* plan, const void* d_in, int row_bytes, 
     else if (al % 2 == 0) TGT_LAUNCH_PERMUTE(uint16_t);
     else TGT_LAUNCH_PERMUTE(uint8_t);
 #undef TGT_LAUNCH_PERMUTE
+    TGT_HIP_CHECK(hipGetLastError());
+    return TGT_OK;
+}
+
+int tgt_plan_edge_order_src(const tgt_plan_t* plan, int64_t* d_out, void* stream) {
+    if (!plan || (plan->E > 0 && !d_out)) { tgt::set_error("tgt_plan_edge_order_src: null pointer"); return TGT_ERR_INVALID_ARG; }
+    if (plan->E == 0) return TGT_OK;
+    hipLaunchKernelGGL(tgt::k_widen, dim3((unsigned)((plan->E + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       plan->src.eid, plan->E, d_out);
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
 }

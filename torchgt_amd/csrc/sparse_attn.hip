@@ -138,6 +138,7 @@ struct Common {
     const void* v;
     const void* g;        // dout (backward)
     const void* bias;
+    const void* bias_src; // the bias as the walk by source reads it (same array, or its source-sorted copy)
     const float2* nd;     // [N, H] (1/(Z+eps), D) (backward)
     int32_t bias_mode;
     int32_t bias_se, bias_sh;   // element strides of the bias per edge / per head: (H, 1) or (1, 0)
@@ -200,7 +201,7 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
     const T* __restrict__ K = static_cast<const T*>(c.k);
     const T* __restrict__ V = static_cast<const T*>(c.v);
     const T* __restrict__ Gd = static_cast<const T*>(c.g);
-    const T* __restrict__ B = static_cast<const T*>(c.bias);
+    const T* __restrict__ B = static_cast<const T*>(MODE == MODE_BWD_SRC ? c.bias_src : c.bias);
     const int64_t row_off = (int64_t)row * HD + el * 8;
 
     float r0[8], r1[8];      // row-resident: fwd q | bwd_dst q, g | bwd_src k, v
@@ -601,29 +602,29 @@ __global__ __launch_bounds__(kBlock, 4) void k_attn_bwd(const Common c, const Si
     int b = blockIdx.x;
     if (b < pad_d) {
         if (b < sd.spread_pad) {
-            if (b < sd.n_spread) block_item<T, LPE, LPH, MODE_BWD_DST, HASB, TILES>(c, sd, b, lds);
+            if (b < sd.n_spread) block_item<T, LPE, LPH, MODE_BWD_DST, (HASB == 3 ? 2 : HASB), TILES>(c, sd, b, lds);
         } else {
             const int bb = b - sd.spread_pad;
             const int it = sd.blk_chunk[bb & 7] + (bb >> 3);
-            if (it < sd.blk_chunk[(bb & 7) + 1]) block_item<T, LPE, LPH, MODE_BWD_DST, HASB, TILES>(c, sd, it, lds);
+            if (it < sd.blk_chunk[(bb & 7) + 1]) block_item<T, LPE, LPH, MODE_BWD_DST, (HASB == 3 ? 2 : HASB), TILES>(c, sd, it, lds);
         }
         return;
     }
     b -= pad_d;
     if (b < pad_s) {
         if (b < ss.spread_pad) {
-            if (b < ss.n_spread) block_item<T, LPE, LPH, MODE_BWD_SRC, (HASB ? 1 : 0), TILES>(c, ss, b, lds);
+            if (b < ss.n_spread) block_item<T, LPE, LPH, MODE_BWD_SRC, (HASB == 3 ? 2 : (HASB ? 1 : 0)), TILES>(c, ss, b, lds);
         } else {
             const int bb = b - ss.spread_pad;
             const int it = ss.blk_chunk[bb & 7] + (bb >> 3);
-            if (it < ss.blk_chunk[(bb & 7) + 1]) block_item<T, LPE, LPH, MODE_BWD_SRC, (HASB ? 1 : 0), TILES>(c, ss, it, lds);
+            if (it < ss.blk_chunk[(bb & 7) + 1]) block_item<T, LPE, LPH, MODE_BWD_SRC, (HASB == 3 ? 2 : (HASB ? 1 : 0)), TILES>(c, ss, it, lds);
         }
         return;
     }
     b -= pad_s;
-    if (b < sd.n_wave_blocks) { wave_block<T, LPE, LPH, MODE_BWD_DST, HASB, TILES>(c, sd, b); return; }
+    if (b < sd.n_wave_blocks) { wave_block<T, LPE, LPH, MODE_BWD_DST, (HASB == 3 ? 2 : HASB), TILES>(c, sd, b); return; }
     b -= sd.n_wave_blocks;
-    wave_block<T, LPE, LPH, MODE_BWD_SRC, (HASB ? 1 : 0), TILES>(c, ss, b);
+    wave_block<T, LPE, LPH, MODE_BWD_SRC, (HASB == 3 ? 2 : (HASB ? 1 : 0)), TILES>(c, ss, b);
 }
 
 // Per-node side vector of the backward: nd[i,h] = (1 / (Z[i,h] + eps), sum_c dout[i,h,c] out[i,h,c]).
@@ -722,7 +723,7 @@ template <typename T, int LPE, int LPH>
 static int run_fwd(const Call& c) {
     const WsLayout L = ws_layout(c.plan, c.H, c.d);
     Common cm{};
-    cm.q = c.q; cm.k = c.k; cm.v = c.v; cm.g = nullptr; cm.bias = c.bias; cm.nd = nullptr;
+    cm.q = c.q; cm.k = c.k; cm.v = c.v; cm.g = nullptr; cm.bias = c.bias; cm.bias_src = c.bias; cm.nd = nullptr;
     cm.bias_mode = c.bias_mode;
     cm.bias_se = (c.bias_mode & 0xf) == TGT_BIAS_EDGE_HEAD ? c.H : 1;
     cm.bias_sh = (c.bias_mode & 0xf) == TGT_BIAS_EDGE_HEAD ? 1 : 0;
@@ -779,6 +780,11 @@ static int run_bwd(const Call& c) {
     if (c.only_node_side) return TGT_OK;
     Common cm{};
     cm.q = c.q; cm.k = c.k; cm.v = c.v; cm.g = c.dout; cm.bias = c.bias; cm.nd = nd;
+    const bool both_orders = (c.bias_mode & TGT_BIAS_BOTH_ORDERS) != 0;
+    // two copies: rows [0, E) destination-sorted, rows [E, 2E) source-sorted
+    cm.bias_src = both_orders ? static_cast<const char*>(c.bias) +
+                                    (size_t)c.plan->E * ((c.bias_mode & 0xf) == TGT_BIAS_EDGE_HEAD ? c.H : 1) * sizeof(T)
+                              : c.bias;
     cm.bias_mode = c.bias_mode;
     cm.bias_se = (c.bias_mode & 0xf) == TGT_BIAS_EDGE_HEAD ? c.H : 1;
     cm.bias_sh = (c.bias_mode & 0xf) == TGT_BIAS_EDGE_HEAD ? 1 : 0;
@@ -793,6 +799,7 @@ static int run_bwd(const Call& c) {
     sd.counters = counters + c.plan->dst.n_split;
     fill_side(ss, c.plan->src, LPE);
     if (c.bias_mode & TGT_BIAS_PLAN_ORDER) ss.eid = c.plan->src.pos;    // source-sorted -> destination-sorted position
+    if (c.bias_mode & TGT_BIAS_BOTH_ORDERS) ss.eid = nullptr;           // its own source-sorted copy
     ss.out0 = c.dk; ss.out1 = c.dv; ss.Z = nullptr;
     if (c.init) { ss.init0 = c.init->dk; ss.init1 = c.init->dv; ss.cover = c.init->cover_src; }
     ss.part = reinterpret_cast<float*>(c.ws + L.dkv_part);
@@ -814,6 +821,8 @@ static int run_bwd(const Call& c) {
                 set_error("block attention: no kernel for this (H, d)");
                 return TGT_ERR_UNSUPPORTED;
             }
+        } else if (hb && (c.bias_mode & TGT_BIAS_BOTH_ORDERS)) {
+            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, 3, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
         } else if (hb && (c.bias_mode & TGT_BIAS_PLAN_ORDER)) {
             hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, 2, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
         } else if (hb) {
@@ -853,12 +862,13 @@ static int check_common(const tgt_plan* plan, const void* q, const void* k, cons
     if (!plan || !q || !k || !v) { set_error("null plan or q/k/v"); return TGT_ERR_INVALID_ARG; }
     {
         const int base = bias_mode & 0xf;
-        if (bias_mode < 0 || (bias_mode & ~(0xf | TGT_BIAS_PLAN_ORDER)) || base > TGT_BIAS_EDGE ||
-            (base == TGT_BIAS_NONE && bias_mode != TGT_BIAS_NONE)) {
+        if (bias_mode < 0 || (bias_mode & ~(0xf | TGT_BIAS_PLAN_ORDER | TGT_BIAS_BOTH_ORDERS)) || base > TGT_BIAS_EDGE ||
+            (base == TGT_BIAS_NONE && bias_mode != TGT_BIAS_NONE) ||
+            ((bias_mode & TGT_BIAS_BOTH_ORDERS) && !(bias_mode & TGT_BIAS_PLAN_ORDER))) {
             set_error("bad bias_mode %d", bias_mode);
             return TGT_ERR_INVALID_ARG;
         }
-        if ((bias_mode & TGT_BIAS_PLAN_ORDER) && !plan->src.pos) {
+        if ((bias_mode & TGT_BIAS_PLAN_ORDER) && !(bias_mode & TGT_BIAS_BOTH_ORDERS) && !plan->src.pos) {
             set_error("TGT_BIAS_PLAN_ORDER needs tgt_plan_enable_bias_order(plan) first");
             return TGT_ERR_INVALID_ARG;
         }

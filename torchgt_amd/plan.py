@@ -77,7 +77,7 @@ class GraphPlan:
     def edge_order(self):
         """int64 [E] on the GPU: the caller's index of every edge in the plan's destination-sorted (stable)
         order.  ``bias[plan.edge_order()]`` is a bias in plan order (see ``sort_bias``).  Also builds, once,
-        the map the walk by source needs for such a bias."""
+        the map the walk by source needs for a bias that is given in that order only."""
         if getattr(self, "_edge_order", None) is None:
             L = _lib.lib()
             out = torch.empty(self.num_edges, dtype=torch.int64, device=self.device)
@@ -88,24 +88,37 @@ class GraphPlan:
             self._edge_order = out
         return self._edge_order
 
-    def sort_bias(self, edge_bias):
-        """A per-edge bias ([E] or [E, H], caller's edge order) in plan order, for
-        ``sparse_attention(..., bias_in_plan_order=True)``.  Differentiable: the gradient comes back in the
-        caller's order.  Permute a bias that several layers share once and pass the result to all of them: the
-        destination walks then stream it instead of gathering 16/32-byte pieces through the edge permutation."""
-        return _SortRows.apply(edge_bias, self)
+    def edge_order_src(self):
+        """The same for the source-sorted order (the walk by source of the backward)."""
+        if getattr(self, "_edge_order_src", None) is None:
+            out = torch.empty(self.num_edges, dtype=torch.int64, device=self.device)
+            with torch.cuda.device(self.device):
+                _lib.check(_lib.lib().tgt_plan_edge_order_src(self.handle, out.data_ptr() if self.num_edges else None,
+                                                              torch.cuda.current_stream(self.device).cuda_stream))
+            self._edge_order_src = out
+        return self._edge_order_src
 
-    def _permute(self, t, inverse):
-        self.edge_order()
+    def sort_bias(self, edge_bias, both_orders=True):
+        """A per-edge bias ([E] or [E, H], caller's edge order) in plan order, for
+        ``sparse_attention(..., bias_in_plan_order=True)``.  With ``both_orders`` the result has 2 E rows: the
+        destination-sorted copy, then the source-sorted one, so that no walk has to gather the bias.
+        Differentiable: the gradient comes back in the caller's order.  Permute a bias that several layers share
+        once and pass the result to all of them."""
+        return _SortRows.apply(edge_bias, self, both_orders)
+
+    def _permute(self, t, direction, out=None):
+        """direction 0: caller's -> destination-sorted; 1: back; 2: caller's -> source-sorted."""
+        if direction != 2:
+            self.edge_order()
         t = t.contiguous()
         if t.shape[0] != self.num_edges:
             raise ValueError(f"expected {self.num_edges} rows, got {t.shape[0]}")
-        out = torch.empty_like(t)
+        if out is None:
+            out = torch.empty_like(t)
         if self.num_edges:
             row_bytes = t.element_size() * (t.numel() // self.num_edges)
             with torch.cuda.device(self.device):
-                _lib.check(_lib.lib().tgt_plan_sort_rows(self.handle, t.data_ptr(), row_bytes, out.data_ptr(),
-                                                         1 if inverse else 0,
+                _lib.check(_lib.lib().tgt_plan_sort_rows(self.handle, t.data_ptr(), row_bytes, out.data_ptr(), int(direction),
                                                          torch.cuda.current_stream(self.device).cuda_stream))
         return out
 
@@ -124,16 +137,24 @@ class GraphPlan:
 
 
 class _SortRows(torch.autograd.Function):
-    """bias in plan order; the gradient is carried back to the caller's order."""
+    """bias in plan order (one or both copies); the gradient is carried back to the caller's order."""
 
     @staticmethod
-    def forward(ctx, t, plan):
+    def forward(ctx, t, plan, both):
         ctx.plan = plan
-        return plan._permute(t, inverse=False)
+        E = plan.num_edges
+        if not both:
+            return plan._permute(t, 0)
+        t = t.contiguous()
+        out = torch.empty((2 * E,) + tuple(t.shape[1:]), dtype=t.dtype, device=t.device)
+        plan._permute(t, 0, out=out[:E])
+        plan._permute(t, 2, out=out[E:])
+        return out
 
     @staticmethod
     def backward(ctx, g):
-        return ctx.plan._permute(g, inverse=True), None
+        E = ctx.plan.num_edges
+        return ctx.plan._permute(g[:E], 1), None, None     # only the destination-sorted rows carry a gradient
 
 
 _CACHE = collections.OrderedDict()
