@@ -29,19 +29,36 @@ def sources():
     return sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
-def _compile(src):
-    obj = os.path.join(OBJ_DIR, src[:-4] + ".o")
-    cmd = [HIPCC] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+# sources compiled as several translation units (-D<macro>=k, k < parts), in parallel: their
+# kernels take minutes to compile in one piece
+SPLIT = {"sparse_attn.hip": ("TGT_SPARSE_PART", 4)}
+
+
+def _jobs():
+    jobs = []
+    for src in sources():
+        if src in SPLIT:
+            macro, parts = SPLIT[src]
+            jobs += [(src, f"{src[:-4]}_p{k}.o", [f"-D{macro}={k}"]) for k in range(parts)]
+        else:
+            jobs.append((src, src[:-4] + ".o", []))
+    return jobs
+
+
+def _compile(job):
+    src, obj_name, extra = job
+    obj = os.path.join(OBJ_DIR, obj_name)
+    cmd = [HIPCC] + FLAGS + extra + ["-c", os.path.join(CSRC, src), "-o", obj]
     t0 = time.time()
     r = subprocess.run(cmd, capture_output=True, text=True)
-    return src, obj, r.returncode, r.stdout + r.stderr, time.time() - t0
+    return src + (" " + " ".join(extra) if extra else ""), obj, r.returncode, r.stdout + r.stderr, time.time() - t0
 
 
 def build(verbose=True):
     os.makedirs(OBJ_DIR, exist_ok=True)
-    srcs = sources()
-    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
-        results = list(ex.map(_compile, srcs))
+    jobs = sorted(_jobs(), key=lambda j: j[0] not in SPLIT)      # the long ones first
+    with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as ex:
+        results = list(ex.map(_compile, jobs))
     objs = []
     for src, obj, rc, log, dt in results:
         noise = "unknown target feature"   # harmless host-pass note about -packed-fp32-ops

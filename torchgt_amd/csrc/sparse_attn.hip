@@ -835,22 +835,71 @@ static int run_bwd(const Call& c) {
     return TGT_OK;
 }
 
+// The kernels of one (lanes per edge, lanes per head) shape take minutes to compile, so this file can be
+// compiled as several translation units: -DTGT_SPARSE_PART=k (k = 0..3) emits the shapes of part k only, and
+// part 0 also holds the entry points.  Without the macro one translation unit holds everything.
+template <typename T, int LPE, int LPH> int run_shape(const Call& c, bool bwd);
+#define TGT_DECLARE_SHAPE(LPE_, LPH_)                                      \
+    template <> int run_shape<float, LPE_, LPH_>(const Call& c, bool bwd); \
+    template <> int run_shape<bf16_t, LPE_, LPH_>(const Call& c, bool bwd);
+#define TGT_DEFINE_SHAPE(LPE_, LPH_)                                                        \
+    template <> int run_shape<float, LPE_, LPH_>(const Call& c, bool bwd) {                 \
+        return bwd ? run_bwd<float, LPE_, LPH_>(c) : run_fwd<float, LPE_, LPH_>(c);         \
+    }                                                                                       \
+    template <> int run_shape<bf16_t, LPE_, LPH_>(const Call& c, bool bwd) {                \
+        return bwd ? run_bwd<bf16_t, LPE_, LPH_>(c) : run_fwd<bf16_t, LPE_, LPH_>(c);       \
+    }
+TGT_DECLARE_SHAPE(8, 1)    // H=8  d=8   (Graphormer-Slim / GT node level, hidden 64)
+#ifndef TGT_ONLY_8x8       // -DTGT_ONLY_8x8: compile one shape only (quick experiments)
+TGT_DECLARE_SHAPE(8, 2)    // H=4  d=16  (attention micro-benchmark, attn_module.py:387)
+TGT_DECLARE_SHAPE(16, 2)   // H=8  d=16  (hidden 128, the parser default)
+TGT_DECLARE_SHAPE(16, 1)   // H=16 d=8
+TGT_DECLARE_SHAPE(4, 1)    // H=4  d=8
+TGT_DECLARE_SHAPE(2, 1)    // H=2  d=8
+TGT_DECLARE_SHAPE(1, 1)    // H=1  d=8
+TGT_DECLARE_SHAPE(4, 2)    // H=2  d=16
+TGT_DECLARE_SHAPE(2, 2)    // H=1  d=16
+#endif
+#if !defined(TGT_SPARSE_PART) || TGT_SPARSE_PART == 0
+TGT_DEFINE_SHAPE(8, 1)
+#ifndef TGT_ONLY_8x8
+TGT_DEFINE_SHAPE(1, 1)
+#endif
+#endif
+#ifndef TGT_ONLY_8x8
+#if !defined(TGT_SPARSE_PART) || TGT_SPARSE_PART == 1
+TGT_DEFINE_SHAPE(8, 2)
+TGT_DEFINE_SHAPE(4, 2)
+#endif
+#if !defined(TGT_SPARSE_PART) || TGT_SPARSE_PART == 2
+TGT_DEFINE_SHAPE(16, 2)
+TGT_DEFINE_SHAPE(2, 2)
+#endif
+#if !defined(TGT_SPARSE_PART) || TGT_SPARSE_PART == 3
+TGT_DEFINE_SHAPE(2, 1)
+TGT_DEFINE_SHAPE(16, 1)
+TGT_DEFINE_SHAPE(4, 1)
+#endif
+#endif
+#undef TGT_DECLARE_SHAPE
+#undef TGT_DEFINE_SHAPE
+
+#if !defined(TGT_SPARSE_PART) || TGT_SPARSE_PART == 0
 template <typename T>
 static int dispatch(const Call& c, bool bwd) {
     const int lph = c.d / 8, lpe = c.H * c.d / 8;
-#define TGT_CASE(LPE_, LPH_)                                                   \
-    if (lpe == LPE_ && lph == LPH_)                                            \
-        return bwd ? run_bwd<T, LPE_, LPH_>(c) : run_fwd<T, LPE_, LPH_>(c);
-    TGT_CASE(8, 1)    // H=8  d=8   (Graphormer-Slim / GT node level, hidden 64)
-#ifndef TGT_ONLY_8x8   // -DTGT_ONLY_8x8: compile one shape only (quick experiments)
-    TGT_CASE(8, 2)    // H=4  d=16  (attention micro-benchmark, attn_module.py:387)
-    TGT_CASE(16, 2)   // H=8  d=16  (hidden 128, the parser default)
-    TGT_CASE(16, 1)   // H=16 d=8
-    TGT_CASE(4, 1)    // H=4  d=8
-    TGT_CASE(2, 1)    // H=2  d=8
-    TGT_CASE(1, 1)    // H=1  d=8
-    TGT_CASE(4, 2)    // H=2  d=16
-    TGT_CASE(2, 2)    // H=1  d=16
+#define TGT_CASE(LPE_, LPH_) \
+    if (lpe == LPE_ && lph == LPH_) return run_shape<T, LPE_, LPH_>(c, bwd);
+    TGT_CASE(8, 1)
+#ifndef TGT_ONLY_8x8
+    TGT_CASE(8, 2)
+    TGT_CASE(16, 2)
+    TGT_CASE(16, 1)
+    TGT_CASE(4, 1)
+    TGT_CASE(2, 1)
+    TGT_CASE(1, 1)
+    TGT_CASE(4, 2)
+    TGT_CASE(2, 2)
 #endif
 #undef TGT_CASE
     set_error("no kernel for H=%d d=%d (d must be 8 or 16 and H*d/8 one of 1,2,4,8,16)", c.H, c.d);
@@ -932,9 +981,11 @@ int sparse_attn_node_side(const tgt_plan_t* plan, int H, int d, int dtype, const
 }
 
 const float2* sparse_attn_nd_ptr(void* d_workspace) { return reinterpret_cast<const float2*>(d_workspace); }
+#endif  // part 0: dispatch and entry points
 
 }  // namespace tgt
 
+#if !defined(TGT_SPARSE_PART) || TGT_SPARSE_PART == 0
 extern "C" {
 
 int64_t tgt_sparse_attn_workspace_bytes(const tgt_plan_t* plan, int H, int d) {
@@ -958,3 +1009,4 @@ int tgt_sparse_attn_bwd(const tgt_plan_t* plan, const void* d_q, const void* d_k
 }
 
 }  // extern "C"
+#endif  // part 0: C entry points
