@@ -471,8 +471,8 @@ __device__ __forceinline__ bool sub_item(const int64_t* __restrict__ ei, int64_t
 template <int PASS>
 __global__ __launch_bounds__(256) void k_sub_compact(const int64_t* __restrict__ ei, int64_t E, int64_t N,
                                                      const int32_t* __restrict__ pos, uint32_t* __restrict__ counts,
-                                                     int64_t* __restrict__ out, int64_t capacity,
-                                                     int* __restrict__ bad) {
+                                                     uint64_t* __restrict__ keep_bits, int64_t* __restrict__ out,
+                                                     int64_t capacity, int* __restrict__ bad) {
     __shared__ uint32_t wave_n[4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t total = E + N;
@@ -480,8 +480,20 @@ __global__ __launch_bounds__(256) void k_sub_compact(const int64_t* __restrict__
     for (int round = 0; round < kSubItems / 256; ++round) {
         const int64_t i = (int64_t)blockIdx.x * kSubItems + round * 256 + threadIdx.x;
         int32_t a = 0, b = 0;
-        const bool keep = i < total && sub_item(ei, E, N, pos, i, a, b, bad);
-        const uint64_t m = __ballot(keep);
+        // one keep bit per item, a 64-bit word per wave and round: the writing pass reads the words and
+        // looks at the endpoints of the kept items only (a few per cent of the edge list)
+        const int64_t word = ((int64_t)blockIdx.x * (kSubItems / 256) + round) * 4 + wave;
+        bool keep;
+        uint64_t m;
+        if (PASS == 0) {
+            keep = i < total && sub_item(ei, E, N, pos, i, a, b, bad);
+            m = __ballot(keep);
+            if (lane == 0) keep_bits[word] = m;
+        } else {
+            m = keep_bits[word];
+            keep = (m >> lane) & 1ull;
+            if (keep) (void)sub_item(ei, E, N, pos, i, a, b, bad);
+        }
         if (lane == 0) wave_n[wave] = (uint32_t)__popcll(m);
         __syncthreads();
         uint32_t before = 0, all = 0;
@@ -530,9 +542,10 @@ static int sub_edge_index_impl(const int64_t* d_ei, int64_t E, int64_t N, const 
                                int64_t* d_out, int64_t capacity, int64_t* h_num, hipStream_t st) {
     const int64_t total = E + N;
     const int nblocks = (int)((total + kSubItems - 1) / kSubItems);
-    DevBuf pos, counts, bad;
+    DevBuf pos, counts, bad, bits;
     TGT_HIP_CHECK(pos.alloc(sizeof(int32_t) * (size_t)N));
     TGT_HIP_CHECK(counts.alloc(sizeof(uint32_t) * (size_t)(nblocks + 1)));
+    TGT_HIP_CHECK(bits.alloc(sizeof(uint64_t) * (size_t)nblocks * (kSubItems / 64)));
     TGT_HIP_CHECK(bad.alloc(sizeof(int)));
     TGT_HIP_CHECK(hipMemsetAsync(bad.p, 0, sizeof(int), st));
     hipLaunchKernelGGL(k_sub_fill, dim3(nblk(N)), dim3(256), 0, st, pos.as<int32_t>(), N);
@@ -540,7 +553,7 @@ static int sub_edge_index_impl(const int64_t* d_ei, int64_t E, int64_t N, const 
         hipLaunchKernelGGL(k_sub_positions, dim3(nblk(S)), dim3(256), 0, st, d_idx, S, N, pos.as<int32_t>(),
                            bad.as<int>());
     hipLaunchKernelGGL((k_sub_compact<0>), dim3(nblocks), dim3(256), 0, st, d_ei, E, N, pos.as<int32_t>(),
-                       counts.as<uint32_t>(), (int64_t*)nullptr, (int64_t)0, bad.as<int>());
+                       counts.as<uint32_t>(), bits.as<uint64_t>(), (int64_t*)nullptr, (int64_t)0, bad.as<int>());
     hipLaunchKernelGGL(k_sub_scan, dim3(1), dim3(256), 0, st, counts.as<uint32_t>(), nblocks);
     TGT_HIP_CHECK(hipGetLastError());
     uint32_t n_keep = 0;
@@ -560,7 +573,7 @@ static int sub_edge_index_impl(const int64_t* d_ei, int64_t E, int64_t N, const 
     }
     if (n_keep > 0) {
         hipLaunchKernelGGL((k_sub_compact<1>), dim3(nblocks), dim3(256), 0, st, d_ei, E, N, pos.as<int32_t>(),
-                           counts.as<uint32_t>(), d_out, capacity, bad.as<int>());
+                           counts.as<uint32_t>(), bits.as<uint64_t>(), d_out, capacity, bad.as<int>());
         TGT_HIP_CHECK(hipGetLastError());
         TGT_HIP_CHECK(hipStreamSynchronize(st));      // the scratch buffers are freed on return
     }
