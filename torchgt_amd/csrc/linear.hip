@@ -18,7 +18,9 @@
 //                        panels and writes one partial; k_linear_gradw_reduce adds the
 //                        partials in a fixed order (no atomics: results are reproducible)
 // Matrix instructions: v_mfma_f32_32x32x2_f32 for float32 (exact fp32 products,
-// fp32 accumulation), v_mfma_f32_32x32x8_bf16_1k for bf16 (fp32 accumulation).
+// fp32 accumulation; the 64-wide forward instead splits every float into three
+// bf16 and uses the bf16 instructions, see k_linear64_split),
+// v_mfma_f32_32x32x8_bf16_1k for bf16 (fp32 accumulation).
 //   A 32xk : lane l holds A[l%32][k-slice of half l/32]
 //   B kx32 : lane l holds B[k-slice of half l/32][l%32]
 //   C 32x32: lane l, register r holds C[8*(r/4) + 4*(l/32) + r%4][l%32]
@@ -373,6 +375,150 @@ __global__ __launch_bounds__(kThreads) void k_linear64(LinArgs a) {
     }
 }
 
+// ---------------------------------------------------------------------------
+// float32 at the bf16 matrix rate.  A float is the exact sum of three bf16 numbers up to 2^-24 of
+// its size (hi = bf16(x), mid = bf16(x - hi), lo = bf16(x - hi - mid); the subtractions are exact),
+// so x * w = hi*hi + hi*mid + mid*hi + mid*mid + hi*lo + lo*hi + terms below 2^-24: six
+// v_mfma_f32_32x32x16_bf16 (fp32 accumulation) give the float32 product to a few 2^-23, and take 0.4 of
+// the time of the eight v_mfma_f32_32x32x2_f32 they replace (measured on this part: 16.8 ns against
+// 30.4 ns per instruction).  The weights are split once per workgroup into three bf16 planes in LDS;
+// the node rows stay float32 in LDS and are split in registers when a wave loads its operand rows.
+// ---------------------------------------------------------------------------
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ void split3(float x, __bf16& hi, __bf16& mid, __bf16& lo) {
+    hi = static_cast<__bf16>(x);
+    const float r1 = x - static_cast<float>(hi);
+    mid = static_cast<__bf16>(r1);
+    lo = static_cast<__bf16>(r1 - static_cast<float>(mid));
+}
+
+constexpr int kPlaneStride = 72;                       // bf16 per row of a weight plane (64 + 8 of padding)
+constexpr int kPlaneElems = 64 * kPlaneStride;
+
+struct Split32 { bf16x8_t hi[4], mid[4], lo[4]; };    // the 32 contraction indices of a lane's half row
+
+// row: 32 consecutive floats in LDS
+__device__ __forceinline__ void load_split(Split32& f, const float* row) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const float4 u0 = *reinterpret_cast<const float4*>(row + 8 * t);
+        const float4 u1 = *reinterpret_cast<const float4*>(row + 8 * t + 4);
+        const float v[8] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            __bf16 a, b, c;
+            split3(v[i], a, b, c);
+            f.hi[t][i] = a; f.mid[t][i] = b; f.lo[t][i] = c;
+        }
+    }
+}
+
+// acc += x_rows W_rows^T over the lane's 32 contraction indices; w: the lane's row in plane 0
+__device__ __forceinline__ void mma_split(const Split32& x, const __bf16* w, float16_t& acc) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const bf16x8_t wh = *reinterpret_cast<const bf16x8_t*>(w + 8 * t);
+        const bf16x8_t wm = *reinterpret_cast<const bf16x8_t*>(w + kPlaneElems + 8 * t);
+        const bf16x8_t wl = *reinterpret_cast<const bf16x8_t*>(w + 2 * kPlaneElems + 8 * t);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x.lo[t], wh, acc, 0, 0, 0);     // small terms first
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x.hi[t], wl, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x.mid[t], wm, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x.mid[t], wh, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x.hi[t], wm, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x.hi[t], wh, acc, 0, 0, 0);
+    }
+}
+
+// Same walk as k_linear64 (64 -> 64 features, weights resident, 64-row panels, register prefetch) for float32
+// through the split.  Weight planes in LDS: [NW][3][64][kPlaneStride] bf16; node rows: [NA][64][68] float.
+template <bool DX, int NW>
+__global__ __launch_bounds__(kThreads) void k_linear64_split(LinArgs a) {
+    constexpr int S = lds_stride<float>(64);
+    constexpr int NA = DX ? NW : 1;
+    constexpr int NO = DX ? 1 : NW;
+    extern __shared__ __align__(16) unsigned char smem[];
+    __bf16* tW = reinterpret_cast<__bf16*>(smem);
+    float* tA = reinterpret_cast<float*>(smem + (size_t)NW * 3 * kPlaneElems * sizeof(__bf16));
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, h = lane >> 5;
+    const int rb = wave >> 1, cb = wave & 1;
+    const int64_t n_panels = (a.N + 63) / 64;
+    TileRegs<float> next[NA];
+    int64_t p = blockIdx.x;
+    if (p < n_panels) {
+#pragma unroll
+        for (int s = 0; s < NA; ++s) tile_fetch(next[s], reinterpret_cast<const float*>(a.A[s]), p * 64, a.N);
+    }
+    {   // weights: 16 elements per thread and weight, split into the three planes
+        uint4 raw[NW][4];
+#pragma unroll
+        for (int j = 0; j < NW; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int v = threadIdx.x + i * kThreads;                       // 16-byte piece: row v / 16, columns 4 (v % 16) ..
+                raw[j][i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const float*>(a.W[j]) + v * 4);
+            }
+#pragma unroll
+        for (int j = 0; j < NW; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int v = threadIdx.x + i * kThreads, r = v >> 4, c = (v & 15) * 4;
+                const float* e = reinterpret_cast<const float*>(&raw[j][i]);
+                __bf16* plane = tW + (size_t)j * 3 * kPlaneElems;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    __bf16 x0, x1, x2;
+                    split3(e[t], x0, x1, x2);
+                    // forward: plane row = output column r, contraction index c + t; input gradient: row = c + t, index r
+                    const int at = DX ? (c + t) * kPlaneStride + r : r * kPlaneStride + c + t;
+                    plane[at] = x0;
+                    plane[kPlaneElems + at] = x1;
+                    plane[2 * kPlaneElems + at] = x2;
+                }
+            }
+    }
+    float bv[NO];
+#pragma unroll
+    for (int o = 0; o < NO; ++o) {
+        const float* bias = DX ? nullptr : reinterpret_cast<const float*>(a.bias[o]);
+        bv[o] = bias ? bias[32 * cb + l32] : 0.f;
+    }
+#pragma unroll
+    for (int o = 0; o < NO; ++o) asm volatile("" ::"v"(bv[o]));      // wait for the bias loads here, not in the loop
+    for (; p < n_panels; p += gridDim.x) {
+        __syncthreads();
+#pragma unroll
+        for (int s = 0; s < NA; ++s) tile_put<float, S>(next[s], tA + s * 64 * S);
+        __syncthreads();
+        if (p + gridDim.x < n_panels) {
+#pragma unroll
+            for (int s = 0; s < NA; ++s)
+                tile_fetch(next[s], reinterpret_cast<const float*>(a.A[s]), (p + gridDim.x) * 64, a.N);
+        }
+        if (!DX) {
+            Split32 x;
+            load_split(x, tA + (32 * rb + l32) * S + h * 32);
+#pragma unroll
+            for (int o = 0; o < NW; ++o) {
+                float16_t acc = zero16();
+                mma_split(x, tW + (size_t)o * 3 * kPlaneElems + (32 * cb + l32) * kPlaneStride + h * 32, acc);
+                float* out = reinterpret_cast<float*>(a.out[o]) + (p * 64 + 32 * rb + 4 * h) * 64 + 32 * cb + l32;
+                store_rows<float>(out, 64, acc, bv[o], a.N - (p * 64 + 32 * rb + 4 * h));
+            }
+        } else {
+            float16_t acc = zero16();
+#pragma unroll
+            for (int s = 0; s < NW; ++s) {
+                Split32 x;
+                load_split(x, tA + (s * 64 + 32 * rb + l32) * S + h * 32);
+                mma_split(x, tW + (size_t)s * 3 * kPlaneElems + (32 * cb + l32) * kPlaneStride + h * 32, acc);
+            }
+            float* out = reinterpret_cast<float*>(a.out[0]) + (p * 64 + 32 * rb + 4 * h) * 64 + 32 * cb + l32;
+            store_rows<float>(out, 64, acc, 0.f, a.N - (p * 64 + 32 * rb + 4 * h));
+        }
+    }
+}
+
 int num_cus() {
     static int cus = 0;
     if (cus == 0) {
@@ -389,17 +535,24 @@ int num_cus() {
 template <typename T, bool DX, int NW>
 int launch_linear64(const LinArgs& a, hipStream_t st) {
     constexpr int NA = DX ? NW : 1;
-    const size_t lds = sizeof(T) * (size_t)(NW + NA) * 64 * lds_stride<T>(64);
+    // float32 forward goes through the three-way bf16 split.  The input gradient keeps the float32 matrix
+    // instructions: it would split three source tiles per panel and stage transposed weight planes, and measured
+    // slower at 64 K rows (28 against 26 us) though faster at 870 K (280 against 297 us).
+    constexpr bool kSplit = sizeof(T) == 4 && !DX;
+    const size_t lds = kSplit ? (size_t)NW * 3 * kPlaneElems * 2 + sizeof(float) * (size_t)NA * 64 * lds_stride<float>(64)
+                              : sizeof(T) * (size_t)(NW + NA) * 64 * lds_stride<T>(64);
+    const void* fn = kSplit ? reinterpret_cast<const void*>(&k_linear64_split<DX, NW>)
+                            : reinterpret_cast<const void*>(&k_linear64<T, DX, NW>);
     static bool raised = false;
     if (!raised && lds > 48 * 1024) {
-        TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_linear64<T, DX, NW>),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        TGT_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         raised = true;
     }
     const int64_t n_panels = (a.N + 63) / 64;
-    const int per_cu = (int)std::max<size_t>(1, std::min<size_t>(4, (size_t)(150 * 1024) / lds));
+    const int per_cu = (int)std::max<size_t>(1, std::min<size_t>(4, (size_t)(160 * 1024) / lds));
     const unsigned grid = (unsigned)std::min<int64_t>(n_panels, (int64_t)num_cus() * per_cu);
-    hipLaunchKernelGGL((k_linear64<T, DX, NW>), dim3(grid), dim3(kThreads), lds, st, a);
+    if (kSplit) hipLaunchKernelGGL((k_linear64_split<DX, NW>), dim3(grid), dim3(kThreads), lds, st, a);
+    else hipLaunchKernelGGL((k_linear64<T, DX, NW>), dim3(grid), dim3(kThreads), lds, st, a);
     return TGT_OK;
 }
 
