@@ -74,6 +74,29 @@ __device__ __forceinline__ void unpack(const Raw8<bf16_t>& r, float (&x)[8]) {
     x[4] = bf16_to_f32(r.u.z & 0xffffu); x[5] = __uint_as_float(r.u.z & 0xffff0000u);
     x[6] = bf16_to_f32(r.u.w & 0xffffu); x[7] = __uint_as_float(r.u.w & 0xffff0000u);
 }
+__device__ __forceinline__ void zero_raw(Raw8<float>& r) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r.x[i] = 0.f;
+}
+__device__ __forceinline__ void zero_raw(Raw8<bf16_t>& r) { r.u = make_uint4(0u, 0u, 0u, 0u); }
+// Dot product of two chunks as they arrived.  bf16 pairs go through v_dot2_f32_bf16 (exact products,
+// fp32 sum): four instructions and no conversion of either operand.
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c, false);
+}
+__device__ __forceinline__ float dot_raw(const Raw8<float>& a, const Raw8<float>& b) {
+    float s = a.x[0] * b.x[0];
+#pragma unroll
+    for (int c = 1; c < 8; ++c) s = fmaf(a.x[c], b.x[c], s);
+    return s;
+}
+__device__ __forceinline__ float dot_raw(const Raw8<bf16_t>& a, const Raw8<bf16_t>& b) {
+    float s = dot2_bf16(a.u.x, b.u.x, 0.f);
+    s = dot2_bf16(a.u.y, b.u.y, s);
+    s = dot2_bf16(a.u.z, b.u.z, s);
+    return dot2_bf16(a.u.w, b.u.w, s);
+}
 __device__ __forceinline__ float raw1(const float* p) { return *p; }
 __device__ __forceinline__ uint32_t raw1(const bf16_t* p) { return p->x; }
 __device__ __forceinline__ float cvt1(float x) { return x; }
@@ -204,22 +227,23 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
     const T* __restrict__ B = static_cast<const T*>(MODE == MODE_BWD_SRC ? c.bias_src : c.bias);
     const int64_t row_off = (int64_t)row * HD + el * 8;
 
-    float r0[8], r1[8];      // row-resident: fwd q | bwd_dst q, g | bwd_src k, v
+    Raw8<T> r0, r1;          // row-resident, as loaded (only dot products use them): fwd q | bwd_dst q, g | bwd_src k, v
     float rz = 0.f, Dh = 0.f;
+    zero_raw(r0); zero_raw(r1);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) { r0[i] = 0.f; r1[i] = 0.f; acc.a0[i] = 0.f; acc.a1[i] = 0.f; }
+    for (int i = 0; i < 8; ++i) { acc.a0[i] = 0.f; acc.a1[i] = 0.f; }
     acc.z = 0.f;
     if (valid) {
         if (MODE == MODE_FWD) {
-            load8(Q + row_off, r0);
+            load_raw(Q + row_off, r0);
         } else if (MODE == MODE_BWD_DST) {
-            load8(Q + row_off, r0);
-            load8(Gd + row_off, r1);
+            load_raw(Q + row_off, r0);
+            load_raw(Gd + row_off, r1);
             const float2 nd = c.nd[(int64_t)row * H + head];
             rz = nd.x; Dh = nd.y;
         } else {
-            load8(K + row_off, r0);
-            load8(V + row_off, r1);
+            load_raw(K + row_off, r0);
+            load_raw(V + row_off, r1);
         }
     }
     const int32_t* __restrict__ col = s.col + start;
@@ -303,7 +327,7 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
                 const float bbu = HASB ? cvt1(braw[u]) : 0.f;
                 // raw score: identical arithmetic in all three walks so that the
                 // recomputed weights and the clamp mask agree bit for bit
-                const float raw = head_sum<LPH>(dot8(r0, x0)) * inv_scale;
+                const float raw = head_sum<LPH>(dot_raw(r0, g0[u])) * inv_scale;
                 const float w = __expf(clamp5(raw) + bbu);
                 if (MODE == MODE_FWD) {
                     acc.z += w;
@@ -312,7 +336,7 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
                 } else {
                     const bool inside = (raw >= -5.0f) & (raw <= 5.0f);   // torch clamp backward: inclusive
                     if (MODE == MODE_BWD_DST) {
-                        const float t = head_sum<LPH>(dot8(r1, x1));   // g_dst . v_src
+                        const float t = head_sum<LPH>(dot_raw(r1, g1[u]));   // g_dst . v_src
                         const float dS = w * rz * (t - Dh);
                         T* __restrict__ dB = static_cast<T*>(s.out1);
                         if (HASB && dB != nullptr) {
@@ -330,7 +354,7 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
                         for (int i = 0; i < 8; ++i) acc.a0[i] = fmaf(md, x0[i], acc.a0[i]);
                     } else {
                         const float p = w * ndv[u].x;
-                        const float t = head_sum<LPH>(dot8(x1, r1));   // g_dst . v_src
+                        const float t = head_sum<LPH>(dot_raw(g1[u], r1));   // g_dst . v_src
                         const float dS = p * (t - ndv[u].y);
                         const float md = inside ? dS : 0.f;
 #pragma unroll
