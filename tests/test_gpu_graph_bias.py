@@ -67,10 +67,13 @@ def test_floyd_warshall_rejects_large_graphs(cuda):
     assert ei.value.code == _lib.ERR_UNSUPPORTED
 
 
+# (heads, edge features): every kernel variant -- eight heads with one feature, with up to four, with more (several
+# passes over the features); more than eight heads (several passes over the heads); fewer than eight
+@pytest.mark.parametrize("H,F", [(8, 3), (8, 1), (8, 6), (16, 2), (4, 1)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_graph_attn_bias_matches_oracle(cuda, dtype):
+def test_graph_attn_bias_matches_oracle(cuda, dtype, H, F):
+    print(f"graph_attn_bias case: H={H} F={F} {dtype}", flush=True)
     data = workloads.erdos_renyi_batch(batch=16, seed=42)
-    H, F = 8, 3
     g = torch.Generator().manual_seed(1)
     m = GraphAttnBias(H, 512, 5, 22, 128, 64, "single_hop", 5)
     with torch.no_grad():
@@ -83,7 +86,9 @@ def test_graph_attn_bias_matches_oracle(cuda, dtype):
     attn_bias = torch.from_numpy(data["attn_bias"])                       # 0 / -inf, [b, S1, S1]
     spatial_pos = torch.from_numpy(data["spatial_pos"]).long()
     et1 = torch.from_numpy(data["edge_type"]).long()
-    edge_type = torch.stack([et1, (et1 * 2) % 5, torch.zeros_like(et1)], -1)       # F = 3 edge features per pair
+    # F edge features per pair; from the third on, every other one is the padding id
+    edge_type = torch.stack([(et1 * (f + 1)) % 5 if f < 2 or f % 2 else torch.zeros_like(et1) for f in range(F)], -1)
+    assert int(spatial_pos.max()) > 6                 # ids beyond the ones the backward keeps in registers occur
     st, et, vd = (p.detach().double() for p in (m.spatial_pos_encoder.weight, m.edge_encoder.weight, m.graph_token_virtual_distance.weight))
     st.requires_grad_(True); et.requires_grad_(True); vd.requires_grad_(True)
     want = oda.graph_attn_bias(attn_bias.double(), spatial_pos, edge_type, st, et, vd)

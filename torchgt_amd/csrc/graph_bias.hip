@@ -76,72 +76,287 @@ __global__ __launch_bounds__(256) void k_graph_bias_fwd(BiasArgs a, T* __restric
     }
 }
 
+// Position (graph, row, column) of a thread in the [b, S1, S1] index space and its step from one
+// iteration of a grid-stride loop to the next, without a 64-bit division per iteration.
+struct BiasPos {
+    int64_t g;
+    int i, j;
+};
+struct BiasStep {
+    int64_t dg;
+    int di, dj;
+};
+__device__ __forceinline__ BiasPos bias_pos(int64_t t, int S1) {
+    const int64_t plane = (int64_t)S1 * S1;
+    BiasPos p;
+    p.g = t / plane;
+    const int ij = (int)(t - p.g * plane);
+    p.i = ij / S1;
+    p.j = ij - p.i * S1;
+    return p;
+}
+__device__ __forceinline__ BiasStep bias_step(int64_t stride, int S1) {
+    const BiasPos p = bias_pos(stride, S1);
+    return BiasStep{p.g, p.i, p.j};
+}
+__device__ __forceinline__ void bias_advance(BiasPos& p, const BiasStep& d, int S1) {
+    p.j += d.dj;
+    if (p.j >= S1) { p.j -= S1; ++p.i; }
+    p.i += d.di;
+    if (p.i >= S1) { p.i -= S1; ++p.g; }
+    p.g += d.dg;
+}
+
+// The same for eight heads and tables that fit LDS: the tables are converted to float once per
+// workgroup, a position reads its table rows with 16-byte LDS loads instead of one global load per
+// head and feature, and the global loads of a position (bias, ids) are issued together.  Same
+// arithmetic in the same order as the kernel above.
+template <typename T>
+__global__ __launch_bounds__(256) void k_graph_bias_fwd8(BiasArgs a, T* __restrict__ out) {
+    constexpr int H = 8;
+    extern __shared__ float4 tab4[];
+    float* tab = reinterpret_cast<float*>(tab4);
+    const int n_sp = a.num_spatial * H, n_e = a.num_edges * H;
+    {
+        const T* sp_tab = reinterpret_cast<const T*>(a.spatial_table);
+        const T* e_tab = reinterpret_cast<const T*>(a.edge_table);
+        const T* vd = reinterpret_cast<const T*>(a.virtual_dist);
+        for (int k = threadIdx.x; k < n_sp + n_e + H; k += 256)
+            tab[k] = k < n_sp ? ldf(sp_tab + k) : (k < n_sp + n_e ? ldf(e_tab + (k - n_sp)) : ldf(vd + (k - n_sp - n_e)));
+    }
+    __syncthreads();
+    const float4* t_sp = tab4;
+    const float4* t_e = tab4 + n_sp / 4;
+    const float4* t_v = t_e + n_e / 4;
+    const int S1 = a.s + 1, F = a.F;
+    const int64_t plane = (int64_t)S1 * S1;
+    const int64_t total = (int64_t)a.b * plane;
+    const float inv_f = 1.f / (float)F;
+    const T* __restrict__ bias = reinterpret_cast<const T*>(a.attn_bias);
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    const BiasStep step = bias_step(stride, S1);
+    BiasPos p = bias_pos((int64_t)blockIdx.x * 256 + threadIdx.x, S1);
+    for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < total; t += stride, bias_advance(p, step, S1)) {
+        const int64_t g = p.g;
+        const int i = p.i, j = p.j, ij = i * S1 + j;
+        const bool inner = i >= 1 && j >= 1;
+        const int64_t pos = inner ? (g * a.s + (i - 1)) * a.s + (j - 1) : 0;
+        const T braw = bias[t];
+        float v[H];
+        if (a.s > 0) {
+            const int64_t spr = a.spatial_pos[pos];
+            float e[H];
+#pragma unroll
+            for (int h = 0; h < H; ++h) e[h] = 0.f;
+            for (int f0 = 0; f0 < F; f0 += 4) {
+                int64_t er[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) er[u] = a.edge_type[pos * F + min(f0 + u, F - 1)];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if (f0 + u < F) {
+                        const int id = clamp_id(er[u], a.num_edges);
+                        const float4 lo = t_e[id * 2], hi = t_e[id * 2 + 1];
+                        e[0] += lo.x; e[1] += lo.y; e[2] += lo.z; e[3] += lo.w;
+                        e[4] += hi.x; e[5] += hi.y; e[6] += hi.z; e[7] += hi.w;
+                    }
+                }
+            }
+            const int sp = clamp_id(spr, a.num_spatial);
+            const float4 lo = t_sp[sp * 2], hi = t_sp[sp * 2 + 1];
+            const float s8[H] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+            const float base = 2.f * ldf(&braw);
+#pragma unroll
+            for (int h = 0; h < H; ++h) {
+                float x = base;
+                if (inner) { x += s8[h]; x += e[h] * inv_f; }
+                v[h] = x;
+            }
+        } else {
+            const float base = 2.f * ldf(&braw);
+#pragma unroll
+            for (int h = 0; h < H; ++h) v[h] = base;
+        }
+        if (!inner) {
+            const float4 lo = t_v[0], hi = t_v[1];
+            v[0] += lo.x; v[1] += lo.y; v[2] += lo.z; v[3] += lo.w;
+            v[4] += hi.x; v[5] += hi.y; v[6] += hi.z; v[7] += hi.w;
+        }
+        T* __restrict__ o = out + g * H * plane + ij;
+#pragma unroll
+        for (int h = 0; h < H; ++h) stf(o + h * plane, v[h]);
+    }
+}
+
 // Table gradients.  Each workgroup keeps the three tables in LDS ([num_spatial + num_edges + 1][H]
 // floats), walks its share of the positions and writes one partial.  Row 0 of the two
 // embedding tables is the padding index: it receives no gradient (nn.Embedding padding_idx=0).
-template <typename T>
+// All loads of a position (ids, then the gradient of eight heads at a time) are issued without a
+// lane-dependent branch around them: out-of-range lanes read a clamped address and add nothing.
+// Shortest-path ids are few and small (most pairs of a graph are two to four hops apart), and an LDS
+// float atomic costs a few cycles per active lane whatever the address: with up to eight heads the
+// ids 1..NHOT are summed in registers (one compare per id, one select + add per id and head), added
+// over the wave at the end and put into LDS by one lane; only the rare other ids, the edge types
+// (most pairs are not edges: id 0) and the virtual-node row and column use atomics per position.
+constexpr int kBiasFeat = 4;      // edge features handled per pass over the heads (1 when there is only one)
+constexpr int kBiasHot = 5;       // spatial ids 1..5 (self, one to four hops) are summed in registers
+
+// What one lane reads for one position and one pass (up to kBiasFeat edge features, eight heads), kept
+// as loaded: converting or clamping a value where it is fetched would make the wave wait for it there.
+template <typename T, int FC>
+struct BiasFetch {
+    int64_t spr, er[FC];
+    T raw[8];
+    bool valid, inner;
+};
+template <typename T, int FC>
+__device__ __forceinline__ void bias_fetch(const BiasArgs& a, const T* __restrict__ dout, const BiasPos& p, bool valid, int f0,
+                                           int h0, BiasFetch<T, FC>& x) {
+    const int S1 = a.s + 1;
+    const int64_t plane = (int64_t)S1 * S1;
+    x.valid = valid;
+    const int64_t g = valid ? p.g : 0;               // past the end: element 0, nothing is added
+    const int i = valid ? p.i : 0, j = valid ? p.j : 0, ij = i * S1 + j;
+    x.inner = valid && i >= 1 && j >= 1;
+    const int64_t pos = x.inner ? (g * a.s + (i - 1)) * a.s + (j - 1) : 0;
+    x.spr = 0;
+#pragma unroll
+    for (int u = 0; u < FC; ++u) x.er[u] = 0;
+    if (a.s > 0) {
+        x.spr = a.spatial_pos[pos];
+#pragma unroll
+        for (int u = 0; u < FC; ++u) x.er[u] = a.edge_type[pos * a.F + min(f0 + u, a.F - 1)];
+    }
+    const T* __restrict__ dg = dout + g * a.H * plane + ij;          // head h of this position: dg[h * plane]
+#pragma unroll
+    for (int u = 0; u < 8; ++u) x.raw[u] = dg[(int64_t)min(h0 + u, a.H - 1) * plane];
+}
+
+template <typename T, int NHOT, int FC>
+__device__ __forceinline__ void bias_consume(const BiasArgs& a, const BiasFetch<T, FC>& x, int f0, int h0, float* acc_sp, float* acc_e,
+                                             float* acc_v, float (&hot)[NHOT > 0 ? NHOT : 1][8]) {
+    const int H = a.H;
+    const int sp = x.inner && f0 == 0 ? clamp_id(x.spr, a.num_spatial) : 0;
+    int e[FC];
+#pragma unroll
+    for (int u = 0; u < FC; ++u) e[u] = x.inner && f0 + u < a.F ? clamp_id(x.er[u], a.num_edges) : 0;
+    const bool virt = x.valid && !x.inner && f0 == 0;
+    const bool cold = sp > NHOT;
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = ldf(&x.raw[u]);
+    if (NHOT > 0) {
+#pragma unroll
+        for (int r = 0; r < NHOT; ++r) {
+            const bool hit = sp == r + 1;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) hot[r][u] += hit ? v[u] : 0.f;
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        const int h = h0 + u;
+        if (h < H && v[u] != 0.f) {              // masked (padded) positions carry exact zeros
+            if (cold) atomicAdd(&acc_sp[sp * H + h], v[u]);
+#pragma unroll
+            for (int w = 0; w < FC; ++w)
+                if (e[w] > 0) atomicAdd(&acc_e[e[w] * H + h], v[u]);
+            if (virt) atomicAdd(&acc_v[h], v[u]);
+        }
+    }
+}
+
+// ONEPASS: H <= 8 and F <= FC, one fetch per position; the fetch of the next position is issued
+// before the current one is consumed.
+template <typename T, int NHOT, bool ONEPASS, int FC>
 __global__ __launch_bounds__(256) void k_graph_bias_bwd(BiasArgs a, const T* __restrict__ dout, float* __restrict__ partial,
                                                         int copies) {
     extern __shared__ float acc_all[];
     const int n_acc = (a.num_spatial + a.num_edges + 1) * a.H;
     for (int k = threadIdx.x; k < n_acc * copies; k += 256) acc_all[k] = 0.f;
     __syncthreads();
-    // few distinct ids meet many positions: neighbouring lanes add into different copies of the tables
+    // neighbouring lanes add into different copies of the tables
     float* acc = acc_all + (threadIdx.x % copies) * n_acc;
     float* acc_sp = acc;
     float* acc_e = acc + a.num_spatial * a.H;
     float* acc_v = acc_e + a.num_edges * a.H;
-    const int S1 = a.s + 1;
-    const int64_t total = (int64_t)a.b * S1 * S1;
-    const float inv_f = 1.f / (float)a.F;
-    for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < total; t += (int64_t)gridDim.x * 256) {
-        const int j = (int)(t % S1), i = (int)((t / S1) % S1);
-        const int64_t g = t / ((int64_t)S1 * S1);
-        const bool inner = i >= 1 && j >= 1;
-        int sp = 0;
-        const int64_t* et = nullptr;
-        if (inner) {
-            const int64_t pos = (g * a.s + (i - 1)) * a.s + (j - 1);
-            sp = clamp_id(a.spatial_pos[pos], a.num_spatial);
-            et = a.edge_type + pos * a.F;
+    const int H = a.H, F = a.F;
+    const int64_t total = (int64_t)a.b * (a.s + 1) * (a.s + 1);
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    float hot[NHOT > 0 ? NHOT : 1][8];
+#pragma unroll
+    for (int r = 0; r < (NHOT > 0 ? NHOT : 1); ++r)
+#pragma unroll
+        for (int u = 0; u < 8; ++u) hot[r][u] = 0.f;
+    if (ONEPASS) {
+        BiasFetch<T, FC> cur, nxt;
+        int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+        const BiasStep step = bias_step(stride, a.s + 1);
+        BiasPos p = bias_pos(t, a.s + 1);
+        if (t - threadIdx.x < total) bias_fetch(a, dout, p, t < total, 0, 0, cur);
+        for (; t - threadIdx.x < total; t += stride) {
+            bias_advance(p, step, a.s + 1);
+            bias_fetch(a, dout, p, t + stride < total, 0, 0, nxt);
+            bias_consume<T, NHOT, FC>(a, cur, 0, 0, acc_sp, acc_e, acc_v, hot);
+            cur = nxt;
         }
-        for (int h = 0; h < a.H; ++h) {
-            const float v = ldf(dout + ((g * a.H + h) * S1 + i) * S1 + j);
-            if (v == 0.f) continue;              // masked (padded) positions carry exact zeros
-            if (inner) {
-                if (sp > 0) atomicAdd(&acc_sp[sp * a.H + h], v);
-                for (int f = 0; f < a.F; ++f) {
-                    const int e = clamp_id(et[f], a.num_edges);
-                    if (e > 0) atomicAdd(&acc_e[e * a.H + h], v * inv_f);
+    } else {
+        for (int64_t t0 = (int64_t)blockIdx.x * 256; t0 < total; t0 += stride)
+            for (int f0 = 0; f0 < F; f0 += FC)
+                for (int h0 = 0; h0 < H; h0 += 8) {
+                    BiasFetch<T, FC> x;
+                    bias_fetch(a, dout, bias_pos(t0 + threadIdx.x, a.s + 1), t0 + threadIdx.x < total, f0, h0, x);
+                    // the spatial id counts once per head pass, in the first feature pass
+                    bias_consume<T, NHOT, FC>(a, x, f0, h0, acc_sp, acc_e, acc_v, hot);
                 }
-            } else {
-                atomicAdd(&acc_v[h], v);
+    }
+    if (NHOT > 0) {
+        // the wave's sums of the ids kept in registers (NHOT > 0 only with H <= 8: one pass over the heads)
+#pragma unroll
+        for (int r = 0; r < NHOT; ++r)
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                float x = hot[r][u];
+#pragma unroll
+                for (int off = 32; off >= 1; off >>= 1) x += __shfl_xor(x, off);
+                if (threadIdx.x % 64 == 0 && u < H && r + 1 < a.num_spatial) atomicAdd(&acc_sp[(r + 1) * H + u], x);
             }
-        }
     }
     __syncthreads();
+    const float inv_f = 1.f / (float)F;                       // mean over the edge features (:150)
+    const int e_lo = a.num_spatial * H, e_hi = e_lo + a.num_edges * H;
     for (int k = threadIdx.x; k < n_acc; k += 256) {
         float t = 0.f;
         for (int c = 0; c < copies; ++c) t += acc_all[c * n_acc + k];       // copies in order
-        partial[(int64_t)blockIdx.x * n_acc + k] = t;
+        partial[(int64_t)blockIdx.x * n_acc + k] = k >= e_lo && k < e_hi ? t * inv_f : t;
     }
 }
 
+// Sum of the workgroup partials in a fixed order: 64 slices of the workers per entry, then the slices.
 template <typename T>
 __global__ __launch_bounds__(256) void k_graph_bias_reduce(const float* __restrict__ partial, int workers, int n_sp, int n_e,
                                                            int n_v, T* __restrict__ d_sp, T* __restrict__ d_e,
                                                            T* __restrict__ d_v) {
+    __shared__ float part[64][4];
     const int n = n_sp + n_e + n_v;
-    const int k = blockIdx.x * 256 + threadIdx.x;
-    if (k >= n) return;
+    const int kl = threadIdx.x % 4, slice = threadIdx.x / 4;
+    const int k = blockIdx.x * 4 + kl;
     float t = 0.f;
-    for (int w = 0; w < workers; ++w) t += partial[(int64_t)w * n + k];
+    if (k < n)
+        for (int w = slice; w < workers; w += 64) t += partial[(int64_t)w * n + k];
+    part[slice][kl] = t;
+    __syncthreads();
+    if (slice != 0 || k >= n) return;
+    t = 0.f;
+#pragma unroll
+    for (int c = 0; c < 64; ++c) t += part[c][kl];
     if (k < n_sp) stf(d_sp + k, t);
     else if (k < n_sp + n_e) stf(d_e + (k - n_sp), t);
     else stf(d_v + (k - n_sp - n_e), t);
 }
 
-constexpr int kBiasWorkers = 256;
+constexpr int kBiasWorkers = 1024;
+constexpr int kBiasCopies = 16;
 
 int bias_check(int b, int s, int H, int F, int num_spatial, int num_edges, int dtype, const char* who) {
     if (b < 0 || s < 0 || H < 1 || F < 1 || num_spatial < 1 || num_edges < 1 ||
@@ -220,8 +435,16 @@ int tgt_graph_attn_bias_fwd(const void* d_attn_bias, const int64_t* d_spatial_po
     const int64_t total = (int64_t)b * (s + 1) * (s + 1);
     const dim3 grid((unsigned)((total + 255) / 256));
     hipStream_t st = (hipStream_t)stream;
-    if (dtype == TGT_DTYPE_F32) hipLaunchKernelGGL((k_graph_bias_fwd<float>), grid, dim3(256), 0, st, a, (float*)d_out);
-    else hipLaunchKernelGGL((k_graph_bias_fwd<gbf16>), grid, dim3(256), 0, st, a, (gbf16*)d_out);
+    const size_t tab_bytes = sizeof(float) * (size_t)(num_spatial + num_edges + 1) * H;
+    if (H == 8 && tab_bytes <= 32 * 1024) {
+        const dim3 g8((unsigned)std::min<int64_t>((total + 255) / 256, 4096));
+        if (dtype == TGT_DTYPE_F32) hipLaunchKernelGGL((k_graph_bias_fwd8<float>), g8, dim3(256), tab_bytes, st, a, (float*)d_out);
+        else hipLaunchKernelGGL((k_graph_bias_fwd8<gbf16>), g8, dim3(256), tab_bytes, st, a, (gbf16*)d_out);
+    } else if (dtype == TGT_DTYPE_F32) {
+        hipLaunchKernelGGL((k_graph_bias_fwd<float>), grid, dim3(256), 0, st, a, (float*)d_out);
+    } else {
+        hipLaunchKernelGGL((k_graph_bias_fwd<gbf16>), grid, dim3(256), 0, st, a, (gbf16*)d_out);
+    }
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
 }
@@ -259,25 +482,40 @@ int tgt_graph_attn_bias_bwd(const void* d_dout, const int64_t* d_spatial_pos, co
     const int workers = (int)std::max<int64_t>(1, std::min<int64_t>((total + 255) / 256, kBiasWorkers));
     hipStream_t st = (hipStream_t)stream;
     float* partial = (float*)d_workspace;
-    int copies = 16;
+    int copies = kBiasCopies;
     while (copies > 1 && (size_t)n_acc * copies * sizeof(float) > 60 * 1024) copies /= 2;
     const size_t lds = (size_t)n_acc * copies * sizeof(float);
-    if (lds > 48 * 1024) {
-        TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_graph_bias_bwd<float>),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, 60 * 1024));
-        TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_graph_bias_bwd<gbf16>),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, 60 * 1024));
-    }
-    const unsigned rgrid = (unsigned)((n_acc + 255) / 256);
+    const unsigned rgrid = (unsigned)((n_acc + 3) / 4);
+    auto launch = [&](auto kernel, auto reduce, auto* dout, auto* dsp, auto* de, auto* dv) -> int {
+        if (lds > 48 * 1024)
+            TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                              60 * 1024));
+        hipLaunchKernelGGL(kernel, dim3(workers), dim3(256), lds, st, a, dout, partial, copies);
+        hipLaunchKernelGGL(reduce, dim3(rgrid), dim3(256), 0, st, (const float*)partial, workers, num_spatial * H, num_edges * H, H,
+                           dsp, de, dv);
+        return TGT_OK;
+    };
+    // registers for the frequent ids need one pass over the heads; the prefetching loop one pass over the features too
+    const int variant = H > 8 ? 0 : (F > kBiasFeat ? 1 : (F > 1 ? 2 : 3));
+    int lrc;
     if (dtype == TGT_DTYPE_F32) {
-        hipLaunchKernelGGL((k_graph_bias_bwd<float>), dim3(workers), dim3(256), lds, st, a, (const float*)d_dout, partial, copies);
-        hipLaunchKernelGGL((k_graph_bias_reduce<float>), dim3(rgrid), dim3(256), 0, st, partial, workers, num_spatial * H,
-                           num_edges * H, H, (float*)d_dspatial_table, (float*)d_dedge_table, (float*)d_dvirtual_dist);
+        auto* red = &k_graph_bias_reduce<float>;
+        const float* dout = (const float*)d_dout;
+        float *dsp = (float*)d_dspatial_table, *de = (float*)d_dedge_table, *dv = (float*)d_dvirtual_dist;
+        lrc = variant == 3   ? launch(&k_graph_bias_bwd<float, kBiasHot, true, 1>, red, dout, dsp, de, dv)
+              : variant == 2 ? launch(&k_graph_bias_bwd<float, kBiasHot, true, kBiasFeat>, red, dout, dsp, de, dv)
+              : variant == 1 ? launch(&k_graph_bias_bwd<float, kBiasHot, false, kBiasFeat>, red, dout, dsp, de, dv)
+                             : launch(&k_graph_bias_bwd<float, 0, false, kBiasFeat>, red, dout, dsp, de, dv);
     } else {
-        hipLaunchKernelGGL((k_graph_bias_bwd<gbf16>), dim3(workers), dim3(256), lds, st, a, (const gbf16*)d_dout, partial, copies);
-        hipLaunchKernelGGL((k_graph_bias_reduce<gbf16>), dim3(rgrid), dim3(256), 0, st, partial, workers, num_spatial * H,
-                           num_edges * H, H, (gbf16*)d_dspatial_table, (gbf16*)d_dedge_table, (gbf16*)d_dvirtual_dist);
+        auto* red = &k_graph_bias_reduce<gbf16>;
+        const gbf16* dout = (const gbf16*)d_dout;
+        gbf16 *dsp = (gbf16*)d_dspatial_table, *de = (gbf16*)d_dedge_table, *dv = (gbf16*)d_dvirtual_dist;
+        lrc = variant == 3   ? launch(&k_graph_bias_bwd<gbf16, kBiasHot, true, 1>, red, dout, dsp, de, dv)
+              : variant == 2 ? launch(&k_graph_bias_bwd<gbf16, kBiasHot, true, kBiasFeat>, red, dout, dsp, de, dv)
+              : variant == 1 ? launch(&k_graph_bias_bwd<gbf16, kBiasHot, false, kBiasFeat>, red, dout, dsp, de, dv)
+                             : launch(&k_graph_bias_bwd<gbf16, 0, false, kBiasFeat>, red, dout, dsp, de, dv);
     }
+    if (lrc != TGT_OK) return lrc;
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
 }
