@@ -8,10 +8,11 @@ the benchmark configuration "configs[1]": N = 64 001, E ~ 530 K, H = 8, d = 8, p
 reported separately).  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype f32|bf16] [--no-cpu-baseline]
-                    [--workload config1|config2|config2-mha|config2-model|config3|config4|config5|config5-blockized]
+                    [--workload config1|config2|config2-mha|config2-model|config3|config4|config4-bias|config5|
+                               config5-blockized]
 
 config3 / config5: larger sparse workloads (bf16); config4: dense biased attention of a graph-level
-batch; config5-blockized: the block path on the reordered config5 graph; config2-mha: one whole
+batch; config4-bias: the bias builder in front of it (GraphAttnBias forward + table gradients); config5-blockized: the block path on the reordered config5 graph; config2-mha: one whole
 MultiHeadAttention layer (projections + sparse attention) on the config2 graph; config2-model: a training
 step of the 4-layer Graphormer-Slim on that graph.
 """
@@ -247,6 +248,77 @@ def bench_dense(args):
                      "avg_us": kernels[dom]["avg_us"]},
         "mfma": {n: {"alg_tflops": flops[n] / (kernels[n]["avg_us"] * 1e-6) / 1e12, "peak_tflops": 2500.0}
                  for n in kernels},
+        "kernels": kernels,
+    }
+    print(json.dumps(result))
+
+
+def bench_graph_bias(args):
+    """The bias builder in front of configs[3]: GraphAttnBias forward and the gradients of its three tables for
+    the batch of 256 padded ER graphs (S = 129, H = 8, one edge feature, tables [22, 8] and [5, 8]).
+    A step = tgt_graph_attn_bias_fwd + tgt_graph_attn_bias_bwd."""
+    import torch
+    from torchgt_amd import _lib, workloads
+    dev = torch.device("cuda:0")
+    b, H, F, n_sp, n_e = 256, 8, 1, 22, 5
+    data = workloads.erdos_renyi_batch(batch=b, seed=42)
+    S1 = data["S"]
+    s = S1 - 1
+    tdt = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    esize = 2 if args.dtype == "bf16" else 4
+    g = torch.Generator().manual_seed(42)
+    attn_bias = torch.from_numpy(data["attn_bias"]).to(dev, tdt)
+    spatial_pos = torch.from_numpy(data["spatial_pos"]).long().to(dev)
+    edge_type = torch.from_numpy(data["edge_type"]).long().unsqueeze(-1).contiguous().to(dev)
+    t_sp, t_e, t_v = ((torch.randn(n, H, generator=g) * 0.02).to(dev, tdt) for n in (n_sp, n_e, 1))
+    out = torch.empty(b, H, S1, S1, device=dev, dtype=tdt)
+    dout = torch.randn(b, H, S1, S1, generator=g).to(dev, tdt)
+    dout[~torch.isfinite(attn_bias).unsqueeze(1).expand_as(dout)] = 0       # masked entries carry no gradient
+    d_sp, d_e, d_v = torch.empty_like(t_sp), torch.empty_like(t_e), torch.empty_like(t_v)
+    L = _lib.lib()
+    dt_code = _lib.DTYPE_BF16 if args.dtype == "bf16" else _lib.DTYPE_F32
+    nbytes = L.tgt_graph_attn_bias_bwd_workspace_bytes(n_sp, n_e, H)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    P = lambda t: t.data_ptr()
+
+    def step():
+        _lib.check(L.tgt_graph_attn_bias_fwd(P(attn_bias), P(spatial_pos), P(edge_type), F, P(t_sp), n_sp, P(t_e), n_e, P(t_v),
+                                             b, s, H, dt_code, P(out), stream))
+        _lib.check(L.tgt_graph_attn_bias_bwd(P(dout), P(spatial_pos), P(edge_type), F, n_sp, n_e, b, s, H, dt_code,
+                                             P(d_sp), P(d_e), P(d_v), P(ws), nbytes, stream))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    L.tgt_timing_reset()
+    L.tgt_timing_enable(1)
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    L.tgt_timing_enable(0)
+    kernels = {n: {"avg_us": t / c * 1e3, "launches": c} for n, (t, c) in _lib.kernel_timings().items() if c}
+    ids_b = b * s * s * 8 * (1 + F)                       # int64 spatial_pos and edge_type
+    bias_b = b * H * S1 * S1 * esize
+    alg = {"graph_bias_fwd": b * S1 * S1 * esize + ids_b + bias_b, "graph_bias_bwd": bias_b + ids_b}
+    dom = max(kernels, key=lambda n: kernels[n]["avg_us"])
+    gbs = alg[dom] / (kernels[dom]["avg_us"] * 1e-6) / 1e9
+    result = {
+        "metric": "GraphAttnBias forward + table gradients (graph-level batch); % HBM roofline",
+        "value": b / (ms * 1e-3), "unit": "graphs/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic",
+        "config": {"workload": "bias builder of configs[3]: 256 ER graphs n~U[16,128] p=0.1 padded to 128 + virtual node",
+                   "b": b, "S": S1, "H": H, "edge_features": F, "tables": [[n_sp, H], [n_e, H], [1, H]],
+                   "step": "tgt_graph_attn_bias_fwd + tgt_graph_attn_bias_bwd", "parallelism": "1 GPU"},
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": gbs / HBM_PEAK_GBS, "traffic": None, "alg_bytes": alg[dom], "avg_us": kernels[dom]["avg_us"]},
+        "alg_bytes": alg,
         "kernels": kernels,
     }
     print(json.dumps(result))
@@ -533,12 +605,14 @@ def main():
         raise SystemExit("bench.py needs a GPU")
     dev = torch.device("cuda:0")
     H, d = 8, 8
-    if args.workload in ("config3", "config4", "config5", "config5-blockized") and "--dtype" not in sys.argv:
+    if args.workload in ("config3", "config4", "config4-bias", "config5", "config5-blockized") and "--dtype" not in sys.argv:
         args.dtype = "bf16"              # the dtype those configurations are quoted on
     tdt = torch.float32 if args.dtype == "f32" else torch.bfloat16
     esize = 4 if args.dtype == "f32" else 2
     if args.workload == "config4":
         return bench_dense(args)
+    if args.workload == "config4-bias":
+        return bench_graph_bias(args)
     if args.workload == "config5-blockized":
         return bench_block(args)
     if args.workload == "config2-mha":

@@ -82,7 +82,8 @@ private:
 
 // Kernel names of the optional per-kernel timing (timing.hip).
 enum KernelSlot { KS_FWD = 0, KS_NODE_SIDE, KS_BWD, KS_DENSE_FWD, KS_DENSE_BWD, KS_TILE_FWD, KS_TILE_BWD, KS_PROBE_GATHER, KS_LINEAR_FWD,
-                  KS_LINEAR_DX, KS_LINEAR_DW, KS_LAYER_NORM_FWD, KS_LAYER_NORM_BWD, KS_GELU, KS_COUNT };
+                  KS_LINEAR_DX, KS_LINEAR_DW, KS_LAYER_NORM_FWD, KS_LAYER_NORM_BWD, KS_GELU, KS_GRAPH_BIAS_FWD,
+                  KS_GRAPH_BIAS_BWD, KS_COUNT };
 
 // Scope guard: records a hipEvent on `st` before and after the launches made in
 // its scope when timing is enabled; does nothing otherwise.

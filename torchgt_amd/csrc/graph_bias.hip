@@ -435,6 +435,7 @@ int tgt_graph_attn_bias_fwd(const void* d_attn_bias, const int64_t* d_spatial_po
     const int64_t total = (int64_t)b * (s + 1) * (s + 1);
     const dim3 grid((unsigned)((total + 255) / 256));
     hipStream_t st = (hipStream_t)stream;
+    KernelTimer timer(KS_GRAPH_BIAS_FWD, st);
     const size_t tab_bytes = sizeof(float) * (size_t)(num_spatial + num_edges + 1) * H;
     if (H == 8 && tab_bytes <= 32 * 1024) {
         const dim3 g8((unsigned)std::min<int64_t>((total + 255) / 256, 4096));
@@ -481,6 +482,7 @@ int tgt_graph_attn_bias_bwd(const void* d_dout, const int64_t* d_spatial_pos, co
     const int64_t total = (int64_t)b * (s + 1) * (s + 1);
     const int workers = (int)std::max<int64_t>(1, std::min<int64_t>((total + 255) / 256, kBiasWorkers));
     hipStream_t st = (hipStream_t)stream;
+    KernelTimer timer(KS_GRAPH_BIAS_BWD, st);
     float* partial = (float*)d_workspace;
     int copies = kBiasCopies;
     while (copies > 1 && (size_t)n_acc * copies * sizeof(float) > 60 * 1024) copies /= 2;
