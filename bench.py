@@ -243,7 +243,7 @@ def bench_dense(args):
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": gbs / HBM_PEAK_GBS,
                      # rocprofv3 FETCH_SIZE x2.000 + WRITE_SIZE x1.000, profiles/dense_attn_config4_bf16.txt
-                     "traffic": {"dense_fwd": 107.5e6, "dense_bwd": 203.9e6}.get(dom) if args.dtype == "bf16" else None,
+                     "traffic": {"dense_fwd": 107.6e6, "dense_bwd": 219.8e6}.get(dom) if args.dtype == "bf16" else None,
                      "alg_bytes": alg[dom],
                      "avg_us": kernels[dom]["avg_us"]},
         "mfma": {n: {"alg_tflops": flops[n] / (kernels[n]["avg_us"] * 1e-6) / 1e12, "peak_tflops": 2500.0}

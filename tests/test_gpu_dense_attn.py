@@ -60,7 +60,11 @@ def test_small_shapes(cuda, dtype):
     run_case("s129", 4, 129, 8, 8, dtype, True, [129, 17, 64, 100], 4, cuda)
 
 
-@pytest.mark.parametrize("S", [1, 31, 64, 65, 96, 160, 161, 200, 256])
+# 1, 4, 34, 65, 100, 131, 161: a last tile of one to four rows (a virtual node behind a multiple of 32), which the
+# kernels treat apart from full tiles; 36 and 69: one row more than that.  (Sequences of two or three rows are left
+# out: with a graph of one real key every dS cancels to zero, and the rounding of the stored bf16 output alone --
+# the same arithmetic in float64 with the kernel's rounding points -- puts dk 3 % off in this error measure.)
+@pytest.mark.parametrize("S", [1, 4, 31, 34, 36, 64, 65, 69, 96, 100, 131, 160, 161, 200, 256])
 def test_every_tile_count(cuda, S):
     run_case(f"S{S}", 2, S, 2, 8, torch.bfloat16, True, [S, max(1, S // 2)], 10 + S, cuda)
 
@@ -69,6 +73,7 @@ def test_every_tile_count(cuda, S):
 def test_other_head_dims(cuda, d):
     run_case(f"d{d}", 2, 70, 4, d, torch.bfloat16, True, [70, 33], 20 + d, cuda)
     run_case(f"d{d}-f32", 1, 129, 2, d, torch.float32, True, None, 30 + d, cuda, bias_grad=False)
+    run_case(f"d{d}-s67", 2, 67, 2, d, torch.bfloat16, True, [67, 40], 40 + d, cuda)        # three rows in the last tile
 
 
 def test_config4_batch_with_bias_from_tables(cuda):

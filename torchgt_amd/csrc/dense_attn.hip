@@ -180,6 +180,180 @@ template <int D, int NT> constexpr int bwd_lds_bytes() {
 constexpr int kLdsLimit = 160 * 1024;
 
 // ---------------------------------------------------------------------------
+// The last tile of a sequence of 32 n + 1 .. 32 n + 4 rows (a virtual node behind a multiple of 32)
+// holds one to four rows.  As a matrix tile it would cost its wave as much as a full one, so the wave
+// that owns it works on the vector unit instead, lane = key (or query), one row at a time: dot
+// products from the LDS images, reductions over the wave.  Probabilities and dS are rounded to bf16
+// where the matrix path rounds them.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) x += __shfl_xor(x, off);
+    return x;
+}
+__device__ __forceinline__ float wave_max(float x) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) x = fmaxf(x, __shfl_xor(x, off));
+    return x;
+}
+__device__ __forceinline__ float round_bf(float x) { return bf2f(f2bf(x)); }
+template <int D>
+__device__ __forceinline__ void lds_row(const short* __restrict__ rm, int row, float (&x)[D]) {
+#pragma unroll
+    for (int c = 0; c < D / 4; ++c) {
+        const short4_t v = *reinterpret_cast<const short4_t*>(&rm[row * D + 4 * c]);
+        x[4 * c + 0] = bf2f(v.x); x[4 * c + 1] = bf2f(v.y); x[4 * c + 2] = bf2f(v.z); x[4 * c + 3] = bf2f(v.w);
+    }
+}
+template <int D>
+__device__ __forceinline__ float dot_d(const float (&a)[D], const float (&b)[D]) {
+    float t = 0.f;
+#pragma unroll
+    for (int c = 0; c < D; ++c) t = fmaf(a[c], b[c], t);
+    return t;
+}
+template <typename T, int D>
+__device__ __forceinline__ void store_row(T* __restrict__ p, const float (&x)[D], float f) {
+#pragma unroll
+    for (int c = 0; c < D; c += 4) st4(p + c, x[c] * f, x[c + 1] * f, x[c + 2] * f, x[c + 3] * f);
+}
+
+// forward of the rows first .. first + count - 1 (all keys), by one wave
+template <typename T, int D, int SP>
+__device__ __forceinline__ void thin_rows_fwd(const T* __restrict__ Q, const short* __restrict__ k_rm,
+                                              const short* __restrict__ v_tr, const T* __restrict__ bias_gh,
+                                              T* __restrict__ out, float* __restrict__ lse, int g, int h, int S, int H,
+                                              float scale, int first, int count, int lane) {
+    constexpr int NC = (SP + 63) / 64;
+    for (int tq = 0; tq < count; ++tq) {
+        const int qi = first + tq;
+        float qv[D];
+#pragma unroll
+        for (int c = 0; c < D / 4; ++c) {
+            const short4_t v = ld4(Q + (((int64_t)g * S + qi) * H + h) * D + 4 * c);
+            qv[4 * c + 0] = bf2f(v.x); qv[4 * c + 1] = bf2f(v.y); qv[4 * c + 2] = bf2f(v.z); qv[4 * c + 3] = bf2f(v.w);
+        }
+        const T* brow = bias_gh ? bias_gh + (int64_t)qi * S : nullptr;
+        float sv[NC], mx = -INFINITY;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            const int key = c * 64 + lane;
+            sv[c] = -INFINITY;
+            if (key < S) {
+                float kv[D];
+                lds_row<D>(k_rm, key, kv);
+                sv[c] = fmaf(dot_d<D>(qv, kv), scale, brow ? ld1(brow + key) : 0.f);
+            }
+            mx = fmaxf(mx, sv[c]);
+        }
+        mx = wave_max(mx);
+        const float m_use = (mx == -INFINITY) ? 0.f : mx;
+        float lsum = 0.f, ov[D];
+#pragma unroll
+        for (int d = 0; d < D; ++d) ov[d] = 0.f;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            const int key = c * 64 + lane;
+            if (key < S) {
+                const float pb = round_bf(fast_exp2((sv[c] - m_use) * kLog2e));
+                lsum += pb;
+#pragma unroll
+                for (int d = 0; d < D; ++d) ov[d] = fmaf(pb, bf2f(v_tr[d * (SP + 4) + key]), ov[d]);
+            }
+        }
+        lsum = wave_sum(lsum);
+#pragma unroll
+        for (int d = 0; d < D; ++d) ov[d] = wave_sum(ov[d]);
+        if (lane == 0) {
+            store_row<T, D>(out + (((int64_t)g * S + qi) * H + h) * D, ov, 1.0f / lsum);
+            lse[((int64_t)g * H + h) * S + qi] = m_use + __logf(lsum);
+        }
+    }
+}
+
+// backward, query side, of the rows first .. first + count - 1: dQ and their rows of dBias
+template <typename T, int D, int SP>
+__device__ __forceinline__ void thin_rows_bwd_q(const short* __restrict__ q_rm, const short* __restrict__ k_rm,
+                                                const short* __restrict__ v_rm, const short* __restrict__ g_rm,
+                                                const float* __restrict__ lse_l, const float* __restrict__ dd_l,
+                                                const T* __restrict__ bias_gh, T* __restrict__ dbias_gh, T* __restrict__ dQ,
+                                                int g, int h, int S, int H, float scale, int first, int count, int lane) {
+    constexpr int NC = (SP + 63) / 64;
+    const float scale2 = scale * kLog2e;
+    for (int tq = 0; tq < count; ++tq) {
+        const int qi = first + tq;
+        float qv[D], gv[D], dq[D];
+        lds_row<D>(q_rm, qi, qv);
+        lds_row<D>(g_rm, qi, gv);
+#pragma unroll
+        for (int d = 0; d < D; ++d) dq[d] = 0.f;
+        const float nL2 = -lse_l[qi], Dq = dd_l[qi];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            const int key = c * 64 + lane;
+            if (key < S) {
+                float kv[D], vv[D];
+                lds_row<D>(k_rm, key, kv);
+                lds_row<D>(v_rm, key, vv);
+                const float b = bias_gh ? ld1(bias_gh + (int64_t)qi * S + key) : 0.f;
+                const float pv = fast_exp2(fmaf(dot_d<D>(qv, kv), scale2, fmaf(b, kLog2e, nL2)));
+                const float dS = pv * (dot_d<D>(gv, vv) - Dq);
+                if (dbias_gh) st1(dbias_gh + (int64_t)qi * S + key, dS);
+                const float dsb = round_bf(dS);
+#pragma unroll
+                for (int d = 0; d < D; ++d) dq[d] = fmaf(dsb, kv[d], dq[d]);
+            }
+        }
+#pragma unroll
+        for (int d = 0; d < D; ++d) dq[d] = wave_sum(dq[d]);
+        if (lane == 0) store_row<T, D>(dQ + (((int64_t)g * S + qi) * H + h) * D, dq, scale);
+    }
+}
+
+// backward, key side, of the keys first .. first + count - 1 (all queries): dK and dV
+template <typename T, int D, int SP>
+__device__ __forceinline__ void thin_rows_bwd_k(const short* __restrict__ q_rm, const short* __restrict__ k_rm,
+                                                const short* __restrict__ v_rm, const short* __restrict__ g_rm,
+                                                const float* __restrict__ lse_l, const float* __restrict__ dd_l,
+                                                const T* __restrict__ bias_gh, T* __restrict__ dK, T* __restrict__ dV,
+                                                int g, int h, int S, int H, float scale, int first, int count, int lane) {
+    constexpr int NC = (SP + 63) / 64;
+    const float scale2 = scale * kLog2e;
+    for (int tk = 0; tk < count; ++tk) {
+        const int ki = first + tk;
+        float kv[D], vv[D], dk[D], dv[D];
+        lds_row<D>(k_rm, ki, kv);
+        lds_row<D>(v_rm, ki, vv);
+#pragma unroll
+        for (int d = 0; d < D; ++d) { dk[d] = 0.f; dv[d] = 0.f; }
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            const int qq = c * 64 + lane;
+            if (qq < S) {
+                float qv[D], gv[D];
+                lds_row<D>(q_rm, qq, qv);
+                lds_row<D>(g_rm, qq, gv);
+                const float b = bias_gh ? ld1(bias_gh + (int64_t)qq * S + ki) : 0.f;
+                const float pv = fast_exp2(fmaf(dot_d<D>(qv, kv), scale2, fmaf(b, kLog2e, -lse_l[qq])));
+                const float dS = pv * (dot_d<D>(gv, vv) - dd_l[qq]);
+                const float pb = round_bf(pv), dsb = round_bf(dS);
+#pragma unroll
+                for (int d = 0; d < D; ++d) {
+                    dk[d] = fmaf(dsb, qv[d], dk[d]);
+                    dv[d] = fmaf(pb, gv[d], dv[d]);
+                }
+            }
+        }
+#pragma unroll
+        for (int d = 0; d < D; ++d) { dk[d] = wave_sum(dk[d]); dv[d] = wave_sum(dv[d]); }
+        if (lane == 0) {
+            store_row<T, D>(dK + (((int64_t)g * S + ki) * H + h) * D, dk, scale);
+            store_row<T, D>(dV + (((int64_t)g * S + ki) * H + h) * D, dv, 1.0f);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // forward: online softmax over key tiles, in the base-2 domain
 // ---------------------------------------------------------------------------
 template <typename T, int D, int NT>
@@ -208,12 +382,14 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
     const int q0 = wave * 32, qi = q0 + col;
     const bool qok = qi < S;
     const bool hasb = bias != nullptr;
+    // a last tile of at most four rows is not worth a matrix tile: its wave takes the vector path
+    const bool vec_wave = wave == NT - 1 && S - (NT - 1) * 32 <= 4;
     // this lane's query row of the bias; the first tile's group of it is requested before anything else
     const T* brow = hasb ? bias + (((int64_t)g * H + h) * S + (qok ? qi : 0)) * S : nullptr;
     Bias16<T> bcur, bnext;
     zero_bias16(bcur);
     zero_bias16(bnext);
-    if (hasb && qok) load_bias16(brow + 16 * half, min(16, S - 16 * half), bcur);
+    if (hasb && qok && !vec_wave) load_bias16(brow + 16 * half, min(16, S - 16 * half), bcur);
     load_head<T, D, SP>(K, g, h, S, H, k_rm, nullptr);
     load_head<T, D, SP>(V, g, h, S, H, nullptr, v_tr);
     short4_t bq[KS];
@@ -223,6 +399,10 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
         if (qok) bq[s] = ld4(Q + (((int64_t)g * S + qi) * H + h) * D + s * 8 + half * 4);
     }
     __syncthreads();
+    if (vec_wave) {
+        thin_rows_fwd<T, D, SP>(Q, k_rm, v_tr, hasb ? bias + ((int64_t)g * H + h) * S * S : nullptr, out, lse, g, h, S, H,
+                                scale, (NT - 1) * 32, S - (NT - 1) * 32, lane);
+    } else {
     const int krow = key_of_row(col);            // key (inside a tile) of this lane's A-operand row
     // Row sums on the matrix unit: with a head dim below 32 the A operand of O^T = V^T P^T has idle
     // rows, and a row of ones there makes row D of the product the sum of the (bf16-rounded)
@@ -231,8 +411,11 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
     const short one_bits = 0x3f80;               // bf16 1.0
     float m = -INFINITY, l = 0.f;                // running maximum and sum (natural units)
     float16_t o = zero16();
+    const int tail = S - (NT - 1) * 32;          // keys in the last tile
+    const bool thin = tail <= 4;
+    const int nt_full = thin ? NT - 1 : NT;      // tiles that take the general path
 #pragma unroll 1
-    for (int kt = 0; kt < NT; ++kt) {
+    for (int kt = 0; kt < nt_full; ++kt) {
         const int kb = kt * 32 + 16 * half;      // this lane's keys: kb .. kb + 15
         if (kt + 1 < NT && hasb && qok) {        // the next tile's group, a whole tile ahead of its use
             const int nv = S - (kb + 32);
@@ -280,6 +463,42 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
         m = m_new;
         bcur = bnext;
         }
+    if (thin) {
+        constexpr int kt = NT - 1;
+        const int kb = kt * 32 + 16 * half;
+        float16_t sc = zero16();
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+        const short4_t a = *reinterpret_cast<const short4_t*>(&k_rm[(kt * 32 + krow) * D + s * 8 + half * 4]);
+        sc = mfma(a, bq[s], sc);
+        }
+        // the last tile holds at most four keys (a virtual node behind a multiple of 32): they are
+        // registers 0..3 of the lower half, one group of the second product instead of four
+        float s4[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s4[r] = (half == 0 && r < tail) ? fmaf(sc[r], scale, bcur.get(r)) : -INFINITY;
+        float tmax = fmaxf(max3(s4[0], s4[1], s4[2]), s4[3]);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+        const float m_new = fmaxf(m, tmax);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = fast_exp2((m - m_use) * kLog2e);
+        const float nm2 = -m_use * kLog2e;
+#pragma unroll
+        for (int r = 0; r < 4 * KS + (kSumOnMfma ? 4 : 0); ++r) o[r] *= alpha;
+        if (!kSumOnMfma) l *= alpha;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            s4[r] = fast_exp2(fmaf(s4[r], kLog2e, nm2));
+            if (!kSumOnMfma) l += s4[r];
+        }
+        short4_t pb;
+        pb.x = f2bf(s4[0]); pb.y = f2bf(s4[1]); pb.z = f2bf(s4[2]); pb.w = f2bf(s4[3]);
+        short4_t av = zero4();
+        if (col < D) av = *reinterpret_cast<const short4_t*>(&v_tr[col * (SP + 4) + kb]);
+        if (kSumOnMfma && col == D) { av.x = one_bits; av.y = one_bits; av.z = one_bits; av.w = one_bits; }
+        o = mfma(av, pb, o);
+        m = m_new;
+    }
     if (kSumOnMfma) l = __shfl(o[4 * KS], col);      // row D sits in the lower half's register 4*KS
     else l += __shfl_xor(l, 32);
     if (qok) {
@@ -290,6 +509,7 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
             st4(op + 8 * rb + 4 * half, o[4 * rb + 0] * inv, o[4 * rb + 1] * inv, o[4 * rb + 2] * inv,
                 o[4 * rb + 3] * inv);
         if (half == 0) lse[((int64_t)g * H + h) * S + qi] = (m == -INFINITY ? 0.f : m) + __logf(l);
+    }
     }
     __syncthreads();     // the LDS images are rewritten for the next pair
     }
@@ -331,6 +551,9 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int col = lane & 31, half = lane >> 5;
     const bool hasb = bias != nullptr;
+    const int tail = S - (NT - 1) * 32;          // rows / keys in the last tile
+    const bool thin = tail <= 4;
+    const int nt_full = thin ? NT - 1 : NT;      // tiles that take the general path
     const T* bias_gh = hasb ? bias + ((int64_t)g * H + h) * S * S : nullptr;
     // the first query-major group of this lane's bias row, requested before anything else
     const int qi = wave * 32 + col;
@@ -339,7 +562,8 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
     Bias16<T> bcur, bnext;
     zero_bias16(bcur);
     zero_bias16(bnext);
-    if (hasb && qok) load_bias16(brow + 16 * half, min(16, S - 16 * half), bcur);
+    const bool vec_wave = thin && wave == NT - 1;     // the wave of a last tile of at most four rows: vector path
+    if (hasb && qok && !vec_wave) load_bias16(brow + 16 * half, min(16, S - 16 * half), bcur);
     load_head<T, D, SP>(Q, g, h, S, H, q_rm, q_tr);
     load_head<T, D, SP>(K, g, h, S, H, k_rm, k_tr);
     load_head<T, D, SP>(V, g, h, S, H, v_rm, nullptr);
@@ -364,7 +588,11 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
     __syncthreads();
 
     // ---- query tile `wave`: dQ -------------------------------------------------
-    {
+    if (vec_wave) {
+        thin_rows_bwd_q<T, D, SP>(q_rm, k_rm, v_rm, g_rm, lse_l, dd_l, bias_gh,
+                                  dbias != nullptr ? dbias + ((int64_t)g * H + h) * S * S : nullptr, dQ, g, h, S, H, scale,
+                                  (NT - 1) * 32, tail, lane);
+    } else {
         short4_t bq[KS], bg[KS];
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
@@ -377,7 +605,7 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
         T* dbrow = dbias != nullptr ? dbias + (((int64_t)g * H + h) * S + (qok ? qi : 0)) * S : nullptr;
         float16_t dq = zero16();
 #pragma unroll 1
-        for (int kt = 0; kt < NT; ++kt) {
+        for (int kt = 0; kt < nt_full; ++kt) {
             const int kb = kt * 32 + 16 * half;
             if (kt + 1 < NT && hasb && qok) {
                 const int nv = S - (kb + 32);
@@ -430,6 +658,35 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
             }
             bcur = bnext;
         }
+        if (thin) {
+            constexpr int kt = NT - 1;
+            const int kb = kt * 32 + 16 * half;
+            float16_t sc = zero16(), dp = zero16();
+#pragma unroll
+            for (int s = 0; s < KS; ++s) {
+            const short4_t ak = *reinterpret_cast<const short4_t*>(&k_rm[(kt * 32 + krow) * D + s * 8 + half * 4]);
+            const short4_t av = *reinterpret_cast<const short4_t*>(&v_rm[(kt * 32 + krow) * D + s * 8 + half * 4]);
+            sc = mfma(ak, bq[s], sc);
+            dp = mfma(av, bg[s], dp);
+            }
+            // at most four keys in the last tile: registers 0..3 of the lower half
+            float s4[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float pv = fast_exp2(fmaf(sc[r], scale2, fmaf(bcur.get(r), kLog2e, nL2)));
+                s4[r] = (half == 0 && r < tail) ? pv * (dp[r] - Dq) : 0.f;
+            }
+            if (dbrow != nullptr && qok && half == 0) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (r < tail) st1(dbrow + kb + r, s4[r]);
+            }
+            short4_t db0;
+            db0.x = f2bf(s4[0]); db0.y = f2bf(s4[1]); db0.z = f2bf(s4[2]); db0.w = f2bf(s4[3]);
+            short4_t ak = zero4();
+            if (col < D) ak = *reinterpret_cast<const short4_t*>(&k_tr[col * (SP + 4) + kb]);
+            dq = mfma(ak, db0, dq);
+        }
         if (qok) {
             T* p = dQ + (((int64_t)g * S + qi) * H + h) * D;
 #pragma unroll
@@ -439,8 +696,11 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
         }
     }
 
-    // ---- key tile `wave`: dK, dV, dBias -----------------------------------------
-    {
+    // ---- key tile `wave`: dK, dV -------------------------------------------------
+    if (vec_wave) {
+        thin_rows_bwd_k<T, D, SP>(q_rm, k_rm, v_rm, g_rm, lse_l, dd_l, bias_gh, dK, dV, g, h, S, H, scale, (NT - 1) * 32, tail,
+                                  lane);
+    } else {
         const int k0 = wave * 32, ki = k0 + col;
         const bool kok = ki < S;
         short4_t bk[KS], bv[KS];
@@ -465,7 +725,7 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
         const float scale2 = scale * kLog2e;
         float16_t dk = zero16(), dv = zero16();
 #pragma unroll 1
-        for (int qt = 0; qt < NT; ++qt) {
+        for (int qt = 0; qt < nt_full; ++qt) {
             if (qt + 1 < NT && hasb && kok) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
@@ -520,6 +780,39 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
             }
 #pragma unroll
             for (int r = 0; r < 16; ++r) braw[r] = braw_next[r];
+        }
+        if (thin) {
+            constexpr int qt = NT - 1;
+            float16_t sc = zero16(), dp = zero16();
+#pragma unroll
+            for (int s = 0; s < KS; ++s) {
+            const short4_t aq = *reinterpret_cast<const short4_t*>(&q_rm[(qt * 32 + col) * D + s * 8 + half * 4]);
+            const short4_t ag = *reinterpret_cast<const short4_t*>(&g_rm[(qt * 32 + col) * D + s * 8 + half * 4]);
+            sc = mfma(aq, bk[s], sc);
+            dp = mfma(ag, bv[s], dp);
+            }
+            // at most four queries in the last tile: registers 0..3 of the lower half
+            const int qb = qt * 32 + 4 * half;
+            const float4_t L4 = *reinterpret_cast<const float4_t*>(&lse_l[qb]);
+            const float4_t D4 = *reinterpret_cast<const float4_t*>(&dd_l[qb]);
+            float p4[4], s4[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const bool in = half == 0 && t < tail;
+                const float pv = fast_exp2(fmaf(sc[t], scale2, fmaf(cvt1(braw[t]), kLog2e, -L4[t])));
+                p4[t] = in ? pv : 0.f;
+                s4[t] = in ? pv * (dp[t] - D4[t]) : 0.f;
+            }
+            short4_t db, pb;
+            db.x = f2bf(s4[0]); db.y = f2bf(s4[1]); db.z = f2bf(s4[2]); db.w = f2bf(s4[3]);
+            pb.x = f2bf(p4[0]); pb.y = f2bf(p4[1]); pb.z = f2bf(p4[2]); pb.w = f2bf(p4[3]);
+            short4_t aq = zero4(), ag = zero4();
+            if (col < D) {
+                aq = *reinterpret_cast<const short4_t*>(&q_tr[col * (SP + 4) + qt * 32 + half * 4]);
+                ag = *reinterpret_cast<const short4_t*>(&g_tr[col * (SP + 4) + qt * 32 + half * 4]);
+            }
+            dk = mfma(aq, db, dk);
+            dv = mfma(ag, pb, dv);
         }
         if (kok) {
             T* pk = dK + (((int64_t)g * S + ki) * H + h) * D;
