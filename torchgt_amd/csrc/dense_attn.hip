@@ -469,8 +469,8 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
         float16_t sc = zero16();
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
-        const short4_t a = *reinterpret_cast<const short4_t*>(&k_rm[(kt * 32 + krow) * D + s * 8 + half * 4]);
-        sc = mfma(a, bq[s], sc);
+            const short4_t a = *reinterpret_cast<const short4_t*>(&k_rm[(kt * 32 + krow) * D + s * 8 + half * 4]);
+            sc = mfma(a, bq[s], sc);
         }
         // the last tile holds at most four keys (a virtual node behind a multiple of 32): they are
         // registers 0..3 of the lower half, one group of the second product instead of four
@@ -664,10 +664,10 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
             float16_t sc = zero16(), dp = zero16();
 #pragma unroll
             for (int s = 0; s < KS; ++s) {
-            const short4_t ak = *reinterpret_cast<const short4_t*>(&k_rm[(kt * 32 + krow) * D + s * 8 + half * 4]);
-            const short4_t av = *reinterpret_cast<const short4_t*>(&v_rm[(kt * 32 + krow) * D + s * 8 + half * 4]);
-            sc = mfma(ak, bq[s], sc);
-            dp = mfma(av, bg[s], dp);
+                const short4_t ak = *reinterpret_cast<const short4_t*>(&k_rm[(kt * 32 + krow) * D + s * 8 + half * 4]);
+                const short4_t av = *reinterpret_cast<const short4_t*>(&v_rm[(kt * 32 + krow) * D + s * 8 + half * 4]);
+                sc = mfma(ak, bq[s], sc);
+                dp = mfma(av, bg[s], dp);
             }
             // at most four keys in the last tile: registers 0..3 of the lower half
             float s4[4];
@@ -786,10 +786,10 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
             float16_t sc = zero16(), dp = zero16();
 #pragma unroll
             for (int s = 0; s < KS; ++s) {
-            const short4_t aq = *reinterpret_cast<const short4_t*>(&q_rm[(qt * 32 + col) * D + s * 8 + half * 4]);
-            const short4_t ag = *reinterpret_cast<const short4_t*>(&g_rm[(qt * 32 + col) * D + s * 8 + half * 4]);
-            sc = mfma(aq, bk[s], sc);
-            dp = mfma(ag, bv[s], dp);
+                const short4_t aq = *reinterpret_cast<const short4_t*>(&q_rm[(qt * 32 + col) * D + s * 8 + half * 4]);
+                const short4_t ag = *reinterpret_cast<const short4_t*>(&g_rm[(qt * 32 + col) * D + s * 8 + half * 4]);
+                sc = mfma(aq, bk[s], sc);
+                dp = mfma(ag, bv[s], dp);
             }
             // at most four queries in the last tile: registers 0..3 of the lower half
             const int qb = qt * 32 + 4 * half;
