@@ -27,6 +27,12 @@ relabel_by_partition           hand-computed known answer
 blockize / reformat_graph      hand-computed known answer (k=1, N=32, bs=16)
                                + structural invariants
 build_csr                      numpy stable argsort + round-trip invariants
+graph_attn_bias_multi_hop      reduces to graph_attn_bias (one hop, identity
+                               hop matrices, adjacent pairs); fp64 loops from
+                               the definition; halves when the distance doubles
+gen_edge_input                 hand-computed known answer (path graph); every
+                               row is a walk of existing edges from i to j of
+                               the shortest length (scipy)
 metis partition labels         PARITY UNPINNED: dgl/METIS is absent; partition
                                ids are always an explicit input here
 =============================  ================================================

@@ -3,7 +3,7 @@
 Restates ``CoreAttention.forward`` of ``models/graphormer_graph_level.py:186-214``
 (same body: ``attn_module.py:99-127``, ``graphormer_dist_graph_level.py:211-235``)
 and the bias producer ``GraphAttnBias.forward``
-(``models/graphormer_graph_level.py:94-156``, edge_type != 'multi_hop' branch).
+(``models/graphormer_graph_level.py:94-156``, both edge-type branches).
 """
 import math
 
@@ -53,6 +53,40 @@ def graph_attn_bias(attn_bias, spatial_pos, attn_edge_type, spatial_table, edge_
     g[:, :, 0, :] = g[:, :, 0, :] + t                                 # :117
     ei = edge_table[attn_edge_type].mean(-2).permute(0, 3, 1, 2)      # :150
     g[:, :, 1:, 1:] = g[:, :, 1:, 1:] + ei                            # :152
+    g = g + attn_bias.unsqueeze(1)                                    # :153
+    return g
+
+
+def graph_attn_bias_multi_hop(attn_bias, spatial_pos, edge_input, spatial_table, edge_table, edge_dis_weight, virtual_dist,
+                              multi_hop_max_dist):
+    """``GraphAttnBias.forward`` (graphormer_graph_level.py:94-156), edge_type == 'multi_hop'
+    (:119-147), op for op.
+
+    edge_input       [b, S, S, D0, F] int64 (features of the edges on the shortest path + 1, 0 = none)
+    edge_dis_weight  [num_edge_dis * H * H, 1] (the weight of ``edge_dis_encoder``)
+    the other arguments as in ``graph_attn_bias``.  Returns [b, H, S+1, S+1].
+    """
+    H = spatial_table.shape[1]
+    n_graph, n_node = spatial_pos.shape[:2]
+    g = attn_bias.clone().unsqueeze(1).repeat(1, H, 1, 1)             # :104-107
+    sp = spatial_table[spatial_pos].permute(0, 3, 1, 2)               # :110
+    g[:, :, 1:, 1:] = g[:, :, 1:, 1:] + sp                            # :111
+    t = virtual_dist.view(1, H, 1)                                    # :115
+    g[:, :, 1:, 0] = g[:, :, 1:, 0] + t                               # :116
+    g[:, :, 0, :] = g[:, :, 0, :] + t                                 # :117
+    sp_ = spatial_pos.clone()                                         # :121
+    sp_[sp_ == 0] = 1                                                 # :122
+    sp_ = torch.where(sp_ > 1, sp_ - 1, sp_)                          # :124
+    if multi_hop_max_dist > 0:
+        sp_ = sp_.clamp(0, multi_hop_max_dist)                        # :126
+        edge_input = edge_input[:, :, :, :multi_hop_max_dist, :]      # :127
+    e = edge_table[edge_input].mean(-2)                               # :129  [b, S, S, D, H]
+    max_dist = e.size(-2)
+    flat = e.permute(3, 0, 1, 2, 4).reshape(max_dist, -1, H)          # :131-133
+    flat = torch.bmm(flat, edge_dis_weight.reshape(-1, H, H)[:max_dist, :, :])     # :134-139
+    e = flat.reshape(max_dist, n_graph, n_node, n_node, H).permute(1, 2, 3, 0, 4)  # :141-143
+    e = (e.sum(-2) / (sp_.to(e.dtype).unsqueeze(-1))).permute(0, 3, 1, 2)          # :145-147
+    g[:, :, 1:, 1:] = g[:, :, 1:, 1:] + e                             # :152
     g = g + attn_bias.unsqueeze(1)                                    # :153
     return g
 

@@ -204,3 +204,34 @@ def floyd_warshall(adjacency_matrix):
     path[far] = FW_UNREACHABLE
     M[far] = FW_UNREACHABLE
     return M, path
+
+
+def get_all_edges(path, i, j):
+    """data/algos.pyx:56-61: the intermediate nodes of the recorded shortest path from i to j."""
+    k = int(path[i][j])
+    if k == -1:
+        return []
+    return get_all_edges(path, i, k) + [k] + get_all_edges(path, k, j)
+
+
+def gen_edge_input(max_dist, path, edge_feat):
+    """data/algos.pyx:64-92, loop for loop.  ``path`` [n, n] from ``floyd_warshall``, ``edge_feat``
+    [n, n, F] integer features of the direct edges.  Returns int64 [n, n, max_dist, F]: entry
+    (i, j, k) = features of the k-th edge on the recorded shortest path from i to j, -1 where there
+    is none (i == j, unreachable pairs, hops past the end of the path).  The reference sizes
+    max_dist to the longest path, so every hop fits; hops at or beyond max_dist are dropped here."""
+    path = np.asarray(path, dtype=np.int64)
+    edge_feat = np.asarray(edge_feat, dtype=np.int64)
+    n = path.shape[0]
+    assert path.shape == (n, n)
+    out = -np.ones((n, n, int(max_dist), edge_feat.shape[-1]), dtype=np.int64)     # :77
+    for i in range(n):
+        for j in range(n):
+            if i == j:                                   # :82
+                continue
+            if path[i][j] == FW_UNREACHABLE:             # :84
+                continue
+            nodes = [i] + get_all_edges(path, i, j) + [j]   # :86
+            for k in range(min(len(nodes) - 1, int(max_dist))):
+                out[i, j, k, :] = edge_feat[nodes[k], nodes[k + 1], :]             # :89
+    return out

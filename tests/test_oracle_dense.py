@@ -54,3 +54,67 @@ def test_graph_attn_bias_against_loops():
                         x = x + vd[0, h]
                     got = out[gi, h, i, j]
                     assert (torch.isinf(x) and torch.isinf(got)) or abs(float(got - x)) < 1e-12
+
+
+def _multi_hop_case(seed, b=2, S=5, H=3, D0=4, F=2, ne=6, nsp=9):
+    g = torch.Generator().manual_seed(seed)
+    attn_bias = torch.zeros(b, S + 1, S + 1, dtype=torch.float64)
+    attn_bias[1, :, S:] = float("-inf")
+    spatial_pos = torch.randint(0, nsp, (b, S, S), generator=g)
+    edge_input = torch.randint(0, ne, (b, S, S, D0, F), generator=g)
+    st = torch.randn(nsp, H, generator=g, dtype=torch.float64)
+    et = torch.randn(ne, H, generator=g, dtype=torch.float64)
+    w = torch.randn(7 * H * H, 1, generator=g, dtype=torch.float64)
+    vd = torch.randn(1, H, generator=g, dtype=torch.float64)
+    return attn_bias, spatial_pos, edge_input, st, et, w, vd
+
+
+def test_multi_hop_bias_matches_loops_from_the_definition():
+    for mhd in (3, 0, 6):       # fewer hops than the input holds, no limit, more
+        attn_bias, sp, ei, st, et, w, vd = _multi_hop_case(mhd)
+        got = oda.graph_attn_bias_multi_hop(attn_bias, sp, ei, st, et, w, vd, mhd)
+        b, S = sp.shape[:2]
+        H, D0, F = st.shape[1], ei.shape[3], ei.shape[4]
+        D = min(D0, mhd) if mhd > 0 else D0
+        W = w.reshape(-1, H, H)
+        want = torch.zeros(b, H, S + 1, S + 1, dtype=torch.float64)
+        for g in range(b):
+            for h in range(H):
+                for i in range(S + 1):
+                    for j in range(S + 1):
+                        x = 2 * attn_bias[g, i, j]
+                        if i == 0 or j == 0:
+                            x = x + vd[0, h]
+                        else:
+                            p = int(sp[g, i - 1, j - 1])
+                            x = x + st[p, h]
+                            hops = 1 if p <= 1 else p - 1            # pad -> 1, distance + 1 -> distance, self -> 1
+                            if mhd > 0:
+                                hops = min(hops, mhd)
+                            acc = 0.0
+                            for dd in range(D):
+                                for h0 in range(H):
+                                    mean = sum(et[int(ei[g, i - 1, j - 1, dd, f]), h0] for f in range(F)) / F
+                                    acc = acc + mean * W[dd, h0, h]
+                            x = x + acc / hops
+                        want[g, h, i, j] = x
+        fin = torch.isfinite(want)
+        assert torch.equal(torch.isfinite(got), fin)
+        torch.testing.assert_close(got[fin], want[fin], rtol=1e-11, atol=1e-12)
+
+
+def test_multi_hop_bias_reduces_to_the_single_hop_branch():
+    # one hop, identity hop matrix, every pair adjacent (or self / pad): the path encoding is the edge encoding
+    attn_bias, sp, ei, st, et, w, vd = _multi_hop_case(5)
+    H = st.shape[1]
+    sp = sp.clamp(0, 2)
+    w = torch.eye(H, dtype=torch.float64).repeat(7, 1, 1).reshape(-1, 1)
+    got = oda.graph_attn_bias_multi_hop(attn_bias, sp, ei, st, et, w, vd, 1)
+    want = oda.graph_attn_bias(attn_bias, sp, ei[:, :, :, 0, :], st, et, vd)
+    fin = torch.isfinite(want)
+    torch.testing.assert_close(got[fin], want[fin], rtol=1e-12, atol=1e-13)
+    # twice the distance halves the edge term: spatial_pos 3 (two hops) against 2 (one hop), zero spatial table
+    z = torch.zeros_like(st)
+    a1 = oda.graph_attn_bias_multi_hop(torch.zeros_like(attn_bias), torch.full_like(sp, 2), ei, z, et, w, vd * 0, 0)
+    a2 = oda.graph_attn_bias_multi_hop(torch.zeros_like(attn_bias), torch.full_like(sp, 3), ei, z, et, w, vd * 0, 0)
+    torch.testing.assert_close(a1[:, :, 1:, 1:], 2 * a2[:, :, 1:, 1:], rtol=1e-12, atol=1e-13)

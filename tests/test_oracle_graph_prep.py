@@ -194,3 +194,50 @@ def test_floyd_warshall_known_answer_and_scipy():
                     assert M[i, j] == M[i, k] + M[k, j]
                 elif k == -1:
                     assert i == j or a[i, j] == 1
+
+
+def test_gen_edge_input_known_answer_and_walk_property():
+    # path graph 0-1-2-3 plus an isolated node 4; the feature of edge (a, b) is (10 a + b, 7)
+    n = 5
+    adj = np.zeros((n, n), dtype=np.int64)
+    for a, b in ((0, 1), (1, 2), (2, 3)):
+        adj[a, b] = adj[b, a] = 1
+    feat = np.zeros((n, n, 2), dtype=np.int64)
+    for a in range(n):
+        for b in range(n):
+            if adj[a, b]:
+                feat[a, b] = (10 * a + b, 7)
+    M, path = gp.floyd_warshall(adj)
+    out = gp.gen_edge_input(3, path, feat)
+    assert out.shape == (n, n, 3, 2) and out.dtype == np.int64
+    np.testing.assert_array_equal(out[0, 3], [[1, 7], [12, 7], [23, 7]])      # 0-1, 1-2, 2-3
+    np.testing.assert_array_equal(out[3, 0], [[32, 7], [21, 7], [10, 7]])     # 3-2, 2-1, 1-0
+    np.testing.assert_array_equal(out[1, 2], [[12, 7], [-1, -1], [-1, -1]])
+    assert (out[2, 2] == -1).all() and (out[0, 4] == -1).all() and (out[4, 1] == -1).all()
+    # a smaller max_dist keeps the first hops
+    np.testing.assert_array_equal(gp.gen_edge_input(2, path, feat)[0, 3], [[1, 7], [12, 7]])
+    # random graphs: the hops of (i, j) form a walk of existing edges from i to j of the shortest length
+    rng = np.random.default_rng(1)
+    for n in (9, 24):
+        a = (rng.random((n, n)) < 0.15).astype(np.int64)
+        a = np.maximum(a, a.T)
+        np.fill_diagonal(a, 0)
+        M, path = gp.floyd_warshall(a)
+        code = np.zeros((n, n, 1), dtype=np.int64)             # the feature names the edge: a * n + b
+        code[:, :, 0] = np.arange(n)[:, None] * n + np.arange(n)[None, :]
+        md = int(M[M < 510].max())
+        out = gp.gen_edge_input(md, path, code)
+        for i in range(n):
+            for j in range(n):
+                hops = out[i, j, :, 0]
+                real = hops[hops >= 0]
+                if i == j or M[i, j] == 510:
+                    assert real.size == 0
+                    continue
+                assert real.size == M[i, j] and (hops[:real.size] >= 0).all()
+                cur = i
+                for h in real:
+                    s_, t_ = divmod(int(h), n)
+                    assert s_ == cur and a[s_, t_] == 1
+                    cur = t_
+                assert cur == j
