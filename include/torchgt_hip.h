@@ -330,6 +330,39 @@ int tgt_graph_attn_bias_bwd(const void* d_dout, const int64_t* d_spatial_pos, co
                             int num_spatial, int num_edges, int b, int s, int H, int dtype, void* d_dspatial_table,
                             void* d_dedge_table, void* d_dvirtual_dist, void* d_workspace, int64_t workspace_bytes,
                             void* stream);
+/* GraphAttnBias.forward with edge_type == 'multi_hop' (models/graphormer_graph_level.py:94-156,
+ * the path-encoding branch :119-147).  As tgt_graph_attn_bias_fwd, with the edge term replaced by
+ *   (1 / hops) * sum_dd  mean_f edge_table[edge_input[g,i-1,j-1,dd,f]]  x  W[dd]        (i, j >= 1)
+ * where W = edge_dis_weight viewed as [num_edge_dis, H, H] (:137), dd runs over the first
+ * D = min(D0, multi_hop_max_dist) hops (all D0 when multi_hop_max_dist is 0; :125-127) and
+ * hops = 1 for spatial ids 0 and 1, id - 1 above, at most multi_hop_max_dist when that is set
+ * (:121-126).  d_edge_input: int64 [b, s, s, D0, F]; d_edge_dis_weight: [num_edge_dis * H * H]
+ * of `dtype`.  D must not exceed num_edge_dis (the reference's bmm would raise); H <= 32. */
+int tgt_graph_attn_bias_multi_hop_fwd(const void* d_attn_bias, const int64_t* d_spatial_pos, const int64_t* d_edge_input, int D0,
+                                      int F, const void* d_spatial_table, int num_spatial, const void* d_edge_table,
+                                      int num_edges, const void* d_edge_dis_weight, int num_edge_dis, const void* d_virtual_dist,
+                                      int multi_hop_max_dist, int b, int s, int H, int dtype, void* d_out, void* stream);
+/* Gradients of the four parameter tensors of that branch for the upstream gradient d_dout
+ * [b, H, S1, S1] (autograd in the reference): spatial table, edge table (row 0 of both is the
+ * padding index and gets zero), the hop matrices ([num_edge_dis * H * H]; matrices beyond the D
+ * hops in use get zero) and the virtual distance.  Workgroup sums are formed in LDS (floating-point
+ * atomics) and added in a fixed order: results agree to rounding between runs, not bit for bit.
+ * D = min(D0, multi_hop_max_dist) (D0 when the limit is 0) sizes the workspace. */
+int64_t tgt_graph_attn_bias_multi_hop_bwd_workspace_bytes(int num_spatial, int num_edges, int H, int D);
+int tgt_graph_attn_bias_multi_hop_bwd(const void* d_dout, const int64_t* d_spatial_pos, const int64_t* d_edge_input, int D0, int F,
+                                      const void* d_edge_table, int num_spatial, int num_edges, const void* d_edge_dis_weight,
+                                      int num_edge_dis, int multi_hop_max_dist, int b, int s, int H, int dtype,
+                                      void* d_dspatial_table, void* d_dedge_table, void* d_dedge_dis_weight,
+                                      void* d_dvirtual_dist, void* d_workspace, int64_t workspace_bytes, void* stream);
+/* gen_edge_input (data/algos.pyx:64-92) for a batch of graphs of at most 128 nodes.
+ * d_path: int32 [num_graphs, n_max, n_max] as tgt_floyd_warshall writes it; d_edge_feat:
+ * [num_graphs, n_max, n_max, F], int64 (feat_is_int64 != 0) or int32; d_n_nodes as there.
+ * d_out: int64 [num_graphs, n_max, n_max, max_dist, F]; entry (i, j, k) = features of the k-th
+ * edge on the recorded shortest path from i to j (the reference's recursive expansion of the
+ * intermediate nodes, :56-61), -1 where there is none: i == j, unreachable pairs, hops past the
+ * end of the path, padding nodes.  Hops at or beyond max_dist are dropped. */
+int tgt_gen_edge_input(const int32_t* d_path, const void* d_edge_feat, int feat_is_int64, int F, const int32_t* d_n_nodes,
+                       int num_graphs, int n_max, int max_dist, int64_t* d_out, void* stream);
 /* floyd_warshall (data/algos.pyx:9-54) for a batch of graphs of at most 128 nodes.
  * d_adj: uint8 [num_graphs, n_max, n_max], entry = edge weight, 0 = no edge;
  * d_n_nodes: int32 [num_graphs] node counts (NULL: all n_max).  d_dist, d_path:

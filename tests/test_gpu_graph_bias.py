@@ -1,5 +1,6 @@
-"""GPU parity of GraphAttnBias (forward and table gradients) and of the Floyd-Warshall
-kernel with the oracle.  Floyd-Warshall is integer work: bit-exact.  The bias is a sum of
+"""GPU parity of GraphAttnBias (both edge-type branches, forward and parameter gradients), of the
+Floyd-Warshall kernel and of gen_edge_input with the oracle.  Floyd-Warshall and gen_edge_input are
+integer work: bit-exact.  The bias is a sum of
 table entries: float32 1e-5 / bf16 2e-2 on max|a-b| / max|b| (finite entries; -inf stays -inf).
 """
 import types
@@ -10,7 +11,7 @@ import torch
 
 from oracle import dense_attention as oda
 from oracle import graph_prep as ogp
-from torchgt_amd import GraphAttnBias, _lib, floyd_warshall, workloads
+from torchgt_amd import GraphAttnBias, _lib, floyd_warshall, gen_edge_input, workloads
 
 pytestmark = pytest.mark.gpu
 TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2}
@@ -119,7 +120,125 @@ def test_graph_attn_bias_matches_oracle(cuda, dtype, H, F):
     assert not got_g[0][0].any() and not got_g[1][0].any()              # padding index rows get no gradient
 
 
-def test_graph_attn_bias_multi_hop_is_not_built(cuda):
-    m = GraphAttnBias(8, 512, 5, 22, 128, 64, "multi_hop", 5)
-    with pytest.raises(NotImplementedError):
-        m(types.SimpleNamespace())
+def _edge_input_of_batch(data, F, max_dist):
+    """Shortest-path edge features of the configuration-4 style batch through the oracle's Floyd-Warshall and
+    gen_edge_input, in the collator's conventions (features + 1, 0 = padding; data/collator.py:59-66)."""
+    sizes = data["n_nodes"]
+    b, s = len(sizes), data["spatial_pos"].shape[1]
+    et1 = data["edge_type"].astype(np.int64)                              # [b, s, s], 0 = no edge
+    edge_input = np.zeros((b, s, s, max_dist, F), dtype=np.int64)
+    for g in range(b):
+        n = int(sizes[g])
+        adj = (data["spatial_pos"][g][:n, :n] == 2).astype(np.int64)
+        feat = np.stack([(et1[g, :n, :n] * (f + 1)) % 4 for f in range(F)], -1) * adj[:, :, None]    # 0..3, ids 1..4
+        _, path = ogp.floyd_warshall(adj)
+        edge_input[g, :n, :n] = ogp.gen_edge_input(max_dist, path, feat) + 1
+    return edge_input
+
+
+# (heads, edge features, hops held by the input, hop limit): eight heads, fewer, sixteen and thirty-two (the wider
+# head tiles); a limit below, at and above the hops the input holds, and no limit
+@pytest.mark.parametrize("H,F,D0,mhd", [(8, 1, 5, 5), (8, 3, 6, 4), (4, 2, 3, 0), (16, 1, 4, 6), (32, 1, 3, 2), (8, 2, 10, 0)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_graph_attn_bias_multi_hop_matches_oracle(cuda, dtype, H, F, D0, mhd):
+    print(f"multi_hop bias case: H={H} F={F} D0={D0} multi_hop_max_dist={mhd} {dtype}", flush=True)
+    data = workloads.erdos_renyi_batch(batch=8, seed=7)
+    g = torch.Generator().manual_seed(2)
+    n_dis = 12
+    m = GraphAttnBias(H, 512, 5, 22, n_dis, 64, "multi_hop", mhd)
+    with torch.no_grad():
+        m.spatial_pos_encoder.weight.normal_(0, 0.5, generator=g); m.spatial_pos_encoder.weight[0] = 0
+        m.edge_encoder.weight.normal_(0, 0.5, generator=g); m.edge_encoder.weight[0] = 0
+        m.edge_dis_encoder.weight.normal_(0, 0.5, generator=g)
+        m.graph_token_virtual_distance.weight.normal_(0, 0.5, generator=g)
+    assert sorted(n for n, _ in m.named_parameters()) == ["edge_dis_encoder.weight", "edge_encoder.weight",
+                                                          "graph_token_virtual_distance.weight", "spatial_pos_encoder.weight"]
+    assert m.edge_dis_encoder.weight.shape == (n_dis * H * H, 1)
+    m = m.to(dtype)
+    attn_bias = torch.from_numpy(data["attn_bias"])
+    spatial_pos = torch.from_numpy(data["spatial_pos"]).long()
+    edge_input = torch.from_numpy(_edge_input_of_batch(data, F, D0))
+    assert int(edge_input.max()) > 0 and int(spatial_pos.max()) > 4           # paths of several hops occur
+    params = [p.detach().double().requires_grad_(True) for p in (m.spatial_pos_encoder.weight, m.edge_encoder.weight,
+                                                                 m.edge_dis_encoder.weight, m.graph_token_virtual_distance.weight)]
+    st, et, wd, vd = params
+    want = oda.graph_attn_bias_multi_hop(attn_bias.double(), spatial_pos, edge_input, st, et, wd, vd, mhd)
+    mc = m.to(cuda)
+    batch = types.SimpleNamespace(attn_bias=attn_bias.to(cuda), spatial_pos=spatial_pos.to(cuda), edge_input=edge_input.to(cuda),
+                                  attn_edge_type=None)
+    got = mc(batch)
+    assert got.shape == want.shape and got.dtype == dtype
+    assert err(got, want) <= TOL[dtype], err(got, want)
+    dout = torch.randn(want.shape, generator=g)
+    dout[~torch.isfinite(want)] = 0
+    dout = dout.to(dtype)
+    finite = torch.where(torch.isfinite(want), want, torch.zeros_like(want))
+    ref = [r.clone() for r in torch.autograd.grad((finite * dout.double()).sum(), params)]
+    ref[0][0] = 0                                  # nn.Embedding(padding_idx=0): row 0 gets no gradient
+    ref[1][0] = 0
+    got_g = torch.autograd.grad(got, [mc.spatial_pos_encoder.weight, mc.edge_encoder.weight, mc.edge_dis_encoder.weight,
+                                      mc.graph_token_virtual_distance.weight], dout.to(cuda))
+    for nm, a, r in zip(("spatial", "edge", "hop matrices", "virtual"), got_g, ref):
+        assert a.shape == r.shape
+        assert err(a, r) <= TOL[dtype], f"d{nm} err {err(a, r)}"
+    assert not got_g[0][0].any() and not got_g[1][0].any()
+    D = min(D0, mhd) if mhd > 0 else D0
+    assert not got_g[2].reshape(n_dis, H, H)[D:].any() and got_g[2].reshape(n_dis, H, H)[:D].any()
+
+
+def test_graph_attn_bias_multi_hop_rejects_more_hops_than_matrices(cuda):
+    m = GraphAttnBias(8, 512, 5, 22, 2, 64, "multi_hop", 0).to(cuda)       # two hop matrices, three hops of input
+    batch = types.SimpleNamespace(attn_bias=torch.zeros(1, 4, 4, device=cuda), spatial_pos=torch.ones(1, 3, 3, dtype=torch.long, device=cuda),
+                                  edge_input=torch.zeros(1, 3, 3, 3, 1, dtype=torch.long, device=cuda))
+    with pytest.raises(_lib.TorchGTHipError) as ei:
+        m(batch)
+    assert ei.value.code == _lib.ERR_INVALID_ARG
+
+
+def test_gen_edge_input_matches_oracle_bit_for_bit(cuda):
+    rng = np.random.default_rng(4)
+    # single graphs, the reference's call shape (max_dist = the longest distance, 510 when a pair is unreachable:
+    # data/wrapper.py passes np.amax of the distance matrix)
+    for n, p, F in ((1, 0.0, 1), (6, 0.4, 2), (23, 0.12, 3), (64, 0.06, 1), (128, 0.03, 2)):
+        a = (rng.random((n, n)) < p).astype(np.int64)
+        a = np.maximum(a, a.T)
+        np.fill_diagonal(a, 0)
+        feat = rng.integers(1, 9, size=(n, n, F)) * a[:, :, None]
+        M, path = ogp.floyd_warshall(a)
+        reach = M[M < 510]
+        for max_dist in sorted({int(reach.max()) if reach.size else 0, 2, 5}):
+            print(f"gen_edge_input case: n={n} p={p} F={F} max_dist={max_dist}", flush=True)
+            want = ogp.gen_edge_input(max_dist, path, feat)
+            got = gen_edge_input(max_dist, path, feat)
+            assert got.dtype == np.int64 and got.shape == want.shape
+            np.testing.assert_array_equal(got, want)
+    # directed graph: paths and features are not symmetric
+    a = (rng.random((40, 40)) < 0.08).astype(np.int64)
+    np.fill_diagonal(a, 0)
+    feat = rng.integers(1, 100, size=(40, 40, 2)) * a[:, :, None]
+    M, path = ogp.floyd_warshall(a)
+    np.testing.assert_array_equal(gen_edge_input(7, path, feat), ogp.gen_edge_input(7, path, feat))
+    # the GPU chain: Floyd-Warshall then gen_edge_input on a padded batch
+    data = workloads.erdos_renyi_batch(batch=10, seed=5)
+    sizes = data["n_nodes"]
+    n_max = int(sizes.max())
+    adj = np.zeros((10, n_max, n_max), dtype=np.uint8)
+    feat = np.zeros((10, n_max, n_max, 1), dtype=np.int64)
+    for g in range(10):
+        n = int(sizes[g])
+        adj[g, :n, :n] = data["spatial_pos"][g][:n, :n] == 2
+        feat[g, :n, :n, 0] = data["edge_type"][g][:n, :n] * adj[g, :n, :n]
+    dist, path = floyd_warshall(torch.from_numpy(adj), sizes)
+    got = gen_edge_input(6, path, torch.from_numpy(feat).to(path.device), sizes)
+    assert got.is_cuda and got.shape == (10, n_max, n_max, 6, 1)
+    for g in range(10):
+        n = int(sizes[g])
+        _, path_ref = ogp.floyd_warshall(adj[g, :n, :n])
+        np.testing.assert_array_equal(got[g, :n, :n].cpu().numpy(), ogp.gen_edge_input(6, path_ref, feat[g, :n, :n]))
+        assert (got[g, n:] == -1).all() and (got[g, :, n:] == -1).all()
+
+
+def test_gen_edge_input_rejects_large_graphs(cuda):
+    with pytest.raises(_lib.TorchGTHipError) as ei:
+        gen_edge_input(3, np.zeros((129, 129), dtype=np.int64), np.zeros((129, 129, 1), dtype=np.int64))
+    assert ei.value.code == _lib.ERR_UNSUPPORTED

@@ -70,6 +70,12 @@ SIGNATURES = {
     "tgt_graph_attn_bias_bwd_workspace_bytes": (_i64, [_i32, _i32, _i32]),
     "tgt_graph_attn_bias_bwd": (_i32, [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _i64, _vp]),
     "tgt_floyd_warshall": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp, _vp]),
+    "tgt_graph_attn_bias_multi_hop_fwd": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp, _i32, _vp, _i32, _vp, _i32, _vp, _i32, _i32, _i32,
+                                                 _i32, _i32, _vp, _vp]),
+    "tgt_graph_attn_bias_multi_hop_bwd_workspace_bytes": (_i64, [_i32, _i32, _i32, _i32]),
+    "tgt_graph_attn_bias_multi_hop_bwd": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp, _i32, _i32, _vp, _i32, _i32, _i32, _i32, _i32, _i32,
+                                                 _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
+    "tgt_gen_edge_input": (_i32, [_vp, _vp, _i32, _i32, _vp, _i32, _i32, _i32, _vp, _vp]),
     "tgt_probe_row_gather": (_i32, [_vp, _i64, _i32, _vp, _i64, _vp, _vp]),
     "tgt_timing_enable": (_i32, [_i32]),
     "tgt_timing_reset": (_i32, []),

@@ -1,11 +1,13 @@
-"""``GraphAttnBias`` and ``floyd_warshall`` on the library's kernels.
+"""``GraphAttnBias``, ``floyd_warshall`` and ``gen_edge_input`` on the library's kernels.
 
 Mirrors of models/graphormer_graph_level.py:63-156 (``GraphAttnBias``: same
 constructor, same embedding parameter names, ``forward(batched_data)``) and of
-data/algos.pyx:9-54 (``floyd_warshall``).  The bias is built by one kernel from
-the id tensors and the three embedding tables; its backward reduces the bias
-gradient into the tables.  ``edge_type='multi_hop'`` (the path-encoding branch,
-:119-147) is not built and raises.
+data/algos.pyx:9-54 (``floyd_warshall``) and :64-92 (``gen_edge_input``).  The
+bias is built by one kernel from the id tensors and the embedding tables; its
+backward reduces the bias gradient into the tables.  Both edge-type branches are
+built: the plain one (mean of the edge-type embeddings, :148-150) and
+``edge_type='multi_hop'`` (embeddings of the edges along the shortest path, one
+H x H matrix per hop, :119-147).
 """
 import numpy as np
 import torch
@@ -61,6 +63,57 @@ class GraphAttnBiasFunction(torch.autograd.Function):
         return None, None, None, d_sp, d_e, d_v.view(vshape)
 
 
+class GraphAttnBiasMultiHopFunction(torch.autograd.Function):
+    """The 'multi_hop' branch (graphormer_graph_level.py:119-147) with gradients for the four parameter tensors."""
+
+    @staticmethod
+    def forward(ctx, attn_bias, spatial_pos, edge_input, spatial_table, edge_table, edge_dis_weight, virtual_dist,
+                multi_hop_max_dist):
+        if not attn_bias.is_cuda:
+            raise RuntimeError("GraphAttnBias runs on the GPU only (no CPU fallback)")
+        dt = spatial_table.dtype
+        if dt not in _DT:
+            raise TypeError(f"unsupported dtype {dt}")
+        b, S1 = attn_bias.shape[0], attn_bias.shape[1]
+        s, H = S1 - 1, spatial_table.shape[1]
+        D0, F = edge_input.shape[-2], edge_input.shape[-1]
+        mhd = int(multi_hop_max_dist)
+        ab = attn_bias.to(dt).contiguous()
+        sp = spatial_pos.to(torch.int64).contiguous()
+        ei = edge_input.to(torch.int64).contiguous()
+        st_, e_, v_ = spatial_table.contiguous(), edge_table.contiguous(), virtual_dist.reshape(-1).contiguous()
+        w_ = edge_dis_weight.to(dt).reshape(-1).contiguous()
+        n_dis = w_.numel() // (H * H)
+        out = torch.empty((b, H, S1, S1), dtype=dt, device=ab.device)
+        with torch.cuda.device(ab.device):
+            _lib.check(_lib.lib().tgt_graph_attn_bias_multi_hop_fwd(
+                ab.data_ptr(), sp.data_ptr(), ei.data_ptr(), D0, F, st_.data_ptr(), st_.shape[0], e_.data_ptr(), e_.shape[0],
+                w_.data_ptr(), n_dis, v_.data_ptr(), mhd, b, s, H, _DT[dt], out.data_ptr(), _stream(ab)))
+        ctx.save_for_backward(sp, ei, e_, w_)
+        ctx.dims = (b, s, H, F, D0, st_.shape[0], e_.shape[0], n_dis, mhd, dt, virtual_dist.shape, edge_dis_weight.shape)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        sp, ei, e_, w_ = ctx.saved_tensors
+        b, s, H, F, D0, ns, ne, n_dis, mhd, dt, vshape, wshape = ctx.dims
+        L = _lib.lib()
+        dout = dout.to(dt).contiguous()
+        dev = dout.device
+        d_sp = torch.empty((ns, H), dtype=dt, device=dev)
+        d_e = torch.empty((ne, H), dtype=dt, device=dev)
+        d_w = torch.empty(n_dis * H * H, dtype=dt, device=dev)
+        d_v = torch.empty(H, dtype=dt, device=dev)
+        D = min(D0, mhd) if mhd > 0 else D0
+        nbytes = L.tgt_graph_attn_bias_multi_hop_bwd_workspace_bytes(ns, ne, H, D)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        with torch.cuda.device(dev):
+            _lib.check(L.tgt_graph_attn_bias_multi_hop_bwd(
+                dout.data_ptr(), sp.data_ptr(), ei.data_ptr(), D0, F, e_.data_ptr(), ns, ne, w_.data_ptr(), n_dis, mhd, b, s, H,
+                _DT[dt], d_sp.data_ptr(), d_e.data_ptr(), d_w.data_ptr(), d_v.data_ptr(), ws.data_ptr(), nbytes, _stream(dout)))
+        return None, None, None, d_sp, d_e, d_w.view(wshape), d_v.view(vshape), None
+
+
 class GraphAttnBias(nn.Module):
     """Attention bias for each head, global token at index 0 (graphormer_graph_level.py:63-156)."""
 
@@ -78,7 +131,10 @@ class GraphAttnBias(nn.Module):
 
     def forward(self, batched_data):
         if self.edge_type == "multi_hop":
-            raise NotImplementedError("the multi_hop edge encoding (graphormer_graph_level.py:119-147) is not built")
+            return GraphAttnBiasMultiHopFunction.apply(batched_data.attn_bias, batched_data.spatial_pos, batched_data.edge_input,
+                                                       self.spatial_pos_encoder.weight, self.edge_encoder.weight,
+                                                       self.edge_dis_encoder.weight, self.graph_token_virtual_distance.weight,
+                                                       self.multi_hop_max_dist)
         return GraphAttnBiasFunction.apply(batched_data.attn_bias, batched_data.spatial_pos, batched_data.attn_edge_type,
                                            self.spatial_pos_encoder.weight, self.edge_encoder.weight,
                                            self.graph_token_virtual_distance.weight)
@@ -112,3 +168,37 @@ def floyd_warshall(adjacency_matrix, n_nodes=None):
     if is_np:
         return dist.cpu().numpy(), path.cpu().numpy()
     return dist, path
+
+
+def gen_edge_input(max_dist, path, edge_feat, n_nodes=None):
+    """``gen_edge_input`` of data/algos.pyx:64-92 on the GPU.
+
+    ``path``: [n, n] (one graph, as in the reference) or [B, n_max, n_max] with ``n_nodes`` [B], as
+    ``floyd_warshall`` returns it; ``edge_feat``: [n, n, F] / [B, n_max, n_max, F] integer features of the
+    direct edges; numpy arrays or tensors.  Returns int64 [..., max_dist, F] of the input's kind: the
+    features of the edges along the recorded shortest path of every pair, -1 where there is none."""
+    is_np = isinstance(path, np.ndarray)
+    pt = torch.as_tensor(path)
+    ft = torch.as_tensor(edge_feat)
+    single = pt.dim() == 2
+    if single:
+        pt, ft = pt.unsqueeze(0), ft.unsqueeze(0)
+    if not torch.cuda.is_available():
+        raise RuntimeError("gen_edge_input runs on the GPU only (no CPU fallback)")
+    dev = pt.device if pt.is_cuda else torch.device("cuda:0")
+    B, n_max = pt.shape[0], pt.shape[1]
+    if ft.shape[:3] != (B, n_max, n_max):
+        raise ValueError(f"edge_feat {tuple(ft.shape)} does not match path {tuple(pt.shape)}")
+    F = ft.shape[3]
+    p32 = pt.to(device=dev, dtype=torch.int32).contiguous()
+    f64 = ft.to(device=dev, dtype=torch.int64).contiguous()
+    nn_ = None if n_nodes is None else torch.as_tensor(n_nodes).to(device=dev, dtype=torch.int32).contiguous()
+    max_dist = int(max_dist)
+    out = torch.empty((B, n_max, n_max, max_dist, F), dtype=torch.int64, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().tgt_gen_edge_input(p32.data_ptr(), f64.data_ptr(), 1, F, None if nn_ is None else nn_.data_ptr(),
+                                                 B, n_max, max_dist, out.data_ptr(),
+                                                 torch.cuda.current_stream(dev).cuda_stream))
+    if single:
+        out = out[0]
+    return out.cpu().numpy() if is_np else out
