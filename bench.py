@@ -8,11 +8,12 @@ the benchmark configuration "configs[1]": N = 64 001, E ~ 530 K, H = 8, d = 8, p
 reported separately).  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype f32|bf16] [--no-cpu-baseline]
-                    [--workload config1|config2|config2-mha|config2-model|config3|config4|config4-bias|config5|
-                               config5-blockized]
+                    [--workload config1|config2|config2-mha|config2-model|config3|config4|config4-bias|
+                               config4-bias-multihop|config5|config5-blockized]
 
 config3 / config5: larger sparse workloads (bf16); config4: dense biased attention of a graph-level
-batch; config4-bias: the bias builder in front of it (GraphAttnBias forward + table gradients); config5-blockized: the block path on the reordered config5 graph; config2-mha: one whole
+batch; config4-bias: the bias builder in front of it (GraphAttnBias forward + table gradients); config4-bias-multihop:
+the same with the path-encoding ('multi_hop') edge term; config5-blockized: the block path on the reordered config5 graph; config2-mha: one whole
 MultiHeadAttention layer (projections + sparse attention) on the config2 graph; config2-model: a training
 step of the 4-layer Graphormer-Slim on that graph.
 """
@@ -281,8 +282,41 @@ def bench_graph_bias(args):
     ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream(dev).cuda_stream
     P = lambda t: t.data_ptr()
+    multi_hop = args.workload == "config4-bias-multihop"
+    prep_ms = None
+    if multi_hop:
+        # the path-encoding branch: edge_input [b, s, s, D, F] from the library's own Floyd-Warshall and gen_edge_input
+        from torchgt_amd import floyd_warshall, gen_edge_input
+        D, n_dis = 5, 128                  # multi_hop_max_dist and num_edge_dis of the reference's graph-level scripts
+        sizes = torch.from_numpy(data["n_nodes"]).to(dev)
+        adj = (spatial_pos == 2).to(torch.uint8)
+        feat = edge_type * adj.unsqueeze(-1).long()
+
+        def prep():
+            _, path = floyd_warshall(adj, sizes)
+            return gen_edge_input(D, path, feat, sizes) + 1        # collator: features + 1, 0 = padding
+        edge_input = prep()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(5):
+            edge_input = prep()
+        torch.cuda.synchronize()
+        prep_ms = (time.perf_counter() - t0) / 5 * 1e3
+        edge_input = edge_input.contiguous()
+        t_w = (torch.randn(n_dis * H * H, generator=g) * 0.02).to(dev, tdt)
+        d_w = torch.empty_like(t_w)
+        nbytes_mh = L.tgt_graph_attn_bias_multi_hop_bwd_workspace_bytes(n_sp, n_e, H, D)
+        ws_mh = torch.empty(nbytes_mh, dtype=torch.uint8, device=dev)
 
     def step():
+        if multi_hop:
+            _lib.check(L.tgt_graph_attn_bias_multi_hop_fwd(P(attn_bias), P(spatial_pos), P(edge_input), D, F, P(t_sp), n_sp,
+                                                           P(t_e), n_e, P(t_w), n_dis, P(t_v), D, b, s, H, dt_code, P(out),
+                                                           stream))
+            _lib.check(L.tgt_graph_attn_bias_multi_hop_bwd(P(dout), P(spatial_pos), P(edge_input), D, F, P(t_e), n_sp, n_e,
+                                                           P(t_w), n_dis, D, b, s, H, dt_code, P(d_sp), P(d_e), P(d_w),
+                                                           P(d_v), P(ws_mh), nbytes_mh, stream))
+            return
         _lib.check(L.tgt_graph_attn_bias_fwd(P(attn_bias), P(spatial_pos), P(edge_type), F, P(t_sp), n_sp, P(t_e), n_e, P(t_v),
                                              b, s, H, dt_code, P(out), stream))
         _lib.check(L.tgt_graph_attn_bias_bwd(P(dout), P(spatial_pos), P(edge_type), F, n_sp, n_e, b, s, H, dt_code,
@@ -303,7 +337,7 @@ def bench_graph_bias(args):
     torch.cuda.synchronize()
     L.tgt_timing_enable(0)
     kernels = {n: {"avg_us": t / c * 1e3, "launches": c} for n, (t, c) in _lib.kernel_timings().items() if c}
-    ids_b = b * s * s * 8 * (1 + F)                       # int64 spatial_pos and edge_type
+    ids_b = b * s * s * 8 * (1 + (D if multi_hop else 1) * F)      # int64 spatial_pos and edge_type / edge_input
     bias_b = b * H * S1 * S1 * esize
     alg = {"graph_bias_fwd": b * S1 * S1 * esize + ids_b + bias_b, "graph_bias_bwd": bias_b + ids_b}
     dom = max(kernels, key=lambda n: kernels[n]["avg_us"])
@@ -315,12 +349,15 @@ def bench_graph_bias(args):
         "dtype": args.dtype, "data": "synthetic",
         "config": {"workload": "bias builder of configs[3]: 256 ER graphs n~U[16,128] p=0.1 padded to 128 + virtual node",
                    "b": b, "S": S1, "H": H, "edge_features": F, "tables": [[n_sp, H], [n_e, H], [1, H]],
-                   "step": "tgt_graph_attn_bias_fwd + tgt_graph_attn_bias_bwd", "parallelism": "1 GPU"},
+                   "step": ("tgt_graph_attn_bias_multi_hop_fwd + _bwd (5 hops, 128 hop matrices)" if multi_hop
+                            else "tgt_graph_attn_bias_fwd + tgt_graph_attn_bias_bwd"), "parallelism": "1 GPU"},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": gbs / HBM_PEAK_GBS, "traffic": None, "alg_bytes": alg[dom], "avg_us": kernels[dom]["avg_us"]},
         "alg_bytes": alg,
         "kernels": kernels,
     }
+    if prep_ms is not None:
+        result["floyd_warshall_plus_gen_edge_input_ms"] = prep_ms
     print(json.dumps(result))
 
 
@@ -605,13 +642,14 @@ def main():
         raise SystemExit("bench.py needs a GPU")
     dev = torch.device("cuda:0")
     H, d = 8, 8
-    if args.workload in ("config3", "config4", "config4-bias", "config5", "config5-blockized") and "--dtype" not in sys.argv:
+    if args.workload in ("config3", "config4", "config4-bias", "config4-bias-multihop", "config5",
+                         "config5-blockized") and "--dtype" not in sys.argv:
         args.dtype = "bf16"              # the dtype those configurations are quoted on
     tdt = torch.float32 if args.dtype == "f32" else torch.bfloat16
     esize = 4 if args.dtype == "f32" else 2
     if args.workload == "config4":
         return bench_dense(args)
-    if args.workload == "config4-bias":
+    if args.workload in ("config4-bias", "config4-bias-multihop"):
         return bench_graph_bias(args)
     if args.workload == "config5-blockized":
         return bench_block(args)

@@ -50,6 +50,38 @@ __device__ __forceinline__ int hop_count(int sp, int max_dist) {
     return n;
 }
 
+// Position (graph, row, column) of a thread in the [b, S1, S1] index space and its step from one
+// iteration of a grid-stride loop to the next, without a 64-bit division per iteration.
+struct HopPos {
+    int64_t g;
+    int i, j;
+};
+__device__ __forceinline__ HopPos hop_pos(int64_t t, int S1) {
+    const int64_t plane = (int64_t)S1 * S1;
+    HopPos p;
+    p.g = t / plane;
+    const int ij = (int)(t - p.g * plane);
+    p.i = ij / S1;
+    p.j = ij - p.i * S1;
+    return p;
+}
+__device__ __forceinline__ void hop_advance(HopPos& p, const HopPos& d, int S1) {
+    p.j += d.j;
+    if (p.j >= S1) { p.j -= S1; ++p.i; }
+    p.i += d.i;
+    if (p.i >= S1) { p.i -= S1; ++p.g; }
+    p.g += d.g;
+}
+
+// Entry idx of the hop matrices read straight from the caller's tensor.  With a uniform index and a
+// pointer the kernel never writes through, the compiler turns these into scalar loads: a hop's 64 values
+// sit in scalar registers and cost the LDS nothing (eight heads only: the layout is then [D][8][8]).
+__device__ __forceinline__ float w_at(const float* __restrict__ w, int idx) { return w[idx]; }
+__device__ __forceinline__ float w_at(const mbf16* __restrict__ w, int idx) {
+    const uint32_t pr = reinterpret_cast<const uint32_t*>(w)[idx >> 1];
+    return __uint_as_float((idx & 1) ? (pr & 0xffff0000u) : (pr << 16));
+}
+
 // Hop matrices into LDS as float, row stride HT (zero beyond H).
 template <typename T, int HT>
 __device__ __forceinline__ void load_hop_weight(const HopArgs& a, float* w_lds) {
@@ -59,11 +91,21 @@ __device__ __forceinline__ void load_hop_weight(const HopArgs& a, float* w_lds) 
         w_lds[k] = h < a.H && h0 < a.H ? ldf(w + (dd * a.H + h0) * a.H + h) : 0.f;
     }
 }
-
-// Averaged edge embedding of hop dd at position pos: mean over the F features (:129).
+// A table [rows, H] into LDS as float, row stride HT (zero beyond H).
 template <typename T, int HT>
-__device__ __forceinline__ void hop_embedding(const HopArgs& a, int64_t pos, int dd, float (&m)[HT]) {
-    const T* e_tab = reinterpret_cast<const T*>(a.edge_table);
+__device__ __forceinline__ void load_table(const void* table, int rows, int H, float* t_lds) {
+    const T* t = reinterpret_cast<const T*>(table);
+    for (int k = threadIdx.x; k < rows * HT; k += 256) {
+        const int h = k % HT, r = k / HT;
+        t_lds[k] = h < H ? ldf(t + r * H + h) : 0.f;
+    }
+}
+
+// Averaged edge embedding of hop dd at position pos: mean over the F features (:129).  The table is
+// either the LDS copy (float, row stride HT) or the caller's (row stride H).
+template <typename TT, int HT>
+__device__ __forceinline__ void hop_embedding(const HopArgs& a, const TT* __restrict__ e_tab, int stride, int64_t pos, int dd,
+                                              float (&m)[HT]) {
     const int64_t* ids = a.edge_input + (pos * a.D0 + dd) * a.F;
 #pragma unroll
     for (int h = 0; h < HT; ++h) m[h] = 0.f;
@@ -71,26 +113,39 @@ __device__ __forceinline__ void hop_embedding(const HopArgs& a, int64_t pos, int
         const int id = clamp_id(ids[f], a.num_edges);
 #pragma unroll
         for (int h = 0; h < HT; ++h)
-            if (h < a.H) m[h] += ldf(e_tab + id * a.H + h);
+            if (h < stride) m[h] += ldf(e_tab + id * stride + h);
     }
     const float inv_f = 1.f / (float)a.F;
 #pragma unroll
     for (int h = 0; h < HT; ++h) m[h] *= inv_f;
 }
 
-template <typename T, int HT>
-__global__ __launch_bounds__(256) void k_multi_hop_fwd(HopArgs a, T* __restrict__ out) {
-    extern __shared__ float w_lds[];          // [D][HT][HT]
-    load_hop_weight<T, HT>(a, w_lds);
+// TAB_LDS: the spatial and edge tables fit LDS next to the hop matrices.
+// WS: eight heads, the hop matrices come through scalar loads from wq instead of LDS.
+template <typename T, int HT, bool TAB_LDS, bool WS>
+__global__ __launch_bounds__(256) void k_multi_hop_fwd(HopArgs a, const T* __restrict__ wq, T* __restrict__ out) {
+    extern __shared__ float w_lds[];          // [D][HT][HT], then [num_edges][HT], [num_spatial][HT] with TAB_LDS
+    float* e_lds = w_lds + a.D * HT * HT;
+    float* sp_lds = e_lds + a.num_edges * HT;
+    if (!WS) load_hop_weight<T, HT>(a, w_lds);
+    if (TAB_LDS) {
+        load_table<T, HT>(a.edge_table, a.num_edges, a.H, e_lds);
+        load_table<T, HT>(a.spatial_table, a.num_spatial, a.H, sp_lds);
+    }
     __syncthreads();
     const int S1 = a.s + 1;
     const int64_t plane = (int64_t)S1 * S1;
     const int64_t total = (int64_t)a.b * plane;
     const T* sp_tab = reinterpret_cast<const T*>(a.spatial_table);
+    const T* e_tab = reinterpret_cast<const T*>(a.edge_table);
     const T* vd = reinterpret_cast<const T*>(a.virtual_dist);
-    for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < total; t += (int64_t)gridDim.x * 256) {
-        const int64_t g = t / plane;
-        const int ij = (int)(t - g * plane), i = ij / S1, j = ij - i * S1;
+    const float inv_f = 1.f / (float)a.F;
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    const HopPos step = hop_pos(stride, S1);
+    HopPos ps = hop_pos((int64_t)blockIdx.x * 256 + threadIdx.x, S1);
+    for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < total; t += stride, hop_advance(ps, step, S1)) {
+        const int64_t g = ps.g;
+        const int i = ps.i, j = ps.j, ij = i * S1 + j;
         const bool inner = i >= 1 && j >= 1;
         const float base = 2.f * ldf(reinterpret_cast<const T*>(a.attn_bias) + t);     // the clone plus the re-add (:104, :153)
         float v[HT];
@@ -102,19 +157,47 @@ __global__ __launch_bounds__(256) void k_multi_hop_fwd(HopArgs a, T* __restrict_
             float y[HT];
 #pragma unroll
             for (int h = 0; h < HT; ++h) y[h] = 0.f;
-            for (int dd = 0; dd < a.D; ++dd) {
-                float m[HT];
-                hop_embedding<T, HT>(a, pos, dd, m);
-                const float* w = w_lds + dd * HT * HT;
+            // the D F ids of the position, eight at a time so that their loads are in flight together; the hop
+            // (dd) and feature (f) counters are uniform, the embedding sum m of a hop is closed after its last feature
+            const int64_t* ids = a.edge_input + pos * a.D0 * a.F;
+            const int n_ids = a.D * a.F;
+            float m[HT];
 #pragma unroll
-                for (int h0 = 0; h0 < HT; ++h0)
+            for (int h = 0; h < HT; ++h) m[h] = 0.f;
+            int dd = 0, f = 0;
+            for (int k0 = 0; k0 < n_ids; k0 += 8) {
+                int64_t idr[8];
 #pragma unroll
-                    for (int h = 0; h < HT; ++h) y[h] += m[h0] * w[h0 * HT + h];       // (:134-139)
+                for (int k = 0; k < 8; ++k) idr[k] = ids[min(k0 + k, n_ids - 1)];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    if (k0 + k < n_ids) {
+                        const int id = clamp_id(idr[k], a.num_edges);
+#pragma unroll
+                        for (int h = 0; h < HT; ++h) {
+                            if (TAB_LDS) m[h] += e_lds[id * HT + h];
+                            else if (h < a.H) m[h] += ldf(e_tab + id * a.H + h);
+                        }
+                        if (++f == a.F) {
+                            const float* w = w_lds + dd * HT * HT;
+#pragma unroll
+                            for (int h0 = 0; h0 < HT; ++h0) {
+                                const float mh = m[h0] * inv_f;                            // mean over the features (:129)
+#pragma unroll
+                                for (int h = 0; h < HT; ++h)                               // (:134-139)
+                                    y[h] += mh * (WS ? w_at(wq, dd * 64 + h0 * 8 + h) : w[h0 * HT + h]);
+                                m[h0] = 0.f;
+                            }
+                            f = 0;
+                            ++dd;
+                        }
+                    }
+                }
             }
             const float hops = (float)hop_count(sp, a.max_dist);
 #pragma unroll
             for (int h = 0; h < HT; ++h)
-                if (h < a.H) v[h] += ldf(sp_tab + sp * a.H + h) + y[h] / hops;         // (:110-111, :145-152)
+                if (h < a.H) v[h] += (TAB_LDS ? sp_lds[sp * HT + h] : ldf(sp_tab + sp * a.H + h)) + y[h] / hops;   // (:110-111, :145-152)
         } else {
 #pragma unroll
             for (int h = 0; h < HT; ++h)
@@ -136,23 +219,38 @@ __host__ __device__ inline HopAcc hop_acc(int num_spatial, int num_edges, int H,
     return HopAcc{num_spatial * H, num_edges * H, H, D * H * H};
 }
 
-constexpr int kHopWorkers = 1024;
+constexpr int kHopWorkers = 768;        // three workgroups of the gradient kernel fit a CU: one round
+constexpr int kStage = 260;            // row stride of the staged positions: rows of consecutive heads start 4 banks apart
+constexpr int kHopHotSp = 5;      // spatial ids 1..5 (self, one to four hops) and
+constexpr int kHopHotE = 4;       // edge ids 1..4 are summed in registers when there are at most eight heads
 
-// DC: hops per pass over the staged positions (the per-lane sums of a pass live in registers).
-template <typename T, int HT, int DC>
-__global__ __launch_bounds__(256) void k_multi_hop_bwd(HopArgs a, const T* __restrict__ dout, float* __restrict__ partial) {
+// Gradients.  An LDS float atomic costs a few cycles per active lane whatever the address, and nearly
+// every position would issue one per head for its spatial id and one per head, hop and feature for its
+// edge ids: with up to eight heads the frequent small ids are summed in registers instead (a compare,
+// a select and an add per id and head), added over the wave at the end and put into LDS by one lane.
+// The hop-matrix gradient is a sum over positions of outer products: the workgroup's 256 positions are
+// staged head-major in LDS and lane (h0, h) of every wave sums m[h0] dy[h] over its wave's 64 positions
+// with 16-byte LDS reads.
+// DC: hops per pass over the positions (the per-lane sums of a pass live in registers).
+template <typename T, int HT, int DC, bool TAB_LDS, bool WS>
+__global__ __launch_bounds__(256) void k_multi_hop_bwd(HopArgs a, const T* __restrict__ wq, const T* __restrict__ dout,
+                                                       float* __restrict__ partial) {
     constexpr int EPL = HT * HT / 64;                 // matrix entries of one hop owned by a lane
+    constexpr bool HOT = HT == 8;
+    constexpr int NHS = HOT ? kHopHotSp : 1, NHE = HOT ? kHopHotE : 1;
     extern __shared__ float lds[];
     const HopAcc L = hop_acc(a.num_spatial, a.num_edges, a.H, a.D);
     float* w_lds = lds;                               // [D][HT][HT]
-    float* st_dy = w_lds + a.D * HT * HT;             // [256][HT]  bias gradient / path length of the staged positions
-    float* st_m = st_dy + 256 * HT;                   // [256][HT]  averaged embedding of one hop
-    float* acc = st_m + 256 * HT;                     // [L.total()]
+    float* st_dy = w_lds + a.D * HT * HT;             // [HT][kStage]  bias gradient / path length of the staged positions
+    float* st_m = st_dy + kStage * HT;                // [min(D, DC)][HT][kStage]  averaged embeddings of the hops of a pass
+    float* acc = st_m + kStage * HT * min(a.D, DC);   // [L.total()]
     float* acc_sp = acc;
     float* acc_e = acc_sp + L.n_sp;
     float* acc_v = acc_e + L.n_e;
     float* acc_w = acc_v + L.n_v;
-    load_hop_weight<T, HT>(a, w_lds);
+    float* e_lds = acc + ((L.total() + 3) & ~3);      // [num_edges][HT] with TAB_LDS
+    if (!WS) load_hop_weight<T, HT>(a, w_lds);
+    if (TAB_LDS) load_table<T, HT>(a.edge_table, a.num_edges, a.H, e_lds);
     for (int k = threadIdx.x; k < L.total(); k += 256) acc[k] = 0.f;
     __syncthreads();
     const int S1 = a.s + 1, H = a.H;
@@ -160,17 +258,29 @@ __global__ __launch_bounds__(256) void k_multi_hop_bwd(HopArgs a, const T* __res
     const int64_t total = (int64_t)a.b * plane;
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
     const float inv_f = 1.f / (float)a.F;
+    const T* e_tab = reinterpret_cast<const T*>(a.edge_table);
+    float hot_sp[NHS][HT], hot_e[NHE][HT];
+#pragma unroll
+    for (int h = 0; h < HT; ++h) {
+#pragma unroll
+        for (int r = 0; r < NHS; ++r) hot_sp[r][h] = 0.f;
+#pragma unroll
+        for (int r = 0; r < NHE; ++r) hot_e[r][h] = 0.f;
+    }
     for (int dc = 0; dc < a.D || dc == 0; dc += DC) {          // one walk per DC hops (one walk when D <= DC)
         float wsum[DC][EPL];
 #pragma unroll
         for (int u = 0; u < DC; ++u)
 #pragma unroll
             for (int e = 0; e < EPL; ++e) wsum[u][e] = 0.f;
-        for (int64_t t0 = (int64_t)blockIdx.x * 256; t0 < total; t0 += (int64_t)gridDim.x * 256) {
+        const int64_t stride = (int64_t)gridDim.x * 256;
+        const HopPos step = hop_pos(stride, S1);
+        HopPos ps = hop_pos((int64_t)blockIdx.x * 256 + threadIdx.x, S1);
+        for (int64_t t0 = (int64_t)blockIdx.x * 256; t0 < total; t0 += stride, hop_advance(ps, step, S1)) {
             const int64_t t = t0 + threadIdx.x;
             const bool valid = t < total;
-            const int64_t g = valid ? t / plane : 0;
-            const int ij = valid ? (int)(t - g * plane) : 0, i = ij / S1, j = ij - i * S1;
+            const int64_t g = valid ? ps.g : 0;
+            const int i = valid ? ps.i : 0, j = valid ? ps.j : 0, ij = i * S1 + j;
             const bool inner = valid && i >= 1 && j >= 1;
             const int64_t pos = inner ? (g * a.s + (i - 1)) * a.s + (j - 1) : 0;
             float dy[HT];
@@ -179,63 +289,101 @@ __global__ __launch_bounds__(256) void k_multi_hop_bwd(HopArgs a, const T* __res
             if (valid) {
                 const T* dg = dout + g * H * plane + ij;
                 const int sp = inner ? clamp_id(a.spatial_pos[pos], a.num_spatial) : 0;
-                const float hops = (float)hop_count(sp, a.max_dist);
+                const float inv_hops = 1.f / (float)hop_count(sp, a.max_dist);
+                float d[HT];
 #pragma unroll
-                for (int h = 0; h < HT; ++h) {
-                    if (h < H) {
-                        const float d = ldf(dg + h * plane);
-                        if (dc == 0 && d != 0.f) {                          // table gradients: first walk only
-                            if (inner) { if (sp > 0) atomicAdd(&acc_sp[sp * H + h], d); }     // row 0 = padding index
-                            else atomicAdd(&acc_v[h], d);
+                for (int h = 0; h < HT; ++h) d[h] = h < H ? ldf(dg + h * plane) : 0.f;
+                if (dc == 0) {                                              // table gradients: first walk only
+                    if (HOT && inner) {
+#pragma unroll
+                        for (int r = 0; r < NHS; ++r) {
+                            const float hit = sp == r + 1 ? 1.f : 0.f;
+#pragma unroll
+                            for (int h = 0; h < HT; ++h) hot_sp[r][h] += hit * d[h];
                         }
-                        dy[h] = inner ? d / hops : 0.f;
+                    }
+                    const bool cold = inner && (HOT ? sp > NHS : sp > 0);   // row 0 = padding index
+#pragma unroll
+                    for (int h = 0; h < HT; ++h) {
+                        if (h < H && d[h] != 0.f) {
+                            if (cold) atomicAdd(&acc_sp[sp * H + h], d[h]);
+                            if (!inner) atomicAdd(&acc_v[h], d[h]);
+                        }
                     }
                 }
+#pragma unroll
+                for (int h = 0; h < HT; ++h) dy[h] = inner ? d[h] * inv_hops : 0.f;
             }
 #pragma unroll
-            for (int h = 0; h < HT; ++h) st_dy[threadIdx.x * HT + h] = dy[h];
+            for (int h = 0; h < HT; ++h) st_dy[h * kStage + threadIdx.x] = dy[h];
 #pragma unroll
             for (int u = 0; u < DC; ++u) {
                 const int dd = dc + u;
                 if (dd < a.D) {                                              // uniform over the workgroup
-                float m[HT];
+                    float m[HT];
 #pragma unroll
-                for (int h = 0; h < HT; ++h) m[h] = 0.f;
-                if (inner) {
-                    hop_embedding<T, HT>(a, pos, dd, m);
-                    // gradient of the averaged embedding, handed to the F edge-table rows it was averaged from
-                    const float* w = w_lds + dd * HT * HT;
-                    const int64_t* ids = a.edge_input + (pos * a.D0 + dd) * a.F;
+                    for (int h = 0; h < HT; ++h) m[h] = 0.f;
+                    if (inner) {
+                        if (TAB_LDS) hop_embedding<float, HT>(a, e_lds, HT, pos, dd, m);
+                        else hop_embedding<T, HT>(a, e_tab, H, pos, dd, m);
+                        // gradient of the averaged embedding, handed to the F edge-table rows it was averaged from
+                        const float* w = w_lds + dd * HT * HT;
+                        float dm[HT];
 #pragma unroll
-                    for (int h0 = 0; h0 < HT; ++h0) {
-                        if (h0 >= H) continue;
-                        float dm = 0.f;
+                        for (int h0 = 0; h0 < HT; ++h0) {
+                            float x = 0.f;
 #pragma unroll
-                        for (int h = 0; h < HT; ++h) dm += w[h0 * HT + h] * dy[h];
-                        dm *= inv_f;
-                        if (dm != 0.f)
-                            for (int f = 0; f < a.F; ++f) {
-                                const int id = clamp_id(ids[f], a.num_edges);
-                                if (id > 0) atomicAdd(&acc_e[id * H + h0], dm);            // row 0 = padding index
+                            for (int h = 0; h < HT; ++h) x += (WS ? w_at(wq, dd * 64 + h0 * 8 + h) : w[h0 * HT + h]) * dy[h];
+                            dm[h0] = x * inv_f;
+                        }
+                        const int64_t* ids = a.edge_input + (pos * a.D0 + dd) * a.F;
+                        for (int f = 0; f < a.F; ++f) {
+                            const int id = clamp_id(ids[f], a.num_edges);
+                            if (HOT) {
+#pragma unroll
+                                for (int r = 0; r < NHE; ++r) {
+                                    const float hit = id == r + 1 ? 1.f : 0.f;
+#pragma unroll
+                                    for (int h0 = 0; h0 < HT; ++h0) hot_e[r][h0] += hit * dm[h0];
+                                }
                             }
-                    }
-                }
+                            if (HOT ? id > NHE : id > 0) {                   // row 0 = padding index
 #pragma unroll
-                for (int h = 0; h < HT; ++h) st_m[threadIdx.x * HT + h] = m[h];
-                __syncthreads();
-                // lane owns entries (h0, h) = divmod(lane + 64 e, HT) of the hop matrix; its wave's 64 positions
-#pragma unroll 4
-                for (int p = 0; p < 64; ++p) {
-                    const int q = (wave * 64 + p) * HT;
-#pragma unroll
-                    for (int e = 0; e < EPL; ++e) {
-                        const int idx = lane + 64 * e;
-                        wsum[u][e] += st_m[q + idx / HT] * st_dy[q + idx % HT];
+                                for (int h0 = 0; h0 < HT; ++h0)
+                                    if (h0 < H && dm[h0] != 0.f) atomicAdd(&acc_e[id * H + h0], dm[h0]);
+                            }
+                        }
                     }
-                }
-                __syncthreads();
+#pragma unroll
+                    for (int h = 0; h < HT; ++h) st_m[(u * HT + h) * kStage + threadIdx.x] = m[h];
                 }
             }
+            __syncthreads();
+            // lane owns entries (h0, h) = divmod(lane + 64 e, HT) of the hop matrices; its wave's 64 positions
+            const int nu = min(DC, a.D - dc);
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) {
+                const int idx = lane + 64 * e;
+                const float4* pm = reinterpret_cast<const float4*>(st_m + (idx / HT) * kStage + wave * 64);
+                const float4* pd = reinterpret_cast<const float4*>(st_dy + (idx % HT) * kStage + wave * 64);
+#pragma unroll 2
+                for (int p = 0; p < 16; ++p) {
+                    const float4 dd4 = pd[p];
+#pragma unroll
+                    for (int u = 0; u < DC; ++u) {
+                        if (u < nu) {                                        // uniform over the workgroup
+                            const float4 mm = pm[u * (HT * kStage / 4) + p];
+                            float x = wsum[u][e];
+                            x += mm.x * dd4.x;
+                            x += mm.y * dd4.y;
+                            x += mm.z * dd4.z;
+                            x += mm.w * dd4.w;
+                            wsum[u][e] = x;
+                        }
+                    }
+                }
+            }
+            __syncthreads();
         }
 #pragma unroll
         for (int u = 0; u < DC; ++u) {
@@ -247,27 +395,59 @@ __global__ __launch_bounds__(256) void k_multi_hop_bwd(HopArgs a, const T* __res
             }
         }
     }
+    if (HOT) {
+        // the wave's sums of the ids kept in registers
+#pragma unroll
+        for (int h = 0; h < HT; ++h) {
+#pragma unroll
+            for (int r = 0; r < NHS; ++r) {
+                float x = hot_sp[r][h];
+#pragma unroll
+                for (int off = 32; off >= 1; off >>= 1) x += __shfl_xor(x, off);
+                if (lane == 0 && h < H && r + 1 < a.num_spatial) atomicAdd(&acc_sp[(r + 1) * H + h], x);
+            }
+#pragma unroll
+            for (int r = 0; r < NHE; ++r) {
+                float x = hot_e[r][h];
+#pragma unroll
+                for (int off = 32; off >= 1; off >>= 1) x += __shfl_xor(x, off);
+                if (lane == 0 && h < H && r + 1 < a.num_edges) atomicAdd(&acc_e[(r + 1) * H + h], x);
+            }
+        }
+    }
     __syncthreads();
     for (int k = threadIdx.x; k < L.total(); k += 256) partial[(int64_t)blockIdx.x * L.total() + k] = acc[k];
 }
 
-// Sum of the workgroup partials in a fixed order; one thread per entry.
+// Sum of the workgroup partials in a fixed order: 64 slices of the workers per entry, then the slices.
+// Four entries per workgroup; the workgroups past the last entry clear the hop matrices that are not in use.
 template <typename T>
 __global__ __launch_bounds__(256) void k_multi_hop_reduce(const float* __restrict__ partial, int workers, HopAcc L, int H,
                                                           T* __restrict__ d_sp, T* __restrict__ d_e, T* __restrict__ d_v,
                                                           T* __restrict__ d_w_used, int64_t n_w_all) {
+    __shared__ float part[64][4];
     const int n = L.total();
-    const int64_t k = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (k < n) {
-        float t = 0.f;
-        for (int w = 0; w < workers; ++w) t += partial[(int64_t)w * n + k];
-        if (k < L.n_sp) stf(d_sp + k, t);
-        else if (k < L.n_sp + L.n_e) stf(d_e + (k - L.n_sp), t);
-        else if (k < L.n_sp + L.n_e + L.n_v) stf(d_v + (k - L.n_sp - L.n_e), t);
-        else stf(d_w_used + (k - L.n_sp - L.n_e - L.n_v), t);
-    } else if (k - n < n_w_all - L.n_w) {
-        stf(d_w_used + L.n_w + (k - n), 0.f);             // hop matrices beyond the hops in use
+    const int n_groups = (n + 3) / 4;
+    if ((int)blockIdx.x >= n_groups) {
+        const int64_t k = (int64_t)(blockIdx.x - n_groups) * 256 + threadIdx.x;
+        if (k < n_w_all - L.n_w) stf(d_w_used + L.n_w + k, 0.f);
+        return;
     }
+    const int kl = threadIdx.x % 4, slice = threadIdx.x / 4;
+    const int k = blockIdx.x * 4 + kl;
+    float t = 0.f;
+    if (k < n)
+        for (int w = slice; w < workers; w += 64) t += partial[(int64_t)w * n + k];
+    part[slice][kl] = t;
+    __syncthreads();
+    if (slice != 0 || k >= n) return;
+    t = 0.f;
+#pragma unroll
+    for (int c = 0; c < 64; ++c) t += part[c][kl];
+    if (k < L.n_sp) stf(d_sp + k, t);
+    else if (k < L.n_sp + L.n_e) stf(d_e + (k - L.n_sp), t);
+    else if (k < L.n_sp + L.n_e + L.n_v) stf(d_v + (k - L.n_sp - L.n_e), t);
+    else stf(d_w_used + (k - L.n_sp - L.n_e - L.n_v), t);
 }
 
 int hop_check(int b, int s, int H, int F, int D0, int num_spatial, int num_edges, int num_edge_dis, int max_dist, int dtype,
@@ -356,23 +536,37 @@ int tgt_graph_attn_bias_multi_hop_fwd(const void* d_attn_bias, const int64_t* d_
         return TGT_ERR_INVALID_ARG;
     }
     const int HT = head_tile(H);
-    const size_t lds = sizeof(float) * (size_t)D * HT * HT;
-    if (lds > 48 * 1024) {
-        set_error("tgt_graph_attn_bias_multi_hop_fwd: %d hop matrices of %d heads exceed the 48 KB kept on chip", D, H);
+    const size_t w_bytes = sizeof(float) * (size_t)D * HT * HT;
+    if (w_bytes > 32 * 1024) {
+        set_error("tgt_graph_attn_bias_multi_hop_fwd: %d hop matrices of %d heads exceed the 32 KB kept on chip", D, H);
         return TGT_ERR_UNSUPPORTED;
     }
+    const size_t tab_bytes = sizeof(float) * (size_t)(num_spatial + num_edges) * HT;
+    const bool tab_lds = w_bytes + tab_bytes <= 48 * 1024;
+    const size_t lds = w_bytes + (tab_lds ? tab_bytes : 0);
     HopArgs a{d_attn_bias, d_spatial_pos, d_edge_input, d_spatial_table, d_edge_table, d_edge_dis_weight, d_virtual_dist,
               b, s, H, F, D0, D, num_spatial, num_edges, multi_hop_max_dist};
     const int64_t total = (int64_t)b * (s + 1) * (s + 1);
     const dim3 grid((unsigned)std::min<int64_t>((total + 255) / 256, 8192));
     hipStream_t st = (hipStream_t)stream;
     KernelTimer timer(KS_GRAPH_BIAS_FWD, st);
-#define TGT_HOP_FWD(T, HTV) hipLaunchKernelGGL((k_multi_hop_fwd<T, HTV>), grid, dim3(256), lds, st, a, (T*)d_out)
-    if (dtype == TGT_DTYPE_F32) {
+    const bool ws = H == 8 && ((uintptr_t)d_edge_dis_weight & 3) == 0;
+#define TGT_HOP_FWD2(T, HTV, TL, WSV) \
+    hipLaunchKernelGGL((k_multi_hop_fwd<T, HTV, TL, WSV>), grid, dim3(256), lds, st, a, (const T*)d_edge_dis_weight, (T*)d_out)
+#define TGT_HOP_FWD(T, HTV)                                                       \
+    do {                                                                          \
+        if (tab_lds) TGT_HOP_FWD2(T, HTV, true, false);                           \
+        else TGT_HOP_FWD2(T, HTV, false, false);                                  \
+    } while (0)
+    if (ws) {
+        if (dtype == TGT_DTYPE_F32) { if (tab_lds) TGT_HOP_FWD2(float, 8, true, true); else TGT_HOP_FWD2(float, 8, false, true); }
+        else { if (tab_lds) TGT_HOP_FWD2(mbf16, 8, true, true); else TGT_HOP_FWD2(mbf16, 8, false, true); }
+    } else if (dtype == TGT_DTYPE_F32) {
         if (HT == 8) TGT_HOP_FWD(float, 8); else if (HT == 16) TGT_HOP_FWD(float, 16); else TGT_HOP_FWD(float, 32);
     } else {
         if (HT == 8) TGT_HOP_FWD(mbf16, 8); else if (HT == 16) TGT_HOP_FWD(mbf16, 16); else TGT_HOP_FWD(mbf16, 32);
     }
+#undef TGT_HOP_FWD2
 #undef TGT_HOP_FWD
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
@@ -407,7 +601,11 @@ int tgt_graph_attn_bias_multi_hop_bwd(const void* d_dout, const int64_t* d_spati
         return TGT_ERR_WORKSPACE;
     }
     const int HT = head_tile(H);
-    const size_t lds = sizeof(float) * ((size_t)D * HT * HT + 2 * 256 * HT + L.total());
+    const int DC = HT == 8 ? 8 : (HT == 16 ? 2 : 1);             // hops per walk, as instantiated below
+    const size_t base_lds = sizeof(float) * ((size_t)D * HT * HT + (size_t)(1 + std::min(D, DC)) * kStage * HT + ((L.total() + 3) & ~3));
+    const size_t tab_bytes = sizeof(float) * (size_t)num_edges * HT;
+    const bool tab_lds = base_lds + tab_bytes <= 64 * 1024;
+    const size_t lds = base_lds + (tab_lds ? tab_bytes : 0);
     if (lds > 128 * 1024) {
         set_error("tgt_graph_attn_bias_multi_hop_bwd: tables of %d entries, %d hops and %d heads need %zu bytes on chip (limit 131072)",
                   L.n_sp + L.n_e + L.n_v, D, H, lds);
@@ -421,34 +619,37 @@ int tgt_graph_attn_bias_multi_hop_bwd(const void* d_dout, const int64_t* d_spati
     KernelTimer timer(KS_GRAPH_BIAS_BWD, st);
     float* partial = (float*)d_workspace;
     const int64_t n_w_all = (int64_t)num_edge_dis * H * H;
-    const unsigned rgrid = (unsigned)((L.total() + (n_w_all - L.n_w) + 255) / 256);
+    const unsigned rgrid = (unsigned)((L.total() + 3) / 4 + (n_w_all - L.n_w + 255) / 256);
     auto launch = [&](auto kernel, auto reduce, auto* dout, auto* dsp, auto* de, auto* dv, auto* dw) -> int {
         if (lds > 48 * 1024)
             TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                               128 * 1024));
-        hipLaunchKernelGGL(kernel, dim3(workers), dim3(256), lds, st, a, dout, partial);
+        hipLaunchKernelGGL(kernel, dim3(workers), dim3(256), lds, st, a, (decltype(dout))d_edge_dis_weight, dout, partial);
         hipLaunchKernelGGL(reduce, dim3(rgrid), dim3(256), 0, st, (const float*)partial, workers, L, H, dsp, de, dv, dw, n_w_all);
         return TGT_OK;
     };
     int lrc;
-    // hops per walk: 8 for up to 16 heads (8 or 32 sums per lane), 2 for 32 heads (32 sums per lane)
+    // hops per walk: as many as are staged in LDS at once
+    const bool ws = H == 8 && ((uintptr_t)d_edge_dis_weight & 3) == 0;
+#define TGT_HOP_BWD(T, HTV, DCV)                                                                          \
+    (ws && HTV == 8 ? (tab_lds ? launch(&k_multi_hop_bwd<T, 8, 8, true, true>, red, dout, dsp, de, dv, dw)        \
+                               : launch(&k_multi_hop_bwd<T, 8, 8, false, true>, red, dout, dsp, de, dv, dw))      \
+     : tab_lds      ? launch(&k_multi_hop_bwd<T, HTV, DCV, true, false>, red, dout, dsp, de, dv, dw)      \
+                    : launch(&k_multi_hop_bwd<T, HTV, DCV, false, false>, red, dout, dsp, de, dv, dw))
     if (dtype == TGT_DTYPE_F32) {
         auto* red = &k_multi_hop_reduce<float>;
         const float* dout = (const float*)d_dout;
         float *dsp = (float*)d_dspatial_table, *de = (float*)d_dedge_table, *dv = (float*)d_dvirtual_dist,
               *dw = (float*)d_dedge_dis_weight;
-        lrc = HT == 8    ? launch(&k_multi_hop_bwd<float, 8, 8>, red, dout, dsp, de, dv, dw)
-              : HT == 16 ? launch(&k_multi_hop_bwd<float, 16, 8>, red, dout, dsp, de, dv, dw)
-                         : launch(&k_multi_hop_bwd<float, 32, 2>, red, dout, dsp, de, dv, dw);
+        lrc = HT == 8 ? TGT_HOP_BWD(float, 8, 8) : HT == 16 ? TGT_HOP_BWD(float, 16, 2) : TGT_HOP_BWD(float, 32, 1);
     } else {
         auto* red = &k_multi_hop_reduce<mbf16>;
         const mbf16* dout = (const mbf16*)d_dout;
         mbf16 *dsp = (mbf16*)d_dspatial_table, *de = (mbf16*)d_dedge_table, *dv = (mbf16*)d_dvirtual_dist,
               *dw = (mbf16*)d_dedge_dis_weight;
-        lrc = HT == 8    ? launch(&k_multi_hop_bwd<mbf16, 8, 8>, red, dout, dsp, de, dv, dw)
-              : HT == 16 ? launch(&k_multi_hop_bwd<mbf16, 16, 8>, red, dout, dsp, de, dv, dw)
-                         : launch(&k_multi_hop_bwd<mbf16, 32, 2>, red, dout, dsp, de, dv, dw);
+        lrc = HT == 8 ? TGT_HOP_BWD(mbf16, 8, 8) : HT == 16 ? TGT_HOP_BWD(mbf16, 16, 2) : TGT_HOP_BWD(mbf16, 32, 1);
     }
+#undef TGT_HOP_BWD
     if (lrc != TGT_OK) return lrc;
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
