@@ -330,6 +330,26 @@ int tgt_graph_attn_bias_bwd(const void* d_dout, const int64_t* d_spatial_pos, co
                             int num_spatial, int num_edges, int b, int s, int H, int dtype, void* d_dspatial_table,
                             void* d_dedge_table, void* d_dvirtual_dist, void* d_workspace, int64_t workspace_bytes,
                             void* stream);
+/* GraphNodeFeature.forward (models/graphormer_graph_level.py:18-60): the input rows of the
+ * graph-level model, virtual node first:
+ *   out[g, 0, :]     = graph_token
+ *   out[g, 1 + i, :] = sum_f atom_table[x[g,i,f]] + in_table[in_degree[g,i]] + out_table[out_degree[g,i]]
+ * d_x: int64 [b, s, Fx]; d_in_degree, d_out_degree: int64 [b, s]; tables [num_*, C], d_graph_token
+ * [C], d_out [b, s + 1, C] of `dtype`.  Ids outside a table are clamped to its range (the
+ * reference's embedding lookup would raise). */
+int tgt_graph_node_feature_fwd(const int64_t* d_x, const int64_t* d_in_degree, const int64_t* d_out_degree, int Fx,
+                               const void* d_atom_table, int num_atoms, const void* d_in_table, int num_in,
+                               const void* d_out_table, int num_out, const void* d_graph_token, int b, int s, int C, int dtype,
+                               void* d_out, void* stream);
+/* Gradients of the four tables for the upstream gradient d_dout [b, s + 1, C] (autograd of the
+ * embedding lookups in the reference; row 0 of the three lookup tables is the padding index and
+ * gets zero).  Sums are formed in float with memory atomics: results agree to rounding between
+ * runs, not bit for bit.  d_workspace: tgt_graph_node_feature_bwd_workspace_bytes(...) bytes. */
+int64_t tgt_graph_node_feature_bwd_workspace_bytes(int num_atoms, int num_in, int num_out, int C);
+int tgt_graph_node_feature_bwd(const void* d_dout, const int64_t* d_x, const int64_t* d_in_degree, const int64_t* d_out_degree,
+                               int Fx, int num_atoms, int num_in, int num_out, int b, int s, int C, int dtype, void* d_datom_table,
+                               void* d_din_table, void* d_dout_table, void* d_dgraph_token, void* d_workspace,
+                               int64_t workspace_bytes, void* stream);
 /* GraphAttnBias.forward with edge_type == 'multi_hop' (models/graphormer_graph_level.py:94-156,
  * the path-encoding branch :119-147).  As tgt_graph_attn_bias_fwd, with the edge term replaced by
  *   (1 / hops) * sum_dd  mean_f edge_table[edge_input[g,i-1,j-1,dd,f]]  x  W[dd]        (i, j >= 1)

@@ -10,10 +10,12 @@ from .plan import GraphPlan, get_plan, clear_plan_cache
 from .multi_head_attention import MultiHeadAttention, LinearFunction, fused_linear
 from .encoder import FeedForwardNetwork, EncoderLayer, Graphormer
 from .graph_bias import GraphAttnBias, floyd_warshall, gen_edge_input
+from .graph_level import GraphNodeFeature, Graphormer as GraphLevelGraphormer
 from .block_attention import BlockAttentionFunction, TileSet, block_attention, expand_tiles
 
 __all__ = ["CoreAttention", "SparseAttentionFunction", "DenseAttentionFunction", "sparse_attention",
            "dense_attention", "gather_dense_bias",
            "GraphPlan", "get_plan", "clear_plan_cache", "BlockAttentionFunction", "TileSet", "block_attention",
            "expand_tiles", "MultiHeadAttention", "LinearFunction", "fused_linear",
-           "FeedForwardNetwork", "EncoderLayer", "Graphormer", "GraphAttnBias", "floyd_warshall", "gen_edge_input"]
+           "FeedForwardNetwork", "EncoderLayer", "Graphormer", "GraphAttnBias", "floyd_warshall", "gen_edge_input",
+           "GraphNodeFeature", "GraphLevelGraphormer"]

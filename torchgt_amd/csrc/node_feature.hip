@@ -1,0 +1,195 @@
+// Input features of the graph-level model: GraphNodeFeature.forward
+// (models/graphormer_graph_level.py:18-60) and the gradients of its four embedding tables.
+//
+//   out[g, 0, :]     = graph_token
+//   out[g, 1 + i, :] = sum_f atom_table[x[g, i, f]] + in_degree_table[in_degree[g, i]]
+//                      + out_degree_table[out_degree[g, i]]
+//
+// The reference runs three embedding lookups, a sum over the features, two adds, a repeat and a
+// concatenation; here one kernel reads the ids and writes every output row once.  The backward adds
+// the output gradient into float copies of the tables with vector-memory atomics (row 0 of the three
+// lookup tables is the padding index and gets none) and a last kernel hands the sums over in the
+// caller's type: results agree to rounding between runs, not bit for bit.
+#include "common.h"
+#include <algorithm>
+
+namespace tgt {
+namespace {
+
+struct nbf16 { uint16_t x; };
+__device__ __forceinline__ float ldf(const float* p) { return *p; }
+__device__ __forceinline__ float ldf(const nbf16* p) { return __uint_as_float(((uint32_t)p->x) << 16); }
+__device__ __forceinline__ void stf(float* p, float v) { *p = v; }
+__device__ __forceinline__ void stf(nbf16* p, float v) {
+    const __bf16 b = static_cast<__bf16>(v);
+    p->x = __builtin_bit_cast(uint16_t, b);
+}
+__device__ __forceinline__ int clamp_id(int64_t v, int n) { return v < 0 ? 0 : (v >= n ? n - 1 : (int)v); }
+
+struct NodeFeatArgs {
+    const int64_t* x;            // [b, s, Fx]
+    const int64_t* in_degree;    // [b, s]
+    const int64_t* out_degree;   // [b, s]
+    int b, s, Fx, C, num_atoms, num_in, num_out;
+};
+
+// one thread per (graph, node, channel), channel fastest
+template <typename T>
+__global__ __launch_bounds__(256) void k_node_feature_fwd(NodeFeatArgs a, const T* __restrict__ atom, const T* __restrict__ tin,
+                                                          const T* __restrict__ tout, const T* __restrict__ token,
+                                                          T* __restrict__ out) {
+    const int64_t total = (int64_t)a.b * (a.s + 1) * a.C;
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= total) return;
+    const int c = (int)(t % a.C);
+    const int64_t row = t / a.C;
+    const int node = (int)(row % (a.s + 1));
+    const int64_t g = row / (a.s + 1);
+    float v;
+    if (node == 0) {
+        v = ldf(token + c);                                           // (:52-56)
+    } else {
+        const int64_t p = g * a.s + (node - 1);
+        v = 0.f;
+        for (int f = 0; f < a.Fx; ++f) v += ldf(atom + (int64_t)clamp_id(a.x[p * a.Fx + f], a.num_atoms) * a.C + c);   // (:45)
+        v += ldf(tin + (int64_t)clamp_id(a.in_degree[p], a.num_in) * a.C + c);                                          // (:46-50)
+        v += ldf(tout + (int64_t)clamp_id(a.out_degree[p], a.num_out) * a.C + c);
+    }
+    stf(out + t, v);
+}
+
+__global__ __launch_bounds__(256) void k_fill_zero(float* __restrict__ p, int64_t n) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t < n) p[t] = 0.f;
+}
+
+// acc: float [num_atoms + num_in + num_out + 1][C]
+template <typename T>
+__global__ __launch_bounds__(256) void k_node_feature_bwd(NodeFeatArgs a, const T* __restrict__ dout, float* __restrict__ acc) {
+    const int64_t total = (int64_t)a.b * (a.s + 1) * a.C;
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= total) return;
+    const int c = (int)(t % a.C);
+    const int64_t row = t / a.C;
+    const int node = (int)(row % (a.s + 1));
+    const int64_t g = row / (a.s + 1);
+    const float d = ldf(dout + t);
+    if (d == 0.f) return;
+    float* acc_in = acc + (int64_t)a.num_atoms * a.C;
+    float* acc_out = acc_in + (int64_t)a.num_in * a.C;
+    float* acc_tok = acc_out + (int64_t)a.num_out * a.C;
+    if (node == 0) {
+        atomicAdd(acc_tok + c, d);
+        return;
+    }
+    const int64_t p = g * a.s + (node - 1);
+    for (int f = 0; f < a.Fx; ++f) {
+        const int id = clamp_id(a.x[p * a.Fx + f], a.num_atoms);
+        if (id > 0) atomicAdd(acc + (int64_t)id * a.C + c, d);        // row 0 = padding index
+    }
+    const int ii = clamp_id(a.in_degree[p], a.num_in), io = clamp_id(a.out_degree[p], a.num_out);
+    if (ii > 0) atomicAdd(acc_in + (int64_t)ii * a.C + c, d);
+    if (io > 0) atomicAdd(acc_out + (int64_t)io * a.C + c, d);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void k_node_feature_finish(const float* __restrict__ acc, int64_t n_atom, int64_t n_in,
+                                                             int64_t n_out, int64_t n_tok, T* __restrict__ d_atom,
+                                                             T* __restrict__ d_in, T* __restrict__ d_out, T* __restrict__ d_tok) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= n_atom + n_in + n_out + n_tok) return;
+    const float v = acc[t];
+    if (t < n_atom) stf(d_atom + t, v);
+    else if (t < n_atom + n_in) stf(d_in + (t - n_atom), v);
+    else if (t < n_atom + n_in + n_out) stf(d_out + (t - n_atom - n_in), v);
+    else stf(d_tok + (t - n_atom - n_in - n_out), v);
+}
+
+int node_feat_check(int b, int s, int Fx, int C, int num_atoms, int num_in, int num_out, int dtype, const char* who) {
+    if (b < 0 || s < 0 || Fx < 1 || C < 1 || num_atoms < 1 || num_in < 1 || num_out < 1 ||
+        (dtype != TGT_DTYPE_F32 && dtype != TGT_DTYPE_BF16)) {
+        set_error("%s: bad size or dtype", who);
+        return TGT_ERR_INVALID_ARG;
+    }
+    return TGT_OK;
+}
+
+}  // namespace
+}  // namespace tgt
+
+extern "C" {
+
+int tgt_graph_node_feature_fwd(const int64_t* d_x, const int64_t* d_in_degree, const int64_t* d_out_degree, int Fx,
+                               const void* d_atom_table, int num_atoms, const void* d_in_table, int num_in,
+                               const void* d_out_table, int num_out, const void* d_graph_token, int b, int s, int C, int dtype,
+                               void* d_out, void* stream) {
+    using namespace tgt;
+    const int rc = node_feat_check(b, s, Fx, C, num_atoms, num_in, num_out, dtype, "tgt_graph_node_feature_fwd");
+    if (rc != TGT_OK) return rc;
+    if (b == 0) return TGT_OK;
+    if (!d_atom_table || !d_in_table || !d_out_table || !d_graph_token || !d_out || (s > 0 && (!d_x || !d_in_degree || !d_out_degree))) {
+        set_error("tgt_graph_node_feature_fwd: null pointer");
+        return TGT_ERR_INVALID_ARG;
+    }
+    NodeFeatArgs a{d_x, d_in_degree, d_out_degree, b, s, Fx, C, num_atoms, num_in, num_out};
+    const int64_t total = (int64_t)b * (s + 1) * C;
+    const dim3 grid((unsigned)((total + 255) / 256));
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == TGT_DTYPE_F32)
+        hipLaunchKernelGGL((k_node_feature_fwd<float>), grid, dim3(256), 0, st, a, (const float*)d_atom_table, (const float*)d_in_table,
+                           (const float*)d_out_table, (const float*)d_graph_token, (float*)d_out);
+    else
+        hipLaunchKernelGGL((k_node_feature_fwd<nbf16>), grid, dim3(256), 0, st, a, (const nbf16*)d_atom_table, (const nbf16*)d_in_table,
+                           (const nbf16*)d_out_table, (const nbf16*)d_graph_token, (nbf16*)d_out);
+    TGT_HIP_CHECK(hipGetLastError());
+    return TGT_OK;
+}
+
+int64_t tgt_graph_node_feature_bwd_workspace_bytes(int num_atoms, int num_in, int num_out, int C) {
+    if (num_atoms < 1 || num_in < 1 || num_out < 1 || C < 1) return 0;
+    return (int64_t)sizeof(float) * ((int64_t)num_atoms + num_in + num_out + 1) * C;
+}
+
+int tgt_graph_node_feature_bwd(const void* d_dout, const int64_t* d_x, const int64_t* d_in_degree, const int64_t* d_out_degree,
+                               int Fx, int num_atoms, int num_in, int num_out, int b, int s, int C, int dtype, void* d_datom_table,
+                               void* d_din_table, void* d_dout_table, void* d_dgraph_token, void* d_workspace,
+                               int64_t workspace_bytes, void* stream) {
+    using namespace tgt;
+    const int rc = node_feat_check(b, s, Fx, C, num_atoms, num_in, num_out, dtype, "tgt_graph_node_feature_bwd");
+    if (rc != TGT_OK) return rc;
+    if (!d_datom_table || !d_din_table || !d_dout_table || !d_dgraph_token ||
+        (b > 0 && (!d_dout || (s > 0 && (!d_x || !d_in_degree || !d_out_degree))))) {
+        set_error("tgt_graph_node_feature_bwd: null pointer");
+        return TGT_ERR_INVALID_ARG;
+    }
+    const int64_t need = tgt_graph_node_feature_bwd_workspace_bytes(num_atoms, num_in, num_out, C);
+    if (!d_workspace || workspace_bytes < need) {
+        set_error("tgt_graph_node_feature_bwd: workspace of %lld bytes needed, got %lld", (long long)need, (long long)workspace_bytes);
+        return TGT_ERR_WORKSPACE;
+    }
+    NodeFeatArgs a{d_x, d_in_degree, d_out_degree, b, s, Fx, C, num_atoms, num_in, num_out};
+    hipStream_t st = (hipStream_t)stream;
+    float* acc = (float*)d_workspace;
+    const int64_t n_acc = need / (int64_t)sizeof(float);
+    hipLaunchKernelGGL(k_fill_zero, dim3((unsigned)((n_acc + 255) / 256)), dim3(256), 0, st, acc, n_acc);
+    const int64_t total = (int64_t)b * (s + 1) * C;
+    const int64_t n_atom = (int64_t)num_atoms * C, n_in = (int64_t)num_in * C, n_out = (int64_t)num_out * C;
+    const dim3 fgrid((unsigned)((n_acc + 255) / 256));
+    if (dtype == TGT_DTYPE_F32) {
+        if (total > 0)
+            hipLaunchKernelGGL((k_node_feature_bwd<float>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, a,
+                               (const float*)d_dout, acc);
+        hipLaunchKernelGGL((k_node_feature_finish<float>), fgrid, dim3(256), 0, st, (const float*)acc, n_atom, n_in, n_out, (int64_t)C,
+                           (float*)d_datom_table, (float*)d_din_table, (float*)d_dout_table, (float*)d_dgraph_token);
+    } else {
+        if (total > 0)
+            hipLaunchKernelGGL((k_node_feature_bwd<nbf16>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, a,
+                               (const nbf16*)d_dout, acc);
+        hipLaunchKernelGGL((k_node_feature_finish<nbf16>), fgrid, dim3(256), 0, st, (const float*)acc, n_atom, n_in, n_out, (int64_t)C,
+                           (nbf16*)d_datom_table, (nbf16*)d_din_table, (nbf16*)d_dout_table, (nbf16*)d_dgraph_token);
+    }
+    TGT_HIP_CHECK(hipGetLastError());
+    return TGT_OK;
+}
+
+}  // extern "C"
