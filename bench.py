@@ -9,11 +9,12 @@ reported separately).  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype f32|bf16] [--no-cpu-baseline]
                     [--workload config1|config2|config2-mha|config2-model|config3|config4|config4-bias|
-                               config4-bias-multihop|config5|config5-blockized]
+                               config4-bias-multihop|config4-model|config5|config5-blockized]
 
 config3 / config5: larger sparse workloads (bf16); config4: dense biased attention of a graph-level
 batch; config4-bias: the bias builder in front of it (GraphAttnBias forward + table gradients); config4-bias-multihop:
-the same with the path-encoding ('multi_hop') edge term; config5-blockized: the block path on the reordered config5 graph; config2-mha: one whole
+the same with the path-encoding ('multi_hop') edge term; config4-model: a training step of the graph-level Graphormer
+on that batch; config5-blockized: the block path on the reordered config5 graph; config2-mha: one whole
 MultiHeadAttention layer (projections + sparse attention) on the config2 graph; config2-model: a training
 step of the 4-layer Graphormer-Slim on that graph.
 """
@@ -614,6 +615,83 @@ def bench_model(args):
     print(json.dumps(result))
 
 
+def bench_graph_model(args):
+    """One training step of the graph-level Graphormer (models/graphormer_graph_level.py; 4 layers, hidden 64, ffn 64,
+    8 heads, ZINC tables, one regression target) on the batch of configs[3]: forward, L1 loss as the graph-level
+    script computes it, backward, AdamW step (torch's optimizer)."""
+    import numpy as np
+    import torch
+    import types
+    from torchgt_amd import _lib, workloads
+    from torchgt_amd.graph_level import Graphormer
+    dev = torch.device("cuda:0")
+    tdt = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    b = 256
+    data = workloads.erdos_renyi_batch(batch=b, seed=42)
+    rng = np.random.default_rng(42)
+    sizes = data["n_nodes"]
+    s = data["spatial_pos"].shape[1]
+    x = np.zeros((b, s, 1), np.int64)
+    deg = np.zeros((b, s), np.int64)
+    for g in range(b):
+        n = int(sizes[g])
+        x[g, :n, 0] = rng.integers(1, 64, size=n)
+        deg[g, :n] = np.minimum((data["spatial_pos"][g][:n, :n] == 2).sum(1) + 1, 63)
+    batch = types.SimpleNamespace(
+        x=torch.from_numpy(x).to(dev), in_degree=torch.from_numpy(deg).to(dev), out_degree=torch.from_numpy(deg).to(dev),
+        attn_bias=torch.from_numpy(data["attn_bias"]).to(dev, tdt), spatial_pos=torch.from_numpy(data["spatial_pos"]).long().to(dev),
+        attn_edge_type=torch.from_numpy(data["edge_type"]).long().unsqueeze(-1).contiguous().to(dev), edge_input=None)
+    torch.manual_seed(42)
+    m = Graphormer(4, 8, 64, 0.0, 0.0, 64, "ZINC", "single_hop", 5, 0.0, 1).to(dev, tdt)
+    opt = torch.optim.AdamW(m.parameters(), lr=1e-3, weight_decay=0.01)
+    y = torch.randn(b, device=dev)
+
+    def step():
+        opt.zero_grad(set_to_none=True)
+        out = m(batch)
+        loss = torch.nn.functional.l1_loss(out.float().view(-1), y)
+        loss.backward()
+        opt.step()
+        return loss
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss = step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    L = _lib.lib()
+    L.tgt_timing_reset()
+    L.tgt_timing_enable(1)
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    L.tgt_timing_enable(0)
+    kernels = {k: {"avg_us": t / c * 1e3, "launches_per_step": c / args.steps} for k, (t, c) in _lib.kernel_timings().items() if c}
+    lib_us = sum(v["avg_us"] * v["launches_per_step"] for v in kernels.values())
+    groups = {"dense attention": ("dense_fwd", "dense_bwd"), "bias builder": ("graph_bias_fwd", "graph_bias_bwd"),
+              "projections and ffn linears": ("linear_fwd", "linear_dx", "linear_dw"),
+              "layer norm + residual": ("layer_norm_fwd", "layer_norm_bwd"), "gelu": ("gelu",)}
+    result = {
+        "metric": "training step of the 4-layer graph-level Graphormer on a batch of 256 padded graphs",
+        "value": b / (ms * 1e-3), "unit": "graphs/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic",
+        "config": {"workload": "configs[3] batch (256 ER graphs n~U[16,128] p=0.1 padded to 128 + virtual node), graph-level "
+                               "Graphormer 4 x (hidden 64, ffn 64, 8 heads), ZINC tables, dropout 0", "b": b, "S": s + 1,
+                   "parameters": sum(p.numel() for p in m.parameters()),
+                   "step": "forward + l1_loss + backward + torch AdamW", "parallelism": "1 GPU"},
+        "loss": float(loss.detach()),
+        "library_kernel_us_per_step": lib_us,
+        "kernel_groups_us": {g: sum(kernels[k]["avg_us"] * kernels[k]["launches_per_step"] for k in ks if k in kernels)
+                             for g, ks in groups.items()},
+        "kernels": kernels,
+    }
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -642,7 +720,7 @@ def main():
         raise SystemExit("bench.py needs a GPU")
     dev = torch.device("cuda:0")
     H, d = 8, 8
-    if args.workload in ("config3", "config4", "config4-bias", "config4-bias-multihop", "config5",
+    if args.workload in ("config3", "config4", "config4-bias", "config4-bias-multihop", "config4-model", "config5",
                          "config5-blockized") and "--dtype" not in sys.argv:
         args.dtype = "bf16"              # the dtype those configurations are quoted on
     tdt = torch.float32 if args.dtype == "f32" else torch.bfloat16
@@ -651,6 +729,8 @@ def main():
         return bench_dense(args)
     if args.workload in ("config4-bias", "config4-bias-multihop"):
         return bench_graph_bias(args)
+    if args.workload == "config4-model":
+        return bench_graph_model(args)
     if args.workload == "config5-blockized":
         return bench_block(args)
     if args.workload == "config2-mha":

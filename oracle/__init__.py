@@ -33,6 +33,10 @@ graph_attn_bias_multi_hop      reduces to graph_attn_bias (one hop, identity
 gen_edge_input                 hand-computed known answer (path graph); every
                                row is a walk of existing edges from i to j of
                                the shortest length (scipy)
+graph_node_feature             torch.nn.functional.embedding; hand-computed answer
+graph-level graphormer_forward torch's layer_norm / linear / gelu / softmax
+                               assembly; closed form without layers; node
+                               relabelling and padding invariance
 metis partition labels         PARITY UNPINNED: dgl/METIS is absent; partition
                                ids are always an explicit input here
 =============================  ================================================
