@@ -377,40 +377,46 @@ int bias_check(int b, int s, int H, int F, int num_spatial, int num_edges, int d
 constexpr int kFwMax = 128;
 constexpr int kFwInf = 510;          // data/algos.pyx:30
 
-__global__ __launch_bounds__(256) void k_floyd_warshall(const uint8_t* __restrict__ adj, const int32_t* __restrict__ n_nodes,
-                                                        int n_max, int32_t* __restrict__ dist, int32_t* __restrict__ path) {
+// 1024 threads: thread (r, j) = (tid / 128, tid % 128) owns column j of rows r, r + 8, ...: no division per
+// element, row i's M[i][k] is one LDS word for all lanes of a row, M[k][j] runs along the lanes.
+__global__ __launch_bounds__(1024) void k_floyd_warshall(const uint8_t* __restrict__ adj, const int32_t* __restrict__ n_nodes,
+                                                         int n_max, int32_t* __restrict__ dist, int32_t* __restrict__ path) {
     extern __shared__ uint16_t lds[];
     const int g = blockIdx.x;
     const int n = n_nodes ? n_nodes[g] : n_max;
     uint16_t* M = lds;                                   // [n][n]
     int16_t* P = reinterpret_cast<int16_t*>(lds + n * n);
     const uint8_t* A = adj + (int64_t)g * n_max * n_max;
-    for (int t = threadIdx.x; t < n * n; t += 256) {
-        const int i = t / n, j = t % n;
-        const uint16_t w = A[i * n_max + j];
-        M[t] = i == j ? 0 : (w == 0 ? kFwInf : w);       // :27-32
-        P[t] = -1;
-    }
+    const int j = threadIdx.x % kFwMax, r = threadIdx.x / kFwMax;
+    constexpr int kRows = 1024 / kFwMax;
+    if (j < n)
+        for (int i = r; i < n; i += kRows) {
+            const uint16_t w = A[i * n_max + j];
+            M[i * n + j] = i == j ? 0 : (w == 0 ? kFwInf : w);       // :27-32
+            P[i * n + j] = -1;
+        }
     __syncthreads();
     for (int k = 0; k < n; ++k) {
-        for (int t = threadIdx.x; t < n * n; t += 256) {
-            const int i = t / n, j = t % n;
-            const uint16_t c = M[i * n + k] + M[k * n + j];
-            if (M[t] > c && i != k && j != k) {          // row k and column k never improve through k
-                M[t] = c;
-                P[t] = (int16_t)k;
+        if (j < n && j != k) {
+            const uint16_t kj = M[k * n + j];
+            for (int i = r; i < n; i += kRows) {
+                const uint16_t c = M[i * n + k] + kj;
+                if (M[i * n + j] > c && i != k) {        // row k and column k never improve through k
+                    M[i * n + j] = c;
+                    P[i * n + j] = (int16_t)k;
+                }
             }
         }
         __syncthreads();
     }
     int32_t* D = dist + (int64_t)g * n_max * n_max;
     int32_t* Q = path + (int64_t)g * n_max * n_max;
-    for (int t = threadIdx.x; t < n * n; t += 256) {
-        const int i = t / n, j = t % n;
-        const bool far = M[t] >= kFwInf;                 // :49-53
-        D[i * n_max + j] = far ? kFwInf : M[t];
-        Q[i * n_max + j] = far ? kFwInf : P[t];
-    }
+    if (j < n)
+        for (int i = r; i < n; i += kRows) {
+            const bool far = M[i * n + j] >= kFwInf;     // :49-53
+            D[i * n_max + j] = far ? kFwInf : M[i * n + j];
+            Q[i * n_max + j] = far ? kFwInf : P[i * n + j];
+        }
 }
 
 }  // namespace
@@ -541,7 +547,7 @@ int tgt_floyd_warshall(const uint8_t* d_adj, const int32_t* d_n_nodes, int num_g
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kFwMax * kFwMax * 4)));
         raised = true;
     }
-    hipLaunchKernelGGL(k_floyd_warshall, dim3(num_graphs), dim3(256), lds, (hipStream_t)stream, d_adj, d_n_nodes, n_max,
+    hipLaunchKernelGGL(k_floyd_warshall, dim3(num_graphs), dim3(1024), lds, (hipStream_t)stream, d_adj, d_n_nodes, n_max,
                        d_dist, d_path);
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
