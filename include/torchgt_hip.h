@@ -304,6 +304,11 @@ int tgt_layer_norm_bwd(const void* d_s, const void* d_gamma, const float* d_mean
  * h = 0.5 u (1 + erf(u / sqrt 2));  backward: du = dh * dh/du evaluated at u. */
 int tgt_gelu_fwd(const void* d_u, int64_t n, int dtype, void* d_h, void* stream);
 int tgt_gelu_bwd(const void* d_u, const void* d_dh, int64_t n, int dtype, void* d_du, void* stream);
+/* F.relu of the GT layers (models/gt_dist_node_level.py:258,285; MLPReadout :272), same shapes
+ * and limits as tgt_gelu_*: h = max(u, 0);  backward: du = dh where u > 0, else 0.  The kernel
+ * time is booked under the gelu slot of the per-kernel timing. */
+int tgt_relu_fwd(const void* d_u, int64_t n, int dtype, void* d_h, void* stream);
+int tgt_relu_bwd(const void* d_u, const void* d_dh, int64_t n, int dtype, void* d_du, void* stream);
 
 /* ---- graph-level attention bias ---------------------------------------------
  * GraphAttnBias.forward (models/graphormer_graph_level.py:94-156), edge_type other than

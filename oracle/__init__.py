@@ -37,6 +37,9 @@ graph_node_feature             torch.nn.functional.embedding; hand-computed answ
 graph-level graphormer_forward torch's layer_norm / linear / gelu / softmax
                                assembly; closed form without layers; node
                                relabelling and padding invariance
+gt_forward (node-level GT)     torch's layer_norm / linear / relu / softmax on a
+                               complete graph; closed form without layers;
+                               commutes with node relabelling
 metis partition labels         PARITY UNPINNED: dgl/METIS is absent; partition
                                ids are always an explicit input here
 =============================  ================================================

@@ -66,6 +66,8 @@ SIGNATURES = {
     "tgt_layer_norm_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _i64, _vp]),
     "tgt_gelu_fwd": (_i32, [_vp, _i64, _i32, _vp, _vp]),
     "tgt_gelu_bwd": (_i32, [_vp, _vp, _i64, _i32, _vp, _vp]),
+    "tgt_relu_fwd": (_i32, [_vp, _i64, _i32, _vp, _vp]),
+    "tgt_relu_bwd": (_i32, [_vp, _vp, _i64, _i32, _vp, _vp]),
     "tgt_graph_attn_bias_fwd": (_i32, [_vp, _vp, _vp, _i32, _vp, _i32, _vp, _i32, _vp, _i32, _i32, _i32, _i32, _vp, _vp]),
     "tgt_graph_attn_bias_bwd_workspace_bytes": (_i64, [_i32, _i32, _i32]),
     "tgt_graph_attn_bias_bwd": (_i32, [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _i64, _vp]),

@@ -205,7 +205,8 @@ __global__ __launch_bounds__(1024) void k_reduce_workers(const float* __restrict
 }
 
 // nn.GELU (exact): h = 0.5 u (1 + erf(u / sqrt 2));  dh/du = 0.5 (1 + erf(u / sqrt 2)) + u exp(-u^2 / 2) / sqrt(2 pi)
-template <typename T, bool BWD>
+// RELU: F.relu instead (the GT layers, models/gt_dist_node_level.py:258,285): h = max(u, 0); dh/du = 1 where u > 0.
+template <typename T, bool BWD, bool RELU = false>
 __global__ __launch_bounds__(kEwBlock) void k_gelu(const T* __restrict__ u, const T* __restrict__ dh, int64_t nvec,
                                                    T* __restrict__ out) {
     constexpr int VE = Vec<T>::N;
@@ -215,6 +216,10 @@ __global__ __launch_bounds__(kEwBlock) void k_gelu(const T* __restrict__ u, cons
         if (BWD) Vec<T>::load(dh + v * VE, d);
 #pragma unroll
         for (int i = 0; i < VE; ++i) {
+            if (RELU) {
+                o[i] = x[i] > 0.f ? (BWD ? d[i] : x[i]) : 0.f;
+                continue;
+            }
             const float cdf = 0.5f * (1.f + erff(x[i] * 0.70710678118654752f));
             if (!BWD) o[i] = x[i] * cdf;
             else o[i] = d[i] * (cdf + x[i] * __expf(-0.5f * x[i] * x[i]) * 0.39894228040143268f);
@@ -335,7 +340,7 @@ int tgt_layer_norm_bwd(const void* d_s, const void* d_gamma, const float* d_mean
     return TGT_OK;
 }
 
-static int gelu_call(const void* d_u, const void* d_dh, int64_t n, int dtype, void* d_out, void* stream, bool bwd) {
+static int gelu_call(const void* d_u, const void* d_dh, int64_t n, int dtype, void* d_out, void* stream, bool bwd, bool relu = false) {
     using namespace tgt;
     if (n < 0 || (dtype != TGT_DTYPE_F32 && dtype != TGT_DTYPE_BF16)) {
         set_error("tgt_gelu: bad size or dtype");
@@ -352,7 +357,15 @@ static int gelu_call(const void* d_u, const void* d_dh, int64_t n, int dtype, vo
     const int64_t nvec = n / ve;
     const dim3 grid(ew_grid(nvec, kEwBlock, 16384));
     KernelTimer t(KS_GELU, st);
-    if (dtype == TGT_DTYPE_F32) {
+    if (relu) {
+        if (dtype == TGT_DTYPE_F32) {
+            if (bwd) hipLaunchKernelGGL((k_gelu<float, true, true>), grid, dim3(kEwBlock), 0, st, (const float*)d_u, (const float*)d_dh, nvec, (float*)d_out);
+            else hipLaunchKernelGGL((k_gelu<float, false, true>), grid, dim3(kEwBlock), 0, st, (const float*)d_u, (const float*)nullptr, nvec, (float*)d_out);
+        } else {
+            if (bwd) hipLaunchKernelGGL((k_gelu<ebf16, true, true>), grid, dim3(kEwBlock), 0, st, (const ebf16*)d_u, (const ebf16*)d_dh, nvec, (ebf16*)d_out);
+            else hipLaunchKernelGGL((k_gelu<ebf16, false, true>), grid, dim3(kEwBlock), 0, st, (const ebf16*)d_u, (const ebf16*)nullptr, nvec, (ebf16*)d_out);
+        }
+    } else if (dtype == TGT_DTYPE_F32) {
         if (bwd) hipLaunchKernelGGL((k_gelu<float, true>), grid, dim3(kEwBlock), 0, st, (const float*)d_u, (const float*)d_dh, nvec, (float*)d_out);
         else hipLaunchKernelGGL((k_gelu<float, false>), grid, dim3(kEwBlock), 0, st, (const float*)d_u, (const float*)nullptr, nvec, (float*)d_out);
     } else {
@@ -369,6 +382,14 @@ int tgt_gelu_fwd(const void* d_u, int64_t n, int dtype, void* d_h, void* stream)
 
 int tgt_gelu_bwd(const void* d_u, const void* d_dh, int64_t n, int dtype, void* d_du, void* stream) {
     return gelu_call(d_u, d_dh, n, dtype, d_du, stream, true);
+}
+
+int tgt_relu_fwd(const void* d_u, int64_t n, int dtype, void* d_h, void* stream) {
+    return gelu_call(d_u, nullptr, n, dtype, d_h, stream, false, true);
+}
+
+int tgt_relu_bwd(const void* d_u, const void* d_dh, int64_t n, int dtype, void* d_du, void* stream) {
+    return gelu_call(d_u, d_dh, n, dtype, d_du, stream, true, true);
 }
 
 }  // extern "C"
