@@ -355,6 +355,16 @@ int tgt_graph_node_feature_bwd(const void* d_dout, const int64_t* d_x, const int
                                int Fx, int num_atoms, int num_in, int num_out, int b, int s, int C, int dtype, void* d_datom_table,
                                void* d_din_table, void* d_dout_table, void* d_dgraph_token, void* d_workspace,
                                int64_t workspace_bytes, void* stream);
+/* The input rows of the graph-level GT, `embedding_h(x).sum(dim=-2)` (models/gt_graph_level.py:301,334):
+ *   out[g, i, :] = sum_f table[x[g,i,f]]
+ * d_x: int64 [b, s, Fx]; d_table [num_rows, C]; d_out [b, s, C] of `dtype`.  No padding index: the
+ * backward gives every row its gradient (float sums with memory atomics, as above).  Ids outside
+ * the table are clamped to its range. */
+int tgt_embedding_sum_fwd(const int64_t* d_x, int Fx, const void* d_table, int num_rows, int b, int s, int C, int dtype, void* d_out,
+                          void* stream);
+int64_t tgt_embedding_sum_bwd_workspace_bytes(int num_rows, int C);
+int tgt_embedding_sum_bwd(const void* d_dout, const int64_t* d_x, int Fx, int num_rows, int b, int s, int C, int dtype, void* d_dtable,
+                          void* d_workspace, int64_t workspace_bytes, void* stream);
 /* GraphAttnBias.forward with edge_type == 'multi_hop' (models/graphormer_graph_level.py:94-156,
  * the path-encoding branch :119-147).  As tgt_graph_attn_bias_fwd, with the edge term replaced by
  *   (1 / hops) * sum_dd  mean_f edge_table[edge_input[g,i-1,j-1,dd,f]]  x  W[dd]        (i, j >= 1)

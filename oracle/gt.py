@@ -60,3 +60,14 @@ def gt_forward(p, x, edge_index, n_layers, num_heads):
         out = encoder_layer(out, p, f"layers.{l}.", edge_index, num_heads)
     out = mlp_readout(out[0], p)                                                          # :340
     return torch.log_softmax(out, dim=1)                                                  # :341
+
+
+def gt_graph_level_forward(p, x_ids, edge_index, n_layers, num_heads):
+    """``GT.forward`` of models/gt_graph_level.py:333-363 (one sequence per graph).  x_ids int64 [b, s, Fx];
+    edge_index over the flattened b * s axis.  Returns [b, output_dim].  Pinned in tests/test_oracle_gt.py by
+    the closed form without layers and by the independence of the graphs of a batch."""
+    out = p["embedding_h.weight"][x_ids].sum(dim=-2)                                      # :334
+    for l in range(n_layers):                                                             # :344-349
+        out = encoder_layer(out, p, f"layers.{l}.", edge_index, num_heads)
+    out = out.mean(dim=1)                                                                 # :357
+    return mlp_readout(out, p)                                                            # :360

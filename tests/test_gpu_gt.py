@@ -98,3 +98,84 @@ def test_gt_forward_backward_matches_oracle(cuda, dtype):
         tail = {k: v for k, v in errs.items() if k.startswith("MLP_layer")}
         assert tail and max(tail.values()) <= 6e-2, tail
         assert np.median(list(errs.values())) <= 6e-2
+
+
+@pytest.mark.parametrize("attn_type", ["sparse", "full"])
+def test_graph_level_gt_matches_oracle(cuda, attn_type):
+    """GT of models/gt_graph_level.py (3 layers, hidden 64, 8 heads, ZINC table) on 10 padded ER graphs whose edges
+    index the flattened batch: outputs [b, 1] and every parameter gradient, float32.  With attn_type 'full' the
+    reference attends densely over all rows of a graph, padding included (no bias, no mask); that path runs on bf16
+    matrix instructions here: the bf16 module bar."""
+    from torchgt_amd.gt import GraphLevelGT
+    import types
+    from oracle import dense_attention as oda
+    print(f"graph-level GT case: {attn_type}", flush=True)
+    data = workloads.erdos_renyi_batch(batch=10, seed=31)
+    sizes = data["n_nodes"]
+    b, s = len(sizes), data["spatial_pos"].shape[1]
+    rng = np.random.default_rng(5)
+    x = np.zeros((b, s, 2), np.int64)
+    edges = []
+    for g in range(b):
+        n = int(sizes[g])
+        x[g, :n] = rng.integers(1, 64, size=(n, 2))
+        src, dst = np.nonzero(data["spatial_pos"][g][:n, :n] == 2)
+        loops = np.arange(n)
+        edges.append(np.stack([np.concatenate([src, loops]), np.concatenate([dst, loops])]) + g * s)
+    ei = torch.from_numpy(np.concatenate(edges, 1))
+    x = torch.from_numpy(x)
+    torch.manual_seed(3)
+    n_layers, H = 3, 8
+    m = GraphLevelGT(n_layers, H, 64, 0.0, 0.0, 64, "ZINC", "single_hop", 5, 0.0, 1)
+    assert {"embedding_h.weight", "graph_token.weight", "MLP_layer.FC_layers.0.weight", "layers.2.O.bias"} <= set(m.state_dict())
+    with torch.no_grad():
+        for k, p in m.named_parameters():
+            if p.dim() == 2:
+                p.normal_(0, 0.05 if ("linear_q" in k or "linear_k" in k) and attn_type == "full" else 0.15)
+    names = [k for k, _ in m.named_parameters()]
+    pd = {k: v.detach().double().requires_grad_(True) for k, v in m.named_parameters()}
+    if attn_type == "sparse":
+        want = ogt.gt_graph_level_forward(pd, x, ei, n_layers, H)
+    else:
+        # the same layers with the dense attention of the graph-level CoreAttention (q * sqrt(d), softmax over all s keys)
+        out = pd["embedding_h.weight"][x].sum(-2)
+        lin = lambda v, nme: v @ pd[nme + ".weight"].t() + pd[nme + ".bias"]
+        for l in range(n_layers):
+            pre = f"layers.{l}."
+            q, k, v = (lin(out, pre + "self_attention." + nme).view(b, s, H, 8) for nme in ("linear_q", "linear_k", "linear_v"))
+            y = lin(oda.dense_attention(q, k, v, None), pre + "O")
+            out = ogt.layer_norm(out + y, pd[pre + "layer_norm1.weight"], pd[pre + "layer_norm1.bias"])
+            y = lin(ogt.relu(lin(y, pre + "FFN_layer1")), pre + "FFN_layer2")
+            out = ogt.layer_norm(out + y, pd[pre + "layer_norm2.weight"], pd[pre + "layer_norm2.bias"])
+        want = ogt.mlp_readout(out.mean(1), pd)
+    target = torch.randn(want.shape, generator=torch.Generator().manual_seed(6)).double()
+    ref = torch.autograd.grad(((want - target) ** 2).mean(), [pd[k] for k in names], allow_unused=True)
+    mc = m.to(cuda)
+    got = mc(types.SimpleNamespace(x=x.to(cuda), edge_index=ei.to(cuda)), attn_type=attn_type)
+    assert got.shape == want.shape == (b, 1)
+    tol = 1e-4 if attn_type == "sparse" else 6e-2
+    assert err(got, want) <= tol, err(got, want)
+    # the same upstream gradient on both sides (the oracle's dL/d output), so that the backward is compared by itself
+    dl = (2 * (want - target) / want.numel()).detach()
+    got_g = torch.autograd.grad(got, [p for _, p in mc.named_parameters()], dl.to(cuda, got.dtype), allow_unused=True)
+    scale = max(r.abs().max().item() for r in ref if r is not None)
+    unused, errs = [], {}
+    for k, a, r in zip(names, got_g, ref):
+        assert (a is None) == (r is None), k
+        if r is None:
+            unused.append(k)
+        elif r.abs().max().item() < 1e-3 * scale:
+            assert a.detach().double().abs().max().item() <= 2e-2 * scale, k
+        else:
+            errs[k] = err(a, r)
+    assert sorted(unused) == sorted([f"layers.{l}.self_attention_norm.{w}" for l in range(n_layers) for w in ("weight", "bias")]
+                                    + ["graph_token.weight"])
+    print("gradient errs", {k: round(v, 6) for k, v in errs.items()}, flush=True)
+    # 'full': the activations carry bf16-sized noise from the dense attention, and a ReLU unit whose input is within
+    # that noise of zero takes the other branch: with ten graphs one such unit of the readout moves its layer's
+    # gradient by several percent.  The bar there is 0.15 on every tensor and the module bar on the median.
+    gtol = tol if attn_type == "sparse" else 0.15
+    bad = {k: v for k, v in errs.items() if v > gtol}
+    assert not bad, bad
+    assert np.median(list(errs.values())) <= tol
+    assert "embedding_h.weight" in errs and got_g[names.index("embedding_h.weight")][0].abs().max() > 0     # row 0 is an ordinary row

@@ -89,3 +89,26 @@ def test_gt_commutes_with_node_relabelling():
     xp[perm] = x
     got = ogt.gt_forward(p, xp, perm[e], 2, H)
     torch.testing.assert_close(got[perm], base, rtol=1e-10, atol=1e-12)
+
+
+def test_graph_level_gt_closed_form_and_batch_independence():
+    g = torch.Generator().manual_seed(8)
+    p = make_params(2, seed=7)
+    p["embedding_h.weight"] = torch.randn(11, HID, generator=g, dtype=torch.float64) * 0.3
+    b, s = 3, 5
+    x = torch.randint(0, 11, (b, s, 2), generator=g)
+    # without layers: readout of the mean of the summed embeddings
+    got = ogt.gt_graph_level_forward(p, x, torch.zeros(2, 0, dtype=torch.long), 0, H)
+    h = torch.stack([sum(p["embedding_h.weight"][int(x[gi, i, f])] for i in range(s) for f in range(2)) / s for gi in range(b)])
+    want = ogt.mlp_readout(h, p)
+    torch.testing.assert_close(got, want, rtol=1e-12, atol=1e-13)
+    # edges inside the graphs only: every graph's output is what it gets alone
+    edges = []
+    for gi in range(b):
+        e = torch.randint(0, s, (2, 8), generator=g)
+        e = torch.cat([e, torch.arange(s).repeat(2, 1)], 1)
+        edges.append(e + gi * s)
+    full = ogt.gt_graph_level_forward(p, x, torch.cat(edges, 1), 2, H)
+    for gi in range(b):
+        alone = ogt.gt_graph_level_forward(p, x[gi:gi + 1], edges[gi] - gi * s, 2, H)
+        torch.testing.assert_close(full[gi:gi + 1], alone, rtol=1e-10, atol=1e-12)

@@ -11,7 +11,7 @@ from .multi_head_attention import MultiHeadAttention, LinearFunction, fused_line
 from .encoder import FeedForwardNetwork, EncoderLayer, Graphormer
 from .graph_bias import GraphAttnBias, floyd_warshall, gen_edge_input
 from .graph_level import GraphNodeFeature, Graphormer as GraphLevelGraphormer
-from .gt import GT, MLPReadout
+from .gt import GT, GraphLevelGT, MLPReadout
 from .block_attention import BlockAttentionFunction, TileSet, block_attention, expand_tiles
 
 __all__ = ["CoreAttention", "SparseAttentionFunction", "DenseAttentionFunction", "sparse_attention",
@@ -19,4 +19,4 @@ __all__ = ["CoreAttention", "SparseAttentionFunction", "DenseAttentionFunction",
            "GraphPlan", "get_plan", "clear_plan_cache", "BlockAttentionFunction", "TileSet", "block_attention",
            "expand_tiles", "MultiHeadAttention", "LinearFunction", "fused_linear",
            "FeedForwardNetwork", "EncoderLayer", "Graphormer", "GraphAttnBias", "floyd_warshall", "gen_edge_input",
-           "GraphNodeFeature", "GraphLevelGraphormer", "GT", "MLPReadout"]
+           "GraphNodeFeature", "GraphLevelGraphormer", "GT", "GraphLevelGT", "MLPReadout"]

@@ -81,6 +81,9 @@ SIGNATURES = {
     "tgt_graph_node_feature_bwd_workspace_bytes": (_i64, [_i32, _i32, _i32, _i32]),
     "tgt_graph_node_feature_bwd": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp,
                                           _i64, _vp]),
+    "tgt_embedding_sum_fwd": (_i32, [_vp, _i32, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp]),
+    "tgt_embedding_sum_bwd_workspace_bytes": (_i64, [_i32, _i32]),
+    "tgt_embedding_sum_bwd": (_i32, [_vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _i64, _vp]),
     "tgt_gen_edge_input": (_i32, [_vp, _vp, _i32, _i32, _vp, _i32, _i32, _i32, _vp, _vp]),
     "tgt_probe_row_gather": (_i32, [_vp, _i64, _i32, _vp, _i64, _vp, _vp]),
     "tgt_timing_enable": (_i32, [_i32]),

@@ -31,6 +31,8 @@ struct NodeFeatArgs {
     const int64_t* in_degree;    // [b, s]
     const int64_t* out_degree;   // [b, s]
     int b, s, Fx, C, num_atoms, num_in, num_out;
+    int pad_rows;                // 1: row 0 of the atom table is a padding index (no gradient); 0: an ordinary row
+    int has_degree, has_token;   // without degrees: the atom sum alone; without token: s rows per graph, no row 0
 };
 
 // one thread per (graph, node, channel), channel fastest
@@ -38,13 +40,14 @@ template <typename T>
 __global__ __launch_bounds__(256) void k_node_feature_fwd(NodeFeatArgs a, const T* __restrict__ atom, const T* __restrict__ tin,
                                                           const T* __restrict__ tout, const T* __restrict__ token,
                                                           T* __restrict__ out) {
-    const int64_t total = (int64_t)a.b * (a.s + 1) * a.C;
+    const int rows = a.s + a.has_token;
+    const int64_t total = (int64_t)a.b * rows * a.C;
     const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (t >= total) return;
     const int c = (int)(t % a.C);
     const int64_t row = t / a.C;
-    const int node = (int)(row % (a.s + 1));
-    const int64_t g = row / (a.s + 1);
+    const int node = (int)(row % rows) + 1 - a.has_token;             // 0 = the graph token's row
+    const int64_t g = row / rows;
     float v;
     if (node == 0) {
         v = ldf(token + c);                                           // (:52-56)
@@ -52,8 +55,10 @@ __global__ __launch_bounds__(256) void k_node_feature_fwd(NodeFeatArgs a, const 
         const int64_t p = g * a.s + (node - 1);
         v = 0.f;
         for (int f = 0; f < a.Fx; ++f) v += ldf(atom + (int64_t)clamp_id(a.x[p * a.Fx + f], a.num_atoms) * a.C + c);   // (:45)
-        v += ldf(tin + (int64_t)clamp_id(a.in_degree[p], a.num_in) * a.C + c);                                          // (:46-50)
-        v += ldf(tout + (int64_t)clamp_id(a.out_degree[p], a.num_out) * a.C + c);
+        if (a.has_degree) {
+            v += ldf(tin + (int64_t)clamp_id(a.in_degree[p], a.num_in) * a.C + c);                                      // (:46-50)
+            v += ldf(tout + (int64_t)clamp_id(a.out_degree[p], a.num_out) * a.C + c);
+        }
     }
     stf(out + t, v);
 }
@@ -66,13 +71,14 @@ __global__ __launch_bounds__(256) void k_fill_zero(float* __restrict__ p, int64_
 // acc: float [num_atoms + num_in + num_out + 1][C]
 template <typename T>
 __global__ __launch_bounds__(256) void k_node_feature_bwd(NodeFeatArgs a, const T* __restrict__ dout, float* __restrict__ acc) {
-    const int64_t total = (int64_t)a.b * (a.s + 1) * a.C;
+    const int rows = a.s + a.has_token;
+    const int64_t total = (int64_t)a.b * rows * a.C;
     const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (t >= total) return;
     const int c = (int)(t % a.C);
     const int64_t row = t / a.C;
-    const int node = (int)(row % (a.s + 1));
-    const int64_t g = row / (a.s + 1);
+    const int node = (int)(row % rows) + 1 - a.has_token;
+    const int64_t g = row / rows;
     const float d = ldf(dout + t);
     if (d == 0.f) return;
     float* acc_in = acc + (int64_t)a.num_atoms * a.C;
@@ -85,8 +91,9 @@ __global__ __launch_bounds__(256) void k_node_feature_bwd(NodeFeatArgs a, const 
     const int64_t p = g * a.s + (node - 1);
     for (int f = 0; f < a.Fx; ++f) {
         const int id = clamp_id(a.x[p * a.Fx + f], a.num_atoms);
-        if (id > 0) atomicAdd(acc + (int64_t)id * a.C + c, d);        // row 0 = padding index
+        if (id >= a.pad_rows) atomicAdd(acc + (int64_t)id * a.C + c, d);        // row 0 = padding index
     }
+    if (!a.has_degree) return;
     const int ii = clamp_id(a.in_degree[p], a.num_in), io = clamp_id(a.out_degree[p], a.num_out);
     if (ii > 0) atomicAdd(acc_in + (int64_t)ii * a.C + c, d);
     if (io > 0) atomicAdd(acc_out + (int64_t)io * a.C + c, d);
@@ -117,6 +124,56 @@ int node_feat_check(int b, int s, int Fx, int C, int num_atoms, int num_in, int 
 }  // namespace
 }  // namespace tgt
 
+namespace tgt {
+namespace {
+
+int node_feature_fwd_impl(NodeFeatArgs a, const void* d_atom_table, const void* d_in_table, const void* d_out_table,
+                          const void* d_graph_token, int dtype, void* d_out, void* stream) {
+    const int64_t total = (int64_t)a.b * (a.s + a.has_token) * a.C;
+    if (total == 0) return TGT_OK;
+    const dim3 grid((unsigned)((total + 255) / 256));
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == TGT_DTYPE_F32)
+        hipLaunchKernelGGL((k_node_feature_fwd<float>), grid, dim3(256), 0, st, a, (const float*)d_atom_table, (const float*)d_in_table,
+                           (const float*)d_out_table, (const float*)d_graph_token, (float*)d_out);
+    else
+        hipLaunchKernelGGL((k_node_feature_fwd<nbf16>), grid, dim3(256), 0, st, a, (const nbf16*)d_atom_table, (const nbf16*)d_in_table,
+                           (const nbf16*)d_out_table, (const nbf16*)d_graph_token, (nbf16*)d_out);
+    TGT_HIP_CHECK(hipGetLastError());
+    return TGT_OK;
+}
+
+// acc layout: [num_atoms][C], [num_in][C], [num_out][C], [1][C]; tables that are not in use have num = 0 rows here
+int node_feature_bwd_impl(NodeFeatArgs a, const void* d_dout, int dtype, void* d_datom, void* d_din, void* d_dout_table,
+                          void* d_dtoken, float* acc, void* stream) {
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t n_atom = (int64_t)a.num_atoms * a.C, n_in = a.has_degree ? (int64_t)a.num_in * a.C : 0,
+                  n_out = a.has_degree ? (int64_t)a.num_out * a.C : 0, n_tok = a.has_token ? a.C : 0;
+    const int64_t n_acc = n_atom + n_in + n_out + n_tok;
+    if (!a.has_degree) a.num_in = a.num_out = 0;          // the kernel's offsets of the sums that follow the atom table
+    hipLaunchKernelGGL(k_fill_zero, dim3((unsigned)((n_acc + 255) / 256)), dim3(256), 0, st, acc, n_acc);
+    const int64_t total = (int64_t)a.b * (a.s + a.has_token) * a.C;
+    const dim3 fgrid((unsigned)((n_acc + 255) / 256));
+    if (dtype == TGT_DTYPE_F32) {
+        if (total > 0)
+            hipLaunchKernelGGL((k_node_feature_bwd<float>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, a,
+                               (const float*)d_dout, acc);
+        hipLaunchKernelGGL((k_node_feature_finish<float>), fgrid, dim3(256), 0, st, (const float*)acc, n_atom, n_in, n_out, n_tok,
+                           (float*)d_datom, (float*)d_din, (float*)d_dout_table, (float*)d_dtoken);
+    } else {
+        if (total > 0)
+            hipLaunchKernelGGL((k_node_feature_bwd<nbf16>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, a,
+                               (const nbf16*)d_dout, acc);
+        hipLaunchKernelGGL((k_node_feature_finish<nbf16>), fgrid, dim3(256), 0, st, (const float*)acc, n_atom, n_in, n_out, n_tok,
+                           (nbf16*)d_datom, (nbf16*)d_din, (nbf16*)d_dout_table, (nbf16*)d_dtoken);
+    }
+    TGT_HIP_CHECK(hipGetLastError());
+    return TGT_OK;
+}
+
+}  // namespace
+}  // namespace tgt
+
 extern "C" {
 
 int tgt_graph_node_feature_fwd(const int64_t* d_x, const int64_t* d_in_degree, const int64_t* d_out_degree, int Fx,
@@ -131,18 +188,8 @@ int tgt_graph_node_feature_fwd(const int64_t* d_x, const int64_t* d_in_degree, c
         set_error("tgt_graph_node_feature_fwd: null pointer");
         return TGT_ERR_INVALID_ARG;
     }
-    NodeFeatArgs a{d_x, d_in_degree, d_out_degree, b, s, Fx, C, num_atoms, num_in, num_out};
-    const int64_t total = (int64_t)b * (s + 1) * C;
-    const dim3 grid((unsigned)((total + 255) / 256));
-    hipStream_t st = (hipStream_t)stream;
-    if (dtype == TGT_DTYPE_F32)
-        hipLaunchKernelGGL((k_node_feature_fwd<float>), grid, dim3(256), 0, st, a, (const float*)d_atom_table, (const float*)d_in_table,
-                           (const float*)d_out_table, (const float*)d_graph_token, (float*)d_out);
-    else
-        hipLaunchKernelGGL((k_node_feature_fwd<nbf16>), grid, dim3(256), 0, st, a, (const nbf16*)d_atom_table, (const nbf16*)d_in_table,
-                           (const nbf16*)d_out_table, (const nbf16*)d_graph_token, (nbf16*)d_out);
-    TGT_HIP_CHECK(hipGetLastError());
-    return TGT_OK;
+    NodeFeatArgs a{d_x, d_in_degree, d_out_degree, b, s, Fx, C, num_atoms, num_in, num_out, 1, 1, 1};
+    return node_feature_fwd_impl(a, d_atom_table, d_in_table, d_out_table, d_graph_token, dtype, d_out, stream);
 }
 
 int64_t tgt_graph_node_feature_bwd_workspace_bytes(int num_atoms, int num_in, int num_out, int C) {
@@ -167,29 +214,45 @@ int tgt_graph_node_feature_bwd(const void* d_dout, const int64_t* d_x, const int
         set_error("tgt_graph_node_feature_bwd: workspace of %lld bytes needed, got %lld", (long long)need, (long long)workspace_bytes);
         return TGT_ERR_WORKSPACE;
     }
-    NodeFeatArgs a{d_x, d_in_degree, d_out_degree, b, s, Fx, C, num_atoms, num_in, num_out};
-    hipStream_t st = (hipStream_t)stream;
-    float* acc = (float*)d_workspace;
-    const int64_t n_acc = need / (int64_t)sizeof(float);
-    hipLaunchKernelGGL(k_fill_zero, dim3((unsigned)((n_acc + 255) / 256)), dim3(256), 0, st, acc, n_acc);
-    const int64_t total = (int64_t)b * (s + 1) * C;
-    const int64_t n_atom = (int64_t)num_atoms * C, n_in = (int64_t)num_in * C, n_out = (int64_t)num_out * C;
-    const dim3 fgrid((unsigned)((n_acc + 255) / 256));
-    if (dtype == TGT_DTYPE_F32) {
-        if (total > 0)
-            hipLaunchKernelGGL((k_node_feature_bwd<float>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, a,
-                               (const float*)d_dout, acc);
-        hipLaunchKernelGGL((k_node_feature_finish<float>), fgrid, dim3(256), 0, st, (const float*)acc, n_atom, n_in, n_out, (int64_t)C,
-                           (float*)d_datom_table, (float*)d_din_table, (float*)d_dout_table, (float*)d_dgraph_token);
-    } else {
-        if (total > 0)
-            hipLaunchKernelGGL((k_node_feature_bwd<nbf16>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, a,
-                               (const nbf16*)d_dout, acc);
-        hipLaunchKernelGGL((k_node_feature_finish<nbf16>), fgrid, dim3(256), 0, st, (const float*)acc, n_atom, n_in, n_out, (int64_t)C,
-                           (nbf16*)d_datom_table, (nbf16*)d_din_table, (nbf16*)d_dout_table, (nbf16*)d_dgraph_token);
+    NodeFeatArgs a{d_x, d_in_degree, d_out_degree, b, s, Fx, C, num_atoms, num_in, num_out, 1, 1, 1};
+    return node_feature_bwd_impl(a, d_dout, dtype, d_datom_table, d_din_table, d_dout_table, d_dgraph_token, (float*)d_workspace, stream);
+}
+
+int tgt_embedding_sum_fwd(const int64_t* d_x, int Fx, const void* d_table, int num_rows, int b, int s, int C, int dtype, void* d_out,
+                          void* stream) {
+    using namespace tgt;
+    const int rc = node_feat_check(b, s, Fx, C, num_rows, 1, 1, dtype, "tgt_embedding_sum_fwd");
+    if (rc != TGT_OK) return rc;
+    if (b == 0 || s == 0) return TGT_OK;
+    if (!d_table || !d_out || !d_x) {
+        set_error("tgt_embedding_sum_fwd: null pointer");
+        return TGT_ERR_INVALID_ARG;
     }
-    TGT_HIP_CHECK(hipGetLastError());
-    return TGT_OK;
+    NodeFeatArgs a{d_x, nullptr, nullptr, b, s, Fx, C, num_rows, 1, 1, 0, 0, 0};
+    return node_feature_fwd_impl(a, d_table, nullptr, nullptr, nullptr, dtype, d_out, stream);
+}
+
+int64_t tgt_embedding_sum_bwd_workspace_bytes(int num_rows, int C) {
+    if (num_rows < 1 || C < 1) return 0;
+    return (int64_t)sizeof(float) * num_rows * C;
+}
+
+int tgt_embedding_sum_bwd(const void* d_dout, const int64_t* d_x, int Fx, int num_rows, int b, int s, int C, int dtype, void* d_dtable,
+                          void* d_workspace, int64_t workspace_bytes, void* stream) {
+    using namespace tgt;
+    const int rc = node_feat_check(b, s, Fx, C, num_rows, 1, 1, dtype, "tgt_embedding_sum_bwd");
+    if (rc != TGT_OK) return rc;
+    if (!d_dtable || (b > 0 && s > 0 && (!d_dout || !d_x))) {
+        set_error("tgt_embedding_sum_bwd: null pointer");
+        return TGT_ERR_INVALID_ARG;
+    }
+    const int64_t need = tgt_embedding_sum_bwd_workspace_bytes(num_rows, C);
+    if (!d_workspace || workspace_bytes < need) {
+        set_error("tgt_embedding_sum_bwd: workspace of %lld bytes needed, got %lld", (long long)need, (long long)workspace_bytes);
+        return TGT_ERR_WORKSPACE;
+    }
+    NodeFeatArgs a{d_x, nullptr, nullptr, b, s, Fx, C, num_rows, 1, 1, 0, 0, 0};
+    return node_feature_bwd_impl(a, d_dout, dtype, d_dtable, nullptr, nullptr, nullptr, (float*)d_workspace, stream);
 }
 
 }  // extern "C"

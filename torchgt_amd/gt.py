@@ -113,3 +113,76 @@ class GT(nn.Module):
             output = enc_layer(output, edge_index=edge_index, attn_type=attn_type)
         output = self.MLP_layer(output[0, :, :])
         return F.log_softmax(output, dim=1)
+
+
+class EmbeddingSumFunction(torch.autograd.Function):
+    """``embedding(x).sum(dim=-2)`` for integer features x [b, s, Fx] and a table without padding index."""
+
+    @staticmethod
+    def forward(ctx, x, table):
+        if not x.is_cuda:
+            raise RuntimeError("torchgt_amd kernels run on the GPU only (no CPU fallback)")
+        dt = table.dtype
+        if dt not in _DT:
+            raise TypeError(f"unsupported dtype {dt}")
+        b, s, Fx = x.shape
+        x = x.to(torch.int64).contiguous()
+        tab = table.contiguous()
+        out = torch.empty((b, s, tab.shape[1]), dtype=dt, device=x.device)
+        with torch.cuda.device(x.device):
+            _lib.check(_lib.lib().tgt_embedding_sum_fwd(x.data_ptr(), Fx, tab.data_ptr(), tab.shape[0], b, s, tab.shape[1], _DT[dt],
+                                                        out.data_ptr(), _stream(x)))
+        ctx.save_for_backward(x)
+        ctx.dims = (b, s, Fx, tab.shape[0], tab.shape[1], dt)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        (x,) = ctx.saved_tensors
+        b, s, Fx, rows, C, dt = ctx.dims
+        L = _lib.lib()
+        dout = dout.to(dt).contiguous()
+        d_tab = torch.empty((rows, C), dtype=dt, device=dout.device)
+        nbytes = L.tgt_embedding_sum_bwd_workspace_bytes(rows, C)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dout.device)
+        with torch.cuda.device(dout.device):
+            _lib.check(L.tgt_embedding_sum_bwd(dout.data_ptr(), x.data_ptr(), Fx, rows, b, s, C, _DT[dt], d_tab.data_ptr(),
+                                               ws.data_ptr(), nbytes, _stream(dout)))
+        return None, d_tab
+
+
+class GraphLevelEncoderLayer(EncoderLayer):
+    """models/gt_graph_level.py:210-254: the same layer with the reference's unused ``mask`` argument."""
+
+    def forward(self, x, attn_bias=None, mask=None, edge_index=None, attn_type=None):
+        if mask is not None:
+            raise NotImplementedError("the reference never passes `mask` (gt_graph_level.py:344-348)")
+        return super().forward(x, attn_bias, edge_index=edge_index, attn_type=attn_type)
+
+
+class GraphLevelGT(nn.Module):
+    """GT for graph-level tasks, one sequence per graph (models/gt_graph_level.py:276-363; class ``GT`` there).
+    The node rows are the summed embeddings of the integer features, the edges of all graphs of the batch
+    index the flattened [b * s] axis, the graph representation is the mean over all s rows (padding included,
+    as in the reference) and the readout is ``MLPReadout``.  ``graph_token`` is constructed and not used."""
+
+    def __init__(self, n_layers, num_heads, hidden_dim, dropout_rate, intput_dropout_rate, ffn_dim, dataset_name, edge_type,
+                 multi_hop_max_dist, attention_dropout_rate, output_dim):
+        super().__init__()
+        num_atoms = {"ZINC": 64, "MalNet": 560000}.get(dataset_name, 7000)          # :294-315
+        self.embedding_h = nn.Embedding(num_atoms, hidden_dim)
+        self.graph_token = nn.Embedding(1, hidden_dim)
+        self.input_dropout = nn.Dropout(intput_dropout_rate)
+        self.layers = nn.ModuleList([GraphLevelEncoderLayer(hidden_dim, ffn_dim, dropout_rate, attention_dropout_rate, num_heads)
+                                     for _ in range(n_layers)])
+        self.MLP_layer = MLPReadout(hidden_dim, output_dim)
+        self.apply(lambda module: init_params(module, n_layers=n_layers))
+
+    def forward(self, batched_data, perturb=None, attn_type=None):
+        x = EmbeddingSumFunction.apply(batched_data.x, self.embedding_h.weight)     # :334
+        output = self.input_dropout(x)
+        edge_index = batched_data.edge_index
+        for enc_layer in self.layers:
+            output = enc_layer(output, edge_index=edge_index, attn_type=attn_type)
+        output = output.mean(dim=1)                                                 # :357
+        return self.MLP_layer(output)
