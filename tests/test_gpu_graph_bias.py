@@ -186,6 +186,37 @@ def test_graph_attn_bias_multi_hop_matches_oracle(cuda, dtype, H, F, D0, mhd):
     assert not got_g[2].reshape(n_dis, H, H)[D:].any() and got_g[2].reshape(n_dis, H, H)[:D].any()
 
 
+def test_graph_attn_bias_multi_hop_without_hops_is_the_spatial_and_virtual_part(cuda):
+    # an edge_input that holds no hops (the reference's reshape raises on it): the edge term vanishes, forward and
+    # gradients still come out; the single-hop oracle with an all-zero edge table is the same sum
+    data = workloads.erdos_renyi_batch(batch=4, seed=9)
+    H = 8
+    m = GraphAttnBias(H, 512, 5, 22, 3, 64, "multi_hop", 5)
+    with torch.no_grad():
+        m.spatial_pos_encoder.weight.normal_(0, 0.5); m.spatial_pos_encoder.weight[0] = 0
+        m.graph_token_virtual_distance.weight.normal_(0, 0.5)
+    attn_bias = torch.from_numpy(data["attn_bias"])
+    spatial_pos = torch.from_numpy(data["spatial_pos"]).long()
+    b, s = spatial_pos.shape[:2]
+    edge_input = torch.zeros(b, s, s, 0, 1, dtype=torch.long)
+    params = [p.detach().double().requires_grad_(True) for p in (m.spatial_pos_encoder.weight, m.edge_encoder.weight,
+                                                                 m.edge_dis_encoder.weight, m.graph_token_virtual_distance.weight)]
+    want = oda.graph_attn_bias(attn_bias.double(), spatial_pos, torch.zeros(b, s, s, 1, dtype=torch.long), params[0],
+                               torch.zeros(5, H, dtype=torch.float64), params[3])
+    mc = m.to(cuda)
+    got = mc(types.SimpleNamespace(attn_bias=attn_bias.to(cuda), spatial_pos=spatial_pos.to(cuda), edge_input=edge_input.to(cuda)))
+    assert err(got, want) <= 1e-5
+    dout = torch.randn(want.shape, generator=torch.Generator().manual_seed(1))
+    dout[~torch.isfinite(want)] = 0
+    finite = torch.where(torch.isfinite(want), want, torch.zeros_like(want))
+    ref = torch.autograd.grad((finite * dout.double()).sum(), [params[0], params[3]])
+    ref[0][0] = 0
+    g = torch.autograd.grad(got, [mc.spatial_pos_encoder.weight, mc.edge_encoder.weight, mc.edge_dis_encoder.weight,
+                                  mc.graph_token_virtual_distance.weight], dout.to(cuda))
+    assert err(g[0], ref[0]) <= 1e-5 and err(g[3], ref[1]) <= 1e-5
+    assert not g[1].any() and not g[2].any()
+
+
 def test_graph_attn_bias_multi_hop_rejects_more_hops_than_matrices(cuda):
     m = GraphAttnBias(8, 512, 5, 22, 2, 64, "multi_hop", 0).to(cuda)       # two hop matrices, three hops of input
     batch = types.SimpleNamespace(attn_bias=torch.zeros(1, 4, 4, device=cuda), spatial_pos=torch.ones(1, 3, 3, dtype=torch.long, device=cuda),
