@@ -671,6 +671,44 @@ def bench_graph_model(args):
     L.tgt_timing_enable(0)
     kernels = {k: {"avg_us": t / c * 1e3, "launches_per_step": c / args.steps} for k, (t, c) in _lib.kernel_timings().items() if c}
     lib_us = sum(v["avg_us"] * v["launches_per_step"] for v in kernels.values())
+    # The same step captured once into a HIP graph and replayed (the library calls only launch kernels); a fresh model
+    # and optimizer, warmed up on a side stream, as for the node-level model.
+    graph_ms = None
+    if args.hip_graph:
+        loss_value = float(loss.detach())
+        del loss
+        torch.manual_seed(42)
+        gm = Graphormer(4, 8, 64, 0.0, 0.0, 64, "ZINC", "single_hop", 5, 0.0, 1).to(dev, tdt)
+        gopt = torch.optim.AdamW(gm.parameters(), lr=1e-3, weight_decay=0.01, capturable=True)
+
+        def gstep():
+            gloss = torch.nn.functional.l1_loss(gm(batch).float().view(-1), y)
+            gloss.backward()
+            gopt.step()
+            return gloss
+
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                gopt.zero_grad(set_to_none=True)
+                gstep()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        gr = torch.cuda.CUDAGraph()
+        gopt.zero_grad(set_to_none=True)
+        with torch.cuda.graph(gr):
+            gstep()
+        for _ in range(args.warmup):
+            gr.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            gr.replay()
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - t0) / args.steps * 1e3
+    else:
+        loss_value = float(loss.detach())
     groups = {"dense attention": ("dense_fwd", "dense_bwd"), "bias builder": ("graph_bias_fwd", "graph_bias_bwd"),
               "projections and ffn linears": ("linear_fwd", "linear_dx", "linear_dw"),
               "layer norm + residual": ("layer_norm_fwd", "layer_norm_bwd"), "gelu": ("gelu",)}
@@ -683,7 +721,8 @@ def bench_graph_model(args):
                                "Graphormer 4 x (hidden 64, ffn 64, 8 heads), ZINC tables, dropout 0", "b": b, "S": s + 1,
                    "parameters": sum(p.numel() for p in m.parameters()),
                    "step": "forward + l1_loss + backward + torch AdamW", "parallelism": "1 GPU"},
-        "loss": float(loss.detach()),
+        "loss": loss_value,
+        "ms_per_step_hip_graph": graph_ms,
         "library_kernel_us_per_step": lib_us,
         "kernel_groups_us": {g: sum(kernels[k]["avg_us"] * kernels[k]["launches_per_step"] for k in ks if k in kernels)
                              for g, ks in groups.items()},
