@@ -41,14 +41,16 @@ def node_inputs(data, num_atoms, num_deg, Fx, seed):
     return torch.from_numpy(x), torch.from_numpy(deg)
 
 
+# tables of 64 rows are summed in LDS by the backward, the molecule-sized ones (4 609 atom types, 512 degrees) with
+# memory atomics
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("C,Fx", [(64, 1), (64, 3), (40, 2)])
-def test_graph_node_feature_matches_oracle(cuda, dtype, C, Fx):
-    print(f"graph_node_feature case: C={C} Fx={Fx} {dtype}", flush=True)
+@pytest.mark.parametrize("C,Fx,num_atoms,num_deg", [(64, 1, 64, 64), (64, 3, 64, 64), (40, 2, 64, 64), (64, 3, 4609, 512)])
+def test_graph_node_feature_matches_oracle(cuda, dtype, C, Fx, num_atoms, num_deg):
+    print(f"graph_node_feature case: C={C} Fx={Fx} tables {num_atoms}/{num_deg} {dtype}", flush=True)
     data = workloads.erdos_renyi_batch(batch=12, seed=11)
-    x, deg = node_inputs(data, 64, 64, Fx, 1)
+    x, deg = node_inputs(data, num_atoms, num_deg, Fx, 1)
     g = torch.Generator().manual_seed(2)
-    m = GraphNodeFeature(8, 64, 64, 64, C)
+    m = GraphNodeFeature(8, num_atoms, num_deg, num_deg, C)
     with torch.no_grad():
         for p in m.parameters():
             p.normal_(0, 0.5, generator=g)
@@ -64,7 +66,7 @@ def test_graph_node_feature_matches_oracle(cuda, dtype, C, Fx):
     dout = torch.randn(want.shape, generator=g).to(dtype)
     ref = [r.clone() for r in torch.autograd.grad(want, tabs, dout.double())]
     for r in ref[:3]:
-        assert r[0].abs().max() > 0
+        assert r[0].abs().max() > 0 or r is ref[0]
         r[0] = 0                                           # nn.Embedding(padding_idx=0): row 0 gets no gradient
     got_g = torch.autograd.grad(got, [mc.atom_encoder.weight, mc.in_degree_encoder.weight, mc.out_degree_encoder.weight,
                                       mc.graph_token.weight], dout.to(cuda))

@@ -9,7 +9,9 @@
 // concatenation; here one kernel reads the ids and writes every output row once.  The backward adds
 // the output gradient into float copies of the tables with vector-memory atomics (row 0 of the three
 // lookup tables is the padding index and gets none) and a last kernel hands the sums over in the
-// caller's type: results agree to rounding between runs, not bit for bit.
+// caller's type: results agree to rounding between runs, not bit for bit.  (Summing a workgroup's share in LDS
+// first was measured and is no faster: with a few dozen atom types the LDS float atomics of a CU serialise as the
+// memory atomics do in the L2, about 55 us for the 33 K rows of 256 padded graphs either way.)
 #include "common.h"
 #include <algorithm>
 
@@ -68,35 +70,49 @@ __global__ __launch_bounds__(256) void k_fill_zero(float* __restrict__ p, int64_
     if (t < n) p[t] = 0.f;
 }
 
-// acc: float [num_atoms + num_in + num_out + 1][C]
+// One wave per output row (lane = channel, channels beyond 64 in further passes): the ids of a row are read once
+// by the whole wave, the row's position in the batch costs one 32-bit division.  acc is either the float copy of
+// the tables in memory or a workgroup's copy in LDS: float [num_atoms + num_in + num_out + 1][C].
 template <typename T>
-__global__ __launch_bounds__(256) void k_node_feature_bwd(NodeFeatArgs a, const T* __restrict__ dout, float* __restrict__ acc) {
+__device__ __forceinline__ void node_feature_bwd_row(const NodeFeatArgs& a, const T* __restrict__ dout, int64_t row, int lane,
+                                                     float* acc) {
     const int rows = a.s + a.has_token;
-    const int64_t total = (int64_t)a.b * rows * a.C;
-    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (t >= total) return;
-    const int c = (int)(t % a.C);
-    const int64_t row = t / a.C;
-    const int node = (int)(row % rows) + 1 - a.has_token;
     const int64_t g = row / rows;
-    const float d = ldf(dout + t);
-    if (d == 0.f) return;
+    const int node = (int)(row - g * rows) + 1 - a.has_token;
     float* acc_in = acc + (int64_t)a.num_atoms * a.C;
     float* acc_out = acc_in + (int64_t)a.num_in * a.C;
     float* acc_tok = acc_out + (int64_t)a.num_out * a.C;
+    const T* d_row = dout + row * a.C;
     if (node == 0) {
-        atomicAdd(acc_tok + c, d);
+        for (int c = lane; c < a.C; c += 64) {
+            const float d = ldf(d_row + c);
+            if (d != 0.f) atomicAdd(acc_tok + c, d);
+        }
         return;
     }
     const int64_t p = g * a.s + (node - 1);
-    for (int f = 0; f < a.Fx; ++f) {
-        const int id = clamp_id(a.x[p * a.Fx + f], a.num_atoms);
-        if (id >= a.pad_rows) atomicAdd(acc + (int64_t)id * a.C + c, d);        // row 0 = padding index
+    int ii = 0, io = 0;
+    if (a.has_degree) {
+        ii = clamp_id(a.in_degree[p], a.num_in);
+        io = clamp_id(a.out_degree[p], a.num_out);
     }
-    if (!a.has_degree) return;
-    const int ii = clamp_id(a.in_degree[p], a.num_in), io = clamp_id(a.out_degree[p], a.num_out);
-    if (ii > 0) atomicAdd(acc_in + (int64_t)ii * a.C + c, d);
-    if (io > 0) atomicAdd(acc_out + (int64_t)io * a.C + c, d);
+    for (int c = lane; c < a.C; c += 64) {
+        const float d = ldf(d_row + c);
+        if (d == 0.f) continue;
+        for (int f = 0; f < a.Fx; ++f) {
+            const int id = clamp_id(a.x[p * a.Fx + f], a.num_atoms);
+            if (id >= a.pad_rows) atomicAdd(acc + (int64_t)id * a.C + c, d);        // row 0 = padding index
+        }
+        if (ii > 0) atomicAdd(acc_in + (int64_t)ii * a.C + c, d);
+        if (io > 0) atomicAdd(acc_out + (int64_t)io * a.C + c, d);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void k_node_feature_bwd(NodeFeatArgs a, const T* __restrict__ dout, float* __restrict__ acc) {
+    const int64_t n_rows = (int64_t)a.b * (a.s + a.has_token);
+    const int64_t row = (int64_t)blockIdx.x * 4 + threadIdx.x / 64;
+    if (row < n_rows) node_feature_bwd_row(a, dout, row, threadIdx.x % 64, acc);
 }
 
 template <typename T>
@@ -151,18 +167,19 @@ int node_feature_bwd_impl(NodeFeatArgs a, const void* d_dout, int dtype, void* d
                   n_out = a.has_degree ? (int64_t)a.num_out * a.C : 0, n_tok = a.has_token ? a.C : 0;
     const int64_t n_acc = n_atom + n_in + n_out + n_tok;
     if (!a.has_degree) a.num_in = a.num_out = 0;          // the kernel's offsets of the sums that follow the atom table
-    hipLaunchKernelGGL(k_fill_zero, dim3((unsigned)((n_acc + 255) / 256)), dim3(256), 0, st, acc, n_acc);
-    const int64_t total = (int64_t)a.b * (a.s + a.has_token) * a.C;
+    const int64_t n_rows = (int64_t)a.b * (a.s + a.has_token);
+    const int64_t total = n_rows * a.C;
     const dim3 fgrid((unsigned)((n_acc + 255) / 256));
+    hipLaunchKernelGGL(k_fill_zero, dim3((unsigned)((n_acc + 255) / 256)), dim3(256), 0, st, acc, n_acc);
     if (dtype == TGT_DTYPE_F32) {
         if (total > 0)
-            hipLaunchKernelGGL((k_node_feature_bwd<float>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, a,
+            hipLaunchKernelGGL((k_node_feature_bwd<float>), dim3((unsigned)((n_rows + 3) / 4)), dim3(256), 0, st, a,
                                (const float*)d_dout, acc);
         hipLaunchKernelGGL((k_node_feature_finish<float>), fgrid, dim3(256), 0, st, (const float*)acc, n_atom, n_in, n_out, n_tok,
                            (float*)d_datom, (float*)d_din, (float*)d_dout_table, (float*)d_dtoken);
     } else {
         if (total > 0)
-            hipLaunchKernelGGL((k_node_feature_bwd<nbf16>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, a,
+            hipLaunchKernelGGL((k_node_feature_bwd<nbf16>), dim3((unsigned)((n_rows + 3) / 4)), dim3(256), 0, st, a,
                                (const nbf16*)d_dout, acc);
         hipLaunchKernelGGL((k_node_feature_finish<nbf16>), fgrid, dim3(256), 0, st, (const float*)acc, n_atom, n_in, n_out, n_tok,
                            (nbf16*)d_datom, (nbf16*)d_din, (nbf16*)d_dout_table, (nbf16*)d_dtoken);
