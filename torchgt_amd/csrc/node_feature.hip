@@ -71,8 +71,8 @@ __global__ __launch_bounds__(256) void k_fill_zero(float* __restrict__ p, int64_
 }
 
 // One wave per output row (lane = channel, channels beyond 64 in further passes): the ids of a row are read once
-// by the whole wave, the row's position in the batch costs one 32-bit division.  acc is either the float copy of
-// the tables in memory or a workgroup's copy in LDS: float [num_atoms + num_in + num_out + 1][C].
+// by the whole wave, the row's position in the batch costs one division.  acc is the float copy of the tables in
+// memory: float [num_atoms + num_in + num_out + 1][C].
 template <typename T>
 __device__ __forceinline__ void node_feature_bwd_row(const NodeFeatArgs& a, const T* __restrict__ dout, int64_t row, int lane,
                                                      float* acc) {
