@@ -383,7 +383,7 @@ __global__ __launch_bounds__(1024) void k_floyd_warshall(const uint8_t* __restri
                                                          int n_max, int32_t* __restrict__ dist, int32_t* __restrict__ path) {
     extern __shared__ uint16_t lds[];
     const int g = blockIdx.x;
-    const int n = n_nodes ? n_nodes[g] : n_max;
+    const int n = n_nodes ? min(max(n_nodes[g], 0), n_max) : n_max;      // a count outside [0, n_max] is clamped
     uint16_t* M = lds;                                   // [n][n]
     int16_t* P = reinterpret_cast<int16_t*>(lds + n * n);
     const uint8_t* A = adj + (int64_t)g * n_max * n_max;

@@ -490,7 +490,7 @@ __global__ __launch_bounds__(128) void k_gen_edge_input(const int32_t* __restric
     const int64_t plane = (int64_t)n_max * n_max;
     const int64_t g = t / plane;
     const int ij = (int)(t - g * plane), i = ij / n_max, j = ij - i * n_max;
-    const int n = n_nodes ? n_nodes[g] : n_max;
+    const int n = n_nodes ? min(max(n_nodes[g], 0), n_max) : n_max;      // a count outside [0, n_max] is clamped
     const int32_t* P = path + g * plane;
     const FeatT* Fg = feat + g * plane * F;
     int64_t* o = out + t * max_dist * F;
