@@ -151,7 +151,9 @@ __global__ __launch_bounds__(256) void k_multi_hop_fwd(HopArgs a, const T* __res
         float v[HT];
 #pragma unroll
         for (int h = 0; h < HT; ++h) v[h] = base;
-        if (inner) {
+        // a masked position (-inf from the collator: padded key columns) stays -inf whatever the finite table
+        // entries add: its lanes sit the hop loop out, and a wave of such lanes skips it altogether
+        if (inner && base != -INFINITY) {
             const int64_t pos = (g * a.s + (i - 1)) * a.s + (j - 1);
             const int sp = clamp_id(a.spatial_pos[pos], a.num_spatial);
             float y[HT];
@@ -198,7 +200,7 @@ __global__ __launch_bounds__(256) void k_multi_hop_fwd(HopArgs a, const T* __res
 #pragma unroll
             for (int h = 0; h < HT; ++h)
                 if (h < a.H) v[h] += (TAB_LDS ? sp_lds[sp * HT + h] : ldf(sp_tab + sp * a.H + h)) + y[h] / hops;   // (:110-111, :145-152)
-        } else {
+        } else if (!inner) {
 #pragma unroll
             for (int h = 0; h < HT; ++h)
                 if (h < a.H) v[h] += ldf(vd + h);                                      // (:115-117)
@@ -208,6 +210,14 @@ __global__ __launch_bounds__(256) void k_multi_hop_fwd(HopArgs a, const T* __res
         for (int h = 0; h < HT; ++h)
             if (h < a.H) stf(o + h * plane, v[h]);
     }
+}
+
+// Orders the LDS writes of a wave's lanes before the LDS reads of the same wave that follow (and the other way
+// round): the hardware runs a wave's LDS instructions in order, this keeps the compiler from moving them.
+__device__ __forceinline__ void wave_sync_lds() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
 // Layout of one workgroup's sums (floats): spatial table, edge table, virtual distance, hop matrices.
@@ -314,6 +324,12 @@ __global__ __launch_bounds__(256) void k_multi_hop_bwd(HopArgs a, const T* __res
 #pragma unroll
                 for (int h = 0; h < HT; ++h) dy[h] = inner ? d[h] * inv_hops : 0.f;
             }
+            // positions without gradient (masked entries, the rows and columns of padding nodes: exact zeros from the
+            // attention's backward) add nothing to any sum: their lanes sit the hop work out, a wave of them skips it
+            bool nz = false;
+#pragma unroll
+            for (int h = 0; h < HT; ++h) nz = nz || dy[h] != 0.f;
+            const bool wave_nz = __any(nz);
 #pragma unroll
             for (int h = 0; h < HT; ++h) st_dy[h * kStage + threadIdx.x] = dy[h];
 #pragma unroll
@@ -323,7 +339,7 @@ __global__ __launch_bounds__(256) void k_multi_hop_bwd(HopArgs a, const T* __res
                     float m[HT];
 #pragma unroll
                     for (int h = 0; h < HT; ++h) m[h] = 0.f;
-                    if (inner) {
+                    if (nz) {
                         if (TAB_LDS) hop_embedding<float, HT>(a, e_lds, HT, pos, dd, m);
                         else hop_embedding<T, HT>(a, e_tab, H, pos, dd, m);
                         // gradient of the averaged embedding, handed to the F edge-table rows it was averaged from
@@ -358,11 +374,12 @@ __global__ __launch_bounds__(256) void k_multi_hop_bwd(HopArgs a, const T* __res
                     for (int h = 0; h < HT; ++h) st_m[(u * HT + h) * kStage + threadIdx.x] = m[h];
                 }
             }
-            __syncthreads();
+            wave_sync_lds();                 // a wave reads back only what its own lanes staged: no workgroup barrier
             // lane owns entries (h0, h) = divmod(lane + 64 e, HT) of the hop matrices; its wave's 64 positions
             const int nu = min(DC, a.D - dc);
 #pragma unroll
             for (int e = 0; e < EPL; ++e) {
+                if (!wave_nz) break;                                         // uniform over the wave: its 64 positions add nothing
                 const int idx = lane + 64 * e;
                 const float4* pm = reinterpret_cast<const float4*>(st_m + (idx / HT) * kStage + wave * 64);
                 const float4* pd = reinterpret_cast<const float4*>(st_dy + (idx % HT) * kStage + wave * 64);
@@ -383,7 +400,7 @@ __global__ __launch_bounds__(256) void k_multi_hop_bwd(HopArgs a, const T* __res
                     }
                 }
             }
-            __syncthreads();
+            wave_sync_lds();                 // the reads are done before the next pass stages over them
         }
 #pragma unroll
         for (int u = 0; u < DC; ++u) {
