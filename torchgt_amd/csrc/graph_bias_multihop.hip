@@ -332,6 +332,11 @@ __global__ __launch_bounds__(256) void k_multi_hop_bwd(HopArgs a, const T* __res
             const bool wave_nz = __any(nz);
 #pragma unroll
             for (int h = 0; h < HT; ++h) st_dy[h * kStage + threadIdx.x] = dy[h];
+            // the first feature's id of every hop of this pass, fetched whether or not the position carries a gradient:
+            // behind the branch these loads would wait for the gradient's own loads to return
+            int64_t id0[DC];
+#pragma unroll
+            for (int u = 0; u < DC; ++u) id0[u] = dc + u < a.D ? a.edge_input[(pos * a.D0 + dc + u) * a.F] : 0;
 #pragma unroll
             for (int u = 0; u < DC; ++u) {
                 const int dd = dc + u;
@@ -340,8 +345,6 @@ __global__ __launch_bounds__(256) void k_multi_hop_bwd(HopArgs a, const T* __res
 #pragma unroll
                     for (int h = 0; h < HT; ++h) m[h] = 0.f;
                     if (nz) {
-                        if (TAB_LDS) hop_embedding<float, HT>(a, e_lds, HT, pos, dd, m);
-                        else hop_embedding<T, HT>(a, e_tab, H, pos, dd, m);
                         // gradient of the averaged embedding, handed to the F edge-table rows it was averaged from
                         const float* w = w_lds + dd * HT * HT;
                         float dm[HT];
@@ -354,7 +357,12 @@ __global__ __launch_bounds__(256) void k_multi_hop_bwd(HopArgs a, const T* __res
                         }
                         const int64_t* ids = a.edge_input + (pos * a.D0 + dd) * a.F;
                         for (int f = 0; f < a.F; ++f) {
-                            const int id = clamp_id(ids[f], a.num_edges);
+                            const int id = clamp_id(f == 0 ? id0[u] : ids[f], a.num_edges);
+#pragma unroll
+                            for (int h = 0; h < HT; ++h) {                   // the averaged embedding itself (:129)
+                                if (TAB_LDS) m[h] += e_lds[id * HT + h];
+                                else if (h < H) m[h] += ldf(e_tab + id * H + h);
+                            }
                             if (HOT) {
 #pragma unroll
                                 for (int r = 0; r < NHE; ++r) {
@@ -369,6 +377,8 @@ __global__ __launch_bounds__(256) void k_multi_hop_bwd(HopArgs a, const T* __res
                                     if (h0 < H && dm[h0] != 0.f) atomicAdd(&acc_e[id * H + h0], dm[h0]);
                             }
                         }
+#pragma unroll
+                        for (int h = 0; h < HT; ++h) m[h] *= inv_f;
                     }
 #pragma unroll
                     for (int h = 0; h < HT; ++h) st_m[(u * HT + h) * kStage + threadIdx.x] = m[h];
