@@ -217,6 +217,25 @@ def test_graph_attn_bias_multi_hop_without_hops_is_the_spatial_and_virtual_part(
     assert not g[1].any() and not g[2].any()
 
 
+def test_graph_attn_bias_multi_hop_on_graphs_without_nodes(cuda):
+    # s = 0: only the virtual node; every entry is 2 * attn_bias + the virtual distance, the id tensors are empty
+    H = 8
+    m = GraphAttnBias(H, 512, 5, 22, 5, 64, "multi_hop", 5).to(cuda)
+    with torch.no_grad():
+        m.graph_token_virtual_distance.weight.normal_(0, 0.5)
+    ab = torch.randn(3, 1, 1, device=cuda)
+    batch = types.SimpleNamespace(attn_bias=ab, spatial_pos=torch.zeros(3, 0, 0, dtype=torch.long, device=cuda),
+                                  edge_input=torch.zeros(3, 0, 0, 4, 1, dtype=torch.long, device=cuda))
+    got = m(batch)
+    want = 2 * ab.unsqueeze(1) + m.graph_token_virtual_distance.weight.view(1, H, 1, 1)
+    assert got.shape == (3, H, 1, 1) and err(got, want) <= 1e-6
+    dout = torch.randn(3, H, 1, 1, device=cuda)
+    g = torch.autograd.grad(got, [m.spatial_pos_encoder.weight, m.edge_encoder.weight, m.edge_dis_encoder.weight,
+                                  m.graph_token_virtual_distance.weight], dout)
+    assert not g[0].any() and not g[1].any() and not g[2].any()
+    assert err(g[3], dout.sum(0).view(1, H)) <= 1e-6
+
+
 def test_graph_attn_bias_multi_hop_rejects_more_hops_than_matrices(cuda):
     m = GraphAttnBias(8, 512, 5, 22, 2, 64, "multi_hop", 0).to(cuda)       # two hop matrices, three hops of input
     batch = types.SimpleNamespace(attn_bias=torch.zeros(1, 4, 4, device=cuda), spatial_pos=torch.ones(1, 3, 3, dtype=torch.long, device=cuda),

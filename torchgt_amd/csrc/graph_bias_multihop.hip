@@ -336,7 +336,7 @@ __global__ __launch_bounds__(256) void k_multi_hop_bwd(HopArgs a, const T* __res
             // behind the branch these loads would wait for the gradient's own loads to return
             int64_t id0[DC];
 #pragma unroll
-            for (int u = 0; u < DC; ++u) id0[u] = dc + u < a.D ? a.edge_input[(pos * a.D0 + dc + u) * a.F] : 0;
+            for (int u = 0; u < DC; ++u) id0[u] = dc + u < a.D && a.s > 0 ? a.edge_input[(pos * a.D0 + dc + u) * a.F] : 0;   // s = 0: no ids at all
 #pragma unroll
             for (int u = 0; u < DC; ++u) {
                 const int dd = dc + u;
