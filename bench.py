@@ -8,7 +8,7 @@ the benchmark configuration "configs[1]": N = 64 001, E ~ 530 K, H = 8, d = 8, p
 reported separately).  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype f32|bf16] [--no-cpu-baseline]
-                    [--workload config1|config2|config2-mha|config2-model|config3|config4|config4-bias|
+                    [--workload config1|config2|config2-mha|config2-model|config2-gt-model|config3|config4|config4-bias|
                                config4-bias-multihop|config4-model|config5|config5-blockized]
 
 config3 / config5: larger sparse workloads (bf16); config4: dense biased attention of a graph-level
@@ -16,7 +16,7 @@ batch; config4-bias: the bias builder in front of it (GraphAttnBias forward + ta
 the same with the path-encoding ('multi_hop') edge term; config4-model: a training step of the graph-level Graphormer
 on that batch; config5-blockized: the block path on the reordered config5 graph; config2-mha: one whole
 MultiHeadAttention layer (projections + sparse attention) on the config2 graph; config2-model: a training
-step of the 4-layer Graphormer-Slim on that graph.
+step of the 4-layer Graphormer-Slim on that graph; config2-gt-model: the same for the node-level GT.
 """
 import argparse
 import json
@@ -521,16 +521,20 @@ def bench_model(args):
     40 classes; 111 913 parameters) on the whole 64 K-node graph as one sequence: forward, nll loss, backward,
     AdamW step (torch's optimizer, as in the reference's training loop)."""
     import torch
-    from torchgt_amd import Graphormer, _lib
+    from torchgt_amd import GT, Graphormer as NodeGraphormer, _lib
     dev = torch.device("cuda:0")
     e, n, label, desc = build_workload("config2")
     tdt = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    gt = args.workload == "config2-gt-model"
+    # the GT of models/gt_dist_node_level.py has no global token: node 0 of the graph is an ordinary node there
+    Graphormer = (lambda *a: GT(*a[:-1], 0)) if gt else NodeGraphormer
+    n_rows = n if gt else n - 1
     torch.manual_seed(42)
     m = Graphormer(4, 8, 128, 64, 40, 1, 0.0, 0.0, 0.0, 64, 1).to(dev, tdt)
     opt = torch.optim.AdamW(m.parameters(), lr=1e-3, weight_decay=0.01)
     ei = torch.from_numpy(e).to(dev)
-    x = torch.randn(n - 1, 128, device=dev).to(tdt)
-    y = torch.randint(0, 40, (n - 1,), device=dev)
+    x = torch.randn(n_rows, 128, device=dev).to(tdt)
+    y = torch.randint(0, 40, (n_rows,), device=dev)
 
     def step():
         opt.zero_grad(set_to_none=True)
@@ -597,11 +601,12 @@ def bench_model(args):
     groups = {"attention": ("attn_fwd", "bwd_node_side", "attn_bwd"), "projections and ffn linears": ("linear_fwd", "linear_dx", "linear_dw"),
               "layer norm + residual": ("layer_norm_fwd", "layer_norm_bwd"), "gelu": ("gelu",)}
     result = {
-        "metric": "training step of the 4-layer Graphormer-Slim on one 64 K-node sequence",
+        "metric": "training step of the 4-layer " + ("GT" if gt else "Graphormer-Slim") + " on one 64 K-node sequence",
         "value": 1e3 / ms, "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic",
-        "config": {"workload": "configs[1] graph as one sequence, Graphormer-Slim 4 x (hidden 64, ffn 64, 8 heads), "
+        "config": {"workload": "configs[1] graph as one sequence, " + ("GT 4 x (hidden 64, ffn 128, 8 heads, MLP readout), " if gt else
+                               "Graphormer-Slim 4 x (hidden 64, ffn 64, 8 heads), ") +
                                "128-d features, 40 classes, no bias, dropout 0", "N": n, "E": int(e.shape[1]),
                    "parameters": sum(p.numel() for p in m.parameters()),
                    "step": "forward + nll_loss + backward + torch AdamW", "parallelism": "1 GPU"},
@@ -774,7 +779,7 @@ def main():
         return bench_block(args)
     if args.workload == "config2-mha":
         return bench_mha(args)
-    if args.workload == "config2-model":
+    if args.workload in ("config2-model", "config2-gt-model"):
         return bench_model(args)
     if args.workload in ("config3", "config5"):
         args.no_cpu_baseline = True      # the CPU restatement needs minutes per step at this size
