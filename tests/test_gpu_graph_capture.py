@@ -111,3 +111,105 @@ def test_model_training_step_replays_from_a_graph(cuda):
         assert torch.isfinite(torch.randn(1000, device=cuda).sum()).item()        # eager work between replays
     for a, b in zip(w_eager, m.parameters()):
         assert torch.equal(a, b.detach())
+
+
+def test_graph_level_training_step_replays_from_a_graph(cuda):
+    """A training step of the graph-level Graphormer mirror (node features, bias builder, dense attention, encoder
+    kernels, L1 loss, backward, SGD) captured once and replayed on other batches' targets and features, with eager
+    work between the replays.  The table gradients are summed with atomics, whose order changes from run to run: the
+    losses and the final weights agree with the eager sequence within the spread that two eager runs show (times 20; at least
+    1e-3 of the loss and of the largest weight: the dense attention rounds its operands to bf16, so a last-bit difference
+    in a sum can move a rounded operand by 2^-9 of its value) with the eager sequence, not bit for
+    bit; SGD keeps that noise proportional (an Adam step would turn a rounding-sized gradient into a full-sized update)."""
+    import types
+    import numpy as np
+    from torchgt_amd.graph_level import Graphormer
+    data = workloads.erdos_renyi_batch(batch=8, seed=13)
+    sizes, s = data["n_nodes"], data["spatial_pos"].shape[1]
+    rng = np.random.default_rng(1)
+    deg = np.zeros((8, s), np.int64)
+    xs = []
+    for g in range(8):
+        n = int(sizes[g])
+        deg[g, :n] = np.minimum((data["spatial_pos"][g][:n, :n] == 2).sum(1) + 1, 63)
+    for _ in range(4):
+        x = np.zeros((8, s, 1), np.int64)
+        for g in range(8):
+            x[g, :int(sizes[g]), 0] = rng.integers(1, 64, size=int(sizes[g]))
+        xs.append(torch.from_numpy(x).to(cuda))
+    ys = [torch.randn(8, generator=torch.Generator().manual_seed(i)).to(cuda) for i in range(4)]
+    batch = types.SimpleNamespace(
+        x=xs[0].clone(), in_degree=torch.from_numpy(deg).to(cuda), out_degree=torch.from_numpy(deg).to(cuda),
+        attn_bias=torch.from_numpy(data["attn_bias"]).float().to(cuda), spatial_pos=torch.from_numpy(data["spatial_pos"]).long().to(cuda),
+        attn_edge_type=torch.from_numpy(data["edge_type"]).long().unsqueeze(-1).contiguous().to(cuda), edge_input=None)
+    static_y = ys[0].clone()
+
+    def make():
+        torch.manual_seed(3)
+        m = Graphormer(2, 8, 64, 0.0, 0.0, 64, "ZINC", "single_hop", 5, 0.0, 1).to(cuda)
+        with torch.no_grad():
+            for p in m.parameters():
+                if p.dim() == 2:
+                    p.mul_(5.0)                       # away from the flat attention of the reference's init
+        return m, torch.optim.SGD(m.parameters(), lr=0.05)
+
+    def step(m, opt):
+        opt.zero_grad(set_to_none=True)
+        loss = torch.nn.functional.l1_loss(m(batch).view(-1), static_y)
+        loss.backward()
+        opt.step()
+        return loss
+
+    def load(i):
+        batch.x.copy_(xs[i])
+        static_y.copy_(ys[i])
+
+    m, opt = make()
+    load(0)
+    for _ in range(2):
+        step(m, opt)
+    eager = []
+    for i in range(1, 4):
+        load(i)
+        eager.append(step(m, opt).item())
+    w_eager = [p.detach().clone() for p in m.parameters()]
+
+    # the run-to-run spread of the eager sequence itself: the yardstick for the replays
+    m, opt = make()
+    load(0)
+    for _ in range(2):
+        step(m, opt)
+    eager2 = []
+    for i in range(1, 4):
+        load(i)
+        eager2.append(step(m, opt).item())
+    wmax = max(p.abs().max().item() for p in w_eager)
+    spread_w = max((a - b.detach()).abs().max().item() for a, b in zip(w_eager, m.parameters()))
+    spread_l = max(abs(a - b) for a, b in zip(eager, eager2))
+    print(f"eager run-to-run spread: loss {spread_l:.3e}, weights {spread_w:.3e} (largest weight {wmax:.3f})", flush=True)
+    tol_l, tol_w = max(1e-3, 20 * spread_l), max(1e-3 * wmax, 20 * spread_w)
+
+    m, opt = make()
+    load(0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step(m, opt)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    gr = torch.cuda.CUDAGraph()
+    opt.zero_grad(set_to_none=True)
+    with torch.cuda.graph(gr):
+        static_loss = torch.nn.functional.l1_loss(m(batch).view(-1), static_y)
+        static_loss.backward()
+        opt.step()
+    for i in range(1, 4):
+        load(i)
+        gr.replay()
+        torch.cuda.synchronize()
+        assert abs(static_loss.item() - eager[i - 1]) <= tol_l, (i, static_loss.item(), eager[i - 1], tol_l)
+        assert torch.isfinite(torch.randn(1000, device=cuda).sum()).item()        # eager work between replays
+    got_w = max((a - b.detach()).abs().max().item() for a, b in zip(w_eager, m.parameters()))
+    print(f"graph replays against eager: weights {got_w:.3e} (bar {tol_w:.3e})", flush=True)
+    assert got_w <= tol_w
