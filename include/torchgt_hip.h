@@ -329,7 +329,8 @@ int tgt_graph_attn_bias_fwd(const void* d_attn_bias, const int64_t* d_spatial_po
  * tables is the padding index and gets zero).  Sums are formed in LDS per workgroup
  * with floating-point atomics and the workgroup partials are added in a fixed order:
  * results agree to rounding between runs, not bit for bit.
- * (num_spatial + num_edges + 1) * H must not exceed 15 360. */
+ * (num_spatial + num_edges + 1) * H must not exceed 32 768 (128 KB of LDS: the molecule tables
+ * of the reference, 512 spatial ids and 1 537 edge types, fit with up to 15 heads). */
 int64_t tgt_graph_attn_bias_bwd_workspace_bytes(int num_spatial, int num_edges, int H);
 int tgt_graph_attn_bias_bwd(const void* d_dout, const int64_t* d_spatial_pos, const int64_t* d_edge_type, int F,
                             int num_spatial, int num_edges, int b, int s, int H, int dtype, void* d_dspatial_table,

@@ -186,6 +186,51 @@ def test_graph_attn_bias_multi_hop_matches_oracle(cuda, dtype, H, F, D0, mhd):
     assert not got_g[2].reshape(n_dis, H, H)[D:].any() and got_g[2].reshape(n_dis, H, H)[:D].any()
 
 
+@pytest.mark.parametrize("edge_type", ["single_hop", "multi_hop"])
+def test_graph_attn_bias_with_molecule_sized_tables(cuda, edge_type):
+    """The tables of the reference's molecule datasets (models/graphormer_graph_level.py:332-338: 512 spatial ids,
+    1 537 edge types, 128 hop matrices) with ids spread over them: the tables no longer fit next to the hop matrices
+    in LDS (the kernels read them from memory) and the gradient sums take 66 KB of LDS per workgroup."""
+    print(f"molecule-sized tables: {edge_type}", flush=True)
+    H, F, D0, mhd = 8, 1, 4, 4
+    data = workloads.erdos_renyi_batch(batch=6, seed=17)
+    g = torch.Generator().manual_seed(3)
+    m = GraphAttnBias(H, 512 * 9 + 1, 512 * 3 + 1, 512, 128, 64, edge_type, mhd)
+    with torch.no_grad():
+        m.spatial_pos_encoder.weight.normal_(0, 0.5, generator=g); m.spatial_pos_encoder.weight[0] = 0
+        m.edge_encoder.weight.normal_(0, 0.5, generator=g); m.edge_encoder.weight[0] = 0
+        m.graph_token_virtual_distance.weight.normal_(0, 0.5, generator=g)
+        if edge_type == "multi_hop":
+            m.edge_dis_encoder.weight.normal_(0, 0.5, generator=g)
+    attn_bias = torch.from_numpy(data["attn_bias"])
+    spatial_pos = torch.from_numpy(data["spatial_pos"]).long() * 20          # 0 stays the padding id, up to 420
+    et = torch.from_numpy(data["edge_type"]).long().unsqueeze(-1) * 300       # up to 1 200
+    edge_input = torch.from_numpy(_edge_input_of_batch(data, F, D0))
+    edge_input = torch.where(edge_input > 0, (edge_input - 1) * 300 + 1, edge_input)
+    names = ["spatial_pos_encoder", "edge_encoder"] + (["edge_dis_encoder"] if edge_type == "multi_hop" else []) \
+        + ["graph_token_virtual_distance"]
+    params = [getattr(m, n).weight.detach().double().requires_grad_(True) for n in names]
+    if edge_type == "multi_hop":
+        # the oracle's path length comes from spatial_pos itself; keep the ids, scale only the table rows they select
+        want = oda.graph_attn_bias_multi_hop(attn_bias.double(), spatial_pos, edge_input, params[0], params[1], params[2], params[3], mhd)
+    else:
+        want = oda.graph_attn_bias(attn_bias.double(), spatial_pos, et, params[0], params[1], params[2])
+    mc = m.to(cuda)
+    got = mc(types.SimpleNamespace(attn_bias=attn_bias.to(cuda), spatial_pos=spatial_pos.to(cuda), attn_edge_type=et.to(cuda),
+                                   edge_input=edge_input.to(cuda)))
+    assert err(got, want) <= 1e-5, err(got, want)
+    dout = torch.randn(want.shape, generator=g)
+    dout[~torch.isfinite(want)] = 0
+    finite = torch.where(torch.isfinite(want), want, torch.zeros_like(want))
+    ref = [r.clone() for r in torch.autograd.grad((finite * dout.double()).sum(), params)]
+    ref[0][0] = 0
+    ref[1][0] = 0
+    got_g = torch.autograd.grad(got, [getattr(mc, n).weight for n in names], dout.to(cuda))
+    for n, a, r in zip(names, got_g, ref):
+        assert err(a, r) <= 1e-5, f"d{n} err {err(a, r)}"
+    assert got_g[0][420].any() and got_g[1][300 if edge_type == "single_hop" else 301].any()
+
+
 def test_graph_attn_bias_multi_hop_without_hops_is_the_spatial_and_virtual_part(cuda):
     # an edge_input that holds no hops (the reference's reshape raises on it): the edge term vanishes, forward and
     # gradients still come out; the single-hop oracle with an all-zero edge table is the same sum

@@ -474,9 +474,9 @@ int tgt_graph_attn_bias_bwd(const void* d_dout, const int64_t* d_spatial_pos, co
         return TGT_ERR_INVALID_ARG;
     }
     const int n_acc = (num_spatial + num_edges + 1) * H;
-    if ((size_t)n_acc * sizeof(float) > 60 * 1024) {
+    if ((size_t)n_acc * sizeof(float) > 128 * 1024) {
         set_error("tgt_graph_attn_bias_bwd: (num_spatial + num_edges + 1) * H = %d table entries exceed the %d kept on chip",
-                  n_acc, 60 * 1024 / 4);
+                  n_acc, 128 * 1024 / 4);
         return TGT_ERR_UNSUPPORTED;
     }
     if (!d_workspace || workspace_bytes < tgt_graph_attn_bias_bwd_workspace_bytes(num_spatial, num_edges, H)) {
@@ -497,7 +497,7 @@ int tgt_graph_attn_bias_bwd(const void* d_dout, const int64_t* d_spatial_pos, co
     auto launch = [&](auto kernel, auto reduce, auto* dout, auto* dsp, auto* de, auto* dv) -> int {
         if (lds > 48 * 1024)
             TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                              60 * 1024));
+                                              128 * 1024));
         hipLaunchKernelGGL(kernel, dim3(workers), dim3(256), lds, st, a, dout, partial, copies);
         hipLaunchKernelGGL(reduce, dim3(rgrid), dim3(256), 0, st, (const float*)partial, workers, num_spatial * H, num_edges * H, H,
                            dsp, de, dv);
