@@ -173,3 +173,32 @@ def test_graph_level_graphormer_matches_oracle(cuda, edge_type, dtype):
     bad = {k: v for k, v in errs.items() if v > tol}
     assert not bad, bad
     assert checked >= len(names) - n_layers - 2
+
+
+def test_graph_level_graphormer_with_molecule_sized_tables(cuda):
+    """The table sizes of the reference's molecule datasets (4 609 atom types, 1 537 edge types, 512 spatial ids and
+    degrees): two layers (with one, only the virtual node's query row reaches the loss and the inner bias tables get
+    no gradient), forward against the oracle, and a backward that reaches every table."""
+    data = workloads.erdos_renyi_batch(batch=6, seed=23)
+    x, deg = node_inputs(data, 4609, 512, 3, 4)
+    torch.manual_seed(8)
+    m = Graphormer(2, 8, 64, 0.0, 0.0, 64, "ogbg-molhiv", "single_hop", 5, 0.0, 2)
+    with torch.no_grad():
+        for k, p in m.named_parameters():
+            if p.dim() == 2:
+                p.normal_(0, 0.3 if "graph_attn_bias" in k else (0.05 if "linear_q" in k or "linear_k" in k else 0.15))
+    pd = {k: v.detach().double() for k, v in m.named_parameters()}
+    batch = {"x": x, "in_degree": deg, "out_degree": deg, "attn_bias": torch.from_numpy(data["attn_bias"]).double(),
+             "spatial_pos": torch.from_numpy(data["spatial_pos"]).long() * 20,
+             "attn_edge_type": torch.from_numpy(data["edge_type"]).long().unsqueeze(-1) * 300}
+    want = ogl.graphormer_forward(pd, batch, 2, 8, "single_hop", 5)
+    mc = m.to(cuda)
+    cb = types.SimpleNamespace(**{k: v.to(cuda) for k, v in batch.items()}, edge_input=None)
+    cb.attn_bias = cb.attn_bias.float()
+    got = mc(cb)
+    assert got.shape == (6, 2) and err(got, want) <= 3 * TOL[torch.bfloat16], err(got, want)
+    got.square().sum().backward()
+    for k, p in mc.named_parameters():
+        assert p.grad is not None and p.grad.shape == p.shape and torch.isfinite(p.grad).all(), k
+    assert mc.graph_node_feature.atom_encoder.weight.grad[1:].any()
+    assert mc.graph_attn_bias.edge_encoder.weight.grad[300].any() and mc.graph_attn_bias.spatial_pos_encoder.weight.grad[40].any()
