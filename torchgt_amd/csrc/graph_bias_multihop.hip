@@ -101,25 +101,6 @@ __device__ __forceinline__ void load_table(const void* table, int rows, int H, f
     }
 }
 
-// Averaged edge embedding of hop dd at position pos: mean over the F features (:129).  The table is
-// either the LDS copy (float, row stride HT) or the caller's (row stride H).
-template <typename TT, int HT>
-__device__ __forceinline__ void hop_embedding(const HopArgs& a, const TT* __restrict__ e_tab, int stride, int64_t pos, int dd,
-                                              float (&m)[HT]) {
-    const int64_t* ids = a.edge_input + (pos * a.D0 + dd) * a.F;
-#pragma unroll
-    for (int h = 0; h < HT; ++h) m[h] = 0.f;
-    for (int f = 0; f < a.F; ++f) {
-        const int id = clamp_id(ids[f], a.num_edges);
-#pragma unroll
-        for (int h = 0; h < HT; ++h)
-            if (h < stride) m[h] += ldf(e_tab + id * stride + h);
-    }
-    const float inv_f = 1.f / (float)a.F;
-#pragma unroll
-    for (int h = 0; h < HT; ++h) m[h] *= inv_f;
-}
-
 // TAB_LDS: the spatial and edge tables fit LDS next to the hop matrices.
 // WS: eight heads, the hop matrices come through scalar loads from wq instead of LDS.
 template <typename T, int HT, bool TAB_LDS, bool WS>
