@@ -9,9 +9,11 @@
 // concatenation; here one kernel reads the ids and writes every output row once.  The backward adds
 // the output gradient into float copies of the tables with vector-memory atomics (row 0 of the three
 // lookup tables is the padding index and gets none) and a last kernel hands the sums over in the
-// caller's type: results agree to rounding between runs, not bit for bit.  (Summing a workgroup's share in LDS
-// first was measured and is no faster: with a few dozen atom types the LDS float atomics of a CU serialise as the
-// memory atomics do in the L2, about 55 us for the 33 K rows of 256 padded graphs either way.)
+// caller's type: results agree to rounding between runs, not bit for bit.  With a few dozen atom types every
+// table row is shared by hundreds of node rows and atomics on one address serialise (55 us for the 33 K rows of
+// 256 padded graphs; summing a workgroup's share in LDS first costs the same, the LDS float atomics of a CU
+// serialise likewise), so neighbouring workgroups add into different copies of the sums (up to 64, at most 16 MB
+// in all) that the last kernel adds up: 21 us.
 #include "common.h"
 #include <algorithm>
 
@@ -109,23 +111,48 @@ __device__ __forceinline__ void node_feature_bwd_row(const NodeFeatArgs& a, cons
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void k_node_feature_bwd(NodeFeatArgs a, const T* __restrict__ dout, float* __restrict__ acc) {
+__global__ __launch_bounds__(256) void k_node_feature_bwd(NodeFeatArgs a, const T* __restrict__ dout, float* __restrict__ acc,
+                                                          int copies, int64_t n_acc) {
     const int64_t n_rows = (int64_t)a.b * (a.s + a.has_token);
     const int64_t row = (int64_t)blockIdx.x * 4 + threadIdx.x / 64;
-    if (row < n_rows) node_feature_bwd_row(a, dout, row, threadIdx.x % 64, acc);
+    // neighbouring workgroups add into different copies of the sums: rows that many positions share serialise less
+    if (row < n_rows) node_feature_bwd_row(a, dout, row, threadIdx.x % 64, acc + (blockIdx.x % copies) * n_acc);
 }
 
+// Sum of the copies, handed over in the caller's type.  64 entries per workgroup along the lanes; the four waves take
+// every fourth copy each (four loads in flight per lane) and their partial sums are added in wave order.
 template <typename T>
 __global__ __launch_bounds__(256) void k_node_feature_finish(const float* __restrict__ acc, int64_t n_atom, int64_t n_in,
-                                                             int64_t n_out, int64_t n_tok, T* __restrict__ d_atom,
+                                                             int64_t n_out, int64_t n_tok, int copies, T* __restrict__ d_atom,
                                                              T* __restrict__ d_in, T* __restrict__ d_out, T* __restrict__ d_tok) {
-    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (t >= n_atom + n_in + n_out + n_tok) return;
-    const float v = acc[t];
+    __shared__ float part[4][64];
+    const int64_t n_acc = n_atom + n_in + n_out + n_tok;
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const int64_t t = (int64_t)blockIdx.x * 64 + lane;
+    float v = 0.f;
+    if (t < n_acc) {
+        for (int c0 = wave; c0 < copies; c0 += 16) {
+            float x[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) x[u] = c0 + 4 * u < copies ? acc[(int64_t)(c0 + 4 * u) * n_acc + t] : 0.f;
+            v += (x[0] + x[1]) + (x[2] + x[3]);
+        }
+    }
+    part[wave][lane] = v;
+    __syncthreads();
+    if (wave != 0 || t >= n_acc) return;
+    v = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
     if (t < n_atom) stf(d_atom + t, v);
     else if (t < n_atom + n_in) stf(d_in + (t - n_atom), v);
     else if (t < n_atom + n_in + n_out) stf(d_out + (t - n_atom - n_in), v);
     else stf(d_tok + (t - n_atom - n_in - n_out), v);
+}
+
+// Copies of the float sums the backward spreads its atomics over: as many as stay under 16 MB in all, at most 64.
+inline int node_feat_copies(int64_t n_acc) {
+    int copies = 64;
+    while (copies > 1 && n_acc * copies * (int64_t)sizeof(float) > (16 << 20)) copies /= 2;
+    return copies;
 }
 
 int node_feat_check(int b, int s, int Fx, int C, int num_atoms, int num_in, int num_out, int dtype, const char* who) {
@@ -169,19 +196,20 @@ int node_feature_bwd_impl(NodeFeatArgs a, const void* d_dout, int dtype, void* d
     if (!a.has_degree) a.num_in = a.num_out = 0;          // the kernel's offsets of the sums that follow the atom table
     const int64_t n_rows = (int64_t)a.b * (a.s + a.has_token);
     const int64_t total = n_rows * a.C;
-    const dim3 fgrid((unsigned)((n_acc + 255) / 256));
-    hipLaunchKernelGGL(k_fill_zero, dim3((unsigned)((n_acc + 255) / 256)), dim3(256), 0, st, acc, n_acc);
+    const dim3 fgrid((unsigned)((n_acc + 63) / 64));
+    const int copies = node_feat_copies(n_acc);
+    hipLaunchKernelGGL(k_fill_zero, dim3((unsigned)((n_acc * copies + 255) / 256)), dim3(256), 0, st, acc, n_acc * copies);
     if (dtype == TGT_DTYPE_F32) {
         if (total > 0)
             hipLaunchKernelGGL((k_node_feature_bwd<float>), dim3((unsigned)((n_rows + 3) / 4)), dim3(256), 0, st, a,
-                               (const float*)d_dout, acc);
-        hipLaunchKernelGGL((k_node_feature_finish<float>), fgrid, dim3(256), 0, st, (const float*)acc, n_atom, n_in, n_out, n_tok,
+                               (const float*)d_dout, acc, copies, n_acc);
+        hipLaunchKernelGGL((k_node_feature_finish<float>), fgrid, dim3(256), 0, st, (const float*)acc, n_atom, n_in, n_out, n_tok, copies,
                            (float*)d_datom, (float*)d_din, (float*)d_dout_table, (float*)d_dtoken);
     } else {
         if (total > 0)
             hipLaunchKernelGGL((k_node_feature_bwd<nbf16>), dim3((unsigned)((n_rows + 3) / 4)), dim3(256), 0, st, a,
-                               (const nbf16*)d_dout, acc);
-        hipLaunchKernelGGL((k_node_feature_finish<nbf16>), fgrid, dim3(256), 0, st, (const float*)acc, n_atom, n_in, n_out, n_tok,
+                               (const nbf16*)d_dout, acc, copies, n_acc);
+        hipLaunchKernelGGL((k_node_feature_finish<nbf16>), fgrid, dim3(256), 0, st, (const float*)acc, n_atom, n_in, n_out, n_tok, copies,
                            (nbf16*)d_datom, (nbf16*)d_din, (nbf16*)d_dout_table, (nbf16*)d_dtoken);
     }
     TGT_HIP_CHECK(hipGetLastError());
@@ -211,7 +239,8 @@ int tgt_graph_node_feature_fwd(const int64_t* d_x, const int64_t* d_in_degree, c
 
 int64_t tgt_graph_node_feature_bwd_workspace_bytes(int num_atoms, int num_in, int num_out, int C) {
     if (num_atoms < 1 || num_in < 1 || num_out < 1 || C < 1) return 0;
-    return (int64_t)sizeof(float) * ((int64_t)num_atoms + num_in + num_out + 1) * C;
+    const int64_t n_acc = ((int64_t)num_atoms + num_in + num_out + 1) * C;
+    return (int64_t)sizeof(float) * n_acc * tgt::node_feat_copies(n_acc);
 }
 
 int tgt_graph_node_feature_bwd(const void* d_dout, const int64_t* d_x, const int64_t* d_in_degree, const int64_t* d_out_degree,
@@ -251,7 +280,8 @@ int tgt_embedding_sum_fwd(const int64_t* d_x, int Fx, const void* d_table, int n
 
 int64_t tgt_embedding_sum_bwd_workspace_bytes(int num_rows, int C) {
     if (num_rows < 1 || C < 1) return 0;
-    return (int64_t)sizeof(float) * num_rows * C;
+    const int64_t n_acc = (int64_t)num_rows * C;
+    return (int64_t)sizeof(float) * n_acc * tgt::node_feat_copies(n_acc);
 }
 
 int tgt_embedding_sum_bwd(const void* d_dout, const int64_t* d_x, int Fx, int num_rows, int b, int s, int C, int dtype, void* d_dtable,
