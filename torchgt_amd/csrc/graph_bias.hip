@@ -491,7 +491,7 @@ int tgt_graph_attn_bias_bwd(const void* d_dout, const int64_t* d_spatial_pos, co
     KernelTimer timer(KS_GRAPH_BIAS_BWD, st);
     float* partial = (float*)d_workspace;
     int copies = kBiasCopies;
-    while (copies > 1 && (size_t)n_acc * copies * sizeof(float) > 60 * 1024) copies /= 2;
+    while (copies > 1 && (size_t)n_acc * copies * sizeof(float) > 16 * 1024) copies /= 2;      // more workgroups per CU beat more copies
     const size_t lds = (size_t)n_acc * copies * sizeof(float);
     const unsigned rgrid = (unsigned)((n_acc + 3) / 4);
     auto launch = [&](auto kernel, auto reduce, auto* dout, auto* dsp, auto* de, auto* dv) -> int {
