@@ -4,6 +4,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <stdarg.h>
+#include <vector>
 #include "../../include/torchgt_hip.h"
 
 namespace tgt {
@@ -12,8 +13,10 @@ constexpr int kWave = 64;            // CDNA wavefront width
 constexpr int kBlock = 256;          // threads per workgroup of the attention kernels (4 waves)
 constexpr int kWaveRowMax = 256;     // a row of up to this many edges is walked by (part of) one wave
 constexpr int kBlockSeg = 1024;      // longer rows are walked by whole workgroups, in segments of at most this many edges
-constexpr int kSpreadSegs = 8;       // rows with more segments than this are spread over all XCDs
-constexpr int kSpreadSeg = 512;      // segment length of such a row (it is alone on the critical path: more, shorter segments)
+constexpr int kSpreadSegs = 8;       // rows with more segments than this get shorter segments:
+constexpr int kSpreadSeg = 128;      // their length (more workgroups, each next to the rows of its sources)
+constexpr int kWindowRows = 128;     // rows of one schedule window (consecutive node ids walked together on one XCD)
+constexpr int kCombineFan = 32;      // partial slots one combine step adds (= lane groups of a workgroup at 8 lanes per edge)
 constexpr int kNumClass = 5;         // wave item length classes: >32, <=32, <=16, <=8, <=4
 
 void set_error(const char* fmt, ...);
@@ -34,23 +37,57 @@ void set_error(const char* fmt, ...);
 // and this item's partial sums go to slot `part` of the workspace.
 struct Item { int32_t row, start, len, part; };
 
+// What one wave of an attention workgroup does.  Workgroup b reads descriptors 4b .. 4b+3.
+//   kind 0..4: wave items [first, first + count) of that length class (count <= rows per wave of the shape)
+//   kind 5:    workgroup item `first` (all four descriptors of the workgroup are equal)
+//   kind 7:    nothing
+// Bit 3 of the code tells the view in the backward launch (0 by destination, 1 by source).
+struct WaveDesc { int32_t first; uint32_t code; };
+constexpr uint32_t kDescBlock = 5, kDescNone = 7, kDescSrcSide = 8;
+__host__ __device__ constexpr uint32_t desc_code(uint32_t kind, uint32_t src_side, uint32_t count) {
+    return kind | (src_side ? kDescSrcSide : 0u) | (count << 8);
+}
+
+// Edge slots of a lane group: natural slot count of the length classes (>32, <=32, <=16, <=8, <=4),
+// capped by the wave (lpe = lanes that cover one edge).
+__host__ __device__ constexpr int slots_for_class(int lpe, int cls) {
+    const int nat = cls == 0 ? 16 : (cls == 1 ? 8 : (cls == 2 ? 4 : (cls == 3 ? 2 : 1)));
+    const int cap = kWave / lpe;
+    return nat < cap ? nat : cap;
+}
+__host__ __device__ constexpr int rows_per_wave(int lpe, int cls) { return kWave / (lpe * slots_for_class(lpe, cls)); }
+
 // One sorted view of the edge list plus its row schedule.
 struct Side {
     int32_t* rowptr = nullptr;   // [N+1]
     int32_t* col = nullptr;      // [E] other endpoint
     int32_t* eid = nullptr;      // [E] caller's edge id
     int32_t* pos = nullptr;      // [E] source side only, built on request: position of the edge in the destination-sorted order
-    Item* items = nullptr;       // [n_items]: workgroup items first, then wave items by length class (longest first)
+    Item* items = nullptr;       // [n_items]: workgroup items first, then wave items by (window, length class, row)
     int32_t* split_row = nullptr;   // [n_split] rows that were split
     int32_t* split_off = nullptr;   // [n_split+1] first partial slot of each split row
     int32_t* part2split = nullptr;  // [n_parts] index into split_row of the row a partial slot belongs to
-    int32_t n_items = 0, n_split = 0, n_parts = 0;
+    int32_t* split_grp = nullptr;   // [n_split+1] first combine group of each split row (a row with more than kCombineFan segments has ceil(segments / kCombineFan) groups)
+    int32_t n_items = 0, n_split = 0, n_parts = 0, n_groups = 0;
     int32_t n_block_items = 0;      // items [0, n_block_items) are walked by one workgroup each
-    int32_t n_spread_items = 0;     // the first of them: segments of rows with more than kSpreadSegs segments,
-                                    // handed to the XCDs round-robin
-    int32_t blk_chunk[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0};   // the others cut into 8 contiguous runs of equal edge count
-    int32_t class_off[kNumClass + 1] = {0, 0, 0, 0, 0, 0};   // item index where each wave class begins
+    // host copies the launch descriptors are made from
+    int32_t n_windows = 0;
+    std::vector<uint32_t> win_class_off;   // [n_windows * (kNumClass + 1)] wave items of (window, class) start at n_block_items + this
+    std::vector<uint32_t> win_class_cnt;   // same shape: how many
+    std::vector<int32_t> block_home;       // [n_block_items] window the workgroup item is scheduled with
+    std::vector<int32_t> block_len;        // [n_block_items] its edges
+    std::vector<uint8_t> block_spread;     // [n_block_items] 1: segment of a row with more than kSpreadSegs segments
 };
+
+// Launch descriptors of one kernel shape (lanes per edge): forward (destination view) and backward
+// (both views, window by window).
+struct Schedule {
+    WaveDesc* fwd = nullptr;
+    WaveDesc* bwd = nullptr;
+    int32_t fwd_blocks = 0, bwd_blocks = 0;
+    bool ready = false;
+};
+constexpr int kNumLpe = 5;   // lanes per edge 1, 2, 4, 8, 16
 
 // Device buffer that frees itself.
 struct DevBuf {
@@ -132,4 +169,10 @@ struct tgt_plan {
     int device = 0;
     tgt::Side dst;   // edges grouped by destination (query) node
     tgt::Side src;   // edges grouped by source (key/value) node
+    tgt::Schedule sched[tgt::kNumLpe];   // by log2(lanes per edge); made on first use of a shape
 };
+namespace tgt {
+// Descriptors for kernels with `lpe` lanes per edge; builds them on first use (allocates, copies and
+// synchronises `st` once per plan and shape).  nullptr on error.
+const Schedule* plan_schedule(const tgt_plan* plan, int lpe, hipStream_t st);
+}

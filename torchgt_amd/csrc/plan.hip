@@ -68,10 +68,11 @@ __global__ void k_gather_col(const uint32_t* __restrict__ eid, const uint32_t* _
 }
 
 // ---------------------------------------------------------------------------
-// schedule kernels: rows are binned on the device, only the few long rows visit the host
+// schedule kernels: rows are binned on the device, window by window; only per-window counts and the
+// few long rows visit the host
 // ---------------------------------------------------------------------------
 constexpr int kSchedCats = kNumClass + 1;   // the wave classes, then "longer than a wave row"
-constexpr int kSchedBlock = 256;
+constexpr int kSchedMaxWaves = 16;          // a window is one workgroup of up to 1024 threads, one per row
 
 __device__ __forceinline__ int sched_category(int len, int wave_row_max) {
     if (len > wave_row_max) return kNumClass;
@@ -82,14 +83,13 @@ __device__ __forceinline__ int sched_category(int len, int wave_row_max) {
     return 4;
 }
 
-// counts[cat * nblocks + block] = rows of that category among the block's 256 rows
-__global__ __launch_bounds__(kSchedBlock) void k_sched_count(const int32_t* __restrict__ rowptr, int64_t N,
-                                                            int wave_row_max, uint32_t* __restrict__ counts,
-                                                            int nblocks) {
+// counts[window * kSchedCats + cat] = rows of that category among the window's rows (blockDim.x rows)
+__global__ void k_sched_count(const int32_t* __restrict__ rowptr, int64_t N, int wave_row_max,
+                              uint32_t* __restrict__ counts) {
     __shared__ uint32_t c[kSchedCats];
     if (threadIdx.x < kSchedCats) c[threadIdx.x] = 0;
     __syncthreads();
-    const int64_t r = (int64_t)blockIdx.x * kSchedBlock + threadIdx.x;
+    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int cat = r < N ? sched_category(rowptr[r + 1] - rowptr[r], wave_row_max) : -1;
 #pragma unroll
     for (int k = 0; k < kSchedCats; ++k) {
@@ -97,20 +97,18 @@ __global__ __launch_bounds__(kSchedBlock) void k_sched_count(const int32_t* __re
         if ((threadIdx.x & 63) == 0 && b) atomicAdd(&c[k], (uint32_t)__popcll(b));   // integer count: order-free
     }
     __syncthreads();
-    if (threadIdx.x < kSchedCats) counts[(int64_t)threadIdx.x * nblocks + blockIdx.x] = c[threadIdx.x];
+    if (threadIdx.x < kSchedCats) counts[(int64_t)blockIdx.x * kSchedCats + threadIdx.x] = c[threadIdx.x];
 }
 
-// Rows keep their order inside a category: position = (rows of the category in earlier blocks)
-// + (rank among the block's rows).  Wave-class rows become schedule items at
-// items[class_base[cat] + position]; long rows are listed (row, first edge, length) for the host.
-struct SchedBases { int32_t v[kSchedCats]; };
-__global__ __launch_bounds__(kSchedBlock) void k_sched_fill(const int32_t* __restrict__ rowptr, int64_t N,
-                                                           int wave_row_max, const uint32_t* __restrict__ offs,
-                                                           int nblocks, SchedBases base, Item* __restrict__ items,
-                                                           int32_t* __restrict__ long_rows) {
-    __shared__ uint32_t wave_cnt[kSchedBlock / 64][kSchedCats];
+// Rows keep their order inside a (window, category): position = offs[window, cat] + rank among the
+// window's rows.  Wave-class rows become schedule items at items[base + position]; long rows are
+// listed (row, first edge, length) for the host.
+__global__ void k_sched_fill(const int32_t* __restrict__ rowptr, int64_t N, int wave_row_max,
+                             const uint32_t* __restrict__ offs, int64_t base, Item* __restrict__ items,
+                             int32_t* __restrict__ long_rows) {
+    __shared__ uint32_t wave_cnt[kSchedMaxWaves][kSchedCats];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int64_t r = (int64_t)blockIdx.x * kSchedBlock + threadIdx.x;
+    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     int start = 0, len = 0, cat = -1;
     if (r < N) {
         start = rowptr[r];
@@ -127,15 +125,22 @@ __global__ __launch_bounds__(kSchedBlock) void k_sched_fill(const int32_t* __res
     }
     __syncthreads();
     if (cat < 0) return;
-    uint32_t pos = offs[(int64_t)cat * nblocks + blockIdx.x] + rank;
+    uint32_t pos = offs[(int64_t)blockIdx.x * kSchedCats + cat] + rank;
     for (int w = 0; w < wave; ++w) pos += wave_cnt[w][cat];
     if (cat < kNumClass) {
-        if (items) items[(int64_t)base.v[cat] + pos] = Item{(int32_t)r, start, len, -1};
+        if (items) items[base + pos] = Item{(int32_t)r, start, len, -1};
     } else if (long_rows) {
         long_rows[3 * (int64_t)pos + 0] = (int32_t)r;
         long_rows[3 * (int64_t)pos + 1] = start;
         long_rows[3 * (int64_t)pos + 2] = len;
     }
+}
+
+// out[i] = col[idx[i]]
+__global__ void k_gather_i32(const int32_t* __restrict__ col, const int32_t* __restrict__ idx, int n,
+                             int32_t* __restrict__ out) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = col[idx[i]];
 }
 
 // ---------------------------------------------------------------------------
@@ -160,13 +165,6 @@ static int build_side(const uint32_t* keys32, const uint32_t* other32, int64_t E
     return TGT_OK;
 }
 
-
-// Row schedule from a host copy of rowptr.  A row of up to kWaveRowMax edges is
-// one wave item; items are grouped by length class (longest first) and keep row
-// order inside a class, so the lanes of a wave see uniform lengths and
-// neighbouring rows stay together.  A longer row is walked by whole workgroups:
-// ceil(len / kBlockSeg) balanced segments, each a workgroup item; if there is more
-// than one segment their partial sums meet in the workspace.
 static int env_int(const char* name, int dflt) {
     const char* v = getenv(name);
     if (!v || !*v) return dflt;
@@ -174,120 +172,114 @@ static int env_int(const char* name, int dflt) {
     return x > 0 ? x : dflt;
 }
 
-// exclusive prefix over the blocks of every category (one workgroup per category) + totals
-__global__ __launch_bounds__(256) void k_sched_scan(uint32_t* __restrict__ counts, int nblocks,
-                                                    uint32_t* __restrict__ totals) {
-    __shared__ uint32_t part[256];
-    const int tid = threadIdx.x;
-    uint32_t* row = counts + (int64_t)blockIdx.x * nblocks;
-    const int chunk = (nblocks + 255) / 256;
-    const int b = tid * chunk, e = min(b + chunk, nblocks);
-    uint32_t sum = 0;
-    for (int i = b; i < e; ++i) sum += row[i];
-    part[tid] = sum;
-    __syncthreads();
-    for (int off = 1; off < 256; off <<= 1) {
-        const uint32_t x = tid >= off ? part[tid - off] : 0u;
-        __syncthreads();
-        part[tid] += x;
-        __syncthreads();
-    }
-    uint32_t run = tid ? part[tid - 1] : 0u;
-    for (int i = b; i < e; ++i) {
-        const uint32_t x = row[i];
-        row[i] = run;
-        run += x;
-    }
-    if (tid == 255) totals[blockIdx.x] = part[255];
+static int window_rows() {
+    int w = env_int("TGT_WINDOW_ROWS", tgt::kWindowRows);
+    w = (w + 63) / 64 * 64;
+    return w > 64 * kSchedMaxWaves ? 64 * kSchedMaxWaves : w;
 }
 
+// Row schedule.  Rows are taken window by window (a window = window_rows() consecutive node ids).
+// A row of up to kWaveRowMax edges is one wave item; the wave items of a window are grouped by length
+// class (longest first) and keep row order inside a class, so the lanes of a wave see uniform lengths.
+// A longer row is walked by whole workgroups: balanced segments, each a workgroup item that is
+// scheduled with the window most of its other endpoints lie in (so that the rows a segment gathers
+// are the ones the window's own rows load); if there is more than one segment their partial sums
+// meet in the workspace.
 static int build_schedule(int64_t N, Side& side, hipStream_t st) {
     // tuning overrides (experiments only; the defaults are the measured best)
     const int kWaveRowMax = env_int("TGT_WAVE_ROW_MAX", tgt::kWaveRowMax);
     const int kBlockSeg = env_int("TGT_BLOCK_SEG", tgt::kBlockSeg);
     const int kSpreadSeg = env_int("TGT_SPREAD_SEG", tgt::kSpreadSeg);
-    const int nblocks = (int)((N + kSchedBlock - 1) / kSchedBlock);
-    DevBuf counts, totals_d, long_d;
-    TGT_HIP_CHECK(counts.alloc(sizeof(uint32_t) * (size_t)kSchedCats * nblocks));
-    TGT_HIP_CHECK(totals_d.alloc(sizeof(uint32_t) * kSchedCats));
-    hipLaunchKernelGGL(k_sched_count, dim3(nblocks), dim3(kSchedBlock), 0, st, side.rowptr, N, kWaveRowMax,
-                       counts.as<uint32_t>(), nblocks);
-    hipLaunchKernelGGL(k_sched_scan, dim3(kSchedCats), dim3(256), 0, st, counts.as<uint32_t>(), nblocks,
-                       totals_d.as<uint32_t>());
+    const int W = window_rows();
+    const int nwin = (int)((N + W - 1) / W);
+    side.n_windows = nwin;
+    DevBuf counts, long_d;
+    const size_t ncnt = (size_t)kSchedCats * nwin;
+    TGT_HIP_CHECK(counts.alloc(sizeof(uint32_t) * ncnt));
+    hipLaunchKernelGGL(k_sched_count, dim3(nwin), dim3(W), 0, st, side.rowptr, N, kWaveRowMax, counts.as<uint32_t>());
     TGT_HIP_CHECK(hipGetLastError());
-    uint32_t totals[kSchedCats];
-    TGT_HIP_CHECK(hipMemcpyAsync(totals, totals_d.p, sizeof(totals), hipMemcpyDeviceToHost, st));
+    std::vector<uint32_t> cnt(ncnt), offs(ncnt);
+    TGT_HIP_CHECK(hipMemcpyAsync(cnt.data(), counts.p, sizeof(uint32_t) * ncnt, hipMemcpyDeviceToHost, st));
     TGT_HIP_CHECK(hipStreamSynchronize(st));
+    // positions: wave items run over (window, class); long rows over windows
+    uint32_t n_wave = 0, n_long = 0;
+    for (int w = 0; w < nwin; ++w) {
+        for (int c = 0; c < kNumClass; ++c) { offs[(size_t)w * kSchedCats + c] = n_wave; n_wave += cnt[(size_t)w * kSchedCats + c]; }
+        offs[(size_t)w * kSchedCats + kNumClass] = n_long;
+        n_long += cnt[(size_t)w * kSchedCats + kNumClass];
+    }
+    side.win_class_off = offs;
+    side.win_class_cnt = cnt;
+    TGT_HIP_CHECK(hipMemcpyAsync(counts.p, offs.data(), sizeof(uint32_t) * ncnt, hipMemcpyHostToDevice, st));
     // the long rows (few) come to the host, which cuts them into workgroup items
-    const int64_t n_long = totals[kNumClass];
-    std::vector<int32_t> longs((size_t)(3 * n_long));
+    std::vector<int32_t> longs((size_t)3 * n_long);
     if (n_long > 0) {
-        TGT_HIP_CHECK(long_d.alloc(sizeof(int32_t) * (size_t)(3 * n_long)));
-        hipLaunchKernelGGL(k_sched_fill, dim3(nblocks), dim3(kSchedBlock), 0, st, side.rowptr, N, kWaveRowMax,
-                           counts.as<uint32_t>(), nblocks, SchedBases{}, (Item*)nullptr, long_d.as<int32_t>());
+        TGT_HIP_CHECK(long_d.alloc(sizeof(int32_t) * (size_t)3 * n_long));
+        hipLaunchKernelGGL(k_sched_fill, dim3(nwin), dim3(W), 0, st, side.rowptr, N, kWaveRowMax, counts.as<uint32_t>(),
+                           (int64_t)0, (Item*)nullptr, long_d.as<int32_t>());
         TGT_HIP_CHECK(hipGetLastError());
         TGT_HIP_CHECK(hipMemcpyAsync(longs.data(), long_d.p, sizeof(int32_t) * longs.size(), hipMemcpyDeviceToHost, st));
         TGT_HIP_CHECK(hipStreamSynchronize(st));
     }
-    std::vector<Item> items;       // segments of very long rows: spread over all XCDs
-    std::vector<Item> local;       // other workgroup items: contiguous runs per XCD
-    std::vector<int32_t> split_row, split_off, part2split;
+    std::vector<Item> items;
+    std::vector<int32_t> split_row, split_off, part2split, split_grp, mid;
+    int32_t n_groups = 0;
     int32_t n_parts = 0;
-    for (int64_t i = 0; i < n_long; ++i) {
+    for (int64_t i = 0; i < (int64_t)n_long; ++i) {
         const int32_t r = longs[3 * i], b = longs[3 * i + 1], len = longs[3 * i + 2];
         int nseg = (len + kBlockSeg - 1) / kBlockSeg;
-        // a row long enough to be spread over all XCDs is alone on the critical path of the launch:
-        // it gets shorter segments (more workgroups, fewer steps each)
-        if (nseg > kSpreadSegs) nseg = (len + kSpreadSeg - 1) / kSpreadSeg;
+        // a row with many segments (a global node) gets short ones: each is scheduled next to the rows it gathers
+        const bool spread = nseg > kSpreadSegs;
+        if (spread) nseg = (len + kSpreadSeg - 1) / kSpreadSeg;
         if (nseg == 1) {
-            local.push_back(Item{r, b, len, -1});
+            items.push_back(Item{r, b, len, -1});
+            mid.push_back(b + len / 2);
+            side.block_spread.push_back(0);
             continue;
         }
-        std::vector<Item>& where = nseg > kSpreadSegs ? items : local;
         const int seg = (len + nseg - 1) / nseg;
         split_off.push_back(n_parts);
         for (int s = 0; s < nseg; ++s) {
             const int o = s * seg;
             const int l = (o + seg <= len) ? seg : (len - o);
             part2split.push_back((int32_t)split_row.size());
-            where.push_back(Item{r, b + o, l, n_parts++});
+            items.push_back(Item{r, b + o, l, n_parts++});
+            mid.push_back(b + o + l / 2);
+            side.block_spread.push_back(spread ? 1 : 0);
         }
         split_row.push_back(r);
+        split_grp.push_back(n_groups);
+        if (nseg > kCombineFan) n_groups += (nseg + kCombineFan - 1) / kCombineFan;
     }
     split_off.push_back(n_parts);
-    side.n_spread_items = (int32_t)items.size();
-    {   // 8 contiguous runs of the other workgroup items with (nearly) equal numbers of edges, one per XCD
-        const int32_t base = side.n_spread_items;
-        int64_t total = 0;
-        for (const Item& it : local) total += it.len;
-        int64_t run = 0;
-        int x = 1;
-        side.blk_chunk[0] = base;
-        for (size_t i = 0; i < local.size() && x < 8; ++i) {
-            run += local[i].len;
-            while (x < 8 && run * 8 >= total * x) side.blk_chunk[x++] = base + (int32_t)(i + 1);
-        }
-        while (x <= 8) side.blk_chunk[x++] = base + (int32_t)local.size();
-    }
-    items.insert(items.end(), local.begin(), local.end());
+    split_grp.push_back(n_groups);
+    side.n_groups = n_groups;
     side.n_block_items = (int32_t)items.size();
-    SchedBases base{};
-    int64_t at = side.n_block_items;
-    for (int c = 0; c < kNumClass; ++c) {
-        side.class_off[c] = (int32_t)at;
-        base.v[c] = (int32_t)at;
-        at += totals[c];
-    }
-    side.class_off[kNumClass] = (int32_t)at;
-    side.n_items = (int32_t)at;
+    side.n_items = (int32_t)(items.size() + n_wave);
     side.n_split = (int32_t)split_row.size();
     side.n_parts = n_parts;
-    TGT_HIP_CHECK(hipMalloc((void**)&side.items, sizeof(Item) * ((size_t)at + 1)));
+    side.block_len.resize(items.size());
+    side.block_home.assign(items.size(), 0);
+    for (size_t i = 0; i < items.size(); ++i) side.block_len[i] = items[i].len;
+    TGT_HIP_CHECK(hipMalloc((void**)&side.items, sizeof(Item) * ((size_t)side.n_items + 1)));
     TGT_HIP_CHECK(hipMalloc((void**)&side.split_row, sizeof(int32_t) * (split_row.size() + 1)));
     TGT_HIP_CHECK(hipMalloc((void**)&side.split_off, sizeof(int32_t) * split_off.size()));
     TGT_HIP_CHECK(hipMalloc((void**)&side.part2split, sizeof(int32_t) * (part2split.size() + 1)));
-    if (!items.empty())
+    TGT_HIP_CHECK(hipMalloc((void**)&side.split_grp, sizeof(int32_t) * split_grp.size()));
+    TGT_HIP_CHECK(hipMemcpyAsync(side.split_grp, split_grp.data(), sizeof(int32_t) * split_grp.size(), hipMemcpyHostToDevice, st));
+    DevBuf mid_d, home_d;
+    if (!items.empty()) {
         TGT_HIP_CHECK(hipMemcpyAsync(side.items, items.data(), sizeof(Item) * items.size(), hipMemcpyHostToDevice, st));
+        // home window of a workgroup item: the window of the other endpoint in the middle of its edges
+        const int nb = (int)items.size();
+        TGT_HIP_CHECK(mid_d.alloc(sizeof(int32_t) * nb));
+        TGT_HIP_CHECK(home_d.alloc(sizeof(int32_t) * nb));
+        TGT_HIP_CHECK(hipMemcpyAsync(mid_d.p, mid.data(), sizeof(int32_t) * nb, hipMemcpyHostToDevice, st));
+        hipLaunchKernelGGL(k_gather_i32, dim3((nb + 255) / 256), dim3(256), 0, st, side.col, mid_d.as<int32_t>(), nb,
+                           home_d.as<int32_t>());
+        TGT_HIP_CHECK(hipGetLastError());
+        TGT_HIP_CHECK(hipMemcpyAsync(side.block_home.data(), home_d.p, sizeof(int32_t) * nb, hipMemcpyDeviceToHost, st));
+    }
     if (!split_row.empty()) {
         TGT_HIP_CHECK(hipMemcpyAsync(side.split_row, split_row.data(), sizeof(int32_t) * split_row.size(),
                                      hipMemcpyHostToDevice, st));
@@ -296,12 +288,142 @@ static int build_schedule(int64_t N, Side& side, hipStream_t st) {
     }
     TGT_HIP_CHECK(hipMemcpyAsync(side.split_off, split_off.data(), sizeof(int32_t) * split_off.size(),
                                  hipMemcpyHostToDevice, st));
-    // the wave items (the bulk) are written by the device, in row order inside every class
-    hipLaunchKernelGGL(k_sched_fill, dim3(nblocks), dim3(kSchedBlock), 0, st, side.rowptr, N, kWaveRowMax,
-                       counts.as<uint32_t>(), nblocks, base, side.items, (int32_t*)nullptr);
+    // the wave items (the bulk) are written by the device
+    hipLaunchKernelGGL(k_sched_fill, dim3(nwin), dim3(W), 0, st, side.rowptr, N, kWaveRowMax, counts.as<uint32_t>(),
+                       (int64_t)side.n_block_items, side.items, (int32_t*)nullptr);
     TGT_HIP_CHECK(hipGetLastError());
     TGT_HIP_CHECK(hipStreamSynchronize(st));   // the host vectors and the scratch buffers die at return
+    for (int32_t& h : side.block_home) h = h / W;   // node id -> window
     return TGT_OK;
+}
+
+// ---------------------------------------------------------------------------
+// launch descriptors
+// ---------------------------------------------------------------------------
+// Workgroups reach the 8 XCDs round-robin (workgroup id mod 8) and every XCD has its own L2.  The
+// windows are cut into 8 contiguous ranges of about equal work, XCD x walks range x in window order,
+// and inside a window the workgroup items homed there come first, then the waves of its rows, longest
+// class first - for the backward both views of the window side by side.  What the rows of a window
+// load (their own q/k/v/dout rows, the rows of their self-loops, the window's share of a global node's
+// segment) then meets in one L2 at about the same time.
+namespace {
+// Workgroup items homed at window w_items and wave descriptors of window w of one view (either may be -1:
+// none), appended to `waves`; `cost` grows by a rough measure of the work.  part 0: the heavy share (segments of ordinary long rows and the rows of the longest class, which
+// run for many steps and whose edges have no tie to the window), part 1: the rest (segments of a row that
+// spans the graph, which gather exactly the window's rows, and the short rows).
+void append_side(std::vector<WaveDesc>& waves, float& cost, const Side& s, int w, int w_items, int lpe, bool src_side,
+                 const std::vector<std::vector<int32_t>>& homed, int part) {
+    if (w_items >= 0) {
+        for (int32_t it : homed[w_items]) {
+            if ((s.block_spread[it] != 0) != (part == 1)) continue;
+            // close a partly filled workgroup first: a workgroup item takes all four waves
+            while (waves.size() % 4) waves.push_back(WaveDesc{0, kDescNone});
+            for (int k = 0; k < 4; ++k) waves.push_back(WaveDesc{it, desc_code(kDescBlock, src_side, 0)});
+            cost += 1.0f + s.block_len[it] / 128.0f;
+        }
+    }
+    if (w < 0) return;
+    for (int c = (part == 0 ? 0 : 1); c < (part == 0 ? 1 : kNumClass); ++c) {
+        const uint32_t n = s.win_class_cnt[(size_t)w * (kNumClass + 1) + c];
+        const uint32_t first = s.n_block_items + s.win_class_off[(size_t)w * (kNumClass + 1) + c];
+        const uint32_t ipw = (uint32_t)rows_per_wave(lpe, c);
+        for (uint32_t i = 0; i < n; i += ipw) {
+            waves.push_back(WaveDesc{(int32_t)(first + i), desc_code((uint32_t)c, src_side, n - i < ipw ? n - i : ipw)});
+            cost += c == 0 ? 0.75f : 0.25f;
+        }
+    }
+}
+
+// descriptors of all windows -> block order.  XCD x gets a contiguous range of windows; it first walks the
+// heavy share of all its windows (long work first keeps the end of the launch short), then window by window.
+int place(const std::vector<const Side*>& sides, int lpe, WaveDesc** d_out, int32_t* n_blocks, hipStream_t st) {
+    const int nwin = sides[0]->n_windows;
+    const bool heavy_first = env_int("TGT_HEAVY_FIRST", 1) == 1;
+    std::vector<std::vector<std::vector<int32_t>>> homed(sides.size());
+    for (size_t k = 0; k < sides.size(); ++k) {
+        homed[k].resize(nwin > 0 ? nwin : 1);
+        for (int32_t i = 0; i < sides[k]->n_block_items; ++i) {
+            int h = sides[k]->block_home[i];
+            h = h < 0 ? 0 : (h >= nwin ? nwin - 1 : h);
+            homed[k][h].push_back(i);
+        }
+    }
+    // 8 contiguous window ranges with about equal numbers of edges and rows
+    int bound[9];
+    bound[0] = 0;
+    {
+        std::vector<double> cost(nwin + 1, 0.0);
+        for (int w = 0; w < nwin; ++w) {
+            double c = 0.0;
+            for (const Side* sd : sides) {
+                for (int32_t it : homed[sd == sides[0] ? 0 : 1][w]) c += 1.0 + sd->block_len[it] / 128.0;
+                for (int k = 0; k < kNumClass; ++k)
+                    c += (k == 0 ? 0.75 : 0.25) * ((sd->win_class_cnt[(size_t)w * (kNumClass + 1) + k] + rows_per_wave(lpe, k) - 1) /
+                                                   rows_per_wave(lpe, k));
+            }
+            cost[w + 1] = cost[w] + c;
+        }
+        int x = 1;
+        for (int w = 0; w < nwin && x < 8; ++w)
+            while (x < 8 && cost[w + 1] * 8 >= cost[nwin] * x) bound[x++] = w + 1;
+        while (x <= 8) bound[x++] = nwin;
+    }
+    // Per XCD and part: runs of whole workgroups.  Part 0 (heavy share) of all windows of the range first.  In
+    // part 1 the segments homed at a window run `lead` windows ahead of the window's rows: close enough in
+    // time for the rows to meet in the L2, and the last windows of a range end with short rows only - the
+    // chain of a split row (partial slot, arrival, sums of the group and of the row) is not left for the end.
+    const int lead = env_int("TGT_SEGMENT_LEAD", 6);
+    std::vector<WaveDesc> xw[8];
+    for (int x = 0; x < 8; ++x) {
+        float c = 0.f;
+        std::vector<WaveDesc>& wv = xw[x];
+        const int w0 = bound[x], w1 = bound[x + 1];
+        if (heavy_first) {
+            for (int w = w0; w < w1; ++w) {
+                for (size_t k = 0; k < sides.size(); ++k) append_side(wv, c, *sides[k], w, w, lpe, k == 1, homed[k], 0);
+            }
+            while (wv.size() % 4) wv.push_back(WaveDesc{0, kDescNone});
+        }
+        // the segments of the last half of the range go first: when the launch ends no split row is still
+        // being added up (those windows give up meeting their segment in the L2)
+        const int w_early = w1 - (w1 - w0) / env_int("TGT_EARLY_SHARE", 2);
+        for (int w = w_early; w < w1; ++w)
+            for (size_t k = 0; k < sides.size(); ++k) append_side(wv, c, *sides[k], -1, w, lpe, k == 1, homed[k], 1);
+        for (int w = w0 - lead; w < w1; ++w) {
+            const int wi = w + lead < w_early ? w + lead : -1;        // segments of the window `lead` ahead
+            for (size_t k = 0; k < sides.size(); ++k) {
+                if (!heavy_first) append_side(wv, c, *sides[k], w >= w0 ? w : -1, w >= w0 ? w : -1, lpe, k == 1, homed[k], 0);
+                append_side(wv, c, *sides[k], w >= w0 ? w : -1, wi >= w0 ? wi : -1, lpe, k == 1, homed[k], 1);
+            }
+            while (wv.size() % 4) wv.push_back(WaveDesc{0, kDescNone});
+        }
+    }
+    size_t per = 0;
+    for (int x = 0; x < 8; ++x) per = std::max(per, xw[x].size() / 4);
+    const size_t nb = per * 8;
+    std::vector<WaveDesc> placed(nb * 4 + 4, WaveDesc{0, kDescNone});
+    for (int x = 0; x < 8; ++x)
+        for (size_t b = 0; b < xw[x].size() / 4; ++b)
+            for (int k = 0; k < 4; ++k) placed[(b * 8 + x) * 4 + k] = xw[x][b * 4 + k];
+    TGT_HIP_CHECK(hipMalloc((void**)d_out, sizeof(WaveDesc) * placed.size()));
+    TGT_HIP_CHECK(hipMemcpyAsync(*d_out, placed.data(), sizeof(WaveDesc) * placed.size(), hipMemcpyHostToDevice, st));
+    TGT_HIP_CHECK(hipStreamSynchronize(st));
+    *n_blocks = (int32_t)nb;
+    return TGT_OK;
+}
+}  // namespace
+
+const Schedule* plan_schedule(const tgt_plan* plan_c, int lpe, hipStream_t st) {
+    int idx = 0;
+    while (idx < kNumLpe && (1 << idx) != lpe) ++idx;
+    if (idx == kNumLpe) { set_error("no schedule for %d lanes per edge", lpe); return nullptr; }
+    tgt_plan* plan = const_cast<tgt_plan*>(plan_c);
+    Schedule& sc = plan->sched[idx];
+    if (sc.ready) return &sc;
+    if (place({&plan->dst}, lpe, &sc.fwd, &sc.fwd_blocks, st) != TGT_OK) return nullptr;
+    if (place({&plan->dst, &plan->src}, lpe, &sc.bwd, &sc.bwd_blocks, st) != TGT_OK) return nullptr;
+    sc.ready = true;
+    return &sc;
 }
 
 // inv[eid[c]] = c, then pos[p] = inv[eid_src[p]]: where each edge of the source-sorted order sits in the
@@ -343,7 +465,16 @@ static void free_side(Side& s) {
     if (s.split_row) (void)hipFree(s.split_row);
     if (s.split_off) (void)hipFree(s.split_off);
     if (s.part2split) (void)hipFree(s.part2split);
+    if (s.split_grp) (void)hipFree(s.split_grp);
     s = Side();
+}
+
+static void free_schedules(tgt_plan* plan) {
+    for (Schedule& sc : plan->sched) {
+        if (sc.fwd) (void)hipFree(sc.fwd);
+        if (sc.bwd) (void)hipFree(sc.bwd);
+        sc = Schedule();
+    }
 }
 
 static int create_impl(const int64_t* d_src, const int64_t* d_dst, int64_t E, int64_t N, hipStream_t st,
@@ -386,7 +517,10 @@ static int create_impl(const int64_t* d_src, const int64_t* d_dst, int64_t E, in
     if (rc) return rc;
     rc = build_schedule(N, plan->dst, st);
     if (rc) return rc;
-    return build_schedule(N, plan->src, st);
+    rc = build_schedule(N, plan->src, st);
+    if (rc) return rc;
+    // the shape of the reference's node-level models (hidden 64: 8 heads of 8, or 4 of 16); other shapes on first use
+    return plan_schedule(plan, 8, st) ? TGT_OK : TGT_ERR_HIP;
 }
 
 }  // namespace tgt
@@ -446,6 +580,7 @@ int tgt_plan_create(const int64_t* d_src, const int64_t* d_dst, int64_t E, int64
     if (rc != TGT_OK) {
         tgt::free_side(plan->dst);
         tgt::free_side(plan->src);
+        tgt::free_schedules(plan);
         delete plan;
         return rc;
     }
@@ -457,6 +592,7 @@ int tgt_plan_destroy(tgt_plan_t* plan) {
     if (!plan) return TGT_OK;
     tgt::free_side(plan->dst);
     tgt::free_side(plan->src);
+    tgt::free_schedules(plan);
     delete plan;
     return TGT_OK;
 }

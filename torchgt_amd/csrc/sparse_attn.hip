@@ -144,13 +144,6 @@ __device__ __forceinline__ float clamp5(float x) { return x < -5.0f ? -5.0f : (x
 constexpr float kEps = 1e-6f;   // attn_module.py:187
 constexpr int kUnroll = 4;      // edges in flight per slot
 
-__host__ __device__ constexpr int slots_for_class(int lpe, int cls) {
-    // natural slot count of the length classes (>32, <=32, <=16, <=8, <=4), capped by the wave
-    const int nat = cls == 0 ? 16 : (cls == 1 ? 8 : (cls == 2 ? 4 : (cls == 3 ? 2 : 1)));
-    const int cap = kWave / lpe;
-    return nat < cap ? nat : cap;
-}
-
 // Which walk a workgroup performs.
 enum { MODE_FWD = 0, MODE_BWD_DST = 1, MODE_BWD_SRC = 2 };
 
@@ -175,6 +168,8 @@ struct SideArgs {
     const int32_t* eid;
     const int32_t* split_off;
     const int32_t* part2split;
+    const int32_t* split_grp;     // first combine group of each split row (rows with more than kCombineFan segments have groups)
+    int32_t n_split, n_parts;     // group counters follow the n_split row counters, group slots the n_parts segment slots
     void* out0;           // fwd: out      bwd_dst: dq     bwd_src: dk
     void* out1;           // fwd: -        bwd_dst: dbias  bwd_src: dv
     float* Z;             // fwd: Z
@@ -186,15 +181,6 @@ struct SideArgs {
     const float* init1;
     const float* initZ;
     const uint8_t* cover; // [N] 1 where the row has such sums
-    int32_t n_block_items;
-    int32_t n_spread;                    // workgroup items [0, n_spread) go to the XCDs round-robin
-    int32_t spread_pad;                  // n_spread rounded up to a multiple of 8
-    int32_t blk_chunk[9];                // XCD x walks workgroup items [blk_chunk[x], blk_chunk[x+1])
-    int32_t n_wave_blocks;               // multiple of 8
-    int32_t class_off[kNumClass + 1];    // item index where each wave class begins
-    int32_t nwaves[kNumClass];           // waves of each class
-    int32_t chunk[kNumClass];            // waves of each class given to one XCD (ceil(nwaves / 8))
-    int32_t voff[kNumClass + 1];         // prefix sums of chunk: wave slots of one XCD
 };
 
 struct Acc {
@@ -416,48 +402,32 @@ __device__ __forceinline__ void write_row(const Common& c, const SideArgs& s, co
     }
 }
 
-// Wave items: rows of at most kWaveRowMax edges, 64 / (LPE*S) rows per wave.
+// Wave items: rows of at most kWaveRowMax edges, 64 / (LPE*S) rows per wave.  The wave takes items
+// [first, first + count).
 template <typename T, int LPE, int LPH, int S, int MODE, int HASB, bool TILES>
-__device__ __forceinline__ void wave_items(const Common& c, const SideArgs& s, const int item_begin,
-                                           const int item_end, const int wave_in_class) {
+__device__ __forceinline__ void wave_items(const Common& c, const SideArgs& s, const int first, const int count) {
     constexpr int G = LPE * S;
-    constexpr int IPW = kWave / G;
     const int lane = threadIdx.x & (kWave - 1);
     const int sub = lane / G, gl = lane % G;
     const int slot = gl / LPE, el = gl % LPE;
-    const int item = item_begin + wave_in_class * IPW + sub;
-    const bool valid = item < item_end;
+    const bool valid = sub < count;
     Item it{0, 0, 0, -1};
-    if (valid) it = s.items[item];
+    if (valid) it = s.items[first + sub];
     Acc acc;
     walk_range<T, LPE, LPH, S, MODE, HASB>(c, s, it.row, it.start, it.len, slot, el, valid, acc);
     if (valid && slot == 0) write_row<T, LPE, LPH, MODE, TILES>(c, s, it.row, el, acc);
 }
 
-// Wave items, XCD-aware.  Workgroups go to the 8 XCDs round-robin (workgroup id mod 8), each
-// XCD has its own L2, and neighbouring rows tend to share sources (clustered / reordered
-// graphs).  So every class's waves are cut into 8 contiguous chunks and XCD x walks chunk x of
-// every class, longest class first: rows that are neighbours in the schedule meet in one L2.
-// `block` counts from the start of this view's wave region, which begins at a workgroup id
-// that is a multiple of 8.
+// The wave's share of a workgroup that walks wave items: its descriptor names the length class.
 template <typename T, int LPE, int LPH, int MODE, int HASB, bool TILES>
-__device__ __forceinline__ void wave_block(const Common& c, const SideArgs& s, const int block) {
-    const int xcd = block & 7;
-    const int v = (block >> 3) * (kBlock / kWave) + (threadIdx.x >> 6);   // wave slot inside the XCD
-    int cls = 0;
-#pragma unroll
-    for (int k = 1; k < kNumClass; ++k) cls += (v >= s.voff[k]) ? 1 : 0;
-    cls = __builtin_amdgcn_readfirstlane(cls);
-    if (v >= s.voff[kNumClass]) return;
-    const int w = xcd * s.chunk[cls] + (v - s.voff[cls]);
-    if (w >= s.nwaves[cls]) return;
-    const int b = s.class_off[cls], e = s.class_off[cls + 1];
-    switch (cls) {
-        case 0: wave_items<T, LPE, LPH, slots_for_class(LPE, 0), MODE, HASB, TILES>(c, s, b, e, w); break;
-        case 1: wave_items<T, LPE, LPH, slots_for_class(LPE, 1), MODE, HASB, TILES>(c, s, b, e, w); break;
-        case 2: wave_items<T, LPE, LPH, slots_for_class(LPE, 2), MODE, HASB, TILES>(c, s, b, e, w); break;
-        case 3: wave_items<T, LPE, LPH, slots_for_class(LPE, 3), MODE, HASB, TILES>(c, s, b, e, w); break;
-        default: wave_items<T, LPE, LPH, slots_for_class(LPE, 4), MODE, HASB, TILES>(c, s, b, e, w); break;
+__device__ __forceinline__ void wave_dispatch(const Common& c, const SideArgs& s, const int kind, const int first,
+                                              const int count) {
+    switch (kind) {
+        case 0: wave_items<T, LPE, LPH, slots_for_class(LPE, 0), MODE, HASB, TILES>(c, s, first, count); break;
+        case 1: wave_items<T, LPE, LPH, slots_for_class(LPE, 1), MODE, HASB, TILES>(c, s, first, count); break;
+        case 2: wave_items<T, LPE, LPH, slots_for_class(LPE, 2), MODE, HASB, TILES>(c, s, first, count); break;
+        case 3: wave_items<T, LPE, LPH, slots_for_class(LPE, 3), MODE, HASB, TILES>(c, s, first, count); break;
+        default: wave_items<T, LPE, LPH, slots_for_class(LPE, 4), MODE, HASB, TILES>(c, s, first, count); break;
     }
 }
 
@@ -472,12 +442,124 @@ struct BlockLds {
     int last;
 };
 
+// Adds the partial slots [first, first + count) of s.part with all threads of the workgroup: the
+// NGROUP groups of LPE threads take slots first + grp, first + grp + NGROUP, ... (two per step, so
+// that the device-scope loads of two slots are in flight together), LDS adds the groups in group order.
+// On return threads 0 .. LPE-1 hold the sums.  The order of the additions is fixed by (first, count).
+template <int LPE, int LPH, int MODE>
+__device__ __forceinline__ void sum_slots(const SideArgs& s, const int first, const int count, BlockLds<LPE>& lds,
+                                          Acc& acc) {
+    constexpr int H = LPE / LPH;
+    constexpr int HD = LPE * 8;
+    constexpr int STRIDE = BlockLds<LPE>::STRIDE;
+    constexpr int NGROUP = BlockLds<LPE>::NGROUP;
+    constexpr int PS = part_stride<MODE, HD, H>();
+    const int tid = threadIdx.x;
+    const int grp2 = tid / LPE, el2 = tid % LPE;
+    {
+        float a0[8], a1[8], z = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { a0[i] = 0.f; a1[i] = 0.f; }
+        for (int p = grp2; p < count; p += 2 * NGROUP) {
+            const bool two = p + NGROUP < count;
+            const float* srcA = s.part + (int64_t)(first + p) * PS;
+            const float* srcB = s.part + (int64_t)(first + (two ? p + NGROUP : p)) * PS;
+            float tA[8], tB[8], uA[8], uB[8], zA = 0.f, zB = 0.f;
+            load8_dev(srcA + el2 * 8, tA);
+            load8_dev(srcB + el2 * 8, tB);
+            if (MODE == MODE_BWD_SRC) {
+                load8_dev(srcA + HD + el2 * 8, uA);
+                load8_dev(srcB + HD + el2 * 8, uB);
+            }
+            if (MODE == MODE_FWD) {
+                zA = load_dev(srcA + HD + el2 / LPH);
+                zB = load_dev(srcB + HD + el2 / LPH);
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                a0[i] += tA[i];
+                if (two) a0[i] += tB[i];
+                if (MODE == MODE_BWD_SRC) {
+                    a1[i] += uA[i];
+                    if (two) a1[i] += uB[i];
+                }
+            }
+            if (MODE == MODE_FWD) {
+                z += zA;
+                if (two) z += zB;
+            }
+        }
+        float* r = lds.red + grp2 * STRIDE;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            r[el2 * 8 + i] = a0[i];
+            if (MODE == MODE_BWD_SRC) r[HD + el2 * 8 + i] = a1[i];
+        }
+        if (MODE == MODE_FWD) r[2 * HD + el2] = z;
+    }
+    __syncthreads();
+    if (tid < LPE) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { acc.a0[i] = 0.f; acc.a1[i] = 0.f; }
+        acc.z = 0.f;
+        const int ng = count < NGROUP ? count : NGROUP;     // groups that added anything
+        for (int gI = 0; gI < ng; ++gI) {
+            const float* r = lds.red + gI * STRIDE;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                acc.a0[i] += r[tid * 8 + i];
+                if (MODE == MODE_BWD_SRC) acc.a1[i] += r[HD + tid * 8 + i];
+            }
+            if (MODE == MODE_FWD) acc.z += r[2 * HD + tid];
+        }
+    }
+}
+
+// Threads 0 .. LPE-1 store their sums into partial slot `slot` with device-scope stores.
+template <int LPE, int LPH, int MODE>
+__device__ __forceinline__ void store_slot(const SideArgs& s, const int slot, const Acc& acc) {
+    constexpr int H = LPE / LPH;
+    constexpr int HD = LPE * 8;
+    constexpr int PS = part_stride<MODE, HD, H>();
+    const int tid = threadIdx.x;
+    float* p = s.part + (int64_t)slot * PS;
+    store8_dev(p + tid * 8, acc.a0);
+    if (MODE == MODE_BWD_SRC) store8_dev(p + HD + tid * 8, acc.a1);
+    if (MODE == MODE_FWD && tid % LPH == 0) store_dev(p + HD + tid / LPH, acc.z);
+}
+
+// Arrival at counter `idx`: the slot written by threads 0 .. LPE-1 (all in wave 0) is published before
+// the counter moves: once wave 0's device-scope stores are acknowledged the slot is visible to all
+// XCDs.  Returns (to every thread) whether this workgroup is the last of `expected` to arrive; the last
+// one also puts the counter back to zero for the next call.
+template <int LPE>
+__device__ __forceinline__ bool arrive(const SideArgs& s, const int idx, const int expected, BlockLds<LPE>& lds) {
+    const int tid = threadIdx.x;
+    if (tid < kWave) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (tid == 0) {
+            const int old = __hip_atomic_fetch_add(&s.counters[idx], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int last = (old == expected - 1) ? 1 : 0;
+            if (last) __hip_atomic_store(&s.counters[idx], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            lds.last = last;
+        }
+    }
+    __syncthreads();
+    const bool last = lds.last != 0;
+    __syncthreads();          // lds.last may be written again by the next arrival
+    return last;
+}
+
 // Workgroup item: one segment (<= kBlockSeg edges) of a long row.  The lane groups
 // of the 4 waves each walk a share of the segment, LDS adds them in a fixed order.
 // If the row has several segments each workgroup stores its sums in a partial
 // slot, and the workgroup that arrives last adds the slots in slot order and
 // writes the row - no second launch, no floating-point atomics, and the order of
-// the additions does not depend on which workgroup is last.
+// the additions does not depend on which workgroup is last.  A row with more than
+// kCombineFan segments does this in two levels: the last arriver of every run of
+// kCombineFan consecutive slots adds them into a group slot, and the last group adds the
+// group slots - the sums of a row with hundreds of segments are formed while the
+// launch is under way, not by one workgroup at its end.
 template <typename T, int LPE, int LPH, int MODE, int HASB, bool TILES>
 __device__ __forceinline__ void block_item(const Common& c, const SideArgs& s, const int item,
                                            BlockLds<LPE>& lds) {
@@ -485,10 +567,8 @@ __device__ __forceinline__ void block_item(const Common& c, const SideArgs& s, c
     constexpr int G = LPE * S;
     constexpr int IPW = kWave / G;
     constexpr int NG = (kBlock / kWave) * IPW;    // lane groups in the workgroup
-    constexpr int H = LPE / LPH;
     constexpr int HD = LPE * 8;
     constexpr int STRIDE = BlockLds<LPE>::STRIDE;
-    constexpr int PS = part_stride<MODE, HD, H>();
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int sub = lane / G, gl = lane % G;
@@ -524,131 +604,98 @@ __device__ __forceinline__ void block_item(const Common& c, const SideArgs& s, c
             }
             if (MODE == MODE_FWD) acc.z += r[2 * HD + tid];
         }
-        if (it.part < 0) {
-            write_row<T, LPE, LPH, MODE, TILES>(c, s, it.row, tid, acc);
-        } else {
-            float* p = s.part + (int64_t)it.part * PS;
-            store8_dev(p + tid * 8, acc.a0);
-            if (MODE == MODE_BWD_SRC) store8_dev(p + HD + tid * 8, acc.a1);
-            if (MODE == MODE_FWD && tid % LPH == 0) store_dev(p + HD + tid / LPH, acc.z);
-        }
+        if (it.part < 0) write_row<T, LPE, LPH, MODE, TILES>(c, s, it.row, tid, acc);
+        else store_slot<LPE, LPH, MODE>(s, it.part, acc);
     }
     if (it.part < 0) return;   // uniform over the workgroup
+    __syncthreads();           // the LDS sums are read; sum_slots writes them again
 
-    // arrival: the partial slot is published before the counter moves.  Wave 0 holds every writer
-    // of the slot; once its device-scope stores are acknowledged the slot is visible to all XCDs.
     const int sidx = s.part2split[it.part];
     const int p0 = s.split_off[sidx], p1 = s.split_off[sidx + 1];
-    if (tid < kWave) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if (tid == 0) {
-            const int old = __hip_atomic_fetch_add(&s.counters[sidx], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            lds.last = (old == p1 - p0 - 1) ? 1 : 0;
-        }
-    }
-    __syncthreads();
-    if (!lds.last) return;
-    // last arriver: NGROUP groups of LPE threads add slots p0 + grp2, p0 + grp2 + NGROUP, ...
-    constexpr int NGROUP = BlockLds<LPE>::NGROUP;
-    const int grp2 = tid / LPE, el2 = tid % LPE;
-    {
-        float a0[8], a1[8], z = 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) { a0[i] = 0.f; a1[i] = 0.f; }
-        for (int p = p0 + grp2; p < p1; p += NGROUP) {
-            const float* src = s.part + (int64_t)p * PS;
-            float t0[8], t1[8];
-            load8_dev(src + el2 * 8, t0);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) a0[i] += t0[i];
-            if (MODE == MODE_BWD_SRC) {
-                load8_dev(src + HD + el2 * 8, t1);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) a1[i] += t1[i];
-            }
-            if (MODE == MODE_FWD) z += load_dev(src + HD + el2 / LPH);
-        }
-        float* r = lds.red + grp2 * STRIDE;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            r[el2 * 8 + i] = a0[i];
-            if (MODE == MODE_BWD_SRC) r[HD + el2 * 8 + i] = a1[i];
-        }
-        if (MODE == MODE_FWD) r[2 * HD + el2] = z;
-    }
-    __syncthreads();
-    if (tid < LPE) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) { acc.a0[i] = 0.f; acc.a1[i] = 0.f; }
-        acc.z = 0.f;
-        for (int gI = 0; gI < NGROUP; ++gI) {
-            const float* r = lds.red + gI * STRIDE;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                acc.a0[i] += r[tid * 8 + i];
-                if (MODE == MODE_BWD_SRC) acc.a1[i] += r[HD + tid * 8 + i];
-            }
-            if (MODE == MODE_FWD) acc.z += r[2 * HD + tid];
-        }
-        write_row<T, LPE, LPH, MODE, TILES>(c, s, it.row, tid, acc);
-        if (tid == 0) s.counters[sidx] = 0;   // ready for the next call
-    }
-}
-
-// Forward: workgroup items of the destination view first (longest work first),
-// then its wave items.
-template <typename T, int LPE, int LPH, int HASB, bool TILES>
-__global__ __launch_bounds__(kBlock) void k_attn_fwd(const Common c, const SideArgs s, const int items_pad) {
-    __shared__ BlockLds<LPE> lds;
-    const int b = blockIdx.x;
-    if (b < items_pad) {
-        // workgroup items are in row order; XCD x (= workgroup id mod 8) takes the x-th contiguous
-        // run of them (runs of equal edge count), so the rows of a cluster share an L2
-        if (b < s.spread_pad) {
-            if (b < s.n_spread) block_item<T, LPE, LPH, MODE_FWD, HASB, TILES>(c, s, b, lds);
-        } else {
-            const int bb = b - s.spread_pad;
-            const int it = s.blk_chunk[bb & 7] + (bb >> 3);
-            if (it < s.blk_chunk[(bb & 7) + 1]) block_item<T, LPE, LPH, MODE_FWD, HASB, TILES>(c, s, it, lds);
-        }
+    const int n = p1 - p0;
+    if (n <= kCombineFan) {
+        if (!arrive<LPE>(s, sidx, n, lds)) return;
+        sum_slots<LPE, LPH, MODE>(s, p0, n, lds, acc);
     } else {
-        wave_block<T, LPE, LPH, MODE_FWD, HASB, TILES>(c, s, b - items_pad);
+        const int g0 = s.split_grp[sidx];                 // first group of this row (groups are numbered over the view)
+        const int ngrp = (n + kCombineFan - 1) / kCombineFan;
+        const int g = (it.part - p0) / kCombineFan;
+        const int gfirst = p0 + g * kCombineFan;
+        const int gcount = min(kCombineFan, p1 - gfirst);
+        if (!arrive<LPE>(s, s.n_split + g0 + g, gcount, lds)) return;
+        sum_slots<LPE, LPH, MODE>(s, gfirst, gcount, lds, acc);
+        if (tid < LPE) store_slot<LPE, LPH, MODE>(s, s.n_parts + g0 + g, acc);
+        __syncthreads();
+        if (!arrive<LPE>(s, sidx, ngrp, lds)) return;
+        sum_slots<LPE, LPH, MODE>(s, s.n_parts + g0, ngrp, lds, acc);
     }
+    if (tid < LPE) write_row<T, LPE, LPH, MODE, TILES>(c, s, it.row, tid, acc);
 }
 
-// Backward: both views in one launch (they are independent once nd is known):
-// workgroup items of the destination view, workgroup items of the source view,
-// wave items of the destination view, wave items of the source view.
+#ifdef TGT_TRACE
+// Experiments only (-DTGT_TRACE): every wave records when it ran and where, 4 x uint64 per wave at
+// g_trace[4 * (4 * workgroup + wave)]: start, end (100 MHz clock), (XCC id << 32 | HW id), descriptor code.
+__device__ uint64_t* g_trace = nullptr;
+struct TraceScope {
+    uint64_t t0; uint32_t code; int idx;
+    __device__ TraceScope(uint32_t c) : t0(wall_clock64()), code(c), idx(blockIdx.x * 4 + (threadIdx.x >> 6)) {}
+    __device__ ~TraceScope() {
+        if (g_trace && (threadIdx.x & 63) == 0) {
+            uint64_t* p = g_trace + 4 * (int64_t)idx;
+            p[0] = t0; p[1] = wall_clock64();
+            p[2] = ((uint64_t)__builtin_amdgcn_s_getreg((3 << 11) | 20) << 32) | (uint32_t)__builtin_amdgcn_s_getreg((31 << 11) | 4);
+            p[3] = code;
+        }
+    }
+};
+#define TGT_TRACE_SCOPE(code) TraceScope trace_scope_(code)
+#else
+#define TGT_TRACE_SCOPE(code)
+#endif
+
+// Forward.  Workgroup b does what descriptors 4b .. 4b+3 say: one workgroup item, or four waves of wave
+// items.  Which rows meet in which workgroup, on which XCD and when is the plan's business.
+template <typename T, int LPE, int LPH, int HASB, bool TILES>
+__global__ __launch_bounds__(kBlock) void k_attn_fwd(const Common c, const SideArgs s,
+                                                     const WaveDesc* __restrict__ desc) {
+    __shared__ BlockLds<LPE> lds;
+    const WaveDesc* d = desc + (int64_t)blockIdx.x * (kBlock / kWave);
+    const uint32_t code0 = d[0].code;
+    if ((code0 & 7u) == kDescBlock) {          // uniform over the workgroup
+        TGT_TRACE_SCOPE(code0);
+        block_item<T, LPE, LPH, MODE_FWD, HASB, TILES>(c, s, d[0].first, lds);
+        return;
+    }
+    const int wave = threadIdx.x >> 6;
+    const uint32_t code = __builtin_amdgcn_readfirstlane(d[wave].code);
+    const int first = __builtin_amdgcn_readfirstlane(d[wave].first);
+    if ((code & 7u) == kDescNone) return;
+    TGT_TRACE_SCOPE(code);
+    wave_dispatch<T, LPE, LPH, MODE_FWD, HASB, TILES>(c, s, code & 7u, first, code >> 8);
+}
+
+// Backward: both views in one launch (they are independent once nd is known); the descriptor tells the view.
 template <typename T, int LPE, int LPH, int HASB, bool TILES>
 __global__ __launch_bounds__(kBlock, 4) void k_attn_bwd(const Common c, const SideArgs sd, const SideArgs ss,
-                                                     const int pad_d, const int pad_s) {
+                                                        const WaveDesc* __restrict__ desc) {
     __shared__ BlockLds<LPE> lds;
-    int b = blockIdx.x;
-    if (b < pad_d) {
-        if (b < sd.spread_pad) {
-            if (b < sd.n_spread) block_item<T, LPE, LPH, MODE_BWD_DST, (HASB == 3 ? 2 : HASB), TILES>(c, sd, b, lds);
-        } else {
-            const int bb = b - sd.spread_pad;
-            const int it = sd.blk_chunk[bb & 7] + (bb >> 3);
-            if (it < sd.blk_chunk[(bb & 7) + 1]) block_item<T, LPE, LPH, MODE_BWD_DST, (HASB == 3 ? 2 : HASB), TILES>(c, sd, it, lds);
-        }
+    constexpr int HB_D = HASB == 3 ? 2 : HASB;
+    constexpr int HB_S = HASB == 3 ? 2 : (HASB ? 1 : 0);
+    const WaveDesc* d = desc + (int64_t)blockIdx.x * (kBlock / kWave);
+    const uint32_t code0 = d[0].code;
+    if ((code0 & 7u) == kDescBlock) {          // uniform over the workgroup
+        TGT_TRACE_SCOPE(code0);
+        if (code0 & kDescSrcSide) block_item<T, LPE, LPH, MODE_BWD_SRC, HB_S, TILES>(c, ss, d[0].first, lds);
+        else block_item<T, LPE, LPH, MODE_BWD_DST, HB_D, TILES>(c, sd, d[0].first, lds);
         return;
     }
-    b -= pad_d;
-    if (b < pad_s) {
-        if (b < ss.spread_pad) {
-            if (b < ss.n_spread) block_item<T, LPE, LPH, MODE_BWD_SRC, (HASB == 3 ? 2 : (HASB ? 1 : 0)), TILES>(c, ss, b, lds);
-        } else {
-            const int bb = b - ss.spread_pad;
-            const int it = ss.blk_chunk[bb & 7] + (bb >> 3);
-            if (it < ss.blk_chunk[(bb & 7) + 1]) block_item<T, LPE, LPH, MODE_BWD_SRC, (HASB == 3 ? 2 : (HASB ? 1 : 0)), TILES>(c, ss, it, lds);
-        }
-        return;
-    }
-    b -= pad_s;
-    if (b < sd.n_wave_blocks) { wave_block<T, LPE, LPH, MODE_BWD_DST, (HASB == 3 ? 2 : HASB), TILES>(c, sd, b); return; }
-    b -= sd.n_wave_blocks;
-    wave_block<T, LPE, LPH, MODE_BWD_SRC, (HASB == 3 ? 2 : (HASB ? 1 : 0)), TILES>(c, ss, b);
+    const int wave = threadIdx.x >> 6;
+    const uint32_t code = __builtin_amdgcn_readfirstlane(d[wave].code);
+    const int first = __builtin_amdgcn_readfirstlane(d[wave].first);
+    if ((code & 7u) == kDescNone) return;
+    TGT_TRACE_SCOPE(code);
+    if (code & kDescSrcSide) wave_dispatch<T, LPE, LPH, MODE_BWD_SRC, HB_S, TILES>(c, ss, code & 7u, first, code >> 8);
+    else wave_dispatch<T, LPE, LPH, MODE_BWD_DST, HB_D, TILES>(c, sd, code & 7u, first, code >> 8);
 }
 
 // Per-node side vector of the backward: nd[i,h] = (1 / (Z[i,h] + eps), sum_c dout[i,h,c] out[i,h,c]).
@@ -688,40 +735,20 @@ static WsLayout ws_layout(const tgt_plan* p, int H, int d) {
     const int64_t HD = (int64_t)H * d;
     WsLayout w;
     w.nd = 0;
+    const int64_t slots_d = (int64_t)p->dst.n_parts + p->dst.n_groups, slots_s = (int64_t)p->src.n_parts + p->src.n_groups;
+    const int64_t cnt_d = (int64_t)p->dst.n_split + p->dst.n_groups, cnt_s = (int64_t)p->src.n_split + p->src.n_groups;
     w.fwd_part = align256(p->N * H * 8);
-    w.dq_part = w.fwd_part + align256((int64_t)p->dst.n_parts * (HD + H) * 4);
-    w.dkv_part = w.dq_part + align256((int64_t)p->dst.n_parts * HD * 4);
-    w.counters = w.dkv_part + align256((int64_t)p->src.n_parts * 2 * HD * 4);
-    w.total = w.counters + align256(((int64_t)2 * p->dst.n_split + p->src.n_split + 1) * 4);
+    w.dq_part = w.fwd_part + align256(slots_d * (HD + H) * 4);
+    w.dkv_part = w.dq_part + align256(slots_d * HD * 4);
+    w.counters = w.dkv_part + align256(slots_s * 2 * HD * 4);
+    w.total = w.counters + align256((2 * cnt_d + cnt_s + 1) * 4);
     return w;
 }
 
-static void fill_side(SideArgs& a, const Side& s, int lpe) {
+static void fill_side(SideArgs& a, const Side& s) {
     a.items = s.items; a.col = s.col; a.eid = s.eid;
-    a.split_off = s.split_off; a.part2split = s.part2split;
-    a.n_block_items = s.n_block_items;
-    for (int x = 0; x < 9; ++x) a.blk_chunk[x] = s.blk_chunk[x];
-    a.n_spread = s.n_spread_items;
-    a.spread_pad = (s.n_spread_items + 7) & ~7;
-    int slots = 0;
-    for (int c = 0; c < kNumClass; ++c) {
-        a.class_off[c] = s.class_off[c];
-        const int ipw = kWave / (lpe * slots_for_class(lpe, c));
-        const int n = s.class_off[c + 1] - s.class_off[c];
-        a.nwaves[c] = (n + ipw - 1) / ipw;
-        a.chunk[c] = (a.nwaves[c] + 7) / 8;
-        a.voff[c] = slots;
-        slots += a.chunk[c];
-    }
-    a.class_off[kNumClass] = s.class_off[kNumClass];
-    a.voff[kNumClass] = slots;
-    a.n_wave_blocks = 8 * ((slots + (kBlock / kWave) - 1) / (kBlock / kWave));
-}
-// workgroups needed so that every XCD can walk its run of workgroup items
-static inline int blk_grid(const Side& s) {
-    int m = 0;
-    for (int x = 0; x < 8; ++x) m = std::max(m, s.blk_chunk[x + 1] - s.blk_chunk[x]);
-    return ((s.n_spread_items + 7) & ~7) + 8 * m;
+    a.split_off = s.split_off; a.part2split = s.part2split; a.split_grp = s.split_grp;
+    a.n_split = s.n_split; a.n_parts = s.n_parts;
 }
 // shapes for which the variant that adds the block path's tile sums is compiled
 template <int LPE, int LPH>
@@ -753,14 +780,16 @@ static int run_fwd(const Call& c) {
     cm.bias_sh = (c.bias_mode & 0xf) == TGT_BIAS_EDGE_HEAD ? 1 : 0;
     cm.inv_scale = 1.0f / sqrtf((float)c.d);
     SideArgs a{};
-    fill_side(a, c.plan->dst, LPE);
+    fill_side(a, c.plan->dst);
+    const Schedule* sch = plan_schedule(c.plan, LPE, c.st);
+    if (!sch) return TGT_ERR_HIP;
+    const WaveDesc* desc = sch->fwd;
     if (c.bias_mode & TGT_BIAS_PLAN_ORDER) a.eid = nullptr;             // bias rows in destination-sorted order
     a.out0 = c.o_out; a.out1 = nullptr; a.Z = c.o_Z;
     if (c.init) { a.init0 = c.init->acc; a.initZ = c.init->Z; a.cover = c.init->cover_dst; }
     a.part = reinterpret_cast<float*>(c.ws + L.fwd_part);
     a.counters = reinterpret_cast<int32_t*>(c.ws + L.counters);
-    const int items_pad = blk_grid(c.plan->dst);
-    const int nb = items_pad + a.n_wave_blocks;
+    const int nb = sch->fwd_blocks;
     if (nb > 0) {
         KernelTimer t(KS_FWD, c.st);
         const bool hb = c.bias_mode != TGT_BIAS_NONE;
@@ -770,18 +799,18 @@ static int run_fwd(const Call& c) {
         }
         if (c.init != nullptr) {
             if constexpr (kTilesShape<LPE, LPH>) {
-                if (hb) hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, 1, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
-                else hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, 0, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
+                if (hb) hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, 1, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, desc);
+                else hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, 0, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, desc);
             } else {
                 set_error("block attention: no kernel for this (H, d)");
                 return TGT_ERR_UNSUPPORTED;
             }
         } else if (hb && (c.bias_mode & TGT_BIAS_PLAN_ORDER)) {
-            hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, 2, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
+            hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, 2, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, desc);
         } else if (hb) {
-            hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, 1, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
+            hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, 1, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, desc);
         } else {
-            hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, 0, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, items_pad);
+            hipLaunchKernelGGL((k_attn_fwd<T, LPE, LPH, 0, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, a, desc);
         }
     }
     TGT_HIP_CHECK(hipGetLastError());
@@ -815,21 +844,23 @@ static int run_bwd(const Call& c) {
     cm.inv_scale = 1.0f / sqrtf((float)c.d);
     int32_t* counters = reinterpret_cast<int32_t*>(c.ws + L.counters);
     SideArgs sd{}, ss{};
-    fill_side(sd, c.plan->dst, LPE);
+    fill_side(sd, c.plan->dst);
+    const Schedule* sch = plan_schedule(c.plan, LPE, c.st);
+    if (!sch) return TGT_ERR_HIP;
+    const WaveDesc* desc = sch->bwd;
     if (c.bias_mode & TGT_BIAS_PLAN_ORDER) sd.eid = nullptr;
     sd.out0 = c.dq; sd.out1 = c.dbias; sd.Z = nullptr;
     if (c.init) { sd.init0 = c.init->dq; sd.cover = c.init->cover_dst; }
     sd.part = reinterpret_cast<float*>(c.ws + L.dq_part);
-    sd.counters = counters + c.plan->dst.n_split;
-    fill_side(ss, c.plan->src, LPE);
+    sd.counters = counters + c.plan->dst.n_split + c.plan->dst.n_groups;
+    fill_side(ss, c.plan->src);
     if (c.bias_mode & TGT_BIAS_PLAN_ORDER) ss.eid = c.plan->src.pos;    // source-sorted -> destination-sorted position
     if (c.bias_mode & TGT_BIAS_BOTH_ORDERS) ss.eid = nullptr;           // its own source-sorted copy
     ss.out0 = c.dk; ss.out1 = c.dv; ss.Z = nullptr;
     if (c.init) { ss.init0 = c.init->dk; ss.init1 = c.init->dv; ss.cover = c.init->cover_src; }
     ss.part = reinterpret_cast<float*>(c.ws + L.dkv_part);
-    ss.counters = counters + 2 * c.plan->dst.n_split;
-    const int pad_d = blk_grid(c.plan->dst), pad_s = blk_grid(c.plan->src);
-    const int nb = pad_d + pad_s + sd.n_wave_blocks + ss.n_wave_blocks;
+    ss.counters = counters + 2 * (c.plan->dst.n_split + c.plan->dst.n_groups);
+    const int nb = sch->bwd_blocks;
     if (nb > 0) {
         KernelTimer t(KS_BWD, c.st);
         const bool hb = c.bias_mode != TGT_BIAS_NONE;
@@ -839,20 +870,20 @@ static int run_bwd(const Call& c) {
         }
         if (c.init != nullptr) {
             if constexpr (kTilesShape<LPE, LPH>) {
-                if (hb) hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, 1, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
-                else hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, 0, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
+                if (hb) hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, 1, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, desc);
+                else hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, 0, true>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, desc);
             } else {
                 set_error("block attention: no kernel for this (H, d)");
                 return TGT_ERR_UNSUPPORTED;
             }
         } else if (hb && (c.bias_mode & TGT_BIAS_BOTH_ORDERS)) {
-            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, 3, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
+            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, 3, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, desc);
         } else if (hb && (c.bias_mode & TGT_BIAS_PLAN_ORDER)) {
-            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, 2, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
+            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, 2, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, desc);
         } else if (hb) {
-            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, 1, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
+            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, 1, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, desc);
         } else {
-            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, 0, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, pad_d, pad_s);
+            hipLaunchKernelGGL((k_attn_bwd<T, LPE, LPH, 0, false>), dim3(nb), dim3(kBlock), 0, c.st, cm, sd, ss, desc);
         }
     }
     TGT_HIP_CHECK(hipGetLastError());
@@ -1011,6 +1042,16 @@ const float2* sparse_attn_nd_ptr(void* d_workspace) { return reinterpret_cast<co
 
 #if !defined(TGT_SPARSE_PART) || TGT_SPARSE_PART == 0
 extern "C" {
+
+#ifdef TGT_TRACE
+int tgt_debug_trace(uint64_t* d_buf) {
+    return hipMemcpyToSymbol(HIP_SYMBOL(tgt::g_trace), &d_buf, sizeof(d_buf)) == hipSuccess ? 0 : -4;
+}
+int tgt_debug_grid(const tgt_plan_t* plan, int lpe, int bwd) {
+    const tgt::Schedule* s = tgt::plan_schedule(plan, lpe, nullptr);
+    return s ? (bwd ? s->bwd_blocks : s->fwd_blocks) : -1;
+}
+#endif
 
 int64_t tgt_sparse_attn_workspace_bytes(const tgt_plan_t* plan, int H, int d) {
     if (!plan || H < 1 || d < 1) return -1;
