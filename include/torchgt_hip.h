@@ -80,6 +80,12 @@ const char*  tgt_last_error(void);
 int tgt_plan_create(const int64_t* d_src, const int64_t* d_dst, int64_t E, int64_t N,
                     void* stream, tgt_plan_t** out_plan);
 int tgt_plan_destroy(tgt_plan_t* plan);
+/* The attention kernels of a (H, d) shape read launch descriptors that are made on the first call
+ * with that shape (a few small allocations, copies and one synchronisation of the stream, once per
+ * plan and H * d / 8); tgt_plan_create makes those of H * d = 64 (the reference's hidden size 64
+ * with 8 x 8 or 4 x 16 heads).  Call this for any other shape before capturing attention calls
+ * into a HIP graph.  Later calls with the same shape return at once. */
+int tgt_plan_prepare(tgt_plan_t* plan, int H, int d, void* stream);
 
 /* info[0]=N, [1]=E, [2]=#schedule items (dst side), [3]=#split rows (dst),
  * [4]=#partial segments (dst), [5..7]= the same for the src side,
@@ -122,7 +128,8 @@ int tgt_plan_sort_rows(const tgt_plan_t* plan, const void* d_in, int row_bytes, 
  * sums of split rows, their arrival counters and per-node side vectors; depends
  * on the plan and H*d.  The caller ZEROES it once after allocating it; after that
  * only this library writes it (the counters return to zero at the end of every
- * call).  Calls that share a workspace must be ordered on one stream. */
+ * call).  Calls that share a workspace must be ordered on one stream.  The attention
+ * calls themselves only launch kernels (see tgt_plan_prepare for the one exception). */
 int64_t tgt_sparse_attn_workspace_bytes(const tgt_plan_t* plan, int H, int d);
 
 /* Forward of CoreAttention.sparse_attention (attn_module.py:133-189) /
@@ -138,6 +145,22 @@ int tgt_sparse_attn_fwd(const tgt_plan_t* plan,
                         int H, int d, int dtype,
                         void* d_out, float* d_Z,
                         void* d_workspace, int64_t workspace_bytes, void* stream);
+
+/* The same forward for callers that cannot allocate device memory or pass a workspace (code under
+ * HIP-graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in
+ * the reference.  The partial sums and arrival counters of split rows live in a fixed array of
+ * 4 MiB per GPU inside the library (held until the process ends); a graph whose split rows need
+ * more is refused with TGT_ERR_WORKSPACE (a few thousand segments of long rows fit; use
+ * tgt_sparse_attn_fwd with a workspace beyond that).  The call allocates nothing and frees nothing:
+ * the launch descriptors of the (H, d) shape must exist already (tgt_plan_create makes those of
+ * H * d = 64; tgt_plan_prepare any other), else TGT_ERR_INVALID_ARG.  Every call on a GPU
+ * uses that GPU's one array: calls that overlap on one GPU (two streams, two threads) race.
+ * Results are bit-identical to tgt_sparse_attn_fwd. */
+int tgt_sparse_attn_fwd_noalloc(const tgt_plan_t* plan,
+                                const void* d_q, const void* d_k, const void* d_v,
+                                const void* d_bias, int bias_mode,
+                                int H, int d, int dtype,
+                                void* d_out, float* d_Z, void* stream);
 
 /* Backward of the same function (autograd in the reference).  d_dout, d_dq,
  * d_dk, d_dv: [N, H, d] dtype; d_dbias: same shape/dtype as d_bias or NULL.

@@ -37,6 +37,8 @@ SIGNATURES = {
     "tgt_plan_sort_rows": (_i32, [_vp, _vp, _i32, _vp, _i32, _vp]),
     "tgt_sparse_attn_workspace_bytes": (_i64, [_vp, _i32, _i32]),
     "tgt_sparse_attn_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _i64, _vp]),
+    "tgt_sparse_attn_fwd_noalloc": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp]),
+    "tgt_plan_prepare": (_i32, [_vp, _i32, _i32, _vp]),
     "tgt_sparse_attn_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp,
                                    _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
     "tgt_dense_attn_fwd": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp]),

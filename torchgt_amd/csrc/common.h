@@ -175,4 +175,6 @@ namespace tgt {
 // Descriptors for kernels with `lpe` lanes per edge; builds them on first use (allocates, copies and
 // synchronises `st` once per plan and shape).  nullptr on error.
 const Schedule* plan_schedule(const tgt_plan* plan, int lpe, hipStream_t st);
+// The same without building anything: nullptr if the shape has not been used or prepared yet.
+const Schedule* plan_schedule_if_ready(const tgt_plan* plan, int lpe);
 }

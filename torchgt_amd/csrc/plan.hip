@@ -413,6 +413,12 @@ int place(const std::vector<const Side*>& sides, int lpe, WaveDesc** d_out, int3
 }
 }  // namespace
 
+const Schedule* plan_schedule_if_ready(const tgt_plan* plan, int lpe) {
+    for (int idx = 0; idx < kNumLpe; ++idx)
+        if ((1 << idx) == lpe) return plan->sched[idx].ready ? &plan->sched[idx] : nullptr;
+    return nullptr;
+}
+
 const Schedule* plan_schedule(const tgt_plan* plan_c, int lpe, hipStream_t st) {
     int idx = 0;
     while (idx < kNumLpe && (1 << idx) != lpe) ++idx;

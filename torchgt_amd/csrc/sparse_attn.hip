@@ -18,6 +18,7 @@
 #include "common.h"
 #include <stdlib.h>
 #include <algorithm>
+#include <mutex>
 
 namespace tgt {
 
@@ -768,6 +769,9 @@ struct Call {
     const TileInit* init;
     bool skip_node_side;   // nd was already computed into the workspace by sparse_attn_node_side
     bool only_node_side;
+    float* fwd_part;       // forward only: partial slots and arrival counters somewhere else than in `ws`
+    int32_t* fwd_counters;
+    bool no_alloc;         // fail instead of building the launch descriptors of a shape seen for the first time
 };
 
 template <typename T, int LPE, int LPH>
@@ -781,14 +785,20 @@ static int run_fwd(const Call& c) {
     cm.inv_scale = 1.0f / sqrtf((float)c.d);
     SideArgs a{};
     fill_side(a, c.plan->dst);
-    const Schedule* sch = plan_schedule(c.plan, LPE, c.st);
-    if (!sch) return TGT_ERR_HIP;
+    const Schedule* sch = c.no_alloc ? plan_schedule_if_ready(c.plan, LPE) : plan_schedule(c.plan, LPE, c.st);
+    if (!sch) {
+        if (c.no_alloc) {
+            set_error("no launch descriptors for H*d = %d yet: call tgt_plan_prepare(plan, H, d, stream) first", LPE * 8);
+            return TGT_ERR_INVALID_ARG;
+        }
+        return TGT_ERR_HIP;
+    }
     const WaveDesc* desc = sch->fwd;
     if (c.bias_mode & TGT_BIAS_PLAN_ORDER) a.eid = nullptr;             // bias rows in destination-sorted order
     a.out0 = c.o_out; a.out1 = nullptr; a.Z = c.o_Z;
     if (c.init) { a.init0 = c.init->acc; a.initZ = c.init->Z; a.cover = c.init->cover_dst; }
-    a.part = reinterpret_cast<float*>(c.ws + L.fwd_part);
-    a.counters = reinterpret_cast<int32_t*>(c.ws + L.counters);
+    a.part = c.fwd_part ? c.fwd_part : reinterpret_cast<float*>(c.ws + L.fwd_part);
+    a.counters = c.fwd_counters ? c.fwd_counters : reinterpret_cast<int32_t*>(c.ws + L.counters);
     const int nb = sch->fwd_blocks;
     if (nb > 0) {
         KernelTimer t(KS_FWD, c.st);
@@ -962,7 +972,7 @@ static int dispatch(const Call& c, bool bwd) {
 }
 
 static int check_common(const tgt_plan* plan, const void* q, const void* k, const void* v, const void* bias,
-                        int bias_mode, int H, int d, int dtype, const void* ws, int64_t ws_bytes) {
+                        int bias_mode, int H, int d, int dtype, const void* ws, int64_t ws_bytes, bool needs_ws = true) {
     if (!plan || !q || !k || !v) { set_error("null plan or q/k/v"); return TGT_ERR_INVALID_ARG; }
     {
         const int base = bias_mode & 0xf;
@@ -981,7 +991,7 @@ static int check_common(const tgt_plan* plan, const void* q, const void* k, cons
     if (dtype != TGT_DTYPE_F32 && dtype != TGT_DTYPE_BF16) { set_error("bad dtype %d", dtype); return TGT_ERR_INVALID_ARG; }
     if (H < 1 || d < 1) { set_error("H and d must be positive"); return TGT_ERR_INVALID_ARG; }
     if (d % 8 != 0) { set_error("head dim %d is not a multiple of 8", d); return TGT_ERR_UNSUPPORTED; }
-    const int64_t need = ws_layout(plan, H, d).total;
+    const int64_t need = needs_ws ? ws_layout(plan, H, d).total : 0;
     if (need > 0 && (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255u))) {
         set_error("workspace: need %lld bytes, 256-byte aligned; got %lld", (long long)need, (long long)ws_bytes);
         return TGT_ERR_WORKSPACE;
@@ -1036,6 +1046,74 @@ int sparse_attn_node_side(const tgt_plan_t* plan, int H, int d, int dtype, const
 }
 
 const float2* sparse_attn_nd_ptr(void* d_workspace) { return reinterpret_cast<const float2*>(d_workspace); }
+
+// ---------------------------------------------------------------------------
+// forward that allocates nothing: partial slots and arrival counters of split rows in a fixed array
+// ---------------------------------------------------------------------------
+constexpr int64_t kScratchBytes = 4ll << 20;      // per GPU, held until the process ends
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+// `scratch` is a host-side stand-in in host code, not a device address: the address of each GPU's copy
+// is looked up once per device and used from then on.
+static void* g_scratch_ptr[kMaxDevices];
+static std::mutex g_scratch_mutex;
+
+static int scratch_for_current_device(void** out) {
+    int dev = 0;
+    TGT_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) { set_error("device %d: at most %d devices", dev, kMaxDevices); return TGT_ERR_UNSUPPORTED; }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        TGT_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return TGT_OK;
+}
+
+__global__ void k_zero_i32(int32_t* __restrict__ p, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+int sparse_attn_fwd_noalloc_impl(const tgt_plan_t* plan, const void* d_q, const void* d_k, const void* d_v,
+                                 const void* d_bias, int bias_mode, int H, int d, int dtype, void* d_out, float* d_Z,
+                                 void* stream) {
+    int rc = check_common(plan, d_q, d_k, d_v, d_bias, bias_mode, H, d, dtype, nullptr, 0, false);
+    if (rc) return rc;
+    if (!d_out || !d_Z) { set_error("null out or Z"); return TGT_ERR_INVALID_ARG; }
+    int dev = 0;
+    TGT_HIP_CHECK(hipGetDevice(&dev));
+    if (dev != plan->device) { set_error("the plan lives on device %d, the current device is %d", plan->device, dev); return TGT_ERR_INVALID_ARG; }
+    // scratch layout: arrival counters (rows, then groups), then the partial slots
+    const int64_t n_cnt = (int64_t)plan->dst.n_split + plan->dst.n_groups;
+    const int64_t slots = (int64_t)plan->dst.n_parts + plan->dst.n_groups;
+    const int64_t part_off = align256(n_cnt * 4);
+    const int64_t need = part_off + slots * ((int64_t)H * d + H) * 4;
+    if (need > kScratchBytes) {
+        set_error("tgt_sparse_attn_fwd_noalloc: the split rows of this graph need %lld bytes of scratch, the fixed array holds %lld; "
+                  "use tgt_sparse_attn_fwd with a workspace", (long long)need, (long long)kScratchBytes);
+        return TGT_ERR_WORKSPACE;
+    }
+    void* base = nullptr;
+    rc = scratch_for_current_device(&base);
+    if (rc) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (n_cnt > 0) {   // the array keeps what the last call left: the counters must start at zero
+        hipLaunchKernelGGL(k_zero_i32, dim3((unsigned)((n_cnt + 255) / 256)), dim3(256), 0, st,
+                           static_cast<int32_t*>(base), (int)n_cnt);
+        TGT_HIP_CHECK(hipGetLastError());
+    }
+    Call c{};
+    c.plan = plan; c.q = d_q; c.k = d_k; c.v = d_v; c.bias = d_bias; c.bias_mode = bias_mode;
+    c.H = H; c.d = d; c.o_out = d_out; c.o_Z = d_Z; c.ws = nullptr;
+    c.st = st;
+    c.fwd_counters = static_cast<int32_t*>(base);
+    c.fwd_part = reinterpret_cast<float*>(static_cast<char*>(base) + part_off);
+    c.no_alloc = true;
+    return dtype == TGT_DTYPE_F32 ? dispatch<float>(c, false) : dispatch<bf16_t>(c, false);
+}
 #endif  // part 0: dispatch and entry points
 
 }  // namespace tgt
@@ -1063,6 +1141,17 @@ int tgt_sparse_attn_fwd(const tgt_plan_t* plan, const void* d_q, const void* d_k
                         void* d_workspace, int64_t workspace_bytes, void* stream) {
     return tgt::sparse_attn_fwd_impl(plan, d_q, d_k, d_v, d_bias, bias_mode, H, d, dtype, d_out, d_Z, d_workspace,
                                      workspace_bytes, stream, nullptr);
+}
+
+int tgt_sparse_attn_fwd_noalloc(const tgt_plan_t* plan, const void* d_q, const void* d_k, const void* d_v,
+                                const void* d_bias, int bias_mode, int H, int d, int dtype, void* d_out, float* d_Z,
+                                void* stream) {
+    return tgt::sparse_attn_fwd_noalloc_impl(plan, d_q, d_k, d_v, d_bias, bias_mode, H, d, dtype, d_out, d_Z, stream);
+}
+
+int tgt_plan_prepare(tgt_plan_t* plan, int H, int d, void* stream) {
+    if (!plan || H < 1 || d < 1 || (H * d) % 8) { tgt::set_error("tgt_plan_prepare: null plan or H*d not a multiple of 8"); return TGT_ERR_INVALID_ARG; }
+    return tgt::plan_schedule(plan, H * d / 8, static_cast<hipStream_t>(stream)) ? TGT_OK : TGT_ERR_UNSUPPORTED;
 }
 
 int tgt_sparse_attn_bwd(const tgt_plan_t* plan, const void* d_q, const void* d_k, const void* d_v,
