@@ -56,6 +56,40 @@ __host__ __device__ constexpr int slots_for_class(int lpe, int cls) {
     return nat < cap ? nat : cap;
 }
 __host__ __device__ constexpr int rows_per_wave(int lpe, int cls) { return kWave / (lpe * slots_for_class(lpe, cls)); }
+// Whether the rows of a class fit one step of their slots (four edges per slot), so that a wave's record can
+// carry their edges: every class but the longest, unless the wave is too narrow for the class's slots.
+__host__ __device__ constexpr bool class_inline(int lpe, int cls) {
+    return cls >= 1 && slots_for_class(lpe, cls) * 4 >= (cls == 1 ? 32 : (cls == 2 ? 16 : (cls == 3 ? 8 : 4)));
+}
+
+// What one wave of an attention workgroup reads first: its share of the launch, complete.  Workgroup b
+// owns records 4b .. 4b+3.  `code` is a descriptor code (kind, view, number of rows).
+//   kind 5: `item` is the workgroup item (all four records of the workgroup carry it);
+//   kind 0: rows row[i] with edges [start[i], start[i] + len[i]) of the view's sorted arrays;
+//   kind 1..4: the same rows, and their edges inline: col / eid hold, for lane group g = (row i of the
+//   wave, slot s) - g = i * S + s, S = slots_for_class - the four edges s, s + S, s + 2S, s + 3S of the row
+//   at [4g, 4g + 4) (an edge past the end of the row repeats the row's last edge; 0 for an empty row).
+// One coalesced read gives a wave everything it needs to issue its gathers.
+template <int LPE>
+struct alignas(128) WaveRec {
+    static constexpr int kRows = kWave / LPE;          // most rows a wave can hold (shortest class)
+    static constexpr int kEdges = 4 * kWave / LPE;     // four edges per lane group
+    uint32_t code;
+    int32_t pad[3];
+    Item item;
+    int32_t row[kRows], start[kRows], len[kRows];
+    int32_t col[kEdges], eid[kEdges];
+};
+// the same layout for code that takes the shape at run time (the builder): offsets in int32 units
+struct WaveRecLayout {
+    int rows, edges, off_row, off_start, off_len, off_col, off_eid, stride;
+    explicit WaveRecLayout(int lpe) {
+        rows = kWave / lpe; edges = 4 * kWave / lpe;
+        off_row = 8; off_start = off_row + rows; off_len = off_start + rows; off_col = off_len + rows;
+        off_eid = off_col + edges;
+        stride = (off_eid + edges + 31) / 32 * 32;
+    }
+};
 
 // One sorted view of the edge list plus its row schedule.
 struct Side {
@@ -79,11 +113,11 @@ struct Side {
     std::vector<uint8_t> block_spread;     // [n_block_items] 1: segment of a row with more than kSpreadSegs segments
 };
 
-// Launch descriptors of one kernel shape (lanes per edge): forward (destination view) and backward
+// Wave records of one kernel shape (lanes per edge): forward (destination view) and backward
 // (both views, window by window).
 struct Schedule {
-    WaveDesc* fwd = nullptr;
-    WaveDesc* bwd = nullptr;
+    void* fwd = nullptr;    // WaveRec<lpe> [4 * fwd_blocks]
+    void* bwd = nullptr;
     int32_t fwd_blocks = 0, bwd_blocks = 0;
     bool ready = false;
 };

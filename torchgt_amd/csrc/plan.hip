@@ -143,6 +143,53 @@ __global__ void k_gather_i32(const int32_t* __restrict__ col, const int32_t* __r
     if (i < n) out[i] = col[idx[i]];
 }
 
+// One workgroup of 64 threads writes one wave record from its descriptor (layout: WaveRec in common.h).
+__global__ __launch_bounds__(64) void k_build_records(const WaveDesc* __restrict__ desc, const Item* __restrict__ items_d,
+                                                      const Item* __restrict__ items_s, const int32_t* __restrict__ col_d,
+                                                      const int32_t* __restrict__ eid_d, const int32_t* __restrict__ col_s,
+                                                      const int32_t* __restrict__ eid_s, WaveRecLayout L, int lpe,
+                                                      int32_t* __restrict__ recs) {
+    const WaveDesc d = desc[blockIdx.x];
+    int32_t* out = recs + (int64_t)blockIdx.x * L.stride;
+    const int t = threadIdx.x;
+    const uint32_t kind = d.code & 7u;
+    const bool src = (d.code & kDescSrcSide) != 0;
+    const int count = (int)(d.code >> 8);
+    const Item* items = src ? items_s : items_d;
+    const int32_t* col = src ? col_s : col_d;
+    const int32_t* eid = src ? eid_s : eid_d;
+    if (t == 0) out[0] = (int32_t)d.code;
+    if (kind == kDescNone) return;
+    if (kind == kDescBlock) {
+        if (t == 0) {
+            const Item it = items[d.first];
+            out[4] = it.row; out[5] = it.start; out[6] = it.len; out[7] = it.part;
+        }
+        return;
+    }
+    if (t < count) {
+        const Item it = items[d.first + t];
+        out[L.off_row + t] = it.row;
+        out[L.off_start + t] = it.start;
+        out[L.off_len + t] = it.len;
+    }
+    if (!class_inline(lpe, (int)kind)) return;
+    const int S = slots_for_class(lpe, (int)kind);
+    const int groups = kWave / lpe;
+    if (t < groups) {
+        const int i = t / S, sl = t % S;
+        if (i < count) {
+            const Item it = items[d.first + i];
+            for (int u = 0; u < 4; ++u) {
+                const int e = sl + u * S;
+                const int ec = e < it.len ? e : it.len - 1;
+                out[L.off_col + 4 * t + u] = it.len > 0 ? col[it.start + ec] : 0;
+                out[L.off_eid + 4 * t + u] = it.len > 0 ? eid[it.start + ec] : 0;
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------
 // host helpers
 // ---------------------------------------------------------------------------
@@ -336,7 +383,7 @@ void append_side(std::vector<WaveDesc>& waves, float& cost, const Side& s, int w
 
 // descriptors of all windows -> block order.  XCD x gets a contiguous range of windows; it first walks the
 // heavy share of all its windows (long work first keeps the end of the launch short), then window by window.
-int place(const std::vector<const Side*>& sides, int lpe, WaveDesc** d_out, int32_t* n_blocks, hipStream_t st) {
+int place(const std::vector<const Side*>& sides, int lpe, void** d_out, int32_t* n_blocks, hipStream_t st) {
     const int nwin = sides[0]->n_windows;
     const bool heavy_first = env_int("TGT_HEAVY_FIRST", 1) == 1;
     std::vector<std::vector<std::vector<int32_t>>> homed(sides.size());
@@ -405,10 +452,23 @@ int place(const std::vector<const Side*>& sides, int lpe, WaveDesc** d_out, int3
     for (int x = 0; x < 8; ++x)
         for (size_t b = 0; b < xw[x].size() / 4; ++b)
             for (int k = 0; k < 4; ++k) placed[(b * 8 + x) * 4 + k] = xw[x][b * 4 + k];
-    TGT_HIP_CHECK(hipMalloc((void**)d_out, sizeof(WaveDesc) * placed.size()));
-    TGT_HIP_CHECK(hipMemcpyAsync(*d_out, placed.data(), sizeof(WaveDesc) * placed.size(), hipMemcpyHostToDevice, st));
-    TGT_HIP_CHECK(hipStreamSynchronize(st));
+    // descriptors -> records, on the device (the edge lists never visit the host)
+    const WaveRecLayout L(lpe);
+    const size_t n_rec = nb * 4;
     *n_blocks = (int32_t)nb;
+    if (n_rec == 0) return TGT_OK;
+    DevBuf desc_d;
+    TGT_HIP_CHECK(desc_d.alloc(sizeof(WaveDesc) * n_rec));
+    TGT_HIP_CHECK(hipMemcpyAsync(desc_d.p, placed.data(), sizeof(WaveDesc) * n_rec, hipMemcpyHostToDevice, st));
+    const size_t bytes = n_rec * (size_t)L.stride * sizeof(int32_t);
+    TGT_HIP_CHECK(hipMalloc(d_out, bytes));
+    TGT_HIP_CHECK(hipMemsetAsync(*d_out, 0, bytes, st));
+    const Side* sd = sides[0];
+    const Side* ss = sides.size() > 1 ? sides[1] : sides[0];
+    hipLaunchKernelGGL(k_build_records, dim3((unsigned)n_rec), dim3(64), 0, st, desc_d.as<WaveDesc>(), sd->items, ss->items,
+                       sd->col, sd->eid, ss->col, ss->eid, L, lpe, static_cast<int32_t*>(*d_out));
+    TGT_HIP_CHECK(hipGetLastError());
+    TGT_HIP_CHECK(hipStreamSynchronize(st));    // the descriptors are freed on return
     return TGT_OK;
 }
 }  // namespace

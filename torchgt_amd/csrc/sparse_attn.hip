@@ -170,6 +170,7 @@ struct SideArgs {
     const int32_t* split_off;
     const int32_t* part2split;
     const int32_t* split_grp;     // first combine group of each split row (rows with more than kCombineFan segments have groups)
+    int32_t eid_is_map;           // `eid` is not the caller's edge ids (which the wave records hold too) but another map
     int32_t n_split, n_parts;     // group counters follow the n_split row counters, group slots the n_parts segment slots
     void* out0;           // fwd: out      bwd_dst: dq     bwd_src: dk
     void* out1;           // fwd: -        bwd_dst: dbias  bwd_src: dv
@@ -196,14 +197,53 @@ __host__ __device__ constexpr int part_stride() {
     return MODE == MODE_FWD ? HD + H : (MODE == MODE_BWD_DST ? HD : 2 * HD);
 }
 
-// Walks `len` edges starting at sorted position `start` of node `row` with S edge
-// slots (this lane is slot `slot`, element chunk `el`).  On return every lane of
-// the S*LPE-lane group holds the sums over all S slots.
-template <typename T, int LPE, int LPH, int S, int MODE, int HASB>
-__device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, const int row, const int start,
-                                           const int len, const int slot, const int el, const bool valid,
-                                           Acc& acc) {
-    constexpr int G = LPE * S;
+// What a lane group keeps of its own row while it walks the row's edges.
+template <typename T>
+struct RowRegs {
+    Raw8<T> r0, r1;      // as loaded (only dot products use them): fwd q | bwd_dst q, g | bwd_src k, v
+    float rz, Dh;        // bwd_dst: 1 / (Z + eps) and dout . out of the row's head
+};
+
+template <typename T, int LPE, int LPH, int MODE>
+__device__ __forceinline__ void load_row(const Common& c, const int row, const int el, const bool valid,
+                                         RowRegs<T>& rr, Acc& acc) {
+    constexpr int H = LPE / LPH;
+    constexpr int HD = LPE * 8;
+    const T* __restrict__ Q = static_cast<const T*>(c.q);
+    const T* __restrict__ K = static_cast<const T*>(c.k);
+    const T* __restrict__ V = static_cast<const T*>(c.v);
+    const T* __restrict__ Gd = static_cast<const T*>(c.g);
+    const int64_t row_off = (int64_t)row * HD + el * 8;
+    rr.rz = 0.f; rr.Dh = 0.f;
+    zero_raw(rr.r0); zero_raw(rr.r1);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { acc.a0[i] = 0.f; acc.a1[i] = 0.f; }
+    acc.z = 0.f;
+    if (valid) {
+        if (MODE == MODE_FWD) {
+            load_raw(Q + row_off, rr.r0);
+        } else if (MODE == MODE_BWD_DST) {
+            load_raw(Q + row_off, rr.r0);
+            load_raw(Gd + row_off, rr.r1);
+            const float2 nd = c.nd[(int64_t)row * H + el / LPH];
+            rr.rz = nd.x; rr.Dh = nd.y;
+        } else {
+            load_raw(K + row_off, rr.r0);
+            load_raw(V + row_off, rr.r1);
+        }
+    }
+}
+
+// kUnroll edges of one slot: nb[u] = the other endpoint, ed[u] = the row of the bias / dbias arrays, ok[u] =
+// whether the edge exists.  All gathers of the step are issued before anything is used.  For 4-byte
+// elements the lanes of a missing edge load nothing; for 2-byte elements every lane loads (a missing edge
+// must then name a valid node and bias row - callers repeat the row's last edge - and only the
+// arithmetic is skipped): with no lane-dependent branch around them the loads go out back to back, and
+// the rows stay packed until they are used.
+template <typename T, int LPE, int LPH, int MODE, int HASB>
+__device__ __forceinline__ void edge_step(const Common& c, const SideArgs& s, const RowRegs<T>& rr,
+                                          const int (&nb)[kUnroll], const int (&ed)[kUnroll],
+                                          const bool (&ok)[kUnroll], const int el, Acc& acc) {
     constexpr int H = LPE / LPH;
     constexpr int HD = LPE * 8;
     const int head = el / LPH;
@@ -212,87 +252,17 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
     const T* __restrict__ V = static_cast<const T*>(c.v);
     const T* __restrict__ Gd = static_cast<const T*>(c.g);
     const T* __restrict__ B = static_cast<const T*>(MODE == MODE_BWD_SRC ? c.bias_src : c.bias);
-    const int64_t row_off = (int64_t)row * HD + el * 8;
-
-    Raw8<T> r0, r1;          // row-resident, as loaded (only dot products use them): fwd q | bwd_dst q, g | bwd_src k, v
-    float rz = 0.f, Dh = 0.f;
-    zero_raw(r0); zero_raw(r1);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) { acc.a0[i] = 0.f; acc.a1[i] = 0.f; }
-    acc.z = 0.f;
-    if (valid) {
-        if (MODE == MODE_FWD) {
-            load_raw(Q + row_off, r0);
-        } else if (MODE == MODE_BWD_DST) {
-            load_raw(Q + row_off, r0);
-            load_raw(Gd + row_off, r1);
-            const float2 nd = c.nd[(int64_t)row * H + head];
-            rz = nd.x; Dh = nd.y;
-        } else {
-            load_raw(K + row_off, r0);
-            load_raw(V + row_off, r1);
-        }
-    }
-    const int32_t* __restrict__ col = s.col + start;
-    // HASB == 2: no edge-id array, the bias rows are in this side's own sorted order (row = sorted position)
-    constexpr bool ident = HASB == 2;
-    const int32_t* __restrict__ eid = ident ? nullptr : s.eid + start;
     const int bias_se = c.bias_se, bias_sh = c.bias_sh;
     const float inv_scale = c.inv_scale;
-    const int n = valid ? len : 0;
-
-#pragma unroll 1
-    for (int e0 = slot; e0 < n; e0 += S * kUnroll) {
-        int nb[kUnroll], ed[kUnroll];
-        bool ok[kUnroll];
-        Raw8<T> g0[kUnroll], g1[kUnroll];          // gathered rows, unconverted
-        decltype(raw1(B)) braw[kUnroll];
-        float2 ndv[kUnroll];
-        if constexpr (sizeof(T) == 4) {
-            // fp32: lanes past the end of the row load nothing and hold zeros
+    Raw8<T> g0[kUnroll], g1[kUnroll];          // gathered rows, unconverted
+    decltype(raw1(B)) braw[kUnroll];
+    float2 ndv[kUnroll];
 #pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-                const int e = e0 + u * S;
-                ok[u] = e < n;
-                nb[u] = 0; ed[u] = 0;
-                if (ok[u]) {
-                    nb[u] = col[e];
-                    if (HASB) ed[u] = ident ? start + e : eid[e];
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u) {
-                braw[u] = 0;
-                ndv[u] = make_float2(0.f, 0.f);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) { g0[u].x[i] = 0.f; g1[u].x[i] = 0.f; }
-                if (ok[u]) {
-                    const int64_t o = (int64_t)nb[u] * HD + el * 8;
-                    if (MODE == MODE_BWD_SRC) {
-                        load_raw(Q + o, g0[u]);
-                        load_raw(Gd + o, g1[u]);
-                        ndv[u] = c.nd[(int64_t)nb[u] * H + head];
-                    } else {
-                        load_raw(K + o, g0[u]);
-                        load_raw(V + o, g1[u]);
-                    }
-                    if (HASB) braw[u] = raw1(B + (int64_t)ed[u] * bias_se + head * bias_sh);
-                }
-            }
-        } else {
-        // 16-bit rows: lanes past the end of the row repeat its last edge (a line the wave is reading
-        // anyway) and skip the arithmetic; with no lane-dependent branch around them the loads of a
-        // step are issued back to back, and the rows stay packed until they are used.
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            const int e = e0 + u * S;
-            ok[u] = e < n;
-            const int ec = min(e, n - 1);
-            nb[u] = col[ec];
-            ed[u] = HASB ? (ident ? start + ec : eid[ec]) : 0;
-        }
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
+    for (int u = 0; u < kUnroll; ++u) {
+        braw[u] = 0;
+        ndv[u] = make_float2(0.f, 0.f);
+        if constexpr (sizeof(T) == 4) { zero_raw(g0[u]); zero_raw(g1[u]); }
+        if (sizeof(T) != 4 || ok[u]) {
             const int64_t o = (int64_t)nb[u] * HD + el * 8;
             if (MODE == MODE_BWD_SRC) {
                 load_raw(Q + o, g0[u]);
@@ -304,57 +274,61 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
             }
             if (HASB) braw[u] = raw1(B + (int64_t)ed[u] * bias_se + head * bias_sh);
         }
-        }
+    }
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            if (ok[u]) {
-                float x0[8], x1[8];
-                unpack(g0[u], x0);
-                unpack(g1[u], x1);
-                const float bbu = HASB ? cvt1(braw[u]) : 0.f;
-                // raw score: identical arithmetic in all three walks so that the
-                // recomputed weights and the clamp mask agree bit for bit
-                const float raw = head_sum<LPH>(dot_raw(r0, g0[u])) * inv_scale;
-                const float w = __expf(clamp5(raw) + bbu);
-                if (MODE == MODE_FWD) {
-                    acc.z += w;
+    for (int u = 0; u < kUnroll; ++u) {
+        if (ok[u]) {
+            float x0[8], x1[8];
+            unpack(g0[u], x0);
+            unpack(g1[u], x1);
+            const float bbu = HASB ? cvt1(braw[u]) : 0.f;
+            // raw score: identical arithmetic in all three walks so that the
+            // recomputed weights and the clamp mask agree bit for bit
+            const float raw = head_sum<LPH>(dot_raw(rr.r0, g0[u])) * inv_scale;
+            const float w = __expf(clamp5(raw) + bbu);
+            if (MODE == MODE_FWD) {
+                acc.z += w;
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) acc.a0[i] = fmaf(w, x1[i], acc.a0[i]);
+                for (int i = 0; i < 8; ++i) acc.a0[i] = fmaf(w, x1[i], acc.a0[i]);
+            } else {
+                const bool inside = (raw >= -5.0f) & (raw <= 5.0f);   // torch clamp backward: inclusive
+                if (MODE == MODE_BWD_DST) {
+                    const float t = head_sum<LPH>(dot_raw(rr.r1, g1[u]));   // g_dst . v_src
+                    const float dS = w * rr.rz * (t - rr.Dh);
+                    T* __restrict__ dB = static_cast<T*>(s.out1);
+                    if (HASB && dB != nullptr) {
+                        if (bias_sh != 0) {       // one value per edge and head
+                            if (el % LPH == 0) store1(dB + (int64_t)ed[u] * H + head, dS);
+                        } else {                  // one value per edge: sum over heads
+                            float t2 = dS;   // sum over heads; every head is held by LPH lanes
+#pragma unroll
+                            for (int off = 1; off < LPE; off <<= 1) t2 += __shfl_xor(t2, off);
+                            if (el == 0) store1(dB + ed[u], t2 * (1.0f / LPH));
+                        }
+                    }
+                    const float md = inside ? dS : 0.f;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) acc.a0[i] = fmaf(md, x0[i], acc.a0[i]);
                 } else {
-                    const bool inside = (raw >= -5.0f) & (raw <= 5.0f);   // torch clamp backward: inclusive
-                    if (MODE == MODE_BWD_DST) {
-                        const float t = head_sum<LPH>(dot_raw(r1, g1[u]));   // g_dst . v_src
-                        const float dS = w * rz * (t - Dh);
-                        T* __restrict__ dB = static_cast<T*>(s.out1);
-                        if (HASB && dB != nullptr) {
-                            if (bias_sh != 0) {       // one value per edge and head
-                                if (el % LPH == 0) store1(dB + (int64_t)ed[u] * H + head, dS);
-                            } else {                  // one value per edge: sum over heads
-                                float t2 = dS;   // sum over heads; every head is held by LPH lanes
+                    const float p = w * ndv[u].x;
+                    const float t = head_sum<LPH>(dot_raw(g1[u], rr.r1));   // g_dst . v_src
+                    const float dS = p * (t - ndv[u].y);
+                    const float md = inside ? dS : 0.f;
 #pragma unroll
-                                for (int off = 1; off < LPE; off <<= 1) t2 += __shfl_xor(t2, off);
-                                if (el == 0) store1(dB + ed[u], t2 * (1.0f / LPH));
-                            }
-                        }
-                        const float md = inside ? dS : 0.f;
-#pragma unroll
-                        for (int i = 0; i < 8; ++i) acc.a0[i] = fmaf(md, x0[i], acc.a0[i]);
-                    } else {
-                        const float p = w * ndv[u].x;
-                        const float t = head_sum<LPH>(dot_raw(g1[u], r1));   // g_dst . v_src
-                        const float dS = p * (t - ndv[u].y);
-                        const float md = inside ? dS : 0.f;
-#pragma unroll
-                        for (int i = 0; i < 8; ++i) {
-                            acc.a0[i] = fmaf(md, x0[i], acc.a0[i]);   // dk += m dS q_dst
-                            acc.a1[i] = fmaf(p, x1[i], acc.a1[i]);    // dv += p g_dst
-                        }
+                    for (int i = 0; i < 8; ++i) {
+                        acc.a0[i] = fmaf(md, x0[i], acc.a0[i]);   // dk += m dS q_dst
+                        acc.a1[i] = fmaf(p, x1[i], acc.a1[i]);    // dv += p g_dst
                     }
                 }
             }
         }
     }
-    // add the S edge slots (all lanes take part)
+}
+
+// add the S edge slots of a lane group (all lanes take part)
+template <int LPE, int S, int MODE>
+__device__ __forceinline__ void add_slots(Acc& acc) {
+    constexpr int G = LPE * S;
 #pragma unroll
     for (int off = LPE; off < G; off <<= 1) {
         if (MODE == MODE_FWD) acc.z += __shfl_xor(acc.z, off);
@@ -364,6 +338,78 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
             if (MODE == MODE_BWD_SRC) acc.a1[i] += __shfl_xor(acc.a1[i], off);
         }
     }
+}
+
+// Walks `len` edges starting at sorted position `start` of node `row` with S edge
+// slots (this lane is slot `slot`, element chunk `el`), reading the plan's sorted view.  On return
+// every lane of the S*LPE-lane group holds the sums over all S slots.
+template <typename T, int LPE, int LPH, int S, int MODE, int HASB>
+__device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, const int row, const int start,
+                                           const int len, const int slot, const int el, const bool valid,
+                                           Acc& acc) {
+    RowRegs<T> rr;
+    load_row<T, LPE, LPH, MODE>(c, row, el, valid, rr, acc);
+    const int32_t* __restrict__ col = s.col + start;
+    // HASB == 2: no edge-id array, the bias rows are in this side's own sorted order (row = sorted position)
+    constexpr bool ident = HASB == 2;
+    const int32_t* __restrict__ eid = ident ? nullptr : s.eid + start;
+    const int n = valid ? len : 0;
+#pragma unroll 1
+    for (int e0 = slot; e0 < n; e0 += S * kUnroll) {
+        int nb[kUnroll], ed[kUnroll];
+        bool ok[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            const int e = e0 + u * S;
+            ok[u] = e < n;
+            if constexpr (sizeof(T) == 4) {
+                nb[u] = 0; ed[u] = 0;
+                if (ok[u]) {
+                    nb[u] = col[e];
+                    if (HASB) ed[u] = ident ? start + e : eid[e];
+                }
+            } else {   // lanes past the end of the row repeat its last edge (a line the wave is reading anyway)
+                const int ec = min(e, n - 1);
+                nb[u] = col[ec];
+                ed[u] = HASB ? (ident ? start + ec : eid[ec]) : 0;
+            }
+        }
+        edge_step<T, LPE, LPH, MODE, HASB>(c, s, rr, nb, ed, ok, el, acc);
+    }
+    add_slots<LPE, S, MODE>(acc);
+}
+
+// The same for a row of at most S * kUnroll edges whose endpoints and bias rows come with the wave's
+// record (one step, no loop): the record lists them in lane order, four consecutive entries per
+// (row, slot), an edge past the end of the row repeats the row's last one.
+template <typename T, int LPE, int LPH, int S, int MODE, int HASB>
+__device__ __forceinline__ void walk_record(const Common& c, const SideArgs& s, const WaveRec<LPE>& rec, const int row,
+                                            const int start, const int len, const int slot, const int el,
+                                            const bool valid, Acc& acc) {
+    RowRegs<T> rr;
+    load_row<T, LPE, LPH, MODE>(c, row, el, valid, rr, acc);
+    const int lg = (threadIdx.x & (kWave - 1)) / LPE;     // lane group = (row of the wave, slot)
+    const int4 cols = *reinterpret_cast<const int4*>(rec.col + lg * kUnroll);
+    int nb[kUnroll] = {cols.x, cols.y, cols.z, cols.w};
+    int ed[kUnroll] = {0, 0, 0, 0};
+    bool ok[kUnroll];
+    const int n = valid ? len : 0;
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) ok[u] = slot + u * S < n;
+    if (HASB == 2) {          // bias rows in this view's sorted order: row = sorted position
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) ed[u] = start + min(slot + u * S, max(n - 1, 0));
+    } else if (HASB) {
+        if (s.eid_is_map) {   // the bias rows are named by a map from sorted positions, not by the caller's edge ids
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) ed[u] = s.eid[start + min(slot + u * S, max(n - 1, 0))];
+        } else {
+            const int4 e4 = *reinterpret_cast<const int4*>(rec.eid + lg * kUnroll);
+            ed[0] = e4.x; ed[1] = e4.y; ed[2] = e4.z; ed[3] = e4.w;
+        }
+    }
+    edge_step<T, LPE, LPH, MODE, HASB>(c, s, rr, nb, ed, ok, el, acc);
+    add_slots<LPE, S, MODE>(acc);
 }
 
 // Final value of a row from its sums, written by the LPE lanes that own the chunks.
@@ -403,32 +449,32 @@ __device__ __forceinline__ void write_row(const Common& c, const SideArgs& s, co
     }
 }
 
-// Wave items: rows of at most kWaveRowMax edges, 64 / (LPE*S) rows per wave.  The wave takes items
-// [first, first + count).
-template <typename T, int LPE, int LPH, int S, int MODE, int HASB, bool TILES>
-__device__ __forceinline__ void wave_items(const Common& c, const SideArgs& s, const int first, const int count) {
+// Rows of one wave: 64 / (LPE*S) rows of one length class, named by the wave's record.  The longest
+// class walks the plan's sorted view step by step; the others find their (at most S * kUnroll) edges
+// in the record itself.
+template <typename T, int LPE, int LPH, int S, int MODE, int HASB, bool TILES, bool INLINE>
+__device__ __forceinline__ void wave_rows(const Common& c, const SideArgs& s, const WaveRec<LPE>& rec) {
     constexpr int G = LPE * S;
     const int lane = threadIdx.x & (kWave - 1);
     const int sub = lane / G, gl = lane % G;
     const int slot = gl / LPE, el = gl % LPE;
-    const bool valid = sub < count;
-    Item it{0, 0, 0, -1};
-    if (valid) it = s.items[first + sub];
+    const bool valid = sub < (int)(__builtin_amdgcn_readfirstlane(rec.code) >> 8);
+    int row = 0, start = 0, len = 0;
+    if (valid) { row = rec.row[sub]; start = rec.start[sub]; len = rec.len[sub]; }
     Acc acc;
-    walk_range<T, LPE, LPH, S, MODE, HASB>(c, s, it.row, it.start, it.len, slot, el, valid, acc);
-    if (valid && slot == 0) write_row<T, LPE, LPH, MODE, TILES>(c, s, it.row, el, acc);
+    if (INLINE) walk_record<T, LPE, LPH, S, MODE, HASB>(c, s, rec, row, start, len, slot, el, valid, acc);
+    else walk_range<T, LPE, LPH, S, MODE, HASB>(c, s, row, start, len, slot, el, valid, acc);
+    if (valid && slot == 0) write_row<T, LPE, LPH, MODE, TILES>(c, s, row, el, acc);
 }
 
-// The wave's share of a workgroup that walks wave items: its descriptor names the length class.
 template <typename T, int LPE, int LPH, int MODE, int HASB, bool TILES>
-__device__ __forceinline__ void wave_dispatch(const Common& c, const SideArgs& s, const int kind, const int first,
-                                              const int count) {
+__device__ __forceinline__ void wave_dispatch(const Common& c, const SideArgs& s, const WaveRec<LPE>& rec, const int kind) {
     switch (kind) {
-        case 0: wave_items<T, LPE, LPH, slots_for_class(LPE, 0), MODE, HASB, TILES>(c, s, first, count); break;
-        case 1: wave_items<T, LPE, LPH, slots_for_class(LPE, 1), MODE, HASB, TILES>(c, s, first, count); break;
-        case 2: wave_items<T, LPE, LPH, slots_for_class(LPE, 2), MODE, HASB, TILES>(c, s, first, count); break;
-        case 3: wave_items<T, LPE, LPH, slots_for_class(LPE, 3), MODE, HASB, TILES>(c, s, first, count); break;
-        default: wave_items<T, LPE, LPH, slots_for_class(LPE, 4), MODE, HASB, TILES>(c, s, first, count); break;
+        case 0: wave_rows<T, LPE, LPH, slots_for_class(LPE, 0), MODE, HASB, TILES, false>(c, s, rec); break;
+        case 1: wave_rows<T, LPE, LPH, slots_for_class(LPE, 1), MODE, HASB, TILES, class_inline(LPE, 1)>(c, s, rec); break;
+        case 2: wave_rows<T, LPE, LPH, slots_for_class(LPE, 2), MODE, HASB, TILES, class_inline(LPE, 2)>(c, s, rec); break;
+        case 3: wave_rows<T, LPE, LPH, slots_for_class(LPE, 3), MODE, HASB, TILES, class_inline(LPE, 3)>(c, s, rec); break;
+        default: wave_rows<T, LPE, LPH, slots_for_class(LPE, 4), MODE, HASB, TILES, class_inline(LPE, 4)>(c, s, rec); break;
     }
 }
 
@@ -562,7 +608,7 @@ __device__ __forceinline__ bool arrive(const SideArgs& s, const int idx, const i
 // group slots - the sums of a row with hundreds of segments are formed while the
 // launch is under way, not by one workgroup at its end.
 template <typename T, int LPE, int LPH, int MODE, int HASB, bool TILES>
-__device__ __forceinline__ void block_item(const Common& c, const SideArgs& s, const int item,
+__device__ __forceinline__ void block_item(const Common& c, const SideArgs& s, const Item it,
                                            BlockLds<LPE>& lds) {
     constexpr int S = slots_for_class(LPE, 0);
     constexpr int G = LPE * S;
@@ -575,7 +621,6 @@ __device__ __forceinline__ void block_item(const Common& c, const SideArgs& s, c
     const int sub = lane / G, gl = lane % G;
     const int slot = gl / LPE, el = gl % LPE;
     const int grp = (tid >> 6) * IPW + sub;
-    const Item it = s.items[item];
     // share of this lane group: consecutive chunk of the segment
     const int share = (it.len + NG - 1) / NG;
     const int lo = min(grp * share, it.len);
@@ -654,49 +699,47 @@ struct TraceScope {
 #define TGT_TRACE_SCOPE(code)
 #endif
 
-// Forward.  Workgroup b does what descriptors 4b .. 4b+3 say: one workgroup item, or four waves of wave
-// items.  Which rows meet in which workgroup, on which XCD and when is the plan's business.
+// Forward.  Workgroup b does what the records 4b .. 4b+3 say: one workgroup item, or four waves of
+// rows.  Which rows meet in which workgroup, on which XCD and when is the plan's business.
 template <typename T, int LPE, int LPH, int HASB, bool TILES>
 __global__ __launch_bounds__(kBlock) void k_attn_fwd(const Common c, const SideArgs s,
-                                                     const WaveDesc* __restrict__ desc) {
+                                                     const WaveRec<LPE>* __restrict__ recs) {
     __shared__ BlockLds<LPE> lds;
-    const WaveDesc* d = desc + (int64_t)blockIdx.x * (kBlock / kWave);
-    const uint32_t code0 = d[0].code;
+    const WaveRec<LPE>* r0 = recs + (int64_t)blockIdx.x * (kBlock / kWave);
+    const uint32_t code0 = r0->code;
     if ((code0 & 7u) == kDescBlock) {          // uniform over the workgroup
         TGT_TRACE_SCOPE(code0);
-        block_item<T, LPE, LPH, MODE_FWD, HASB, TILES>(c, s, d[0].first, lds);
+        block_item<T, LPE, LPH, MODE_FWD, HASB, TILES>(c, s, r0->item, lds);
         return;
     }
-    const int wave = threadIdx.x >> 6;
-    const uint32_t code = __builtin_amdgcn_readfirstlane(d[wave].code);
-    const int first = __builtin_amdgcn_readfirstlane(d[wave].first);
+    const WaveRec<LPE>& rec = r0[threadIdx.x >> 6];
+    const uint32_t code = __builtin_amdgcn_readfirstlane(rec.code);
     if ((code & 7u) == kDescNone) return;
     TGT_TRACE_SCOPE(code);
-    wave_dispatch<T, LPE, LPH, MODE_FWD, HASB, TILES>(c, s, code & 7u, first, code >> 8);
+    wave_dispatch<T, LPE, LPH, MODE_FWD, HASB, TILES>(c, s, rec, code & 7u);
 }
 
-// Backward: both views in one launch (they are independent once nd is known); the descriptor tells the view.
+// Backward: both views in one launch (they are independent once nd is known); the record tells the view.
 template <typename T, int LPE, int LPH, int HASB, bool TILES>
 __global__ __launch_bounds__(kBlock, 4) void k_attn_bwd(const Common c, const SideArgs sd, const SideArgs ss,
-                                                        const WaveDesc* __restrict__ desc) {
+                                                        const WaveRec<LPE>* __restrict__ recs) {
     __shared__ BlockLds<LPE> lds;
     constexpr int HB_D = HASB == 3 ? 2 : HASB;
     constexpr int HB_S = HASB == 3 ? 2 : (HASB ? 1 : 0);
-    const WaveDesc* d = desc + (int64_t)blockIdx.x * (kBlock / kWave);
-    const uint32_t code0 = d[0].code;
+    const WaveRec<LPE>* r0 = recs + (int64_t)blockIdx.x * (kBlock / kWave);
+    const uint32_t code0 = r0->code;
     if ((code0 & 7u) == kDescBlock) {          // uniform over the workgroup
         TGT_TRACE_SCOPE(code0);
-        if (code0 & kDescSrcSide) block_item<T, LPE, LPH, MODE_BWD_SRC, HB_S, TILES>(c, ss, d[0].first, lds);
-        else block_item<T, LPE, LPH, MODE_BWD_DST, HB_D, TILES>(c, sd, d[0].first, lds);
+        if (code0 & kDescSrcSide) block_item<T, LPE, LPH, MODE_BWD_SRC, HB_S, TILES>(c, ss, r0->item, lds);
+        else block_item<T, LPE, LPH, MODE_BWD_DST, HB_D, TILES>(c, sd, r0->item, lds);
         return;
     }
-    const int wave = threadIdx.x >> 6;
-    const uint32_t code = __builtin_amdgcn_readfirstlane(d[wave].code);
-    const int first = __builtin_amdgcn_readfirstlane(d[wave].first);
+    const WaveRec<LPE>& rec = r0[threadIdx.x >> 6];
+    const uint32_t code = __builtin_amdgcn_readfirstlane(rec.code);
     if ((code & 7u) == kDescNone) return;
     TGT_TRACE_SCOPE(code);
-    if (code & kDescSrcSide) wave_dispatch<T, LPE, LPH, MODE_BWD_SRC, HB_S, TILES>(c, ss, code & 7u, first, code >> 8);
-    else wave_dispatch<T, LPE, LPH, MODE_BWD_DST, HB_D, TILES>(c, sd, code & 7u, first, code >> 8);
+    if (code & kDescSrcSide) wave_dispatch<T, LPE, LPH, MODE_BWD_SRC, HB_S, TILES>(c, ss, rec, code & 7u);
+    else wave_dispatch<T, LPE, LPH, MODE_BWD_DST, HB_D, TILES>(c, sd, rec, code & 7u);
 }
 
 // Per-node side vector of the backward: nd[i,h] = (1 / (Z[i,h] + eps), sum_c dout[i,h,c] out[i,h,c]).
@@ -793,7 +836,7 @@ static int run_fwd(const Call& c) {
         }
         return TGT_ERR_HIP;
     }
-    const WaveDesc* desc = sch->fwd;
+    const WaveRec<LPE>* desc = static_cast<const WaveRec<LPE>*>(sch->fwd);
     if (c.bias_mode & TGT_BIAS_PLAN_ORDER) a.eid = nullptr;             // bias rows in destination-sorted order
     a.out0 = c.o_out; a.out1 = nullptr; a.Z = c.o_Z;
     if (c.init) { a.init0 = c.init->acc; a.initZ = c.init->Z; a.cover = c.init->cover_dst; }
@@ -857,14 +900,14 @@ static int run_bwd(const Call& c) {
     fill_side(sd, c.plan->dst);
     const Schedule* sch = plan_schedule(c.plan, LPE, c.st);
     if (!sch) return TGT_ERR_HIP;
-    const WaveDesc* desc = sch->bwd;
+    const WaveRec<LPE>* desc = static_cast<const WaveRec<LPE>*>(sch->bwd);
     if (c.bias_mode & TGT_BIAS_PLAN_ORDER) sd.eid = nullptr;
     sd.out0 = c.dq; sd.out1 = c.dbias; sd.Z = nullptr;
     if (c.init) { sd.init0 = c.init->dq; sd.cover = c.init->cover_dst; }
     sd.part = reinterpret_cast<float*>(c.ws + L.dq_part);
     sd.counters = counters + c.plan->dst.n_split + c.plan->dst.n_groups;
     fill_side(ss, c.plan->src);
-    if (c.bias_mode & TGT_BIAS_PLAN_ORDER) ss.eid = c.plan->src.pos;    // source-sorted -> destination-sorted position
+    if (c.bias_mode & TGT_BIAS_PLAN_ORDER) { ss.eid = c.plan->src.pos; ss.eid_is_map = 1; }   // source-sorted -> destination-sorted position
     if (c.bias_mode & TGT_BIAS_BOTH_ORDERS) ss.eid = nullptr;           // its own source-sorted copy
     ss.out0 = c.dk; ss.out1 = c.dv; ss.Z = nullptr;
     if (c.init) { ss.init0 = c.init->dk; ss.init1 = c.init->dv; ss.cover = c.init->cover_src; }
