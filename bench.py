@@ -86,7 +86,17 @@ def build_workload(name):
     return e, n, label, workloads.describe(e, n)
 
 
-def cpu_baseline(e, n, H, d, seconds_budget=25.0):
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(e, n, H, d, seconds_budget=30.0):
     """The oracle (op-for-op restatement of the reference's PyTorch path, fp32,
     autograd backward) timed on this host's cores with the same seeded inputs."""
     import torch
@@ -107,14 +117,15 @@ def cpu_baseline(e, n, H, d, seconds_budget=25.0):
 
     times = []
     t_start = time.perf_counter()
-    step()                                       # warm-up
-    while len(times) < 10 and (time.perf_counter() - t_start) < seconds_budget:
+    for _ in range(3):                           # warm-up
+        step()
+    while len(times) < 10 and (len(times) < 3 or (time.perf_counter() - t_start) < seconds_budget):
         t0 = time.perf_counter()
         step()
         times.append(time.perf_counter() - t0)
     med = statistics.median(times)
-    return {"value": E / med, "unit": "edges/s", "cores": cores, "kind": "port",
-            "sample": f"full workload (E={E}), fp32, {len(times)} fwd+bwd iterations after 1 warm-up, median",
+    return {"value": E / med, "unit": "edges/s", "cores": cores, "cpu_model": cpu_model(), "kind": "port",
+            "sample": f"full workload (E={E}), fp32, {len(times)} fwd+bwd iterations after 3 warm-ups, median",
             "ms_per_step": med * 1e3}
 
 
@@ -252,7 +263,7 @@ def bench_dense(args):
                  for n in kernels},
         "kernels": kernels,
     }
-    print(json.dumps(result))
+    return result
 
 
 def bench_graph_bias(args):
@@ -359,7 +370,7 @@ def bench_graph_bias(args):
     }
     if prep_ms is not None:
         result["floyd_warshall_plus_gen_edge_input_ms"] = prep_ms
-    print(json.dumps(result))
+    return result
 
 
 def bench_block(args):
@@ -376,10 +387,15 @@ def bench_block(args):
     H, d = 8, 8
     tdt = torch.bfloat16 if args.dtype == "bf16" else torch.float32
     e, n, cluster = workloads.stochastic_block_model(seed=42)
+    hybrid = args.workload == "config5-hybrid"
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    new_e, _, tiles, raw = graph_prep.reformat_graph(torch.from_numpy(e).to(dev), 64, 16,
-                                                     partition_ids=torch.from_numpy(cluster), return_tiles=True)
+    if hybrid:
+        tiles, raw, new_e = workloads.hybrid_tiles(e, cluster, 64, 16, seed=42)
+        raw, new_e = torch.from_numpy(raw).to(dev), torch.from_numpy(new_e).to(dev)
+    else:
+        new_e, _, tiles, raw = graph_prep.reformat_graph(torch.from_numpy(e).to(dev), 64, 16,
+                                                         partition_ids=torch.from_numpy(cluster), return_tiles=True)
     torch.cuda.synchronize()
     reorder_ms = (time.perf_counter() - t0) * 1e3
     E = int(new_e.shape[1])
@@ -432,13 +448,15 @@ def bench_block(args):
     esize = 2 if args.dtype == "bf16" else 4
     R = H * d * esize
     # every node row once per pass; a tile is 8 bytes; fp32 tile sums written and read once per pass
-    alg = 12 * n * R + 8 * n * H + 3 * 8 * len(tiles) + 2 * 4 * (n * H * d * 4 + n * H)
+    alg = 12 * n * R + 8 * n * H + 3 * 8 * len(tiles) + 2 * 4 * (n * H * d * 4 + n * H) + 16 * int(raw.shape[1])
     result = {
         "metric": "fwd+bwd block attention (16x16 tiles on MFMA + sparse remainder) edges/sec; ms/layer",
         "value": E / (ms_block * 1e-3), "unit": "edges/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_block, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic",
-        "config": {"workload": "configs[4]: SBM 64 x 4096 reordered by the reference's blockize (k=64, 16x16 blocks)",
+        "config": {"workload": ("configs[4]: SBM 64 x 4096, hybrid: intra-cluster edges as 16x16 tiles, inter-cluster edges raw, one softmax"
+                                if hybrid else
+                                "configs[4]: SBM 64 x 4096 reordered by the reference's blockize (k=64, 16x16 blocks)"),
                    "N": n, "tiles": int(len(tiles)), "E_expanded": E, "E_remainder": int(raw.shape[1]), "H": H, "d": d,
                    "step": "tgt_block_attn_fwd + tgt_block_attn_bwd", "parallelism": "1 GPU"},
         "roofline": {"bound": "hbm", "kernel": "whole step", "achieved": alg / (ms_block * 1e-3) / 1e9,
@@ -448,7 +466,7 @@ def bench_block(args):
         "sparse_path_same_edges_ms": ms_sparse,
         "reorder_ms": reorder_ms,
     }
-    print(json.dumps(result))
+    return result
 
 
 def bench_mha(args):
@@ -513,7 +531,7 @@ def bench_mha(args):
                         "mfma_peak_tflops": 157.3 if args.dtype == "f32" else 2500.0},
         "kernels": kernels,
     }
-    print(json.dumps(result))
+    return result
 
 
 def bench_model(args):
@@ -617,7 +635,7 @@ def bench_model(args):
                              for g, ks in groups.items()},
         "kernels": kernels,
     }
-    print(json.dumps(result))
+    return result
 
 
 def bench_graph_model(args):
@@ -733,56 +751,19 @@ def bench_graph_model(args):
                              for g, ks in groups.items()},
         "kernels": kernels,
     }
-    print(json.dumps(result))
+    return result
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--dtype", default="f32", choices=["f32", "bf16"])
-    ap.add_argument("--workload", default="config2")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-reference-ops", action="store_true",
-                    help="skip the datapoint that runs the reference's op chain with stock torch kernels (profiling runs)")
-    ap.add_argument("--hip-graph", action="store_true",
-                    help="config2-model: also time the step captured into a HIP graph and replayed")
-    ap.add_argument("--calibration-copy", action="store_true",
-                    help="also run one 256 MiB device copy (a kernel of known traffic, for scaling rocprofv3 "
-                         "FETCH_SIZE / WRITE_SIZE readings)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        raise SystemExit("bench.py: this build runs on ONE GPU (sequence-parallel size 1); "
-                         "--gpus N with N > 1 is not supported")
-
+def bench_sparse(args):
+    """Sparse attention fwd+bwd of one layer through the C ABI on the graph of args.workload (config1, config2,
+    config3, config5): the headline measurement for config2."""
     import torch
     from torchgt_amd import _lib
     from torchgt_amd.plan import GraphPlan
-
-    if not torch.cuda.is_available():
-        raise SystemExit("bench.py needs a GPU")
     dev = torch.device("cuda:0")
     H, d = 8, 8
-    if args.workload in ("config3", "config4", "config4-bias", "config4-bias-multihop", "config4-model", "config5",
-                         "config5-blockized") and "--dtype" not in sys.argv:
-        args.dtype = "bf16"              # the dtype those configurations are quoted on
     tdt = torch.float32 if args.dtype == "f32" else torch.bfloat16
     esize = 4 if args.dtype == "f32" else 2
-    if args.workload == "config4":
-        return bench_dense(args)
-    if args.workload in ("config4-bias", "config4-bias-multihop"):
-        return bench_graph_bias(args)
-    if args.workload == "config4-model":
-        return bench_graph_model(args)
-    if args.workload == "config5-blockized":
-        return bench_block(args)
-    if args.workload == "config2-mha":
-        return bench_mha(args)
-    if args.workload in ("config2-model", "config2-gt-model"):
-        return bench_model(args)
-    if args.workload in ("config3", "config5"):
-        args.no_cpu_baseline = True      # the CPU restatement needs minutes per step at this size
     e, n, label, desc = build_workload(args.workload)
     E = e.shape[1]
 
@@ -888,7 +869,7 @@ def main():
                 "mode": "TGT_BIAS_PLAN_ORDER | TGT_BIAS_BOTH_ORDERS"}
 
     plan_order = plan_order_point()
-    probe = gather_probe(plan, n, E, H * d * esize, stream)
+    probe = gather_probe(plan, n, E, H * d * esize, stream) if not args.brief else None
     bpe = H * esize
     dom = max((kk for kk in kernels if kernel_alg_bytes(kk, n, E, H, d, esize, bpe)),
               key=lambda kk: kernels[kk]["avg_us"])
@@ -925,6 +906,98 @@ def main():
         result["reference_ops_on_gpu"] = reference_ops_on_gpu(ei, q, k, v, bias, dout)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(e, n, H, d)
+    plan.close()
+    return result
+
+
+DISPATCH = {"config4": bench_dense, "config4-bias": bench_graph_bias, "config4-bias-multihop": bench_graph_bias,
+            "config4-model": bench_graph_model, "config5-blockized": bench_block, "config5-hybrid": bench_block,
+            "config2-mha": bench_mha, "config2-model": bench_model, "config2-gt-model": bench_model}
+BF16_BY_DEFAULT = ("config3", "config4", "config4-bias", "config4-bias-multihop", "config4-model", "config5",
+                   "config5-blockized", "config5-hybrid")
+
+
+def run_workload(args):
+    fn = DISPATCH.get(args.workload)
+    if fn is not None:
+        return fn(args)
+    if args.workload in ("config3", "config5"):
+        args.no_cpu_baseline = True      # the CPU restatement needs minutes per step at this size
+    return bench_sparse(args)
+
+
+def other_configs(args):
+    """The other benchmark configurations, each timed by its own workload function inside this run (so that
+    they sit under the same clock as the headline): step time, algorithmic bytes, fraction of the 8 TB/s roofline."""
+    import copy
+    import gc
+    import torch
+    out = {}
+    todo = [("configs[1] bf16", "config2", "bf16", 100, 10), ("configs[2] bf16", "config3", "bf16", 10, 3),
+            ("configs[3] bf16 dense", "config4", "bf16", 100, 10), ("configs[4] bf16 sparse path", "config5", "bf16", 50, 5),
+            ("configs[4] bf16 hybrid (tiles + remaining edges)", "config5-hybrid", "bf16", 50, 5),
+            ("configs[4] bf16 blockized by the reference's reordering", "config5-blockized", "bf16", 50, 5)]
+    for tag, workload, dtype, steps, warmup in todo:
+        a = copy.copy(args)
+        a.workload, a.dtype, a.steps, a.warmup = workload, dtype, steps, warmup
+        a.no_cpu_baseline = a.no_reference_ops = a.brief = True
+        a.calibration_copy = False
+        t0 = time.perf_counter()
+        try:
+            r = run_workload(a)
+        except Exception as exc:                       # one configuration must not take the headline line down
+            out[tag] = {"error": f"{type(exc).__name__}: {exc}"}
+            continue
+        roof = r.get("roofline", {})
+        entry = {"workload": r["config"]["workload"], "ms_per_step": r["ms_per_step"], "value": r["value"], "unit": r["unit"],
+                 "steps": steps, "alg_bytes_step": r.get("alg_bytes_step", roof.get("alg_bytes")),
+                 "hbm_roofline_frac_step": r.get("hbm_roofline_frac_step"),
+                 "roofline": {kk: roof.get(kk) for kk in ("kernel", "frac", "alg_bytes", "avg_us")},
+                 "kernels_avg_us": {kk: round(vv["avg_us"], 2) for kk, vv in r.get("kernels", {}).items()},
+                 "seconds_spent": None}
+        for extra in ("bias_in_plan_order", "mfma", "sparse_path_same_edges_ms", "ids_and_tables"):
+            if extra in r:
+                entry[extra] = r[extra]
+        entry["seconds_spent"] = round(time.perf_counter() - t0, 1)
+        out[tag] = entry
+        del r
+        gc.collect()
+        torch.cuda.empty_cache()
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--dtype", default="f32", choices=["f32", "bf16"])
+    ap.add_argument("--workload", default="config2")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-reference-ops", action="store_true",
+                    help="skip the datapoint that runs the reference's op chain with stock torch kernels (profiling runs)")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="config2 / f32 only: skip the other benchmark configurations (they are timed in the default run)")
+    ap.add_argument("--hip-graph", action="store_true",
+                    help="config2-model: also time the step captured into a HIP graph and replayed")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run one 256 MiB device copy (a kernel of known traffic, for scaling rocprofv3 "
+                         "FETCH_SIZE / WRITE_SIZE readings)")
+    args = ap.parse_args()
+    args.brief = False
+    if args.gpus != 1:
+        raise SystemExit("bench.py: this build runs on ONE GPU (sequence-parallel size 1); "
+                         "--gpus N with N > 1 is not supported")
+
+    import torch
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU")
+    if args.workload in BF16_BY_DEFAULT and "--dtype" not in sys.argv:
+        args.dtype = "bf16"              # the dtype those configurations are quoted on
+    headline = args.workload == "config2" and args.dtype == "f32"
+    result = run_workload(args)
+    if headline and not args.no_other_configs:
+        result["other_configs"] = other_configs(args)
     print(json.dumps(result))
 
 

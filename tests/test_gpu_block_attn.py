@@ -133,6 +133,18 @@ def test_config5_blockized_full_size(cuda):
     run_case("config5-blockized", n, tiles, raw.cpu(), 8, 8, torch.bfloat16, "none", 9, cuda)
 
 
+def test_config5_hybrid_full_size(cuda):
+    # configs[4] as the benchmark words it: the intra-cluster edges of the 64 clusters as dense 16 x 16 tiles on the
+    # matrix cores, the ~5 % inter-cluster edges raw on the sparse kernels (with a per-edge bias), one softmax per
+    # node - against the float64 oracle on the expanded edge list, outputs and all gradients, at full size
+    e, n, cluster = workloads.stochastic_block_model()
+    tiles, raw, expanded = workloads.hybrid_tiles(e, cluster, 64, 16, seed=42)
+    print(f"config5 hybrid: T={tiles.shape[0]} raw={raw.shape[1]} expanded={expanded.shape[1]}", flush=True)
+    assert n == 262144 and 0.03 < raw.shape[1] / e.shape[1] < 0.07
+    assert expanded.shape[1] == 256 * tiles.shape[0] + raw.shape[1]
+    run_case("config5-hybrid", n, tiles, torch.from_numpy(raw), 8, 8, torch.bfloat16, "edge_head", 10, cuda)
+
+
 def test_block_loud_failures(cuda):
     q = torch.randn(100, 8, 8, device=cuda, dtype=torch.bfloat16)
     with pytest.raises(_lib.TorchGTHipError) as exc:

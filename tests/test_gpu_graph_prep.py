@@ -73,6 +73,23 @@ def test_reformat_raw_branch_when_duplicates_exceed_capacity(cuda):
     _check_reformat(np.concatenate([rest, dense, rest2], 1), part, 2, 2, True, cuda)
 
 
+def test_reformat_hand_computed_compact_counts_and_raw_branch(cuda):
+    # the hand-computed example of tests/test_oracle_graph_prep.py (compact edge counts read at the wrong
+    # pair, raw-edge branch, duplicate blocks): 7 nodes in parts of 2, 3, 2, block size 2, no random draw matters
+    part = np.array([0, 0, 1, 1, 1, 2, 2])
+    pairs = [(1, 0), (0, 1), (0, 1), (1, 1), (0, 0), (1, 6), (0, 5), (0, 5), (1, 5), (0, 6), (1, 6), (0, 5),
+             (4, 0), (2, 0), (3, 1), (2, 5), (6, 6), (5, 5), (5, 6), (6, 5), (5, 5)]
+    blk = lambda r0, c0: [(r0, c0), (r0, c0 + 1), (r0 + 1, c0), (r0 + 1, c0 + 1)]
+    emitted = ([(0, 0), (0, 1), (0, 1), (1, 0), (1, 1)] + [(0, 5), (0, 5), (0, 5), (0, 6), (1, 5), (1, 6), (1, 6)]
+               + blk(0, 5) + blk(2, 0) + blk(2, 2) + blk(2, 2) + blk(2, 5) + blk(5, 0) + blk(5, 2) + blk(5, 5))
+    emitted = np.array(emitted).T
+    want = emitted[:, np.argsort(emitted[0], kind="stable")]
+    got_e, got_s = graph_prep.reformat_graph(torch.tensor(pairs).t().contiguous().to(cuda), 3, 2,
+                                             partition_ids=torch.from_numpy(part))
+    np.testing.assert_array_equal(got_e.cpu().numpy(), want)
+    np.testing.assert_array_equal(got_s.cpu().numpy(), np.arange(7))
+
+
 def test_relabel_and_sort_without_blockize(cuda):
     rng = np.random.default_rng(3)
     N, k = 70000, 8

@@ -354,6 +354,52 @@ def test_bias_in_plan_order_is_the_same_computation(cuda, dtype, per_head):
                 assert torch.equal(a, b_), nm
 
 
+def test_module_bias_cache_respects_autograd_state(cuda):
+    """A leaf per-edge bias first seen under no_grad (an evaluation pass) must still get its gradient in the
+    training pass that follows, and a second training step over the same bias object must not walk a freed
+    graph: the module's plan-order copy of the bias is tied to the autograd state and dropped at backward."""
+    e, n = workloads.barabasi_albert(n=512, m=3, seed=5)
+    ei = torch.from_numpy(e).to(cuda)
+    H, d = 8, 8
+    g = torch.Generator().manual_seed(9)
+    q, k, v = (torch.randn(1, n, H, d, generator=g).to(cuda).requires_grad_(True) for _ in range(3))
+    bias = (torch.randn(e.shape[1], H, generator=g) * 0.3).to(cuda).requires_grad_(True)
+    layers = [CoreAttention(H * d, 0.0, H).to(cuda) for _ in range(2)]
+    with torch.no_grad():
+        ref = sum(m(q, k, v, bias, ei, "sparse") for m in layers)
+    for step in range(2):
+        out = sum(m(q, k, v, bias, ei, "sparse") for m in layers)
+        assert torch.equal(out, ref)
+        bias.grad = None
+        out.square().sum().backward()
+        assert bias.grad is not None and torch.isfinite(bias.grad).all() and bias.grad.abs().max() > 0
+    # the gradient equals the one of the functional path
+    b2 = bias.detach().clone().requires_grad_(True)
+    out2 = 2 * sparse_attention(q.detach()[0], k.detach()[0], v.detach()[0], ei, b2).view(1, n, -1)
+    out2.square().sum().backward()
+    assert err(bias.grad, b2.grad) <= 1e-5
+    from torchgt_amd import core_attention
+    assert not core_attention._BIAS_CACHE      # nothing outlives the step
+
+
+def test_plan_cache_is_bounded_by_bytes(cuda):
+    from torchgt_amd import plan as plan_mod, get_plan, set_plan_cache_bytes, clear_plan_cache
+    clear_plan_cache()
+    rng = np.random.default_rng(0)
+    keep = [torch.from_numpy(rng.integers(0, 1000, (2, 5000))).to(cuda) for _ in range(6)]
+    try:
+        set_plan_cache_bytes(3 * (56 * 5000 + 450 * 1000 + 16 * 5000))     # room for three such plans
+        plans = [get_plan(t, 1000) for t in keep]
+        assert len(plan_mod._CACHE) == 3
+        assert get_plan(keep[-1], 1000) is plans[-1]                         # still cached
+        assert get_plan(keep[0], 1000) is not plans[0]                       # evicted and rebuilt
+        set_plan_cache_bytes(1)
+        assert len(plan_mod._CACHE) == 1                                     # the last one always stays
+    finally:
+        set_plan_cache_bytes(1 << 30)
+        clear_plan_cache()
+
+
 def test_plan_order_needs_the_map(cuda):
     e, n = workloads.barabasi_albert()
     ei = torch.from_numpy(e).to(cuda)

@@ -83,6 +83,38 @@ def test_blockize_counts_and_offsets_two_partitions():
     assert pos == out.shape[1]
 
 
+def test_blockize_compact_counts_and_raw_edge_branch_by_hand():
+    """Hand-computed answer for the two branches nothing else pins (gt_sp/utils.py:237-246, 270-283).
+    7 nodes in 3 parts of 2, 3, 2 nodes (already in part order, so the relabelling is the identity), block
+    size 2: every part holds exactly one block row, so every randint(0, 1) is 0 and no random stream enters.
+    Non-empty partition pairs in sorted order: (0,0) 5 edges, (0,2) 7, (1,0) 3, (1,2) 1, (2,2) 5.  The reference
+    stores these counts compactly, [5, 7, 3, 1, 5, 0, 0, 0, 0], and reads entry i*3+j for pair (i, j):
+      (0,0) reads 5 > 2*2      -> raw branch: the 5 sorted edges of slice [0, 5)
+      (0,1) reads 7 > 2*3      -> raw branch: slice [5, 12), which holds the edges of pair (0,2)
+      (0,2) reads 3 <= 4       -> int(3/4)+1 = 1 block on rows {0,1} x columns {5,6}
+      (1,0) reads 1            -> 1 block rows {2,3} x columns {0,1}
+      (1,1) reads 5 <= 9       -> int(5/4)+1 = 2 (identical) blocks rows {2,3} x columns {2,3}
+      (1,2), (2,0), (2,1), (2,2) read 0 -> 1 block each."""
+    part = np.array([0, 0, 1, 1, 1, 2, 2])
+    pairs = [(1, 0), (0, 1), (0, 1), (1, 1), (0, 0),                          # (0,0), unsorted on purpose
+             (1, 6), (0, 5), (0, 5), (1, 5), (0, 6), (1, 6), (0, 5),          # (0,2)
+             (4, 0), (2, 0), (3, 1),                                          # (1,0)
+             (2, 5),                                                          # (1,2)
+             (6, 6), (5, 5), (5, 6), (6, 5), (5, 5)]                          # (2,2)
+    ei = np.array(pairs).T
+    mapping = gp.relabel_by_partition(part, 3)
+    np.testing.assert_array_equal(mapping, np.arange(7))
+    out = gp.blockize(ei, 3, part, 1, 2, mapping)
+
+    def block(r0, c0):
+        return [(r0, c0), (r0, c0 + 1), (r0 + 1, c0), (r0 + 1, c0 + 1)]
+    want = ([(0, 0), (0, 1), (0, 1), (1, 0), (1, 1)]
+            + [(0, 5), (0, 5), (0, 5), (0, 6), (1, 5), (1, 6), (1, 6)]
+            + block(0, 5) + block(2, 0) + block(2, 2) + block(2, 2) + block(2, 5)
+            + block(5, 0) + block(5, 2) + block(5, 5))
+    np.testing.assert_array_equal(out, np.array(want).T)
+
+
 def test_reformat_graph_sorted_by_source_stably():
     rng = np.random.default_rng(1)
     N, k = 96, 3

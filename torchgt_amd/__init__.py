@@ -6,7 +6,7 @@ The compute lives in ``libtorchgt_hip.so`` (sources in ``csrc/``, C ABI in
 """
 from .core_attention import (CoreAttention, SparseAttentionFunction, DenseAttentionFunction, sparse_attention,
                              dense_attention, gather_dense_bias)
-from .plan import GraphPlan, get_plan, clear_plan_cache
+from .plan import GraphPlan, get_plan, clear_plan_cache, set_plan_cache_bytes
 from .multi_head_attention import MultiHeadAttention, LinearFunction, fused_linear
 from .encoder import FeedForwardNetwork, EncoderLayer, Graphormer
 from .graph_bias import GraphAttnBias, floyd_warshall, gen_edge_input
@@ -16,7 +16,7 @@ from .block_attention import BlockAttentionFunction, TileSet, block_attention, e
 
 __all__ = ["CoreAttention", "SparseAttentionFunction", "DenseAttentionFunction", "sparse_attention",
            "dense_attention", "gather_dense_bias",
-           "GraphPlan", "get_plan", "clear_plan_cache", "BlockAttentionFunction", "TileSet", "block_attention",
+           "GraphPlan", "get_plan", "clear_plan_cache", "set_plan_cache_bytes", "BlockAttentionFunction", "TileSet", "block_attention",
            "expand_tiles", "MultiHeadAttention", "LinearFunction", "fused_linear",
            "FeedForwardNetwork", "EncoderLayer", "Graphormer", "GraphAttnBias", "floyd_warshall", "gen_edge_input",
            "GraphNodeFeature", "GraphLevelGraphormer", "GT", "GraphLevelGT", "MLPReadout"]

@@ -14,6 +14,7 @@ There is no CPU or eager fallback: tensors must live on the GPU and the HIP
 library must be built, otherwise an exception is raised.
 """
 import math
+import weakref
 
 import torch
 import torch.nn as nn
@@ -92,6 +93,8 @@ class SparseAttentionFunction(torch.autograd.Function):
             dbias = torch.empty_like(edge_bias)
             if ctx.mode & _lib.BIAS_BOTH_ORDERS:
                 dbias[plan.num_edges:].zero_()      # the source-sorted copy gets no gradient of its own
+        if ctx.mode & _lib.BIAS_PLAN_ORDER:
+            _BIAS_CACHE.clear()     # the step is over: the next forward brings its bias into plan order afresh
         ws = plan.workspace(H, d)
         with torch.cuda.device(q.device):
             stream = torch.cuda.current_stream(q.device).cuda_stream
@@ -190,16 +193,20 @@ def gather_dense_bias(attn_bias, edge_index, layout):
     return attn_bias[src // S, src % S, dst % S, :]
 
 
-_BIAS_CACHE = {}      # one entry: (bias tensor, its version, plan, dtype, layout) -> per-edge bias in plan order
+_BIAS_CACHE = {}      # at most one entry: the per-edge bias in plan order of the bias tensor seen last
 
 
 def _plan_order_bias(module, attn_bias, edge_index, plan, dtype):
-    """Per-edge bias in the plan's destination-sorted order for a dense or per-edge ``attn_bias``; the last
-    result is kept (with the tensor it came from, so its identity cannot be recycled) and reused while the same
-    bias object comes in again - the other layers of the same step.  Differentiable."""
-    key = (id(attn_bias), attn_bias._version, id(plan), dtype, module.dense_bias_layout)
+    """Per-edge bias in the plan's sorted orders for a dense or per-edge ``attn_bias``.  The layers of one
+    forward pass get one and the same bias tensor: the first brings it into plan order, the others reuse the
+    result.  The entry is tied to the tensor (held weakly), its version, the plan, the dtype and the autograd
+    state it was made under - a result made under ``no_grad`` carries no graph and is not handed to a pass that
+    needs one - and it is dropped by the first backward that follows, so neither the bias nor its 2E-row copy
+    outlives the step.  Differentiable."""
+    key = (id(attn_bias), attn_bias._version, id(plan), dtype, module.dense_bias_layout,
+           torch.is_grad_enabled(), attn_bias.requires_grad)
     hit = _BIAS_CACHE.get("entry")
-    if hit is not None and hit[0] == key and hit[1] is attn_bias and hit[2] is plan:
+    if hit is not None and hit[0] == key and hit[1]() is attn_bias and hit[2] is plan:
         return hit[3]
     if attn_bias.dim() <= 2:
         eb = plan.sort_bias(attn_bias.to(dtype))
@@ -211,7 +218,7 @@ def _plan_order_bias(module, attn_bias, edge_index, plan, dtype):
         if eb.shape[-1] == 1:
             eb = eb.squeeze(-1)
         eb = eb.to(dtype)
-    _BIAS_CACHE["entry"] = (key, attn_bias, plan, eb)
+    _BIAS_CACHE["entry"] = (key, weakref.ref(attn_bias), plan, eb)
     return eb
 
 

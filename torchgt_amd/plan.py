@@ -158,13 +158,36 @@ class _SortRows(torch.autograd.Function):
 
 
 _CACHE = collections.OrderedDict()
-_CACHE_SIZE = 16
+_CACHE_BYTES = 1 << 30        # device memory the cached plans (and the edge_index tensors they were built from) may hold
+
+
+def set_plan_cache_bytes(nbytes):
+    """Bound on the device memory held by ``get_plan``'s cache (default 1 GiB).  The plan asked for last is
+    always kept, whatever its size."""
+    global _CACHE_BYTES
+    _CACHE_BYTES = int(nbytes)
+    _evict()
+
+
+def _plan_bytes(plan, edge_index):
+    # two sorted views (rowptr, col, eid), items, wave records of one shape, and the edge_index kept alive
+    return 56 * plan.num_edges + 450 * plan.num_nodes + edge_index.numel() * edge_index.element_size()
+
+
+def _evict():
+    total = sum(v[2] for v in _CACHE.values())
+    while len(_CACHE) > 1 and total > _CACHE_BYTES:
+        _, (_, _, nbytes) = _CACHE.popitem(last=False)      # freed when its last user (a pending backward) lets go
+        total -= nbytes
 
 
 def get_plan(edge_index, num_nodes):
     """Plan for ``edge_index``, cached on (storage address, shape, version, N) so
     that the layers of a model and the iterations over a pre-packed batch share
-    one plan.  The cache keeps the tensor alive, so the address cannot be reused."""
+    one plan.  The cache keeps the tensor alive, so the address cannot be reused; it is bounded by bytes
+    (``set_plan_cache_bytes``), least recently used plans go first.  A driver that moves a fresh edge_index
+    to the GPU for every iteration therefore holds one large plan at a time, not sixteen.  Build plans before
+    capturing a HIP graph: building one allocates and synchronises."""
     key = (edge_index.data_ptr(), tuple(edge_index.shape), edge_index._version, edge_index.dtype,
            str(edge_index.device), int(num_nodes))
     hit = _CACHE.get(key)
@@ -172,9 +195,8 @@ def get_plan(edge_index, num_nodes):
         _CACHE.move_to_end(key)
         return hit[0]
     plan = GraphPlan(edge_index, num_nodes)
-    _CACHE[key] = (plan, edge_index)
-    while len(_CACHE) > _CACHE_SIZE:
-        _CACHE.popitem(last=False)
+    _CACHE[key] = (plan, edge_index, _plan_bytes(plan, edge_index))
+    _evict()
     return plan
 
 

@@ -145,6 +145,37 @@ def stochastic_block_model(n_clusters=64, cluster_size=4096, p_intra=0.004, inte
     return e, n, np.repeat(np.arange(n_clusters, dtype=np.int64), cluster_size)
 
 
+def hybrid_tiles(edge_index, cluster, n_clusters, block_size, seed=42):
+    """Config 5 as a hybrid: every cluster's intra-cluster edges are replaced by int(count / bs^2) + 1 random
+    dense bs x bs tiles inside the cluster (the recipe of generate_new_edges_optimized for one partition pair,
+    gt_sp/utils.py:284-299, applied to the diagonal pairs only, with this module's own seeded generator); the
+    inter-cluster edges stay as they are.  Nodes must be ordered contiguously by cluster.  Returns (tiles int32
+    [T, 2] = first source / first destination, raw inter-cluster edges int64 [2, E_raw], the equivalent
+    expanded edge list int64 [2, T * bs^2 + E_raw])."""
+    rng = np.random.default_rng(seed)
+    src, dst = np.asarray(edge_index[0]), np.asarray(edge_index[1])
+    cs, cd = cluster[src], cluster[dst]
+    intra = cs == cd
+    counts = np.bincount(cs[intra], minlength=n_clusters)
+    sizes = np.bincount(cluster, minlength=n_clusters)
+    offs = np.concatenate([[0], np.cumsum(sizes)[:-1]])
+    tiles = []
+    for c in range(n_clusters):
+        nb = sizes[c] // block_size
+        if nb == 0:
+            continue
+        t = counts[c] // (block_size * block_size) + 1
+        tiles.append(np.stack([rng.integers(0, nb, t) * block_size + offs[c],
+                               rng.integers(0, nb, t) * block_size + offs[c]], 1))
+    tiles = np.concatenate(tiles).astype(np.int32)
+    raw = np.ascontiguousarray(np.stack([src[~intra], dst[~intra]]).astype(np.int64))
+    ar = np.arange(block_size)
+    a = (tiles[:, 0:1, None] + ar[None, :, None] + 0 * ar[None, None, :]).reshape(-1)
+    b = (tiles[:, 1:2, None] + 0 * ar[None, :, None] + ar[None, None, :]).reshape(-1)
+    expanded = np.concatenate([np.stack([a, b]).astype(np.int64), raw], axis=1)
+    return tiles, raw, np.ascontiguousarray(expanded)
+
+
 def clustered_power_law_graph(n=870_000, exponent=2.0, directed_edges=44_000_000, n_clusters=64,
                               intra_fraction=0.8, seed=42, oversample=None):
     """Config 3: power-law graph (mean degree ~50) whose nodes are grouped into contiguous
