@@ -35,6 +35,9 @@ extern "C" {
 /* element type of q, k, v, out, bias and the gradients */
 #define TGT_DTYPE_F32   0
 #define TGT_DTYPE_BF16  1
+/* dense attention only: float32 tensors whose matrix products run on the bf16 matrix cores (operands
+ * rounded to bf16, fp32 accumulation and softmax): about 2e-2 instead of 1e-5, for callers that ask for it */
+#define TGT_DTYPE_F32_BF16_PRODUCTS 2
 
 /* how the additive attention bias is supplied (added AFTER the +-5 clamp,
  * models/graphormer_dist_graph_level.py:262-267) */
@@ -178,10 +181,11 @@ int tgt_sparse_attn_bwd(const tgt_plan_t* plan,
  * attn_module.py:99-127):  x = (q * sqrt(d)) k^T + bias ; softmax over keys ; x v.
  * d_q, d_k, d_v: [b, S, H, d]; d_bias: [b, H, S, S] (may hold -inf on padded
  * keys) or NULL; d_out: [b, S, H*d]; all of `dtype`.  d_lse: [b, H, S] float32
- * (log-sum-exp of every score row, saved for the backward).  bf16 matrix
- * instructions with fp32 accumulation and fp32 softmax; float32 inputs are rounded
- * to bf16 on load.  d in {8, 16, 32}, S <= 256.  Dropout and the reference's
- * unused `mask` argument are not applied. */
+ * (log-sum-exp of every score row, saved for the backward).  TGT_DTYPE_BF16 and
+ * TGT_DTYPE_F32_BF16_PRODUCTS: bf16 matrix instructions with fp32 accumulation and fp32 softmax
+ * (S <= 256).  TGT_DTYPE_F32: float32 arithmetic throughout, like the reference (vector units; any S
+ * whose four head images and one bias strip fit the LDS, S * (4 d + 35) <= 40 000).  d in {8, 16, 32}.  No dropout (see tgt_dense_attn_dropout_fwd);
+ * the reference's unused `mask` argument is not applied. */
 int tgt_dense_attn_fwd(const void* d_q, const void* d_k, const void* d_v, const void* d_bias,
                        int b, int S, int H, int d, int dtype,
                        void* d_out, float* d_lse, void* stream);
@@ -190,6 +194,23 @@ int tgt_dense_attn_bwd(const void* d_q, const void* d_k, const void* d_v, const 
                        int b, int S, int H, int d, int dtype,
                        const void* d_out, const float* d_lse, const void* d_dout,
                        void* d_dq, void* d_dk, void* d_dv, void* d_dbias, void* stream);
+
+/* The same with attention dropout (models/graphormer_graph_level.py:207-209, attn_module.py:121: Dropout(p) on the
+ * softmax output, kept probabilities scaled by 1 / (1 - p); the reference's defaults are p = 0.1 / 0.5,
+ * utils/parser_graph_level.py:20, utils/parser_node_level.py:20).  Whether the probability of (graph, head,
+ * query, key) is kept is a counter-based hash of (seed, graph, head, query, key): the backward regenerates the
+ * forward's choice from the same (p_drop, seed), nothing is stored.  p_drop in [0, 1); p_drop = 0 is
+ * tgt_dense_attn_fwd / _bwd.  d_lse is the log-sum-exp of the undropped scores. */
+int tgt_dense_attn_dropout_fwd(const void* d_q, const void* d_k, const void* d_v, const void* d_bias,
+                               int b, int S, int H, int d, int dtype, float p_drop, uint64_t seed,
+                               void* d_out, float* d_lse, void* stream);
+int tgt_dense_attn_dropout_bwd(const void* d_q, const void* d_k, const void* d_v, const void* d_bias,
+                               int b, int S, int H, int d, int dtype, float p_drop, uint64_t seed,
+                               const void* d_out, const float* d_lse, const void* d_dout,
+                               void* d_dq, void* d_dk, void* d_dv, void* d_dbias, void* stream);
+/* d_keep: uint8 [b, H, S, S], 1 where the kernels keep the probability for (p_drop, seed) - what torch's
+ * Dropout would hold as its mask; for tests and for callers that want to inspect it. */
+int tgt_dense_attn_dropout_mask(int b, int S, int H, float p_drop, uint64_t seed, uint8_t* d_keep, void* stream);
 
 /* ---- block path: dense 16 x 16 tiles + remaining edges, one softmax per node ----
  * A tile (r0, c0) stands for the 256 edges a -> b, a in [r0, r0+16), b in

@@ -10,11 +10,12 @@ import math
 import torch
 
 
-def dense_attention(q, k, v, attn_bias=None, mask=None):
+def dense_attention(q, k, v, attn_bias=None, mask=None, drop_keep=None, p_drop=0.0):
     """q, k, v: [b, S, H, d]; attn_bias [b, H, S, S] (additive, -inf on padded
     keys); mask [b, S, S] bool or None.  NOTE the reference MULTIPLIES q by
-    sqrt(d) (graphormer_graph_level.py:198).  Dropout is the identity here
-    (eval / p = 0).  Returns [b, S, H*d]."""
+    sqrt(d) (graphormer_graph_level.py:198).  ``att_dropout`` (:208) is the identity
+    (eval / p = 0) unless ``drop_keep`` [b, H, S, S] (1 = kept) is given: torch's Dropout
+    with that mask, i.e. kept probabilities times 1 / (1 - p_drop).  Returns [b, S, H*d]."""
     b, S, H, d = q.shape
     scale = math.sqrt(d)
     qt = q.transpose(1, 2)                      # :192  [b, H, S, d]
@@ -27,6 +28,8 @@ def dense_attention(q, k, v, attn_bias=None, mask=None):
     if mask is not None:
         x = x.masked_fill(mask.unsqueeze(1), 0)  # :204-205
     x = torch.softmax(x, dim=3)                 # :207
+    if drop_keep is not None:
+        x = x * drop_keep.to(x.dtype) / (1.0 - p_drop)   # :208 with the mask made explicit
     x = x.matmul(vt)                            # :209
     x = x.transpose(1, 2).contiguous()          # :211
     return x.view(b, S, -1)                     # :212

@@ -118,3 +118,26 @@ def test_multi_hop_bias_reduces_to_the_single_hop_branch():
     a1 = oda.graph_attn_bias_multi_hop(torch.zeros_like(attn_bias), torch.full_like(sp, 2), ei, z, et, w, vd * 0, 0)
     a2 = oda.graph_attn_bias_multi_hop(torch.zeros_like(attn_bias), torch.full_like(sp, 3), ei, z, et, w, vd * 0, 0)
     torch.testing.assert_close(a1[:, :, 1:, 1:], 2 * a2[:, :, 1:, 1:], rtol=1e-12, atol=1e-13)
+
+
+def test_dropout_mask_is_dropout_of_the_softmax_output():
+    """``att_dropout`` with an explicit mask: the oracle equals softmax -> torch's dropout arithmetic (zero the
+    dropped entries, scale the kept ones by 1 / (1 - p)) -> times v, written out with loops; an all-ones mask with
+    p = 0 is the plain forward."""
+    import math
+    g = torch.Generator().manual_seed(3)
+    b, S, H, d, p = 2, 5, 2, 4, 0.25
+    q, k, v = (torch.randn(b, S, H, d, generator=g, dtype=torch.float64) for _ in range(3))
+    bias = torch.randn(b, H, S, S, generator=g, dtype=torch.float64)
+    keep = (torch.rand(b, H, S, S, generator=g) > p)
+    got = oda.dense_attention(q, k, v, bias, drop_keep=keep, p_drop=p)
+    want = torch.zeros(b, S, H * d, dtype=torch.float64)
+    for gi in range(b):
+        for h in range(H):
+            for i in range(S):
+                sc = torch.stack([(q[gi, i, h] * math.sqrt(d) * k[gi, j, h]).sum() + bias[gi, h, i, j] for j in range(S)])
+                w = torch.softmax(sc, 0) * keep[gi, h, i].double() / (1 - p)
+                want[gi, i, h * d:(h + 1) * d] = (w.unsqueeze(1) * v[gi, :, h]).sum(0)
+    assert (got - want).abs().max() < 1e-12
+    ones = torch.ones(b, H, S, S)
+    assert torch.equal(oda.dense_attention(q, k, v, bias, drop_keep=ones, p_drop=0.0), oda.dense_attention(q, k, v, bias))

@@ -11,7 +11,7 @@ LIB_PATH = os.path.join(HERE, "libtorchgt_hip.so")
 
 OK = 0
 ERR_INVALID_ARG, ERR_INDEX_RANGE, ERR_UNSUPPORTED, ERR_HIP, ERR_WORKSPACE = -1, -2, -3, -4, -5
-DTYPE_F32, DTYPE_BF16 = 0, 1
+DTYPE_F32, DTYPE_BF16, DTYPE_F32_BF16_PRODUCTS = 0, 1, 2
 BIAS_NONE, BIAS_EDGE_HEAD, BIAS_EDGE = 0, 1, 2
 BIAS_PLAN_ORDER = 0x10
 BIAS_BOTH_ORDERS = 0x20
@@ -41,6 +41,10 @@ SIGNATURES = {
     "tgt_plan_prepare": (_i32, [_vp, _i32, _i32, _vp]),
     "tgt_sparse_attn_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp,
                                    _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
+    "tgt_dense_attn_dropout_fwd": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _c.c_float, _c.c_uint64, _vp, _vp, _vp]),
+    "tgt_dense_attn_dropout_bwd": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _c.c_float, _c.c_uint64, _vp, _vp, _vp,
+                                          _vp, _vp, _vp, _vp, _vp]),
+    "tgt_dense_attn_dropout_mask": (_i32, [_i32, _i32, _i32, _c.c_float, _c.c_uint64, _vp, _vp]),
     "tgt_dense_attn_fwd": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp]),
     "tgt_dense_attn_bwd": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp,
                                   _vp, _vp, _vp, _vp, _vp]),

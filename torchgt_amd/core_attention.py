@@ -106,11 +106,14 @@ class SparseAttentionFunction(torch.autograd.Function):
 
 
 class DenseAttentionFunction(torch.autograd.Function):
-    """out[b,S,H*d] = softmax((q*sqrt(d)) k^T + bias) v, the dense ``CoreAttention.forward`` of
-    models/graphormer_graph_level.py:186-214, on the library's MFMA kernels."""
+    """out[b,S,H*d] = dropout(softmax((q*sqrt(d)) k^T + bias)) v, the dense ``CoreAttention.forward`` of
+    models/graphormer_graph_level.py:186-214.  bfloat16 tensors run on the matrix cores (bf16 products, fp32
+    accumulation and softmax); float32 tensors run in float32 arithmetic like the reference, unless
+    ``bf16_products`` asks for the matrix cores (about 2e-2 instead of 1e-5).  ``p_drop`` / ``seed``: attention
+    dropout regenerated in the backward from the same pair, no mask is stored."""
 
     @staticmethod
-    def forward(ctx, q, k, v, bias):
+    def forward(ctx, q, k, v, bias, p_drop=0.0, seed=0, bf16_products=False):
         if not (q.is_cuda and k.is_cuda and v.is_cuda):
             raise RuntimeError("dense attention needs GPU tensors (no CPU implementation)")
         if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
@@ -124,14 +127,18 @@ class DenseAttentionFunction(torch.autograd.Function):
                 raise ValueError(f"attn_bias must be {q.dtype} [b, H, S, S] = {(b, H, S, S)}, "
                                  f"got {bias.dtype} {tuple(bias.shape)}")
             bias = bias.contiguous()
+        code = _DTYPES[q.dtype]
+        if q.dtype == torch.float32 and bf16_products:
+            code = _lib.DTYPE_F32_BF16_PRODUCTS
         out = torch.empty((b, S, H * d), dtype=q.dtype, device=q.device)
         lse = torch.empty((b, H, S), dtype=torch.float32, device=q.device)
         with torch.cuda.device(q.device):
             stream = torch.cuda.current_stream(q.device).cuda_stream
-            _lib.check(_lib.lib().tgt_dense_attn_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(bias), b, S, H, d,
-                                                     _DTYPES[q.dtype], _ptr(out), _ptr(lse), stream))
+            _lib.check(_lib.lib().tgt_dense_attn_dropout_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(bias), b, S, H, d, code,
+                                                             float(p_drop), int(seed), _ptr(out), _ptr(lse), stream))
         ctx.save_for_backward(q, k, v, bias, out, lse)
         ctx.has_bias = bias is not None
+        ctx.code, ctx.p_drop, ctx.seed = code, float(p_drop), int(seed)
         return out
 
     @staticmethod
@@ -143,22 +150,36 @@ class DenseAttentionFunction(torch.autograd.Function):
         dbias = torch.empty_like(bias) if (ctx.has_bias and ctx.needs_input_grad[3]) else None
         with torch.cuda.device(q.device):
             stream = torch.cuda.current_stream(q.device).cuda_stream
-            _lib.check(_lib.lib().tgt_dense_attn_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(bias), b, S, H, d,
-                                                     _DTYPES[q.dtype], _ptr(out), _ptr(lse), _ptr(dout),
-                                                     _ptr(dq), _ptr(dk), _ptr(dv), _ptr(dbias), stream))
-        return dq, dk, dv, dbias
+            _lib.check(_lib.lib().tgt_dense_attn_dropout_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(bias), b, S, H, d, ctx.code,
+                                                             ctx.p_drop, ctx.seed, _ptr(out), _ptr(lse), _ptr(dout),
+                                                             _ptr(dq), _ptr(dk), _ptr(dv), _ptr(dbias), stream))
+        return dq, dk, dv, dbias, None, None, None
 
 
-def dense_attention(q, k, v, attn_bias=None):
+def dense_dropout_mask(b, S, H, p_drop, seed, device):
+    """uint8 [b, H, S, S]: 1 where the dense kernels keep a probability for (p_drop, seed) - the mask torch's
+    Dropout would hold."""
+    keep = torch.empty((b, H, S, S), dtype=torch.uint8, device=device)
+    with torch.cuda.device(device):
+        _lib.check(_lib.lib().tgt_dense_attn_dropout_mask(b, S, H, float(p_drop), int(seed), keep.data_ptr(),
+                                                          torch.cuda.current_stream(device).cuda_stream))
+    return keep
+
+
+def dense_attention(q, k, v, attn_bias=None, p_drop=0.0, seed=None, bf16_products=False):
     """Functional form of the dense path: q, k, v [b, S, H, d], attn_bias [b, H, S, S] or None;
     returns [b, S, H*d].  A bias of another float dtype or with a broadcast head axis
-    ([b, 1, S, S]) is converted / expanded here, where autograd sees it."""
+    ([b, 1, S, S]) is converted / expanded here, where autograd sees it.  ``p_drop`` > 0 applies attention
+    dropout; ``seed`` (default: drawn from torch's CPU generator, so ``torch.manual_seed`` governs it) names
+    the mask."""
     if attn_bias is not None:
         b, S, H = q.shape[0], q.shape[1], q.shape[2]
         if attn_bias.dim() == 4 and attn_bias.shape[1] == 1 and H != 1:
             attn_bias = attn_bias.expand(b, H, S, S)
         attn_bias = attn_bias.to(q.dtype)
-    return DenseAttentionFunction.apply(q, k, v, attn_bias)
+    if p_drop > 0 and seed is None:
+        seed = int(torch.randint(0, 2 ** 62, (1,)).item())
+    return DenseAttentionFunction.apply(q, k, v, attn_bias, p_drop, seed or 0, bf16_products)
 
 
 def sparse_attention(q, k, v, edge_index=None, edge_bias=None, plan=None, return_z=False, bias_in_plan_order=False):
@@ -240,6 +261,9 @@ class CoreAttention(nn.Module):
         fourth = extra[0] if extra else kw.get("attn_bias_dim", kw.get("device"))
         self.attn_bias_dim = fourth if isinstance(fourth, int) else None
         self.dense_bias_layout = "bssh" if self.attn_bias_dim is not None else "bhss"
+        # float32 dense attention runs in float32 arithmetic like the reference; True moves its products to the
+        # bf16 matrix cores (faster, about 2e-2 instead of 1e-5)
+        self.dense_bf16_products = False
 
     # -- helpers ---------------------------------------------------------
     def _edge_bias(self, attn_bias, edge_index):
@@ -284,11 +308,10 @@ class CoreAttention(nn.Module):
         if mask is not None:
             raise NotImplementedError("the reference never passes `mask` (graphormer_graph_level.py:380); "
                                       "it is not supported")
-        if self.training and self.attention_dropout_rate > 0:
-            raise NotImplementedError(
-                "attention dropout inside the dense kernel is not implemented; construct CoreAttention "
-                "with attention_dropout_rate=0 or call it in eval mode")
-        return dense_attention(q, k, v, attn_bias)
+        # the reference applies att_dropout to the softmax output (graphormer_graph_level.py:207-209); here the
+        # kernels do, in training mode
+        p = float(self.attention_dropout_rate) if self.training else 0.0
+        return dense_attention(q, k, v, attn_bias, p_drop=p, bf16_products=self.dense_bf16_products)
 
     def forward(self, q, k, v, attn_bias=None, edge_index=None, attn_type=None, mask=None,
                 flash_attn=False, full=False):

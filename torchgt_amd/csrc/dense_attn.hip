@@ -19,6 +19,7 @@
 // The bias is read straight from global memory in the layout each walk needs (see
 // key_of_row and the backward kernel); only q/k/v/dout heads are staged in LDS.
 #include "common.h"
+#include "dense_dropout.h"
 #include <algorithm>
 #include <stdlib.h>
 
@@ -219,11 +220,11 @@ __device__ __forceinline__ void store_row(T* __restrict__ p, const float (&x)[D]
 }
 
 // forward of the rows first .. first + count - 1 (all keys), by one wave
-template <typename T, int D, int SP>
+template <typename T, int D, int SP, bool DROP>
 __device__ __forceinline__ void thin_rows_fwd(const T* __restrict__ Q, const short* __restrict__ k_rm,
                                               const short* __restrict__ v_tr, const T* __restrict__ bias_gh,
                                               T* __restrict__ out, float* __restrict__ lse, int g, int h, int S, int H,
-                                              float scale, int first, int count, int lane) {
+                                              float scale, int first, int count, int lane, const DropArgs da) {
     constexpr int NC = (SP + 63) / 64;
     for (int tq = 0; tq < count; ++tq) {
         const int qi = first + tq;
@@ -251,33 +252,36 @@ __device__ __forceinline__ void thin_rows_fwd(const T* __restrict__ Q, const sho
         float lsum = 0.f, ov[D];
 #pragma unroll
         for (int d = 0; d < D; ++d) ov[d] = 0.f;
+        const uint32_t rh = DROP ? drop_row_hash(da, g * H + h, qi) : 0u;
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             const int key = c * 64 + lane;
             if (key < S) {
                 const float pb = round_bf(fast_exp2((sv[c] - m_use) * kLog2e));
                 lsum += pb;
+                const float pk = (!DROP || drop_keep(da, rh, key)) ? pb : 0.f;
 #pragma unroll
-                for (int d = 0; d < D; ++d) ov[d] = fmaf(pb, bf2f(v_tr[d * (SP + 4) + key]), ov[d]);
+                for (int d = 0; d < D; ++d) ov[d] = fmaf(pk, bf2f(v_tr[d * (SP + 4) + key]), ov[d]);
             }
         }
         lsum = wave_sum(lsum);
 #pragma unroll
         for (int d = 0; d < D; ++d) ov[d] = wave_sum(ov[d]);
         if (lane == 0) {
-            store_row<T, D>(out + (((int64_t)g * S + qi) * H + h) * D, ov, 1.0f / lsum);
+            store_row<T, D>(out + (((int64_t)g * S + qi) * H + h) * D, ov, (DROP ? da.inv_keep : 1.0f) / lsum);
             lse[((int64_t)g * H + h) * S + qi] = m_use + __logf(lsum);
         }
     }
 }
 
 // backward, query side, of the rows first .. first + count - 1: dQ and their rows of dBias
-template <typename T, int D, int SP>
+template <typename T, int D, int SP, bool DROP>
 __device__ __forceinline__ void thin_rows_bwd_q(const short* __restrict__ q_rm, const short* __restrict__ k_rm,
                                                 const short* __restrict__ v_rm, const short* __restrict__ g_rm,
                                                 const float* __restrict__ lse_l, const float* __restrict__ dd_l,
                                                 const T* __restrict__ bias_gh, T* __restrict__ dbias_gh, T* __restrict__ dQ,
-                                                int g, int h, int S, int H, float scale, int first, int count, int lane) {
+                                                int g, int h, int S, int H, float scale, int first, int count, int lane,
+                                                const DropArgs da) {
     constexpr int NC = (SP + 63) / 64;
     const float scale2 = scale * kLog2e;
     for (int tq = 0; tq < count; ++tq) {
@@ -288,6 +292,7 @@ __device__ __forceinline__ void thin_rows_bwd_q(const short* __restrict__ q_rm, 
 #pragma unroll
         for (int d = 0; d < D; ++d) dq[d] = 0.f;
         const float nL2 = -lse_l[qi], Dq = dd_l[qi];
+        const uint32_t rh = DROP ? drop_row_hash(da, g * H + h, qi) : 0u;
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             const int key = c * 64 + lane;
@@ -297,7 +302,8 @@ __device__ __forceinline__ void thin_rows_bwd_q(const short* __restrict__ q_rm, 
                 lds_row<D>(v_rm, key, vv);
                 const float b = bias_gh ? ld1(bias_gh + (int64_t)qi * S + key) : 0.f;
                 const float pv = fast_exp2(fmaf(dot_d<D>(qv, kv), scale2, fmaf(b, kLog2e, nL2)));
-                const float dS = pv * (dot_d<D>(gv, vv) - Dq);
+                const float ks = !DROP ? 1.0f : (drop_keep(da, rh, key) ? da.inv_keep : 0.f);
+                const float dS = pv * (dot_d<D>(gv, vv) * ks - Dq);
                 if (dbias_gh) st1(dbias_gh + (int64_t)qi * S + key, dS);
                 const float dsb = round_bf(dS);
 #pragma unroll
@@ -311,12 +317,13 @@ __device__ __forceinline__ void thin_rows_bwd_q(const short* __restrict__ q_rm, 
 }
 
 // backward, key side, of the keys first .. first + count - 1 (all queries): dK and dV
-template <typename T, int D, int SP>
+template <typename T, int D, int SP, bool DROP>
 __device__ __forceinline__ void thin_rows_bwd_k(const short* __restrict__ q_rm, const short* __restrict__ k_rm,
                                                 const short* __restrict__ v_rm, const short* __restrict__ g_rm,
                                                 const float* __restrict__ lse_l, const float* __restrict__ dd_l,
                                                 const T* __restrict__ bias_gh, T* __restrict__ dK, T* __restrict__ dV,
-                                                int g, int h, int S, int H, float scale, int first, int count, int lane) {
+                                                int g, int h, int S, int H, float scale, int first, int count, int lane,
+                                                const DropArgs da) {
     constexpr int NC = (SP + 63) / 64;
     const float scale2 = scale * kLog2e;
     for (int tk = 0; tk < count; ++tk) {
@@ -335,8 +342,9 @@ __device__ __forceinline__ void thin_rows_bwd_k(const short* __restrict__ q_rm, 
                 lds_row<D>(g_rm, qq, gv);
                 const float b = bias_gh ? ld1(bias_gh + (int64_t)qq * S + ki) : 0.f;
                 const float pv = fast_exp2(fmaf(dot_d<D>(qv, kv), scale2, fmaf(b, kLog2e, -lse_l[qq])));
-                const float dS = pv * (dot_d<D>(gv, vv) - dd_l[qq]);
-                const float pb = round_bf(pv), dsb = round_bf(dS);
+                const float ks = !DROP ? 1.0f : (drop_keep(da, drop_row_hash(da, g * H + h, qq), ki) ? da.inv_keep : 0.f);
+                const float dS = pv * (dot_d<D>(gv, vv) * ks - dd_l[qq]);
+                const float pb = round_bf(pv * ks), dsb = round_bf(dS);
 #pragma unroll
                 for (int d = 0; d < D; ++d) {
                     dk[d] = fmaf(dsb, qv[d], dk[d]);
@@ -356,11 +364,11 @@ __device__ __forceinline__ void thin_rows_bwd_k(const short* __restrict__ q_rm, 
 // ---------------------------------------------------------------------------
 // forward: online softmax over key tiles, in the base-2 domain
 // ---------------------------------------------------------------------------
-template <typename T, int D, int NT>
+template <typename T, int D, int NT, bool DROP>
 __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, const T* __restrict__ K,
                                                        const T* __restrict__ V, const T* __restrict__ bias,
                                                        T* __restrict__ out, float* __restrict__ lse, int S,
-                                                       int H, float scale, int nb) {
+                                                       int H, float scale, int nb, const DropArgs da) {
     constexpr int KS = D / 8;
     constexpr int SP = NT * 32;
     extern __shared__ __align__(16) char smem[];
@@ -400,15 +408,17 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
     }
     __syncthreads();
     if (vec_wave) {
-        thin_rows_fwd<T, D, SP>(Q, k_rm, v_tr, hasb ? bias + ((int64_t)g * H + h) * S * S : nullptr, out, lse, g, h, S, H,
-                                scale, (NT - 1) * 32, S - (NT - 1) * 32, lane);
+        thin_rows_fwd<T, D, SP, DROP>(Q, k_rm, v_tr, hasb ? bias + ((int64_t)g * H + h) * S * S : nullptr, out, lse, g, h, S,
+                                      H, scale, (NT - 1) * 32, S - (NT - 1) * 32, lane, da);
     } else {
     const int krow = key_of_row(col);            // key (inside a tile) of this lane's A-operand row
     // Row sums on the matrix unit: with a head dim below 32 the A operand of O^T = V^T P^T has idle
     // rows, and a row of ones there makes row D of the product the sum of the (bf16-rounded)
     // probabilities, the very numbers the numerator was built from.  It is C register 4*KS of the lower half.
-    constexpr bool kSumOnMfma = D < 32;
+    // (not with dropout: the sum runs over all probabilities, the numerator over the kept ones)
+    constexpr bool kSumOnMfma = D < 32 && !DROP;
     const short one_bits = 0x3f80;               // bf16 1.0
+    const uint32_t rh = DROP ? drop_row_hash(da, g * H + h, qi) : 0u;
     float m = -INFINITY, l = 0.f;                // running maximum and sum (natural units)
     float16_t o = zero16();
     const int tail = S - (NT - 1) * 32;          // keys in the last tile
@@ -449,6 +459,7 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
         for (int r = 0; r < 16; ++r) {
             sc[r] = fast_exp2(fmaf(sc[r], kLog2e, nm2));
             if (!kSumOnMfma) l += sc[r];
+            if (DROP) sc[r] = drop_keep(da, rh, kb + r) ? sc[r] : 0.f;
         }
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
@@ -490,6 +501,7 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
         for (int r = 0; r < 4; ++r) {
             s4[r] = fast_exp2(fmaf(s4[r], kLog2e, nm2));
             if (!kSumOnMfma) l += s4[r];
+            if (DROP) s4[r] = drop_keep(da, rh, kb + r) ? s4[r] : 0.f;
         }
         short4_t pb;
         pb.x = f2bf(s4[0]); pb.y = f2bf(s4[1]); pb.z = f2bf(s4[2]); pb.w = f2bf(s4[3]);
@@ -502,7 +514,7 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
     if (kSumOnMfma) l = __shfl(o[4 * KS], col);      // row D sits in the lower half's register 4*KS
     else l += __shfl_xor(l, 32);
     if (qok) {
-        const float inv = 1.0f / l;
+        const float inv = (DROP ? da.inv_keep : 1.0f) / l;
         T* op = out + (((int64_t)g * S + qi) * H + h) * D;
 #pragma unroll
         for (int rb = 0; rb < KS; ++rb)
@@ -524,13 +536,14 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
 // bias straight from global memory in the layout their lanes need (a lane's own row
 // in the first, 32 lanes on 32 consecutive keys of one row in the second); the second
 // read of a (graph, head) slice comes from L2.
-template <typename T, int D, int NT>
+template <typename T, int D, int NT, bool DROP>
 __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, const T* __restrict__ K,
                                                        const T* __restrict__ V, const T* __restrict__ bias,
                                                        const T* __restrict__ O, const float* __restrict__ lse,
                                                        const T* __restrict__ dO, T* __restrict__ dQ,
                                                        T* __restrict__ dK, T* __restrict__ dV,
-                                                       T* __restrict__ dbias, int S, int H, float scale, int nb) {
+                                                       T* __restrict__ dbias, int S, int H, float scale, int nb,
+                                                       const DropArgs da) {
     constexpr int KS = D / 8;
     constexpr int SP = NT * 32;
     extern __shared__ __align__(16) char smem[];
@@ -589,9 +602,9 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
 
     // ---- query tile `wave`: dQ -------------------------------------------------
     if (vec_wave) {
-        thin_rows_bwd_q<T, D, SP>(q_rm, k_rm, v_rm, g_rm, lse_l, dd_l, bias_gh,
-                                  dbias != nullptr ? dbias + ((int64_t)g * H + h) * S * S : nullptr, dQ, g, h, S, H, scale,
-                                  (NT - 1) * 32, tail, lane);
+        thin_rows_bwd_q<T, D, SP, DROP>(q_rm, k_rm, v_rm, g_rm, lse_l, dd_l, bias_gh,
+                                        dbias != nullptr ? dbias + ((int64_t)g * H + h) * S * S : nullptr, dQ, g, h, S, H,
+                                        scale, (NT - 1) * 32, tail, lane, da);
     } else {
         short4_t bq[KS], bg[KS];
 #pragma unroll
@@ -602,6 +615,7 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
         const float nL2 = -lse_l[qi], Dq = dd_l[qi];
         const float scale2 = scale * kLog2e;
         const int krow = key_of_row(col);
+        const uint32_t rh = DROP ? drop_row_hash(da, g * H + h, qi) : 0u;
         T* dbrow = dbias != nullptr ? dbias + (((int64_t)g * H + h) * S + (qok ? qi : 0)) * S : nullptr;
         float16_t dq = zero16();
 #pragma unroll 1
@@ -623,6 +637,7 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const float pv = fast_exp2(fmaf(sc[r], scale2, fmaf(bcur.get(r), kLog2e, nL2)));
+                if (DROP) dp[r] = drop_keep(da, rh, kb + r) ? dp[r] * da.inv_keep : 0.f;
                 sc[r] = pv * (dp[r] - Dq);
             }
             if (kt * 32 + 32 > S) {               // the row ends inside this tile (wave-uniform)
@@ -674,6 +689,7 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const float pv = fast_exp2(fmaf(sc[r], scale2, fmaf(bcur.get(r), kLog2e, nL2)));
+                if (DROP) dp[r] = drop_keep(da, rh, kb + r) ? dp[r] * da.inv_keep : 0.f;
                 s4[r] = (half == 0 && r < tail) ? pv * (dp[r] - Dq) : 0.f;
             }
             if (dbrow != nullptr && qok && half == 0) {
@@ -698,8 +714,8 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
 
     // ---- key tile `wave`: dK, dV -------------------------------------------------
     if (vec_wave) {
-        thin_rows_bwd_k<T, D, SP>(q_rm, k_rm, v_rm, g_rm, lse_l, dd_l, bias_gh, dK, dV, g, h, S, H, scale, (NT - 1) * 32, tail,
-                                  lane);
+        thin_rows_bwd_k<T, D, SP, DROP>(q_rm, k_rm, v_rm, g_rm, lse_l, dd_l, bias_gh, dK, dV, g, h, S, H, scale,
+                                        (NT - 1) * 32, tail, lane, da);
     } else {
         const int k0 = wave * 32, ki = k0 + col;
         const bool kok = ki < S;
@@ -752,7 +768,10 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
                 for (int t = 0; t < 4; ++t) {
                     const int r = 4 * j + t;
                     pr[r] = fast_exp2(fmaf(sc[r], scale2, fmaf(cvt1(braw[r]), kLog2e, -L4[t])));
-                    sc[r] = pr[r] * (dp[r] - D4[t]);
+                    float ks = 1.0f;
+                    if (DROP) ks = drop_keep(da, drop_row_hash(da, g * H + h, qb + t), ki) ? da.inv_keep : 0.f;
+                    sc[r] = pr[r] * (dp[r] * ks - D4[t]);
+                    if (DROP) pr[r] *= ks;
                 }
             }
             if (!full) {                          // queries past the end of the batch entry (wave-uniform branch)
@@ -800,8 +819,10 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
             for (int t = 0; t < 4; ++t) {
                 const bool in = half == 0 && t < tail;
                 const float pv = fast_exp2(fmaf(sc[t], scale2, fmaf(cvt1(braw[t]), kLog2e, -L4[t])));
-                p4[t] = in ? pv : 0.f;
-                s4[t] = in ? pv * (dp[t] - D4[t]) : 0.f;
+                float ks = 1.0f;
+                if (DROP) ks = drop_keep(da, drop_row_hash(da, g * H + h, qb + t), ki) ? da.inv_keep : 0.f;
+                p4[t] = in ? pv * ks : 0.f;
+                s4[t] = in ? pv * (dp[t] * ks - D4[t]) : 0.f;
             }
             short4_t db, pb;
             db.x = f2bf(s4[0]); db.y = f2bf(s4[1]); db.z = f2bf(s4[2]); db.w = f2bf(s4[3]);
@@ -837,6 +858,8 @@ struct DenseCall {
     float* o_lse;
     int b, S, H, d;
     hipStream_t st;
+    float p_drop;          // 0: no dropout
+    uint64_t seed;
 };
 
 template <typename T, int D, int NT>
@@ -851,12 +874,18 @@ static int launch_dense(const DenseCall& c, bool bwd) {
         const dim3 block(64 * NT);
         static bool attr_done = false;     // raise the dynamic-LDS cap once per instantiation
         if (!attr_done) {
-            if (lds_f > 48 * 1024)
-                TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_dense_fwd<T, D, NT>),
+            if (lds_f > 48 * 1024) {
+                TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_dense_fwd<T, D, NT, false>),
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds_f));
-            if (lds_b > 48 * 1024)
-                TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_dense_bwd<T, D, NT>),
+                TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_dense_fwd<T, D, NT, true>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_f));
+            }
+            if (lds_b > 48 * 1024) {
+                TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_dense_bwd<T, D, NT, false>),
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds_b));
+                TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_dense_bwd<T, D, NT, true>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_b));
+            }
             attr_done = true;
         }
         const int total_pairs = ((c.b + 7) / 8) * 8 * c.H;
@@ -872,15 +901,26 @@ static int launch_dense(const DenseCall& c, bool bwd) {
         }
         const int nblk = bwd ? total_pairs : std::min(total_pairs, fwd_grid);
         const dim3 grid((unsigned)nblk);
+        const bool drop = c.p_drop > 0.f;
+        const DropArgs da = drop_args(c.p_drop, c.seed);
         if (!bwd) {
             KernelTimer t(KS_DENSE_FWD, c.st);
-            hipLaunchKernelGGL((k_dense_fwd<T, D, NT>), grid, block, lds_f, c.st, (const T*)c.q, (const T*)c.k,
-                               (const T*)c.v, (const T*)c.bias, (T*)c.o_out, c.o_lse, c.S, c.H, scale, c.b);
+            if (drop)
+                hipLaunchKernelGGL((k_dense_fwd<T, D, NT, true>), grid, block, lds_f, c.st, (const T*)c.q, (const T*)c.k,
+                                   (const T*)c.v, (const T*)c.bias, (T*)c.o_out, c.o_lse, c.S, c.H, scale, c.b, da);
+            else
+                hipLaunchKernelGGL((k_dense_fwd<T, D, NT, false>), grid, block, lds_f, c.st, (const T*)c.q, (const T*)c.k,
+                                   (const T*)c.v, (const T*)c.bias, (T*)c.o_out, c.o_lse, c.S, c.H, scale, c.b, da);
         } else {
             KernelTimer t(KS_DENSE_BWD, c.st);
-            hipLaunchKernelGGL((k_dense_bwd<T, D, NT>), grid, block, lds_b, c.st, (const T*)c.q, (const T*)c.k,
-                               (const T*)c.v, (const T*)c.bias, (const T*)c.out, c.lse, (const T*)c.dout,
-                               (T*)c.dq, (T*)c.dk, (T*)c.dv, (T*)c.dbias, c.S, c.H, scale, c.b);
+            if (drop)
+                hipLaunchKernelGGL((k_dense_bwd<T, D, NT, true>), grid, block, lds_b, c.st, (const T*)c.q, (const T*)c.k,
+                                   (const T*)c.v, (const T*)c.bias, (const T*)c.out, c.lse, (const T*)c.dout,
+                                   (T*)c.dq, (T*)c.dk, (T*)c.dv, (T*)c.dbias, c.S, c.H, scale, c.b, da);
+            else
+                hipLaunchKernelGGL((k_dense_bwd<T, D, NT, false>), grid, block, lds_b, c.st, (const T*)c.q, (const T*)c.k,
+                                   (const T*)c.v, (const T*)c.bias, (const T*)c.out, c.lse, (const T*)c.dout,
+                                   (T*)c.dq, (T*)c.dk, (T*)c.dv, (T*)c.dbias, c.S, c.H, scale, c.b, da);
         }
         TGT_HIP_CHECK(hipGetLastError());
         return TGT_OK;
@@ -916,10 +956,25 @@ static int dispatch_d(const DenseCall& c, bool bwd) {
     }
 }
 
+// keep[g, h, q, k] (1 = kept) of the dropout the attention kernels apply for (p, seed)
+__global__ void k_dropout_mask(uint8_t* __restrict__ out, int S, int H, int64_t total, const DropArgs da) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int k = (int)(i % S);
+    const int64_t r = i / S;
+    const int q = (int)(r % S);
+    const int pair = (int)(r / S);
+    out[i] = drop_keep(da, drop_row_hash(da, pair, q), k) ? 1 : 0;
+}
+
 static int check_dense(const void* q, const void* k, const void* v, int b, int S, int H, int d, int dtype) {
     if (!q || !k || !v) { set_error("dense attention: null q/k/v"); return TGT_ERR_INVALID_ARG; }
     if (b < 1 || S < 1 || H < 1 || d < 1) { set_error("dense attention: non-positive size"); return TGT_ERR_INVALID_ARG; }
-    if (dtype != TGT_DTYPE_F32 && dtype != TGT_DTYPE_BF16) { set_error("bad dtype %d", dtype); return TGT_ERR_INVALID_ARG; }
+    if (dtype != TGT_DTYPE_F32 && dtype != TGT_DTYPE_BF16 && dtype != TGT_DTYPE_F32_BF16_PRODUCTS) {
+        set_error("bad dtype %d", dtype);
+        return TGT_ERR_INVALID_ARG;
+    }
+    if (S > 256 && dtype != TGT_DTYPE_F32) { set_error("dense attention: sequence length %d exceeds 256", S); return TGT_ERR_UNSUPPORTED; }
     if ((int64_t)b * H > 0x7fffffffLL) { set_error("dense attention: b*H too large"); return TGT_ERR_INVALID_ARG; }
     return TGT_OK;
 }
@@ -928,22 +983,58 @@ static int check_dense(const void* q, const void* k, const void* v, int b, int S
 
 extern "C" {
 
-int tgt_dense_attn_fwd(const void* d_q, const void* d_k, const void* d_v, const void* d_bias, int b, int S, int H,
-                       int d, int dtype, void* d_out, float* d_lse, void* stream) {
+int tgt_dense_attn_dropout_fwd(const void* d_q, const void* d_k, const void* d_v, const void* d_bias, int b, int S,
+                               int H, int d, int dtype, float p_drop, uint64_t seed, void* d_out, float* d_lse,
+                               void* stream) {
     int rc = tgt::check_dense(d_q, d_k, d_v, b, S, H, d, dtype);
     if (rc) return rc;
     if (!d_out || !d_lse) { tgt::set_error("dense attention: null out or lse"); return TGT_ERR_INVALID_ARG; }
+    if (!(p_drop >= 0.f && p_drop < 1.f)) { tgt::set_error("dense attention: dropout rate %g outside [0, 1)", p_drop); return TGT_ERR_INVALID_ARG; }
     tgt::DenseCall c{};
     c.q = d_q; c.k = d_k; c.v = d_v; c.bias = d_bias; c.o_out = d_out; c.o_lse = d_lse;
     c.b = b; c.S = S; c.H = H; c.d = d; c.st = (hipStream_t)stream;
-    return dtype == TGT_DTYPE_F32 ? tgt::dispatch_d<float>(c, false) : tgt::dispatch_d<tgt::dbf16>(c, false);
+    c.p_drop = p_drop; c.seed = seed;
+    if (dtype == TGT_DTYPE_F32) {
+        tgt::DenseF32Call f{};
+        f.q = (const float*)d_q; f.k = (const float*)d_k; f.v = (const float*)d_v; f.bias = (const float*)d_bias;
+        f.o_out = (float*)d_out; f.o_lse = d_lse; f.b = b; f.S = S; f.H = H; f.d = d; f.st = c.st;
+        f.p_drop = p_drop; f.seed = seed;
+        return tgt::dense_attn_f32(f, false);
+    }
+    return dtype == TGT_DTYPE_F32_BF16_PRODUCTS ? tgt::dispatch_d<float>(c, false) : tgt::dispatch_d<tgt::dbf16>(c, false);
+}
+
+int tgt_dense_attn_fwd(const void* d_q, const void* d_k, const void* d_v, const void* d_bias, int b, int S, int H,
+                       int d, int dtype, void* d_out, float* d_lse, void* stream) {
+    return tgt_dense_attn_dropout_fwd(d_q, d_k, d_v, d_bias, b, S, H, d, dtype, 0.f, 0, d_out, d_lse, stream);
+}
+
+int tgt_dense_attn_dropout_mask(int b, int S, int H, float p_drop, uint64_t seed, uint8_t* d_keep, void* stream) {
+    if (b < 1 || S < 1 || H < 1 || !d_keep || !(p_drop >= 0.f && p_drop < 1.f)) {
+        tgt::set_error("tgt_dense_attn_dropout_mask: bad size, null pointer or rate outside [0, 1)");
+        return TGT_ERR_INVALID_ARG;
+    }
+    const int64_t total = (int64_t)b * H * S * S;
+    hipLaunchKernelGGL(tgt::k_dropout_mask, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, d_keep,
+                       S, H, total, tgt::drop_args(p_drop, seed));
+    TGT_HIP_CHECK(hipGetLastError());
+    return TGT_OK;
 }
 
 int tgt_dense_attn_bwd(const void* d_q, const void* d_k, const void* d_v, const void* d_bias, int b, int S, int H,
                        int d, int dtype, const void* d_out, const float* d_lse, const void* d_dout, void* d_dq,
                        void* d_dk, void* d_dv, void* d_dbias, void* stream) {
+    return tgt_dense_attn_dropout_bwd(d_q, d_k, d_v, d_bias, b, S, H, d, dtype, 0.f, 0, d_out, d_lse, d_dout, d_dq, d_dk,
+                                      d_dv, d_dbias, stream);
+}
+
+int tgt_dense_attn_dropout_bwd(const void* d_q, const void* d_k, const void* d_v, const void* d_bias, int b, int S,
+                               int H, int d, int dtype, float p_drop, uint64_t seed, const void* d_out,
+                               const float* d_lse, const void* d_dout, void* d_dq, void* d_dk, void* d_dv,
+                               void* d_dbias, void* stream) {
     int rc = tgt::check_dense(d_q, d_k, d_v, b, S, H, d, dtype);
     if (rc) return rc;
+    if (!(p_drop >= 0.f && p_drop < 1.f)) { tgt::set_error("dense attention: dropout rate %g outside [0, 1)", p_drop); return TGT_ERR_INVALID_ARG; }
     if (!d_out || !d_lse || !d_dout || !d_dq || !d_dk || !d_dv) {
         tgt::set_error("dense attention backward: null out/lse/dout/dq/dk/dv");
         return TGT_ERR_INVALID_ARG;
@@ -952,7 +1043,16 @@ int tgt_dense_attn_bwd(const void* d_q, const void* d_k, const void* d_v, const 
     c.q = d_q; c.k = d_k; c.v = d_v; c.bias = d_bias; c.out = d_out; c.lse = d_lse; c.dout = d_dout;
     c.dq = d_dq; c.dk = d_dk; c.dv = d_dv; c.dbias = d_dbias;
     c.b = b; c.S = S; c.H = H; c.d = d; c.st = (hipStream_t)stream;
-    return dtype == TGT_DTYPE_F32 ? tgt::dispatch_d<float>(c, true) : tgt::dispatch_d<tgt::dbf16>(c, true);
+    c.p_drop = p_drop; c.seed = seed;
+    if (dtype == TGT_DTYPE_F32) {
+        tgt::DenseF32Call f{};
+        f.q = (const float*)d_q; f.k = (const float*)d_k; f.v = (const float*)d_v; f.bias = (const float*)d_bias;
+        f.out = (const float*)d_out; f.lse = d_lse; f.dout = (const float*)d_dout;
+        f.dq = (float*)d_dq; f.dk = (float*)d_dk; f.dv = (float*)d_dv; f.dbias = (float*)d_dbias;
+        f.b = b; f.S = S; f.H = H; f.d = d; f.st = c.st; f.p_drop = p_drop; f.seed = seed;
+        return tgt::dense_attn_f32(f, true);
+    }
+    return dtype == TGT_DTYPE_F32_BF16_PRODUCTS ? tgt::dispatch_d<float>(c, true) : tgt::dispatch_d<tgt::dbf16>(c, true);
 }
 
 }  // extern "C"
