@@ -61,8 +61,8 @@ def kernel_alg_bytes(name, N, E, H, d, esize, bpe):
 # profiles/sparse_attn_config2_hbm_traffic_pmc.txt.  Counters cannot be read from inside this process,
 # so the figures are carried here and only reported for the workload / dtype they were measured on.
 MEASURED_TRAFFIC = {
-    ("config2", "f32"): {"attn_fwd": 252.4e6, "bwd_node_side": 38.9e6, "attn_bwd": 637.1e6},
-    ("config2", "bf16"): {"attn_fwd": 138.3e6, "bwd_node_side": 22.6e6, "attn_bwd": 371.7e6},
+    ("config2", "f32"): {"attn_fwd": 242.6e6, "bwd_node_side": 38.9e6, "attn_bwd": 577.7e6},
+    ("config2", "bf16"): {"attn_fwd": 131.4e6, "bwd_node_side": 22.6e6, "attn_bwd": 324.0e6},
 }
 
 
