@@ -50,3 +50,18 @@ def test_host_only_entry_points():
     assert L.tgt_sparse_attn_workspace_bytes(None, 8, 8) == -1
     assert L.tgt_sparse_attn_fwd(None, None, None, None, None, 0, 8, 8, 0, None, None, None, 0, None) \
         == _lib.ERR_INVALID_ARG
+
+
+def test_torch_extension_loads_and_registers_its_operators():
+    """The PyTorch-ROCm extension (csrc/torch_binding.cpp) loads without a GPU, registers every operator the Python
+    layer calls, and refuses CPU tensors instead of falling back."""
+    import torch
+    from torchgt_amd import _ext
+    ops = _ext.ops()
+    for name in ("sparse_attention", "dense_attention", "linear", "add_layer_norm", "add", "gelu", "relu"):
+        assert hasattr(ops, name), name
+    assert hasattr(torch.classes.torchgt, "PlanHolder")
+    with pytest.raises(RuntimeError, match="GPU"):
+        ops.gelu(torch.zeros(8))
+    with pytest.raises(RuntimeError, match="GPU"):
+        ops.linear(torch.zeros(4, 8), [torch.zeros(8, 8)], [None])

@@ -208,14 +208,13 @@ def test_rows_sum_to_one_property_full_size(cuda):
 
 def test_dense_loud_failures(cuda):
     q = torch.randn(2, 300, 2, 8, device=cuda, dtype=torch.bfloat16)
-    with pytest.raises(_lib.TorchGTHipError) as exc:
-        dense_attention(q, q, q)
-    assert exc.value.code == _lib.ERR_UNSUPPORTED          # S > 256
+    with pytest.raises(RuntimeError, match="exceeds 256"):
+        dense_attention(q, q, q)                            # S > 256 on the matrix path
     q = torch.randn(2, 10, 2, 12, device=cuda, dtype=torch.bfloat16)
-    with pytest.raises(_lib.TorchGTHipError):
+    with pytest.raises(RuntimeError, match="head dim"):
         dense_attention(q, q, q)                            # head dim 12
     q = torch.randn(2, 10, 8, 8, device=cuda)
-    with pytest.raises(_lib.TorchGTHipError):
+    with pytest.raises(RuntimeError, match="dropout rate"):
         dense_attention(q, q, q, p_drop=1.0, seed=1)        # rate outside [0, 1)
     with pytest.raises(RuntimeError):
         dense_attention(q.cpu(), q.cpu(), q.cpu())

@@ -54,9 +54,8 @@ def test_add_layer_norm_forward_backward(cuda, dtype, C):
 def test_layer_norm_rejects_unsupported_width(cuda):
     x = torch.zeros(4, 24, device=cuda)
     w = torch.ones(24, device=cuda)
-    with pytest.raises(_lib.TorchGTHipError) as ei:
+    with pytest.raises(RuntimeError, match="unsupported"):
         AddLayerNormFunction.apply(x, None, w, w, 1e-5)          # 24 / 4 = 6 lanes: not a power of two
-    assert ei.value.code == _lib.ERR_UNSUPPORTED
     with pytest.raises(RuntimeError):
         GeluFunction.apply(torch.zeros(8))                        # CPU tensor: no fallback
 

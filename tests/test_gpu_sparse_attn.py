@@ -268,9 +268,8 @@ def test_module_api_matches_reference_conventions(cuda):
 def test_loud_failures(cuda):
     q = torch.randn(10, 8, 4, device=cuda)        # d = 4: no kernel
     ei = torch.tensor([[0, 1], [1, 2]], device=cuda)
-    with pytest.raises(_lib.TorchGTHipError) as exc:
+    with pytest.raises(RuntimeError, match="unsupported"):     # the C entry point's error, through the torch operator
         sparse_attention(q, q, q, ei)
-    assert exc.value.code == _lib.ERR_UNSUPPORTED
     qc = torch.randn(10, 8, 8)
     with pytest.raises(RuntimeError):
         sparse_attention(qc, qc, qc, ei.cpu())     # CPU tensors: no fallback

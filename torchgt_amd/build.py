@@ -14,6 +14,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 LIB_PATH = os.path.join(HERE, "libtorchgt_hip.so")
+EXT_SRC = os.path.join(CSRC, "torch_binding.cpp")
+EXT_PATH = os.path.join(HERE, "_torchgt_ext.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # packed-fp32 instructions are switched off on purpose: the compiler otherwise
@@ -78,7 +80,29 @@ def build(verbose=True):
     os.replace(tmp, LIB_PATH)
     if verbose:
         print(f"[torchgt_amd.build] linked {LIB_PATH}")
+    build_extension(verbose)
     return LIB_PATH
+
+
+def build_extension(verbose=True):
+    """The PyTorch-ROCm extension: host code only (g++), torch's headers, linked against libtorchgt_hip.so
+    next to it (rpath $ORIGIN) and torch's libraries."""
+    import torch
+    from torch.utils import cpp_extension
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__", "-DUSE_ROCM",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}"]
+    cmd += [f"-I{p}" for p in cpp_extension.include_paths()] + ["-I/opt/rocm/include", EXT_SRC, "-o", EXT_PATH + ".tmp",
+            f"-L{tlib}", "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_hip", f"-L{HERE}", "-ltorchgt_hip",
+            "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{tlib}"]
+    t0 = time.time()
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building the torch extension failed:\n" + r.stdout + r.stderr)
+    os.replace(EXT_PATH + ".tmp", EXT_PATH)
+    if verbose:
+        print(f"[torchgt_amd.build] torch_binding.cpp: {time.time() - t0:.1f}s -> {EXT_PATH}")
+    return EXT_PATH
 
 
 if __name__ == "__main__":

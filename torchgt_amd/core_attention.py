@@ -19,7 +19,7 @@ import weakref
 import torch
 import torch.nn as nn
 
-from . import _lib
+from . import _ext, _lib
 from .plan import GraphPlan, get_plan
 
 _DTYPES = {torch.float32: _lib.DTYPE_F32, torch.bfloat16: _lib.DTYPE_BF16}
@@ -29,13 +29,13 @@ def _ptr(t):
     return t.data_ptr() if t is not None else None
 
 
-class SparseAttentionFunction(torch.autograd.Function):
-    """out[N,H,d] = sparse_attention(q, k, v, plan, edge_bias) with the backward
-    kernels of the library (the reference relies on autograd through ATen /
-    torch_scatter ops, attn_module.py:146-187)."""
+class SparseAttentionFunction:
+    """out[N,H,d], Z[N,H] = sparse_attention(q, k, v, plan, edge_bias): ``torch.ops.torchgt.sparse_attention`` (a C++
+    autograd function over ``tgt_sparse_attn_fwd`` / ``_bwd``; the reference relies on autograd through ATen /
+    torch_scatter ops, attn_module.py:146-187).  ``apply`` keeps the call convention of an autograd function."""
 
     @staticmethod
-    def forward(ctx, q, k, v, edge_bias, plan, bias_in_plan_order=False):
+    def apply(q, k, v, edge_bias, plan, bias_in_plan_order=False):
         if not (q.is_cuda and k.is_cuda and v.is_cuda):
             raise RuntimeError("sparse attention needs GPU tensors (no CPU implementation)")
         if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
@@ -45,12 +45,10 @@ class SparseAttentionFunction(torch.autograd.Function):
         N, H, d = q.shape
         if N != plan.num_nodes:
             raise ValueError(f"q has {N} rows but the plan was built for {plan.num_nodes} nodes")
-        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
         mode = _lib.BIAS_NONE
         if edge_bias is not None:
             if edge_bias.dtype != q.dtype:
                 raise TypeError("edge bias must have the dtype of q (convert it outside, where autograd sees it)")
-            edge_bias = edge_bias.contiguous()
             E = plan.num_edges
             both = bias_in_plan_order and edge_bias.shape[0] == 2 * E and E > 0
             rows = 2 * E if both else E
@@ -66,94 +64,20 @@ class SparseAttentionFunction(torch.autograd.Function):
                     mode |= _lib.BIAS_BOTH_ORDERS      # [2E, ...]: destination-sorted rows, then source-sorted rows
                 else:
                     plan.edge_order()                  # makes sure the plan holds the map for this mode
-        out = torch.empty_like(q)
-        Z = torch.empty((N, H), dtype=torch.float32, device=q.device)
-        ws = plan.workspace(H, d)
-        with torch.cuda.device(q.device):
-            stream = torch.cuda.current_stream(q.device).cuda_stream
-            _lib.check(_lib.lib().tgt_sparse_attn_fwd(
-                plan.handle, _ptr(q), _ptr(k), _ptr(v), _ptr(edge_bias), mode, H, d, _DTYPES[q.dtype],
-                _ptr(out), _ptr(Z), _ptr(ws), ws.numel(), stream))
-        ctx.plan = plan
-        ctx.mode = mode
-        ctx.has_bias = edge_bias is not None
-        ctx.save_for_backward(q, k, v, edge_bias, out, Z)
-        ctx.mark_non_differentiable(Z)
-        return out, Z
-
-    @staticmethod
-    def backward(ctx, dout, _dZ):
-        q, k, v, edge_bias, out, Z = ctx.saved_tensors
-        plan = ctx.plan
-        N, H, d = q.shape
-        dout = dout.contiguous()
-        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-        dbias = None
-        if ctx.has_bias and ctx.needs_input_grad[3]:
-            dbias = torch.empty_like(edge_bias)
-            if ctx.mode & _lib.BIAS_BOTH_ORDERS:
-                dbias[plan.num_edges:].zero_()      # the source-sorted copy gets no gradient of its own
-        if ctx.mode & _lib.BIAS_PLAN_ORDER:
-            _BIAS_CACHE.clear()     # the step is over: the next forward brings its bias into plan order afresh
-        ws = plan.workspace(H, d)
-        with torch.cuda.device(q.device):
-            stream = torch.cuda.current_stream(q.device).cuda_stream
-            _lib.check(_lib.lib().tgt_sparse_attn_bwd(
-                plan.handle, _ptr(q), _ptr(k), _ptr(v), _ptr(edge_bias), ctx.mode, H, d, _DTYPES[q.dtype],
-                _ptr(out), _ptr(Z), _ptr(dout), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(dbias),
-                _ptr(ws), ws.numel(), stream))
-        return dq, dk, dv, dbias, None, None
+        plan.handle      # raises if the plan was closed
+        return _ext.ops().sparse_attention(q, k, v, edge_bias, plan.holder, mode, plan.workspace(H, d))
 
 
-class DenseAttentionFunction(torch.autograd.Function):
+class DenseAttentionFunction:
     """out[b,S,H*d] = dropout(softmax((q*sqrt(d)) k^T + bias)) v, the dense ``CoreAttention.forward`` of
-    models/graphormer_graph_level.py:186-214.  bfloat16 tensors run on the matrix cores (bf16 products, fp32
-    accumulation and softmax); float32 tensors run in float32 arithmetic like the reference, unless
-    ``bf16_products`` asks for the matrix cores (about 2e-2 instead of 1e-5).  ``p_drop`` / ``seed``: attention
-    dropout regenerated in the backward from the same pair, no mask is stored."""
+    models/graphormer_graph_level.py:186-214: ``torch.ops.torchgt.dense_attention``.  bfloat16 tensors run on the
+    matrix cores (bf16 products, fp32 accumulation and softmax); float32 tensors run in float32 arithmetic like the
+    reference, unless ``bf16_products`` asks for the matrix cores (about 2e-2 instead of 1e-5).  ``p_drop`` / ``seed``:
+    attention dropout regenerated in the backward from the same pair, no mask is stored."""
 
     @staticmethod
-    def forward(ctx, q, k, v, bias, p_drop=0.0, seed=0, bf16_products=False):
-        if not (q.is_cuda and k.is_cuda and v.is_cuda):
-            raise RuntimeError("dense attention needs GPU tensors (no CPU implementation)")
-        if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
-            raise TypeError(f"q/k/v must share dtype float32 or bfloat16, got {q.dtype}/{k.dtype}/{v.dtype}")
-        if q.dim() != 4 or q.shape != k.shape or q.shape != v.shape:
-            raise ValueError("q, k, v must be [b, S, H, d] with equal shapes")
-        b, S, H, d = q.shape
-        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-        if bias is not None:
-            if tuple(bias.shape) != (b, H, S, S) or bias.dtype != q.dtype:
-                raise ValueError(f"attn_bias must be {q.dtype} [b, H, S, S] = {(b, H, S, S)}, "
-                                 f"got {bias.dtype} {tuple(bias.shape)}")
-            bias = bias.contiguous()
-        code = _DTYPES[q.dtype]
-        if q.dtype == torch.float32 and bf16_products:
-            code = _lib.DTYPE_F32_BF16_PRODUCTS
-        out = torch.empty((b, S, H * d), dtype=q.dtype, device=q.device)
-        lse = torch.empty((b, H, S), dtype=torch.float32, device=q.device)
-        with torch.cuda.device(q.device):
-            stream = torch.cuda.current_stream(q.device).cuda_stream
-            _lib.check(_lib.lib().tgt_dense_attn_dropout_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(bias), b, S, H, d, code,
-                                                             float(p_drop), int(seed), _ptr(out), _ptr(lse), stream))
-        ctx.save_for_backward(q, k, v, bias, out, lse)
-        ctx.has_bias = bias is not None
-        ctx.code, ctx.p_drop, ctx.seed = code, float(p_drop), int(seed)
-        return out
-
-    @staticmethod
-    def backward(ctx, dout):
-        q, k, v, bias, out, lse = ctx.saved_tensors
-        b, S, H, d = q.shape
-        dout = dout.contiguous()
-        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-        dbias = torch.empty_like(bias) if (ctx.has_bias and ctx.needs_input_grad[3]) else None
-        with torch.cuda.device(q.device):
-            stream = torch.cuda.current_stream(q.device).cuda_stream
-            _lib.check(_lib.lib().tgt_dense_attn_dropout_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(bias), b, S, H, d, ctx.code,
-                                                             ctx.p_drop, ctx.seed, _ptr(out), _ptr(lse), _ptr(dout),
-                                                             _ptr(dq), _ptr(dk), _ptr(dv), _ptr(dbias), stream))
-        return dq, dk, dv, dbias, None, None, None
+    def apply(q, k, v, bias, p_drop=0.0, seed=0, bf16_products=False):
+        return _ext.ops().dense_attention(q, k, v, bias, float(p_drop), int(seed), bool(bf16_products))
 
 
 def dense_dropout_mask(b, S, H, p_drop, seed, device):
@@ -214,6 +138,10 @@ def gather_dense_bias(attn_bias, edge_index, layout):
     return attn_bias[src // S, src % S, dst % S, :]
 
 
+def _drop_bias_cache(_grad):
+    _BIAS_CACHE.clear()
+
+
 _BIAS_CACHE = {}      # at most one entry: the per-edge bias in plan order of the bias tensor seen last
 
 
@@ -222,7 +150,7 @@ def _plan_order_bias(module, attn_bias, edge_index, plan, dtype):
     forward pass get one and the same bias tensor: the first brings it into plan order, the others reuse the
     result.  The entry is tied to the tensor (held weakly), its version, the plan, the dtype and the autograd
     state it was made under - a result made under ``no_grad`` carries no graph and is not handed to a pass that
-    needs one - and it is dropped by the first backward that follows, so neither the bias nor its 2E-row copy
+    needs one - and it is dropped when the backward of any layer that used it begins, so neither the bias nor its 2E-row copy
     outlives the step.  Differentiable."""
     key = (id(attn_bias), attn_bias._version, id(plan), dtype, module.dense_bias_layout,
            torch.is_grad_enabled(), attn_bias.requires_grad)
@@ -289,6 +217,8 @@ class CoreAttention(nn.Module):
         # (by the first layer that sees it) and every layer then streams it.
         eb = _plan_order_bias(self, attn_bias, edge_index, plan, q3.dtype)
         out, _ = SparseAttentionFunction.apply(q3, k3, v3, eb, plan, True)
+        if out.requires_grad:
+            out.register_hook(_drop_bias_cache)     # the backward has begun: the step's forward passes are over
         return out
 
     # -- reference method names -------------------------------------------

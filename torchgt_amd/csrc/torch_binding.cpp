@@ -1,0 +1,392 @@
+// PyTorch-ROCm binding of the library's hot operators: TORCH_LIBRARY ops with C++ autograd functions over the C ABI
+// of include/torchgt_hip.h.  Host code only (g++): it validates the tensors, allocates the outputs with torch's
+// allocator, takes the current HIP stream and calls the C entry points; nothing else happens between Python and
+// the kernels.  The reference has no such layer - its hot path is a chain of ATen / torch_scatter calls from Python
+// (attn_module.py:133-189, models/graphormer_dist_node_level.py:246-314) - these ops stand where that chain stood.
+//
+//   torchgt::sparse_attention(q, k, v, bias?, plan holder, bias_mode, workspace) -> (out, Z)
+//   torchgt::dense_attention(q, k, v, bias?, p_drop, seed, bf16_products) -> out
+//   torchgt::linear(x, weights[], biases?[]) -> Tensor[]                      (1 to 3 layers of one shape)
+//   torchgt::add_layer_norm(x, r?, gamma, beta, eps) -> (sum, y)
+//   torchgt::add(x, r) -> sum
+//   torchgt::gelu(u) / torchgt::relu(u) -> h
+#include <torch/library.h>
+#include <torch/custom_class.h>
+#include <torch/autograd.h>
+#include <ATen/ATen.h>
+#include <c10/hip/HIPStream.h>
+#include <c10/core/DeviceGuard.h>
+
+#include "../../include/torchgt_hip.h"
+
+namespace {
+
+using at::Tensor;
+using torch::autograd::AutogradContext;
+using torch::autograd::variable_list;
+
+void check(int rc, const char* what) {
+    TORCH_CHECK(rc == TGT_OK, what, ": ", tgt_error_string(rc), " (", tgt_last_error(), ")");
+}
+int dtype_code(const Tensor& t) {
+    if (t.scalar_type() == at::kFloat) return TGT_DTYPE_F32;
+    if (t.scalar_type() == at::kBFloat16) return TGT_DTYPE_BF16;
+    TORCH_CHECK(false, "torchgt: unsupported dtype ", t.scalar_type(), " (float32 or bfloat16)");
+}
+void* stream_of(const Tensor& t) { return c10::hip::getCurrentHIPStream(t.device().index()).stream(); }
+const void* ptr(const c10::optional<Tensor>& t) { return (t.has_value() && t->defined()) ? t->data_ptr() : nullptr; }
+void on_gpu(const Tensor& t, const char* op) {
+    TORCH_CHECK(t.is_cuda(), op, " needs GPU tensors (there is no CPU implementation)");
+}
+
+// Owner of a tgt_plan_t: the Python plan object holds one, and so does every autograd node that will need the plan
+// in its backward - the plan lives until the last of them lets go.
+struct PlanHolder : torch::CustomClassHolder {
+    int64_t h;
+    explicit PlanHolder(int64_t handle) : h(handle) {}
+    ~PlanHolder() override {
+        if (h) tgt_plan_destroy(reinterpret_cast<tgt_plan_t*>(h));
+    }
+    int64_t handle() const { return h; }
+};
+
+// ---------------------------------------------------------------------------------------------------------------
+// sparse attention
+// ---------------------------------------------------------------------------------------------------------------
+struct SparseAttention : public torch::autograd::Function<SparseAttention> {
+    static variable_list forward(AutogradContext* ctx, Tensor q, Tensor k, Tensor v, c10::optional<Tensor> bias,
+                                 c10::intrusive_ptr<PlanHolder> holder, int64_t mode, Tensor ws) {
+        const int64_t plan = holder->h;
+        on_gpu(q, "sparse attention");
+        TORCH_CHECK(q.dim() == 3 && q.sizes() == k.sizes() && q.sizes() == v.sizes(), "q, k, v must be [N, H, d] with equal shapes");
+        TORCH_CHECK(k.scalar_type() == q.scalar_type() && v.scalar_type() == q.scalar_type(), "q/k/v must share a dtype");
+        const int code = dtype_code(q);
+        q = q.contiguous(); k = k.contiguous(); v = v.contiguous();
+        Tensor b;
+        if (bias.has_value() && bias->defined()) {
+            TORCH_CHECK(bias->scalar_type() == q.scalar_type(), "edge bias must have the dtype of q");
+            b = bias->contiguous();
+        }
+        const int64_t N = q.size(0), H = q.size(1), d = q.size(2);
+        c10::DeviceGuard guard(q.device());
+        Tensor out = at::empty_like(q);
+        Tensor Z = at::empty({N, H}, q.options().dtype(at::kFloat));
+        check(tgt_sparse_attn_fwd(reinterpret_cast<const tgt_plan_t*>(plan), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                  b.defined() ? b.data_ptr() : nullptr, (int)mode, (int)H, (int)d, code, out.data_ptr(),
+                                  Z.data_ptr<float>(), ws.data_ptr(), ws.numel(), stream_of(q)),
+              "tgt_sparse_attn_fwd");
+        ctx->save_for_backward({q, k, v, b, out, Z, ws});
+        ctx->saved_data["plan"] = holder;
+        ctx->saved_data["mode"] = mode;
+        ctx->saved_data["bias_grad"] = b.defined() && bias->requires_grad();
+        ctx->mark_non_differentiable({Z});
+        return {out, Z};
+    }
+    static variable_list backward(AutogradContext* ctx, variable_list grads) {
+        auto saved = ctx->get_saved_variables();
+        const Tensor &q = saved[0], &k = saved[1], &v = saved[2], &b = saved[3], &out = saved[4], &Z = saved[5], &ws = saved[6];
+        const int64_t plan = ctx->saved_data["plan"].toCustomClass<PlanHolder>()->h, mode = ctx->saved_data["mode"].toInt();
+        const int64_t H = q.size(1), d = q.size(2);
+        Tensor dout = grads[0].contiguous();
+        c10::DeviceGuard guard(q.device());
+        Tensor dq = at::empty_like(q), dk = at::empty_like(k), dv = at::empty_like(v), dbias;
+        if (b.defined() && ctx->saved_data["bias_grad"].toBool()) {
+            dbias = at::empty_like(b);
+            if (mode & TGT_BIAS_BOTH_ORDERS) dbias.narrow(0, b.size(0) / 2, b.size(0) / 2).zero_();   // the source-sorted copy gets none
+        }
+        check(tgt_sparse_attn_bwd(reinterpret_cast<const tgt_plan_t*>(plan), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                  b.defined() ? b.data_ptr() : nullptr, (int)mode, (int)H, (int)d, dtype_code(q), out.data_ptr(),
+                                  Z.data_ptr<float>(), dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+                                  dbias.defined() ? dbias.data_ptr() : nullptr, ws.data_ptr(), ws.numel(), stream_of(q)),
+              "tgt_sparse_attn_bwd");
+        return {dq, dk, dv, dbias, Tensor(), Tensor(), Tensor()};
+    }
+};
+std::tuple<Tensor, Tensor> sparse_attention(const Tensor& q, const Tensor& k, const Tensor& v, const c10::optional<Tensor>& bias,
+                                            const c10::intrusive_ptr<PlanHolder>& plan, int64_t mode, const Tensor& ws) {
+    auto r = SparseAttention::apply(q, k, v, bias, plan, mode, ws);
+    return {r[0], r[1]};
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// dense attention
+// ---------------------------------------------------------------------------------------------------------------
+struct DenseAttention : public torch::autograd::Function<DenseAttention> {
+    static Tensor forward(AutogradContext* ctx, Tensor q, Tensor k, Tensor v, c10::optional<Tensor> bias, double p_drop,
+                          int64_t seed, bool bf16_products) {
+        on_gpu(q, "dense attention");
+        TORCH_CHECK(q.dim() == 4 && q.sizes() == k.sizes() && q.sizes() == v.sizes(), "q, k, v must be [b, S, H, d] with equal shapes");
+        TORCH_CHECK(k.scalar_type() == q.scalar_type() && v.scalar_type() == q.scalar_type(), "q/k/v must share a dtype");
+        int code = dtype_code(q);
+        if (code == TGT_DTYPE_F32 && bf16_products) code = TGT_DTYPE_F32_BF16_PRODUCTS;
+        q = q.contiguous(); k = k.contiguous(); v = v.contiguous();
+        const int64_t b = q.size(0), S = q.size(1), H = q.size(2), d = q.size(3);
+        Tensor bb;
+        if (bias.has_value() && bias->defined()) {
+            TORCH_CHECK(bias->scalar_type() == q.scalar_type() && bias->dim() == 4 && bias->size(0) == b && bias->size(1) == H &&
+                            bias->size(2) == S && bias->size(3) == S,
+                        "attn_bias must be [b, H, S, S] of q's dtype");
+            bb = bias->contiguous();
+        }
+        c10::DeviceGuard guard(q.device());
+        Tensor out = at::empty({b, S, H * d}, q.options());
+        Tensor lse = at::empty({b, H, S}, q.options().dtype(at::kFloat));
+        check(tgt_dense_attn_dropout_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), bb.defined() ? bb.data_ptr() : nullptr, (int)b,
+                                         (int)S, (int)H, (int)d, code, (float)p_drop, (uint64_t)seed, out.data_ptr(),
+                                         lse.data_ptr<float>(), stream_of(q)),
+              "tgt_dense_attn_dropout_fwd");
+        ctx->save_for_backward({q, k, v, bb, out, lse});
+        ctx->saved_data["code"] = (int64_t)code;
+        ctx->saved_data["p"] = p_drop;
+        ctx->saved_data["seed"] = seed;
+        ctx->saved_data["bias_grad"] = bb.defined() && bias->requires_grad();
+        return out;
+    }
+    static variable_list backward(AutogradContext* ctx, variable_list grads) {
+        auto saved = ctx->get_saved_variables();
+        const Tensor &q = saved[0], &k = saved[1], &v = saved[2], &bb = saved[3], &out = saved[4], &lse = saved[5];
+        const int64_t b = q.size(0), S = q.size(1), H = q.size(2), d = q.size(3);
+        Tensor dout = grads[0].contiguous();
+        c10::DeviceGuard guard(q.device());
+        Tensor dq = at::empty_like(q), dk = at::empty_like(k), dv = at::empty_like(v), dbias;
+        if (bb.defined() && ctx->saved_data["bias_grad"].toBool()) dbias = at::empty_like(bb);
+        check(tgt_dense_attn_dropout_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), bb.defined() ? bb.data_ptr() : nullptr, (int)b,
+                                         (int)S, (int)H, (int)d, (int)ctx->saved_data["code"].toInt(),
+                                         (float)ctx->saved_data["p"].toDouble(), (uint64_t)ctx->saved_data["seed"].toInt(),
+                                         out.data_ptr(), lse.data_ptr<float>(), dout.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                                         dv.data_ptr(), dbias.defined() ? dbias.data_ptr() : nullptr, stream_of(q)),
+              "tgt_dense_attn_dropout_bwd");
+        return {dq, dk, dv, dbias, Tensor(), Tensor(), Tensor()};
+    }
+};
+Tensor dense_attention(const Tensor& q, const Tensor& k, const Tensor& v, const c10::optional<Tensor>& bias, double p_drop,
+                       int64_t seed, bool bf16_products) {
+    return DenseAttention::apply(q, k, v, bias, p_drop, seed, bf16_products);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// 1 to 3 linear layers of one shape on the same input
+// ---------------------------------------------------------------------------------------------------------------
+struct Linear : public torch::autograd::Function<Linear> {
+    // wb: the n weights, then the biases that exist (bit j of bias_mask: layer j has one), in layer order
+    static variable_list forward(AutogradContext* ctx, Tensor x, at::TensorList wb, int64_t n64, int64_t bias_mask) {
+        on_gpu(x, "linear");
+        const int n = (int)n64;
+        TORCH_CHECK(n >= 1 && n <= 3 && (int)wb.size() >= n, "linear takes 1 to 3 (weight, bias) pairs");
+        const int code = dtype_code(x);
+        const int64_t out_f = wb[0].size(0), in_f = wb[0].size(1);
+        TORCH_CHECK(x.size(-1) == in_f, "x has ", x.size(-1), " features, the weights take ", in_f);
+        Tensor x2 = x.reshape({-1, in_f}).contiguous();
+        const int64_t N = x2.size(0);
+        std::vector<Tensor> save{x2};
+        const void *W[3] = {nullptr, nullptr, nullptr}, *B[3] = {nullptr, nullptr, nullptr};
+        void* Y[3] = {nullptr, nullptr, nullptr};
+        variable_list ys;
+        c10::DeviceGuard guard(x.device());
+        std::vector<Tensor> keep;
+        int next_bias = n;
+        for (int j = 0; j < n; ++j) {
+            const Tensor& w = wb[j];
+            TORCH_CHECK(w.dim() == 2 && w.size(0) == out_f && w.size(1) == in_f && w.scalar_type() == x.scalar_type(),
+                        "all weights must be [out, in] of x's dtype");
+            Tensor wc = w.contiguous();
+            save.push_back(wc);
+            W[j] = wc.data_ptr();
+            if (bias_mask & (1 << j)) {
+                TORCH_CHECK(next_bias < (int)wb.size(), "fewer biases than the mask says");
+                const Tensor& bj = wb[next_bias++];
+                TORCH_CHECK(bj.numel() == out_f && bj.scalar_type() == x.scalar_type(), "all biases must be [out] of x's dtype");
+                keep.push_back(bj.contiguous());
+                B[j] = keep.back().data_ptr();
+            }
+            ys.push_back(at::empty({N, out_f}, x.options()));
+            Y[j] = ys.back().data_ptr();
+        }
+        check(tgt_linear_fwd(x2.data_ptr(), W, B, Y, n, N, (int)in_f, (int)out_f, code, stream_of(x)), "tgt_linear_fwd");
+        ctx->save_for_backward(save);
+        ctx->saved_data["bias_mask"] = bias_mask;
+        ctx->saved_data["x_shape"] = x.sizes().vec();
+        std::vector<int64_t> oshape(x.sizes().vec());
+        oshape.back() = out_f;
+        for (auto& y : ys) y = y.view(oshape);
+        return ys;
+    }
+    static variable_list backward(AutogradContext* ctx, variable_list dys) {
+        auto saved = ctx->get_saved_variables();
+        const Tensor& x2 = saved[0];
+        const int n = (int)saved.size() - 1;
+        const int64_t out_f = saved[1].size(0), in_f = saved[1].size(1), N = x2.size(0);
+        const int64_t bias_mask = ctx->saved_data["bias_mask"].toInt();
+        int n_bias = 0;
+        for (int j = 0; j < n; ++j) n_bias += (bias_mask >> j) & 1;
+        const bool need_dx = ctx->needs_input_grad(0);
+        bool need_dw = false;
+        for (int j = 0; j < n + n_bias; ++j) need_dw = need_dw || ctx->needs_input_grad(1 + j);
+        c10::DeviceGuard guard(x2.device());
+        const void *W[3] = {nullptr, nullptr, nullptr}, *DY[3] = {nullptr, nullptr, nullptr};
+        void *DW[3] = {nullptr, nullptr, nullptr}, *DB[3] = {nullptr, nullptr, nullptr};
+        std::vector<Tensor> dyc, dWs(n), dbs(n);
+        for (int j = 0; j < n; ++j) {
+            W[j] = saved[1 + j].data_ptr();
+            dyc.push_back(dys[j].defined() ? dys[j].reshape({N, out_f}).contiguous() : at::zeros({N, out_f}, x2.options()));
+            DY[j] = dyc.back().data_ptr();
+            if (need_dw) {
+                dWs[j] = at::empty_like(saved[1 + j]);
+                DW[j] = dWs[j].data_ptr();
+                if (bias_mask & (1 << j)) {
+                    dbs[j] = at::empty({out_f}, x2.options());
+                    DB[j] = dbs[j].data_ptr();
+                }
+            }
+        }
+        Tensor dx, ws;
+        if (need_dx) dx = at::empty_like(x2);
+        int64_t ws_bytes = 0;
+        if (need_dw) {
+            ws_bytes = tgt_linear_bwd_workspace_bytes(n, (int)in_f, (int)out_f);
+            ws = at::empty({ws_bytes}, x2.options().dtype(at::kByte));
+        }
+        check(tgt_linear_bwd(x2.data_ptr(), W, DY, n, N, (int)in_f, (int)out_f, dtype_code(x2), need_dx ? dx.data_ptr() : nullptr,
+                             need_dw ? DW : nullptr, need_dw ? DB : nullptr, need_dw ? ws.data_ptr() : nullptr, ws_bytes,
+                             stream_of(x2)),
+              "tgt_linear_bwd");
+        variable_list out;
+        out.push_back(need_dx ? dx.view(ctx->saved_data["x_shape"].toIntVector()) : Tensor());
+        for (int j = 0; j < n; ++j) out.push_back(dWs[j]);
+        for (int j = 0; j < n; ++j)
+            if (bias_mask & (1 << j)) out.push_back(dbs[j]);
+        out.push_back(Tensor());     // n
+        out.push_back(Tensor());     // bias_mask
+        return out;
+    }
+};
+std::vector<Tensor> linear(const Tensor& x, at::TensorList weights, const c10::List<c10::optional<Tensor>>& biases) {
+    TORCH_CHECK(weights.size() == biases.size(), "one bias slot per weight");
+    variable_list wb(weights.begin(), weights.end());
+    int64_t mask = 0;
+    for (size_t j = 0; j < biases.size(); ++j) {
+        c10::optional<Tensor> b = biases.get(j);
+        if (b.has_value() && b->defined()) {
+            wb.push_back(*b);
+            mask |= (int64_t)1 << j;
+        }
+    }
+    return Linear::apply(x, at::TensorList(wb), (int64_t)weights.size(), mask);      // a TensorList: every entry is an autograd input
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// residual add + LayerNorm, add, GELU / ReLU
+// ---------------------------------------------------------------------------------------------------------------
+struct AddLayerNorm : public torch::autograd::Function<AddLayerNorm> {
+    static variable_list forward(AutogradContext* ctx, Tensor x, c10::optional<Tensor> r, Tensor gamma, Tensor beta, double eps) {
+        on_gpu(x, "add_layer_norm");
+        const int code = dtype_code(x);
+        const int64_t C = x.size(-1);
+        Tensor x2 = x.reshape({-1, C}).contiguous(), r2;
+        const bool has_r = r.has_value() && r->defined();
+        if (has_r) r2 = r->reshape({-1, C}).contiguous();
+        const int64_t N = x2.size(0);
+        c10::DeviceGuard guard(x.device());
+        Tensor s = has_r ? at::empty_like(x2) : x2, y = at::empty_like(x2);
+        Tensor mean = at::empty({N}, x.options().dtype(at::kFloat)), rstd = at::empty({N}, x.options().dtype(at::kFloat));
+        Tensor g = gamma.contiguous(), b = beta.contiguous();
+        check(tgt_add_layer_norm_fwd(x2.data_ptr(), has_r ? r2.data_ptr() : nullptr, g.data_ptr(), b.data_ptr(), N, (int)C, (float)eps,
+                                     code, has_r ? s.data_ptr() : nullptr, y.data_ptr(), mean.data_ptr<float>(),
+                                     rstd.data_ptr<float>(), stream_of(x)),
+              "tgt_add_layer_norm_fwd");
+        ctx->save_for_backward({s, g, mean, rstd});
+        ctx->saved_data["has_r"] = has_r;
+        ctx->saved_data["shape"] = x.sizes().vec();
+        return {s.view(x.sizes()), y.view(x.sizes())};
+    }
+    static variable_list backward(AutogradContext* ctx, variable_list grads) {
+        auto saved = ctx->get_saved_variables();
+        const Tensor &s = saved[0], &g = saved[1], &mean = saved[2], &rstd = saved[3];
+        const int64_t N = s.size(0), C = s.size(1);
+        c10::DeviceGuard guard(s.device());
+        Tensor dy = grads[1].defined() ? grads[1].reshape({N, C}).contiguous() : at::zeros_like(s);
+        Tensor extra;
+        if (grads[0].defined()) extra = grads[0].reshape({N, C}).contiguous();
+        Tensor ds = at::empty_like(s), dg = at::empty_like(g), db = at::empty_like(g);
+        const int64_t nbytes = tgt_layer_norm_bwd_workspace_bytes((int)C);
+        Tensor ws = at::empty({nbytes}, s.options().dtype(at::kByte));
+        check(tgt_layer_norm_bwd(s.data_ptr(), g.data_ptr(), mean.data_ptr<float>(), rstd.data_ptr<float>(), dy.data_ptr(),
+                                 extra.defined() ? extra.data_ptr() : nullptr, N, (int)C, dtype_code(s), ds.data_ptr(), dg.data_ptr(),
+                                 db.data_ptr(), ws.data_ptr(), nbytes, stream_of(s)),
+              "tgt_layer_norm_bwd");
+        Tensor dsv = ds.view(ctx->saved_data["shape"].toIntVector());
+        return {dsv, ctx->saved_data["has_r"].toBool() ? dsv : Tensor(), dg, db, Tensor()};
+    }
+};
+std::tuple<Tensor, Tensor> add_layer_norm(const Tensor& x, const c10::optional<Tensor>& r, const Tensor& gamma, const Tensor& beta,
+                                          double eps) {
+    auto o = AddLayerNorm::apply(x, r, gamma, beta, eps);
+    return {o[0], o[1]};
+}
+
+struct Add : public torch::autograd::Function<Add> {
+    static Tensor forward(AutogradContext* ctx, Tensor x, Tensor r) {
+        on_gpu(x, "add");
+        const int64_t C = x.size(-1);
+        Tensor x2 = x.reshape({-1, C}).contiguous(), r2 = r.reshape({-1, C}).contiguous();
+        c10::DeviceGuard guard(x.device());
+        Tensor s = at::empty_like(x2);
+        check(tgt_add_layer_norm_fwd(x2.data_ptr(), r2.data_ptr(), nullptr, nullptr, x2.size(0), (int)C, 0.f, dtype_code(x), s.data_ptr(),
+                                     nullptr, nullptr, nullptr, stream_of(x)),
+              "tgt_add_layer_norm_fwd");
+        return s.view(x.sizes());
+    }
+    static variable_list backward(AutogradContext*, variable_list grads) { return {grads[0], grads[0]}; }
+};
+Tensor add(const Tensor& x, const Tensor& r) { return Add::apply(x, r); }
+
+template <bool GELU>
+struct Activation : public torch::autograd::Function<Activation<GELU>> {
+    static Tensor forward(AutogradContext* ctx, Tensor u) {
+        on_gpu(u, GELU ? "gelu" : "relu");
+        Tensor u2 = u.contiguous();
+        c10::DeviceGuard guard(u.device());
+        Tensor h = at::empty_like(u2);
+        check((GELU ? tgt_gelu_fwd : tgt_relu_fwd)(u2.data_ptr(), u2.numel(), dtype_code(u), h.data_ptr(), stream_of(u)),
+              GELU ? "tgt_gelu_fwd" : "tgt_relu_fwd");
+        ctx->save_for_backward({u2});
+        return h;
+    }
+    static variable_list backward(AutogradContext* ctx, variable_list grads) {
+        const Tensor u = ctx->get_saved_variables()[0];
+        Tensor dh = grads[0].contiguous();
+        c10::DeviceGuard guard(u.device());
+        Tensor du = at::empty_like(u);
+        check((GELU ? tgt_gelu_bwd : tgt_relu_bwd)(u.data_ptr(), dh.data_ptr(), u.numel(), dtype_code(u), du.data_ptr(), stream_of(u)),
+              GELU ? "tgt_gelu_bwd" : "tgt_relu_bwd");
+        return {du};
+    }
+};
+Tensor gelu(const Tensor& u) { return Activation<true>::apply(u); }
+Tensor relu(const Tensor& u) { return Activation<false>::apply(u); }
+
+}  // namespace
+
+TORCH_LIBRARY(torchgt, m) {
+    m.class_<PlanHolder>("PlanHolder").def(torch::init<int64_t>()).def("handle", &PlanHolder::handle);
+    m.def("sparse_attention(Tensor q, Tensor k, Tensor v, Tensor? bias, __torch__.torch.classes.torchgt.PlanHolder plan, int bias_mode, "
+          "Tensor workspace) -> (Tensor, Tensor)");
+    m.def("dense_attention(Tensor q, Tensor k, Tensor v, Tensor? bias, float p_drop, int seed, bool bf16_products) -> Tensor");
+    m.def("linear(Tensor x, Tensor[] weights, Tensor?[] biases) -> Tensor[]");
+    m.def("add_layer_norm(Tensor x, Tensor? r, Tensor gamma, Tensor beta, float eps) -> (Tensor, Tensor)");
+    m.def("add(Tensor x, Tensor r) -> Tensor");
+    m.def("gelu(Tensor u) -> Tensor");
+    m.def("relu(Tensor u) -> Tensor");
+}
+
+// One implementation per op, registered for every backend and for autograd alike: each is an autograd function
+// whose forward calls the C ABI directly (no further dispatch).
+TORCH_LIBRARY_IMPL(torchgt, CompositeImplicitAutograd, m) {
+    m.impl("sparse_attention", sparse_attention);
+    m.impl("dense_attention", dense_attention);
+    m.impl("linear", linear);
+    m.impl("add_layer_norm", add_layer_norm);
+    m.impl("add", add);
+    m.impl("gelu", gelu);
+    m.impl("relu", relu);
+}

@@ -18,101 +18,33 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from . import _lib
+from . import _ext, _lib
 from .multi_head_attention import MultiHeadAttention, fused_linear, _DT
 
 
-def _stream(t):
-    return torch.cuda.current_stream(t.device).cuda_stream
-
-
-class AddLayerNormFunction(torch.autograd.Function):
-    """``s = x + r`` (r may be None) and ``y = LayerNorm(s)`` in one pass; returns (s, y)."""
+class AddLayerNormFunction:
+    """``s = x + r`` (r may be None) and ``y = LayerNorm(s)`` in one pass; returns (s, y):
+    ``torch.ops.torchgt.add_layer_norm`` (C++ autograd function over ``tgt_add_layer_norm_fwd`` / ``tgt_layer_norm_bwd``)."""
 
     @staticmethod
-    def forward(ctx, x, r, gamma, beta, eps):
-        if not x.is_cuda:
-            raise RuntimeError("torchgt_amd encoder kernels run on the GPU only (no CPU fallback)")
-        if x.dtype not in _DT:
-            raise TypeError(f"unsupported dtype {x.dtype}")
-        C = x.shape[-1]
-        x2 = x.reshape(-1, C).contiguous()
-        r2 = None if r is None else r.reshape(-1, C).contiguous()
-        N = x2.shape[0]
-        s = x2 if r2 is None else torch.empty_like(x2)
-        y = torch.empty_like(x2)
-        mean = torch.empty(N, dtype=torch.float32, device=x.device)
-        rstd = torch.empty(N, dtype=torch.float32, device=x.device)
-        g, b = gamma.contiguous(), beta.contiguous()
-        with torch.cuda.device(x.device):
-            _lib.check(_lib.lib().tgt_add_layer_norm_fwd(
-                x2.data_ptr(), None if r2 is None else r2.data_ptr(), g.data_ptr(), b.data_ptr(), N, C, float(eps),
-                _DT[x.dtype], None if r2 is None else s.data_ptr(), y.data_ptr(), mean.data_ptr(), rstd.data_ptr(),
-                _stream(x)))
-        ctx.save_for_backward(s, g, mean, rstd)
-        ctx.has_r = r is not None
-        ctx.shape = x.shape
-        return s.view(x.shape), y.view(x.shape)
-
-    @staticmethod
-    def backward(ctx, ds_out, dy):
-        s, g, mean, rstd = ctx.saved_tensors
-        N, C = s.shape
-        L = _lib.lib()
-        if dy is None:
-            dy = torch.zeros_like(s)
-        dy2 = dy.reshape(N, C).contiguous()
-        extra = None if ds_out is None else ds_out.reshape(N, C).contiguous()
-        ds = torch.empty_like(s)
-        dg, db = torch.empty_like(g), torch.empty_like(g)
-        nbytes = L.tgt_layer_norm_bwd_workspace_bytes(C)
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=s.device)
-        with torch.cuda.device(s.device):
-            _lib.check(L.tgt_layer_norm_bwd(s.data_ptr(), g.data_ptr(), mean.data_ptr(), rstd.data_ptr(), dy2.data_ptr(),
-                                            None if extra is None else extra.data_ptr(), N, C, _DT[s.dtype],
-                                            ds.data_ptr(), dg.data_ptr(), db.data_ptr(), ws.data_ptr(), nbytes, _stream(s)))
-        ds = ds.view(ctx.shape)
-        return ds, (ds if ctx.has_r else None), dg, db, None
+    def apply(x, r, gamma, beta, eps):
+        return _ext.ops().add_layer_norm(x, r, gamma, beta, float(eps))
 
 
-class AddFunction(torch.autograd.Function):
+class AddFunction:
     """``x + r`` through the same kernel (no normalisation)."""
 
     @staticmethod
-    def forward(ctx, x, r):
-        C = x.shape[-1]
-        x2, r2 = x.reshape(-1, C).contiguous(), r.reshape(-1, C).contiguous()
-        s = torch.empty_like(x2)
-        with torch.cuda.device(x.device):
-            _lib.check(_lib.lib().tgt_add_layer_norm_fwd(x2.data_ptr(), r2.data_ptr(), None, None, x2.shape[0], C, 0.0,
-                                                         _DT[x.dtype], s.data_ptr(), None, None, None, _stream(x)))
-        return s.view(x.shape)
+    def apply(x, r):
+        return _ext.ops().add(x, r)
+
+
+class GeluFunction:
+    """Exact (erf) GELU: ``torch.ops.torchgt.gelu``."""
 
     @staticmethod
-    def backward(ctx, ds):
-        return ds, ds
-
-
-class GeluFunction(torch.autograd.Function):
-    @staticmethod
-    def forward(ctx, u):
-        if not u.is_cuda:
-            raise RuntimeError("torchgt_amd encoder kernels run on the GPU only (no CPU fallback)")
-        u2 = u.contiguous()
-        h = torch.empty_like(u2)
-        with torch.cuda.device(u.device):
-            _lib.check(_lib.lib().tgt_gelu_fwd(u2.data_ptr(), u2.numel(), _DT[u.dtype], h.data_ptr(), _stream(u)))
-        ctx.save_for_backward(u2)
-        return h
-
-    @staticmethod
-    def backward(ctx, dh):
-        (u,) = ctx.saved_tensors
-        dh2 = dh.contiguous()
-        du = torch.empty_like(u)
-        with torch.cuda.device(u.device):
-            _lib.check(_lib.lib().tgt_gelu_bwd(u.data_ptr(), dh2.data_ptr(), u.numel(), _DT[u.dtype], du.data_ptr(), _stream(u)))
-        return du
+    def apply(u):
+        return _ext.ops().gelu(u)
 
 
 def init_params(module, n_layers):

@@ -9,7 +9,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from . import _lib
+from . import _ext, _lib
 from .encoder import AddLayerNormFunction, init_params
 from .multi_head_attention import MultiHeadAttention, fused_linear
 
@@ -20,26 +20,12 @@ def _stream(t):
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
-class ReluFunction(torch.autograd.Function):
-    @staticmethod
-    def forward(ctx, u):
-        if not u.is_cuda:
-            raise RuntimeError("torchgt_amd kernels run on the GPU only (no CPU fallback)")
-        u2 = u.contiguous()
-        h = torch.empty_like(u2)
-        with torch.cuda.device(u.device):
-            _lib.check(_lib.lib().tgt_relu_fwd(u2.data_ptr(), u2.numel(), _DT[u.dtype], h.data_ptr(), _stream(u)))
-        ctx.save_for_backward(u2)
-        return h
+class ReluFunction:
+    """``torch.ops.torchgt.relu`` (C++ autograd function over ``tgt_relu_fwd`` / ``_bwd``)."""
 
     @staticmethod
-    def backward(ctx, dh):
-        (u,) = ctx.saved_tensors
-        dh2 = dh.contiguous()
-        du = torch.empty_like(u)
-        with torch.cuda.device(u.device):
-            _lib.check(_lib.lib().tgt_relu_bwd(u.data_ptr(), dh2.data_ptr(), u.numel(), _DT[u.dtype], du.data_ptr(), _stream(u)))
-        return du
+    def apply(u):
+        return _ext.ops().relu(u)
 
 
 class EncoderLayer(nn.Module):

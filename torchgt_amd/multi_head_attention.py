@@ -12,91 +12,28 @@ weight and bias gradients.  At sequence-parallel size 1 the reference's
 ``DistributedAttentionNoMerge`` (gt_sp/layer.py:502-550) hands q, k, v to the local
 attention unchanged, which is what ``dist_attn`` does here.
 """
-import ctypes
-
 import torch
 import torch.nn as nn
 
-from . import _lib
+from . import _ext, _lib
 from .core_attention import CoreAttention
 
 _DT = {torch.float32: _lib.DTYPE_F32, torch.bfloat16: _lib.DTYPE_BF16}
 
 
-def _ptr_array(tensors):
-    arr = (ctypes.c_void_p * 3)()
-    for i, t in enumerate(tensors):
-        arr[i] = None if t is None else t.data_ptr()
-    return arr
-
-
-class LinearFunction(torch.autograd.Function):
-    """``(x W_0^T + b_0, ..., x W_{n-1}^T + b_{n-1})`` for n <= 3 weights of one shape.
+class LinearFunction:
+    """``(x W_0^T + b_0, ..., x W_{n-1}^T + b_{n-1})`` for n <= 3 weights of one shape:
+    ``torch.ops.torchgt.linear`` (a C++ autograd function over ``tgt_linear_fwd`` / ``_bwd``).
 
     ``apply(x, W_0, b_0, W_1, b_1, ...)``; x ``[..., in]``, W_j ``[out, in]``, b_j
     ``[out]`` or None.  Returns a tuple of ``[..., out]`` tensors."""
 
     @staticmethod
-    def forward(ctx, x, *wb):
-        L = _lib.lib()
+    def apply(x, *wb):
         Ws, bs = list(wb[0::2]), list(wb[1::2])
-        n = len(Ws)
-        if not 1 <= n <= 3 or len(bs) != n:
+        if not 1 <= len(Ws) <= 3 or len(bs) != len(Ws):
             raise ValueError("LinearFunction takes 1 to 3 (weight, bias) pairs")
-        if not x.is_cuda:
-            raise RuntimeError("torchgt_amd projections run on the GPU only (no CPU fallback)")
-        if x.dtype not in _DT:
-            raise TypeError(f"unsupported dtype {x.dtype}")
-        out_f, in_f = Ws[0].shape
-        for W, b in zip(Ws, bs):
-            if W.shape != (out_f, in_f) or W.dtype != x.dtype or (b is not None and (b.shape != (out_f,) or b.dtype != x.dtype)):
-                raise ValueError("all weights must be [out, in] of x's dtype and all biases [out]")
-        if x.shape[-1] != in_f:
-            raise ValueError(f"x has {x.shape[-1]} features, the weights take {in_f}")
-        x2 = x.reshape(-1, in_f).contiguous()
-        Ws = [W.contiguous() for W in Ws]
-        bs = [None if b is None else b.contiguous() for b in bs]
-        N = x2.shape[0]
-        ys = [torch.empty((N, out_f), dtype=x.dtype, device=x.device) for _ in range(n)]
-        stream = torch.cuda.current_stream(x.device).cuda_stream
-        with torch.cuda.device(x.device):
-            _lib.check(L.tgt_linear_fwd(x2.data_ptr(), _ptr_array(Ws), _ptr_array(bs), _ptr_array(ys), n, N, in_f, out_f,
-                                        _DT[x.dtype], stream))
-        ctx.save_for_backward(x2, *Ws)
-        ctx.has_bias = [b is not None for b in bs]
-        ctx.x_shape = x.shape
-        return tuple(y.view(*x.shape[:-1], out_f) for y in ys)
-
-    @staticmethod
-    def backward(ctx, *dys):
-        L = _lib.lib()
-        x2, *Ws = ctx.saved_tensors
-        n = len(Ws)
-        out_f, in_f = Ws[0].shape
-        N = x2.shape[0]
-        dys = [torch.zeros((N, out_f), dtype=x2.dtype, device=x2.device) if g is None
-               else g.reshape(N, out_f).contiguous() for g in dys]
-        need_dx = ctx.needs_input_grad[0]
-        need_dw = any(ctx.needs_input_grad[1:])
-        dx = torch.empty_like(x2) if need_dx else None
-        dWs = [torch.empty_like(W) for W in Ws] if need_dw else None
-        dbs = [torch.empty(out_f, dtype=x2.dtype, device=x2.device) if hb else None for hb in ctx.has_bias] if need_dw else None
-        ws, ws_bytes = None, 0
-        if need_dw:
-            ws_bytes = L.tgt_linear_bwd_workspace_bytes(n, in_f, out_f)
-            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x2.device)
-        stream = torch.cuda.current_stream(x2.device).cuda_stream
-        with torch.cuda.device(x2.device):
-            _lib.check(L.tgt_linear_bwd(x2.data_ptr(), _ptr_array(Ws), _ptr_array(dys), n, N, in_f, out_f, _DT[x2.dtype],
-                                        None if dx is None else dx.data_ptr(),
-                                        None if dWs is None else _ptr_array(dWs),
-                                        None if dbs is None else _ptr_array(dbs),
-                                        None if ws is None else ws.data_ptr(), ws_bytes, stream))
-        grads = [None if dx is None else dx.view(ctx.x_shape)]
-        for j in range(n):
-            grads.append(dWs[j] if need_dw else None)
-            grads.append(dbs[j] if need_dw and dbs[j] is not None else None)
-        return tuple(grads)
+        return tuple(_ext.ops().linear(x, Ws, bs))
 
 
 def fused_linear(x, *layers):

@@ -13,7 +13,7 @@ import ctypes
 import numpy as np
 import torch
 
-from . import _lib
+from . import _ext, _lib
 
 
 class GraphPlan:
@@ -38,6 +38,10 @@ class GraphPlan:
             dst_ptr = ei[1].data_ptr() if self.num_edges else None
             _lib.check(L.tgt_plan_create(src_ptr, dst_ptr, self.num_edges, self.num_nodes, stream,
                                          ctypes.byref(self._handle)))
+        # the owner of the C plan: shared with every autograd node that needs the plan in its backward, so that
+        # the plan outlives this object if a backward is still pending
+        _ext.ops()
+        self.holder = torch.classes.torchgt.PlanHolder(self._handle.value)
 
     @property
     def handle(self):
@@ -46,8 +50,11 @@ class GraphPlan:
         return self._handle
 
     def close(self):
+        """Lets go of the plan; its device memory is freed when the last pending backward that uses it has run."""
         if getattr(self, "_handle", None):
-            _lib.lib().tgt_plan_destroy(self._handle)
+            if getattr(self, "holder", None) is None:
+                _lib.lib().tgt_plan_destroy(self._handle)        # creation failed half-way: nobody else owns it
+            self.holder = None
             self._handle = ctypes.c_void_p()
             self._workspaces = {}
 
