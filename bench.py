@@ -243,6 +243,52 @@ def bench_dense(args):
     bias_b = b * H * S * S * esize
     alg = {"dense_fwd": 4 * node_b + bias_b + 4 * b * H * S, "dense_bwd": 8 * node_b + 2 * bias_b + 4 * b * H * S}
     flops = {"dense_fwd": 4 * b * H * S * S * d, "dense_bwd": 10 * b * H * S * S * d}
+    # The same attention with the bias formed on chip from 16-bit ids and the three tables of the graph-level model
+    # (tgt_dense_attn_ids_fwd / _bwd, table gradients included): no [b, H, S, S] tensor in either direction.
+    from_ids = None
+    if args.dtype == "bf16":
+        n_sp, n_e, F = 40, 64, 1                                   # the ZINC tables of models/graphormer_graph_level.py:325-339
+        sp = torch.from_numpy(data["spatial_pos"]).long().to(dev)
+        et = torch.from_numpy(data["edge_type"]).long().unsqueeze(-1).contiguous().to(dev)
+        sp16 = torch.empty(b, S, S, dtype=torch.int16, device=dev)
+        et16 = torch.empty(b, S, S, F, dtype=torch.int16, device=dev)
+        _lib.check(L.tgt_dense_ids_pack(P(sp), P(et), b, S - 1, F, n_sp, n_e, P(sp16), P(et16), stream))
+        ab = torch.from_numpy(data["attn_bias"]).to(dev, tdt)
+        t_sp, t_e, t_v = ((torch.randn(n, H, generator=g) * 0.02).to(dev, tdt) for n in (n_sp, n_e, 1))
+        d_sp, d_e, d_v = torch.empty_like(t_sp), torch.empty_like(t_e), torch.empty_like(t_v)
+        code = dt_code
+        nbytes = L.tgt_dense_attn_ids_bwd_workspace_bytes(b, H, n_sp, n_e)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+
+        def step_ids():
+            _lib.check(L.tgt_dense_attn_ids_fwd(P(q), P(k), P(v), P(ab), P(sp16), P(et16), F, P(t_sp), n_sp, P(t_e), n_e, P(t_v),
+                                                b, S, H, d, code, 0.0, 0, P(out), P(lse), stream))
+            _lib.check(L.tgt_dense_attn_ids_bwd(P(q), P(k), P(v), P(ab), P(sp16), P(et16), F, P(t_sp), n_sp, P(t_e), n_e, P(t_v),
+                                                b, S, H, d, code, 0.0, 0, P(out), P(lse), P(dout), P(dq), P(dk), P(dv),
+                                                P(d_sp), P(d_e), P(d_v), P(ws), nbytes, stream))
+
+        for _ in range(args.warmup):
+            step_ids()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step_ids()
+        torch.cuda.synchronize()
+        ms_ids = (time.perf_counter() - t0) / args.steps * 1e3
+        L.tgt_timing_reset()
+        L.tgt_timing_enable(1)
+        for _ in range(args.steps):
+            step_ids()
+        torch.cuda.synchronize()
+        L.tgt_timing_enable(0)
+        k_ids = {n: {"avg_us": t / c * 1e3, "launches": c} for n, (t, c) in _lib.kernel_timings().items() if c}
+        ids_b = b * S * S * (2 + 2 * F + esize)
+        alg_ids = {"dense_fwd": 4 * node_b + ids_b + 4 * b * H * S, "dense_bwd": 8 * node_b + ids_b + 4 * b * H * S}
+        from_ids = {"ms_per_step": ms_ids, "graphs_per_s": b / (ms_ids * 1e-3), "tables": [n_sp, n_e, 1], "edge_features": F,
+                    "step": "tgt_dense_attn_ids_fwd + tgt_dense_attn_ids_bwd (dq, dk, dv and the three table gradients)",
+                    "kernels": {n: dict(v, alg_bytes=alg_ids[n], hbm_frac=alg_ids[n] / (v["avg_us"] * 1e-6) / 1e9 / HBM_PEAK_GBS,
+                                        alg_tflops=flops[n] / (v["avg_us"] * 1e-6) / 1e12) for n, v in k_ids.items() if n in alg_ids},
+                    "bias_tensor_bytes_avoided": 3 * bias_b}
     dom = max(kernels, key=lambda n: kernels[n]["avg_us"])
     gbs = alg[dom] / (kernels[dom]["avg_us"] * 1e-6) / 1e9
     result = {
@@ -262,6 +308,7 @@ def bench_dense(args):
         "mfma": {n: {"alg_tflops": flops[n] / (kernels[n]["avg_us"] * 1e-6) / 1e12, "peak_tflops": 2500.0}
                  for n in kernels},
         "kernels": kernels,
+        "from_ids": from_ids,
     }
     return result
 
@@ -666,6 +713,7 @@ def bench_graph_model(args):
         attn_edge_type=torch.from_numpy(data["edge_type"]).long().unsqueeze(-1).contiguous().to(dev), edge_input=None)
     torch.manual_seed(42)
     m = Graphormer(4, 8, 64, 0.0, 0.0, 64, "ZINC", "single_hop", 5, 0.0, 1).to(dev, tdt)
+    m.bias_from_ids = bool(args.bias_from_ids)
     opt = torch.optim.AdamW(m.parameters(), lr=1e-3, weight_decay=0.01)
     y = torch.randn(b, device=dev)
 
@@ -702,6 +750,7 @@ def bench_graph_model(args):
         del loss
         torch.manual_seed(42)
         gm = Graphormer(4, 8, 64, 0.0, 0.0, 64, "ZINC", "single_hop", 5, 0.0, 1).to(dev, tdt)
+        gm.bias_from_ids = bool(args.bias_from_ids)
         gopt = torch.optim.AdamW(gm.parameters(), lr=1e-3, weight_decay=0.01, capturable=True)
 
         def gstep():
@@ -978,6 +1027,8 @@ def main():
                     help="skip the datapoint that runs the reference's op chain with stock torch kernels (profiling runs)")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="config2 / f32 only: skip the other benchmark configurations (they are timed in the default run)")
+    ap.add_argument("--bias-from-ids", action="store_true",
+                    help="config4-model: the attention kernels form the bias from ids and tables instead of reading a [b,H,S,S] tensor")
     ap.add_argument("--hip-graph", action="store_true",
                     help="config2-model: also time the step captured into a HIP graph and replayed")
     ap.add_argument("--calibration-copy", action="store_true",

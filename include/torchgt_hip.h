@@ -212,6 +212,43 @@ int tgt_dense_attn_dropout_bwd(const void* d_q, const void* d_k, const void* d_v
  * Dropout would hold as its mask; for tests and for callers that want to inspect it. */
 int tgt_dense_attn_dropout_mask(int b, int S, int H, float p_drop, uint64_t seed, uint8_t* d_keep, void* stream);
 
+/* ---- dense attention with the bias formed in the kernels from ids and tables -----------------
+ * GraphAttnBias.forward (models/graphormer_graph_level.py:94-156, edge_type other than 'multi_hop') feeding
+ * CoreAttention.forward (:186-214) without the [b, H, S, S] bias tensor in memory in either direction:
+ *   bias[g,h,i,j] = 2 attn_bias[g,i,j] + spatial_table[sp[g,i,j]][h] + mean_f edge_table[et[g,i,j,f]][h]
+ * over the padded index space S = s + 1 (virtual node first), i.e. the tensor tgt_graph_attn_bias_fwd would
+ * write (the kernels round it to bf16, as a bf16 bias tensor is).
+ *
+ * tgt_dense_ids_pack: once per batch, the reference's int64 spatial_pos [b, s, s] and attn_edge_type
+ * [b, s, s, F] to 16-bit ids over [b, S, S] and [b, S, S, F]: clamped to their tables like
+ * tgt_graph_attn_bias_fwd does; on the virtual node's row and column the spatial id is num_spatial (the
+ * kernels read the virtual distance there) and the edge id num_edges (reads as 0).  Table sizes 1..65534. */
+int tgt_dense_ids_pack(const int64_t* d_spatial_pos, const int64_t* d_edge_type, int b, int s, int F, int num_spatial,
+                       int num_edges, uint16_t* d_sp16, uint16_t* d_et16, void* stream);
+/* Forward.  d_attn_bias: [b, S, S] of `dtype` (0 / -inf padding mask of the collator, any values allowed) or
+ * NULL; tables [num_spatial, H], [num_edges, H], [H] of `dtype`; everything else as
+ * tgt_dense_attn_dropout_fwd.  dtype TGT_DTYPE_BF16 or TGT_DTYPE_F32_BF16_PRODUCTS (the float32-arithmetic
+ * kernels take a bias tensor: TGT_ERR_UNSUPPORTED); H <= 32; the [S, S] bias of one (graph, head) as bf16 plus
+ * one column of both tables as float must fit the LDS next to the q/k/v images (S = 129 with the molecule
+ * tables, 512 + 1537 rows: 52 KB forward, 79 KB backward), else TGT_ERR_UNSUPPORTED. */
+int tgt_dense_attn_ids_fwd(const void* d_q, const void* d_k, const void* d_v, const void* d_attn_bias,
+                           const uint16_t* d_sp16, const uint16_t* d_et16, int F, const void* d_spatial_table, int num_spatial,
+                           const void* d_edge_table, int num_edges, const void* d_virtual_dist, int b, int S, int H, int d,
+                           int dtype, float p_drop, uint64_t seed, void* d_out, float* d_lse, void* stream);
+/* Backward: dq, dk, dv as tgt_dense_attn_dropout_bwd, and the gradients of the three tables (all three or
+ * all NULL; autograd of the embedding lookups in the reference, row 0 of the spatial and edge tables is the
+ * padding index and gets zero) summed over this call's batch: workgroups add dS into LDS accumulators with
+ * floating-point atomics and their partials are added in a fixed order (results agree to rounding between
+ * runs, not bit for bit).  d_workspace: tgt_dense_attn_ids_bwd_workspace_bytes(...) bytes, 16-byte aligned,
+ * needed only with table gradients. */
+int64_t tgt_dense_attn_ids_bwd_workspace_bytes(int b, int H, int num_spatial, int num_edges);
+int tgt_dense_attn_ids_bwd(const void* d_q, const void* d_k, const void* d_v, const void* d_attn_bias,
+                           const uint16_t* d_sp16, const uint16_t* d_et16, int F, const void* d_spatial_table, int num_spatial,
+                           const void* d_edge_table, int num_edges, const void* d_virtual_dist, int b, int S, int H, int d,
+                           int dtype, float p_drop, uint64_t seed, const void* d_out, const float* d_lse, const void* d_dout,
+                           void* d_dq, void* d_dk, void* d_dv, void* d_dspatial_table, void* d_dedge_table,
+                           void* d_dvirtual_dist, void* d_workspace, int64_t workspace_bytes, void* stream);
+
 /* ---- block path: dense 16 x 16 tiles + remaining edges, one softmax per node ----
  * A tile (r0, c0) stands for the 256 edges a -> b, a in [r0, r0+16), b in
  * [c0, c0+16) that the reference's cluster reordering emits as an expanded edge

@@ -45,6 +45,12 @@ SIGNATURES = {
     "tgt_dense_attn_dropout_bwd": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _c.c_float, _c.c_uint64, _vp, _vp, _vp,
                                           _vp, _vp, _vp, _vp, _vp]),
     "tgt_dense_attn_dropout_mask": (_i32, [_i32, _i32, _i32, _c.c_float, _c.c_uint64, _vp, _vp]),
+    "tgt_dense_ids_pack": (_i32, [_vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp]),
+    "tgt_dense_attn_ids_fwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _i32, _vp, _i32, _vp, _i32, _i32, _i32, _i32, _i32,
+                                      _c.c_float, _c.c_uint64, _vp, _vp, _vp]),
+    "tgt_dense_attn_ids_bwd_workspace_bytes": (_i64, [_i32, _i32, _i32, _i32]),
+    "tgt_dense_attn_ids_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _i32, _vp, _i32, _vp, _i32, _i32, _i32, _i32, _i32,
+                                      _c.c_float, _c.c_uint64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
     "tgt_dense_attn_fwd": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp]),
     "tgt_dense_attn_bwd": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp,
                                   _vp, _vp, _vp, _vp, _vp]),

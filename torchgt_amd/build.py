@@ -33,7 +33,7 @@ def sources():
 
 # sources compiled as several translation units (-D<macro>=k, k < parts), in parallel: their
 # kernels take minutes to compile in one piece
-SPLIT = {"sparse_attn.hip": ("TGT_SPARSE_PART", 4)}
+SPLIT = {"sparse_attn.hip": ("TGT_SPARSE_PART", 4), "dense_attn.hip": ("TGT_DENSE_PART", 2)}
 
 
 def _jobs():

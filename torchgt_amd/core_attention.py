@@ -90,19 +90,53 @@ def dense_dropout_mask(b, S, H, p_drop, seed, device):
     return keep
 
 
+class GraphBiasIds:
+    """The graph-level attention bias in unbuilt form: what ``GraphAttnBias`` (models/graphormer_graph_level.py:94-156,
+    plain edge-type branch) would turn into a [b, H, S, S] tensor, kept as 16-bit ids over the padded [b, S, S] index
+    space (``torch.ops.torchgt.dense_ids_pack``), the [b, S, S] ``attn_bias`` of the batch and the three embedding
+    tables.  ``dense_attention`` accepts it in place of the bias tensor: the kernels then form the bias on chip and
+    return the table gradients directly (bf16 matrix-product kernels only).  ``materialize()`` builds the tensor the
+    reference would pass, once, for the float32-arithmetic kernels and for shapes whose bias does not fit the LDS."""
+
+    def __init__(self, attn_bias, sp16, et16, spatial_table, edge_table, virtual_dist, build):
+        self.attn_bias, self.sp16, self.et16 = attn_bias, sp16, et16
+        self.spatial_table, self.edge_table, self.virtual_dist = spatial_table, edge_table, virtual_dist
+        self._build = build            # () -> [b, H, S, S] tensor with autograd to the tables
+        self._tensor = None
+        self.fits = True               # cleared when the kernels report that this shape needs the tensor
+
+    def materialize(self):
+        if self._tensor is None:
+            self._tensor = self._build()
+        return self._tensor
+
+
 def dense_attention(q, k, v, attn_bias=None, p_drop=0.0, seed=None, bf16_products=False):
     """Functional form of the dense path: q, k, v [b, S, H, d], attn_bias [b, H, S, S] or None;
     returns [b, S, H*d].  A bias of another float dtype or with a broadcast head axis
     ([b, 1, S, S]) is converted / expanded here, where autograd sees it.  ``p_drop`` > 0 applies attention
     dropout; ``seed`` (default: drawn from torch's CPU generator, so ``torch.manual_seed`` governs it) names
-    the mask."""
+    the mask.  ``attn_bias`` may be a ``GraphBiasIds``."""
+    if p_drop > 0 and seed is None:
+        seed = int(torch.randint(0, 2 ** 62, (1,)).item())
+    if isinstance(attn_bias, GraphBiasIds):
+        ids = attn_bias
+        if ids.fits and (q.dtype == torch.bfloat16 or bf16_products):
+            ab = None if ids.attn_bias is None else ids.attn_bias.to(q.dtype)
+            try:
+                return _ext.ops().dense_attention_ids(q, k, v, ab, ids.sp16, ids.et16, ids.spatial_table.to(q.dtype),
+                                                      ids.edge_table.to(q.dtype), ids.virtual_dist.to(q.dtype), float(p_drop),
+                                                      int(seed or 0), bool(bf16_products))
+            except RuntimeError as exc:
+                if "bytes of LDS" not in str(exc):
+                    raise
+                ids.fits = False       # this shape needs the bias tensor: build it once, below
+        attn_bias = ids.materialize()
     if attn_bias is not None:
         b, S, H = q.shape[0], q.shape[1], q.shape[2]
         if attn_bias.dim() == 4 and attn_bias.shape[1] == 1 and H != 1:
             attn_bias = attn_bias.expand(b, H, S, S)
         attn_bias = attn_bias.to(q.dtype)
-    if p_drop > 0 and seed is None:
-        seed = int(torch.randint(0, 2 ** 62, (1,)).item())
     return DenseAttentionFunction.apply(q, k, v, attn_bias, p_drop, seed or 0, bf16_products)
 
 

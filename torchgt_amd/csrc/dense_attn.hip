@@ -153,6 +153,184 @@ __device__ __forceinline__ float raw1(const float* p) { return *p; }
 __device__ __forceinline__ float cvt1(uint32_t x) { return __uint_as_float(x << 16); }
 __device__ __forceinline__ float cvt1(float x) { return x; }
 
+// ---------------------------------------------------------------------------
+// The bias of the graph-level Graphormer formed inside the attention kernels (BSRC = 1) instead of
+// read from a [b, H, S, S] tensor (GraphAttnBias.forward, models/graphormer_graph_level.py:94-156,
+// simple edge-type branch, feeding CoreAttention.forward :186-214):
+//   bias[g,h,i,j] = 2 attn_bias[g,i,j] + spatial_table[sp[g,i,j]][h] + mean_f edge_table[et[g,i,j,f]][h]
+// with the ids packed beforehand to 16 bits over the padded [S, S] index space: on the virtual
+// node's row and column sp holds the extra id num_spatial (its table slot is the virtual
+// distance of head h) and et the extra id num_edges (slot 0.0).  A workgroup keeps the tables of
+// its head in LDS as float, builds the [S, S] bias of its (graph, head) pair in LDS as bf16 once,
+// and both walks read it from there.  In the backward the bias gradient dS never leaves the
+// chip either: the query-major walk adds every dS into LDS accumulators indexed by the ids (ids
+// below kHotIds into one of kHotCopies copies chosen by the lane, which keeps lanes that meet the
+// same few shortest-path lengths off each other's address).  The accumulators are 32-bit
+// integers: LDS integer atomics run about nine times faster than the floating-point ones on this
+// part (measured: 16 against 54 ns per wave-wide add under this id distribution), and integer
+// sums do not depend on the order of the adds, so the table gradients are reproducible bit for
+// bit.  Every (graph, head) pair gets its own power-of-two scale from a bound on its dS: the rows
+// of the softmax sum to one, so sum_k |dS[q,k]| <= 2 max_q |dout_q|_1 max|v| / (1 - p) =: B and no
+// accumulator of one pair can exceed S B; with scale = 2^22 / B' (B' = B rounded up to a power of
+// two) that stays below 2^30 for S <= 256, and one unit is 2^-22 B'.  After each pair the
+// workgroup converts its integer sums to float and adds them to its partial in global memory.
+// ---------------------------------------------------------------------------
+struct IdsArgs {
+    const void* ab;            // [b, S, S] of T, or null
+    const uint16_t* sp;        // [b, S, S]
+    const uint16_t* et;        // [b, S, S, F]
+    const void* sp_tab;        // [ns, H] of T
+    const void* e_tab;         // [ne, H] of T
+    const void* vd;            // [H] of T
+    float* partial;            // backward: [gridDim.x][ns + ne + 1], or null when no table gradient is wanted
+    int F, ns, ne;
+};
+constexpr int kHotIds = 32, kHotCopies = 16, kHotStride = kHotIds + 1;
+
+struct IdsLds {
+    short* tile;               // [S][bst] bf16 bits
+    float *tabS, *tabE;        // [ns + 1], [ne + 1]: the head's table columns (edge entries already divided by F)
+    int *hot, *accS, *accE;    // backward only: fixed-point sums of the current pair ([kHotCopies][kHotStride], [ns + 1], [ne + 1])
+    int* bound;                // backward only: max_q |dout_q|_1 and max |v| of the current pair, as float bits
+    int bst;
+};
+__host__ __device__ __forceinline__ int ids_tile_stride(int S) { return (S + 7) & ~7; }
+__host__ __device__ __forceinline__ size_t ids_tile_bytes(int S) { return (((size_t)S * ids_tile_stride(S) * 2) + 15) & ~(size_t)15; }
+inline size_t ids_lds_bytes(int S, int ns, int ne, bool bwd) {
+    // (+ 32: a lane's sixteen-key group of the last row may end up to 30 bytes behind the tile)
+    return ids_tile_bytes(S) + 32 + sizeof(float) * ((size_t)(ns + ne + 2) * (bwd ? 2 : 1) + (bwd ? kHotCopies * kHotStride + 4 : 0));
+}
+__device__ __forceinline__ IdsLds ids_lds(char* base, int S, int ns, int ne) {
+    IdsLds l;
+    l.bst = ids_tile_stride(S);
+    l.tile = reinterpret_cast<short*>(base);
+    l.tabS = reinterpret_cast<float*>(base + ids_tile_bytes(S));
+    l.tabE = l.tabS + ns + 1;
+    l.hot = reinterpret_cast<int*>(l.tabE + ne + 1);
+    l.accS = l.hot + kHotCopies * kHotStride;
+    l.accE = l.accS + ns + 1;
+    l.bound = l.accE + ne + 1;
+    return l;
+}
+__device__ __forceinline__ float ldT(const float* p) { return *p; }
+__device__ __forceinline__ float ldT(const dbf16* p) { return __uint_as_float(((uint32_t)p->x) << 16); }
+
+template <typename T>
+__device__ __forceinline__ void ids_load_tables(const IdsArgs& a, int h, int H, const IdsLds& l) {
+    const T* st = reinterpret_cast<const T*>(a.sp_tab);
+    const T* et = reinterpret_cast<const T*>(a.e_tab);
+    for (int i = threadIdx.x; i < a.ns; i += blockDim.x) l.tabS[i] = ldT(st + (int64_t)i * H + h);
+    const float inv_f = 1.f / (float)a.F;
+    for (int i = threadIdx.x; i < a.ne; i += blockDim.x) l.tabE[i] = ldT(et + (int64_t)i * H + h) * inv_f;
+    if (threadIdx.x == 0) {
+        l.tabS[a.ns] = ldT(reinterpret_cast<const T*>(a.vd) + h);
+        l.tabE[a.ne] = 0.f;
+    }
+}
+
+// tile[i][j] = bias of (query i, key j) of graph g for the head whose tables are in LDS; columns S .. bst-1 are zero.
+// A thread takes sixteen consecutive keys of a row at a time: three 32-byte requests (attn_bias, spatial ids, first
+// edge feature) in flight together, sixteen pairs of table look-ups, one 32-byte LDS write; GB such groups per thread
+// are requested before the first is used (a thread has only a handful of groups per pair: one after the other they
+// would cost a memory round trip each).  The columns behind the last whole group of a row are done one per thread.
+__device__ __forceinline__ float ids_bias_value(const IdsArgs& a, const IdsLds& l, float ab2, uint32_t sp, int64_t at) {
+    float v = ab2 + l.tabS[min((int)sp, a.ns)];
+    for (int f = 0; f < a.F; ++f) v += l.tabE[min((int)a.et[at * a.F + f], a.ne)];
+    return v;
+}
+// x / d for 0 <= x < 65536 and 1 <= d <= 65536 through a multiplication: with m = ceil(2^32 / d), (x m) >> 32 is exact
+// in that range (d = 1 has no 32-bit m: it is coded as 0)
+__device__ __forceinline__ uint32_t div_magic(int d) { return d == 1 ? 0u : (uint32_t)((0x100000000ull + (uint32_t)d - 1) / (uint32_t)d); }
+__device__ __forceinline__ int div_by(int x, uint32_t m) { return m == 0u ? x : (int)__umulhi((uint32_t)x, m); }
+
+template <typename T, int GB>
+__device__ __forceinline__ void ids_build_tile(const IdsArgs& a, int g, int S, const IdsLds& l) {
+    const T* ab = reinterpret_cast<const T*>(a.ab);
+    const int64_t base = (int64_t)g * S * S;
+    const int bst = l.bst;
+    const int gpr = S >> 4;                          // whole groups per row
+    const int n_groups = S * gpr;
+    const uint32_t m_gpr = div_magic(max(gpr, 1));
+    for (int grp0 = threadIdx.x; grp0 < n_groups; grp0 += GB * blockDim.x) {
+        Bias16<T> abr[GB];
+        Bias16<dbf16> spr[GB], etr[GB];
+#pragma unroll
+        for (int u = 0; u < GB; ++u) {
+            const int grp = min(grp0 + u * (int)blockDim.x, n_groups - 1);      // past the end: the last group again, not stored
+            const int i = div_by(grp, m_gpr), j0 = (grp - i * gpr) * 16;
+            const int64_t at = base + (int64_t)i * S + j0;
+            zero_bias16(abr[u]);
+            zero_bias16(etr[u]);
+            if (ab) load_bias16(ab + at, 16, abr[u]);
+            load_bias16(reinterpret_cast<const dbf16*>(a.sp) + at, 16, spr[u]);
+            if (a.F == 1) load_bias16(reinterpret_cast<const dbf16*>(a.et) + at, 16, etr[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < GB; ++u) {
+            const int grp = grp0 + u * (int)blockDim.x;
+            const int gc = min(grp, n_groups - 1);
+            const int i = div_by(gc, m_gpr), j0 = (gc - i * gpr) * 16;
+            const int64_t at = base + (int64_t)i * S + j0;
+            short v16[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float ab2 = 2.f * abr[u].get(r);                   // the clone plus the final re-add (:104, :153)
+                const uint32_t sp = (spr[u].w[r >> 1] >> (16 * (r & 1))) & 0xffffu;
+                float v;
+                if (a.F == 1) v = ab2 + l.tabS[min((int)sp, a.ns)] + l.tabE[min((int)((etr[u].w[r >> 1] >> (16 * (r & 1))) & 0xffffu), a.ne)];
+                else v = ids_bias_value(a, l, ab2, sp, at + r);
+                v16[r] = f2bf(v);
+            }
+            if (grp < n_groups) __builtin_memcpy(l.tile + i * bst + j0, v16, 32);
+        }
+    }
+    const int j_rest = gpr * 16, w_rest = bst - j_rest;        // columns j_rest .. bst-1 of every row, one per thread
+    const uint32_t m_rest = div_magic(max(w_rest, 1));
+    for (int e = threadIdx.x; e < S * w_rest; e += blockDim.x) {
+        const int i = div_by(e, m_rest), j = j_rest + (e - i * w_rest);
+        float v = 0.f;
+        if (j < S) {
+            const int64_t at = base + (int64_t)i * S + j;
+            v = ids_bias_value(a, l, ab ? 2.f * ldT(ab + at) : 0.f, a.sp[at], at);
+        }
+        l.tile[i * bst + j] = f2bf(v);
+    }
+}
+
+// sixteen consecutive bf16 of a tile row, from a 32-byte aligned position
+__device__ __forceinline__ void load_tile16(const short* __restrict__ p, Bias16<dbf16>& b) {
+    const uint4 u0 = *reinterpret_cast<const uint4*>(p), u1 = *reinterpret_cast<const uint4*>(p + 8);
+    b.w[0] = u0.x; b.w[1] = u0.y; b.w[2] = u0.z; b.w[3] = u0.w;
+    b.w[4] = u1.x; b.w[5] = u1.y; b.w[6] = u1.z; b.w[7] = u1.w;
+}
+
+// Where the backward adds one dS.  id 0 of either table is the padding index and gets no gradient
+// (nn.Embedding(padding_idx=0), :82, :86); masked positions carry exact zeros.
+struct IdsAcc {
+    const uint16_t *sp, *et;   // of this graph: [S, S], [S, S, F]
+    int *hot_copy, *accS, *accE;
+    int F, ns, ne, hot_n;
+    float scale;               // of the current pair: dS * scale is what the accumulators count
+    bool on;
+};
+// (id 0 is added too, into a slot that is never read: one test less per position)
+__device__ __forceinline__ void acc_spatial(const IdsAcc& c, float ds, uint32_t id) {
+    if (ds != 0.f) {
+        id = min(id, (uint32_t)c.ns);
+        atomicAdd((int)id < c.hot_n ? c.hot_copy + id : c.accS + id, __float2int_rn(ds * c.scale));
+    }
+}
+__device__ __forceinline__ void acc_edge(const IdsAcc& c, float ds, uint32_t e) {
+    if (ds != 0.f && e != 0 && (int)e < c.ne) atomicAdd(c.accE + e, __float2int_rn(ds * c.scale));
+}
+// one position whose ids are still in memory
+__device__ __forceinline__ void acc_position(const IdsAcc& c, float ds, int64_t at) {
+    if (ds != 0.f) {
+        acc_spatial(c, ds, c.sp[at]);
+        for (int f = 0; f < c.F; ++f) acc_edge(c, ds, c.et[at * c.F + f]);
+    }
+}
+
 // The keys of a 32-key tile are assigned to the rows of the MFMA A operand in a permuted order,
 // row 8j + 4h + t  <->  key 16h + 4j + t, so that in the transposed score tile (lane = query,
 // half h = lane / 32) register r of a lane is key 16h + r: sixteen CONSECUTIVE keys per lane,
@@ -220,9 +398,9 @@ __device__ __forceinline__ void store_row(T* __restrict__ p, const float (&x)[D]
 }
 
 // forward of the rows first .. first + count - 1 (all keys), by one wave
-template <typename T, int D, int SP, bool DROP>
+template <typename T, typename BT, int D, int SP, bool DROP>
 __device__ __forceinline__ void thin_rows_fwd(const T* __restrict__ Q, const short* __restrict__ k_rm,
-                                              const short* __restrict__ v_tr, const T* __restrict__ bias_gh,
+                                              const short* __restrict__ v_tr, const BT* __restrict__ bias_gh, int bstride,
                                               T* __restrict__ out, float* __restrict__ lse, int g, int h, int S, int H,
                                               float scale, int first, int count, int lane, const DropArgs da) {
     constexpr int NC = (SP + 63) / 64;
@@ -234,7 +412,7 @@ __device__ __forceinline__ void thin_rows_fwd(const T* __restrict__ Q, const sho
             const short4_t v = ld4(Q + (((int64_t)g * S + qi) * H + h) * D + 4 * c);
             qv[4 * c + 0] = bf2f(v.x); qv[4 * c + 1] = bf2f(v.y); qv[4 * c + 2] = bf2f(v.z); qv[4 * c + 3] = bf2f(v.w);
         }
-        const T* brow = bias_gh ? bias_gh + (int64_t)qi * S : nullptr;
+        const BT* brow = bias_gh ? bias_gh + (int64_t)qi * bstride : nullptr;
         float sv[NC], mx = -INFINITY;
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
@@ -275,13 +453,13 @@ __device__ __forceinline__ void thin_rows_fwd(const T* __restrict__ Q, const sho
 }
 
 // backward, query side, of the rows first .. first + count - 1: dQ and their rows of dBias
-template <typename T, int D, int SP, bool DROP>
+template <typename T, typename BT, int D, int SP, bool DROP>
 __device__ __forceinline__ void thin_rows_bwd_q(const short* __restrict__ q_rm, const short* __restrict__ k_rm,
                                                 const short* __restrict__ v_rm, const short* __restrict__ g_rm,
                                                 const float* __restrict__ lse_l, const float* __restrict__ dd_l,
-                                                const T* __restrict__ bias_gh, T* __restrict__ dbias_gh, T* __restrict__ dQ,
-                                                int g, int h, int S, int H, float scale, int first, int count, int lane,
-                                                const DropArgs da) {
+                                                const BT* __restrict__ bias_gh, int bstride, T* __restrict__ dbias_gh,
+                                                T* __restrict__ dQ, int g, int h, int S, int H, float scale, int first,
+                                                int count, int lane, const DropArgs da, const IdsAcc& acc) {
     constexpr int NC = (SP + 63) / 64;
     const float scale2 = scale * kLog2e;
     for (int tq = 0; tq < count; ++tq) {
@@ -300,11 +478,12 @@ __device__ __forceinline__ void thin_rows_bwd_q(const short* __restrict__ q_rm, 
                 float kv[D], vv[D];
                 lds_row<D>(k_rm, key, kv);
                 lds_row<D>(v_rm, key, vv);
-                const float b = bias_gh ? ld1(bias_gh + (int64_t)qi * S + key) : 0.f;
+                const float b = bias_gh ? ld1(bias_gh + (int64_t)qi * bstride + key) : 0.f;
                 const float pv = fast_exp2(fmaf(dot_d<D>(qv, kv), scale2, fmaf(b, kLog2e, nL2)));
                 const float ks = !DROP ? 1.0f : (drop_keep(da, rh, key) ? da.inv_keep : 0.f);
                 const float dS = pv * (dot_d<D>(gv, vv) * ks - Dq);
                 if (dbias_gh) st1(dbias_gh + (int64_t)qi * S + key, dS);
+                if (acc.on) acc_position(acc, dS, (int64_t)qi * S + key);
                 const float dsb = round_bf(dS);
 #pragma unroll
                 for (int d = 0; d < D; ++d) dq[d] = fmaf(dsb, kv[d], dq[d]);
@@ -317,11 +496,11 @@ __device__ __forceinline__ void thin_rows_bwd_q(const short* __restrict__ q_rm, 
 }
 
 // backward, key side, of the keys first .. first + count - 1 (all queries): dK and dV
-template <typename T, int D, int SP, bool DROP>
+template <typename T, typename BT, int D, int SP, bool DROP>
 __device__ __forceinline__ void thin_rows_bwd_k(const short* __restrict__ q_rm, const short* __restrict__ k_rm,
                                                 const short* __restrict__ v_rm, const short* __restrict__ g_rm,
                                                 const float* __restrict__ lse_l, const float* __restrict__ dd_l,
-                                                const T* __restrict__ bias_gh, T* __restrict__ dK, T* __restrict__ dV,
+                                                const BT* __restrict__ bias_gh, int bstride, T* __restrict__ dK, T* __restrict__ dV,
                                                 int g, int h, int S, int H, float scale, int first, int count, int lane,
                                                 const DropArgs da) {
     constexpr int NC = (SP + 63) / 64;
@@ -340,7 +519,7 @@ __device__ __forceinline__ void thin_rows_bwd_k(const short* __restrict__ q_rm, 
                 float qv[D], gv[D];
                 lds_row<D>(q_rm, qq, qv);
                 lds_row<D>(g_rm, qq, gv);
-                const float b = bias_gh ? ld1(bias_gh + (int64_t)qq * S + ki) : 0.f;
+                const float b = bias_gh ? ld1(bias_gh + (int64_t)qq * bstride + ki) : 0.f;
                 const float pv = fast_exp2(fmaf(dot_d<D>(qv, kv), scale2, fmaf(b, kLog2e, -lse_l[qq])));
                 const float ks = !DROP ? 1.0f : (drop_keep(da, drop_row_hash(da, g * H + h, qq), ki) ? da.inv_keep : 0.f);
                 const float dS = pv * (dot_d<D>(gv, vv) * ks - dd_l[qq]);
@@ -364,16 +543,24 @@ __device__ __forceinline__ void thin_rows_bwd_k(const short* __restrict__ q_rm, 
 // ---------------------------------------------------------------------------
 // forward: online softmax over key tiles, in the base-2 domain
 // ---------------------------------------------------------------------------
-template <typename T, int D, int NT, bool DROP>
+template <typename T, int D, int NT, bool DROP, int BSRC>
 __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, const T* __restrict__ K,
                                                        const T* __restrict__ V, const T* __restrict__ bias,
                                                        T* __restrict__ out, float* __restrict__ lse, int S,
-                                                       int H, float scale, int nb, const DropArgs da) {
+                                                       int H, float scale, int nb, const DropArgs da, const IdsArgs ia) {
     constexpr int KS = D / 8;
     constexpr int SP = NT * 32;
+    using BT = typename std::conditional<BSRC == 1, dbf16, T>::type;     // element type of the bias as the walks read it
     extern __shared__ __align__(16) char smem[];
     short* k_rm = reinterpret_cast<short*>(smem);
     short* v_tr = k_rm + rm_elems<D, SP>();
+    IdsLds il{};
+    if constexpr (BSRC == 1) {
+        // the grid is a multiple of 8 H, so every pair of this workgroup has the same head: its tables are loaded once
+        il = ids_lds(smem + fwd_lds_bytes<D, NT>(), S, ia.ns, ia.ne);
+        ids_load_tables<T>(ia, (blockIdx.x % (8 * H)) >> 3, H, il);
+        __syncthreads();
+    }
     // XCD-aware placement: workgroups go to the 8 XCDs round-robin, and the H heads of a graph
     // share every 128-byte line of q/k/v ([b,S,H,d] layout), so the heads of graph g are given the
     // workgroup ids congruent to g mod 8 inside a window of 8*H ids - same XCD, same L2, same time.
@@ -389,15 +576,20 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
     const int col = lane & 31, half = lane >> 5;
     const int q0 = wave * 32, qi = q0 + col;
     const bool qok = qi < S;
-    const bool hasb = bias != nullptr;
+    const bool hasb = BSRC == 1 || bias != nullptr;
     // a last tile of at most four rows is not worth a matrix tile: its wave takes the vector path
     const bool vec_wave = wave == NT - 1 && S - (NT - 1) * 32 <= 4;
     // this lane's query row of the bias; the first tile's group of it is requested before anything else
-    const T* brow = hasb ? bias + (((int64_t)g * H + h) * S + (qok ? qi : 0)) * S : nullptr;
-    Bias16<T> bcur, bnext;
+    const T* brow = (BSRC == 0 && hasb) ? bias + (((int64_t)g * H + h) * S + (qok ? qi : 0)) * S : nullptr;
+    const short* trow = BSRC == 1 ? il.tile + (qok ? qi : 0) * il.bst : nullptr;      // the same row of the LDS tile
+    Bias16<BT> bcur, bnext;
     zero_bias16(bcur);
     zero_bias16(bnext);
-    if (hasb && qok && !vec_wave) load_bias16(brow + 16 * half, min(16, S - 16 * half), bcur);
+    if constexpr (BSRC == 0) {
+        if (hasb && qok && !vec_wave) load_bias16(brow + 16 * half, min(16, S - 16 * half), bcur);
+    } else {
+        ids_build_tile<T, 2>(ia, g, S, il);
+    }
     load_head<T, D, SP>(K, g, h, S, H, k_rm, nullptr);
     load_head<T, D, SP>(V, g, h, S, H, nullptr, v_tr);
     short4_t bq[KS];
@@ -407,9 +599,15 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
         if (qok) bq[s] = ld4(Q + (((int64_t)g * S + qi) * H + h) * D + s * 8 + half * 4);
     }
     __syncthreads();
+    if constexpr (BSRC == 1) {
+        if (qok && !vec_wave && 16 * half < S) load_tile16(trow + 16 * half, bcur);
+    }
     if (vec_wave) {
-        thin_rows_fwd<T, D, SP, DROP>(Q, k_rm, v_tr, hasb ? bias + ((int64_t)g * H + h) * S * S : nullptr, out, lse, g, h, S,
-                                      H, scale, (NT - 1) * 32, S - (NT - 1) * 32, lane, da);
+        const BT* bias_gh = nullptr;
+        if constexpr (BSRC == 1) bias_gh = reinterpret_cast<const dbf16*>(il.tile);
+        else bias_gh = hasb ? bias + ((int64_t)g * H + h) * S * S : nullptr;
+        thin_rows_fwd<T, BT, D, SP, DROP>(Q, k_rm, v_tr, bias_gh, BSRC == 1 ? il.bst : S, out, lse, g, h, S, H, scale,
+                                          (NT - 1) * 32, S - (NT - 1) * 32, lane, da);
     } else {
     const int krow = key_of_row(col);            // key (inside a tile) of this lane's A-operand row
     // Row sums on the matrix unit: with a head dim below 32 the A operand of O^T = V^T P^T has idle
@@ -429,7 +627,11 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
         const int kb = kt * 32 + 16 * half;      // this lane's keys: kb .. kb + 15
         if (kt + 1 < NT && hasb && qok) {        // the next tile's group, a whole tile ahead of its use
             const int nv = S - (kb + 32);
-            if (nv > 0) load_bias16(brow + kb + 32, min(16, nv), bnext);
+            if constexpr (BSRC == 1) {
+                if (nv > 0) load_tile16(trow + kb + 32, bnext);
+            } else {
+                if (nv > 0) load_bias16(brow + kb + 32, min(16, nv), bnext);
+            }
         }
         float16_t sc = zero16();
 #pragma unroll
@@ -536,16 +738,17 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
 // bias straight from global memory in the layout their lanes need (a lane's own row
 // in the first, 32 lanes on 32 consecutive keys of one row in the second); the second
 // read of a (graph, head) slice comes from L2.
-template <typename T, int D, int NT, bool DROP>
+template <typename T, int D, int NT, bool DROP, int BSRC>
 __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, const T* __restrict__ K,
                                                        const T* __restrict__ V, const T* __restrict__ bias,
                                                        const T* __restrict__ O, const float* __restrict__ lse,
                                                        const T* __restrict__ dO, T* __restrict__ dQ,
                                                        T* __restrict__ dK, T* __restrict__ dV,
                                                        T* __restrict__ dbias, int S, int H, float scale, int nb,
-                                                       const DropArgs da) {
+                                                       const DropArgs da, const IdsArgs ia) {
     constexpr int KS = D / 8;
     constexpr int SP = NT * 32;
+    using BT = typename std::conditional<BSRC == 1, dbf16, T>::type;
     extern __shared__ __align__(16) char smem[];
     constexpr int RM = rm_elems<D, SP>(), TR = tr_elems<D, SP>();
     short* q_rm = reinterpret_cast<short*>(smem);
@@ -557,32 +760,71 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
     short* g_tr = k_tr + TR;
     float* lse_l = reinterpret_cast<float*>(g_tr + TR);   // lse * log2(e)
     float* dd_l = lse_l + SP;
-    // XCD-aware placement as in the forward; one workgroup per (graph, head) pair
-    const int win = blockIdx.x / (8 * H), rem = blockIdx.x % (8 * H);
+    IdsLds il{};
+    IdsAcc acc{};
+    if constexpr (BSRC == 1) {
+        // the grid is a multiple of 8 H: one head per workgroup, whose tables are loaded and whose accumulators are
+        // cleared once
+        il = ids_lds(smem + bwd_lds_bytes<D, NT>(), S, ia.ns, ia.ne);
+        ids_load_tables<T>(ia, (blockIdx.x % (8 * H)) >> 3, H, il);
+        for (int i = threadIdx.x; i < kHotCopies * kHotStride + ia.ns + ia.ne + 2 + 2; i += blockDim.x) il.hot[i] = 0;   // .. and the bound words
+        acc.F = ia.F; acc.ns = ia.ns; acc.ne = ia.ne; acc.hot_n = min(kHotIds, ia.ns);
+        acc.hot_copy = il.hot + (threadIdx.x % kHotCopies) * kHotStride;
+        acc.accS = il.accS; acc.accE = il.accE;
+        acc.on = ia.partial != nullptr;
+        if (acc.on)       // the partial starts at zero (a workgroup whose pairs all lie past the batch adds nothing)
+            for (int k = threadIdx.x; k < ia.ns + ia.ne + 1; k += blockDim.x) ia.partial[(int64_t)blockIdx.x * (ia.ns + ia.ne + 1) + k] = 0.f;
+        __syncthreads();
+    }
+    // XCD-aware placement as in the forward.  With the bias in memory one workgroup per (graph, head) pair (it runs
+    // longer per pair than the forward, persistence does not pay); with ids the grid is what the GPU keeps resident
+    // and a workgroup walks pairs of its head, so that it writes its table partial once.
+    const int total_pairs = ((nb + 7) / 8) * 8 * H;
+    for (int pair = blockIdx.x; pair < total_pairs; pair += gridDim.x) {
+    const int win = pair / (8 * H), rem = pair % (8 * H);
     const int g = win * 8 + (rem & 7), h = rem >> 3;
-    if (g >= nb) return;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (g >= nb) {
+        if constexpr (BSRC == 0) return;
+        else continue;
+    }
+    // In the loop over pairs the compiler would compute everything that depends on the lane alone once, ahead of
+    // the loop, and keep it in registers through both walks (256 registers and spills instead of 160): the thread
+    // id is handed to it as a value it cannot see through, once per pair.
+    int tid = threadIdx.x;
+    if constexpr (BSRC == 1) asm volatile("v_mov_b32 %0, %1" : "=v"(tid) : "v"(tid));
+    const int wave = BSRC == 1 ? __builtin_amdgcn_readfirstlane(tid >> 6) : tid >> 6, lane = tid & 63;
     const int col = lane & 31, half = lane >> 5;
-    const bool hasb = bias != nullptr;
+    const bool hasb = BSRC == 1 || bias != nullptr;
     const int tail = S - (NT - 1) * 32;          // rows / keys in the last tile
     const bool thin = tail <= 4;
     const int nt_full = thin ? NT - 1 : NT;      // tiles that take the general path
-    const T* bias_gh = hasb ? bias + ((int64_t)g * H + h) * S * S : nullptr;
+    const int bstride = BSRC == 1 ? il.bst : S;  // row stride of the bias as the walks read it
+    const BT* bias_gh = nullptr;
+    if constexpr (BSRC == 1) bias_gh = reinterpret_cast<const dbf16*>(il.tile);
+    else bias_gh = hasb ? bias + ((int64_t)g * H + h) * S * S : nullptr;
     // the first query-major group of this lane's bias row, requested before anything else
     const int qi = wave * 32 + col;
     const bool qok = qi < S;
-    const T* brow = hasb ? bias_gh + (int64_t)(qok ? qi : 0) * S : nullptr;
-    Bias16<T> bcur, bnext;
+    const T* brow = nullptr;
+    if constexpr (BSRC == 0) brow = hasb ? bias_gh + (int64_t)(qok ? qi : 0) * S : nullptr;
+    const short* trow = BSRC == 1 ? il.tile + (qok ? qi : 0) * il.bst : nullptr;
+    Bias16<BT> bcur, bnext;
     zero_bias16(bcur);
     zero_bias16(bnext);
     const bool vec_wave = thin && wave == NT - 1;     // the wave of a last tile of at most four rows: vector path
-    if (hasb && qok && !vec_wave) load_bias16(brow + 16 * half, min(16, S - 16 * half), bcur);
+    if constexpr (BSRC == 0) {
+        if (hasb && qok && !vec_wave) load_bias16(brow + 16 * half, min(16, S - 16 * half), bcur);
+    } else {
+        ids_build_tile<T, 4>(ia, g, S, il);
+        acc.sp = ia.sp + (int64_t)g * S * S;
+        acc.et = ia.et + (int64_t)g * S * S * ia.F;
+    }
     load_head<T, D, SP>(Q, g, h, S, H, q_rm, q_tr);
     load_head<T, D, SP>(K, g, h, S, H, k_rm, k_tr);
     load_head<T, D, SP>(V, g, h, S, H, v_rm, nullptr);
     load_head<T, D, SP>(dO, g, h, S, H, g_rm, g_tr);
     for (int i = threadIdx.x; i < SP; i += blockDim.x) {
-        float dsum = 0.f, L = 0.f;
+        float dsum = 0.f, L = 0.f, g1 = 0.f, vm = 0.f;
         if (i < S) {
             L = lse[((int64_t)g * H + h) * S + i];
             const T* op = O + (((int64_t)g * S + i) * H + h) * D;
@@ -593,18 +835,42 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
                 const short4_t gv = ld4(gp + c);
                 dsum += bf2f(ov.x) * bf2f(gv.x) + bf2f(ov.y) * bf2f(gv.y) + bf2f(ov.z) * bf2f(gv.z) +
                         bf2f(ov.w) * bf2f(gv.w);
+                if (BSRC == 1) g1 += fabsf(bf2f(gv.x)) + fabsf(bf2f(gv.y)) + fabsf(bf2f(gv.z)) + fabsf(bf2f(gv.w));
+            }
+            if (BSRC == 1 && acc.on) {
+                const T* vp = V + (((int64_t)g * S + i) * H + h) * D;
+#pragma unroll
+                for (int c = 0; c < D; c += 4) {
+                    const short4_t vv = ld4(vp + c);
+                    vm = fmaxf(fmaxf(vm, fmaxf(fabsf(bf2f(vv.x)), fabsf(bf2f(vv.y)))), fmaxf(fabsf(bf2f(vv.z)), fabsf(bf2f(vv.w))));
+                }
             }
         }
         lse_l[i] = L * kLog2e;
         dd_l[i] = dsum;          // D[q] = sum_dd dout[q,dd] out[q,dd]
+        if (BSRC == 1 && acc.on && i < S) {      // non-negative floats order like their bit patterns (a NaN ends up largest)
+            atomicMax(il.bound, __float_as_int(g1));
+            atomicMax(il.bound + 1, __float_as_int(vm));
+        }
     }
     __syncthreads();
+    if constexpr (BSRC == 1) {
+        if (qok && !vec_wave && 16 * half < S) load_tile16(trow + 16 * half, bcur);
+        // this pair's scale: 2^22 / B', B' = the bound on a row's sum of |dS| rounded up to a power of two (0: nothing to add)
+        const float B = 2.f * (DROP ? da.inv_keep : 1.0f) * __int_as_float(il.bound[0]) * __int_as_float(il.bound[1]);
+        int e = 0;
+        acc.scale = 0.f;
+        if (acc.on && B > 0.f && B < INFINITY) {
+            (void)frexpf(B, &e);
+            acc.scale = ldexpf(1.f, 22 - e);
+        }
+    }
 
     // ---- query tile `wave`: dQ -------------------------------------------------
     if (vec_wave) {
-        thin_rows_bwd_q<T, D, SP, DROP>(q_rm, k_rm, v_rm, g_rm, lse_l, dd_l, bias_gh,
-                                        dbias != nullptr ? dbias + ((int64_t)g * H + h) * S * S : nullptr, dQ, g, h, S, H,
-                                        scale, (NT - 1) * 32, tail, lane, da);
+        thin_rows_bwd_q<T, BT, D, SP, DROP>(q_rm, k_rm, v_rm, g_rm, lse_l, dd_l, bias_gh, bstride,
+                                            dbias != nullptr ? dbias + ((int64_t)g * H + h) * S * S : nullptr, dQ, g, h, S, H,
+                                            scale, (NT - 1) * 32, tail, lane, da, acc);
     } else {
         short4_t bq[KS], bg[KS];
 #pragma unroll
@@ -617,13 +883,26 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
         const int krow = key_of_row(col);
         const uint32_t rh = DROP ? drop_row_hash(da, g * H + h, qi) : 0u;
         T* dbrow = dbias != nullptr ? dbias + (((int64_t)g * H + h) * S + (qok ? qi : 0)) * S : nullptr;
+        const bool acc_here = BSRC == 1 && acc.on && qok;
         float16_t dq = zero16();
 #pragma unroll 1
         for (int kt = 0; kt < nt_full; ++kt) {
             const int kb = kt * 32 + 16 * half;
             if (kt + 1 < NT && hasb && qok) {
                 const int nv = S - (kb + 32);
-                if (nv > 0) load_bias16(brow + kb + 32, min(16, nv), bnext);
+                if constexpr (BSRC == 1) {
+                    if (nv > 0) load_tile16(trow + kb + 32, bnext);
+                } else {
+                    if (nv > 0) load_bias16(brow + kb + 32, min(16, nv), bnext);
+                }
+            }
+            // the ids of this lane's sixteen positions, asked for now and used after the products
+            Bias16<dbf16> spraw, etraw;
+            zero_bias16(spraw);
+            zero_bias16(etraw);
+            if (acc_here && kb < S) {
+                load_bias16(reinterpret_cast<const dbf16*>(acc.sp) + (int64_t)qi * S + kb, min(16, S - kb), spraw);
+                if (acc.F == 1) load_bias16(reinterpret_cast<const dbf16*>(acc.et) + (int64_t)qi * S + kb, min(16, S - kb), etraw);
             }
             float16_t sc = zero16(), dp = zero16();
 #pragma unroll
@@ -649,6 +928,20 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
             for (int t = 0; t < 4; ++t) {
                 db[t].x = f2bf(sc[4 * t + 0]); db[t].y = f2bf(sc[4 * t + 1]);
                 db[t].z = f2bf(sc[4 * t + 2]); db[t].w = f2bf(sc[4 * t + 3]);
+            }
+            if (acc_here && kb < S) {      // dS into the table accumulators (keys past the end carry zeros)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc_spatial(acc, sc[r], (spraw.w[r >> 1] >> (16 * (r & 1))) & 0xffffu);
+                // most pairs of nodes are not edges (id 0): a lane whose sixteen edge ids are all zero skips them
+                if (acc.F == 1 && (etraw.w[0] | etraw.w[1] | etraw.w[2] | etraw.w[3] | etraw.w[4] | etraw.w[5] | etraw.w[6] | etraw.w[7])) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc_edge(acc, sc[r], (etraw.w[r >> 1] >> (16 * (r & 1))) & 0xffffu);
+                }
+                if (acc.F != 1) {
+                    for (int r = 0; r < 16; ++r)
+                        if (sc[r] != 0.f)
+                            for (int f = 0; f < acc.F; ++f) acc_edge(acc, sc[r], acc.et[((int64_t)qi * S + kb + r) * acc.F + f]);
+                }
             }
             // dBias = dS: this lane holds 16 consecutive keys of its query row, one 32/64-byte piece
             if (dbrow != nullptr && qok) {
@@ -697,6 +990,11 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
                 for (int r = 0; r < 4; ++r)
                     if (r < tail) st1(dbrow + kb + r, s4[r]);
             }
+            if (acc_here && half == 0) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (r < tail) acc_position(acc, s4[r], (int64_t)qi * S + kb + r);
+            }
             short4_t db0;
             db0.x = f2bf(s4[0]); db0.y = f2bf(s4[1]); db0.z = f2bf(s4[2]); db0.w = f2bf(s4[3]);
             short4_t ak = zero4();
@@ -714,8 +1012,8 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
 
     // ---- key tile `wave`: dK, dV -------------------------------------------------
     if (vec_wave) {
-        thin_rows_bwd_k<T, D, SP, DROP>(q_rm, k_rm, v_rm, g_rm, lse_l, dd_l, bias_gh, dK, dV, g, h, S, H, scale,
-                                        (NT - 1) * 32, tail, lane, da);
+        thin_rows_bwd_k<T, BT, D, SP, DROP>(q_rm, k_rm, v_rm, g_rm, lse_l, dd_l, bias_gh, bstride, dK, dV, g, h, S, H, scale,
+                                            (NT - 1) * 32, tail, lane, da);
     } else {
         const int k0 = wave * 32, ki = k0 + col;
         const bool kok = ki < S;
@@ -727,7 +1025,7 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
         }
         // register r of a lane is query qt*32 + 8*(r/4) + 4*half + r%4; for one r the 32 lanes of a
         // half read 32 consecutive keys of that query's bias row (second read of the slice: L2)
-        const T* bcol = hasb ? bias_gh + (kok ? ki : 0) : nullptr;
+        const BT* bcol = hasb ? bias_gh + (kok ? ki : 0) : nullptr;
         decltype(raw1(bcol)) braw[16], braw_next[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) { braw[r] = 0; braw_next[r] = 0; }
@@ -735,7 +1033,7 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int qq = 8 * (r / 4) + 4 * half + (r % 4);
-                if (qq < S) braw[r] = raw1(bcol + (int64_t)qq * S);
+                if (qq < S) braw[r] = raw1(bcol + (int64_t)qq * bstride);
             }
         }
         const float scale2 = scale * kLog2e;
@@ -746,7 +1044,7 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int qq = (qt + 1) * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-                    if (qq < S) braw_next[r] = raw1(bcol + (int64_t)qq * S);
+                    if (qq < S) braw_next[r] = raw1(bcol + (int64_t)qq * bstride);
                 }
             }
             float16_t sc = zero16(), dp = zero16();
@@ -846,6 +1144,31 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
             }
         }
     }
+    if constexpr (BSRC == 0) break;      // one pair per workgroup: no loop as far as the compiler is concerned
+    __syncthreads();     // the LDS images and the bias tile are rewritten for the next pair
+    if (acc.on) {
+        // This pair's integer sums, converted with its scale, go into the workgroup's partial in global memory -
+        // [ns] spatial, [ne] edge (with the mean's 1 / F), [1] virtual - and the accumulators start the next pair at
+        // zero.  Only this workgroup touches its partial, one thread per entry.
+        float* mine = ia.partial + (int64_t)blockIdx.x * (ia.ns + ia.ne + 1);
+        const float unit = acc.scale > 0.f ? 1.f / acc.scale : 0.f, unit_e = unit / (float)ia.F;
+        for (int k = threadIdx.x; k <= ia.ns; k += blockDim.x) {
+            int t = il.accS[k];
+            il.accS[k] = 0;
+            if (k < acc.hot_n)
+                for (int c = 0; c < kHotCopies; ++c) { t += il.hot[c * kHotStride + k]; il.hot[c * kHotStride + k] = 0; }
+            const int at = k < ia.ns ? k : ia.ns + ia.ne;           // slot ns of the spatial accumulators is the virtual distance's
+            if (k != 0) mine[at] += (float)t * unit;                // slot 0: the padding index, no gradient
+        }
+        for (int k = threadIdx.x; k < ia.ne; k += blockDim.x) {
+            const int t = il.accE[k];
+            il.accE[k] = 0;
+            mine[ia.ns + k] += (float)t * unit_e;
+        }
+        if (threadIdx.x == 0) { il.bound[0] = 0; il.bound[1] = 0; }
+        __syncthreads();
+    }
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -860,102 +1183,130 @@ struct DenseCall {
     hipStream_t st;
     float p_drop;          // 0: no dropout
     uint64_t seed;
+    IdsArgs ids;           // BSRC = 1 only
 };
 
-template <typename T, int D, int NT>
+static int device_cus() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
+            n > 0)
+            cus = n;
+        else
+            cus = 256;
+    }
+    return cus;
+}
+// Workgroups of the id form's backward: what the GPU keeps resident at two per CU, a multiple of 8 H so that a
+// workgroup stays with one head, at most one per pair.  It also sizes the workspace of table partials.
+static int ids_bwd_grid(int b, int H) {
+    const int unit = 8 * H, total_pairs = ((b + 7) / 8) * unit;
+    return std::min(total_pairs, std::max(unit, 2 * device_cus() / unit * unit));
+}
+
+template <typename T, int D, int NT, int BSRC>
 static int launch_dense(const DenseCall& c, bool bwd) {
-    constexpr int lds_f = fwd_lds_bytes<D, NT>(), lds_b = bwd_lds_bytes<D, NT>();
-    if constexpr (lds_f > kLdsLimit || lds_b > kLdsLimit) {
+    constexpr int lds_f0 = fwd_lds_bytes<D, NT>(), lds_b0 = bwd_lds_bytes<D, NT>();
+    if constexpr (lds_f0 > kLdsLimit || lds_b0 > kLdsLimit) {
         set_error("dense attention: S=%d with head dim %d needs %d bytes of LDS (limit %d)", c.S, c.d,
-                  lds_b > lds_f ? lds_b : lds_f, kLdsLimit);
+                  lds_b0 > lds_f0 ? lds_b0 : lds_f0, kLdsLimit);
         return TGT_ERR_UNSUPPORTED;
     } else {
+        const size_t lds_f = lds_f0 + (BSRC == 1 ? ids_lds_bytes(c.S, c.ids.ns, c.ids.ne, false) : 0);
+        const size_t lds_b = lds_b0 + (BSRC == 1 ? ids_lds_bytes(c.S, c.ids.ns, c.ids.ne, true) : 0);
+        if ((bwd ? lds_b : lds_f) > (size_t)kLdsLimit) {
+            set_error("dense attention from ids: S=%d with tables of %d + %d rows needs %zu bytes of LDS (limit %d); "
+                      "build the bias tensor instead", c.S, c.ids.ns, c.ids.ne, bwd ? lds_b : lds_f, kLdsLimit);
+            return TGT_ERR_UNSUPPORTED;
+        }
         const float scale = sqrtf((float)c.d);     // the reference MULTIPLIES q by sqrt(d)
         const dim3 block(64 * NT);
         static bool attr_done = false;     // raise the dynamic-LDS cap once per instantiation
         if (!attr_done) {
-            if (lds_f > 48 * 1024) {
-                TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_dense_fwd<T, D, NT, false>),
-                                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_f));
-                TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_dense_fwd<T, D, NT, true>),
-                                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_f));
+            const int cap_f = BSRC == 1 ? kLdsLimit : lds_f0, cap_b = BSRC == 1 ? kLdsLimit : lds_b0;
+            if (cap_f > 48 * 1024) {
+                TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_dense_fwd<T, D, NT, false, BSRC>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, cap_f));
+                TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_dense_fwd<T, D, NT, true, BSRC>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, cap_f));
             }
-            if (lds_b > 48 * 1024) {
-                TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_dense_bwd<T, D, NT, false>),
-                                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_b));
-                TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_dense_bwd<T, D, NT, true>),
-                                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_b));
+            if (cap_b > 48 * 1024) {
+                TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_dense_bwd<T, D, NT, false, BSRC>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, cap_b));
+                TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_dense_bwd<T, D, NT, true, BSRC>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, cap_b));
             }
             attr_done = true;
         }
-        const int total_pairs = ((c.b + 7) / 8) * 8 * c.H;
+        const int unit = 8 * c.H, total_pairs = ((c.b + 7) / 8) * unit;
         // Forward: a persistent grid of about three workgroups per CU (measured best; more resident
-        // workgroups only add cache pressure), a multiple of 8 (one share per XCD).  Backward: one
-        // workgroup per pair (it runs longer per pair, persistence does not pay there).
-        static int fwd_grid = 0;
-        if (fwd_grid == 0) {
-            int dev = 0, cus = 0;
-            TGT_HIP_CHECK(hipGetDevice(&dev));
-            TGT_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-            fwd_grid = std::max(8, (3 * cus) & ~7);
-        }
-        const int nblk = bwd ? total_pairs : std::min(total_pairs, fwd_grid);
+        // workgroups only add cache pressure), a multiple of 8 (one share per XCD; of 8 H with ids: one
+        // head per workgroup).  Backward with the bias in memory: one workgroup per pair.
+        int fwd_grid = std::max(8, (3 * device_cus()) & ~7);
+        if (BSRC == 1) fwd_grid = std::max(unit, fwd_grid / unit * unit);
+        const int nblk = bwd ? (BSRC == 1 ? ids_bwd_grid(c.b, c.H) : total_pairs) : std::min(total_pairs, fwd_grid);
         const dim3 grid((unsigned)nblk);
         const bool drop = c.p_drop > 0.f;
         const DropArgs da = drop_args(c.p_drop, c.seed);
         if (!bwd) {
             KernelTimer t(KS_DENSE_FWD, c.st);
             if (drop)
-                hipLaunchKernelGGL((k_dense_fwd<T, D, NT, true>), grid, block, lds_f, c.st, (const T*)c.q, (const T*)c.k,
-                                   (const T*)c.v, (const T*)c.bias, (T*)c.o_out, c.o_lse, c.S, c.H, scale, c.b, da);
+                hipLaunchKernelGGL((k_dense_fwd<T, D, NT, true, BSRC>), grid, block, lds_f, c.st, (const T*)c.q, (const T*)c.k,
+                                   (const T*)c.v, (const T*)c.bias, (T*)c.o_out, c.o_lse, c.S, c.H, scale, c.b, da, c.ids);
             else
-                hipLaunchKernelGGL((k_dense_fwd<T, D, NT, false>), grid, block, lds_f, c.st, (const T*)c.q, (const T*)c.k,
-                                   (const T*)c.v, (const T*)c.bias, (T*)c.o_out, c.o_lse, c.S, c.H, scale, c.b, da);
+                hipLaunchKernelGGL((k_dense_fwd<T, D, NT, false, BSRC>), grid, block, lds_f, c.st, (const T*)c.q, (const T*)c.k,
+                                   (const T*)c.v, (const T*)c.bias, (T*)c.o_out, c.o_lse, c.S, c.H, scale, c.b, da, c.ids);
         } else {
             KernelTimer t(KS_DENSE_BWD, c.st);
             if (drop)
-                hipLaunchKernelGGL((k_dense_bwd<T, D, NT, true>), grid, block, lds_b, c.st, (const T*)c.q, (const T*)c.k,
+                hipLaunchKernelGGL((k_dense_bwd<T, D, NT, true, BSRC>), grid, block, lds_b, c.st, (const T*)c.q, (const T*)c.k,
                                    (const T*)c.v, (const T*)c.bias, (const T*)c.out, c.lse, (const T*)c.dout,
-                                   (T*)c.dq, (T*)c.dk, (T*)c.dv, (T*)c.dbias, c.S, c.H, scale, c.b, da);
+                                   (T*)c.dq, (T*)c.dk, (T*)c.dv, (T*)c.dbias, c.S, c.H, scale, c.b, da, c.ids);
             else
-                hipLaunchKernelGGL((k_dense_bwd<T, D, NT, false>), grid, block, lds_b, c.st, (const T*)c.q, (const T*)c.k,
+                hipLaunchKernelGGL((k_dense_bwd<T, D, NT, false, BSRC>), grid, block, lds_b, c.st, (const T*)c.q, (const T*)c.k,
                                    (const T*)c.v, (const T*)c.bias, (const T*)c.out, c.lse, (const T*)c.dout,
-                                   (T*)c.dq, (T*)c.dk, (T*)c.dv, (T*)c.dbias, c.S, c.H, scale, c.b, da);
+                                   (T*)c.dq, (T*)c.dk, (T*)c.dv, (T*)c.dbias, c.S, c.H, scale, c.b, da, c.ids);
         }
         TGT_HIP_CHECK(hipGetLastError());
         return TGT_OK;
     }
 }
 
-template <typename T, int D>
+template <typename T, int D, int BSRC>
 static int dispatch_nt(const DenseCall& c, bool bwd) {
     switch ((c.S + 31) / 32) {
-        case 1: return launch_dense<T, D, 1>(c, bwd);
-        case 2: return launch_dense<T, D, 2>(c, bwd);
-        case 3: return launch_dense<T, D, 3>(c, bwd);
-        case 4: return launch_dense<T, D, 4>(c, bwd);
-        case 5: return launch_dense<T, D, 5>(c, bwd);
-        case 6: return launch_dense<T, D, 6>(c, bwd);
-        case 7: return launch_dense<T, D, 7>(c, bwd);
-        case 8: return launch_dense<T, D, 8>(c, bwd);
+        case 1: return launch_dense<T, D, 1, BSRC>(c, bwd);
+        case 2: return launch_dense<T, D, 2, BSRC>(c, bwd);
+        case 3: return launch_dense<T, D, 3, BSRC>(c, bwd);
+        case 4: return launch_dense<T, D, 4, BSRC>(c, bwd);
+        case 5: return launch_dense<T, D, 5, BSRC>(c, bwd);
+        case 6: return launch_dense<T, D, 6, BSRC>(c, bwd);
+        case 7: return launch_dense<T, D, 7, BSRC>(c, bwd);
+        case 8: return launch_dense<T, D, 8, BSRC>(c, bwd);
         default:
             set_error("dense attention: sequence length %d exceeds 256", c.S);
             return TGT_ERR_UNSUPPORTED;
     }
 }
 
-template <typename T>
+template <typename T, int BSRC>
 static int dispatch_d(const DenseCall& c, bool bwd) {
     switch (c.d) {
-        case 8: return dispatch_nt<T, 8>(c, bwd);
-        case 16: return dispatch_nt<T, 16>(c, bwd);
-        case 32: return dispatch_nt<T, 32>(c, bwd);
+        case 8: return dispatch_nt<T, 8, BSRC>(c, bwd);
+        case 16: return dispatch_nt<T, 16, BSRC>(c, bwd);
+        case 32: return dispatch_nt<T, 32, BSRC>(c, bwd);
         default:
             set_error("dense attention: head dim %d not in {8, 16, 32}", c.d);
             return TGT_ERR_UNSUPPORTED;
     }
 }
 
+#ifndef TGT_DENSE_PART
+#error "compile with -DTGT_DENSE_PART=0 (bias tensor entry points) or 1 (id + table entry points)"
+#endif
+
+#if TGT_DENSE_PART == 0
 // keep[g, h, q, k] (1 = kept) of the dropout the attention kernels apply for (p, seed)
 __global__ void k_dropout_mask(uint8_t* __restrict__ out, int S, int H, int64_t total, const DropArgs da) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -966,6 +1317,8 @@ __global__ void k_dropout_mask(uint8_t* __restrict__ out, int S, int H, int64_t 
     const int pair = (int)(r / S);
     out[i] = drop_keep(da, drop_row_hash(da, pair, q), k) ? 1 : 0;
 }
+
+#endif
 
 static int check_dense(const void* q, const void* k, const void* v, int b, int S, int H, int d, int dtype) {
     if (!q || !k || !v) { set_error("dense attention: null q/k/v"); return TGT_ERR_INVALID_ARG; }
@@ -981,6 +1334,7 @@ static int check_dense(const void* q, const void* k, const void* v, int b, int S
 
 }  // namespace tgt
 
+#if TGT_DENSE_PART == 0
 extern "C" {
 
 int tgt_dense_attn_dropout_fwd(const void* d_q, const void* d_k, const void* d_v, const void* d_bias, int b, int S,
@@ -1001,7 +1355,7 @@ int tgt_dense_attn_dropout_fwd(const void* d_q, const void* d_k, const void* d_v
         f.p_drop = p_drop; f.seed = seed;
         return tgt::dense_attn_f32(f, false);
     }
-    return dtype == TGT_DTYPE_F32_BF16_PRODUCTS ? tgt::dispatch_d<float>(c, false) : tgt::dispatch_d<tgt::dbf16>(c, false);
+    return dtype == TGT_DTYPE_F32_BF16_PRODUCTS ? tgt::dispatch_d<float, 0>(c, false) : tgt::dispatch_d<tgt::dbf16, 0>(c, false);
 }
 
 int tgt_dense_attn_fwd(const void* d_q, const void* d_k, const void* d_v, const void* d_bias, int b, int S, int H,
@@ -1052,7 +1406,163 @@ int tgt_dense_attn_dropout_bwd(const void* d_q, const void* d_k, const void* d_v
         f.b = b; f.S = S; f.H = H; f.d = d; f.st = c.st; f.p_drop = p_drop; f.seed = seed;
         return tgt::dense_attn_f32(f, true);
     }
-    return dtype == TGT_DTYPE_F32_BF16_PRODUCTS ? tgt::dispatch_d<float>(c, true) : tgt::dispatch_d<tgt::dbf16>(c, true);
+    return dtype == TGT_DTYPE_F32_BF16_PRODUCTS ? tgt::dispatch_d<float, 0>(c, true) : tgt::dispatch_d<tgt::dbf16, 0>(c, true);
 }
 
 }  // extern "C"
+#endif
+
+#if TGT_DENSE_PART == 1
+// ---------------------------------------------------------------------------
+// The id + table form: entry points
+// ---------------------------------------------------------------------------
+namespace tgt {
+
+__device__ __forceinline__ uint16_t pack_id(int64_t v, int n) { return (uint16_t)(v < 0 ? 0 : (v >= n ? n - 1 : v)); }
+
+// one thread per position of the padded [S1, S1] index space
+__global__ __launch_bounds__(256) void k_ids_pack(const int64_t* __restrict__ spatial_pos, const int64_t* __restrict__ edge_type,
+                                                  int b, int s, int F, int ns, int ne, uint16_t* __restrict__ sp16,
+                                                  uint16_t* __restrict__ et16) {
+    const int S1 = s + 1;
+    const int64_t total = (int64_t)b * S1 * S1;
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= total) return;
+    const int j = (int)(t % S1), i = (int)((t / S1) % S1);
+    const int64_t g = t / ((int64_t)S1 * S1);
+    if (i >= 1 && j >= 1) {
+        const int64_t pos = (g * s + (i - 1)) * s + (j - 1);
+        sp16[t] = pack_id(spatial_pos[pos], ns);
+        for (int f = 0; f < F; ++f) et16[t * F + f] = pack_id(edge_type[pos * F + f], ne);
+    } else {
+        sp16[t] = (uint16_t)ns;                       // the virtual distance's slot
+        for (int f = 0; f < F; ++f) et16[t * F + f] = (uint16_t)ne;     // a slot that holds 0
+    }
+}
+
+// Table gradients from the workgroup partials: thread (h, k) adds the partials of the workgroups of head h
+// (ids 8 h .. 8 h + 7 in every window of 8 H) in workgroup order.
+template <typename T>
+__global__ __launch_bounds__(256) void k_ids_reduce(const float* __restrict__ partial, int grid, int H, int ns, int ne,
+                                                    T* __restrict__ d_sp, T* __restrict__ d_e, T* __restrict__ d_v) {
+    const int n_acc = ns + ne + 1;
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n_acc * H) return;
+    const int h = idx / n_acc, k = idx - h * n_acc;
+    float t = 0.f;
+    for (int w0 = 8 * h; w0 < grid; w0 += 8 * H)
+        for (int x = 0; x < 8; ++x) t += partial[(int64_t)(w0 + x) * n_acc + k];
+    if (k < ns) st1(d_sp + (int64_t)k * H + h, t);
+    else if (k < ns + ne) st1(d_e + (int64_t)(k - ns) * H + h, t);
+    else st1(d_v + h, t);
+}
+
+static int check_ids(const void* sp16, const void* et16, int F, const void* sp_tab, int ns, const void* e_tab, int ne,
+                     const void* vd, int H, int dtype) {
+    if (!sp16 || !et16 || !sp_tab || !e_tab || !vd) { set_error("dense attention from ids: null ids or tables"); return TGT_ERR_INVALID_ARG; }
+    if (F < 1 || ns < 1 || ne < 1 || ns > 65534 || ne > 65534) {
+        set_error("dense attention from ids: F >= 1 and table sizes in 1..65534 needed (F=%d, %d, %d)", F, ns, ne);
+        return TGT_ERR_INVALID_ARG;
+    }
+    if (dtype == TGT_DTYPE_F32) {
+        set_error("dense attention from ids: the float32-arithmetic kernels read a bias tensor; build it with "
+                  "tgt_graph_attn_bias_fwd, or pass TGT_DTYPE_F32_BF16_PRODUCTS");
+        return TGT_ERR_UNSUPPORTED;
+    }
+    if (H > 32) { set_error("dense attention from ids: at most 32 heads"); return TGT_ERR_UNSUPPORTED; }
+    return TGT_OK;
+}
+
+}  // namespace tgt
+
+extern "C" {
+
+int tgt_dense_ids_pack(const int64_t* d_spatial_pos, const int64_t* d_edge_type, int b, int s, int F, int num_spatial,
+                       int num_edges, uint16_t* d_sp16, uint16_t* d_et16, void* stream) {
+    using namespace tgt;
+    if (b < 1 || s < 0 || F < 1 || num_spatial < 1 || num_edges < 1 || num_spatial > 65534 || num_edges > 65534 || !d_sp16 ||
+        !d_et16 || (s > 0 && (!d_spatial_pos || !d_edge_type))) {
+        set_error("tgt_dense_ids_pack: bad size (table sizes must be 1..65534) or null pointer");
+        return TGT_ERR_INVALID_ARG;
+    }
+    const int64_t total = (int64_t)b * (s + 1) * (s + 1);
+    hipLaunchKernelGGL(k_ids_pack, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, d_spatial_pos,
+                       d_edge_type, b, s, F, num_spatial, num_edges, d_sp16, d_et16);
+    TGT_HIP_CHECK(hipGetLastError());
+    return TGT_OK;
+}
+
+int tgt_dense_attn_ids_fwd(const void* d_q, const void* d_k, const void* d_v, const void* d_attn_bias,
+                           const uint16_t* d_sp16, const uint16_t* d_et16, int F, const void* d_spatial_table, int num_spatial,
+                           const void* d_edge_table, int num_edges, const void* d_virtual_dist, int b, int S, int H, int d,
+                           int dtype, float p_drop, uint64_t seed, void* d_out, float* d_lse, void* stream) {
+    using namespace tgt;
+    int rc = check_dense(d_q, d_k, d_v, b, S, H, d, dtype);
+    if (rc) return rc;
+    rc = check_ids(d_sp16, d_et16, F, d_spatial_table, num_spatial, d_edge_table, num_edges, d_virtual_dist, H, dtype);
+    if (rc) return rc;
+    if (!d_out || !d_lse) { set_error("dense attention: null out or lse"); return TGT_ERR_INVALID_ARG; }
+    if (!(p_drop >= 0.f && p_drop < 1.f)) { set_error("dense attention: dropout rate %g outside [0, 1)", p_drop); return TGT_ERR_INVALID_ARG; }
+    DenseCall c{};
+    c.q = d_q; c.k = d_k; c.v = d_v; c.o_out = d_out; c.o_lse = d_lse;
+    c.b = b; c.S = S; c.H = H; c.d = d; c.st = (hipStream_t)stream;
+    c.p_drop = p_drop; c.seed = seed;
+    c.ids = IdsArgs{d_attn_bias, d_sp16, d_et16, d_spatial_table, d_edge_table, d_virtual_dist, nullptr, F, num_spatial, num_edges};
+    return dtype == TGT_DTYPE_F32_BF16_PRODUCTS ? dispatch_d<float, 1>(c, false) : dispatch_d<dbf16, 1>(c, false);
+}
+
+int64_t tgt_dense_attn_ids_bwd_workspace_bytes(int b, int H, int num_spatial, int num_edges) {
+    using namespace tgt;
+    if (b < 1 || H < 1 || num_spatial < 1 || num_edges < 1) return 0;
+    return (int64_t)sizeof(float) * ids_bwd_grid(b, H) * (num_spatial + num_edges + 1);
+}
+
+int tgt_dense_attn_ids_bwd(const void* d_q, const void* d_k, const void* d_v, const void* d_attn_bias,
+                           const uint16_t* d_sp16, const uint16_t* d_et16, int F, const void* d_spatial_table, int num_spatial,
+                           const void* d_edge_table, int num_edges, const void* d_virtual_dist, int b, int S, int H, int d,
+                           int dtype, float p_drop, uint64_t seed, const void* d_out, const float* d_lse, const void* d_dout,
+                           void* d_dq, void* d_dk, void* d_dv, void* d_dspatial_table, void* d_dedge_table,
+                           void* d_dvirtual_dist, void* d_workspace, int64_t workspace_bytes, void* stream) {
+    using namespace tgt;
+    int rc = check_dense(d_q, d_k, d_v, b, S, H, d, dtype);
+    if (rc) return rc;
+    rc = check_ids(d_sp16, d_et16, F, d_spatial_table, num_spatial, d_edge_table, num_edges, d_virtual_dist, H, dtype);
+    if (rc) return rc;
+    if (!(p_drop >= 0.f && p_drop < 1.f)) { set_error("dense attention: dropout rate %g outside [0, 1)", p_drop); return TGT_ERR_INVALID_ARG; }
+    if (!d_out || !d_lse || !d_dout || !d_dq || !d_dk || !d_dv) {
+        set_error("dense attention backward: null out/lse/dout/dq/dk/dv");
+        return TGT_ERR_INVALID_ARG;
+    }
+    const bool tables = d_dspatial_table || d_dedge_table || d_dvirtual_dist;
+    if (tables && !(d_dspatial_table && d_dedge_table && d_dvirtual_dist)) {
+        set_error("dense attention from ids, backward: the three table gradients come together (all or none)");
+        return TGT_ERR_INVALID_ARG;
+    }
+    if (tables && (!d_workspace || ((uintptr_t)d_workspace & 15) ||
+                   workspace_bytes < tgt_dense_attn_ids_bwd_workspace_bytes(b, H, num_spatial, num_edges))) {
+        set_error("dense attention from ids, backward: workspace of %lld bytes (16-byte aligned) needed, got %lld",
+                  (long long)tgt_dense_attn_ids_bwd_workspace_bytes(b, H, num_spatial, num_edges), (long long)workspace_bytes);
+        return TGT_ERR_WORKSPACE;
+    }
+    DenseCall c{};
+    c.q = d_q; c.k = d_k; c.v = d_v; c.out = d_out; c.lse = d_lse; c.dout = d_dout;
+    c.dq = d_dq; c.dk = d_dk; c.dv = d_dv;
+    c.b = b; c.S = S; c.H = H; c.d = d; c.st = (hipStream_t)stream;
+    c.p_drop = p_drop; c.seed = seed;
+    c.ids = IdsArgs{d_attn_bias, d_sp16, d_et16, d_spatial_table, d_edge_table, d_virtual_dist,
+                    tables ? (float*)d_workspace : nullptr, F, num_spatial, num_edges};
+    rc = dtype == TGT_DTYPE_F32_BF16_PRODUCTS ? dispatch_d<float, 1>(c, true) : dispatch_d<dbf16, 1>(c, true);
+    if (rc != TGT_OK || !tables) return rc;
+    const int grid = ids_bwd_grid(b, H), n = (num_spatial + num_edges + 1) * H;
+    if (dtype == TGT_DTYPE_F32_BF16_PRODUCTS)
+        hipLaunchKernelGGL((k_ids_reduce<float>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, c.st, (const float*)d_workspace,
+                           grid, H, num_spatial, num_edges, (float*)d_dspatial_table, (float*)d_dedge_table, (float*)d_dvirtual_dist);
+    else
+        hipLaunchKernelGGL((k_ids_reduce<dbf16>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, c.st, (const float*)d_workspace,
+                           grid, H, num_spatial, num_edges, (dbf16*)d_dspatial_table, (dbf16*)d_dedge_table, (dbf16*)d_dvirtual_dist);
+    TGT_HIP_CHECK(hipGetLastError());
+    return TGT_OK;
+}
+
+}  // extern "C"
+#endif

@@ -80,6 +80,7 @@ struct SparseAttention : public torch::autograd::Function<SparseAttention> {
         ctx->saved_data["mode"] = mode;
         ctx->saved_data["bias_grad"] = b.defined() && bias->requires_grad();
         ctx->mark_non_differentiable({Z});
+        ctx->set_materialize_grads(false);       // no zero tensor is made for Z's absent gradient
         return {out, Z};
     }
     static variable_list backward(AutogradContext* ctx, variable_list grads) {
@@ -87,6 +88,7 @@ struct SparseAttention : public torch::autograd::Function<SparseAttention> {
         const Tensor &q = saved[0], &k = saved[1], &v = saved[2], &b = saved[3], &out = saved[4], &Z = saved[5], &ws = saved[6];
         const int64_t plan = ctx->saved_data["plan"].toCustomClass<PlanHolder>()->h, mode = ctx->saved_data["mode"].toInt();
         const int64_t H = q.size(1), d = q.size(2);
+        if (!grads[0].defined()) return {Tensor(), Tensor(), Tensor(), Tensor(), Tensor(), Tensor(), Tensor()};
         Tensor dout = grads[0].contiguous();
         c10::DeviceGuard guard(q.device());
         Tensor dq = at::empty_like(q), dk = at::empty_like(k), dv = at::empty_like(v), dbias;
@@ -162,6 +164,102 @@ struct DenseAttention : public torch::autograd::Function<DenseAttention> {
 Tensor dense_attention(const Tensor& q, const Tensor& k, const Tensor& v, const c10::optional<Tensor>& bias, double p_drop,
                        int64_t seed, bool bf16_products) {
     return DenseAttention::apply(q, k, v, bias, p_drop, seed, bf16_products);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// dense attention with the bias formed in the kernels from packed ids and the three tables
+// ---------------------------------------------------------------------------------------------------------------
+struct DenseAttentionIds : public torch::autograd::Function<DenseAttentionIds> {
+    static Tensor forward(AutogradContext* ctx, Tensor q, Tensor k, Tensor v, c10::optional<Tensor> attn_bias, Tensor sp16,
+                          Tensor et16, Tensor sp_tab, Tensor e_tab, Tensor vd, double p_drop, int64_t seed, bool bf16_products) {
+        on_gpu(q, "dense attention from ids");
+        TORCH_CHECK(q.dim() == 4 && q.sizes() == k.sizes() && q.sizes() == v.sizes(), "q, k, v must be [b, S, H, d] with equal shapes");
+        TORCH_CHECK(k.scalar_type() == q.scalar_type() && v.scalar_type() == q.scalar_type(), "q/k/v must share a dtype");
+        int code = dtype_code(q);
+        TORCH_CHECK(code != TGT_DTYPE_F32 || bf16_products,
+                    "dense attention from ids computes with bf16 matrix products: pass bf16 tensors, or float32 with bf16_products");
+        if (code == TGT_DTYPE_F32) code = TGT_DTYPE_F32_BF16_PRODUCTS;
+        q = q.contiguous(); k = k.contiguous(); v = v.contiguous();
+        const int64_t b = q.size(0), S = q.size(1), H = q.size(2), d = q.size(3);
+        TORCH_CHECK(sp16.scalar_type() == at::kShort && sp16.dim() == 3 && sp16.size(0) == b && sp16.size(1) == S && sp16.size(2) == S &&
+                        sp16.is_contiguous(), "sp16 must be a contiguous int16 [b, S, S] (tgt_dense_ids_pack)");
+        TORCH_CHECK(et16.scalar_type() == at::kShort && et16.dim() == 4 && et16.size(0) == b && et16.size(1) == S && et16.size(2) == S &&
+                        et16.is_contiguous(), "et16 must be a contiguous int16 [b, S, S, F] (tgt_dense_ids_pack)");
+        const int64_t F = et16.size(3);
+        TORCH_CHECK(sp_tab.dim() == 2 && e_tab.dim() == 2 && sp_tab.size(1) == H && e_tab.size(1) == H && vd.numel() == H &&
+                        sp_tab.scalar_type() == q.scalar_type() && e_tab.scalar_type() == q.scalar_type() &&
+                        vd.scalar_type() == q.scalar_type(), "tables must be [rows, H] / [H] of q's dtype");
+        Tensor ab;
+        if (attn_bias.has_value() && attn_bias->defined()) {
+            TORCH_CHECK(attn_bias->scalar_type() == q.scalar_type() && attn_bias->dim() == 3 && attn_bias->size(0) == b &&
+                            attn_bias->size(1) == S && attn_bias->size(2) == S, "attn_bias must be [b, S, S] of q's dtype");
+            ab = attn_bias->contiguous();
+        }
+        Tensor st = sp_tab.contiguous(), et = e_tab.contiguous(), vdc = vd.reshape({-1}).contiguous();
+        c10::DeviceGuard guard(q.device());
+        Tensor out = at::empty({b, S, H * d}, q.options());
+        Tensor lse = at::empty({b, H, S}, q.options().dtype(at::kFloat));
+        check(tgt_dense_attn_ids_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), ab.defined() ? ab.data_ptr() : nullptr,
+                                     reinterpret_cast<const uint16_t*>(sp16.data_ptr()), reinterpret_cast<const uint16_t*>(et16.data_ptr()),
+                                     (int)F, st.data_ptr(), (int)st.size(0), et.data_ptr(), (int)et.size(0), vdc.data_ptr(), (int)b,
+                                     (int)S, (int)H, (int)d, code, (float)p_drop, (uint64_t)seed, out.data_ptr(),
+                                     lse.data_ptr<float>(), stream_of(q)),
+              "tgt_dense_attn_ids_fwd");
+        ctx->save_for_backward({q, k, v, ab, sp16, et16, st, et, vdc, out, lse});
+        ctx->saved_data["code"] = (int64_t)code;
+        ctx->saved_data["p"] = p_drop;
+        ctx->saved_data["seed"] = seed;
+        ctx->saved_data["vd_shape"] = vd.sizes().vec();
+        return out;
+    }
+    static variable_list backward(AutogradContext* ctx, variable_list grads) {
+        auto saved = ctx->get_saved_variables();
+        const Tensor &q = saved[0], &k = saved[1], &v = saved[2], &ab = saved[3], &sp16 = saved[4], &et16 = saved[5], &st = saved[6],
+                     &et = saved[7], &vd = saved[8], &out = saved[9], &lse = saved[10];
+        const int64_t b = q.size(0), S = q.size(1), H = q.size(2), d = q.size(3), F = et16.size(3);
+        Tensor dout = grads[0].contiguous();
+        c10::DeviceGuard guard(q.device());
+        Tensor dq = at::empty_like(q), dk = at::empty_like(k), dv = at::empty_like(v), dst, det, dvd, ws;
+        const bool tables = ctx->needs_input_grad(6) || ctx->needs_input_grad(7) || ctx->needs_input_grad(8);
+        int64_t ws_bytes = 0;
+        if (tables) {
+            dst = at::empty_like(st); det = at::empty_like(et); dvd = at::empty_like(vd);
+            ws_bytes = tgt_dense_attn_ids_bwd_workspace_bytes((int)b, (int)H, (int)st.size(0), (int)et.size(0));
+            ws = at::empty({ws_bytes}, q.options().dtype(at::kByte));
+        }
+        check(tgt_dense_attn_ids_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), ab.defined() ? ab.data_ptr() : nullptr,
+                                     reinterpret_cast<const uint16_t*>(sp16.data_ptr()), reinterpret_cast<const uint16_t*>(et16.data_ptr()),
+                                     (int)F, st.data_ptr(), (int)st.size(0), et.data_ptr(), (int)et.size(0), vd.data_ptr(), (int)b, (int)S,
+                                     (int)H, (int)d, (int)ctx->saved_data["code"].toInt(), (float)ctx->saved_data["p"].toDouble(),
+                                     (uint64_t)ctx->saved_data["seed"].toInt(), out.data_ptr(), lse.data_ptr<float>(), dout.data_ptr(),
+                                     dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), tables ? dst.data_ptr() : nullptr,
+                                     tables ? det.data_ptr() : nullptr, tables ? dvd.data_ptr() : nullptr,
+                                     tables ? ws.data_ptr() : nullptr, ws_bytes, stream_of(q)),
+              "tgt_dense_attn_ids_bwd");
+        if (tables) dvd = dvd.view(ctx->saved_data["vd_shape"].toIntVector());
+        return {dq, dk, dv, Tensor(), Tensor(), Tensor(), dst, det, dvd, Tensor(), Tensor(), Tensor()};
+    }
+};
+Tensor dense_attention_ids(const Tensor& q, const Tensor& k, const Tensor& v, const c10::optional<Tensor>& attn_bias, const Tensor& sp16,
+                           const Tensor& et16, const Tensor& sp_tab, const Tensor& e_tab, const Tensor& vd, double p_drop, int64_t seed,
+                           bool bf16_products) {
+    return DenseAttentionIds::apply(q, k, v, attn_bias, sp16, et16, sp_tab, e_tab, vd, p_drop, seed, bf16_products);
+}
+// the reference's int64 ids to the packed form, once per batch
+std::tuple<Tensor, Tensor> dense_ids_pack(const Tensor& spatial_pos, const Tensor& edge_type, int64_t num_spatial, int64_t num_edges) {
+    on_gpu(spatial_pos, "dense_ids_pack");
+    TORCH_CHECK(spatial_pos.dim() == 3 && edge_type.dim() == 4 && spatial_pos.size(1) == spatial_pos.size(2) &&
+                    edge_type.size(0) == spatial_pos.size(0) && edge_type.size(1) == spatial_pos.size(1) &&
+                    edge_type.size(2) == spatial_pos.size(1), "spatial_pos [b, s, s] and attn_edge_type [b, s, s, F] expected");
+    Tensor sp = spatial_pos.to(at::kLong).contiguous(), et = edge_type.to(at::kLong).contiguous();
+    const int64_t b = sp.size(0), s = sp.size(1), F = et.size(3);
+    c10::DeviceGuard guard(sp.device());
+    Tensor sp16 = at::empty({b, s + 1, s + 1}, sp.options().dtype(at::kShort));
+    Tensor et16 = at::empty({b, s + 1, s + 1, F}, sp.options().dtype(at::kShort));
+    check(tgt_dense_ids_pack(sp.data_ptr<int64_t>(), et.data_ptr<int64_t>(), (int)b, (int)s, (int)F, (int)num_spatial, (int)num_edges,
+                             reinterpret_cast<uint16_t*>(sp16.data_ptr()), reinterpret_cast<uint16_t*>(et16.data_ptr()), stream_of(sp)),
+          "tgt_dense_ids_pack");
+    return {sp16, et16};
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -297,6 +395,7 @@ struct AddLayerNorm : public torch::autograd::Function<AddLayerNorm> {
         ctx->save_for_backward({s, g, mean, rstd});
         ctx->saved_data["has_r"] = has_r;
         ctx->saved_data["shape"] = x.sizes().vec();
+        ctx->set_materialize_grads(false);       // an output nobody differentiates costs no zero tensor
         return {s.view(x.sizes()), y.view(x.sizes())};
     }
     static variable_list backward(AutogradContext* ctx, variable_list grads) {
@@ -372,6 +471,9 @@ TORCH_LIBRARY(torchgt, m) {
     m.def("sparse_attention(Tensor q, Tensor k, Tensor v, Tensor? bias, __torch__.torch.classes.torchgt.PlanHolder plan, int bias_mode, "
           "Tensor workspace) -> (Tensor, Tensor)");
     m.def("dense_attention(Tensor q, Tensor k, Tensor v, Tensor? bias, float p_drop, int seed, bool bf16_products) -> Tensor");
+    m.def("dense_attention_ids(Tensor q, Tensor k, Tensor v, Tensor? attn_bias, Tensor sp16, Tensor et16, Tensor spatial_table, "
+          "Tensor edge_table, Tensor virtual_dist, float p_drop, int seed, bool bf16_products) -> Tensor");
+    m.def("dense_ids_pack(Tensor spatial_pos, Tensor edge_type, int num_spatial, int num_edges) -> (Tensor, Tensor)");
     m.def("linear(Tensor x, Tensor[] weights, Tensor?[] biases) -> Tensor[]");
     m.def("add_layer_norm(Tensor x, Tensor? r, Tensor gamma, Tensor beta, float eps) -> (Tensor, Tensor)");
     m.def("add(Tensor x, Tensor r) -> Tensor");
@@ -384,6 +486,8 @@ TORCH_LIBRARY(torchgt, m) {
 TORCH_LIBRARY_IMPL(torchgt, CompositeImplicitAutograd, m) {
     m.impl("sparse_attention", sparse_attention);
     m.impl("dense_attention", dense_attention);
+    m.impl("dense_attention_ids", dense_attention_ids);
+    m.impl("dense_ids_pack", dense_ids_pack);
     m.impl("linear", linear);
     m.impl("add_layer_norm", add_layer_norm);
     m.impl("add", add);

@@ -129,7 +129,19 @@ class GraphAttnBias(nn.Module):
         self.spatial_pos_encoder = nn.Embedding(num_spatial, num_heads, padding_idx=0)
         self.graph_token_virtual_distance = nn.Embedding(1, num_heads)
 
-    def forward(self, batched_data):
+    def forward(self, batched_data, as_ids=False):
+        """The [b, H, S, S] bias; with ``as_ids=True`` (plain edge-type branch only) a ``GraphBiasIds`` that the dense
+        attention takes in its place and that builds the tensor only if a layer needs it."""
+        if as_ids and self.edge_type != "multi_hop":
+            from . import _ext
+            from .core_attention import GraphBiasIds
+            sp_w, e_w, vd_w = self.spatial_pos_encoder.weight, self.edge_encoder.weight, self.graph_token_virtual_distance.weight
+            if not batched_data.attn_bias.is_cuda:
+                raise RuntimeError("GraphAttnBias runs on the GPU only (no CPU fallback)")
+            sp16, et16 = _ext.ops().dense_ids_pack(batched_data.spatial_pos, batched_data.attn_edge_type, sp_w.shape[0], e_w.shape[0])
+            build = lambda: GraphAttnBiasFunction.apply(batched_data.attn_bias, batched_data.spatial_pos,
+                                                        batched_data.attn_edge_type, sp_w, e_w, vd_w)
+            return GraphBiasIds(batched_data.attn_bias, sp16, et16, sp_w, e_w, vd_w, build)
         if self.edge_type == "multi_hop":
             return GraphAttnBiasMultiHopFunction.apply(batched_data.attn_bias, batched_data.spatial_pos, batched_data.edge_input,
                                                        self.spatial_pos_encoder.weight, self.edge_encoder.weight,

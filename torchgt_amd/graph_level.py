@@ -136,10 +136,13 @@ class Graphormer(nn.Module):
         else:
             self.downstream_out_proj = nn.Linear(hidden_dim, output_dim)
         self.apply(lambda module: init_params(module, n_layers=n_layers))
+        # True: the layers get the bias as ids + tables and the bf16 attention kernels form it on chip (the [b, H, S, S]
+        # tensor is built only for layers that cannot: float32 arithmetic, the multi-hop branch, very long sequences)
+        self.bias_from_ids = True
 
     def forward(self, batched_data, perturb=None):
         x = self.graph_node_feature(batched_data)            # [b, s + 1, h]
-        attn_bias = self.graph_attn_bias(batched_data)       # [b, H, s + 1, s + 1]
+        attn_bias = self.graph_attn_bias(batched_data, as_ids=self.bias_from_ids)       # [b, H, s + 1, s + 1], or its ids
         output = self.input_dropout(x)
         pending = None
         for enc_layer in self.layers:
