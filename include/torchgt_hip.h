@@ -237,9 +237,10 @@ int tgt_dense_attn_ids_fwd(const void* d_q, const void* d_k, const void* d_v, co
                            int dtype, float p_drop, uint64_t seed, void* d_out, float* d_lse, void* stream);
 /* Backward: dq, dk, dv as tgt_dense_attn_dropout_bwd, and the gradients of the three tables (all three or
  * all NULL; autograd of the embedding lookups in the reference, row 0 of the spatial and edge tables is the
- * padding index and gets zero) summed over this call's batch: workgroups add dS into LDS accumulators with
- * floating-point atomics and their partials are added in a fixed order (results agree to rounding between
- * runs, not bit for bit).  d_workspace: tgt_dense_attn_ids_bwd_workspace_bytes(...) bytes, 16-byte aligned,
+ * padding index and gets zero) summed over this call's batch: workgroups add dS into fixed-point LDS
+ * accumulators (integer atomics, one power-of-two scale per (graph, head) from a bound on its dS; one unit is
+ * at most 2^-21 of that bound) and their partials are added in a fixed order: results are reproducible bit
+ * for bit.  d_workspace: tgt_dense_attn_ids_bwd_workspace_bytes(...) bytes, 16-byte aligned,
  * needed only with table gradients. */
 int64_t tgt_dense_attn_ids_bwd_workspace_bytes(int b, int H, int num_spatial, int num_edges);
 int tgt_dense_attn_ids_bwd(const void* d_q, const void* d_k, const void* d_v, const void* d_attn_bias,

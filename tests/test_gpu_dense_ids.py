@@ -113,6 +113,11 @@ def test_dense_from_ids_matches_oracle(cuda, dtype, case):
     for nm, a, r in zip(("q", "k", "v", "spatial", "edge", "virtual"), g_got, g_ref):
         assert err(a, r) <= (TOL if len(nm) == 1 else TOL_TABLE), f"d{nm} err {err(a, r)}"
     assert not g_got[3][0].any() and not g_got[4][0].any()      # padding index rows
+    # integer accumulators and fixed-order sums: a second run gives the same bits
+    g_again = torch.autograd.grad(_ext.ops().dense_attention_ids(tc[0], tc[1], tc[2], ab.to(cuda, dtype), sp16, et16, tc[3], tc[4], tc[5],
+                                                                 0.0, 0, dtype == torch.float32), tc, dout.reshape(b, S, -1).to(cuda))
+    for a, r in zip(g_again, g_got):
+        assert torch.equal(a, r)
     # the same numbers through the bias tensor (the library's other form): both round the bias to bf16 in bf16 runs
     if dtype == torch.bfloat16:
         bias = oda.graph_attn_bias(ab, sp.clamp(0, ns - 1), et_ids.clamp(0, ne - 1), st.float(), et.float(), vd.float()).to(dtype)
