@@ -168,3 +168,45 @@ def test_graphormer_forward_backward_matches_oracle(cuda):
     out = torch.log_softmax(lin(h[0, 1:, :], pd["downstream_out_proj.weight"], pd["downstream_out_proj.bias"]), 1)
     (gx_ref,) = torch.autograd.grad(torch.nn.functional.nll_loss(out, y), xd)
     assert err(gx, gx_ref) <= 1e-4, err(gx, gx_ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_layer_as_one_operator_equals_layer_op_by_op(cuda, dtype):
+    """``torch.ops.torchgt.encoder_layer`` launches the kernels the modules launch one by one, in the same order on the
+    same inputs: outputs and every gradient agree bit for bit (the attention is reproducible, the weight-gradient sums
+    have a fixed order)."""
+    torch.manual_seed(3)
+    e, n_nodes = workloads.barabasi_albert()
+    ei = torch.as_tensor(e).to(cuda)
+    m = EncoderLayer(64, 96, 0.0, 0.0, 8, 1)
+    with torch.no_grad():
+        for p in m.parameters():
+            if p.dim() == 2:
+                p.normal_(0, 0.1)
+    m = m.to(cuda, dtype)
+    x = torch.randn(1, n_nodes, 64).to(cuda, dtype)
+    r = torch.randn(1, n_nodes, 64).to(cuda, dtype)
+    gy = torch.randn(1, n_nodes, 64).to(cuda, dtype)
+    results = []
+    for fused in (False, True):
+        m.one_operator = fused
+        for residual, defer in ((None, False), (r, True)):
+            xc = x.clone().requires_grad_(True)
+            rc = None if residual is None else residual.clone().requires_grad_(True)
+            out = m(xc, None, ei, "sparse", residual=rc, defer_residual=defer)
+            outs = list(out) if defer else [out]
+            leaves = [xc] + ([rc] if rc is not None else []) + list(m.parameters())
+            grads = torch.autograd.grad(outs, leaves, [gy] * len(outs))
+            results.append([o.detach() for o in outs] + list(grads))
+    half = len(results) // 2
+    for a_case, b_case in zip(results[:half], results[half:]):
+        assert len(a_case) == len(b_case)
+        for a, b in zip(a_case, b_case):
+            assert torch.equal(a, b)
+    # in training mode with a positive dropout rate the layer runs operator by operator (torch's dropout)
+    m.one_operator = True
+    m.ffn_dropout.p = 0.5
+    m.train()
+    assert not m._one_operator(x, None, ei, "sparse")
+    m.eval()
+    assert m._one_operator(x, None, ei, "sparse")

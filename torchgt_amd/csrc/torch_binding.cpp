@@ -8,6 +8,7 @@
 //   torchgt::dense_attention(q, k, v, bias?, p_drop, seed, bf16_products) -> out
 //   torchgt::linear(x, weights[], biases?[]) -> Tensor[]                      (1 to 3 layers of one shape)
 //   torchgt::add_layer_norm(x, r?, gamma, beta, eps) -> (sum, y)
+//   torchgt::encoder_layer(x, residual?, params[16], plan holder, workspace, heads, eps1, eps2) -> (x + attention, ffn output)
 //   torchgt::add(x, r) -> sum
 //   torchgt::gelu(u) / torchgt::relu(u) -> h
 #include <torch/library.h>
@@ -464,6 +465,156 @@ struct Activation : public torch::autograd::Function<Activation<GELU>> {
 Tensor gelu(const Tensor& u) { return Activation<true>::apply(u); }
 Tensor relu(const Tensor& u) { return Activation<false>::apply(u); }
 
+// ---------------------------------------------------------------------------------------------------------------
+// one whole encoder layer of the node-level Graphormer (models/graphormer_dist_node_level.py:276-314) with sparse
+// attention, no bias, no dropout: the eight kernels of the forward and the fourteen of the backward launched from one
+// operator and one autograd node instead of eight of each.  Same kernels, same order, same numbers as the modules give
+// op by op; what goes away is the per-operator cost of the dispatcher and of autograd between the launches.
+//   s1 = x (+ residual); y1 = LN1(s1); q, k, v = y1 W^T + b; o = attention(q, k, v); a = o Wo^T + bo
+//   s2 = s1 + a; y2 = LN2(s2); u = y2 W1^T + b1; h = gelu(u); f = h W2^T + b2;  returns (s2, f)
+// params: n1.weight, n1.bias, Wq, bq, Wk, bk, Wv, bv, Wo, bo, n2.weight, n2.bias, W1, b1, W2, b2
+// ---------------------------------------------------------------------------------------------------------------
+namespace layer {
+void ln_fwd(const Tensor& x, const Tensor& r, const Tensor& g, const Tensor& b, double eps, Tensor& sum, Tensor& y, Tensor& mean,
+            Tensor& rstd) {
+    const int64_t N = x.size(0), C = x.size(1);
+    sum = r.defined() ? at::empty_like(x) : x;
+    y = at::empty_like(x);
+    mean = at::empty({N}, x.options().dtype(at::kFloat));
+    rstd = at::empty({N}, x.options().dtype(at::kFloat));
+    check(tgt_add_layer_norm_fwd(x.data_ptr(), r.defined() ? r.data_ptr() : nullptr, g.data_ptr(), b.data_ptr(), N, (int)C, (float)eps,
+                                 dtype_code(x), r.defined() ? sum.data_ptr() : nullptr, y.data_ptr(), mean.data_ptr<float>(),
+                                 rstd.data_ptr<float>(), stream_of(x)),
+          "tgt_add_layer_norm_fwd");
+}
+// ds = LN backward of dy (+ extra), dgamma, dbeta
+void ln_bwd(const Tensor& s, const Tensor& g, const Tensor& mean, const Tensor& rstd, const Tensor& dy, const Tensor& extra, Tensor& ds,
+            Tensor& dg, Tensor& db) {
+    const int64_t N = s.size(0), C = s.size(1);
+    ds = at::empty_like(s); dg = at::empty_like(g); db = at::empty_like(g);
+    const int64_t nbytes = tgt_layer_norm_bwd_workspace_bytes((int)C);
+    Tensor ws = at::empty({nbytes}, s.options().dtype(at::kByte));
+    check(tgt_layer_norm_bwd(s.data_ptr(), g.data_ptr(), mean.data_ptr<float>(), rstd.data_ptr<float>(), dy.data_ptr(),
+                             extra.defined() ? extra.data_ptr() : nullptr, N, (int)C, dtype_code(s), ds.data_ptr(), dg.data_ptr(),
+                             db.data_ptr(), ws.data_ptr(), nbytes, stream_of(s)),
+          "tgt_layer_norm_bwd");
+}
+// ys[j] = x W[j]^T + b[j]
+void lin_fwd(const Tensor& x, std::initializer_list<const Tensor*> W, std::initializer_list<const Tensor*> b, std::vector<Tensor>& ys) {
+    const int n = (int)W.size();
+    const int64_t N = x.size(0), in_f = x.size(1), out_f = (*W.begin())->size(0);
+    const void *Wp[3] = {nullptr, nullptr, nullptr}, *Bp[3] = {nullptr, nullptr, nullptr};
+    void* Yp[3] = {nullptr, nullptr, nullptr};
+    ys.clear();
+    int j = 0;
+    for (const Tensor* w : W) Wp[j++] = w->data_ptr();
+    j = 0;
+    for (const Tensor* bb : b) Bp[j++] = bb->data_ptr();
+    for (j = 0; j < n; ++j) { ys.push_back(at::empty({N, out_f}, x.options())); Yp[j] = ys.back().data_ptr(); }
+    check(tgt_linear_fwd(x.data_ptr(), Wp, Bp, Yp, n, N, (int)in_f, (int)out_f, dtype_code(x), stream_of(x)), "tgt_linear_fwd");
+}
+// dx = sum_j dy[j] W[j]; dW[j] = dy[j]^T x; db[j] = column sums of dy[j]
+void lin_bwd(const Tensor& x, std::initializer_list<const Tensor*> W, std::initializer_list<const Tensor*> dy, Tensor& dx,
+             std::vector<Tensor>& dW, std::vector<Tensor>& db) {
+    const int n = (int)W.size();
+    const int64_t N = x.size(0), in_f = x.size(1), out_f = (*W.begin())->size(0);
+    const void *Wp[3] = {nullptr, nullptr, nullptr}, *DYp[3] = {nullptr, nullptr, nullptr};
+    void *DWp[3] = {nullptr, nullptr, nullptr}, *DBp[3] = {nullptr, nullptr, nullptr};
+    dW.clear(); db.clear();
+    int j = 0;
+    for (const Tensor* w : W) { Wp[j] = w->data_ptr(); dW.push_back(at::empty_like(*w)); DWp[j] = dW.back().data_ptr();
+                                db.push_back(at::empty({out_f}, x.options())); DBp[j] = db.back().data_ptr(); ++j; }
+    j = 0;
+    for (const Tensor* d : dy) DYp[j++] = d->data_ptr();
+    dx = at::empty_like(x);
+    const int64_t ws_bytes = tgt_linear_bwd_workspace_bytes(n, (int)in_f, (int)out_f);
+    Tensor ws = at::empty({ws_bytes}, x.options().dtype(at::kByte));
+    check(tgt_linear_bwd(x.data_ptr(), Wp, DYp, n, N, (int)in_f, (int)out_f, dtype_code(x), dx.data_ptr(), DWp, DBp, ws.data_ptr(), ws_bytes,
+                         stream_of(x)),
+          "tgt_linear_bwd");
+}
+}  // namespace layer
+
+struct EncoderLayerFn : public torch::autograd::Function<EncoderLayerFn> {
+    static variable_list forward(AutogradContext* ctx, Tensor x, c10::optional<Tensor> residual, at::TensorList P,
+                                 c10::intrusive_ptr<PlanHolder> holder, Tensor ws, int64_t H, double eps1, double eps2) {
+        on_gpu(x, "encoder_layer");
+        TORCH_CHECK(P.size() == 16, "encoder_layer takes 16 parameter tensors");
+        const int64_t C = x.size(-1);
+        TORCH_CHECK(C % H == 0, "hidden size ", C, " is not a multiple of ", H, " heads");
+        for (const Tensor& p : P) TORCH_CHECK(p.defined() && p.is_cuda() && p.scalar_type() == x.scalar_type(), "parameters must be GPU tensors of x's dtype");
+        std::vector<Tensor> p;
+        for (const Tensor& t : P) p.push_back(t.contiguous());
+        c10::DeviceGuard guard(x.device());
+        Tensor x2 = x.reshape({-1, C}).contiguous(), r2;
+        if (residual.has_value() && residual->defined()) r2 = residual->reshape({-1, C}).contiguous();
+        const int64_t N = x2.size(0), d = C / H;
+        Tensor s1, y1, mean1, rstd1, s2, y2, mean2, rstd2;
+        std::vector<Tensor> qkv, a, u, f;
+        layer::ln_fwd(x2, r2, p[0], p[1], eps1, s1, y1, mean1, rstd1);
+        layer::lin_fwd(y1, {&p[2], &p[4], &p[6]}, {&p[3], &p[5], &p[7]}, qkv);
+        Tensor o = at::empty_like(qkv[0]), Z = at::empty({N, H}, x.options().dtype(at::kFloat));
+        check(tgt_sparse_attn_fwd(reinterpret_cast<const tgt_plan_t*>(holder->h), qkv[0].data_ptr(), qkv[1].data_ptr(), qkv[2].data_ptr(), nullptr,
+                                  TGT_BIAS_NONE, (int)H, (int)d, dtype_code(x), o.data_ptr(), Z.data_ptr<float>(), ws.data_ptr(), ws.numel(),
+                                  stream_of(x)),
+              "tgt_sparse_attn_fwd");
+        layer::lin_fwd(o, {&p[8]}, {&p[9]}, a);
+        layer::ln_fwd(s1, a[0], p[10], p[11], eps2, s2, y2, mean2, rstd2);
+        layer::lin_fwd(y2, {&p[12]}, {&p[13]}, u);
+        Tensor h = at::empty_like(u[0]);
+        check(tgt_gelu_fwd(u[0].data_ptr(), u[0].numel(), dtype_code(x), h.data_ptr(), stream_of(x)), "tgt_gelu_fwd");
+        layer::lin_fwd(h, {&p[14]}, {&p[15]}, f);
+        std::vector<Tensor> save{s1, mean1, rstd1, y1, qkv[0], qkv[1], qkv[2], o, Z, s2, mean2, rstd2, y2, u[0], h, ws};
+        save.insert(save.end(), p.begin(), p.end());
+        ctx->save_for_backward(save);
+        ctx->saved_data["plan"] = holder;
+        ctx->saved_data["H"] = H;
+        ctx->saved_data["has_r"] = r2.defined();
+        ctx->saved_data["shape"] = x.sizes().vec();
+        ctx->set_materialize_grads(false);
+        return {s2.view(x.sizes()), f[0].view(x.sizes())};
+    }
+    static variable_list backward(AutogradContext* ctx, variable_list grads) {
+        auto sv = ctx->get_saved_variables();
+        const Tensor &s1 = sv[0], &mean1 = sv[1], &rstd1 = sv[2], &y1 = sv[3], &q = sv[4], &k = sv[5], &v = sv[6], &o = sv[7], &Z = sv[8],
+                     &s2 = sv[9], &mean2 = sv[10], &rstd2 = sv[11], &y2 = sv[12], &u = sv[13], &h = sv[14], &ws = sv[15];
+        const Tensor* p = &sv[16];
+        const int64_t N = s1.size(0), C = s1.size(1), H = ctx->saved_data["H"].toInt(), d = C / H;
+        c10::DeviceGuard guard(s1.device());
+        Tensor d_s2, d_f;
+        if (grads[0].defined()) d_s2 = grads[0].reshape({N, C}).contiguous();
+        d_f = grads[1].defined() ? grads[1].reshape({N, C}).contiguous() : at::zeros_like(s1);
+        const int code = dtype_code(s1);
+        Tensor dh, du, dy2, ds2, do_, dy1, dx;
+        std::vector<Tensor> dW2, db2, dW1, db1, dWo, dbo, dWqkv, dbqkv;
+        layer::lin_bwd(h, {&p[14]}, {&d_f}, dh, dW2, db2);
+        du = at::empty_like(u);
+        check(tgt_gelu_bwd(u.data_ptr(), dh.data_ptr(), u.numel(), code, du.data_ptr(), stream_of(u)), "tgt_gelu_bwd");
+        layer::lin_bwd(y2, {&p[12]}, {&du}, dy2, dW1, db1);
+        Tensor dg2, dbn2, dg1, dbn1;
+        layer::ln_bwd(s2, p[10], mean2, rstd2, dy2, d_s2, ds2, dg2, dbn2);           // gradient of s2 = s1 + a: to both
+        layer::lin_bwd(o, {&p[8]}, {&ds2}, do_, dWo, dbo);
+        Tensor dq = at::empty_like(q), dk = at::empty_like(k), dv = at::empty_like(v);
+        check(tgt_sparse_attn_bwd(reinterpret_cast<const tgt_plan_t*>(ctx->saved_data["plan"].toCustomClass<PlanHolder>()->h), q.data_ptr(),
+                                  k.data_ptr(), v.data_ptr(), nullptr, TGT_BIAS_NONE, (int)H, (int)d, code, o.data_ptr(), Z.data_ptr<float>(),
+                                  do_.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), nullptr, ws.data_ptr(), ws.numel(), stream_of(q)),
+              "tgt_sparse_attn_bwd");
+        layer::lin_bwd(y1, {&p[2], &p[4], &p[6]}, {&dq, &dk, &dv}, dy1, dWqkv, dbqkv);
+        layer::ln_bwd(s1, p[0], mean1, rstd1, dy1, ds2, dx, dg1, dbn1);              // gradient of s1 = x (+ residual)
+        Tensor dxv = dx.view(ctx->saved_data["shape"].toIntVector());
+        variable_list out{dxv, ctx->saved_data["has_r"].toBool() ? dxv : Tensor(),
+                          dg1, dbn1, dWqkv[0], dbqkv[0], dWqkv[1], dbqkv[1], dWqkv[2], dbqkv[2], dWo[0], dbo[0], dg2, dbn2, dW1[0], db1[0],
+                          dW2[0], db2[0]};
+        for (int i = 0; i < 5; ++i) out.push_back(Tensor());
+        return out;
+    }
+};
+std::tuple<Tensor, Tensor> encoder_layer(const Tensor& x, const c10::optional<Tensor>& residual, at::TensorList params,
+                                         const c10::intrusive_ptr<PlanHolder>& plan, const Tensor& ws, int64_t H, double eps1, double eps2) {
+    auto r = EncoderLayerFn::apply(x, residual, params, plan, ws, H, eps1, eps2);
+    return {r[0], r[1]};
+}
+
 }  // namespace
 
 TORCH_LIBRARY(torchgt, m) {
@@ -476,6 +627,8 @@ TORCH_LIBRARY(torchgt, m) {
     m.def("dense_ids_pack(Tensor spatial_pos, Tensor edge_type, int num_spatial, int num_edges) -> (Tensor, Tensor)");
     m.def("linear(Tensor x, Tensor[] weights, Tensor?[] biases) -> Tensor[]");
     m.def("add_layer_norm(Tensor x, Tensor? r, Tensor gamma, Tensor beta, float eps) -> (Tensor, Tensor)");
+    m.def("encoder_layer(Tensor x, Tensor? residual, Tensor[] params, __torch__.torch.classes.torchgt.PlanHolder plan, Tensor workspace, "
+          "int num_heads, float eps1, float eps2) -> (Tensor, Tensor)");
     m.def("add(Tensor x, Tensor r) -> Tensor");
     m.def("gelu(Tensor u) -> Tensor");
     m.def("relu(Tensor u) -> Tensor");
@@ -490,6 +643,7 @@ TORCH_LIBRARY_IMPL(torchgt, CompositeImplicitAutograd, m) {
     m.impl("dense_ids_pack", dense_ids_pack);
     m.impl("linear", linear);
     m.impl("add_layer_norm", add_layer_norm);
+    m.impl("encoder_layer", encoder_layer);
     m.impl("add", add);
     m.impl("gelu", gelu);
     m.impl("relu", relu);

@@ -20,6 +20,7 @@ import torch.nn.functional as F
 
 from . import _ext, _lib
 from .multi_head_attention import MultiHeadAttention, fused_linear, _DT
+from .plan import GraphPlan, get_plan
 
 
 class AddLayerNormFunction:
@@ -81,11 +82,40 @@ class EncoderLayer(nn.Module):
         self.ffn = FeedForwardNetwork(hidden_size, ffn_size, dropout_rate)
         self.ffn_dropout = nn.Dropout(dropout_rate)
 
+    one_operator = True      # False: always run the layer operator by operator
+
+    def _one_operator(self, x, attn_bias, edge_index, attn_type):
+        """Whether ``torch.ops.torchgt.encoder_layer`` covers this call: sparse attention without a bias, no dropout at
+        work, feature widths the kernels read without padding."""
+        if not self.one_operator or attn_type != "sparse" or attn_bias is not None or edge_index is None or not x.is_cuda:
+            return False
+        if self.training and (self.self_attention_dropout.p > 0 or self.ffn_dropout.p > 0):
+            return False
+        att = self.self_attention
+        if att.output_layer is None or x.dtype not in _DT:
+            return False
+        ve = 4 if x.dtype == torch.float32 else 8
+        widths = (x.shape[-1], self.ffn.layer1.out_features, att.num_heads * att.att_size)
+        return all(w % ve == 0 for w in widths) and att.num_heads * att.att_size == x.shape[-1] and all(
+            lin.bias is not None for lin in (att.linear_q, att.linear_k, att.linear_v, att.output_layer, self.ffn.layer1, self.ffn.layer2))
+
     def forward(self, x, attn_bias=None, edge_index=None, attn_type=None, residual=None, defer_residual=False):
         """``residual``: a tensor still to be added to x (the previous layer's FFN output when it was
         called with ``defer_residual=True``); the add rides on this layer's first LayerNorm.
         ``defer_residual=True`` returns (x, ffn_output) instead of their sum."""
         n1, n2 = self.self_attention_norm, self.ffn_norm
+        if self._one_operator(x, attn_bias, edge_index, attn_type):
+            # the whole layer as one operator and one autograd node: the same kernels in the same order, without the
+            # per-operator cost of dispatcher and autograd between the launches
+            att = self.self_attention
+            plan = edge_index if isinstance(edge_index, GraphPlan) else get_plan(edge_index, x.numel() // x.shape[-1])
+            params = [n1.weight, n1.bias, att.linear_q.weight, att.linear_q.bias, att.linear_k.weight, att.linear_k.bias,
+                      att.linear_v.weight, att.linear_v.bias, att.output_layer.weight, att.output_layer.bias, n2.weight, n2.bias,
+                      self.ffn.layer1.weight, self.ffn.layer1.bias, self.ffn.layer2.weight, self.ffn.layer2.bias]
+            plan.handle      # raises if the plan was closed
+            x, y = _ext.ops().encoder_layer(x, residual, params, plan.holder, plan.workspace(att.num_heads, att.att_size),
+                                            att.num_heads, n1.eps, n2.eps)
+            return (x, y) if defer_residual else AddFunction.apply(x, y)
         x, y = AddLayerNormFunction.apply(x, residual, n1.weight, n1.bias, n1.eps)
         y = self.self_attention(y, attn_bias, edge_index, attn_type=attn_type)
         y = self.self_attention_dropout(y)
