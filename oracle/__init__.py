@@ -21,11 +21,17 @@ sparse_attention (gradients)   torch autograd of the restatement; analytic
                                formulas checked by fp64 gradcheck
 dense_bias_to_edge_bias        brute-force indexing loops
 dense_attention                torch.softmax/matmul library routine with the
-                               q*sqrt(d) quirk; brute-force loops
+                               q*sqrt(d) quirk; brute-force loops; with a keep
+                               mask: loops from the definition (softmax, mask /
+                               (1 - p), times v) and the p = 0 reduction
+graph_attn_bias                loops from the definition; torch's embedding for
+                               the padding-index rows of the table gradients
 fix_edge_index                 hand-computed known answer (N=3)
 relabel_by_partition           hand-computed known answer
-blockize / reformat_graph      hand-computed known answer (k=1, N=32, bs=16)
-                               + structural invariants
+blockize / reformat_graph      hand-computed known answers (k=1, N=32, bs=16;
+                               the compact-count misalignment after an empty
+                               partition pair; the raw-edge branch of a sparse
+                               tile) + structural invariants
 build_csr                      numpy stable argsort + round-trip invariants
 graph_attn_bias_multi_hop      reduces to graph_attn_bias (one hop, identity
                                hop matrices, adjacent pairs); fp64 loops from
