@@ -218,3 +218,18 @@ def test_dense_loud_failures(cuda):
         dense_attention(q, q, q, p_drop=1.0, seed=1)        # rate outside [0, 1)
     with pytest.raises(RuntimeError):
         dense_attention(q.cpu(), q.cpu(), q.cpu())
+
+
+def test_node_level_bias_layout_is_reinterpreted_like_the_reference(cuda):
+    """models/graphormer_dist_node_level.py:157-161: the node-level 'full' path receives [b, S, S, H] and views that
+    memory as [b, H, S, S] (no permute).  The module does the same."""
+    b, S, H, d = 1, 40, 4, 8
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(b, S, H, d, generator=g).to(torch.bfloat16).to(cuda) for _ in range(3))
+    bias = torch.randn(b, S, S, H, generator=g).to(torch.bfloat16).to(cuda)
+    mod = CoreAttention(H * d, 0.0, H, 1).to(cuda)
+    got = mod(q, k, v, bias, None, "full")
+    want = dense_attention(q, k, v, bias.contiguous().view(b, H, S, S))
+    assert torch.equal(got, want)
+    o_ref = oda.dense_attention(q.double().cpu(), k.double().cpu(), v.double().cpu(), bias.double().cpu().contiguous().view(b, H, S, S))
+    assert err(got, o_ref) <= TOL

@@ -136,6 +136,10 @@ def dense_attention(q, k, v, attn_bias=None, p_drop=0.0, seed=None, bf16_product
         b, S, H = q.shape[0], q.shape[1], q.shape[2]
         if attn_bias.dim() == 4 and attn_bias.shape[1] == 1 and H != 1:
             attn_bias = attn_bias.expand(b, H, S, S)
+        elif attn_bias.dim() == 4 and tuple(attn_bias.shape) == (b, S, S, H) and S != H:
+            # the node-level models hand over [b, S, S, H] and the reference REINTERPRETS that memory as [b, H, S, S]
+            # (`attn_bias.view(*output_size)`, models/graphormer_dist_node_level.py:160 - a view, not a permute)
+            attn_bias = attn_bias.contiguous().view(b, H, S, S)
         attn_bias = attn_bias.to(q.dtype)
     return DenseAttentionFunction.apply(q, k, v, attn_bias, p_drop, seed or 0, bf16_products)
 

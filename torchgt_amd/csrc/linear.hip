@@ -643,6 +643,162 @@ __global__ __launch_bounds__(kThreads) void k_linear_gradw(GradWArgs a) {
     }
 }
 
+// ---------------------------------------------------------------------------
+// in_features = out_features = 64: the whole backward in one pass over dy.  A workgroup walks panels of 64 node
+// rows; for each it forms the panel of dx = sum_j dy_j W_j (weights resident in LDS, transposed) and adds
+// dy_j^T x and the column sums of dy_j to the 64 x 64 weight-gradient tiles it keeps in registers; at its end it
+// writes one partial like k_linear_gradw (k_linear_gradw_reduce adds them).  dy is read once instead of twice and
+// one launch replaces two.  Wave w owns the 32 x 32 block (w/2, w%2) of the dx panel and of every dW_j.
+//   float32: dy and x tiles stay in their natural [node][feature] layout; the products over nodes read them with
+//            4-byte LDS accesses (the 32x32x2 instruction takes one value per lane and operand).
+//   bf16:    the products over nodes need the node index contiguous: dy and x are also scattered into transposed
+//            tiles, as in k_linear_gradw.
+// ---------------------------------------------------------------------------
+struct Bwd64Args {
+    const void* x;         // [N, 64]
+    const void* dy[3];     // [N, 64]
+    const void* W[3];      // [64, 64]
+    void* dx;              // [N, 64]
+    float* partial;        // [workers][nw][64*64 + 64]
+    int64_t N;
+};
+
+template <typename T, int NW> constexpr size_t bwd64_lds_bytes() {
+    // W^T and natural dy per weight; float32: natural x; bf16: transposed dy per weight and transposed x
+    return sizeof(T) * (size_t)64 * lds_stride<T>(64) * (sizeof(T) == 4 ? 2 * NW + 1 : 3 * NW + 1);
+}
+
+template <typename T, int NW>
+__global__ __launch_bounds__(kThreads) void k_linear64_bwd(Bwd64Args a) {
+    constexpr int S = lds_stride<T>(64);
+    constexpr bool F32 = sizeof(T) == 4;
+    extern __shared__ __align__(16) unsigned char smem[];
+    T* tW = reinterpret_cast<T*>(smem);            // [NW][64 k][S]: W_j transposed, contraction index m contiguous
+    T* tD = tW + NW * 64 * S;                      // [NW][64 nodes][S]: dy_j as in memory
+    T* tX = tD + NW * 64 * S;                      // float32: [64 nodes][S] x as in memory; bf16: [64 k][S] x transposed
+    T* tDt = tX + 64 * S;                          // bf16 only: [NW][64 m][S] dy_j transposed
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, h = lane >> 5;
+    const int rb = wave >> 1, cb = wave & 1;
+    const int64_t n_panels = (a.N + 63) / 64;
+    const T* X = reinterpret_cast<const T*>(a.x);
+    // a panel on its way from memory: natural pieces for float32, the transposing piece order for bf16 (a piece is
+    // written to the natural tile as it is and scattered into the transposed one)
+    TileRegs<T> nx_n, nd_n[NW];
+    PieceRegs<T> nx_p, nd_p[NW];
+    auto fetch = [&](int64_t p) {
+        if constexpr (F32) {
+            tile_fetch(nx_n, X, p * 64, a.N);
+#pragma unroll
+            for (int j = 0; j < NW; ++j) tile_fetch(nd_n[j], reinterpret_cast<const T*>(a.dy[j]), p * 64, a.N);
+        } else {
+            fetch_t(nx_p, X, 64, p * 64, a.N, 0, 64);
+#pragma unroll
+            for (int j = 0; j < NW; ++j) fetch_t(nd_p[j], reinterpret_cast<const T*>(a.dy[j]), 64, p * 64, a.N, 0, 64);
+        }
+    };
+    int64_t p = blockIdx.x;
+    if (p < n_panels) fetch(p);
+#pragma unroll
+    for (int j = 0; j < NW; ++j) stage_transposed<T, 64, S>(tW + j * 64 * S, reinterpret_cast<const T*>(a.W[j]), 64, 0, 64, 0, 64);
+    float16_t accw[NW];
+#pragma unroll
+    for (int j = 0; j < NW; ++j) accw[j] = zero16();
+    float colsum = 0.f;
+    for (; p < n_panels; p += gridDim.x) {
+        __syncthreads();                 // the previous panel has been read
+        if constexpr (F32) {
+            // rows past the end of the batch must read as zero here: they enter the sums over nodes
+            constexpr int VE = 4, VPR = 64 / VE, NV = (int)(sizeof(TileRegs<T>) / 16);
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int v = threadIdx.x + i * kThreads, r = v / VPR, c = (v % VPR) * VE;
+                const bool in = p * 64 + r < a.N;
+                *reinterpret_cast<uint4*>(tX + r * S + c) = zero_unless(in, nx_n.v[i]);
+#pragma unroll
+                for (int j = 0; j < NW; ++j) *reinterpret_cast<uint4*>(tD + j * 64 * S + r * S + c) = zero_unless(in, nd_n[j].v[i]);
+            }
+        } else {
+            constexpr int NV = (int)(sizeof(PieceRegs<T>) / 16);
+            put_t<T, S>(nx_p, tX, p * 64, a.N, 0, 64);
+#pragma unroll
+            for (int j = 0; j < NW; ++j) {
+                put_t<T, S>(nd_p[j], tDt + j * 64 * S, p * 64, a.N, 0, 64);
+#pragma unroll
+                for (int i = 0; i < NV; ++i) {
+                    int r, c;
+                    piece_pos<T, 64>(i, r, c);
+                    *reinterpret_cast<uint4*>(tD + j * 64 * S + r * S + c) = zero_unless(p * 64 + r < a.N, nd_p[j].v[i]);
+                }
+            }
+        }
+        __syncthreads();
+        if (p + gridDim.x < n_panels) fetch(p + gridDim.x);
+        // dx panel: rows = nodes, contraction over m
+        {
+            float16_t acc = zero16();
+#pragma unroll
+            for (int j = 0; j < NW; ++j)
+                Mma<T, 64>::run(tD + j * 64 * S + (32 * rb + l32) * S + h * 32, tW + j * 64 * S + (32 * cb + l32) * S + h * 32, acc);
+            T* out = reinterpret_cast<T*>(a.dx) + (p * 64 + 32 * rb + 4 * h) * 64 + 32 * cb + l32;
+            store_rows<T>(out, 64, acc, 0.f, a.N - (p * 64 + 32 * rb + 4 * h));
+        }
+        // dW_j block (m = 32 rb + ., k = 32 cb + .): contraction over the 64 nodes of the panel
+        if constexpr (F32) {
+            const float* ap = tD + (32 * h) * S + 32 * rb + l32;      // dy_j[node 32 h + i][m], weight j at + j * 64 * S
+            const float* bp = tX + (32 * h) * S + 32 * cb + l32;      // x[node 32 h + i][k]
+#pragma unroll 8
+            for (int i = 0; i < 32; ++i) {
+                const float xv = bp[i * S];
+#pragma unroll
+                for (int j = 0; j < NW; ++j)
+                    accw[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[j * 64 * S + i * S], xv, accw[j], 0, 0, 0);
+            }
+        } else {
+            const T* bp = tX + (32 * cb + l32) * S + h * 32;
+#pragma unroll
+            for (int j = 0; j < NW; ++j) Mma<T, 64>::run(tDt + j * 64 * S + (32 * rb + l32) * S + h * 32, bp, accw[j]);
+        }
+        if (wave < NW) {      // wave j adds up the columns of dy_j: lane = column
+            float sacc = 0.f;
+            if constexpr (F32) {
+                const float* col = tD + wave * 64 * S + lane;
+#pragma unroll 16
+                for (int i = 0; i < 64; ++i) sacc += col[i * S];
+            } else {
+                const T* row = tDt + wave * 64 * S + lane * S;
+#pragma unroll 16
+                for (int i = 0; i < 64; ++i) sacc += ld1(row + i);
+            }
+            colsum += sacc;
+        }
+    }
+    constexpr int64_t per = 64 * 64 + 64;
+    float* mine = a.partial + (int64_t)blockIdx.x * NW * per;
+#pragma unroll
+    for (int j = 0; j < NW; ++j) {
+        const int k = 32 * cb + l32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m = 32 * rb + 8 * (r >> 2) + 4 * h + (r & 3);
+            mine[j * per + (int64_t)m * 64 + k] = accw[j][r];
+        }
+    }
+    if (wave < NW) mine[wave * per + 64 * 64 + lane] = colsum;
+}
+
+template <typename T, int NW>
+int launch_bwd64(const Bwd64Args& a, int workers, hipStream_t st) {
+    constexpr size_t lds = bwd64_lds_bytes<T, NW>();
+    static bool raised = false;
+    if (!raised && lds > 48 * 1024) {
+        TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_linear64_bwd<T, NW>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        raised = true;
+    }
+    hipLaunchKernelGGL((k_linear64_bwd<T, NW>), dim3(workers), dim3(kThreads), lds, st, a);
+    return TGT_OK;
+}
+
 struct ReduceArgs {
     const float* partial;
     void* dW[3];
@@ -730,6 +886,34 @@ int launch_gradw(const GradWArgs& g, int workers, int tiles, hipStream_t st) {
 template <typename T>
 int linear_bwd_t(const void* d_x, const void* const* d_W, const void* const* d_dy, int n_out, int64_t N, int K, int M,
                  void* d_dx, void* const* d_dW, void* const* d_db, float* partial, hipStream_t st) {
+    if (d_dx && d_dW && N > 0 && K == 64 && M == 64) {
+        // one pass for dx and the weight gradients
+        constexpr size_t lds1 = bwd64_lds_bytes<T, 1>();
+        const size_t lds = lds1 + (n_out - 1) * (bwd64_lds_bytes<T, 2>() - lds1);
+        const int64_t n_panels = (N + 63) / 64;
+        const int per_cu = (int)std::max<size_t>(1, std::min<size_t>(2, (size_t)(160 * 1024) / lds));
+        const int workers = (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(n_panels, grad_workers(K, M)),
+                                                                        (int64_t)num_cus() * per_cu));
+        Bwd64Args b{};
+        b.x = d_x; b.dx = d_dx; b.partial = partial; b.N = N;
+        for (int j = 0; j < n_out; ++j) { b.dy[j] = d_dy[j]; b.W[j] = d_W[j]; }
+        int rc = TGT_OK;
+        {
+            KernelTimer t(KS_LINEAR_DX, st);
+            if (n_out == 1) rc = launch_bwd64<T, 1>(b, workers, st);
+            else if (n_out == 2) rc = launch_bwd64<T, 2>(b, workers, st);
+            else rc = launch_bwd64<T, 3>(b, workers, st);
+        }
+        if (rc != TGT_OK) return rc;
+        KernelTimer t(KS_LINEAR_DW, st);
+        ReduceArgs r{};
+        r.partial = partial; r.workers = workers; r.nw = n_out; r.K = K; r.M = M;
+        for (int j = 0; j < n_out; ++j) { r.dW[j] = d_dW[j]; r.db[j] = d_db ? d_db[j] : nullptr; }
+        const int64_t total = ((int64_t)M * K + M) * n_out;
+        hipLaunchKernelGGL((k_linear_gradw_reduce<T>), dim3((unsigned)((total + 63) / 64)), dim3(1024), 0, st, r);
+        TGT_HIP_CHECK(hipGetLastError());
+        return TGT_OK;
+    }
     if (d_dx && N > 0) {
         LinArgs a{};
         for (int j = 0; j < n_out; ++j) { a.A[j] = d_dy[j]; a.W[j] = d_W[j]; }
