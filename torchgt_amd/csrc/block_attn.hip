@@ -65,13 +65,15 @@ __device__ __forceinline__ void t_st4(tbf16* p, float a, float b, float c, float
     *reinterpret_cast<bshort4*>(p) = r;
 }
 
-// Rows no tile covers get zeros when the tile kernels write final results (no remaining edges).
+// Rows no tile covers get zeros when the tile kernels write final results (no remaining edges).  The rows are
+// listed when the tile set is built: a reordered graph normally leaves none and then nothing is launched.
 template <typename T>
-__global__ void k_zero_uncovered(const uint8_t* __restrict__ cover, int64_t N, int HD, int H, T* __restrict__ a,
+__global__ void k_zero_uncovered(const int32_t* __restrict__ rows, int64_t n_rows, int HD, int H, T* __restrict__ a,
                                  T* __restrict__ b, float* __restrict__ Z) {
-    const int64_t row = (int64_t)blockIdx.x * (blockDim.x / 8) + threadIdx.x / 8;
+    const int64_t i = (int64_t)blockIdx.x * (blockDim.x / 8) + threadIdx.x / 8;
     const int part = threadIdx.x % 8;
-    if (row >= N || cover[row]) return;
+    if (i >= n_rows) return;
+    const int64_t row = rows[i];
     for (int e = part; e < HD; e += 8) {
         if (a) a[row * HD + e] = T{};
         if (b) b[row * HD + e] = T{};
@@ -385,6 +387,8 @@ struct tgt_tiles {
     tgt::DevBuf dst_c0, dst_off, dst_r0;     // [G], [G+1], [T]
     tgt::DevBuf src_r0, src_off, src_c0;     // [Gs], [Gs+1], [T]
     tgt::DevBuf cover_dst, cover_src;        // [N] bytes
+    tgt::DevBuf bare_dst, bare_src;          // the rows cover_* marks 0
+    int64_t n_bare_dst = 0, n_bare_src = 0;
 };
 
 namespace tgt {
@@ -445,8 +449,9 @@ static int tile_fwd_launch_s(const tgt_tiles* tl, const void* q, const void* k, 
     KernelTimer t(KS_TILE_FWD, st);
     const dim3 grid((tl->n_dst_groups + W - 1) / W), block(64 * W);
     if (final_out) {
-        hipLaunchKernelGGL((k_zero_uncovered<T>), dim3((unsigned)((tl->N + 31) / 32)), dim3(256), 0, st,
-                           tl->cover_dst.as<uint8_t>(), tl->N, H * D, H, (T*)final_out, (T*)nullptr, Zp);
+        if (tl->n_bare_dst > 0)
+            hipLaunchKernelGGL((k_zero_uncovered<T>), dim3((unsigned)((tl->n_bare_dst + 31) / 32)), dim3(256), 0, st,
+                               tl->bare_dst.as<int32_t>(), tl->n_bare_dst, H * D, H, (T*)final_out, (T*)nullptr, Zp);
         if (tl->n_dst_groups > 0)
             hipLaunchKernelGGL((k_tile_fwd<T, D, H, true>), grid, block, 0, st, tl->dst_c0.as<int32_t>(),
                                tl->dst_off.as<int32_t>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
@@ -469,11 +474,12 @@ static int tile_bwd_launch_s(const tgt_tiles* tl, const void* q, const void* k, 
     KernelTimer t(KS_TILE_BWD, st);
     const dim3 gd((tl->n_dst_groups + W - 1) / W), gs((tl->n_src_groups + W - 1) / W), block(64 * W);
     if (f_dq) {
-        const dim3 gz((unsigned)((tl->N + 31) / 32));
-        hipLaunchKernelGGL((k_zero_uncovered<T>), gz, dim3(256), 0, st, tl->cover_dst.as<uint8_t>(), tl->N, H * D, H,
-                           (T*)f_dq, (T*)nullptr, (float*)nullptr);
-        hipLaunchKernelGGL((k_zero_uncovered<T>), gz, dim3(256), 0, st, tl->cover_src.as<uint8_t>(), tl->N, H * D, H,
-                           (T*)f_dk, (T*)f_dv, (float*)nullptr);
+        if (tl->n_bare_dst > 0)
+            hipLaunchKernelGGL((k_zero_uncovered<T>), dim3((unsigned)((tl->n_bare_dst + 31) / 32)), dim3(256), 0, st,
+                               tl->bare_dst.as<int32_t>(), tl->n_bare_dst, H * D, H, (T*)f_dq, (T*)nullptr, (float*)nullptr);
+        if (tl->n_bare_src > 0)
+            hipLaunchKernelGGL((k_zero_uncovered<T>), dim3((unsigned)((tl->n_bare_src + 31) / 32)), dim3(256), 0, st,
+                               tl->bare_src.as<int32_t>(), tl->n_bare_src, H * D, H, (T*)f_dk, (T*)f_dv, (float*)nullptr);
         if (tl->n_dst_groups > 0)
             hipLaunchKernelGGL((k_tile_bwd_dst<T, D, H, true>), gd, block, 0, st, tl->dst_c0.as<int32_t>(),
                                tl->dst_off.as<int32_t>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
@@ -579,6 +585,17 @@ int tgt_tiles_create(const int32_t* h_tiles, int64_t T, int block_size, int64_t 
     if (!rc) rc = tgt::upload(tl->src_c0, xs, st);
     if (!rc) rc = tgt::upload(tl->cover_dst, cd, st);
     if (!rc) rc = tgt::upload(tl->cover_src, cs, st);
+    std::vector<int32_t> bd, bs;
+    if (!rc) {
+        for (int64_t i = 0; i < N; ++i) {
+            if (i >= (int64_t)cd.size() || !cd[i]) bd.push_back((int32_t)i);
+            if (i >= (int64_t)cs.size() || !cs[i]) bs.push_back((int32_t)i);
+        }
+    }
+    tl->n_bare_dst = (int64_t)bd.size();
+    tl->n_bare_src = (int64_t)bs.size();
+    if (!rc && !bd.empty()) rc = tgt::upload(tl->bare_dst, bd, st);
+    if (!rc && !bs.empty()) rc = tgt::upload(tl->bare_src, bs, st);
     if (!rc && hipStreamSynchronize(st) != hipSuccess) rc = TGT_ERR_HIP;
     if (rc) { delete tl; return rc; }
     tl->n_dst_groups = (int32_t)kd.size();
