@@ -103,9 +103,9 @@ def _edge_input(data, D0):
     return torch.from_numpy(out)
 
 
-@pytest.mark.parametrize("edge_type,dtype", [("single_hop", torch.float32), ("multi_hop", torch.float32),
-                                             ("single_hop", torch.bfloat16)])
-def test_graph_level_graphormer_matches_oracle(cuda, edge_type, dtype):
+@pytest.mark.parametrize("edge_type,dtype,from_ids", [("single_hop", torch.float32, False), ("multi_hop", torch.float32, False),
+                                                      ("single_hop", torch.bfloat16, False), ("single_hop", torch.bfloat16, True)])
+def test_graph_level_graphormer_matches_oracle(cuda, edge_type, dtype, from_ids):
     """Graphormer-Slim shape of the graph-level scripts (hidden 64, ffn 64, 8 heads), 3 layers, ZINC tables,
     on 12 padded ER graphs: output [b, 1] and the gradient of every parameter against float64 autograd."""
     print(f"graph-level model case: {edge_type} {dtype}", flush=True)
@@ -114,6 +114,7 @@ def test_graph_level_graphormer_matches_oracle(cuda, edge_type, dtype):
     x, deg = node_inputs(data, 64, 64, 1, 3)
     torch.manual_seed(5)
     m = Graphormer(n_layers, H, 64, 0.0, 0.0, 64, "ZINC", edge_type, mhd, 0.0, 1)
+    m.bias_from_ids = from_ids          # the attention kernels form the bias from ids + tables (no [b, H, S, S] tensor)
     assert sorted(k for k in m.state_dict() if not k.startswith("layers.")) == sorted(
         ["graph_node_feature.atom_encoder.weight", "graph_node_feature.in_degree_encoder.weight",
          "graph_node_feature.out_degree_encoder.weight", "graph_node_feature.graph_token.weight",
@@ -202,3 +203,44 @@ def test_graph_level_graphormer_with_molecule_sized_tables(cuda):
         assert p.grad is not None and p.grad.shape == p.shape and torch.isfinite(p.grad).all(), k
     assert mc.graph_node_feature.atom_encoder.weight.grad[1:].any()
     assert mc.graph_attn_bias.edge_encoder.weight.grad[300].any() and mc.graph_attn_bias.spatial_pos_encoder.weight.grad[40].any()
+
+
+@pytest.mark.parametrize("dtype,from_ids", [(torch.bfloat16, True), (torch.bfloat16, False), (torch.float32, False)])
+def test_dense_layer_as_one_operator_equals_layer_op_by_op(cuda, dtype, from_ids):
+    """``torch.ops.torchgt.dense_encoder_layer`` launches the kernels the modules launch one by one: the model's output
+    and every parameter gradient agree bit for bit between the two ways of running the layers (bias tensor and bias
+    from ids; the id form's table gradients are integer sums, the weight gradients have a fixed order)."""
+    import types
+    from torchgt_amd import workloads
+    from torchgt_amd.graph_level import Graphormer
+    data = workloads.erdos_renyi_batch(batch=6, seed=9)
+    b, S = 6, data["S"]
+    rng = np.random.default_rng(1)
+    torch.manual_seed(4)
+    m = Graphormer(2, 8, 64, 0.0, 0.0, 64, "ZINC", "single_hop", 5, 0.0, 1)
+    with torch.no_grad():
+        for p_ in m.parameters():
+            if p_.dim() == 2 and p_.shape[0] > 1:
+                p_.normal_(0, 0.1)
+    m = m.to(cuda, dtype)
+    m.bias_from_ids = from_ids
+    batch = types.SimpleNamespace(
+        x=torch.from_numpy(rng.integers(1, 60, size=(b, S - 1, 1))).to(cuda), in_degree=torch.from_numpy(rng.integers(1, 60, size=(b, S - 1))).to(cuda),
+        out_degree=torch.from_numpy(rng.integers(1, 60, size=(b, S - 1))).to(cuda), attn_bias=torch.from_numpy(data["attn_bias"]).to(cuda, dtype),
+        spatial_pos=torch.from_numpy(data["spatial_pos"]).long().to(cuda),
+        attn_edge_type=torch.from_numpy(data["edge_type"]).long().unsqueeze(-1).contiguous().to(cuda), edge_input=None)
+    results = []
+    for fused in (False, True):
+        for layer in m.layers:
+            layer.one_operator = fused
+        out = m(batch)
+        named = list(m.named_parameters())
+        grads = torch.autograd.grad(out.float().sum(), [p_ for _, p_ in named], allow_unused=True)
+        results.append([("out", out.detach())] + [(n_, g_) for (n_, _), g_ in zip(named, grads) if g_ is not None])
+    assert len(results[0]) == len(results[1]) and len(results[0]) > 20
+    for (name, a), (_, r) in zip(*results):
+        if name.startswith("graph_node_feature.") or (name.startswith("graph_attn_bias.") and not from_ids):
+            # the node-feature and bias-builder backward kernels sum with floating-point atomics: equal to rounding from run to run
+            assert (a.double() - r.double()).abs().max().item() <= 1e-5 * max(r.double().abs().max().item(), 1e-30), name
+        else:
+            assert torch.equal(a, r), name

@@ -9,6 +9,8 @@
 //   torchgt::linear(x, weights[], biases?[]) -> Tensor[]                      (1 to 3 layers of one shape)
 //   torchgt::add_layer_norm(x, r?, gamma, beta, eps) -> (sum, y)
 //   torchgt::encoder_layer(x, residual?, params[16], plan holder, workspace, heads, eps1, eps2) -> (x + attention, ffn output)
+//   torchgt::dense_encoder_layer(x, residual?, params[16], extra[], attn_bias?, sp16?, et16?, heads, eps1, eps2, p_drop, seed,
+//                                bf16_products) -> (x + attention, ffn output)      the graph-level layer around the dense attention
 //   torchgt::add(x, r) -> sum
 //   torchgt::gelu(u) / torchgt::relu(u) -> h
 #include <torch/library.h>
@@ -615,6 +617,158 @@ std::tuple<Tensor, Tensor> encoder_layer(const Tensor& x, const c10::optional<Te
     return {r[0], r[1]};
 }
 
+// The same layer around the dense attention of the graph-level models (models/graphormer_graph_level.py:267-306).
+// x: [b, S, C].  extra: nothing, [bias [b, H, S, S]] (kind 1: its gradient is returned when it needs one), or
+// [spatial_table, edge_table, virtual_dist] (kind 2: the bias is formed in the kernels from ab / sp16 / et16, the
+// table gradients are returned).  Attention dropout runs inside the kernels from (p_drop, seed).
+struct DenseEncoderLayerFn : public torch::autograd::Function<DenseEncoderLayerFn> {
+    static variable_list forward(AutogradContext* ctx, Tensor x, c10::optional<Tensor> residual, at::TensorList P, at::TensorList extra,
+                                 c10::optional<Tensor> ab_o, c10::optional<Tensor> sp16_o, c10::optional<Tensor> et16_o, int64_t H,
+                                 double eps1, double eps2, double p_drop, int64_t seed, bool bf16_products) {
+        on_gpu(x, "dense_encoder_layer");
+        TORCH_CHECK(x.dim() == 3, "x must be [b, S, C]");
+        TORCH_CHECK(P.size() == 16, "dense_encoder_layer takes 16 parameter tensors");
+        TORCH_CHECK(extra.size() == 0 || extra.size() == 1 || extra.size() == 3, "extra: nothing, a bias tensor, or the three tables");
+        const int kind = extra.size() == 3 ? 2 : (int)extra.size();
+        const int64_t b = x.size(0), S = x.size(1), C = x.size(2);
+        TORCH_CHECK(C % H == 0, "hidden size ", C, " is not a multiple of ", H, " heads");
+        const int64_t d = C / H;
+        for (const Tensor& t : P) TORCH_CHECK(t.defined() && t.is_cuda() && t.scalar_type() == x.scalar_type(), "parameters must be GPU tensors of x's dtype");
+        for (const Tensor& t : extra) TORCH_CHECK(t.defined() && t.is_cuda() && t.scalar_type() == x.scalar_type(), "bias / tables must be GPU tensors of x's dtype");
+        int code = dtype_code(x);
+        if (code == TGT_DTYPE_F32 && bf16_products) code = TGT_DTYPE_F32_BF16_PRODUCTS;
+        TORCH_CHECK(kind != 2 || code != TGT_DTYPE_F32, "the bias from ids needs bf16 tensors or bf16_products");
+        std::vector<Tensor> p, ex;
+        for (const Tensor& t : P) p.push_back(t.contiguous());
+        for (const Tensor& t : extra) ex.push_back(t.contiguous());
+        Tensor ab, sp16, et16;
+        if (kind == 1) {
+            TORCH_CHECK(ex[0].dim() == 4 && ex[0].size(0) == b && ex[0].size(1) == H && ex[0].size(2) == S && ex[0].size(3) == S,
+                        "attn_bias must be [b, H, S, S]");
+        } else if (kind == 2) {
+            TORCH_CHECK(sp16_o.has_value() && et16_o.has_value(), "the id form needs sp16 and et16");
+            sp16 = *sp16_o; et16 = *et16_o;
+            TORCH_CHECK(sp16.scalar_type() == at::kShort && sp16.is_contiguous() && sp16.dim() == 3 && sp16.size(0) == b && sp16.size(1) == S &&
+                            sp16.size(2) == S, "sp16 must be a contiguous int16 [b, S, S]");
+            TORCH_CHECK(et16.scalar_type() == at::kShort && et16.is_contiguous() && et16.dim() == 4 && et16.size(0) == b && et16.size(1) == S &&
+                            et16.size(2) == S, "et16 must be a contiguous int16 [b, S, S, F]");
+            TORCH_CHECK(ex[0].dim() == 2 && ex[1].dim() == 2 && ex[0].size(1) == H && ex[1].size(1) == H && ex[2].numel() == H,
+                        "tables must be [rows, H] / [H]");
+            if (ab_o.has_value() && ab_o->defined()) {
+                TORCH_CHECK(ab_o->scalar_type() == x.scalar_type() && ab_o->dim() == 3 && ab_o->size(0) == b && ab_o->size(1) == S &&
+                                ab_o->size(2) == S, "attn_bias must be [b, S, S] of x's dtype");
+                ab = ab_o->contiguous();
+            }
+        }
+        c10::DeviceGuard guard(x.device());
+        Tensor x2 = x.reshape({-1, C}).contiguous(), r2;
+        if (residual.has_value() && residual->defined()) r2 = residual->reshape({-1, C}).contiguous();
+        Tensor s1, y1, mean1, rstd1, s2, y2, mean2, rstd2;
+        std::vector<Tensor> qkv, a, u, f;
+        layer::ln_fwd(x2, r2, p[0], p[1], eps1, s1, y1, mean1, rstd1);
+        layer::lin_fwd(y1, {&p[2], &p[4], &p[6]}, {&p[3], &p[5], &p[7]}, qkv);
+        Tensor o = at::empty_like(qkv[0]), lse = at::empty({b, H, S}, x.options().dtype(at::kFloat));
+        if (kind == 2) {
+            Tensor vd = ex[2].reshape({-1});
+            check(tgt_dense_attn_ids_fwd(qkv[0].data_ptr(), qkv[1].data_ptr(), qkv[2].data_ptr(), ab.defined() ? ab.data_ptr() : nullptr,
+                                         reinterpret_cast<const uint16_t*>(sp16.data_ptr()), reinterpret_cast<const uint16_t*>(et16.data_ptr()),
+                                         (int)et16.size(3), ex[0].data_ptr(), (int)ex[0].size(0), ex[1].data_ptr(), (int)ex[1].size(0),
+                                         vd.data_ptr(), (int)b, (int)S, (int)H, (int)d, code, (float)p_drop, (uint64_t)seed, o.data_ptr(),
+                                         lse.data_ptr<float>(), stream_of(x)),
+                  "tgt_dense_attn_ids_fwd");
+        } else {
+            check(tgt_dense_attn_dropout_fwd(qkv[0].data_ptr(), qkv[1].data_ptr(), qkv[2].data_ptr(), kind == 1 ? ex[0].data_ptr() : nullptr, (int)b,
+                                             (int)S, (int)H, (int)d, code, (float)p_drop, (uint64_t)seed, o.data_ptr(), lse.data_ptr<float>(),
+                                             stream_of(x)),
+                  "tgt_dense_attn_dropout_fwd");
+        }
+        layer::lin_fwd(o, {&p[8]}, {&p[9]}, a);
+        layer::ln_fwd(s1, a[0], p[10], p[11], eps2, s2, y2, mean2, rstd2);
+        layer::lin_fwd(y2, {&p[12]}, {&p[13]}, u);
+        Tensor h = at::empty_like(u[0]);
+        check(tgt_gelu_fwd(u[0].data_ptr(), u[0].numel(), dtype_code(x), h.data_ptr(), stream_of(x)), "tgt_gelu_fwd");
+        layer::lin_fwd(h, {&p[14]}, {&p[15]}, f);
+        std::vector<Tensor> save{s1, mean1, rstd1, y1, qkv[0], qkv[1], qkv[2], o, lse, s2, mean2, rstd2, y2, u[0], h, ab, sp16, et16};
+        save.insert(save.end(), p.begin(), p.end());
+        save.insert(save.end(), ex.begin(), ex.end());
+        ctx->save_for_backward(save);
+        ctx->saved_data["kind"] = (int64_t)kind;
+        ctx->saved_data["H"] = H;
+        ctx->saved_data["code"] = (int64_t)code;
+        ctx->saved_data["p"] = p_drop;
+        ctx->saved_data["seed"] = seed;
+        ctx->saved_data["has_r"] = r2.defined();
+        ctx->saved_data["bias_grad"] = kind == 1 && extra[0].requires_grad();
+        ctx->saved_data["vd_shape"] = kind == 2 ? extra[2].sizes().vec() : std::vector<int64_t>{};
+        ctx->set_materialize_grads(false);
+        return {s2.view(x.sizes()), f[0].view(x.sizes())};
+    }
+    static variable_list backward(AutogradContext* ctx, variable_list grads) {
+        auto sv = ctx->get_saved_variables();
+        const Tensor &s1 = sv[0], &mean1 = sv[1], &rstd1 = sv[2], &y1 = sv[3], &q = sv[4], &k = sv[5], &v = sv[6], &o = sv[7], &lse = sv[8],
+                     &s2 = sv[9], &mean2 = sv[10], &rstd2 = sv[11], &y2 = sv[12], &u = sv[13], &h = sv[14], &ab = sv[15], &sp16 = sv[16],
+                     &et16 = sv[17];
+        const Tensor* p = sv.data() + 18;
+        const Tensor* ex = sv.data() + 34;
+        const int kind = (int)ctx->saved_data["kind"].toInt(), code = (int)ctx->saved_data["code"].toInt();
+        const int64_t H = ctx->saved_data["H"].toInt(), b = lse.size(0), S = lse.size(2), N = s1.size(0), C = s1.size(1), d = C / H;
+        const float p_drop = (float)ctx->saved_data["p"].toDouble();
+        const uint64_t seed = (uint64_t)ctx->saved_data["seed"].toInt();
+        c10::DeviceGuard guard(s1.device());
+        Tensor d_s2, d_f;
+        if (grads[0].defined()) d_s2 = grads[0].reshape({N, C}).contiguous();
+        d_f = grads[1].defined() ? grads[1].reshape({N, C}).contiguous() : at::zeros_like(s1);
+        Tensor dh, du, dy2, ds2, do_, dy1, dx, dg2, dbn2, dg1, dbn1;
+        std::vector<Tensor> dW2, db2, dW1, db1, dWo, dbo, dWqkv, dbqkv;
+        layer::lin_bwd(h, {&p[14]}, {&d_f}, dh, dW2, db2);
+        du = at::empty_like(u);
+        check(tgt_gelu_bwd(u.data_ptr(), dh.data_ptr(), u.numel(), dtype_code(s1), du.data_ptr(), stream_of(u)), "tgt_gelu_bwd");
+        layer::lin_bwd(y2, {&p[12]}, {&du}, dy2, dW1, db1);
+        layer::ln_bwd(s2, p[10], mean2, rstd2, dy2, d_s2, ds2, dg2, dbn2);
+        layer::lin_bwd(o, {&p[8]}, {&ds2}, do_, dWo, dbo);
+        Tensor dq = at::empty_like(q), dk = at::empty_like(k), dv = at::empty_like(v);
+        variable_list dextra;
+        if (kind == 2) {
+            Tensor dst = at::empty_like(ex[0]), det = at::empty_like(ex[1]), vd = ex[2].reshape({-1}), dvd = at::empty_like(vd);
+            const int64_t ws_bytes = tgt_dense_attn_ids_bwd_workspace_bytes((int)b, (int)H, (int)ex[0].size(0), (int)ex[1].size(0));
+            Tensor ws = at::empty({ws_bytes}, s1.options().dtype(at::kByte));
+            check(tgt_dense_attn_ids_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), ab.defined() ? ab.data_ptr() : nullptr,
+                                         reinterpret_cast<const uint16_t*>(sp16.data_ptr()), reinterpret_cast<const uint16_t*>(et16.data_ptr()),
+                                         (int)et16.size(3), ex[0].data_ptr(), (int)ex[0].size(0), ex[1].data_ptr(), (int)ex[1].size(0),
+                                         vd.data_ptr(), (int)b, (int)S, (int)H, (int)d, code, p_drop, seed, o.data_ptr(), lse.data_ptr<float>(),
+                                         do_.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dst.data_ptr(), det.data_ptr(),
+                                         dvd.data_ptr(), ws.data_ptr(), ws_bytes, stream_of(q)),
+                  "tgt_dense_attn_ids_bwd");
+            dextra = {dst, det, dvd.view(ctx->saved_data["vd_shape"].toIntVector())};
+        } else {
+            Tensor dbias;
+            if (kind == 1 && ctx->saved_data["bias_grad"].toBool()) dbias = at::empty_like(ex[0]);
+            check(tgt_dense_attn_dropout_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), kind == 1 ? ex[0].data_ptr() : nullptr, (int)b, (int)S,
+                                             (int)H, (int)d, code, p_drop, seed, o.data_ptr(), lse.data_ptr<float>(), do_.data_ptr(),
+                                             dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dbias.defined() ? dbias.data_ptr() : nullptr,
+                                             stream_of(q)),
+                  "tgt_dense_attn_dropout_bwd");
+            if (kind == 1) dextra = {dbias};
+        }
+        layer::lin_bwd(y1, {&p[2], &p[4], &p[6]}, {&dq, &dk, &dv}, dy1, dWqkv, dbqkv);
+        layer::ln_bwd(s1, p[0], mean1, rstd1, dy1, ds2, dx, dg1, dbn1);
+        Tensor dxv = dx.view({b, S, C});
+        variable_list out{dxv, ctx->saved_data["has_r"].toBool() ? dxv : Tensor(),
+                          dg1, dbn1, dWqkv[0], dbqkv[0], dWqkv[1], dbqkv[1], dWqkv[2], dbqkv[2], dWo[0], dbo[0], dg2, dbn2, dW1[0], db1[0],
+                          dW2[0], db2[0]};
+        out.insert(out.end(), dextra.begin(), dextra.end());
+        for (int i = 0; i < 9; ++i) out.push_back(Tensor());      // ab, sp16, et16, H, eps1, eps2, p_drop, seed, bf16_products
+        return out;
+    }
+};
+std::tuple<Tensor, Tensor> dense_encoder_layer(const Tensor& x, const c10::optional<Tensor>& residual, at::TensorList params,
+                                               at::TensorList extra, const c10::optional<Tensor>& ab, const c10::optional<Tensor>& sp16,
+                                               const c10::optional<Tensor>& et16, int64_t H, double eps1, double eps2, double p_drop,
+                                               int64_t seed, bool bf16_products) {
+    auto r = DenseEncoderLayerFn::apply(x, residual, params, extra, ab, sp16, et16, H, eps1, eps2, p_drop, seed, bf16_products);
+    return {r[0], r[1]};
+}
+
 }  // namespace
 
 TORCH_LIBRARY(torchgt, m) {
@@ -629,6 +783,8 @@ TORCH_LIBRARY(torchgt, m) {
     m.def("add_layer_norm(Tensor x, Tensor? r, Tensor gamma, Tensor beta, float eps) -> (Tensor, Tensor)");
     m.def("encoder_layer(Tensor x, Tensor? residual, Tensor[] params, __torch__.torch.classes.torchgt.PlanHolder plan, Tensor workspace, "
           "int num_heads, float eps1, float eps2) -> (Tensor, Tensor)");
+    m.def("dense_encoder_layer(Tensor x, Tensor? residual, Tensor[] params, Tensor[] extra, Tensor? attn_bias, Tensor? sp16, Tensor? et16, "
+          "int num_heads, float eps1, float eps2, float p_drop, int seed, bool bf16_products) -> (Tensor, Tensor)");
     m.def("add(Tensor x, Tensor r) -> Tensor");
     m.def("gelu(Tensor u) -> Tensor");
     m.def("relu(Tensor u) -> Tensor");
@@ -644,6 +800,7 @@ TORCH_LIBRARY_IMPL(torchgt, CompositeImplicitAutograd, m) {
     m.impl("linear", linear);
     m.impl("add_layer_norm", add_layer_norm);
     m.impl("encoder_layer", encoder_layer);
+    m.impl("dense_encoder_layer", dense_encoder_layer);
     m.impl("add", add);
     m.impl("gelu", gelu);
     m.impl("relu", relu);

@@ -9,7 +9,8 @@ per step and is shared by all layers, the input rows from one gather kernel.
 import torch
 import torch.nn as nn
 
-from . import _lib
+from . import _ext, _lib
+from .core_attention import GraphBiasIds
 from .encoder import AddFunction, AddLayerNormFunction, FeedForwardNetwork, init_params
 from .graph_bias import GraphAttnBias
 from .multi_head_attention import MultiHeadAttention, fused_linear
@@ -96,10 +97,58 @@ class EncoderLayer(nn.Module):
         self.ffn = FeedForwardNetwork(hidden_size, ffn_size, dropout_rate)
         self.ffn_dropout = nn.Dropout(dropout_rate)
 
+    one_operator = True      # False: always run the layer operator by operator
+
+    def _one_operator(self, x, attn_bias):
+        """``(extra, attn_bias[b,S,S], sp16, et16)`` for ``torch.ops.torchgt.dense_encoder_layer`` when it covers this call
+        (no torch dropout at work, widths the kernels read without padding, a bias it can take as it is), else None."""
+        if not self.one_operator or not x.is_cuda or x.dim() != 3 or x.dtype not in (torch.float32, torch.bfloat16):
+            return None
+        if self.training and (self.self_attention_dropout.p > 0 or self.ffn_dropout.p > 0):
+            return None
+        att = self.self_attention
+        core = att.dist_attn.local_attn
+        ve = 4 if x.dtype == torch.float32 else 8
+        if att.output_layer is None or any(w % ve for w in (x.shape[-1], self.ffn.layer1.out_features)) or \
+                att.num_heads * att.att_size != x.shape[-1]:
+            return None
+        b, S, H = x.shape[0], x.shape[1], att.num_heads
+        if attn_bias is None:
+            return [], None, None, None
+        if isinstance(attn_bias, GraphBiasIds):
+            ids = attn_bias
+            if ids.fits and (x.dtype == torch.bfloat16 or core.dense_bf16_products) and all(
+                    t.dtype == x.dtype for t in (ids.spatial_table, ids.edge_table, ids.virtual_dist)):
+                ab = None if ids.attn_bias is None else ids.attn_bias.to(x.dtype)
+                return [ids.spatial_table, ids.edge_table, ids.virtual_dist], ab, ids.sp16, ids.et16
+            attn_bias = ids.materialize()
+        if isinstance(attn_bias, torch.Tensor) and tuple(attn_bias.shape) == (b, H, S, S) and attn_bias.dtype == x.dtype:
+            return [attn_bias], None, None, None
+        return None
+
     def forward(self, x, attn_bias=None, mask=None, residual=None, defer_residual=False):
         if mask is not None:
             raise NotImplementedError("the reference never passes `mask` (graphormer_graph_level.py:380)")
         n1, n2 = self.self_attention_norm, self.ffn_norm
+        fused = self._one_operator(x, attn_bias)
+        if fused is not None:
+            # the whole layer as one operator and one autograd node (same kernels, same order, same numbers)
+            extra, ab, sp16, et16 = fused
+            att = self.self_attention
+            core = att.dist_attn.local_attn
+            p = float(core.attention_dropout_rate) if self.training else 0.0
+            seed = int(torch.randint(0, 2 ** 62, (1,)).item()) if p > 0 else 0
+            params = [n1.weight, n1.bias, att.linear_q.weight, att.linear_q.bias, att.linear_k.weight, att.linear_k.bias,
+                      att.linear_v.weight, att.linear_v.bias, att.output_layer.weight, att.output_layer.bias, n2.weight, n2.bias,
+                      self.ffn.layer1.weight, self.ffn.layer1.bias, self.ffn.layer2.weight, self.ffn.layer2.bias]
+            try:
+                x2, y = _ext.ops().dense_encoder_layer(x, residual, params, extra, ab, sp16, et16, att.num_heads, n1.eps, n2.eps, p,
+                                                       seed, bool(core.dense_bf16_products))
+                return (x2, y) if defer_residual else AddFunction.apply(x2, y)
+            except RuntimeError as exc:
+                if sp16 is None or "bytes of LDS" not in str(exc):
+                    raise
+                attn_bias.fits = False       # this shape needs the bias tensor: the attention below builds it once
         x, y = AddLayerNormFunction.apply(x, residual, n1.weight, n1.bias, n1.eps)
         y = self.self_attention(y, attn_bias, None, attn_type="full")
         y = self.self_attention_dropout(y)
@@ -137,8 +186,11 @@ class Graphormer(nn.Module):
             self.downstream_out_proj = nn.Linear(hidden_dim, output_dim)
         self.apply(lambda module: init_params(module, n_layers=n_layers))
         # True: the layers get the bias as ids + tables and the bf16 attention kernels form it on chip (the [b, H, S, S]
-        # tensor is built only for layers that cannot: float32 arithmetic, the multi-hop branch, very long sequences)
-        self.bias_from_ids = True
+        # tensor is built only for layers that cannot: float32 arithmetic, the multi-hop branch, very long sequences).
+        # It saves the bias tensor and one bias-gradient tensor per layer (68 MB each for 256 graphs of 129 nodes in bf16)
+        # and costs GPU time: every attention launch rebuilds the bias of its (graph, head) pairs and every backward runs
+        # the id histogram the tensor form runs once per step (1.85 against 2.30 ms per training step on that batch).
+        self.bias_from_ids = False
 
     def forward(self, batched_data, perturb=None):
         x = self.graph_node_feature(batched_data)            # [b, s + 1, h]
