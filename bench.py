@@ -586,7 +586,8 @@ def bench_model(args):
     40 classes; 111 913 parameters) on the whole 64 K-node graph as one sequence: forward, nll loss, backward,
     AdamW step (torch's optimizer, as in the reference's training loop)."""
     import torch
-    from torchgt_amd import GT, Graphormer as NodeGraphormer, _lib
+    from torchgt_amd import GT, Graphormer as NodeGraphormer, _lib, nll_loss as lib_nll_loss
+    nll_loss = torch.nn.functional.nll_loss if args.torch_loss else lib_nll_loss
     dev = torch.device("cuda:0")
     e, n, label, desc = build_workload("config2")
     tdt = torch.bfloat16 if args.dtype == "bf16" else torch.float32
@@ -596,7 +597,7 @@ def bench_model(args):
     n_rows = n if gt else n - 1
     torch.manual_seed(42)
     m = Graphormer(4, 8, 128, 64, 40, 1, 0.0, 0.0, 0.0, 64, 1).to(dev, tdt)
-    opt = torch.optim.AdamW(m.parameters(), lr=1e-3, weight_decay=0.01)
+    opt = torch.optim.AdamW(m.parameters(), lr=1e-3, weight_decay=0.01, fused=not args.foreach_adamw)
     ei = torch.from_numpy(e).to(dev)
     x = torch.randn(n_rows, 128, device=dev).to(tdt)
     y = torch.randint(0, 40, (n_rows,), device=dev)
@@ -604,7 +605,7 @@ def bench_model(args):
     def step():
         opt.zero_grad(set_to_none=True)
         out = m(x, None, ei, attn_type="sparse")
-        loss = torch.nn.functional.nll_loss(out.float(), y)
+        loss = nll_loss(out.float(), y)
         loss.backward()
         opt.step()
         return loss
@@ -638,7 +639,7 @@ def bench_model(args):
         gopt = torch.optim.AdamW(gm.parameters(), lr=1e-3, weight_decay=0.01, capturable=True)
 
         def gstep():
-            gloss = torch.nn.functional.nll_loss(gm(x, None, ei, attn_type="sparse").float(), y)
+            gloss = nll_loss(gm(x, None, ei, attn_type="sparse").float(), y)
             gloss.backward()
             gopt.step()
             return gloss
@@ -664,7 +665,7 @@ def bench_model(args):
         torch.cuda.synchronize()
         graph_ms = (time.perf_counter() - t0) / args.steps * 1e3
     groups = {"attention": ("attn_fwd", "bwd_node_side", "attn_bwd"), "projections and ffn linears": ("linear_fwd", "linear_dx", "linear_dw"),
-              "layer norm + residual": ("layer_norm_fwd", "layer_norm_bwd"), "gelu": ("gelu",)}
+              "layer norm + residual": ("layer_norm_fwd", "layer_norm_bwd"), "gelu": ("gelu",), "nll loss": ("nll_loss",)}
     result = {
         "metric": "training step of the 4-layer " + ("GT" if gt else "Graphormer-Slim") + " on one 64 K-node sequence",
         "value": 1e3 / ms, "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -674,7 +675,8 @@ def bench_model(args):
                                "Graphormer-Slim 4 x (hidden 64, ffn 64, 8 heads), ") +
                                "128-d features, 40 classes, no bias, dropout 0", "N": n, "E": int(e.shape[1]),
                    "parameters": sum(p.numel() for p in m.parameters()),
-                   "step": "forward + nll_loss + backward + torch AdamW", "parallelism": "1 GPU"},
+                   "step": "forward + nll_loss (" + ("torch's" if args.torch_loss else "the library's") + ") + backward + torch AdamW (" + ("foreach" if args.foreach_adamw else "fused") + ")",
+                   "parallelism": "1 GPU"},
         "loss": loss_value,
         "ms_per_step_hip_graph": graph_ms,
         "library_kernel_us_per_step": lib_us,
@@ -714,7 +716,7 @@ def bench_graph_model(args):
     torch.manual_seed(42)
     m = Graphormer(4, 8, 64, 0.0, 0.0, 64, "ZINC", "single_hop", 5, 0.0, 1).to(dev, tdt)
     m.bias_from_ids = bool(args.bias_from_ids)
-    opt = torch.optim.AdamW(m.parameters(), lr=1e-3, weight_decay=0.01)
+    opt = torch.optim.AdamW(m.parameters(), lr=1e-3, weight_decay=0.01, fused=not args.foreach_adamw)
     y = torch.randn(b, device=dev)
 
     def step():
@@ -792,7 +794,7 @@ def bench_graph_model(args):
         "config": {"workload": "configs[3] batch (256 ER graphs n~U[16,128] p=0.1 padded to 128 + virtual node), graph-level "
                                "Graphormer 4 x (hidden 64, ffn 64, 8 heads), ZINC tables, dropout 0", "b": b, "S": s + 1,
                    "parameters": sum(p.numel() for p in m.parameters()),
-                   "step": "forward + l1_loss + backward + torch AdamW", "parallelism": "1 GPU"},
+                   "step": "forward + l1_loss + backward + torch AdamW (" + ("foreach" if args.foreach_adamw else "fused") + ")", "parallelism": "1 GPU"},
         "loss": loss_value,
         "ms_per_step_hip_graph": graph_ms,
         "library_kernel_us_per_step": lib_us,
@@ -1029,6 +1031,11 @@ def main():
                     help="config2 / f32 only: skip the other benchmark configurations (they are timed in the default run)")
     ap.add_argument("--bias-from-ids", action="store_true",
                     help="config4-model: the attention kernels form the bias from ids and tables instead of reading a [b,H,S,S] tensor")
+    ap.add_argument("--foreach-adamw", action="store_true",
+                    help="model workloads: torch.optim.AdamW's default multi-tensor implementation instead of fused=True "
+                         "(the same update from one kernel; the default one issues a dozen launches per step from Python)")
+    ap.add_argument("--torch-loss", action="store_true",
+                    help="config2-model / config2-gt-model: torch's F.nll_loss instead of the library's kernel")
     ap.add_argument("--hip-graph", action="store_true",
                     help="config2-model: also time the step captured into a HIP graph and replayed")
     ap.add_argument("--calibration-copy", action="store_true",

@@ -355,6 +355,41 @@ int tgt_linear_fwd(const void* d_x, const void* const* d_W, const void* const* d
  * the same bits).  d_workspace: tgt_linear_bwd_workspace_bytes(...) bytes,
  * 16-byte aligned, needed when d_dW is given; contents need no initialisation. */
 int64_t tgt_linear_bwd_workspace_bytes(int n_out, int in_features, int out_features);
+/* A sum over per-workgroup partials that a *_deferred call leaves to its caller: element e of the result is the sum
+ * over w of partial[w * n + e], added in a fixed order, and goes to out[i] + (e - begin[i]) for the last i with
+ * begin[i] <= e (an out[i] of NULL: not wanted).  The caller only carries descriptors from a *_deferred call to
+ * tgt_reduce_partials; the workspace the call was given must live until that launch has run. */
+typedef struct {
+    const float* partial;
+    int32_t workers, n, n_out;
+    void* out[6];
+    int32_t begin[6];
+} tgt_reduce_desc;
+/* Up to eight such sums in one launch (a layer's backward has six: four linears, two LayerNorms, each a few
+ * microseconds of launch latency on its own).  The result of a sum does not depend on what else is in the launch:
+ * tgt_linear_bwd is tgt_linear_bwd_deferred followed by tgt_reduce_partials of its one descriptor.  dtype: of the
+ * outputs.  No counterpart in the reference (autograd of nn.Linear / nn.LayerNorm reduces inside its own kernels). */
+int tgt_reduce_partials(const tgt_reduce_desc* descs, int count, int dtype, void* stream);
+/* tgt_linear_bwd without its last step: dx is complete on return (in stream order), the weight and bias gradients
+ * are the sum `desc` describes.  d_dW must be given. */
+int tgt_linear_bwd_deferred(const void* d_x, const void* const* d_W, const void* const* d_dy, int n_out, int64_t N,
+                            int in_features, int out_features, int dtype, void* d_dx, void* const* d_dW, void* const* d_db,
+                            void* d_workspace, int64_t workspace_bytes, void* stream, tgt_reduce_desc* desc);
+/* FeedForwardNetwork's first layer with its activation (models/graphormer_dist_node_level.py:36-37:
+ * x = self.layer1(x); x = self.gelu(x)) in one pass: u = x W^T + b goes to d_u and act(u) to d_h, both [N, out_features].
+ * act: TGT_ACT_GELU (exact erf form, as tgt_gelu_fwd) or TGT_ACT_RELU.  The same bits as tgt_linear_fwd followed by
+ * tgt_gelu_fwd / tgt_relu_fwd (which is what runs for shapes whose kernel has no such epilogue: only 64 -> 64 has). */
+#define TGT_ACT_GELU 1
+#define TGT_ACT_RELU 2
+int tgt_linear_act_fwd(const void* d_x, const void* d_W, const void* d_b, int64_t N, int in_features, int out_features, int dtype,
+                       int act, void* d_u, void* d_h, void* stream);
+/* Backward of the layer that follows such an activation (FeedForwardNetwork.layer2, :38): its input was h = act(u)
+ * [N, in_features].  d_du = (dy W) * act'(u), the gradient of u, instead of the gradient of h; d_dW = dy^T h and
+ * d_db (may be NULL) as in tgt_linear_bwd.  The same bits as tgt_linear_bwd followed by tgt_gelu_bwd / tgt_relu_bwd.
+ * desc: NULL, or a descriptor to fill instead of summing the weight-gradient partials (see tgt_reduce_partials). */
+int tgt_linear_act_bwd(const void* d_h, const void* d_W, const void* d_dy, const void* d_u, int64_t N, int in_features,
+                       int out_features, int dtype, int act, void* d_du, void* d_dW, void* d_db, void* d_workspace,
+                       int64_t workspace_bytes, void* stream, tgt_reduce_desc* desc);
 int tgt_linear_bwd(const void* d_x, const void* const* d_W, const void* const* d_dy, int n_out, int64_t N,
                    int in_features, int out_features, int dtype, void* d_dx, void* const* d_dW, void* const* d_db,
                    void* d_workspace, int64_t workspace_bytes, void* stream);
@@ -378,9 +413,13 @@ int tgt_add_layer_norm_fwd(const void* d_x, const void* d_r, const void* d_gamma
  * The column sums are formed per workgroup and added in a fixed order.
  * d_workspace: tgt_layer_norm_bwd_workspace_bytes(C) bytes, 16-byte aligned. */
 int64_t tgt_layer_norm_bwd_workspace_bytes(int C);
+/* (tgt_layer_norm_bwd_deferred: the same with dgamma and dbeta left as the sum `desc` describes, see tgt_reduce_partials) */
 int tgt_layer_norm_bwd(const void* d_s, const void* d_gamma, const float* d_mean, const float* d_rstd, const void* d_dy,
                        const void* d_ds_extra, int64_t N, int C, int dtype, void* d_ds, void* d_dgamma, void* d_dbeta,
                        void* d_workspace, int64_t workspace_bytes, void* stream);
+int tgt_layer_norm_bwd_deferred(const void* d_s, const void* d_gamma, const float* d_mean, const float* d_rstd, const void* d_dy,
+                       const void* d_ds_extra, int64_t N, int C, int dtype, void* d_ds, void* d_dgamma, void* d_dbeta,
+                       void* d_workspace, int64_t workspace_bytes, void* stream, tgt_reduce_desc* desc);
 /* nn.GELU() of FeedForwardNetwork (models/graphormer_dist_node_level.py:32,37), exact
  * erf form, on n elements (n a multiple of 4 for fp32, 8 for bf16):
  * h = 0.5 u (1 + erf(u / sqrt 2));  backward: du = dh * dh/du evaluated at u. */
@@ -391,6 +430,20 @@ int tgt_gelu_bwd(const void* d_u, const void* d_dh, int64_t n, int dtype, void* 
  * time is booked under the gelu slot of the per-kernel timing. */
 int tgt_relu_fwd(const void* d_u, int64_t n, int dtype, void* d_h, void* stream);
 int tgt_relu_bwd(const void* d_u, const void* d_dh, int64_t n, int dtype, void* d_du, void* stream);
+/* F.nll_loss(log_probs, target) of the node-level training and evaluation loops (main_sp_sparse_node_level.py:200,
+ * gt_sp/evaluate.py:52,77): reduction 'mean', no class weights.  log_probs [N, C] (float32 or bf16), target [N]
+ * int64:  loss = - sum_i log_probs[i, target_i] / count over the rows with target_i != ignore_index (torch's default
+ * is -100), count = their number (0 rows: nan, like torch).  A target outside [0, C) other than ignore_index counts
+ * as ignored (torch raises a device-side assertion there).  d_loss: one element of dtype; d_count: one float, kept
+ * for the backward.  The sum is formed per workgroup and then in a fixed order: the same inputs give the same bits.
+ * d_workspace: tgt_nll_loss_workspace_bytes(N) bytes, 4-byte aligned.
+ * Backward: d_dlog_probs[i, c] = - dloss / count where c == target_i (and the row counts), else 0; d_dloss is one
+ * element of dtype on the device. */
+int64_t tgt_nll_loss_workspace_bytes(int64_t N);
+int tgt_nll_loss_fwd(const void* d_log_probs, const int64_t* d_target, int64_t N, int C, int dtype, int64_t ignore_index, void* d_loss,
+                     float* d_count, void* d_workspace, int64_t workspace_bytes, void* stream);
+int tgt_nll_loss_bwd(const int64_t* d_target, const void* d_dloss, const float* d_count, int64_t N, int C, int dtype, int64_t ignore_index,
+                     void* d_dlog_probs, void* stream);
 
 /* ---- graph-level attention bias ---------------------------------------------
  * GraphAttnBias.forward (models/graphormer_graph_level.py:94-156), edge_type other than

@@ -46,6 +46,8 @@ graph-level graphormer_forward torch's layer_norm / linear / gelu / softmax
 gt_forward (node-level GT)     torch's layer_norm / linear / relu / softmax on a
                                complete graph; closed form without layers;
                                commutes with node relabelling
+nll_loss                       torch's CPU F.nll_loss (library routine); log C
+                               for a uniform prediction
 metis partition labels         PARITY UNPINNED: dgl/METIS is absent; partition
                                ids are always an explicit input here
 =============================  ================================================

@@ -13,10 +13,13 @@ Restates, in plain numpy on top of ``oracle.projections`` and
   token row 0, the layers, final LayerNorm, output projection of rows 1.., and
   ``log_softmax``.
 
+* ``F.nll_loss`` of the training loop (main_sp_sparse_node_level.py:200), reduction 'mean' with ``ignore_index``.
+
 Pinned in ``tests/test_oracle_encoder.py`` against ``torch.nn.functional.layer_norm``
 and ``gelu`` (independent library routines), closed forms (constant rows, the GELU
 reflection identity ``gelu(x) - gelu(-x) = x``, a layer with zero attention/FFN
-output weights is the identity) and the parameter counts of README.md:70,114.
+output weights is the identity) and the parameter counts of README.md:70,114; ``nll_loss`` against torch's CPU
+``F.nll_loss`` and the closed form log C of a uniform prediction.
 """
 import math
 
@@ -71,3 +74,17 @@ def graphormer_forward(x, params, edge_index, n_layers, num_heads):
     out = _proj.linear_forward(h[0, 1:, :], params["downstream_out_proj.weight"], params["downstream_out_proj.bias"])
     out = out - out.max(axis=1, keepdims=True)
     return out - np.log(np.exp(out).sum(axis=1, keepdims=True))                                      # log_softmax
+
+
+def nll_loss(log_probs, target, ignore_index=-100):
+    """``F.nll_loss(log_probs, target)`` (main_sp_sparse_node_level.py:200): minus the mean, over the rows whose
+    target is not ``ignore_index``, of the log-probability of the target class.  Returns (loss, d loss / d log_probs)."""
+    lp = np.asarray(log_probs, np.float64)
+    t = np.asarray(target, np.int64)
+    rows = np.nonzero(t != ignore_index)[0]
+    grad = np.zeros_like(lp)
+    if rows.size == 0:
+        return float("nan"), grad
+    loss = -lp[rows, t[rows]].sum() / rows.size
+    grad[rows, t[rows]] = -1.0 / rows.size
+    return float(loss), grad

@@ -12,7 +12,7 @@ import torch
 from oracle import encoder_layer as E
 from oracle import graph_prep as ogp
 from oracle import sparse_attention as osa
-from torchgt_amd import EncoderLayer, Graphormer, _lib, workloads
+from torchgt_amd import EncoderLayer, Graphormer, _lib, nll_loss, workloads
 from torchgt_amd.encoder import AddFunction, AddLayerNormFunction, GeluFunction
 
 pytestmark = pytest.mark.gpu
@@ -89,6 +89,47 @@ def _ref_layer(p, x, ei, H, prefix=""):
     x1 = x + lin(o.reshape(b, S, hidden), g("self_attention.output_layer.weight"), g("self_attention.output_layer.bias"))
     y = F.layer_norm(x1, (hidden,), g("ffn_norm.weight"), g("ffn_norm.bias"))
     return x1 + lin(F.gelu(lin(y, g("ffn.layer1.weight"), g("ffn.layer1.bias"))), g("ffn.layer2.weight"), g("ffn.layer2.bias"))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("N,C", [(64000, 40), (1000, 47), (5, 3), (1, 1)])
+def test_nll_loss_matches_oracle(cuda, dtype, N, C):
+    """loss and its gradient against the oracle; float32 1e-6 (one fp32 sum of N terms in a tree), bf16: the loss is
+    rounded to bf16 once (4e-3), the gradient likewise."""
+    print(f"nll_loss case: N={N} C={C} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(N + C)
+    lp = torch.log_softmax(torch.randn(N, C, generator=g), 1).to(dtype)
+    t = torch.randint(0, C, (N,), generator=g)
+    if N > 3:
+        t[torch.randperm(N, generator=g)[: N // 10]] = -100
+    want, want_grad = E.nll_loss(lp.double().numpy(), t.numpy())
+    x = lp.to(cuda).requires_grad_(True)
+    loss = nll_loss(x, t.to(cuda))
+    assert loss.dtype == dtype and loss.dim() == 0
+    (gx,) = torch.autograd.grad(loss, x, torch.tensor(2.0, dtype=dtype, device=cuda))
+    tol = 1e-6 if dtype == torch.float32 else 4e-3
+    assert abs(loss.item() - want) <= tol * abs(want)
+    assert np.abs(gx.double().cpu().numpy() - 2.0 * want_grad).max() <= tol * np.abs(2.0 * want_grad).max()
+    assert ((gx != 0).sum(1) <= 1).all()
+    # the same bits from call to call, and another ignore_index
+    assert torch.equal(loss, nll_loss(x, t.to(cuda)))
+    if N > 3:
+        t2 = torch.where(t == -100, torch.tensor(1 % C), t)
+        want2, _ = E.nll_loss(lp.double().numpy(), t2.numpy(), ignore_index=0)
+        got2 = nll_loss(x, t2.to(cuda), ignore_index=0).item()
+        assert abs(got2 - want2) <= tol * abs(want2)
+
+
+def test_nll_loss_edge_cases(cuda):
+    x = torch.log_softmax(torch.randn(6, 4), 1).to(cuda).requires_grad_(True)
+    every_row_ignored = nll_loss(x, torch.full((6,), -100, device=cuda))
+    assert torch.isnan(every_row_ignored)                      # 0 / 0 like torch
+    empty = nll_loss(torch.zeros(0, 4, device=cuda), torch.zeros(0, dtype=torch.int64, device=cuda))
+    assert torch.isnan(empty)
+    with pytest.raises(RuntimeError):
+        nll_loss(torch.zeros(4, 3), torch.zeros(4, dtype=torch.int64))              # CPU tensors: no fallback
+    with pytest.raises(RuntimeError):
+        nll_loss(x, torch.zeros(6, dtype=torch.int32, device=cuda))
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

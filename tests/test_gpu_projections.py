@@ -79,6 +79,114 @@ def test_linear_weight_gradient_is_reproducible(cuda):
         assert torch.equal(ga, gb)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_deferred_sums_in_one_launch_equal_the_plain_entry_points(cuda, dtype):
+    """tgt_linear_bwd_deferred (two projections, one of them the 64-wide one-pass form) and tgt_layer_norm_bwd_deferred
+    followed by ONE tgt_reduce_partials give the bits of tgt_linear_bwd / tgt_layer_norm_bwd."""
+    L = _lib.lib()
+    code = 0 if dtype == torch.float32 else 1
+    g = torch.Generator().manual_seed(21)
+    vp3 = ctypes.c_void_p * 3
+    descs = (_lib.ReduceDesc * 3)()
+    keep, pairs = [], []
+
+    def linear(idx, N, in_f, out_f, n):
+        print(f"deferred linear: N={N} in={in_f} out={out_f} n={n} {dtype}", flush=True)
+        x = torch.randn(N, in_f, generator=g).to(dtype).to(cuda)
+        Ws = [torch.randn(out_f, in_f, generator=g).to(dtype).to(cuda) for _ in range(n)]
+        dys = [torch.randn(N, out_f, generator=g).to(dtype).to(cuda) for _ in range(n)]
+        nbytes = L.tgt_linear_bwd_workspace_bytes(n, in_f, out_f)
+        outs = []
+        for deferred in (False, True):
+            dx = torch.empty_like(x)
+            dW = [torch.full_like(W, 7.0) for W in Ws]
+            db = [torch.full((out_f,), 7.0, dtype=dtype, device=cuda) for _ in range(n)]
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=cuda)
+            a = (x.data_ptr(), vp3(*[W.data_ptr() for W in Ws]), vp3(*[d.data_ptr() for d in dys]), n, N, in_f, out_f, code,
+                 dx.data_ptr(), vp3(*[t.data_ptr() for t in dW]), vp3(*[t.data_ptr() for t in db]), ws.data_ptr(), nbytes, None)
+            if deferred:
+                _lib.check(L.tgt_linear_bwd_deferred(*a, ctypes.byref(descs[idx])))
+            else:
+                _lib.check(L.tgt_linear_bwd(*a))
+            outs.append([dx] + dW + db)
+            keep.append((ws, x, Ws, dys))
+        pairs.append(outs)
+
+    linear(0, 3000, 64, 64, 3)
+    linear(1, 1111, 128, 72, 1)
+    N, C = 2500, 64
+    print(f"deferred LayerNorm backward: N={N} C={C} {dtype}", flush=True)
+    s_ = torch.randn(N, C, generator=g).to(dtype).to(cuda)
+    gam = torch.randn(C, generator=g).to(dtype).to(cuda)
+    dy = torch.randn(N, C, generator=g).to(dtype).to(cuda)
+    mean = s_.float().mean(1).contiguous()
+    rstd = (s_.float().var(1, unbiased=False) + 1e-5).rsqrt().contiguous()
+    nbytes = L.tgt_layer_norm_bwd_workspace_bytes(C)
+    outs = []
+    for deferred in (False, True):
+        ds, dg, dbt = torch.empty_like(s_), torch.full_like(gam, 7.0), torch.full_like(gam, 7.0)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=cuda)
+        a = (s_.data_ptr(), gam.data_ptr(), mean.data_ptr(), rstd.data_ptr(), dy.data_ptr(), None, N, C, code, ds.data_ptr(),
+             dg.data_ptr(), dbt.data_ptr(), ws.data_ptr(), nbytes, None)
+        if deferred:
+            _lib.check(L.tgt_layer_norm_bwd_deferred(*a, ctypes.byref(descs[2])))
+        else:
+            _lib.check(L.tgt_layer_norm_bwd(*a))
+        outs.append([ds, dg, dbt])
+        keep.append(ws)
+    pairs.append(outs)
+    assert [d.n for d in descs] == [3 * (64 * 64 + 64), 128 * 72 + 72, 2 * C]
+    _lib.check(L.tgt_reduce_partials(descs, 3, code, None))
+    torch.cuda.synchronize()
+    for plain, later in pairs:
+        for a, b in zip(plain, later):
+            assert torch.equal(a, b)
+    assert L.tgt_reduce_partials(descs, 9, code, None) == _lib.ERR_INVALID_ARG
+    assert L.tgt_reduce_partials((_lib.ReduceDesc * 1)(), 1, code, None) == _lib.ERR_INVALID_ARG      # not filled in
+    assert L.tgt_linear_bwd_deferred(None, None, None, 1, 0, 64, 64, code, None, None, None, None, 0, None, None) == _lib.ERR_INVALID_ARG
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("act", ["gelu", "relu"])
+@pytest.mark.parametrize("N,in_f,out_f", [(3000, 64, 64), (70, 64, 64), (257, 64, 128), (100, 128, 64)])
+def test_linear_with_activation_equals_linear_then_activation(cuda, dtype, act, N, in_f, out_f):
+    """tgt_linear_act_fwd / tgt_linear_act_bwd (the activation in the epilogue of the 64 -> 64 kernels; two launches for
+    other shapes) give the bits of tgt_linear_fwd + tgt_gelu_fwd and of tgt_linear_bwd + tgt_gelu_bwd, which the
+    other tests hold against the oracle."""
+    print(f"linear+activation case: N={N} in={in_f} out={out_f} {act} {dtype}", flush=True)
+    L = _lib.lib()
+    code = 0 if dtype == torch.float32 else 1
+    a = 1 if act == "gelu" else 2
+    fwd_act, bwd_act = (L.tgt_gelu_fwd, L.tgt_gelu_bwd) if act == "gelu" else (L.tgt_relu_fwd, L.tgt_relu_bwd)
+    g = torch.Generator().manual_seed(N + out_f)
+    vp3 = ctypes.c_void_p * 3
+    x = torch.randn(N, in_f, generator=g).to(dtype).to(cuda)
+    W1 = (torch.randn(out_f, in_f, generator=g) / in_f ** 0.5).to(dtype).to(cuda)
+    b1 = torch.randn(out_f, generator=g).to(dtype).to(cuda)
+    # forward
+    u0, h0, u1, h1 = (torch.empty(N, out_f, dtype=dtype, device=cuda) for _ in range(4))
+    _lib.check(L.tgt_linear_fwd(x.data_ptr(), vp3(W1.data_ptr()), vp3(b1.data_ptr()), vp3(u0.data_ptr()), 1, N, in_f, out_f, code, None))
+    _lib.check(fwd_act(u0.data_ptr(), N * out_f, code, h0.data_ptr(), None))
+    _lib.check(L.tgt_linear_act_fwd(x.data_ptr(), W1.data_ptr(), b1.data_ptr(), N, in_f, out_f, code, a, u1.data_ptr(), h1.data_ptr(), None))
+    assert torch.equal(u0, u1) and torch.equal(h0, h1)
+    # backward of the next layer: its input is h = act(u), [N, out_f] -> [N, in_f]
+    W2 = (torch.randn(in_f, out_f, generator=g) / out_f ** 0.5).to(dtype).to(cuda)
+    dy = torch.randn(N, in_f, generator=g).to(dtype).to(cuda)
+    nbytes = L.tgt_linear_bwd_workspace_bytes(1, out_f, in_f)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=cuda)
+    dh, du0, du1 = (torch.empty(N, out_f, dtype=dtype, device=cuda) for _ in range(3))
+    dW0, dW1 = torch.empty_like(W2), torch.empty_like(W2)
+    db0, db1 = (torch.empty(in_f, dtype=dtype, device=cuda) for _ in range(2))
+    _lib.check(L.tgt_linear_bwd(h0.data_ptr(), vp3(W2.data_ptr()), vp3(dy.data_ptr()), 1, N, out_f, in_f, code, dh.data_ptr(),
+                                vp3(dW0.data_ptr()), vp3(db0.data_ptr()), ws.data_ptr(), nbytes, None))
+    _lib.check(bwd_act(u0.data_ptr(), dh.data_ptr(), N * out_f, code, du0.data_ptr(), None))
+    _lib.check(L.tgt_linear_act_bwd(h0.data_ptr(), W2.data_ptr(), dy.data_ptr(), u0.data_ptr(), N, out_f, in_f, code, a, du1.data_ptr(),
+                                    dW1.data_ptr(), db1.data_ptr(), ws.data_ptr(), nbytes, None, None))
+    torch.cuda.synchronize()
+    assert torch.equal(du0, du1) and torch.equal(dW0, dW1) and torch.equal(db0, db1)
+    assert L.tgt_linear_act_fwd(x.data_ptr(), W1.data_ptr(), None, N, in_f, out_f, code, 3, u1.data_ptr(), h1.data_ptr(), None) == _lib.ERR_INVALID_ARG
+
+
 def test_linear_empty_input(cuda):
     x = torch.zeros(0, 64, device=cuda, requires_grad=True)
     W = torch.randn(64, 64, device=cuda, requires_grad=True)

@@ -92,3 +92,22 @@ def test_graphormer_forward_rows_are_log_probabilities():
     out = E.graphormer_forward(x, _params(m), ei, 2, 4)
     assert out.shape == (S, 5)
     np.testing.assert_allclose(np.exp(out).sum(axis=1), 1.0, rtol=1e-12)
+
+
+def test_nll_loss_matches_torch_and_the_uniform_closed_form():
+    rng = np.random.default_rng(5)
+    N, C = 37, 7
+    lp = np.log(rng.dirichlet(np.ones(C), size=N))
+    t = rng.integers(0, C, size=N)
+    t[[3, 11, 30]] = -100
+    loss, grad = E.nll_loss(lp, t)
+    x = torch.tensor(lp, requires_grad=True)
+    want = torch.nn.functional.nll_loss(x, torch.tensor(t))
+    want.backward()
+    assert abs(loss - want.item()) < 1e-12
+    assert np.abs(grad - x.grad.numpy()).max() < 1e-15
+    # a uniform prediction costs log C whatever the targets; a dropped sign or a division by N instead of the count shows here
+    loss_u, grad_u = E.nll_loss(np.full((N, C), -np.log(C)), t)
+    assert abs(loss_u - np.log(C)) < 1e-12
+    assert abs(grad_u.sum() + 1.0) < 1e-12 and (grad_u[[3, 11, 30]] == 0).all()
+    assert np.isnan(E.nll_loss(lp, np.full(N, -100))[0])

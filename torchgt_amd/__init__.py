@@ -8,7 +8,7 @@ from .core_attention import (CoreAttention, SparseAttentionFunction, DenseAttent
                              dense_attention, gather_dense_bias)
 from .plan import GraphPlan, get_plan, clear_plan_cache, set_plan_cache_bytes
 from .multi_head_attention import MultiHeadAttention, LinearFunction, fused_linear
-from .encoder import FeedForwardNetwork, EncoderLayer, Graphormer
+from .encoder import FeedForwardNetwork, EncoderLayer, Graphormer, nll_loss
 from .graph_bias import GraphAttnBias, floyd_warshall, gen_edge_input
 from .graph_level import GraphNodeFeature, Graphormer as GraphLevelGraphormer
 from .gt import GT, GraphLevelGT, MLPReadout
@@ -18,5 +18,5 @@ __all__ = ["CoreAttention", "SparseAttentionFunction", "DenseAttentionFunction",
            "dense_attention", "gather_dense_bias",
            "GraphPlan", "get_plan", "clear_plan_cache", "set_plan_cache_bytes", "BlockAttentionFunction", "TileSet", "block_attention",
            "expand_tiles", "MultiHeadAttention", "LinearFunction", "fused_linear",
-           "FeedForwardNetwork", "EncoderLayer", "Graphormer", "GraphAttnBias", "floyd_warshall", "gen_edge_input",
+           "FeedForwardNetwork", "EncoderLayer", "Graphormer", "nll_loss", "GraphAttnBias", "floyd_warshall", "gen_edge_input",
            "GraphNodeFeature", "GraphLevelGraphormer", "GT", "GraphLevelGT", "MLPReadout"]

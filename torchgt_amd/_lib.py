@@ -73,13 +73,21 @@ SIGNATURES = {
     "tgt_linear_fwd": (_i32, [_vp, _vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp]),
     "tgt_linear_bwd_workspace_bytes": (_i64, [_i32, _i32, _i32]),
     "tgt_linear_bwd": (_i32, [_vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _i64, _vp]),
+    "tgt_linear_bwd_deferred": (_i32, [_vp, _vp, _vp, _i32, _i64, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _i64, _vp, _vp]),
+    "tgt_reduce_partials": (_i32, [_vp, _i32, _i32, _vp]),
+    "tgt_linear_act_fwd": (_i32, [_vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _vp]),
+    "tgt_linear_act_bwd": (_i32, [_vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _i64, _vp, _vp]),
     "tgt_add_layer_norm_fwd": (_i32, [_vp, _vp, _vp, _vp, _i64, _i32, _c.c_float, _i32, _vp, _vp, _vp, _vp, _vp]),
     "tgt_layer_norm_bwd_workspace_bytes": (_i64, [_i32]),
     "tgt_layer_norm_bwd": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _i64, _vp]),
+    "tgt_layer_norm_bwd_deferred": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _i64, _vp, _vp]),
     "tgt_gelu_fwd": (_i32, [_vp, _i64, _i32, _vp, _vp]),
     "tgt_gelu_bwd": (_i32, [_vp, _vp, _i64, _i32, _vp, _vp]),
     "tgt_relu_fwd": (_i32, [_vp, _i64, _i32, _vp, _vp]),
     "tgt_relu_bwd": (_i32, [_vp, _vp, _i64, _i32, _vp, _vp]),
+    "tgt_nll_loss_workspace_bytes": (_i64, [_i64]),
+    "tgt_nll_loss_fwd": (_i32, [_vp, _vp, _i64, _i32, _i32, _i64, _vp, _vp, _vp, _i64, _vp]),
+    "tgt_nll_loss_bwd": (_i32, [_vp, _vp, _vp, _i64, _i32, _i32, _i64, _vp, _vp]),
     "tgt_graph_attn_bias_fwd": (_i32, [_vp, _vp, _vp, _i32, _vp, _i32, _vp, _i32, _vp, _i32, _i32, _i32, _i32, _vp, _vp]),
     "tgt_graph_attn_bias_bwd_workspace_bytes": (_i64, [_i32, _i32, _i32]),
     "tgt_graph_attn_bias_bwd": (_i32, [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _i64, _vp]),
@@ -103,6 +111,13 @@ SIGNATURES = {
     "tgt_timing_slots": (_i32, []),
     "tgt_timing_read": (_i32, [_i32, _c.POINTER(_c.c_char_p), _c.POINTER(_c.c_double), _c.POINTER(_i64)]),
 }
+
+
+class ReduceDesc(_c.Structure):
+    """tgt_reduce_desc of include/torchgt_hip.h: a sum over workgroup partials that a *_deferred call leaves to
+    tgt_reduce_partials."""
+    _fields_ = [("partial", _c.c_void_p), ("workers", _c.c_int32), ("n", _c.c_int32), ("n_out", _c.c_int32),
+                ("out", _c.c_void_p * 6), ("begin", _c.c_int32 * 6)]
 
 
 def kernel_timings():

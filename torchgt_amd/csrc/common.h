@@ -20,6 +20,8 @@ constexpr int kCombineFan = 32;      // partial slots one combine step adds (= l
 constexpr int kNumClass = 5;         // wave item length classes: >32, <=32, <=16, <=8, <=4
 
 void set_error(const char* fmt, ...);
+// reduce.hip: up to eight fixed-order sums of workgroup partials in one launch
+int reduce_partials(const tgt_reduce_desc* descs, int count, int dtype, hipStream_t st);
 
 #define TGT_HIP_CHECK(expr)                                                        \
     do {                                                                           \
@@ -151,10 +153,27 @@ private:
     int nblocks_ = 0;
 };
 
+// nn.GELU() (exact erf form) and F.relu on one value, and dh * d act / du.  One definition for the elementwise kernels
+// and for the epilogues of the projections that apply the activation themselves: both give the same bits.
+//   GELU: h = 0.5 u (1 + erf(u / sqrt 2));  dh/du = 0.5 (1 + erf(u / sqrt 2)) + u exp(-u^2 / 2) / sqrt(2 pi)
+//   RELU: h = max(u, 0);  dh/du = 1 where u > 0
+template <bool RELU>
+__device__ __forceinline__ float act_value(float u) {
+    if (RELU) return u > 0.f ? u : 0.f;
+    const float cdf = 0.5f * (1.f + erff(u * 0.70710678118654752f));
+    return u * cdf;
+}
+template <bool RELU>
+__device__ __forceinline__ float act_grad(float u, float dh) {
+    if (RELU) return u > 0.f ? dh : 0.f;
+    const float cdf = 0.5f * (1.f + erff(u * 0.70710678118654752f));
+    return dh * (cdf + u * __expf(-0.5f * u * u) * 0.39894228040143268f);
+}
+
 // Kernel names of the optional per-kernel timing (timing.hip).
 enum KernelSlot { KS_FWD = 0, KS_NODE_SIDE, KS_BWD, KS_DENSE_FWD, KS_DENSE_BWD, KS_TILE_FWD, KS_TILE_BWD, KS_PROBE_GATHER, KS_LINEAR_FWD,
                   KS_LINEAR_DX, KS_LINEAR_DW, KS_LAYER_NORM_FWD, KS_LAYER_NORM_BWD, KS_GELU, KS_GRAPH_BIAS_FWD,
-                  KS_GRAPH_BIAS_BWD, KS_COUNT };
+                  KS_GRAPH_BIAS_BWD, KS_LOSS, KS_COUNT };
 
 // Scope guard: records a hipEvent on `st` before and after the launches made in
 // its scope when timing is enabled; does nothing otherwise.

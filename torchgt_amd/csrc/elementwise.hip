@@ -166,44 +166,6 @@ __global__ __launch_bounds__(kEwBlock) void k_layer_norm_bwd(const T* __restrict
     }
 }
 
-// out[e] = sum over workers of partial[w][e], e < n: 64 consecutive elements x 16
-// slices of the workers per workgroup; the slices are added in order, so the sum
-// does not depend on the launch.
-template <typename T>
-__global__ __launch_bounds__(1024) void k_reduce_workers(const float* __restrict__ partial, int workers, int n,
-                                                         T* __restrict__ out_a, T* __restrict__ out_b, int split) {
-    __shared__ float part[16][64];
-    const int el = threadIdx.x & 63, sl = threadIdx.x >> 6;
-    const int e = blockIdx.x * 64 + el;
-    const int w0 = (int)((int64_t)workers * sl / 16), w1 = (int)((int64_t)workers * (sl + 1) / 16);
-    float t = 0.f;
-    if (e < n) {
-        const float* __restrict__ src = partial + e;
-        int w = w0;
-        for (; w + 8 <= w1; w += 8) {
-            float v[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] = src[(int64_t)(w + i) * n];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) t += v[i];
-        }
-        for (; w < w1; ++w) t += src[(int64_t)w * n];
-    }
-    part[sl][el] = t;
-    __syncthreads();
-    if (sl == 0 && e < n) {
-        float sum = 0.f;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) sum += part[i][el];
-        T* dst = e < split ? out_a + e : out_b + (e - split);
-        if constexpr (sizeof(T) == 4) *reinterpret_cast<float*>(dst) = sum;
-        else {
-            const __bf16 b = static_cast<__bf16>(sum);
-            reinterpret_cast<ebf16*>(dst)->x = __builtin_bit_cast(uint16_t, b);
-        }
-    }
-}
-
 // nn.GELU (exact): h = 0.5 u (1 + erf(u / sqrt 2));  dh/du = 0.5 (1 + erf(u / sqrt 2)) + u exp(-u^2 / 2) / sqrt(2 pi)
 // RELU: F.relu instead (the GT layers, models/gt_dist_node_level.py:258,285): h = max(u, 0); dh/du = 1 where u > 0.
 template <typename T, bool BWD, bool RELU = false>
@@ -215,15 +177,7 @@ __global__ __launch_bounds__(kEwBlock) void k_gelu(const T* __restrict__ u, cons
         Vec<T>::load(u + v * VE, x);
         if (BWD) Vec<T>::load(dh + v * VE, d);
 #pragma unroll
-        for (int i = 0; i < VE; ++i) {
-            if (RELU) {
-                o[i] = x[i] > 0.f ? (BWD ? d[i] : x[i]) : 0.f;
-                continue;
-            }
-            const float cdf = 0.5f * (1.f + erff(x[i] * 0.70710678118654752f));
-            if (!BWD) o[i] = x[i] * cdf;
-            else o[i] = d[i] * (cdf + x[i] * __expf(-0.5f * x[i] * x[i]) * 0.39894228040143268f);
-        }
+        for (int i = 0; i < VE; ++i) o[i] = BWD ? act_grad<RELU>(x[i], d[i]) : act_value<RELU>(x[i]);
         Vec<T>::store(out + v * VE, o);
     }
 }
@@ -307,9 +261,9 @@ int64_t tgt_layer_norm_bwd_workspace_bytes(int C) {
     return C > 0 ? (int64_t)sizeof(float) * tgt::kLnWorkers * 2 * C : 0;
 }
 
-int tgt_layer_norm_bwd(const void* d_s, const void* d_gamma, const float* d_mean, const float* d_rstd, const void* d_dy,
-                       const void* d_ds_extra, int64_t N, int C, int dtype, void* d_ds, void* d_dgamma, void* d_dbeta,
-                       void* d_workspace, int64_t workspace_bytes, void* stream) {
+static int layer_norm_bwd_entry(const void* d_s, const void* d_gamma, const float* d_mean, const float* d_rstd, const void* d_dy,
+                                const void* d_ds_extra, int64_t N, int C, int dtype, void* d_ds, void* d_dgamma, void* d_dbeta,
+                                void* d_workspace, int64_t workspace_bytes, void* stream, tgt_reduce_desc* defer) {
     using namespace tgt;
     const int rc = ln_check(N, C, dtype, "tgt_layer_norm_bwd");
     if (rc != TGT_OK) return rc;
@@ -326,18 +280,35 @@ int tgt_layer_norm_bwd(const void* d_s, const void* d_gamma, const float* d_mean
     const int lpr = lanes_per_row(C, dtype);
     const int workers = (int)ew_grid(N, kEwBlock / lpr, kLnWorkers);
     float* partial = (float*)d_workspace;
-    KernelTimer t(KS_LAYER_NORM_BWD, st);
-    if (dtype == TGT_DTYPE_F32) launch_ln_bwd<float>(lpr, workers, d_s, d_gamma, d_mean, d_rstd, d_dy, d_ds_extra, N, d_ds, partial, st);
-    else launch_ln_bwd<ebf16>(lpr, workers, d_s, d_gamma, d_mean, d_rstd, d_dy, d_ds_extra, N, d_ds, partial, st);
-    const unsigned rgrid = (unsigned)((2 * C + 63) / 64);
-    if (dtype == TGT_DTYPE_F32)
-        hipLaunchKernelGGL((k_reduce_workers<float>), dim3(rgrid), dim3(1024), 0, st, partial, workers, 2 * C,
-                           (float*)d_dgamma, (float*)d_dbeta, C);
-    else
-        hipLaunchKernelGGL((k_reduce_workers<ebf16>), dim3(rgrid), dim3(1024), 0, st, partial, workers, 2 * C,
-                           (ebf16*)d_dgamma, (ebf16*)d_dbeta, C);
+    {
+        KernelTimer t(KS_LAYER_NORM_BWD, st);
+        if (dtype == TGT_DTYPE_F32) launch_ln_bwd<float>(lpr, workers, d_s, d_gamma, d_mean, d_rstd, d_dy, d_ds_extra, N, d_ds, partial, st);
+        else launch_ln_bwd<ebf16>(lpr, workers, d_s, d_gamma, d_mean, d_rstd, d_dy, d_ds_extra, N, d_ds, partial, st);
+    }
     TGT_HIP_CHECK(hipGetLastError());
-    return TGT_OK;
+    // the workgroups' column sums ([workers][2 C]: dgamma, then dbeta), added in a fixed order
+    tgt_reduce_desc r{};
+    r.partial = partial; r.workers = workers; r.n = 2 * C; r.n_out = 2;
+    r.out[0] = d_dgamma; r.begin[0] = 0;
+    r.out[1] = d_dbeta;  r.begin[1] = C;
+    if (defer) { *defer = r; return TGT_OK; }
+    return reduce_partials(&r, 1, dtype, st);
+}
+
+int tgt_layer_norm_bwd(const void* d_s, const void* d_gamma, const float* d_mean, const float* d_rstd, const void* d_dy,
+                       const void* d_ds_extra, int64_t N, int C, int dtype, void* d_ds, void* d_dgamma, void* d_dbeta,
+                       void* d_workspace, int64_t workspace_bytes, void* stream) {
+    return layer_norm_bwd_entry(d_s, d_gamma, d_mean, d_rstd, d_dy, d_ds_extra, N, C, dtype, d_ds, d_dgamma, d_dbeta, d_workspace,
+                                workspace_bytes, stream, nullptr);
+}
+
+int tgt_layer_norm_bwd_deferred(const void* d_s, const void* d_gamma, const float* d_mean, const float* d_rstd, const void* d_dy,
+                                const void* d_ds_extra, int64_t N, int C, int dtype, void* d_ds, void* d_dgamma, void* d_dbeta,
+                                void* d_workspace, int64_t workspace_bytes, void* stream, tgt_reduce_desc* desc) {
+    if (!desc) { tgt::set_error("tgt_layer_norm_bwd_deferred: a descriptor is needed"); return TGT_ERR_INVALID_ARG; }
+    *desc = tgt_reduce_desc{};
+    return layer_norm_bwd_entry(d_s, d_gamma, d_mean, d_rstd, d_dy, d_ds_extra, N, C, dtype, d_ds, d_dgamma, d_dbeta, d_workspace,
+                                workspace_bytes, stream, desc);
 }
 
 static int gelu_call(const void* d_u, const void* d_dh, int64_t n, int dtype, void* d_out, void* stream, bool bwd, bool relu = false) {

@@ -15,7 +15,7 @@
 //   k_linear<DX=true>    dx  = sum_j dy_j W_j         same walk, W staged transposed
 //   k_linear_gradw       dW_j = dy_j^T x, db_j = colsum(dy_j): each workgroup keeps a
 //                        64 x 64 tile of every dW_j in registers over its share of the
-//                        panels and writes one partial; k_linear_gradw_reduce adds the
+//                        panels and writes one partial; the fixed-order sum of reduce.hip adds the
 //                        partials in a fixed order (no atomics: results are reproducible)
 // Matrix instructions: v_mfma_f32_32x32x2_f32 for float32 (exact fp32 products,
 // fp32 accumulation; the 64-wide forward instead splits every float into three
@@ -82,6 +82,35 @@ __device__ __forceinline__ void store_rows(T* __restrict__ out, int64_t ld, cons
 #pragma unroll
         for (int r = 0; r < 16; ++r)
             if (8 * (r >> 2) + (r & 3) < rows_left) st1(out + (8 * (r >> 2) + (r & 3)) * ld, v[r]);
+    }
+}
+
+// The same with an activation on top: u = acc + bias goes to out_u and act(u) to out_h.  The activation is taken of
+// the value as it is stored (rounded to bf16 for bf16 outputs), so a separate activation kernel that reads out_u
+// gives the same bits.
+__device__ __forceinline__ float as_stored(float v, const float*) { return v; }
+__device__ __forceinline__ float as_stored(float v, const pbf16*) { return static_cast<float>(static_cast<__bf16>(v)); }
+template <typename T, bool RELU>
+__device__ __forceinline__ void store_rows_act(T* __restrict__ out_u, T* __restrict__ out_h, int64_t ld, const float16_t& acc,
+                                               float bias, int64_t rows_left) {
+    float v[16], w[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        v[r] = acc[r] + bias;
+        w[r] = act_value<RELU>(as_stored(v[r], out_u));
+    }
+    if (__builtin_amdgcn_readfirstlane(rows_left >= 32 ? 1 : 0)) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) st1(out_u + (8 * (r >> 2) + (r & 3)) * ld, v[r]);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) st1(out_h + (8 * (r >> 2) + (r & 3)) * ld, w[r]);
+    } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            if (8 * (r >> 2) + (r & 3) < rows_left) {
+                st1(out_u + (8 * (r >> 2) + (r & 3)) * ld, v[r]);
+                st1(out_h + (8 * (r >> 2) + (r & 3)) * ld, w[r]);
+            }
     }
 }
 
@@ -319,8 +348,10 @@ __device__ __forceinline__ void tile_put(const TileRegs<T>& t, T* __restrict__ t
 // for the life of the workgroup, which walks panels of 64 node rows; the next
 // panel's rows are fetched into registers while the current panel is multiplied.
 // Wave w owns the 32 x 32 block (w/2, w%2) of every 64 x 64 output tile.
-template <typename T, bool DX, int NW>
+// ACT (forward with one weight only): 1 = GELU, 2 = RELU: out[0] gets u = x W^T + b and out[1] the activation of u.
+template <typename T, bool DX, int NW, int ACT = 0>
 __global__ __launch_bounds__(kThreads) void k_linear64(LinArgs a) {
+    static_assert(ACT == 0 || (!DX && NW == 1), "the activation rides on a forward with one weight");
     constexpr int S = lds_stride<T>(64);
     constexpr int NA = DX ? NW : 1;      // source tiles per panel
     constexpr int NO = DX ? 1 : NW;      // output tiles per panel
@@ -369,8 +400,10 @@ __global__ __launch_bounds__(kThreads) void k_linear64(LinArgs a) {
             for (int s = 0; s < NA; ++s)
                 Mma<T, 64>::run(tA + (s * 64 + 32 * rb + l32) * S + h * 32,
                                 tW + ((DX ? s : o) * 64 + 32 * cb + l32) * S + h * 32, acc);
-            T* out = reinterpret_cast<T*>(a.out[o]) + (p * 64 + 32 * rb + 4 * h) * 64 + 32 * cb + l32;
-            store_rows<T>(out, 64, acc, bv[o], a.N - (p * 64 + 32 * rb + 4 * h));
+            const int64_t at = (p * 64 + 32 * rb + 4 * h) * 64 + 32 * cb + l32;
+            T* out = reinterpret_cast<T*>(a.out[o]) + at;
+            if constexpr (ACT != 0) store_rows_act<T, ACT == 2>(out, reinterpret_cast<T*>(a.out[1]) + at, 64, acc, bv[o], a.N - (p * 64 + 32 * rb + 4 * h));
+            else store_rows<T>(out, 64, acc, bv[o], a.N - (p * 64 + 32 * rb + 4 * h));
         }
     }
 }
@@ -432,8 +465,9 @@ __device__ __forceinline__ void mma_split(const Split32& x, const __bf16* w, flo
 
 // Same walk as k_linear64 (64 -> 64 features, weights resident, 64-row panels, register prefetch) for float32
 // through the split.  Weight planes in LDS: [NW][3][64][kPlaneStride] bf16; node rows: [NA][64][68] float.
-template <bool DX, int NW>
+template <bool DX, int NW, int ACT = 0>
 __global__ __launch_bounds__(kThreads) void k_linear64_split(LinArgs a) {
+    static_assert(ACT == 0 || (!DX && NW == 1), "the activation rides on a forward with one weight");
     constexpr int S = lds_stride<float>(64);
     constexpr int NA = DX ? NW : 1;
     constexpr int NO = DX ? 1 : NW;
@@ -502,8 +536,10 @@ __global__ __launch_bounds__(kThreads) void k_linear64_split(LinArgs a) {
             for (int o = 0; o < NW; ++o) {
                 float16_t acc = zero16();
                 mma_split(x, tW + (size_t)o * 3 * kPlaneElems + (32 * cb + l32) * kPlaneStride + h * 32, acc);
-                float* out = reinterpret_cast<float*>(a.out[o]) + (p * 64 + 32 * rb + 4 * h) * 64 + 32 * cb + l32;
-                store_rows<float>(out, 64, acc, bv[o], a.N - (p * 64 + 32 * rb + 4 * h));
+                const int64_t at = (p * 64 + 32 * rb + 4 * h) * 64 + 32 * cb + l32;
+                float* out = reinterpret_cast<float*>(a.out[o]) + at;
+                if constexpr (ACT != 0) store_rows_act<float, ACT == 2>(out, reinterpret_cast<float*>(a.out[1]) + at, 64, acc, bv[o], a.N - (p * 64 + 32 * rb + 4 * h));
+                else store_rows<float>(out, 64, acc, bv[o], a.N - (p * 64 + 32 * rb + 4 * h));
             }
         } else {
             float16_t acc = zero16();
@@ -532,7 +568,7 @@ int num_cus() {
     return cus;
 }
 
-template <typename T, bool DX, int NW>
+template <typename T, bool DX, int NW, int ACT = 0>
 int launch_linear64(const LinArgs& a, hipStream_t st) {
     constexpr int NA = DX ? NW : 1;
     // float32 forward goes through the three-way bf16 split.  The input gradient keeps the float32 matrix
@@ -541,8 +577,8 @@ int launch_linear64(const LinArgs& a, hipStream_t st) {
     constexpr bool kSplit = sizeof(T) == 4 && !DX;
     const size_t lds = kSplit ? (size_t)NW * 3 * kPlaneElems * 2 + sizeof(float) * (size_t)NA * 64 * lds_stride<float>(64)
                               : sizeof(T) * (size_t)(NW + NA) * 64 * lds_stride<T>(64);
-    const void* fn = kSplit ? reinterpret_cast<const void*>(&k_linear64_split<DX, NW>)
-                            : reinterpret_cast<const void*>(&k_linear64<T, DX, NW>);
+    const void* fn = kSplit ? reinterpret_cast<const void*>(&k_linear64_split<DX, NW, ACT>)
+                            : reinterpret_cast<const void*>(&k_linear64<T, DX, NW, ACT>);
     static bool raised = false;
     if (!raised && lds > 48 * 1024) {
         TGT_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
@@ -551,8 +587,8 @@ int launch_linear64(const LinArgs& a, hipStream_t st) {
     const int64_t n_panels = (a.N + 63) / 64;
     const int per_cu = (int)std::max<size_t>(1, std::min<size_t>(4, (size_t)(160 * 1024) / lds));
     const unsigned grid = (unsigned)std::min<int64_t>(n_panels, (int64_t)num_cus() * per_cu);
-    if (kSplit) hipLaunchKernelGGL((k_linear64_split<DX, NW>), dim3(grid), dim3(kThreads), lds, st, a);
-    else hipLaunchKernelGGL((k_linear64<T, DX, NW>), dim3(grid), dim3(kThreads), lds, st, a);
+    if (kSplit) hipLaunchKernelGGL((k_linear64_split<DX, NW, ACT>), dim3(grid), dim3(kThreads), lds, st, a);
+    else hipLaunchKernelGGL((k_linear64<T, DX, NW, ACT>), dim3(grid), dim3(kThreads), lds, st, a);
     return TGT_OK;
 }
 
@@ -647,7 +683,7 @@ __global__ __launch_bounds__(kThreads) void k_linear_gradw(GradWArgs a) {
 // in_features = out_features = 64: the whole backward in one pass over dy.  A workgroup walks panels of 64 node
 // rows; for each it forms the panel of dx = sum_j dy_j W_j (weights resident in LDS, transposed) and adds
 // dy_j^T x and the column sums of dy_j to the 64 x 64 weight-gradient tiles it keeps in registers; at its end it
-// writes one partial like k_linear_gradw (k_linear_gradw_reduce adds them).  dy is read once instead of twice and
+// writes one partial like k_linear_gradw (the fixed-order sum of reduce.hip adds them).  dy is read once instead of twice and
 // one launch replaces two.  Wave w owns the 32 x 32 block (w/2, w%2) of the dx panel and of every dW_j.
 //   float32: dy and x tiles stay in their natural [node][feature] layout; the products over nodes read them with
 //            4-byte LDS accesses (the 32x32x2 instruction takes one value per lane and operand).
@@ -661,6 +697,7 @@ struct Bwd64Args {
     void* dx;              // [N, 64]
     float* partial;        // [workers][nw][64*64 + 64]
     int64_t N;
+    const void* u;         // [N, 64], ACT only: x = act(u), and dx leaves as dx * act'(u)
 };
 
 template <typename T, int NW> constexpr size_t bwd64_lds_bytes() {
@@ -668,8 +705,11 @@ template <typename T, int NW> constexpr size_t bwd64_lds_bytes() {
     return sizeof(T) * (size_t)64 * lds_stride<T>(64) * (sizeof(T) == 4 ? 2 * NW + 1 : 3 * NW + 1);
 }
 
-template <typename T, int NW>
+// ACT (one weight only; 1 = GELU, 2 = RELU): the layer's input was x = act(u); what leaves in dx is the gradient of u,
+// dx * act'(u), with dx rounded as it would have been stored.
+template <typename T, int NW, int ACT = 0>
 __global__ __launch_bounds__(kThreads) void k_linear64_bwd(Bwd64Args a) {
+    static_assert(ACT == 0 || NW == 1, "the activation rides on a backward with one weight");
     constexpr int S = lds_stride<T>(64);
     constexpr bool F32 = sizeof(T) == 4;
     extern __shared__ __align__(16) unsigned char smem[];
@@ -736,10 +776,23 @@ __global__ __launch_bounds__(kThreads) void k_linear64_bwd(Bwd64Args a) {
         // dx panel: rows = nodes, contraction over m
         {
             float16_t acc = zero16();
+            float uu[ACT != 0 ? 16 : 1];
+            if constexpr (ACT != 0) {      // u where this lane writes; rows past the end repeat the last row and are not stored
+                const T* U = reinterpret_cast<const T*>(a.u) + 32 * cb + l32;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int64_t row = p * 64 + 32 * rb + 4 * h + 8 * (r >> 2) + (r & 3);
+                    uu[r] = ld1(U + (row < a.N ? row : a.N - 1) * 64);
+                }
+            }
 #pragma unroll
             for (int j = 0; j < NW; ++j)
                 Mma<T, 64>::run(tD + j * 64 * S + (32 * rb + l32) * S + h * 32, tW + j * 64 * S + (32 * cb + l32) * S + h * 32, acc);
             T* out = reinterpret_cast<T*>(a.dx) + (p * 64 + 32 * rb + 4 * h) * 64 + 32 * cb + l32;
+            if constexpr (ACT != 0) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[r] = act_grad<ACT == 2>(uu[r], as_stored(acc[r], out));
+            }
             store_rows<T>(out, 64, acc, 0.f, a.N - (p * 64 + 32 * rb + 4 * h));
         }
         // dW_j block (m = 32 rb + ., k = 32 cb + .): contraction over the 64 nodes of the panel
@@ -786,60 +839,29 @@ __global__ __launch_bounds__(kThreads) void k_linear64_bwd(Bwd64Args a) {
     if (wave < NW) mine[wave * per + 64 * 64 + lane] = colsum;
 }
 
-template <typename T, int NW>
+template <typename T, int NW, int ACT = 0>
 int launch_bwd64(const Bwd64Args& a, int workers, hipStream_t st) {
     constexpr size_t lds = bwd64_lds_bytes<T, NW>();
     static bool raised = false;
     if (!raised && lds > 48 * 1024) {
-        TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_linear64_bwd<T, NW>),
+        TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_linear64_bwd<T, NW, ACT>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         raised = true;
     }
-    hipLaunchKernelGGL((k_linear64_bwd<T, NW>), dim3(workers), dim3(kThreads), lds, st, a);
+    hipLaunchKernelGGL((k_linear64_bwd<T, NW, ACT>), dim3(workers), dim3(kThreads), lds, st, a);
     return TGT_OK;
 }
 
-struct ReduceArgs {
-    const float* partial;
-    void* dW[3];
-    void* db[3];           // entries may be null
-    int workers, nw, K, M;
-};
-
-// 64 consecutive elements x 16 slices of the workers per workgroup; the slices are
-// added in order, so the sum does not depend on the launch.
-template <typename T>
-__global__ __launch_bounds__(1024) void k_linear_gradw_reduce(ReduceArgs a) {
-    __shared__ float part[16][64];
-    const int el = threadIdx.x & 63, sl = threadIdx.x >> 6;
-    const int64_t per = (int64_t)a.M * a.K + a.M;
-    const int64_t total = per * a.nw;
-    const int64_t e = (int64_t)blockIdx.x * 64 + el;
-    const int w0 = (int)((int64_t)a.workers * sl / 16), w1 = (int)((int64_t)a.workers * (sl + 1) / 16);
-    float s = 0.f;
-    if (e < total) {
-        const float* __restrict__ src = a.partial + e;
-        int w = w0;
-        for (; w + 8 <= w1; w += 8) {      // eight loads in flight, added in worker order
-            float t[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) t[i] = src[(int64_t)(w + i) * total];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) s += t[i];
-        }
-        for (; w < w1; ++w) s += src[(int64_t)w * total];
+// What remains of a weight-gradient pass: the sum of the workers' partials ([workers][nw][M*K + M]) into dW_j and db_j.
+tgt_reduce_desc gradw_sum(const float* partial, int workers, int nw, int K, int M, void* const* d_dW, void* const* d_db) {
+    tgt_reduce_desc r{};
+    const int per = M * K + M;
+    r.partial = partial; r.workers = workers; r.n = per * nw; r.n_out = 2 * nw;
+    for (int j = 0; j < nw; ++j) {
+        r.out[2 * j] = d_dW[j];                      r.begin[2 * j] = j * per;
+        r.out[2 * j + 1] = d_db ? d_db[j] : nullptr; r.begin[2 * j + 1] = j * per + M * K;
     }
-    part[sl][el] = s;
-    __syncthreads();
-    if (sl == 0 && e < total) {
-        float t = 0.f;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) t += part[i][el];
-        const int j = (int)(e / per);
-        const int64_t off = e % per;
-        if (off < (int64_t)a.M * a.K) st1(reinterpret_cast<T*>(a.dW[j]) + off, t);
-        else if (a.db[j]) st1(reinterpret_cast<T*>(a.db[j]) + (off - (int64_t)a.M * a.K), t);
-    }
+    return r;
 }
 
 int check_shape(int n_out, int64_t N, int in_features, int out_features, int dtype) {
@@ -885,7 +907,15 @@ int launch_gradw(const GradWArgs& g, int workers, int tiles, hipStream_t st) {
 
 template <typename T>
 int linear_bwd_t(const void* d_x, const void* const* d_W, const void* const* d_dy, int n_out, int64_t N, int K, int M,
-                 void* d_dx, void* const* d_dW, void* const* d_db, float* partial, hipStream_t st) {
+                 void* d_dx, void* const* d_dW, void* const* d_db, float* partial, hipStream_t st, tgt_reduce_desc* defer,
+                 int act = 0, const void* d_u = nullptr) {
+    if (act != 0 && !(d_dx && d_dW && N > 0 && K == 64 && M == 64 && n_out == 1)) {
+        // no kernel of this shape applies the activation itself: the plain backward, then dx * act'(u) in place
+        const int rc = linear_bwd_t<T>(d_x, d_W, d_dy, n_out, N, K, M, d_dx, d_dW, d_db, partial, st, defer);
+        if (rc != TGT_OK || !d_dx || N == 0) return rc;
+        const int code = sizeof(T) == 4 ? TGT_DTYPE_F32 : TGT_DTYPE_BF16;
+        return act == TGT_ACT_RELU ? tgt_relu_bwd(d_u, d_dx, N * K, code, d_dx, st) : tgt_gelu_bwd(d_u, d_dx, N * K, code, d_dx, st);
+    }
     if (d_dx && d_dW && N > 0 && K == 64 && M == 64) {
         // one pass for dx and the weight gradients
         constexpr size_t lds1 = bwd64_lds_bytes<T, 1>();
@@ -895,24 +925,22 @@ int linear_bwd_t(const void* d_x, const void* const* d_W, const void* const* d_d
         const int workers = (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(n_panels, grad_workers(K, M)),
                                                                         (int64_t)num_cus() * per_cu));
         Bwd64Args b{};
-        b.x = d_x; b.dx = d_dx; b.partial = partial; b.N = N;
+        b.x = d_x; b.dx = d_dx; b.partial = partial; b.N = N; b.u = d_u;
         for (int j = 0; j < n_out; ++j) { b.dy[j] = d_dy[j]; b.W[j] = d_W[j]; }
         int rc = TGT_OK;
         {
             KernelTimer t(KS_LINEAR_DX, st);
-            if (n_out == 1) rc = launch_bwd64<T, 1>(b, workers, st);
+            if (act == TGT_ACT_GELU) rc = launch_bwd64<T, 1, 1>(b, workers, st);
+            else if (act == TGT_ACT_RELU) rc = launch_bwd64<T, 1, 2>(b, workers, st);
+            else if (n_out == 1) rc = launch_bwd64<T, 1>(b, workers, st);
             else if (n_out == 2) rc = launch_bwd64<T, 2>(b, workers, st);
             else rc = launch_bwd64<T, 3>(b, workers, st);
         }
         if (rc != TGT_OK) return rc;
-        KernelTimer t(KS_LINEAR_DW, st);
-        ReduceArgs r{};
-        r.partial = partial; r.workers = workers; r.nw = n_out; r.K = K; r.M = M;
-        for (int j = 0; j < n_out; ++j) { r.dW[j] = d_dW[j]; r.db[j] = d_db ? d_db[j] : nullptr; }
-        const int64_t total = ((int64_t)M * K + M) * n_out;
-        hipLaunchKernelGGL((k_linear_gradw_reduce<T>), dim3((unsigned)((total + 63) / 64)), dim3(1024), 0, st, r);
         TGT_HIP_CHECK(hipGetLastError());
-        return TGT_OK;
+        const tgt_reduce_desc r = gradw_sum(partial, workers, n_out, K, M, d_dW, d_db);
+        if (defer) { *defer = r; return TGT_OK; }
+        return reduce_partials(&r, 1, sizeof(T) == 4 ? TGT_DTYPE_F32 : TGT_DTYPE_BF16, st);
     }
     if (d_dx && N > 0) {
         LinArgs a{};
@@ -931,17 +959,18 @@ int linear_bwd_t(const void* d_x, const void* const* d_W, const void* const* d_d
         g.x = d_x;
         for (int j = 0; j < n_out; ++j) g.dy[j] = d_dy[j];
         g.partial = partial; g.N = N; g.K = K; g.M = M;
-        KernelTimer t(KS_LINEAR_DW, st);
         int rc = TGT_OK;
-        if (n_out == 1) rc = launch_gradw<T, 1>(g, workers, tiles, st);
-        else if (n_out == 2) rc = launch_gradw<T, 2>(g, workers, tiles, st);
-        else rc = launch_gradw<T, 3>(g, workers, tiles, st);
+        {
+            KernelTimer t(KS_LINEAR_DW, st);
+            if (n_out == 1) rc = launch_gradw<T, 1>(g, workers, tiles, st);
+            else if (n_out == 2) rc = launch_gradw<T, 2>(g, workers, tiles, st);
+            else rc = launch_gradw<T, 3>(g, workers, tiles, st);
+        }
         if (rc != TGT_OK) return rc;
-        ReduceArgs r{};
-        r.partial = partial; r.workers = workers; r.nw = n_out; r.K = K; r.M = M;
-        for (int j = 0; j < n_out; ++j) { r.dW[j] = d_dW[j]; r.db[j] = d_db ? d_db[j] : nullptr; }
-        const int64_t total = ((int64_t)M * K + M) * n_out;
-        hipLaunchKernelGGL((k_linear_gradw_reduce<T>), dim3((unsigned)((total + 63) / 64)), dim3(1024), 0, st, r);
+        TGT_HIP_CHECK(hipGetLastError());
+        const tgt_reduce_desc r = gradw_sum(partial, workers, n_out, K, M, d_dW, d_db);
+        if (defer) { *defer = r; return TGT_OK; }
+        return reduce_partials(&r, 1, sizeof(T) == 4 ? TGT_DTYPE_F32 : TGT_DTYPE_BF16, st);
     }
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
@@ -983,9 +1012,10 @@ int64_t tgt_linear_bwd_workspace_bytes(int n_out, int in_features, int out_featu
            ((int64_t)in_features * out_features + out_features);
 }
 
-int tgt_linear_bwd(const void* d_x, const void* const* d_W, const void* const* d_dy, int n_out, int64_t N,
-                   int in_features, int out_features, int dtype, void* d_dx, void* const* d_dW, void* const* d_db,
-                   void* d_workspace, int64_t workspace_bytes, void* stream) {
+static int linear_bwd_entry(const void* d_x, const void* const* d_W, const void* const* d_dy, int n_out, int64_t N,
+                            int in_features, int out_features, int dtype, void* d_dx, void* const* d_dW, void* const* d_db,
+                            void* d_workspace, int64_t workspace_bytes, void* stream, tgt_reduce_desc* defer, int act = 0,
+                            const void* d_u = nullptr) {
     using namespace tgt;
     const int rc = check_shape(n_out, N, in_features, out_features, dtype);
     if (rc != TGT_OK) return rc;
@@ -1006,9 +1036,69 @@ int tgt_linear_bwd(const void* d_x, const void* const* d_W, const void* const* d
     hipStream_t st = (hipStream_t)stream;
     if (dtype == TGT_DTYPE_F32)
         return linear_bwd_t<float>(d_x, d_W, d_dy, n_out, N, in_features, out_features, d_dx, d_dW, d_db,
-                                   (float*)d_workspace, st);
+                                   (float*)d_workspace, st, defer, act, d_u);
     return linear_bwd_t<pbf16>(d_x, d_W, d_dy, n_out, N, in_features, out_features, d_dx, d_dW, d_db,
-                               (float*)d_workspace, st);
+                               (float*)d_workspace, st, defer, act, d_u);
+}
+
+int tgt_linear_act_fwd(const void* d_x, const void* d_W, const void* d_b, int64_t N, int in_features, int out_features, int dtype,
+                       int act, void* d_u, void* d_h, void* stream) {
+    using namespace tgt;
+    const int rc = check_shape(1, N, in_features, out_features, dtype);
+    if (rc != TGT_OK) return rc;
+    if (act != TGT_ACT_GELU && act != TGT_ACT_RELU) { set_error("linear_act_fwd: unknown activation %d", act); return TGT_ERR_INVALID_ARG; }
+    if (!d_W || (N > 0 && (!d_x || !d_u || !d_h))) { set_error("linear_act_fwd: null pointer"); return TGT_ERR_INVALID_ARG; }
+    if (N == 0) return TGT_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (in_features != 64 || out_features != 64) {
+        // no kernel of this shape applies the activation itself: the plain forward, then the activation kernel
+        const void* W[1] = {d_W};
+        const void* b[1] = {d_b};
+        void* y[1] = {d_u};
+        const int lrc = tgt_linear_fwd(d_x, W, b, y, 1, N, in_features, out_features, dtype, stream);
+        if (lrc != TGT_OK) return lrc;
+        return act == TGT_ACT_RELU ? tgt_relu_fwd(d_u, N * out_features, dtype, d_h, stream) : tgt_gelu_fwd(d_u, N * out_features, dtype, d_h, stream);
+    }
+    LinArgs a{};
+    a.A[0] = d_x; a.W[0] = d_W; a.bias[0] = d_b; a.out[0] = d_u; a.out[1] = d_h;
+    a.nw = 1; a.N = N; a.K = 64; a.M = 64;
+    KernelTimer t(KS_LINEAR_FWD, st);
+    int lrc;
+    if (dtype == TGT_DTYPE_F32) lrc = act == TGT_ACT_GELU ? launch_linear64<float, false, 1, 1>(a, st) : launch_linear64<float, false, 1, 2>(a, st);
+    else lrc = act == TGT_ACT_GELU ? launch_linear64<pbf16, false, 1, 1>(a, st) : launch_linear64<pbf16, false, 1, 2>(a, st);
+    if (lrc != TGT_OK) return lrc;
+    TGT_HIP_CHECK(hipGetLastError());
+    return TGT_OK;
+}
+
+int tgt_linear_act_bwd(const void* d_h, const void* d_W, const void* d_dy, const void* d_u, int64_t N, int in_features,
+                       int out_features, int dtype, int act, void* d_du, void* d_dW, void* d_db, void* d_workspace,
+                       int64_t workspace_bytes, void* stream, tgt_reduce_desc* desc) {
+    if (act != TGT_ACT_GELU && act != TGT_ACT_RELU) { tgt::set_error("linear_act_bwd: unknown activation %d", act); return TGT_ERR_INVALID_ARG; }
+    if (!d_du || !d_dW || (N > 0 && !d_u)) { tgt::set_error("linear_act_bwd: null pointer"); return TGT_ERR_INVALID_ARG; }
+    const void* W[1] = {d_W};
+    const void* dy[1] = {d_dy};
+    void* dW[1] = {d_dW};
+    void* db[1] = {d_db};
+    if (desc) *desc = tgt_reduce_desc{};
+    return linear_bwd_entry(d_h, W, dy, 1, N, in_features, out_features, dtype, d_du, dW, d_db ? db : nullptr, d_workspace,
+                            workspace_bytes, stream, desc, act, d_u);
+}
+
+int tgt_linear_bwd(const void* d_x, const void* const* d_W, const void* const* d_dy, int n_out, int64_t N,
+                   int in_features, int out_features, int dtype, void* d_dx, void* const* d_dW, void* const* d_db,
+                   void* d_workspace, int64_t workspace_bytes, void* stream) {
+    return linear_bwd_entry(d_x, d_W, d_dy, n_out, N, in_features, out_features, dtype, d_dx, d_dW, d_db, d_workspace,
+                            workspace_bytes, stream, nullptr);
+}
+
+int tgt_linear_bwd_deferred(const void* d_x, const void* const* d_W, const void* const* d_dy, int n_out, int64_t N,
+                            int in_features, int out_features, int dtype, void* d_dx, void* const* d_dW, void* const* d_db,
+                            void* d_workspace, int64_t workspace_bytes, void* stream, tgt_reduce_desc* desc) {
+    if (!desc || !d_dW) { tgt::set_error("linear_bwd_deferred: a descriptor and weight-gradient outputs are needed"); return TGT_ERR_INVALID_ARG; }
+    *desc = tgt_reduce_desc{};
+    return linear_bwd_entry(d_x, d_W, d_dy, n_out, N, in_features, out_features, dtype, d_dx, d_dW, d_db, d_workspace,
+                            workspace_bytes, stream, desc);
 }
 
 }  // extern "C"

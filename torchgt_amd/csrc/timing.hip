@@ -14,7 +14,7 @@ namespace tgt {
 static const char* kSlotNames[KS_COUNT] = {
     "attn_fwd", "bwd_node_side", "attn_bwd", "dense_fwd", "dense_bwd", "tile_fwd", "tile_bwd", "probe_row_gather",
     "linear_fwd", "linear_dx", "linear_dw", "layer_norm_fwd", "layer_norm_bwd", "gelu",
-    "graph_bias_fwd", "graph_bias_bwd",
+    "graph_bias_fwd", "graph_bias_bwd", "nll_loss",
 };
 
 struct Pending { hipEvent_t start, stop; int slot; };

@@ -13,6 +13,7 @@
 //                                bf16_products) -> (x + attention, ffn output)      the graph-level layer around the dense attention
 //   torchgt::add(x, r) -> sum
 //   torchgt::gelu(u) / torchgt::relu(u) -> h
+//   torchgt::nll_loss(log_probs, target, ignore_index) -> loss                (mean over the rows that count)
 #include <torch/library.h>
 #include <torch/custom_class.h>
 #include <torch/autograd.h>
@@ -467,16 +468,66 @@ struct Activation : public torch::autograd::Function<Activation<GELU>> {
 Tensor gelu(const Tensor& u) { return Activation<true>::apply(u); }
 Tensor relu(const Tensor& u) { return Activation<false>::apply(u); }
 
+// F.nll_loss(log_probs [N, C], target [N] int64), reduction 'mean' (main_sp_sparse_node_level.py:200)
+struct NllLoss : public torch::autograd::Function<NllLoss> {
+    static Tensor forward(AutogradContext* ctx, Tensor logp, Tensor target, int64_t ignore_index) {
+        on_gpu(logp, "nll_loss");
+        TORCH_CHECK(logp.dim() == 2, "nll_loss: log_probs must be [N, C]");
+        TORCH_CHECK(target.is_cuda() && target.scalar_type() == at::kLong && target.dim() == 1 && target.size(0) == logp.size(0),
+                    "nll_loss: target must be an int64 GPU tensor [N]");
+        Tensor lp = logp.contiguous(), t = target.contiguous();
+        c10::DeviceGuard guard(logp.device());
+        const int64_t N = lp.size(0), C = lp.size(1);
+        Tensor loss = at::empty({}, lp.options()), count = at::empty({1}, lp.options().dtype(at::kFloat));
+        const int64_t nbytes = tgt_nll_loss_workspace_bytes(N);
+        Tensor ws = at::empty({nbytes}, lp.options().dtype(at::kByte));
+        check(tgt_nll_loss_fwd(lp.data_ptr(), t.data_ptr<int64_t>(), N, (int)C, dtype_code(lp), ignore_index, loss.data_ptr(),
+                               count.data_ptr<float>(), ws.data_ptr(), nbytes, stream_of(lp)),
+              "tgt_nll_loss_fwd");
+        ctx->save_for_backward({t, count});
+        ctx->saved_data["C"] = C;
+        ctx->saved_data["ignore"] = ignore_index;
+        ctx->saved_data["bf16"] = lp.scalar_type() == at::kBFloat16;
+        return loss;
+    }
+    static variable_list backward(AutogradContext* ctx, variable_list grads) {
+        auto sv = ctx->get_saved_variables();
+        const Tensor &t = sv[0], &count = sv[1];
+        c10::DeviceGuard guard(t.device());
+        const int64_t N = t.size(0), C = ctx->saved_data["C"].toInt();
+        const auto dt = ctx->saved_data["bf16"].toBool() ? at::kBFloat16 : at::kFloat;
+        Tensor g = grads[0].to(dt).contiguous();
+        Tensor d = at::empty({N, C}, t.options().dtype(dt));
+        check(tgt_nll_loss_bwd(t.data_ptr<int64_t>(), g.data_ptr(), count.data_ptr<float>(), N, (int)C, dtype_code(d),
+                               ctx->saved_data["ignore"].toInt(), d.data_ptr(), stream_of(d)),
+              "tgt_nll_loss_bwd");
+        return {d, Tensor(), Tensor()};
+    }
+};
+Tensor nll_loss(const Tensor& logp, const Tensor& target, int64_t ignore_index) { return NllLoss::apply(logp, target, ignore_index); }
+
 // ---------------------------------------------------------------------------------------------------------------
 // one whole encoder layer of the node-level Graphormer (models/graphormer_dist_node_level.py:276-314) with sparse
-// attention, no bias, no dropout: the eight kernels of the forward and the fourteen of the backward launched from one
-// operator and one autograd node instead of eight of each.  Same kernels, same order, same numbers as the modules give
-// op by op; what goes away is the per-operator cost of the dispatcher and of autograd between the launches.
+// attention, no bias, no dropout: the seven kernels of the forward and the nine of the backward launched from one
+// operator and one autograd node instead of eight of each.  The same numbers as the modules give op by op; what goes
+// away is the per-operator cost of the dispatcher and of autograd between the launches, and what only a whole layer
+// can do: GELU rides on the FFN linears (tgt_linear_act_fwd / _bwd) and the six sums over weight-gradient partials
+// share one launch at the end of the backward (tgt_reduce_partials).
 //   s1 = x (+ residual); y1 = LN1(s1); q, k, v = y1 W^T + b; o = attention(q, k, v); a = o Wo^T + bo
 //   s2 = s1 + a; y2 = LN2(s2); u = y2 W1^T + b1; h = gelu(u); f = h W2^T + b2;  returns (s2, f)
 // params: n1.weight, n1.bias, Wq, bq, Wk, bk, Wv, bv, Wo, bo, n2.weight, n2.bias, W1, b1, W2, b2
 // ---------------------------------------------------------------------------------------------------------------
 namespace layer {
+// The sums over workgroup partials that the backward kernels of a layer leave behind, for one launch at the layer's end.
+struct Deferred {
+    std::vector<tgt_reduce_desc> sums;
+    std::vector<Tensor> workspaces;       // hold the partials until the launch
+    void run(int code, void* stream) {
+        for (size_t i = 0; i < sums.size(); i += 8)
+            check(tgt_reduce_partials(sums.data() + i, (int)std::min<size_t>(8, sums.size() - i), code, stream), "tgt_reduce_partials");
+        sums.clear();
+    }
+};
 void ln_fwd(const Tensor& x, const Tensor& r, const Tensor& g, const Tensor& b, double eps, Tensor& sum, Tensor& y, Tensor& mean,
             Tensor& rstd) {
     const int64_t N = x.size(0), C = x.size(1);
@@ -491,15 +542,18 @@ void ln_fwd(const Tensor& x, const Tensor& r, const Tensor& g, const Tensor& b, 
 }
 // ds = LN backward of dy (+ extra), dgamma, dbeta
 void ln_bwd(const Tensor& s, const Tensor& g, const Tensor& mean, const Tensor& rstd, const Tensor& dy, const Tensor& extra, Tensor& ds,
-            Tensor& dg, Tensor& db) {
+            Tensor& dg, Tensor& db, Deferred& later) {
     const int64_t N = s.size(0), C = s.size(1);
     ds = at::empty_like(s); dg = at::empty_like(g); db = at::empty_like(g);
     const int64_t nbytes = tgt_layer_norm_bwd_workspace_bytes((int)C);
     Tensor ws = at::empty({nbytes}, s.options().dtype(at::kByte));
-    check(tgt_layer_norm_bwd(s.data_ptr(), g.data_ptr(), mean.data_ptr<float>(), rstd.data_ptr<float>(), dy.data_ptr(),
-                             extra.defined() ? extra.data_ptr() : nullptr, N, (int)C, dtype_code(s), ds.data_ptr(), dg.data_ptr(),
-                             db.data_ptr(), ws.data_ptr(), nbytes, stream_of(s)),
-          "tgt_layer_norm_bwd");
+    tgt_reduce_desc sum;
+    check(tgt_layer_norm_bwd_deferred(s.data_ptr(), g.data_ptr(), mean.data_ptr<float>(), rstd.data_ptr<float>(), dy.data_ptr(),
+                                      extra.defined() ? extra.data_ptr() : nullptr, N, (int)C, dtype_code(s), ds.data_ptr(), dg.data_ptr(),
+                                      db.data_ptr(), ws.data_ptr(), nbytes, stream_of(s), &sum),
+          "tgt_layer_norm_bwd_deferred");
+    later.sums.push_back(sum);
+    later.workspaces.push_back(ws);
 }
 // ys[j] = x W[j]^T + b[j]
 void lin_fwd(const Tensor& x, std::initializer_list<const Tensor*> W, std::initializer_list<const Tensor*> b, std::vector<Tensor>& ys) {
@@ -517,7 +571,7 @@ void lin_fwd(const Tensor& x, std::initializer_list<const Tensor*> W, std::initi
 }
 // dx = sum_j dy[j] W[j]; dW[j] = dy[j]^T x; db[j] = column sums of dy[j]
 void lin_bwd(const Tensor& x, std::initializer_list<const Tensor*> W, std::initializer_list<const Tensor*> dy, Tensor& dx,
-             std::vector<Tensor>& dW, std::vector<Tensor>& db) {
+             std::vector<Tensor>& dW, std::vector<Tensor>& db, Deferred& later) {
     const int n = (int)W.size();
     const int64_t N = x.size(0), in_f = x.size(1), out_f = (*W.begin())->size(0);
     const void *Wp[3] = {nullptr, nullptr, nullptr}, *DYp[3] = {nullptr, nullptr, nullptr};
@@ -531,9 +585,37 @@ void lin_bwd(const Tensor& x, std::initializer_list<const Tensor*> W, std::initi
     dx = at::empty_like(x);
     const int64_t ws_bytes = tgt_linear_bwd_workspace_bytes(n, (int)in_f, (int)out_f);
     Tensor ws = at::empty({ws_bytes}, x.options().dtype(at::kByte));
-    check(tgt_linear_bwd(x.data_ptr(), Wp, DYp, n, N, (int)in_f, (int)out_f, dtype_code(x), dx.data_ptr(), DWp, DBp, ws.data_ptr(), ws_bytes,
-                         stream_of(x)),
-          "tgt_linear_bwd");
+    tgt_reduce_desc sum;
+    check(tgt_linear_bwd_deferred(x.data_ptr(), Wp, DYp, n, N, (int)in_f, (int)out_f, dtype_code(x), dx.data_ptr(), DWp, DBp, ws.data_ptr(),
+                                  ws_bytes, stream_of(x), &sum),
+          "tgt_linear_bwd_deferred");
+    later.sums.push_back(sum);
+    later.workspaces.push_back(ws);
+}
+// u = x W^T + b, h = gelu(u) from one kernel
+void lin_gelu_fwd(const Tensor& x, const Tensor& W, const Tensor& b, Tensor& u, Tensor& h) {
+    const int64_t N = x.size(0), in_f = x.size(1), out_f = W.size(0);
+    u = at::empty({N, out_f}, x.options());
+    h = at::empty({N, out_f}, x.options());
+    check(tgt_linear_act_fwd(x.data_ptr(), W.data_ptr(), b.data_ptr(), N, (int)in_f, (int)out_f, dtype_code(x), TGT_ACT_GELU, u.data_ptr(),
+                             h.data_ptr(), stream_of(x)),
+          "tgt_linear_act_fwd");
+}
+// backward of y = h W^T + b with h = gelu(u): du = (dy W) gelu'(u), dW = dy^T h, db
+void lin_gelu_bwd(const Tensor& h, const Tensor& W, const Tensor& dy, const Tensor& u, Tensor& du, std::vector<Tensor>& dW,
+                  std::vector<Tensor>& db, Deferred& later) {
+    const int64_t N = h.size(0), in_f = h.size(1), out_f = W.size(0);
+    du = at::empty_like(u);
+    dW.assign(1, at::empty_like(W));
+    db.assign(1, at::empty({out_f}, h.options()));
+    const int64_t ws_bytes = tgt_linear_bwd_workspace_bytes(1, (int)in_f, (int)out_f);
+    Tensor ws = at::empty({ws_bytes}, h.options().dtype(at::kByte));
+    tgt_reduce_desc sum;
+    check(tgt_linear_act_bwd(h.data_ptr(), W.data_ptr(), dy.data_ptr(), u.data_ptr(), N, (int)in_f, (int)out_f, dtype_code(h), TGT_ACT_GELU,
+                             du.data_ptr(), dW[0].data_ptr(), db[0].data_ptr(), ws.data_ptr(), ws_bytes, stream_of(h), &sum),
+          "tgt_linear_act_bwd");
+    later.sums.push_back(sum);
+    later.workspaces.push_back(ws);
 }
 }  // namespace layer
 
@@ -562,9 +644,9 @@ struct EncoderLayerFn : public torch::autograd::Function<EncoderLayerFn> {
               "tgt_sparse_attn_fwd");
         layer::lin_fwd(o, {&p[8]}, {&p[9]}, a);
         layer::ln_fwd(s1, a[0], p[10], p[11], eps2, s2, y2, mean2, rstd2);
-        layer::lin_fwd(y2, {&p[12]}, {&p[13]}, u);
-        Tensor h = at::empty_like(u[0]);
-        check(tgt_gelu_fwd(u[0].data_ptr(), u[0].numel(), dtype_code(x), h.data_ptr(), stream_of(x)), "tgt_gelu_fwd");
+        Tensor h;
+        u.resize(1);
+        layer::lin_gelu_fwd(y2, p[12], p[13], u[0], h);
         layer::lin_fwd(h, {&p[14]}, {&p[15]}, f);
         std::vector<Tensor> save{s1, mean1, rstd1, y1, qkv[0], qkv[1], qkv[2], o, Z, s2, mean2, rstd2, y2, u[0], h, ws};
         save.insert(save.end(), p.begin(), p.end());
@@ -587,22 +669,22 @@ struct EncoderLayerFn : public torch::autograd::Function<EncoderLayerFn> {
         if (grads[0].defined()) d_s2 = grads[0].reshape({N, C}).contiguous();
         d_f = grads[1].defined() ? grads[1].reshape({N, C}).contiguous() : at::zeros_like(s1);
         const int code = dtype_code(s1);
-        Tensor dh, du, dy2, ds2, do_, dy1, dx;
+        Tensor du, dy2, ds2, do_, dy1, dx;
         std::vector<Tensor> dW2, db2, dW1, db1, dWo, dbo, dWqkv, dbqkv;
-        layer::lin_bwd(h, {&p[14]}, {&d_f}, dh, dW2, db2);
-        du = at::empty_like(u);
-        check(tgt_gelu_bwd(u.data_ptr(), dh.data_ptr(), u.numel(), code, du.data_ptr(), stream_of(u)), "tgt_gelu_bwd");
-        layer::lin_bwd(y2, {&p[12]}, {&du}, dy2, dW1, db1);
+        layer::Deferred later;
+        layer::lin_gelu_bwd(h, p[14], d_f, u, du, dW2, db2, later);
+        layer::lin_bwd(y2, {&p[12]}, {&du}, dy2, dW1, db1, later);
         Tensor dg2, dbn2, dg1, dbn1;
-        layer::ln_bwd(s2, p[10], mean2, rstd2, dy2, d_s2, ds2, dg2, dbn2);           // gradient of s2 = s1 + a: to both
-        layer::lin_bwd(o, {&p[8]}, {&ds2}, do_, dWo, dbo);
+        layer::ln_bwd(s2, p[10], mean2, rstd2, dy2, d_s2, ds2, dg2, dbn2, later);           // gradient of s2 = s1 + a: to both
+        layer::lin_bwd(o, {&p[8]}, {&ds2}, do_, dWo, dbo, later);
         Tensor dq = at::empty_like(q), dk = at::empty_like(k), dv = at::empty_like(v);
         check(tgt_sparse_attn_bwd(reinterpret_cast<const tgt_plan_t*>(ctx->saved_data["plan"].toCustomClass<PlanHolder>()->h), q.data_ptr(),
                                   k.data_ptr(), v.data_ptr(), nullptr, TGT_BIAS_NONE, (int)H, (int)d, code, o.data_ptr(), Z.data_ptr<float>(),
                                   do_.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), nullptr, ws.data_ptr(), ws.numel(), stream_of(q)),
               "tgt_sparse_attn_bwd");
-        layer::lin_bwd(y1, {&p[2], &p[4], &p[6]}, {&dq, &dk, &dv}, dy1, dWqkv, dbqkv);
-        layer::ln_bwd(s1, p[0], mean1, rstd1, dy1, ds2, dx, dg1, dbn1);              // gradient of s1 = x (+ residual)
+        layer::lin_bwd(y1, {&p[2], &p[4], &p[6]}, {&dq, &dk, &dv}, dy1, dWqkv, dbqkv, later);
+        layer::ln_bwd(s1, p[0], mean1, rstd1, dy1, ds2, dx, dg1, dbn1, later);              // gradient of s1 = x (+ residual)
+        later.run(dtype_code(s1), stream_of(s1));        // the six weight-gradient sums of the layer in one launch
         Tensor dxv = dx.view(ctx->saved_data["shape"].toIntVector());
         variable_list out{dxv, ctx->saved_data["has_r"].toBool() ? dxv : Tensor(),
                           dg1, dbn1, dWqkv[0], dbqkv[0], dWqkv[1], dbqkv[1], dWqkv[2], dbqkv[2], dWo[0], dbo[0], dg2, dbn2, dW1[0], db1[0],
@@ -684,9 +766,9 @@ struct DenseEncoderLayerFn : public torch::autograd::Function<DenseEncoderLayerF
         }
         layer::lin_fwd(o, {&p[8]}, {&p[9]}, a);
         layer::ln_fwd(s1, a[0], p[10], p[11], eps2, s2, y2, mean2, rstd2);
-        layer::lin_fwd(y2, {&p[12]}, {&p[13]}, u);
-        Tensor h = at::empty_like(u[0]);
-        check(tgt_gelu_fwd(u[0].data_ptr(), u[0].numel(), dtype_code(x), h.data_ptr(), stream_of(x)), "tgt_gelu_fwd");
+        Tensor h;
+        u.resize(1);
+        layer::lin_gelu_fwd(y2, p[12], p[13], u[0], h);
         layer::lin_fwd(h, {&p[14]}, {&p[15]}, f);
         std::vector<Tensor> save{s1, mean1, rstd1, y1, qkv[0], qkv[1], qkv[2], o, lse, s2, mean2, rstd2, y2, u[0], h, ab, sp16, et16};
         save.insert(save.end(), p.begin(), p.end());
@@ -718,14 +800,13 @@ struct DenseEncoderLayerFn : public torch::autograd::Function<DenseEncoderLayerF
         Tensor d_s2, d_f;
         if (grads[0].defined()) d_s2 = grads[0].reshape({N, C}).contiguous();
         d_f = grads[1].defined() ? grads[1].reshape({N, C}).contiguous() : at::zeros_like(s1);
-        Tensor dh, du, dy2, ds2, do_, dy1, dx, dg2, dbn2, dg1, dbn1;
+        Tensor du, dy2, ds2, do_, dy1, dx, dg2, dbn2, dg1, dbn1;
         std::vector<Tensor> dW2, db2, dW1, db1, dWo, dbo, dWqkv, dbqkv;
-        layer::lin_bwd(h, {&p[14]}, {&d_f}, dh, dW2, db2);
-        du = at::empty_like(u);
-        check(tgt_gelu_bwd(u.data_ptr(), dh.data_ptr(), u.numel(), dtype_code(s1), du.data_ptr(), stream_of(u)), "tgt_gelu_bwd");
-        layer::lin_bwd(y2, {&p[12]}, {&du}, dy2, dW1, db1);
-        layer::ln_bwd(s2, p[10], mean2, rstd2, dy2, d_s2, ds2, dg2, dbn2);
-        layer::lin_bwd(o, {&p[8]}, {&ds2}, do_, dWo, dbo);
+        layer::Deferred later;
+        layer::lin_gelu_bwd(h, p[14], d_f, u, du, dW2, db2, later);
+        layer::lin_bwd(y2, {&p[12]}, {&du}, dy2, dW1, db1, later);
+        layer::ln_bwd(s2, p[10], mean2, rstd2, dy2, d_s2, ds2, dg2, dbn2, later);
+        layer::lin_bwd(o, {&p[8]}, {&ds2}, do_, dWo, dbo, later);
         Tensor dq = at::empty_like(q), dk = at::empty_like(k), dv = at::empty_like(v);
         variable_list dextra;
         if (kind == 2) {
@@ -750,8 +831,9 @@ struct DenseEncoderLayerFn : public torch::autograd::Function<DenseEncoderLayerF
                   "tgt_dense_attn_dropout_bwd");
             if (kind == 1) dextra = {dbias};
         }
-        layer::lin_bwd(y1, {&p[2], &p[4], &p[6]}, {&dq, &dk, &dv}, dy1, dWqkv, dbqkv);
-        layer::ln_bwd(s1, p[0], mean1, rstd1, dy1, ds2, dx, dg1, dbn1);
+        layer::lin_bwd(y1, {&p[2], &p[4], &p[6]}, {&dq, &dk, &dv}, dy1, dWqkv, dbqkv, later);
+        layer::ln_bwd(s1, p[0], mean1, rstd1, dy1, ds2, dx, dg1, dbn1, later);
+        later.run(dtype_code(s1), stream_of(s1));        // the six weight-gradient sums of the layer in one launch
         Tensor dxv = dx.view({b, S, C});
         variable_list out{dxv, ctx->saved_data["has_r"].toBool() ? dxv : Tensor(),
                           dg1, dbn1, dWqkv[0], dbqkv[0], dWqkv[1], dbqkv[1], dWqkv[2], dbqkv[2], dWo[0], dbo[0], dg2, dbn2, dW1[0], db1[0],
@@ -788,6 +870,7 @@ TORCH_LIBRARY(torchgt, m) {
     m.def("add(Tensor x, Tensor r) -> Tensor");
     m.def("gelu(Tensor u) -> Tensor");
     m.def("relu(Tensor u) -> Tensor");
+    m.def("nll_loss(Tensor log_probs, Tensor target, int ignore_index=-100) -> Tensor");
 }
 
 // One implementation per op, registered for every backend and for autograd alike: each is an autograd function
@@ -804,4 +887,5 @@ TORCH_LIBRARY_IMPL(torchgt, CompositeImplicitAutograd, m) {
     m.impl("add", add);
     m.impl("gelu", gelu);
     m.impl("relu", relu);
+    m.impl("nll_loss", nll_loss);
 }

@@ -48,6 +48,15 @@ class GeluFunction:
         return _ext.ops().gelu(u)
 
 
+def nll_loss(log_probs, target, ignore_index=-100):
+    """``F.nll_loss(log_probs, target)`` of the training and evaluation loops (main_sp_sparse_node_level.py:200,
+    gt_sp/evaluate.py:52): mean over the rows whose target is not ``ignore_index``, no class weights.
+    ``torch.ops.torchgt.nll_loss``: one row per lane and a fixed-order sum (torch's kernel walks the rows with a
+    single workgroup, ~95 + 60 us forward + backward for 64 K rows against ~5 + 3 here).  A target outside
+    [0, C) other than ``ignore_index`` counts as ignored."""
+    return _ext.ops().nll_loss(log_probs, target, int(ignore_index))
+
+
 def init_params(module, n_layers):
     """models/graphormer_dist_node_level.py:18-24."""
     if isinstance(module, nn.Linear):
@@ -154,7 +163,7 @@ class Graphormer(nn.Module):
         (node_feature,) = fused_linear(x, self.node_encoder)
         if perturb is not None:
             node_feature = node_feature + perturb
-        global_node_feature = self.graph_token.weight.unsqueeze(0).repeat(n_graph, 1, 1)
+        global_node_feature = self.graph_token.weight.unsqueeze(0).expand(n_graph, -1, -1)      # a view: cat makes the copy
         node_feature = torch.cat([global_node_feature, node_feature], dim=1)
         output = self.input_dropout(node_feature)
         if attn_bias is not None:
