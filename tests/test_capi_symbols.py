@@ -58,7 +58,8 @@ def test_torch_extension_loads_and_registers_its_operators():
     import torch
     from torchgt_amd import _ext
     ops = _ext.ops()
-    for name in ("sparse_attention", "dense_attention", "linear", "add_layer_norm", "add", "gelu", "relu"):
+    for name in ("sparse_attention", "dense_attention", "dense_attention_ids", "linear", "add_layer_norm", "add", "gelu", "relu",
+                 "ffn", "nll_loss", "encoder_layer", "dense_encoder_layer"):
         assert hasattr(ops, name), name
     assert hasattr(torch.classes.torchgt, "PlanHolder")
     with pytest.raises(RuntimeError, match="GPU"):

@@ -12,7 +12,7 @@ import torch
 from oracle import encoder_layer as E
 from oracle import graph_prep as ogp
 from oracle import sparse_attention as osa
-from torchgt_amd import EncoderLayer, Graphormer, _lib, nll_loss, workloads
+from torchgt_amd import EncoderLayer, FeedForwardNetwork, Graphormer, _lib, fused_linear, nll_loss, workloads
 from torchgt_amd.encoder import AddFunction, AddLayerNormFunction, GeluFunction
 
 pytestmark = pytest.mark.gpu
@@ -89,6 +89,44 @@ def _ref_layer(p, x, ei, H, prefix=""):
     x1 = x + lin(o.reshape(b, S, hidden), g("self_attention.output_layer.weight"), g("self_attention.output_layer.bias"))
     y = F.layer_norm(x1, (hidden,), g("ffn_norm.weight"), g("ffn_norm.bias"))
     return x1 + lin(F.gelu(lin(y, g("ffn.layer1.weight"), g("ffn.layer1.bias"))), g("ffn.layer2.weight"), g("ffn.layer2.bias"))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hidden,ffn", [(64, 64), (64, 128), (40, 24)])
+def test_ffn_operator_matches_oracle_and_the_separate_operators(cuda, dtype, hidden, ffn):
+    """FeedForwardNetwork.forward as one operator (torch.ops.torchgt.ffn): against the oracle (layer2(gelu(layer1 x)),
+    float32 1e-5 / bf16 2e-2) and bit for bit against linear -> gelu -> linear through the separate operators."""
+    print(f"ffn case: hidden={hidden} ffn={ffn} {dtype}", flush=True)
+    torch.manual_seed(hidden + ffn)
+    m = FeedForwardNetwork(hidden, ffn, 0.0)
+    with torch.no_grad():
+        for p in m.parameters():
+            p.normal_(0, 0.3)
+    m = m.to(dtype)
+    x = torch.randn(3, 333, hidden).to(dtype)
+    dy = torch.randn(3, 333, hidden).to(dtype)
+    pd = {k: v.detach().double().numpy() for k, v in m.named_parameters()}
+    want = E.gelu(x.double().numpy() @ pd["layer1.weight"].T + pd["layer1.bias"]) @ pd["layer2.weight"].T + pd["layer2.bias"]
+    mc = m.to(cuda)
+    xc = x.to(cuda).requires_grad_(True)
+    got = mc(xc)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    assert np.abs(got.detach().double().cpu().numpy() - want).max() <= tol * np.abs(want).max()
+    grads = torch.autograd.grad(got, [xc] + list(mc.parameters()), dy.to(cuda))
+    xs = x.to(cuda).requires_grad_(True)
+    (u,) = fused_linear(xs, mc.layer1)
+    (ys,) = fused_linear(GeluFunction.apply(u), mc.layer2)
+    assert torch.equal(got, ys)
+    for a, b in zip(grads, torch.autograd.grad(ys, [xs] + list(mc.parameters()), dy.to(cuda))):
+        assert torch.equal(a, b)
+    # gradients against torch autograd of the same composition in float64 on the CPU
+    md = FeedForwardNetwork(hidden, ffn, 0.0).double()
+    md.load_state_dict({k: v.double() for k, v in m.state_dict().items()})
+    xd = x.double().requires_grad_(True)
+    yd = torch.nn.functional.linear(torch.nn.functional.gelu(torch.nn.functional.linear(xd, md.layer1.weight, md.layer1.bias)),
+                                    md.layer2.weight, md.layer2.bias)
+    for a, b in zip(grads, torch.autograd.grad(yd, [xd] + list(md.parameters()), dy.double())):
+        assert (a.double().cpu() - b).abs().max() <= tol * b.abs().max()
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

@@ -14,6 +14,7 @@
 //   torchgt::add(x, r) -> sum
 //   torchgt::gelu(u) / torchgt::relu(u) -> h
 //   torchgt::nll_loss(log_probs, target, ignore_index) -> loss                (mean over the rows that count)
+//   torchgt::ffn(x, W1, b1, W2, b2) -> layer2(gelu(layer1(x)))
 #include <torch/library.h>
 #include <torch/custom_class.h>
 #include <torch/autograd.h>
@@ -619,6 +620,45 @@ void lin_gelu_bwd(const Tensor& h, const Tensor& W, const Tensor& dy, const Tens
 }
 }  // namespace layer
 
+// FeedForwardNetwork.forward (models/graphormer_dist_node_level.py:35-39): layer2(gelu(layer1(x))) as one operator and
+// one autograd node: the activation rides on the linears and the two sums of weight-gradient partials share a launch.
+struct FfnFn : public torch::autograd::Function<FfnFn> {
+    static Tensor forward(AutogradContext* ctx, Tensor x, Tensor W1, Tensor b1, Tensor W2, Tensor b2) {
+        on_gpu(x, "ffn");
+        const int64_t C = x.size(-1);
+        for (const Tensor* t : {&W1, &b1, &W2, &b2})
+            TORCH_CHECK(t->defined() && t->is_cuda() && t->scalar_type() == x.scalar_type(), "ffn: parameters must be GPU tensors of x's dtype");
+        TORCH_CHECK(W1.dim() == 2 && W1.size(1) == C && W2.dim() == 2 && W2.size(1) == W1.size(0) && b1.numel() == W1.size(0) &&
+                    b2.numel() == W2.size(0), "ffn: weight shapes do not chain");
+        c10::DeviceGuard guard(x.device());
+        Tensor x2 = x.reshape({-1, C}).contiguous(), w1 = W1.contiguous(), w2 = W2.contiguous(), c1 = b1.contiguous(), c2 = b2.contiguous();
+        Tensor u, h;
+        std::vector<Tensor> f;
+        layer::lin_gelu_fwd(x2, w1, c1, u, h);
+        layer::lin_fwd(h, {&w2}, {&c2}, f);
+        ctx->save_for_backward({x2, u, h, w1, w2});
+        std::vector<int64_t> shape = x.sizes().vec();
+        shape.back() = w2.size(0);
+        return f[0].view(shape);
+    }
+    static variable_list backward(AutogradContext* ctx, variable_list grads) {
+        auto sv = ctx->get_saved_variables();
+        const Tensor &x2 = sv[0], &u = sv[1], &h = sv[2], &w1 = sv[3], &w2 = sv[4];
+        c10::DeviceGuard guard(x2.device());
+        Tensor d_f = grads[0].reshape({x2.size(0), w2.size(0)}).contiguous();
+        Tensor du, dx;
+        std::vector<Tensor> dW2, db2, dW1, db1;
+        layer::Deferred later;
+        layer::lin_gelu_bwd(h, w2, d_f, u, du, dW2, db2, later);
+        layer::lin_bwd(x2, {&w1}, {&du}, dx, dW1, db1, later);
+        later.run(dtype_code(x2), stream_of(x2));
+        std::vector<int64_t> shape = grads[0].sizes().vec();
+        shape.back() = x2.size(1);
+        return {dx.view(shape), dW1[0], db1[0], dW2[0], db2[0]};
+    }
+};
+Tensor ffn(const Tensor& x, const Tensor& W1, const Tensor& b1, const Tensor& W2, const Tensor& b2) { return FfnFn::apply(x, W1, b1, W2, b2); }
+
 struct EncoderLayerFn : public torch::autograd::Function<EncoderLayerFn> {
     static variable_list forward(AutogradContext* ctx, Tensor x, c10::optional<Tensor> residual, at::TensorList P,
                                  c10::intrusive_ptr<PlanHolder> holder, Tensor ws, int64_t H, double eps1, double eps2) {
@@ -871,6 +911,7 @@ TORCH_LIBRARY(torchgt, m) {
     m.def("gelu(Tensor u) -> Tensor");
     m.def("relu(Tensor u) -> Tensor");
     m.def("nll_loss(Tensor log_probs, Tensor target, int ignore_index=-100) -> Tensor");
+    m.def("ffn(Tensor x, Tensor W1, Tensor b1, Tensor W2, Tensor b2) -> Tensor");
 }
 
 // One implementation per op, registered for every backend and for autograd alike: each is an autograd function
@@ -888,4 +929,5 @@ TORCH_LIBRARY_IMPL(torchgt, CompositeImplicitAutograd, m) {
     m.impl("gelu", gelu);
     m.impl("relu", relu);
     m.impl("nll_loss", nll_loss);
+    m.impl("ffn", ffn);
 }
