@@ -59,7 +59,7 @@ def test_torch_extension_loads_and_registers_its_operators():
     from torchgt_amd import _ext
     ops = _ext.ops()
     for name in ("sparse_attention", "dense_attention", "dense_attention_ids", "linear", "add_layer_norm", "add", "gelu", "relu",
-                 "ffn", "nll_loss", "encoder_layer", "dense_encoder_layer"):
+                 "ffn", "nll_loss", "multi_head_attention", "encoder_layer", "dense_encoder_layer"):
         assert hasattr(ops, name), name
     assert hasattr(torch.classes.torchgt, "PlanHolder")
     with pytest.raises(RuntimeError, match="GPU"):

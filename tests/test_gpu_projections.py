@@ -12,7 +12,7 @@ import pytest
 import torch
 
 from oracle import projections as P
-from torchgt_amd import MultiHeadAttention, _lib, fused_linear, workloads
+from torchgt_amd import MultiHeadAttention, _lib, fused_linear, get_plan, workloads
 from torchgt_amd.multi_head_attention import LinearFunction
 
 pytestmark = pytest.mark.gpu
@@ -260,6 +260,31 @@ def test_module_matches_oracle_and_reference_state_dict(cuda, dtype):
         else:
             e = err(a, r.numpy())
         assert e <= tol, f"d{nm} err {e}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("with_output_layer", [True, False])
+def test_module_as_one_operator_equals_operator_by_operator(cuda, dtype, with_output_layer):
+    """torch.ops.torchgt.multi_head_attention (projections, sparse attention, output layer: one operator, one autograd
+    node, one launch for the weight-gradient sums) gives the bits of the three operators one after the other."""
+    torch.manual_seed(3)
+    e, n_nodes = workloads.barabasi_albert()
+    ei = torch.as_tensor(e).to(cuda)
+    m = (MultiHeadAttention(64, 0.0, 8, 1) if with_output_layer else MultiHeadAttention(64, 0.0, 8)).to(cuda, dtype)
+    x = torch.randn(1, n_nodes, 64, device=cuda).to(dtype)
+    gy = torch.randn(1, n_nodes, 64, device=cuda).to(dtype)
+    results = []
+    for one in (True, False):
+        m.one_operator = one
+        xc = x.clone().requires_grad_(True)
+        y = m(xc, None, ei, "sparse")
+        results.append([y] + list(torch.autograd.grad(y, [xc] + list(m.parameters()), gy)))
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+    # rows that do not match the plan are refused before any kernel runs
+    m.one_operator = True
+    with pytest.raises(RuntimeError, match="plan was built for"):
+        m(x[:, :-1], None, get_plan(ei, n_nodes), "sparse")
 
 
 def test_module_without_output_layer(cuda):

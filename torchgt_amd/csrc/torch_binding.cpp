@@ -15,6 +15,7 @@
 //   torchgt::gelu(u) / torchgt::relu(u) -> h
 //   torchgt::nll_loss(log_probs, target, ignore_index) -> loss                (mean over the rows that count)
 //   torchgt::ffn(x, W1, b1, W2, b2) -> layer2(gelu(layer1(x)))
+//   torchgt::multi_head_attention(x, params[6 | 8], plan holder, workspace, heads) -> y     (sparse attention, no bias)
 #include <torch/library.h>
 #include <torch/custom_class.h>
 #include <torch/autograd.h>
@@ -55,6 +56,13 @@ struct PlanHolder : torch::CustomClassHolder {
     int64_t handle() const { return h; }
 };
 
+// the attention entry points take the number of rows from the plan: tensors of another length must not reach them
+void rows_match_plan(const c10::intrusive_ptr<PlanHolder>& holder, int64_t N, const char* op) {
+    int64_t info[16];
+    check(tgt_plan_info(reinterpret_cast<const tgt_plan_t*>(holder->h), info), "tgt_plan_info");
+    TORCH_CHECK(info[0] == N, op, ": ", N, " rows, but the plan was built for ", info[0], " nodes");
+}
+
 // ---------------------------------------------------------------------------------------------------------------
 // sparse attention
 // ---------------------------------------------------------------------------------------------------------------
@@ -73,6 +81,7 @@ struct SparseAttention : public torch::autograd::Function<SparseAttention> {
             b = bias->contiguous();
         }
         const int64_t N = q.size(0), H = q.size(1), d = q.size(2);
+        rows_match_plan(holder, N, "sparse_attention");
         c10::DeviceGuard guard(q.device());
         Tensor out = at::empty_like(q);
         Tensor Z = at::empty({N, H}, q.options().dtype(at::kFloat));
@@ -659,6 +668,73 @@ struct FfnFn : public torch::autograd::Function<FfnFn> {
 };
 Tensor ffn(const Tensor& x, const Tensor& W1, const Tensor& b1, const Tensor& W2, const Tensor& b2) { return FfnFn::apply(x, W1, b1, W2, b2); }
 
+// MultiHeadAttention.forward with sparse attention and no bias (models/graphormer_dist_node_level.py:246-273; the GT
+// flavour of gt_dist_node_level.py:186-216 has no output layer) as one operator and one autograd node:
+// q, k, v = x W^T + b from one kernel, the attention, the output layer; the backward ends with one launch for both
+// sums of weight-gradient partials.  P: Wq, bq, Wk, bk, Wv, bv (, Wo, bo).
+struct MhaFn : public torch::autograd::Function<MhaFn> {
+    static Tensor forward(AutogradContext* ctx, Tensor x, at::TensorList P, c10::intrusive_ptr<PlanHolder> holder, Tensor ws, int64_t H) {
+        on_gpu(x, "multi_head_attention");
+        TORCH_CHECK(P.size() == 6 || P.size() == 8, "multi_head_attention takes 6 parameter tensors, or 8 with an output layer");
+        for (const Tensor& t : P) TORCH_CHECK(t.defined() && t.is_cuda() && t.scalar_type() == x.scalar_type(), "parameters must be GPU tensors of x's dtype");
+        const int64_t C = x.size(-1), HD = P[0].size(0);
+        TORCH_CHECK(HD % H == 0, "projection width ", HD, " is not a multiple of ", H, " heads");
+        std::vector<Tensor> p;
+        for (const Tensor& t : P) p.push_back(t.contiguous());
+        c10::DeviceGuard guard(x.device());
+        Tensor x2 = x.reshape({-1, C}).contiguous();
+        const int64_t N = x2.size(0), d = HD / H;
+        rows_match_plan(holder, N, "multi_head_attention");
+        std::vector<Tensor> qkv, y;
+        layer::lin_fwd(x2, {&p[0], &p[2], &p[4]}, {&p[1], &p[3], &p[5]}, qkv);
+        Tensor o = at::empty_like(qkv[0]), Z = at::empty({N, H}, x.options().dtype(at::kFloat));
+        check(tgt_sparse_attn_fwd(reinterpret_cast<const tgt_plan_t*>(holder->h), qkv[0].data_ptr(), qkv[1].data_ptr(), qkv[2].data_ptr(), nullptr,
+                                  TGT_BIAS_NONE, (int)H, (int)d, dtype_code(x), o.data_ptr(), Z.data_ptr<float>(), ws.data_ptr(), ws.numel(),
+                                  stream_of(x)),
+              "tgt_sparse_attn_fwd");
+        const bool has_o = p.size() == 8;
+        if (has_o) layer::lin_fwd(o, {&p[6]}, {&p[7]}, y);
+        std::vector<Tensor> save{x2, qkv[0], qkv[1], qkv[2], o, Z, ws};
+        save.insert(save.end(), p.begin(), p.end());
+        ctx->save_for_backward(save);
+        ctx->saved_data["plan"] = holder;
+        ctx->saved_data["H"] = H;
+        std::vector<int64_t> shape = x.sizes().vec();
+        shape.back() = has_o ? p[6].size(0) : HD;
+        return (has_o ? y[0] : o).view(shape);
+    }
+    static variable_list backward(AutogradContext* ctx, variable_list grads) {
+        auto sv = ctx->get_saved_variables();
+        const Tensor &x2 = sv[0], &q = sv[1], &k = sv[2], &v = sv[3], &o = sv[4], &Z = sv[5], &ws = sv[6];
+        const Tensor* p = &sv[7];
+        const bool has_o = sv.size() == 7 + 8;
+        const int64_t N = x2.size(0), H = ctx->saved_data["H"].toInt(), d = q.size(1) / H;
+        c10::DeviceGuard guard(x2.device());
+        const int code = dtype_code(x2);
+        Tensor dy = grads[0].reshape({N, -1}).contiguous(), do_, dx;
+        std::vector<Tensor> dWo, dbo, dWqkv, dbqkv;
+        layer::Deferred later;
+        if (has_o) layer::lin_bwd(o, {&p[6]}, {&dy}, do_, dWo, dbo, later);
+        else do_ = dy;
+        Tensor dq = at::empty_like(q), dk = at::empty_like(k), dv = at::empty_like(v);
+        check(tgt_sparse_attn_bwd(reinterpret_cast<const tgt_plan_t*>(ctx->saved_data["plan"].toCustomClass<PlanHolder>()->h), q.data_ptr(),
+                                  k.data_ptr(), v.data_ptr(), nullptr, TGT_BIAS_NONE, (int)H, (int)d, code, o.data_ptr(), Z.data_ptr<float>(),
+                                  do_.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), nullptr, ws.data_ptr(), ws.numel(), stream_of(q)),
+              "tgt_sparse_attn_bwd");
+        layer::lin_bwd(x2, {&p[0], &p[2], &p[4]}, {&dq, &dk, &dv}, dx, dWqkv, dbqkv, later);
+        later.run(code, stream_of(x2));
+        std::vector<int64_t> shape = grads[0].sizes().vec();
+        shape.back() = x2.size(1);
+        variable_list out{dx.view(shape), dWqkv[0], dbqkv[0], dWqkv[1], dbqkv[1], dWqkv[2], dbqkv[2]};
+        if (has_o) { out.push_back(dWo[0]); out.push_back(dbo[0]); }
+        for (int i = 0; i < 3; ++i) out.push_back(Tensor());
+        return out;
+    }
+};
+Tensor multi_head_attention(const Tensor& x, at::TensorList params, const c10::intrusive_ptr<PlanHolder>& plan, const Tensor& ws, int64_t H) {
+    return MhaFn::apply(x, params, plan, ws, H);
+}
+
 struct EncoderLayerFn : public torch::autograd::Function<EncoderLayerFn> {
     static variable_list forward(AutogradContext* ctx, Tensor x, c10::optional<Tensor> residual, at::TensorList P,
                                  c10::intrusive_ptr<PlanHolder> holder, Tensor ws, int64_t H, double eps1, double eps2) {
@@ -673,6 +749,7 @@ struct EncoderLayerFn : public torch::autograd::Function<EncoderLayerFn> {
         Tensor x2 = x.reshape({-1, C}).contiguous(), r2;
         if (residual.has_value() && residual->defined()) r2 = residual->reshape({-1, C}).contiguous();
         const int64_t N = x2.size(0), d = C / H;
+        rows_match_plan(holder, N, "encoder_layer");
         Tensor s1, y1, mean1, rstd1, s2, y2, mean2, rstd2;
         std::vector<Tensor> qkv, a, u, f;
         layer::ln_fwd(x2, r2, p[0], p[1], eps1, s1, y1, mean1, rstd1);
@@ -912,6 +989,7 @@ TORCH_LIBRARY(torchgt, m) {
     m.def("relu(Tensor u) -> Tensor");
     m.def("nll_loss(Tensor log_probs, Tensor target, int ignore_index=-100) -> Tensor");
     m.def("ffn(Tensor x, Tensor W1, Tensor b1, Tensor W2, Tensor b2) -> Tensor");
+    m.def("multi_head_attention(Tensor x, Tensor[] params, __torch__.torch.classes.torchgt.PlanHolder plan, Tensor workspace, int heads) -> Tensor");
 }
 
 // One implementation per op, registered for every backend and for autograd alike: each is an autograd function
@@ -930,4 +1008,5 @@ TORCH_LIBRARY_IMPL(torchgt, CompositeImplicitAutograd, m) {
     m.impl("relu", relu);
     m.impl("nll_loss", nll_loss);
     m.impl("ffn", ffn);
+    m.impl("multi_head_attention", multi_head_attention);
 }

@@ -188,5 +188,6 @@ class Graphormer(nn.Module):
                                         residual=pending, defer_residual=True)
         fl = self.final_ln
         _, output = AddLayerNormFunction.apply(output, pending, fl.weight, fl.bias, fl.eps)
-        (output,) = fused_linear(output[0, 1:, :], self.downstream_out_proj)
+        # rows 1.. of graph 0 (:391 `output[0, 1:, :]`); through a view, so that autograd pads the gradient once, not twice
+        (output,) = fused_linear(output.reshape(-1, self.hidden_dim)[1:output.shape[1]], self.downstream_out_proj)
         return F.log_softmax(output, dim=1)

@@ -17,6 +17,7 @@ import torch.nn as nn
 
 from . import _ext, _lib
 from .core_attention import CoreAttention
+from .plan import GraphPlan, get_plan
 
 _DT = {torch.float32: _lib.DTYPE_F32, torch.bfloat16: _lib.DTYPE_BF16}
 
@@ -93,7 +94,28 @@ class MultiHeadAttention(nn.Module):
             self.output_layer = None
         self.dist_attn = _LocalAttention(local_attn)
 
+    one_operator = True      # False: always run projections and attention operator by operator
+
+    def _one_operator(self, x, attn_bias, edge_index, attn_type):
+        """Whether ``torch.ops.torchgt.multi_head_attention`` covers this call: sparse attention without a bias, feature
+        widths the kernels read without padding, every layer with its bias."""
+        if not self.one_operator or attn_type != "sparse" or attn_bias is not None or edge_index is None or not x.is_cuda:
+            return False
+        ve = 4 if x.dtype == torch.float32 else 8
+        layers = [self.linear_q, self.linear_k, self.linear_v] + ([] if self.output_layer is None else [self.output_layer])
+        return all(l.bias is not None and l.in_features % ve == 0 and l.out_features % ve == 0 for l in layers)
+
     def forward(self, x, attn_bias=None, edge_index=None, attn_type=None):
+        if self._one_operator(x, attn_bias, edge_index, attn_type):
+            # projections, attention and output layer as one operator and one autograd node: the same kernels and
+            # numbers, without the per-operator cost of dispatcher and autograd between the launches
+            plan = edge_index if isinstance(edge_index, GraphPlan) else get_plan(edge_index, x.numel() // x.shape[-1])
+            params = [self.linear_q.weight, self.linear_q.bias, self.linear_k.weight, self.linear_k.bias, self.linear_v.weight,
+                      self.linear_v.bias]
+            if self.output_layer is not None:
+                params += [self.output_layer.weight, self.output_layer.bias]
+            plan.handle      # raises if the plan was closed
+            return _ext.ops().multi_head_attention(x, params, plan.holder, plan.workspace(self.num_heads, self.att_size), self.num_heads)
         batch_size = x.size(0)
         q, k, v = fused_linear(x, self.linear_q, self.linear_k, self.linear_v)
         q = q.view(batch_size, -1, self.num_heads, self.att_size)
