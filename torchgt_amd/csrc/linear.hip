@@ -684,11 +684,11 @@ __global__ __launch_bounds__(kThreads) void k_linear_gradw(GradWArgs a) {
 // rows; for each it forms the panel of dx = sum_j dy_j W_j (weights resident in LDS, transposed) and adds
 // dy_j^T x and the column sums of dy_j to the 64 x 64 weight-gradient tiles it keeps in registers; at its end it
 // writes one partial like k_linear_gradw (the fixed-order sum of reduce.hip adds them).  dy is read once instead of twice and
-// one launch replaces two.  Wave w owns the 32 x 32 block (w/2, w%2) of the dx panel and of every dW_j.
-//   float32: dy and x tiles stay in their natural [node][feature] layout; the products over nodes read them with
-//            4-byte LDS accesses (the 32x32x2 instruction takes one value per lane and operand).
-//   bf16:    the products over nodes need the node index contiguous: dy and x are also scattered into transposed
+// one launch replaces two.
+//   bf16 (k_linear64_bwd, four waves): wave w owns the 32 x 32 block (w/2, w%2) of the dx panel and of every dW_j;
+//            the products over nodes need the node index contiguous: dy and x are also scattered into transposed
 //            tiles, as in k_linear_gradw.
+//   float32 (k_linear64_bwd_split, eight waves): see there.
 // ---------------------------------------------------------------------------
 struct Bwd64Args {
     const void* x;         // [N, 64]
@@ -701,8 +701,8 @@ struct Bwd64Args {
 };
 
 template <typename T, int NW> constexpr size_t bwd64_lds_bytes() {
-    // W^T and natural dy per weight; float32: natural x; bf16: transposed dy per weight and transposed x
-    return sizeof(T) * (size_t)64 * lds_stride<T>(64) * (sizeof(T) == 4 ? 2 * NW + 1 : 3 * NW + 1);
+    // W^T, natural dy and transposed dy per weight, transposed x
+    return sizeof(T) * (size_t)64 * lds_stride<T>(64) * (3 * NW + 1);
 }
 
 // ACT (one weight only; 1 = GELU, 2 = RELU): the layer's input was x = act(u); what leaves in dx is the gradient of u,
@@ -710,31 +710,24 @@ template <typename T, int NW> constexpr size_t bwd64_lds_bytes() {
 template <typename T, int NW, int ACT = 0>
 __global__ __launch_bounds__(kThreads) void k_linear64_bwd(Bwd64Args a) {
     static_assert(ACT == 0 || NW == 1, "the activation rides on a backward with one weight");
+    static_assert(sizeof(T) == 2, "float32 takes k_linear64_bwd_split");
     constexpr int S = lds_stride<T>(64);
-    constexpr bool F32 = sizeof(T) == 4;
     extern __shared__ __align__(16) unsigned char smem[];
     T* tW = reinterpret_cast<T*>(smem);            // [NW][64 k][S]: W_j transposed, contraction index m contiguous
     T* tD = tW + NW * 64 * S;                      // [NW][64 nodes][S]: dy_j as in memory
-    T* tX = tD + NW * 64 * S;                      // float32: [64 nodes][S] x as in memory; bf16: [64 k][S] x transposed
-    T* tDt = tX + 64 * S;                          // bf16 only: [NW][64 m][S] dy_j transposed
+    T* tX = tD + NW * 64 * S;                      // [64 k][S]: x transposed
+    T* tDt = tX + 64 * S;                          // [NW][64 m][S]: dy_j transposed
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, h = lane >> 5;
     const int rb = wave >> 1, cb = wave & 1;
     const int64_t n_panels = (a.N + 63) / 64;
     const T* X = reinterpret_cast<const T*>(a.x);
-    // a panel on its way from memory: natural pieces for float32, the transposing piece order for bf16 (a piece is
-    // written to the natural tile as it is and scattered into the transposed one)
-    TileRegs<T> nx_n, nd_n[NW];
+    // a panel on its way from memory, in the transposing piece order (a piece is written to the natural tile as it
+    // is and scattered into the transposed one)
     PieceRegs<T> nx_p, nd_p[NW];
     auto fetch = [&](int64_t p) {
-        if constexpr (F32) {
-            tile_fetch(nx_n, X, p * 64, a.N);
+        fetch_t(nx_p, X, 64, p * 64, a.N, 0, 64);
 #pragma unroll
-            for (int j = 0; j < NW; ++j) tile_fetch(nd_n[j], reinterpret_cast<const T*>(a.dy[j]), p * 64, a.N);
-        } else {
-            fetch_t(nx_p, X, 64, p * 64, a.N, 0, 64);
-#pragma unroll
-            for (int j = 0; j < NW; ++j) fetch_t(nd_p[j], reinterpret_cast<const T*>(a.dy[j]), 64, p * 64, a.N, 0, 64);
-        }
+        for (int j = 0; j < NW; ++j) fetch_t(nd_p[j], reinterpret_cast<const T*>(a.dy[j]), 64, p * 64, a.N, 0, 64);
     };
     int64_t p = blockIdx.x;
     if (p < n_panels) fetch(p);
@@ -746,18 +739,8 @@ __global__ __launch_bounds__(kThreads) void k_linear64_bwd(Bwd64Args a) {
     float colsum = 0.f;
     for (; p < n_panels; p += gridDim.x) {
         __syncthreads();                 // the previous panel has been read
-        if constexpr (F32) {
+        {
             // rows past the end of the batch must read as zero here: they enter the sums over nodes
-            constexpr int VE = 4, VPR = 64 / VE, NV = (int)(sizeof(TileRegs<T>) / 16);
-#pragma unroll
-            for (int i = 0; i < NV; ++i) {
-                const int v = threadIdx.x + i * kThreads, r = v / VPR, c = (v % VPR) * VE;
-                const bool in = p * 64 + r < a.N;
-                *reinterpret_cast<uint4*>(tX + r * S + c) = zero_unless(in, nx_n.v[i]);
-#pragma unroll
-                for (int j = 0; j < NW; ++j) *reinterpret_cast<uint4*>(tD + j * 64 * S + r * S + c) = zero_unless(in, nd_n[j].v[i]);
-            }
-        } else {
             constexpr int NV = (int)(sizeof(PieceRegs<T>) / 16);
             put_t<T, S>(nx_p, tX, p * 64, a.N, 0, 64);
 #pragma unroll
@@ -796,32 +779,16 @@ __global__ __launch_bounds__(kThreads) void k_linear64_bwd(Bwd64Args a) {
             store_rows<T>(out, 64, acc, 0.f, a.N - (p * 64 + 32 * rb + 4 * h));
         }
         // dW_j block (m = 32 rb + ., k = 32 cb + .): contraction over the 64 nodes of the panel
-        if constexpr (F32) {
-            const float* ap = tD + (32 * h) * S + 32 * rb + l32;      // dy_j[node 32 h + i][m], weight j at + j * 64 * S
-            const float* bp = tX + (32 * h) * S + 32 * cb + l32;      // x[node 32 h + i][k]
-#pragma unroll 8
-            for (int i = 0; i < 32; ++i) {
-                const float xv = bp[i * S];
-#pragma unroll
-                for (int j = 0; j < NW; ++j)
-                    accw[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(ap[j * 64 * S + i * S], xv, accw[j], 0, 0, 0);
-            }
-        } else {
+        {
             const T* bp = tX + (32 * cb + l32) * S + h * 32;
 #pragma unroll
             for (int j = 0; j < NW; ++j) Mma<T, 64>::run(tDt + j * 64 * S + (32 * rb + l32) * S + h * 32, bp, accw[j]);
         }
         if (wave < NW) {      // wave j adds up the columns of dy_j: lane = column
             float sacc = 0.f;
-            if constexpr (F32) {
-                const float* col = tD + wave * 64 * S + lane;
+            const T* row = tDt + wave * 64 * S + lane * S;
 #pragma unroll 16
-                for (int i = 0; i < 64; ++i) sacc += col[i * S];
-            } else {
-                const T* row = tDt + wave * 64 * S + lane * S;
-#pragma unroll 16
-                for (int i = 0; i < 64; ++i) sacc += ld1(row + i);
-            }
+            for (int i = 0; i < 64; ++i) sacc += ld1(row + i);
             colsum += sacc;
         }
     }
@@ -837,6 +804,187 @@ __global__ __launch_bounds__(kThreads) void k_linear64_bwd(Bwd64Args a) {
         }
     }
     if (wave < NW) mine[wave * per + 64 * 64 + lane] = colsum;
+}
+
+// float32: the same pass with eight waves and the three-way bf16 split of k_linear64_split.  With the float32 matrix
+// instructions this backward is bound by their rate (the two products of the q/k/v backward are 3.1 GFLOP: 20 us at
+// the peak), and splitting the operands in the wave that multiplies them only trades matrix time for vector time.
+// Here waves 0-3 form the dx panel (and the column sums) and waves 4-7 the weight-gradient blocks, both from the same
+// staged tiles, so every SIMD holds one wave of each kind: while one splits its operands on the vector ALU the other
+// runs its products.  W_j^T sits in LDS as three bf16 planes (split once per workgroup); dy and x stay float32 in
+// their natural [node][feature] layout: the dx waves read their rows of dy (contraction over features, contiguous),
+// the dW waves gather eight nodes of one column per product (contraction over nodes) and split them in registers.
+// Six v_mfma_f32_32x32x16_bf16 per 16 contraction indices as in the forward: the float32 product to a few 2^-23.
+constexpr int kThreads8 = 512;
+
+template <int NW> constexpr size_t bwd64_split_lds_bytes() {
+    return (size_t)NW * 3 * kPlaneElems * sizeof(__bf16) + sizeof(float) * (size_t)(NW + 1) * 64 * lds_stride<float>(64);
+}
+
+struct Split8 { bf16x8_t hi, mid, lo; };
+// eight floats at p[0], p[stride], ...: one column of eight consecutive node rows
+__device__ __forceinline__ void gather_split(Split8& f, const float* p, int stride) {
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = p[i * stride];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        __bf16 a, b, c;
+        split3(v[i], a, b, c);
+        f.hi[i] = a; f.mid[i] = b; f.lo[i] = c;
+    }
+}
+
+template <int NW, int ACT = 0>
+__global__ __launch_bounds__(kThreads8, NW == 1 && ACT == 0 ? 4 : 2) void k_linear64_bwd_split(Bwd64Args a) {
+    // one weight: two workgroups per CU (128 registers); with the activation's erf and exp that would spill: one
+    static_assert(ACT == 0 || NW == 1, "the activation rides on a backward with one weight");
+    constexpr int S = lds_stride<float>(64);
+    extern __shared__ __align__(16) unsigned char smem[];
+    __bf16* tW = reinterpret_cast<__bf16*>(smem);                                            // [NW][3][64 k][kPlaneStride]: W_j^T planes
+    float* tD = reinterpret_cast<float*>(smem + (size_t)NW * 3 * kPlaneElems * sizeof(__bf16));   // [NW][64 nodes][S]: dy_j as in memory
+    float* tX = tD + NW * 64 * S;                                                            // [64 nodes][S]: x as in memory
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, h = lane >> 5;
+    const int role = wave >> 2, w4 = wave & 3, rb = w4 >> 1, cb = w4 & 1;
+    const int64_t n_panels = (a.N + 63) / 64;
+    const float* X = reinterpret_cast<const float*>(a.x);
+    constexpr int NV = 64 * 64 * 4 / (16 * kThreads8);      // 16-byte pieces of a tile per thread: 2
+    uint4 nx[NV], nd[NW][NV];
+    auto fetch = [&](int64_t p) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int v = threadIdx.x + i * kThreads8, r = v >> 4, c = (v & 15) * 4;
+            nx[i] = load16_clamped(X, 64, p * 64 + r, a.N, c, 64);
+#pragma unroll
+            for (int j = 0; j < NW; ++j) nd[j][i] = load16_clamped(reinterpret_cast<const float*>(a.dy[j]), 64, p * 64 + r, a.N, c, 64);
+        }
+    };
+    int64_t p = blockIdx.x;
+    if (p < n_panels) fetch(p);
+    {   // weights: W_j[m][k] goes to plane row k, contraction index m, split into the three planes
+        uint4 raw[NW][NV];
+#pragma unroll
+        for (int j = 0; j < NW; ++j)
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int v = threadIdx.x + i * kThreads8;
+                raw[j][i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const float*>(a.W[j]) + v * 4);
+            }
+#pragma unroll
+        for (int j = 0; j < NW; ++j)
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int v = threadIdx.x + i * kThreads8, m = v >> 4, k = (v & 15) * 4;
+                const float* e = reinterpret_cast<const float*>(&raw[j][i]);
+                __bf16* plane = tW + (size_t)j * 3 * kPlaneElems;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    __bf16 x0, x1, x2;
+                    split3(e[t], x0, x1, x2);
+                    const int at = (k + t) * kPlaneStride + m;
+                    plane[at] = x0;
+                    plane[kPlaneElems + at] = x1;
+                    plane[2 * kPlaneElems + at] = x2;
+                }
+            }
+    }
+    float16_t accw[NW];
+#pragma unroll
+    for (int j = 0; j < NW; ++j) accw[j] = zero16();
+    float colsum = 0.f;
+    for (; p < n_panels; p += gridDim.x) {
+        __syncthreads();                 // the previous panel has been read
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {   // rows past the end of the batch must read as zero: they enter the sums over nodes
+            const int v = threadIdx.x + i * kThreads8, r = v >> 4, c = (v & 15) * 4;
+            const bool in = p * 64 + r < a.N;
+            *reinterpret_cast<uint4*>(tX + r * S + c) = zero_unless(in, nx[i]);
+#pragma unroll
+            for (int j = 0; j < NW; ++j) *reinterpret_cast<uint4*>(tD + j * 64 * S + r * S + c) = zero_unless(in, nd[j][i]);
+        }
+        __syncthreads();
+        if (p + gridDim.x < n_panels) fetch(p + gridDim.x);
+        if (role == 0) {
+            // dx panel: rows = nodes, contraction over m
+            float16_t acc = zero16();
+            float uu[ACT != 0 ? 16 : 1];
+            if constexpr (ACT != 0) {      // u where this lane writes; rows past the end repeat the last row and are not stored
+                const float* U = reinterpret_cast<const float*>(a.u) + 32 * cb + l32;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int64_t row = p * 64 + 32 * rb + 4 * h + 8 * (r >> 2) + (r & 3);
+                    uu[r] = U[(row < a.N ? row : a.N - 1) * 64];
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < NW; ++j) {
+                Split32 d;
+                load_split(d, tD + j * 64 * S + (32 * rb + l32) * S + h * 32);
+                mma_split(d, tW + (size_t)j * 3 * kPlaneElems + (32 * cb + l32) * kPlaneStride + h * 32, acc);
+            }
+            float* out = reinterpret_cast<float*>(a.dx) + (p * 64 + 32 * rb + 4 * h) * 64 + 32 * cb + l32;
+            if constexpr (ACT != 0) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[r] = act_grad<ACT == 2>(uu[r], acc[r]);
+            }
+            store_rows<float>(out, 64, acc, 0.f, a.N - (p * 64 + 32 * rb + 4 * h));
+            if (w4 < NW) {      // wave j adds up the columns of dy_j: lane = column
+                float sacc = 0.f;
+                const float* col = tD + w4 * 64 * S + lane;
+#pragma unroll 16
+                for (int i = 0; i < 64; ++i) sacc += col[i * S];
+                colsum += sacc;
+            }
+        } else {
+            // dW_j block (m = 32 rb + ., k = 32 cb + .): contraction over the 64 nodes of the panel, sixteen per step,
+            // of which this half of the wave takes eight
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n0 = 16 * g + 8 * h;
+                Split8 xs;
+                gather_split(xs, tX + n0 * S + 32 * cb + l32, S);
+#pragma unroll
+                for (int j = 0; j < NW; ++j) {
+                    Split8 ds;
+                    gather_split(ds, tD + j * 64 * S + n0 * S + 32 * rb + l32, S);
+                    accw[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ds.lo, xs.hi, accw[j], 0, 0, 0);     // small terms first
+                    accw[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ds.hi, xs.lo, accw[j], 0, 0, 0);
+                    accw[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ds.mid, xs.mid, accw[j], 0, 0, 0);
+                    accw[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ds.mid, xs.hi, accw[j], 0, 0, 0);
+                    accw[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ds.hi, xs.mid, accw[j], 0, 0, 0);
+                    accw[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ds.hi, xs.hi, accw[j], 0, 0, 0);
+                }
+            }
+        }
+    }
+    constexpr int64_t per = 64 * 64 + 64;
+    float* mine = a.partial + (int64_t)blockIdx.x * NW * per;
+    if (role == 1) {
+#pragma unroll
+        for (int j = 0; j < NW; ++j) {
+            const int k = 32 * cb + l32;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = 32 * rb + 8 * (r >> 2) + 4 * h + (r & 3);
+                mine[j * per + (int64_t)m * 64 + k] = accw[j][r];
+            }
+        }
+    } else if (w4 < NW) {
+        mine[w4 * per + 64 * 64 + lane] = colsum;
+    }
+}
+
+template <int NW, int ACT = 0>
+int launch_bwd64_split(const Bwd64Args& a, int workers, hipStream_t st) {
+    constexpr size_t lds = bwd64_split_lds_bytes<NW>();
+    static bool raised = false;
+    if (!raised && lds > 48 * 1024) {
+        TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_linear64_bwd_split<NW, ACT>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        raised = true;
+    }
+    hipLaunchKernelGGL((k_linear64_bwd_split<NW, ACT>), dim3(workers), dim3(kThreads8), lds, st, a);
+    return TGT_OK;
 }
 
 template <typename T, int NW, int ACT = 0>
@@ -918,10 +1066,12 @@ int linear_bwd_t(const void* d_x, const void* const* d_W, const void* const* d_d
     }
     if (d_dx && d_dW && N > 0 && K == 64 && M == 64) {
         // one pass for dx and the weight gradients
-        constexpr size_t lds1 = bwd64_lds_bytes<T, 1>();
-        const size_t lds = lds1 + (n_out - 1) * (bwd64_lds_bytes<T, 2>() - lds1);
+        constexpr bool split = sizeof(T) == 4;       // float32: eight waves and the bf16 split; bf16: four waves
+        constexpr size_t lds1 = split ? bwd64_split_lds_bytes<1>() : bwd64_lds_bytes<T, 1>();
+        constexpr size_t lds2 = split ? bwd64_split_lds_bytes<2>() : bwd64_lds_bytes<T, 2>();
+        const size_t lds = lds1 + (n_out - 1) * (lds2 - lds1);
         const int64_t n_panels = (N + 63) / 64;
-        const int per_cu = (int)std::max<size_t>(1, std::min<size_t>(2, (size_t)(160 * 1024) / lds));
+        const int per_cu = split && act != 0 ? 1 : (int)std::max<size_t>(1, std::min<size_t>(2, (size_t)(160 * 1024) / lds));
         const int workers = (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(n_panels, grad_workers(K, M)),
                                                                         (int64_t)num_cus() * per_cu));
         Bwd64Args b{};
@@ -930,11 +1080,19 @@ int linear_bwd_t(const void* d_x, const void* const* d_W, const void* const* d_d
         int rc = TGT_OK;
         {
             KernelTimer t(KS_LINEAR_DX, st);
-            if (act == TGT_ACT_GELU) rc = launch_bwd64<T, 1, 1>(b, workers, st);
-            else if (act == TGT_ACT_RELU) rc = launch_bwd64<T, 1, 2>(b, workers, st);
-            else if (n_out == 1) rc = launch_bwd64<T, 1>(b, workers, st);
-            else if (n_out == 2) rc = launch_bwd64<T, 2>(b, workers, st);
-            else rc = launch_bwd64<T, 3>(b, workers, st);
+            if constexpr (split) {
+                if (act == TGT_ACT_GELU) rc = launch_bwd64_split<1, 1>(b, workers, st);
+                else if (act == TGT_ACT_RELU) rc = launch_bwd64_split<1, 2>(b, workers, st);
+                else if (n_out == 1) rc = launch_bwd64_split<1>(b, workers, st);
+                else if (n_out == 2) rc = launch_bwd64_split<2>(b, workers, st);
+                else rc = launch_bwd64_split<3>(b, workers, st);
+            } else {
+                if (act == TGT_ACT_GELU) rc = launch_bwd64<T, 1, 1>(b, workers, st);
+                else if (act == TGT_ACT_RELU) rc = launch_bwd64<T, 1, 2>(b, workers, st);
+                else if (n_out == 1) rc = launch_bwd64<T, 1>(b, workers, st);
+                else if (n_out == 2) rc = launch_bwd64<T, 2>(b, workers, st);
+                else rc = launch_bwd64<T, 3>(b, workers, st);
+            }
         }
         if (rc != TGT_OK) return rc;
         TGT_HIP_CHECK(hipGetLastError());
