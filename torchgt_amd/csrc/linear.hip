@@ -409,21 +409,34 @@ __global__ __launch_bounds__(kThreads) void k_linear64(LinArgs a) {
 }
 
 // ---------------------------------------------------------------------------
-// float32 at the bf16 matrix rate.  A float is the exact sum of three bf16 numbers up to 2^-24 of
-// its size (hi = bf16(x), mid = bf16(x - hi), lo = bf16(x - hi - mid); the subtractions are exact),
-// so x * w = hi*hi + hi*mid + mid*hi + mid*mid + hi*lo + lo*hi + terms below 2^-24: six
-// v_mfma_f32_32x32x16_bf16 (fp32 accumulation) give the float32 product to a few 2^-23, and take 0.4 of
-// the time of the eight v_mfma_f32_32x32x2_f32 they replace (measured on this part: 16.8 ns against
-// 30.4 ns per instruction).  The weights are split once per workgroup into three bf16 planes in LDS;
-// the node rows stay float32 in LDS and are split in registers when a wave loads its operand rows.
+// float32 at the bf16 matrix rate.  A float is the exact sum of three bf16 numbers: hi = its upper 16 bits (sign,
+// exponent, the first 8 bits of the significand), mid = the upper 16 bits of x - hi, lo = x - hi - mid (what is left
+// has at most 8 significant bits; every subtraction is exact).  So x * w = hi*hi + hi*mid + mid*hi + mid*mid + hi*lo +
+// lo*hi + terms below 2^-24: six v_mfma_f32_32x32x16_bf16 (fp32 accumulation) give the float32 product to a few 2^-23,
+// and take 0.4 of the time of the eight v_mfma_f32_32x32x2_f32 they replace (measured on this part: 16.8 ns against
+// 30.4 ns per instruction).  Cutting the words costs four full-rate vector instructions per value and one byte
+// permute per pair and plane; the rounding conversions (v_cvt_pk_bf16_f32) it was first written with run at a quarter
+// of that rate and made the split the longest part of the backward.  The weights are split once per workgroup into
+// three bf16 planes in LDS; the node rows stay float32 in LDS and are split in registers when a wave loads them.
 // ---------------------------------------------------------------------------
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 
-__device__ __forceinline__ void split3(float x, __bf16& hi, __bf16& mid, __bf16& lo) {
-    hi = static_cast<__bf16>(x);
-    const float r1 = x - static_cast<float>(hi);
-    mid = static_cast<__bf16>(r1);
-    lo = static_cast<__bf16>(r1 - static_cast<float>(mid));
+// the three parts as float32 words: each is a bf16 in its upper half (the lower half is zero)
+__device__ __forceinline__ void split3(float x, uint32_t& hi, uint32_t& mid, uint32_t& lo) {
+    hi = __float_as_uint(x) & 0xffff0000u;
+    const float r1 = x - __uint_as_float(hi);
+    mid = __float_as_uint(r1) & 0xffff0000u;
+    lo = __float_as_uint(r1 - __uint_as_float(mid));
+}
+__device__ __forceinline__ __bf16 upper_bf16(uint32_t w) { return __builtin_bit_cast(__bf16, (uint16_t)(w >> 16)); }
+// the upper halves of eight such words as one matrix operand
+__device__ __forceinline__ bf16x8_t pack8(const uint32_t (&w)[8]) {
+    uint4 u;
+    u.x = __builtin_amdgcn_perm(w[1], w[0], 0x07060302u);
+    u.y = __builtin_amdgcn_perm(w[3], w[2], 0x07060302u);
+    u.z = __builtin_amdgcn_perm(w[5], w[4], 0x07060302u);
+    u.w = __builtin_amdgcn_perm(w[7], w[6], 0x07060302u);
+    return __builtin_bit_cast(bf16x8_t, u);
 }
 
 constexpr int kPlaneStride = 72;                       // bf16 per row of a weight plane (64 + 8 of padding)
@@ -438,12 +451,10 @@ __device__ __forceinline__ void load_split(Split32& f, const float* row) {
         const float4 u0 = *reinterpret_cast<const float4*>(row + 8 * t);
         const float4 u1 = *reinterpret_cast<const float4*>(row + 8 * t + 4);
         const float v[8] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
+        uint32_t a[8], b[8], c[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            __bf16 a, b, c;
-            split3(v[i], a, b, c);
-            f.hi[t][i] = a; f.mid[t][i] = b; f.lo[t][i] = c;
-        }
+        for (int i = 0; i < 8; ++i) split3(v[i], a[i], b[i], c[i]);
+        f.hi[t] = pack8(a); f.mid[t] = pack8(b); f.lo[t] = pack8(c);
     }
 }
 
@@ -501,8 +512,9 @@ __global__ __launch_bounds__(kThreads) void k_linear64_split(LinArgs a) {
                 __bf16* plane = tW + (size_t)j * 3 * kPlaneElems;
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
-                    __bf16 x0, x1, x2;
-                    split3(e[t], x0, x1, x2);
+                    uint32_t w0, w1, w2;
+                    split3(e[t], w0, w1, w2);
+                    const __bf16 x0 = upper_bf16(w0), x1 = upper_bf16(w1), x2 = upper_bf16(w2);
                     // forward: plane row = output column r, contraction index c + t; input gradient: row = c + t, index r
                     const int at = DX ? (c + t) * kPlaneStride + r : r * kPlaneStride + c + t;
                     plane[at] = x0;
@@ -827,12 +839,10 @@ __device__ __forceinline__ void gather_split(Split8& f, const float* p, int stri
     float v[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) v[i] = p[i * stride];
+    uint32_t a[8], b[8], c[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        __bf16 a, b, c;
-        split3(v[i], a, b, c);
-        f.hi[i] = a; f.mid[i] = b; f.lo[i] = c;
-    }
+    for (int i = 0; i < 8; ++i) split3(v[i], a[i], b[i], c[i]);
+    f.hi = pack8(a); f.mid = pack8(b); f.lo = pack8(c);
 }
 
 template <int NW, int ACT = 0>
@@ -879,8 +889,9 @@ __global__ __launch_bounds__(kThreads8, NW == 1 && ACT == 0 ? 4 : 2) void k_line
                 __bf16* plane = tW + (size_t)j * 3 * kPlaneElems;
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
-                    __bf16 x0, x1, x2;
-                    split3(e[t], x0, x1, x2);
+                    uint32_t w0, w1, w2;
+                    split3(e[t], w0, w1, w2);
+                    const __bf16 x0 = upper_bf16(w0), x1 = upper_bf16(w1), x2 = upper_bf16(w2);
                     const int at = (k + t) * kPlaneStride + m;
                     plane[at] = x0;
                     plane[kPlaneElems + at] = x1;
