@@ -318,3 +318,37 @@ def test_fused_linear_pads_widths_that_do_not_fit(cuda):
         assert err(y, torch.nn.functional.linear(xd, Wd, bd).detach().numpy()) <= TOL[dtype]
         for a, r in zip(got, ref):
             assert a.shape == r.shape and err(a, r.numpy()) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_linear_at_the_row_count_of_the_largest_configuration(cuda, dtype):
+    """870 001 rows (configs[2]), q/k/v shape: the float64 oracle is out of reach at this size, so the outputs and the
+    input gradient are held against float64 products on a sample of rows, and the weight gradients - sums over all
+    rows - against torch's float64 matmul on the GPU (an independent library routine)."""
+    N, n = 870001, 3
+    print(f"linear at N={N} x{n} {dtype}", flush=True)
+    g = torch.Generator(device="cuda").manual_seed(11)
+    x = torch.randn(N, 64, device=cuda, generator=g).to(dtype).requires_grad_(True)
+    Ws = [(torch.randn(64, 64, device=cuda, generator=g) / 8).to(dtype).requires_grad_(True) for _ in range(n)]
+    bs = [torch.randn(64, device=cuda, generator=g).to(dtype).requires_grad_(True) for _ in range(n)]
+    dys = [torch.randn(N, 64, device=cuda, generator=g).to(dtype) for _ in range(n)]
+    args = []
+    for W, b in zip(Ws, bs):
+        args += [W, b]
+    ys = LinearFunction.apply(x, *args)
+    grads = torch.autograd.grad(ys, [x] + Ws + bs, dys)
+    tol = TOL[dtype]
+    rows = torch.cat([torch.arange(0, 70, device=cuda), torch.randint(0, N, (2000,), device=cuda, generator=g),
+                      torch.arange(N - 70, N, device=cuda)])
+    xd = x.detach().double()
+    dx_ref = 0
+    for j in range(n):
+        Wd, dyd = Ws[j].detach().double(), dys[j].double()
+        y_ref = xd[rows] @ Wd.T + bs[j].detach().double()
+        assert ((ys[j][rows].double() - y_ref).abs().max() / y_ref.abs().max()).item() <= tol
+        dx_ref = dx_ref + dyd[rows] @ Wd
+        dW_ref = dyd.T @ xd
+        assert ((grads[1 + j].double() - dW_ref).abs().max() / dW_ref.abs().max()).item() <= tol
+        db_ref = dyd.sum(0)
+        assert ((grads[1 + n + j].double() - db_ref).abs().max() / db_ref.abs().max()).item() <= tol
+    assert ((grads[0][rows].double() - dx_ref).abs().max() / dx_ref.abs().max()).item() <= tol
