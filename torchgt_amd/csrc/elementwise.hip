@@ -124,32 +124,43 @@ __global__ __launch_bounds__(kEwBlock) void k_layer_norm_bwd(const T* __restrict
     Vec<T>::load(gamma + sub * VE, g);
 #pragma unroll
     for (int i = 0; i < VE; ++i) { dg[i] = 0.f; db[i] = 0.f; }
-    for (int64_t row = (int64_t)blockIdx.x * RPB + slot; row < N; row += (int64_t)gridDim.x * RPB) {
-        float s[VE], d[VE];
-        Vec<T>::load(s_in + row * C + sub * VE, s);
-        Vec<T>::load(dy + row * C + sub * VE, d);
-        const float mean = mean_in[row], rstd = rstd_in[row];
-        float xh[VE], gg[VE], a1 = 0.f, a2 = 0.f;
+    // two rows of the walk per step, all their loads issued before the first is used (a lane has six 16-byte loads
+    // in flight instead of three); the rows enter the column sums in the order of the one-row walk: same bits
+    const int64_t step = (int64_t)gridDim.x * RPB;
+    for (int64_t row0 = (int64_t)blockIdx.x * RPB + slot; row0 < N; row0 += 2 * step) {
+        const bool two = row0 + step < N;
+        const int64_t rows[2] = {row0, two ? row0 + step : row0};
+        float s[2][VE], d[2][VE], t[2][VE], mean[2], rstd[2];
 #pragma unroll
-        for (int i = 0; i < VE; ++i) {
-            xh[i] = (s[i] - mean) * rstd;
-            gg[i] = d[i] * g[i];
-            a1 += gg[i];
-            a2 += gg[i] * xh[i];
-            dg[i] += d[i] * xh[i];
-            db[i] += d[i];
+        for (int u = 0; u < 2; ++u) {
+            Vec<T>::load(s_in + rows[u] * C + sub * VE, s[u]);
+            Vec<T>::load(dy + rows[u] * C + sub * VE, d[u]);
+            mean[u] = mean_in[rows[u]]; rstd[u] = rstd_in[rows[u]];
+            if (extra) Vec<T>::load(extra + rows[u] * C + sub * VE, t[u]);
         }
-        const float m1 = row_sum<LPR>(a1) * (1.f / C), m2 = row_sum<LPR>(a2) * (1.f / C);
-        float o[VE];
 #pragma unroll
-        for (int i = 0; i < VE; ++i) o[i] = rstd * (gg[i] - m1 - xh[i] * m2);
-        if (extra) {
-            float t[VE];
-            Vec<T>::load(extra + row * C + sub * VE, t);
+        for (int u = 0; u < 2; ++u) {
+            if (u == 1 && !two) break;
+            float xh[VE], gg[VE], a1 = 0.f, a2 = 0.f;
 #pragma unroll
-            for (int i = 0; i < VE; ++i) o[i] += t[i];
+            for (int i = 0; i < VE; ++i) {
+                xh[i] = (s[u][i] - mean[u]) * rstd[u];
+                gg[i] = d[u][i] * g[i];
+                a1 += gg[i];
+                a2 += gg[i] * xh[i];
+                dg[i] += d[u][i] * xh[i];
+                db[i] += d[u][i];
+            }
+            const float m1 = row_sum<LPR>(a1) * (1.f / C), m2 = row_sum<LPR>(a2) * (1.f / C);
+            float o[VE];
+#pragma unroll
+            for (int i = 0; i < VE; ++i) o[i] = rstd[u] * (gg[i] - m1 - xh[i] * m2);
+            if (extra) {
+#pragma unroll
+                for (int i = 0; i < VE; ++i) o[i] += t[u][i];
+            }
+            Vec<T>::store(ds + rows[u] * C + sub * VE, o);
         }
-        Vec<T>::store(ds + row * C + sub * VE, o);
     }
 #pragma unroll
     for (int i = 0; i < VE; ++i) {
