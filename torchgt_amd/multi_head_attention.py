@@ -7,8 +7,10 @@ models/graphormer_dist_graph_level.py): same constructor, same parameter names
 ``state_dict`` loads), same ``forward(x, attn_bias, edge_index, attn_type)``.
 The three input projections run as ONE kernel that reads ``x`` once and writes q, k
 and v in the ``[N, H, d]`` layout the attention kernels read; their backward is
-one kernel for ``dx`` and one (plus a small fixed-order reduction) for all three
-weight and bias gradients.  At sequence-parallel size 1 the reference's
+one pass over the three output gradients for ``dx`` and all weight and bias
+gradients (64 -> 64 features; two kernels for other widths) plus a small
+fixed-order sum of per-workgroup partials.  With sparse attention and no bias
+the whole module is one operator (``torch.ops.torchgt.multi_head_attention``).  At sequence-parallel size 1 the reference's
 ``DistributedAttentionNoMerge`` (gt_sp/layer.py:502-550) hands q, k, v to the local
 attention unchanged, which is what ``dist_attn`` does here.
 """
