@@ -352,3 +352,25 @@ def test_linear_at_the_row_count_of_the_largest_configuration(cuda, dtype):
         db_ref = dyd.sum(0)
         assert ((grads[1 + n + j].double() - db_ref).abs().max() / db_ref.abs().max()).item() <= tol
     assert ((grads[0][rows].double() - dx_ref).abs().max() / dx_ref.abs().max()).item() <= tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_module_as_one_operator_on_the_benchmark_graph(cuda, dtype):
+    """The same equality at the size the benchmark runs (configs[1]: 64 001 nodes, ~530 K edges, 1001 panels of rows,
+    256 partial sums per weight): one operator and three operators give the same bits, and the output is finite."""
+    e, n_nodes = workloads.power_law_graph(n=64000, exponent=2.1, directed_edges=530_000, seed=42)
+    print(f"module at N={n_nodes} E={e.shape[1]} {dtype}", flush=True)
+    torch.manual_seed(4)
+    ei = torch.as_tensor(e).to(cuda)
+    m = MultiHeadAttention(64, 0.0, 8, 1).to(cuda, dtype)
+    x = torch.randn(1, n_nodes, 64, device=cuda).to(dtype)
+    gy = torch.randn(1, n_nodes, 64, device=cuda).to(dtype)
+    results = []
+    for one in (True, False):
+        m.one_operator = one
+        xc = x.clone().requires_grad_(True)
+        y = m(xc, None, ei, "sparse")
+        results.append([y] + list(torch.autograd.grad(y, [xc] + list(m.parameters()), gy)))
+    for a, b in zip(*results):
+        assert torch.isfinite(a).all()
+        assert torch.equal(a, b)
