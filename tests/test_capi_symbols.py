@@ -50,6 +50,18 @@ def test_host_only_entry_points():
     assert L.tgt_sparse_attn_workspace_bytes(None, 8, 8) == -1
     assert L.tgt_sparse_attn_fwd(None, None, None, None, None, 0, 8, 8, 0, None, None, None, 0, None) \
         == _lib.ERR_INVALID_ARG
+    # the entry points around the path refuse bad arguments before they touch the GPU as well
+    assert L.tgt_nll_loss_workspace_bytes(-1) == -1 and L.tgt_nll_loss_workspace_bytes(64000) == 8 * 250
+    assert L.tgt_nll_loss_fwd(None, None, -1, 40, 0, -100, None, None, None, 0, None) == _lib.ERR_INVALID_ARG
+    assert L.tgt_nll_loss_fwd(None, None, 10, 40, 7, -100, None, None, None, 0, None) == _lib.ERR_INVALID_ARG      # dtype
+    assert L.tgt_nll_loss_bwd(None, None, None, 0, 40, 0, -100, None, None) == 0                                   # nothing to do
+    assert L.tgt_reduce_partials(None, 0, 0, None) == 0
+    assert L.tgt_reduce_partials(None, 3, 0, None) == _lib.ERR_INVALID_ARG
+    empty = (_lib.ReduceDesc * 2)()
+    assert L.tgt_reduce_partials(empty, 2, 0, None) == _lib.ERR_INVALID_ARG                                        # not filled in
+    assert L.tgt_linear_act_fwd(None, None, None, 16, 64, 64, 0, 0, None, None, None) == _lib.ERR_INVALID_ARG       # activation
+    assert L.tgt_linear_act_bwd(None, None, None, None, 16, 64, 64, 0, 1, None, None, None, None, 0, None, None) == _lib.ERR_INVALID_ARG
+    assert ctypes.sizeof(_lib.ReduceDesc) == 8 + 3 * 4 + 4 + 6 * 8 + 6 * 4                                       # the C struct's layout
 
 
 def test_torch_extension_loads_and_registers_its_operators():
