@@ -159,44 +159,6 @@ def reference_ops_on_gpu(ei, q, k, v, bias, dout, steps=20):
             "what": "reference op chain with stock PyTorch-ROCm kernels (index gathers + index_add_, autograd)"}
 
 
-def gather_probe(plan, n, E, row_bytes, stream, repeats=20):
-    """Rate the memory system sustains for the bare access pattern of the forward walk: the same
-    source rows in the same (destination-sorted) order, k then v (two tables of n rows of
-    row_bytes each), read by the library's row-gather probe kernel: no index chain, no arithmetic,
-    no outputs.  Also the same number of uniformly random rows.  Returns None if the row size
-    has no probe variant."""
-    import torch
-    from torchgt_amd import _lib
-    if row_bytes not in (128, 256):
-        return None
-    dev = torch.device("cuda:0")
-    L = _lib.lib()
-    col = torch.from_numpy(plan.export(_lib.PLAN_COL_DST)).to(dev, torch.int32)
-    idx_real = torch.cat([col, col + n]).contiguous()
-    idx_real = idx_real[: idx_real.numel() // 4 * 4]
-    gen = torch.Generator().manual_seed(7)
-    idx_rand = torch.randint(0, 2 * n, (idx_real.numel(),), generator=gen, dtype=torch.int32).to(dev)
-    table = torch.ones(2 * n * row_bytes // 4, dtype=torch.int32, device=dev)
-    sink = torch.zeros(1, dtype=torch.int32, device=dev)
-    out = {"row_bytes": row_bytes, "table_bytes": 2 * n * row_bytes, "rows_gathered": int(idx_real.numel())}
-    for tag, idx in (("graph_order", idx_real), ("uniform_random", idx_rand)):
-        for _ in range(3):
-            _lib.check(L.tgt_probe_row_gather(table.data_ptr(), 2 * n, row_bytes, idx.data_ptr(), idx.numel(),
-                                              sink.data_ptr(), stream))
-        torch.cuda.synchronize()
-        L.tgt_timing_reset()
-        L.tgt_timing_enable(1)
-        for _ in range(repeats):
-            _lib.check(L.tgt_probe_row_gather(table.data_ptr(), 2 * n, row_bytes, idx.data_ptr(), idx.numel(),
-                                              sink.data_ptr(), stream))
-        torch.cuda.synchronize()
-        L.tgt_timing_enable(0)
-        ms, cnt = _lib.kernel_timings()["probe_row_gather"]
-        us = ms / cnt * 1e3
-        out[tag] = {"avg_us": us, "GB/s": idx.numel() * row_bytes / (us * 1e-6) / 1e9}
-    return out
-
-
 def bench_dense(args):
     """Benchmark configuration configs[3]: dense biased attention on a batch of 256 padded ER graphs (S = 129,
     H = 8, d = 8, bf16, bias [b,H,S,S] with gradient).  A step = tgt_dense_attn_fwd + _bwd."""
@@ -494,8 +456,10 @@ def bench_block(args):
     ms_sparse = timed(step_sparse)
     esize = 2 if args.dtype == "bf16" else 4
     R = H * d * esize
-    # every node row once per pass; a tile is 8 bytes; fp32 tile sums written and read once per pass
-    alg = 12 * n * R + 8 * n * H + 3 * 8 * len(tiles) + 2 * 4 * (n * H * d * 4 + n * H) + 16 * int(raw.shape[1])
+    # compulsory bytes: every node row once per pass (12 N R), Z written and read (8 N H), a tile is 8 bytes and
+    # is read by the forward and by both walks of the backward, 16 bytes of sorted views per remaining edge.  The
+    # fp32 tile sums the hybrid mode passes between its kernels are the implementation's own traffic: not counted.
+    alg = 12 * n * R + 8 * n * H + 3 * 8 * len(tiles) + 16 * int(raw.shape[1])
     result = {
         "metric": "fwd+bwd block attention (16x16 tiles on MFMA + sparse remainder) edges/sec; ms/layer",
         "value": E / (ms_block * 1e-3), "unit": "edges/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -618,6 +582,29 @@ def bench_model(args):
         loss = step()
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) / args.steps * 1e3
+    # The reference's loop moves the CPU-resident edge_index of a pre-packed batch to the GPU in every iteration
+    # (main_sp_sparse_node_level.py:178-183): the same step with a fresh copy each time.  The first such step
+    # finds the plan by its content key; no step builds one.
+    from torchgt_amd import plan as plan_mod
+    ei_cpu = torch.from_numpy(e).pin_memory()
+    builds_before = plan_mod.plan_cache_stats()["builds"]
+
+    def fresh_step():
+        opt.zero_grad(set_to_none=True)
+        out = m(x, None, ei_cpu.to(dev, non_blocking=True), attn_type="sparse")
+        loss = nll_loss(out.float(), y)
+        loss.backward()
+        opt.step()
+
+    for _ in range(3):
+        fresh_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        fresh_step()
+    torch.cuda.synchronize()
+    fresh_ms = (time.perf_counter() - t0) / args.steps * 1e3
+    fresh_builds = plan_mod.plan_cache_stats()["builds"] - builds_before
     L = _lib.lib()
     L.tgt_timing_reset()
     L.tgt_timing_enable(1)
@@ -678,6 +665,8 @@ def bench_model(args):
                    "step": "forward + nll_loss (" + ("torch's" if args.torch_loss else "the library's") + ") + backward + torch AdamW (" + ("foreach" if args.foreach_adamw else "fused") + ")",
                    "parallelism": "1 GPU"},
         "loss": loss_value,
+        "step_with_fresh_edge_index_ms": fresh_ms,
+        "plans_built_by_the_fresh_edge_index_steps": fresh_builds,
         "ms_per_step_hip_graph": graph_ms,
         "library_kernel_us_per_step": lib_us,
         "kernel_groups_us": {g: sum(kernels[k]["avg_us"] * kernels[k]["launches_per_step"] for k in ks if k in kernels)
@@ -796,6 +785,8 @@ def bench_graph_model(args):
                    "parameters": sum(p.numel() for p in m.parameters()),
                    "step": "forward + l1_loss + backward + torch AdamW (" + ("foreach" if args.foreach_adamw else "fused") + ")", "parallelism": "1 GPU"},
         "loss": loss_value,
+        "step_with_fresh_edge_index_ms": fresh_ms,
+        "plans_built_by_the_fresh_edge_index_steps": fresh_builds,
         "ms_per_step_hip_graph": graph_ms,
         "library_kernel_us_per_step": lib_us,
         "kernel_groups_us": {g: sum(kernels[k]["avg_us"] * kernels[k]["launches_per_step"] for k in ks if k in kernels)
@@ -920,7 +911,6 @@ def bench_sparse(args):
                 "mode": "TGT_BIAS_PLAN_ORDER | TGT_BIAS_BOTH_ORDERS"}
 
     plan_order = plan_order_point()
-    probe = gather_probe(plan, n, E, H * d * esize, stream) if not args.brief else None
     bpe = H * esize
     dom = max((kk for kk in kernels if kernel_alg_bytes(kk, n, E, H, d, esize, bpe)),
               key=lambda kk: kernels[kk]["avg_us"])
@@ -949,8 +939,6 @@ def bench_sparse(args):
                      "avg_us": kernels[dom]["avg_us"]},
         "kernels": kernels,
         "bias_in_plan_order": plan_order,
-        # what a bare gather of the forward walk's k and v rows costs (no arithmetic, no index chain)
-        "row_gather_probe": probe,
         "plan_build_ms": plan_ms, "plan_build_first_ms": plan_first_ms,
     }
     if E <= 4_000_000 and not args.no_reference_ops:      # the op chain materialises several [E,H,d] fp32 tensors
@@ -987,7 +975,8 @@ def other_configs(args):
     todo = [("configs[1] bf16", "config2", "bf16", 100, 10), ("configs[2] bf16", "config3", "bf16", 10, 3),
             ("configs[3] bf16 dense", "config4", "bf16", 100, 10), ("configs[4] bf16 sparse path", "config5", "bf16", 50, 5),
             ("configs[4] bf16 hybrid (tiles + remaining edges)", "config5-hybrid", "bf16", 50, 5),
-            ("configs[4] bf16 blockized by the reference's reordering", "config5-blockized", "bf16", 50, 5)]
+            ("configs[4] bf16 blockized by the reference's reordering", "config5-blockized", "bf16", 50, 5),
+            ("configs[1] f32 model step (4-layer Graphormer-Slim)", "config2-model", "f32", 30, 5)]
     for tag, workload, dtype, steps, warmup in todo:
         a = copy.copy(args)
         a.workload, a.dtype, a.steps, a.warmup = workload, dtype, steps, warmup
@@ -1006,7 +995,8 @@ def other_configs(args):
                  "roofline": {kk: roof.get(kk) for kk in ("kernel", "frac", "alg_bytes", "avg_us")},
                  "kernels_avg_us": {kk: round(vv["avg_us"], 2) for kk, vv in r.get("kernels", {}).items()},
                  "seconds_spent": None}
-        for extra in ("bias_in_plan_order", "mfma", "sparse_path_same_edges_ms", "ids_and_tables"):
+        for extra in ("bias_in_plan_order", "mfma", "sparse_path_same_edges_ms", "ids_and_tables", "plan_build_ms",
+                      "step_with_fresh_edge_index_ms", "plans_built_by_the_fresh_edge_index_steps"):
             if extra in r:
                 entry[extra] = r[extra]
         entry["seconds_spent"] = round(time.perf_counter() - t0, 1)

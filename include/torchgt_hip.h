@@ -19,6 +19,7 @@
 #ifndef TORCHGT_HIP_H
 #define TORCHGT_HIP_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -61,6 +62,21 @@ extern "C" {
 
 typedef struct tgt_plan tgt_plan_t;   /* opaque, owns device memory */
 
+/* ---- device memory of the library's own ----------------------------------
+ * Plans, tile sets and the scratch buffers of the edge preparation come from hipMalloc / hipFree
+ * unless the host gives an allocator: `alloc(bytes, stream, user)` returns device memory that is
+ * safe to use on `stream` (NULL on failure), `free_fn(ptr, user)` takes it back and may hand it
+ * out again to later allocations for the same stream while kernels already launched there still
+ * read it (what a stream-ordered caching allocator does).  The PyTorch extension registers torch's
+ * caching allocator when it is loaded, so that building a plan per training iteration - the
+ * reference moves edge_index to the GPU in every iteration, main_sp_sparse_node_level.py:178-183 -
+ * costs no hipMalloc / hipFree (both synchronise the device).  Give both functions, or NULL for
+ * both to return to hipMalloc; memory goes back to the allocator it came from.  No counterpart in
+ * the reference (torch owns all of its memory). */
+typedef void* (*tgt_alloc_fn)(size_t bytes, void* stream, void* user);
+typedef void (*tgt_free_fn)(void* ptr, void* user);
+int tgt_set_allocator(tgt_alloc_fn alloc, tgt_free_fn free_fn, void* user);
+
 int          tgt_version(void);
 const char*  tgt_error_string(int code);
 const char*  tgt_last_error(void);
@@ -78,11 +94,19 @@ const char*  tgt_last_error(void);
  * plan holds a degree-binned row schedule (long rows split into segments).
  *
  * d_src / d_dst: int64 device arrays of length E (edge_index[0], edge_index[1]).
- * Synchronises `stream`.  TGT_ERR_INDEX_RANGE if any endpoint is outside [0,N).
+ * Synchronises `stream` (once; a second time if the graph has rows of more than 256 edges,
+ * a third for the launch descriptors).  TGT_ERR_INDEX_RANGE if any endpoint is outside [0,N).
  */
 int tgt_plan_create(const int64_t* d_src, const int64_t* d_dst, int64_t E, int64_t N,
                     void* stream, tgt_plan_t** out_plan);
 int tgt_plan_destroy(tgt_plan_t* plan);
+/* A 128-bit content key of an edge list (values and their positions), for caches of plans that must
+ * recognise an edge_index they have seen at another address: the reference's training loops move the
+ * same CPU-resident edge_index to the GPU in every iteration (main_sp_sparse_node_level.py:178-183,
+ * gt_sp/utils.py:455-458), and its layers and iterations are meant to share one plan.  Two small
+ * kernels on `stream`, a 16-byte copy to h_key and one synchronisation of the stream; the key does
+ * not depend on the launch shape. */
+int tgt_edge_index_hash(const int64_t* d_src, const int64_t* d_dst, int64_t E, void* stream, uint64_t h_key[2]);
 /* The attention kernels of a (H, d) shape read launch descriptors that are made on the first call
  * with that shape (a few small allocations, copies and one synchronisation of the stream, once per
  * plan and H * d / 8); tgt_plan_create makes those of H * d = 64 (the reference's hidden size 64
@@ -230,7 +254,9 @@ int tgt_dense_ids_pack(const int64_t* d_spatial_pos, const int64_t* d_edge_type,
  * tgt_dense_attn_dropout_fwd.  dtype TGT_DTYPE_BF16 or TGT_DTYPE_F32_BF16_PRODUCTS (the float32-arithmetic
  * kernels take a bias tensor: TGT_ERR_UNSUPPORTED); H <= 32; the [S, S] bias of one (graph, head) as bf16 plus
  * one column of both tables as float must fit the LDS next to the q/k/v images (S = 129 with the molecule
- * tables, 512 + 1537 rows: 52 KB forward, 79 KB backward), else TGT_ERR_UNSUPPORTED. */
+ * tables, 512 + 1537 rows: 52 KB forward, 79 KB backward), else TGT_ERR_UNSUPPORTED.  The forward applies the
+ * backward's (larger) need: a shape it accepts is a shape tgt_dense_attn_ids_bwd accepts.  The same holds for
+ * tgt_dense_attn_fwd / _bwd. */
 int tgt_dense_attn_ids_fwd(const void* d_q, const void* d_k, const void* d_v, const void* d_attn_bias,
                            const uint16_t* d_sp16, const uint16_t* d_et16, int F, const void* d_spatial_table, int num_spatial,
                            const void* d_edge_table, int num_edges, const void* d_virtual_dist, int b, int S, int H, int d,
@@ -554,17 +580,6 @@ int tgt_timing_enable(int on);
 int tgt_timing_reset(void);
 int tgt_timing_slots(void);
 int tgt_timing_read(int slot, const char** name, double* total_ms, int64_t* launches);
-
-/* ---- row-gather probe ----------------------------------------------------
- * Measurement aid with no counterpart in the reference.  Launches one kernel in
- * which every group of 8 lanes reads the rows d_idx[4g .. 4g+3] (row_bytes = 128
- * or 256, values in [0, n_rows), not checked) of d_table and discards them: the
- * per-edge k[src] / v[src] access of tgt_sparse_attn_fwd (attn_module.py:146-147)
- * without arithmetic, index chains or outputs.  Its rate (n_idx * row_bytes over
- * the "probe_row_gather" timing slot) is what the memory system sustains for
- * this access pattern at this table size.  d_sink: 4 writable bytes. */
-int tgt_probe_row_gather(const void* d_table, int64_t n_rows, int row_bytes, const int32_t* d_idx,
-                         int64_t n_idx, void* d_sink, void* stream);
 
 #ifdef __cplusplus
 }

@@ -62,6 +62,13 @@ def test_host_only_entry_points():
     assert L.tgt_linear_act_fwd(None, None, None, 16, 64, 64, 0, 0, None, None, None) == _lib.ERR_INVALID_ARG       # activation
     assert L.tgt_linear_act_bwd(None, None, None, None, 16, 64, 64, 0, 1, None, None, None, None, 0, None, None) == _lib.ERR_INVALID_ARG
     assert ctypes.sizeof(_lib.ReduceDesc) == 8 + 3 * 4 + 4 + 6 * 8 + 6 * 4                                       # the C struct's layout
+    key = (ctypes.c_uint64 * 2)()
+    assert L.tgt_edge_index_hash(None, None, -1, None, key) == _lib.ERR_INVALID_ARG
+    assert L.tgt_edge_index_hash(None, None, 4, None, key) == _lib.ERR_INVALID_ARG
+    assert L.tgt_edge_index_hash(None, None, 0, None, None) == _lib.ERR_INVALID_ARG
+    # an allocator is both functions or neither
+    CB = ctypes.CFUNCTYPE(ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p)
+    assert L.tgt_set_allocator(ctypes.cast(CB(lambda n, s, u: None), ctypes.c_void_p), None, None) == _lib.ERR_INVALID_ARG
 
 
 def test_torch_extension_loads_and_registers_its_operators():

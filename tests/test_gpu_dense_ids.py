@@ -203,3 +203,29 @@ def test_module_passes_ids_and_falls_back(cuda):
     # float32 tensors without the bf16-products flag are refused by the operator itself
     with pytest.raises(RuntimeError, match="bf16"):
         _ext.ops().dense_attention_ids(q.float(), q.float(), q.float(), None, sp16, et16, st.float(), et.float(), vd.float(), 0.0, 0, False)
+
+
+def test_a_shape_the_forward_accepts_can_be_trained(cuda):
+    """The id form keeps the bias of a (graph, head) pair and the table columns in LDS and its backward needs more of it
+    than its forward: the forward applies the backward's limit, so that a training step never passes the forward and
+    dies inside autograd.  Swept over the sizes around the limit with the molecule tables (512 + 1537 rows)."""
+    H, d, b, ns, ne = 8, 8, 2, 512, 1537
+    g = torch.Generator().manual_seed(4)
+    st, et, vd = (x.to(cuda, torch.bfloat16) for x in _tables(H, ns, ne, seed=2))
+    accepted = refused = 0
+    for s in (128, 160, 192, 208, 224, 232, 240, 248, 255):
+        print(f"id-form limit case: S={s + 1}", flush=True)
+        _, sp, et_ids, _ = make_batch(b, s, 1, ns, ne, seed=s)
+        sp16, et16 = _ext.ops().dense_ids_pack(sp.to(cuda), et_ids.to(cuda), ns, ne)
+        q, k, v = (torch.randn(b, s + 1, H, d, generator=g).to(cuda, torch.bfloat16).requires_grad_(True) for _ in range(3))
+        tabs = [t.clone().requires_grad_(True) for t in (st, et, vd)]
+        try:
+            o = _ext.ops().dense_attention_ids(q, k, v, None, sp16, et16, tabs[0], tabs[1], tabs[2], 0.0, 0, False)
+        except RuntimeError as exc:
+            assert "bytes of LDS" in str(exc)
+            refused += 1
+            continue
+        accepted += 1
+        grads = torch.autograd.grad(o, [q, k, v] + tabs, torch.ones_like(o))          # must not raise
+        assert all(torch.isfinite(x).all() for x in grads)
+    assert accepted >= 1 and refused >= 1, (accepted, refused)       # the sweep straddles the limit

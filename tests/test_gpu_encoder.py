@@ -13,7 +13,7 @@ from oracle import encoder_layer as E
 from oracle import graph_prep as ogp
 from oracle import sparse_attention as osa
 from torchgt_amd import EncoderLayer, FeedForwardNetwork, Graphormer, _lib, fused_linear, nll_loss, workloads
-from torchgt_amd.encoder import AddFunction, AddLayerNormFunction, GeluFunction
+from torchgt_amd import _ext
 
 pytestmark = pytest.mark.gpu
 TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2}
@@ -43,7 +43,7 @@ def test_add_layer_norm_forward_backward(cuda, dtype, C):
         y_ref = torch.nn.functional.layer_norm(s_ref, (C,), leaves[-2], leaves[-1], 1e-5)
         g_ref = torch.autograd.grad([s_ref, y_ref], leaves, [ds_out.double(), dy.double()])
         cl = [t.to(cuda).requires_grad_(True) for t in ([x, r] if with_r else [x]) + [gamma, beta]]
-        s, y = AddLayerNormFunction.apply(cl[0], cl[1] if with_r else None, cl[-2], cl[-1], 1e-5)
+        s, y = _ext.ops().add_layer_norm(cl[0], cl[1] if with_r else None, cl[-2], cl[-1], float(1e-5))
         g_got = torch.autograd.grad([s, y], cl, [ds_out.to(cuda), dy.to(cuda)])
         tol = TOL[dtype]
         assert err(s, s_ref) <= tol and err(y, y_ref) <= tol, (err(s, s_ref), err(y, y_ref))
@@ -55,9 +55,9 @@ def test_layer_norm_rejects_unsupported_width(cuda):
     x = torch.zeros(4, 24, device=cuda)
     w = torch.ones(24, device=cuda)
     with pytest.raises(RuntimeError, match="unsupported"):
-        AddLayerNormFunction.apply(x, None, w, w, 1e-5)          # 24 / 4 = 6 lanes: not a power of two
+        _ext.ops().add_layer_norm(x, None, w, w, float(1e-5))          # 24 / 4 = 6 lanes: not a power of two
     with pytest.raises(RuntimeError):
-        GeluFunction.apply(torch.zeros(8))                        # CPU tensor: no fallback
+        _ext.ops().gelu(torch.zeros(8))                        # CPU tensor: no fallback
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -69,11 +69,11 @@ def test_gelu_and_add(cuda, dtype):
     h_ref = torch.nn.functional.gelu(ud)
     (du_ref,) = torch.autograd.grad(h_ref, ud, dh.double())
     uc = u.to(cuda).requires_grad_(True)
-    h = GeluFunction.apply(uc)
+    h = _ext.ops().gelu(uc)
     (du,) = torch.autograd.grad(h, uc, dh.to(cuda))
     np.testing.assert_allclose(h.detach().double().cpu().numpy(), E.gelu(u.double().numpy()), rtol=0, atol=TOL[dtype] * 10)
     assert err(h, h_ref) <= TOL[dtype] and err(du, du_ref) <= TOL[dtype]
-    s = AddFunction.apply(uc, dh.to(cuda))
+    s = _ext.ops().add(uc, dh.to(cuda))
     assert torch.equal(s.detach().cpu(), u + dh)        # one rounding of the exact sum, in either dtype
 
 
@@ -115,7 +115,7 @@ def test_ffn_operator_matches_oracle_and_the_separate_operators(cuda, dtype, hid
     grads = torch.autograd.grad(got, [xc] + list(mc.parameters()), dy.to(cuda))
     xs = x.to(cuda).requires_grad_(True)
     (u,) = fused_linear(xs, mc.layer1)
-    (ys,) = fused_linear(GeluFunction.apply(u), mc.layer2)
+    (ys,) = fused_linear(_ext.ops().gelu(u), mc.layer2)
     assert torch.equal(got, ys)
     for a, b in zip(grads, torch.autograd.grad(ys, [xs] + list(mc.parameters()), dy.to(cuda))):
         assert torch.equal(a, b)

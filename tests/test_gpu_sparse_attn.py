@@ -399,6 +399,49 @@ def test_plan_cache_is_bounded_by_bytes(cuda):
         clear_plan_cache()
 
 
+def test_plan_survives_a_fresh_copy_of_edge_index(cuda):
+    """The reference's training loops move the CPU-resident edge_index of a pre-packed batch to the GPU in every
+    iteration (main_sp_sparse_node_level.py:178-183): the second copy, at whatever address, must find the plan
+    of the first (one build), and the results are bit-identical.  A different edge list of the same shape gets
+    its own plan."""
+    from torchgt_amd import plan as plan_mod, get_plan, clear_plan_cache
+    clear_plan_cache()
+    e, n = workloads.barabasi_albert(n=2048, m=4, seed=11)
+    ei_cpu = torch.from_numpy(e)
+    H, d = 8, 8
+    g = torch.Generator().manual_seed(21)
+    q, k, v, dout = (torch.randn(n, H, d, generator=g).to(cuda) for _ in range(4))
+    bias = (torch.randn(e.shape[1], H, generator=g) * 0.1).to(cuda)
+    layer = CoreAttention(H * d, 0.0, H).to(cuda)
+    results, plans, held = [], [], []
+    for it in range(3):
+        ei = ei_cpu.to(cuda)                      # a new tensor every iteration
+        held.append(ei)                           # kept alive: the copies sit at different addresses
+        t = [x.clone().requires_grad_(True) for x in (q, k, v, bias)]
+        out = layer(t[0][None], t[1][None], t[2][None], t[3], ei, "sparse")
+        out2 = layer(t[0][None], t[1][None], t[2][None], t[3], ei, "sparse")          # second layer of the step
+        results.append((out,) + torch.autograd.grad(out + out2, t, dout.view(1, n, -1)))
+        plans.append(get_plan(ei, n))
+    stats = plan_mod.plan_cache_stats()
+    assert stats["builds"] == 1 and stats["content_hits"] == 2, stats
+    assert stats["tensor_hits"] >= 3            # the second layer and the explicit look-up never hash
+    assert plans[0] is plans[1] is plans[2]
+    for r in results[1:]:
+        for a, b in zip(results[0], r):
+            assert torch.equal(a, b)
+    # same shape, other content: a plan of its own; the key looks at positions too
+    e2 = np.ascontiguousarray(e[:, ::-1])          # the same edges in another order
+    assert get_plan(torch.from_numpy(e2).to(cuda), n) is not plans[0]
+    e3 = e.copy()
+    e3[0, 5] = (e3[0, 5] + 1) % n
+    assert get_plan(torch.from_numpy(e3).to(cuda), n) is not plans[0]
+    assert plan_mod.plan_cache_stats()["builds"] == 3
+    # the key itself: equal for equal content, whatever the address
+    assert plan_mod.edge_index_key(held[0]) == plan_mod.edge_index_key(held[1])
+    assert plan_mod.edge_index_key(held[0]) != plan_mod.edge_index_key(torch.from_numpy(e3).to(cuda))
+    clear_plan_cache()
+
+
 def test_plan_order_needs_the_map(cuda):
     e, n = workloads.barabasi_albert()
     ei = torch.from_numpy(e).to(cuda)

@@ -28,6 +28,8 @@ SIGNATURES = {
     "tgt_last_error": (_c.c_char_p, []),
     "tgt_plan_create": (_i32, [_vp, _vp, _i64, _i64, _vp, _c.POINTER(_vp)]),
     "tgt_plan_destroy": (_i32, [_vp]),
+    "tgt_set_allocator": (_i32, [_vp, _vp, _vp]),
+    "tgt_edge_index_hash": (_i32, [_vp, _vp, _i64, _vp, _c.POINTER(_c.c_uint64)]),
     "tgt_plan_info": (_i32, [_vp, _c.POINTER(_i64)]),
     "tgt_plan_array_len": (_i64, [_vp, _i32]),
     "tgt_plan_export": (_i32, [_vp, _i32, _vp, _i64]),
@@ -105,7 +107,6 @@ SIGNATURES = {
     "tgt_embedding_sum_bwd_workspace_bytes": (_i64, [_i32, _i32]),
     "tgt_embedding_sum_bwd": (_i32, [_vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _i64, _vp]),
     "tgt_gen_edge_input": (_i32, [_vp, _vp, _i32, _i32, _vp, _i32, _i32, _i32, _vp, _vp]),
-    "tgt_probe_row_gather": (_i32, [_vp, _i64, _i32, _vp, _i64, _vp, _vp]),
     "tgt_timing_enable": (_i32, [_i32]),
     "tgt_timing_reset": (_i32, []),
     "tgt_timing_slots": (_i32, []),

@@ -4,6 +4,7 @@
 #include <stdint.h>
 #include <stdio.h>
 #include <stdarg.h>
+#include <mutex>
 #include <vector>
 #include "../../include/torchgt_hip.h"
 
@@ -99,16 +100,17 @@ struct Side {
     int32_t* col = nullptr;      // [E] other endpoint
     int32_t* eid = nullptr;      // [E] caller's edge id
     int32_t* pos = nullptr;      // [E] source side only, built on request: position of the edge in the destination-sorted order
-    Item* items = nullptr;       // [n_items]: workgroup items first, then wave items by (window, length class, row)
+    Item* items = nullptr;       // wave items (rows one wave walks) by (window, length class, row); room for N
+    Item* block_items = nullptr; // [n_block_items] workgroup items: segments of the rows longer than a wave row
     int32_t* split_row = nullptr;   // [n_split] rows that were split
     int32_t* split_off = nullptr;   // [n_split+1] first partial slot of each split row
     int32_t* part2split = nullptr;  // [n_parts] index into split_row of the row a partial slot belongs to
     int32_t* split_grp = nullptr;   // [n_split+1] first combine group of each split row (a row with more than kCombineFan segments has ceil(segments / kCombineFan) groups)
     int32_t n_items = 0, n_split = 0, n_parts = 0, n_groups = 0;
-    int32_t n_block_items = 0;      // items [0, n_block_items) are walked by one workgroup each
+    int32_t n_block_items = 0;      // workgroup items (n_items counts both kinds)
     // host copies the launch descriptors are made from
     int32_t n_windows = 0;
-    std::vector<uint32_t> win_class_off;   // [n_windows * (kNumClass + 1)] wave items of (window, class) start at n_block_items + this
+    std::vector<uint32_t> win_class_off;   // [n_windows * (kNumClass + 1)] wave items of (window, class) start here
     std::vector<uint32_t> win_class_cnt;   // same shape: how many
     std::vector<int32_t> block_home;       // [n_block_items] window the workgroup item is scheduled with
     std::vector<int32_t> block_len;        // [n_block_items] its edges
@@ -125,14 +127,21 @@ struct Schedule {
 };
 constexpr int kNumLpe = 5;   // lanes per edge 1, 2, 4, 8, 16
 
-// Device buffer that frees itself.
+// Device memory of the library's own (plans, tile sets, scratch of the edge preparation): from the
+// allocator set with tgt_set_allocator, hipMalloc / hipFree without one.  `st` is the stream the memory
+// is first used on (a caching allocator hands back memory that is safe to reuse on that stream).
+hipError_t dev_alloc(void** p, size_t bytes, hipStream_t st);
+void dev_free(void* p);
+
+// Device buffer that frees itself.  Freed memory may still be read by kernels already launched on the
+// stream it was allocated for: a stream-ordered allocator reuses it behind them, hipFree waits for them.
 struct DevBuf {
     void* p = nullptr;
     DevBuf() = default;
     DevBuf(const DevBuf&) = delete;
     DevBuf& operator=(const DevBuf&) = delete;
     ~DevBuf();
-    hipError_t alloc(size_t bytes);
+    hipError_t alloc(size_t bytes, hipStream_t st = nullptr);
     template <typename T> T* as() const { return (T*)p; }
 };
 
@@ -141,7 +150,7 @@ int bits_for(int64_t n);   // bits needed to hold values in [0, n)
 // Stable LSD radix sort of (uint32 key, uint32 value) pairs (radix_sort.hip).
 class RadixSorter {
 public:
-    int init(int64_t capacity);
+    int init(int64_t capacity, hipStream_t st = nullptr);
     // Sorts by the low `bits` bits of the keys.  vals_in == nullptr means values 0..n-1.
     // The results live in the sorter's buffers until the next sort() call; copy a
     // result before passing it as input of another sort().
@@ -171,7 +180,7 @@ __device__ __forceinline__ float act_grad(float u, float dh) {
 }
 
 // Kernel names of the optional per-kernel timing (timing.hip).
-enum KernelSlot { KS_FWD = 0, KS_NODE_SIDE, KS_BWD, KS_DENSE_FWD, KS_DENSE_BWD, KS_TILE_FWD, KS_TILE_BWD, KS_PROBE_GATHER, KS_LINEAR_FWD,
+enum KernelSlot { KS_FWD = 0, KS_NODE_SIDE, KS_BWD, KS_DENSE_FWD, KS_DENSE_BWD, KS_TILE_FWD, KS_TILE_BWD, KS_LINEAR_FWD,
                   KS_LINEAR_DX, KS_LINEAR_DW, KS_LAYER_NORM_FWD, KS_LAYER_NORM_BWD, KS_GELU, KS_GRAPH_BIAS_FWD,
                   KS_GRAPH_BIAS_BWD, KS_LOSS, KS_COUNT };
 
@@ -223,6 +232,7 @@ struct tgt_plan {
     tgt::Side dst;   // edges grouped by destination (query) node
     tgt::Side src;   // edges grouped by source (key/value) node
     tgt::Schedule sched[tgt::kNumLpe];   // by log2(lanes per edge); made on first use of a shape
+    std::mutex sched_mutex;              // guards that first use
 };
 namespace tgt {
 // Descriptors for kernels with `lpe` lanes per edge; builds them on first use (allocates, copies and

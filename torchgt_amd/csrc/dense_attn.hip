@@ -1215,9 +1215,11 @@ static int launch_dense(const DenseCall& c, bool bwd) {
     } else {
         const size_t lds_f = lds_f0 + (BSRC == 1 ? ids_lds_bytes(c.S, c.ids.ns, c.ids.ne, false) : 0);
         const size_t lds_b = lds_b0 + (BSRC == 1 ? ids_lds_bytes(c.S, c.ids.ns, c.ids.ne, true) : 0);
-        if ((bwd ? lds_b : lds_f) > (size_t)kLdsLimit) {
+        // the forward refuses what its backward could not run: a training step must not pass the forward and fail
+        // inside autograd
+        if (std::max(lds_f, lds_b) > (size_t)kLdsLimit) {
             set_error("dense attention from ids: S=%d with tables of %d + %d rows needs %zu bytes of LDS (limit %d); "
-                      "build the bias tensor instead", c.S, c.ids.ns, c.ids.ne, bwd ? lds_b : lds_f, kLdsLimit);
+                      "build the bias tensor instead", c.S, c.ids.ns, c.ids.ne, std::max(lds_f, lds_b), kLdsLimit);
             return TGT_ERR_UNSUPPORTED;
         }
         const float scale = sqrtf((float)c.d);     // the reference MULTIPLIES q by sqrt(d)

@@ -248,9 +248,10 @@ __global__ __launch_bounds__(kF32Block) void k_dense_f32_bwd(const float* __rest
 
 template <int D>
 static int launch_f32(const DenseF32Call& c, bool bwd) {
-    const int lds = (bwd ? (4 * c.S * D + 2 * c.S) : 2 * c.S * D) * 4 + c.S * kF32StripLd * 4;
-    if (lds > 160 * 1024) {
-        set_error("dense attention (float32): S=%d with head dim %d needs %d bytes of LDS (limit %d)", c.S, D, lds, 160 * 1024);
+    const int lds_bwd = (4 * c.S * D + 2 * c.S) * 4 + c.S * kF32StripLd * 4;
+    const int lds = bwd ? lds_bwd : 2 * c.S * D * 4 + c.S * kF32StripLd * 4;
+    if (lds_bwd > 160 * 1024) {      // the forward refuses what its backward could not run
+        set_error("dense attention (float32): S=%d with head dim %d needs %d bytes of LDS (limit %d)", c.S, D, lds_bwd, 160 * 1024);
         return TGT_ERR_UNSUPPORTED;
     }
     const float scale = sqrtf((float)D);      // the reference MULTIPLIES q by sqrt(d)

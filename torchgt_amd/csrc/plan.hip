@@ -13,6 +13,9 @@
 #include "common.h"
 #include <vector>
 #include <new>
+#include <mutex>
+#include <utility>
+#include <algorithm>
 #include <stdlib.h>
 
 namespace tgt {
@@ -100,12 +103,45 @@ __global__ void k_sched_count(const int32_t* __restrict__ rowptr, int64_t N, int
     if (threadIdx.x < kSchedCats) counts[(int64_t)blockIdx.x * kSchedCats + threadIdx.x] = c[threadIdx.x];
 }
 
+// Per side, written by the device and read back once: how many of everything the schedule holds.
+struct SchedHeader { int32_t n_wave, n_long, n_block, n_split, n_parts, n_groups, pad0, pad1; };
+
+// offs[window, cat]: first position of the window's rows of a category - wave classes count through
+// (window, class) in that order, long rows through the windows - and the two totals.  One workgroup.
+__global__ __launch_bounds__(1024) void k_sched_scan(const uint32_t* __restrict__ counts, int nwin,
+                                                     uint32_t* __restrict__ offs, SchedHeader* __restrict__ hdr) {
+    __shared__ uint32_t sw[1024], sl[1024];
+    const int tid = threadIdx.x;
+    const int chunk = (nwin + 1023) / 1024;
+    const int b = min(tid * chunk, nwin), e = min(b + chunk, nwin);
+    uint32_t ws = 0, ls = 0;
+    for (int w = b; w < e; ++w) {
+        for (int c = 0; c < kNumClass; ++c) ws += counts[(int64_t)w * kSchedCats + c];
+        ls += counts[(int64_t)w * kSchedCats + kNumClass];
+    }
+    sw[tid] = ws; sl[tid] = ls;
+    __syncthreads();
+    for (int off = 1; off < 1024; off <<= 1) {
+        const uint32_t x = tid >= off ? sw[tid - off] : 0u, y = tid >= off ? sl[tid - off] : 0u;
+        __syncthreads();
+        sw[tid] += x; sl[tid] += y;
+        __syncthreads();
+    }
+    uint32_t rw = tid ? sw[tid - 1] : 0u, rl = tid ? sl[tid - 1] : 0u;
+    for (int w = b; w < e; ++w) {
+        for (int c = 0; c < kNumClass; ++c) { offs[(int64_t)w * kSchedCats + c] = rw; rw += counts[(int64_t)w * kSchedCats + c]; }
+        offs[(int64_t)w * kSchedCats + kNumClass] = rl;
+        rl += counts[(int64_t)w * kSchedCats + kNumClass];
+    }
+    if (tid == 1023) { hdr->n_wave = (int32_t)sw[1023]; hdr->n_long = (int32_t)sl[1023]; }
+}
+
 // Rows keep their order inside a (window, category): position = offs[window, cat] + rank among the
-// window's rows.  Wave-class rows become schedule items at items[base + position]; long rows are
-// listed (row, first edge, length) for the host.
+// window's rows.  Wave-class rows become wave items at items[position]; long rows are listed (row, first
+// edge, length) for the kernels that cut them into workgroup items.
 __global__ void k_sched_fill(const int32_t* __restrict__ rowptr, int64_t N, int wave_row_max,
-                             const uint32_t* __restrict__ offs, int64_t base, Item* __restrict__ items,
-                             int32_t* __restrict__ long_rows) {
+                             const uint32_t* __restrict__ offs, Item* __restrict__ items,
+                             int32_t* __restrict__ long_rows, int64_t cap_long) {
     __shared__ uint32_t wave_cnt[kSchedMaxWaves][kSchedCats];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -128,24 +164,126 @@ __global__ void k_sched_fill(const int32_t* __restrict__ rowptr, int64_t N, int 
     uint32_t pos = offs[(int64_t)blockIdx.x * kSchedCats + cat] + rank;
     for (int w = 0; w < wave; ++w) pos += wave_cnt[w][cat];
     if (cat < kNumClass) {
-        if (items) items[base + pos] = Item{(int32_t)r, start, len, -1};
-    } else if (long_rows) {
+        items[pos] = Item{(int32_t)r, start, len, -1};
+    } else if ((int64_t)pos < cap_long) {
         long_rows[3 * (int64_t)pos + 0] = (int32_t)r;
         long_rows[3 * (int64_t)pos + 1] = start;
         long_rows[3 * (int64_t)pos + 2] = len;
     }
 }
 
-// out[i] = col[idx[i]]
-__global__ void k_gather_i32(const int32_t* __restrict__ col, const int32_t* __restrict__ idx, int n,
-                             int32_t* __restrict__ out) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) out[i] = col[idx[i]];
+// How a long row is cut (the same arithmetic on the device and wherever it is checked): balanced segments
+// of at most block_seg edges; a row with more than spread_segs of those (a global node) gets segments of
+// spread_seg edges instead, each scheduled next to the rows it gathers.
+struct CutParams { int block_seg, spread_segs, spread_seg, combine_fan, window; };
+__host__ __device__ inline void cut_row(const CutParams& cp, int len, int& nseg, int& seg, bool& spread) {
+    nseg = (len + cp.block_seg - 1) / cp.block_seg;
+    spread = nseg > cp.spread_segs;
+    if (spread) nseg = (len + cp.spread_seg - 1) / cp.spread_seg;
+    seg = (len + nseg - 1) / nseg;
+}
+
+// Long rows -> where their workgroup items, partial slots and combine groups start.  One workgroup: every
+// thread takes a run of consecutive rows of the list (it is short: rows of more than a wave row's edges), the
+// runs' totals are scanned in LDS, then every thread writes its rows.
+__global__ __launch_bounds__(1024) void k_cut_rows(const int32_t* __restrict__ long_rows, SchedHeader* __restrict__ hdr,
+                                                   CutParams cp, int32_t* __restrict__ row_item_off,
+                                                   int32_t* __restrict__ row_split_idx, int32_t* __restrict__ row_part_off,
+                                                   int32_t* __restrict__ split_row, int32_t* __restrict__ split_off,
+                                                   int32_t* __restrict__ split_grp) {
+    __shared__ uint32_t sh[4][1024];
+    const int n_long = hdr->n_long;
+    const int tid = threadIdx.x;
+    const int chunk = (n_long + 1023) / 1024;
+    const int b = min(tid * chunk, n_long), e = min(b + chunk, n_long);
+    uint32_t items = 0, splits = 0, parts = 0, groups = 0;
+    for (int i = b; i < e; ++i) {
+        int nseg, seg;
+        bool spread;
+        cut_row(cp, long_rows[3 * i + 2], nseg, seg, spread);
+        items += (uint32_t)nseg;
+        if (nseg > 1) { splits += 1; parts += (uint32_t)nseg; }
+        if (nseg > cp.combine_fan) groups += (uint32_t)((nseg + cp.combine_fan - 1) / cp.combine_fan);
+    }
+    sh[0][tid] = items; sh[1][tid] = splits; sh[2][tid] = parts; sh[3][tid] = groups;
+    __syncthreads();
+    for (int off = 1; off < 1024; off <<= 1) {
+        uint32_t x[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) x[k] = tid >= off ? sh[k][tid - off] : 0u;
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 4; ++k) sh[k][tid] += x[k];
+        __syncthreads();
+    }
+    // running totals in front of this thread's rows
+    items = tid ? sh[0][tid - 1] : 0u; splits = tid ? sh[1][tid - 1] : 0u;
+    parts = tid ? sh[2][tid - 1] : 0u; groups = tid ? sh[3][tid - 1] : 0u;
+    for (int i = b; i < e; ++i) {
+        int nseg, seg;
+        bool spread;
+        cut_row(cp, long_rows[3 * i + 2], nseg, seg, spread);
+        const bool is_split = nseg > 1;
+        row_item_off[i] = (int32_t)items;
+        row_split_idx[i] = is_split ? (int32_t)splits : -1;
+        row_part_off[i] = (int32_t)parts;
+        if (is_split) {
+            split_row[splits] = long_rows[3 * i];
+            split_off[splits] = (int32_t)parts;
+            split_grp[splits] = (int32_t)groups;
+            splits += 1; parts += (uint32_t)nseg;
+        }
+        items += (uint32_t)nseg;
+        if (nseg > cp.combine_fan) groups += (uint32_t)((nseg + cp.combine_fan - 1) / cp.combine_fan);
+    }
+    if (tid == 1023) {
+        row_item_off[n_long] = (int32_t)sh[0][1023];
+        split_off[sh[1][1023]] = (int32_t)sh[2][1023];
+        split_grp[sh[1][1023]] = (int32_t)sh[3][1023];
+        hdr->n_block = (int32_t)sh[0][1023];
+        hdr->n_split = (int32_t)sh[1][1023];
+        hdr->n_parts = (int32_t)sh[2][1023];
+        hdr->n_groups = (int32_t)sh[3][1023];
+    }
+}
+
+// What the host needs to know of a workgroup item to place it: the window it is scheduled with (the one
+// of the other endpoint in the middle of its edges), its edges, whether it is a short segment of a row
+// that spans the graph.
+struct BlockMeta { int32_t home, len, spread; };
+
+// One thread per workgroup item: finds its row in the offsets and writes the item.
+__global__ void k_emit_items(const int32_t* __restrict__ long_rows, const SchedHeader* __restrict__ hdr, CutParams cp,
+                             const int32_t* __restrict__ row_item_off, const int32_t* __restrict__ row_split_idx,
+                             const int32_t* __restrict__ row_part_off, const int32_t* __restrict__ col,
+                             Item* __restrict__ block_items, BlockMeta* __restrict__ meta,
+                             int32_t* __restrict__ part2split) {
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= hdr->n_block) return;
+    int lo = 0, hi = hdr->n_long - 1;               // last row whose first item is <= j
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (row_item_off[mid] <= j) lo = mid;
+        else hi = mid - 1;
+    }
+    const int i = lo, sgm = j - row_item_off[i];
+    const int r = long_rows[3 * i], b = long_rows[3 * i + 1], len = long_rows[3 * i + 2];
+    int nseg, seg;
+    bool spread;
+    cut_row(cp, len, nseg, seg, spread);
+    const int o = sgm * seg;
+    const int l = (o + seg <= len) ? seg : (len - o);
+    const int sidx = row_split_idx[i];
+    const int part = sidx >= 0 ? row_part_off[i] + sgm : -1;
+    block_items[j] = Item{r, b + o, l, part};
+    meta[j] = BlockMeta{col[b + o + l / 2] / cp.window, l, spread ? 1 : 0};
+    if (part >= 0) part2split[part] = sidx;
 }
 
 // One workgroup of 64 threads writes one wave record from its descriptor (layout: WaveRec in common.h).
 __global__ __launch_bounds__(64) void k_build_records(const WaveDesc* __restrict__ desc, const Item* __restrict__ items_d,
-                                                      const Item* __restrict__ items_s, const int32_t* __restrict__ col_d,
+                                                      const Item* __restrict__ items_s, const Item* __restrict__ bitems_d,
+                                                      const Item* __restrict__ bitems_s, const int32_t* __restrict__ col_d,
                                                       const int32_t* __restrict__ eid_d, const int32_t* __restrict__ col_s,
                                                       const int32_t* __restrict__ eid_s, WaveRecLayout L, int lpe,
                                                       int32_t* __restrict__ recs) {
@@ -162,7 +300,7 @@ __global__ __launch_bounds__(64) void k_build_records(const WaveDesc* __restrict
     if (kind == kDescNone) return;
     if (kind == kDescBlock) {
         if (t == 0) {
-            const Item it = items[d.first];
+            const Item it = (src ? bitems_s : bitems_d)[d.first];
             out[4] = it.row; out[5] = it.start; out[6] = it.len; out[7] = it.part;
         }
         return;
@@ -231,117 +369,78 @@ static int window_rows() {
 // A longer row is walked by whole workgroups: balanced segments, each a workgroup item that is
 // scheduled with the window most of its other endpoints lie in (so that the rows a segment gathers
 // are the ones the window's own rows load); if there is more than one segment their partial sums
-// meet in the workspace.
-static int build_schedule(int64_t N, Side& side, hipStream_t st) {
+// meet in the workspace.  All of it is made on the device; the host reads back the counts (one copy for
+// both views, together with the range-check flag) and, if there are long rows, what it needs to place
+// their workgroup items.
+struct SideScratch {
+    DevBuf long_rows, row_item_off, row_split_idx, row_part_off, meta;
+    int64_t cap_long = 0, cap_block = 0;
+    CutParams cp{};
+    int wave_row_max = 0, W = 0, nwin = 0;
+};
+
+// ints of the report in front of the per-window counts: two headers, the flag, padding
+constexpr int kReportHead = 32;
+constexpr int kReportFlag = 16;
+
+static int schedule_device(int64_t N, int64_t E, Side& side, SideScratch& sc, int32_t* report, int side_idx,
+                           hipStream_t st) {
     // tuning overrides (experiments only; the defaults are the measured best)
-    const int kWaveRowMax = env_int("TGT_WAVE_ROW_MAX", tgt::kWaveRowMax);
-    const int kBlockSeg = env_int("TGT_BLOCK_SEG", tgt::kBlockSeg);
-    const int kSpreadSeg = env_int("TGT_SPREAD_SEG", tgt::kSpreadSeg);
-    const int W = window_rows();
-    const int nwin = (int)((N + W - 1) / W);
-    side.n_windows = nwin;
-    DevBuf counts, long_d;
-    const size_t ncnt = (size_t)kSchedCats * nwin;
-    TGT_HIP_CHECK(counts.alloc(sizeof(uint32_t) * ncnt));
-    hipLaunchKernelGGL(k_sched_count, dim3(nwin), dim3(W), 0, st, side.rowptr, N, kWaveRowMax, counts.as<uint32_t>());
+    sc.wave_row_max = env_int("TGT_WAVE_ROW_MAX", tgt::kWaveRowMax);
+    sc.cp.block_seg = env_int("TGT_BLOCK_SEG", tgt::kBlockSeg);
+    sc.cp.spread_seg = env_int("TGT_SPREAD_SEG", tgt::kSpreadSeg);
+    sc.cp.spread_segs = kSpreadSegs;
+    sc.cp.combine_fan = kCombineFan;
+    sc.W = window_rows();
+    sc.cp.window = sc.W;
+    sc.nwin = (int)((N + sc.W - 1) / sc.W);
+    side.n_windows = sc.nwin;
+    const size_t ncnt = (size_t)kSchedCats * sc.nwin;
+    SchedHeader* hdr = reinterpret_cast<SchedHeader*>(report) + side_idx;
+    uint32_t* counts = reinterpret_cast<uint32_t*>(report) + kReportHead + (size_t)side_idx * 2 * ncnt;
+    uint32_t* offs = counts + ncnt;
+    // bounds known before anything is counted: a long row has more than wave_row_max edges, a row of len edges
+    // is cut into at most len / min(block_seg, spread_seg) + 1 segments
+    sc.cap_long = std::min<int64_t>(N, E / (sc.wave_row_max + 1)) + 1;
+    const int min_seg = std::max(1, std::min(sc.cp.block_seg, sc.cp.spread_seg));
+    sc.cap_block = E / min_seg + sc.cap_long + 1;
+    TGT_HIP_CHECK(dev_alloc((void**)&side.items, sizeof(Item) * (size_t)(N + 1), st));
+    TGT_HIP_CHECK(dev_alloc((void**)&side.block_items, sizeof(Item) * (size_t)sc.cap_block, st));
+    TGT_HIP_CHECK(dev_alloc((void**)&side.split_row, sizeof(int32_t) * (size_t)(sc.cap_long + 1), st));
+    TGT_HIP_CHECK(dev_alloc((void**)&side.split_off, sizeof(int32_t) * (size_t)(sc.cap_long + 1), st));
+    TGT_HIP_CHECK(dev_alloc((void**)&side.split_grp, sizeof(int32_t) * (size_t)(sc.cap_long + 1), st));
+    TGT_HIP_CHECK(dev_alloc((void**)&side.part2split, sizeof(int32_t) * (size_t)(sc.cap_block + 1), st));
+    TGT_HIP_CHECK(sc.long_rows.alloc(sizeof(int32_t) * 3 * (size_t)sc.cap_long, st));
+    TGT_HIP_CHECK(sc.row_item_off.alloc(sizeof(int32_t) * (size_t)(sc.cap_long + 1), st));
+    TGT_HIP_CHECK(sc.row_split_idx.alloc(sizeof(int32_t) * (size_t)sc.cap_long, st));
+    TGT_HIP_CHECK(sc.row_part_off.alloc(sizeof(int32_t) * (size_t)sc.cap_long, st));
+    TGT_HIP_CHECK(sc.meta.alloc(sizeof(BlockMeta) * (size_t)sc.cap_block, st));
+    hipLaunchKernelGGL(k_sched_count, dim3(sc.nwin), dim3(sc.W), 0, st, side.rowptr, N, sc.wave_row_max, counts);
+    hipLaunchKernelGGL(k_sched_scan, dim3(1), dim3(1024), 0, st, counts, sc.nwin, offs, hdr);
+    hipLaunchKernelGGL(k_sched_fill, dim3(sc.nwin), dim3(sc.W), 0, st, side.rowptr, N, sc.wave_row_max, offs, side.items,
+                       sc.long_rows.as<int32_t>(), sc.cap_long);
+    hipLaunchKernelGGL(k_cut_rows, dim3(1), dim3(1024), 0, st, sc.long_rows.as<int32_t>(), hdr, sc.cp,
+                       sc.row_item_off.as<int32_t>(), sc.row_split_idx.as<int32_t>(), sc.row_part_off.as<int32_t>(),
+                       side.split_row, side.split_off, side.split_grp);
+    hipLaunchKernelGGL(k_emit_items, dim3((unsigned)((sc.cap_block + 255) / 256)), dim3(256), 0, st, sc.long_rows.as<int32_t>(),
+                       hdr, sc.cp, sc.row_item_off.as<int32_t>(), sc.row_split_idx.as<int32_t>(), sc.row_part_off.as<int32_t>(),
+                       side.col, side.block_items, sc.meta.as<BlockMeta>(), side.part2split);
     TGT_HIP_CHECK(hipGetLastError());
-    std::vector<uint32_t> cnt(ncnt), offs(ncnt);
-    TGT_HIP_CHECK(hipMemcpyAsync(cnt.data(), counts.p, sizeof(uint32_t) * ncnt, hipMemcpyDeviceToHost, st));
-    TGT_HIP_CHECK(hipStreamSynchronize(st));
-    // positions: wave items run over (window, class); long rows over windows
-    uint32_t n_wave = 0, n_long = 0;
-    for (int w = 0; w < nwin; ++w) {
-        for (int c = 0; c < kNumClass; ++c) { offs[(size_t)w * kSchedCats + c] = n_wave; n_wave += cnt[(size_t)w * kSchedCats + c]; }
-        offs[(size_t)w * kSchedCats + kNumClass] = n_long;
-        n_long += cnt[(size_t)w * kSchedCats + kNumClass];
-    }
-    side.win_class_off = offs;
-    side.win_class_cnt = cnt;
-    TGT_HIP_CHECK(hipMemcpyAsync(counts.p, offs.data(), sizeof(uint32_t) * ncnt, hipMemcpyHostToDevice, st));
-    // the long rows (few) come to the host, which cuts them into workgroup items
-    std::vector<int32_t> longs((size_t)3 * n_long);
-    if (n_long > 0) {
-        TGT_HIP_CHECK(long_d.alloc(sizeof(int32_t) * (size_t)3 * n_long));
-        hipLaunchKernelGGL(k_sched_fill, dim3(nwin), dim3(W), 0, st, side.rowptr, N, kWaveRowMax, counts.as<uint32_t>(),
-                           (int64_t)0, (Item*)nullptr, long_d.as<int32_t>());
-        TGT_HIP_CHECK(hipGetLastError());
-        TGT_HIP_CHECK(hipMemcpyAsync(longs.data(), long_d.p, sizeof(int32_t) * longs.size(), hipMemcpyDeviceToHost, st));
-        TGT_HIP_CHECK(hipStreamSynchronize(st));
-    }
-    std::vector<Item> items;
-    std::vector<int32_t> split_row, split_off, part2split, split_grp, mid;
-    int32_t n_groups = 0;
-    int32_t n_parts = 0;
-    for (int64_t i = 0; i < (int64_t)n_long; ++i) {
-        const int32_t r = longs[3 * i], b = longs[3 * i + 1], len = longs[3 * i + 2];
-        int nseg = (len + kBlockSeg - 1) / kBlockSeg;
-        // a row with many segments (a global node) gets short ones: each is scheduled next to the rows it gathers
-        const bool spread = nseg > kSpreadSegs;
-        if (spread) nseg = (len + kSpreadSeg - 1) / kSpreadSeg;
-        if (nseg == 1) {
-            items.push_back(Item{r, b, len, -1});
-            mid.push_back(b + len / 2);
-            side.block_spread.push_back(0);
-            continue;
-        }
-        const int seg = (len + nseg - 1) / nseg;
-        split_off.push_back(n_parts);
-        for (int s = 0; s < nseg; ++s) {
-            const int o = s * seg;
-            const int l = (o + seg <= len) ? seg : (len - o);
-            part2split.push_back((int32_t)split_row.size());
-            items.push_back(Item{r, b + o, l, n_parts++});
-            mid.push_back(b + o + l / 2);
-            side.block_spread.push_back(spread ? 1 : 0);
-        }
-        split_row.push_back(r);
-        split_grp.push_back(n_groups);
-        if (nseg > kCombineFan) n_groups += (nseg + kCombineFan - 1) / kCombineFan;
-    }
-    split_off.push_back(n_parts);
-    split_grp.push_back(n_groups);
-    side.n_groups = n_groups;
-    side.n_block_items = (int32_t)items.size();
-    side.n_items = (int32_t)(items.size() + n_wave);
-    side.n_split = (int32_t)split_row.size();
-    side.n_parts = n_parts;
-    side.block_len.resize(items.size());
-    side.block_home.assign(items.size(), 0);
-    for (size_t i = 0; i < items.size(); ++i) side.block_len[i] = items[i].len;
-    TGT_HIP_CHECK(hipMalloc((void**)&side.items, sizeof(Item) * ((size_t)side.n_items + 1)));
-    TGT_HIP_CHECK(hipMalloc((void**)&side.split_row, sizeof(int32_t) * (split_row.size() + 1)));
-    TGT_HIP_CHECK(hipMalloc((void**)&side.split_off, sizeof(int32_t) * split_off.size()));
-    TGT_HIP_CHECK(hipMalloc((void**)&side.part2split, sizeof(int32_t) * (part2split.size() + 1)));
-    TGT_HIP_CHECK(hipMalloc((void**)&side.split_grp, sizeof(int32_t) * split_grp.size()));
-    TGT_HIP_CHECK(hipMemcpyAsync(side.split_grp, split_grp.data(), sizeof(int32_t) * split_grp.size(), hipMemcpyHostToDevice, st));
-    DevBuf mid_d, home_d;
-    if (!items.empty()) {
-        TGT_HIP_CHECK(hipMemcpyAsync(side.items, items.data(), sizeof(Item) * items.size(), hipMemcpyHostToDevice, st));
-        // home window of a workgroup item: the window of the other endpoint in the middle of its edges
-        const int nb = (int)items.size();
-        TGT_HIP_CHECK(mid_d.alloc(sizeof(int32_t) * nb));
-        TGT_HIP_CHECK(home_d.alloc(sizeof(int32_t) * nb));
-        TGT_HIP_CHECK(hipMemcpyAsync(mid_d.p, mid.data(), sizeof(int32_t) * nb, hipMemcpyHostToDevice, st));
-        hipLaunchKernelGGL(k_gather_i32, dim3((nb + 255) / 256), dim3(256), 0, st, side.col, mid_d.as<int32_t>(), nb,
-                           home_d.as<int32_t>());
-        TGT_HIP_CHECK(hipGetLastError());
-        TGT_HIP_CHECK(hipMemcpyAsync(side.block_home.data(), home_d.p, sizeof(int32_t) * nb, hipMemcpyDeviceToHost, st));
-    }
-    if (!split_row.empty()) {
-        TGT_HIP_CHECK(hipMemcpyAsync(side.split_row, split_row.data(), sizeof(int32_t) * split_row.size(),
-                                     hipMemcpyHostToDevice, st));
-        TGT_HIP_CHECK(hipMemcpyAsync(side.part2split, part2split.data(), sizeof(int32_t) * part2split.size(),
-                                     hipMemcpyHostToDevice, st));
-    }
-    TGT_HIP_CHECK(hipMemcpyAsync(side.split_off, split_off.data(), sizeof(int32_t) * split_off.size(),
-                                 hipMemcpyHostToDevice, st));
-    // the wave items (the bulk) are written by the device
-    hipLaunchKernelGGL(k_sched_fill, dim3(nwin), dim3(W), 0, st, side.rowptr, N, kWaveRowMax, counts.as<uint32_t>(),
-                       (int64_t)side.n_block_items, side.items, (int32_t*)nullptr);
-    TGT_HIP_CHECK(hipGetLastError());
-    TGT_HIP_CHECK(hipStreamSynchronize(st));   // the host vectors and the scratch buffers die at return
-    for (int32_t& h : side.block_home) h = h / W;   // node id -> window
     return TGT_OK;
+}
+
+// The counts are on the host: sizes of the view's schedule and the per-window tables the placement reads.
+static void schedule_counts(Side& side, const SideScratch& sc, const int32_t* report, int side_idx) {
+    const SchedHeader& h = reinterpret_cast<const SchedHeader*>(report)[side_idx];
+    const size_t ncnt = (size_t)kSchedCats * sc.nwin;
+    const uint32_t* counts = reinterpret_cast<const uint32_t*>(report) + kReportHead + (size_t)side_idx * 2 * ncnt;
+    side.win_class_cnt.assign(counts, counts + ncnt);
+    side.win_class_off.assign(counts + ncnt, counts + 2 * ncnt);
+    side.n_block_items = h.n_block;
+    side.n_items = h.n_block + h.n_wave;
+    side.n_split = h.n_split;
+    side.n_parts = h.n_parts;
+    side.n_groups = h.n_groups;
 }
 
 // ---------------------------------------------------------------------------
@@ -372,7 +471,7 @@ void append_side(std::vector<WaveDesc>& waves, float& cost, const Side& s, int w
     if (w < 0) return;
     for (int c = (part == 0 ? 0 : 1); c < (part == 0 ? 1 : kNumClass); ++c) {
         const uint32_t n = s.win_class_cnt[(size_t)w * (kNumClass + 1) + c];
-        const uint32_t first = s.n_block_items + s.win_class_off[(size_t)w * (kNumClass + 1) + c];
+        const uint32_t first = s.win_class_off[(size_t)w * (kNumClass + 1) + c];
         const uint32_t ipw = (uint32_t)rows_per_wave(lpe, c);
         for (uint32_t i = 0; i < n; i += ipw) {
             waves.push_back(WaveDesc{(int32_t)(first + i), desc_code((uint32_t)c, src_side, n - i < ipw ? n - i : ipw)});
@@ -383,7 +482,10 @@ void append_side(std::vector<WaveDesc>& waves, float& cost, const Side& s, int w
 
 // descriptors of all windows -> block order.  XCD x gets a contiguous range of windows; it first walks the
 // heavy share of all its windows (long work first keeps the end of the launch short), then window by window.
-int place(const std::vector<const Side*>& sides, int lpe, void** d_out, int32_t* n_blocks, hipStream_t st) {
+// `placed` and `desc_d` feed an asynchronous copy and the kernel behind it: the caller keeps them until the stream
+// has been synchronised.
+int place(const std::vector<const Side*>& sides, int lpe, void** d_out, int32_t* n_blocks, hipStream_t st,
+          std::vector<WaveDesc>& placed, DevBuf& desc_d) {
     const int nwin = sides[0]->n_windows;
     const bool heavy_first = env_int("TGT_HEAVY_FIRST", 1) == 1;
     std::vector<std::vector<std::vector<int32_t>>> homed(sides.size());
@@ -450,7 +552,7 @@ int place(const std::vector<const Side*>& sides, int lpe, void** d_out, int32_t*
     size_t per = 0;
     for (int x = 0; x < 8; ++x) per = std::max(per, xw[x].size() / 4);
     const size_t nb = per * 8;
-    std::vector<WaveDesc> placed(nb * 4 + 4, WaveDesc{0, kDescNone});
+    placed.assign(nb * 4 + 4, WaveDesc{0, kDescNone});
     for (int x = 0; x < 8; ++x)
         for (size_t b = 0; b < xw[x].size() / 4; ++b)
             for (int k = 0; k < 4; ++k) placed[(b * 8 + x) * 4 + k] = xw[x][b * 4 + k];
@@ -459,18 +561,16 @@ int place(const std::vector<const Side*>& sides, int lpe, void** d_out, int32_t*
     const size_t n_rec = nb * 4;
     *n_blocks = (int32_t)nb;
     if (n_rec == 0) return TGT_OK;
-    DevBuf desc_d;
-    TGT_HIP_CHECK(desc_d.alloc(sizeof(WaveDesc) * n_rec));
+    TGT_HIP_CHECK(desc_d.alloc(sizeof(WaveDesc) * n_rec, st));
     TGT_HIP_CHECK(hipMemcpyAsync(desc_d.p, placed.data(), sizeof(WaveDesc) * n_rec, hipMemcpyHostToDevice, st));
     const size_t bytes = n_rec * (size_t)L.stride * sizeof(int32_t);
-    TGT_HIP_CHECK(hipMalloc(d_out, bytes));
+    TGT_HIP_CHECK(dev_alloc(d_out, bytes, st));
     TGT_HIP_CHECK(hipMemsetAsync(*d_out, 0, bytes, st));
     const Side* sd = sides[0];
     const Side* ss = sides.size() > 1 ? sides[1] : sides[0];
     hipLaunchKernelGGL(k_build_records, dim3((unsigned)n_rec), dim3(64), 0, st, desc_d.as<WaveDesc>(), sd->items, ss->items,
-                       sd->col, sd->eid, ss->col, ss->eid, L, lpe, static_cast<int32_t*>(*d_out));
+                       sd->block_items, ss->block_items, sd->col, sd->eid, ss->col, ss->eid, L, lpe, static_cast<int32_t*>(*d_out));
     TGT_HIP_CHECK(hipGetLastError());
-    TGT_HIP_CHECK(hipStreamSynchronize(st));    // the descriptors are freed on return
     return TGT_OK;
 }
 }  // namespace
@@ -487,9 +587,20 @@ const Schedule* plan_schedule(const tgt_plan* plan_c, int lpe, hipStream_t st) {
     if (idx == kNumLpe) { set_error("no schedule for %d lanes per edge", lpe); return nullptr; }
     tgt_plan* plan = const_cast<tgt_plan*>(plan_c);
     Schedule& sc = plan->sched[idx];
+    // the descriptors of a shape are made once, whichever thread or stream asks first
+    std::lock_guard<std::mutex> lock(plan->sched_mutex);
     if (sc.ready) return &sc;
-    if (place({&plan->dst}, lpe, &sc.fwd, &sc.fwd_blocks, st) != TGT_OK) return nullptr;
-    if (place({&plan->dst, &plan->src}, lpe, &sc.bwd, &sc.bwd_blocks, st) != TGT_OK) return nullptr;
+    std::vector<WaveDesc> placed_f, placed_b;
+    DevBuf desc_f, desc_b;
+    int rc = place({&plan->dst}, lpe, &sc.fwd, &sc.fwd_blocks, st, placed_f, desc_f);
+    if (rc == TGT_OK) rc = place({&plan->dst, &plan->src}, lpe, &sc.bwd, &sc.bwd_blocks, st, placed_b, desc_b);
+    // the host vectors feed asynchronous copies: they may go once the stream is idle
+    if (hipStreamSynchronize(st) != hipSuccess && rc == TGT_OK) { set_error("hipStreamSynchronize failed"); rc = TGT_ERR_HIP; }
+    if (rc != TGT_OK) {
+        dev_free(sc.fwd); dev_free(sc.bwd);
+        sc = Schedule();
+        return nullptr;
+    }
     sc.ready = true;
     return &sc;
 }
@@ -525,22 +636,15 @@ __global__ void k_permute_rows(const V* __restrict__ in, const int32_t* __restri
 }
 
 static void free_side(Side& s) {
-    if (s.rowptr) (void)hipFree(s.rowptr);
-    if (s.col) (void)hipFree(s.col);
-    if (s.eid) (void)hipFree(s.eid);
-    if (s.pos) (void)hipFree(s.pos);
-    if (s.items) (void)hipFree(s.items);
-    if (s.split_row) (void)hipFree(s.split_row);
-    if (s.split_off) (void)hipFree(s.split_off);
-    if (s.part2split) (void)hipFree(s.part2split);
-    if (s.split_grp) (void)hipFree(s.split_grp);
+    dev_free(s.rowptr); dev_free(s.col); dev_free(s.eid); dev_free(s.pos);
+    dev_free(s.items); dev_free(s.block_items);
+    dev_free(s.split_row); dev_free(s.split_off); dev_free(s.part2split); dev_free(s.split_grp);
     s = Side();
 }
 
 static void free_schedules(tgt_plan* plan) {
     for (Schedule& sc : plan->sched) {
-        if (sc.fwd) (void)hipFree(sc.fwd);
-        if (sc.bwd) (void)hipFree(sc.bwd);
+        dev_free(sc.fwd); dev_free(sc.bwd);
         sc = Schedule();
     }
 }
@@ -551,44 +655,106 @@ static int create_impl(const int64_t* d_src, const int64_t* d_dst, int64_t E, in
     plan->E = E;
     TGT_HIP_CHECK(hipGetDevice(&plan->device));
     for (Side* s : {&plan->dst, &plan->src}) {
-        TGT_HIP_CHECK(hipMalloc((void**)&s->rowptr, sizeof(int32_t) * (N + 1)));
-        TGT_HIP_CHECK(hipMalloc((void**)&s->col, sizeof(int32_t) * (E ? E : 1)));
-        TGT_HIP_CHECK(hipMalloc((void**)&s->eid, sizeof(int32_t) * (E ? E : 1)));
+        TGT_HIP_CHECK(dev_alloc((void**)&s->rowptr, sizeof(int32_t) * (N + 1), st));
+        TGT_HIP_CHECK(dev_alloc((void**)&s->col, sizeof(int32_t) * (E ? E : 1), st));
+        TGT_HIP_CHECK(dev_alloc((void**)&s->eid, sizeof(int32_t) * (E ? E : 1), st));
     }
-    DevBuf s32, d32, flag;
+    DevBuf s32, d32, report_d;
     RadixSorter sorter;
     const size_t eb = sizeof(uint32_t) * (size_t)(E ? E : 1);
-    TGT_HIP_CHECK(s32.alloc(eb));
-    TGT_HIP_CHECK(d32.alloc(eb));
-    TGT_HIP_CHECK(flag.alloc(sizeof(int)));
+    TGT_HIP_CHECK(s32.alloc(eb, st));
+    TGT_HIP_CHECK(d32.alloc(eb, st));
     {
-        int rc0 = sorter.init(E);
+        int rc0 = sorter.init(E, st);
         if (rc0) return rc0;
     }
-    TGT_HIP_CHECK(hipMemsetAsync(flag.p, 0, sizeof(int), st));
+    // what comes back to the host, in one copy: the two schedule headers, the range-check flag, and per view the
+    // per-window row counts and their offsets
+    const int W = window_rows();
+    const int nwin = (int)((N + W - 1) / W);
+    const size_t report_ints = kReportHead + 4 * (size_t)kSchedCats * nwin;
+    TGT_HIP_CHECK(report_d.alloc(sizeof(int32_t) * report_ints, st));
+    TGT_HIP_CHECK(hipMemsetAsync(report_d.p, 0, sizeof(int32_t) * kReportHead, st));
+    int32_t* report = report_d.as<int32_t>();
     if (E > 0) {
         const int T = 256;
         hipLaunchKernelGGL(k_convert_validate, dim3((unsigned)((E + T - 1) / T)), dim3(T), 0, st, d_src,
-                           d_dst, E, N, s32.as<uint32_t>(), d32.as<uint32_t>(), flag.as<int>());
+                           d_dst, E, N, s32.as<uint32_t>(), d32.as<uint32_t>(), report + kReportFlag);
         TGT_HIP_CHECK(hipGetLastError());
     }
-    int h_flag = 0;
-    TGT_HIP_CHECK(hipMemcpyAsync(&h_flag, flag.p, sizeof(int), hipMemcpyDeviceToHost, st));
-    TGT_HIP_CHECK(hipStreamSynchronize(st));
-    if (h_flag) {
-        set_error("edge_index holds a node id outside [0, %lld)", (long long)N);
-        return TGT_ERR_INDEX_RANGE;
-    }
+    // out-of-range endpoints were replaced by node 0 (and flagged): everything below runs on valid ids
     int rc = build_side(d32.as<uint32_t>(), s32.as<uint32_t>(), E, N, sorter, plan->dst, st);
     if (rc) return rc;
     rc = build_side(s32.as<uint32_t>(), d32.as<uint32_t>(), E, N, sorter, plan->src, st);
     if (rc) return rc;
-    rc = build_schedule(N, plan->dst, st);
+    SideScratch scr_d, scr_s;
+    rc = schedule_device(N, E, plan->dst, scr_d, report, 0, st);
     if (rc) return rc;
-    rc = build_schedule(N, plan->src, st);
+    rc = schedule_device(N, E, plan->src, scr_s, report, 1, st);
     if (rc) return rc;
+    std::vector<int32_t> h_report(report_ints);
+    TGT_HIP_CHECK(hipMemcpyAsync(h_report.data(), report, sizeof(int32_t) * report_ints, hipMemcpyDeviceToHost, st));
+    TGT_HIP_CHECK(hipStreamSynchronize(st));
+    if (h_report[kReportFlag]) {
+        set_error("edge_index holds a node id outside [0, %lld)", (long long)N);
+        return TGT_ERR_INDEX_RANGE;
+    }
+    schedule_counts(plan->dst, scr_d, h_report.data(), 0);
+    schedule_counts(plan->src, scr_s, h_report.data(), 1);
+    // graphs with rows longer than a wave row: where their workgroup items go (second and last read-back)
+    std::vector<BlockMeta> meta_d(plan->dst.n_block_items), meta_s(plan->src.n_block_items);
+    if (!meta_d.empty())
+        TGT_HIP_CHECK(hipMemcpyAsync(meta_d.data(), scr_d.meta.p, sizeof(BlockMeta) * meta_d.size(), hipMemcpyDeviceToHost, st));
+    if (!meta_s.empty())
+        TGT_HIP_CHECK(hipMemcpyAsync(meta_s.data(), scr_s.meta.p, sizeof(BlockMeta) * meta_s.size(), hipMemcpyDeviceToHost, st));
+    if (!meta_d.empty() || !meta_s.empty()) TGT_HIP_CHECK(hipStreamSynchronize(st));
+    for (auto sm : {std::make_pair(&plan->dst, &meta_d), std::make_pair(&plan->src, &meta_s)}) {
+        Side& sd = *sm.first;
+        const std::vector<BlockMeta>& m = *sm.second;
+        sd.block_home.resize(m.size()); sd.block_len.resize(m.size()); sd.block_spread.resize(m.size());
+        for (size_t i = 0; i < m.size(); ++i) {
+            sd.block_home[i] = m[i].home; sd.block_len[i] = m[i].len; sd.block_spread[i] = (uint8_t)m[i].spread;
+        }
+    }
     // the shape of the reference's node-level models (hidden 64: 8 heads of 8, or 4 of 16); other shapes on first use
     return plan_schedule(plan, 8, st) ? TGT_OK : TGT_ERR_HIP;
+}
+
+// ---------------------------------------------------------------------------
+// content key of an edge list
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ uint64_t mix64(uint64_t x) {
+    x ^= x >> 33; x *= 0xff51afd7ed558ccdull;
+    x ^= x >> 33; x *= 0xc4ceb9fe1a85ec53ull;
+    x ^= x >> 33;
+    return x;
+}
+constexpr int kHashBlocks = 1024;
+// Two 64-bit sums over all 2E endpoints of mixed (value, position) pairs: a sum does not depend on the order
+// of the additions, so the key is the same whatever the grid does, and a value that moves or changes moves it.
+__global__ __launch_bounds__(256) void k_hash_partial(const int64_t* __restrict__ src, const int64_t* __restrict__ dst,
+                                                      int64_t E, uint64_t* __restrict__ partial) {
+    __shared__ uint64_t sh[2][4];
+    uint64_t a = 0, b = 0;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < 2 * E; i += (int64_t)gridDim.x * blockDim.x) {
+        const uint64_t v = (uint64_t)(i < E ? src[i] : dst[i - E]);
+        a += mix64(v * 0x9e3779b97f4a7c15ull + (uint64_t)i * 0xd6e8feb86659fd93ull + 0x2545f4914f6cdd1dull);
+        b += mix64((v + (uint64_t)i * 0xa0761d6478bd642full) ^ 0xe7037ed1a0b428dbull);
+    }
+    for (int off = 32; off > 0; off >>= 1) { a += __shfl_xor(a, off); b += __shfl_xor(b, off); }
+    if ((threadIdx.x & 63) == 0) { sh[0][threadIdx.x >> 6] = a; sh[1][threadIdx.x >> 6] = b; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        partial[2 * blockIdx.x] = sh[0][0] + sh[0][1] + sh[0][2] + sh[0][3];
+        partial[2 * blockIdx.x + 1] = sh[1][0] + sh[1][1] + sh[1][2] + sh[1][3];
+    }
+}
+__global__ __launch_bounds__(64) void k_hash_final(const uint64_t* __restrict__ partial, int n, int64_t E,
+                                                   uint64_t* __restrict__ out) {
+    uint64_t a = 0, b = 0;
+    for (int i = threadIdx.x; i < n; i += 64) { a += partial[2 * i]; b += partial[2 * i + 1]; }
+    for (int off = 32; off > 0; off >>= 1) { a += __shfl_xor(a, off); b += __shfl_xor(b, off); }
+    if (threadIdx.x == 0) { out[0] = mix64(a ^ (uint64_t)E); out[1] = mix64(b + (uint64_t)E); }
 }
 
 }  // namespace tgt
@@ -605,17 +771,16 @@ int tgt_plan_enable_bias_order(tgt_plan_t* plan, void* stream) {
     if (plan->src.pos) return TGT_OK;
     const int64_t E = plan->E;
     hipStream_t st = (hipStream_t)stream;
-    TGT_HIP_CHECK(hipMalloc((void**)&plan->src.pos, sizeof(int32_t) * (size_t)(E ? E : 1)));
+    TGT_HIP_CHECK(tgt::dev_alloc((void**)&plan->src.pos, sizeof(int32_t) * (size_t)(E ? E : 1), st));
     if (E == 0) return TGT_OK;
     tgt::DevBuf inv;
-    TGT_HIP_CHECK(inv.alloc(sizeof(int32_t) * (size_t)E));
+    TGT_HIP_CHECK(inv.alloc(sizeof(int32_t) * (size_t)E, st));
     const unsigned grid = (unsigned)((E + 255) / 256);
     hipLaunchKernelGGL(tgt::k_invert_perm, dim3(grid), dim3(256), 0, st, plan->dst.eid, E, inv.as<int32_t>());
     hipLaunchKernelGGL(tgt::k_compose_perm, dim3(grid), dim3(256), 0, st, plan->src.eid, inv.as<int32_t>(), E,
                        plan->src.pos);
     TGT_HIP_CHECK(hipGetLastError());
-    TGT_HIP_CHECK(hipStreamSynchronize(st));      // the scratch buffer is freed on return
-    return TGT_OK;
+    return TGT_OK;      // the scratch buffer goes back to its allocator behind the kernels that read it
 }
 
 const char* tgt_error_string(int code) {
@@ -631,6 +796,24 @@ const char* tgt_error_string(int code) {
 }
 
 const char* tgt_last_error(void) { return tgt::last_error(); }
+
+int tgt_edge_index_hash(const int64_t* d_src, const int64_t* d_dst, int64_t E, void* stream, uint64_t h_key[2]) {
+    if (!h_key || E < 0 || (E > 0 && (!d_src || !d_dst))) {
+        tgt::set_error("tgt_edge_index_hash: null pointer or E < 0");
+        return TGT_ERR_INVALID_ARG;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    const int nb = (int)std::min<int64_t>(tgt::kHashBlocks, std::max<int64_t>(1, (2 * E + 1023) / 1024));
+    tgt::DevBuf buf;
+    TGT_HIP_CHECK(buf.alloc(sizeof(uint64_t) * (2 * (size_t)nb + 2), st));
+    uint64_t* partial = buf.as<uint64_t>();
+    hipLaunchKernelGGL(tgt::k_hash_partial, dim3(nb), dim3(256), 0, st, d_src, d_dst, E, partial);
+    hipLaunchKernelGGL(tgt::k_hash_final, dim3(1), dim3(64), 0, st, partial, nb, E, partial + 2 * nb);
+    TGT_HIP_CHECK(hipGetLastError());
+    TGT_HIP_CHECK(hipMemcpyAsync(h_key, partial + 2 * nb, 2 * sizeof(uint64_t), hipMemcpyDeviceToHost, st));
+    TGT_HIP_CHECK(hipStreamSynchronize(st));
+    return TGT_OK;
+}
 
 int tgt_plan_create(const int64_t* d_src, const int64_t* d_dst, int64_t E, int64_t N, void* stream,
                     tgt_plan_t** out_plan) {
@@ -702,6 +885,14 @@ int tgt_plan_export(const tgt_plan_t* plan, int which, int32_t* h_out, int64_t c
         tgt::set_error("tgt_plan_export: bad array id or capacity");
         return TGT_ERR_INVALID_ARG;
     }
+    if (n == 0) return TGT_OK;
+    if (which == TGT_PLAN_ITEMS_DST || which == TGT_PLAN_ITEMS_SRC) {   // workgroup items, then wave items
+        const tgt::Side& s = which == TGT_PLAN_ITEMS_DST ? plan->dst : plan->src;
+        const int64_t nb = 4 * (int64_t)s.n_block_items;
+        if (nb > 0) TGT_HIP_CHECK(hipMemcpy(h_out, s.block_items, sizeof(int32_t) * nb, hipMemcpyDeviceToHost));
+        if (n > nb) TGT_HIP_CHECK(hipMemcpy(h_out + nb, s.items, sizeof(int32_t) * (n - nb), hipMemcpyDeviceToHost));
+        return TGT_OK;
+    }
     const void* p = nullptr;
     switch (which) {
         case TGT_PLAN_ROWPTR_DST: p = plan->dst.rowptr; break;
@@ -711,10 +902,7 @@ int tgt_plan_export(const tgt_plan_t* plan, int which, int32_t* h_out, int64_t c
         case TGT_PLAN_COL_SRC: p = plan->src.col; break;
         case TGT_PLAN_EID_SRC: p = plan->src.eid; break;
         case TGT_PLAN_POS_SRC: p = plan->src.pos; break;
-        case TGT_PLAN_ITEMS_DST: p = plan->dst.items; break;
-        case TGT_PLAN_ITEMS_SRC: p = plan->src.items; break;
     }
-    if (n == 0) return TGT_OK;
     TGT_HIP_CHECK(hipMemcpy(h_out, p, sizeof(int32_t) * n, hipMemcpyDeviceToHost));
     return TGT_OK;
 }

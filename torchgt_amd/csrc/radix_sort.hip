@@ -6,6 +6,9 @@
 // Used for the CSR/CSC build (keys = destination / source node) and for the
 // graph reordering (keys = partition id, new source id).
 #include "common.h"
+#include <mutex>
+#include <unordered_map>
+#include <utility>
 
 namespace tgt {
 
@@ -157,11 +160,44 @@ __global__ __launch_bounds__(RS_THREADS) void k_rs_scatter(
 }
 
 
-hipError_t DevBuf::alloc(size_t bytes) {
-    if (p) { (void)hipFree(p); p = nullptr; }
-    return hipMalloc(&p, bytes ? bytes : 4);
+// allocator hooks (tgt_set_allocator); read on every call, set before the first plan is made
+static tgt_alloc_fn g_alloc = nullptr;
+static tgt_free_fn g_free = nullptr;
+static void* g_alloc_user = nullptr;
+// what the hook handed out and has not taken back: memory goes back to where it came from even if the
+// hooks were set or cleared in between
+static std::mutex g_hooked_mutex;
+static std::unordered_map<void*, std::pair<tgt_free_fn, void*>> g_hooked;
+
+hipError_t dev_alloc(void** p, size_t bytes, hipStream_t st) {
+    if (bytes == 0) bytes = 4;
+    const tgt_alloc_fn alloc = g_alloc;
+    if (alloc) {
+        *p = alloc(bytes, (void*)st, g_alloc_user);
+        if (!*p) return hipErrorOutOfMemory;
+        std::lock_guard<std::mutex> lock(g_hooked_mutex);
+        g_hooked[*p] = std::make_pair(g_free, g_alloc_user);
+        return hipSuccess;
+    }
+    return hipMalloc(p, bytes);
 }
-DevBuf::~DevBuf() { if (p) (void)hipFree(p); }
+void dev_free(void* p) {
+    if (!p) return;
+    std::pair<tgt_free_fn, void*> how(nullptr, nullptr);
+    {
+        std::lock_guard<std::mutex> lock(g_hooked_mutex);
+        auto it = g_hooked.find(p);
+        if (it != g_hooked.end()) { how = it->second; g_hooked.erase(it); }
+    }
+    if (how.first) how.first(p, how.second);
+    else (void)hipFree(p);
+}
+
+hipError_t DevBuf::alloc(size_t bytes, hipStream_t st) {
+    if (p) { dev_free(p); p = nullptr; }
+    return dev_alloc(&p, bytes, st);
+}
+DevBuf::~DevBuf() { dev_free(p); }
 
 int bits_for(int64_t n) {
     int bits = 1;
@@ -169,16 +205,16 @@ int bits_for(int64_t n) {
     return bits;
 }
 
-int RadixSorter::init(int64_t n) {
+int RadixSorter::init(int64_t n, hipStream_t st) {
     cap_ = n > 0 ? n : 1;
     nblocks_ = (int)((cap_ + RS_TILE - 1) / RS_TILE);
     const size_t eb = sizeof(uint32_t) * (size_t)cap_;
-    TGT_HIP_CHECK(keysA_.alloc(eb));
-    TGT_HIP_CHECK(keysB_.alloc(eb));
-    TGT_HIP_CHECK(valsA_.alloc(eb));
-    TGT_HIP_CHECK(valsB_.alloc(eb));
-    TGT_HIP_CHECK(hist_.alloc(sizeof(uint32_t) * 256 * (size_t)nblocks_));
-    TGT_HIP_CHECK(totals_.alloc(sizeof(uint32_t) * 256));
+    TGT_HIP_CHECK(keysA_.alloc(eb, st));
+    TGT_HIP_CHECK(keysB_.alloc(eb, st));
+    TGT_HIP_CHECK(valsA_.alloc(eb, st));
+    TGT_HIP_CHECK(valsB_.alloc(eb, st));
+    TGT_HIP_CHECK(hist_.alloc(sizeof(uint32_t) * 256 * (size_t)nblocks_, st));
+    TGT_HIP_CHECK(totals_.alloc(sizeof(uint32_t) * 256, st));
     return TGT_OK;
 }
 
@@ -212,3 +248,14 @@ int RadixSorter::sort(const uint32_t* keys_in, const uint32_t* vals_in, int64_t 
 }
 
 }  // namespace tgt
+
+extern "C" int tgt_set_allocator(tgt_alloc_fn alloc, tgt_free_fn free_fn, void* user) {
+    if ((alloc == nullptr) != (free_fn == nullptr)) {
+        tgt::set_error("tgt_set_allocator: give both functions or neither");
+        return TGT_ERR_INVALID_ARG;
+    }
+    tgt::g_alloc = alloc;
+    tgt::g_free = free_fn;
+    tgt::g_alloc_user = user;
+    return TGT_OK;
+}

@@ -678,27 +678,6 @@ __device__ __forceinline__ void block_item(const Common& c, const SideArgs& s, c
     if (tid < LPE) write_row<T, LPE, LPH, MODE, TILES>(c, s, it.row, tid, acc);
 }
 
-#ifdef TGT_TRACE
-// Experiments only (-DTGT_TRACE): every wave records when it ran and where, 4 x uint64 per wave at
-// g_trace[4 * (4 * workgroup + wave)]: start, end (100 MHz clock), (XCC id << 32 | HW id), descriptor code.
-__device__ uint64_t* g_trace = nullptr;
-struct TraceScope {
-    uint64_t t0; uint32_t code; int idx;
-    __device__ TraceScope(uint32_t c) : t0(wall_clock64()), code(c), idx(blockIdx.x * 4 + (threadIdx.x >> 6)) {}
-    __device__ ~TraceScope() {
-        if (g_trace && (threadIdx.x & 63) == 0) {
-            uint64_t* p = g_trace + 4 * (int64_t)idx;
-            p[0] = t0; p[1] = wall_clock64();
-            p[2] = ((uint64_t)__builtin_amdgcn_s_getreg((3 << 11) | 20) << 32) | (uint32_t)__builtin_amdgcn_s_getreg((31 << 11) | 4);
-            p[3] = code;
-        }
-    }
-};
-#define TGT_TRACE_SCOPE(code) TraceScope trace_scope_(code)
-#else
-#define TGT_TRACE_SCOPE(code)
-#endif
-
 // Forward.  Workgroup b does what the records 4b .. 4b+3 say: one workgroup item, or four waves of
 // rows.  Which rows meet in which workgroup, on which XCD and when is the plan's business.
 template <typename T, int LPE, int LPH, int HASB, bool TILES>
@@ -708,14 +687,12 @@ __global__ __launch_bounds__(kBlock) void k_attn_fwd(const Common c, const SideA
     const WaveRec<LPE>* r0 = recs + (int64_t)blockIdx.x * (kBlock / kWave);
     const uint32_t code0 = r0->code;
     if ((code0 & 7u) == kDescBlock) {          // uniform over the workgroup
-        TGT_TRACE_SCOPE(code0);
         block_item<T, LPE, LPH, MODE_FWD, HASB, TILES>(c, s, r0->item, lds);
         return;
     }
     const WaveRec<LPE>& rec = r0[threadIdx.x >> 6];
     const uint32_t code = __builtin_amdgcn_readfirstlane(rec.code);
     if ((code & 7u) == kDescNone) return;
-    TGT_TRACE_SCOPE(code);
     wave_dispatch<T, LPE, LPH, MODE_FWD, HASB, TILES>(c, s, rec, code & 7u);
 }
 
@@ -729,7 +706,6 @@ __global__ __launch_bounds__(kBlock, 4) void k_attn_bwd(const Common c, const Si
     const WaveRec<LPE>* r0 = recs + (int64_t)blockIdx.x * (kBlock / kWave);
     const uint32_t code0 = r0->code;
     if ((code0 & 7u) == kDescBlock) {          // uniform over the workgroup
-        TGT_TRACE_SCOPE(code0);
         if (code0 & kDescSrcSide) block_item<T, LPE, LPH, MODE_BWD_SRC, HB_S, TILES>(c, ss, r0->item, lds);
         else block_item<T, LPE, LPH, MODE_BWD_DST, HB_D, TILES>(c, sd, r0->item, lds);
         return;
@@ -737,7 +713,6 @@ __global__ __launch_bounds__(kBlock, 4) void k_attn_bwd(const Common c, const Si
     const WaveRec<LPE>& rec = r0[threadIdx.x >> 6];
     const uint32_t code = __builtin_amdgcn_readfirstlane(rec.code);
     if ((code & 7u) == kDescNone) return;
-    TGT_TRACE_SCOPE(code);
     if (code & kDescSrcSide) wave_dispatch<T, LPE, LPH, MODE_BWD_SRC, HB_S, TILES>(c, ss, rec, code & 7u);
     else wave_dispatch<T, LPE, LPH, MODE_BWD_DST, HB_D, TILES>(c, sd, rec, code & 7u);
 }
@@ -1163,16 +1138,6 @@ int sparse_attn_fwd_noalloc_impl(const tgt_plan_t* plan, const void* d_q, const 
 
 #if !defined(TGT_SPARSE_PART) || TGT_SPARSE_PART == 0
 extern "C" {
-
-#ifdef TGT_TRACE
-int tgt_debug_trace(uint64_t* d_buf) {
-    return hipMemcpyToSymbol(HIP_SYMBOL(tgt::g_trace), &d_buf, sizeof(d_buf)) == hipSuccess ? 0 : -4;
-}
-int tgt_debug_grid(const tgt_plan_t* plan, int lpe, int bwd) {
-    const tgt::Schedule* s = tgt::plan_schedule(plan, lpe, nullptr);
-    return s ? (bwd ? s->bwd_blocks : s->fwd_blocks) : -1;
-}
-#endif
 
 int64_t tgt_sparse_attn_workspace_bytes(const tgt_plan_t* plan, int H, int d) {
     if (!plan || H < 1 || d < 1) return -1;

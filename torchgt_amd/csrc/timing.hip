@@ -12,7 +12,7 @@
 namespace tgt {
 
 static const char* kSlotNames[KS_COUNT] = {
-    "attn_fwd", "bwd_node_side", "attn_bwd", "dense_fwd", "dense_bwd", "tile_fwd", "tile_bwd", "probe_row_gather",
+    "attn_fwd", "bwd_node_side", "attn_bwd", "dense_fwd", "dense_bwd", "tile_fwd", "tile_bwd",
     "linear_fwd", "linear_dx", "linear_dw", "layer_norm_fwd", "layer_norm_bwd", "gelu",
     "graph_bias_fwd", "graph_bias_bwd", "nll_loss",
 };
@@ -70,57 +70,9 @@ static void drain() {
     g_pending.clear();
 }
 
-// Row-gather probe: the access pattern of the sparse walk with nothing else around it.  Eight
-// lanes read one row of 128 * VPL bytes picked by idx[], four rows in flight per lane group.
-template <int VPL>
-__global__ __launch_bounds__(kBlock) void k_probe_row_gather(const uint4* __restrict__ table,
-                                                             const int32_t* __restrict__ idx, int64_t n_groups,
-                                                             uint32_t* __restrict__ sink) {
-    constexpr int U = 4;
-    const int64_t g = ((int64_t)blockIdx.x * kBlock + threadIdx.x) >> 3;
-    const int l = threadIdx.x & 7;
-    if (g >= n_groups) return;
-    int id[U];
-#pragma unroll
-    for (int u = 0; u < U; ++u) id[u] = idx[g * U + u];
-    uint4 x[U][VPL];
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-        for (int v = 0; v < VPL; ++v) x[u][v] = table[((int64_t)id[u] * 8 + l) * VPL + v];
-    uint32_t a = 0;
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-        for (int v = 0; v < VPL; ++v) a ^= x[u][v].x ^ x[u][v].y ^ x[u][v].z ^ x[u][v].w;
-    if (a == 0x9e3779b9u) sink[0] = a;   // keeps the loads alive; practically never taken
-}
-
 }  // namespace tgt
 
 extern "C" {
-
-int tgt_probe_row_gather(const void* d_table, int64_t n_rows, int row_bytes, const int32_t* d_idx, int64_t n_idx,
-                         void* d_sink, void* stream) {
-    if (!d_table || !d_idx || !d_sink || n_rows < 1 || n_idx < 4 || (row_bytes != 128 && row_bytes != 256)) {
-        tgt::set_error("tgt_probe_row_gather: null pointer, fewer than 4 indices, or row_bytes not 128 / 256");
-        return TGT_ERR_INVALID_ARG;
-    }
-    hipStream_t st = (hipStream_t)stream;
-    const int64_t n_groups = n_idx / 4;
-    const unsigned nb = (unsigned)((n_groups * 8 + tgt::kBlock - 1) / tgt::kBlock);
-    {
-        tgt::KernelTimer t(tgt::KS_PROBE_GATHER, st);
-        if (row_bytes == 128)
-            hipLaunchKernelGGL((tgt::k_probe_row_gather<1>), dim3(nb), dim3(tgt::kBlock), 0, st,
-                               (const uint4*)d_table, d_idx, n_groups, (uint32_t*)d_sink);
-        else
-            hipLaunchKernelGGL((tgt::k_probe_row_gather<2>), dim3(nb), dim3(tgt::kBlock), 0, st,
-                               (const uint4*)d_table, d_idx, n_groups, (uint32_t*)d_sink);
-    }
-    TGT_HIP_CHECK(hipGetLastError());
-    return TGT_OK;
-}
 
 int tgt_timing_enable(int on) {
     std::lock_guard<std::mutex> lk(tgt::g_mu);

@@ -21,6 +21,7 @@
 #include <torch/autograd.h>
 #include <ATen/ATen.h>
 #include <c10/hip/HIPStream.h>
+#include <c10/hip/HIPCachingAllocator.h>
 #include <c10/core/DeviceGuard.h>
 
 #include "../../include/torchgt_hip.h"
@@ -44,6 +45,21 @@ const void* ptr(const c10::optional<Tensor>& t) { return (t.has_value() && t->de
 void on_gpu(const Tensor& t, const char* op) {
     TORCH_CHECK(t.is_cuda(), op, " needs GPU tensors (there is no CPU implementation)");
 }
+
+// The library's own device memory (plans, tile sets, scratch of the edge preparation) comes from torch's caching
+// allocator once this extension is loaded: a plan built per training iteration then costs no hipMalloc / hipFree.
+void* torch_alloc(size_t bytes, void* stream, void*) {
+    try {
+        return c10::hip::HIPCachingAllocator::raw_alloc_with_stream(bytes, static_cast<hipStream_t>(stream));
+    } catch (const std::exception&) {
+        return nullptr;
+    }
+}
+void torch_free(void* p, void*) { c10::hip::HIPCachingAllocator::raw_delete(p); }
+struct AllocatorRegistration {
+    AllocatorRegistration() { tgt_set_allocator(&torch_alloc, &torch_free, nullptr); }
+};
+const AllocatorRegistration allocator_registration;
 
 // Owner of a tgt_plan_t: the Python plan object holds one, and so does every autograd node that will need the plan
 // in its backward - the plan lives until the last of them lets go.

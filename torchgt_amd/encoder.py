@@ -23,31 +23,6 @@ from .multi_head_attention import MultiHeadAttention, fused_linear, _DT
 from .plan import GraphPlan, get_plan
 
 
-class AddLayerNormFunction:
-    """``s = x + r`` (r may be None) and ``y = LayerNorm(s)`` in one pass; returns (s, y):
-    ``torch.ops.torchgt.add_layer_norm`` (C++ autograd function over ``tgt_add_layer_norm_fwd`` / ``tgt_layer_norm_bwd``)."""
-
-    @staticmethod
-    def apply(x, r, gamma, beta, eps):
-        return _ext.ops().add_layer_norm(x, r, gamma, beta, float(eps))
-
-
-class AddFunction:
-    """``x + r`` through the same kernel (no normalisation)."""
-
-    @staticmethod
-    def apply(x, r):
-        return _ext.ops().add(x, r)
-
-
-class GeluFunction:
-    """Exact (erf) GELU: ``torch.ops.torchgt.gelu``."""
-
-    @staticmethod
-    def apply(u):
-        return _ext.ops().gelu(u)
-
-
 def nll_loss(log_probs, target, ignore_index=-100):
     """``F.nll_loss(log_probs, target)`` of the training and evaluation loops (main_sp_sparse_node_level.py:200,
     gt_sp/evaluate.py:52): mean over the rows whose target is not ``ignore_index``, no class weights.
@@ -81,7 +56,7 @@ class FeedForwardNetwork(nn.Module):
             # one operator: GELU in the epilogue of layer1 (64 -> 64) and in the input gradient of layer2
             return _ext.ops().ffn(x, l1.weight, l1.bias, l2.weight, l2.bias)
         (u,) = fused_linear(x, l1)
-        h = GeluFunction.apply(u)
+        h = _ext.ops().gelu(u)
         (y,) = fused_linear(h, l2)
         return y
 
@@ -129,16 +104,16 @@ class EncoderLayer(nn.Module):
             plan.handle      # raises if the plan was closed
             x, y = _ext.ops().encoder_layer(x, residual, params, plan.holder, plan.workspace(att.num_heads, att.att_size),
                                             att.num_heads, n1.eps, n2.eps)
-            return (x, y) if defer_residual else AddFunction.apply(x, y)
-        x, y = AddLayerNormFunction.apply(x, residual, n1.weight, n1.bias, n1.eps)
+            return (x, y) if defer_residual else _ext.ops().add(x, y)
+        x, y = _ext.ops().add_layer_norm(x, residual, n1.weight, n1.bias, float(n1.eps))
         y = self.self_attention(y, attn_bias, edge_index, attn_type=attn_type)
         y = self.self_attention_dropout(y)
-        x, y = AddLayerNormFunction.apply(x, y, n2.weight, n2.bias, n2.eps)
+        x, y = _ext.ops().add_layer_norm(x, y, n2.weight, n2.bias, float(n2.eps))
         y = self.ffn(y)
         y = self.ffn_dropout(y)
         if defer_residual:
             return x, y
-        return AddFunction.apply(x, y)
+        return _ext.ops().add(x, y)
 
 
 class Graphormer(nn.Module):
@@ -187,7 +162,7 @@ class Graphormer(nn.Module):
             output, pending = enc_layer(output, attn_bias=graph_attn_bias, edge_index=edge_index, attn_type=attn_type,
                                         residual=pending, defer_residual=True)
         fl = self.final_ln
-        _, output = AddLayerNormFunction.apply(output, pending, fl.weight, fl.bias, fl.eps)
+        _, output = _ext.ops().add_layer_norm(output, pending, fl.weight, fl.bias, float(fl.eps))
         # rows 1.. of graph 0 (:391 `output[0, 1:, :]`); through a view, so that autograd pads the gradient once, not twice
         (output,) = fused_linear(output.reshape(-1, self.hidden_dim)[1:output.shape[1]], self.downstream_out_proj)
         return F.log_softmax(output, dim=1)

@@ -11,7 +11,7 @@ import torch.nn as nn
 
 from . import _ext, _lib
 from .core_attention import GraphBiasIds
-from .encoder import AddFunction, AddLayerNormFunction, FeedForwardNetwork, init_params
+from .encoder import FeedForwardNetwork, init_params
 from .graph_bias import GraphAttnBias
 from .multi_head_attention import MultiHeadAttention, fused_linear
 
@@ -144,20 +144,20 @@ class EncoderLayer(nn.Module):
             try:
                 x2, y = _ext.ops().dense_encoder_layer(x, residual, params, extra, ab, sp16, et16, att.num_heads, n1.eps, n2.eps, p,
                                                        seed, bool(core.dense_bf16_products))
-                return (x2, y) if defer_residual else AddFunction.apply(x2, y)
+                return (x2, y) if defer_residual else _ext.ops().add(x2, y)
             except RuntimeError as exc:
                 if sp16 is None or "bytes of LDS" not in str(exc):
                     raise
                 attn_bias.fits = False       # this shape needs the bias tensor: the attention below builds it once
-        x, y = AddLayerNormFunction.apply(x, residual, n1.weight, n1.bias, n1.eps)
+        x, y = _ext.ops().add_layer_norm(x, residual, n1.weight, n1.bias, float(n1.eps))
         y = self.self_attention(y, attn_bias, None, attn_type="full")
         y = self.self_attention_dropout(y)
-        x, y = AddLayerNormFunction.apply(x, y, n2.weight, n2.bias, n2.eps)
+        x, y = _ext.ops().add_layer_norm(x, y, n2.weight, n2.bias, float(n2.eps))
         y = self.ffn(y)
         y = self.ffn_dropout(y)
         if defer_residual:
             return x, y
-        return AddFunction.apply(x, y)
+        return _ext.ops().add(x, y)
 
 
 class Graphormer(nn.Module):
@@ -200,7 +200,7 @@ class Graphormer(nn.Module):
         for enc_layer in self.layers:
             output, pending = enc_layer(output, attn_bias, mask=None, residual=pending, defer_residual=True)
         fl = self.final_ln
-        _, output = AddLayerNormFunction.apply(output, pending, fl.weight, fl.bias, fl.eps)
+        _, output = _ext.ops().add_layer_norm(output, pending, fl.weight, fl.bias, float(fl.eps))
         head = self.out_proj if hasattr(self, "out_proj") else self.downstream_out_proj
         (output,) = fused_linear(output[:, 0, :].contiguous(), head)      # the virtual node's row (:387)
         return output

@@ -10,7 +10,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from . import _ext, _lib
-from .encoder import AddLayerNormFunction, init_params
+from .encoder import init_params
 from .multi_head_attention import MultiHeadAttention, fused_linear
 
 _DT = {torch.float32: _lib.DTYPE_F32, torch.bfloat16: _lib.DTYPE_BF16}
@@ -49,12 +49,12 @@ class EncoderLayer(nn.Module):
         y = self.self_attention(x, attn_bias, edge_index=edge_index, attn_type=attn_type)      # :244
         y = self.self_attention_dropout(y)
         (y,) = fused_linear(y, self.O)                                                         # :246
-        _, x = AddLayerNormFunction.apply(x, y, n1.weight, n1.bias, n1.eps)                    # :247-248
+        _, x = _ext.ops().add_layer_norm(x, y, n1.weight, n1.bias, float(n1.eps))                    # :247-248
         (y,) = fused_linear(y, self.FFN_layer1)                                                # :254
         y = ReluFunction.apply(y)
         y = self.self_attention_dropout(y)
         (y,) = fused_linear(y, self.FFN_layer2)
-        _, x = AddLayerNormFunction.apply(x, y, n2.weight, n2.bias, n2.eps)                    # :258-259
+        _, x = _ext.ops().add_layer_norm(x, y, n2.weight, n2.bias, float(n2.eps))                    # :258-259
         return x
 
 

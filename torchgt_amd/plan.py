@@ -9,6 +9,7 @@ of a step and by all steps of a pre-packed batch
 """
 import collections
 import ctypes
+import weakref
 
 import numpy as np
 import torch
@@ -31,6 +32,7 @@ class GraphPlan:
         self.device = ei.device
         self._handle = ctypes.c_void_p()
         self._workspaces = {}
+        _ext.ops()                       # registers torch's caching allocator with the library: no hipMalloc per plan
         L = _lib.lib()
         with torch.cuda.device(self.device):
             stream = torch.cuda.current_stream(self.device).cuda_stream
@@ -40,7 +42,6 @@ class GraphPlan:
                                          ctypes.byref(self._handle)))
         # the owner of the C plan: shared with every autograd node that needs the plan in its backward, so that
         # the plan outlives this object if a backward is still pending
-        _ext.ops()
         self.holder = torch.classes.torchgt.PlanHolder(self._handle.value)
 
     @property
@@ -164,8 +165,10 @@ class _SortRows(torch.autograd.Function):
         return ctx.plan._permute(g[:E], 1), None, None     # only the destination-sorted rows carry a gradient
 
 
-_CACHE = collections.OrderedDict()
-_CACHE_BYTES = 1 << 30        # device memory the cached plans (and the edge_index tensors they were built from) may hold
+_CACHE = collections.OrderedDict()      # content key -> (plan, bytes)
+_BY_TENSOR = {}                          # id(tensor) -> (weak reference, version, plan): the layers of one step
+_CACHE_BYTES = 1 << 30                   # device memory the cached plans may hold
+_STATS = {"builds": 0, "content_hits": 0, "tensor_hits": 0}
 
 
 def set_plan_cache_bytes(nbytes):
@@ -176,38 +179,86 @@ def set_plan_cache_bytes(nbytes):
     _evict()
 
 
-def _plan_bytes(plan, edge_index):
-    # two sorted views (rowptr, col, eid), items, wave records of one shape, and the edge_index kept alive
-    return 56 * plan.num_edges + 450 * plan.num_nodes + edge_index.numel() * edge_index.element_size()
+def plan_cache_stats():
+    """Counters since the last ``clear_plan_cache``: plans built, look-ups answered by the content key, look-ups
+    answered by the tensor itself."""
+    return dict(_STATS)
+
+
+def _plan_bytes(plan):
+    # two sorted views (rowptr, col, eid), items, wave records of one shape
+    return 56 * plan.num_edges + 450 * plan.num_nodes
 
 
 def _evict():
-    total = sum(v[2] for v in _CACHE.values())
+    total = sum(v[1] for v in _CACHE.values())
     while len(_CACHE) > 1 and total > _CACHE_BYTES:
-        _, (_, _, nbytes) = _CACHE.popitem(last=False)      # freed when its last user (a pending backward) lets go
+        _, (gone, nbytes) = _CACHE.popitem(last=False)      # freed when its last user (a pending backward) lets go
         total -= nbytes
+        for tid in [t for t, ent in _BY_TENSOR.items() if ent[2] is gone]:
+            del _BY_TENSOR[tid]
+
+
+def edge_index_key(edge_index):
+    """128-bit content key of ``edge_index`` (values and positions), computed on the GPU."""
+    ei = edge_index if (edge_index.dtype == torch.int64 and edge_index.is_contiguous()) else edge_index.to(torch.int64).contiguous()
+    E = int(ei.size(1))
+    key = (ctypes.c_uint64 * 2)()
+    with torch.cuda.device(ei.device):
+        _ext.ops()
+        _lib.check(_lib.lib().tgt_edge_index_hash(ei[0].data_ptr() if E else None, ei[1].data_ptr() if E else None, E,
+                                                  torch.cuda.current_stream(ei.device).cuda_stream, key))
+    return int(key[0]), int(key[1])
 
 
 def get_plan(edge_index, num_nodes):
-    """Plan for ``edge_index``, cached on (storage address, shape, version, N) so
-    that the layers of a model and the iterations over a pre-packed batch share
-    one plan.  The cache keeps the tensor alive, so the address cannot be reused; it is bounded by bytes
-    (``set_plan_cache_bytes``), least recently used plans go first.  A driver that moves a fresh edge_index
-    to the GPU for every iteration therefore holds one large plan at a time, not sixteen.  Build plans before
-    capturing a HIP graph: building one allocates and synchronises."""
-    key = (edge_index.data_ptr(), tuple(edge_index.shape), edge_index._version, edge_index.dtype,
-           str(edge_index.device), int(num_nodes))
+    """Plan for ``edge_index``, shared by the layers of a model and by the iterations over a pre-packed batch.
+
+    The cache is keyed on the CONTENT of ``edge_index`` (a 128-bit key computed by two small kernels and one
+    16-byte read-back), so a driver that moves the same CPU-resident edge list to the GPU in every iteration -
+    the reference's loops do (main_sp_sparse_node_level.py:178-183, gt_sp/utils.py:455-458) - gets the plan it
+    built the first time.  The tensor object itself is remembered through a weak reference (no hashing for the
+    second and later layers of a step; the tensor is not kept alive).  The cache is bounded by bytes
+    (``set_plan_cache_bytes``), least recently used plans go first.  Build plans before capturing a HIP graph:
+    the look-up synchronises the stream, building allocates."""
+    ent = _BY_TENSOR.get(id(edge_index))
+    if ent is not None:
+        ref, version, plan, n = ent
+        if ref() is edge_index and version == edge_index._version and n == int(num_nodes) and plan._handle:
+            _STATS["tensor_hits"] += 1
+            return plan
+    if not edge_index.is_cuda:
+        raise RuntimeError("get_plan needs edge_index on the GPU (there is no CPU implementation)")
+    key = (edge_index_key(edge_index), tuple(edge_index.shape), str(edge_index.device), int(num_nodes))
     hit = _CACHE.get(key)
-    if hit is not None:
+    if hit is not None and hit[0]._handle:
         _CACHE.move_to_end(key)
-        return hit[0]
-    plan = GraphPlan(edge_index, num_nodes)
-    _CACHE[key] = (plan, edge_index, _plan_bytes(plan, edge_index))
-    _evict()
+        plan = hit[0]
+        _STATS["content_hits"] += 1
+    else:
+        plan = GraphPlan(edge_index, num_nodes)
+        _STATS["builds"] += 1
+        _CACHE[key] = (plan, _plan_bytes(plan))
+        _evict()
+    _remember(edge_index, plan, int(num_nodes))
     return plan
+
+
+def _remember(edge_index, plan, n):
+    tid = id(edge_index)
+
+    def forget(_ref, tid=tid):
+        ent = _BY_TENSOR.get(tid)
+        if ent is not None and ent[0] is _ref:
+            del _BY_TENSOR[tid]
+
+    _BY_TENSOR[tid] = (weakref.ref(edge_index, forget), edge_index._version, plan, n)
 
 
 def clear_plan_cache():
     _CACHE.clear()
+    _BY_TENSOR.clear()
+    for k in _STATS:
+        _STATS[k] = 0
     from . import core_attention
     core_attention._BIAS_CACHE.clear()
