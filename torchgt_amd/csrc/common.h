@@ -40,12 +40,11 @@ int reduce_partials(const tgt_reduce_desc* descs, int count, int dtype, hipStrea
 // and this item's partial sums go to slot `part` of the workspace.
 struct Item { int32_t row, start, len, part; };
 
-// What one wave of an attention workgroup does.  Workgroup b reads descriptors 4b .. 4b+3.
-//   kind 0..4: wave items [first, first + count) of that length class (count <= rows per wave of the shape)
-//   kind 5:    workgroup item `first` (all four descriptors of the workgroup are equal)
+// Code of a wave record: bits 0-2 kind, bit 3 the view in the backward launch (0 by destination, 1 by source),
+// bits 8.. number of rows.
+//   kind 0..4: wave items of that length class (count <= rows per wave of the shape)
+//   kind 5:    a workgroup item (all four records of the workgroup are equal)
 //   kind 7:    nothing
-// Bit 3 of the code tells the view in the backward launch (0 by destination, 1 by source).
-struct WaveDesc { int32_t first; uint32_t code; };
 constexpr uint32_t kDescBlock = 5, kDescNone = 7, kDescSrcSide = 8;
 __host__ __device__ constexpr uint32_t desc_code(uint32_t kind, uint32_t src_side, uint32_t count) {
     return kind | (src_side ? kDescSrcSide : 0u) | (count << 8);
@@ -115,6 +114,7 @@ struct Side {
     std::vector<int32_t> block_home;       // [n_block_items] window the workgroup item is scheduled with
     std::vector<int32_t> block_len;        // [n_block_items] its edges
     std::vector<uint8_t> block_spread;     // [n_block_items] 1: segment of a row with more than kSpreadSegs segments
+    std::vector<int32_t> homed_off, homed_idx;   // workgroup items by home window: items homed_idx[homed_off[w] .. homed_off[w+1])
 };
 
 // Wave records of one kernel shape (lanes per edge): forward (destination view) and backward

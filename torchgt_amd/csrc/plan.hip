@@ -280,44 +280,60 @@ __global__ void k_emit_items(const int32_t* __restrict__ long_rows, const SchedH
     if (part >= 0) part2split[part] = sidx;
 }
 
-// One workgroup of 64 threads writes one wave record from its descriptor (layout: WaveRec in common.h).
-__global__ __launch_bounds__(64) void k_build_records(const WaveDesc* __restrict__ desc, const Item* __restrict__ items_d,
-                                                      const Item* __restrict__ items_s, const Item* __restrict__ bitems_d,
-                                                      const Item* __restrict__ bitems_s, const int32_t* __restrict__ col_d,
-                                                      const int32_t* __restrict__ eid_d, const int32_t* __restrict__ col_s,
-                                                      const int32_t* __restrict__ eid_s, WaveRecLayout L, int lpe,
-                                                      int32_t* __restrict__ recs) {
-    const WaveDesc d = desc[blockIdx.x];
-    int32_t* out = recs + (int64_t)blockIdx.x * L.stride;
-    const int t = threadIdx.x;
-    const uint32_t kind = d.code & 7u;
-    const bool src = (d.code & kDescSrcSide) != 0;
-    const int count = (int)(d.code >> 8);
+// A run: `waves` consecutive waves of the list of XCD `xcd` that do the same kind of thing.
+//   rows:       the wave items [first, first + n) of one (window, class), rows_per_wave of them per wave
+//   block item: workgroup item `first`; its four waves carry the same record
+//   nothing:    padding to whole workgroups, and behind the end of a list
+struct Run { int32_t wave0, waves, first, n; uint32_t code; int32_t xcd; int32_t pad[2]; };
+
+// One workgroup per run; its waves write the run's wave records in turn (layout: WaveRec in common.h).  Wave lw of
+// XCD x's list is wave lw % 4 of that XCD's (lw / 4)-th workgroup, and workgroup b of the launch runs on XCD b mod 8:
+// record ((lw / 4) * 8 + x) * 4 + lw % 4.  Everything a kernel may read of a record is written: no clearing pass.
+__global__ __launch_bounds__(256) void k_build_records(const Run* __restrict__ runs, const Item* __restrict__ items_d,
+                                                       const Item* __restrict__ items_s, const Item* __restrict__ bitems_d,
+                                                       const Item* __restrict__ bitems_s, const int32_t* __restrict__ col_d,
+                                                       const int32_t* __restrict__ eid_d, const int32_t* __restrict__ col_s,
+                                                       const int32_t* __restrict__ eid_s, WaveRecLayout L, int lpe,
+                                                       int32_t* __restrict__ recs) {
+    const Run run = runs[blockIdx.x];
+    const int t = threadIdx.x & 63;
+    const uint32_t kind = run.code & 7u;
+    const bool src = (run.code & kDescSrcSide) != 0;
     const Item* items = src ? items_s : items_d;
     const int32_t* col = src ? col_s : col_d;
     const int32_t* eid = src ? eid_s : eid_d;
-    if (t == 0) out[0] = (int32_t)d.code;
-    if (kind == kDescNone) return;
-    if (kind == kDescBlock) {
-        if (t == 0) {
-            const Item it = (src ? bitems_s : bitems_d)[d.first];
-            out[4] = it.row; out[5] = it.start; out[6] = it.len; out[7] = it.part;
-        }
-        return;
-    }
-    if (t < count) {
-        const Item it = items[d.first + t];
-        out[L.off_row + t] = it.row;
-        out[L.off_start + t] = it.start;
-        out[L.off_len + t] = it.len;
-    }
-    if (!class_inline(lpe, (int)kind)) return;
-    const int S = slots_for_class(lpe, (int)kind);
+    const int ipw = kind < (uint32_t)kNumClass ? rows_per_wave(lpe, (int)kind) : 1;
+    const int S = kind < (uint32_t)kNumClass ? slots_for_class(lpe, (int)kind) : 1;
+    const bool inl = kind < (uint32_t)kNumClass && class_inline(lpe, (int)kind);
     const int groups = kWave / lpe;
-    if (t < groups) {
-        const int i = t / S, sl = t % S;
-        if (i < count) {
-            const Item it = items[d.first + i];
+    for (int w = threadIdx.x >> 6; w < run.waves; w += 4) {
+        const int lw = run.wave0 + w;
+        int32_t* out = recs + (((int64_t)(lw >> 2) * 8 + run.xcd) * 4 + (lw & 3)) * L.stride;
+        if (kind == kDescNone) {
+            if (t == 0) out[0] = (int32_t)kDescNone;
+            continue;
+        }
+        if (kind == kDescBlock) {
+            if (t == 0) {
+                const Item it = (src ? bitems_s : bitems_d)[run.first];
+                out[0] = (int32_t)run.code;
+                out[4] = it.row; out[5] = it.start; out[6] = it.len; out[7] = it.part;
+            }
+            continue;
+        }
+        const int first = run.first + w * ipw;
+        const int count = min(ipw, run.n - w * ipw);
+        if (t == 0) out[0] = (int32_t)desc_code(kind, src, (uint32_t)count);
+        if (t < count) {
+            const Item it = items[first + t];
+            out[L.off_row + t] = it.row;
+            out[L.off_start + t] = it.start;
+            out[L.off_len + t] = it.len;
+        }
+        if (inl && t < groups) {                        // every lane group's entries, zeros behind the last row
+            const int i = t / S, sl = t % S;
+            Item it{0, 0, 0, -1};
+            if (i < count) it = items[first + i];
             for (int u = 0; u < 4; ++u) {
                 const int e = sl + u * S;
                 const int ec = e < it.len ? e : it.len - 1;
@@ -453,50 +469,48 @@ static void schedule_counts(Side& side, const SideScratch& sc, const int32_t* re
 // load (their own q/k/v/dout rows, the rows of their self-loops, the window's share of a global node's
 // segment) then meets in one L2 at about the same time.
 namespace {
-// Workgroup items homed at window w_items and wave descriptors of window w of one view (either may be -1:
-// none), appended to `waves`; `cost` grows by a rough measure of the work.  part 0: the heavy share (segments of ordinary long rows and the rows of the longest class, which
+// One XCD's list as runs of waves.
+struct XcdList {
+    std::vector<Run> runs;
+    int32_t waves = 0, xcd = 0;
+    void add(uint32_t code, int32_t first, int32_t n, int32_t waves_of_run) {
+        if (waves_of_run <= 0) return;
+        runs.push_back(Run{waves, waves_of_run, first, n, code, xcd, {0, 0}});
+        waves += waves_of_run;
+    }
+    void pad4() { if (waves % 4) add(kDescNone, 0, 0, 4 - waves % 4); }
+};
+
+// Workgroup items homed at window w_items and the waves of window w of one view (either may be -1: none), appended
+// to the list.  part 0: the heavy share (segments of ordinary long rows and the rows of the longest class, which
 // run for many steps and whose edges have no tie to the window), part 1: the rest (segments of a row that
 // spans the graph, which gather exactly the window's rows, and the short rows).
-void append_side(std::vector<WaveDesc>& waves, float& cost, const Side& s, int w, int w_items, int lpe, bool src_side,
-                 const std::vector<std::vector<int32_t>>& homed, int part) {
+void append_side(XcdList& xl, const Side& s, int w, int w_items, int lpe, bool src_side, int part) {
     if (w_items >= 0) {
-        for (int32_t it : homed[w_items]) {
+        for (int32_t q = s.homed_off[w_items]; q < s.homed_off[w_items + 1]; ++q) {
+            const int32_t it = s.homed_idx[q];
             if ((s.block_spread[it] != 0) != (part == 1)) continue;
-            // close a partly filled workgroup first: a workgroup item takes all four waves
-            while (waves.size() % 4) waves.push_back(WaveDesc{0, kDescNone});
-            for (int k = 0; k < 4; ++k) waves.push_back(WaveDesc{it, desc_code(kDescBlock, src_side, 0)});
-            cost += 1.0f + s.block_len[it] / 128.0f;
+            xl.pad4();      // close a partly filled workgroup first: a workgroup item takes all four waves
+            xl.add(desc_code(kDescBlock, src_side, 0), it, 1, 4);
         }
     }
     if (w < 0) return;
     for (int c = (part == 0 ? 0 : 1); c < (part == 0 ? 1 : kNumClass); ++c) {
         const uint32_t n = s.win_class_cnt[(size_t)w * (kNumClass + 1) + c];
-        const uint32_t first = s.win_class_off[(size_t)w * (kNumClass + 1) + c];
-        const uint32_t ipw = (uint32_t)rows_per_wave(lpe, c);
-        for (uint32_t i = 0; i < n; i += ipw) {
-            waves.push_back(WaveDesc{(int32_t)(first + i), desc_code((uint32_t)c, src_side, n - i < ipw ? n - i : ipw)});
-            cost += c == 0 ? 0.75f : 0.25f;
-        }
+        const int ipw = rows_per_wave(lpe, c);
+        xl.add(desc_code((uint32_t)c, src_side, 0), (int32_t)s.win_class_off[(size_t)w * (kNumClass + 1) + c], (int32_t)n,
+               (int32_t)((n + ipw - 1) / ipw));
     }
 }
 
-// descriptors of all windows -> block order.  XCD x gets a contiguous range of windows; it first walks the
+// runs of all windows -> block order.  XCD x gets a contiguous range of windows; it first walks the
 // heavy share of all its windows (long work first keeps the end of the launch short), then window by window.
-// `placed` and `desc_d` feed an asynchronous copy and the kernel behind it: the caller keeps them until the stream
-// has been synchronised.
+// The host vectors and device buffers handed back feed an asynchronous copy and the kernel behind it: the caller
+// keeps them until the stream has been synchronised.
 int place(const std::vector<const Side*>& sides, int lpe, void** d_out, int32_t* n_blocks, hipStream_t st,
-          std::vector<WaveDesc>& placed, DevBuf& desc_d) {
+          std::vector<Run>& all_runs, DevBuf& runs_d) {
     const int nwin = sides[0]->n_windows;
     const bool heavy_first = env_int("TGT_HEAVY_FIRST", 1) == 1;
-    std::vector<std::vector<std::vector<int32_t>>> homed(sides.size());
-    for (size_t k = 0; k < sides.size(); ++k) {
-        homed[k].resize(nwin > 0 ? nwin : 1);
-        for (int32_t i = 0; i < sides[k]->n_block_items; ++i) {
-            int h = sides[k]->block_home[i];
-            h = h < 0 ? 0 : (h >= nwin ? nwin - 1 : h);
-            homed[k][h].push_back(i);
-        }
-    }
     // 8 contiguous window ranges with about equal numbers of edges and rows
     int bound[9];
     bound[0] = 0;
@@ -504,11 +518,12 @@ int place(const std::vector<const Side*>& sides, int lpe, void** d_out, int32_t*
         std::vector<double> cost(nwin + 1, 0.0);
         for (int w = 0; w < nwin; ++w) {
             double c = 0.0;
-            for (const Side* sd : sides) {
-                for (int32_t it : homed[sd == sides[0] ? 0 : 1][w]) c += 1.0 + sd->block_len[it] / 128.0;
-                for (int k = 0; k < kNumClass; ++k)
-                    c += (k == 0 ? 0.75 : 0.25) * ((sd->win_class_cnt[(size_t)w * (kNumClass + 1) + k] + rows_per_wave(lpe, k) - 1) /
-                                                   rows_per_wave(lpe, k));
+            for (size_t k = 0; k < sides.size(); ++k) {
+                const Side* sd = sides[k];
+                for (int32_t q = sd->homed_off[w]; q < sd->homed_off[w + 1]; ++q) c += 1.0 + sd->block_len[sd->homed_idx[q]] / 128.0;
+                for (int kk = 0; kk < kNumClass; ++kk)
+                    c += (kk == 0 ? 0.75 : 0.25) * ((sd->win_class_cnt[(size_t)w * (kNumClass + 1) + kk] + rows_per_wave(lpe, kk) - 1) /
+                                                    rows_per_wave(lpe, kk));
             }
             cost[w + 1] = cost[w] + c;
         }
@@ -522,53 +537,53 @@ int place(const std::vector<const Side*>& sides, int lpe, void** d_out, int32_t*
     // time for the rows to meet in the L2, and the last windows of a range end with short rows only - the
     // chain of a split row (partial slot, arrival, sums of the group and of the row) is not left for the end.
     const int lead = env_int("TGT_SEGMENT_LEAD", 6);
-    std::vector<WaveDesc> xw[8];
+    XcdList xl[8];
     for (int x = 0; x < 8; ++x) {
-        float c = 0.f;
-        std::vector<WaveDesc>& wv = xw[x];
+        XcdList& wv = xl[x];
+        wv.xcd = x;
+        wv.runs.reserve((size_t)(bound[x + 1] - bound[x] + 8) * 8 * sides.size());
         const int w0 = bound[x], w1 = bound[x + 1];
         if (heavy_first) {
             // one view after the other: the long rows of the destination view gather k and v rows, those of the source
             // view q, dout and the per-node scalars; side by side the two sets compete for the L2 (870 K nodes with
             // 50 edges per row: 3 % faster one after the other; no difference where long rows are few)
             for (size_t k = 0; k < sides.size(); ++k)
-                for (int w = w0; w < w1; ++w) append_side(wv, c, *sides[k], w, w, lpe, k == 1, homed[k], 0);
-            while (wv.size() % 4) wv.push_back(WaveDesc{0, kDescNone});
+                for (int w = w0; w < w1; ++w) append_side(wv, *sides[k], w, w, lpe, k == 1, 0);
+            wv.pad4();
         }
         // the segments of the last half of the range go first: when the launch ends no split row is still
         // being added up (those windows give up meeting their segment in the L2)
         const int w_early = w1 - (w1 - w0) / env_int("TGT_EARLY_SHARE", 2);
         for (int w = w_early; w < w1; ++w)
-            for (size_t k = 0; k < sides.size(); ++k) append_side(wv, c, *sides[k], -1, w, lpe, k == 1, homed[k], 1);
+            for (size_t k = 0; k < sides.size(); ++k) append_side(wv, *sides[k], -1, w, lpe, k == 1, 1);
         for (int w = w0 - lead; w < w1; ++w) {
             const int wi = w + lead < w_early ? w + lead : -1;        // segments of the window `lead` ahead
             for (size_t k = 0; k < sides.size(); ++k) {
-                if (!heavy_first) append_side(wv, c, *sides[k], w >= w0 ? w : -1, w >= w0 ? w : -1, lpe, k == 1, homed[k], 0);
-                append_side(wv, c, *sides[k], w >= w0 ? w : -1, wi >= w0 ? wi : -1, lpe, k == 1, homed[k], 1);
+                if (!heavy_first) append_side(wv, *sides[k], w >= w0 ? w : -1, w >= w0 ? w : -1, lpe, k == 1, 0);
+                append_side(wv, *sides[k], w >= w0 ? w : -1, wi >= w0 ? wi : -1, lpe, k == 1, 1);
             }
-            while (wv.size() % 4) wv.push_back(WaveDesc{0, kDescNone});
+            wv.pad4();
         }
     }
-    size_t per = 0;
-    for (int x = 0; x < 8; ++x) per = std::max(per, xw[x].size() / 4);
-    const size_t nb = per * 8;
-    placed.assign(nb * 4 + 4, WaveDesc{0, kDescNone});
-    for (int x = 0; x < 8; ++x)
-        for (size_t b = 0; b < xw[x].size() / 4; ++b)
-            for (int k = 0; k < 4; ++k) placed[(b * 8 + x) * 4 + k] = xw[x][b * 4 + k];
-    // descriptors -> records, on the device (the edge lists never visit the host)
+    int32_t per = 0;
+    for (int x = 0; x < 8; ++x) per = std::max(per, (xl[x].waves + 3) / 4);
+    const size_t nb = (size_t)per * 8;
     const WaveRecLayout L(lpe);
     const size_t n_rec = nb * 4;
     *n_blocks = (int32_t)nb;
     if (n_rec == 0) return TGT_OK;
-    TGT_HIP_CHECK(desc_d.alloc(sizeof(WaveDesc) * n_rec, st));
-    TGT_HIP_CHECK(hipMemcpyAsync(desc_d.p, placed.data(), sizeof(WaveDesc) * n_rec, hipMemcpyHostToDevice, st));
+    all_runs.clear();
+    for (int x = 0; x < 8; ++x) {
+        xl[x].add(kDescNone, 0, 0, per * 4 - xl[x].waves);       // behind the end of the list: records that say "nothing"
+        all_runs.insert(all_runs.end(), xl[x].runs.begin(), xl[x].runs.end());
+    }
+    TGT_HIP_CHECK(runs_d.alloc(sizeof(Run) * all_runs.size(), st));
+    TGT_HIP_CHECK(hipMemcpyAsync(runs_d.p, all_runs.data(), sizeof(Run) * all_runs.size(), hipMemcpyHostToDevice, st));
     const size_t bytes = n_rec * (size_t)L.stride * sizeof(int32_t);
     TGT_HIP_CHECK(dev_alloc(d_out, bytes, st));
-    TGT_HIP_CHECK(hipMemsetAsync(*d_out, 0, bytes, st));
     const Side* sd = sides[0];
     const Side* ss = sides.size() > 1 ? sides[1] : sides[0];
-    hipLaunchKernelGGL(k_build_records, dim3((unsigned)n_rec), dim3(64), 0, st, desc_d.as<WaveDesc>(), sd->items, ss->items,
+    hipLaunchKernelGGL(k_build_records, dim3((unsigned)all_runs.size()), dim3(256), 0, st, runs_d.as<Run>(), sd->items, ss->items,
                        sd->block_items, ss->block_items, sd->col, sd->eid, ss->col, ss->eid, L, lpe, static_cast<int32_t*>(*d_out));
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
@@ -590,10 +605,10 @@ const Schedule* plan_schedule(const tgt_plan* plan_c, int lpe, hipStream_t st) {
     // the descriptors of a shape are made once, whichever thread or stream asks first
     std::lock_guard<std::mutex> lock(plan->sched_mutex);
     if (sc.ready) return &sc;
-    std::vector<WaveDesc> placed_f, placed_b;
-    DevBuf desc_f, desc_b;
-    int rc = place({&plan->dst}, lpe, &sc.fwd, &sc.fwd_blocks, st, placed_f, desc_f);
-    if (rc == TGT_OK) rc = place({&plan->dst, &plan->src}, lpe, &sc.bwd, &sc.bwd_blocks, st, placed_b, desc_b);
+    std::vector<Run> runs_f, runs_b;
+    DevBuf rf, rb;
+    int rc = place({&plan->dst}, lpe, &sc.fwd, &sc.fwd_blocks, st, runs_f, rf);
+    if (rc == TGT_OK) rc = place({&plan->dst, &plan->src}, lpe, &sc.bwd, &sc.bwd_blocks, st, runs_b, rb);
     // the host vectors feed asynchronous copies: they may go once the stream is idle
     if (hipStreamSynchronize(st) != hipSuccess && rc == TGT_OK) { set_error("hipStreamSynchronize failed"); rc = TGT_ERR_HIP; }
     if (rc != TGT_OK) {
@@ -715,6 +730,14 @@ static int create_impl(const int64_t* d_src, const int64_t* d_dst, int64_t E, in
         for (size_t i = 0; i < m.size(); ++i) {
             sd.block_home[i] = m[i].home; sd.block_len[i] = m[i].len; sd.block_spread[i] = (uint8_t)m[i].spread;
         }
+        // workgroup items by the window they are scheduled with (counting sort: item order is kept inside a window)
+        const int nw = sd.n_windows > 0 ? sd.n_windows : 1;
+        sd.homed_off.assign((size_t)nw + 1, 0);
+        for (int32_t& h : sd.block_home) { h = h < 0 ? 0 : (h >= nw ? nw - 1 : h); sd.homed_off[(size_t)h + 1]++; }
+        for (int w = 0; w < nw; ++w) sd.homed_off[(size_t)w + 1] += sd.homed_off[w];
+        sd.homed_idx.resize(m.size());
+        std::vector<int32_t> at(sd.homed_off.begin(), sd.homed_off.end() - 1);
+        for (size_t i = 0; i < m.size(); ++i) sd.homed_idx[at[sd.block_home[i]]++] = (int32_t)i;
     }
     // the shape of the reference's node-level models (hidden 64: 8 heads of 8, or 4 of 16); other shapes on first use
     return plan_schedule(plan, 8, st) ? TGT_OK : TGT_ERR_HIP;
