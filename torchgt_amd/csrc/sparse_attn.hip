@@ -340,9 +340,119 @@ __device__ __forceinline__ void add_slots(Acc& acc) {
     }
 }
 
+// x of lane (l ^ OFF).  The exchange between the two halves of a row of 16 lanes is a DPP operand of the
+// add that uses it, the others go through the LDS crossbar.
+template <int OFF>
+__device__ __forceinline__ float lane_xor(float x) {
+    if constexpr (OFF == 8) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x128 /* row_ror:8 */,
+                                                                     0xf, 0xf, false));
+    } else {
+        return __shfl_xor(x, OFF);
+    }
+}
+
+// One level of the reduce-scatter below: the 2 N values of a lane become N, the sums with lane (l ^ OFF) of
+// the lower (bit OFF of the lane clear) or upper (set) half of them.
+template <int N, int OFF>
+__device__ __forceinline__ void halve(float (&a)[8], const bool upper) {
+    if constexpr (N >= 1) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const float keep = upper ? a[i + N] : a[i];
+            const float send = upper ? a[i] : a[i + N];
+            a[i] = keep + lane_xor<OFF>(send);
+        }
+    }
+}
+
+// Adds the S edge slots of a lane group so that the sums end up spread over the slots: afterwards the
+// lane of slot t holds, in a[0 .. 8/S), the sums of the elements t * (8/S) ... of its chunk - log2(S) levels
+// with 4, 2, 1 exchanges instead of 8 each, and every lane has a share of the row to finish and store.
+// The additions pair the same values as add_slots does, so both give the same bits.
+template <int LPE, int S>
+__device__ __forceinline__ void reduce_slots(float (&a)[8], const int slot) {
+    if constexpr (S >= 2) halve<4, LPE * S / 2>(a, (slot & (S / 2)) != 0);
+    if constexpr (S >= 4) halve<2, LPE * S / 4>(a, (slot & (S / 4)) != 0);
+    if constexpr (S >= 8) halve<1, LPE * S / 8>(a, (slot & (S / 8)) != 0);
+}
+
+template <int CNT>
+__device__ __forceinline__ void store_n(float* __restrict__ p, const float (&x)[8]) {
+    if constexpr (CNT == 1) *p = x[0];
+    else if constexpr (CNT == 2) *reinterpret_cast<float2*>(p) = make_float2(x[0], x[1]);
+    else {
+        *reinterpret_cast<float4*>(p) = make_float4(x[0], x[1], x[2], x[3]);
+        if constexpr (CNT == 8) *reinterpret_cast<float4*>(p + 4) = make_float4(x[4], x[5], x[6], x[7]);
+    }
+}
+template <int CNT>
+__device__ __forceinline__ void store_n(bf16_t* __restrict__ p, const float (&x)[8]) {
+    if constexpr (CNT == 1) p->x = (uint16_t)f32_to_bf16(x[0]);
+    else if constexpr (CNT == 2) *reinterpret_cast<uint32_t*>(p) = f32_to_bf16(x[0]) | (f32_to_bf16(x[1]) << 16);
+    else if constexpr (CNT == 4)
+        *reinterpret_cast<uint2*>(p) = make_uint2(f32_to_bf16(x[0]) | (f32_to_bf16(x[1]) << 16),
+                                                  f32_to_bf16(x[2]) | (f32_to_bf16(x[3]) << 16));
+    else store8(p, x);
+}
+template <int CNT>
+__device__ __forceinline__ void add_n(const float* __restrict__ p, float (&x)[8]) {
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) x[i] += p[i];
+}
+
+// Final value of a row of a wave item from the sums of its S slots: all S * LPE lanes of the row's lane
+// group take part, each finishes and stores 8 / S elements.
+template <typename T, int LPE, int LPH, int S, int MODE, bool TILES>
+__device__ __forceinline__ void finish_row(const Common& c, const SideArgs& s, const int row, const int slot,
+                                           const int el, const bool valid, Acc& acc) {
+    constexpr int H = LPE / LPH;
+    constexpr int HD = LPE * 8;
+    constexpr int SR = S > 8 ? 8 : S;     // slots the 8 elements of a chunk are spread over
+    constexpr int CNT = 8 / SR;
+    if constexpr (S > SR) {               // more slots than elements: the upper slot bits are plain sums
+#pragma unroll
+        for (int off = LPE * SR; off < LPE * S; off <<= 1) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                acc.a0[i] += __shfl_xor(acc.a0[i], off);
+                if (MODE == MODE_BWD_SRC) acc.a1[i] += __shfl_xor(acc.a1[i], off);
+            }
+        }
+    }
+    const int sl = slot % SR;
+    reduce_slots<LPE, SR>(acc.a0, sl);
+    if (MODE == MODE_BWD_SRC) reduce_slots<LPE, SR>(acc.a1, sl);
+    if (MODE == MODE_FWD) {
+#pragma unroll
+        for (int off = LPE; off < LPE * S; off <<= 1) acc.z += __shfl_xor(acc.z, off);
+    }
+    if (!valid || slot >= SR) return;
+    const int64_t off = (int64_t)row * HD + el * 8 + sl * CNT;
+    if (MODE != MODE_FWD) {
+#pragma unroll
+        for (int i = 0; i < CNT; ++i) acc.a0[i] *= c.inv_scale;
+    }
+    if (TILES) {   // sums of the dense tiles of the block path for this row, if it has any
+        if (s.cover[row] != 0) {
+            add_n<CNT>(s.init0 + off, acc.a0);
+            if (MODE == MODE_FWD) acc.z += s.initZ[(int64_t)row * H + el / LPH];
+            if (MODE == MODE_BWD_SRC) add_n<CNT>(s.init1 + off, acc.a1);
+        }
+    }
+    if (MODE == MODE_FWD) {
+        const float inv = 1.0f / (acc.z + kEps);
+#pragma unroll
+        for (int i = 0; i < CNT; ++i) acc.a0[i] *= inv;
+        if (sl == 0 && el % LPH == 0) s.Z[(int64_t)row * H + el / LPH] = acc.z;
+    }
+    store_n<CNT>(static_cast<T*>(s.out0) + off, acc.a0);
+    if (MODE == MODE_BWD_SRC) store_n<CNT>(static_cast<T*>(s.out1) + off, acc.a1);
+}
+
 // Walks `len` edges starting at sorted position `start` of node `row` with S edge
 // slots (this lane is slot `slot`, element chunk `el`), reading the plan's sorted view.  On return
-// every lane of the S*LPE-lane group holds the sums over all S slots.
+// every lane holds the sums of its own slot (add_slots or reduce_slots adds the slots).
 template <typename T, int LPE, int LPH, int S, int MODE, int HASB>
 __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, const int row, const int start,
                                            const int len, const int slot, const int el, const bool valid,
@@ -354,17 +464,14 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
     constexpr bool ident = HASB == 2;
     const int32_t* __restrict__ eid = ident ? nullptr : s.eid + start;
     const int n = valid ? len : 0;
-#pragma unroll 1
-    for (int e0 = slot; e0 < n; e0 += S * kUnroll) {
-        int nb[kUnroll], ed[kUnroll];
-        bool ok[kUnroll];
+    // endpoints and bias rows of the step that starts at edge e0 of the row
+    auto load_ids = [&](const int e0, int (&nb)[kUnroll], int (&ed)[kUnroll]) {
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
             const int e = e0 + u * S;
-            ok[u] = e < n;
             if constexpr (sizeof(T) == 4) {
                 nb[u] = 0; ed[u] = 0;
-                if (ok[u]) {
+                if (e < n) {
                     nb[u] = col[e];
                     if (HASB) ed[u] = ident ? start + e : eid[e];
                 }
@@ -374,9 +481,35 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
                 ed[u] = HASB ? (ident ? start + ec : eid[ec]) : 0;
             }
         }
-        edge_step<T, LPE, LPH, MODE, HASB>(c, s, rr, nb, ed, ok, el, acc);
+    };
+    if (n <= 0) return;
+    if constexpr (sizeof(T) == 4) {
+#pragma unroll 1
+        for (int e0 = slot; e0 < n; e0 += S * kUnroll) {
+            int nb[kUnroll], ed[kUnroll];
+            bool ok[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) ok[u] = e0 + u * S < n;
+            load_ids(e0, nb, ed);
+            edge_step<T, LPE, LPH, MODE, HASB>(c, s, rr, nb, ed, ok, el, acc);
+        }
+    } else {
+        // the ids of the next step are asked for before this step's gathers: a step waits for one memory
+        // round trip, not for two in a row (2-byte elements leave the registers for it)
+        int nb[kUnroll], ed[kUnroll];
+        load_ids(slot, nb, ed);
+#pragma unroll 1
+        for (int e0 = slot; e0 < n; e0 += S * kUnroll) {
+            int nb2[kUnroll], ed2[kUnroll];
+            bool ok[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) ok[u] = e0 + u * S < n;
+            load_ids(e0 + S * kUnroll, nb2, ed2);
+            edge_step<T, LPE, LPH, MODE, HASB>(c, s, rr, nb, ed, ok, el, acc);
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u) { nb[u] = nb2[u]; ed[u] = ed2[u]; }
+        }
     }
-    add_slots<LPE, S, MODE>(acc);
 }
 
 // The same for a row of at most S * kUnroll edges whose endpoints and bias rows come with the wave's
@@ -409,7 +542,6 @@ __device__ __forceinline__ void walk_record(const Common& c, const SideArgs& s, 
         }
     }
     edge_step<T, LPE, LPH, MODE, HASB>(c, s, rr, nb, ed, ok, el, acc);
-    add_slots<LPE, S, MODE>(acc);
 }
 
 // Final value of a row from its sums, written by the LPE lanes that own the chunks.
@@ -438,9 +570,9 @@ __device__ __forceinline__ void write_row(const Common& c, const SideArgs& s, co
         }
     }
     if (MODE == MODE_FWD) {
-        const float den = acc.z + kEps;
+        const float inv = 1.0f / (acc.z + kEps);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc.a0[i] = acc.a0[i] / den;
+        for (int i = 0; i < 8; ++i) acc.a0[i] *= inv;
         store8(static_cast<T*>(s.out0) + row_off, acc.a0);
         if (el % LPH == 0) s.Z[(int64_t)row * H + el / LPH] = acc.z;
     } else {
@@ -464,7 +596,7 @@ __device__ __forceinline__ void wave_rows(const Common& c, const SideArgs& s, co
     Acc acc;
     if (INLINE) walk_record<T, LPE, LPH, S, MODE, HASB>(c, s, rec, row, start, len, slot, el, valid, acc);
     else walk_range<T, LPE, LPH, S, MODE, HASB>(c, s, row, start, len, slot, el, valid, acc);
-    if (valid && slot == 0) write_row<T, LPE, LPH, MODE, TILES>(c, s, row, el, acc);
+    finish_row<T, LPE, LPH, S, MODE, TILES>(c, s, row, slot, el, valid, acc);
 }
 
 template <typename T, int LPE, int LPH, int MODE, int HASB, bool TILES>
@@ -627,6 +759,7 @@ __device__ __forceinline__ void block_item(const Common& c, const SideArgs& s, c
     const int hi = min(lo + share, it.len);
     Acc acc;
     walk_range<T, LPE, LPH, S, MODE, HASB>(c, s, it.row, it.start + lo, hi - lo, slot, el, true, acc);
+    add_slots<LPE, S, MODE>(acc);
     if (slot == 0) {
         float* r = lds.red + grp * STRIDE;
 #pragma unroll
