@@ -551,7 +551,7 @@ int tgt_graph_attn_bias_multi_hop_bwd(const void* d_dout, const int64_t* d_spati
                                       int num_edge_dis, int multi_hop_max_dist, int b, int s, int H, int dtype,
                                       void* d_dspatial_table, void* d_dedge_table, void* d_dedge_dis_weight,
                                       void* d_dvirtual_dist, void* d_workspace, int64_t workspace_bytes, void* stream);
-/* gen_edge_input (data/algos.pyx:64-92) for a batch of graphs of at most 128 nodes.
+/* gen_edge_input (data/algos.pyx:64-92) for a batch of graphs of at most 256 nodes.
  * d_path: int32 [num_graphs, n_max, n_max] as tgt_floyd_warshall writes it; d_edge_feat:
  * [num_graphs, n_max, n_max, F], int64 (feat_is_int64 != 0) or int32; d_n_nodes as there.
  * d_out: int64 [num_graphs, n_max, n_max, max_dist, F]; entry (i, j, k) = features of the k-th
@@ -560,7 +560,7 @@ int tgt_graph_attn_bias_multi_hop_bwd(const void* d_dout, const int64_t* d_spati
  * end of the path, padding nodes.  Hops at or beyond max_dist are dropped. */
 int tgt_gen_edge_input(const int32_t* d_path, const void* d_edge_feat, int feat_is_int64, int F, const int32_t* d_n_nodes,
                        int num_graphs, int n_max, int max_dist, int64_t* d_out, void* stream);
-/* floyd_warshall (data/algos.pyx:9-54) for a batch of graphs of at most 128 nodes.
+/* floyd_warshall (data/algos.pyx:9-54) for a batch of graphs of at most 256 nodes.
  * d_adj: uint8 [num_graphs, n_max, n_max], entry = edge weight, 0 = no edge;
  * d_n_nodes: int32 [num_graphs] node counts (NULL: all n_max).  d_dist, d_path:
  * int32 [num_graphs, n_max, n_max]; entries with i or j >= n_nodes[g] are left

@@ -206,6 +206,28 @@ def floyd_warshall(adjacency_matrix):
     return M, path
 
 
+def floyd_warshall_by_steps(adjacency_matrix):
+    """The same result as ``floyd_warshall`` with one array operation per k, for graphs too large for the
+    triple loop.  Step k of the loop reads only row k and column k of M, and neither changes during the step
+    (M[k][k] = 0, so M[i][k] > M[i][k] + 0 and M[k][j] > 0 + M[k][j] never hold): all (i, j) of a step can be
+    relaxed at once.  tests/test_oracle_graph_prep.py compares the two on random graphs."""
+    M = np.array(adjacency_matrix, dtype=np.int64)
+    n = M.shape[0]
+    assert M.shape == (n, n)
+    path = -np.ones((n, n), dtype=np.int64)
+    M[M == 0] = FW_UNREACHABLE
+    np.fill_diagonal(M, 0)
+    for k in range(n):
+        cost = M[:, k][:, None] + M[k, :][None, :]
+        better = M > cost
+        M[better] = cost[better]
+        path[better] = k
+    far = M >= FW_UNREACHABLE
+    path[far] = FW_UNREACHABLE
+    M[far] = FW_UNREACHABLE
+    return M, path
+
+
 def get_all_edges(path, i, j):
     """data/algos.pyx:56-61: the intermediate nodes of the recorded shortest path from i to j."""
     k = int(path[i][j])

@@ -112,6 +112,43 @@ def test_attention_dropout_matches_oracle_with_the_exported_mask(cuda, dtype, p)
     if dtype == torch.float32:
         run_case("drop-f32-bf16mm", 2, 100, 4, 8, dtype, True, None, 63, cuda, p_drop=p, bf16_products=True)
 
+# Keep mask of seed 2024, p = 0.5 for b = 2, H = 2, S = 4, listed by hand: [graph][head][query][key].  It comes from
+# the documented generator evaluated with pencil-and-paper integer arithmetic (32-bit multiply / xor-shift rounds on
+# (seed, graph * H + head, query, key)), not from the library.
+HAND_MASK = [[[[1, 1, 1, 1], [1, 1, 1, 1], [0, 0, 0, 1], [0, 0, 1, 1]],
+              [[1, 1, 1, 1], [1, 1, 0, 0], [1, 0, 0, 0], [0, 1, 0, 0]]],
+             [[[1, 0, 0, 1], [1, 0, 1, 0], [1, 1, 0, 1], [1, 0, 1, 0]],
+              [[0, 1, 0, 1], [0, 1, 1, 1], [1, 0, 0, 0], [1, 0, 0, 0]]]]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_dropout_mask_indexing_read_off_the_kernels(cuda, dtype):
+    """Which (graph, head, query, key) the kernels drop, read off their outputs and compared with the hand-listed
+    mask - the exported mask plays no part.  With q = k = 0 and no bias every probability is 1/4; values that are
+    unit vectors (v[key] = e_key) make out[g, q, h, c] = keep[g, h, q, c] / (4 (1 - p)), and an upstream gradient
+    of unit vectors (dout[q] = e_q) makes dv[g, k, h, c] = keep[g, h, c, k] / (4 (1 - p)): the forward's mask and
+    the backward's, position by position."""
+    b, S, H, d, p = 2, 4, 2, 8, 0.5
+    want = torch.tensor(HAND_MASK, dtype=torch.bool)                     # [b, H, q, k]
+    q = torch.zeros(b, S, H, d, dtype=dtype, device=cuda)
+    v = torch.zeros(b, S, H, d, dtype=dtype)
+    for key in range(S):
+        v[:, key, :, key] = 1.0
+    v = v.to(cuda).requires_grad_(True)
+    out = dense_attention(q, q.clone(), v, None, p_drop=p, seed=2024)
+    o = out.view(b, S, H, d).float().cpu()                               # [g, q, h, c]
+    assert torch.equal(o[..., S:], torch.zeros(b, S, H, d - S))
+    shown = o[..., :S].permute(0, 2, 1, 3)                               # [g, h, q, key]
+    assert torch.equal(shown, want.float() * 0.5), shown                 # 1/4 * 1/(1 - p), exact in bf16 as well
+    dout = torch.zeros(b, S, H, d, dtype=dtype)
+    for qq in range(S):
+        dout[:, qq, :, qq] = 1.0
+    dv, = torch.autograd.grad(out, v, dout.reshape(b, S, H * d).to(cuda))
+    shown_b = dv.float().cpu()[..., :S].permute(0, 2, 3, 1)              # dv[g, k, h, c=q] -> [g, h, q, k]
+    assert torch.equal(shown_b, want.float() * 0.5), shown_b
+    # and the exported mask is the same one
+    assert torch.equal(dense_dropout_mask(b, S, H, p, 2024, cuda).cpu().bool(), want)
+
 
 def test_dropout_mask_statistics_and_module(cuda):
     b, S, H = 4, 129, 8

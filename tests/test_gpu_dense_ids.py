@@ -19,7 +19,7 @@ from torchgt_amd.graph_bias import GraphAttnBias
 
 pytestmark = pytest.mark.gpu
 TOL = 2e-2
-TOL_TABLE = 3e-2
+TOL_TABLE = 2e-2
 
 
 def err(a, b):

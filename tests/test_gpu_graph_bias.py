@@ -29,12 +29,12 @@ def err(a, b):
 def test_floyd_warshall_matches_oracle_bit_for_bit(cuda):
     rng = np.random.default_rng(0)
     # single graphs, the reference's call shape
-    for n, p in ((1, 0.0), (5, 0.5), (23, 0.12), (64, 0.05), (128, 0.03)):
+    for n, p in ((1, 0.0), (5, 0.5), (23, 0.12), (64, 0.05), (128, 0.03), (129, 0.03), (222, 0.012), (256, 0.02)):
         print(f"floyd_warshall case: n={n} p={p}", flush=True)
         a = (rng.random((n, n)) < p).astype(np.int64)
         a = np.maximum(a, a.T)
         M, path = floyd_warshall(a)
-        M_ref, path_ref = ogp.floyd_warshall(a)
+        M_ref, path_ref = ogp.floyd_warshall(a) if n <= 128 else ogp.floyd_warshall_by_steps(a)
         assert M.dtype == np.int64 and path.dtype == np.int64
         np.testing.assert_array_equal(M, M_ref)
         np.testing.assert_array_equal(path, path_ref)
@@ -60,11 +60,28 @@ def test_floyd_warshall_matches_oracle_bit_for_bit(cuda):
         np.testing.assert_array_equal(dist[g, :n, :n].cpu().numpy(), M_ref)
         np.testing.assert_array_equal(path[g, :n, :n].cpu().numpy(), path_ref)
         assert not dist[g, n:, :].any() and not dist[g, :, n:].any()
+    # a padded batch with graphs of more than 128 nodes (intermediate nodes kept in the output array), one of them
+    # a ring: the longest shortest paths a graph of that size can have
+    sizes = np.array([130, 222, 17, 200], dtype=np.int64)
+    adj = np.zeros((4, 222, 222), dtype=np.uint8)
+    for g, n in enumerate(sizes):
+        if g == 3:
+            idx = np.arange(n)
+            adj[g, idx, (idx + 1) % n] = 1
+            adj[g, (idx + 1) % n, idx] = 1
+        else:
+            a = rng.random((n, n)) < 2.5 / n
+            adj[g, :n, :n] = np.maximum(a, a.T)
+    dist, path = floyd_warshall(torch.from_numpy(adj), sizes)
+    for g, n in enumerate(sizes):
+        M_ref, path_ref = ogp.floyd_warshall_by_steps(adj[g, :n, :n])
+        np.testing.assert_array_equal(dist[g, :n, :n].cpu().numpy(), M_ref)
+        np.testing.assert_array_equal(path[g, :n, :n].cpu().numpy(), path_ref)
 
 
 def test_floyd_warshall_rejects_large_graphs(cuda):
     with pytest.raises(_lib.TorchGTHipError) as ei:
-        floyd_warshall(np.zeros((129, 129), dtype=np.int64))
+        floyd_warshall(np.zeros((257, 257), dtype=np.int64))
     assert ei.value.code == _lib.ERR_UNSUPPORTED
 
 
@@ -294,12 +311,12 @@ def test_gen_edge_input_matches_oracle_bit_for_bit(cuda):
     rng = np.random.default_rng(4)
     # single graphs, the reference's call shape (max_dist = the longest distance, 510 when a pair is unreachable:
     # data/wrapper.py passes np.amax of the distance matrix)
-    for n, p, F in ((1, 0.0, 1), (6, 0.4, 2), (23, 0.12, 3), (64, 0.06, 1), (128, 0.03, 2)):
+    for n, p, F in ((1, 0.0, 1), (6, 0.4, 2), (23, 0.12, 3), (64, 0.06, 1), (128, 0.03, 2), (222, 0.012, 1)):
         a = (rng.random((n, n)) < p).astype(np.int64)
         a = np.maximum(a, a.T)
         np.fill_diagonal(a, 0)
         feat = rng.integers(1, 9, size=(n, n, F)) * a[:, :, None]
-        M, path = ogp.floyd_warshall(a)
+        M, path = ogp.floyd_warshall(a) if n <= 128 else ogp.floyd_warshall_by_steps(a)
         reach = M[M < 510]
         for max_dist in sorted({int(reach.max()) if reach.size else 0, 2, 5}):
             print(f"gen_edge_input case: n={n} p={p} F={F} max_dist={max_dist}", flush=True)
@@ -307,6 +324,14 @@ def test_gen_edge_input_matches_oracle_bit_for_bit(cuda):
             got = gen_edge_input(max_dist, path, feat)
             assert got.dtype == np.int64 and got.shape == want.shape
             np.testing.assert_array_equal(got, want)
+    # a ring of 200 nodes: paths of up to 100 hops
+    idx = np.arange(200)
+    a = np.zeros((200, 200), dtype=np.int64)
+    a[idx, (idx + 1) % 200] = 1
+    a[(idx + 1) % 200, idx] = 1
+    feat = rng.integers(1, 9, size=(200, 200, 1)) * a[:, :, None]
+    M, path = ogp.floyd_warshall_by_steps(a)
+    np.testing.assert_array_equal(gen_edge_input(100, path, feat), ogp.gen_edge_input(100, path, feat))
     # directed graph: paths and features are not symmetric
     a = (rng.random((40, 40)) < 0.08).astype(np.int64)
     np.fill_diagonal(a, 0)
@@ -335,5 +360,5 @@ def test_gen_edge_input_matches_oracle_bit_for_bit(cuda):
 
 def test_gen_edge_input_rejects_large_graphs(cuda):
     with pytest.raises(_lib.TorchGTHipError) as ei:
-        gen_edge_input(3, np.zeros((129, 129), dtype=np.int64), np.zeros((129, 129, 1), dtype=np.int64))
+        gen_edge_input(3, np.zeros((257, 257), dtype=np.int64), np.zeros((257, 257, 1), dtype=np.int64))
     assert ei.value.code == _lib.ERR_UNSUPPORTED

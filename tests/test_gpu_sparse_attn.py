@@ -100,7 +100,7 @@ def test_config1_with_learned_spd_table(cuda):
         assert err(a, b) <= 1e-5
 
 
-SHAPES = [(8, 8), (4, 16), (8, 16), (16, 8), (4, 8), (2, 8), (1, 8), (2, 16), (1, 16)]
+SHAPES = [(8, 8), (4, 16), (8, 16), (16, 8), (4, 8), (2, 8), (1, 8), (2, 16), (1, 16), (4, 32), (2, 32), (1, 32)]
 
 
 @pytest.mark.parametrize("H,d", SHAPES)

@@ -228,6 +228,30 @@ def test_floyd_warshall_known_answer_and_scipy():
                     assert i == j or a[i, j] == 1
 
 
+def test_floyd_warshall_by_steps_is_the_loop():
+    """The one-array-operation-per-k form used for graphs of more than 128 nodes gives the loop's matrices
+    (distances and recorded intermediate nodes), on undirected, directed and weighted graphs."""
+    rng = np.random.default_rng(3)
+    for n, p, directed, wmax in ((1, 0.0, False, 1), (9, 0.3, False, 1), (33, 0.08, False, 1), (40, 0.06, True, 1),
+                                 (25, 0.15, True, 4), (30, 0.02, False, 1)):
+        a = (rng.random((n, n)) < p) * rng.integers(1, wmax + 1, size=(n, n))
+        if not directed:
+            a = np.maximum(a, a.T)
+        M0, P0 = gp.floyd_warshall(a)
+        M1, P1 = gp.floyd_warshall_by_steps(a)
+        np.testing.assert_array_equal(M0, M1)
+        np.testing.assert_array_equal(P0, P1)
+    # and against scipy's distances at a size the loop is too slow for
+    from scipy.sparse.csgraph import shortest_path
+    a = (rng.random((200, 200)) < 0.012).astype(np.int64)
+    a = np.maximum(a, a.T)
+    np.fill_diagonal(a, 0)
+    M, _ = gp.floyd_warshall_by_steps(a)
+    d = shortest_path(a, method="D", unweighted=True)
+    d[np.isinf(d)] = 510
+    np.testing.assert_array_equal(M, d.astype(np.int64))
+
+
 def test_gen_edge_input_known_answer_and_walk_property():
     # path graph 0-1-2-3 plus an isolated node 4; the feature of edge (a, b) is (10 a + b, 7)
     n = 5

@@ -371,14 +371,17 @@ int bias_check(int b, int s, int H, int F, int num_spatial, int num_edges, int d
     return TGT_OK;
 }
 
-// One workgroup per graph.  Distances (uint16: at most 2 * 510) and intermediate nodes (int16)
-// live in LDS.  Within one k the k-th row and column do not change (M[k][k] = 0), so all
-// (i, j) of a step can be relaxed at once and give exactly the sequential result.
-constexpr int kFwMax = 128;
+// One workgroup per graph.  Distances (uint16: at most 2 * 510) live in LDS; the intermediate nodes (int16) too
+// for graphs of up to 128 nodes, beyond that they are kept in the output array itself (every (i, j) has one
+// owner thread, so nobody else reads them).  Within one k the k-th row and column do not change
+// (M[k][k] = 0), so all (i, j) of a step can be relaxed at once and give exactly the sequential result.
+constexpr int kFwMax = 256;
+constexpr int kFwLdsPath = 128;      // largest graph whose intermediate nodes fit in LDS beside the distances
 constexpr int kFwInf = 510;          // data/algos.pyx:30
 
-// 1024 threads: thread (r, j) = (tid / 128, tid % 128) owns column j of rows r, r + 8, ...: no division per
-// element, row i's M[i][k] is one LDS word for all lanes of a row, M[k][j] runs along the lanes.
+// 1024 threads: thread (r, j) = (tid / COLS, tid % COLS) owns column j of rows r, r + 1024 / COLS, ...: no
+// division per element, row i's M[i][k] is one LDS word for all lanes of a row, M[k][j] runs along the lanes.
+template <int COLS, bool PATH_IN_LDS>
 __global__ __launch_bounds__(1024) void k_floyd_warshall(const uint8_t* __restrict__ adj, const int32_t* __restrict__ n_nodes,
                                                          int n_max, int32_t* __restrict__ dist, int32_t* __restrict__ path) {
     extern __shared__ uint16_t lds[];
@@ -387,13 +390,16 @@ __global__ __launch_bounds__(1024) void k_floyd_warshall(const uint8_t* __restri
     uint16_t* M = lds;                                   // [n][n]
     int16_t* P = reinterpret_cast<int16_t*>(lds + n * n);
     const uint8_t* A = adj + (int64_t)g * n_max * n_max;
-    const int j = threadIdx.x % kFwMax, r = threadIdx.x / kFwMax;
-    constexpr int kRows = 1024 / kFwMax;
+    int32_t* D = dist + (int64_t)g * n_max * n_max;
+    int32_t* Q = path + (int64_t)g * n_max * n_max;
+    const int j = threadIdx.x % COLS, r = threadIdx.x / COLS;
+    constexpr int kRows = 1024 / COLS;
     if (j < n)
         for (int i = r; i < n; i += kRows) {
             const uint16_t w = A[i * n_max + j];
             M[i * n + j] = i == j ? 0 : (w == 0 ? kFwInf : w);       // :27-32
-            P[i * n + j] = -1;
+            if (PATH_IN_LDS) P[i * n + j] = -1;
+            else Q[i * n_max + j] = -1;
         }
     __syncthreads();
     for (int k = 0; k < n; ++k) {
@@ -403,19 +409,19 @@ __global__ __launch_bounds__(1024) void k_floyd_warshall(const uint8_t* __restri
                 const uint16_t c = M[i * n + k] + kj;
                 if (M[i * n + j] > c && i != k) {        // row k and column k never improve through k
                     M[i * n + j] = c;
-                    P[i * n + j] = (int16_t)k;
+                    if (PATH_IN_LDS) P[i * n + j] = (int16_t)k;
+                    else Q[i * n_max + j] = k;
                 }
             }
         }
         __syncthreads();
     }
-    int32_t* D = dist + (int64_t)g * n_max * n_max;
-    int32_t* Q = path + (int64_t)g * n_max * n_max;
     if (j < n)
         for (int i = r; i < n; i += kRows) {
             const bool far = M[i * n + j] >= kFwInf;     // :49-53
             D[i * n_max + j] = far ? kFwInf : M[i * n + j];
-            Q[i * n_max + j] = far ? kFwInf : P[i * n + j];
+            if (PATH_IN_LDS) Q[i * n_max + j] = far ? kFwInf : P[i * n + j];
+            else if (far) Q[i * n_max + j] = kFwInf;
         }
 }
 
@@ -540,15 +546,28 @@ int tgt_floyd_warshall(const uint8_t* d_adj, const int32_t* d_n_nodes, int num_g
         return TGT_ERR_UNSUPPORTED;
     }
     if (num_graphs == 0) return TGT_OK;
-    const size_t lds = (size_t)n_max * n_max * 4;
-    static bool raised = false;
-    if (!raised && lds > 48 * 1024) {
-        TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_floyd_warshall),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kFwMax * kFwMax * 4)));
-        raised = true;
+    hipStream_t st = (hipStream_t)stream;
+    if (n_max <= kFwLdsPath) {
+        const size_t lds = (size_t)n_max * n_max * 4;
+        static bool raised = false;
+        if (!raised && lds > 48 * 1024) {
+            TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_floyd_warshall<128, true>),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kFwLdsPath * kFwLdsPath * 4)));
+            raised = true;
+        }
+        hipLaunchKernelGGL((k_floyd_warshall<128, true>), dim3(num_graphs), dim3(1024), lds, st, d_adj, d_n_nodes, n_max, d_dist,
+                           d_path);
+    } else {
+        const size_t lds = (size_t)n_max * n_max * 2;      // up to 128 KB of the CU's 160
+        static bool raised = false;
+        if (!raised) {
+            TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_floyd_warshall<256, false>),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)(kFwMax * kFwMax * 2)));
+            raised = true;
+        }
+        hipLaunchKernelGGL((k_floyd_warshall<256, false>), dim3(num_graphs), dim3(1024), lds, st, d_adj, d_n_nodes, n_max, d_dist,
+                           d_path);
     }
-    hipLaunchKernelGGL(k_floyd_warshall, dim3(num_graphs), dim3(1024), lds, (hipStream_t)stream, d_adj, d_n_nodes, n_max,
-                       d_dist, d_path);
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
 }

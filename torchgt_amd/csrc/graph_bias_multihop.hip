@@ -485,14 +485,14 @@ inline int head_tile(int H) { return H <= 8 ? 8 : (H <= 16 ? 16 : 32); }
 // right ends on a stack: with the current node a and the top b, a direct pair (path[a][b] == -1) is
 // the next hop, anything else pushes path[a][b].  Every stack entry is a distinct node of one shortest
 // path, so n entries suffice.
-constexpr int kGeiMaxNodes = 128;
+constexpr int kGeiMaxNodes = 256;
 constexpr int kGeiFar = 510;
 
-template <typename FeatT>
+template <typename FeatT, int MAXN>
 __global__ __launch_bounds__(128) void k_gen_edge_input(const int32_t* __restrict__ path, const FeatT* __restrict__ feat,
                                                         const int32_t* __restrict__ n_nodes, int n_max, int F, int max_dist,
                                                         int64_t total, int64_t* __restrict__ out) {
-    __shared__ uint8_t stack[kGeiMaxNodes][128];          // [depth][thread]: a thread's entries sit in its own bank column
+    __shared__ uint8_t stack[MAXN][128];                  // [depth][thread]: a thread's entries sit in its own bank column
     const int64_t t = (int64_t)blockIdx.x * 128 + threadIdx.x;
     if (t >= total) return;
     const int64_t plane = (int64_t)n_max * n_max;
@@ -509,7 +509,7 @@ __global__ __launch_bounds__(128) void k_gen_edge_input(const int32_t* __restric
         while (depth > 0 && hop < max_dist) {
             const int b = stack[depth - 1][threadIdx.x];
             const int k = P[a * n_max + b];
-            if (k < 0 || k >= n || depth >= kGeiMaxNodes) {        // a direct edge: the next hop (:89)
+            if (k < 0 || k >= n || depth >= MAXN) {        // a direct edge: the next hop (:89)
                 for (int f = 0; f < F; ++f) o[hop * F + f] = (int64_t)Fg[((int64_t)a * n_max + b) * F + f];
                 ++hop;
                 a = b;
@@ -679,12 +679,17 @@ int tgt_gen_edge_input(const int32_t* d_path, const void* d_edge_feat, int feat_
     const int64_t total = (int64_t)num_graphs * n_max * n_max;
     const dim3 grid((unsigned)((total + 127) / 128));
     hipStream_t st = (hipStream_t)stream;
-    if (feat_is_int64)
-        hipLaunchKernelGGL((k_gen_edge_input<int64_t>), grid, dim3(128), 0, st, d_path, (const int64_t*)d_edge_feat, d_n_nodes,
-                           n_max, F, max_dist, total, d_out);
-    else
-        hipLaunchKernelGGL((k_gen_edge_input<int32_t>), grid, dim3(128), 0, st, d_path, (const int32_t*)d_edge_feat, d_n_nodes,
-                           n_max, F, max_dist, total, d_out);
+#define TGT_GEI(FEAT_, MAXN_)                                                                                              \
+    hipLaunchKernelGGL((k_gen_edge_input<FEAT_, MAXN_>), grid, dim3(128), 0, st, d_path, (const FEAT_*)d_edge_feat, d_n_nodes, \
+                       n_max, F, max_dist, total, d_out)
+    if (n_max <= 128) {          // the stack of a walk is as deep as the graph is large
+        if (feat_is_int64) TGT_GEI(int64_t, 128);
+        else TGT_GEI(int32_t, 128);
+    } else {
+        if (feat_is_int64) TGT_GEI(int64_t, kGeiMaxNodes);
+        else TGT_GEI(int32_t, kGeiMaxNodes);
+    }
+#undef TGT_GEI
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
 }

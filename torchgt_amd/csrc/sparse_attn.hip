@@ -1075,21 +1075,27 @@ TGT_DECLARE_SHAPE(2, 1)    // H=2  d=8
 TGT_DECLARE_SHAPE(1, 1)    // H=1  d=8
 TGT_DECLARE_SHAPE(4, 2)    // H=2  d=16
 TGT_DECLARE_SHAPE(2, 2)    // H=1  d=16
+TGT_DECLARE_SHAPE(16, 4)   // H=4  d=32  (hidden 128 with 4 heads)
+TGT_DECLARE_SHAPE(8, 4)    // H=2  d=32
+TGT_DECLARE_SHAPE(4, 4)    // H=1  d=32
 #endif
 #if !defined(TGT_SPARSE_PART) || TGT_SPARSE_PART == 0
 TGT_DEFINE_SHAPE(8, 1)
 #ifndef TGT_ONLY_8x8
 TGT_DEFINE_SHAPE(1, 1)
+TGT_DEFINE_SHAPE(16, 4)
 #endif
 #endif
 #ifndef TGT_ONLY_8x8
 #if !defined(TGT_SPARSE_PART) || TGT_SPARSE_PART == 1
 TGT_DEFINE_SHAPE(8, 2)
 TGT_DEFINE_SHAPE(4, 2)
+TGT_DEFINE_SHAPE(8, 4)
 #endif
 #if !defined(TGT_SPARSE_PART) || TGT_SPARSE_PART == 2
 TGT_DEFINE_SHAPE(16, 2)
 TGT_DEFINE_SHAPE(2, 2)
+TGT_DEFINE_SHAPE(4, 4)
 #endif
 #if !defined(TGT_SPARSE_PART) || TGT_SPARSE_PART == 3
 TGT_DEFINE_SHAPE(2, 1)
@@ -1116,9 +1122,12 @@ static int dispatch(const Call& c, bool bwd) {
     TGT_CASE(1, 1)
     TGT_CASE(4, 2)
     TGT_CASE(2, 2)
+    TGT_CASE(16, 4)
+    TGT_CASE(8, 4)
+    TGT_CASE(4, 4)
 #endif
 #undef TGT_CASE
-    set_error("no kernel for H=%d d=%d (d must be 8 or 16 and H*d/8 one of 1,2,4,8,16)", c.H, c.d);
+    set_error("no kernel for H=%d d=%d (d must be 8, 16 or 32 and H*d/8 one of 1,2,4,8,16, at least d/8)", c.H, c.d);
     return TGT_ERR_UNSUPPORTED;
 }
 
