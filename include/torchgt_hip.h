@@ -264,9 +264,10 @@ int tgt_dense_attn_ids_fwd(const void* d_q, const void* d_k, const void* d_v, co
 /* Backward: dq, dk, dv as tgt_dense_attn_dropout_bwd, and the gradients of the three tables (all three or
  * all NULL; autograd of the embedding lookups in the reference, row 0 of the spatial and edge tables is the
  * padding index and gets zero) summed over this call's batch: workgroups add dS into fixed-point LDS
- * accumulators (integer atomics, one power-of-two scale per (graph, head) from a bound on its dS; one unit is
- * at most 2^-21 of that bound) and their partials are added in a fixed order: results are reproducible bit
- * for bit.  d_workspace: tgt_dense_attn_ids_bwd_workspace_bytes(...) bytes, 16-byte aligned,
+ * accumulators (integer atomics, one power-of-two scale per (graph, head) from a bound B on a row's sum of |dS|:
+ * no spatial accumulator exceeds S B, no edge accumulator F S B - a position adds its dS once per edge feature -
+ * and one unit is at most 2^-21 B, for the edge table 2^-21 B times F rounded up to a power of two) and their
+ * partials are added in a fixed order: results are reproducible bit for bit.  d_workspace: tgt_dense_attn_ids_bwd_workspace_bytes(...) bytes, 16-byte aligned,
  * needed only with table gradients. */
 int64_t tgt_dense_attn_ids_bwd_workspace_bytes(int b, int H, int num_spatial, int num_edges);
 int tgt_dense_attn_ids_bwd(const void* d_q, const void* d_k, const void* d_v, const void* d_attn_bias,

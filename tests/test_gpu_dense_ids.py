@@ -88,7 +88,9 @@ def _oracle(q, k, v, ab, sp, et_ids, st, et, vd, dout, keep=None, p=0.0):
 CASES = [(9, 128, 8, 8, 1, 22, 5), (5, 31, 8, 8, 1, 22, 5), (10, 49, 4, 16, 3, 40, 64), (3, 96, 8, 8, 2, 512, 1537),
          (17, 19, 16, 8, 1, 7, 3), (4, 66, 2, 32, 1, 22, 5),
          # S = 4 (no whole group of sixteen keys), S = 16 (exactly one), S = 33 (a one-row last tile behind one full tile)
-         (3, 3, 2, 8, 1, 5, 4), (2, 15, 8, 8, 2, 22, 5), (3, 32, 8, 8, 1, 22, 5)]
+         (3, 3, 2, 8, 1, 5, 4), (2, 15, 8, 8, 2, 22, 5), (3, 32, 8, 8, 1, 22, 5),
+         # one edge id in all four features of every edge position: the edge accumulator collects F dS per position
+         (4, 40, 8, 8, 4, 5, 2)]
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])

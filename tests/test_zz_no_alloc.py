@@ -41,9 +41,16 @@ def _fwd_both(e, n, H, d, dtype, seed, cuda):
     Z_a, Z_b = torch.empty(n, H, device=cuda), torch.full((n, H), float("nan"), device=cuda)
     _lib.check(L.tgt_sparse_attn_fwd(plan.handle, P(q), P(k), P(v), P(bias), _lib.BIAS_EDGE_HEAD, H, d, code, P(out_a),
                                      P(Z_a), P(ws), ws.numel(), stream))
+    # with kernel timing switched on (the workspace forward then takes events from a pool that grows on demand):
+    # the call neither creates events nor moves the device's free memory
+    torch.cuda.synchronize()
+    L.tgt_timing_enable(1)
+    free_before = torch.cuda.mem_get_info(cuda)[0]
     _lib.check(L.tgt_sparse_attn_fwd_noalloc(plan.handle, P(q), P(k), P(v), P(bias), _lib.BIAS_EDGE_HEAD, H, d, code,
                                              P(out_b), P(Z_b), stream))
     torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info(cuda)[0] == free_before
+    L.tgt_timing_enable(0)
     assert torch.equal(out_a, out_b) and torch.equal(Z_a, Z_b)
     ref, _ = osa.sparse_attention(q.double().cpu(), k.double().cpu(), v.double().cpu(), ei.cpu(), bias.double().cpu())
     rel = (out_b.double().cpu() - ref).abs().max().item() / ref.abs().max().item()

@@ -188,7 +188,8 @@ enum KernelSlot { KS_FWD = 0, KS_NODE_SIDE, KS_BWD, KS_DENSE_FWD, KS_DENSE_BWD, 
 // its scope when timing is enabled; does nothing otherwise.
 class KernelTimer {
 public:
-    KernelTimer(int slot, hipStream_t st);
+    // `on` false: times nothing (a caller that must not create events, which taking one from an empty pool does)
+    KernelTimer(int slot, hipStream_t st, bool on = true);
     ~KernelTimer();
     KernelTimer(const KernelTimer&) = delete;
     KernelTimer& operator=(const KernelTimer&) = delete;

@@ -172,7 +172,8 @@ __device__ __forceinline__ float cvt1(float x) { return x; }
 // bit.  Every (graph, head) pair gets its own power-of-two scale from a bound on its dS: the rows
 // of the softmax sum to one, so sum_k |dS[q,k]| <= 2 max_q |dout_q|_1 max|v| / (1 - p) =: B and no
 // accumulator of one pair can exceed S B; with scale = 2^22 / B' (B' = B rounded up to a power of
-// two) that stays below 2^30 for S <= 256, and one unit is 2^-22 B'.  After each pair the
+// two) that stays below 2^30 for S <= 256, and one unit is 2^-22 B'.  A position adds its dS to the edge table once
+// per edge feature, so an edge accumulator is bounded by F S B: its scale is 2^ceil(log2 F) times smaller.  After each pair the
 // workgroup converts its integer sums to float and adds them to its partial in global memory.
 // ---------------------------------------------------------------------------
 struct IdsArgs {
@@ -311,6 +312,7 @@ struct IdsAcc {
     int *hot_copy, *accS, *accE;
     int F, ns, ne, hot_n;
     float scale;               // of the current pair: dS * scale is what the accumulators count
+    float scale_e;             // the same for the edge table: scale / 2^ceil(log2 F), a position adds its dS once per feature
     bool on;
 };
 // (id 0 is added too, into a slot that is never read: one test less per position)
@@ -321,7 +323,7 @@ __device__ __forceinline__ void acc_spatial(const IdsAcc& c, float ds, uint32_t 
     }
 }
 __device__ __forceinline__ void acc_edge(const IdsAcc& c, float ds, uint32_t e) {
-    if (ds != 0.f && e != 0 && (int)e < c.ne) atomicAdd(c.accE + e, __float2int_rn(ds * c.scale));
+    if (ds != 0.f && e != 0 && (int)e < c.ne) atomicAdd(c.accE + e, __float2int_rn(ds * c.scale_e));
 }
 // one position whose ids are still in memory
 __device__ __forceinline__ void acc_position(const IdsAcc& c, float ds, int64_t at) {
@@ -860,9 +862,13 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
         const float B = 2.f * (DROP ? da.inv_keep : 1.0f) * __int_as_float(il.bound[0]) * __int_as_float(il.bound[1]);
         int e = 0;
         acc.scale = 0.f;
+        acc.scale_e = 0.f;
         if (acc.on && B > 0.f && B < INFINITY) {
             (void)frexpf(B, &e);
             acc.scale = ldexpf(1.f, 22 - e);
+            // an edge id repeated in all F features of a position collects F dS: the bound of an edge accumulator is
+            // F S B, and its unit is 2^ceil(log2 F) times coarser
+            acc.scale_e = ldexpf(1.f, 22 - e - (ia.F > 1 ? 32 - __clz(ia.F - 1) : 0));
         }
     }
 
@@ -1151,7 +1157,7 @@ __global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, 
         // [ns] spatial, [ne] edge (with the mean's 1 / F), [1] virtual - and the accumulators start the next pair at
         // zero.  Only this workgroup touches its partial, one thread per entry.
         float* mine = ia.partial + (int64_t)blockIdx.x * (ia.ns + ia.ne + 1);
-        const float unit = acc.scale > 0.f ? 1.f / acc.scale : 0.f, unit_e = unit / (float)ia.F;
+        const float unit = acc.scale > 0.f ? 1.f / acc.scale : 0.f, unit_e = (acc.scale_e > 0.f ? 1.f / acc.scale_e : 0.f) / (float)ia.F;
         for (int k = threadIdx.x; k <= ia.ns; k += blockDim.x) {
             int t = il.accS[k];
             il.accS[k] = 0;

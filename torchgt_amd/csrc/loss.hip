@@ -26,22 +26,25 @@ __device__ __forceinline__ void st(uint16_t* p, float v) {
 template <typename T>
 __global__ __launch_bounds__(kLossBlock) void k_nll_fwd(const T* __restrict__ logp, const int64_t* __restrict__ target, int64_t N,
                                                          int C, int64_t ignore_index, float* __restrict__ partial) {
-    __shared__ float red[2][kLossBlock / 64];
-    float s = 0.f, n = 0.f;
+    __shared__ float red[kLossBlock / 64];
+    __shared__ int cnt[kLossBlock / 64];
+    float s = 0.f;
+    int n = 0;      // rows counted as integers: a float count is exact only up to 2^24 rows
     for (int64_t i = (int64_t)blockIdx.x * kLossBlock + threadIdx.x; i < N; i += (int64_t)gridDim.x * kLossBlock) {
         const int64_t t = target[i];
-        if (t != ignore_index && t >= 0 && t < C) { s += ld(logp + i * C + t); n += 1.f; }
+        if (t != ignore_index && t >= 0 && t < C) { s += ld(logp + i * C + t); n += 1; }
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) { s += __shfl_xor(s, o); n += __shfl_xor(n, o); }
-    if ((threadIdx.x & 63) == 0) { red[0][threadIdx.x >> 6] = s; red[1][threadIdx.x >> 6] = n; }
+    if ((threadIdx.x & 63) == 0) { red[threadIdx.x >> 6] = s; cnt[threadIdx.x >> 6] = n; }
     __syncthreads();
     if (threadIdx.x == 0) {
-        float a = 0.f, b = 0.f;
+        float a = 0.f;
+        int b = 0;
 #pragma unroll
-        for (int w = 0; w < kLossBlock / 64; ++w) { a += red[0][w]; b += red[1][w]; }
+        for (int w = 0; w < kLossBlock / 64; ++w) { a += red[w]; b += cnt[w]; }
         partial[2 * blockIdx.x] = a;
-        partial[2 * blockIdx.x + 1] = b;
+        partial[2 * blockIdx.x + 1] = __int_as_float(b);       // the count travels as its bit pattern
     }
 }
 
@@ -49,16 +52,18 @@ __global__ __launch_bounds__(kLossBlock) void k_nll_fwd(const T* __restrict__ lo
 template <typename T>
 __global__ __launch_bounds__(kLossBlock) void k_nll_finish(const float* __restrict__ partial, int workers, T* __restrict__ loss,
                                                             float* __restrict__ count) {
-    __shared__ float red[2][kLossBlock];
-    float s = 0.f, n = 0.f;
-    for (int w = threadIdx.x; w < workers; w += kLossBlock) { s += partial[2 * w]; n += partial[2 * w + 1]; }
-    red[0][threadIdx.x] = s; red[1][threadIdx.x] = n;
+    __shared__ float red[kLossBlock];
+    __shared__ long long cnt[kLossBlock];
+    float s = 0.f;
+    long long n = 0;
+    for (int w = threadIdx.x; w < workers; w += kLossBlock) { s += partial[2 * w]; n += __float_as_int(partial[2 * w + 1]); }
+    red[threadIdx.x] = s; cnt[threadIdx.x] = n;
     __syncthreads();
     for (int o = kLossBlock / 2; o > 0; o >>= 1) {
-        if ((int)threadIdx.x < o) { red[0][threadIdx.x] += red[0][threadIdx.x + o]; red[1][threadIdx.x] += red[1][threadIdx.x + o]; }
+        if ((int)threadIdx.x < o) { red[threadIdx.x] += red[threadIdx.x + o]; cnt[threadIdx.x] += cnt[threadIdx.x + o]; }
         __syncthreads();
     }
-    if (threadIdx.x == 0) { st(loss, -red[0][0] / red[1][0]); *count = red[1][0]; }
+    if (threadIdx.x == 0) { st(loss, -red[0] / (float)cnt[0]); *count = (float)cnt[0]; }
 }
 
 // VE consecutive elements of the flattened [N, C] per lane (N * C is a multiple of VE)

@@ -952,7 +952,7 @@ static int run_fwd(const Call& c) {
     a.counters = c.fwd_counters ? c.fwd_counters : reinterpret_cast<int32_t*>(c.ws + L.counters);
     const int nb = sch->fwd_blocks;
     if (nb > 0) {
-        KernelTimer t(KS_FWD, c.st);
+        KernelTimer t(KS_FWD, c.st, !c.no_alloc);       // the entry point that allocates nothing creates no events either
         const bool hb = c.bias_mode != TGT_BIAS_NONE;
         if (c.init != nullptr && (c.bias_mode & TGT_BIAS_PLAN_ORDER)) {
             set_error("block attention takes the bias in the caller's edge order");

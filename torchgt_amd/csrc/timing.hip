@@ -39,8 +39,8 @@ static hipEvent_t take_event() {
 
 bool timing_enabled() { return g_enabled; }
 
-KernelTimer::KernelTimer(int slot, hipStream_t st) : slot_(slot), st_(st), start_(nullptr) {
-    if (!g_enabled) return;
+KernelTimer::KernelTimer(int slot, hipStream_t st, bool on) : slot_(slot), st_(st), start_(nullptr) {
+    if (!g_enabled || !on) return;
     std::lock_guard<std::mutex> lk(g_mu);
     start_ = take_event();
     if (start_) (void)hipEventRecord(start_, st_);

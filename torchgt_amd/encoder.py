@@ -28,7 +28,8 @@ def nll_loss(log_probs, target, ignore_index=-100):
     gt_sp/evaluate.py:52): mean over the rows whose target is not ``ignore_index``, no class weights.
     ``torch.ops.torchgt.nll_loss``: one row per lane and a fixed-order sum (torch's kernel walks the rows with a
     single workgroup, ~95 + 60 us forward + backward for 64 K rows against ~5 + 3 here).  A target outside
-    [0, C) other than ``ignore_index`` counts as ignored."""
+    [0, C) other than ``ignore_index`` counts as ignored - torch raises there: check labels that may be corrupt
+    before they reach the loss."""
     return _ext.ops().nll_loss(log_probs, target, int(ignore_index))
 
 
