@@ -148,7 +148,8 @@ __device__ __forceinline__ void wave_lds_fence() {
 // heads at once.  The K and V rows of a tile are staged in LDS once (coalesced) and every head's
 // two products take their operands from there.
 // FINAL: the tiles are all there is (no remaining edges): the kernel divides by Z + eps and writes
-// the output rows and Z themselves; otherwise it leaves fp32 sums for the sparse kernel to add.
+// the output rows and Z themselves; otherwise it does so for the destinations that have no remaining edge and
+// leaves fp32 sums of the others for the sparse kernel to add (which skips the former).
 template <typename T, int D, int H, bool FINAL>
 __global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_fwd(const int32_t* __restrict__ grp_c0,
                                                               const int32_t* __restrict__ grp_off,
@@ -156,7 +157,8 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_fwd(const int
                                                               const T* __restrict__ Q, const T* __restrict__ K,
                                                               const T* __restrict__ V, float* __restrict__ acc,
                                                               float* __restrict__ Zp, T* __restrict__ out,
-                                                              float inv_scale) {
+                                                              float* __restrict__ Zout,
+                                                              const int32_t* __restrict__ rem_rowptr, float inv_scale) {
     constexpr int HD = H * D;
     constexpr int kTileWaves = tile_waves<HD>();
     __shared__ short lds[kTileWaves * (rm_size<HD>() + tr_size<HD>())];
@@ -200,18 +202,20 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_fwd(const int
             o[h] = mfma16(av, t_pack(w), o[h]);                    // O^T[dd 4kq+r][destination col]
         }
     }
+    // a destination without remaining edges (row pointers of the plan that holds them) is finished here as well
+    const bool fin = FINAL || rem_rowptr[c0 + col + 1] == rem_rowptr[c0 + col];
 #pragma unroll
     for (int h = 0; h < H; ++h) {
         float zz = z[h];
         zz += __shfl_xor(zz, 16);
         zz += __shfl_xor(zz, 32);
-        if (FINAL) {
+        if (fin) {
             const float inv = 1.0f / (zz + kTileEps);
             if (kval) t_st4(out + (int64_t)(c0 + col) * HD + h * D + kq * 4, o[h].x * inv, o[h].y * inv, o[h].z * inv, o[h].w * inv);
         } else if (kval) {
             *reinterpret_cast<bfloat4*>(acc + (int64_t)(c0 + col) * HD + h * D + kq * 4) = o[h];
         }
-        if (kq == 0) Zp[(int64_t)(c0 + col) * H + h] = zz;
+        if (kq == 0) (fin ? Zout : Zp)[(int64_t)(c0 + col) * H + h] = zz;
     }
 }
 
@@ -224,6 +228,7 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_bwd_dst(const
                                                                   const T* __restrict__ V, const T* __restrict__ dO,
                                                                   const float2* __restrict__ nd,
                                                                   float* __restrict__ dq_part, T* __restrict__ dq_out,
+                                                                  const int32_t* __restrict__ rem_rowptr,
                                                                   float inv_scale) {
     constexpr int HD = H * D;
     constexpr int kTileWaves = tile_waves<HD>();
@@ -280,11 +285,12 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_bwd_dst(const
         }
     }
     if (kval) {
+        const bool fin = FINAL || rem_rowptr[c0 + col + 1] == rem_rowptr[c0 + col];      // no remaining edge into this row
 #pragma unroll
         for (int h = 0; h < H; ++h) {
             bfloat4 o;
             o.x = dq[h].x * inv_scale; o.y = dq[h].y * inv_scale; o.z = dq[h].z * inv_scale; o.w = dq[h].w * inv_scale;
-            if (FINAL) t_st4(dq_out + (int64_t)(c0 + col) * HD + h * D + kq * 4, o.x, o.y, o.z, o.w);
+            if (fin) t_st4(dq_out + (int64_t)(c0 + col) * HD + h * D + kq * 4, o.x, o.y, o.z, o.w);
             else *reinterpret_cast<bfloat4*>(dq_part + (int64_t)(c0 + col) * HD + h * D + kq * 4) = o;
         }
     }
@@ -300,7 +306,8 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_bwd_src(const
                                                                   const float2* __restrict__ nd,
                                                                   float* __restrict__ dk_part,
                                                                   float* __restrict__ dv_part, T* __restrict__ dk_out,
-                                                                  T* __restrict__ dv_out, float inv_scale) {
+                                                                  T* __restrict__ dv_out,
+                                                                  const int32_t* __restrict__ rem_rowptr, float inv_scale) {
     constexpr int HD = H * D;
     constexpr int kTileWaves = tile_waves<HD>();
     constexpr int PER_WAVE = 2 * rm_size<HD>() + 2 * tr_size<HD>() + 4 * kTile * H;   // + nd tile (float2 = 4 shorts)
@@ -363,11 +370,12 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_bwd_src(const
         }
     }
     if (kval) {
+        const bool fin = FINAL || rem_rowptr[r0 + col + 1] == rem_rowptr[r0 + col];      // no remaining edge out of this row
 #pragma unroll
         for (int h = 0; h < H; ++h) {
             bfloat4 o;
             o.x = dk[h].x * inv_scale; o.y = dk[h].y * inv_scale; o.z = dk[h].z * inv_scale; o.w = dk[h].w * inv_scale;
-            if (FINAL) {
+            if (fin) {
                 t_st4(dk_out + (int64_t)(r0 + col) * HD + h * D + kq * 4, o.x, o.y, o.z, o.w);
                 t_st4(dv_out + (int64_t)(r0 + col) * HD + h * D + kq * 4, dv[h].x, dv[h].y, dv[h].z, dv[h].w);
             } else {
@@ -443,7 +451,7 @@ static int upload(DevBuf& b, const std::vector<X>& v, hipStream_t st) {
 // rows without tiles) and the sparse kernels are not run.
 template <typename T, int D, int H>
 static int tile_fwd_launch_s(const tgt_tiles* tl, const void* q, const void* k, const void* v, float* acc, float* Zp,
-                             void* final_out, hipStream_t st) {
+                             void* final_out, void* out, float* Zout, const int32_t* rem_rowptr, hipStream_t st) {
     constexpr int W = tile_waves<H * D>();
     const float inv_scale = 1.0f / sqrtf((float)D);
     KernelTimer t(KS_TILE_FWD, st);
@@ -455,11 +463,11 @@ static int tile_fwd_launch_s(const tgt_tiles* tl, const void* q, const void* k, 
         if (tl->n_dst_groups > 0)
             hipLaunchKernelGGL((k_tile_fwd<T, D, H, true>), grid, block, 0, st, tl->dst_c0.as<int32_t>(),
                                tl->dst_off.as<int32_t>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
-                               (const T*)k, (const T*)v, acc, Zp, (T*)final_out, inv_scale);
+                               (const T*)k, (const T*)v, acc, Zp, (T*)final_out, Zp, (const int32_t*)nullptr, inv_scale);
     } else if (tl->n_dst_groups > 0) {
         hipLaunchKernelGGL((k_tile_fwd<T, D, H, false>), grid, block, 0, st, tl->dst_c0.as<int32_t>(),
                            tl->dst_off.as<int32_t>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
-                           (const T*)k, (const T*)v, acc, Zp, (T*)nullptr, inv_scale);
+                           (const T*)k, (const T*)v, acc, Zp, (T*)out, Zout, rem_rowptr, inv_scale);
     }
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
@@ -468,6 +476,7 @@ static int tile_fwd_launch_s(const tgt_tiles* tl, const void* q, const void* k, 
 template <typename T, int D, int H>
 static int tile_bwd_launch_s(const tgt_tiles* tl, const void* q, const void* k, const void* v, const void* dout,
                              const float2* nd, float* dq, float* dk, float* dv, void* f_dq, void* f_dk, void* f_dv,
+                             void* o_dq, void* o_dk, void* o_dv, const int32_t* rem_dst, const int32_t* rem_src,
                              hipStream_t st) {
     constexpr int W = tile_waves<H * D>();
     const float inv_scale = 1.0f / sqrtf((float)D);
@@ -483,20 +492,20 @@ static int tile_bwd_launch_s(const tgt_tiles* tl, const void* q, const void* k, 
         if (tl->n_dst_groups > 0)
             hipLaunchKernelGGL((k_tile_bwd_dst<T, D, H, true>), gd, block, 0, st, tl->dst_c0.as<int32_t>(),
                                tl->dst_off.as<int32_t>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
-                               (const T*)k, (const T*)v, (const T*)dout, nd, dq, (T*)f_dq, inv_scale);
+                               (const T*)k, (const T*)v, (const T*)dout, nd, dq, (T*)f_dq, (const int32_t*)nullptr, inv_scale);
         if (tl->n_src_groups > 0)
             hipLaunchKernelGGL((k_tile_bwd_src<T, D, H, true>), gs, block, 0, st, tl->src_r0.as<int32_t>(),
                                tl->src_off.as<int32_t>(), tl->src_c0.as<int32_t>(), tl->n_src_groups, (const T*)q,
-                               (const T*)k, (const T*)v, (const T*)dout, nd, dk, dv, (T*)f_dk, (T*)f_dv, inv_scale);
+                               (const T*)k, (const T*)v, (const T*)dout, nd, dk, dv, (T*)f_dk, (T*)f_dv, (const int32_t*)nullptr, inv_scale);
     } else {
         if (tl->n_dst_groups > 0)
             hipLaunchKernelGGL((k_tile_bwd_dst<T, D, H, false>), gd, block, 0, st, tl->dst_c0.as<int32_t>(),
                                tl->dst_off.as<int32_t>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
-                               (const T*)k, (const T*)v, (const T*)dout, nd, dq, (T*)nullptr, inv_scale);
+                               (const T*)k, (const T*)v, (const T*)dout, nd, dq, (T*)o_dq, rem_dst, inv_scale);
         if (tl->n_src_groups > 0)
             hipLaunchKernelGGL((k_tile_bwd_src<T, D, H, false>), gs, block, 0, st, tl->src_r0.as<int32_t>(),
                                tl->src_off.as<int32_t>(), tl->src_c0.as<int32_t>(), tl->n_src_groups, (const T*)q,
-                               (const T*)k, (const T*)v, (const T*)dout, nd, dk, dv, (T*)nullptr, (T*)nullptr,
+                               (const T*)k, (const T*)v, (const T*)dout, nd, dk, dv, (T*)o_dk, (T*)o_dv, rem_src,
                                inv_scale);
     }
     TGT_HIP_CHECK(hipGetLastError());
@@ -508,8 +517,9 @@ static int tile_bwd_launch_s(const tgt_tiles* tl, const void* q, const void* k, 
 
 template <typename T>
 static int tile_fwd_launch(const tgt_tiles* tl, const void* q, const void* k, const void* v, float* acc, float* Zp,
-                           void* final_out, int H, int d, hipStream_t st) {
-#define X(D_, H_) if (d == D_ && H == H_) return tile_fwd_launch_s<T, D_, H_>(tl, q, k, v, acc, Zp, final_out, st);
+                           void* final_out, void* out, float* Zout, const int32_t* rem_rowptr, int H, int d, hipStream_t st) {
+#define X(D_, H_) \
+    if (d == D_ && H == H_) return tile_fwd_launch_s<T, D_, H_>(tl, q, k, v, acc, Zp, final_out, out, Zout, rem_rowptr, st);
     TGT_TILE_SHAPES(X)
 #undef X
     set_error("block attention: no tile kernel for H=%d, d=%d", H, d);
@@ -519,9 +529,12 @@ static int tile_fwd_launch(const tgt_tiles* tl, const void* q, const void* k, co
 template <typename T>
 static int tile_bwd_launch(const tgt_tiles* tl, const void* q, const void* k, const void* v, const void* dout,
                            const float2* nd, float* dq, float* dk, float* dv, void* f_dq, void* f_dk, void* f_dv,
-                           int H, int d, hipStream_t st) {
-#define X(D_, H_) \
-    if (d == D_ && H == H_) return tile_bwd_launch_s<T, D_, H_>(tl, q, k, v, dout, nd, dq, dk, dv, f_dq, f_dk, f_dv, st);
+                           void* o_dq, void* o_dk, void* o_dv, const int32_t* rem_dst, const int32_t* rem_src, int H, int d,
+                           hipStream_t st) {
+#define X(D_, H_)                                                                                                        \
+    if (d == D_ && H == H_)                                                                                              \
+        return tile_bwd_launch_s<T, D_, H_>(tl, q, k, v, dout, nd, dq, dk, dv, f_dq, f_dk, f_dv, o_dq, o_dk, o_dv, rem_dst, \
+                                            rem_src, st);
     TGT_TILE_SHAPES(X)
 #undef X
     set_error("block attention: no tile kernel for H=%d, d=%d", H, d);
@@ -629,8 +642,10 @@ int tgt_block_attn_fwd(const tgt_tiles_t* tiles, const tgt_plan_t* plan, const v
     const bool tiles_only = plan->E == 0;
     void* fin = tiles_only ? d_out : nullptr;
     float* Zdst = tiles_only ? d_Z : Zp;
-    rc = dtype == TGT_DTYPE_F32 ? tgt::tile_fwd_launch<float>(tiles, d_q, d_k, d_v, acc, Zdst, fin, H, d, st)
-                                : tgt::tile_fwd_launch<tgt::tbf16>(tiles, d_q, d_k, d_v, acc, Zdst, fin, H, d, st);
+    // with remaining edges: the tile kernels still finish the rows that have none (the sparse kernels skip them)
+    const int32_t* rem = plan->dst.rowptr;
+    rc = dtype == TGT_DTYPE_F32 ? tgt::tile_fwd_launch<float>(tiles, d_q, d_k, d_v, acc, Zdst, fin, d_out, d_Z, rem, H, d, st)
+                                : tgt::tile_fwd_launch<tgt::tbf16>(tiles, d_q, d_k, d_v, acc, Zdst, fin, d_out, d_Z, rem, H, d, st);
     if (rc || tiles_only) return rc;
     tgt::TileInit init{};
     init.acc = acc; init.Z = Zp; init.cover_dst = tiles->cover_dst.as<uint8_t>();
@@ -662,8 +677,10 @@ int tgt_block_attn_bwd(const tgt_tiles_t* tiles, const tgt_plan_t* plan, const v
     void* f_dk = tiles_only ? d_dk : nullptr;
     void* f_dv = tiles_only ? d_dv : nullptr;
     rc = dtype == TGT_DTYPE_F32
-             ? tgt::tile_bwd_launch<float>(tiles, d_q, d_k, d_v, d_dout, nd, dq, dk, dv, f_dq, f_dk, f_dv, H, d, st)
-             : tgt::tile_bwd_launch<tgt::tbf16>(tiles, d_q, d_k, d_v, d_dout, nd, dq, dk, dv, f_dq, f_dk, f_dv, H, d, st);
+             ? tgt::tile_bwd_launch<float>(tiles, d_q, d_k, d_v, d_dout, nd, dq, dk, dv, f_dq, f_dk, f_dv, d_dq, d_dk, d_dv,
+                                           plan->dst.rowptr, plan->src.rowptr, H, d, st)
+             : tgt::tile_bwd_launch<tgt::tbf16>(tiles, d_q, d_k, d_v, d_dout, nd, dq, dk, dv, f_dq, f_dk, f_dv, d_dq, d_dk,
+                                                d_dv, plan->dst.rowptr, plan->src.rowptr, H, d, st);
     if (rc || tiles_only) return rc;     // (no edges: there is no per-edge bias gradient to write either)
     tgt::TileInit init{};
     init.dq = dq; init.dk = dk; init.dv = dv;

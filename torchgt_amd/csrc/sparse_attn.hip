@@ -117,13 +117,30 @@ __device__ __forceinline__ void store_dev(float* p, float v) {
 __device__ __forceinline__ float load_dev(const float* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// Eight consecutive floats (32-byte aligned) at device scope: two 16-byte accesses with the sc1 bit, which the
+// atomic builtins above would split into eight 4-byte ones.
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ void store8_dev(float* p, const float (&x)[8]) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) store_dev(p + i, x[i]);
+    const f32x4_t a = {x[0], x[1], x[2], x[3]}, b = {x[4], x[5], x[6], x[7]};
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\tglobal_store_dwordx4 %0, %2, off offset:16 sc1"
+                 :: "v"(p), "v"(a), "v"(b) : "memory");
 }
-__device__ __forceinline__ void load8_dev(const float* p, float (&x)[8]) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) x[i] = load_dev(p + i);
+// The load in two steps, so that several can be in flight: dev_load8 asks, dev_arrived waits for everything asked
+// (the registers pass through it, which keeps their uses behind it).
+struct Dev8 { f32x4_t a, b; };
+__device__ __forceinline__ void dev_load8(const float* p, Dev8& r) {
+    asm volatile("global_load_dwordx4 %0, %2, off sc1\n\tglobal_load_dwordx4 %1, %2, off offset:16 sc1"
+                 : "=&v"(r.a), "=&v"(r.b) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void dev_arrived(Dev8& r0, Dev8& r1) {
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(r0.a), "+v"(r0.b), "+v"(r1.a), "+v"(r1.b) :: "memory");
+}
+__device__ __forceinline__ void dev_arrived(Dev8& r0, Dev8& r1, Dev8& r2, Dev8& r3) {
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+v"(r0.a), "+v"(r0.b), "+v"(r1.a), "+v"(r1.b), "+v"(r2.a), "+v"(r2.b), "+v"(r3.a), "+v"(r3.b) :: "memory");
+}
+__device__ __forceinline__ void dev_unpack(const Dev8& r, float (&x)[8]) {
+    x[0] = r.a.x; x[1] = r.a.y; x[2] = r.a.z; x[3] = r.a.w; x[4] = r.b.x; x[5] = r.b.y; x[6] = r.b.z; x[7] = r.b.w;
 }
 
 __device__ __forceinline__ float dot8(const float (&a)[8], const float (&b)[8]) {
@@ -590,9 +607,12 @@ __device__ __forceinline__ void wave_rows(const Common& c, const SideArgs& s, co
     const int lane = threadIdx.x & (kWave - 1);
     const int sub = lane / G, gl = lane % G;
     const int slot = gl / LPE, el = gl % LPE;
-    const bool valid = sub < (int)(__builtin_amdgcn_readfirstlane(rec.code) >> 8);
+    bool valid = sub < (int)(__builtin_amdgcn_readfirstlane(rec.code) >> 8);
     int row = 0, start = 0, len = 0;
     if (valid) { row = rec.row[sub]; start = rec.start[sub]; len = rec.len[sub]; }
+    // block path: a row that has tiles and no edge here was written by the tile kernels (they see the same row
+    // pointers); nothing of it is loaded or stored
+    if (TILES) valid = valid && !(len == 0 && s.cover[row] != 0);
     Acc acc;
     if (INLINE) walk_record<T, LPE, LPH, S, MODE, HASB>(c, s, rec, row, start, len, slot, el, valid, acc);
     else walk_range<T, LPE, LPH, S, MODE, HASB>(c, s, row, start, len, slot, el, valid, acc);
@@ -644,16 +664,26 @@ __device__ __forceinline__ void sum_slots(const SideArgs& s, const int first, co
             const float* srcA = s.part + (int64_t)(first + p) * PS;
             const float* srcB = s.part + (int64_t)(first + (two ? p + NGROUP : p)) * PS;
             float tA[8], tB[8], uA[8], uB[8], zA = 0.f, zB = 0.f;
-            load8_dev(srcA + el2 * 8, tA);
-            load8_dev(srcB + el2 * 8, tB);
+            Dev8 rA, rB, sA, sB;
+            dev_load8(srcA + el2 * 8, rA);
+            dev_load8(srcB + el2 * 8, rB);
             if (MODE == MODE_BWD_SRC) {
-                load8_dev(srcA + HD + el2 * 8, uA);
-                load8_dev(srcB + HD + el2 * 8, uB);
+                dev_load8(srcA + HD + el2 * 8, sA);
+                dev_load8(srcB + HD + el2 * 8, sB);
             }
             if (MODE == MODE_FWD) {
                 zA = load_dev(srcA + HD + el2 / LPH);
                 zB = load_dev(srcB + HD + el2 / LPH);
             }
+            if (MODE == MODE_BWD_SRC) {
+                dev_arrived(rA, rB, sA, sB);
+                dev_unpack(sA, uA);
+                dev_unpack(sB, uB);
+            } else {
+                dev_arrived(rA, rB);
+            }
+            dev_unpack(rA, tA);
+            dev_unpack(rB, tB);
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 a0[i] += tA[i];
