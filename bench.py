@@ -810,16 +810,24 @@ def bench_sparse(args):
     E = e.shape[1]
 
     ei = torch.from_numpy(e).to(dev)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    plan = GraphPlan(ei, n)
-    torch.cuda.synchronize()
-    plan_first_ms = (time.perf_counter() - t0) * 1e3
-    t0 = time.perf_counter()
-    plan2 = GraphPlan(ei, n)
-    torch.cuda.synchronize()
-    plan_ms = (time.perf_counter() - t0) * 1e3
-    plan2.close()
+
+    def build_plan():
+        # everything a first attention call on a new edge list pays for: sorted views, schedule, wave records
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        p = GraphPlan(ei, n)
+        _lib.check(_lib.lib().tgt_plan_prepare(p.handle, H, d, torch.cuda.current_stream(dev).cuda_stream))
+        torch.cuda.synchronize()
+        return p, (time.perf_counter() - t0) * 1e3
+
+    plan, plan_first_ms = build_plan()
+    samples = []
+    for _ in range(5):          # later builds find their memory in torch's caching allocator
+        p2, ms = build_plan()
+        p2.close()
+        del p2
+        samples.append(ms)
+    plan_ms = sorted(samples)[len(samples) // 2]
 
     g = torch.Generator().manual_seed(42)
     q, k, v = (torch.randn(n, H, d, generator=g).to(dev, tdt) for _ in range(3))

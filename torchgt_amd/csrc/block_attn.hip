@@ -66,17 +66,26 @@ __device__ __forceinline__ void t_st4(tbf16* p, float a, float b, float c, float
 }
 
 // Rows no tile covers get zeros when the tile kernels write final results (no remaining edges).  The rows are
-// listed when the tile set is built: a reordered graph normally leaves none and then nothing is launched.
+// listed when the tile set is built; the workgroups behind the last tile group of a launch write them (eight
+// lanes per row, 16-byte stores), so they cost no launch of their own.
+struct BareRows {
+    const int32_t* rows;
+    int32_t n_rows;
+    int32_t first_block;       // workgroups from here on zero rows instead of walking tiles
+};
 template <typename T>
-__global__ void k_zero_uncovered(const int32_t* __restrict__ rows, int64_t n_rows, int HD, int H, T* __restrict__ a,
-                                 T* __restrict__ b, float* __restrict__ Z) {
-    const int64_t i = (int64_t)blockIdx.x * (blockDim.x / 8) + threadIdx.x / 8;
+__device__ __forceinline__ void zero_bare_rows(const BareRows& br, int HD, int H, T* __restrict__ a, T* __restrict__ b,
+                                               float* __restrict__ Z) {
+    const int per_block = blockDim.x / 8;
+    const int64_t i = (int64_t)(blockIdx.x - br.first_block) * per_block + threadIdx.x / 8;
     const int part = threadIdx.x % 8;
-    if (i >= n_rows) return;
-    const int64_t row = rows[i];
-    for (int e = part; e < HD; e += 8) {
-        if (a) a[row * HD + e] = T{};
-        if (b) b[row * HD + e] = T{};
+    if (i >= br.n_rows) return;
+    const int64_t row = br.rows[i];
+    const int bytes = HD * (int)sizeof(T);                 // a multiple of 16: HD is a multiple of 8
+    const uint4 z4 = make_uint4(0u, 0u, 0u, 0u);
+    for (int o = part * 16; o < bytes; o += 128) {
+        if (a) *reinterpret_cast<uint4*>(reinterpret_cast<char*>(a + row * HD) + o) = z4;
+        if (b) *reinterpret_cast<uint4*>(reinterpret_cast<char*>(b + row * HD) + o) = z4;
     }
     if (Z) for (int h = part; h < H; h += 8) Z[row * H + h] = 0.f;
 }
@@ -158,10 +167,15 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_fwd(const int
                                                               const T* __restrict__ V, float* __restrict__ acc,
                                                               float* __restrict__ Zp, T* __restrict__ out,
                                                               float* __restrict__ Zout,
-                                                              const int32_t* __restrict__ rem_rowptr, float inv_scale) {
+                                                              const int32_t* __restrict__ rem_rowptr, const BareRows bare,
+                                                              float inv_scale) {
     constexpr int HD = H * D;
     constexpr int kTileWaves = tile_waves<HD>();
     __shared__ short lds[kTileWaves * (rm_size<HD>() + tr_size<HD>())];
+    if (FINAL && (int)blockIdx.x >= bare.first_block) {      // uniform over the workgroup
+        zero_bare_rows<T>(bare, HD, H, out, (T*)nullptr, Zp);
+        return;
+    }
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int g = blockIdx.x * kTileWaves + wave;
     if (g >= n_groups) return;
@@ -229,11 +243,15 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_bwd_dst(const
                                                                   const float2* __restrict__ nd,
                                                                   float* __restrict__ dq_part, T* __restrict__ dq_out,
                                                                   const int32_t* __restrict__ rem_rowptr,
-                                                                  float inv_scale) {
+                                                                  const BareRows bare, float inv_scale) {
     constexpr int HD = H * D;
     constexpr int kTileWaves = tile_waves<HD>();
     constexpr int PER_WAVE = 2 * rm_size<HD>() + tr_size<HD>();
     __shared__ short lds[kTileWaves * PER_WAVE];
+    if (FINAL && (int)blockIdx.x >= bare.first_block) {
+        zero_bare_rows<T>(bare, HD, H, dq_out, (T*)nullptr, (float*)nullptr);
+        return;
+    }
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int g = blockIdx.x * kTileWaves + wave;
     if (g >= n_groups) return;
@@ -307,11 +325,16 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_bwd_src(const
                                                                   float* __restrict__ dk_part,
                                                                   float* __restrict__ dv_part, T* __restrict__ dk_out,
                                                                   T* __restrict__ dv_out,
-                                                                  const int32_t* __restrict__ rem_rowptr, float inv_scale) {
+                                                                  const int32_t* __restrict__ rem_rowptr, const BareRows bare,
+                                                                  float inv_scale) {
     constexpr int HD = H * D;
     constexpr int kTileWaves = tile_waves<HD>();
     constexpr int PER_WAVE = 2 * rm_size<HD>() + 2 * tr_size<HD>() + 4 * kTile * H;   // + nd tile (float2 = 4 shorts)
     __shared__ __align__(16) short lds[kTileWaves * PER_WAVE];
+    if (FINAL && (int)blockIdx.x >= bare.first_block) {
+        zero_bare_rows<T>(bare, HD, H, dk_out, dv_out, (float*)nullptr);
+        return;
+    }
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int g = blockIdx.x * kTileWaves + wave;
     if (g >= n_groups) return;
@@ -455,19 +478,21 @@ static int tile_fwd_launch_s(const tgt_tiles* tl, const void* q, const void* k, 
     constexpr int W = tile_waves<H * D>();
     const float inv_scale = 1.0f / sqrtf((float)D);
     KernelTimer t(KS_TILE_FWD, st);
-    const dim3 grid((tl->n_dst_groups + W - 1) / W), block(64 * W);
+    const int gblocks = (tl->n_dst_groups + W - 1) / W;
+    const dim3 grid(gblocks), block(64 * W);
+    const BareRows none{nullptr, 0, 0x7fffffff};
     if (final_out) {
-        if (tl->n_bare_dst > 0)
-            hipLaunchKernelGGL((k_zero_uncovered<T>), dim3((unsigned)((tl->n_bare_dst + 31) / 32)), dim3(256), 0, st,
-                               tl->bare_dst.as<int32_t>(), tl->n_bare_dst, H * D, H, (T*)final_out, (T*)nullptr, Zp);
-        if (tl->n_dst_groups > 0)
-            hipLaunchKernelGGL((k_tile_fwd<T, D, H, true>), grid, block, 0, st, tl->dst_c0.as<int32_t>(),
+        // the rows without tiles are zeroed by workgroups appended to the same launch
+        const int per = 64 * W / 8, zblocks = (int)((tl->n_bare_dst + per - 1) / per);
+        const BareRows bare{tl->bare_dst.as<int32_t>(), (int32_t)tl->n_bare_dst, gblocks};
+        if (gblocks + zblocks > 0)
+            hipLaunchKernelGGL((k_tile_fwd<T, D, H, true>), dim3(gblocks + zblocks), block, 0, st, tl->dst_c0.as<int32_t>(),
                                tl->dst_off.as<int32_t>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
-                               (const T*)k, (const T*)v, acc, Zp, (T*)final_out, Zp, (const int32_t*)nullptr, inv_scale);
+                               (const T*)k, (const T*)v, acc, Zp, (T*)final_out, Zp, (const int32_t*)nullptr, bare, inv_scale);
     } else if (tl->n_dst_groups > 0) {
         hipLaunchKernelGGL((k_tile_fwd<T, D, H, false>), grid, block, 0, st, tl->dst_c0.as<int32_t>(),
                            tl->dst_off.as<int32_t>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
-                           (const T*)k, (const T*)v, acc, Zp, (T*)out, Zout, rem_rowptr, inv_scale);
+                           (const T*)k, (const T*)v, acc, Zp, (T*)out, Zout, rem_rowptr, none, inv_scale);
     }
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
@@ -481,31 +506,33 @@ static int tile_bwd_launch_s(const tgt_tiles* tl, const void* q, const void* k, 
     constexpr int W = tile_waves<H * D>();
     const float inv_scale = 1.0f / sqrtf((float)D);
     KernelTimer t(KS_TILE_BWD, st);
-    const dim3 gd((tl->n_dst_groups + W - 1) / W), gs((tl->n_src_groups + W - 1) / W), block(64 * W);
+    const int gdb = (tl->n_dst_groups + W - 1) / W, gsb = (tl->n_src_groups + W - 1) / W;
+    const dim3 gd(gdb), gs(gsb), block(64 * W);
+    const BareRows none{nullptr, 0, 0x7fffffff};
     if (f_dq) {
-        if (tl->n_bare_dst > 0)
-            hipLaunchKernelGGL((k_zero_uncovered<T>), dim3((unsigned)((tl->n_bare_dst + 31) / 32)), dim3(256), 0, st,
-                               tl->bare_dst.as<int32_t>(), tl->n_bare_dst, H * D, H, (T*)f_dq, (T*)nullptr, (float*)nullptr);
-        if (tl->n_bare_src > 0)
-            hipLaunchKernelGGL((k_zero_uncovered<T>), dim3((unsigned)((tl->n_bare_src + 31) / 32)), dim3(256), 0, st,
-                               tl->bare_src.as<int32_t>(), tl->n_bare_src, H * D, H, (T*)f_dk, (T*)f_dv, (float*)nullptr);
-        if (tl->n_dst_groups > 0)
-            hipLaunchKernelGGL((k_tile_bwd_dst<T, D, H, true>), gd, block, 0, st, tl->dst_c0.as<int32_t>(),
+        const int per = 64 * W / 8;
+        const int zd = (int)((tl->n_bare_dst + per - 1) / per), zs = (int)((tl->n_bare_src + per - 1) / per);
+        const BareRows bare_d{tl->bare_dst.as<int32_t>(), (int32_t)tl->n_bare_dst, gdb};
+        const BareRows bare_s{tl->bare_src.as<int32_t>(), (int32_t)tl->n_bare_src, gsb};
+        if (gdb + zd > 0)
+            hipLaunchKernelGGL((k_tile_bwd_dst<T, D, H, true>), dim3(gdb + zd), block, 0, st, tl->dst_c0.as<int32_t>(),
                                tl->dst_off.as<int32_t>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
-                               (const T*)k, (const T*)v, (const T*)dout, nd, dq, (T*)f_dq, (const int32_t*)nullptr, inv_scale);
-        if (tl->n_src_groups > 0)
-            hipLaunchKernelGGL((k_tile_bwd_src<T, D, H, true>), gs, block, 0, st, tl->src_r0.as<int32_t>(),
+                               (const T*)k, (const T*)v, (const T*)dout, nd, dq, (T*)f_dq, (const int32_t*)nullptr, bare_d,
+                               inv_scale);
+        if (gsb + zs > 0)
+            hipLaunchKernelGGL((k_tile_bwd_src<T, D, H, true>), dim3(gsb + zs), block, 0, st, tl->src_r0.as<int32_t>(),
                                tl->src_off.as<int32_t>(), tl->src_c0.as<int32_t>(), tl->n_src_groups, (const T*)q,
-                               (const T*)k, (const T*)v, (const T*)dout, nd, dk, dv, (T*)f_dk, (T*)f_dv, (const int32_t*)nullptr, inv_scale);
+                               (const T*)k, (const T*)v, (const T*)dout, nd, dk, dv, (T*)f_dk, (T*)f_dv,
+                               (const int32_t*)nullptr, bare_s, inv_scale);
     } else {
         if (tl->n_dst_groups > 0)
             hipLaunchKernelGGL((k_tile_bwd_dst<T, D, H, false>), gd, block, 0, st, tl->dst_c0.as<int32_t>(),
                                tl->dst_off.as<int32_t>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
-                               (const T*)k, (const T*)v, (const T*)dout, nd, dq, (T*)o_dq, rem_dst, inv_scale);
+                               (const T*)k, (const T*)v, (const T*)dout, nd, dq, (T*)o_dq, rem_dst, none, inv_scale);
         if (tl->n_src_groups > 0)
             hipLaunchKernelGGL((k_tile_bwd_src<T, D, H, false>), gs, block, 0, st, tl->src_r0.as<int32_t>(),
                                tl->src_off.as<int32_t>(), tl->src_c0.as<int32_t>(), tl->n_src_groups, (const T*)q,
-                               (const T*)k, (const T*)v, (const T*)dout, nd, dk, dv, (T*)o_dk, (T*)o_dv, rem_src,
+                               (const T*)k, (const T*)v, (const T*)dout, nd, dk, dv, (T*)o_dk, (T*)o_dv, rem_src, none,
                                inv_scale);
     }
     TGT_HIP_CHECK(hipGetLastError());
