@@ -59,11 +59,15 @@ def kernel_alg_bytes(name, N, E, H, d, esize, bpe):
 # HBM-side bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each
 # scaled by the reading of a copy kernel of known size: FETCH x2.000, WRITE x1.000); the summary is
 # profiles/sparse_attn_config2_hbm_traffic_pmc.txt.  Counters cannot be read from inside this process,
-# so the figures are carried here and only reported for the workload / dtype they were measured on.
+# so the figures are carried here, reported only for the workload / dtype they were measured on, and the
+# bench line says when and on which commit of the kernels they were taken (a kernel change after that
+# commit makes them stale: measure again).
 MEASURED_TRAFFIC = {
-    ("config2", "f32"): {"attn_fwd": 242.6e6, "bwd_node_side": 38.9e6, "attn_bwd": 577.7e6},
-    ("config2", "bf16"): {"attn_fwd": 131.4e6, "bwd_node_side": 22.6e6, "attn_bwd": 324.0e6},
+    ("config2", "f32"): {"attn_fwd": 241.5e6, "bwd_node_side": 38.9e6, "attn_bwd": 570.6e6},
+    ("config2", "bf16"): {"attn_fwd": 130.5e6, "bwd_node_side": 22.6e6, "attn_bwd": 320.9e6},
 }
+MEASURED_TRAFFIC_AT = {"date": "2026-11-26", "kernels_as_of_commit": "a1e9bfa",
+                       "summary": "profiles/sparse_attn_config2_hbm_traffic_pmc.txt"}
 
 
 def build_workload(name):
@@ -605,6 +609,18 @@ def bench_model(args):
     torch.cuda.synchronize()
     fresh_ms = (time.perf_counter() - t0) / args.steps * 1e3
     fresh_builds = plan_mod.plan_cache_stats()["builds"] - builds_before
+    # what of that is the copy itself (the reference's loop pays it too) and what the look-up by content costs
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        fresh = ei_cpu.to(dev, non_blocking=True)
+        torch.cuda.synchronize()
+    copy_ms = (time.perf_counter() - t0) / args.steps * 1e3
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        fresh = ei_cpu.to(dev, non_blocking=True)
+        plan_mod.get_plan(fresh, n)
+        torch.cuda.synchronize()
+    lookup_ms = (time.perf_counter() - t0) / args.steps * 1e3 - copy_ms
     L = _lib.lib()
     L.tgt_timing_reset()
     L.tgt_timing_enable(1)
@@ -667,6 +683,8 @@ def bench_model(args):
         "loss": loss_value,
         "step_with_fresh_edge_index_ms": fresh_ms,
         "plans_built_by_the_fresh_edge_index_steps": fresh_builds,
+        "edge_index_host_to_device_copy_ms": copy_ms,
+        "plan_lookup_by_content_ms": lookup_ms,
         "ms_per_step_hip_graph": graph_ms,
         "library_kernel_us_per_step": lib_us,
         "kernel_groups_us": {g: sum(kernels[k]["avg_us"] * kernels[k]["launches_per_step"] for k in ks if k in kernels)
@@ -785,8 +803,6 @@ def bench_graph_model(args):
                    "parameters": sum(p.numel() for p in m.parameters()),
                    "step": "forward + l1_loss + backward + torch AdamW (" + ("foreach" if args.foreach_adamw else "fused") + ")", "parallelism": "1 GPU"},
         "loss": loss_value,
-        "step_with_fresh_edge_index_ms": fresh_ms,
-        "plans_built_by_the_fresh_edge_index_steps": fresh_builds,
         "ms_per_step_hip_graph": graph_ms,
         "library_kernel_us_per_step": lib_us,
         "kernel_groups_us": {g: sum(kernels[k]["avg_us"] * kernels[k]["launches_per_step"] for k in ks if k in kernels)
@@ -943,6 +959,7 @@ def bench_sparse(args):
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": dom_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": dom_gbs / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC.get((args.workload, args.dtype), {}).get(dom),
+                     "traffic_measured_at": MEASURED_TRAFFIC_AT if (args.workload, args.dtype) in MEASURED_TRAFFIC else None,
                      "alg_bytes": dom_bytes,
                      "avg_us": kernels[dom]["avg_us"]},
         "kernels": kernels,
@@ -1004,7 +1021,8 @@ def other_configs(args):
                  "kernels_avg_us": {kk: round(vv["avg_us"], 2) for kk, vv in r.get("kernels", {}).items()},
                  "seconds_spent": None}
         for extra in ("bias_in_plan_order", "mfma", "sparse_path_same_edges_ms", "ids_and_tables", "plan_build_ms",
-                      "step_with_fresh_edge_index_ms", "plans_built_by_the_fresh_edge_index_steps"):
+                      "step_with_fresh_edge_index_ms", "plans_built_by_the_fresh_edge_index_steps",
+                      "edge_index_host_to_device_copy_ms", "plan_lookup_by_content_ms"):
             if extra in r:
                 entry[extra] = r[extra]
         entry["seconds_spent"] = round(time.perf_counter() - t0, 1)
