@@ -504,7 +504,11 @@ __device__ __forceinline__ void thin_rows_bwd_k(const short* __restrict__ q_rm, 
                                                 const float* __restrict__ lse_l, const float* __restrict__ dd_l,
                                                 const BT* __restrict__ bias_gh, int bstride, T* __restrict__ dK, T* __restrict__ dV,
                                                 int g, int h, int S, int H, float scale, int first, int count, int lane,
-                                                const DropArgs da) {
+                                                const DropArgs da, float* __restrict__ dq_slab = nullptr,
+                                                T* __restrict__ dbias_gh = nullptr) {
+    // dq_slab (one-walk backward): this wave's share of dQ, [query][D] floats in LDS - the sums over these keys of
+    // dS k for the queries in front of `first` (the rows from `first` on get their dQ from thin_rows_bwd_q) - and
+    // dbias_gh: the keys' column of dBias for the same queries.
     constexpr int NC = (SP + 63) / 64;
     const float scale2 = scale * kLog2e;
     for (int tk = 0; tk < count; ++tk) {
@@ -530,6 +534,11 @@ __device__ __forceinline__ void thin_rows_bwd_k(const short* __restrict__ q_rm, 
                 for (int d = 0; d < D; ++d) {
                     dk[d] = fmaf(dsb, qv[d], dk[d]);
                     dv[d] = fmaf(pb, gv[d], dv[d]);
+                }
+                if (dq_slab != nullptr && qq < first) {       // the same lane owns query qq for every key
+#pragma unroll
+                    for (int d = 0; d < D; ++d) dq_slab[qq * D + d] = (tk == 0 ? 0.f : dq_slab[qq * D + d]) + dsb * kv[d];
+                    if (dbias_gh != nullptr) st1(dbias_gh + (int64_t)qq * S + ki, dS);
                 }
             }
         }
@@ -1204,6 +1213,315 @@ static int device_cus() {
     }
     return cus;
 }
+// ---------------------------------------------------------------------------
+// Backward in one walk (bias tensor or no bias).  The kernel above forms every score tile twice: once with a lane
+// per query (dQ, dBias) and once with a lane per key (dK, dV).  Here wave w owns key tile w only and walks the query
+// tiles once.  dS of a tile leaves the lane-per-key registers through a wave-private LDS tile [query][key] (bf16):
+// read back with a lane per query it is the B operand of dQ^T += K^T dS^T and the 32-byte pieces of the dBias rows.
+// A wave's dQ covers its own 32 keys; it goes to the wave's slab in LDS and the workgroup adds the slabs in wave
+// order at the end (fixed order: reproducible).  Per tile that is 16 + 8 LDS accesses and four matrix instructions
+// more, two matrix instructions, sixteen exponentials and the whole second pass over the bias less.
+// ---------------------------------------------------------------------------
+// The bias of one query tile as the lane-per-key walk needs it: 16 queries x this lane's key, one element each from 16
+// rows.  2-byte elements sit two to a register, so that the elements of three tiles can be in flight (the walk is
+// bound by the latency of these loads: 2 KB per wave and tile).
+typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+template <typename T> struct ColRegs;
+template <> struct ColRegs<dbf16> {
+    static constexpr int kDepth = 3;
+    u16x2_t v[8];
+    __device__ __forceinline__ void set(int r, const dbf16* p) { if (r & 1) v[r >> 1].y = p->x; else v[r >> 1].x = p->x; }
+    __device__ __forceinline__ float get(int r) const { return __uint_as_float(((uint32_t)((r & 1) ? v[r >> 1].y : v[r >> 1].x)) << 16); }
+};
+template <> struct ColRegs<float> {
+    static constexpr int kDepth = 2;
+    float v[16];
+    __device__ __forceinline__ void set(int r, const float* p) { v[r] = *p; }
+    __device__ __forceinline__ float get(int r) const { return v[r]; }
+};
+// rows past the end repeat the last one (a valid address; their scores are masked)
+template <typename T>
+__device__ __forceinline__ void load_col(const T* __restrict__ bcol, int qt, int half, int S, ColRegs<T>& c) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int qq = min(qt * 32 + 8 * (r / 4) + 4 * half + (r % 4), S - 1);
+        c.set(r, bcol + (int64_t)qq * S);
+    }
+}
+template <typename T>
+__device__ __forceinline__ void zero_col(ColRegs<T>& c) {
+    if constexpr (sizeof(T) == 2) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { c.v[i].x = 0; c.v[i].y = 0; }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) c.v[i] = 0.f;
+    }
+}
+
+constexpr int kTqPitch = 36;      // shorts per query row of the dS tile (8-byte reads two to a bank at worst)
+// slab_rows: the queries whose dQ the waves share out (all of them, or those in front of a thin last tile)
+template <int D, int NT> constexpr int bwd1_lds_bytes(int slab_rows = NT * 32) {
+    return bwd_lds_bytes<D, NT>() + NT * 32 * kTqPitch * 2 + NT * slab_rows * D * 4;
+}
+// the one-walk kernel is used where two workgroups still fit a CU's LDS
+template <int D, int NT> constexpr bool bwd1_fits() { return bwd1_lds_bytes<D, NT>() <= 72 * 1024; }
+
+template <typename T, int D, int NT, bool DROP>
+__global__ __launch_bounds__(64 * NT, D == 8 ? 4 : 3) void k_dense_bwd1(const T* __restrict__ Q, const T* __restrict__ K,
+                                                        const T* __restrict__ V, const T* __restrict__ bias,
+                                                        const T* __restrict__ O, const float* __restrict__ lse,
+                                                        const T* __restrict__ dO, T* __restrict__ dQ,
+                                                        T* __restrict__ dK, T* __restrict__ dV,
+                                                        T* __restrict__ dbias, int S, int H, float scale, int nb,
+                                                        const DropArgs da) {
+    constexpr int KS = D / 8;
+    constexpr int SP = NT * 32;
+    extern __shared__ __align__(16) char smem[];
+    constexpr int RM = rm_elems<D, SP>(), TR = tr_elems<D, SP>();
+    short* q_rm = reinterpret_cast<short*>(smem);
+    short* k_rm = q_rm + RM;
+    short* v_rm = k_rm + RM;
+    short* g_rm = v_rm + RM;          // g = dout
+    short* q_tr = g_rm + RM;
+    short* k_tr = q_tr + TR;
+    short* g_tr = k_tr + TR;
+    float* lse_l = reinterpret_cast<float*>(g_tr + TR);   // lse * log2(e)
+    float* dd_l = lse_l + SP;
+    short* tq_all = reinterpret_cast<short*>(dd_l + SP);  // [NT][32][kTqPitch]
+    float* slab_all = reinterpret_cast<float*>(tq_all + NT * 32 * kTqPitch);   // [NT][slab_rows][D]
+    const int pair = blockIdx.x;
+    const int win = pair / (8 * H), rem = pair % (8 * H);
+    const int g = win * 8 + (rem & 7), h = rem >> 3;
+    if (g >= nb) return;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int col = lane & 31, half = lane >> 5;
+    const bool hasb = bias != nullptr;
+    const int tail = S - (NT - 1) * 32;          // rows / keys in the last tile
+    const bool thin = tail <= 4;
+    const int nt_full = thin ? NT - 1 : NT;      // tiles that take the matrix path
+    const T* bias_gh = hasb ? bias + ((int64_t)g * H + h) * S * S : nullptr;
+    T* dbias_gh = dbias != nullptr ? dbias + ((int64_t)g * H + h) * S * S : nullptr;
+    const bool vec_wave = thin && wave == NT - 1;
+    short* tq = tq_all + wave * 32 * kTqPitch;
+    const int slab_rows = thin ? (NT - 1) * 32 : SP;
+    float* slab = slab_all + wave * slab_rows * D;
+    // this lane's key and the first slice of its bias column, requested before anything else
+    const int k0 = wave * 32, ki = k0 + col;
+    const bool kok = ki < S;
+    const T* bcol = hasb ? bias_gh + (kok ? ki : 0) : nullptr;
+    constexpr int kDepth = ColRegs<T>::kDepth;       // tiles whose bias is in flight or in use
+    ColRegs<T> b0, b1, b2;                            // of query tiles qt, qt + 1, qt + 2
+    zero_col(b0); zero_col(b1); zero_col(b2);
+    const bool bload = hasb && kok && !vec_wave;
+    if (bload) {
+        load_col(bcol, 0, half, S, b0);
+        if (NT > 1) load_col(bcol, 1, half, S, b1);
+    }
+    load_head<T, D, SP>(Q, g, h, S, H, q_rm, q_tr);
+    load_head<T, D, SP>(K, g, h, S, H, k_rm, k_tr);
+    load_head<T, D, SP>(V, g, h, S, H, v_rm, nullptr);
+    load_head<T, D, SP>(dO, g, h, S, H, g_rm, g_tr);
+    for (int i = threadIdx.x; i < SP; i += blockDim.x) {
+        float dsum = 0.f, L = 0.f;
+        if (i < S) {
+            L = lse[((int64_t)g * H + h) * S + i];
+            const T* op = O + (((int64_t)g * S + i) * H + h) * D;
+            const T* gp = dO + (((int64_t)g * S + i) * H + h) * D;
+#pragma unroll
+            for (int c = 0; c < D; c += 4) {
+                const short4_t ov = ld4(op + c);
+                const short4_t gv = ld4(gp + c);
+                dsum += bf2f(ov.x) * bf2f(gv.x) + bf2f(ov.y) * bf2f(gv.y) + bf2f(ov.z) * bf2f(gv.z) +
+                        bf2f(ov.w) * bf2f(gv.w);
+            }
+        }
+        lse_l[i] = L * kLog2e;
+        dd_l[i] = dsum;          // D[q] = sum_dd dout[q,dd] out[q,dd]
+    }
+    __syncthreads();
+
+    if (vec_wave) {
+        // the one to four rows of the last tile: as queries (dQ and dBias of those rows), then as keys (dK, dV, their
+        // column of dBias and their share of everybody's dQ)
+        thin_rows_bwd_q<T, T, D, SP, DROP>(q_rm, k_rm, v_rm, g_rm, lse_l, dd_l, bias_gh, S, dbias_gh, dQ, g, h, S, H, scale,
+                                           (NT - 1) * 32, tail, lane, da, IdsAcc{});
+        thin_rows_bwd_k<T, T, D, SP, DROP>(q_rm, k_rm, v_rm, g_rm, lse_l, dd_l, bias_gh, S, dK, dV, g, h, S, H, scale,
+                                           (NT - 1) * 32, tail, lane, da, slab, dbias_gh);
+    } else {
+        short4_t bk[KS], bv[KS];
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            bk[s] = *reinterpret_cast<const short4_t*>(&k_rm[ki * D + s * 8 + half * 4]);
+            bv[s] = *reinterpret_cast<const short4_t*>(&v_rm[ki * D + s * 8 + half * 4]);
+        }
+        const float scale2 = scale * kLog2e;
+        float16_t dk = zero16(), dv = zero16();
+#pragma unroll 1
+        for (int qt = 0; qt < nt_full; ++qt) {
+            if (bload) {      // the tile that will be needed kDepth - 1 tiles from now
+                if (kDepth == 3 && qt + 2 < NT) load_col(bcol, qt + 2, half, S, b2);
+                if (kDepth == 2 && qt + 1 < NT) load_col(bcol, qt + 1, half, S, b1);
+            }
+            float16_t sc = zero16(), dp = zero16();
+#pragma unroll
+            for (int s = 0; s < KS; ++s) {
+                const short4_t aq = *reinterpret_cast<const short4_t*>(&q_rm[(qt * 32 + col) * D + s * 8 + half * 4]);
+                const short4_t ag = *reinterpret_cast<const short4_t*>(&g_rm[(qt * 32 + col) * D + s * 8 + half * 4]);
+                sc = mfma(aq, bk[s], sc);     // S[query, key]
+                dp = mfma(ag, bv[s], dp);     // dP[query, key] = dout V^T
+            }
+            const bool full = qt * 32 + 32 <= S;
+            float pr[16];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int qb = qt * 32 + 8 * j + 4 * half;          // four consecutive queries
+                const float4_t L4 = *reinterpret_cast<const float4_t*>(&lse_l[qb]);
+                const float4_t D4 = *reinterpret_cast<const float4_t*>(&dd_l[qb]);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const int r = 4 * j + t;
+                    pr[r] = fast_exp2(fmaf(sc[r], scale2, fmaf(b0.get(r), kLog2e, -L4[t])));
+                    float ks = 1.0f;
+                    if (DROP) ks = drop_keep(da, drop_row_hash(da, g * H + h, qb + t), ki) ? da.inv_keep : 0.f;
+                    sc[r] = pr[r] * (dp[r] * ks - D4[t]);
+                    if (DROP) pr[r] *= ks;
+                }
+            }
+            if (!full || !kok) {                  // queries past the end of the batch entry (wave-uniform) or a key past it
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const bool in = kok && qt * 32 + 8 * (r / 4) + 4 * half + (r % 4) < S;
+                    pr[r] = in ? pr[r] : 0.f;
+                    sc[r] = in ? sc[r] : 0.f;
+                }
+            }
+            // dS of the tile, rounded to bf16 once: into the wave's LDS tile [query][key] ...
+            short dsb[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                dsb[r] = f2bf(sc[r]);
+                tq[(8 * (r / 4) + 4 * half + (r % 4)) * kTqPitch + col] = dsb[r];
+            }
+            // ... and, as it is, the B operand of dK^T += Q^T dS (P likewise for dV^T += dout^T P)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                short4_t db, pb;
+                db.x = dsb[4 * t + 0]; db.y = dsb[4 * t + 1]; db.z = dsb[4 * t + 2]; db.w = dsb[4 * t + 3];
+                pb.x = f2bf(pr[4 * t + 0]); pb.y = f2bf(pr[4 * t + 1]);
+                pb.z = f2bf(pr[4 * t + 2]); pb.w = f2bf(pr[4 * t + 3]);
+                short4_t aq = zero4(), ag = zero4();
+                if (col < D) {
+                    aq = *reinterpret_cast<const short4_t*>(&q_tr[col * (SP + 4) + qt * 32 + t * 8 + half * 4]);
+                    ag = *reinterpret_cast<const short4_t*>(&g_tr[col * (SP + 4) + qt * 32 + t * 8 + half * 4]);
+                }
+                dk = mfma(aq, db, dk);        // dK^T[dd, key] += Q^T dS
+                dv = mfma(ag, pb, dv);        // dV^T[dd, key] += dout^T P
+            }
+            // the tile read back with a lane per query: the writes are the wave's own and the LDS serves a wave's
+            // accesses in the order they were issued, so only the compiler has to be kept from reordering them
+            asm volatile("" ::: "memory");
+            const int qi = qt * 32 + col;
+            float16_t dq = zero16();
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const short4_t dsT = *reinterpret_cast<const short4_t*>(&tq[col * kTqPitch + 8 * t + 4 * half]);
+                short4_t ak = zero4();
+                if (col < D) ak = *reinterpret_cast<const short4_t*>(&k_tr[col * (SP + 4) + k0 + 8 * t + 4 * half]);
+                dq = mfma(ak, dsT, dq);       // dQ^T[dd, query] += K^T dS^T over this wave's keys
+            }
+            if (dbias_gh != nullptr && qi < S) {          // 16 keys of the query's dBias row: 32 / 64 contiguous bytes
+                const int kb = k0 + 16 * half;
+                short4_t piece[4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) piece[t] = *reinterpret_cast<const short4_t*>(&tq[col * kTqPitch + 16 * half + 4 * t]);
+                T* dbrow = dbias_gh + (int64_t)qi * S;
+                if (kb + 16 <= S && sizeof(T) == 2) {
+                    __builtin_memcpy(dbrow + kb, piece, 32);
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        if (kb + 4 * t + 0 < S) st1(dbrow + kb + 4 * t + 0, bf2f(piece[t].x));
+                        if (kb + 4 * t + 1 < S) st1(dbrow + kb + 4 * t + 1, bf2f(piece[t].y));
+                        if (kb + 4 * t + 2 < S) st1(dbrow + kb + 4 * t + 2, bf2f(piece[t].z));
+                        if (kb + 4 * t + 3 < S) st1(dbrow + kb + 4 * t + 3, bf2f(piece[t].w));
+                    }
+                }
+            }
+            // this wave's share of dQ of the 32 queries: rows dd = 8 rb + 4 half .. + 3 of the accumulator
+#pragma unroll
+            for (int rb = 0; rb < KS; ++rb) {
+                float4_t o;
+                o[0] = dq[4 * rb + 0]; o[1] = dq[4 * rb + 1]; o[2] = dq[4 * rb + 2]; o[3] = dq[4 * rb + 3];
+                *reinterpret_cast<float4_t*>(&slab[qi * D + 8 * rb + 4 * half]) = o;
+            }
+            asm volatile("" ::: "memory");      // the tile is read before the next one is written (issue order)
+            b0 = b1;
+            if (kDepth == 3) b1 = b2;
+        }
+        if (thin) {
+            constexpr int qt = NT - 1;
+            float16_t sc = zero16(), dp = zero16();
+#pragma unroll
+            for (int s = 0; s < KS; ++s) {
+                const short4_t aq = *reinterpret_cast<const short4_t*>(&q_rm[(qt * 32 + col) * D + s * 8 + half * 4]);
+                const short4_t ag = *reinterpret_cast<const short4_t*>(&g_rm[(qt * 32 + col) * D + s * 8 + half * 4]);
+                sc = mfma(aq, bk[s], sc);
+                dp = mfma(ag, bv[s], dp);
+            }
+            // at most four queries in the last tile: registers 0..3 of the lower half; their dQ and dBias rows are
+            // the vector wave's
+            const int qb = qt * 32 + 4 * half;
+            const float4_t L4 = *reinterpret_cast<const float4_t*>(&lse_l[qb]);
+            const float4_t D4 = *reinterpret_cast<const float4_t*>(&dd_l[qb]);
+            float p4[4], s4[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const bool in = half == 0 && t < tail;
+                const float pv = fast_exp2(fmaf(sc[t], scale2, fmaf(b0.get(t), kLog2e, -L4[t])));
+                float ks = 1.0f;
+                if (DROP) ks = drop_keep(da, drop_row_hash(da, g * H + h, qb + t), ki) ? da.inv_keep : 0.f;
+                p4[t] = in ? pv * ks : 0.f;
+                s4[t] = in ? pv * (dp[t] * ks - D4[t]) : 0.f;
+            }
+            short4_t db, pb;
+            db.x = f2bf(s4[0]); db.y = f2bf(s4[1]); db.z = f2bf(s4[2]); db.w = f2bf(s4[3]);
+            pb.x = f2bf(p4[0]); pb.y = f2bf(p4[1]); pb.z = f2bf(p4[2]); pb.w = f2bf(p4[3]);
+            short4_t aq = zero4(), ag = zero4();
+            if (col < D) {
+                aq = *reinterpret_cast<const short4_t*>(&q_tr[col * (SP + 4) + qt * 32 + half * 4]);
+                ag = *reinterpret_cast<const short4_t*>(&g_tr[col * (SP + 4) + qt * 32 + half * 4]);
+            }
+            dk = mfma(aq, db, dk);
+            dv = mfma(ag, pb, dv);
+        }
+        if (kok) {
+            T* pk = dK + (((int64_t)g * S + ki) * H + h) * D;
+            T* pv = dV + (((int64_t)g * S + ki) * H + h) * D;
+#pragma unroll
+            for (int rb = 0; rb < KS; ++rb) {
+                st4(pk + 8 * rb + 4 * half, dk[4 * rb + 0] * scale, dk[4 * rb + 1] * scale, dk[4 * rb + 2] * scale,
+                    dk[4 * rb + 3] * scale);
+                st4(pv + 8 * rb + 4 * half, dv[4 * rb + 0], dv[4 * rb + 1], dv[4 * rb + 2], dv[4 * rb + 3]);
+            }
+        }
+    }
+    __syncthreads();
+    // dQ = scale * (the waves' shares, in wave order); the rows of a thin last tile were written by their wave
+    const int q_end = thin ? (NT - 1) * 32 : S;
+    for (int c = threadIdx.x; c < q_end * (D / 4); c += blockDim.x) {
+        const int row = c / (D / 4), part = c % (D / 4);
+        float4_t a = *reinterpret_cast<const float4_t*>(&slab_all[row * D + part * 4]);
+#pragma unroll
+        for (int w = 1; w < NT; ++w) {
+            const float4_t b = *reinterpret_cast<const float4_t*>(&slab_all[(w * slab_rows + row) * D + part * 4]);
+            a[0] += b[0]; a[1] += b[1]; a[2] += b[2]; a[3] += b[3];
+        }
+        st4(dQ + (((int64_t)g * S + row) * H + h) * D + part * 4, a[0] * scale, a[1] * scale, a[2] * scale, a[3] * scale);
+    }
+}
+
 // Workgroups of the id form's backward: what the GPU keeps resident at two per CU, a multiple of 8 H so that a
 // workgroup stays with one head, at most one per pair.  It also sizes the workspace of table partials.
 static int ids_bwd_grid(int b, int H) {
@@ -1230,6 +1548,7 @@ static int launch_dense(const DenseCall& c, bool bwd) {
         }
         const float scale = sqrtf((float)c.d);     // the reference MULTIPLIES q by sqrt(d)
         const dim3 block(64 * NT);
+        const bool thin = c.S - (NT - 1) * 32 <= 4;      // a last tile of at most four rows
         static bool attr_done = false;     // raise the dynamic-LDS cap once per instantiation
         if (!attr_done) {
             const int cap_f = BSRC == 1 ? kLdsLimit : lds_f0, cap_b = BSRC == 1 ? kLdsLimit : lds_b0;
@@ -1265,6 +1584,27 @@ static int launch_dense(const DenseCall& c, bool bwd) {
             else
                 hipLaunchKernelGGL((k_dense_fwd<T, D, NT, false, BSRC>), grid, block, lds_f, c.st, (const T*)c.q, (const T*)c.k,
                                    (const T*)c.v, (const T*)c.bias, (T*)c.o_out, c.o_lse, c.S, c.H, scale, c.b, da, c.ids);
+        } else if constexpr (BSRC == 0 && bwd1_fits<D, NT>()) {
+            // bias tensor (or none) and a shape whose dQ shares fit the LDS: every score tile is formed once
+            constexpr int lds1_max = bwd1_lds_bytes<D, NT>();
+            const int lds1 = bwd1_lds_bytes<D, NT>(thin ? (NT - 1) * 32 : NT * 32);
+            static bool attr1_done = false;
+            if (!attr1_done) {
+                TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_dense_bwd1<T, D, NT, false>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds1_max));
+                TGT_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&k_dense_bwd1<T, D, NT, true>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds1_max));
+                attr1_done = true;
+            }
+            KernelTimer t(KS_DENSE_BWD, c.st);
+            if (drop)
+                hipLaunchKernelGGL((k_dense_bwd1<T, D, NT, true>), grid, block, lds1, c.st, (const T*)c.q, (const T*)c.k,
+                                   (const T*)c.v, (const T*)c.bias, (const T*)c.out, c.lse, (const T*)c.dout,
+                                   (T*)c.dq, (T*)c.dk, (T*)c.dv, (T*)c.dbias, c.S, c.H, scale, c.b, da);
+            else
+                hipLaunchKernelGGL((k_dense_bwd1<T, D, NT, false>), grid, block, lds1, c.st, (const T*)c.q, (const T*)c.k,
+                                   (const T*)c.v, (const T*)c.bias, (const T*)c.out, c.lse, (const T*)c.dout,
+                                   (T*)c.dq, (T*)c.dk, (T*)c.dv, (T*)c.dbias, c.S, c.H, scale, c.b, da);
         } else {
             KernelTimer t(KS_DENSE_BWD, c.st);
             if (drop)
