@@ -160,8 +160,7 @@ __device__ __forceinline__ void wave_lds_fence() {
 // the output rows and Z themselves; otherwise it does so for the destinations that have no remaining edge and
 // leaves fp32 sums of the others for the sparse kernel to add (which skips the former).
 template <typename T, int D, int H, bool FINAL>
-__global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_fwd(const int32_t* __restrict__ grp_c0,
-                                                              const int32_t* __restrict__ grp_off,
+__global__ __launch_bounds__(64 * tile_waves<H * D>(), 4) void k_tile_fwd(const int4* __restrict__ grp_rec,
                                                               const int32_t* __restrict__ tile_r0, int n_groups,
                                                               const T* __restrict__ Q, const T* __restrict__ K,
                                                               const T* __restrict__ V, float* __restrict__ acc,
@@ -183,7 +182,10 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_fwd(const int
     short* v_tr = k_rm + rm_size<HD>();
     const int col = lane & 15, kq = lane >> 4;
     const bool kval = kq * 4 < D;
-    const int c0 = grp_c0[g], t0 = grp_off[g], t1 = grp_off[g + 1];
+    // one 16-byte record per group: (first node, tile range, the first tile's other side) - a wave with one tile, the
+    // usual case, needs no second look-up before it can ask for the tile's rows
+    const int4 gr = grp_rec[g];
+    const int c0 = gr.x, t0 = gr.y, t1 = gr.z;
     bshort4 bq[H];
 #pragma unroll
     for (int h = 0; h < H; ++h) {
@@ -195,7 +197,7 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_fwd(const int
 #pragma unroll
     for (int h = 0; h < H; ++h) { o[h] = t_zerof(); z[h] = 0.f; }
     for (int t = t0; t < t1; ++t) {
-        const int r0 = tile_r0[t];
+        const int r0 = t == t0 ? gr.w : tile_r0[t];
         wave_lds_fence();                      // the previous tile's reads are done
         stage_rows<T, HD>(K, r0, k_rm, nullptr, lane);
         stage_rows<T, HD>(V, r0, nullptr, v_tr, lane);
@@ -235,8 +237,7 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_fwd(const int
 
 // Same grouping: dQ of the tiles.  nd[i,h] = (1/(Z+eps), dout.out) of the FINAL output.
 template <typename T, int D, int H, bool FINAL>
-__global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_bwd_dst(const int32_t* __restrict__ grp_c0,
-                                                                  const int32_t* __restrict__ grp_off,
+__global__ __launch_bounds__(64 * tile_waves<H * D>(), 3) void k_tile_bwd_dst(const int4* __restrict__ grp_rec,
                                                                   const int32_t* __restrict__ tile_r0, int n_groups,
                                                                   const T* __restrict__ Q, const T* __restrict__ K,
                                                                   const T* __restrict__ V, const T* __restrict__ dO,
@@ -260,7 +261,10 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_bwd_dst(const
     short* k_tr = v_rm + rm_size<HD>();
     const int col = lane & 15, kq = lane >> 4;
     const bool kval = kq * 4 < D;
-    const int c0 = grp_c0[g], t0 = grp_off[g], t1 = grp_off[g + 1];
+    // one 16-byte record per group: (first node, tile range, the first tile's other side) - a wave with one tile, the
+    // usual case, needs no second look-up before it can ask for the tile's rows
+    const int4 gr = grp_rec[g];
+    const int c0 = gr.x, t0 = gr.y, t1 = gr.z;
     bshort4 bq[H], bg[H];
     float2 ndv[H];
     bfloat4 dq[H];
@@ -275,7 +279,7 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_bwd_dst(const
         dq[h] = t_zerof();
     }
     for (int t = t0; t < t1; ++t) {
-        const int r0 = tile_r0[t];
+        const int r0 = t == t0 ? gr.w : tile_r0[t];
         wave_lds_fence();
         stage_rows<T, HD>(K, r0, k_rm, k_tr, lane);
         stage_rows<T, HD>(V, r0, v_rm, nullptr, lane);
@@ -316,8 +320,7 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_bwd_dst(const
 
 // One wave per group of tiles that share their 16 SOURCES: dK and dV of the tiles.
 template <typename T, int D, int H, bool FINAL>
-__global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_bwd_src(const int32_t* __restrict__ grp_r0,
-                                                                  const int32_t* __restrict__ grp_off,
+__global__ __launch_bounds__(64 * tile_waves<H * D>(), 3) void k_tile_bwd_src(const int4* __restrict__ grp_rec,
                                                                   const int32_t* __restrict__ tile_c0, int n_groups,
                                                                   const T* __restrict__ Q, const T* __restrict__ K,
                                                                   const T* __restrict__ V, const T* __restrict__ dO,
@@ -345,7 +348,8 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_bwd_src(const
     float2* nd_l = reinterpret_cast<float2*>(g_tr + tr_size<HD>());     // [16 destinations][H]
     const int col = lane & 15, kq = lane >> 4;
     const bool kval = kq * 4 < D;
-    const int r0 = grp_r0[g], t0 = grp_off[g], t1 = grp_off[g + 1];
+    const int4 gr = grp_rec[g];
+    const int r0 = gr.x, t0 = gr.y, t1 = gr.z;
     bshort4 bk[H], bv[H];
     bfloat4 dk[H], dv[H];
 #pragma unroll
@@ -358,7 +362,7 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>()) void k_tile_bwd_src(const
         dk[h] = t_zerof(); dv[h] = t_zerof();
     }
     for (int t = t0; t < t1; ++t) {
-        const int c0 = tile_c0[t];
+        const int c0 = t == t0 ? gr.w : tile_c0[t];
         wave_lds_fence();
         stage_rows<T, HD>(Q, c0, q_rm, q_tr, lane);
         stage_rows<T, HD>(dO, c0, g_rm, g_tr, lane);
@@ -416,6 +420,7 @@ struct tgt_tiles {
     int64_t N = 0, T = 0;
     int32_t n_dst_groups = 0, n_src_groups = 0;
     tgt::DevBuf dst_c0, dst_off, dst_r0;     // [G], [G+1], [T]
+    tgt::DevBuf dst_rec, src_rec;            // [G] / [Gs] int4 (group's first node, off[g], off[g + 1], first tile's other side)
     tgt::DevBuf src_r0, src_off, src_c0;     // [Gs], [Gs+1], [T]
     tgt::DevBuf cover_dst, cover_src;        // [N] bytes
     tgt::DevBuf bare_dst, bare_src;          // the rows cover_* marks 0
@@ -486,12 +491,10 @@ static int tile_fwd_launch_s(const tgt_tiles* tl, const void* q, const void* k, 
         const int per = 64 * W / 8, zblocks = (int)((tl->n_bare_dst + per - 1) / per);
         const BareRows bare{tl->bare_dst.as<int32_t>(), (int32_t)tl->n_bare_dst, gblocks};
         if (gblocks + zblocks > 0)
-            hipLaunchKernelGGL((k_tile_fwd<T, D, H, true>), dim3(gblocks + zblocks), block, 0, st, tl->dst_c0.as<int32_t>(),
-                               tl->dst_off.as<int32_t>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
+            hipLaunchKernelGGL((k_tile_fwd<T, D, H, true>), dim3(gblocks + zblocks), block, 0, st, tl->dst_rec.as<int4>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
                                (const T*)k, (const T*)v, acc, Zp, (T*)final_out, Zp, (const int32_t*)nullptr, bare, inv_scale);
     } else if (tl->n_dst_groups > 0) {
-        hipLaunchKernelGGL((k_tile_fwd<T, D, H, false>), grid, block, 0, st, tl->dst_c0.as<int32_t>(),
-                           tl->dst_off.as<int32_t>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
+        hipLaunchKernelGGL((k_tile_fwd<T, D, H, false>), grid, block, 0, st, tl->dst_rec.as<int4>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
                            (const T*)k, (const T*)v, acc, Zp, (T*)out, Zout, rem_rowptr, none, inv_scale);
     }
     TGT_HIP_CHECK(hipGetLastError());
@@ -515,23 +518,19 @@ static int tile_bwd_launch_s(const tgt_tiles* tl, const void* q, const void* k, 
         const BareRows bare_d{tl->bare_dst.as<int32_t>(), (int32_t)tl->n_bare_dst, gdb};
         const BareRows bare_s{tl->bare_src.as<int32_t>(), (int32_t)tl->n_bare_src, gsb};
         if (gdb + zd > 0)
-            hipLaunchKernelGGL((k_tile_bwd_dst<T, D, H, true>), dim3(gdb + zd), block, 0, st, tl->dst_c0.as<int32_t>(),
-                               tl->dst_off.as<int32_t>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
+            hipLaunchKernelGGL((k_tile_bwd_dst<T, D, H, true>), dim3(gdb + zd), block, 0, st, tl->dst_rec.as<int4>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
                                (const T*)k, (const T*)v, (const T*)dout, nd, dq, (T*)f_dq, (const int32_t*)nullptr, bare_d,
                                inv_scale);
         if (gsb + zs > 0)
-            hipLaunchKernelGGL((k_tile_bwd_src<T, D, H, true>), dim3(gsb + zs), block, 0, st, tl->src_r0.as<int32_t>(),
-                               tl->src_off.as<int32_t>(), tl->src_c0.as<int32_t>(), tl->n_src_groups, (const T*)q,
+            hipLaunchKernelGGL((k_tile_bwd_src<T, D, H, true>), dim3(gsb + zs), block, 0, st, tl->src_rec.as<int4>(), tl->src_c0.as<int32_t>(), tl->n_src_groups, (const T*)q,
                                (const T*)k, (const T*)v, (const T*)dout, nd, dk, dv, (T*)f_dk, (T*)f_dv,
                                (const int32_t*)nullptr, bare_s, inv_scale);
     } else {
         if (tl->n_dst_groups > 0)
-            hipLaunchKernelGGL((k_tile_bwd_dst<T, D, H, false>), gd, block, 0, st, tl->dst_c0.as<int32_t>(),
-                               tl->dst_off.as<int32_t>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
+            hipLaunchKernelGGL((k_tile_bwd_dst<T, D, H, false>), gd, block, 0, st, tl->dst_rec.as<int4>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
                                (const T*)k, (const T*)v, (const T*)dout, nd, dq, (T*)o_dq, rem_dst, none, inv_scale);
         if (tl->n_src_groups > 0)
-            hipLaunchKernelGGL((k_tile_bwd_src<T, D, H, false>), gs, block, 0, st, tl->src_r0.as<int32_t>(),
-                               tl->src_off.as<int32_t>(), tl->src_c0.as<int32_t>(), tl->n_src_groups, (const T*)q,
+            hipLaunchKernelGGL((k_tile_bwd_src<T, D, H, false>), gs, block, 0, st, tl->src_rec.as<int4>(), tl->src_c0.as<int32_t>(), tl->n_src_groups, (const T*)q,
                                (const T*)k, (const T*)v, (const T*)dout, nd, dk, dv, (T*)o_dk, (T*)o_dv, rem_src, none,
                                inv_scale);
     }
@@ -623,6 +622,13 @@ int tgt_tiles_create(const int32_t* h_tiles, int64_t T, int block_size, int64_t 
     if (!rc) rc = tgt::upload(tl->src_r0, ks, st);
     if (!rc) rc = tgt::upload(tl->src_off, os, st);
     if (!rc) rc = tgt::upload(tl->src_c0, xs, st);
+    {
+        std::vector<int4> rd(kd.size()), rs(ks.size());
+        for (size_t g = 0; g < kd.size(); ++g) rd[g] = make_int4(kd[g], od[g], od[g + 1], xd[od[g]]);
+        for (size_t g = 0; g < ks.size(); ++g) rs[g] = make_int4(ks[g], os[g], os[g + 1], xs[os[g]]);
+        if (!rc && !rd.empty()) rc = tgt::upload(tl->dst_rec, rd, st);
+        if (!rc && !rs.empty()) rc = tgt::upload(tl->src_rec, rs, st);
+    }
     if (!rc) rc = tgt::upload(tl->cover_dst, cd, st);
     if (!rc) rc = tgt::upload(tl->cover_src, cs, st);
     std::vector<int32_t> bd, bs;

@@ -555,7 +555,7 @@ __device__ __forceinline__ void thin_rows_bwd_k(const short* __restrict__ q_rm, 
 // forward: online softmax over key tiles, in the base-2 domain
 // ---------------------------------------------------------------------------
 template <typename T, int D, int NT, bool DROP, int BSRC>
-__global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, const T* __restrict__ K,
+__global__ __launch_bounds__(64 * NT, 2) void k_dense_fwd(const T* __restrict__ Q, const T* __restrict__ K,
                                                        const T* __restrict__ V, const T* __restrict__ bias,
                                                        T* __restrict__ out, float* __restrict__ lse, int S,
                                                        int H, float scale, int nb, const DropArgs da, const IdsArgs ia) {
@@ -750,7 +750,7 @@ __global__ __launch_bounds__(64 * NT) void k_dense_fwd(const T* __restrict__ Q, 
 // in the first, 32 lanes on 32 consecutive keys of one row in the second); the second
 // read of a (graph, head) slice comes from L2.
 template <typename T, int D, int NT, bool DROP, int BSRC>
-__global__ __launch_bounds__(64 * NT) void k_dense_bwd(const T* __restrict__ Q, const T* __restrict__ K,
+__global__ __launch_bounds__(64 * NT, 2) void k_dense_bwd(const T* __restrict__ Q, const T* __restrict__ K,
                                                        const T* __restrict__ V, const T* __restrict__ bias,
                                                        const T* __restrict__ O, const float* __restrict__ lse,
                                                        const T* __restrict__ dO, T* __restrict__ dQ,
