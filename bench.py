@@ -413,7 +413,7 @@ def bench_block(args):
     reorder_ms = (time.perf_counter() - t0) * 1e3
     E = int(new_e.shape[1])
     ts = TileSet(tiles, n, dev)
-    plan_rest = GraphPlan(raw, n)
+    plan_rest = GraphPlan(raw, n, rows_with_edges_only=True)
     plan_full = GraphPlan(new_e, n)
     g = torch.Generator().manual_seed(42)
     q, k, v, dout = (torch.randn(n, H, d, generator=g).to(dev, tdt) for _ in range(4))

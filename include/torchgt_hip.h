@@ -100,6 +100,14 @@ const char*  tgt_last_error(void);
 int tgt_plan_create(const int64_t* d_src, const int64_t* d_dst, int64_t E, int64_t N,
                     void* stream, tgt_plan_t** out_plan);
 int tgt_plan_destroy(tgt_plan_t* plan);
+/* The same for the edges that remain beside a tile set (tgt_block_attn_*; the reference's reordering
+ * leaves them as the tail of its edge list, gt_sp/utils.py:284-299): the schedules hold only the rows
+ * that have edges, the tile kernels write the others (most rows, when the tiles hold most edges: the
+ * sparse kernels then start a fraction of the waves).  Accepted by tgt_block_attn_* and every tgt_plan_*
+ * call; tgt_sparse_attn_* refuse such a plan with TGT_ERR_INVALID_ARG, since on their own they would
+ * leave the rows without edges unwritten. */
+int tgt_plan_create_remaining(const int64_t* d_src, const int64_t* d_dst, int64_t E, int64_t N,
+                              void* stream, tgt_plan_t** out_plan);
 /* A 128-bit content key of an edge list (values and their positions), for caches of plans that must
  * recognise an edge_index they have seen at another address: the reference's training loops move the
  * same CPU-resident edge_index to the GPU in every iteration (main_sp_sparse_node_level.py:178-183,

@@ -10,7 +10,7 @@ import torch
 
 from oracle import graph_prep as ogp
 from oracle import sparse_attention as osa
-from torchgt_amd import _lib, block_attention, expand_tiles, graph_prep, sparse_attention, workloads
+from torchgt_amd import GraphPlan, _lib, block_attention, expand_tiles, graph_prep, sparse_attention, workloads
 
 pytestmark = pytest.mark.gpu
 TOL = 2e-2
@@ -143,6 +143,35 @@ def test_config5_hybrid_full_size(cuda):
     assert n == 262144 and 0.03 < raw.shape[1] / e.shape[1] < 0.07
     assert expanded.shape[1] == 256 * tiles.shape[0] + raw.shape[1]
     run_case("config5-hybrid", n, tiles, torch.from_numpy(raw), 8, 8, torch.bfloat16, "edge_head", 10, cuda)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_plan_of_the_remaining_edges_schedules_only_rows_with_edges(cuda, dtype):
+    # few remaining edges: most rows have none - some under tiles (finished by the tile kernels), some under
+    # nothing (zeros from the tile launches), a few with edges only (sparse kernels), a few with both
+    rng = np.random.default_rng(5)
+    N = 1000
+    tiles = _random_tiles(rng, 640, 50)                      # nodes 640.. have no tiles
+    rest = torch.from_numpy(np.concatenate([rng.integers(0, N, (2, 150)), rng.integers(700, 720, (2, 60))], 1))
+    run_case("few remaining edges", N, tiles, rest, 8, 8, dtype, "edge_head", 11, cuda)
+    run_case("few remaining edges, no tiles", N, np.zeros((0, 2), np.int32), rest, 8, 8, dtype, "edge", 12, cuda)
+    # the same numbers whichever kind of plan holds the remaining edges
+    g = torch.Generator().manual_seed(13)
+    q, k, v, dout = (torch.randn(N, 8, 8, generator=g).to(cuda, dtype) for _ in range(4))
+    bias = (torch.randn(rest.shape[1], 8, generator=g) * 0.5).to(cuda, dtype)
+    res = []
+    for only in (False, True):
+        plan = GraphPlan(rest.to(cuda), N, rows_with_edges_only=only)
+        tc = [x.clone().requires_grad_(True) for x in (q, k, v, bias)]
+        o = block_attention(tc[0], tc[1], tc[2], tiles, edge_bias=tc[3], plan=plan)
+        res.append([o] + list(torch.autograd.grad(o, tc, dout)))
+        info = plan.info()
+        assert info["items_dst"] == (len(np.unique(rest[1].numpy())) if only else N)
+    for a, b in zip(*res):
+        assert torch.equal(a, b)
+    # on their own the sparse kernels would leave the other rows unwritten: refused
+    with pytest.raises(RuntimeError, match="tgt_block_attn"):
+        sparse_attention(q, k, v, rest.to(cuda), plan=plan)
 
 
 def test_block_loud_failures(cuda):

@@ -27,6 +27,7 @@ SIGNATURES = {
     "tgt_error_string": (_c.c_char_p, [_i32]),
     "tgt_last_error": (_c.c_char_p, []),
     "tgt_plan_create": (_i32, [_vp, _vp, _i64, _i64, _vp, _c.POINTER(_vp)]),
+    "tgt_plan_create_remaining": (_i32, [_vp, _vp, _i64, _i64, _vp, _c.POINTER(_vp)]),
     "tgt_plan_destroy": (_i32, [_vp]),
     "tgt_set_allocator": (_i32, [_vp, _vp, _vp]),
     "tgt_edge_index_hash": (_i32, [_vp, _vp, _i64, _vp, _c.POINTER(_c.c_uint64)]),

@@ -131,7 +131,7 @@ def block_attention(q, k, v, tiles, edge_index=None, edge_bias=None, plan=None):
     if plan is None:
         if edge_index is None:
             edge_index = torch.zeros((2, 0), dtype=torch.int64, device=q.device)
-        plan = GraphPlan(edge_index, N)
+        plan = GraphPlan(edge_index, N, rows_with_edges_only=True)
     if edge_bias is not None:
         edge_bias = edge_bias.to(q3.dtype)
     return BlockAttentionFunction.apply(q3, k3, v3, edge_bias, tiles, plan)

@@ -65,9 +65,10 @@ __device__ __forceinline__ void t_st4(tbf16* p, float a, float b, float c, float
     *reinterpret_cast<bshort4*>(p) = r;
 }
 
-// Rows no tile covers get zeros when the tile kernels write final results (no remaining edges).  The rows are
-// listed when the tile set is built; the workgroups behind the last tile group of a launch write them (eight
-// lanes per row, 16-byte stores), so they cost no launch of their own.
+// Rows no tile covers get zeros when the tile kernels write final results (no remaining edges, or a plan of the
+// remaining edges that schedules only rows with edges: then the rows without, rem_rowptr[row + 1] ==
+// rem_rowptr[row]).  The rows are listed when the tile set is built; the workgroups behind the last tile group of
+// a launch write them (eight lanes per row, 16-byte stores), so they cost no launch of their own.
 struct BareRows {
     const int32_t* rows;
     int32_t n_rows;
@@ -75,12 +76,13 @@ struct BareRows {
 };
 template <typename T>
 __device__ __forceinline__ void zero_bare_rows(const BareRows& br, int HD, int H, T* __restrict__ a, T* __restrict__ b,
-                                               float* __restrict__ Z) {
+                                               float* __restrict__ Z, const int32_t* __restrict__ rem_rowptr) {
     const int per_block = blockDim.x / 8;
     const int64_t i = (int64_t)(blockIdx.x - br.first_block) * per_block + threadIdx.x / 8;
     const int part = threadIdx.x % 8;
     if (i >= br.n_rows) return;
     const int64_t row = br.rows[i];
+    if (rem_rowptr && rem_rowptr[row + 1] != rem_rowptr[row]) return;      // the sparse kernels write this row
     const int bytes = HD * (int)sizeof(T);                 // a multiple of 16: HD is a multiple of 8
     const uint4 z4 = make_uint4(0u, 0u, 0u, 0u);
     for (int o = part * 16; o < bytes; o += 128) {
@@ -99,31 +101,48 @@ template <int HD> constexpr int tile_waves() { return HD > 64 ? 2 : 4; }
 template <int HD> constexpr int rm_size() { return kTile * (HD + 4); }
 template <int HD> constexpr int tr_size() { return HD * 20; }
 
-// Coalesced copy of rows row0 .. row0+15 of X ([N, HD]) into the LDS images (either may be null):
-// every lane fetches 16-byte pieces of consecutive memory.
+// Coalesced copy of rows row0 .. row0+15 of X ([N, HD]) into the LDS images (either may be null): every lane
+// fetches 16-byte pieces of consecutive memory.  Loading and storing are separate steps so that a kernel can ask
+// for the rows of all its tensors before it waits for the first of them.
+// a piece in registers: eight bf16 values (float inputs are rounded as they arrive)
+template <typename T, int HD> struct RowPieces {
+    static constexpr int CPR = HD / 8;                      // 8-element pieces per row
+    static constexpr int ITERS = (kTile * CPR + 63) / 64;
+    uint4 p[ITERS];
+};
+__device__ __forceinline__ uint32_t pack2(short lo, short hi) { return (uint32_t)(uint16_t)lo | ((uint32_t)(uint16_t)hi << 16); }
+__device__ __forceinline__ void load_piece(const tbf16* p, uint4& r) { r = *reinterpret_cast<const uint4*>(p); }
+__device__ __forceinline__ void load_piece(const float* p, uint4& r) {
+    const bfloat4 a = *reinterpret_cast<const bfloat4*>(p);
+    const bfloat4 b = *reinterpret_cast<const bfloat4*>(p + 4);
+    r.x = pack2(t_f2bf(a.x), t_f2bf(a.y)); r.y = pack2(t_f2bf(a.z), t_f2bf(a.w));
+    r.z = pack2(t_f2bf(b.x), t_f2bf(b.y)); r.w = pack2(t_f2bf(b.z), t_f2bf(b.w));
+}
+__device__ __forceinline__ void unpack_piece(const uint4& u, short (&v)[8]) {
+    v[0] = (short)(u.x & 0xffffu); v[1] = (short)(u.x >> 16);
+    v[2] = (short)(u.y & 0xffffu); v[3] = (short)(u.y >> 16);
+    v[4] = (short)(u.z & 0xffffu); v[5] = (short)(u.z >> 16);
+    v[6] = (short)(u.w & 0xffffu); v[7] = (short)(u.w >> 16);
+}
 template <typename T, int HD>
-__device__ __forceinline__ void stage_rows(const T* __restrict__ X, int row0, short* __restrict__ rm,
-                                           short* __restrict__ tr, int lane) {
-    constexpr int CPR = HD / 8;                     // 8-element pieces per row
+__device__ __forceinline__ void load_rows(const T* __restrict__ X, int row0, int lane, RowPieces<T, HD>& rp) {
+    constexpr int CPR = RowPieces<T, HD>::CPR;
 #pragma unroll
-    for (int i = 0; i < (kTile * CPR + 63) / 64; ++i) {
+    for (int i = 0; i < RowPieces<T, HD>::ITERS; ++i) {
+        const int c = i * 64 + lane;
+        if (kTile * CPR % 64 == 0 || c < kTile * CPR) load_piece(X + (int64_t)row0 * HD + c * 8, rp.p[i]);   // rows are contiguous
+    }
+}
+template <typename T, int HD>
+__device__ __forceinline__ void store_rows(const RowPieces<T, HD>& rp, short* __restrict__ rm, short* __restrict__ tr, int lane) {
+    constexpr int CPR = RowPieces<T, HD>::CPR;
+#pragma unroll
+    for (int i = 0; i < RowPieces<T, HD>::ITERS; ++i) {
         const int c = i * 64 + lane;
         if (kTile * CPR % 64 != 0 && c >= kTile * CPR) break;
         const int row = c / CPR, e0 = (c % CPR) * 8;
-        const T* p = X + (int64_t)(row0 + row) * HD + e0;
         short v[8];
-        if (sizeof(T) == 2) {
-            const uint4 u = *reinterpret_cast<const uint4*>(p);
-            v[0] = (short)(u.x & 0xffffu); v[1] = (short)(u.x >> 16);
-            v[2] = (short)(u.y & 0xffffu); v[3] = (short)(u.y >> 16);
-            v[4] = (short)(u.z & 0xffffu); v[5] = (short)(u.z >> 16);
-            v[6] = (short)(u.w & 0xffffu); v[7] = (short)(u.w >> 16);
-        } else {
-            const bfloat4 f0 = *reinterpret_cast<const bfloat4*>(p);
-            const bfloat4 f1 = *reinterpret_cast<const bfloat4*>(reinterpret_cast<const float*>(p) + 4);
-            v[0] = t_f2bf(f0.x); v[1] = t_f2bf(f0.y); v[2] = t_f2bf(f0.z); v[3] = t_f2bf(f0.w);
-            v[4] = t_f2bf(f1.x); v[5] = t_f2bf(f1.y); v[6] = t_f2bf(f1.z); v[7] = t_f2bf(f1.w);
-        }
+        unpack_piece(rp.p[i], v);
         if (rm) {
             bshort4 lo, hi;
             lo.x = v[0]; lo.y = v[1]; lo.z = v[2]; lo.w = v[3];
@@ -137,6 +156,12 @@ __device__ __forceinline__ void stage_rows(const T* __restrict__ X, int row0, sh
         }
     }
 }
+// Whether the next tile's rows are asked for while the current one is worked on: where the pieces in flight fit the
+// registers next to the accumulators (2-byte elements, up to 64 per row)
+template <typename T, int HD> constexpr bool tile_prefetch() { return sizeof(T) == 2 && HD <= 64; }
+// the first lane's value as a scalar: what every lane of a wave holds alike (a group's record) steers loops and
+// addresses from scalar registers
+__device__ __forceinline__ int wave_uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
 // A operand "rows x 4 consecutive elements": lane (col, kq) reads row `col`, elements e .. e+3
 template <int HD>
 __device__ __forceinline__ bshort4 a_rows(const short* __restrict__ rm, int col, int e) {
@@ -170,9 +195,10 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 4) void k_tile_fwd(const 
                                                               float inv_scale) {
     constexpr int HD = H * D;
     constexpr int kTileWaves = tile_waves<HD>();
+    constexpr bool kPrefetch = tile_prefetch<T, HD>();
     __shared__ short lds[kTileWaves * (rm_size<HD>() + tr_size<HD>())];
-    if (FINAL && (int)blockIdx.x >= bare.first_block) {      // uniform over the workgroup
-        zero_bare_rows<T>(bare, HD, H, out, (T*)nullptr, Zp);
+    if ((int)blockIdx.x >= bare.first_block) {      // uniform over the workgroup
+        zero_bare_rows<T>(bare, HD, H, out, (T*)nullptr, Zout, rem_rowptr);
         return;
     }
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -185,23 +211,39 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 4) void k_tile_fwd(const 
     // one 16-byte record per group: (first node, tile range, the first tile's other side) - a wave with one tile, the
     // usual case, needs no second look-up before it can ask for the tile's rows
     const int4 gr = grp_rec[g];
-    const int c0 = gr.x, t0 = gr.y, t1 = gr.z;
+    const int c0 = wave_uniform(gr.x), t0 = wave_uniform(gr.y), t1 = wave_uniform(gr.z);
+    int r0 = wave_uniform(gr.w);
+    RowPieces<T, HD> pk, pv;
+    load_rows<T, HD>(K, r0, lane, pk);         // asked for before anything waits
+    load_rows<T, HD>(V, r0, lane, pv);
     bshort4 bq[H];
 #pragma unroll
     for (int h = 0; h < H; ++h) {
         bq[h] = t_zero4();
         if (kval) bq[h] = t_ld4(Q + (int64_t)(c0 + col) * HD + h * D + kq * 4);
     }
+    // a destination without remaining edges (row pointers of the plan that holds them) is finished here as well
+    bool fin = true;
+    if (!FINAL) fin = rem_rowptr[c0 + col + 1] == rem_rowptr[c0 + col];
     bfloat4 o[H];
     float z[H];
 #pragma unroll
     for (int h = 0; h < H; ++h) { o[h] = t_zerof(); z[h] = 0.f; }
     for (int t = t0; t < t1; ++t) {
-        const int r0 = t == t0 ? gr.w : tile_r0[t];
+        if (!kPrefetch && t > t0) {
+            r0 = wave_uniform(tile_r0[t]);
+            load_rows<T, HD>(K, r0, lane, pk);
+            load_rows<T, HD>(V, r0, lane, pv);
+        }
         wave_lds_fence();                      // the previous tile's reads are done
-        stage_rows<T, HD>(K, r0, k_rm, nullptr, lane);
-        stage_rows<T, HD>(V, r0, nullptr, v_tr, lane);
+        store_rows<T, HD>(pk, k_rm, nullptr, lane);
+        store_rows<T, HD>(pv, nullptr, v_tr, lane);
         wave_lds_fence();
+        if (kPrefetch && t + 1 < t1) {         // the next tile's rows travel while this one is worked on
+            r0 = wave_uniform(tile_r0[t + 1]);
+            load_rows<T, HD>(K, r0, lane, pk);
+            load_rows<T, HD>(V, r0, lane, pv);
+        }
 #pragma unroll
         for (int h = 0; h < H; ++h) {
             bshort4 ak = t_zero4();
@@ -218,8 +260,6 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 4) void k_tile_fwd(const 
             o[h] = mfma16(av, t_pack(w), o[h]);                    // O^T[dd 4kq+r][destination col]
         }
     }
-    // a destination without remaining edges (row pointers of the plan that holds them) is finished here as well
-    const bool fin = FINAL || rem_rowptr[c0 + col + 1] == rem_rowptr[c0 + col];
 #pragma unroll
     for (int h = 0; h < H; ++h) {
         float zz = z[h];
@@ -247,10 +287,11 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 3) void k_tile_bwd_dst(co
                                                                   const BareRows bare, float inv_scale) {
     constexpr int HD = H * D;
     constexpr int kTileWaves = tile_waves<HD>();
+    constexpr bool kPrefetch = tile_prefetch<T, HD>();
     constexpr int PER_WAVE = 2 * rm_size<HD>() + tr_size<HD>();
     __shared__ short lds[kTileWaves * PER_WAVE];
-    if (FINAL && (int)blockIdx.x >= bare.first_block) {
-        zero_bare_rows<T>(bare, HD, H, dq_out, (T*)nullptr, (float*)nullptr);
+    if ((int)blockIdx.x >= bare.first_block) {
+        zero_bare_rows<T>(bare, HD, H, dq_out, (T*)nullptr, (float*)nullptr, rem_rowptr);
         return;
     }
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -264,7 +305,13 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 3) void k_tile_bwd_dst(co
     // one 16-byte record per group: (first node, tile range, the first tile's other side) - a wave with one tile, the
     // usual case, needs no second look-up before it can ask for the tile's rows
     const int4 gr = grp_rec[g];
-    const int c0 = gr.x, t0 = gr.y, t1 = gr.z;
+    const int c0 = wave_uniform(gr.x), t0 = wave_uniform(gr.y), t1 = wave_uniform(gr.z);
+    int r0 = wave_uniform(gr.w);
+    RowPieces<T, HD> pk, pv;
+    load_rows<T, HD>(K, r0, lane, pk);
+    load_rows<T, HD>(V, r0, lane, pv);
+    bool fin = true;                            // no remaining edge into this row
+    if (!FINAL) fin = rem_rowptr[c0 + col + 1] == rem_rowptr[c0 + col];
     bshort4 bq[H], bg[H];
     float2 ndv[H];
     bfloat4 dq[H];
@@ -279,11 +326,20 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 3) void k_tile_bwd_dst(co
         dq[h] = t_zerof();
     }
     for (int t = t0; t < t1; ++t) {
-        const int r0 = t == t0 ? gr.w : tile_r0[t];
+        if (!kPrefetch && t > t0) {
+            r0 = wave_uniform(tile_r0[t]);
+            load_rows<T, HD>(K, r0, lane, pk);
+            load_rows<T, HD>(V, r0, lane, pv);
+        }
         wave_lds_fence();
-        stage_rows<T, HD>(K, r0, k_rm, k_tr, lane);
-        stage_rows<T, HD>(V, r0, v_rm, nullptr, lane);
+        store_rows<T, HD>(pk, k_rm, k_tr, lane);
+        store_rows<T, HD>(pv, v_rm, nullptr, lane);
         wave_lds_fence();
+        if (kPrefetch && t + 1 < t1) {
+            r0 = wave_uniform(tile_r0[t + 1]);
+            load_rows<T, HD>(K, r0, lane, pk);
+            load_rows<T, HD>(V, r0, lane, pv);
+        }
 #pragma unroll
         for (int h = 0; h < H; ++h) {
             bshort4 ak = t_zero4(), av = t_zero4();
@@ -307,7 +363,6 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 3) void k_tile_bwd_dst(co
         }
     }
     if (kval) {
-        const bool fin = FINAL || rem_rowptr[c0 + col + 1] == rem_rowptr[c0 + col];      // no remaining edge into this row
 #pragma unroll
         for (int h = 0; h < H; ++h) {
             bfloat4 o;
@@ -332,10 +387,11 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 3) void k_tile_bwd_src(co
                                                                   float inv_scale) {
     constexpr int HD = H * D;
     constexpr int kTileWaves = tile_waves<HD>();
+    constexpr bool kPrefetch = tile_prefetch<T, HD>();
     constexpr int PER_WAVE = 2 * rm_size<HD>() + 2 * tr_size<HD>() + 4 * kTile * H;   // + nd tile (float2 = 4 shorts)
     __shared__ __align__(16) short lds[kTileWaves * PER_WAVE];
-    if (FINAL && (int)blockIdx.x >= bare.first_block) {
-        zero_bare_rows<T>(bare, HD, H, dk_out, dv_out, (float*)nullptr);
+    if ((int)blockIdx.x >= bare.first_block) {
+        zero_bare_rows<T>(bare, HD, H, dk_out, dv_out, (float*)nullptr, rem_rowptr);
         return;
     }
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -349,7 +405,18 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 3) void k_tile_bwd_src(co
     const int col = lane & 15, kq = lane >> 4;
     const bool kval = kq * 4 < D;
     const int4 gr = grp_rec[g];
-    const int r0 = gr.x, t0 = gr.y, t1 = gr.z;
+    const int r0 = wave_uniform(gr.x), t0 = wave_uniform(gr.y), t1 = wave_uniform(gr.z);
+    int c0 = wave_uniform(gr.w);
+    RowPieces<T, HD> pq, pg;
+    load_rows<T, HD>(Q, c0, lane, pq);
+    load_rows<T, HD>(dO, c0, lane, pg);
+    constexpr int ND_ITERS = (kTile * H + 63) / 64;
+    float2 ndr[ND_ITERS];
+#pragma unroll
+    for (int i = 0; i < ND_ITERS; ++i)
+        if (kTile * H % 64 == 0 || i * 64 + lane < kTile * H) ndr[i] = nd[(int64_t)c0 * H + i * 64 + lane];   // rows c0..c0+15 are contiguous
+    bool fin = true;                            // no remaining edge out of this row
+    if (!FINAL) fin = rem_rowptr[r0 + col + 1] == rem_rowptr[r0 + col];
     bshort4 bk[H], bv[H];
     bfloat4 dk[H], dv[H];
 #pragma unroll
@@ -362,12 +429,29 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 3) void k_tile_bwd_src(co
         dk[h] = t_zerof(); dv[h] = t_zerof();
     }
     for (int t = t0; t < t1; ++t) {
-        const int c0 = t == t0 ? gr.w : tile_c0[t];
+        if (!kPrefetch && t > t0) {
+            c0 = wave_uniform(tile_c0[t]);
+            load_rows<T, HD>(Q, c0, lane, pq);
+            load_rows<T, HD>(dO, c0, lane, pg);
+#pragma unroll
+            for (int i = 0; i < ND_ITERS; ++i)
+                if (kTile * H % 64 == 0 || i * 64 + lane < kTile * H) ndr[i] = nd[(int64_t)c0 * H + i * 64 + lane];
+        }
         wave_lds_fence();
-        stage_rows<T, HD>(Q, c0, q_rm, q_tr, lane);
-        stage_rows<T, HD>(dO, c0, g_rm, g_tr, lane);
-        for (int i = lane; i < kTile * H; i += 64) nd_l[i] = nd[(int64_t)c0 * H + i];   // rows c0..c0+15 are contiguous
+        store_rows<T, HD>(pq, q_rm, q_tr, lane);
+        store_rows<T, HD>(pg, g_rm, g_tr, lane);
+#pragma unroll
+        for (int i = 0; i < ND_ITERS; ++i)
+            if (kTile * H % 64 == 0 || i * 64 + lane < kTile * H) nd_l[i * 64 + lane] = ndr[i];
         wave_lds_fence();
+        if (kPrefetch && t + 1 < t1) {
+            c0 = wave_uniform(tile_c0[t + 1]);
+            load_rows<T, HD>(Q, c0, lane, pq);
+            load_rows<T, HD>(dO, c0, lane, pg);
+#pragma unroll
+            for (int i = 0; i < ND_ITERS; ++i)
+                if (kTile * H % 64 == 0 || i * 64 + lane < kTile * H) ndr[i] = nd[(int64_t)c0 * H + i * 64 + lane];
+        }
 #pragma unroll
         for (int h = 0; h < H; ++h) {
             bshort4 aq = t_zero4(), ag = t_zero4();
@@ -397,7 +481,6 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 3) void k_tile_bwd_src(co
         }
     }
     if (kval) {
-        const bool fin = FINAL || rem_rowptr[r0 + col + 1] == rem_rowptr[r0 + col];      // no remaining edge out of this row
 #pragma unroll
         for (int h = 0; h < H; ++h) {
             bfloat4 o;
@@ -479,23 +562,23 @@ static int upload(DevBuf& b, const std::vector<X>& v, hipStream_t st) {
 // rows without tiles) and the sparse kernels are not run.
 template <typename T, int D, int H>
 static int tile_fwd_launch_s(const tgt_tiles* tl, const void* q, const void* k, const void* v, float* acc, float* Zp,
-                             void* final_out, void* out, float* Zout, const int32_t* rem_rowptr, hipStream_t st) {
+                             void* final_out, void* out, float* Zout, const int32_t* rem_rowptr, bool zero_rows, hipStream_t st) {
     constexpr int W = tile_waves<H * D>();
     const float inv_scale = 1.0f / sqrtf((float)D);
     KernelTimer t(KS_TILE_FWD, st);
     const int gblocks = (tl->n_dst_groups + W - 1) / W;
-    const dim3 grid(gblocks), block(64 * W);
-    const BareRows none{nullptr, 0, 0x7fffffff};
+    const dim3 block(64 * W);
+    // the rows without tiles are zeroed by workgroups appended to the same launch: all of them when the tiles are all
+    // there is, else (zero_rows: the plan of the remaining edges schedules only rows with edges) those without edges
+    const int per = 64 * W / 8, zblocks = final_out || zero_rows ? (int)((tl->n_bare_dst + per - 1) / per) : 0;
+    const BareRows bare{tl->bare_dst.as<int32_t>(), (int32_t)tl->n_bare_dst, zblocks ? gblocks : 0x7fffffff};
+    if (gblocks + zblocks == 0) return TGT_OK;
     if (final_out) {
-        // the rows without tiles are zeroed by workgroups appended to the same launch
-        const int per = 64 * W / 8, zblocks = (int)((tl->n_bare_dst + per - 1) / per);
-        const BareRows bare{tl->bare_dst.as<int32_t>(), (int32_t)tl->n_bare_dst, gblocks};
-        if (gblocks + zblocks > 0)
-            hipLaunchKernelGGL((k_tile_fwd<T, D, H, true>), dim3(gblocks + zblocks), block, 0, st, tl->dst_rec.as<int4>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
-                               (const T*)k, (const T*)v, acc, Zp, (T*)final_out, Zp, (const int32_t*)nullptr, bare, inv_scale);
-    } else if (tl->n_dst_groups > 0) {
-        hipLaunchKernelGGL((k_tile_fwd<T, D, H, false>), grid, block, 0, st, tl->dst_rec.as<int4>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
-                           (const T*)k, (const T*)v, acc, Zp, (T*)out, Zout, rem_rowptr, none, inv_scale);
+        hipLaunchKernelGGL((k_tile_fwd<T, D, H, true>), dim3(gblocks + zblocks), block, 0, st, tl->dst_rec.as<int4>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
+                           (const T*)k, (const T*)v, acc, Zp, (T*)final_out, Zp, (const int32_t*)nullptr, bare, inv_scale);
+    } else {
+        hipLaunchKernelGGL((k_tile_fwd<T, D, H, false>), dim3(gblocks + zblocks), block, 0, st, tl->dst_rec.as<int4>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
+                           (const T*)k, (const T*)v, acc, Zp, (T*)out, Zout, rem_rowptr, bare, inv_scale);
     }
     TGT_HIP_CHECK(hipGetLastError());
     return TGT_OK;
@@ -505,18 +588,18 @@ template <typename T, int D, int H>
 static int tile_bwd_launch_s(const tgt_tiles* tl, const void* q, const void* k, const void* v, const void* dout,
                              const float2* nd, float* dq, float* dk, float* dv, void* f_dq, void* f_dk, void* f_dv,
                              void* o_dq, void* o_dk, void* o_dv, const int32_t* rem_dst, const int32_t* rem_src,
-                             hipStream_t st) {
+                             bool zero_rows, hipStream_t st) {
     constexpr int W = tile_waves<H * D>();
     const float inv_scale = 1.0f / sqrtf((float)D);
     KernelTimer t(KS_TILE_BWD, st);
     const int gdb = (tl->n_dst_groups + W - 1) / W, gsb = (tl->n_src_groups + W - 1) / W;
-    const dim3 gd(gdb), gs(gsb), block(64 * W);
-    const BareRows none{nullptr, 0, 0x7fffffff};
+    const dim3 block(64 * W);
+    const bool zr = f_dq || zero_rows;
+    const int per = 64 * W / 8;
+    const int zd = zr ? (int)((tl->n_bare_dst + per - 1) / per) : 0, zs = zr ? (int)((tl->n_bare_src + per - 1) / per) : 0;
+    const BareRows bare_d{tl->bare_dst.as<int32_t>(), (int32_t)tl->n_bare_dst, zd ? gdb : 0x7fffffff};
+    const BareRows bare_s{tl->bare_src.as<int32_t>(), (int32_t)tl->n_bare_src, zs ? gsb : 0x7fffffff};
     if (f_dq) {
-        const int per = 64 * W / 8;
-        const int zd = (int)((tl->n_bare_dst + per - 1) / per), zs = (int)((tl->n_bare_src + per - 1) / per);
-        const BareRows bare_d{tl->bare_dst.as<int32_t>(), (int32_t)tl->n_bare_dst, gdb};
-        const BareRows bare_s{tl->bare_src.as<int32_t>(), (int32_t)tl->n_bare_src, gsb};
         if (gdb + zd > 0)
             hipLaunchKernelGGL((k_tile_bwd_dst<T, D, H, true>), dim3(gdb + zd), block, 0, st, tl->dst_rec.as<int4>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
                                (const T*)k, (const T*)v, (const T*)dout, nd, dq, (T*)f_dq, (const int32_t*)nullptr, bare_d,
@@ -526,12 +609,12 @@ static int tile_bwd_launch_s(const tgt_tiles* tl, const void* q, const void* k, 
                                (const T*)k, (const T*)v, (const T*)dout, nd, dk, dv, (T*)f_dk, (T*)f_dv,
                                (const int32_t*)nullptr, bare_s, inv_scale);
     } else {
-        if (tl->n_dst_groups > 0)
-            hipLaunchKernelGGL((k_tile_bwd_dst<T, D, H, false>), gd, block, 0, st, tl->dst_rec.as<int4>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
-                               (const T*)k, (const T*)v, (const T*)dout, nd, dq, (T*)o_dq, rem_dst, none, inv_scale);
-        if (tl->n_src_groups > 0)
-            hipLaunchKernelGGL((k_tile_bwd_src<T, D, H, false>), gs, block, 0, st, tl->src_rec.as<int4>(), tl->src_c0.as<int32_t>(), tl->n_src_groups, (const T*)q,
-                               (const T*)k, (const T*)v, (const T*)dout, nd, dk, dv, (T*)o_dk, (T*)o_dv, rem_src, none,
+        if (gdb + zd > 0)
+            hipLaunchKernelGGL((k_tile_bwd_dst<T, D, H, false>), dim3(gdb + zd), block, 0, st, tl->dst_rec.as<int4>(), tl->dst_r0.as<int32_t>(), tl->n_dst_groups, (const T*)q,
+                               (const T*)k, (const T*)v, (const T*)dout, nd, dq, (T*)o_dq, rem_dst, bare_d, inv_scale);
+        if (gsb + zs > 0)
+            hipLaunchKernelGGL((k_tile_bwd_src<T, D, H, false>), dim3(gsb + zs), block, 0, st, tl->src_rec.as<int4>(), tl->src_c0.as<int32_t>(), tl->n_src_groups, (const T*)q,
+                               (const T*)k, (const T*)v, (const T*)dout, nd, dk, dv, (T*)o_dk, (T*)o_dv, rem_src, bare_s,
                                inv_scale);
     }
     TGT_HIP_CHECK(hipGetLastError());
@@ -543,9 +626,10 @@ static int tile_bwd_launch_s(const tgt_tiles* tl, const void* q, const void* k, 
 
 template <typename T>
 static int tile_fwd_launch(const tgt_tiles* tl, const void* q, const void* k, const void* v, float* acc, float* Zp,
-                           void* final_out, void* out, float* Zout, const int32_t* rem_rowptr, int H, int d, hipStream_t st) {
+                           void* final_out, void* out, float* Zout, const int32_t* rem_rowptr, bool zero_rows, int H, int d,
+                           hipStream_t st) {
 #define X(D_, H_) \
-    if (d == D_ && H == H_) return tile_fwd_launch_s<T, D_, H_>(tl, q, k, v, acc, Zp, final_out, out, Zout, rem_rowptr, st);
+    if (d == D_ && H == H_) return tile_fwd_launch_s<T, D_, H_>(tl, q, k, v, acc, Zp, final_out, out, Zout, rem_rowptr, zero_rows, st);
     TGT_TILE_SHAPES(X)
 #undef X
     set_error("block attention: no tile kernel for H=%d, d=%d", H, d);
@@ -555,12 +639,12 @@ static int tile_fwd_launch(const tgt_tiles* tl, const void* q, const void* k, co
 template <typename T>
 static int tile_bwd_launch(const tgt_tiles* tl, const void* q, const void* k, const void* v, const void* dout,
                            const float2* nd, float* dq, float* dk, float* dv, void* f_dq, void* f_dk, void* f_dv,
-                           void* o_dq, void* o_dk, void* o_dv, const int32_t* rem_dst, const int32_t* rem_src, int H, int d,
-                           hipStream_t st) {
+                           void* o_dq, void* o_dk, void* o_dv, const int32_t* rem_dst, const int32_t* rem_src, bool zero_rows,
+                           int H, int d, hipStream_t st) {
 #define X(D_, H_)                                                                                                        \
     if (d == D_ && H == H_)                                                                                              \
         return tile_bwd_launch_s<T, D_, H_>(tl, q, k, v, dout, nd, dq, dk, dv, f_dq, f_dk, f_dv, o_dq, o_dk, o_dv, rem_dst, \
-                                            rem_src, st);
+                                            rem_src, zero_rows, st);
     TGT_TILE_SHAPES(X)
 #undef X
     set_error("block attention: no tile kernel for H=%d, d=%d", H, d);
@@ -677,8 +761,10 @@ int tgt_block_attn_fwd(const tgt_tiles_t* tiles, const tgt_plan_t* plan, const v
     float* Zdst = tiles_only ? d_Z : Zp;
     // with remaining edges: the tile kernels still finish the rows that have none (the sparse kernels skip them)
     const int32_t* rem = plan->dst.rowptr;
-    rc = dtype == TGT_DTYPE_F32 ? tgt::tile_fwd_launch<float>(tiles, d_q, d_k, d_v, acc, Zdst, fin, d_out, d_Z, rem, H, d, st)
-                                : tgt::tile_fwd_launch<tgt::tbf16>(tiles, d_q, d_k, d_v, acc, Zdst, fin, d_out, d_Z, rem, H, d, st);
+    // a plan that schedules only rows with edges leaves the rows without edges and without tiles to the tile launch
+    const bool zr = plan->rows_with_edges_only;
+    rc = dtype == TGT_DTYPE_F32 ? tgt::tile_fwd_launch<float>(tiles, d_q, d_k, d_v, acc, Zdst, fin, d_out, d_Z, rem, zr, H, d, st)
+                                : tgt::tile_fwd_launch<tgt::tbf16>(tiles, d_q, d_k, d_v, acc, Zdst, fin, d_out, d_Z, rem, zr, H, d, st);
     if (rc || tiles_only) return rc;
     tgt::TileInit init{};
     init.acc = acc; init.Z = Zp; init.cover_dst = tiles->cover_dst.as<uint8_t>();
@@ -711,9 +797,9 @@ int tgt_block_attn_bwd(const tgt_tiles_t* tiles, const tgt_plan_t* plan, const v
     void* f_dv = tiles_only ? d_dv : nullptr;
     rc = dtype == TGT_DTYPE_F32
              ? tgt::tile_bwd_launch<float>(tiles, d_q, d_k, d_v, d_dout, nd, dq, dk, dv, f_dq, f_dk, f_dv, d_dq, d_dk, d_dv,
-                                           plan->dst.rowptr, plan->src.rowptr, H, d, st)
+                                           plan->dst.rowptr, plan->src.rowptr, plan->rows_with_edges_only, H, d, st)
              : tgt::tile_bwd_launch<tgt::tbf16>(tiles, d_q, d_k, d_v, d_dout, nd, dq, dk, dv, f_dq, f_dk, f_dv, d_dq, d_dk,
-                                                d_dv, plan->dst.rowptr, plan->src.rowptr, H, d, st);
+                                                d_dv, plan->dst.rowptr, plan->src.rowptr, plan->rows_with_edges_only, H, d, st);
     if (rc || tiles_only) return rc;     // (no edges: there is no per-edge bias gradient to write either)
     tgt::TileInit init{};
     init.dq = dq; init.dk = dk; init.dv = dv;

@@ -230,6 +230,9 @@ const float2* sparse_attn_nd_ptr(void* d_workspace);
 struct tgt_plan {
     int64_t N = 0, E = 0;
     int device = 0;
+    // a plan of the edges that remain beside a tile set: rows without edges have no place in its schedules
+    // (the tile kernels write them), so the sparse entry points on their own must refuse it
+    bool rows_with_edges_only = false;
     tgt::Side dst;   // edges grouped by destination (query) node
     tgt::Side src;   // edges grouped by source (key/value) node
     tgt::Schedule sched[tgt::kNumLpe];   // by log2(lanes per edge); made on first use of a shape

@@ -77,7 +77,9 @@ __global__ void k_gather_col(const uint32_t* __restrict__ eid, const uint32_t* _
 constexpr int kSchedCats = kNumClass + 1;   // the wave classes, then "longer than a wave row"
 constexpr int kSchedMaxWaves = 16;          // a window is one workgroup of up to 1024 threads, one per row
 
-__device__ __forceinline__ int sched_category(int len, int wave_row_max) {
+// skip_empty: rows without edges get no place in the schedule (-1)
+__device__ __forceinline__ int sched_category(int len, int wave_row_max, bool skip_empty) {
+    if (skip_empty && len == 0) return -1;
     if (len > wave_row_max) return kNumClass;
     if (len > 32) return 0;
     if (len > 16) return 1;
@@ -87,13 +89,13 @@ __device__ __forceinline__ int sched_category(int len, int wave_row_max) {
 }
 
 // counts[window * kSchedCats + cat] = rows of that category among the window's rows (blockDim.x rows)
-__global__ void k_sched_count(const int32_t* __restrict__ rowptr, int64_t N, int wave_row_max,
+__global__ void k_sched_count(const int32_t* __restrict__ rowptr, int64_t N, int wave_row_max, bool skip_empty,
                               uint32_t* __restrict__ counts) {
     __shared__ uint32_t c[kSchedCats];
     if (threadIdx.x < kSchedCats) c[threadIdx.x] = 0;
     __syncthreads();
     const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int cat = r < N ? sched_category(rowptr[r + 1] - rowptr[r], wave_row_max) : -1;
+    const int cat = r < N ? sched_category(rowptr[r + 1] - rowptr[r], wave_row_max, skip_empty) : -1;
 #pragma unroll
     for (int k = 0; k < kSchedCats; ++k) {
         const uint64_t b = __ballot(cat == k);
@@ -139,7 +141,7 @@ __global__ __launch_bounds__(1024) void k_sched_scan(const uint32_t* __restrict_
 // Rows keep their order inside a (window, category): position = offs[window, cat] + rank among the
 // window's rows.  Wave-class rows become wave items at items[position]; long rows are listed (row, first
 // edge, length) for the kernels that cut them into workgroup items.
-__global__ void k_sched_fill(const int32_t* __restrict__ rowptr, int64_t N, int wave_row_max,
+__global__ void k_sched_fill(const int32_t* __restrict__ rowptr, int64_t N, int wave_row_max, bool skip_empty,
                              const uint32_t* __restrict__ offs, Item* __restrict__ items,
                              int32_t* __restrict__ long_rows, int64_t cap_long) {
     __shared__ uint32_t wave_cnt[kSchedMaxWaves][kSchedCats];
@@ -149,7 +151,7 @@ __global__ void k_sched_fill(const int32_t* __restrict__ rowptr, int64_t N, int 
     if (r < N) {
         start = rowptr[r];
         len = rowptr[r + 1] - start;
-        cat = sched_category(len, wave_row_max);
+        cat = sched_category(len, wave_row_max, skip_empty);
     }
     const uint64_t lower = lane == 0 ? 0ull : (~0ull >> (64 - lane));
     uint32_t rank = 0;
@@ -400,7 +402,7 @@ constexpr int kReportHead = 32;
 constexpr int kReportFlag = 16;
 
 static int schedule_device(int64_t N, int64_t E, Side& side, SideScratch& sc, int32_t* report, int side_idx,
-                           hipStream_t st) {
+                           bool skip_empty, hipStream_t st) {
     // tuning overrides (experiments only; the defaults are the measured best)
     sc.wave_row_max = env_int("TGT_WAVE_ROW_MAX", tgt::kWaveRowMax);
     sc.cp.block_seg = env_int("TGT_BLOCK_SEG", tgt::kBlockSeg);
@@ -431,9 +433,9 @@ static int schedule_device(int64_t N, int64_t E, Side& side, SideScratch& sc, in
     TGT_HIP_CHECK(sc.row_split_idx.alloc(sizeof(int32_t) * (size_t)sc.cap_long, st));
     TGT_HIP_CHECK(sc.row_part_off.alloc(sizeof(int32_t) * (size_t)sc.cap_long, st));
     TGT_HIP_CHECK(sc.meta.alloc(sizeof(BlockMeta) * (size_t)sc.cap_block, st));
-    hipLaunchKernelGGL(k_sched_count, dim3(sc.nwin), dim3(sc.W), 0, st, side.rowptr, N, sc.wave_row_max, counts);
+    hipLaunchKernelGGL(k_sched_count, dim3(sc.nwin), dim3(sc.W), 0, st, side.rowptr, N, sc.wave_row_max, skip_empty, counts);
     hipLaunchKernelGGL(k_sched_scan, dim3(1), dim3(1024), 0, st, counts, sc.nwin, offs, hdr);
-    hipLaunchKernelGGL(k_sched_fill, dim3(sc.nwin), dim3(sc.W), 0, st, side.rowptr, N, sc.wave_row_max, offs, side.items,
+    hipLaunchKernelGGL(k_sched_fill, dim3(sc.nwin), dim3(sc.W), 0, st, side.rowptr, N, sc.wave_row_max, skip_empty, offs, side.items,
                        sc.long_rows.as<int32_t>(), sc.cap_long);
     hipLaunchKernelGGL(k_cut_rows, dim3(1), dim3(1024), 0, st, sc.long_rows.as<int32_t>(), hdr, sc.cp,
                        sc.row_item_off.as<int32_t>(), sc.row_split_idx.as<int32_t>(), sc.row_part_off.as<int32_t>(),
@@ -703,9 +705,9 @@ static int create_impl(const int64_t* d_src, const int64_t* d_dst, int64_t E, in
     rc = build_side(s32.as<uint32_t>(), d32.as<uint32_t>(), E, N, sorter, plan->src, st);
     if (rc) return rc;
     SideScratch scr_d, scr_s;
-    rc = schedule_device(N, E, plan->dst, scr_d, report, 0, st);
+    rc = schedule_device(N, E, plan->dst, scr_d, report, 0, plan->rows_with_edges_only, st);
     if (rc) return rc;
-    rc = schedule_device(N, E, plan->src, scr_s, report, 1, st);
+    rc = schedule_device(N, E, plan->src, scr_s, report, 1, plan->rows_with_edges_only, st);
     if (rc) return rc;
     std::vector<int32_t> h_report(report_ints);
     TGT_HIP_CHECK(hipMemcpyAsync(h_report.data(), report, sizeof(int32_t) * report_ints, hipMemcpyDeviceToHost, st));
@@ -838,8 +840,8 @@ int tgt_edge_index_hash(const int64_t* d_src, const int64_t* d_dst, int64_t E, v
     return TGT_OK;
 }
 
-int tgt_plan_create(const int64_t* d_src, const int64_t* d_dst, int64_t E, int64_t N, void* stream,
-                    tgt_plan_t** out_plan) {
+static int plan_create_checked(const int64_t* d_src, const int64_t* d_dst, int64_t E, int64_t N, void* stream,
+                               bool rows_with_edges_only, tgt_plan_t** out_plan) {
     if (!out_plan || E < 0 || N < 1 || (E > 0 && (!d_src || !d_dst))) {
         tgt::set_error("tgt_plan_create: null pointer, E < 0 or N < 1");
         return TGT_ERR_INVALID_ARG;
@@ -850,6 +852,7 @@ int tgt_plan_create(const int64_t* d_src, const int64_t* d_dst, int64_t E, int64
     }
     tgt_plan* plan = new (std::nothrow) tgt_plan();
     if (!plan) return TGT_ERR_INVALID_ARG;
+    plan->rows_with_edges_only = rows_with_edges_only;
     int rc = tgt::create_impl(d_src, d_dst, E, N, (hipStream_t)stream, plan);
     if (rc != TGT_OK) {
         tgt::free_side(plan->dst);
@@ -860,6 +863,16 @@ int tgt_plan_create(const int64_t* d_src, const int64_t* d_dst, int64_t E, int64
     }
     *out_plan = plan;
     return TGT_OK;
+}
+
+int tgt_plan_create(const int64_t* d_src, const int64_t* d_dst, int64_t E, int64_t N, void* stream,
+                    tgt_plan_t** out_plan) {
+    return plan_create_checked(d_src, d_dst, E, N, stream, false, out_plan);
+}
+
+int tgt_plan_create_remaining(const int64_t* d_src, const int64_t* d_dst, int64_t E, int64_t N, void* stream,
+                              tgt_plan_t** out_plan) {
+    return plan_create_checked(d_src, d_dst, E, N, stream, true, out_plan);
 }
 
 int tgt_plan_destroy(tgt_plan_t* plan) {

@@ -1309,6 +1309,16 @@ int sparse_attn_fwd_noalloc_impl(const tgt_plan_t* plan, const void* d_q, const 
 }  // namespace tgt
 
 #if !defined(TGT_SPARSE_PART) || TGT_SPARSE_PART == 0
+// A plan made by tgt_plan_create_remaining schedules no row without edges: only the block path, whose tile
+// kernels write those rows, may run it.
+static int refuse_remaining(const tgt_plan_t* plan) {
+    if (plan && plan->rows_with_edges_only) {
+        tgt::set_error("this plan holds the edges beside a tile set (tgt_plan_create_remaining): use tgt_block_attn_*");
+        return TGT_ERR_INVALID_ARG;
+    }
+    return TGT_OK;
+}
+
 extern "C" {
 
 int64_t tgt_sparse_attn_workspace_bytes(const tgt_plan_t* plan, int H, int d) {
@@ -1319,6 +1329,7 @@ int64_t tgt_sparse_attn_workspace_bytes(const tgt_plan_t* plan, int H, int d) {
 int tgt_sparse_attn_fwd(const tgt_plan_t* plan, const void* d_q, const void* d_k, const void* d_v,
                         const void* d_bias, int bias_mode, int H, int d, int dtype, void* d_out, float* d_Z,
                         void* d_workspace, int64_t workspace_bytes, void* stream) {
+    if (int rc = refuse_remaining(plan)) return rc;
     return tgt::sparse_attn_fwd_impl(plan, d_q, d_k, d_v, d_bias, bias_mode, H, d, dtype, d_out, d_Z, d_workspace,
                                      workspace_bytes, stream, nullptr);
 }
@@ -1326,6 +1337,7 @@ int tgt_sparse_attn_fwd(const tgt_plan_t* plan, const void* d_q, const void* d_k
 int tgt_sparse_attn_fwd_noalloc(const tgt_plan_t* plan, const void* d_q, const void* d_k, const void* d_v,
                                 const void* d_bias, int bias_mode, int H, int d, int dtype, void* d_out, float* d_Z,
                                 void* stream) {
+    if (int rc = refuse_remaining(plan)) return rc;
     return tgt::sparse_attn_fwd_noalloc_impl(plan, d_q, d_k, d_v, d_bias, bias_mode, H, d, dtype, d_out, d_Z, stream);
 }
 
@@ -1338,6 +1350,7 @@ int tgt_sparse_attn_bwd(const tgt_plan_t* plan, const void* d_q, const void* d_k
                         const void* d_bias, int bias_mode, int H, int d, int dtype, const void* d_out,
                         const float* d_Z, const void* d_dout, void* d_dq, void* d_dk, void* d_dv,
                         void* d_dbias, void* d_workspace, int64_t workspace_bytes, void* stream) {
+    if (int rc = refuse_remaining(plan)) return rc;
     return tgt::sparse_attn_bwd_impl(plan, d_q, d_k, d_v, d_bias, bias_mode, H, d, dtype, d_out, d_Z, d_dout, d_dq,
                                      d_dk, d_dv, d_dbias, d_workspace, workspace_bytes, stream, nullptr, false);
 }

@@ -19,9 +19,11 @@ from . import _ext, _lib
 
 class GraphPlan:
     """Stable CSR-by-destination / CSC-by-source views of ``edge_index`` plus the
-    row schedule, resident on the GPU."""
+    row schedule, resident on the GPU.  ``rows_with_edges_only``: a plan of the edges beside a tile set
+    (``block_attention``): rows without edges are left out of the schedule and written by the tile kernels;
+    ``sparse_attention`` refuses such a plan."""
 
-    def __init__(self, edge_index, num_nodes):
+    def __init__(self, edge_index, num_nodes, rows_with_edges_only=False):
         if not isinstance(edge_index, torch.Tensor) or edge_index.dim() != 2 or edge_index.size(0) != 2:
             raise ValueError("edge_index must be a [2, E] tensor")
         if not edge_index.is_cuda:
@@ -30,6 +32,7 @@ class GraphPlan:
         self.num_nodes = int(num_nodes)
         self.num_edges = int(ei.size(1))
         self.device = ei.device
+        self.rows_with_edges_only = bool(rows_with_edges_only)
         self._handle = ctypes.c_void_p()
         self._workspaces = {}
         _ext.ops()                       # registers torch's caching allocator with the library: no hipMalloc per plan
@@ -38,8 +41,8 @@ class GraphPlan:
             stream = torch.cuda.current_stream(self.device).cuda_stream
             src_ptr = ei[0].data_ptr() if self.num_edges else None
             dst_ptr = ei[1].data_ptr() if self.num_edges else None
-            _lib.check(L.tgt_plan_create(src_ptr, dst_ptr, self.num_edges, self.num_nodes, stream,
-                                         ctypes.byref(self._handle)))
+            create = L.tgt_plan_create_remaining if rows_with_edges_only else L.tgt_plan_create
+            _lib.check(create(src_ptr, dst_ptr, self.num_edges, self.num_nodes, stream, ctypes.byref(self._handle)))
         # the owner of the C plan: shared with every autograd node that needs the plan in its backward, so that
         # the plan outlives this object if a backward is still pending
         self.holder = torch.classes.torchgt.PlanHolder(self._handle.value)
