@@ -44,14 +44,41 @@ __device__ __forceinline__ short t_ld1(const tbf16* p) { return (short)p->x; }
 __device__ __forceinline__ short t_ld1(const float* p) { return t_f2bf(*p); }
 __device__ __forceinline__ bshort4 t_zero4() { bshort4 z; z.x = 0; z.y = 0; z.z = 0; z.w = 0; return z; }
 __device__ __forceinline__ bfloat4 t_zerof() { bfloat4 z; z.x = 0.f; z.y = 0.f; z.z = 0.f; z.w = 0.f; return z; }
+// the operand of the lanes whose four elements lie beyond the head's D must be zero whatever the memory holds
+// (0 x Inf would not be): an AND with 0 or ~0 instead of a load under a lane mask
+__device__ __forceinline__ bshort4 t_and4(bshort4 v, int m) {
+    typedef int i2 __attribute__((ext_vector_type(2)));
+    i2 x = __builtin_bit_cast(i2, v);
+    x.x &= m; x.y &= m;
+    return __builtin_bit_cast(bshort4, x);
+}
 __device__ __forceinline__ bfloat4 mfma16(bshort4 a, bshort4 b, bfloat4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, c, 0, 0, 0);
 }
-__device__ __forceinline__ float t_clamp5(float x) { return x < -5.0f ? -5.0f : (x > 5.0f ? 5.0f : x); }
+// exp(clamp(s / sqrt(d), -5, 5)) (attn_module.py:160-161) from x2 = s * log2(e) / sqrt(d): one multiply, a median of
+// three and the hardware's exp2 (its argument stays within +-7.3); NaN stays NaN, like torch.clamp
+constexpr float kLog2e = 1.44269504088896340736f;
+constexpr float kClamp2 = 5.0f * kLog2e;
+__device__ __forceinline__ float t_weight(float x2) {
+    const float w = __builtin_amdgcn_exp2f(__builtin_amdgcn_fmed3f(x2, -kClamp2, kClamp2));
+    return x2 != x2 ? x2 : w;
+}
+// the clamp lets a gradient through where the score is inside [-5, 5] (inclusive, like torch.clamp's backward)
+__device__ __forceinline__ bool t_inside(float x2) { return fabsf(x2) <= kClamp2; }
+// four floats -> four bf16 (round to nearest even), two values per conversion instruction
+__device__ __forceinline__ int t_cvt_pk(float lo, float hi) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    f32x2 x;
+    x.x = lo; x.y = hi;
+    return __builtin_bit_cast(int, __builtin_convertvector(x, bf16x2));
+}
 __device__ __forceinline__ bshort4 t_pack(const float (&x)[4]) {
-    bshort4 r;
-    r.x = t_f2bf(x[0]); r.y = t_f2bf(x[1]); r.z = t_f2bf(x[2]); r.w = t_f2bf(x[3]);
-    return r;
+    typedef int i2 __attribute__((ext_vector_type(2)));
+    i2 r;
+    r.x = t_cvt_pk(x[0], x[1]);
+    r.y = t_cvt_pk(x[2], x[3]);
+    return __builtin_bit_cast(bshort4, r);
 }
 constexpr int kTile = 16;
 constexpr float kTileEps = 1e-6f;   // attn_module.py:187
@@ -61,8 +88,8 @@ __device__ __forceinline__ void t_st4(float* p, float a, float b, float c, float
     *reinterpret_cast<bfloat4*>(p) = r;
 }
 __device__ __forceinline__ void t_st4(tbf16* p, float a, float b, float c, float d) {
-    bshort4 r; r.x = t_f2bf(a); r.y = t_f2bf(b); r.z = t_f2bf(c); r.w = t_f2bf(d);
-    *reinterpret_cast<bshort4*>(p) = r;
+    const float x[4] = {a, b, c, d};
+    *reinterpret_cast<bshort4*>(p) = t_pack(x);
 }
 
 // Rows no tile covers get zeros when the tile kernels write final results (no remaining edges, or a plan of the
@@ -91,6 +118,16 @@ __device__ __forceinline__ void zero_bare_rows(const BareRows& br, int HD, int H
     }
     if (Z) for (int h = part; h < H; h += 8) Z[row * H + h] = 0.f;
 }
+// Waves per SIMD the kernels are compiled for (the register budget follows from it).  Without a bound the compiler
+// budgets 512 registers, puts the matrix accumulators into AGPRs and copies them around every matrix instruction.
+#ifndef TGT_TILE_FWD_OCC
+#define TGT_TILE_FWD_OCC 4
+#endif
+#ifndef TGT_TILE_DST_OCC
+#define TGT_TILE_DST_OCC 4
+#endif
+template <int HD> constexpr int fwd_occupancy() { return HD <= 64 ? TGT_TILE_FWD_OCC : 4; }
+template <typename T, int HD> constexpr int dst_occupancy() { return HD <= 64 && sizeof(T) == 2 ? TGT_TILE_DST_OCC : 3; }
 // waves (= tile groups) per workgroup of the tile kernels: as many as keep the static LDS under 64 KB
 template <int HD> constexpr int tile_waves() { return HD > 64 ? 2 : 4; }
 
@@ -110,13 +147,12 @@ template <typename T, int HD> struct RowPieces {
     static constexpr int ITERS = (kTile * CPR + 63) / 64;
     uint4 p[ITERS];
 };
-__device__ __forceinline__ uint32_t pack2(short lo, short hi) { return (uint32_t)(uint16_t)lo | ((uint32_t)(uint16_t)hi << 16); }
 __device__ __forceinline__ void load_piece(const tbf16* p, uint4& r) { r = *reinterpret_cast<const uint4*>(p); }
 __device__ __forceinline__ void load_piece(const float* p, uint4& r) {
     const bfloat4 a = *reinterpret_cast<const bfloat4*>(p);
     const bfloat4 b = *reinterpret_cast<const bfloat4*>(p + 4);
-    r.x = pack2(t_f2bf(a.x), t_f2bf(a.y)); r.y = pack2(t_f2bf(a.z), t_f2bf(a.w));
-    r.z = pack2(t_f2bf(b.x), t_f2bf(b.y)); r.w = pack2(t_f2bf(b.z), t_f2bf(b.w));
+    r.x = (uint32_t)t_cvt_pk(a.x, a.y); r.y = (uint32_t)t_cvt_pk(a.z, a.w);
+    r.z = (uint32_t)t_cvt_pk(b.x, b.y); r.w = (uint32_t)t_cvt_pk(b.z, b.w);
 }
 __device__ __forceinline__ void unpack_piece(const uint4& u, short (&v)[8]) {
     v[0] = (short)(u.x & 0xffffu); v[1] = (short)(u.x >> 16);
@@ -130,7 +166,12 @@ __device__ __forceinline__ void load_rows(const T* __restrict__ X, int row0, int
 #pragma unroll
     for (int i = 0; i < RowPieces<T, HD>::ITERS; ++i) {
         const int c = i * 64 + lane;
-        if (kTile * CPR % 64 == 0 || c < kTile * CPR) load_piece(X + (int64_t)row0 * HD + c * 8, rp.p[i]);   // rows are contiguous
+        // rows are contiguous: a scalar base (row0 is the same in all lanes) plus a 32-bit lane offset; the empty
+        // statement keeps the sum from being re-associated into a 64-bit address per lane held across the tile loop
+        const char* base = reinterpret_cast<const char*>(X) + (int64_t)row0 * HD * (int)sizeof(T);
+        asm volatile("" : "+s"(base));
+        if (kTile * CPR % 64 == 0 || c < kTile * CPR)
+            load_piece(reinterpret_cast<const T*>(base + (uint32_t)(c * 8 * (int)sizeof(T))), rp.p[i]);
     }
 }
 template <typename T, int HD>
@@ -159,6 +200,9 @@ __device__ __forceinline__ void store_rows(const RowPieces<T, HD>& rp, short* __
 // Whether the next tile's rows are asked for while the current one is worked on: where the pieces in flight fit the
 // registers next to the accumulators (2-byte elements, up to 64 per row)
 template <typename T, int HD> constexpr bool tile_prefetch() { return sizeof(T) == 2 && HD <= 64; }
+// Hides where a scalar came from: addresses formed from the result cannot be computed before this point.  Put
+// behind a kernel's tile loop it keeps the epilogue's pointers out of the registers the loop needs.
+__device__ __forceinline__ int late_scalar(int x) { asm volatile("" : "+s"(x)); return x; }
 // the first lane's value as a scalar: what every lane of a wave holds alike (a group's record) steers loops and
 // addresses from scalar registers
 __device__ __forceinline__ int wave_uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
@@ -185,7 +229,7 @@ __device__ __forceinline__ void wave_lds_fence() {
 // the output rows and Z themselves; otherwise it does so for the destinations that have no remaining edge and
 // leaves fp32 sums of the others for the sparse kernel to add (which skips the former).
 template <typename T, int D, int H, bool FINAL>
-__global__ __launch_bounds__(64 * tile_waves<H * D>(), 4) void k_tile_fwd(const int4* __restrict__ grp_rec,
+__global__ __launch_bounds__(64 * tile_waves<H * D>(), fwd_occupancy<H * D>()) void k_tile_fwd(const int4* __restrict__ grp_rec,
                                                               const int32_t* __restrict__ tile_r0, int n_groups,
                                                               const T* __restrict__ Q, const T* __restrict__ K,
                                                               const T* __restrict__ V, float* __restrict__ acc,
@@ -196,6 +240,7 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 4) void k_tile_fwd(const 
     constexpr int HD = H * D;
     constexpr int kTileWaves = tile_waves<HD>();
     constexpr bool kPrefetch = tile_prefetch<T, HD>();
+    const float scale2 = inv_scale * kLog2e;
     __shared__ short lds[kTileWaves * (rm_size<HD>() + tr_size<HD>())];
     if ((int)blockIdx.x >= bare.first_block) {      // uniform over the workgroup
         zero_bare_rows<T>(bare, HD, H, out, (T*)nullptr, Zout, rem_rowptr);
@@ -208,6 +253,7 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 4) void k_tile_fwd(const 
     short* v_tr = k_rm + rm_size<HD>();
     const int col = lane & 15, kq = lane >> 4;
     const bool kval = kq * 4 < D;
+    const int kmask = kval ? -1 : 0;
     // one 16-byte record per group: (first node, tile range, the first tile's other side) - a wave with one tile, the
     // usual case, needs no second look-up before it can ask for the tile's rows
     const int4 gr = grp_rec[g];
@@ -246,20 +292,21 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 4) void k_tile_fwd(const 
         }
 #pragma unroll
         for (int h = 0; h < H; ++h) {
-            bshort4 ak = t_zero4();
-            if (kval) ak = a_rows<HD>(k_rm, col, h * D + kq * 4);
+            // every lane reads (no lane mask around the LDS reads): lanes beyond the head's D get zeros by an AND, and
+            // what the rows dd >= D of the second product hold is never stored
+            const bshort4 ak = t_and4(a_rows<HD>(k_rm, col, h * D + (kq * 4) % D), kmask);
             const bfloat4 sc = mfma16(ak, bq[h], t_zerof());       // S^T[source 4kq+r][destination col]
             float w[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                w[r] = __expf(t_clamp5(sc[r] * inv_scale));
+                w[r] = t_weight(sc[r] * scale2);
                 z[h] += w[r];
             }
-            bshort4 av = t_zero4();
-            if (col < D) av = a_cols(v_tr, h * D + col, kq);
+            const bshort4 av = a_cols(v_tr, h * D + col % D, kq);
             o[h] = mfma16(av, t_pack(w), o[h]);                    // O^T[dd 4kq+r][destination col]
         }
     }
+    const int c0e = late_scalar(c0);
 #pragma unroll
     for (int h = 0; h < H; ++h) {
         float zz = z[h];
@@ -267,17 +314,17 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 4) void k_tile_fwd(const 
         zz += __shfl_xor(zz, 32);
         if (fin) {
             const float inv = 1.0f / (zz + kTileEps);
-            if (kval) t_st4(out + (int64_t)(c0 + col) * HD + h * D + kq * 4, o[h].x * inv, o[h].y * inv, o[h].z * inv, o[h].w * inv);
+            if (kval) t_st4(out + (int64_t)(c0e + col) * HD + h * D + kq * 4, o[h].x * inv, o[h].y * inv, o[h].z * inv, o[h].w * inv);
         } else if (kval) {
-            *reinterpret_cast<bfloat4*>(acc + (int64_t)(c0 + col) * HD + h * D + kq * 4) = o[h];
+            *reinterpret_cast<bfloat4*>(acc + (int64_t)(c0e + col) * HD + h * D + kq * 4) = o[h];
         }
-        if (kq == 0) (fin ? Zout : Zp)[(int64_t)(c0 + col) * H + h] = zz;
+        if (kq == 0) (fin ? Zout : Zp)[(int64_t)(c0e + col) * H + h] = zz;
     }
 }
 
 // Same grouping: dQ of the tiles.  nd[i,h] = (1/(Z+eps), dout.out) of the FINAL output.
 template <typename T, int D, int H, bool FINAL>
-__global__ __launch_bounds__(64 * tile_waves<H * D>(), 3) void k_tile_bwd_dst(const int4* __restrict__ grp_rec,
+__global__ __launch_bounds__(64 * tile_waves<H * D>(), (dst_occupancy<T, H * D>())) void k_tile_bwd_dst(const int4* __restrict__ grp_rec,
                                                                   const int32_t* __restrict__ tile_r0, int n_groups,
                                                                   const T* __restrict__ Q, const T* __restrict__ K,
                                                                   const T* __restrict__ V, const T* __restrict__ dO,
@@ -288,6 +335,7 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 3) void k_tile_bwd_dst(co
     constexpr int HD = H * D;
     constexpr int kTileWaves = tile_waves<HD>();
     constexpr bool kPrefetch = tile_prefetch<T, HD>();
+    const float scale2 = inv_scale * kLog2e;
     constexpr int PER_WAVE = 2 * rm_size<HD>() + tr_size<HD>();
     __shared__ short lds[kTileWaves * PER_WAVE];
     if ((int)blockIdx.x >= bare.first_block) {
@@ -342,6 +390,8 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 3) void k_tile_bwd_dst(co
         }
 #pragma unroll
         for (int h = 0; h < H; ++h) {
+            // operands of the lanes beyond the head's D: reads under a lane mask here - read by all lanes as in the
+            // forward, the compiler moves more reads to the front than the registers of this occupancy hold
             bshort4 ak = t_zero4(), av = t_zero4();
             if (kval) {
                 ak = a_rows<HD>(k_rm, col, h * D + kq * 4);
@@ -352,23 +402,23 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 3) void k_tile_bwd_dst(co
             float md[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const float raw = sc[r] * inv_scale;
-                const float wv = __expf(t_clamp5(raw));
-                const float dS = wv * ndv[h].x * (dp[r] - ndv[h].y);
-                md[r] = ((raw >= -5.0f) & (raw <= 5.0f)) ? dS : 0.f;
+                const float x2 = sc[r] * scale2;
+                const float dS = t_weight(x2) * ndv[h].x * (dp[r] - ndv[h].y);
+                md[r] = t_inside(x2) ? dS : 0.f;
             }
             bshort4 akT = t_zero4();
             if (col < D) akT = a_cols(k_tr, h * D + col, kq);
             dq[h] = mfma16(akT, t_pack(md), dq[h]);                // dQ^T[dd][destination] += K^T (m dS)^T
         }
     }
+    const int c0e = late_scalar(c0);
     if (kval) {
 #pragma unroll
         for (int h = 0; h < H; ++h) {
             bfloat4 o;
             o.x = dq[h].x * inv_scale; o.y = dq[h].y * inv_scale; o.z = dq[h].z * inv_scale; o.w = dq[h].w * inv_scale;
-            if (fin) t_st4(dq_out + (int64_t)(c0 + col) * HD + h * D + kq * 4, o.x, o.y, o.z, o.w);
-            else *reinterpret_cast<bfloat4*>(dq_part + (int64_t)(c0 + col) * HD + h * D + kq * 4) = o;
+            if (fin) t_st4(dq_out + (int64_t)(c0e + col) * HD + h * D + kq * 4, o.x, o.y, o.z, o.w);
+            else *reinterpret_cast<bfloat4*>(dq_part + (int64_t)(c0e + col) * HD + h * D + kq * 4) = o;
         }
     }
 }
@@ -387,7 +437,8 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 3) void k_tile_bwd_src(co
                                                                   float inv_scale) {
     constexpr int HD = H * D;
     constexpr int kTileWaves = tile_waves<HD>();
-    constexpr bool kPrefetch = tile_prefetch<T, HD>();
+    constexpr bool kPrefetch = false;
+    const float scale2 = inv_scale * kLog2e;
     constexpr int PER_WAVE = 2 * rm_size<HD>() + 2 * tr_size<HD>() + 4 * kTile * H;   // + nd tile (float2 = 4 shorts)
     __shared__ __align__(16) short lds[kTileWaves * PER_WAVE];
     if ((int)blockIdx.x >= bare.first_block) {
@@ -465,11 +516,11 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 3) void k_tile_bwd_src(co
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const float2 ndv = nd_l[(4 * kq + r) * H + h];
-                const float raw = sc[r] * inv_scale;
-                const float p = __expf(t_clamp5(raw)) * ndv.x;
+                const float x2 = sc[r] * scale2;
+                const float p = t_weight(x2) * ndv.x;
                 const float dS = p * (dp[r] - ndv.y);
                 pw[r] = p;
-                md[r] = ((raw >= -5.0f) & (raw <= 5.0f)) ? dS : 0.f;
+                md[r] = t_inside(x2) ? dS : 0.f;
             }
             bshort4 agT = t_zero4(), aqT = t_zero4();
             if (col < D) {
@@ -480,17 +531,18 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 3) void k_tile_bwd_src(co
             dk[h] = mfma16(aqT, t_pack(md), dk[h]);                // dK^T[dd][source] += Q^T (m dS)
         }
     }
+    const int r0e = late_scalar(r0);
     if (kval) {
 #pragma unroll
         for (int h = 0; h < H; ++h) {
             bfloat4 o;
             o.x = dk[h].x * inv_scale; o.y = dk[h].y * inv_scale; o.z = dk[h].z * inv_scale; o.w = dk[h].w * inv_scale;
             if (fin) {
-                t_st4(dk_out + (int64_t)(r0 + col) * HD + h * D + kq * 4, o.x, o.y, o.z, o.w);
-                t_st4(dv_out + (int64_t)(r0 + col) * HD + h * D + kq * 4, dv[h].x, dv[h].y, dv[h].z, dv[h].w);
+                t_st4(dk_out + (int64_t)(r0e + col) * HD + h * D + kq * 4, o.x, o.y, o.z, o.w);
+                t_st4(dv_out + (int64_t)(r0e + col) * HD + h * D + kq * 4, dv[h].x, dv[h].y, dv[h].z, dv[h].w);
             } else {
-                *reinterpret_cast<bfloat4*>(dk_part + (int64_t)(r0 + col) * HD + h * D + kq * 4) = o;
-                *reinterpret_cast<bfloat4*>(dv_part + (int64_t)(r0 + col) * HD + h * D + kq * 4) = dv[h];
+                *reinterpret_cast<bfloat4*>(dk_part + (int64_t)(r0e + col) * HD + h * D + kq * 4) = o;
+                *reinterpret_cast<bfloat4*>(dv_part + (int64_t)(r0e + col) * HD + h * D + kq * 4) = dv[h];
             }
         }
     }
