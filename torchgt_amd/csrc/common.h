@@ -67,11 +67,15 @@ __host__ __device__ constexpr bool class_inline(int lpe, int cls) {
 // What one wave of an attention workgroup reads first: its share of the launch, complete.  Workgroup b
 // owns records 4b .. 4b+3.  `code` is a descriptor code (kind, view, number of rows).
 //   kind 5: `item` is the workgroup item (all four records of the workgroup carry it);
-//   kind 0: rows row[i] with edges [start[i], start[i] + len[i]) of the view's sorted arrays;
-//   kind 1..4: the same rows, and their edges inline: col / eid hold, for lane group g = (row i of the
-//   wave, slot s) - g = i * S + s, S = slots_for_class - the four edges s, s + S, s + 2S, s + 3S of the row
-//   at [4g, 4g + 4) (an edge past the end of the row repeats the row's last edge; 0 for an empty row).
-// One coalesced read gives a wave everything it needs to issue its gathers.
+//   kind 0: lane group g = (row i of the wave, slot s), g = i * S + s, S = slots_for_class, works on row row[g]
+//   with edges [start[g], start[g] + len[g]) of the view's sorted arrays (the S groups of a row hold the same
+//   three numbers; zeros behind the wave's last row);
+//   kind 1..4: the same, and the edges inline: col / eid hold for lane group g the four edges s, s + S, s + 2S,
+//   s + 3S of its row at [4g, 4g + 4) (an edge past the end of the row repeats the row's last edge; 0 for an
+//   empty row).
+// No address in a record depends on the kind: a lane asks for code, row, start, len and its four edges at once,
+// and one memory round trip gives a wave everything it needs to issue its gathers.  (Kinds without inline edges
+// leave col / eid unwritten; what a lane reads there is never used.)
 template <int LPE>
 struct alignas(128) WaveRec {
     static constexpr int kRows = kWave / LPE;          // most rows a wave can hold (shortest class)

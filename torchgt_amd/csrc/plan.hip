@@ -290,7 +290,7 @@ struct Run { int32_t wave0, waves, first, n; uint32_t code; int32_t xcd; int32_t
 
 // One workgroup per run; its waves write the run's wave records in turn (layout: WaveRec in common.h).  Wave lw of
 // XCD x's list is wave lw % 4 of that XCD's (lw / 4)-th workgroup, and workgroup b of the launch runs on XCD b mod 8:
-// record ((lw / 4) * 8 + x) * 4 + lw % 4.  Everything a kernel may read of a record is written: no clearing pass.
+// record ((lw / 4) * 8 + x) * 4 + lw % 4.  Everything a kernel uses of a record is written: no clearing pass.
 __global__ __launch_bounds__(256) void k_build_records(const Run* __restrict__ runs, const Item* __restrict__ items_d,
                                                        const Item* __restrict__ items_s, const Item* __restrict__ bitems_d,
                                                        const Item* __restrict__ bitems_s, const int32_t* __restrict__ col_d,
@@ -326,17 +326,14 @@ __global__ __launch_bounds__(256) void k_build_records(const Run* __restrict__ r
         const int first = run.first + w * ipw;
         const int count = min(ipw, run.n - w * ipw);
         if (t == 0) out[0] = (int32_t)desc_code(kind, src, (uint32_t)count);
-        if (t < count) {
-            const Item it = items[first + t];
-            out[L.off_row + t] = it.row;
-            out[L.off_start + t] = it.start;
-            out[L.off_len + t] = it.len;
-        }
-        if (inl && t < groups) {                        // every lane group's entries, zeros behind the last row
+        if (t < groups) {                               // every lane group's entries, zeros behind the last row
             const int i = t / S, sl = t % S;
             Item it{0, 0, 0, -1};
             if (i < count) it = items[first + i];
-            for (int u = 0; u < 4; ++u) {
+            out[L.off_row + t] = it.row;                // per lane group: a lane finds its row without knowing the class
+            out[L.off_start + t] = it.start;
+            out[L.off_len + t] = it.len;
+            if (inl) for (int u = 0; u < 4; ++u) {
                 const int e = sl + u * S;
                 const int ec = e < it.len ? e : it.len - 1;
                 out[L.off_col + 4 * t + u] = it.len > 0 ? col[it.start + ec] : 0;

@@ -274,6 +274,13 @@ __device__ __forceinline__ void edge_step(const Common& c, const SideArgs& s, co
     Raw8<T> g0[kUnroll], g1[kUnroll];          // gathered rows, unconverted
     decltype(raw1(B)) braw[kUnroll];
     float2 ndv[kUnroll];
+    if constexpr (sizeof(T) == 4) {
+        // The edge ids are waited for here, on every path.  Otherwise the wait sits inside the first lane-masked
+        // block below, and behind that block the compiler must assume the ids may still be in flight: it then
+        // waits for everything outstanding - the first edge's rows - before it asks for the second edge's.
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) asm volatile("" ::"v"(nb[u]), "v"(ed[u]));
+    }
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
         braw[u] = 0;
@@ -529,17 +536,44 @@ __device__ __forceinline__ void walk_range(const Common& c, const SideArgs& s, c
     }
 }
 
+// What one lane takes from its wave's record, asked for in one go when the kernel starts: none of the addresses
+// depends on the row class (the record lists row, start and length per lane group), so the wave has its rows and
+// its edges after one memory round trip, whatever the code then says they are.
+struct RecLane {
+    uint32_t code;
+    int row, start, len;     // of the row this lane group works on (zeros behind the record's last row)
+    int4 cols, eids;         // inline classes: the lane group's four edges (other endpoint, bias row)
+    const int32_t* col_p;    // EDGES == false: where cols and eids are, for a read at the point of use
+    const int32_t* eid_p;
+};
+// EDGES: whether the four edges come along at once.  The 4-byte backward holds two gathered rows per edge in
+// registers and has none to spare for edges that wait through the class dispatch: it reads them where it uses them.
+template <int LPE, bool EDGES>
+__device__ __forceinline__ RecLane load_rec_lane(const WaveRec<LPE>& rec) {
+    const int lg = (threadIdx.x & (kWave - 1)) / LPE;
+    RecLane r;
+    r.code = rec.code;
+    r.row = rec.row[lg];
+    r.start = rec.start[lg];
+    r.len = rec.len[lg];
+    r.col_p = rec.col + lg * kUnroll;
+    r.eid_p = rec.eid + lg * kUnroll;
+    if (EDGES) {
+        r.cols = *reinterpret_cast<const int4*>(r.col_p);
+        r.eids = *reinterpret_cast<const int4*>(r.eid_p);
+    }
+    return r;
+}
+template <typename T, int MODE> constexpr bool rec_edges_early() { return sizeof(T) == 2 || MODE == MODE_FWD; }
+
 // The same for a row of at most S * kUnroll edges whose endpoints and bias rows come with the wave's
 // record (one step, no loop): the record lists them in lane order, four consecutive entries per
 // (row, slot), an edge past the end of the row repeats the row's last one.
 template <typename T, int LPE, int LPH, int S, int MODE, int HASB>
-__device__ __forceinline__ void walk_record(const Common& c, const SideArgs& s, const WaveRec<LPE>& rec, const int row,
+__device__ __forceinline__ void walk_record(const Common& c, const SideArgs& s, const RecLane& rec, const int row,
                                             const int start, const int len, const int slot, const int el,
                                             const bool valid, Acc& acc) {
-    RowRegs<T> rr;
-    load_row<T, LPE, LPH, MODE>(c, row, el, valid, rr, acc);
-    const int lg = (threadIdx.x & (kWave - 1)) / LPE;     // lane group = (row of the wave, slot)
-    const int4 cols = *reinterpret_cast<const int4*>(rec.col + lg * kUnroll);
+    const int4 cols = rec_edges_early<T, MODE>() ? rec.cols : *reinterpret_cast<const int4*>(rec.col_p);
     int nb[kUnroll] = {cols.x, cols.y, cols.z, cols.w};
     int ed[kUnroll] = {0, 0, 0, 0};
     bool ok[kUnroll];
@@ -554,10 +588,17 @@ __device__ __forceinline__ void walk_record(const Common& c, const SideArgs& s, 
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u) ed[u] = s.eid[start + min(slot + u * S, max(n - 1, 0))];
         } else {
-            const int4 e4 = *reinterpret_cast<const int4*>(rec.eid + lg * kUnroll);
+            const int4 e4 = rec_edges_early<T, MODE>() ? rec.eids : *reinterpret_cast<const int4*>(rec.eid_p);
             ed[0] = e4.x; ed[1] = e4.y; ed[2] = e4.z; ed[3] = e4.w;
         }
     }
+    // The ids are complete here, on every path (the map above is a second look-up that only some calls make), and
+    // only then is the row's own data asked for: it and the gathers of the step go out back to back, and nothing
+    // behind a branch makes the gathers wait for the row.
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) asm volatile("" ::"v"(nb[u]), "v"(ed[u]));
+    RowRegs<T> rr;
+    load_row<T, LPE, LPH, MODE>(c, row, el, valid, rr, acc);
     edge_step<T, LPE, LPH, MODE, HASB>(c, s, rr, nb, ed, ok, el, acc);
 }
 
@@ -602,14 +643,21 @@ __device__ __forceinline__ void write_row(const Common& c, const SideArgs& s, co
 // class walks the plan's sorted view step by step; the others find their (at most S * kUnroll) edges
 // in the record itself.
 template <typename T, int LPE, int LPH, int S, int MODE, int HASB, bool TILES, bool INLINE>
-__device__ __forceinline__ void wave_rows(const Common& c, const SideArgs& s, const WaveRec<LPE>& rec) {
+__device__ __forceinline__ void wave_rows(const Common& c, const SideArgs& s, const RecLane& rec) {
     constexpr int G = LPE * S;
     const int lane = threadIdx.x & (kWave - 1);
     const int sub = lane / G, gl = lane % G;
     const int slot = gl / LPE, el = gl % LPE;
     bool valid = sub < (int)(__builtin_amdgcn_readfirstlane(rec.code) >> 8);
-    int row = 0, start = 0, len = 0;
-    if (valid) { row = rec.row[sub]; start = rec.start[sub]; len = rec.len[sub]; }
+    int row = rec.row, start = rec.start, len = rec.len;
+    // The record's words are waited for here, by all lanes: a wait that first happens inside a lane-masked block
+    // (the row's own loads below) makes the compiler wait for everything outstanding behind that block - the
+    // row's data - before the gathers may go out.
+    asm volatile("" ::"v"(row), "v"(start), "v"(len));
+    if (INLINE && rec_edges_early<T, MODE>())
+        asm volatile("" ::"v"(rec.cols.x), "v"(rec.cols.y), "v"(rec.cols.z), "v"(rec.cols.w), "v"(rec.eids.x), "v"(rec.eids.y),
+                     "v"(rec.eids.z), "v"(rec.eids.w));
+    if (!valid) { row = 0; start = 0; len = 0; }
     // block path: a row that has tiles and no edge here was written by the tile kernels (they see the same row
     // pointers); nothing of it is loaded or stored
     if (TILES) valid = valid && !(len == 0 && s.cover[row] != 0);
@@ -620,7 +668,7 @@ __device__ __forceinline__ void wave_rows(const Common& c, const SideArgs& s, co
 }
 
 template <typename T, int LPE, int LPH, int MODE, int HASB, bool TILES>
-__device__ __forceinline__ void wave_dispatch(const Common& c, const SideArgs& s, const WaveRec<LPE>& rec, const int kind) {
+__device__ __forceinline__ void wave_dispatch(const Common& c, const SideArgs& s, const RecLane& rec, const int kind) {
     switch (kind) {
         case 0: wave_rows<T, LPE, LPH, slots_for_class(LPE, 0), MODE, HASB, TILES, false>(c, s, rec); break;
         case 1: wave_rows<T, LPE, LPH, slots_for_class(LPE, 1), MODE, HASB, TILES, class_inline(LPE, 1)>(c, s, rec); break;
@@ -848,12 +896,12 @@ __global__ __launch_bounds__(kBlock) void k_attn_fwd(const Common c, const SideA
                                                      const WaveRec<LPE>* __restrict__ recs) {
     __shared__ BlockLds<LPE> lds;
     const WaveRec<LPE>* r0 = recs + (int64_t)blockIdx.x * (kBlock / kWave);
+    const RecLane rec = load_rec_lane<LPE, true>(r0[threadIdx.x >> 6]);      // in flight while the workgroup's code is looked at
     const uint32_t code0 = r0->code;
     if ((code0 & 7u) == kDescBlock) {          // uniform over the workgroup
         block_item<T, LPE, LPH, MODE_FWD, HASB, TILES>(c, s, r0->item, lds);
         return;
     }
-    const WaveRec<LPE>& rec = r0[threadIdx.x >> 6];
     const uint32_t code = __builtin_amdgcn_readfirstlane(rec.code);
     if ((code & 7u) == kDescNone) return;
     wave_dispatch<T, LPE, LPH, MODE_FWD, HASB, TILES>(c, s, rec, code & 7u);
@@ -867,13 +915,13 @@ __global__ __launch_bounds__(kBlock, 4) void k_attn_bwd(const Common c, const Si
     constexpr int HB_D = HASB == 3 ? 2 : HASB;
     constexpr int HB_S = HASB == 3 ? 2 : (HASB ? 1 : 0);
     const WaveRec<LPE>* r0 = recs + (int64_t)blockIdx.x * (kBlock / kWave);
+    const RecLane rec = load_rec_lane<LPE, sizeof(T) == 2>(r0[threadIdx.x >> 6]);      // in flight while the workgroup's code is looked at
     const uint32_t code0 = r0->code;
     if ((code0 & 7u) == kDescBlock) {          // uniform over the workgroup
         if (code0 & kDescSrcSide) block_item<T, LPE, LPH, MODE_BWD_SRC, HB_S, TILES>(c, ss, r0->item, lds);
         else block_item<T, LPE, LPH, MODE_BWD_DST, HB_D, TILES>(c, sd, r0->item, lds);
         return;
     }
-    const WaveRec<LPE>& rec = r0[threadIdx.x >> 6];
     const uint32_t code = __builtin_amdgcn_readfirstlane(rec.code);
     if ((code & 7u) == kDescNone) return;
     if (code & kDescSrcSide) wave_dispatch<T, LPE, LPH, MODE_BWD_SRC, HB_S, TILES>(c, ss, rec, code & 7u);
