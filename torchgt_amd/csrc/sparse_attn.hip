@@ -301,6 +301,13 @@ __device__ __forceinline__ void edge_step(const Common& c, const SideArgs& s, co
     }
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
+        if constexpr (sizeof(T) == 2) {
+            // The edge's rows are named here, outside the lane-masked block that uses them: the compiler otherwise
+            // moves their loads into that block (its only user), where they are asked for and waited for one edge
+            // at a time instead of with the other gathers of the step.
+            asm volatile("" ::"v"(g0[u].u.x), "v"(g0[u].u.y), "v"(g0[u].u.z), "v"(g0[u].u.w), "v"(g1[u].u.x), "v"(g1[u].u.y),
+                         "v"(g1[u].u.z), "v"(g1[u].u.w));
+        }
         if (ok[u]) {
             float x0[8], x1[8];
             unpack(g0[u], x0);
