@@ -36,6 +36,22 @@ __device__ __forceinline__ short f2bf(float f) {
     return __builtin_bit_cast(short, b);
 }
 __device__ __forceinline__ float bf2f(short s) { return __uint_as_float(((uint32_t)(uint16_t)s) << 16); }
+// two / four floats -> bf16 (round to nearest even), two values per conversion instruction
+__device__ __forceinline__ uint32_t cvt_pk(float lo, float hi) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    f32x2 x;
+    x.x = lo; x.y = hi;
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
+}
+typedef short short4_pk __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ short4_pk pack4(float a, float b, float c, float d) {
+    typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+    u2 r;
+    r.x = cvt_pk(a, b);
+    r.y = cvt_pk(c, d);
+    return __builtin_bit_cast(short4_pk, r);
+}
 
 // four consecutive elements as bf16 bits
 __device__ __forceinline__ short4_t ld4(const dbf16* p) {
@@ -43,14 +59,10 @@ __device__ __forceinline__ short4_t ld4(const dbf16* p) {
 }
 __device__ __forceinline__ short4_t ld4(const float* p) {
     const float4_t f = *reinterpret_cast<const float4_t*>(p);
-    short4_t r;
-    r.x = f2bf(f.x); r.y = f2bf(f.y); r.z = f2bf(f.z); r.w = f2bf(f.w);
-    return r;
+    return pack4(f.x, f.y, f.z, f.w);
 }
 __device__ __forceinline__ void st4(dbf16* p, float a, float b, float c, float d) {
-    short4_t r;
-    r.x = f2bf(a); r.y = f2bf(b); r.z = f2bf(c); r.w = f2bf(d);
-    *reinterpret_cast<short4_t*>(p) = r;
+    *reinterpret_cast<short4_t*>(p) = pack4(a, b, c, d);
 }
 __device__ __forceinline__ void st4(float* p, float a, float b, float c, float d) {
     float4_t r;
@@ -677,8 +689,7 @@ __global__ __launch_bounds__(64 * NT, 2) void k_dense_fwd(const T* __restrict__ 
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             short4_t pb;
-            pb.x = f2bf(sc[4 * t + 0]); pb.y = f2bf(sc[4 * t + 1]);
-            pb.z = f2bf(sc[4 * t + 2]); pb.w = f2bf(sc[4 * t + 3]);
+            pb = pack4(sc[4 * t + 0], sc[4 * t + 1], sc[4 * t + 2], sc[4 * t + 3]);
             short4_t av = zero4();
             if (col < D) av = *reinterpret_cast<const short4_t*>(&v_tr[col * (SP + 4) + kb + 4 * t]);
             if (kSumOnMfma && col == D) { av.x = one_bits; av.y = one_bits; av.z = one_bits; av.w = one_bits; }
@@ -717,7 +728,7 @@ __global__ __launch_bounds__(64 * NT, 2) void k_dense_fwd(const T* __restrict__ 
             if (DROP) s4[r] = drop_keep(da, rh, kb + r) ? s4[r] : 0.f;
         }
         short4_t pb;
-        pb.x = f2bf(s4[0]); pb.y = f2bf(s4[1]); pb.z = f2bf(s4[2]); pb.w = f2bf(s4[3]);
+        pb = pack4(s4[0], s4[1], s4[2], s4[3]);
         short4_t av = zero4();
         if (col < D) av = *reinterpret_cast<const short4_t*>(&v_tr[col * (SP + 4) + kb]);
         if (kSumOnMfma && col == D) { av.x = one_bits; av.y = one_bits; av.z = one_bits; av.w = one_bits; }
@@ -941,8 +952,7 @@ __global__ __launch_bounds__(64 * NT, 2) void k_dense_bwd(const T* __restrict__ 
             short4_t db[4];
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-                db[t].x = f2bf(sc[4 * t + 0]); db[t].y = f2bf(sc[4 * t + 1]);
-                db[t].z = f2bf(sc[4 * t + 2]); db[t].w = f2bf(sc[4 * t + 3]);
+                db[t] = pack4(sc[4 * t + 0], sc[4 * t + 1], sc[4 * t + 2], sc[4 * t + 3]);
             }
             if (acc_here && kb < S) {      // dS into the table accumulators (keys past the end carry zeros)
 #pragma unroll
@@ -1011,7 +1021,7 @@ __global__ __launch_bounds__(64 * NT, 2) void k_dense_bwd(const T* __restrict__ 
                     if (r < tail) acc_position(acc, s4[r], (int64_t)qi * S + kb + r);
             }
             short4_t db0;
-            db0.x = f2bf(s4[0]); db0.y = f2bf(s4[1]); db0.z = f2bf(s4[2]); db0.w = f2bf(s4[3]);
+            db0 = pack4(s4[0], s4[1], s4[2], s4[3]);
             short4_t ak = zero4();
             if (col < D) ak = *reinterpret_cast<const short4_t*>(&k_tr[col * (SP + 4) + kb]);
             dq = mfma(ak, db0, dq);
@@ -1098,10 +1108,8 @@ __global__ __launch_bounds__(64 * NT, 2) void k_dense_bwd(const T* __restrict__ 
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
                 short4_t db, pb;
-                db.x = f2bf(sc[4 * t + 0]); db.y = f2bf(sc[4 * t + 1]);
-                db.z = f2bf(sc[4 * t + 2]); db.w = f2bf(sc[4 * t + 3]);
-                pb.x = f2bf(pr[4 * t + 0]); pb.y = f2bf(pr[4 * t + 1]);
-                pb.z = f2bf(pr[4 * t + 2]); pb.w = f2bf(pr[4 * t + 3]);
+                db = pack4(sc[4 * t + 0], sc[4 * t + 1], sc[4 * t + 2], sc[4 * t + 3]);
+                pb = pack4(pr[4 * t + 0], pr[4 * t + 1], pr[4 * t + 2], pr[4 * t + 3]);
                 short4_t aq = zero4(), ag = zero4();
                 if (col < D) {
                     aq = *reinterpret_cast<const short4_t*>(&q_tr[col * (SP + 4) + qt * 32 + t * 8 + half * 4]);
@@ -1138,8 +1146,8 @@ __global__ __launch_bounds__(64 * NT, 2) void k_dense_bwd(const T* __restrict__ 
                 s4[t] = in ? pv * (dp[t] * ks - D4[t]) : 0.f;
             }
             short4_t db, pb;
-            db.x = f2bf(s4[0]); db.y = f2bf(s4[1]); db.z = f2bf(s4[2]); db.w = f2bf(s4[3]);
-            pb.x = f2bf(p4[0]); pb.y = f2bf(p4[1]); pb.z = f2bf(p4[2]); pb.w = f2bf(p4[3]);
+            db = pack4(s4[0], s4[1], s4[2], s4[3]);
+            pb = pack4(p4[0], p4[1], p4[2], p4[3]);
             short4_t aq = zero4(), ag = zero4();
             if (col < D) {
                 aq = *reinterpret_cast<const short4_t*>(&q_tr[col * (SP + 4) + qt * 32 + half * 4]);
@@ -1239,13 +1247,22 @@ template <> struct ColRegs<float> {
     __device__ __forceinline__ void set(int r, const float* p) { v[r] = *p; }
     __device__ __forceinline__ float get(int r) const { return v[r]; }
 };
-// rows past the end repeat the last one (a valid address; their scores are masked)
+// bias_gh: the [S, S] bias of this (graph, head), the same in all lanes; key: this lane's column.  Offsets are 32-bit
+// byte offsets (S * S elements): the per-element part (8 (r / 4) + r % 4) S is the same in all lanes, so an element costs
+// one add and one min next to a scalar base.  The min keeps rows past the end of a last, partial tile on the last
+// row of the column (a valid address; their scores are masked): o_last is that row's offset.
 template <typename T>
-__device__ __forceinline__ void load_col(const T* __restrict__ bcol, int qt, int half, int S, ColRegs<T>& c) {
+__device__ __forceinline__ void load_col(const T* __restrict__ bias_gh, int key, int qt, int half, int S, uint32_t o_last,
+                                         ColRegs<T>& c) {
+    const char* base = reinterpret_cast<const char*>(bias_gh);
+    uint32_t o0 = (uint32_t)((qt * 32 + 4 * half) * S + key) * (uint32_t)sizeof(T);
+    // (kept as one register: the compiler would otherwise carry the 16 element offsets through the tile loop, one
+    // increment each per tile, in registers the loop does not have)
+    asm volatile("" : "+v"(o0));
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-        const int qq = min(qt * 32 + 8 * (r / 4) + 4 * half + (r % 4), S - 1);
-        c.set(r, bcol + (int64_t)qq * S);
+        const uint32_t o = min(o0 + (uint32_t)((8 * (r / 4) + (r % 4)) * S) * (uint32_t)sizeof(T), o_last);
+        c.set(r, reinterpret_cast<const T*>(base + o));
     }
 }
 template <typename T>
@@ -1310,14 +1327,15 @@ __global__ __launch_bounds__(64 * NT, D == 8 ? 4 : 3) void k_dense_bwd1(const T*
     // this lane's key and the first slice of its bias column, requested before anything else
     const int k0 = wave * 32, ki = k0 + col;
     const bool kok = ki < S;
-    const T* bcol = hasb ? bias_gh + (kok ? ki : 0) : nullptr;
+    const int bkey = kok ? ki : 0;
+    const uint32_t o_last = (uint32_t)((S - 1) * S + bkey) * (uint32_t)sizeof(T);
     constexpr int kDepth = ColRegs<T>::kDepth;       // tiles whose bias is in flight or in use
     ColRegs<T> b0, b1, b2;                            // of query tiles qt, qt + 1, qt + 2
     zero_col(b0); zero_col(b1); zero_col(b2);
     const bool bload = hasb && kok && !vec_wave;
     if (bload) {
-        load_col(bcol, 0, half, S, b0);
-        if (NT > 1) load_col(bcol, 1, half, S, b1);
+        load_col(bias_gh, bkey, 0, half, S, o_last, b0);
+        if (NT > 1) load_col(bias_gh, bkey, 1, half, S, o_last, b1);
     }
     load_head<T, D, SP>(Q, g, h, S, H, q_rm, q_tr);
     load_head<T, D, SP>(K, g, h, S, H, k_rm, k_tr);
@@ -1361,8 +1379,8 @@ __global__ __launch_bounds__(64 * NT, D == 8 ? 4 : 3) void k_dense_bwd1(const T*
 #pragma unroll 1
         for (int qt = 0; qt < nt_full; ++qt) {
             if (bload) {      // the tile that will be needed kDepth - 1 tiles from now
-                if (kDepth == 3 && qt + 2 < NT) load_col(bcol, qt + 2, half, S, b2);
-                if (kDepth == 2 && qt + 1 < NT) load_col(bcol, qt + 1, half, S, b1);
+                if (kDepth == 3 && qt + 2 < NT) load_col(bias_gh, bkey, qt + 2, half, S, o_last, b2);
+                if (kDepth == 2 && qt + 1 < NT) load_col(bias_gh, bkey, qt + 1, half, S, o_last, b1);
             }
             float16_t sc = zero16(), dp = zero16();
 #pragma unroll
@@ -1398,19 +1416,21 @@ __global__ __launch_bounds__(64 * NT, D == 8 ? 4 : 3) void k_dense_bwd1(const T*
                 }
             }
             // dS of the tile, rounded to bf16 once: into the wave's LDS tile [query][key] ...
-            short dsb[16];
+            uint32_t dsp[8];          // pairs (r, r + 1), converted two at a time
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                dsb[r] = f2bf(sc[r]);
-                tq[(8 * (r / 4) + 4 * half + (r % 4)) * kTqPitch + col] = dsb[r];
+            for (int r = 0; r < 16; r += 2) {
+                dsp[r / 2] = cvt_pk(sc[r], sc[r + 1]);
+                tq[(8 * (r / 4) + 4 * half + (r % 4)) * kTqPitch + col] = (short)(dsp[r / 2] & 0xffffu);
+                tq[(8 * (r / 4) + 4 * half + (r % 4) + 1) * kTqPitch + col] = (short)(dsp[r / 2] >> 16);
             }
             // ... and, as it is, the B operand of dK^T += Q^T dS (P likewise for dV^T += dout^T P)
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-                short4_t db, pb;
-                db.x = dsb[4 * t + 0]; db.y = dsb[4 * t + 1]; db.z = dsb[4 * t + 2]; db.w = dsb[4 * t + 3];
-                pb.x = f2bf(pr[4 * t + 0]); pb.y = f2bf(pr[4 * t + 1]);
-                pb.z = f2bf(pr[4 * t + 2]); pb.w = f2bf(pr[4 * t + 3]);
+                typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+                u2 dd2;
+                dd2.x = dsp[2 * t]; dd2.y = dsp[2 * t + 1];
+                const short4_t db = __builtin_bit_cast(short4_t, dd2);
+                const short4_t pb = pack4(pr[4 * t + 0], pr[4 * t + 1], pr[4 * t + 2], pr[4 * t + 3]);
                 short4_t aq = zero4(), ag = zero4();
                 if (col < D) {
                     aq = *reinterpret_cast<const short4_t*>(&q_tr[col * (SP + 4) + qt * 32 + t * 8 + half * 4]);
@@ -1486,8 +1506,8 @@ __global__ __launch_bounds__(64 * NT, D == 8 ? 4 : 3) void k_dense_bwd1(const T*
                 s4[t] = in ? pv * (dp[t] * ks - D4[t]) : 0.f;
             }
             short4_t db, pb;
-            db.x = f2bf(s4[0]); db.y = f2bf(s4[1]); db.z = f2bf(s4[2]); db.w = f2bf(s4[3]);
-            pb.x = f2bf(p4[0]); pb.y = f2bf(p4[1]); pb.z = f2bf(p4[2]); pb.w = f2bf(p4[3]);
+            db = pack4(s4[0], s4[1], s4[2], s4[3]);
+            pb = pack4(p4[0], p4[1], p4[2], p4[3]);
             short4_t aq = zero4(), ag = zero4();
             if (col < D) {
                 aq = *reinterpret_cast<const short4_t*>(&q_tr[col * (SP + 4) + qt * 32 + half * 4]);
