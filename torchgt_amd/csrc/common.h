@@ -15,7 +15,7 @@ constexpr int kBlock = 256;          // threads per workgroup of the attention k
 constexpr int kWaveRowMax = 256;     // a row of up to this many edges is walked by (part of) one wave
 constexpr int kBlockSeg = 1024;      // longer rows are walked by whole workgroups, in segments of at most this many edges
 constexpr int kSpreadSegs = 8;       // rows with more segments than this get shorter segments:
-constexpr int kSpreadSeg = 128;      // their length (more workgroups, each next to the rows of its sources)
+constexpr int kSpreadSeg = 256;      // their length (more workgroups, each next to the rows of its sources; 128 and 512 measured slower)
 constexpr int kWindowRows = 128;     // rows of one schedule window (consecutive node ids walked together on one XCD)
 constexpr int kCombineFan = 32;      // partial slots one combine step adds (= lane groups of a workgroup at 8 lanes per edge)
 constexpr int kNumClass = 5;         // wave item length classes: >32, <=32, <=16, <=8, <=4
