@@ -126,10 +126,21 @@ __device__ __forceinline__ void zero_bare_rows(const BareRows& br, int HD, int H
 #ifndef TGT_TILE_DST_OCC
 #define TGT_TILE_DST_OCC 4
 #endif
-template <int HD> constexpr int fwd_occupancy() { return HD <= 64 ? TGT_TILE_FWD_OCC : 4; }
-template <typename T, int HD> constexpr int dst_occupancy() { return HD <= 64 && sizeof(T) == 2 ? TGT_TILE_DST_OCC : 3; }
+#ifndef TGT_TILE_SRC_OCC
+#define TGT_TILE_SRC_OCC 4
+#endif
+template <int HDL> constexpr int fwd_occupancy() { return TGT_TILE_FWD_OCC; }
+template <typename T, int HDL> constexpr int dst_occupancy() { return TGT_TILE_DST_OCC; }
+// Heads one wave works on.  A group of tiles is shared out over H / heads_per_wave waves, each with its own 32
+// elements of every row (four heads of 8, two of 16): half the accumulators and half the LDS per wave of what all
+// eight heads took, so that twice the waves are resident - the kernels wait on chains of loads, LDS and matrix steps,
+// and the number of waves in flight is what hides them.  Each wave stages just its 64-byte share of the rows.
+#ifndef TGT_TILE_HDL
+#define TGT_TILE_HDL 32
+#endif
+template <int D, int H> constexpr int heads_per_wave() { return H * D <= TGT_TILE_HDL ? H : (TGT_TILE_HDL / D > 0 ? TGT_TILE_HDL / D : 1); }
 // waves (= tile groups) per workgroup of the tile kernels: as many as keep the static LDS under 64 KB
-template <int HD> constexpr int tile_waves() { return HD > 64 ? 2 : 4; }
+template <int HDL> constexpr int tile_waves() { return 4; }
 
 // LDS images of a block of 16 node rows (all heads, HD = H*D elements per row, bf16 bits):
 //   row-major   rm[row * (HD + 4) + e]   - the A operand "16 rows x 4 consecutive elements"
@@ -142,8 +153,8 @@ template <int HD> constexpr int tr_size() { return HD * 20; }
 // fetches 16-byte pieces of consecutive memory.  Loading and storing are separate steps so that a kernel can ask
 // for the rows of all its tensors before it waits for the first of them.
 // a piece in registers: eight bf16 values (float inputs are rounded as they arrive)
-template <typename T, int HD> struct RowPieces {
-    static constexpr int CPR = HD / 8;                      // 8-element pieces per row
+template <typename T, int HDL> struct RowPieces {
+    static constexpr int CPR = HDL / 8;                     // 8-element pieces per row
     static constexpr int ITERS = (kTile * CPR + 63) / 64;
     uint4 p[ITERS];
 };
@@ -160,25 +171,26 @@ __device__ __forceinline__ void unpack_piece(const uint4& u, short (&v)[8]) {
     v[4] = (short)(u.z & 0xffffu); v[5] = (short)(u.z >> 16);
     v[6] = (short)(u.w & 0xffffu); v[7] = (short)(u.w >> 16);
 }
-template <typename T, int HD>
-__device__ __forceinline__ void load_rows(const T* __restrict__ X, int row0, int lane, RowPieces<T, HD>& rp) {
-    constexpr int CPR = RowPieces<T, HD>::CPR;
+// elements [e_off, e_off + HDL) of rows row0 .. row0 + 15 of X ([N, HD])
+template <typename T, int HD, int HDL>
+__device__ __forceinline__ void load_rows(const T* __restrict__ X, int row0, int e_off, int lane, RowPieces<T, HDL>& rp) {
+    constexpr int CPR = RowPieces<T, HDL>::CPR;
 #pragma unroll
-    for (int i = 0; i < RowPieces<T, HD>::ITERS; ++i) {
+    for (int i = 0; i < RowPieces<T, HDL>::ITERS; ++i) {
         const int c = i * 64 + lane;
-        // rows are contiguous: a scalar base (row0 is the same in all lanes) plus a 32-bit lane offset; the empty
-        // statement keeps the sum from being re-associated into a 64-bit address per lane held across the tile loop
-        const char* base = reinterpret_cast<const char*>(X) + (int64_t)row0 * HD * (int)sizeof(T);
+        // a scalar base (row0 and e_off are the same in all lanes) plus a 32-bit lane offset; the empty statement
+        // keeps the sum from being re-associated into a 64-bit address per lane held across the tile loop
+        const char* base = reinterpret_cast<const char*>(X) + ((int64_t)row0 * HD + e_off) * (int)sizeof(T);
         asm volatile("" : "+s"(base));
         if (kTile * CPR % 64 == 0 || c < kTile * CPR)
-            load_piece(reinterpret_cast<const T*>(base + (uint32_t)(c * 8 * (int)sizeof(T))), rp.p[i]);
+            load_piece(reinterpret_cast<const T*>(base + (uint32_t)(((c / CPR) * HD + (c % CPR) * 8) * (int)sizeof(T))), rp.p[i]);
     }
 }
-template <typename T, int HD>
-__device__ __forceinline__ void store_rows(const RowPieces<T, HD>& rp, short* __restrict__ rm, short* __restrict__ tr, int lane) {
-    constexpr int CPR = RowPieces<T, HD>::CPR;
+template <typename T, int HDL>
+__device__ __forceinline__ void store_rows(const RowPieces<T, HDL>& rp, short* __restrict__ rm, short* __restrict__ tr, int lane) {
+    constexpr int CPR = RowPieces<T, HDL>::CPR;
 #pragma unroll
-    for (int i = 0; i < RowPieces<T, HD>::ITERS; ++i) {
+    for (int i = 0; i < RowPieces<T, HDL>::ITERS; ++i) {
         const int c = i * 64 + lane;
         if (kTile * CPR % 64 != 0 && c >= kTile * CPR) break;
         const int row = c / CPR, e0 = (c % CPR) * 8;
@@ -188,8 +200,8 @@ __device__ __forceinline__ void store_rows(const RowPieces<T, HD>& rp, short* __
             bshort4 lo, hi;
             lo.x = v[0]; lo.y = v[1]; lo.z = v[2]; lo.w = v[3];
             hi.x = v[4]; hi.y = v[5]; hi.z = v[6]; hi.w = v[7];
-            *reinterpret_cast<bshort4*>(&rm[row * (HD + 4) + e0]) = lo;
-            *reinterpret_cast<bshort4*>(&rm[row * (HD + 4) + e0 + 4]) = hi;
+            *reinterpret_cast<bshort4*>(&rm[row * (HDL + 4) + e0]) = lo;
+            *reinterpret_cast<bshort4*>(&rm[row * (HDL + 4) + e0 + 4]) = hi;
         }
         if (tr) {
 #pragma unroll
@@ -198,8 +210,8 @@ __device__ __forceinline__ void store_rows(const RowPieces<T, HD>& rp, short* __
     }
 }
 // Whether the next tile's rows are asked for while the current one is worked on: where the pieces in flight fit the
-// registers next to the accumulators (2-byte elements, up to 64 per row)
-template <typename T, int HD> constexpr bool tile_prefetch() { return sizeof(T) == 2 && HD <= 64; }
+// registers next to the accumulators (2-byte elements)
+template <typename T, int HDL> constexpr bool tile_prefetch() { return sizeof(T) == 2 && HDL <= 64; }
 // Hides where a scalar came from: addresses formed from the result cannot be computed before this point.  Put
 // behind a kernel's tile loop it keeps the epilogue's pointers out of the registers the loop needs.
 __device__ __forceinline__ int late_scalar(int x) { asm volatile("" : "+s"(x)); return x; }
@@ -229,7 +241,7 @@ __device__ __forceinline__ void wave_lds_fence() {
 // the output rows and Z themselves; otherwise it does so for the destinations that have no remaining edge and
 // leaves fp32 sums of the others for the sparse kernel to add (which skips the former).
 template <typename T, int D, int H, bool FINAL>
-__global__ __launch_bounds__(64 * tile_waves<H * D>(), fwd_occupancy<H * D>()) void k_tile_fwd(const int4* __restrict__ grp_rec,
+__global__ __launch_bounds__((64 * tile_waves<heads_per_wave<D, H>() * D>()), (fwd_occupancy<heads_per_wave<D, H>() * D>())) void k_tile_fwd(const int4* __restrict__ grp_rec,
                                                               const int32_t* __restrict__ tile_r0, int n_groups,
                                                               const T* __restrict__ Q, const T* __restrict__ K,
                                                               const T* __restrict__ V, float* __restrict__ acc,
@@ -238,19 +250,21 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), fwd_occupancy<H * D>()) v
                                                               const int32_t* __restrict__ rem_rowptr, const BareRows bare,
                                                               float inv_scale) {
     constexpr int HD = H * D;
-    constexpr int kTileWaves = tile_waves<HD>();
-    constexpr bool kPrefetch = tile_prefetch<T, HD>();
+    constexpr int HW = heads_per_wave<D, H>(), NP = H / HW, HDL = HW * D;     // this wave's heads: h0 .. h0 + HW - 1
+    constexpr int kTileWaves = tile_waves<HDL>();
+    constexpr bool kPrefetch = tile_prefetch<T, HDL>();
     const float scale2 = inv_scale * kLog2e;
-    __shared__ short lds[kTileWaves * (rm_size<HD>() + tr_size<HD>())];
+    __shared__ short lds[kTileWaves * (rm_size<HDL>() + tr_size<HDL>())];
     if ((int)blockIdx.x >= bare.first_block) {      // uniform over the workgroup
         zero_bare_rows<T>(bare, HD, H, out, (T*)nullptr, Zout, rem_rowptr);
         return;
     }
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int g = blockIdx.x * kTileWaves + wave;
+    const int wave = wave_uniform(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int gw = blockIdx.x * kTileWaves + wave;
+    const int g = gw / NP, h0 = (gw % NP) * HW;
     if (g >= n_groups) return;
-    short* k_rm = lds + wave * (rm_size<HD>() + tr_size<HD>());
-    short* v_tr = k_rm + rm_size<HD>();
+    short* k_rm = lds + wave * (rm_size<HDL>() + tr_size<HDL>());
+    short* v_tr = k_rm + rm_size<HDL>();
     const int col = lane & 15, kq = lane >> 4;
     const bool kval = kq * 4 < D;
     const int kmask = kval ? -1 : 0;
@@ -259,42 +273,42 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), fwd_occupancy<H * D>()) v
     const int4 gr = grp_rec[g];
     const int c0 = wave_uniform(gr.x), t0 = wave_uniform(gr.y), t1 = wave_uniform(gr.z);
     int r0 = wave_uniform(gr.w);
-    RowPieces<T, HD> pk, pv;
-    load_rows<T, HD>(K, r0, lane, pk);         // asked for before anything waits
-    load_rows<T, HD>(V, r0, lane, pv);
-    bshort4 bq[H];
+    RowPieces<T, HDL> pk, pv;
+    load_rows<T, HD, HDL>(K, r0, h0 * D, lane, pk);         // asked for before anything waits
+    load_rows<T, HD, HDL>(V, r0, h0 * D, lane, pv);
+    bshort4 bq[HW];
 #pragma unroll
-    for (int h = 0; h < H; ++h) {
+    for (int h = 0; h < HW; ++h) {
         bq[h] = t_zero4();
-        if (kval) bq[h] = t_ld4(Q + (int64_t)(c0 + col) * HD + h * D + kq * 4);
+        if (kval) bq[h] = t_ld4(Q + (int64_t)(c0 + col) * HD + (h0 + h) * D + kq * 4);
     }
     // a destination without remaining edges (row pointers of the plan that holds them) is finished here as well
     bool fin = true;
     if (!FINAL) fin = rem_rowptr[c0 + col + 1] == rem_rowptr[c0 + col];
-    bfloat4 o[H];
-    float z[H];
+    bfloat4 o[HW];
+    float z[HW];
 #pragma unroll
-    for (int h = 0; h < H; ++h) { o[h] = t_zerof(); z[h] = 0.f; }
+    for (int h = 0; h < HW; ++h) { o[h] = t_zerof(); z[h] = 0.f; }
     for (int t = t0; t < t1; ++t) {
         if (!kPrefetch && t > t0) {
             r0 = wave_uniform(tile_r0[t]);
-            load_rows<T, HD>(K, r0, lane, pk);
-            load_rows<T, HD>(V, r0, lane, pv);
+            load_rows<T, HD, HDL>(K, r0, h0 * D, lane, pk);
+            load_rows<T, HD, HDL>(V, r0, h0 * D, lane, pv);
         }
         wave_lds_fence();                      // the previous tile's reads are done
-        store_rows<T, HD>(pk, k_rm, nullptr, lane);
-        store_rows<T, HD>(pv, nullptr, v_tr, lane);
+        store_rows<T, HDL>(pk, k_rm, nullptr, lane);
+        store_rows<T, HDL>(pv, nullptr, v_tr, lane);
         wave_lds_fence();
         if (kPrefetch && t + 1 < t1) {         // the next tile's rows travel while this one is worked on
             r0 = wave_uniform(tile_r0[t + 1]);
-            load_rows<T, HD>(K, r0, lane, pk);
-            load_rows<T, HD>(V, r0, lane, pv);
+            load_rows<T, HD, HDL>(K, r0, h0 * D, lane, pk);
+            load_rows<T, HD, HDL>(V, r0, h0 * D, lane, pv);
         }
 #pragma unroll
-        for (int h = 0; h < H; ++h) {
+        for (int h = 0; h < HW; ++h) {
             // every lane reads (no lane mask around the LDS reads): lanes beyond the head's D get zeros by an AND, and
             // what the rows dd >= D of the second product hold is never stored
-            const bshort4 ak = t_and4(a_rows<HD>(k_rm, col, h * D + (kq * 4) % D), kmask);
+            const bshort4 ak = t_and4(a_rows<HDL>(k_rm, col, h * D + (kq * 4) % D), kmask);
             const bfloat4 sc = mfma16(ak, bq[h], t_zerof());       // S^T[source 4kq+r][destination col]
             float w[4];
 #pragma unroll
@@ -308,23 +322,23 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), fwd_occupancy<H * D>()) v
     }
     const int c0e = late_scalar(c0);
 #pragma unroll
-    for (int h = 0; h < H; ++h) {
+    for (int h = 0; h < HW; ++h) {
         float zz = z[h];
         zz += __shfl_xor(zz, 16);
         zz += __shfl_xor(zz, 32);
         if (fin) {
             const float inv = 1.0f / (zz + kTileEps);
-            if (kval) t_st4(out + (int64_t)(c0e + col) * HD + h * D + kq * 4, o[h].x * inv, o[h].y * inv, o[h].z * inv, o[h].w * inv);
+            if (kval) t_st4(out + (int64_t)(c0e + col) * HD + (h0 + h) * D + kq * 4, o[h].x * inv, o[h].y * inv, o[h].z * inv, o[h].w * inv);
         } else if (kval) {
-            *reinterpret_cast<bfloat4*>(acc + (int64_t)(c0e + col) * HD + h * D + kq * 4) = o[h];
+            *reinterpret_cast<bfloat4*>(acc + (int64_t)(c0e + col) * HD + (h0 + h) * D + kq * 4) = o[h];
         }
-        if (kq == 0) (fin ? Zout : Zp)[(int64_t)(c0e + col) * H + h] = zz;
+        if (kq == 0) (fin ? Zout : Zp)[(int64_t)(c0e + col) * H + h0 + h] = zz;
     }
 }
 
 // Same grouping: dQ of the tiles.  nd[i,h] = (1/(Z+eps), dout.out) of the FINAL output.
 template <typename T, int D, int H, bool FINAL>
-__global__ __launch_bounds__(64 * tile_waves<H * D>(), (dst_occupancy<T, H * D>())) void k_tile_bwd_dst(const int4* __restrict__ grp_rec,
+__global__ __launch_bounds__((64 * tile_waves<heads_per_wave<D, H>() * D>()), (dst_occupancy<T, heads_per_wave<D, H>() * D>())) void k_tile_bwd_dst(const int4* __restrict__ grp_rec,
                                                                   const int32_t* __restrict__ tile_r0, int n_groups,
                                                                   const T* __restrict__ Q, const T* __restrict__ K,
                                                                   const T* __restrict__ V, const T* __restrict__ dO,
@@ -333,21 +347,23 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), (dst_occupancy<T, H * D>(
                                                                   const int32_t* __restrict__ rem_rowptr,
                                                                   const BareRows bare, float inv_scale) {
     constexpr int HD = H * D;
-    constexpr int kTileWaves = tile_waves<HD>();
-    constexpr bool kPrefetch = tile_prefetch<T, HD>();
+    constexpr int HW = heads_per_wave<D, H>(), NP = H / HW, HDL = HW * D;     // this wave's heads: h0 .. h0 + HW - 1
+    constexpr int kTileWaves = tile_waves<HDL>();
+    constexpr bool kPrefetch = tile_prefetch<T, HDL>();
     const float scale2 = inv_scale * kLog2e;
-    constexpr int PER_WAVE = 2 * rm_size<HD>() + tr_size<HD>();
+    constexpr int PER_WAVE = 2 * rm_size<HDL>() + tr_size<HDL>();
     __shared__ short lds[kTileWaves * PER_WAVE];
     if ((int)blockIdx.x >= bare.first_block) {
         zero_bare_rows<T>(bare, HD, H, dq_out, (T*)nullptr, (float*)nullptr, rem_rowptr);
         return;
     }
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int g = blockIdx.x * kTileWaves + wave;
+    const int wave = wave_uniform(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int gw = blockIdx.x * kTileWaves + wave;
+    const int g = gw / NP, h0 = (gw % NP) * HW;
     if (g >= n_groups) return;
     short* k_rm = lds + wave * PER_WAVE;
-    short* v_rm = k_rm + rm_size<HD>();
-    short* k_tr = v_rm + rm_size<HD>();
+    short* v_rm = k_rm + rm_size<HDL>();
+    short* k_tr = v_rm + rm_size<HDL>();
     const int col = lane & 15, kq = lane >> 4;
     const bool kval = kq * 4 < D;
     // one 16-byte record per group: (first node, tile range, the first tile's other side) - a wave with one tile, the
@@ -355,47 +371,47 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), (dst_occupancy<T, H * D>(
     const int4 gr = grp_rec[g];
     const int c0 = wave_uniform(gr.x), t0 = wave_uniform(gr.y), t1 = wave_uniform(gr.z);
     int r0 = wave_uniform(gr.w);
-    RowPieces<T, HD> pk, pv;
-    load_rows<T, HD>(K, r0, lane, pk);
-    load_rows<T, HD>(V, r0, lane, pv);
+    RowPieces<T, HDL> pk, pv;
+    load_rows<T, HD, HDL>(K, r0, h0 * D, lane, pk);
+    load_rows<T, HD, HDL>(V, r0, h0 * D, lane, pv);
     bool fin = true;                            // no remaining edge into this row
     if (!FINAL) fin = rem_rowptr[c0 + col + 1] == rem_rowptr[c0 + col];
-    bshort4 bq[H], bg[H];
-    float2 ndv[H];
-    bfloat4 dq[H];
+    bshort4 bq[HW], bg[HW];
+    float2 ndv[HW];
+    bfloat4 dq[HW];
 #pragma unroll
-    for (int h = 0; h < H; ++h) {
+    for (int h = 0; h < HW; ++h) {
         bq[h] = t_zero4(); bg[h] = t_zero4();
         if (kval) {
-            bq[h] = t_ld4(Q + (int64_t)(c0 + col) * HD + h * D + kq * 4);
-            bg[h] = t_ld4(dO + (int64_t)(c0 + col) * HD + h * D + kq * 4);
+            bq[h] = t_ld4(Q + (int64_t)(c0 + col) * HD + (h0 + h) * D + kq * 4);
+            bg[h] = t_ld4(dO + (int64_t)(c0 + col) * HD + (h0 + h) * D + kq * 4);
         }
-        ndv[h] = nd[(int64_t)(c0 + col) * H + h];
+        ndv[h] = nd[(int64_t)(c0 + col) * H + h0 + h];
         dq[h] = t_zerof();
     }
     for (int t = t0; t < t1; ++t) {
         if (!kPrefetch && t > t0) {
             r0 = wave_uniform(tile_r0[t]);
-            load_rows<T, HD>(K, r0, lane, pk);
-            load_rows<T, HD>(V, r0, lane, pv);
+            load_rows<T, HD, HDL>(K, r0, h0 * D, lane, pk);
+            load_rows<T, HD, HDL>(V, r0, h0 * D, lane, pv);
         }
         wave_lds_fence();
-        store_rows<T, HD>(pk, k_rm, k_tr, lane);
-        store_rows<T, HD>(pv, v_rm, nullptr, lane);
+        store_rows<T, HDL>(pk, k_rm, k_tr, lane);
+        store_rows<T, HDL>(pv, v_rm, nullptr, lane);
         wave_lds_fence();
         if (kPrefetch && t + 1 < t1) {
             r0 = wave_uniform(tile_r0[t + 1]);
-            load_rows<T, HD>(K, r0, lane, pk);
-            load_rows<T, HD>(V, r0, lane, pv);
+            load_rows<T, HD, HDL>(K, r0, h0 * D, lane, pk);
+            load_rows<T, HD, HDL>(V, r0, h0 * D, lane, pv);
         }
 #pragma unroll
-        for (int h = 0; h < H; ++h) {
+        for (int h = 0; h < HW; ++h) {
             // operands of the lanes beyond the head's D: reads under a lane mask here - read by all lanes as in the
             // forward, the compiler moves more reads to the front than the registers of this occupancy hold
             bshort4 ak = t_zero4(), av = t_zero4();
             if (kval) {
-                ak = a_rows<HD>(k_rm, col, h * D + kq * 4);
-                av = a_rows<HD>(v_rm, col, h * D + kq * 4);
+                ak = a_rows<HDL>(k_rm, col, h * D + kq * 4);
+                av = a_rows<HDL>(v_rm, col, h * D + kq * 4);
             }
             const bfloat4 sc = mfma16(ak, bq[h], t_zerof());       // S^T[source][destination]
             const bfloat4 dp = mfma16(av, bg[h], t_zerof());       // dP^T = V dout^T
@@ -414,18 +430,18 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), (dst_occupancy<T, H * D>(
     const int c0e = late_scalar(c0);
     if (kval) {
 #pragma unroll
-        for (int h = 0; h < H; ++h) {
+        for (int h = 0; h < HW; ++h) {
             bfloat4 o;
             o.x = dq[h].x * inv_scale; o.y = dq[h].y * inv_scale; o.z = dq[h].z * inv_scale; o.w = dq[h].w * inv_scale;
-            if (fin) t_st4(dq_out + (int64_t)(c0e + col) * HD + h * D + kq * 4, o.x, o.y, o.z, o.w);
-            else *reinterpret_cast<bfloat4*>(dq_part + (int64_t)(c0e + col) * HD + h * D + kq * 4) = o;
+            if (fin) t_st4(dq_out + (int64_t)(c0e + col) * HD + (h0 + h) * D + kq * 4, o.x, o.y, o.z, o.w);
+            else *reinterpret_cast<bfloat4*>(dq_part + (int64_t)(c0e + col) * HD + (h0 + h) * D + kq * 4) = o;
         }
     }
 }
 
 // One wave per group of tiles that share their 16 SOURCES: dK and dV of the tiles.
 template <typename T, int D, int H, bool FINAL>
-__global__ __launch_bounds__(64 * tile_waves<H * D>(), 3) void k_tile_bwd_src(const int4* __restrict__ grp_rec,
+__global__ __launch_bounds__((64 * tile_waves<heads_per_wave<D, H>() * D>()), TGT_TILE_SRC_OCC) void k_tile_bwd_src(const int4* __restrict__ grp_rec,
                                                                   const int32_t* __restrict__ tile_c0, int n_groups,
                                                                   const T* __restrict__ Q, const T* __restrict__ K,
                                                                   const T* __restrict__ V, const T* __restrict__ dO,
@@ -436,86 +452,90 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 3) void k_tile_bwd_src(co
                                                                   const int32_t* __restrict__ rem_rowptr, const BareRows bare,
                                                                   float inv_scale) {
     constexpr int HD = H * D;
-    constexpr int kTileWaves = tile_waves<HD>();
-    constexpr bool kPrefetch = false;
+    constexpr int HW = heads_per_wave<D, H>(), NP = H / HW, HDL = HW * D;     // this wave's heads: h0 .. h0 + HW - 1
+    constexpr int kTileWaves = tile_waves<HDL>();
+    constexpr bool kPrefetch = tile_prefetch<T, HDL>();
     const float scale2 = inv_scale * kLog2e;
-    constexpr int PER_WAVE = 2 * rm_size<HD>() + 2 * tr_size<HD>() + 4 * kTile * H;   // + nd tile (float2 = 4 shorts)
+    constexpr int PER_WAVE = 2 * rm_size<HDL>() + 2 * tr_size<HDL>() + 4 * kTile * HW;   // + nd tile (float2 = 4 shorts)
     __shared__ __align__(16) short lds[kTileWaves * PER_WAVE];
     if ((int)blockIdx.x >= bare.first_block) {
         zero_bare_rows<T>(bare, HD, H, dk_out, dv_out, (float*)nullptr, rem_rowptr);
         return;
     }
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int g = blockIdx.x * kTileWaves + wave;
+    const int wave = wave_uniform(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int gw = blockIdx.x * kTileWaves + wave;
+    const int g = gw / NP, h0 = (gw % NP) * HW;
     if (g >= n_groups) return;
     short* q_rm = lds + wave * PER_WAVE;
-    short* g_rm = q_rm + rm_size<HD>();
-    short* q_tr = g_rm + rm_size<HD>();
-    short* g_tr = q_tr + tr_size<HD>();
-    float2* nd_l = reinterpret_cast<float2*>(g_tr + tr_size<HD>());     // [16 destinations][H]
+    short* g_rm = q_rm + rm_size<HDL>();
+    short* q_tr = g_rm + rm_size<HDL>();
+    short* g_tr = q_tr + tr_size<HDL>();
+    float2* nd_l = reinterpret_cast<float2*>(g_tr + tr_size<HDL>());     // [16 destinations][HW]
     const int col = lane & 15, kq = lane >> 4;
     const bool kval = kq * 4 < D;
     const int4 gr = grp_rec[g];
     const int r0 = wave_uniform(gr.x), t0 = wave_uniform(gr.y), t1 = wave_uniform(gr.z);
     int c0 = wave_uniform(gr.w);
-    RowPieces<T, HD> pq, pg;
-    load_rows<T, HD>(Q, c0, lane, pq);
-    load_rows<T, HD>(dO, c0, lane, pg);
-    constexpr int ND_ITERS = (kTile * H + 63) / 64;
+    RowPieces<T, HDL> pq, pg;
+    load_rows<T, HD, HDL>(Q, c0, h0 * D, lane, pq);
+    load_rows<T, HD, HDL>(dO, c0, h0 * D, lane, pg);
+    constexpr int ND_ITERS = (kTile * HW + 63) / 64;
     float2 ndr[ND_ITERS];
+    // entry e of the [16][HW] tile: destination c0 + e / HW, head h0 + e % HW
+    auto load_nd = [&](const int cc) {
 #pragma unroll
-    for (int i = 0; i < ND_ITERS; ++i)
-        if (kTile * H % 64 == 0 || i * 64 + lane < kTile * H) ndr[i] = nd[(int64_t)c0 * H + i * 64 + lane];   // rows c0..c0+15 are contiguous
+        for (int i = 0; i < ND_ITERS; ++i) {
+            const int e = i * 64 + lane;
+            if (kTile * HW % 64 == 0 || e < kTile * HW) ndr[i] = nd[(int64_t)(cc + e / HW) * H + h0 + e % HW];
+        }
+    };
+    load_nd(c0);
     bool fin = true;                            // no remaining edge out of this row
     if (!FINAL) fin = rem_rowptr[r0 + col + 1] == rem_rowptr[r0 + col];
-    bshort4 bk[H], bv[H];
-    bfloat4 dk[H], dv[H];
+    bshort4 bk[HW], bv[HW];
+    bfloat4 dk[HW], dv[HW];
 #pragma unroll
-    for (int h = 0; h < H; ++h) {
+    for (int h = 0; h < HW; ++h) {
         bk[h] = t_zero4(); bv[h] = t_zero4();
         if (kval) {
-            bk[h] = t_ld4(K + (int64_t)(r0 + col) * HD + h * D + kq * 4);
-            bv[h] = t_ld4(V + (int64_t)(r0 + col) * HD + h * D + kq * 4);
+            bk[h] = t_ld4(K + (int64_t)(r0 + col) * HD + (h0 + h) * D + kq * 4);
+            bv[h] = t_ld4(V + (int64_t)(r0 + col) * HD + (h0 + h) * D + kq * 4);
         }
         dk[h] = t_zerof(); dv[h] = t_zerof();
     }
     for (int t = t0; t < t1; ++t) {
         if (!kPrefetch && t > t0) {
             c0 = wave_uniform(tile_c0[t]);
-            load_rows<T, HD>(Q, c0, lane, pq);
-            load_rows<T, HD>(dO, c0, lane, pg);
-#pragma unroll
-            for (int i = 0; i < ND_ITERS; ++i)
-                if (kTile * H % 64 == 0 || i * 64 + lane < kTile * H) ndr[i] = nd[(int64_t)c0 * H + i * 64 + lane];
+            load_rows<T, HD, HDL>(Q, c0, h0 * D, lane, pq);
+            load_rows<T, HD, HDL>(dO, c0, h0 * D, lane, pg);
+            load_nd(c0);
         }
         wave_lds_fence();
-        store_rows<T, HD>(pq, q_rm, q_tr, lane);
-        store_rows<T, HD>(pg, g_rm, g_tr, lane);
+        store_rows<T, HDL>(pq, q_rm, q_tr, lane);
+        store_rows<T, HDL>(pg, g_rm, g_tr, lane);
 #pragma unroll
         for (int i = 0; i < ND_ITERS; ++i)
-            if (kTile * H % 64 == 0 || i * 64 + lane < kTile * H) nd_l[i * 64 + lane] = ndr[i];
+            if (kTile * HW % 64 == 0 || i * 64 + lane < kTile * HW) nd_l[i * 64 + lane] = ndr[i];
         wave_lds_fence();
         if (kPrefetch && t + 1 < t1) {
             c0 = wave_uniform(tile_c0[t + 1]);
-            load_rows<T, HD>(Q, c0, lane, pq);
-            load_rows<T, HD>(dO, c0, lane, pg);
-#pragma unroll
-            for (int i = 0; i < ND_ITERS; ++i)
-                if (kTile * H % 64 == 0 || i * 64 + lane < kTile * H) ndr[i] = nd[(int64_t)c0 * H + i * 64 + lane];
+            load_rows<T, HD, HDL>(Q, c0, h0 * D, lane, pq);
+            load_rows<T, HD, HDL>(dO, c0, h0 * D, lane, pg);
+            load_nd(c0);
         }
 #pragma unroll
-        for (int h = 0; h < H; ++h) {
+        for (int h = 0; h < HW; ++h) {
             bshort4 aq = t_zero4(), ag = t_zero4();
             if (kval) {
-                aq = a_rows<HD>(q_rm, col, h * D + kq * 4);
-                ag = a_rows<HD>(g_rm, col, h * D + kq * 4);
+                aq = a_rows<HDL>(q_rm, col, h * D + kq * 4);
+                ag = a_rows<HDL>(g_rm, col, h * D + kq * 4);
             }
             const bfloat4 sc = mfma16(aq, bk[h], t_zerof());       // S[destination 4kq+r][source col]
             const bfloat4 dp = mfma16(ag, bv[h], t_zerof());       // dP = dout V^T
             float pw[4], md[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const float2 ndv = nd_l[(4 * kq + r) * H + h];
+                const float2 ndv = nd_l[(4 * kq + r) * HW + h];
                 const float x2 = sc[r] * scale2;
                 const float p = t_weight(x2) * ndv.x;
                 const float dS = p * (dp[r] - ndv.y);
@@ -534,15 +554,15 @@ __global__ __launch_bounds__(64 * tile_waves<H * D>(), 3) void k_tile_bwd_src(co
     const int r0e = late_scalar(r0);
     if (kval) {
 #pragma unroll
-        for (int h = 0; h < H; ++h) {
+        for (int h = 0; h < HW; ++h) {
             bfloat4 o;
             o.x = dk[h].x * inv_scale; o.y = dk[h].y * inv_scale; o.z = dk[h].z * inv_scale; o.w = dk[h].w * inv_scale;
             if (fin) {
-                t_st4(dk_out + (int64_t)(r0e + col) * HD + h * D + kq * 4, o.x, o.y, o.z, o.w);
-                t_st4(dv_out + (int64_t)(r0e + col) * HD + h * D + kq * 4, dv[h].x, dv[h].y, dv[h].z, dv[h].w);
+                t_st4(dk_out + (int64_t)(r0e + col) * HD + (h0 + h) * D + kq * 4, o.x, o.y, o.z, o.w);
+                t_st4(dv_out + (int64_t)(r0e + col) * HD + (h0 + h) * D + kq * 4, dv[h].x, dv[h].y, dv[h].z, dv[h].w);
             } else {
-                *reinterpret_cast<bfloat4*>(dk_part + (int64_t)(r0e + col) * HD + h * D + kq * 4) = o;
-                *reinterpret_cast<bfloat4*>(dv_part + (int64_t)(r0e + col) * HD + h * D + kq * 4) = dv[h];
+                *reinterpret_cast<bfloat4*>(dk_part + (int64_t)(r0e + col) * HD + (h0 + h) * D + kq * 4) = o;
+                *reinterpret_cast<bfloat4*>(dv_part + (int64_t)(r0e + col) * HD + (h0 + h) * D + kq * 4) = dv[h];
             }
         }
     }
@@ -615,10 +635,11 @@ static int upload(DevBuf& b, const std::vector<X>& v, hipStream_t st) {
 template <typename T, int D, int H>
 static int tile_fwd_launch_s(const tgt_tiles* tl, const void* q, const void* k, const void* v, float* acc, float* Zp,
                              void* final_out, void* out, float* Zout, const int32_t* rem_rowptr, bool zero_rows, hipStream_t st) {
-    constexpr int W = tile_waves<H * D>();
+    constexpr int NP = H / heads_per_wave<D, H>();          // waves per group
+    constexpr int W = tile_waves<heads_per_wave<D, H>() * D>();
     const float inv_scale = 1.0f / sqrtf((float)D);
     KernelTimer t(KS_TILE_FWD, st);
-    const int gblocks = (tl->n_dst_groups + W - 1) / W;
+    const int gblocks = (tl->n_dst_groups * NP + W - 1) / W;
     const dim3 block(64 * W);
     // the rows without tiles are zeroed by workgroups appended to the same launch: all of them when the tiles are all
     // there is, else (zero_rows: the plan of the remaining edges schedules only rows with edges) those without edges
@@ -641,10 +662,11 @@ static int tile_bwd_launch_s(const tgt_tiles* tl, const void* q, const void* k, 
                              const float2* nd, float* dq, float* dk, float* dv, void* f_dq, void* f_dk, void* f_dv,
                              void* o_dq, void* o_dk, void* o_dv, const int32_t* rem_dst, const int32_t* rem_src,
                              bool zero_rows, hipStream_t st) {
-    constexpr int W = tile_waves<H * D>();
+    constexpr int NP = H / heads_per_wave<D, H>();          // waves per group
+    constexpr int W = tile_waves<heads_per_wave<D, H>() * D>();
     const float inv_scale = 1.0f / sqrtf((float)D);
     KernelTimer t(KS_TILE_BWD, st);
-    const int gdb = (tl->n_dst_groups + W - 1) / W, gsb = (tl->n_src_groups + W - 1) / W;
+    const int gdb = (tl->n_dst_groups * NP + W - 1) / W, gsb = (tl->n_src_groups * NP + W - 1) / W;
     const dim3 block(64 * W);
     const bool zr = f_dq || zero_rows;
     const int per = 64 * W / 8;
