@@ -535,7 +535,7 @@ int place(const std::vector<const Side*>& sides, int lpe, void** d_out, int32_t*
     // part 1 the segments homed at a window run `lead` windows ahead of the window's rows: close enough in
     // time for the rows to meet in the L2, and the last windows of a range end with short rows only - the
     // chain of a split row (partial slot, arrival, sums of the group and of the row) is not left for the end.
-    const int lead = env_int("TGT_SEGMENT_LEAD", 6);
+    const int lead = env_int("TGT_SEGMENT_LEAD", 3);
     XcdList xl[8];
     for (int x = 0; x < 8; ++x) {
         XcdList& wv = xl[x];
