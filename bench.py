@@ -63,10 +63,10 @@ def kernel_alg_bytes(name, N, E, H, d, esize, bpe):
 # bench line says when and on which commit of the kernels they were taken (a kernel change after that
 # commit makes them stale: measure again).
 MEASURED_TRAFFIC = {
-    ("config2", "f32"): {"attn_fwd": 239.2e6, "bwd_node_side": 38.9e6, "attn_bwd": 560.0e6},
-    ("config2", "bf16"): {"attn_fwd": 131.2e6, "bwd_node_side": 22.5e6, "attn_bwd": 320.1e6},
+    ("config2", "f32"): {"attn_fwd": 237.2e6, "bwd_node_side": 38.9e6, "attn_bwd": 546.6e6},
+    ("config2", "bf16"): {"attn_fwd": 131.1e6, "bwd_node_side": 22.5e6, "attn_bwd": 318.7e6},
 }
-MEASURED_TRAFFIC_AT = {"date": "2026-11-26", "kernels_as_of_commit": "b9b1fef",
+MEASURED_TRAFFIC_AT = {"date": "2026-11-26", "kernels_as_of_commit": "95a5294",
                        "summary": "profiles/sparse_attn_config2_hbm_traffic_pmc.txt"}
 
 
