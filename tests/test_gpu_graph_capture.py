@@ -4,7 +4,9 @@ against the eager result, with the program's own eager work and synchronisations
 import pytest
 import torch
 
-from torchgt_amd import GraphPlan, _lib, workloads
+import numpy as np
+
+from torchgt_amd import GraphPlan, TileSet, _lib, workloads
 
 pytestmark = pytest.mark.gpu
 
@@ -58,6 +60,56 @@ def test_sparse_step_replays_from_a_graph(cuda, dtype):
         for a, b in zip(got, (out, Z, dq, dk, dv, db)):
             assert torch.equal(a, b), f"replay {replay} differs from the eager step"
     plan.close()
+
+
+def test_block_step_replays_from_a_graph(cuda):
+    """The block path (tile kernels, the per-node side, the sparse kernels on the remaining edges with their plan
+    of rows that have edges) is kernel launches only as well: captured once, replayed on fresh inputs."""
+    rng = np.random.default_rng(3)
+    n, H, d = 2048, 8, 8
+    nb = n // 16
+    tiles = np.stack([rng.integers(0, nb, 300) * 16, rng.integers(0, nb, 300) * 16], 1).astype(np.int32)
+    rest = torch.from_numpy(rng.integers(0, n, (2, 1500))).to(cuda)
+    E = rest.shape[1]
+    ts = TileSet(tiles, n, cuda)
+    plan = GraphPlan(rest, n, rows_with_edges_only=True)
+    ws = ts.workspace(plan, H, d)
+    L = _lib.lib()
+    dtype, code = torch.bfloat16, _lib.DTYPE_BF16
+    q, k, v, dout, bias = _buffers(n, E, H, d, dtype, cuda, 0)
+    out = torch.empty_like(q)
+    Z = torch.empty(n, H, device=cuda)
+    dq, dk, dv, db = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q), torch.empty_like(bias)
+    P = lambda t: t.data_ptr()
+
+    def step(stream):
+        _lib.check(L.tgt_block_attn_fwd(ts.handle, plan.handle, P(q), P(k), P(v), P(bias), _lib.BIAS_EDGE_HEAD, H, d, code,
+                                        P(out), P(Z), P(ws), ws.numel(), stream))
+        _lib.check(L.tgt_block_attn_bwd(ts.handle, plan.handle, P(q), P(k), P(v), P(bias), _lib.BIAS_EDGE_HEAD, H, d, code,
+                                        P(out), P(Z), P(dout), P(dq), P(dk), P(dv), P(db), P(ws), ws.numel(), stream))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step(side.cuda_stream)                   # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(torch.cuda.current_stream().cuda_stream)
+    for replay in range(3):
+        nq, nk, nv, ndout, nbias = _buffers(n, E, H, d, dtype, cuda, 20 + replay)
+        for dst_t, src_t in ((q, nq), (k, nk), (v, nv), (dout, ndout), (bias, nbias)):
+            dst_t.copy_(src_t)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in (out, Z, dq, dk, dv, db)]
+        step(torch.cuda.current_stream().cuda_stream)      # eager, same buffers
+        torch.cuda.synchronize()
+        for a, b in zip(got, (out, Z, dq, dk, dv, db)):
+            assert torch.equal(a, b), f"replay {replay} differs from the eager step"
+    plan.close()
+    ts.close()
 
 
 def test_model_training_step_replays_from_a_graph(cuda):
